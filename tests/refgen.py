@@ -1,0 +1,122 @@
+"""Closed-form input generators taken from the reference's own tests.
+
+Only the formulas are restated (they are the reference's test vectors); each
+cites where the reference defines it.  All return numpy arrays.
+"""
+import numpy as np
+
+from oxydllm_amd import synth
+
+
+def awq_kat_small():
+    """awq.rs:954-1011: K=8, N=16, g=4; returns (qweight, qzeros, scales, expected[N,K])."""
+    K, N, g = 8, 16, 4
+    G = K // g
+    i = np.arange(K)[:, None]
+    j = np.arange(N)[None, :]
+    iweight = (i * 3 + j * 5 + 1) & 0xF
+    gi = np.arange(G)[:, None]
+    izero = (gi * 7 + j) & 0xF
+    scales = (np.float32(0.01) * (gi + 1).astype(np.float32)
+              + np.float32(0.001) * (j + 1).astype(np.float32)).astype(np.float32)
+    expected = np.zeros((N, K), dtype=np.float32)
+    for ii in range(K):
+        for jj in range(N):
+            w = int(iweight[ii, jj]) - int(izero[ii // g, jj])
+            expected[jj, ii] = np.float32(w) * scales[ii // g, jj]
+    return synth.pack_awq(iweight), synth.pack_awq(izero), scales, expected
+
+
+def gptq_kat(bits):
+    """awq.rs:1170-1283: K=32, N=16, g=16; 8-bit and 4-bit variants."""
+    K, N, g = 32, 16, 16
+    G = K // g
+    i = np.arange(K)[:, None]
+    j = np.arange(N)[None, :]
+    gi = np.arange(G)[:, None]
+    if bits == 8:
+        iweight = (i * 11 + j * 7) & 0xFF
+        izero = (gi * 31 + j * 17 + 1) & 0xFF
+        scales = (np.float32(0.02) * (gi + 1).astype(np.float32)
+                  + np.float32(0.003) * (j + 1).astype(np.float32)).astype(np.float32)
+    else:
+        iweight = (i * 3 + j * 5) & 0xF
+        izero = (gi * 2 + j) & 0xF
+        scales = (np.float32(0.01) * (gi + 1).astype(np.float32)
+                  + np.float32(0.002) * (j + 1).astype(np.float32)).astype(np.float32)
+    expected = np.zeros((N, K), dtype=np.float32)
+    for ii in range(K):
+        for jj in range(N):
+            q = int(iweight[ii, jj])
+            z = int(izero[ii // g, jj]) + 1
+            expected[jj, ii] = np.float32(q - z) * scales[ii // g, jj]
+    return (synth.pack_gptq_qweight(iweight, bits), synth.pack_gptq_qzeros(izero, bits),
+            scales, expected)
+
+
+def build_awq_triplet(K, N, g):
+    """metal_ops.rs:3668-3711: q=(5i+3j+1)&15, z=(7g+j+2)&15, s=0.01+0.003*((g+j)%5)."""
+    G = K // g
+    i = np.arange(K)[:, None]
+    j = np.arange(N)[None, :]
+    gi = np.arange(G)[:, None]
+    iweight = (i * 5 + j * 3 + 1) & 0xF
+    izero = (gi * 7 + j + 2) & 0xF
+    scales = (np.float32(0.01) + np.float32(0.003) * ((gi + j) % 5).astype(np.float32))
+    return synth.pack_awq(iweight), synth.pack_awq(izero), scales.astype(np.float32)
+
+
+def build_w8a16_triplet(K, N, g):
+    """metal_ops.rs:3975-4028; also returns ref_w [N,K] f32 built from the unpacked ints."""
+    G = K // g
+    i = np.arange(K)[:, None]
+    j = np.arange(N)[None, :]
+    gi = np.arange(G)[:, None]
+    iweight = (i * 11 + j * 7) & 0xFF
+    izero = (gi * 31 + j * 5 + 2) & 0xFF
+    scales = (np.float32(0.001) + np.float32(0.0007) * ((gi + j) % 17).astype(np.float32))
+    scales = scales.astype(np.float32)
+    zfull = np.repeat(izero, g, axis=0)
+    sfull = np.repeat(scales, g, axis=0)
+    ref_w = ((iweight - zfull).astype(np.float32) * sfull).T.copy()
+    return synth.pack_awq_8bit(iweight), synth.pack_awq_8bit(izero), scales, ref_w
+
+
+def build_gptq_triplet(bits, K, N, g):
+    """metal_ops.rs:4134-4183: q=(13i+7o)&mask, z=(31g+17o+1)&mask, s=0.002+0.0005*((g+o)%11)."""
+    G = K // g
+    mask = (1 << bits) - 1
+    i = np.arange(K)[:, None]
+    o = np.arange(N)[None, :]
+    gi = np.arange(G)[:, None]
+    iweight = (i * 13 + o * 7) & mask
+    izero = (gi * 31 + o * 17 + 1) & mask
+    scales = (np.float32(0.002) + np.float32(0.0005) * ((gi + o) % 11).astype(np.float32))
+    return (synth.pack_gptq_qweight(iweight, bits), synth.pack_gptq_qzeros(izero, bits),
+            scales.astype(np.float32))
+
+
+def x_gemv(K, mod=13, off=6.0, step=0.03):
+    """metal_ops.rs:3727-3729 (AWQ M=1): ((i % 13) - 6) * 0.03; GPTQ uses (17, 8, 0.02)."""
+    i = np.arange(K)
+    return (((i % mod).astype(np.float32) - np.float32(off)) * np.float32(step)).reshape(1, K)
+
+
+def batch_x(M, K):
+    """metal_ops.rs:3771-3779: ((i % 17) - 8) * 0.03 over the flat [M*K] index."""
+    i = np.arange(M * K)
+    return (((i % 17).astype(np.float32) - np.float32(8.0)) * np.float32(0.03)).reshape(M, K)
+
+
+def mxfp4_case(n=10, k=64):
+    """metal_ops.rs:6626-6631: blocks=(37i+11)&255, scales=125+i%5."""
+    nb = k // 32
+    blocks = ((np.arange(n * nb * 16) * 37 + 11) & 0xFF).astype(np.uint8)
+    scales = (125 + (np.arange(n * nb) % 5)).astype(np.uint8)
+    return blocks, scales
+
+
+def mxfp4_x(m, k):
+    """metal_ops.rs:6642: ((i % 13) - 6) * 0.05."""
+    i = np.arange(m * k)
+    return (((i % 13).astype(np.float32) - np.float32(6.0)) * np.float32(0.05)).reshape(m, k)

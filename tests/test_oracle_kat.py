@@ -1,0 +1,428 @@
+"""Pins the CPU oracle before anything is compared against it.
+
+Each oracle function is checked against something it was not written from:
+the reference's hand-packed known-answer tests, closed forms, IEEE casts done
+by numpy/torch, brute force on small inputs, or an independently structured
+restatement of the public ggml block formats.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from oxydllm_amd import synth
+from tests import refgen
+
+
+# ------------------------------------------------------------------ conversions
+def test_f16_conversion_matches_ieee_rne():
+    rng = np.random.default_rng(1)
+    vals = np.concatenate([
+        rng.standard_normal(20000).astype(np.float32) * np.float32(10.0),
+        rng.uniform(-7e4, 7e4, 5000).astype(np.float32),
+        (rng.standard_normal(5000) * 1e-5).astype(np.float32),
+        (rng.standard_normal(5000) * 1e-7).astype(np.float32),
+        np.array([0.0, -0.0, 65504.0, 65519.9, 65520.0, 1e9, -1e9, np.inf, -np.inf,
+                  2.0 ** -24, 2.0 ** -25, 2.0 ** -25 * 1.0001, 2.0 ** -14, 1.0009765625,
+                  1.00048828125, 1.00146484375], dtype=np.float32),
+    ])
+    got = oracle.convert_f32(vals, oracle.F16)
+    want = vals.astype(np.float16).view(np.uint16)
+    np.testing.assert_array_equal(got, want)
+    # every f16 bit pattern widens exactly
+    allbits = np.arange(65536, dtype=np.uint16)
+    wide = oracle.widen_to_f32(allbits, oracle.F16)
+    ref = allbits.view(np.float16).astype(np.float32)
+    np.testing.assert_array_equal(wide.view(np.uint32), ref.view(np.uint32))
+
+
+def test_bf16_conversion_matches_torch_rne():
+    rng = np.random.default_rng(2)
+    vals = np.concatenate([
+        rng.standard_normal(30000).astype(np.float32) * np.float32(100.0),
+        (rng.standard_normal(5000) * 1e-30).astype(np.float32),
+        np.array([0.0, -0.0, 1.00390625, 1.01171875, 3.3895314e38, np.inf, -np.inf],
+                 dtype=np.float32),
+    ])
+    got = oracle.convert_f32(vals, oracle.BF16)
+    want = torch.from_numpy(vals).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    np.testing.assert_array_equal(got, want)
+    back = oracle.widen_to_f32(got, oracle.BF16)
+    ref = torch.from_numpy(vals).to(torch.bfloat16).to(torch.float32).numpy()
+    np.testing.assert_array_equal(back.view(np.uint32), ref.view(np.uint32))
+
+
+# ------------------------------------------------------------------ AWQ / GPTQ KATs
+def test_awq_dequant_known_answer():
+    """awq.rs:954-1011 dequantize_awq_recovers_original_matrix, tol 1e-6."""
+    qw, qz, sc, expected = refgen.awq_kat_small()
+    got = oracle.dequantize_awq(qw, qz, sc)
+    assert got.shape == (16, 8)
+    assert np.max(np.abs(got - expected)) < 1e-6
+    np.testing.assert_array_equal(got, expected)  # and in fact bit-equal
+
+
+def test_awq_hand_packed_word():
+    """One word by hand: slot k of the word is column ORDER[k]."""
+    # columns 0..7 hold values 1..8 -> slots hold columns 0,2,4,6,1,3,5,7 = 1,3,5,7,2,4,6,8
+    word = 0
+    for k, v in enumerate([1, 3, 5, 7, 2, 4, 6, 8]):
+        word |= v << (4 * k)
+    qw = np.array([[word]], dtype=np.uint32)
+    qz = np.zeros((1, 1), dtype=np.uint32)
+    sc = np.ones((1, 8), dtype=np.float32)
+    got = oracle.dequantize_awq(qw, qz, sc)  # [8,1]
+    np.testing.assert_array_equal(got[:, 0], np.arange(1, 9, dtype=np.float32))
+    assert synth.pack_awq(np.arange(1, 9).reshape(1, 8)).view(np.uint32)[0, 0] == word
+
+
+def test_awq_accepts_i32_u32_i64():
+    """read_packed_to_u32 (awq.rs:158-179)."""
+    qw, qz, sc, expected = refgen.awq_kat_small()
+    for dt in (np.int32, np.uint32, np.int64):
+        a = qw.view(np.uint32).astype(dt) if dt != np.int32 else qw
+        b = qz.view(np.uint32).astype(dt) if dt != np.int32 else qz
+        np.testing.assert_array_equal(oracle.dequantize_awq(a, b, sc), expected)
+    with pytest.raises(TypeError):
+        oracle.dequantize_awq(qw.astype(np.float32), qz, sc)
+
+
+def test_awq_rejects_wrong_shapes():
+    """awq.rs:1096-1121: qweight [8,2], qzeros [2,2], scales [2,8] must be rejected."""
+    with pytest.raises(ValueError):
+        oracle.dequantize_awq(np.zeros((8, 2), np.int32), np.zeros((2, 2), np.int32),
+                              np.zeros((2, 8), np.float32))
+
+
+def test_awq_compressed_tensors_closed_form():
+    """awq.rs:754-800: signed int4 q in [-8,7] stored as q+8 with zero 8 gives q*scale."""
+    out_f, in_f, group = 16, 64, 32
+    groups = in_f // group
+    q = (np.arange(out_f * in_f) % 16 - 8).reshape(out_f, in_f)
+    scale = (np.float32(0.01) + (np.arange(out_f * groups) % 7).astype(np.float32)
+             * np.float32(0.003)).reshape(out_f, groups)
+    qweight = synth.pack_awq((q + 8).T)                       # [in, out/8]
+    qzeros = synth.pack_awq(np.full((groups, out_f), 8))
+    scales = scale.T.copy()                                   # [groups, out]
+    dq = oracle.dequantize_awq(qweight, qzeros, scales)
+    expected = q.astype(np.float32) * np.repeat(scale, group, axis=1)
+    assert np.max(np.abs(dq - expected)) < 1e-6
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_gptq_dequant_known_answer(bits):
+    """awq.rs:1170-1283, tol 1e-5."""
+    qw, qz, sc, expected = refgen.gptq_kat(bits)
+    got = oracle.dequantize_gptq(qw, qz, sc, bits)
+    assert got.shape == (16, 32)
+    assert np.max(np.abs(got - expected)) < 1e-5
+    np.testing.assert_array_equal(got, expected)
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_gptq_symmetric_zero(bits):
+    """awq.rs:567, 580-585: no qzeros -> zero+1 = 2^(bits-1)."""
+    qw, _, sc, _ = refgen.gptq_kat(bits)
+    got = oracle.dequantize_gptq(qw, None, sc, bits)
+    pf = 32 // bits
+    q = np.zeros((32, 16), dtype=np.int64)
+    w = qw.view(np.uint32)
+    for i in range(32):
+        q[i] = (w[i // pf] >> np.uint32(bits * (i % pf))) & ((1 << bits) - 1)
+    want = ((q - (1 << (bits - 1))).astype(np.float32) * np.repeat(sc, 16, axis=0)).T
+    np.testing.assert_array_equal(got, want)
+    # stored zero 2^(bits-1)-1 with explicit qzeros gives the same matrix
+    z = synth.pack_gptq_qzeros(np.full((2, 16), (1 << (bits - 1)) - 1), bits)
+    np.testing.assert_array_equal(oracle.dequantize_gptq(qw, z, sc, bits), want)
+
+
+def test_gptq_rejects_bad_bits():
+    qw, qz, sc, _ = refgen.gptq_kat(4)
+    with pytest.raises(ValueError):
+        oracle.dequantize_gptq(qw, qz, sc, 3)
+
+
+def test_awq8_matches_reference_generator():
+    """metal_ops.rs:3975-4009: ref_w built from the unpacked ints."""
+    qw, qz, sc, ref_w = refgen.build_w8a16_triplet(256, 128, 64)
+    np.testing.assert_array_equal(oracle.dequantize_awq8(qw, qz, sc), ref_w)
+
+
+@pytest.mark.parametrize("K,N,g", [(256, 128, 128), (256, 128, 64), (512, 256, 128)])
+def test_awq_bruteforce_on_reference_triplets(K, N, g):
+    """Brute force per element on the reference's GPU-test generator shapes."""
+    qw, qz, sc = refgen.build_awq_triplet(K, N, g)
+    got = oracle.dequantize_awq(qw, qz, sc)
+    i = np.arange(K)[:, None]
+    j = np.arange(N)[None, :]
+    q = (i * 5 + j * 3 + 1) & 0xF
+    z = np.repeat((np.arange(K // g)[:, None] * 7 + j + 2) & 0xF, g, axis=0)
+    want = ((q - z).astype(np.float32) * np.repeat(sc, g, axis=0)).T
+    np.testing.assert_array_equal(got, want)
+
+
+def test_transpose_convert_is_single_rounding():
+    qw, qz, sc = refgen.build_awq_triplet(256, 128, 64)
+    for dt, npdt in ((oracle.F16, np.float16),):
+        s16 = oracle.round_through(sc, dt)
+        w = oracle.dequantize_awq(qw, qz, s16)
+        kn = oracle.transpose_convert(w, dt)
+        np.testing.assert_array_equal(kn, w.T.astype(npdt).view(np.uint16))
+    s16 = oracle.round_through(sc, oracle.BF16)
+    w = oracle.dequantize_awq(qw, qz, s16)
+    kn = oracle.transpose_convert(w, oracle.BF16)
+    want = torch.from_numpy(w.T.copy()).to(torch.bfloat16).view(torch.int16).numpy()
+    np.testing.assert_array_equal(kn, want.view(np.uint16))
+
+
+# ------------------------------------------------------------------ MXFP4
+def test_mxfp4_known_values():
+    """mxfp4.rs:178-197: codes 0..15 at scale 128 (x2)."""
+    blocks = [(2 * i) | ((2 * i + 1) << 4) for i in range(8)] + [0] * 8
+    out = oracle.dequantize_mxfp4_f32(np.array(blocks, np.uint8), np.array([128], np.uint8), 1, 32)
+    exp = np.array([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0,
+                    -0.0, -0.5, -1.0, -1.5, -2.0, -3.0, -4.0, -6.0], np.float32) * 2
+    np.testing.assert_array_equal(out[0, :16], exp)
+    assert np.signbit(out[0, 8])
+    assert np.all(out[0, 16:] == 0.0)
+
+
+def test_mxfp4_linear_manual_dot():
+    """mxfp4.rs:199-214: two rows both dot to 32 with all-ones x."""
+    blocks = np.array([0x22] * 16 + [0x44] * 16, np.uint8)
+    scales = np.array([127, 126], np.uint8)
+    w = oracle.dequantize_mxfp4_f32(blocks, scales, 2, 32)
+    y = oracle.matmul_nt_f32(np.ones((1, 32), np.float32), w)
+    np.testing.assert_array_equal(y, np.array([[32.0, 32.0]], np.float32))
+
+
+def test_mxfp4_nan_scale_and_size_check():
+    out = oracle.dequantize_mxfp4_f32(np.zeros(16, np.uint8), np.array([255], np.uint8), 1, 32)
+    assert np.all(np.isnan(out))
+    with pytest.raises(ValueError):
+        oracle.dequantize_mxfp4_f32(np.zeros(15, np.uint8), np.array([127], np.uint8), 1, 32)
+    with pytest.raises(ValueError):
+        oracle.dequantize_mxfp4_f32(np.zeros(16, np.uint8), np.array([127], np.uint8), 1, 33)
+
+
+def test_mxfp4_e8m0_is_exact_power_of_two():
+    for s in (0, 1, 100, 118, 126, 127, 128, 200, 254):
+        out = oracle.dequantize_mxfp4_f32(np.full(16, 0x22, np.uint8), np.array([s], np.uint8), 1, 32)
+        assert out[0, 0] == np.float32(2.0) ** np.float32(s - 127)
+
+
+# ------------------------------------------------------------------ GGUF
+def _ggml_q4_0(blk):
+    d = blk[0:2].view(np.float16).astype(np.float32)[0]
+    qs = blk[2:18].astype(np.int32)
+    y = np.empty(32, np.float32)
+    for j in range(16):  # ggml dequantize_row_q4_0: y[j] low nibble, y[j+16] high nibble
+        y[j] = np.float32((qs[j] & 0xF) - 8) * d
+        y[j + 16] = np.float32((qs[j] >> 4) - 8) * d
+    return y
+
+
+def _ggml_q8_0(blk):
+    d = blk[0:2].view(np.float16).astype(np.float32)[0]
+    return blk[2:34].view(np.int8).astype(np.float32) * d
+
+
+def _k4(j, q):
+    if j < 4:
+        return q[j] & 63, q[j + 4] & 63
+    return (q[j + 4] & 0xF) | ((q[j - 4] >> 6) << 4), (q[j + 4] >> 4) | ((q[j] >> 6) << 4)
+
+
+def _ggml_q4_k(blk):
+    d = blk[0:2].view(np.float16).astype(np.float32)[0]
+    dmin = blk[2:4].view(np.float16).astype(np.float32)[0]
+    sc = blk[4:16].astype(np.int32)
+    q = blk[16:144].astype(np.int32)
+    y = []
+    is_ = 0
+    for j in range(0, 256, 64):  # ggml dequantize_row_q4_K walks 64 elements per 32 bytes
+        s1, m1 = _k4(is_, sc)
+        s2, m2 = _k4(is_ + 1, sc)
+        d1, mm1 = d * np.float32(s1), dmin * np.float32(m1)
+        d2, mm2 = d * np.float32(s2), dmin * np.float32(m2)
+        qq = q[(j // 64) * 32:(j // 64) * 32 + 32]
+        y.extend(d1 * (qq & 0xF).astype(np.float32) - mm1)
+        y.extend(d2 * (qq >> 4).astype(np.float32) - mm2)
+        is_ += 2
+    return np.array(y, np.float32)
+
+
+def _ggml_q6_k(blk):
+    ql = blk[0:128].astype(np.int32)
+    qh = blk[128:192].astype(np.int32)
+    sc = blk[192:208].view(np.int8).astype(np.int32)
+    d = blk[208:210].view(np.float16).astype(np.float32)[0]
+    y = np.empty(256, np.float32)
+    for n in range(0, 256, 128):  # ggml dequantize_row_q6_K
+        h = n // 128
+        qlh, qhh, sch = ql[64 * h:], qh[32 * h:], sc[8 * h:]
+        for l in range(32):
+            is_ = l // 16
+            q1 = ((qlh[l] & 0xF) | (((qhh[l] >> 0) & 3) << 4)) - 32
+            q2 = ((qlh[l + 32] & 0xF) | (((qhh[l] >> 2) & 3) << 4)) - 32
+            q3 = ((qlh[l] >> 4) | (((qhh[l] >> 4) & 3) << 4)) - 32
+            q4 = ((qlh[l + 32] >> 4) | (((qhh[l] >> 6) & 3) << 4)) - 32
+            y[n + l] = d * np.float32(sch[is_]) * np.float32(q1)
+            y[n + l + 32] = d * np.float32(sch[is_ + 2]) * np.float32(q2)
+            y[n + l + 64] = d * np.float32(sch[is_ + 4]) * np.float32(q3)
+            y[n + l + 96] = d * np.float32(sch[is_ + 6]) * np.float32(q4)
+    return y
+
+
+_GGML = {synth.GGUF_Q4_0: _ggml_q4_0, synth.GGUF_Q8_0: _ggml_q8_0,
+         synth.GGUF_Q4_K: _ggml_q4_k, synth.GGUF_Q6_K: _ggml_q6_k}
+
+
+@pytest.mark.parametrize("fmt", [synth.GGUF_Q4_0, synth.GGUF_Q8_0, synth.GGUF_Q4_K, synth.GGUF_Q6_K])
+def test_gguf_dequant_matches_ggml_row_loops(fmt):
+    """Block formats per the public ggml spec, walked the way ggml's own
+    dequantize_row_* loops walk them (not the per-element index formula)."""
+    elems, bbytes = synth.GGUF_BLOCK_LAYOUT[fmt]
+    N, K = 3, 2 * elems
+    data = synth.gguf_weight(fmt, N, K, seed=11 + fmt)
+    got = oracle.dequantize_gguf(fmt, data, N, K)
+    blocks = data.reshape(N * 2, bbytes)
+    want = np.stack([_GGML[fmt](b) for b in blocks]).reshape(N, K)
+    np.testing.assert_array_equal(got, want)
+
+
+def test_gguf_closed_forms():
+    # Q4_0 all-zero quants -> -8 d ; Q8_0 quant 1 -> d
+    d = np.array([0.0123], np.float16)
+    blk = np.zeros(18, np.uint8)
+    blk[0:2] = d.view(np.uint8)
+    out = oracle.dequantize_gguf(oracle.Q4_0, blk, 1, 32)
+    np.testing.assert_array_equal(out, np.full((1, 32), np.float32(-8) * d.astype(np.float32)[0]))
+    blk = np.ones(34, np.uint8)
+    blk[0:2] = d.view(np.uint8)
+    out = oracle.dequantize_gguf(oracle.Q8_0, blk, 1, 32)
+    np.testing.assert_array_equal(out, np.full((1, 32), d.astype(np.float32)[0]))
+    # Q6_K all-zero ql/qh -> -32 * d * scale[sub-block]
+    blk = np.zeros(210, np.uint8)
+    blk[192:208] = np.arange(1, 17, dtype=np.uint8)
+    blk[208:210] = d.view(np.uint8)
+    out = oracle.dequantize_gguf(oracle.Q6_K, blk, 1, 256)[0]
+    for j in range(256):
+        sub = j // 16
+        assert out[j] == d.astype(np.float32)[0] * np.float32(sub + 1) * np.float32(-32)
+    # Q4_K: scales bytes give sc=j+1 (j<4), min=0 -> w = d*sc*nib
+    blk = np.zeros(144, np.uint8)
+    blk[0:2] = d.view(np.uint8)
+    blk[2:4] = d.view(np.uint8)
+    blk[4:8] = [1, 2, 3, 4]
+    blk[16:144] = 0x21  # low nibble 1, high nibble 2
+    out = oracle.dequantize_gguf(oracle.Q4_K, blk, 1, 256)[0]
+    df = d.astype(np.float32)[0]
+    assert np.all(out[0:32] == df * 1 * 1) and np.all(out[32:64] == df * 2 * 2)
+    assert np.all(out[64:96] == df * 3 * 1) and np.all(out[96:128] == df * 4 * 2)
+    assert np.all(out[128:] == 0)
+
+
+def test_gguf_size_checks():
+    with pytest.raises(ValueError):
+        oracle.dequantize_gguf(oracle.Q4_0, np.zeros(17, np.uint8), 1, 32)
+    with pytest.raises(ValueError):
+        oracle.dequantize_gguf(oracle.Q4_K, np.zeros(144, np.uint8), 1, 128)
+
+
+# ------------------------------------------------------------------ matmul / MoE
+def test_matmul_against_numpy_float64():
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((5, 300)).astype(np.float32)
+    w = rng.standard_normal((17, 300)).astype(np.float32)
+    b = rng.standard_normal(17).astype(np.float32)
+    want = x.astype(np.float64) @ w.astype(np.float64).T + b
+    np.testing.assert_allclose(oracle.matmul_nt_f32(x, w, b), want, rtol=1e-5, atol=1e-4)
+    np.testing.assert_array_equal(oracle.matmul_nt_f64acc(x, w, b), want.astype(np.float32))
+    # transposed-operand mistake would fail this non-square case
+    assert oracle.matmul_nt_f32(x, w).shape == (5, 17)
+
+
+def test_linear_from_awq_matches_dense():
+    """linear.rs:688-787 shape: K=4, N=8, g=2, bias; y = x.W^T + b from the dequantized W."""
+    K, N, g = 4, 8, 2
+    rng = np.random.default_rng(3)
+    q = rng.integers(0, 16, (K, N))
+    z = rng.integers(0, 16, (K // g, N))
+    s = rng.uniform(0.01, 0.1, (K // g, N)).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    x = rng.standard_normal((3, K)).astype(np.float32)
+    w = oracle.dequantize_awq(synth.pack_awq(q), synth.pack_awq(z), s)
+    dense = ((q - np.repeat(z, g, 0)).astype(np.float32) * np.repeat(s, g, 0)).T
+    want = x.astype(np.float64) @ dense.astype(np.float64).T + bias
+    np.testing.assert_allclose(oracle.matmul_nt_f32(x, w, bias), want, rtol=1e-5, atol=1e-5)
+
+
+def test_moe_route_matches_numpy():
+    rng = np.random.default_rng(7)
+    logits = rng.standard_normal((8, 32)).astype(np.float32)
+    idx, vals = oracle.moe_route(logits, 4, True)
+    p = np.exp(logits - logits.max(1, keepdims=True))
+    p /= p.sum(1, keepdims=True)
+    order = np.argsort(-p, axis=1, kind="stable")[:, :4]
+    np.testing.assert_array_equal(idx, order.astype(np.uint32))
+    tv = np.take_along_axis(p, order, 1)
+    np.testing.assert_allclose(vals, tv / tv.sum(1, keepdims=True), rtol=1e-5)
+    np.testing.assert_allclose(vals.sum(1), 1.0, rtol=1e-5)
+    _, raw = oracle.moe_route(logits, 4, False)
+    np.testing.assert_allclose(raw, tv, rtol=1e-5)
+    offsets, tokens, weights = oracle.moe_group(idx, vals, 32)
+    assert offsets[-1] == 32 and offsets[0] == 0
+    for e in range(32):
+        toks = tokens[offsets[e]:offsets[e + 1]]
+        want = [t for t in range(8) if e in idx[t]]
+        assert list(toks) == want  # token-major order, like dispatch_sparse
+        for t, w_ in zip(toks, weights[offsets[e]:offsets[e + 1]]):
+            assert w_ == vals[t, list(idx[t]).index(e)]
+
+
+def test_gpt_oss_expert_scalar_reference():
+    """moe.rs:705-788 gpt_oss_expert_matches_scalar_reference (tol 1e-3*max + 1e-3)."""
+    hidden = inter = 32
+    limit = np.float32(7.0)
+    gu_out, nb = 2 * inter, 1
+    gu_blocks = ((np.arange(gu_out * nb * 16) * 23 + 7) & 0xFF).astype(np.uint8)
+    gu_scales = (125 + np.arange(gu_out * nb) % 5).astype(np.uint8)
+    dn_blocks = ((np.arange(hidden * nb * 16) * 41 + 3) & 0xFF).astype(np.uint8)
+    dn_scales = (126 + np.arange(hidden * nb) % 3).astype(np.uint8)
+    gu_bias = (np.sin(np.arange(gu_out, dtype=np.float32) * np.float32(0.7)) * 2).astype(np.float32)
+    dn_bias = (np.cos(np.arange(hidden, dtype=np.float32) * np.float32(0.3)) * 0.5).astype(np.float32)
+    x = (np.sin(np.arange(hidden, dtype=np.float32) * np.float32(0.21)) * 3).astype(np.float32)
+
+    # oracle path: dequant + matmul + swiglu + matmul
+    w_gu = oracle.dequantize_mxfp4_f32(gu_blocks, gu_scales, gu_out, hidden)
+    w_dn = oracle.dequantize_mxfp4_f32(dn_blocks, dn_scales, hidden, inter)
+    gu = oracle.matmul_nt_f32(x[None, :], w_gu, gu_bias)
+    h = oracle.gpt_oss_swiglu(gu, float(limit))
+    y = oracle.matmul_nt_f32(h, w_dn, dn_bias)[0]
+
+    # independent scalar reference written from the MX spec tables
+    lut = [0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0]
+
+    def deq(blocks, scales, rows, cols):
+        w = np.zeros((rows, cols))
+        for r in range(rows):
+            for b in range(cols // 32):
+                sc = 2.0 ** (int(scales[r * (cols // 32) + b]) - 127)
+                for i in range(16):
+                    byte = int(blocks[(r * (cols // 32) + b) * 16 + i])
+                    for half, code in enumerate((byte & 0xF, byte >> 4)):
+                        v = lut[code & 7] * (-1 if code & 8 else 1)
+                        w[r, b * 32 + 2 * i + half] = v * sc
+        return w
+
+    wg, wd = deq(gu_blocks, gu_scales, gu_out, hidden), deq(dn_blocks, dn_scales, hidden, inter)
+    gate_up = gu_bias + wg @ x
+    hh = np.zeros(inter)
+    for k in range(inter):
+        gate = min(gate_up[2 * k], 7.0)
+        up = min(max(gate_up[2 * k + 1], -7.0), 7.0)
+        hh[k] = (up + 1.0) * gate * (1.0 / (1.0 + np.exp(-gate * 1.702)))
+    expected = dn_bias + wd @ hh
+    tol = 1e-3 * np.max(np.abs(expected)) + 1e-3
+    assert np.max(np.abs(y - expected)) < tol
