@@ -1,0 +1,250 @@
+/*
+ * oxq.h - C ABI of the MI355X (gfx950) quantized-weight matmul library.
+ *
+ * The library replaces, one for one, the op functions oxydLLM's linear layers
+ * call for packed-quantized weights (reference: src/common/metal_ops.rs) and
+ * the three layer types that route to them (src/common/linear.rs,
+ * src/common/mxfp4.rs).  Each declaration cites the reference interface it
+ * stands in for.
+ *
+ * Conventions
+ *  - Every tensor argument is an `oxq_tensor` descriptor: a device pointer to
+ *    element 0 (any storage offset already applied), element type, rank and
+ *    dims.  The library never owns, frees or reallocates caller memory.
+ *  - Outputs are caller-allocated (the reference ops allocate their result;
+ *    a C ABI cannot return a framework tensor).  Shapes are checked.
+ *  - All validation runs on the host before anything is enqueued and mirrors
+ *    the reference's `bail!` conditions; a failed call enqueues nothing.
+ *  - Calls return 0 on success or a negative `oxq_status`; the message of the
+ *    last failure on the calling thread is available from oxq_last_error().
+ *  - Work is enqueued asynchronously on `stream` (a hipStream_t, NULL = the
+ *    default stream).  No call synchronizes the device.
+ *  - One `oxq_ctx` per engine thread / stream: the ctx owns a split-K
+ *    workspace that concurrent calls on the same ctx would race on.
+ *  - A ctx created with device = OXQ_DEVICE_PLAN_ONLY validates arguments and
+ *    computes the launch plan but launches nothing; it needs no GPU.
+ */
+#ifndef OXQ_H
+#define OXQ_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define OXQ_VERSION_MAJOR 0
+#define OXQ_VERSION_MINOR 1
+
+#define OXQ_DEVICE_HOST (-1)      /* oxq_tensor.device: host memory (always rejected by ops) */
+#define OXQ_DEVICE_PLAN_ONLY (-1) /* oxq_ctx_create: validate + plan, never launch */
+
+typedef enum oxq_status {
+    OXQ_OK = 0,
+    OXQ_ERR_ARG = -1,        /* NULL pointer / bad enum */
+    OXQ_ERR_DTYPE = -2,      /* element type not accepted by the op */
+    OXQ_ERR_SHAPE = -3,      /* rank / dims / byte-count mismatch */
+    OXQ_ERR_CONTIGUOUS = -4, /* x (or qweight) must be contiguous */
+    OXQ_ERR_M_RANGE = -5,    /* m outside the op's decode range [1, 8] */
+    OXQ_ERR_GROUP = -6,      /* group size not a power of two / not dividing K */
+    OXQ_ERR_DEVICE = -7,     /* tensor not resident on the ctx device */
+    OXQ_ERR_BITS = -8,       /* bits not in {4, 8} */
+    OXQ_ERR_RUNTIME = -9,    /* HIP runtime failure */
+    OXQ_ERR_WORKSPACE = -10, /* problem needs more split-K workspace than the ctx holds */
+    OXQ_ERR_UNSUPPORTED = -11
+} oxq_status;
+
+typedef enum oxq_dtype {
+    OXQ_F32 = 0,
+    OXQ_F16 = 1,
+    OXQ_BF16 = 2,
+    OXQ_U8 = 3,
+    OXQ_I32 = 4,
+    OXQ_U32 = 5,
+    OXQ_I64 = 6
+} oxq_dtype;
+
+/* reference: awq.rs:27-31 (PackDim).  OUT = AWQ layout, IN = GPTQ layout. */
+typedef enum oxq_pack_dim { OXQ_PACK_OUT = 0, OXQ_PACK_IN = 1 } oxq_pack_dim;
+
+/* reference: metal_ops.rs:5211-5223 (GgufFastQuant); the four formats built here. */
+typedef enum oxq_gguf_quant {
+    OXQ_GGUF_Q4_0 = 0,
+    OXQ_GGUF_Q8_0 = 1,
+    OXQ_GGUF_Q4_K = 2,
+    OXQ_GGUF_Q6_K = 3
+} oxq_gguf_quant;
+
+#define OXQ_MAX_RANK 4
+
+typedef struct oxq_tensor {
+    void *data;                 /* device pointer to element 0 */
+    int32_t dtype;              /* oxq_dtype */
+    int32_t rank;               /* 1..OXQ_MAX_RANK */
+    int64_t dims[OXQ_MAX_RANK]; /* row-major */
+    int32_t contiguous;         /* non-zero when densely packed row-major */
+    int32_t device;             /* HIP device ordinal, OXQ_DEVICE_HOST for host memory */
+} oxq_tensor;
+
+/* What the last successful call on a ctx launched (or would launch). */
+typedef struct oxq_plan {
+    char kernel[64];
+    uint32_t grid[3];
+    uint32_t block[3];
+    uint32_t split_k;         /* number of K slices combined in fixed order */
+    uint32_t launches;        /* kernel launches the call enqueued */
+    uint64_t workspace_bytes; /* split-K partials used */
+} oxq_plan;
+
+typedef struct oxq_ctx oxq_ctx;
+
+/* ---- context -------------------------------------------------------------
+ * No counterpart in the reference (candle owns its Metal device/encoder,
+ * metal_ops.rs:1367-1403); holds the device ordinal and split-K workspace. */
+int oxq_ctx_create(int device, oxq_ctx **out);
+int oxq_ctx_destroy(oxq_ctx *ctx);
+int oxq_ctx_device(const oxq_ctx *ctx);
+int oxq_ctx_last_plan(const oxq_ctx *ctx, oxq_plan *out);
+const char *oxq_last_error(void);
+const char *oxq_status_name(int status);
+void oxq_version(int *major, int *minor);
+
+/* Block layout of a GGUF format: metal_ops.rs:5228-5241 (block_layout). */
+int oxq_gguf_block_layout(int quant, int64_t *block_elems, int64_t *block_bytes);
+
+/* ---- decode GEMV ops (1 <= m <= 8) ---------------------------------------
+ * y[m,N] = x[m,K] . dequant(W), f32 accumulate, result in x's dtype.
+ * x, scales: F16 or BF16 (same type); qweight/qzeros: I32 or U32. */
+
+/* metal_ops.rs:1821 w4a16_matmul(x, qweight, qzeros, scales)
+ * qweight [K, N/8] AWQ-interleaved, qzeros [K/g, N/8], scales [K/g, N]. */
+int oxq_w4a16_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x, const oxq_tensor *qweight,
+                     const oxq_tensor *qzeros, const oxq_tensor *scales, const oxq_tensor *out);
+
+/* metal_ops.rs:1835 w8a16_matmul: qweight [K, N/4] identity slot order. */
+int oxq_w8a16_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x, const oxq_tensor *qweight,
+                     const oxq_tensor *qzeros, const oxq_tensor *scales, const oxq_tensor *out);
+
+/* metal_ops.rs:2281 gptq_matmul(x, qweight, qzeros, scales, bits)
+ * qweight [K/pf, N] sequential along K, qzeros [K/g, N/pf] (stored zero-1). */
+int oxq_gptq_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x, const oxq_tensor *qweight,
+                    const oxq_tensor *qzeros, const oxq_tensor *scales, uint32_t bits,
+                    const oxq_tensor *out);
+
+/* ---- dense dequant ops: out [K, N] in the scales' dtype ------------------ */
+
+/* metal_ops.rs:1873 dequantize_w4 */
+int oxq_dequantize_w4(oxq_ctx *ctx, void *stream, const oxq_tensor *qweight,
+                      const oxq_tensor *qzeros, const oxq_tensor *scales, const oxq_tensor *out);
+/* metal_ops.rs:1886 dequantize_w8 */
+int oxq_dequantize_w8(oxq_ctx *ctx, void *stream, const oxq_tensor *qweight,
+                      const oxq_tensor *qzeros, const oxq_tensor *scales, const oxq_tensor *out);
+/* metal_ops.rs:2305 dequantize_gptq_packed(qweight, qzeros, scales, bits) */
+int oxq_dequantize_gptq_packed(oxq_ctx *ctx, void *stream, const oxq_tensor *qweight,
+                               const oxq_tensor *qzeros, const oxq_tensor *scales, uint32_t bits,
+                               const oxq_tensor *out);
+
+/* ---- batched tile GEMM (matrix cores) ------------------------------------
+ * metal_ops.rs:2748 mpp_quant_matmul / 2771 maybe_mpp_quant_matmul
+ * y[m,N] = x[m,K] . dequant(W) on MFMA tiles, any m >= 1, F16 or BF16.
+ * The `maybe_` form declines (returns OXQ_OK with *taken = 0, nothing
+ * enqueued) when m < OXQ_MFMA_MIN_M or x is not contiguous, as the reference
+ * declines below MPP_GEMM_MIN_M (metal_ops.rs:2326). */
+#define OXQ_MFMA_MIN_M 9
+int oxq_mpp_quant_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x,
+                         const oxq_tensor *qweight, const oxq_tensor *qzeros,
+                         const oxq_tensor *scales, uint32_t bits, int pack_dim,
+                         const oxq_tensor *out);
+int oxq_maybe_mpp_quant_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x,
+                               const oxq_tensor *qweight, const oxq_tensor *qzeros,
+                               const oxq_tensor *scales, uint32_t bits, int pack_dim,
+                               const oxq_tensor *out, int *taken);
+
+/* ---- GGUF block-quant ops -------------------------------------------------
+ * weight_bytes: U8 [N * K/block_elems * block_bytes], row n = consecutive
+ * ggml blocks.  x and out: BF16 (the reference's contract) or F32 (the
+ * benchmark's f32-activation configuration); x and out share a dtype. */
+
+/* metal_ops.rs:5819 gguf_quant_matmul: 1 <= m <= 8 */
+int oxq_gguf_quant_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x,
+                          const oxq_tensor *weight_bytes, int64_t in_features,
+                          int64_t out_features, int quant, const oxq_tensor *out);
+/* metal_ops.rs:5973 gguf_quant_mul_mm: any m */
+int oxq_gguf_quant_mul_mm(oxq_ctx *ctx, void *stream, const oxq_tensor *x,
+                          const oxq_tensor *weight_bytes, int64_t in_features,
+                          int64_t out_features, int quant, const oxq_tensor *out);
+/* Dense dequant [N, K] f32 of a GGUF weight (no reference op: the reference
+ * tests compare against candle's QTensor::dequantize, metal_ops.rs:6405-6417;
+ * this exposes the kernels' own decode so it can be checked bit for bit). */
+int oxq_gguf_dequantize(oxq_ctx *ctx, void *stream, const oxq_tensor *weight_bytes,
+                        int64_t in_features, int64_t out_features, int quant,
+                        const oxq_tensor *out);
+
+/* ---- MXFP4 ----------------------------------------------------------------
+ * metal_ops.rs:6197 mxfp4_matmul(x, blocks, scales, k, n): x/out BF16,
+ * blocks U8 [n*k/32*16], scales U8 [n*k/32], any m >= 1 (gemv kernel for
+ * m <= 8, tiled beyond, metal_ops.rs:6204-6222). */
+int oxq_mxfp4_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x, const oxq_tensor *blocks,
+                     const oxq_tensor *scales, int64_t k, int64_t n, const oxq_tensor *out);
+/* Dense dequant [n, k] f32 (device twin of mxfp4.rs:35 dequantize_mxfp4_f32). */
+int oxq_mxfp4_dequantize(oxq_ctx *ctx, void *stream, const oxq_tensor *blocks,
+                         const oxq_tensor *scales, int64_t k, int64_t n, const oxq_tensor *out);
+
+/* Grouped expert GEMV: every active expert of one MoE projection in a single
+ * launch.  Stands in for the per-expert loop of moe.rs:593-605 over
+ * Mxfp4Linear::forward (mxfp4.rs:119-154).
+ *  x           BF16 [n_tokens, k]           (gather_rows != 0) or
+ *              BF16 [n_pairs, k]            (gather_rows == 0: row i is pair i)
+ *  blocks      U8 [n_experts, n, k/32, 16]; scales U8 [n_experts, n, k/32]
+ *  bias        BF16 [n_experts, n] or NULL
+ *  expert_offsets I32 [n_experts + 1]: pairs of expert e are
+ *              [offsets[e], offsets[e+1]) in token_ids / out rows
+ *  token_ids   I32 [n_pairs]: source row of x for each pair (gather_rows != 0)
+ *  out         BF16 [n_pairs, n]: out[p] = x[row(p)] . W_e^T + bias_e */
+int oxq_mxfp4_moe_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x,
+                         const oxq_tensor *blocks, const oxq_tensor *scales,
+                         const oxq_tensor *bias, const oxq_tensor *expert_offsets,
+                         const oxq_tensor *token_ids, int gather_rows, int64_t k, int64_t n,
+                         const oxq_tensor *out);
+
+/* ---- layers ----------------------------------------------------------------
+ * Host-side mirrors of the reference layer types; they hold descriptors of
+ * caller-owned resident weights and route by m exactly where the reference
+ * routes.  `x` may have any leading dims; m is their product. */
+
+/* linear.rs:403-534 PackedQuantLinear::{new, forward}.  scales must already be
+ * in the runtime dtype (`dtype`), as after the cast at linear.rs:437. */
+typedef struct oxq_packed_quant_linear oxq_packed_quant_linear;
+int oxq_packed_quant_linear_new(oxq_ctx *ctx, uint32_t bits, int pack_dim,
+                                const oxq_tensor *qweight, const oxq_tensor *qzeros,
+                                const oxq_tensor *scales, const oxq_tensor *bias_or_null,
+                                int dtype, oxq_packed_quant_linear **out);
+int oxq_packed_quant_linear_forward(oxq_packed_quant_linear *layer, void *stream,
+                                    const oxq_tensor *x, const oxq_tensor *out);
+int oxq_packed_quant_linear_in_features(const oxq_packed_quant_linear *layer, int64_t *k);
+int oxq_packed_quant_linear_out_features(const oxq_packed_quant_linear *layer, int64_t *n);
+void oxq_packed_quant_linear_free(oxq_packed_quant_linear *layer);
+
+/* linear.rs:179-393 QLinear / GgufFastPath::{build, forward_decode, forward_prefill}. */
+typedef struct oxq_qlinear oxq_qlinear;
+int oxq_qlinear_new(oxq_ctx *ctx, int quant, const oxq_tensor *weight_bytes, int64_t in_features,
+                    int64_t out_features, const oxq_tensor *bias_or_null, int out_dtype,
+                    oxq_qlinear **out);
+int oxq_qlinear_forward(oxq_qlinear *layer, void *stream, const oxq_tensor *x,
+                        const oxq_tensor *out);
+void oxq_qlinear_free(oxq_qlinear *layer);
+
+/* mxfp4.rs:67-169 Mxfp4Linear::{new, forward}. */
+typedef struct oxq_mxfp4_linear oxq_mxfp4_linear;
+int oxq_mxfp4_linear_new(oxq_ctx *ctx, const oxq_tensor *blocks, const oxq_tensor *scales,
+                         const oxq_tensor *bias_or_null, int64_t in_features,
+                         int64_t out_features, oxq_mxfp4_linear **out);
+int oxq_mxfp4_linear_forward(oxq_mxfp4_linear *layer, void *stream, const oxq_tensor *x,
+                             const oxq_tensor *out);
+void oxq_mxfp4_linear_free(oxq_mxfp4_linear *layer);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* OXQ_H */

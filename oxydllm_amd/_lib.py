@@ -1,0 +1,114 @@
+"""ctypes loader for ``liboxq_hip.so`` (the C ABI declared in ``include/oxq.h``).
+
+There is no fallback: if the library is missing the import of any op fails with
+an error that says how to build it.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "liboxq_hip.so")
+
+OXQ_MAX_RANK = 4
+(F32, F16, BF16, U8, I32, U32, I64) = range(7)
+PACK_OUT, PACK_IN = 0, 1
+GGUF_Q4_0, GGUF_Q8_0, GGUF_Q4_K, GGUF_Q6_K = range(4)
+DEVICE_HOST = -1
+DEVICE_PLAN_ONLY = -1
+MFMA_MIN_M = 9
+
+STATUS = {
+    0: "OXQ_OK", -1: "OXQ_ERR_ARG", -2: "OXQ_ERR_DTYPE", -3: "OXQ_ERR_SHAPE",
+    -4: "OXQ_ERR_CONTIGUOUS", -5: "OXQ_ERR_M_RANGE", -6: "OXQ_ERR_GROUP", -7: "OXQ_ERR_DEVICE",
+    -8: "OXQ_ERR_BITS", -9: "OXQ_ERR_RUNTIME", -10: "OXQ_ERR_WORKSPACE", -11: "OXQ_ERR_UNSUPPORTED",
+}
+
+
+class OxqTensor(C.Structure):
+    _fields_ = [("data", C.c_void_p), ("dtype", C.c_int32), ("rank", C.c_int32),
+                ("dims", C.c_int64 * OXQ_MAX_RANK), ("contiguous", C.c_int32),
+                ("device", C.c_int32)]
+
+
+class OxqPlan(C.Structure):
+    _fields_ = [("kernel", C.c_char * 64), ("grid", C.c_uint32 * 3), ("block", C.c_uint32 * 3),
+                ("split_k", C.c_uint32), ("launches", C.c_uint32),
+                ("workspace_bytes", C.c_uint64)]
+
+
+class OxqError(RuntimeError):
+    def __init__(self, status: int, message: str):
+        super().__init__(f"{STATUS.get(status, status)}: {message}")
+        self.status = status
+        self.message = message
+
+
+# Every symbol include/oxq.h declares, with its argument types.
+_TP = C.POINTER(OxqTensor)
+_VP = C.c_void_p
+SIGNATURES = {
+    "oxq_ctx_create": (C.c_int, [C.c_int, C.POINTER(_VP)]),
+    "oxq_ctx_destroy": (C.c_int, [_VP]),
+    "oxq_ctx_device": (C.c_int, [_VP]),
+    "oxq_ctx_last_plan": (C.c_int, [_VP, C.POINTER(OxqPlan)]),
+    "oxq_last_error": (C.c_char_p, []),
+    "oxq_status_name": (C.c_char_p, [C.c_int]),
+    "oxq_version": (None, [C.POINTER(C.c_int), C.POINTER(C.c_int)]),
+    "oxq_gguf_block_layout": (C.c_int, [C.c_int, C.POINTER(C.c_int64), C.POINTER(C.c_int64)]),
+    "oxq_w4a16_matmul": (C.c_int, [_VP, _VP, _TP, _TP, _TP, _TP, _TP]),
+    "oxq_w8a16_matmul": (C.c_int, [_VP, _VP, _TP, _TP, _TP, _TP, _TP]),
+    "oxq_gptq_matmul": (C.c_int, [_VP, _VP, _TP, _TP, _TP, _TP, C.c_uint32, _TP]),
+    "oxq_dequantize_w4": (C.c_int, [_VP, _VP, _TP, _TP, _TP, _TP]),
+    "oxq_dequantize_w8": (C.c_int, [_VP, _VP, _TP, _TP, _TP, _TP]),
+    "oxq_dequantize_gptq_packed": (C.c_int, [_VP, _VP, _TP, _TP, _TP, C.c_uint32, _TP]),
+    "oxq_mpp_quant_matmul": (C.c_int, [_VP, _VP, _TP, _TP, _TP, _TP, C.c_uint32, C.c_int, _TP]),
+    "oxq_maybe_mpp_quant_matmul": (C.c_int, [_VP, _VP, _TP, _TP, _TP, _TP, C.c_uint32, C.c_int,
+                                             _TP, C.POINTER(C.c_int)]),
+    "oxq_gguf_quant_matmul": (C.c_int, [_VP, _VP, _TP, _TP, C.c_int64, C.c_int64, C.c_int, _TP]),
+    "oxq_gguf_quant_mul_mm": (C.c_int, [_VP, _VP, _TP, _TP, C.c_int64, C.c_int64, C.c_int, _TP]),
+    "oxq_gguf_dequantize": (C.c_int, [_VP, _VP, _TP, C.c_int64, C.c_int64, C.c_int, _TP]),
+    "oxq_mxfp4_matmul": (C.c_int, [_VP, _VP, _TP, _TP, _TP, C.c_int64, C.c_int64, _TP]),
+    "oxq_mxfp4_dequantize": (C.c_int, [_VP, _VP, _TP, _TP, C.c_int64, C.c_int64, _TP]),
+    "oxq_mxfp4_moe_matmul": (C.c_int, [_VP, _VP, _TP, _TP, _TP, _TP, _TP, _TP, C.c_int,
+                                       C.c_int64, C.c_int64, _TP]),
+    "oxq_packed_quant_linear_new": (C.c_int, [_VP, C.c_uint32, C.c_int, _TP, _TP, _TP, _TP,
+                                              C.c_int, C.POINTER(_VP)]),
+    "oxq_packed_quant_linear_forward": (C.c_int, [_VP, _VP, _TP, _TP]),
+    "oxq_packed_quant_linear_in_features": (C.c_int, [_VP, C.POINTER(C.c_int64)]),
+    "oxq_packed_quant_linear_out_features": (C.c_int, [_VP, C.POINTER(C.c_int64)]),
+    "oxq_packed_quant_linear_free": (None, [_VP]),
+    "oxq_qlinear_new": (C.c_int, [_VP, C.c_int, _TP, C.c_int64, C.c_int64, _TP, C.c_int,
+                                  C.POINTER(_VP)]),
+    "oxq_qlinear_forward": (C.c_int, [_VP, _VP, _TP, _TP]),
+    "oxq_qlinear_free": (None, [_VP]),
+    "oxq_mxfp4_linear_new": (C.c_int, [_VP, _TP, _TP, _TP, C.c_int64, C.c_int64, C.POINTER(_VP)]),
+    "oxq_mxfp4_linear_forward": (C.c_int, [_VP, _VP, _TP, _TP]),
+    "oxq_mxfp4_linear_free": (None, [_VP]),
+}
+
+_lib = None
+
+
+def load() -> C.CDLL:
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `python -m oxydllm_amd.build` "
+            "(hipcc --offload-arch=gfx950); there is no CPU fallback")
+    lib = C.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError if the library does not export it
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def check(rc: int):
+    if rc != 0:
+        msg = load().oxq_last_error()
+        raise OxqError(rc, msg.decode() if msg else "")

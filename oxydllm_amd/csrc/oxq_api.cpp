@@ -1,0 +1,914 @@
+// Host side of the C ABI: context, argument validation (device-free, mirrors
+// the reference's checks in src/common/metal_ops.rs before every dispatch) and
+// routing to the kernel launchers.
+
+#include "oxq_internal.hpp"
+
+#include <cstdlib>
+#include <new>
+
+namespace oxq {
+
+static thread_local char g_last_error[512] = "";
+
+int fail(int status, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_last_error, sizeof g_last_error, fmt, ap);
+    va_end(ap);
+    return status;
+}
+
+const char *dtype_name(int dtype) {
+    switch (dtype) {
+    case OXQ_F32: return "F32";
+    case OXQ_F16: return "F16";
+    case OXQ_BF16: return "BF16";
+    case OXQ_U8: return "U8";
+    case OXQ_I32: return "I32";
+    case OXQ_U32: return "U32";
+    case OXQ_I64: return "I64";
+    default: return "?";
+    }
+}
+
+void set_plan(oxq_ctx *ctx, const char *kernel, dim3 grid, dim3 block, uint32_t split_k,
+              uint32_t launches, uint64_t ws_bytes) {
+    oxq_plan &pl = ctx->plan;
+    memset(&pl, 0, sizeof pl);
+    snprintf(pl.kernel, sizeof pl.kernel, "%s", kernel);
+    pl.grid[0] = grid.x; pl.grid[1] = grid.y; pl.grid[2] = grid.z;
+    pl.block[0] = block.x; pl.block[1] = block.y; pl.block[2] = block.z;
+    pl.split_k = split_k;
+    pl.launches = launches;
+    pl.workspace_bytes = ws_bytes;
+}
+
+void add_launch(oxq_ctx *ctx) { ctx->plan.launches++; }
+
+static void dims_str(const oxq_tensor *t, char *buf, size_t n) {
+    size_t off = 0;
+    off += snprintf(buf + off, n - off, "[");
+    for (int i = 0; i < t->rank && off < n; ++i)
+        off += snprintf(buf + off, n - off, "%s%lld", i ? ", " : "", (long long)t->dims[i]);
+    if (off < n) snprintf(buf + off, n - off, "]");
+}
+
+// Basic descriptor sanity + residency.  `op` prefixes the message.
+static int check_tensor(const oxq_ctx *ctx, const char *op, const char *what, const oxq_tensor *t) {
+    if (!t) return fail(OXQ_ERR_ARG, "%s: %s is NULL", op, what);
+    if (t->rank < 1 || t->rank > OXQ_MAX_RANK)
+        return fail(OXQ_ERR_SHAPE, "%s: %s rank %d out of [1, %d]", op, what, t->rank, OXQ_MAX_RANK);
+    for (int i = 0; i < t->rank; ++i)
+        if (t->dims[i] < 0) return fail(OXQ_ERR_SHAPE, "%s: %s has a negative dim", op, what);
+    if (dtype_size(t->dtype) == 0) return fail(OXQ_ERR_DTYPE, "%s: %s has an unknown dtype", op, what);
+    if (t->device == OXQ_DEVICE_HOST)
+        return fail(OXQ_ERR_DEVICE,
+                    "%s: %s must be GPU-resident (HIP-only path; host tensors go through the CPU "
+                    "dequantize path)", op, what);
+    if (!ctx->plan_only) {
+        if (t->device != ctx->device)
+            return fail(OXQ_ERR_DEVICE, "%s: %s is on device %d, ctx is on device %d", op, what,
+                        t->device, ctx->device);
+        if (!t->data && numel(t) > 0) return fail(OXQ_ERR_ARG, "%s: %s has a NULL data pointer", op, what);
+    }
+    return OXQ_OK;
+}
+
+#define OXQ_TRY(expr)              \
+    do {                           \
+        int _rc = (expr);          \
+        if (_rc != OXQ_OK) return _rc; \
+    } while (0)
+
+static bool is_packed_dtype(int dt) { return dt == OXQ_I32 || dt == OXQ_U32; }
+
+// Validation shared by the AWQ/GPTQ GEMV, dequant and tile-GEMM ops.
+// Order follows W4A16Matmul::metal_fwd (metal_ops.rs:1506-1566),
+// GptqMatmul::metal_fwd (1975-2044), DequantizeW4 (1736-1754),
+// DequantizeGptqPacked (2187-2214) and MppQuantMatmul (2631-2684).
+enum Wna16Kind { KIND_GEMV, KIND_DEQUANT, KIND_TILE };
+
+static int check_wna16(oxq_ctx *ctx, const char *op, Wna16Kind kind, const oxq_tensor *x,
+                       const oxq_tensor *qweight, const oxq_tensor *qzeros,
+                       const oxq_tensor *scales, uint32_t bits, int pack_dim,
+                       const oxq_tensor *out, Wna16Problem *p) {
+    if (!ctx) return fail(OXQ_ERR_ARG, "%s: ctx is NULL", op);
+    if (bits != 4 && bits != 8)
+        return fail(OXQ_ERR_BITS, "%s: bits must be 4 or 8, got %u", op, bits);
+    if (pack_dim != OXQ_PACK_OUT && pack_dim != OXQ_PACK_IN)
+        return fail(OXQ_ERR_ARG, "%s: bad pack_dim %d", op, pack_dim);
+    if (kind != KIND_DEQUANT) OXQ_TRY(check_tensor(ctx, op, "x", x));
+    OXQ_TRY(check_tensor(ctx, op, "qweight", qweight));
+    OXQ_TRY(check_tensor(ctx, op, "qzeros", qzeros));
+    OXQ_TRY(check_tensor(ctx, op, "scales", scales));
+    OXQ_TRY(check_tensor(ctx, op, "out", out));
+    char b0[96], b1[96];
+
+    int64_t m = 1, in_features = 0;
+    if (kind != KIND_DEQUANT) {
+        if (!x->contiguous) return fail(OXQ_ERR_CONTIGUOUS, "%s: x must be contiguous", op);
+        dims_str(x, b0, sizeof b0);
+        if (x->rank != 2) return fail(OXQ_ERR_SHAPE, "%s: x must be 2-D [m, in], got %s", op, b0);
+        if (kind == KIND_GEMV && !(x->dims[0] >= 1 && x->dims[0] <= 8))
+            return fail(OXQ_ERR_M_RANGE,
+                        "%s: x must be [m, in] with m in 1..=8 (decode GEMV path), got %s", op, b0);
+        if (x->dims[0] < 1) return fail(OXQ_ERR_SHAPE, "%s: x has no rows, got %s", op, b0);
+        m = x->dims[0];
+        in_features = x->dims[1];
+    } else if (!qweight->contiguous) {
+        return fail(OXQ_ERR_CONTIGUOUS, "%s: qweight must be contiguous", op);
+    }
+    if (qweight->rank != 2)
+        return fail(OXQ_ERR_SHAPE, "%s: qweight must be 2-D", op);
+    if (scales->rank != 2) return fail(OXQ_ERR_SHAPE, "%s: scales must be 2-D [groups, out]", op);
+    if (!is_packed_dtype(qweight->dtype) || !is_packed_dtype(qzeros->dtype))
+        return fail(OXQ_ERR_DTYPE, "%s: qweight/qzeros must be I32 or U32, got %s/%s", op,
+                    dtype_name(qweight->dtype), dtype_name(qzeros->dtype));
+    if (!qweight->contiguous || !qzeros->contiguous || !scales->contiguous)
+        return fail(OXQ_ERR_CONTIGUOUS, "%s: qweight, qzeros and scales must be contiguous", op);
+
+    const int64_t pf = 32 / bits;
+    const int64_t groups = scales->dims[0], out_features = scales->dims[1];
+    int64_t K;
+    if (pack_dim == OXQ_PACK_OUT) {
+        const int64_t qw_in = qweight->dims[0], packed_out = qweight->dims[1];
+        if (qzeros->rank != 2 || qzeros->dims[0] != groups || qzeros->dims[1] != packed_out) {
+            dims_str(qzeros, b0, sizeof b0);
+            return fail(OXQ_ERR_SHAPE, "%s: qzeros shape %s != [%lld, %lld]", op, b0,
+                        (long long)groups, (long long)packed_out);
+        }
+        // AwqShape::new_bits (metal_ops.rs:1434-1458)
+        if (packed_out * pf != out_features)
+            return fail(OXQ_ERR_SHAPE, "W%uA16: qweight packed_out %lld (x%lld) != scales out %lld",
+                        bits, (long long)packed_out, (long long)pf, (long long)out_features);
+        if (groups == 0 || qw_in % groups != 0)
+            return fail(OXQ_ERR_GROUP, "W%uA16: in_features %lld not divisible by groups %lld", bits,
+                        (long long)qw_in, (long long)groups);
+        K = qw_in;
+    } else {
+        const int64_t packed_in = qweight->dims[0], qw_out = qweight->dims[1];
+        if (qw_out != out_features)
+            return fail(OXQ_ERR_SHAPE, "%s: qweight dim1 %lld != scales out_features %lld", op,
+                        (long long)qw_out, (long long)out_features);
+        if (qzeros->rank != 2 || qzeros->dims[0] != groups || qzeros->dims[1] * pf != out_features) {
+            dims_str(qzeros, b0, sizeof b0);
+            return fail(OXQ_ERR_SHAPE, "%s: qzeros shape %s != [%lld, %lld]", op, b0,
+                        (long long)groups, (long long)(out_features / pf));
+        }
+        // GptqShape::new_bits (metal_ops.rs:1923-1943)
+        K = packed_in * pf;
+        if (groups == 0 || K % groups != 0)
+            return fail(OXQ_ERR_GROUP, "GPTQ-W%uA16: in_features %lld not divisible by groups %lld",
+                        bits, (long long)K, (long long)groups);
+        if (out_features % pf != 0)
+            return fail(OXQ_ERR_SHAPE,
+                        "GPTQ-W%uA16: out_features %lld not divisible by pack_factor %lld", bits,
+                        (long long)out_features, (long long)pf);
+    }
+    const int64_t group_size = K / groups;
+    if (kind != KIND_DEQUANT && in_features != K)
+        return fail(OXQ_ERR_SHAPE, "%s: x in_features %lld != weight in_features %lld", op,
+                    (long long)in_features, (long long)K);
+    dims_str(out, b1, sizeof b1);
+    if (kind == KIND_DEQUANT) {
+        if (out->rank != 2 || out->dims[0] != K || out->dims[1] != out_features)
+            return fail(OXQ_ERR_SHAPE, "%s: output shape %s != [%lld, %lld]", op, b1, (long long)K,
+                        (long long)out_features);
+    } else if (out->rank != 2 || out->dims[0] != m || out->dims[1] != out_features) {
+        return fail(OXQ_ERR_SHAPE, "%s: output shape %s != [%lld, %lld]", op, b1, (long long)m,
+                    (long long)out_features);
+    }
+    if (!out->contiguous) return fail(OXQ_ERR_CONTIGUOUS, "%s: out must be contiguous", op);
+    const int act = kind == KIND_DEQUANT ? scales->dtype : x->dtype;
+    if (kind != KIND_DEQUANT && scales->dtype != x->dtype)
+        return fail(OXQ_ERR_DTYPE, "%s: scales dtype %s must match x dtype %s", op,
+                    dtype_name(scales->dtype), dtype_name(x->dtype));
+    if (act != OXQ_F16 && act != OXQ_BF16)
+        return fail(OXQ_ERR_DTYPE, "%s: unsupported (bits, dtype) combo (%u, %s)", op, bits,
+                    dtype_name(act));
+    if (out->dtype != act)
+        return fail(OXQ_ERR_DTYPE, "%s: out dtype %s must be %s", op, dtype_name(out->dtype),
+                    dtype_name(act));
+    if (!is_pow2(group_size))
+        return fail(OXQ_ERR_GROUP, "%s: group_size %lld must be a power of two", op,
+                    (long long)group_size);
+    if (pack_dim == OXQ_PACK_IN && group_size % pf != 0)
+        return fail(OXQ_ERR_GROUP, "%s: group_size %lld must be a multiple of pack_factor %lld", op,
+                    (long long)group_size, (long long)pf);
+    if (K > INT32_MAX || out_features > INT32_MAX || m > INT32_MAX)
+        return fail(OXQ_ERR_SHAPE, "%s: dimension exceeds 2^31-1", op);
+
+    p->x = x ? x->data : nullptr;
+    p->qweight = (const uint32_t *)qweight->data;
+    p->qzeros = (const uint32_t *)qzeros->data;
+    p->scales = scales->data;
+    p->bias = nullptr;
+    p->y = out->data;
+    p->M = m;
+    p->K = K;
+    p->N = out_features;
+    p->group_size = group_size;
+    p->group_shift = ilog2(group_size);
+    p->bits = (int)bits;
+    p->pack_dim = pack_dim;
+    p->dtype = act;
+    return OXQ_OK;
+}
+
+static int check_bias(const oxq_ctx *ctx, const char *op, const oxq_tensor *bias, int64_t n, int dtype) {
+    if (!bias) return OXQ_OK;
+    OXQ_TRY(check_tensor(ctx, op, "bias", bias));
+    if (numel(bias) != n || !bias->contiguous)
+        return fail(OXQ_ERR_SHAPE, "%s: bias must be a contiguous [%lld] tensor", op, (long long)n);
+    if (bias->dtype != dtype)
+        return fail(OXQ_ERR_DTYPE, "%s: bias dtype %s must be %s", op, dtype_name(bias->dtype),
+                    dtype_name(dtype));
+    return OXQ_OK;
+}
+
+// ---- GGUF -------------------------------------------------------------------
+static const char *gguf_name(int q) {
+    switch (q) {
+    case OXQ_GGUF_Q4_0: return "Q4_0";
+    case OXQ_GGUF_Q8_0: return "Q8_0";
+    case OXQ_GGUF_Q4_K: return "Q4K";
+    case OXQ_GGUF_Q6_K: return "Q6K";
+    default: return "?";
+    }
+}
+
+// GgufQuantMatmul::metal_fwd (metal_ops.rs:5357-5431) / GgufQuantMulMM (5872-5919).
+static int check_gguf(oxq_ctx *ctx, const char *op, bool decode, bool dequant, const oxq_tensor *x,
+                      const oxq_tensor *w, int64_t in_features, int64_t out_features, int quant,
+                      const oxq_tensor *out, GgufProblem *p) {
+    if (!ctx) return fail(OXQ_ERR_ARG, "%s: ctx is NULL", op);
+    int64_t be, bb;
+    if (oxq_gguf_block_layout(quant, &be, &bb) != OXQ_OK)
+        return fail(OXQ_ERR_ARG, "%s: unknown GGUF quant %d", op, quant);
+    const char *qn = gguf_name(quant);
+    if (!dequant) OXQ_TRY(check_tensor(ctx, op, "x", x));
+    OXQ_TRY(check_tensor(ctx, op, "weight_bytes", w));
+    OXQ_TRY(check_tensor(ctx, op, "out", out));
+    char b0[96];
+    int act = OXQ_F32;
+    int64_t m = 1;
+    if (!dequant) {
+        act = x->dtype;
+        if (out->dtype != OXQ_BF16 && out->dtype != OXQ_F32)
+            return fail(OXQ_ERR_DTYPE, "%s (%s): out must be BF16 or F32, got %s", op, qn,
+                        dtype_name(out->dtype));
+        if (act != OXQ_BF16 && act != OXQ_F32)
+            return fail(OXQ_ERR_DTYPE, "%s (%s): x must be BF16 or F32, got %s", op, qn, dtype_name(act));
+        if (out->dtype != act)
+            return fail(OXQ_ERR_DTYPE, "%s (%s): out dtype %s must match x dtype %s", op, qn,
+                        dtype_name(out->dtype), dtype_name(act));
+    } else if (out->dtype != OXQ_F32) {
+        return fail(OXQ_ERR_DTYPE, "%s (%s): out must be F32, got %s", op, qn, dtype_name(out->dtype));
+    }
+    if (w->dtype != OXQ_U8)
+        return fail(OXQ_ERR_DTYPE, "%s (%s): weight_bytes must be U8, got %s", op, qn,
+                    dtype_name(w->dtype));
+    if (in_features <= 0 || out_features <= 0 || in_features % be != 0)
+        return fail(OXQ_ERR_SHAPE, "%s (%s): in_features %lld must be a multiple of %lld", op, qn,
+                    (long long)in_features, (long long)be);
+    if (!dequant) {
+        m = x->rank >= 1 ? x->dims[0] : 0;
+        if (decode && !(m >= 1 && m <= 8))
+            return fail(OXQ_ERR_M_RANGE, "%s (%s): m %lld out of [1, 8]", op, qn, (long long)m);
+        if (!x->contiguous) return fail(OXQ_ERR_CONTIGUOUS, "%s (%s): x must be contiguous", op, qn);
+        dims_str(x, b0, sizeof b0);
+        if (x->rank != 2 || x->dims[1] != in_features || m < 1)
+            return fail(OXQ_ERR_SHAPE, "%s (%s): x shape %s != [%s, %lld]", op, qn, b0,
+                        decode ? "m" : "M", (long long)in_features);
+    }
+    dims_str(out, b0, sizeof b0);
+    const int64_t o0 = dequant ? out_features : m, o1 = dequant ? in_features : out_features;
+    if (out->rank != 2 || out->dims[0] != o0 || out->dims[1] != o1 || !out->contiguous)
+        return fail(OXQ_ERR_SHAPE, "%s (%s): output shape %s != [%lld, %lld]", op, qn, b0,
+                    (long long)o0, (long long)o1);
+    const int64_t expected = out_features * (in_features / be) * bb;
+    if (numel(w) != expected || !w->contiguous)
+        return fail(OXQ_ERR_SHAPE,
+                    "%s (%s): weight_bytes has %lld bytes, expected %lld (out=%lld x "
+                    "blocks_per_row=%lld x %lld)", op, qn, (long long)numel(w), (long long)expected,
+                    (long long)out_features, (long long)(in_features / be), (long long)bb);
+    if (in_features > INT32_MAX || out_features > INT32_MAX)
+        return fail(OXQ_ERR_SHAPE, "%s: dimension exceeds 2^31-1", op);
+    p->x = x ? x->data : nullptr;
+    p->w = (const uint8_t *)w->data;
+    p->bias = nullptr;
+    p->y = out->data;
+    p->M = m;
+    p->K = in_features;
+    p->N = out_features;
+    p->quant = quant;
+    p->act_dtype = act;
+    return OXQ_OK;
+}
+
+// Mxfp4Matmul::metal_fwd (metal_ops.rs:6009-6058)
+static int check_mxfp4(oxq_ctx *ctx, const char *op, bool dequant, const oxq_tensor *x,
+                       const oxq_tensor *blocks, const oxq_tensor *scales, int64_t k, int64_t n,
+                       int64_t n_experts, const oxq_tensor *out, Mxfp4Problem *p) {
+    if (!ctx) return fail(OXQ_ERR_ARG, "%s: ctx is NULL", op);
+    if (!dequant) OXQ_TRY(check_tensor(ctx, op, "x", x));
+    OXQ_TRY(check_tensor(ctx, op, "blocks", blocks));
+    OXQ_TRY(check_tensor(ctx, op, "scales", scales));
+    OXQ_TRY(check_tensor(ctx, op, "out", out));
+    char b0[96];
+    if (!dequant && (out->dtype != OXQ_BF16 || x->dtype != OXQ_BF16))
+        return fail(OXQ_ERR_DTYPE, "%s: x/out must be BF16, got %s/%s", op, dtype_name(x->dtype),
+                    dtype_name(out->dtype));
+    if (dequant && out->dtype != OXQ_F32)
+        return fail(OXQ_ERR_DTYPE, "%s: out must be F32, got %s", op, dtype_name(out->dtype));
+    if (blocks->dtype != OXQ_U8 || scales->dtype != OXQ_U8)
+        return fail(OXQ_ERR_DTYPE, "%s: blocks/scales must be U8", op);
+    if (k <= 0 || n <= 0 || k % 32 != 0)
+        return fail(OXQ_ERR_SHAPE, "%s: K %lld must be a multiple of 32", op, (long long)k);
+    const int64_t nb = k / 32;
+    const int64_t e = n_experts > 0 ? n_experts : 1;
+    if (numel(blocks) != e * n * nb * 16 || numel(scales) != e * n * nb || !blocks->contiguous ||
+        !scales->contiguous)
+        return fail(OXQ_ERR_SHAPE, "%s: blocks %lld / scales %lld elements don't match [%lld, %lld]",
+                    op, (long long)numel(blocks), (long long)numel(scales), (long long)n, (long long)k);
+    int64_t m = 1;
+    if (!dequant) {
+        if (!x->contiguous) return fail(OXQ_ERR_CONTIGUOUS, "%s: x must be contiguous", op);
+        dims_str(x, b0, sizeof b0);
+        if (x->rank != 2 || x->dims[1] != k || x->dims[0] < 1)
+            return fail(OXQ_ERR_SHAPE, "%s: x shape %s != [m, %lld]", op, b0, (long long)k);
+        m = x->dims[0];
+    }
+    if (k > INT32_MAX || n > INT32_MAX) return fail(OXQ_ERR_SHAPE, "%s: dimension exceeds 2^31-1", op);
+    p->x = x ? x->data : nullptr;
+    p->blocks = (const uint8_t *)blocks->data;
+    p->scales = (const uint8_t *)scales->data;
+    p->bias = nullptr;
+    p->y = out->data;
+    p->M = m;
+    p->K = k;
+    p->N = n;
+    p->n_experts = 0;
+    p->expert_offsets = nullptr;
+    p->token_ids = nullptr;
+    p->n_pairs = 0;
+    return OXQ_OK;
+}
+
+}  // namespace oxq
+
+using namespace oxq;
+
+// =============================================================================
+// C ABI
+// =============================================================================
+extern "C" {
+
+void oxq_version(int *major, int *minor) {
+    if (major) *major = OXQ_VERSION_MAJOR;
+    if (minor) *minor = OXQ_VERSION_MINOR;
+}
+
+const char *oxq_last_error(void) { return g_last_error; }
+
+const char *oxq_status_name(int status) {
+    switch (status) {
+    case OXQ_OK: return "OXQ_OK";
+    case OXQ_ERR_ARG: return "OXQ_ERR_ARG";
+    case OXQ_ERR_DTYPE: return "OXQ_ERR_DTYPE";
+    case OXQ_ERR_SHAPE: return "OXQ_ERR_SHAPE";
+    case OXQ_ERR_CONTIGUOUS: return "OXQ_ERR_CONTIGUOUS";
+    case OXQ_ERR_M_RANGE: return "OXQ_ERR_M_RANGE";
+    case OXQ_ERR_GROUP: return "OXQ_ERR_GROUP";
+    case OXQ_ERR_DEVICE: return "OXQ_ERR_DEVICE";
+    case OXQ_ERR_BITS: return "OXQ_ERR_BITS";
+    case OXQ_ERR_RUNTIME: return "OXQ_ERR_RUNTIME";
+    case OXQ_ERR_WORKSPACE: return "OXQ_ERR_WORKSPACE";
+    case OXQ_ERR_UNSUPPORTED: return "OXQ_ERR_UNSUPPORTED";
+    default: return "OXQ_ERR_?";
+    }
+}
+
+int oxq_gguf_block_layout(int quant, int64_t *block_elems, int64_t *block_bytes) {
+    int64_t e, b;
+    switch (quant) {
+    case OXQ_GGUF_Q4_0: e = 32; b = 18; break;
+    case OXQ_GGUF_Q8_0: e = 32; b = 34; break;
+    case OXQ_GGUF_Q4_K: e = 256; b = 144; break;
+    case OXQ_GGUF_Q6_K: e = 256; b = 210; break;
+    default: return fail(OXQ_ERR_ARG, "unknown GGUF quant %d", quant);
+    }
+    if (block_elems) *block_elems = e;
+    if (block_bytes) *block_bytes = b;
+    return OXQ_OK;
+}
+
+int oxq_ctx_create(int device, oxq_ctx **out) {
+    if (!out) return fail(OXQ_ERR_ARG, "oxq_ctx_create: out is NULL");
+    *out = nullptr;
+    oxq_ctx *ctx = new (std::nothrow) oxq_ctx();
+    if (!ctx) return fail(OXQ_ERR_RUNTIME, "oxq_ctx_create: out of host memory");
+    memset(ctx, 0, sizeof *ctx);
+    ctx->device = device;
+    ctx->plan_only = device == OXQ_DEVICE_PLAN_ONLY;
+    ctx->num_cus = 256;
+    const char *ws_env = getenv("OXQ_WORKSPACE_MB");
+    const size_t ws_mb = (ws_env && atoi(ws_env) > 0) ? (size_t)atoi(ws_env) : 64;
+    ctx->workspace_bytes = ws_mb << 20;
+    ctx->n_counters = 16384;
+    if (ctx->plan_only) {
+        *out = ctx;
+        return OXQ_OK;
+    }
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || device < 0 || device >= count) {
+        delete ctx;
+        return fail(OXQ_ERR_DEVICE, "oxq_ctx_create: no HIP device %d (%d visible%s%s)", device,
+                    count, e != hipSuccess ? ": " : "", e != hipSuccess ? hipGetErrorString(e) : "");
+    }
+    int prev = 0;
+    (void)hipGetDevice(&prev);
+    int rc = OXQ_OK;
+    do {
+        if ((e = hipSetDevice(device)) != hipSuccess) break;
+        int cus = 0;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess &&
+            cus > 0)
+            ctx->num_cus = cus;
+        if ((e = hipMalloc(&ctx->workspace, ctx->workspace_bytes)) != hipSuccess) break;
+        if ((e = hipMalloc((void **)&ctx->counters, ctx->n_counters * sizeof(unsigned))) != hipSuccess)
+            break;
+        if ((e = hipMemset(ctx->counters, 0, ctx->n_counters * sizeof(unsigned))) != hipSuccess) break;
+        e = hipDeviceSynchronize();
+    } while (0);
+    (void)hipSetDevice(prev);
+    if (e != hipSuccess) {
+        rc = fail(OXQ_ERR_RUNTIME, "oxq_ctx_create: %s", hipGetErrorString(e));
+        if (ctx->workspace) (void)hipFree(ctx->workspace);
+        if (ctx->counters) (void)hipFree(ctx->counters);
+        delete ctx;
+        return rc;
+    }
+    *out = ctx;
+    return OXQ_OK;
+}
+
+int oxq_ctx_destroy(oxq_ctx *ctx) {
+    if (!ctx) return OXQ_OK;
+    if (!ctx->plan_only) {
+        if (ctx->workspace) (void)hipFree(ctx->workspace);
+        if (ctx->counters) (void)hipFree(ctx->counters);
+    }
+    delete ctx;
+    return OXQ_OK;
+}
+
+int oxq_ctx_device(const oxq_ctx *ctx) { return ctx ? ctx->device : OXQ_DEVICE_PLAN_ONLY; }
+
+int oxq_ctx_last_plan(const oxq_ctx *ctx, oxq_plan *out) {
+    if (!ctx || !out) return fail(OXQ_ERR_ARG, "oxq_ctx_last_plan: NULL argument");
+    *out = ctx->plan;
+    return OXQ_OK;
+}
+
+// ---- AWQ / GPTQ -------------------------------------------------------------
+int oxq_w4a16_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x, const oxq_tensor *qweight,
+                     const oxq_tensor *qzeros, const oxq_tensor *scales, const oxq_tensor *out) {
+    Wna16Problem p;
+    OXQ_TRY(check_wna16(ctx, "W4A16Matmul", KIND_GEMV, x, qweight, qzeros, scales, 4, OXQ_PACK_OUT,
+                        out, &p));
+    return launch_wna16_gemv(ctx, (hipStream_t)stream, p);
+}
+
+int oxq_w8a16_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x, const oxq_tensor *qweight,
+                     const oxq_tensor *qzeros, const oxq_tensor *scales, const oxq_tensor *out) {
+    Wna16Problem p;
+    OXQ_TRY(check_wna16(ctx, "W8A16Matmul", KIND_GEMV, x, qweight, qzeros, scales, 8, OXQ_PACK_OUT,
+                        out, &p));
+    return launch_wna16_gemv(ctx, (hipStream_t)stream, p);
+}
+
+int oxq_gptq_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x, const oxq_tensor *qweight,
+                    const oxq_tensor *qzeros, const oxq_tensor *scales, uint32_t bits,
+                    const oxq_tensor *out) {
+    Wna16Problem p;
+    OXQ_TRY(check_wna16(ctx, "GptqMatmul", KIND_GEMV, x, qweight, qzeros, scales, bits, OXQ_PACK_IN,
+                        out, &p));
+    return launch_wna16_gemv(ctx, (hipStream_t)stream, p);
+}
+
+int oxq_dequantize_w4(oxq_ctx *ctx, void *stream, const oxq_tensor *qweight,
+                      const oxq_tensor *qzeros, const oxq_tensor *scales, const oxq_tensor *out) {
+    Wna16Problem p;
+    OXQ_TRY(check_wna16(ctx, "DequantizeW4", KIND_DEQUANT, nullptr, qweight, qzeros, scales, 4,
+                        OXQ_PACK_OUT, out, &p));
+    return launch_wna16_dequant(ctx, (hipStream_t)stream, p, out->data);
+}
+
+int oxq_dequantize_w8(oxq_ctx *ctx, void *stream, const oxq_tensor *qweight,
+                      const oxq_tensor *qzeros, const oxq_tensor *scales, const oxq_tensor *out) {
+    Wna16Problem p;
+    OXQ_TRY(check_wna16(ctx, "DequantizeW8", KIND_DEQUANT, nullptr, qweight, qzeros, scales, 8,
+                        OXQ_PACK_OUT, out, &p));
+    return launch_wna16_dequant(ctx, (hipStream_t)stream, p, out->data);
+}
+
+int oxq_dequantize_gptq_packed(oxq_ctx *ctx, void *stream, const oxq_tensor *qweight,
+                               const oxq_tensor *qzeros, const oxq_tensor *scales, uint32_t bits,
+                               const oxq_tensor *out) {
+    Wna16Problem p;
+    OXQ_TRY(check_wna16(ctx, "DequantizeGptq", KIND_DEQUANT, nullptr, qweight, qzeros, scales, bits,
+                        OXQ_PACK_IN, out, &p));
+    return launch_wna16_dequant(ctx, (hipStream_t)stream, p, out->data);
+}
+
+int oxq_mpp_quant_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x,
+                         const oxq_tensor *qweight, const oxq_tensor *qzeros,
+                         const oxq_tensor *scales, uint32_t bits, int pack_dim,
+                         const oxq_tensor *out) {
+    Wna16Problem p;
+    OXQ_TRY(check_wna16(ctx, "MppQuantMatmul", KIND_TILE, x, qweight, qzeros, scales, bits, pack_dim,
+                        out, &p));
+    return launch_wna16_mfma(ctx, (hipStream_t)stream, p);
+}
+
+int oxq_maybe_mpp_quant_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x,
+                               const oxq_tensor *qweight, const oxq_tensor *qzeros,
+                               const oxq_tensor *scales, uint32_t bits, int pack_dim,
+                               const oxq_tensor *out, int *taken) {
+    if (!taken) return fail(OXQ_ERR_ARG, "maybe_mpp_quant_matmul: taken is NULL");
+    *taken = 0;
+    // decline rules: metal_ops.rs:2779-2791
+    if (!x || !scales) return fail(OXQ_ERR_ARG, "maybe_mpp_quant_matmul: NULL tensor");
+    if ((x->dtype != OXQ_BF16 && x->dtype != OXQ_F16) || scales->dtype != x->dtype) return OXQ_OK;
+    if (x->device == OXQ_DEVICE_HOST) return OXQ_OK;
+    if (x->rank != 2 || x->dims[0] < OXQ_MFMA_MIN_M || !x->contiguous) return OXQ_OK;
+    int rc = oxq_mpp_quant_matmul(ctx, stream, x, qweight, qzeros, scales, bits, pack_dim, out);
+    if (rc == OXQ_OK) *taken = 1;
+    return rc;
+}
+
+// ---- GGUF ---------------------------------------------------------------------
+int oxq_gguf_quant_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x,
+                          const oxq_tensor *weight_bytes, int64_t in_features,
+                          int64_t out_features, int quant, const oxq_tensor *out) {
+    GgufProblem p;
+    OXQ_TRY(check_gguf(ctx, "GgufQuantMatmul", true, false, x, weight_bytes, in_features,
+                       out_features, quant, out, &p));
+    return launch_gguf_gemv(ctx, (hipStream_t)stream, p);
+}
+
+int oxq_gguf_quant_mul_mm(oxq_ctx *ctx, void *stream, const oxq_tensor *x,
+                          const oxq_tensor *weight_bytes, int64_t in_features,
+                          int64_t out_features, int quant, const oxq_tensor *out) {
+    GgufProblem p;
+    OXQ_TRY(check_gguf(ctx, "GgufQuantMulMM", false, false, x, weight_bytes, in_features,
+                       out_features, quant, out, &p));
+    return launch_gguf_gemv(ctx, (hipStream_t)stream, p);
+}
+
+int oxq_gguf_dequantize(oxq_ctx *ctx, void *stream, const oxq_tensor *weight_bytes,
+                        int64_t in_features, int64_t out_features, int quant,
+                        const oxq_tensor *out) {
+    GgufProblem p;
+    OXQ_TRY(check_gguf(ctx, "GgufDequantize", false, true, nullptr, weight_bytes, in_features,
+                       out_features, quant, out, &p));
+    return launch_gguf_dequant(ctx, (hipStream_t)stream, p, (float *)out->data);
+}
+
+// ---- MXFP4 ---------------------------------------------------------------------
+int oxq_mxfp4_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x, const oxq_tensor *blocks,
+                     const oxq_tensor *scales, int64_t k, int64_t n, const oxq_tensor *out) {
+    Mxfp4Problem p;
+    OXQ_TRY(check_mxfp4(ctx, "Mxfp4Matmul", false, x, blocks, scales, k, n, 0, out, &p));
+    char b0[96];
+    dims_str(out, b0, sizeof b0);
+    if (out->rank != 2 || out->dims[0] != p.M || out->dims[1] != n || !out->contiguous)
+        return fail(OXQ_ERR_SHAPE, "Mxfp4Matmul: output shape %s != [%lld, %lld]", b0,
+                    (long long)p.M, (long long)n);
+    return launch_mxfp4_gemv(ctx, (hipStream_t)stream, p);
+}
+
+int oxq_mxfp4_dequantize(oxq_ctx *ctx, void *stream, const oxq_tensor *blocks,
+                         const oxq_tensor *scales, int64_t k, int64_t n, const oxq_tensor *out) {
+    Mxfp4Problem p;
+    OXQ_TRY(check_mxfp4(ctx, "Mxfp4Dequantize", true, nullptr, blocks, scales, k, n, 0, out, &p));
+    if (out->rank != 2 || out->dims[0] != n || out->dims[1] != k || !out->contiguous)
+        return fail(OXQ_ERR_SHAPE, "Mxfp4Dequantize: output must be a contiguous [%lld, %lld]",
+                    (long long)n, (long long)k);
+    return launch_mxfp4_dequant(ctx, (hipStream_t)stream, p, (float *)out->data);
+}
+
+int oxq_mxfp4_moe_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x,
+                         const oxq_tensor *blocks, const oxq_tensor *scales,
+                         const oxq_tensor *bias, const oxq_tensor *expert_offsets,
+                         const oxq_tensor *token_ids, int gather_rows, int64_t k, int64_t n,
+                         const oxq_tensor *out) {
+    const char *op = "Mxfp4MoeMatmul";
+    if (!ctx) return fail(OXQ_ERR_ARG, "%s: ctx is NULL", op);
+    OXQ_TRY(check_tensor(ctx, op, "expert_offsets", expert_offsets));
+    if (expert_offsets->dtype != OXQ_I32 || expert_offsets->rank != 1 || expert_offsets->dims[0] < 2 ||
+        !expert_offsets->contiguous)
+        return fail(OXQ_ERR_SHAPE, "%s: expert_offsets must be a contiguous I32 [n_experts + 1]", op);
+    const int64_t n_experts = expert_offsets->dims[0] - 1;
+    Mxfp4Problem p;
+    OXQ_TRY(check_mxfp4(ctx, op, false, x, blocks, scales, k, n, n_experts, out, &p));
+    if (out->rank != 2 || out->dims[1] != n || !out->contiguous)
+        return fail(OXQ_ERR_SHAPE, "%s: out must be a contiguous [n_pairs, %lld]", op, (long long)n);
+    const int64_t n_pairs = out->dims[0];
+    if (gather_rows) {
+        OXQ_TRY(check_tensor(ctx, op, "token_ids", token_ids));
+        if (token_ids->dtype != OXQ_I32 || numel(token_ids) != n_pairs || !token_ids->contiguous)
+            return fail(OXQ_ERR_SHAPE, "%s: token_ids must be a contiguous I32 [%lld]", op,
+                        (long long)n_pairs);
+    } else if (x->dims[0] != n_pairs) {
+        return fail(OXQ_ERR_SHAPE, "%s: x has %lld rows, out has %lld", op, (long long)x->dims[0],
+                    (long long)n_pairs);
+    }
+    if (bias) {
+        OXQ_TRY(check_tensor(ctx, op, "bias", bias));
+        if (bias->dtype != OXQ_BF16 || numel(bias) != n_experts * n || !bias->contiguous)
+            return fail(OXQ_ERR_SHAPE, "%s: bias must be a contiguous BF16 [%lld, %lld]", op,
+                        (long long)n_experts, (long long)n);
+        p.bias = bias->data;
+    }
+    p.n_experts = n_experts;
+    p.expert_offsets = (const int32_t *)expert_offsets->data;
+    p.token_ids = gather_rows ? (const int32_t *)token_ids->data : nullptr;
+    p.n_pairs = n_pairs;
+    return launch_mxfp4_gemv(ctx, (hipStream_t)stream, p);
+}
+
+}  // extern "C"
+
+// =============================================================================
+// Layers: host mirrors of linear.rs / mxfp4.rs
+// =============================================================================
+namespace oxq {
+
+static int flatten_rows(const char *op, const oxq_tensor *x, int64_t in_features, oxq_tensor *x2,
+                        int64_t *m_out) {
+    if (!x) return fail(OXQ_ERR_ARG, "%s: x is NULL", op);
+    if (x->rank < 1 || x->rank > OXQ_MAX_RANK) return fail(OXQ_ERR_SHAPE, "%s: bad x rank", op);
+    const int64_t last = x->dims[x->rank - 1];
+    if (last != in_features)
+        return fail(OXQ_ERR_SHAPE, "%s: input last dim %lld != in_features %lld", op, (long long)last,
+                    (long long)in_features);
+    if (!x->contiguous)
+        return fail(OXQ_ERR_CONTIGUOUS, "%s: x must be contiguous (the caller owns the copy the "
+                                        "reference makes with .contiguous())", op);
+    int64_t m = 1;
+    for (int i = 0; i < x->rank - 1; ++i) m *= x->dims[i];
+    *x2 = *x;
+    x2->rank = 2;
+    x2->dims[0] = m;
+    x2->dims[1] = in_features;
+    *m_out = m;
+    return OXQ_OK;
+}
+
+static int flatten_out(const char *op, const oxq_tensor *out, int64_t m, int64_t n, oxq_tensor *o2) {
+    if (!out) return fail(OXQ_ERR_ARG, "%s: out is NULL", op);
+    if (out->rank < 1 || out->rank > OXQ_MAX_RANK || out->dims[out->rank - 1] != n || numel(out) != m * n ||
+        !out->contiguous)
+        return fail(OXQ_ERR_SHAPE, "%s: out must be contiguous with %lld rows of %lld", op,
+                    (long long)m, (long long)n);
+    *o2 = *out;
+    o2->rank = 2;
+    o2->dims[0] = m;
+    o2->dims[1] = n;
+    return OXQ_OK;
+}
+
+}  // namespace oxq
+
+struct oxq_packed_quant_linear {
+    oxq_ctx *ctx;
+    oxq_tensor qweight, qzeros, scales, bias;
+    bool has_bias;
+    int64_t in_features, out_features;
+    uint32_t bits;
+    int pack_dim;
+    int dtype;
+    // linear.rs:450-455 gemv_max_m: the reference keeps batches up to 16 (AWQ) /
+    // 32 (GPTQ) on the GEMV kernel in chunks of 8 because its only alternative
+    // below m = 64 is a full dense dequant.  Here every m > 8 runs the MFMA tile
+    // kernel, which reads the packed weights once.
+    int64_t gemv_max_m() const { return 8; }
+};
+
+struct oxq_qlinear {
+    oxq_ctx *ctx;
+    oxq_tensor weight_bytes, bias;
+    bool has_bias;
+    int64_t in_features, out_features;
+    int quant;
+    int out_dtype;
+};
+
+struct oxq_mxfp4_linear {
+    oxq_ctx *ctx;
+    oxq_tensor blocks, scales, bias;
+    bool has_bias;
+    int64_t in_features, out_features;
+};
+
+extern "C" {
+
+int oxq_packed_quant_linear_new(oxq_ctx *ctx, uint32_t bits, int pack_dim,
+                                const oxq_tensor *qweight, const oxq_tensor *qzeros,
+                                const oxq_tensor *scales, const oxq_tensor *bias, int dtype,
+                                oxq_packed_quant_linear **out) {
+    const char *op = "PackedQuantLinear";
+    if (!ctx || !out) return fail(OXQ_ERR_ARG, "%s: NULL argument", op);
+    *out = nullptr;
+    if (bits != 4 && bits != 8)  // linear.rs:417-419
+        return fail(OXQ_ERR_BITS, "%s: bits must be 4 or 8, got %u", op, bits);
+    if (!qzeros) return fail(OXQ_ERR_ARG, "%s: qzeros missing", op);  // linear.rs:420-422
+    if (pack_dim != OXQ_PACK_OUT && pack_dim != OXQ_PACK_IN)
+        return fail(OXQ_ERR_ARG, "%s: bad pack_dim %d", op, pack_dim);
+    OXQ_TRY(check_tensor(ctx, op, "qweight", qweight));
+    OXQ_TRY(check_tensor(ctx, op, "qzeros", qzeros));
+    OXQ_TRY(check_tensor(ctx, op, "scales", scales));
+    if (qweight->rank != 2 || scales->rank != 2)
+        return fail(OXQ_ERR_SHAPE, "%s: qweight and scales must be 2-D", op);
+    const int64_t pf = 32 / bits;
+    int64_t in_f, out_f;  // linear.rs:423-430
+    if (pack_dim == OXQ_PACK_OUT) {
+        in_f = qweight->dims[0];
+        out_f = qweight->dims[1] * pf;
+    } else {
+        in_f = qweight->dims[0] * pf;
+        out_f = qweight->dims[1];
+    }
+    if (scales->dims[1] != out_f)  // linear.rs:431-436
+        return fail(OXQ_ERR_SHAPE, "%s: scales out_features %lld != derived %lld", op,
+                    (long long)scales->dims[1], (long long)out_f);
+    if (dtype != OXQ_F16 && dtype != OXQ_BF16)
+        return fail(OXQ_ERR_DTYPE, "%s: runtime dtype must be F16 or BF16", op);
+    if (scales->dtype != dtype)
+        return fail(OXQ_ERR_DTYPE, "%s: scales must already be cast to %s (linear.rs:437), got %s",
+                    op, dtype_name(dtype), dtype_name(scales->dtype));
+    OXQ_TRY(check_bias(ctx, op, bias, out_f, dtype));
+    oxq_packed_quant_linear *l = new (std::nothrow) oxq_packed_quant_linear();
+    if (!l) return fail(OXQ_ERR_RUNTIME, "%s: out of host memory", op);
+    l->ctx = ctx;
+    l->qweight = *qweight;
+    l->qzeros = *qzeros;
+    l->scales = *scales;
+    l->has_bias = bias != nullptr;
+    if (bias) l->bias = *bias;
+    l->in_features = in_f;
+    l->out_features = out_f;
+    l->bits = bits;
+    l->pack_dim = pack_dim;
+    l->dtype = dtype;
+    *out = l;
+    return OXQ_OK;
+}
+
+// linear.rs:482-533 PackedQuantLinear::forward
+int oxq_packed_quant_linear_forward(oxq_packed_quant_linear *l, void *stream, const oxq_tensor *x,
+                                    const oxq_tensor *out) {
+    const char *op = "PackedQuantLinear";
+    if (!l) return fail(OXQ_ERR_ARG, "%s: layer is NULL", op);
+    oxq_tensor x2, o2;
+    int64_t m;
+    OXQ_TRY(flatten_rows(op, x, l->in_features, &x2, &m));
+    OXQ_TRY(flatten_out(op, out, m, l->out_features, &o2));
+    Wna16Problem p;
+    const bool gemv = m <= l->gemv_max_m();
+    OXQ_TRY(check_wna16(l->ctx, op, gemv ? KIND_GEMV : KIND_TILE, &x2, &l->qweight, &l->qzeros,
+                        &l->scales, l->bits, l->pack_dim, &o2, &p));
+    p.bias = l->has_bias ? l->bias.data : nullptr;
+    return gemv ? launch_wna16_gemv(l->ctx, (hipStream_t)stream, p)
+                : launch_wna16_mfma(l->ctx, (hipStream_t)stream, p);
+}
+
+int oxq_packed_quant_linear_in_features(const oxq_packed_quant_linear *l, int64_t *k) {
+    if (!l || !k) return fail(OXQ_ERR_ARG, "PackedQuantLinear: NULL argument");
+    *k = l->in_features;
+    return OXQ_OK;
+}
+int oxq_packed_quant_linear_out_features(const oxq_packed_quant_linear *l, int64_t *n) {
+    if (!l || !n) return fail(OXQ_ERR_ARG, "PackedQuantLinear: NULL argument");
+    *n = l->out_features;
+    return OXQ_OK;
+}
+void oxq_packed_quant_linear_free(oxq_packed_quant_linear *l) { delete l; }
+
+// linear.rs:197-247 GgufFastPath::build
+int oxq_qlinear_new(oxq_ctx *ctx, int quant, const oxq_tensor *weight_bytes, int64_t in_features,
+                    int64_t out_features, const oxq_tensor *bias, int out_dtype, oxq_qlinear **out) {
+    const char *op = "QLinear";
+    if (!ctx || !out) return fail(OXQ_ERR_ARG, "%s: NULL argument", op);
+    *out = nullptr;
+    int64_t be, bb;
+    OXQ_TRY(oxq_gguf_block_layout(quant, &be, &bb));
+    OXQ_TRY(check_tensor(ctx, op, "weight_bytes", weight_bytes));
+    if (weight_bytes->dtype != OXQ_U8) return fail(OXQ_ERR_DTYPE, "%s: weight_bytes must be U8", op);
+    if (in_features <= 0 || out_features <= 0 || in_features % be != 0)
+        return fail(OXQ_ERR_SHAPE, "%s: in_features %lld must be a multiple of %lld", op,
+                    (long long)in_features, (long long)be);
+    const int64_t expected = out_features * (in_features / be) * bb;  // linear.rs:227-237
+    if (numel(weight_bytes) != expected)
+        return fail(OXQ_ERR_SHAPE,
+                    "GGUF fast path: weight has %lld bytes, expected %lld for shape [%lld, %lld]",
+                    (long long)numel(weight_bytes), (long long)expected, (long long)out_features,
+                    (long long)in_features);
+    if (out_dtype != OXQ_BF16 && out_dtype != OXQ_F32)
+        return fail(OXQ_ERR_DTYPE, "%s: out dtype must be BF16 or F32", op);
+    OXQ_TRY(check_bias(ctx, op, bias, out_features, out_dtype));
+    oxq_qlinear *l = new (std::nothrow) oxq_qlinear();
+    if (!l) return fail(OXQ_ERR_RUNTIME, "%s: out of host memory", op);
+    l->ctx = ctx;
+    l->weight_bytes = *weight_bytes;
+    l->has_bias = bias != nullptr;
+    if (bias) l->bias = *bias;
+    l->in_features = in_features;
+    l->out_features = out_features;
+    l->quant = quant;
+    l->out_dtype = out_dtype;
+    *out = l;
+    return OXQ_OK;
+}
+
+// linear.rs:324-351 QLinear::forward (fast-path arm), 250-284 forward_decode/prefill
+int oxq_qlinear_forward(oxq_qlinear *l, void *stream, const oxq_tensor *x, const oxq_tensor *out) {
+    const char *op = "QLinear";
+    if (!l) return fail(OXQ_ERR_ARG, "%s: layer is NULL", op);
+    oxq_tensor x2, o2;
+    int64_t m;
+    OXQ_TRY(flatten_rows(op, x, l->in_features, &x2, &m));
+    OXQ_TRY(flatten_out(op, out, m, l->out_features, &o2));
+    if (out->dtype != l->out_dtype)
+        return fail(OXQ_ERR_DTYPE, "%s: out dtype %s != layer out dtype %s", op,
+                    dtype_name(out->dtype), dtype_name(l->out_dtype));
+    GgufProblem p;
+    const bool decode = m >= 1 && m <= 8;  // GGUF_BATCH_MAX, metal_ops.rs:5324
+    OXQ_TRY(check_gguf(l->ctx, decode ? "GgufQuantMatmul" : "GgufQuantMulMM", decode, false, &x2,
+                       &l->weight_bytes, l->in_features, l->out_features, l->quant, &o2, &p));
+    p.bias = l->has_bias ? l->bias.data : nullptr;
+    return launch_gguf_gemv(l->ctx, (hipStream_t)stream, p);
+}
+
+void oxq_qlinear_free(oxq_qlinear *l) { delete l; }
+
+// mxfp4.rs:78-116 Mxfp4Linear::new
+int oxq_mxfp4_linear_new(oxq_ctx *ctx, const oxq_tensor *blocks, const oxq_tensor *scales,
+                         const oxq_tensor *bias, int64_t in_features, int64_t out_features,
+                         oxq_mxfp4_linear **out) {
+    const char *op = "Mxfp4Linear";
+    if (!ctx || !out) return fail(OXQ_ERR_ARG, "%s: NULL argument", op);
+    *out = nullptr;
+    OXQ_TRY(check_tensor(ctx, op, "blocks", blocks));
+    OXQ_TRY(check_tensor(ctx, op, "scales", scales));
+    if (blocks->dtype != OXQ_U8 || scales->dtype != OXQ_U8)
+        return fail(OXQ_ERR_DTYPE, "%s: blocks/scales must be U8, got %s/%s", op,
+                    dtype_name(blocks->dtype), dtype_name(scales->dtype));
+    if (in_features <= 0 || in_features % 32 != 0)
+        return fail(OXQ_ERR_SHAPE, "%s: in_features %lld must be a multiple of 32", op,
+                    (long long)in_features);
+    const int64_t nb = in_features / 32;
+    if (numel(blocks) != out_features * nb * 16 || numel(scales) != out_features * nb)
+        return fail(OXQ_ERR_SHAPE, "%s: blocks %lld / scales %lld elements don't match [%lld, %lld]",
+                    op, (long long)numel(blocks), (long long)numel(scales), (long long)out_features,
+                    (long long)in_features);
+    OXQ_TRY(check_bias(ctx, op, bias, out_features, OXQ_BF16));
+    oxq_mxfp4_linear *l = new (std::nothrow) oxq_mxfp4_linear();
+    if (!l) return fail(OXQ_ERR_RUNTIME, "%s: out of host memory", op);
+    l->ctx = ctx;
+    l->blocks = *blocks;
+    l->scales = *scales;
+    l->has_bias = bias != nullptr;
+    if (bias) l->bias = *bias;
+    l->in_features = in_features;
+    l->out_features = out_features;
+    *out = l;
+    return OXQ_OK;
+}
+
+// mxfp4.rs:119-154 Mxfp4Linear::forward
+int oxq_mxfp4_linear_forward(oxq_mxfp4_linear *l, void *stream, const oxq_tensor *x,
+                             const oxq_tensor *out) {
+    const char *op = "Mxfp4Linear";
+    if (!l) return fail(OXQ_ERR_ARG, "%s: layer is NULL", op);
+    oxq_tensor x2, o2;
+    int64_t m;
+    if (x && x->rank >= 1 && x->dims[x->rank - 1] != l->in_features)
+        return fail(OXQ_ERR_SHAPE, "%s: x last dim %lld != in_features %lld", op,
+                    (long long)x->dims[x->rank - 1], (long long)l->in_features);
+    OXQ_TRY(flatten_rows(op, x, l->in_features, &x2, &m));
+    OXQ_TRY(flatten_out(op, out, m, l->out_features, &o2));
+    Mxfp4Problem p;
+    OXQ_TRY(check_mxfp4(l->ctx, "Mxfp4Matmul", false, &x2, &l->blocks, &l->scales, l->in_features,
+                        l->out_features, 0, &o2, &p));
+    p.bias = l->has_bias ? l->bias.data : nullptr;
+    return launch_mxfp4_gemv(l->ctx, (hipStream_t)stream, p);
+}
+
+void oxq_mxfp4_linear_free(oxq_mxfp4_linear *l) { delete l; }
+
+}  // extern "C"

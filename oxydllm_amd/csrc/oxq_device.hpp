@@ -1,0 +1,144 @@
+// Device-side helpers shared by the gfx950 kernels: 16-bit type traits,
+// packed-nibble unpack into dot2/MFMA operand pairs, wave reductions and the
+// deterministic split-K arrival protocol.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+namespace oxq {
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+constexpr int WAVE = 64;
+
+__device__ __forceinline__ uint32_t perm_b32(uint32_t hi, uint32_t lo, uint32_t sel) {
+    return __builtin_amdgcn_perm(hi, lo, sel);
+}
+// (lo16(a), lo16(b)) and (hi16(a), hi16(b)) as {low half, high half}
+__device__ __forceinline__ uint32_t pack_lo16(uint32_t a, uint32_t b) {
+    return perm_b32(b, a, 0x05040100u);
+}
+__device__ __forceinline__ uint32_t pack_hi16(uint32_t a, uint32_t b) {
+    return perm_b32(b, a, 0x07060302u);
+}
+
+// AWQ 4-bit slot -> column offset inside the 8 columns of a word.
+__device__ __forceinline__ constexpr int awq_slot_col(int slot) {
+    return ((slot & 3) << 1) | (slot >> 2);
+}
+
+// ---------------------------------------------------------------------------
+// Element-type traits.  `pair` registers hold two 16-bit floats.
+//
+// unpack4(t, p): t holds two 16-bit halves of 4 nibbles each; p[i] receives
+// the pair {nibble i of the low half, nibble i of the high half} as two
+// floats equal to BIAS(i) + nibble.  The OR-with-exponent trick makes the
+// conversion exact: an f16 with exponent 2^10 (2^6) has ulp 1 at mantissa bit
+// 0 (bit 4); a bf16 with exponent 2^7 has ulp 1 at mantissa bit 0.
+// ---------------------------------------------------------------------------
+struct F16Traits {
+    using elem_t = _Float16;
+    static constexpr int DTYPE = 1;
+    static constexpr uint32_t ONES = 0x3C003C00u;
+    __device__ static __forceinline__ float bias(int i) { return (i & 1) ? 64.0f : 1024.0f; }
+    __device__ static __forceinline__ void unpack4(uint32_t t, uint32_t p[4]) {
+        p[0] = (t & 0x000F000Fu) | 0x64006400u;
+        p[1] = (t & 0x00F000F0u) | 0x54005400u;
+        const uint32_t t8 = t >> 8;
+        p[2] = (t8 & 0x000F000Fu) | 0x64006400u;
+        p[3] = (t8 & 0x00F000F0u) | 0x54005400u;
+    }
+    // two bytes (low byte of each half) -> pair of 1024 + byte
+    __device__ static __forceinline__ uint32_t unpack_bytes(uint32_t t) {
+        return (t & 0x00FF00FFu) | 0x64006400u;
+    }
+    static constexpr float BYTE_BIAS = 1024.0f;
+    __device__ static __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, a),
+                                      __builtin_bit_cast(half2_t, b), c, false);
+    }
+    __device__ static __forceinline__ float to_f32(uint16_t v) {
+        return (float)__builtin_bit_cast(_Float16, v);
+    }
+    __device__ static __forceinline__ uint16_t from_f32(float f) {
+        return __builtin_bit_cast(uint16_t, (_Float16)f);
+    }
+};
+
+struct BF16Traits {
+    using elem_t = __bf16;
+    static constexpr int DTYPE = 2;
+    static constexpr uint32_t ONES = 0x3F803F80u;
+    __device__ static __forceinline__ float bias(int) { return 128.0f; }
+    __device__ static __forceinline__ void unpack4(uint32_t t, uint32_t p[4]) {
+        p[0] = (t & 0x000F000Fu) | 0x43004300u;
+        p[1] = ((t >> 4) & 0x000F000Fu) | 0x43004300u;
+        p[2] = ((t >> 8) & 0x000F000Fu) | 0x43004300u;
+        p[3] = ((t >> 12) & 0x000F000Fu) | 0x43004300u;
+    }
+    // bytes need 8 significant bits: go through f32 (exact), keep the high halves
+    __device__ static __forceinline__ uint32_t unpack_bytes(uint32_t t) {
+        const float lo = (float)(t & 0xFFu);
+        const float hi = (float)((t >> 16) & 0xFFu);
+        return (__builtin_bit_cast(uint32_t, lo) >> 16) |
+               (__builtin_bit_cast(uint32_t, hi) & 0xFFFF0000u);
+    }
+    static constexpr float BYTE_BIAS = 0.0f;
+    __device__ static __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a),
+                                               __builtin_bit_cast(bf16x2_t, b), c, false);
+    }
+    __device__ static __forceinline__ float to_f32(uint16_t v) {
+        return __builtin_bit_cast(float, ((uint32_t)v) << 16);
+    }
+    __device__ static __forceinline__ uint16_t from_f32(float f) {  // round to nearest even
+        uint32_t u = __builtin_bit_cast(uint32_t, f);
+        if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
+        u += 0x7fffu + ((u >> 16) & 1u);
+        return (uint16_t)(u >> 16);
+    }
+};
+
+// ---------------------------------------------------------------------------
+// Reductions
+// ---------------------------------------------------------------------------
+template <int WIDTH>
+__device__ __forceinline__ float wave_sum_xor(float v) {  // butterfly over WIDTH lanes
+#pragma unroll
+    for (int off = WIDTH / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, WAVE);
+    return v;
+}
+
+// ---------------------------------------------------------------------------
+// Deterministic split-K.
+//
+// Each of `splits` workgroups that share an output tile stores its f32 partial
+// tile to the workspace, then calls splitk_arrive().  Exactly one caller - the
+// last to arrive - gets `true`; it then sums the partials of all slices in
+// slice order 0..splits-1, so the result does not depend on arrival order.
+// The counter is left at zero for the next launch.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ bool splitk_arrive(unsigned *counters, unsigned tile, unsigned splits) {
+    __shared__ unsigned s_last;
+    __threadfence();  // release this thread's partial stores at device scope
+    __syncthreads();
+    if (threadIdx.x == 0 && threadIdx.y == 0 && threadIdx.z == 0) {
+        const unsigned old = atomicAdd(&counters[tile], 1u);
+        const unsigned last = (old + 1u == splits) ? 1u : 0u;
+        if (last) counters[tile] = 0u;
+        s_last = last;
+    }
+    __syncthreads();
+    const bool last = s_last != 0u;
+    if (last) __threadfence();  // acquire the other slices' stores
+    return last;
+}
+
+}  // namespace oxq

@@ -1,0 +1,116 @@
+// Internal declarations shared by the host API and the kernel launchers.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+
+#include "oxq.h"
+
+struct oxq_ctx {
+    int device;             // HIP ordinal, or OXQ_DEVICE_PLAN_ONLY
+    bool plan_only;
+    void *workspace;        // split-K partial sums (f32)
+    size_t workspace_bytes;
+    unsigned *counters;     // arrival counters, zero between calls
+    size_t n_counters;
+    int num_cus;
+    oxq_plan plan;
+};
+
+namespace oxq {
+
+int fail(int status, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+const char *dtype_name(int dtype);
+
+inline size_t dtype_size(int dtype) {
+    switch (dtype) {
+    case OXQ_F32: case OXQ_I32: case OXQ_U32: return 4;
+    case OXQ_F16: case OXQ_BF16: return 2;
+    case OXQ_U8: return 1;
+    case OXQ_I64: return 8;
+    default: return 0;
+    }
+}
+
+inline int64_t numel(const oxq_tensor *t) {
+    int64_t n = 1;
+    for (int i = 0; i < t->rank; ++i) n *= t->dims[i];
+    return n;
+}
+
+inline bool is_pow2(int64_t v) { return v > 0 && (v & (v - 1)) == 0; }
+inline int ilog2(int64_t v) {
+    int s = 0;
+    while ((int64_t(1) << s) < v) ++s;
+    return s;
+}
+inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+void set_plan(oxq_ctx *ctx, const char *kernel, dim3 grid, dim3 block, uint32_t split_k,
+              uint32_t launches, uint64_t ws_bytes);
+void add_launch(oxq_ctx *ctx);
+
+#define OXQ_HIP_CHECK(expr)                                                                   \
+    do {                                                                                      \
+        hipError_t _e = (expr);                                                               \
+        if (_e != hipSuccess)                                                                 \
+            return ::oxq::fail(OXQ_ERR_RUNTIME, "%s failed: %s", #expr, hipGetErrorString(_e)); \
+    } while (0)
+
+// ---- problem descriptors handed to the launchers (all validated) ----------
+
+struct Wna16Problem {
+    const void *x;          // [M, K] T
+    const uint32_t *qweight;
+    const uint32_t *qzeros;
+    const void *scales;     // [G, N] T
+    const void *bias;       // [N] T or nullptr
+    void *y;                // [M, N] T
+    int64_t M, K, N;
+    int64_t group_size;
+    int group_shift;
+    int bits;               // 4 or 8
+    int pack_dim;           // OXQ_PACK_OUT (AWQ) / OXQ_PACK_IN (GPTQ)
+    int dtype;              // OXQ_F16 / OXQ_BF16
+};
+
+struct GgufProblem {
+    const void *x;          // [M, K] act dtype
+    const uint8_t *w;       // raw blocks
+    const void *bias;       // [N] or nullptr (act dtype)
+    void *y;                // [M, N]
+    int64_t M, K, N;
+    int quant;
+    int act_dtype;          // OXQ_BF16 or OXQ_F32
+};
+
+struct Mxfp4Problem {
+    const void *x;          // bf16
+    const uint8_t *blocks;
+    const uint8_t *scales;
+    const void *bias;       // bf16 [E, N] / [N] or nullptr
+    void *y;                // bf16
+    int64_t M, K, N;
+    // grouped form (n_experts > 0)
+    int64_t n_experts;
+    const int32_t *expert_offsets;
+    const int32_t *token_ids;   // nullptr => identity
+    int64_t n_pairs;
+};
+
+// ---- launchers (defined in the .hip files) ---------------------------------
+int launch_wna16_gemv(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p);
+int launch_wna16_mfma(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p);
+int launch_wna16_dequant(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p, void *out_kn);
+int launch_gguf_gemv(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p);
+int launch_gguf_dequant(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p, float *out_nk);
+int launch_mxfp4_gemv(oxq_ctx *ctx, hipStream_t s, const Mxfp4Problem &p);
+int launch_mxfp4_dequant(oxq_ctx *ctx, hipStream_t s, const Mxfp4Problem &p, float *out_nk);
+int launch_bias_add(oxq_ctx *ctx, hipStream_t s, void *y, const void *bias, int64_t M, int64_t N,
+                    int dtype);
+
+}  // namespace oxq

@@ -1,0 +1,488 @@
+// Fused dequant + GEMV for AWQ / GPTQ packed weights, 1 <= M <= 8 rows.
+//
+//   y[m, n] = sum_k x[m, k] * (q[k, n] - z[k/g, n]) * s[k/g, n]      (AWQ)
+//   y[m, n] = sum_k x[m, k] * (q[k, n] - (z[k/g, n] + 1)) * s[k/g, n] (GPTQ)
+//
+// Reference semantics: quant_kernels.metal:3349-3499 (awq_gemv[_batch]_det_impl)
+// and 3501-3648 (gptq_gemv[_batch]_det_impl): f32 accumulation, deterministic
+// fixed-order reduction of the K slices, result cast to the activation dtype.
+//
+// Two kernel families:
+//   *_generic  one packed word per lane per row, f32 math exactly as the
+//              reference writes it; accepts every shape the reference accepts.
+//   awq4_gemv_fast  the bandwidth path for 4-bit AWQ: 128/64/32-bit coalesced
+//              loads, nibbles turned into exact 16-bit floats with one
+//              AND-OR, rows paired so v_dot2_f32_{f16,bf16} does two MACs
+//              per lane, zero-point and scale applied once per group.
+//
+// Both split K across workgroups and combine the slices with the
+// last-arriver protocol of oxq_device.hpp (bitwise run-to-run deterministic).
+// HBM-bound: the packed weights are read exactly once.
+
+#include "oxq_device.hpp"
+#include "oxq_internal.hpp"
+
+#include <cstdlib>
+
+namespace oxq {
+
+// ---------------------------------------------------------------------------
+// Shared epilogue: the last workgroup of a column tile sums the slices.
+// ---------------------------------------------------------------------------
+template <typename TT>
+__device__ __forceinline__ void splitk_finish(const float *__restrict__ ws,
+                                              const uint16_t *__restrict__ bias,
+                                              uint16_t *__restrict__ y, int M, int N, int S,
+                                              int n0, int tile_cols, int nthreads, int tid) {
+    for (int idx = tid; idx < M * tile_cols; idx += nthreads) {
+        const int m = idx / tile_cols;
+        const int n = n0 + idx % tile_cols;
+        if (n >= N) continue;
+        float tot = 0.0f;
+        for (int s = 0; s < S; ++s) tot += ws[((size_t)s * M + m) * N + n];
+        if (bias) tot += TT::to_f32(bias[n]);
+        y[(size_t)m * N + n] = TT::from_f32(tot);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Generic AWQ-layout kernel (4- and 8-bit).  256 threads = 64 word columns x 4
+// interleaved row phases.
+// ---------------------------------------------------------------------------
+template <typename TT, int BITS, int MB>
+__global__ __launch_bounds__(256) void awq_gemv_generic(
+    const uint16_t *__restrict__ x, const uint32_t *__restrict__ qw,
+    const uint32_t *__restrict__ qz, const uint16_t *__restrict__ sc,
+    const uint16_t *__restrict__ bias, uint16_t *__restrict__ y, float *__restrict__ ws,
+    unsigned *__restrict__ counters, int M, int K, int N, int packed_out, int gshift, int kchunk,
+    int S) {
+    constexpr int PF = 32 / BITS;
+    constexpr uint32_t MASK = (1u << BITS) - 1u;
+    __shared__ float red[4][64][PF];
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    const int j = blockIdx.x * 64 + tx;
+    const int slice = blockIdx.y;
+    const int k0 = slice * kchunk;
+    const int k1 = min(K, k0 + kchunk);
+
+    float acc[MB][PF];
+#pragma unroll
+    for (int m = 0; m < MB; ++m)
+#pragma unroll
+        for (int s = 0; s < PF; ++s) acc[m][s] = 0.0f;
+
+    if (j < packed_out) {
+        int last_g = -1;
+        float zf[PF], sf[PF];
+        for (int i = k0 + ty; i < k1; i += 4) {
+            const int g = i >> gshift;
+            if (g != last_g) {
+                const uint32_t zw = qz[(size_t)g * packed_out + j];
+#pragma unroll
+                for (int s = 0; s < PF; ++s) {
+                    const int col = (BITS == 4) ? awq_slot_col(s) : s;
+                    zf[s] = (float)((zw >> (BITS * s)) & MASK);
+                    sf[s] = TT::to_f32(sc[(size_t)g * N + (size_t)j * PF + col]);
+                }
+                last_g = g;
+            }
+            const uint32_t ww = qw[(size_t)i * packed_out + j];
+            float w[PF];
+#pragma unroll
+            for (int s = 0; s < PF; ++s) w[s] = ((float)((ww >> (BITS * s)) & MASK) - zf[s]) * sf[s];
+#pragma unroll
+            for (int m = 0; m < MB; ++m) {
+                if (m < M) {
+                    const float xv = TT::to_f32(x[(size_t)m * K + i]);
+#pragma unroll
+                    for (int s = 0; s < PF; ++s) acc[m][s] = fmaf(xv, w[s], acc[m][s]);
+                }
+            }
+        }
+    }
+
+    const int tile_cols = 64 * PF;
+    const int n0 = blockIdx.x * tile_cols;
+#pragma unroll
+    for (int m = 0; m < MB; ++m) {
+        if (m < M) {
+#pragma unroll
+            for (int s = 0; s < PF; ++s) red[ty][tx][s] = acc[m][s];
+            __syncthreads();
+            if (ty == 0 && j < packed_out) {
+#pragma unroll
+                for (int s = 0; s < PF; ++s) {
+                    const int col = (BITS == 4) ? awq_slot_col(s) : s;
+                    const float tot = red[0][tx][s] + red[1][tx][s] + red[2][tx][s] + red[3][tx][s];
+                    const int n = j * PF + col;
+                    if (S == 1) {
+                        const float b = bias ? TT::to_f32(bias[n]) : 0.0f;
+                        y[(size_t)m * N + n] = TT::from_f32(tot + b);
+                    } else {
+                        ws[((size_t)slice * M + m) * N + n] = tot;
+                    }
+                }
+            }
+            __syncthreads();
+        }
+    }
+    if (S > 1 && splitk_arrive(counters, blockIdx.x, S))
+        splitk_finish<TT>(ws, bias, y, M, N, S, n0, tile_cols, 256, threadIdx.x);
+}
+
+// ---------------------------------------------------------------------------
+// Generic GPTQ-layout kernel (4- and 8-bit).  One output column per lane; a
+// word holds PF consecutive k for that column.  256 threads = 64 columns x 4
+// interleaved word-row phases.
+// ---------------------------------------------------------------------------
+template <typename TT, int BITS, int MB>
+__global__ __launch_bounds__(256) void gptq_gemv_generic(
+    const uint16_t *__restrict__ x, const uint32_t *__restrict__ qw,
+    const uint32_t *__restrict__ qz, const uint16_t *__restrict__ sc,
+    const uint16_t *__restrict__ bias, uint16_t *__restrict__ y, float *__restrict__ ws,
+    unsigned *__restrict__ counters, int M, int K, int N, int gshift, int wchunk, int S) {
+    constexpr int PF = 32 / BITS;
+    constexpr uint32_t MASK = (1u << BITS) - 1u;
+    __shared__ float red[4][64];
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    const int n = blockIdx.x * 64 + tx;
+    const int slice = blockIdx.y;
+    const int packed_in = K / PF;
+    const int w0 = slice * wchunk;
+    const int w1 = min(packed_in, w0 + wchunk);
+    const int packed_out = N / PF;
+
+    float acc[MB];
+#pragma unroll
+    for (int m = 0; m < MB; ++m) acc[m] = 0.0f;
+
+    if (n < N) {
+        int last_g = -1;
+        float zp1 = 0.0f, sv = 0.0f;
+        const uint32_t zshift = BITS * (n % PF);
+        for (int iw = w0 + ty; iw < w1; iw += 4) {
+            const int g = (iw * PF) >> gshift;
+            if (g != last_g) {
+                const uint32_t zw = qz[(size_t)g * packed_out + n / PF];
+                zp1 = (float)((zw >> zshift) & MASK) + 1.0f;
+                sv = TT::to_f32(sc[(size_t)g * N + n]);
+                last_g = g;
+            }
+            const uint32_t ww = qw[(size_t)iw * N + n];
+            float w[PF];
+#pragma unroll
+            for (int s = 0; s < PF; ++s) w[s] = sv * ((float)((ww >> (BITS * s)) & MASK) - zp1);
+#pragma unroll
+            for (int m = 0; m < MB; ++m) {
+                if (m < M) {
+                    const uint16_t *xr = x + (size_t)m * K + (size_t)iw * PF;
+#pragma unroll
+                    for (int s = 0; s < PF; ++s) acc[m] = fmaf(TT::to_f32(xr[s]), w[s], acc[m]);
+                }
+            }
+        }
+    }
+    const int n0 = blockIdx.x * 64;
+#pragma unroll
+    for (int m = 0; m < MB; ++m) {
+        if (m < M) {
+            red[ty][tx] = acc[m];
+            __syncthreads();
+            if (ty == 0 && n < N) {
+                const float tot = red[0][tx] + red[1][tx] + red[2][tx] + red[3][tx];
+                if (S == 1) {
+                    const float b = bias ? TT::to_f32(bias[n]) : 0.0f;
+                    y[(size_t)m * N + n] = TT::from_f32(tot + b);
+                } else {
+                    ws[((size_t)slice * M + m) * N + n] = tot;
+                }
+            }
+            __syncthreads();
+        }
+    }
+    if (S > 1 && splitk_arrive(counters, blockIdx.x, S))
+        splitk_finish<TT>(ws, bias, y, M, N, S, n0, 64, 256, threadIdx.x);
+}
+
+// ---------------------------------------------------------------------------
+// Fast 4-bit AWQ kernel.
+//
+// Geometry: a workgroup of WAVES waves owns a slab of LPR*WPL packed words
+// (LPR*WPL*8 output columns) and `gpw` consecutive quantization groups of K.
+// A lane owns WPL consecutive words of a row (one 32*WPL-bit load) and walks
+// row pairs (k, k+1): the low/high 16-bit halves of the two rows' words are
+// interleaved with one v_perm, after which a single AND-OR per slot yields the
+// pair {bias+q[k], bias+q[k+1]} as 16-bit floats, consumed by one dot2 against
+// {x[k], x[k+1]}.  Per group and column the lane then applies
+//     y += s * (acc - (bias + z) * sum_k x[k])
+// which removes both the conversion bias and the zero-point in f32.
+// ---------------------------------------------------------------------------
+template <int WPL> struct WordVec;
+template <> struct WordVec<4> { typedef uint32_t type __attribute__((ext_vector_type(4))); };
+template <> struct WordVec<2> { typedef uint32_t type __attribute__((ext_vector_type(2))); };
+template <> struct WordVec<1> { typedef uint32_t type __attribute__((ext_vector_type(1))); };
+
+template <typename TT, int MB, int WPL, int WAVES, int RPW, int PS>
+__global__ __launch_bounds__(WAVES * 64) void awq4_gemv_fast(
+    const uint16_t *__restrict__ x, const uint32_t *__restrict__ qw,
+    const uint32_t *__restrict__ qz, const uint16_t *__restrict__ sc,
+    const uint16_t *__restrict__ bias, uint16_t *__restrict__ y, float *__restrict__ ws,
+    unsigned *__restrict__ counters, int M, int K, int N, int gshift, int gpw, int S) {
+    typedef typename WordVec<WPL>::type wvec_t;
+    constexpr int LPR = 64 / RPW;          // lanes per row
+    constexpr int NC = WPL * 8;            // columns per lane
+    constexpr int SLAB_COLS = LPR * NC;
+    constexpr int ROWS_PER_CHUNK = 2 * WAVES * RPW * PS;
+    __shared__ float red[WAVES][SLAB_COLS];
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int cl = lane % LPR, sub = lane / LPR;
+    const int PW = N >> 3;                 // words per row
+    const int jw = (blockIdx.x * LPR + cl) * WPL;
+    const bool valid = jw < PW;
+    const int G = K >> gshift;
+    const int slice = blockIdx.y;
+    const int g0 = slice * gpw;
+    const int g1 = min(G, g0 + gpw);
+    const int chunks = (1 << gshift) / ROWS_PER_CHUNK;
+
+    float yacc[MB][NC];
+#pragma unroll
+    for (int m = 0; m < MB; ++m)
+#pragma unroll
+        for (int c = 0; c < NC; ++c) yacc[m][c] = 0.0f;
+
+    if (valid) {
+        for (int g = g0; g < g1; ++g) {
+            const wvec_t zw = *(const wvec_t *)(qz + (size_t)g * PW + jw);
+            float acc[MB][NC];
+            float xs[MB];
+#pragma unroll
+            for (int m = 0; m < MB; ++m) {
+                xs[m] = 0.0f;
+#pragma unroll
+                for (int c = 0; c < NC; ++c) acc[m][c] = 0.0f;
+            }
+            for (int ch = 0; ch < chunks; ++ch) {
+                const int kb = (g << gshift) + ch * ROWS_PER_CHUNK;
+                wvec_t wa[PS], wb[PS];
+                uint32_t xp[MB][PS];
+#pragma unroll
+                for (int t = 0; t < PS; ++t) {
+                    const int r = kb + 2 * (wave * RPW + sub + t * (WAVES * RPW));
+                    wa[t] = *(const wvec_t *)(qw + (size_t)r * PW + jw);
+                    wb[t] = *(const wvec_t *)(qw + (size_t)(r + 1) * PW + jw);
+#pragma unroll
+                    for (int m = 0; m < MB; ++m) {
+                        const int mm = m < M ? m : M - 1;
+                        xp[m][t] = *(const uint32_t *)(x + (size_t)mm * K + r);
+                    }
+                }
+#pragma unroll
+                for (int t = 0; t < PS; ++t) {
+#pragma unroll
+                    for (int c = 0; c < WPL; ++c) {
+                        uint32_t p[8];
+                        TT::unpack4(pack_lo16(wa[t][c], wb[t][c]), p);
+                        TT::unpack4(pack_hi16(wa[t][c], wb[t][c]), p + 4);
+#pragma unroll
+                        for (int m = 0; m < MB; ++m)
+#pragma unroll
+                            for (int s = 0; s < 8; ++s)
+                                acc[m][c * 8 + s] = TT::dot2(p[s], xp[m][t], acc[m][c * 8 + s]);
+                    }
+#pragma unroll
+                    for (int m = 0; m < MB; ++m) xs[m] = TT::dot2(TT::ONES, xp[m][t], xs[m]);
+                }
+            }
+            // group epilogue: remove bias and zero-point, apply the scale
+            const uint16_t *srow = sc + (size_t)g * N + (size_t)jw * 8;
+#pragma unroll
+            for (int c = 0; c < WPL; ++c) {
+                const uint32_t zword = zw[c];
+                const u32x4_t sv = *(const u32x4_t *)(srow + c * 8);  // 8 scales
+#pragma unroll
+                for (int s = 0; s < 8; ++s) {
+                    const int col = awq_slot_col(s);
+                    const uint32_t spair = sv[col >> 1];
+                    const uint16_t sbits = (col & 1) ? (uint16_t)(spair >> 16) : (uint16_t)(spair & 0xFFFFu);
+                    const float scale = TT::to_f32(sbits);
+                    const float zb = (float)((zword >> (4 * s)) & 0xFu) + TT::bias(s);
+#pragma unroll
+                    for (int m = 0; m < MB; ++m) {
+                        const float v = fmaf(-zb, xs[m], acc[m][c * 8 + s]);
+                        yacc[m][c * 8 + s] = fmaf(scale, v, yacc[m][c * 8 + s]);
+                    }
+                }
+            }
+        }
+    }
+
+    // combine the RPW row phases inside the wave, then the waves through LDS
+    const int n0 = blockIdx.x * SLAB_COLS;
+#pragma unroll
+    for (int m = 0; m < MB; ++m) {
+        if (m < M) {
+#pragma unroll
+            for (int c = 0; c < NC; ++c) {
+                float v = yacc[m][c];
+#pragma unroll
+                for (int off = LPR; off < 64; off <<= 1) v += __shfl_xor(v, off, WAVE);
+                yacc[m][c] = v;
+            }
+            if (sub == 0) {
+#pragma unroll
+                for (int c = 0; c < WPL; ++c)
+#pragma unroll
+                    for (int s = 0; s < 8; ++s)
+                        red[wave][cl * NC + c * 8 + awq_slot_col(s)] = yacc[m][c * 8 + s];
+            }
+            __syncthreads();
+            for (int col = threadIdx.x; col < SLAB_COLS; col += WAVES * 64) {
+                const int n = n0 + col;
+                if (n < N) {
+                    float tot = 0.0f;
+#pragma unroll
+                    for (int w = 0; w < WAVES; ++w) tot += red[w][col];
+                    if (S == 1) {
+                        const float b = bias ? TT::to_f32(bias[n]) : 0.0f;
+                        y[(size_t)m * N + n] = TT::from_f32(tot + b);
+                    } else {
+                        ws[((size_t)slice * M + m) * N + n] = tot;
+                    }
+                }
+            }
+            __syncthreads();
+        }
+    }
+    if (S > 1 && splitk_arrive(counters, blockIdx.x, S))
+        splitk_finish<TT>(ws, bias, y, M, N, S, n0, SLAB_COLS, WAVES * 64, threadIdx.x);
+}
+
+// ---------------------------------------------------------------------------
+// Host dispatch
+// ---------------------------------------------------------------------------
+static int env_int(const char *name, int dflt) {
+    const char *v = getenv(name);
+    return (v && *v) ? atoi(v) : dflt;
+}
+
+static int pick_mb(int64_t M) { return M <= 1 ? 1 : (M <= 2 ? 2 : (M <= 4 ? 4 : 8)); }
+
+template <typename TT, int MB, int WPL, int PS>
+static int launch_awq4_fast_t(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p, int gpw, int S) {
+    constexpr int WAVES = 4, RPW = 2;
+    constexpr int LPR = 64 / RPW;
+    const int PW = (int)(p.N / 8);
+    dim3 grid((unsigned)ceil_div(PW, LPR * WPL), (unsigned)S);
+    dim3 block(WAVES * 64);
+    const uint64_t ws_bytes = S > 1 ? (uint64_t)S * p.M * p.N * 4 : 0;
+    char name[64];
+    snprintf(name, sizeof name, "awq4_gemv_fast_%s_m%d_w%d_p%d", TT::DTYPE == 1 ? "f16" : "bf16", MB,
+             WPL, PS);
+    set_plan(ctx, name, grid, block, S, 1, ws_bytes);
+    if (ctx->plan_only) return OXQ_OK;
+    if (ws_bytes > ctx->workspace_bytes || grid.x > ctx->n_counters)
+        return fail(OXQ_ERR_WORKSPACE, "w4a16 gemv: needs %llu workspace bytes, ctx holds %zu",
+                    (unsigned long long)ws_bytes, ctx->workspace_bytes);
+    hipLaunchKernelGGL((awq4_gemv_fast<TT, MB, WPL, WAVES, RPW, PS>), grid, block, 0, s,
+                       (const uint16_t *)p.x, p.qweight, p.qzeros, (const uint16_t *)p.scales,
+                       (const uint16_t *)p.bias, (uint16_t *)p.y, (float *)ctx->workspace,
+                       ctx->counters, (int)p.M, (int)p.K, (int)p.N, p.group_shift, gpw, S);
+    OXQ_HIP_CHECK(hipGetLastError());
+    return OXQ_OK;
+}
+
+template <typename TT>
+static int launch_awq4_fast(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p) {
+    const int mb = pick_mb(p.M);
+    const int wpl = mb == 1 ? 4 : (mb == 2 ? 4 : (mb == 4 ? 2 : 1));
+    const int G = (int)(p.K >> p.group_shift);
+    const int slabs = (int)ceil_div(p.N / 8, 32 * wpl);
+    // enough workgroups for ~2 per CU, whole groups per workgroup
+    int target = env_int("OXQ_GEMV_TARGET_WGS", 2 * ctx->num_cus);
+    int S = (int)ceil_div(target, slabs);
+    if (S > G) S = G;
+    if (S < 1) S = 1;
+    int gpw = (int)ceil_div(G, S);
+    gpw = env_int("OXQ_GEMV_GPW", gpw);
+    S = (int)ceil_div(G, gpw);
+    const bool ps8 = p.group_size >= 128;
+#define OXQ_CASE(MBv, WPLv)                                                          \
+    if (mb == MBv && wpl == WPLv)                                                    \
+        return ps8 ? launch_awq4_fast_t<TT, MBv, WPLv, 8>(ctx, s, p, gpw, S)         \
+                   : launch_awq4_fast_t<TT, MBv, WPLv, 4>(ctx, s, p, gpw, S);
+    OXQ_CASE(1, 4)
+    OXQ_CASE(2, 4)
+    OXQ_CASE(4, 2)
+    OXQ_CASE(8, 1)
+#undef OXQ_CASE
+    return fail(OXQ_ERR_UNSUPPORTED, "w4a16 gemv: no kernel for m=%lld", (long long)p.M);
+}
+
+static bool awq4_fast_ok(const Wna16Problem &p) {
+    if (p.bits != 4 || p.pack_dim != OXQ_PACK_OUT) return false;
+    if (p.N % 32 != 0 || p.K % 2 != 0) return false;
+    if (p.group_size < 64) return false;  // 2 * WAVES * RPW * PS rows per chunk
+    if (((uintptr_t)p.qweight | (uintptr_t)p.qzeros | (uintptr_t)p.scales) & 15) return false;
+    if ((uintptr_t)p.x & 3) return false;
+    return true;
+}
+
+template <typename TT, int BITS>
+static int launch_generic_t(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p) {
+    constexpr int PF = 32 / BITS;
+    const int mb = pick_mb(p.M);
+    const bool awq = p.pack_dim == OXQ_PACK_OUT;
+    const int tiles = awq ? (int)ceil_div(p.N / PF, 64) : (int)ceil_div(p.N, 64);
+    const int64_t units = awq ? p.K : p.K / PF;  // rows (AWQ) or word rows (GPTQ) to split
+    int S = (int)ceil_div(2 * ctx->num_cus, tiles);
+    // keep whole groups per slice so each slice reloads scales rarely
+    const int64_t unit_group = awq ? p.group_size : (p.group_size / PF > 0 ? p.group_size / PF : 1);
+    int64_t chunk = ceil_div(units, S);
+    chunk = ceil_div(chunk, unit_group) * unit_group;
+    if (chunk < 4) chunk = 4;
+    S = (int)ceil_div(units, chunk);
+    dim3 grid((unsigned)tiles, (unsigned)S), block(256);
+    const uint64_t ws_bytes = S > 1 ? (uint64_t)S * p.M * p.N * 4 : 0;
+    char name[64];
+    snprintf(name, sizeof name, "%s_gemv_generic_w%d_%s_m%d", awq ? "awq" : "gptq", BITS,
+             TT::DTYPE == 1 ? "f16" : "bf16", mb);
+    set_plan(ctx, name, grid, block, S, 1, ws_bytes);
+    if (ctx->plan_only) return OXQ_OK;
+    if (ws_bytes > ctx->workspace_bytes || grid.x > ctx->n_counters)
+        return fail(OXQ_ERR_WORKSPACE, "wna16 gemv: needs %llu workspace bytes, ctx holds %zu",
+                    (unsigned long long)ws_bytes, ctx->workspace_bytes);
+#define OXQ_GO(MBv)                                                                              \
+    if (awq)                                                                                     \
+        hipLaunchKernelGGL((awq_gemv_generic<TT, BITS, MBv>), grid, block, 0, s,                 \
+                           (const uint16_t *)p.x, p.qweight, p.qzeros, (const uint16_t *)p.scales, \
+                           (const uint16_t *)p.bias, (uint16_t *)p.y, (float *)ctx->workspace,   \
+                           ctx->counters, (int)p.M, (int)p.K, (int)p.N, (int)(p.N / PF),         \
+                           p.group_shift, (int)chunk, S);                                        \
+    else                                                                                         \
+        hipLaunchKernelGGL((gptq_gemv_generic<TT, BITS, MBv>), grid, block, 0, s,                \
+                           (const uint16_t *)p.x, p.qweight, p.qzeros, (const uint16_t *)p.scales, \
+                           (const uint16_t *)p.bias, (uint16_t *)p.y, (float *)ctx->workspace,   \
+                           ctx->counters, (int)p.M, (int)p.K, (int)p.N, p.group_shift, (int)chunk, S)
+    switch (mb) {
+    case 1: OXQ_GO(1); break;
+    case 2: OXQ_GO(2); break;
+    case 4: OXQ_GO(4); break;
+    default: OXQ_GO(8); break;
+    }
+#undef OXQ_GO
+    OXQ_HIP_CHECK(hipGetLastError());
+    return OXQ_OK;
+}
+
+int launch_wna16_gemv(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p) {
+    const bool f16 = p.dtype == OXQ_F16;
+    if (awq4_fast_ok(p) && !env_int("OXQ_FORCE_GENERIC", 0))
+        return f16 ? launch_awq4_fast<F16Traits>(ctx, s, p) : launch_awq4_fast<BF16Traits>(ctx, s, p);
+    if (p.bits == 4)
+        return f16 ? launch_generic_t<F16Traits, 4>(ctx, s, p) : launch_generic_t<BF16Traits, 4>(ctx, s, p);
+    return f16 ? launch_generic_t<F16Traits, 8>(ctx, s, p) : launch_generic_t<BF16Traits, 8>(ctx, s, p);
+}
+
+}  // namespace oxq

@@ -1,0 +1,353 @@
+"""Torch-facing binding of the C ABI, named after the reference's op functions
+(``src/common/metal_ops.rs``) and layer types (``src/common/linear.rs``,
+``src/common/mxfp4.rs``).
+
+torch is plumbing only: it owns device memory and the current stream.  All
+validation, routing and compute happen behind the C ABI; this module builds
+descriptors, allocates the output the reference op would have allocated, and
+raises :class:`OxqError` with the library's message on failure.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Optional
+
+import torch
+
+from . import _lib
+from ._lib import (BF16, F16, F32, GGUF_Q4_0, GGUF_Q4_K, GGUF_Q6_K, GGUF_Q8_0, I32, I64, PACK_IN,
+                   PACK_OUT, U8, U32, OxqError, OxqPlan, OxqTensor)
+
+_DTYPES = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16, torch.uint8: U8,
+           torch.int32: I32, torch.int64: I64}
+if hasattr(torch, "uint32"):
+    _DTYPES[torch.uint32] = U32
+_TORCH_OF = {F32: torch.float32, F16: torch.float16, BF16: torch.bfloat16}
+
+
+def desc(t: Optional[torch.Tensor]):
+    """Tensor -> pointer to an oxq_tensor descriptor (None -> NULL)."""
+    if t is None:
+        return None
+    if isinstance(t, OxqTensor):
+        return C.byref(t)
+    if t.dtype not in _DTYPES:
+        raise OxqError(-2, f"unsupported torch dtype {t.dtype}")
+    if t.dim() < 1 or t.dim() > _lib.OXQ_MAX_RANK:
+        raise OxqError(-3, f"rank {t.dim()} out of [1, {_lib.OXQ_MAX_RANK}]")
+    d = OxqTensor()
+    d.data = t.data_ptr()
+    d.dtype = _DTYPES[t.dtype]
+    d.rank = t.dim()
+    for i, s in enumerate(t.shape):
+        d.dims[i] = s
+    d.contiguous = 1 if t.is_contiguous() else 0
+    d.device = t.device.index if t.device.type == "cuda" else _lib.DEVICE_HOST
+    if t.device.type == "cuda" and d.device is None:
+        d.device = torch.cuda.current_device()
+    return C.byref(d)
+
+
+class Context:
+    """One per engine thread / stream (owns the split-K workspace)."""
+
+    def __init__(self, device: Optional[int] = None, plan_only: bool = False):
+        self._lib = _lib.load()
+        self.handle = C.c_void_p()
+        if plan_only:
+            dev = _lib.DEVICE_PLAN_ONLY
+        else:
+            dev = torch.cuda.current_device() if device is None else device
+        _lib.check(self._lib.oxq_ctx_create(dev, C.byref(self.handle)))
+        self.device = dev
+        self.plan_only = plan_only
+
+    def close(self):
+        if self.handle:
+            self._lib.oxq_ctx_destroy(self.handle)
+            self.handle = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def last_plan(self) -> dict:
+        p = OxqPlan()
+        _lib.check(self._lib.oxq_ctx_last_plan(self.handle, C.byref(p)))
+        return {"kernel": p.kernel.decode(), "grid": tuple(p.grid), "block": tuple(p.block),
+                "split_k": p.split_k, "launches": p.launches, "workspace_bytes": p.workspace_bytes}
+
+    def stream(self) -> int:
+        if self.plan_only:
+            return 0
+        return torch.cuda.current_stream().cuda_stream
+
+
+_default_ctx: dict = {}
+
+
+def default_context() -> Context:
+    dev = torch.cuda.current_device()
+    if dev not in _default_ctx:
+        _default_ctx[dev] = Context(dev)
+    return _default_ctx[dev]
+
+
+def _ctx(ctx: Optional[Context]) -> Context:
+    return ctx if ctx is not None else default_context()
+
+
+def _out_for(x: torch.Tensor, n: int, out, ctx):
+    if out is not None:
+        return out
+    return torch.empty((x.shape[0], n), dtype=x.dtype, device=x.device)
+
+
+# ---------------------------------------------------------------- AWQ / GPTQ ops
+def w4a16_matmul(x, qweight, qzeros, scales, *, out=None, ctx: Optional[Context] = None):
+    """metal_ops.rs:1821.  x [m,K] (m in 1..=8) -> [m,N] in x's dtype."""
+    ctx = _ctx(ctx)
+    out = _out_for(x, scales.shape[1], out, ctx)
+    _lib.check(ctx._lib.oxq_w4a16_matmul(ctx.handle, ctx.stream(), desc(x), desc(qweight),
+                                         desc(qzeros), desc(scales), desc(out)))
+    return out
+
+
+def w8a16_matmul(x, qweight, qzeros, scales, *, out=None, ctx: Optional[Context] = None):
+    """metal_ops.rs:1835."""
+    ctx = _ctx(ctx)
+    out = _out_for(x, scales.shape[1], out, ctx)
+    _lib.check(ctx._lib.oxq_w8a16_matmul(ctx.handle, ctx.stream(), desc(x), desc(qweight),
+                                         desc(qzeros), desc(scales), desc(out)))
+    return out
+
+
+def gptq_matmul(x, qweight, qzeros, scales, bits: int, *, out=None, ctx: Optional[Context] = None):
+    """metal_ops.rs:2281."""
+    ctx = _ctx(ctx)
+    out = _out_for(x, scales.shape[1], out, ctx)
+    _lib.check(ctx._lib.oxq_gptq_matmul(ctx.handle, ctx.stream(), desc(x), desc(qweight),
+                                        desc(qzeros), desc(scales), bits, desc(out)))
+    return out
+
+
+def _dequant_out(qweight, scales, bits, pack_dim, out):
+    if out is not None:
+        return out
+    pf = 32 // bits if bits in (4, 8) else 8
+    k = qweight.shape[0] if pack_dim == PACK_OUT else qweight.shape[0] * pf
+    return torch.empty((k, scales.shape[1]), dtype=scales.dtype, device=scales.device)
+
+
+def dequantize_w4(qweight, qzeros, scales, *, out=None, ctx: Optional[Context] = None):
+    """metal_ops.rs:1873 -> dense [K,N] in the scales' dtype."""
+    ctx = _ctx(ctx)
+    out = _dequant_out(qweight, scales, 4, PACK_OUT, out)
+    _lib.check(ctx._lib.oxq_dequantize_w4(ctx.handle, ctx.stream(), desc(qweight), desc(qzeros),
+                                          desc(scales), desc(out)))
+    return out
+
+
+def dequantize_w8(qweight, qzeros, scales, *, out=None, ctx: Optional[Context] = None):
+    """metal_ops.rs:1886."""
+    ctx = _ctx(ctx)
+    out = _dequant_out(qweight, scales, 8, PACK_OUT, out)
+    _lib.check(ctx._lib.oxq_dequantize_w8(ctx.handle, ctx.stream(), desc(qweight), desc(qzeros),
+                                          desc(scales), desc(out)))
+    return out
+
+
+def dequantize_gptq_packed(qweight, qzeros, scales, bits: int, *, out=None,
+                           ctx: Optional[Context] = None):
+    """metal_ops.rs:2305."""
+    ctx = _ctx(ctx)
+    out = _dequant_out(qweight, scales, bits, PACK_IN, out)
+    _lib.check(ctx._lib.oxq_dequantize_gptq_packed(ctx.handle, ctx.stream(), desc(qweight),
+                                                   desc(qzeros), desc(scales), bits, desc(out)))
+    return out
+
+
+def mpp_quant_matmul(x, qweight, qzeros, scales, bits: int, pack_dim: int, *, out=None,
+                     ctx: Optional[Context] = None):
+    """metal_ops.rs:2748: tile GEMM on the matrix cores, any m."""
+    ctx = _ctx(ctx)
+    out = _out_for(x, scales.shape[1], out, ctx)
+    _lib.check(ctx._lib.oxq_mpp_quant_matmul(ctx.handle, ctx.stream(), desc(x), desc(qweight),
+                                             desc(qzeros), desc(scales), bits, pack_dim, desc(out)))
+    return out
+
+
+def maybe_mpp_quant_matmul(x, qweight, qzeros, scales, bits: int, pack_dim: int, *,
+                           ctx: Optional[Context] = None):
+    """metal_ops.rs:2771: returns None when the op declines (small m, wrong dtype...)."""
+    ctx = _ctx(ctx)
+    out = _out_for(x, scales.shape[1], None, ctx)
+    taken = C.c_int(0)
+    _lib.check(ctx._lib.oxq_maybe_mpp_quant_matmul(ctx.handle, ctx.stream(), desc(x), desc(qweight),
+                                                   desc(qzeros), desc(scales), bits, pack_dim,
+                                                   desc(out), C.byref(taken)))
+    return out if taken.value else None
+
+
+# ---------------------------------------------------------------- GGUF
+def gguf_block_layout(quant: int):
+    e, b = C.c_int64(), C.c_int64()
+    _lib.check(_lib.load().oxq_gguf_block_layout(quant, C.byref(e), C.byref(b)))
+    return e.value, b.value
+
+
+def gguf_quant_matmul(x, weight_bytes, in_features: int, out_features: int, quant: int, *,
+                      out=None, ctx: Optional[Context] = None):
+    """metal_ops.rs:5819 (1 <= m <= 8)."""
+    ctx = _ctx(ctx)
+    out = _out_for(x, out_features, out, ctx)
+    _lib.check(ctx._lib.oxq_gguf_quant_matmul(ctx.handle, ctx.stream(), desc(x), desc(weight_bytes),
+                                              in_features, out_features, quant, desc(out)))
+    return out
+
+
+def gguf_quant_mul_mm(x, weight_bytes, in_features: int, out_features: int, quant: int, *,
+                      out=None, ctx: Optional[Context] = None):
+    """metal_ops.rs:5973 (any m)."""
+    ctx = _ctx(ctx)
+    out = _out_for(x, out_features, out, ctx)
+    _lib.check(ctx._lib.oxq_gguf_quant_mul_mm(ctx.handle, ctx.stream(), desc(x), desc(weight_bytes),
+                                              in_features, out_features, quant, desc(out)))
+    return out
+
+
+def gguf_dequantize(weight_bytes, in_features: int, out_features: int, quant: int, *,
+                    ctx: Optional[Context] = None):
+    ctx = _ctx(ctx)
+    out = torch.empty((out_features, in_features), dtype=torch.float32, device=weight_bytes.device)
+    _lib.check(ctx._lib.oxq_gguf_dequantize(ctx.handle, ctx.stream(), desc(weight_bytes),
+                                            in_features, out_features, quant, desc(out)))
+    return out
+
+
+# ---------------------------------------------------------------- MXFP4
+def mxfp4_matmul(x, blocks, scales, k: int, n: int, *, out=None, ctx: Optional[Context] = None):
+    """metal_ops.rs:6197."""
+    ctx = _ctx(ctx)
+    out = _out_for(x, n, out, ctx)
+    _lib.check(ctx._lib.oxq_mxfp4_matmul(ctx.handle, ctx.stream(), desc(x), desc(blocks),
+                                         desc(scales), k, n, desc(out)))
+    return out
+
+
+def mxfp4_dequantize(blocks, scales, k: int, n: int, *, ctx: Optional[Context] = None):
+    ctx = _ctx(ctx)
+    out = torch.empty((n, k), dtype=torch.float32, device=blocks.device)
+    _lib.check(ctx._lib.oxq_mxfp4_dequantize(ctx.handle, ctx.stream(), desc(blocks), desc(scales),
+                                             k, n, desc(out)))
+    return out
+
+
+def mxfp4_moe_matmul(x, blocks, scales, bias, expert_offsets, token_ids, k: int, n: int, *,
+                     out=None, ctx: Optional[Context] = None):
+    """Grouped expert GEMV: out[p] = x[row(p)] . W_e^T + bias_e for every routed pair."""
+    ctx = _ctx(ctx)
+    gather = token_ids is not None
+    n_pairs = token_ids.numel() if gather else x.shape[0]
+    if out is None:
+        out = torch.empty((n_pairs, n), dtype=x.dtype, device=x.device)
+    _lib.check(ctx._lib.oxq_mxfp4_moe_matmul(ctx.handle, ctx.stream(), desc(x), desc(blocks),
+                                             desc(scales), desc(bias), desc(expert_offsets),
+                                             desc(token_ids), 1 if gather else 0, k, n, desc(out)))
+    return out
+
+
+# ---------------------------------------------------------------- layers
+class PackedQuantLinear:
+    """linear.rs:403-534.  Holds resident packed weights; routes by m."""
+
+    def __init__(self, bits: int, pack_dim: int, qweight, qzeros, scales, bias=None,
+                 dtype=torch.float16, ctx: Optional[Context] = None):
+        self.ctx = _ctx(ctx)
+        self._keep = (qweight, qzeros, scales, bias)
+        self.handle = C.c_void_p()
+        _lib.check(self.ctx._lib.oxq_packed_quant_linear_new(
+            self.ctx.handle, bits, pack_dim, desc(qweight), desc(qzeros), desc(scales), desc(bias),
+            _DTYPES[dtype], C.byref(self.handle)))
+        k, n = C.c_int64(), C.c_int64()
+        self.ctx._lib.oxq_packed_quant_linear_in_features(self.handle, C.byref(k))
+        self.ctx._lib.oxq_packed_quant_linear_out_features(self.handle, C.byref(n))
+        self.in_features, self.out_features = k.value, n.value
+
+    def forward(self, x: torch.Tensor, out=None) -> torch.Tensor:
+        if out is None:
+            out = torch.empty(tuple(x.shape[:-1]) + (self.out_features,), dtype=x.dtype,
+                              device=x.device)
+        _lib.check(self.ctx._lib.oxq_packed_quant_linear_forward(self.handle, self.ctx.stream(),
+                                                                 desc(x), desc(out)))
+        return out
+
+    def __del__(self):
+        try:
+            if self.handle:
+                self.ctx._lib.oxq_packed_quant_linear_free(self.handle)
+                self.handle = C.c_void_p()
+        except Exception:
+            pass
+
+
+class QLinear:
+    """linear.rs:179-393 (GGUF fast path)."""
+
+    def __init__(self, quant: int, weight_bytes, in_features: int, out_features: int, bias=None,
+                 out_dtype=torch.bfloat16, ctx: Optional[Context] = None):
+        self.ctx = _ctx(ctx)
+        self._keep = (weight_bytes, bias)
+        self.handle = C.c_void_p()
+        self.out_features = out_features
+        _lib.check(self.ctx._lib.oxq_qlinear_new(
+            self.ctx.handle, quant, desc(weight_bytes), in_features, out_features, desc(bias),
+            _DTYPES[out_dtype], C.byref(self.handle)))
+
+    def forward(self, x: torch.Tensor, out=None) -> torch.Tensor:
+        if out is None:
+            out = torch.empty(tuple(x.shape[:-1]) + (self.out_features,), dtype=x.dtype,
+                              device=x.device)
+        _lib.check(self.ctx._lib.oxq_qlinear_forward(self.handle, self.ctx.stream(), desc(x),
+                                                     desc(out)))
+        return out
+
+    def __del__(self):
+        try:
+            if self.handle:
+                self.ctx._lib.oxq_qlinear_free(self.handle)
+                self.handle = C.c_void_p()
+        except Exception:
+            pass
+
+
+class Mxfp4Linear:
+    """mxfp4.rs:67-169."""
+
+    def __init__(self, blocks, scales, bias, in_features: int, out_features: int,
+                 ctx: Optional[Context] = None):
+        self.ctx = _ctx(ctx)
+        self._keep = (blocks, scales, bias)
+        self.handle = C.c_void_p()
+        self.out_features = out_features
+        _lib.check(self.ctx._lib.oxq_mxfp4_linear_new(
+            self.ctx.handle, desc(blocks), desc(scales), desc(bias), in_features, out_features,
+            C.byref(self.handle)))
+
+    def forward(self, x: torch.Tensor, out=None) -> torch.Tensor:
+        if out is None:
+            out = torch.empty(tuple(x.shape[:-1]) + (self.out_features,), dtype=x.dtype,
+                              device=x.device)
+        _lib.check(self.ctx._lib.oxq_mxfp4_linear_forward(self.handle, self.ctx.stream(), desc(x),
+                                                          desc(out)))
+        return out
+
+    def __del__(self):
+        try:
+            if self.handle:
+                self.ctx._lib.oxq_mxfp4_linear_free(self.handle)
+                self.handle = C.c_void_p()
+        except Exception:
+            pass

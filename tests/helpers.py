@@ -1,0 +1,60 @@
+"""Shared helpers for the parity tests."""
+import numpy as np
+import torch
+
+import oracle
+from oxydllm_amd import _lib
+
+TORCH_DT = {oracle.F16: torch.float16, oracle.BF16: torch.bfloat16, oracle.F32: torch.float32}
+
+# north-star tolerance: 2e-3 relative / 1e-2 absolute of the f32-accumulated reference
+RTOL, ATOL = 2e-3, 1e-2
+
+
+def fake(shape, dtype, device=0, contiguous=True):
+    """Descriptor of a tensor that is never dereferenced (plan-only contexts)."""
+    d = _lib.OxqTensor()
+    d.data = 0
+    d.dtype = dtype
+    d.rank = len(shape)
+    for i, s in enumerate(shape):
+        d.dims[i] = s
+    d.contiguous = 1 if contiguous else 0
+    d.device = device
+    return d
+
+
+def to_dev(a: np.ndarray, dtype=None):
+    t = torch.from_numpy(np.ascontiguousarray(a))
+    if dtype is not None:
+        t = t.to(dtype)
+    return t.cuda()
+
+
+def bits_of(t: torch.Tensor) -> np.ndarray:
+    """Raw 16-bit patterns of an f16/bf16 tensor (uint16), or the f32 array."""
+    t = t.detach().cpu().contiguous()
+    if t.dtype in (torch.float16, torch.bfloat16):
+        return t.view(torch.int16).numpy().view(np.uint16)
+    return t.numpy()
+
+
+def as_f32(t: torch.Tensor) -> np.ndarray:
+    return t.detach().float().cpu().numpy()
+
+
+def assert_close(got: np.ndarray, ref: np.ndarray, what="", rtol=RTOL, atol=ATOL):
+    got = np.asarray(got, dtype=np.float64)
+    ref = np.asarray(ref, dtype=np.float64)
+    assert got.shape == ref.shape, f"{what}: shape {got.shape} != {ref.shape}"
+    assert np.all(np.isfinite(got)), f"{what}: non-finite output"
+    err = np.abs(got - ref)
+    bound = atol + rtol * np.abs(ref)
+    bad = err > bound
+    assert not bad.any(), (f"{what}: {bad.sum()} of {bad.size} outside {rtol} rel / {atol} abs; "
+                           f"max err {err.max():.3e} at ref {ref.flat[err.argmax()]:.4f}")
+
+
+def round_x(x_f32: np.ndarray, dt: int) -> np.ndarray:
+    """The activation values the kernel actually sees (x rounded to its 16-bit dtype)."""
+    return oracle.round_through(x_f32, dt)

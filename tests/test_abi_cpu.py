@@ -1,0 +1,308 @@
+"""No-GPU tests of the C ABI: the library loads, exports every declared symbol,
+and its device-free validation layer rejects what the reference rejects
+(metal_ops.rs:1507-1566, 1984-2044, 5357-5431, 6011-6058; awq.rs:1096-1121;
+metal_ops.rs:3943-3958) before anything would be launched.
+"""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+from oxydllm_amd import _lib
+from tests.helpers import fake
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+F16, BF16, F32, U8, I32, I64 = _lib.F16, _lib.BF16, _lib.F32, _lib.U8, _lib.I32, _lib.I64
+
+
+@pytest.fixture(scope="module")
+def lib():
+    return _lib.load()
+
+
+@pytest.fixture()
+def ctx(lib):
+    h = C.c_void_p()
+    assert lib.oxq_ctx_create(_lib.DEVICE_PLAN_ONLY, C.byref(h)) == 0
+    yield h
+    lib.oxq_ctx_destroy(h)
+
+
+def err(lib):
+    return lib.oxq_last_error().decode()
+
+
+def plan(lib, ctx):
+    p = _lib.OxqPlan()
+    assert lib.oxq_ctx_last_plan(ctx, C.byref(p)) == 0
+    return p
+
+
+def test_library_exports_every_declared_symbol(lib):
+    header = open(os.path.join(ROOT, "include", "oxq.h")).read()
+    declared = set(re.findall(r"\b(oxq_[a-z0-9_]+)\s*\(", header))
+    assert len(declared) >= 30
+    missing = [n for n in sorted(declared) if not hasattr(lib, n)]
+    assert not missing, f"not exported: {missing}"
+    assert declared == set(_lib.SIGNATURES), "binding table out of sync with include/oxq.h"
+
+
+def test_version_and_status_names(lib):
+    a, b = C.c_int(-1), C.c_int(-1)
+    lib.oxq_version(C.byref(a), C.byref(b))
+    assert (a.value, b.value) == (0, 1)
+    assert lib.oxq_status_name(-5) == b"OXQ_ERR_M_RANGE"
+    for code, name in _lib.STATUS.items():
+        assert lib.oxq_status_name(code).decode() == name
+
+
+def test_gguf_block_layout_matches_reference(lib):
+    """metal_ops.rs:5228-5241."""
+    want = {_lib.GGUF_Q4_0: (32, 18), _lib.GGUF_Q8_0: (32, 34), _lib.GGUF_Q4_K: (256, 144),
+            _lib.GGUF_Q6_K: (256, 210)}
+    for q, (e, b) in want.items():
+        ee, bb = C.c_int64(), C.c_int64()
+        assert lib.oxq_gguf_block_layout(q, C.byref(ee), C.byref(bb)) == 0
+        assert (ee.value, bb.value) == (e, b)
+    assert lib.oxq_gguf_block_layout(17, None, None) == -1
+
+
+def _awq(K, N, g, dt=F16, bits=4):
+    pf = 32 // bits
+    return (fake((K, N // pf), I32), fake((K // g, N // pf), I32), fake((K // g, N), dt))
+
+
+def test_w4a16_accepts_valid_and_reports_plan(lib, ctx):
+    qw, qz, sc = _awq(4096, 14336, 128)
+    x, out = fake((1, 4096), F16), fake((1, 14336), F16)
+    assert lib.oxq_w4a16_matmul(ctx, None, C.byref(x), C.byref(qw), C.byref(qz), C.byref(sc),
+                                C.byref(out)) == 0, err(lib)
+    p = plan(lib, ctx)
+    assert p.kernel.decode().startswith("awq4_gemv_fast_f16_m1")
+    assert p.block[0] == 256 and p.grid[0] == 14 and p.split_k == p.grid[1] >= 1
+    assert p.workspace_bytes == (p.split_k * 14336 * 4 if p.split_k > 1 else 0)
+    # odd shape falls to the generic kernel (N not a multiple of 32)
+    qw, qz, sc = _awq(192, 104, 64)
+    x, out = fake((3, 192), BF16), fake((3, 104), BF16)
+    sc.dtype = BF16
+    assert lib.oxq_w4a16_matmul(ctx, None, C.byref(x), C.byref(qw), C.byref(qz), C.byref(sc),
+                                C.byref(out)) == 0, err(lib)
+    assert "awq_gemv_generic_w4_bf16_m4" in plan(lib, ctx).kernel.decode()
+
+
+def test_w4a16_rejects_host_tensors(lib, ctx):
+    """metal_ops.rs:3943-3958 w4a16_matmul_rejects_cpu_tensors."""
+    qw, qz, sc = _awq(64, 64, 32)
+    x, out = fake((1, 64), F16, device=_lib.DEVICE_HOST), fake((1, 64), F16)
+    rc = lib.oxq_w4a16_matmul(ctx, None, C.byref(x), C.byref(qw), C.byref(qz), C.byref(sc), C.byref(out))
+    assert rc == -7 and "GPU-resident" in err(lib)
+
+
+@pytest.mark.parametrize("m", [0, 9, 64])
+def test_gemv_m_range(lib, ctx, m):
+    qw, qz, sc = _awq(256, 128, 64)
+    x, out = fake((m, 256), F16), fake((m, 128), F16)
+    rc = lib.oxq_w4a16_matmul(ctx, None, C.byref(x), C.byref(qw), C.byref(qz), C.byref(sc), C.byref(out))
+    assert rc == -5 and "m in 1..=8" in err(lib)
+    g = (fake((256 // 8, 128), I32), fake((4, 128 // 8), I32), fake((4, 128), F16))
+    rc = lib.oxq_gptq_matmul(ctx, None, C.byref(x), C.byref(g[0]), C.byref(g[1]), C.byref(g[2]), 4,
+                             C.byref(out))
+    assert rc == -5
+
+
+def test_wna16_validation_errors(lib, ctx):
+    K, N, g = 256, 128, 64
+    qw, qz, sc = _awq(K, N, g)
+    x, out = fake((1, K), F16), fake((1, N), F16)
+
+    def call(x=x, qw=qw, qz=qz, sc=sc, out=out):
+        return lib.oxq_w4a16_matmul(ctx, None, C.byref(x), C.byref(qw), C.byref(qz), C.byref(sc),
+                                    C.byref(out))
+
+    assert call() == 0
+    assert call(x=fake((1, K), F16, contiguous=False)) == -4 and "contiguous" in err(lib)
+    assert call(x=fake((K,), F16)) == -3
+    assert call(qz=fake((K // g, N // 8 + 1), I32)) == -3 and "qzeros shape" in err(lib)
+    assert call(qw=fake((K, N // 8 - 1), I32), qz=fake((K // g, N // 8 - 1), I32)) == -3
+    assert "packed_out" in err(lib)
+    assert call(x=fake((1, K + 32), F16)) == -3 and "in_features" in err(lib)
+    assert call(out=fake((1, N + 8), F16)) == -3 and "output shape" in err(lib)
+    assert call(x=fake((1, K), BF16)) == -2 and "must match x dtype" in err(lib)
+    assert call(x=fake((1, K), F32), sc=fake((K // g, N), F32), out=fake((1, N), F32)) == -2
+    assert "unsupported (bits, dtype) combo" in err(lib)
+    assert call(qw=fake((K, N // 8), I64)) == -2
+    # 3 groups of 85.33: not divisible
+    assert call(qz=fake((3, N // 8), I32), sc=fake((3, N), F16)) == -6 and "not divisible" in err(lib)
+    # group size 96 (K=288): not a power of two
+    qw2, qz2, sc2 = _awq(288, N, 96)
+    assert call(x=fake((1, 288), F16), qw=qw2, qz=qz2, sc=sc2) == -6 and "power of two" in err(lib)
+    assert lib.oxq_w4a16_matmul(None, None, C.byref(x), C.byref(qw), C.byref(qz), C.byref(sc),
+                                C.byref(out)) == -1
+    assert lib.oxq_w4a16_matmul(ctx, None, None, C.byref(qw), C.byref(qz), C.byref(sc), C.byref(out)) == -1
+
+
+def test_awq_shape_rejection_from_reference(lib, ctx):
+    """awq.rs:1096-1121: qweight [8,2], qzeros [2,2], scales [2,8]."""
+    qw, qz, sc = fake((8, 2), I32), fake((2, 2), I32), fake((2, 8), F16)
+    out = fake((8, 8), F16)
+    assert lib.oxq_dequantize_w4(ctx, None, C.byref(qw), C.byref(qz), C.byref(sc), C.byref(out)) == -3
+
+
+def test_gptq_validation(lib, ctx):
+    K, N, g = 5120, 13824, 128
+    for bits in (4, 8):
+        pf = 32 // bits
+        qw, qz, sc = fake((K // pf, N), I32), fake((K // g, N // pf), I32), fake((K // g, N), BF16)
+        x, out = fake((8, K), BF16), fake((8, N), BF16)
+        assert lib.oxq_gptq_matmul(ctx, None, C.byref(x), C.byref(qw), C.byref(qz), C.byref(sc), bits,
+                                   C.byref(out)) == 0, err(lib)
+        assert f"gptq_gemv_generic_w{bits}_bf16_m8" in plan(lib, ctx).kernel.decode()
+        bad = fake((K // g, N // pf + 1), I32)
+        assert lib.oxq_gptq_matmul(ctx, None, C.byref(x), C.byref(qw), C.byref(bad), C.byref(sc),
+                                   bits, C.byref(out)) == -3
+        w = fake((K, N), BF16)
+        assert lib.oxq_dequantize_gptq_packed(ctx, None, C.byref(qw), C.byref(qz), C.byref(sc), bits,
+                                              C.byref(w)) == 0
+    assert lib.oxq_gptq_matmul(ctx, None, C.byref(x), C.byref(qw), C.byref(qz), C.byref(sc), 3,
+                               C.byref(out)) == -8
+    assert "bits must be 4 or 8" in err(lib)
+    qw_bad = fake((K // 8, N + 8), I32)
+    assert lib.oxq_gptq_matmul(ctx, None, C.byref(x), C.byref(qw_bad), C.byref(qz), C.byref(sc), 8,
+                               C.byref(out)) == -3 and "qweight dim1" in err(lib)
+
+
+def test_maybe_mpp_declines_like_reference(lib, ctx):
+    """metal_ops.rs:2779-2791: small m, wrong dtype, non-contiguous -> Ok(None)."""
+    qw, qz, sc = _awq(4096, 14336, 128)
+    taken = C.c_int(7)
+
+    def call(x, out, sc=sc):
+        return lib.oxq_maybe_mpp_quant_matmul(ctx, None, C.byref(x), C.byref(qw), C.byref(qz),
+                                              C.byref(sc), 4, _lib.PACK_OUT, C.byref(out),
+                                              C.byref(taken))
+
+    assert call(fake((4, 4096), F16), fake((4, 14336), F16)) == 0 and taken.value == 0
+    assert call(fake((64, 4096), F32), fake((64, 14336), F32)) == 0 and taken.value == 0
+    assert call(fake((64, 4096), F16, contiguous=False), fake((64, 14336), F16)) == 0
+    assert taken.value == 0
+    assert call(fake((64, 4096), F16), fake((64, 14336), F16)) == 0 and taken.value == 1
+    p = plan(lib, ctx)
+    assert p.kernel.decode() == "awq4_mfma_f16_mt4" and p.grid[0] == 28 and p.grid[2] == 1
+    assert call(fake((16, 4096), F16), fake((16, 14336), F16)) == 0 and taken.value == 1
+    assert plan(lib, ctx).kernel.decode() == "awq4_mfma_f16_mt1"
+    # a real error is still an error
+    assert call(fake((64, 4000), F16), fake((64, 14336), F16)) == -3 and taken.value == 0
+
+
+def test_gguf_validation(lib, ctx):
+    K, N = 4096, 4096
+    for q, (be, bb) in {_lib.GGUF_Q4_0: (32, 18), _lib.GGUF_Q6_K: (256, 210)}.items():
+        w = fake((N * (K // be) * bb,), U8)
+        x, out = fake((1, K), BF16), fake((1, N), BF16)
+
+        def call(x=x, w=w, out=out, k=K, n=N, fn=lib.oxq_gguf_quant_matmul):
+            return fn(ctx, None, C.byref(x), C.byref(w), k, n, q, C.byref(out))
+
+        assert call() == 0, err(lib)
+        assert call(x=fake((1, K), F32), out=fake((1, N), F32)) == 0, err(lib)
+        assert call(x=fake((1, K), F16), out=fake((1, N), F16)) == -2 and "BF16" in err(lib)
+        assert call(w=fake((N * (K // be) * bb,), I32)) == -2 and "U8" in err(lib)
+        assert call(k=K + 8, x=fake((1, K + 8), BF16)) == -3 and "multiple of" in err(lib)
+        assert call(x=fake((9, K), BF16), out=fake((9, N), BF16)) == -5 and "out of [1, 8]" in err(lib)
+        assert call(x=fake((9, K), BF16), out=fake((9, N), BF16), fn=lib.oxq_gguf_quant_mul_mm) == 0
+        assert call(x=fake((1, K), BF16, contiguous=False)) == -4
+        assert call(x=fake((1, K - 256), BF16)) == -3 and "x shape" in err(lib)
+        assert call(out=fake((1, N - 1), BF16)) == -3 and "output shape" in err(lib)
+        assert call(w=fake((N * (K // be) * bb - bb,), U8)) == -3 and "expected" in err(lib)
+        assert call(x=fake((1, K), BF16, device=_lib.DEVICE_HOST)) == -7
+    # odd N (reference tests n in {1001, 49159}, metal_ops.rs:6471-6536)
+    w = fake((1001 * 128 * 18,), U8)
+    assert lib.oxq_gguf_quant_matmul(ctx, None, C.byref(fake((1, 4096), BF16)), C.byref(w), 4096,
+                                     1001, _lib.GGUF_Q4_0, C.byref(fake((1, 1001), BF16))) == 0
+
+
+def test_mxfp4_validation(lib, ctx):
+    K, N = 2880, 5760
+    nb = K // 32
+    blocks, scales = fake((N * nb * 16,), U8), fake((N * nb,), U8)
+    x, out = fake((8, K), BF16), fake((8, N), BF16)
+
+    def call(x=x, b=blocks, s=scales, out=out, k=K, n=N):
+        return lib.oxq_mxfp4_matmul(ctx, None, C.byref(x), C.byref(b), C.byref(s), k, n, C.byref(out))
+
+    assert call() == 0, err(lib)
+    assert call(x=fake((33, K), BF16), out=fake((33, N), BF16)) == 0  # any m (mul_mm above 8)
+    assert call(x=fake((8, K), F16)) == -2 and "BF16" in err(lib)
+    assert call(b=fake((N * nb * 16,), I32)) == -2
+    assert call(k=K + 16, x=fake((8, K + 16), BF16)) == -3 and "multiple of 32" in err(lib)
+    assert call(b=fake((N * nb * 16 - 16,), U8)) == -3 and "don't match" in err(lib)
+    assert call(x=fake((8, K), BF16, contiguous=False)) == -4
+    assert call(x=fake((8, K - 32), BF16)) == -3
+    assert call(out=fake((7, N), BF16)) == -3 and "output shape" in err(lib)
+
+
+def test_layers_validate_like_reference(lib, ctx):
+    h = C.c_void_p()
+    qw, qz, sc = _awq(4096, 14336, 128, BF16)
+    # linear.rs:417-419 bits; 420-422 qzeros missing; 431-436 scales mismatch
+    assert lib.oxq_packed_quant_linear_new(ctx, 3, 0, C.byref(qw), C.byref(qz), C.byref(sc), None,
+                                           BF16, C.byref(h)) == -8
+    assert lib.oxq_packed_quant_linear_new(ctx, 4, 0, C.byref(qw), None, C.byref(sc), None, BF16,
+                                           C.byref(h)) == -1 and "qzeros missing" in err(lib)
+    bad_sc = fake((32, 14336 + 8), BF16)
+    assert lib.oxq_packed_quant_linear_new(ctx, 4, 0, C.byref(qw), C.byref(qz), C.byref(bad_sc), None,
+                                           BF16, C.byref(h)) == -3 and "derived" in err(lib)
+    assert lib.oxq_packed_quant_linear_new(ctx, 4, 0, C.byref(qw), C.byref(qz), C.byref(sc), None,
+                                           BF16, C.byref(h)) == 0, err(lib)
+    k, n = C.c_int64(), C.c_int64()
+    lib.oxq_packed_quant_linear_in_features(h, C.byref(k))
+    lib.oxq_packed_quant_linear_out_features(h, C.byref(n))
+    assert (k.value, n.value) == (4096, 14336)
+    # routing (linear.rs:494-524): m <= 8 -> GEMV kernel, above -> tile GEMM; leading dims flatten
+    for shape, kern in [((1, 4096), "awq4_gemv_fast_bf16_m1"), ((2, 3, 4096), "awq4_gemv_fast_bf16_m8"),
+                        ((16, 4096), "awq4_mfma_bf16_mt1"), ((4, 16, 4096), "awq4_mfma_bf16_mt4")]:
+        x = fake(shape, BF16)
+        out = fake(shape[:-1] + (14336,), BF16)
+        assert lib.oxq_packed_quant_linear_forward(h, None, C.byref(x), C.byref(out)) == 0, err(lib)
+        assert plan(lib, ctx).kernel.decode().startswith(kern), plan(lib, ctx).kernel
+    x = fake((1, 4000), BF16)
+    assert lib.oxq_packed_quant_linear_forward(h, None, C.byref(x), C.byref(fake((1, 14336), BF16))) == -3
+    assert "input last dim 4000 != in_features 4096" in err(lib)
+    lib.oxq_packed_quant_linear_free(h)
+
+    # Mxfp4Linear::new (mxfp4.rs:85-105)
+    m = C.c_void_p()
+    b, s = fake((10 * 2 * 16,), U8), fake((10 * 2,), U8)
+    assert lib.oxq_mxfp4_linear_new(ctx, C.byref(b), C.byref(s), None, 64, 10, C.byref(m)) == 0
+    assert lib.oxq_mxfp4_linear_forward(m, None, C.byref(fake((3, 64), BF16)),
+                                        C.byref(fake((3, 10), BF16))) == 0, err(lib)
+    assert lib.oxq_mxfp4_linear_forward(m, None, C.byref(fake((3, 32), BF16)),
+                                        C.byref(fake((3, 10), BF16))) == -3
+    assert "x last dim 32 != in_features 64" in err(lib)
+    lib.oxq_mxfp4_linear_free(m)
+    assert lib.oxq_mxfp4_linear_new(ctx, C.byref(b), C.byref(s), None, 48, 10, C.byref(m)) == -3
+    assert lib.oxq_mxfp4_linear_new(ctx, C.byref(fake((320,), I32)), C.byref(s), None, 64, 10,
+                                    C.byref(m)) == -2
+    assert lib.oxq_mxfp4_linear_new(ctx, C.byref(b), C.byref(s), None, 64, 11, C.byref(m)) == -3
+
+    # QLinear / GgufFastPath::build (linear.rs:197-247)
+    q = C.c_void_p()
+    w = fake((4096 * 16 * 144,), U8)
+    assert lib.oxq_qlinear_new(ctx, _lib.GGUF_Q4_K, C.byref(w), 4096, 4096, None, BF16, C.byref(q)) == 0
+    for m_rows, kern in [(1, "gguf_q4k_gemv_bf16"), (8, "gguf_q4k_gemv_bf16"), (33, "gguf_q4k_gemv_bf16")]:
+        assert lib.oxq_qlinear_forward(q, None, C.byref(fake((m_rows, 4096), BF16)),
+                                       C.byref(fake((m_rows, 4096), BF16))) == 0, err(lib)
+        p = plan(lib, ctx)
+        assert p.kernel.decode() == kern and p.launches == (m_rows + 7) // 8
+    lib.oxq_qlinear_free(q)
+    assert lib.oxq_qlinear_new(ctx, _lib.GGUF_Q4_K, C.byref(w), 4096, 4095, None, BF16, C.byref(q)) == -3
+
+
+def test_real_context_without_gpu_fails_loudly(lib):
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("GPU present")
+    h = C.c_void_p()
+    rc = lib.oxq_ctx_create(0, C.byref(h))
+    assert rc == -7 and "no HIP device" in err(lib)

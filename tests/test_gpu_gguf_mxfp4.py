@@ -1,0 +1,207 @@
+"""GPU parity tests for the GGUF block-quant GEMV and the MXFP4 expert GEMV.
+
+GGUF: no golden vectors exist in the reference (its tests quantize with the
+third-party candle QTensor, metal_ops.rs:6405-6417); inputs here are seeded
+random block bytes (benchmark config 3) and the oracle is the ggml-format
+restatement pinned in test_oracle_kat.py.  Dequant is compared bit for bit,
+GEMV at 2e-3 rel / 1e-2 abs of the f32-accumulated oracle.
+MXFP4: generators of metal_ops.rs:6622-6670 plus benchmark config 4.
+"""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from oxydllm_amd import synth
+from tests import refgen
+from tests.helpers import as_f32, assert_close, round_x, to_dev
+
+pytestmark = pytest.mark.gpu
+ops = None
+FMTS = [synth.GGUF_Q4_0, synth.GGUF_Q8_0, synth.GGUF_Q4_K, synth.GGUF_Q6_K]
+
+
+def setup_module(module):
+    from oxydllm_amd import ops as _ops
+    module.ops = _ops
+
+
+def say(msg):
+    print(f"[case] {msg}", flush=True)
+    sys.stdout.flush()
+
+
+# ------------------------------------------------------------------ GGUF
+@pytest.mark.parametrize("fmt", FMTS)
+def test_gguf_dequant_bit_exact(fmt):
+    say(f"gguf dequant {synth.GGUF_NAMES[fmt]}")
+    N, K = 37, 1024
+    data = synth.gguf_weight(fmt, N, K, seed=40 + fmt)
+    want = oracle.dequantize_gguf(fmt, data, N, K)
+    got = ops.gguf_dequantize(to_dev(data), K, N, fmt)
+    np.testing.assert_array_equal(got.cpu().numpy().view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+@pytest.mark.parametrize("act", ["f32", "bf16"])
+def test_gguf_gemv_config3(fmt, act):
+    """Benchmark config 3: M=1, K=N=4096, x~N(0,1) f32 (and the reference's bf16 contract)."""
+    say(f"gguf gemv {synth.GGUF_NAMES[fmt]} {act}")
+    N = K = 4096
+    data = synth.gguf_weight(fmt, N, K, seed=0x0A0D11E8 + fmt)
+    w = oracle.dequantize_gguf(fmt, data, N, K)
+    x = np.random.default_rng(50 + fmt).standard_normal((1, K)).astype(np.float32)
+    if act == "bf16":
+        xd, xr = to_dev(x, torch.bfloat16), round_x(x, oracle.BF16)
+    else:
+        xd, xr = to_dev(x), x
+    ref = oracle.matmul_nt_f32(xr, w)
+    y = ops.gguf_quant_matmul(xd, to_dev(data), K, N, fmt)
+    assert y.shape == (1, N) and y.dtype == xd.dtype
+    assert_close(as_f32(y), ref, f"gguf {synth.GGUF_NAMES[fmt]} {act}")
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+def test_gguf_gemv_batch_and_odd_n(fmt):
+    """metal_ops.rs:6544-6617 (M in {2,4,8}) and 6471-6536 (odd N: 1001)."""
+    elems, _ = synth.GGUF_BLOCK_LAYOUT[fmt]
+    N, K = 1001, 4 * 256
+    data = synth.gguf_weight(fmt, N, K, seed=60 + fmt)
+    w = oracle.dequantize_gguf(fmt, data, N, K)
+    wd = to_dev(data)
+    for m in (1, 2, 4, 8):
+        say(f"gguf batch {synth.GGUF_NAMES[fmt]} m={m} N={N}")
+        x = np.random.default_rng(70 + m).standard_normal((m, K)).astype(np.float32)
+        ref = oracle.matmul_nt_f32(round_x(x, oracle.BF16), w)
+        y = ops.gguf_quant_matmul(to_dev(x, torch.bfloat16), wd, K, N, fmt)
+        assert_close(as_f32(y), ref, f"gguf batch m{m}")
+
+
+@pytest.mark.parametrize("fmt", [synth.GGUF_Q4_0, synth.GGUF_Q6_K])
+@pytest.mark.parametrize("m", [9, 33, 70])
+def test_gguf_mul_mm(fmt, m):
+    """metal_ops.rs:6387-6463: M in {9, 33, 70}."""
+    say(f"gguf mul_mm {synth.GGUF_NAMES[fmt]} m={m}")
+    N, K = 200, 512
+    data = synth.gguf_weight(fmt, N, K, seed=80 + fmt)
+    w = oracle.dequantize_gguf(fmt, data, N, K)
+    x = np.random.default_rng(90 + m).standard_normal((m, K)).astype(np.float32)
+    ref = oracle.matmul_nt_f32(round_x(x, oracle.BF16), w)
+    y = ops.gguf_quant_mul_mm(to_dev(x, torch.bfloat16), to_dev(data), K, N, fmt)
+    assert_close(as_f32(y), ref, f"gguf mul_mm m{m}")
+    with pytest.raises(ops.OxqError, match=r"out of \[1, 8\]"):
+        ops.gguf_quant_matmul(to_dev(x, torch.bfloat16), to_dev(data), K, N, fmt)
+
+
+def test_qlinear_layer_bias_and_routing():
+    """linear.rs:324-351: decode vs prefill routing, out dtype, bias."""
+    say("QLinear")
+    fmt, N, K = synth.GGUF_Q4_K, 96, 512
+    data = synth.gguf_weight(fmt, N, K, seed=99)
+    w = oracle.dequantize_gguf(fmt, data, N, K)
+    bias = np.linspace(-1, 1, N).astype(np.float32)
+    layer = ops.QLinear(fmt, to_dev(data), K, N, to_dev(bias, torch.bfloat16), torch.bfloat16)
+    for shape in [(1, K), (2, 4, K), (3, 5, K)]:
+        m = int(np.prod(shape[:-1]))
+        x = np.random.default_rng(m).standard_normal((m, K)).astype(np.float32)
+        y = layer.forward(to_dev(x.reshape(shape), torch.bfloat16))
+        assert tuple(y.shape) == shape[:-1] + (N,)
+        ref = oracle.matmul_nt_f32(round_x(x, oracle.BF16), w, round_x(bias, oracle.BF16))
+        assert_close(as_f32(y).reshape(m, N), ref, f"QLinear {shape}")
+
+
+# ------------------------------------------------------------------ MXFP4
+def test_mxfp4_dequant_bit_exact():
+    say("mxfp4 dequant")
+    n, k = 64, 2880
+    blocks, scales = synth.mxfp4_weight(n, k, seed=7, exp_lo=0, exp_hi=254)
+    blocks[:16] = np.arange(16, dtype=np.uint8) * 17  # every code in both nibbles
+    scales[3] = 255                                   # E8M0 NaN encoding (mxfp4.rs:26-29)
+    want = oracle.dequantize_mxfp4_f32(blocks, scales, n, k)
+    got = ops.mxfp4_dequantize(to_dev(blocks), to_dev(scales), k, n).cpu().numpy()
+    nan = np.isnan(want)
+    assert nan.any() and np.array_equal(np.isnan(got), nan)
+    np.testing.assert_array_equal(got.view(np.uint32)[~nan], want.view(np.uint32)[~nan])
+
+
+@pytest.mark.parametrize("m", [1, 4, 8, 33])
+def test_mxfp4_matmul_reference_case(m):
+    """metal_ops.rs:6622-6670: n=10 (unaligned), k=64, M in {1,4,8,33}."""
+    say(f"mxfp4 matmul m={m}")
+    n, k = 10, 64
+    blocks, scales = refgen.mxfp4_case(n, k)
+    w = oracle.dequantize_mxfp4_f32(blocks, scales, n, k)
+    x = refgen.mxfp4_x(m, k)
+    ref = oracle.matmul_nt_f32(round_x(x, oracle.BF16), w)
+    y = ops.mxfp4_matmul(to_dev(x, torch.bfloat16), to_dev(blocks), to_dev(scales), k, n)
+    assert y.shape == (m, n) and y.dtype == torch.bfloat16
+    assert_close(as_f32(y), ref, f"mxfp4 m{m}")
+
+
+def _config4(seed=0x0A0D11E9):
+    E, top_k, hidden, inter, T = 32, 4, 2880, 2880, 8
+    rng = np.random.default_rng(seed)
+    gu_b, gu_s = synth.mxfp4_weight(E * 2 * inter, hidden, seed=seed + 1)
+    dn_b, dn_s = synth.mxfp4_weight(E * hidden, inter, seed=seed + 2)
+    gu_bias = (rng.standard_normal((E, 2 * inter)) * 0.1).astype(np.float32)
+    dn_bias = (rng.standard_normal((E, hidden)) * 0.1).astype(np.float32)
+    x = rng.standard_normal((T, hidden)).astype(np.float32)
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    return dict(E=E, top_k=top_k, hidden=hidden, inter=inter, T=T, gu_b=gu_b, gu_s=gu_s, dn_b=dn_b,
+                dn_s=dn_s, gu_bias=gu_bias, dn_bias=dn_bias, x=x, logits=logits)
+
+
+def test_mxfp4_moe_config4():
+    """Benchmark config 4: 32 experts, top-4, hidden 2880, gate_up N=5760, down K=2880, 8 tokens.
+    Routing lists come from the oracle's restatement of moe.rs:466-607."""
+    c = _config4()
+    E, H, I = c["E"], c["hidden"], c["inter"]
+    idx, vals = oracle.moe_route(c["logits"], c["top_k"], True)
+    offsets, tokens, _ = oracle.moe_group(idx, vals, E)
+    n_pairs = int(offsets[-1])
+    assert n_pairs == c["T"] * c["top_k"]
+    say(f"mxfp4 moe gate_up: {int((np.diff(offsets) > 0).sum())} active experts, {n_pairs} pairs")
+    xb = round_x(c["x"], oracle.BF16)
+    gub = round_x(c["gu_bias"], oracle.BF16)
+    dnb = round_x(c["dn_bias"], oracle.BF16)
+    nb = H // 32
+
+    # oracle, per active expert (Mxfp4Linear::forward = x.W^T + bias, mxfp4.rs:119-154)
+    ref_gu = np.zeros((n_pairs, 2 * I), np.float32)
+    ref_dn = np.zeros((n_pairs, H), np.float32)
+    h_in = np.random.default_rng(5).standard_normal((n_pairs, I)).astype(np.float32)
+    hb = round_x(h_in, oracle.BF16)
+    for e in range(E):
+        lo, hi = int(offsets[e]), int(offsets[e + 1])
+        if hi == lo:
+            continue
+        wg = oracle.dequantize_mxfp4_f32(c["gu_b"][e * 2 * I * nb * 16:(e + 1) * 2 * I * nb * 16],
+                                         c["gu_s"][e * 2 * I * nb:(e + 1) * 2 * I * nb], 2 * I, H)
+        ref_gu[lo:hi] = oracle.matmul_nt_f32(xb[tokens[lo:hi]], wg, gub[e])
+        wd = oracle.dequantize_mxfp4_f32(c["dn_b"][e * H * nb * 16:(e + 1) * H * nb * 16],
+                                         c["dn_s"][e * H * nb:(e + 1) * H * nb], H, I)
+        ref_dn[lo:hi] = oracle.matmul_nt_f32(hb[lo:hi], wd, dnb[e])
+
+    off_d = to_dev(offsets.astype(np.int32))
+    tok_d = to_dev(tokens.astype(np.int32))
+    y = ops.mxfp4_moe_matmul(to_dev(c["x"], torch.bfloat16), to_dev(c["gu_b"]), to_dev(c["gu_s"]),
+                             to_dev(c["gu_bias"], torch.bfloat16), off_d, tok_d, H, 2 * I)
+    assert y.shape == (n_pairs, 2 * I)
+    assert_close(as_f32(y), ref_gu, "moe gate_up")
+    say("mxfp4 moe down")
+    y2 = ops.mxfp4_moe_matmul(to_dev(h_in, torch.bfloat16), to_dev(c["dn_b"]), to_dev(c["dn_s"]),
+                              to_dev(c["dn_bias"], torch.bfloat16), off_d, None, I, H)
+    assert_close(as_f32(y2), ref_dn, "moe down")
+
+    # one expert through the layer type equals its slice of the grouped launch
+    e = int(np.argmax(np.diff(offsets)))
+    lo, hi = int(offsets[e]), int(offsets[e + 1])
+    say(f"Mxfp4Linear expert {e} rows {hi - lo}")
+    lay = ops.Mxfp4Linear(to_dev(c["gu_b"][e * 2 * I * nb * 16:(e + 1) * 2 * I * nb * 16]),
+                          to_dev(c["gu_s"][e * 2 * I * nb:(e + 1) * 2 * I * nb]),
+                          to_dev(c["gu_bias"][e], torch.bfloat16), H, 2 * I)
+    ys = lay.forward(to_dev(c["x"][tokens[lo:hi]], torch.bfloat16))
+    assert_close(as_f32(ys), ref_gu[lo:hi], "Mxfp4Linear")
+    assert torch.equal(ys, y[lo:hi])
