@@ -60,7 +60,7 @@ def test_gguf_gemv_config3(fmt, act):
     ref = oracle.matmul_nt_f32(xr, w)
     y = ops.gguf_quant_matmul(xd, to_dev(data), K, N, fmt)
     assert y.shape == (1, N) and y.dtype == xd.dtype
-    assert_close(as_f32(y), ref, f"gguf {synth.GGUF_NAMES[fmt]} {act}")
+    assert_close(y, ref, f"gguf {synth.GGUF_NAMES[fmt]} {act}")
 
 
 @pytest.mark.parametrize("fmt", FMTS)
@@ -76,7 +76,7 @@ def test_gguf_gemv_batch_and_odd_n(fmt):
         x = np.random.default_rng(70 + m).standard_normal((m, K)).astype(np.float32)
         ref = oracle.matmul_nt_f32(round_x(x, oracle.BF16), w)
         y = ops.gguf_quant_matmul(to_dev(x, torch.bfloat16), wd, K, N, fmt)
-        assert_close(as_f32(y), ref, f"gguf batch m{m}")
+        assert_close(y, ref, f"gguf batch m{m}")
 
 
 @pytest.mark.parametrize("fmt", [synth.GGUF_Q4_0, synth.GGUF_Q6_K])
@@ -90,7 +90,7 @@ def test_gguf_mul_mm(fmt, m):
     x = np.random.default_rng(90 + m).standard_normal((m, K)).astype(np.float32)
     ref = oracle.matmul_nt_f32(round_x(x, oracle.BF16), w)
     y = ops.gguf_quant_mul_mm(to_dev(x, torch.bfloat16), to_dev(data), K, N, fmt)
-    assert_close(as_f32(y), ref, f"gguf mul_mm m{m}")
+    assert_close(y, ref, f"gguf mul_mm m{m}")
     with pytest.raises(ops.OxqError, match=r"out of \[1, 8\]"):
         ops.gguf_quant_matmul(to_dev(x, torch.bfloat16), to_dev(data), K, N, fmt)
 
@@ -109,7 +109,7 @@ def test_qlinear_layer_bias_and_routing():
         y = layer.forward(to_dev(x.reshape(shape), torch.bfloat16))
         assert tuple(y.shape) == shape[:-1] + (N,)
         ref = oracle.matmul_nt_f32(round_x(x, oracle.BF16), w, round_x(bias, oracle.BF16))
-        assert_close(as_f32(y).reshape(m, N), ref, f"QLinear {shape}")
+        assert_close(y.reshape(m, N), ref, f"QLinear {shape}")
 
 
 # ------------------------------------------------------------------ MXFP4
@@ -137,7 +137,7 @@ def test_mxfp4_matmul_reference_case(m):
     ref = oracle.matmul_nt_f32(round_x(x, oracle.BF16), w)
     y = ops.mxfp4_matmul(to_dev(x, torch.bfloat16), to_dev(blocks), to_dev(scales), k, n)
     assert y.shape == (m, n) and y.dtype == torch.bfloat16
-    assert_close(as_f32(y), ref, f"mxfp4 m{m}")
+    assert_close(y, ref, f"mxfp4 m{m}")
 
 
 def _config4(seed=0x0A0D11E9):
@@ -189,11 +189,11 @@ def test_mxfp4_moe_config4():
     y = ops.mxfp4_moe_matmul(to_dev(c["x"], torch.bfloat16), to_dev(c["gu_b"]), to_dev(c["gu_s"]),
                              to_dev(c["gu_bias"], torch.bfloat16), off_d, tok_d, H, 2 * I)
     assert y.shape == (n_pairs, 2 * I)
-    assert_close(as_f32(y), ref_gu, "moe gate_up")
+    assert_close(y, ref_gu, "moe gate_up")
     say("mxfp4 moe down")
     y2 = ops.mxfp4_moe_matmul(to_dev(h_in, torch.bfloat16), to_dev(c["dn_b"]), to_dev(c["dn_s"]),
                               to_dev(c["dn_bias"], torch.bfloat16), off_d, None, I, H)
-    assert_close(as_f32(y2), ref_dn, "moe down")
+    assert_close(y2, ref_dn, "moe down")
 
     # one expert through the layer type equals its slice of the grouped launch
     e = int(np.argmax(np.diff(offsets)))
@@ -203,5 +203,5 @@ def test_mxfp4_moe_config4():
                           to_dev(c["gu_s"][e * 2 * I * nb:(e + 1) * 2 * I * nb]),
                           to_dev(c["gu_bias"][e], torch.bfloat16), H, 2 * I)
     ys = lay.forward(to_dev(c["x"][tokens[lo:hi]], torch.bfloat16))
-    assert_close(as_f32(ys), ref_gu[lo:hi], "Mxfp4Linear")
+    assert_close(ys, ref_gu[lo:hi], "Mxfp4Linear")
     assert torch.equal(ys, y[lo:hi])
