@@ -1,0 +1,216 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-weight matmul path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--all]
+
+Workload (BASELINE.json configs[1]): AWQ W4A16, K=4096, N=14336, g=128, f16
+activations/scales, at M = 1 (GEMV), 16 and 64 (MFMA tile GEMM).  A "step" is
+one call of the hot path at M=1 on synthetic inputs already resident in HBM;
+consecutive steps rotate over enough weight copies (> 256 MB) that no step finds
+its weights in L2 or the memory-side cache.  The K timed steps are replayed from
+one HIP graph so that host launch overhead is not what is measured.
+
+Prints ONE JSON line: `value` is the M=1 throughput in GB/s of algorithmic
+bytes (packed weights + zeros + scales + x + y per call); the M=16 / M=64
+results, in GB/s and TFLOP/s, ride along in `cases`.  `roofline` describes the
+dominant kernel (the M=1 GEMV, HBM-bound); `cpu_baseline` times the CPU oracle's
+restatement of the reference's CPU path (dequantize at load, then a dense f32
+x.W^T per call, linear.rs:40-79, 597-600) on this machine's cores.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
+MFMA_F16_PEAK_TFLOPS = 2500.0
+K, N, G = 4096, 14336, 128
+
+
+def algo_bytes(M: int, k: int = K, n: int = N, g: int = G, bits: int = 4) -> int:
+    """Algorithmic bytes per call: packed weights + zeros + scales + x + y (16-bit)."""
+    w = k * n * bits // 8
+    z = (k // g) * n * bits // 8
+    s = (k // g) * n * 2
+    return w + z + s + M * k * 2 + M * n * 2
+
+
+def time_graph(fn_of_step, steps: int, warmup: int, stream):
+    """Capture `steps` consecutive calls into one HIP graph, replay, time with HIP events
+    recorded on the stream the kernels run on.  Returns (wall_ms, event_ms) for `steps` calls."""
+    import torch
+    for i in range(warmup):
+        fn_of_step(i)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        for i in range(steps):
+            fn_of_step(i)
+    torch.cuda.synchronize()
+    graph.replay()          # untimed replay (first replay uploads the graph)
+    torch.cuda.synchronize()
+    ev0 = torch.cuda.Event(enable_timing=True)
+    ev1 = torch.cuda.Event(enable_timing=True)
+    cur = torch.cuda.current_stream()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ev0.record(cur)
+    graph.replay()
+    ev1.record(cur)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    return wall_ms, ev0.elapsed_time(ev1)
+
+
+def cpu_baseline(qw, qz, sc, x_f32):
+    """Reference CPU path restated by the oracle: dequantize once (load time), then per
+    call a dense f32 y = x.W^T over the [N,K] f32 weight.  Bounded sample."""
+    import oracle
+    cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    t0 = time.perf_counter()
+    w = oracle.dequantize_awq(qw, qz, oracle.round_through(sc, oracle.F16))
+    t_deq = time.perf_counter() - t0
+    xr = oracle.round_through(x_f32, oracle.F16)
+    oracle.matmul_nt_f32(xr, w)  # warm
+    calls, t_total = 0, 0.0
+    while t_total < 4.0 and calls < 200:
+        t0 = time.perf_counter()
+        oracle.matmul_nt_f32(xr, w)
+        t_total += time.perf_counter() - t0
+        calls += 1
+    per_call = t_total / calls
+    return {
+        "value": round(algo_bytes(1) / per_call / 1e9, 3),
+        "unit": "GB/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": (f"{calls} calls of the dense f32 GEMV over the dequantized {N}x{K} weight "
+                   f"({per_call * 1e3:.2f} ms/call, OpenMP over rows); one-time dequant-at-load "
+                   f"{t_deq:.2f} s not included; GB/s counts the same packed-weight bytes as `value`"),
+        "ms_per_call": round(per_call * 1e3, 3),
+        "dequant_at_load_s": round(t_deq, 3),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=400)
+    ap.add_argument("--warmup", type=int, default=40)
+    ap.add_argument("--copies", type=int, default=16, help="weight copies rotated to defeat caches")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--all", action="store_true", help="also time GPTQ / GGUF / MXFP4 (stderr)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)")
+
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    from oxydllm_amd import ops, synth
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    ctx = ops.default_context()
+    stream = torch.cuda.Stream()
+
+    qw, qz, sc = synth.awq_checkpoint(K, N, G, 4, seed=0x0A0D11E6)
+    copies = max(1, args.copies)
+    qw_d = [torch.from_numpy(qw).to(dev) for _ in range(copies)]
+    qz_d = [torch.from_numpy(qz).to(dev) for _ in range(copies)]
+    sc_d = [torch.from_numpy(sc).to(dev, torch.float16) for _ in range(copies)]
+    rng = np.random.default_rng(1)
+    x_host = {m: rng.standard_normal((m, K)).astype(np.float32) for m in (1, 16, 64)}
+    x_d = {m: torch.from_numpy(v).to(dev, torch.float16) for m, v in x_host.items()}
+    y_d = {m: torch.empty((m, N), dtype=torch.float16, device=dev) for m in (1, 16, 64)}
+
+    cases = []
+    for m in (1, 16, 64):
+        if m <= 8:
+            def step(i, m=m):
+                c = i % copies
+                ops.w4a16_matmul(x_d[m], qw_d[c], qz_d[c], sc_d[c], out=y_d[m], ctx=ctx)
+        else:
+            def step(i, m=m):
+                c = i % copies
+                ops.mpp_quant_matmul(x_d[m], qw_d[c], qz_d[c], sc_d[c], 4, ops.PACK_OUT,
+                                     out=y_d[m], ctx=ctx)
+        step(0)
+        plan = ctx.last_plan()
+        wall_ms, ev_ms = time_graph(step, args.steps, args.warmup, stream)
+        # same weights every call: the 30 MB stay in the 256 MB memory-side cache
+        def hot(i, m=m):
+            if m <= 8:
+                ops.w4a16_matmul(x_d[m], qw_d[0], qz_d[0], sc_d[0], out=y_d[m], ctx=ctx)
+            else:
+                ops.mpp_quant_matmul(x_d[m], qw_d[0], qz_d[0], sc_d[0], 4, ops.PACK_OUT,
+                                     out=y_d[m], ctx=ctx)
+        _, hot_ms = time_graph(hot, args.steps, args.warmup, stream)
+        us = ev_ms * 1e3 / args.steps
+        b = algo_bytes(m)
+        flops = 2.0 * m * K * N
+        cases.append({
+            "M": m, "kernel": plan["kernel"], "grid": list(plan["grid"]), "split_k": plan["split_k"],
+            "us_per_call": round(us, 3), "us_per_call_wall": round(wall_ms * 1e3 / args.steps, 3),
+            "us_per_call_hot_cache": round(hot_ms * 1e3 / args.steps, 3),
+            "algorithmic_bytes": b, "GB_per_s": round(b / us / 1e3, 1),
+            "hbm_frac": round(b / us / 1e3 / HBM_PEAK_GBS, 4),
+            "TFLOP_per_s": round(flops / us / 1e6, 2),
+            "mfma_frac": round(flops / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 4),
+        })
+        print(f"[bench] M={m}: {cases[-1]}", file=sys.stderr, flush=True)
+
+    c1 = cases[0]
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "awq4_gemv_m1_traffic.json")
+    if os.path.exists(tpath):
+        try:
+            traffic = json.load(open(tpath)).get("hbm_bytes_per_launch")
+        except Exception:
+            traffic = None
+    result = {
+        "metric": "int4 GEMV/GEMM HBM GB/s (% peak) + TFLOPS at M=1/16/64, K=4096 N=14336",
+        "value": c1["GB_per_s"],
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(c1["us_per_call_wall"] / 1e3, 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": "AWQ W4A16 GEMV M=1, K=4096 N=14336 g=128, f16 in/out, f32 accumulate "
+                               "(BASELINE configs[1]); M=16/64 tile GEMM in `cases`",
+                   "weight_copies_rotated": copies, "timing": "HIP graph of `steps` launches"},
+        "roofline": {"bound": "hbm", "achieved": c1["GB_per_s"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(c1["GB_per_s"] / HBM_PEAK_GBS, 4), "traffic": traffic,
+                     "kernel": c1["kernel"], "algorithmic_bytes_per_launch": c1["algorithmic_bytes"],
+                     "us_per_launch": c1["us_per_call"]},
+        "roofline_m64": {"bound": "mfma", "achieved": cases[2]["TFLOP_per_s"],
+                         "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                         "frac": cases[2]["mfma_frac"], "traffic": None,
+                         "kernel": cases[2]["kernel"], "hbm_frac": cases[2]["hbm_frac"]},
+        "cases": cases,
+    }
+    if args.all:
+        from oxydllm_amd import bench_extra
+        result["other_configs"] = bench_extra.run(ops, ctx, stream, args.steps, args.warmup, time_graph)
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(qw, qz, sc, x_host[1])
+    else:
+        result["cpu_baseline"] = None
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -417,6 +417,10 @@ int oxq_ctx_create(int device, oxq_ctx **out) {
     const size_t ws_mb = (ws_env && atoi(ws_env) > 0) ? (size_t)atoi(ws_env) : 64;
     ctx->workspace_bytes = ws_mb << 20;
     ctx->n_counters = 16384;
+    {
+        const char *m = getenv("OXQ_SPLITK_MODE");
+        ctx->splitk_mode = (m && *m) ? atoi(m) : 0;
+    }
     if (ctx->plan_only) {
         *out = ctx;
         return OXQ_OK;

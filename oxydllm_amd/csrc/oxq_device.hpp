@@ -34,6 +34,28 @@ __device__ __forceinline__ constexpr int awq_slot_col(int slot) {
     return ((slot & 3) << 1) | (slot >> 2);
 }
 
+// The AND masks live in VGPRs: v_and_or_b32 may read only one scalar/literal
+// operand, and with both the mask and the exponent pattern as literals the
+// compiler splits every unpack into v_and + v_or.
+struct NibbleMasks {
+    uint32_t m0, m1;
+};
+__device__ __forceinline__ uint32_t vgpr_const(uint32_t c) {
+    uint32_t r;
+    asm volatile("v_mov_b32 %0, %1" : "=v"(r) : "s"(c));
+    return r;
+}
+__device__ __forceinline__ NibbleMasks nibble_masks() {
+    return NibbleMasks{vgpr_const(0x000F000Fu), vgpr_const(0x00F000F0u)};
+}
+
+// Raw buffer resources: base + 32-bit lane offset + scalar offset addressing, so
+// row addresses cost scalar ALU only; out-of-range reads return zero.
+constexpr int BUFFER_RSRC_FLAGS = 0x00020000;
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *p, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, (int)bytes, BUFFER_RSRC_FLAGS);
+}
+
 // ---------------------------------------------------------------------------
 // Element-type traits.  `pair` registers hold two 16-bit floats.
 //
@@ -48,12 +70,17 @@ struct F16Traits {
     static constexpr int DTYPE = 1;
     static constexpr uint32_t ONES = 0x3C003C00u;
     __device__ static __forceinline__ float bias(int i) { return (i & 1) ? 64.0f : 1024.0f; }
-    __device__ static __forceinline__ void unpack4(uint32_t t, uint32_t p[4]) {
-        p[0] = (t & 0x000F000Fu) | 0x64006400u;
-        p[1] = (t & 0x00F000F0u) | 0x54005400u;
+    __device__ static __forceinline__ void unpack4(uint32_t t, uint32_t p[4], const NibbleMasks &k) {
+        p[0] = (t & k.m0) | 0x64006400u;
+        p[1] = (t & k.m1) | 0x54005400u;
         const uint32_t t8 = t >> 8;
-        p[2] = (t8 & 0x000F000Fu) | 0x64006400u;
-        p[3] = (t8 & 0x00F000F0u) | 0x54005400u;
+        p[2] = (t8 & k.m0) | 0x64006400u;
+        p[3] = (t8 & k.m1) | 0x54005400u;
+    }
+    // one nibble position (0..3 of each 16-bit half) -> pair of bias(i) + nibble
+    __device__ static __forceinline__ uint32_t unpack1(uint32_t t, int i, const NibbleMasks &k) {
+        const uint32_t u = (i & 2) ? (t >> 8) : t;
+        return (i & 1) ? ((u & k.m1) | 0x54005400u) : ((u & k.m0) | 0x64006400u);
     }
     // two bytes (low byte of each half) -> pair of 1024 + byte
     __device__ static __forceinline__ uint32_t unpack_bytes(uint32_t t) {
@@ -77,11 +104,15 @@ struct BF16Traits {
     static constexpr int DTYPE = 2;
     static constexpr uint32_t ONES = 0x3F803F80u;
     __device__ static __forceinline__ float bias(int) { return 128.0f; }
-    __device__ static __forceinline__ void unpack4(uint32_t t, uint32_t p[4]) {
-        p[0] = (t & 0x000F000Fu) | 0x43004300u;
-        p[1] = ((t >> 4) & 0x000F000Fu) | 0x43004300u;
-        p[2] = ((t >> 8) & 0x000F000Fu) | 0x43004300u;
-        p[3] = ((t >> 12) & 0x000F000Fu) | 0x43004300u;
+    __device__ static __forceinline__ void unpack4(uint32_t t, uint32_t p[4], const NibbleMasks &k) {
+        p[0] = (t & k.m0) | 0x43004300u;
+        p[1] = ((t >> 4) & k.m0) | 0x43004300u;
+        p[2] = ((t >> 8) & k.m0) | 0x43004300u;
+        p[3] = ((t >> 12) & k.m0) | 0x43004300u;
+    }
+    __device__ static __forceinline__ uint32_t unpack1(uint32_t t, int i, const NibbleMasks &k) {
+        const uint32_t u = i ? (t >> (4 * i)) : t;
+        return (u & k.m0) | 0x43004300u;
     }
     // bytes need 8 significant bits: go through f32 (exact), keep the high halves
     __device__ static __forceinline__ uint32_t unpack_bytes(uint32_t t) {
@@ -120,25 +151,43 @@ __device__ __forceinline__ float wave_sum_xor(float v) {  // butterfly over WIDT
 // Deterministic split-K.
 //
 // Each of `splits` workgroups that share an output tile stores its f32 partial
-// tile to the workspace, then calls splitk_arrive().  Exactly one caller - the
-// last to arrive - gets `true`; it then sums the partials of all slices in
-// slice order 0..splits-1, so the result does not depend on arrival order.
-// The counter is left at zero for the next launch.
+// tile to the workspace; the partials are summed in slice order 0..splits-1,
+// so the result does not depend on which workgroup finishes first.  Two ways
+// to run that sum:
+//
+//  * a second kernel (splitk_reduce_kernel): plain stores, the kernel boundary
+//    publishes them, every CU takes part in the reduction;
+//  * fused: the last workgroup to arrive at the tile's counter does the sum.
+//    Partials are written and read with device-scope relaxed atomics
+//    (write-through / cache-bypassing accesses on gfx950), the arrival is a
+//    device-scope atomic add issued after the workgroup's stores have
+//    completed (s_waitcnt + barrier).  No cache write-back or invalidate is
+//    needed, which on this part costs more than the whole GEMV.  The counter is
+//    left at zero for the next launch.
 // ---------------------------------------------------------------------------
+__device__ __forceinline__ void st_agent(float *p, float v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float ld_agent(const float *p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 __device__ __forceinline__ bool splitk_arrive(unsigned *counters, unsigned tile, unsigned splits) {
     __shared__ unsigned s_last;
-    __threadfence();  // release this thread's partial stores at device scope
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);
+    __builtin_amdgcn_s_waitcnt(0);  // this wave's partial stores have completed
     __syncthreads();
     if (threadIdx.x == 0 && threadIdx.y == 0 && threadIdx.z == 0) {
-        const unsigned old = atomicAdd(&counters[tile], 1u);
+        const unsigned old = __hip_atomic_fetch_add(&counters[tile], 1u, __ATOMIC_RELAXED,
+                                                    __HIP_MEMORY_SCOPE_AGENT);
         const unsigned last = (old + 1u == splits) ? 1u : 0u;
-        if (last) counters[tile] = 0u;
+        if (last)
+            __hip_atomic_store(&counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         s_last = last;
     }
     __syncthreads();
-    const bool last = s_last != 0u;
-    if (last) __threadfence();  // acquire the other slices' stores
-    return last;
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);
+    return s_last != 0u;
 }
 
 }  // namespace oxq

@@ -18,6 +18,7 @@ struct oxq_ctx {
     unsigned *counters;     // arrival counters, zero between calls
     size_t n_counters;
     int num_cus;
+    int splitk_mode;        // 0 auto, 1 fused last-arriver, 2 separate reduce kernel
     oxq_plan plan;
 };
 
@@ -110,7 +111,8 @@ int launch_gguf_gemv(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p);
 int launch_gguf_dequant(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p, float *out_nk);
 int launch_mxfp4_gemv(oxq_ctx *ctx, hipStream_t s, const Mxfp4Problem &p);
 int launch_mxfp4_dequant(oxq_ctx *ctx, hipStream_t s, const Mxfp4Problem &p, float *out_nk);
-int launch_bias_add(oxq_ctx *ctx, hipStream_t s, void *y, const void *bias, int64_t M, int64_t N,
-                    int dtype);
+// y[M,N] = sum over S slices of ws[s][M][N] (+ bias), slices added in index order.
+int launch_splitk_reduce(oxq_ctx *ctx, hipStream_t s, const float *ws, const void *bias, void *y,
+                         int64_t M, int64_t N, int S, int dtype);
 
 }  // namespace oxq

@@ -34,15 +34,87 @@ __device__ __forceinline__ void splitk_finish(const float *__restrict__ ws,
                                               const uint16_t *__restrict__ bias,
                                               uint16_t *__restrict__ y, int M, int N, int S,
                                               int n0, int tile_cols, int nthreads, int tid) {
-    for (int idx = tid; idx < M * tile_cols; idx += nthreads) {
-        const int m = idx / tile_cols;
-        const int n = n0 + idx % tile_cols;
-        if (n >= N) continue;
-        float tot = 0.0f;
-        for (int s = 0; s < S; ++s) tot += ws[((size_t)s * M + m) * N + n];
-        if (bias) tot += TT::to_f32(bias[n]);
-        y[(size_t)m * N + n] = TT::from_f32(tot);
+    constexpr int CPT = 4;  // outputs per thread whose slice loads are in flight together
+    const int total = M * tile_cols;
+    for (int base = tid; base < total; base += nthreads * CPT) {
+        float tot[CPT];
+#pragma unroll
+        for (int c = 0; c < CPT; ++c) tot[c] = 0.0f;
+        for (int s0 = 0; s0 < S; s0 += 8) {
+            float v[CPT][8];
+#pragma unroll
+            for (int c = 0; c < CPT; ++c) {
+                const int idx = base + c * nthreads;
+                const int m = idx / tile_cols;
+                const int n = n0 + idx % tile_cols;
+                const bool ok = idx < total && n < N;
+#pragma unroll
+                for (int u = 0; u < 8; ++u)
+                    v[c][u] = (ok && s0 + u < S) ? ld_agent(ws + ((size_t)(s0 + u) * M + m) * N + n) : 0.0f;
+            }
+#pragma unroll
+            for (int c = 0; c < CPT; ++c)
+#pragma unroll
+                for (int u = 0; u < 8; ++u) tot[c] += v[c][u];  // slice order
+        }
+#pragma unroll
+        for (int c = 0; c < CPT; ++c) {
+            const int idx = base + c * nthreads;
+            const int m = idx / tile_cols;
+            const int n = n0 + idx % tile_cols;
+            if (idx < total && n < N) {
+                float t = tot[c];
+                if (bias) t += TT::to_f32(bias[n]);
+                y[(size_t)m * N + n] = TT::from_f32(t);
+            }
+        }
     }
+}
+
+// Stand-alone reduction of the K slices (second launch): every thread owns 4
+// consecutive outputs and issues the loads of 8 slices at a time.
+template <typename TT>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *__restrict__ ws,
+                                                            const uint16_t *__restrict__ bias,
+                                                            uint16_t *__restrict__ y, size_t total,
+                                                            int N, int S) {
+    const size_t i4 = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i4 >= total) return;
+    float4_t tot = {0.f, 0.f, 0.f, 0.f};
+    for (int s0 = 0; s0 < S; s0 += 8) {
+        float4_t v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            v[u] = (s0 + u < S) ? *(const float4_t *)(ws + (size_t)(s0 + u) * total + i4)
+                                : float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int u = 0; u < 8; ++u) tot += v[u];
+    }
+    uint16_t o[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        float t = tot[c];
+        if (bias) t += TT::to_f32(bias[(i4 + c) % N]);
+        o[c] = TT::from_f32(t);
+    }
+    *(uint2 *)(y + i4) = uint2{(uint32_t)o[0] | ((uint32_t)o[1] << 16),
+                               (uint32_t)o[2] | ((uint32_t)o[3] << 16)};
+}
+
+int launch_splitk_reduce(oxq_ctx *ctx, hipStream_t s, const float *ws, const void *bias, void *y,
+                         int64_t M, int64_t N, int S, int dtype) {
+    const size_t total = (size_t)M * N;  // N % 4 == 0 for every caller
+    dim3 grid((unsigned)ceil_div((int64_t)(total / 4), 256)), block(256);
+    add_launch(ctx);
+    if (ctx->plan_only) return OXQ_OK;
+    if (dtype == OXQ_F16)
+        hipLaunchKernelGGL((splitk_reduce_kernel<F16Traits>), grid, block, 0, s, ws,
+                           (const uint16_t *)bias, (uint16_t *)y, total, (int)N, S);
+    else
+        hipLaunchKernelGGL((splitk_reduce_kernel<BF16Traits>), grid, block, 0, s, ws,
+                           (const uint16_t *)bias, (uint16_t *)y, total, (int)N, S);
+    OXQ_HIP_CHECK(hipGetLastError());
+    return OXQ_OK;
 }
 
 // ---------------------------------------------------------------------------
@@ -55,7 +127,7 @@ __global__ __launch_bounds__(256) void awq_gemv_generic(
     const uint32_t *__restrict__ qz, const uint16_t *__restrict__ sc,
     const uint16_t *__restrict__ bias, uint16_t *__restrict__ y, float *__restrict__ ws,
     unsigned *__restrict__ counters, int M, int K, int N, int packed_out, int gshift, int kchunk,
-    int S) {
+    int S, int fused) {
     constexpr int PF = 32 / BITS;
     constexpr uint32_t MASK = (1u << BITS) - 1u;
     __shared__ float red[4][64][PF];
@@ -118,6 +190,8 @@ __global__ __launch_bounds__(256) void awq_gemv_generic(
                     if (S == 1) {
                         const float b = bias ? TT::to_f32(bias[n]) : 0.0f;
                         y[(size_t)m * N + n] = TT::from_f32(tot + b);
+                    } else if (fused) {
+                        st_agent(ws + ((size_t)slice * M + m) * N + n, tot);
                     } else {
                         ws[((size_t)slice * M + m) * N + n] = tot;
                     }
@@ -126,7 +200,7 @@ __global__ __launch_bounds__(256) void awq_gemv_generic(
             __syncthreads();
         }
     }
-    if (S > 1 && splitk_arrive(counters, blockIdx.x, S))
+    if (S > 1 && fused && splitk_arrive(counters, blockIdx.x, S))
         splitk_finish<TT>(ws, bias, y, M, N, S, n0, tile_cols, 256, threadIdx.x);
 }
 
@@ -140,7 +214,7 @@ __global__ __launch_bounds__(256) void gptq_gemv_generic(
     const uint16_t *__restrict__ x, const uint32_t *__restrict__ qw,
     const uint32_t *__restrict__ qz, const uint16_t *__restrict__ sc,
     const uint16_t *__restrict__ bias, uint16_t *__restrict__ y, float *__restrict__ ws,
-    unsigned *__restrict__ counters, int M, int K, int N, int gshift, int wchunk, int S) {
+    unsigned *__restrict__ counters, int M, int K, int N, int gshift, int wchunk, int S, int fused) {
     constexpr int PF = 32 / BITS;
     constexpr uint32_t MASK = (1u << BITS) - 1u;
     __shared__ float red[4][64];
@@ -193,6 +267,8 @@ __global__ __launch_bounds__(256) void gptq_gemv_generic(
                 if (S == 1) {
                     const float b = bias ? TT::to_f32(bias[n]) : 0.0f;
                     y[(size_t)m * N + n] = TT::from_f32(tot + b);
+                } else if (fused) {
+                    st_agent(ws + ((size_t)slice * M + m) * N + n, tot);
                 } else {
                     ws[((size_t)slice * M + m) * N + n] = tot;
                 }
@@ -200,7 +276,7 @@ __global__ __launch_bounds__(256) void gptq_gemv_generic(
             __syncthreads();
         }
     }
-    if (S > 1 && splitk_arrive(counters, blockIdx.x, S))
+    if (S > 1 && fused && splitk_arrive(counters, blockIdx.x, S))
         splitk_finish<TT>(ws, bias, y, M, N, S, n0, 64, 256, threadIdx.x);
 }
 
@@ -218,26 +294,50 @@ __global__ __launch_bounds__(256) void gptq_gemv_generic(
 // which removes both the conversion bias and the zero-point in f32.
 // ---------------------------------------------------------------------------
 template <int WPL> struct WordVec;
-template <> struct WordVec<4> { typedef uint32_t type __attribute__((ext_vector_type(4))); };
-template <> struct WordVec<2> { typedef uint32_t type __attribute__((ext_vector_type(2))); };
-template <> struct WordVec<1> { typedef uint32_t type __attribute__((ext_vector_type(1))); };
+template <> struct WordVec<4> {
+    typedef uint32_t type __attribute__((ext_vector_type(4)));
+    __device__ static __forceinline__ type load(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
+        return __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0);
+    }
+};
+template <> struct WordVec<2> {
+    typedef uint32_t type __attribute__((ext_vector_type(2)));
+    __device__ static __forceinline__ type load(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
+        return __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, 0);
+    }
+};
+template <> struct WordVec<1> {
+    typedef uint32_t type __attribute__((ext_vector_type(1)));
+    __device__ static __forceinline__ type load(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
+        type v;
+        v[0] = __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0);
+        return v;
+    }
+};
 
-template <typename TT, int MB, int WPL, int WAVES, int RPW, int PS>
-__global__ __launch_bounds__(WAVES * 64) void awq4_gemv_fast(
+template <typename TT, int MB, int WPL, int WPG, int GPB, int RPW, int PS>
+__global__ __launch_bounds__(WPG * GPB * 64) void awq4_gemv_fast(
     const uint16_t *__restrict__ x, const uint32_t *__restrict__ qw,
     const uint32_t *__restrict__ qz, const uint16_t *__restrict__ sc,
     const uint16_t *__restrict__ bias, uint16_t *__restrict__ y, float *__restrict__ ws,
-    unsigned *__restrict__ counters, int M, int K, int N, int gshift, int gpw, int S) {
-    typedef typename WordVec<WPL>::type wvec_t;
+    unsigned *__restrict__ counters, int M, int K, int N, int gshift, int gpw, int S, int fused) {
+    // WPG waves share one quantization group (they take interleaved row pairs),
+    // GPB groups are processed side by side by one workgroup.
+    typedef WordVec<WPL> WV;
+    typedef typename WV::type wvec_t;
+    constexpr int WAVES = WPG * GPB;
     constexpr int LPR = 64 / RPW;          // lanes per row
     constexpr int NC = WPL * 8;            // columns per lane
     constexpr int SLAB_COLS = LPR * NC;
-    constexpr int ROWS_PER_CHUNK = 2 * WAVES * RPW * PS;
+    constexpr int ROWS_PER_CHUNK = 2 * WPG * RPW * PS;
     __shared__ float red[WAVES][SLAB_COLS];
 
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wg = wave / WPG, wr = wave % WPG;  // group slot, row phase (wave-uniform)
     const int cl = lane % LPR, sub = lane / LPR;
     const int PW = N >> 3;                 // words per row
+    const int rowbytes = PW * 4;
     const int jw = (blockIdx.x * LPR + cl) * WPL;
     const bool valid = jw < PW;
     const int G = K >> gshift;
@@ -246,6 +346,12 @@ __global__ __launch_bounds__(WAVES * 64) void awq4_gemv_fast(
     const int g1 = min(G, g0 + gpw);
     const int chunks = (1 << gshift) / ROWS_PER_CHUNK;
 
+    const __amdgpu_buffer_rsrc_t rs_w = make_rsrc(qw, (uint32_t)K * (uint32_t)rowbytes);
+    const __amdgpu_buffer_rsrc_t rs_x = make_rsrc(x, (uint32_t)M * (uint32_t)K * 2u);
+    const int voff_w = (2 * sub * PW + jw) * 4;  // this lane's row pair and word column
+    const int voff_x = 2 * sub * 2;
+    const NibbleMasks nm = nibble_masks();
+
     float yacc[MB][NC];
 #pragma unroll
     for (int m = 0; m < MB; ++m)
@@ -253,8 +359,12 @@ __global__ __launch_bounds__(WAVES * 64) void awq4_gemv_fast(
         for (int c = 0; c < NC; ++c) yacc[m][c] = 0.0f;
 
     if (valid) {
-        for (int g = g0; g < g1; ++g) {
+        for (int g = g0 + wg; g < g1; g += GPB) {
             const wvec_t zw = *(const wvec_t *)(qz + (size_t)g * PW + jw);
+            const uint16_t *srow = sc + (size_t)g * N + (size_t)jw * 8;
+            u32x4_t sv[WPL];
+#pragma unroll
+            for (int c = 0; c < WPL; ++c) sv[c] = *(const u32x4_t *)(srow + c * 8);  // 8 scales
             float acc[MB][NC];
             float xs[MB];
 #pragma unroll
@@ -269,13 +379,13 @@ __global__ __launch_bounds__(WAVES * 64) void awq4_gemv_fast(
                 uint32_t xp[MB][PS];
 #pragma unroll
                 for (int t = 0; t < PS; ++t) {
-                    const int r = kb + 2 * (wave * RPW + sub + t * (WAVES * RPW));
-                    wa[t] = *(const wvec_t *)(qw + (size_t)r * PW + jw);
-                    wb[t] = *(const wvec_t *)(qw + (size_t)(r + 1) * PW + jw);
+                    const int ru = kb + 2 * (wr * RPW + t * (WPG * RPW));  // wave-uniform row
+                    wa[t] = WV::load(rs_w, voff_w, ru * rowbytes);
+                    wb[t] = WV::load(rs_w, voff_w, (ru + 1) * rowbytes);
 #pragma unroll
                     for (int m = 0; m < MB; ++m) {
                         const int mm = m < M ? m : M - 1;
-                        xp[m][t] = *(const uint32_t *)(x + (size_t)mm * K + r);
+                        xp[m][t] = __builtin_amdgcn_raw_buffer_load_b32(rs_x, voff_x, (mm * K + ru) * 2, 0);
                     }
                 }
 #pragma unroll
@@ -283,8 +393,8 @@ __global__ __launch_bounds__(WAVES * 64) void awq4_gemv_fast(
 #pragma unroll
                     for (int c = 0; c < WPL; ++c) {
                         uint32_t p[8];
-                        TT::unpack4(pack_lo16(wa[t][c], wb[t][c]), p);
-                        TT::unpack4(pack_hi16(wa[t][c], wb[t][c]), p + 4);
+                        TT::unpack4(pack_lo16(wa[t][c], wb[t][c]), p, nm);
+                        TT::unpack4(pack_hi16(wa[t][c], wb[t][c]), p + 4, nm);
 #pragma unroll
                         for (int m = 0; m < MB; ++m)
 #pragma unroll
@@ -296,15 +406,13 @@ __global__ __launch_bounds__(WAVES * 64) void awq4_gemv_fast(
                 }
             }
             // group epilogue: remove bias and zero-point, apply the scale
-            const uint16_t *srow = sc + (size_t)g * N + (size_t)jw * 8;
 #pragma unroll
             for (int c = 0; c < WPL; ++c) {
                 const uint32_t zword = zw[c];
-                const u32x4_t sv = *(const u32x4_t *)(srow + c * 8);  // 8 scales
 #pragma unroll
                 for (int s = 0; s < 8; ++s) {
                     const int col = awq_slot_col(s);
-                    const uint32_t spair = sv[col >> 1];
+                    const uint32_t spair = sv[c][col >> 1];
                     const uint16_t sbits = (col & 1) ? (uint16_t)(spair >> 16) : (uint16_t)(spair & 0xFFFFu);
                     const float scale = TT::to_f32(sbits);
                     const float zb = (float)((zword >> (4 * s)) & 0xFu) + TT::bias(s);
@@ -347,6 +455,8 @@ __global__ __launch_bounds__(WAVES * 64) void awq4_gemv_fast(
                     if (S == 1) {
                         const float b = bias ? TT::to_f32(bias[n]) : 0.0f;
                         y[(size_t)m * N + n] = TT::from_f32(tot + b);
+                    } else if (fused) {
+                        st_agent(ws + ((size_t)slice * M + m) * N + n, tot);
                     } else {
                         ws[((size_t)slice * M + m) * N + n] = tot;
                     }
@@ -355,7 +465,7 @@ __global__ __launch_bounds__(WAVES * 64) void awq4_gemv_fast(
             __syncthreads();
         }
     }
-    if (S > 1 && splitk_arrive(counters, blockIdx.x, S))
+    if (S > 1 && fused && splitk_arrive(counters, blockIdx.x, S))
         splitk_finish<TT>(ws, bias, y, M, N, S, n0, SLAB_COLS, WAVES * 64, threadIdx.x);
 }
 
@@ -367,63 +477,99 @@ static int env_int(const char *name, int dflt) {
     return (v && *v) ? atoi(v) : dflt;
 }
 
+// 1: the last workgroup of a tile sums the slices; 0: a second launch does.
+// The fused form saves a launch but its sum runs on one workgroup per tile, so
+// it only pays for few slices.
+static int splitk_fused(const oxq_ctx *ctx, int S) {
+    if (S <= 1) return 0;
+    if (ctx->splitk_mode == 1) return 1;
+    if (ctx->splitk_mode == 2) return 0;
+    return S <= 4 ? 1 : 0;
+}
+
 static int pick_mb(int64_t M) { return M <= 1 ? 1 : (M <= 2 ? 2 : (M <= 4 ? 4 : 8)); }
 
-template <typename TT, int MB, int WPL, int PS>
-static int launch_awq4_fast_t(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p, int gpw, int S) {
-    constexpr int WAVES = 4, RPW = 2;
+template <typename TT, int MB, int WPL, int WPG, int GPB, int RPW, int PS>
+static int launch_awq4_fast_t(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p, int gpw) {
     constexpr int LPR = 64 / RPW;
     const int PW = (int)(p.N / 8);
+    const int G = (int)(p.K >> p.group_shift);
+    const int S = (int)ceil_div(G, gpw);
     dim3 grid((unsigned)ceil_div(PW, LPR * WPL), (unsigned)S);
-    dim3 block(WAVES * 64);
+    dim3 block(WPG * GPB * 64);
     const uint64_t ws_bytes = S > 1 ? (uint64_t)S * p.M * p.N * 4 : 0;
     char name[64];
-    snprintf(name, sizeof name, "awq4_gemv_fast_%s_m%d_w%d_p%d", TT::DTYPE == 1 ? "f16" : "bf16", MB,
-             WPL, PS);
+    snprintf(name, sizeof name, "awq4_gemv_fast_%s_m%d_w%d_g%dx%d_r%d_p%d",
+             TT::DTYPE == 1 ? "f16" : "bf16", MB, WPL, WPG, GPB, RPW, PS);
     set_plan(ctx, name, grid, block, S, 1, ws_bytes);
-    if (ctx->plan_only) return OXQ_OK;
+    if (ctx->plan_only) {
+        if (S > 1 && !splitk_fused(ctx, S)) add_launch(ctx);
+        return OXQ_OK;
+    }
     if (ws_bytes > ctx->workspace_bytes || grid.x > ctx->n_counters)
         return fail(OXQ_ERR_WORKSPACE, "w4a16 gemv: needs %llu workspace bytes, ctx holds %zu",
                     (unsigned long long)ws_bytes, ctx->workspace_bytes);
-    hipLaunchKernelGGL((awq4_gemv_fast<TT, MB, WPL, WAVES, RPW, PS>), grid, block, 0, s,
+    const int fused = splitk_fused(ctx, S);
+    hipLaunchKernelGGL((awq4_gemv_fast<TT, MB, WPL, WPG, GPB, RPW, PS>), grid, block, 0, s,
                        (const uint16_t *)p.x, p.qweight, p.qzeros, (const uint16_t *)p.scales,
                        (const uint16_t *)p.bias, (uint16_t *)p.y, (float *)ctx->workspace,
-                       ctx->counters, (int)p.M, (int)p.K, (int)p.N, p.group_shift, gpw, S);
+                       ctx->counters, (int)p.M, (int)p.K, (int)p.N, p.group_shift, gpw, S, fused);
     OXQ_HIP_CHECK(hipGetLastError());
+    if (S > 1 && !fused)
+        return launch_splitk_reduce(ctx, s, (const float *)ctx->workspace, p.bias, p.y, p.M, p.N, S,
+                                    p.dtype);
     return OXQ_OK;
 }
 
+// Geometry table.  rows per chunk = 2 * WPG * RPW * PS must divide the group size.
 template <typename TT>
 static int launch_awq4_fast(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p) {
     const int mb = pick_mb(p.M);
-    const int wpl = mb == 1 ? 4 : (mb == 2 ? 4 : (mb == 4 ? 2 : 1));
     const int G = (int)(p.K >> p.group_shift);
-    const int slabs = (int)ceil_div(p.N / 8, 32 * wpl);
-    // enough workgroups for ~2 per CU, whole groups per workgroup
-    int target = env_int("OXQ_GEMV_TARGET_WGS", 2 * ctx->num_cus);
-    int S = (int)ceil_div(target, slabs);
-    if (S > G) S = G;
-    if (S < 1) S = 1;
-    int gpw = (int)ceil_div(G, S);
-    gpw = env_int("OXQ_GEMV_GPW", gpw);
-    S = (int)ceil_div(G, gpw);
-    const bool ps8 = p.group_size >= 128;
-#define OXQ_CASE(MBv, WPLv)                                                          \
-    if (mb == MBv && wpl == WPLv)                                                    \
-        return ps8 ? launch_awq4_fast_t<TT, MBv, WPLv, 8>(ctx, s, p, gpw, S)         \
-                   : launch_awq4_fast_t<TT, MBv, WPLv, 4>(ctx, s, p, gpw, S);
-    OXQ_CASE(1, 4)
-    OXQ_CASE(2, 4)
-    OXQ_CASE(4, 2)
-    OXQ_CASE(8, 1)
-#undef OXQ_CASE
-    return fail(OXQ_ERR_UNSUPPORTED, "w4a16 gemv: no kernel for m=%lld", (long long)p.M);
+    const int gs = (int)p.group_size;
+    int cfg = env_int("OXQ_GEMV_CFG", -1);
+    int gpw_env = env_int("OXQ_GEMV_GPW", 0);
+    auto gpw_for = [&](int slab_cols, int gpb) {
+        if (gpw_env > 0) return gpw_env;
+        const int slabs = (int)ceil_div(p.N, slab_cols);
+        int S = (int)ceil_div(ctx->num_cus, slabs);  // about one workgroup per CU
+        if (S > G) S = G;
+        if (S < 1) S = 1;
+        int gpw = (int)ceil_div(G, S);
+        gpw = (int)ceil_div(gpw, gpb) * gpb;       // whole rounds of GPB groups
+        return gpw;
+    };
+    if (mb == 1) {
+        if (cfg < 0) cfg = gs >= 128 ? 4 : 0;  // measured best on MI355X at K=4096, N=14336
+        if (gs >= 128) {
+            switch (cfg) {
+            case 1: return launch_awq4_fast_t<TT, 1, 4, 4, 2, 2, 8>(ctx, s, p, gpw_for(1024, 2));
+            case 2: return launch_awq4_fast_t<TT, 1, 4, 4, 4, 4, 4>(ctx, s, p, gpw_for(512, 4));
+            case 4: return launch_awq4_fast_t<TT, 1, 4, 2, 4, 4, 8>(ctx, s, p, gpw_for(512, 4));
+            case 5: return launch_awq4_fast_t<TT, 1, 4, 1, 8, 8, 8>(ctx, s, p, gpw_for(256, 8));
+            case 6: return launch_awq4_fast_t<TT, 1, 4, 1, 4, 8, 8>(ctx, s, p, gpw_for(256, 4));
+            default: return launch_awq4_fast_t<TT, 1, 4, 4, 1, 2, 8>(ctx, s, p, gpw_for(1024, 1));
+            }
+        }
+        return launch_awq4_fast_t<TT, 1, 4, 4, 1, 2, 4>(ctx, s, p, gpw_for(1024, 1));
+    }
+    const bool ps8 = gs >= 128;
+    if (mb == 2)
+        return ps8 ? launch_awq4_fast_t<TT, 2, 4, 4, 1, 2, 8>(ctx, s, p, gpw_for(1024, 1))
+                   : launch_awq4_fast_t<TT, 2, 4, 4, 1, 2, 4>(ctx, s, p, gpw_for(1024, 1));
+    if (mb == 4)
+        return ps8 ? launch_awq4_fast_t<TT, 4, 2, 4, 1, 2, 8>(ctx, s, p, gpw_for(512, 1))
+                   : launch_awq4_fast_t<TT, 4, 2, 4, 1, 2, 4>(ctx, s, p, gpw_for(512, 1));
+    return ps8 ? launch_awq4_fast_t<TT, 8, 1, 4, 1, 2, 8>(ctx, s, p, gpw_for(256, 1))
+               : launch_awq4_fast_t<TT, 8, 1, 4, 1, 2, 4>(ctx, s, p, gpw_for(256, 1));
 }
 
 static bool awq4_fast_ok(const Wna16Problem &p) {
     if (p.bits != 4 || p.pack_dim != OXQ_PACK_OUT) return false;
     if (p.N % 32 != 0 || p.K % 2 != 0) return false;
-    if (p.group_size < 64) return false;  // 2 * WAVES * RPW * PS rows per chunk
+    if (p.group_size < 64) return false;  // 2 * WPG * RPW * PS rows per chunk
+    if ((uint64_t)p.K * (uint64_t)(p.N / 2) >= (1ull << 31)) return false;  // 32-bit buffer offsets
+    if ((uint64_t)p.M * (uint64_t)p.K * 2 >= (1ull << 31)) return false;
     if (((uintptr_t)p.qweight | (uintptr_t)p.qzeros | (uintptr_t)p.scales) & 15) return false;
     if ((uintptr_t)p.x & 3) return false;
     return true;
@@ -449,7 +595,12 @@ static int launch_generic_t(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p) 
     snprintf(name, sizeof name, "%s_gemv_generic_w%d_%s_m%d", awq ? "awq" : "gptq", BITS,
              TT::DTYPE == 1 ? "f16" : "bf16", mb);
     set_plan(ctx, name, grid, block, S, 1, ws_bytes);
-    if (ctx->plan_only) return OXQ_OK;
+    // the stand-alone reduce handles 4 outputs per thread
+    const int fused = (p.N % 4 != 0 && S > 1) ? 1 : splitk_fused(ctx, S);
+    if (ctx->plan_only) {
+        if (S > 1 && !fused) add_launch(ctx);
+        return OXQ_OK;
+    }
     if (ws_bytes > ctx->workspace_bytes || grid.x > ctx->n_counters)
         return fail(OXQ_ERR_WORKSPACE, "wna16 gemv: needs %llu workspace bytes, ctx holds %zu",
                     (unsigned long long)ws_bytes, ctx->workspace_bytes);
@@ -459,12 +610,12 @@ static int launch_generic_t(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p) 
                            (const uint16_t *)p.x, p.qweight, p.qzeros, (const uint16_t *)p.scales, \
                            (const uint16_t *)p.bias, (uint16_t *)p.y, (float *)ctx->workspace,   \
                            ctx->counters, (int)p.M, (int)p.K, (int)p.N, (int)(p.N / PF),         \
-                           p.group_shift, (int)chunk, S);                                        \
+                           p.group_shift, (int)chunk, S, fused);                                 \
     else                                                                                         \
         hipLaunchKernelGGL((gptq_gemv_generic<TT, BITS, MBv>), grid, block, 0, s,                \
                            (const uint16_t *)p.x, p.qweight, p.qzeros, (const uint16_t *)p.scales, \
                            (const uint16_t *)p.bias, (uint16_t *)p.y, (float *)ctx->workspace,   \
-                           ctx->counters, (int)p.M, (int)p.K, (int)p.N, p.group_shift, (int)chunk, S)
+                           ctx->counters, (int)p.M, (int)p.K, (int)p.N, p.group_shift, (int)chunk, S, fused)
     switch (mb) {
     case 1: OXQ_GO(1); break;
     case 2: OXQ_GO(2); break;
@@ -473,6 +624,9 @@ static int launch_generic_t(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p) 
     }
 #undef OXQ_GO
     OXQ_HIP_CHECK(hipGetLastError());
+    if (S > 1 && !fused)
+        return launch_splitk_reduce(ctx, s, (const float *)ctx->workspace, p.bias, p.y, p.M, p.N, S,
+                                    p.dtype);
     return OXQ_OK;
 }
 

@@ -17,7 +17,7 @@
 // exact 16-bit integers, then (q - z) * s is a packed add + packed multiply.
 //
 // A workgroup of 4 waves covers 16*MT rows x 512 columns; K is split across
-// workgroups and combined with the deterministic last-arriver protocol.
+// workgroups; the slices are summed in index order by a second launch.
 
 #include "oxq_device.hpp"
 #include "oxq_internal.hpp"
@@ -71,11 +71,13 @@ __global__ __launch_bounds__(256) void awq4_mfma_kernel(
     const uint16_t *__restrict__ x, const uint32_t *__restrict__ qw,
     const uint32_t *__restrict__ qz, const uint16_t *__restrict__ sc,
     const uint16_t *__restrict__ bias, uint16_t *__restrict__ y, float *__restrict__ ws,
-    unsigned *__restrict__ counters, int M, int K, int N, int gshift, int kslice, int S) {
+    int M, int K, int N, int gshift, int kslice, int S) {
     typedef MfmaOps<TT> Ops;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int c = lane & 15, kb = lane >> 4;
     const int PW = N >> 3;
+    const int rowbytes = PW * 4;
     const int jw = blockIdx.x * 64 + wave * 16 + c;  // packed word column of this lane
     const bool col_ok = jw < PW;
     const int jws = col_ok ? jw : PW - 1;            // clamp loads, discard results
@@ -83,6 +85,24 @@ __global__ __launch_bounds__(256) void awq4_mfma_kernel(
     const int m0 = blockIdx.z * (16 * MT);
     const int k_begin = slice * kslice;
     const int k_end = min(K, k_begin + kslice);
+    const int gsize = 1 << gshift;
+
+    // Raw buffer addressing: lane part in a VGPR offset, row part in a scalar offset.
+    const __amdgpu_buffer_rsrc_t rs_w = make_rsrc(qw, (uint32_t)K * (uint32_t)rowbytes);
+    const __amdgpu_buffer_rsrc_t rs_x = make_rsrc(x, (uint32_t)M * (uint32_t)K * 2u);
+    const __amdgpu_buffer_rsrc_t rs_z = make_rsrc(qz, (uint32_t)(K >> gshift) * (uint32_t)rowbytes);
+    const __amdgpu_buffer_rsrc_t rs_s = make_rsrc(sc, (uint32_t)(K >> gshift) * (uint32_t)N * 2u);
+    const int voff_w = (kb * 8 * PW + jws) * 4;
+    const int voff_z = jws * 4;
+    const int voff_s = jws * 16;
+    int voff_a[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        int r = m0 + mt * 16 + c;
+        r = r < M ? r : M - 1;  // extra rows are computed and discarded
+        voff_a[mt] = (r * K + kb * 8) * 2;
+    }
+    const NibbleMasks nm = nibble_masks();
 
     float4_t acc[MT][8];
 #pragma unroll
@@ -90,54 +110,84 @@ __global__ __launch_bounds__(256) void awq4_mfma_kernel(
 #pragma unroll
         for (int s = 0; s < 8; ++s) acc[mt][s] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-    // activation rows of this lane's A fragments (clamped; extra rows are discarded)
-    const uint16_t *xrow[MT];
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-        int r = m0 + mt * 16 + c;
-        r = r < M ? r : M - 1;
-        xrow[mt] = x + (size_t)r * K;
-    }
-
-    uint32_t negzb[8], sp[8];
-    int cur_g = -1;
-    for (int k0 = k_begin; k0 < k_end; k0 += 32) {
-        const int g = k0 >> gshift;
-        if (g != cur_g) {  // wave-uniform
-            const uint32_t zw = qz[(size_t)g * PW + jws];
-            const u32x4_t sv = *(const u32x4_t *)(sc + (size_t)g * N + (size_t)jws * 8);
-#pragma unroll
-            for (int s = 0; s < 8; ++s) {
-                const int col = awq_slot_col(s);
-                const uint32_t pr = sv[col >> 1];
-                const uint32_t sb = (col & 1) ? (pr >> 16) : (pr & 0xFFFFu);
-                sp[s] = sb | (sb << 16);
-                negzb[s] = Ops::splat(-((float)((zw >> (4 * s)) & 0xFu) + TT::bias(s)));
-            }
-            cur_g = g;
-        }
+    struct Step {
         uint32_t w[8];
+        u32x4_t a[MT];
+    };
+    auto load_step = [&](int k0, Step &st) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) w[i] = qw[(size_t)(k0 + kb * 8 + i) * PW + jws];
-        uint32_t a[MT][4];
+        for (int i = 0; i < 8; ++i)
+            st.w[i] = __builtin_amdgcn_raw_buffer_load_b32(rs_w, voff_w, (k0 + i) * rowbytes, 0);
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            const u32x4_t av = *(const u32x4_t *)(xrow[mt] + k0 + kb * 8);
-            a[mt][0] = av[0]; a[mt][1] = av[1]; a[mt][2] = av[2]; a[mt][3] = av[3];
+        for (int mt = 0; mt < MT; ++mt)
+            st.a[mt] = __builtin_amdgcn_raw_buffer_load_b128(rs_x, voff_a[mt], k0 * 2, 0);
+    };
+
+    // group parameters, fetched one group ahead of use
+    uint32_t zw_next;
+    u32x4_t sv_next;
+    auto load_group = [&](int g) {
+        zw_next = __builtin_amdgcn_raw_buffer_load_b32(rs_z, voff_z, g * rowbytes, 0);
+        sv_next = __builtin_amdgcn_raw_buffer_load_b128(rs_s, voff_s, g * N * 2, 0);
+    };
+    uint32_t negzb[8], sp[8];
+    auto use_group = [&]() {
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            const int col = awq_slot_col(s);
+            const uint32_t pr = sv_next[col >> 1];
+            const uint32_t sb = (col & 1) ? (pr >> 16) : (pr & 0xFFFFu);
+            sp[s] = sb | (sb << 16);
+            negzb[s] = Ops::splat(-((float)((zw_next >> (4 * s)) & 0xFu) + TT::bias(s)));
         }
-        uint32_t b[8][4];
+    };
+    auto compute = [&](const Step &st) {
+        // one fragment (8 consecutive k of one column set) at a time keeps few registers live
+        uint32_t tl[4], th[4];
 #pragma unroll
         for (int pp = 0; pp < 4; ++pp) {
-            uint32_t p[8];
-            TT::unpack4(pack_lo16(w[2 * pp], w[2 * pp + 1]), p);
-            TT::unpack4(pack_hi16(w[2 * pp], w[2 * pp + 1]), p + 4);
-#pragma unroll
-            for (int s = 0; s < 8; ++s) b[s][pp] = Ops::dequant_pair(p[s], negzb[s], sp[s]);
+            tl[pp] = pack_lo16(st.w[2 * pp], st.w[2 * pp + 1]);
+            th[pp] = pack_hi16(st.w[2 * pp], st.w[2 * pp + 1]);
         }
 #pragma unroll
-        for (int s = 0; s < 8; ++s)
+        for (int s = 0; s < 8; ++s) {
+            uint32_t b[4];
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) acc[mt][s] = Ops::mfma(a[mt], b[s], acc[mt][s]);
+            for (int pp = 0; pp < 4; ++pp) {
+                const uint32_t pr = TT::unpack1(s < 4 ? tl[pp] : th[pp], s & 3, nm);
+                b[pp] = Ops::dequant_pair(pr, negzb[s], sp[s]);
+            }
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const uint32_t a[4] = {st.a[mt][0], st.a[mt][1], st.a[mt][2], st.a[mt][3]};
+                acc[mt][s] = Ops::mfma(a, b, acc[mt][s]);
+            }
+        }
+    };
+    // A K-step of 32 rows never straddles a group (group size is a multiple of 32).
+    auto step_group = [&](int k0) {
+        if ((k0 & (gsize - 1)) == 0 || k0 == k_begin) {  // wave-uniform
+            use_group();
+            const int gn = (k0 >> gshift) + 1;
+            if ((gn << gshift) < k_end) load_group(gn);
+        }
+    };
+
+    Step sa, sb;
+    if (k_begin < k_end) {
+        load_group(k_begin >> gshift);
+        load_step(k_begin, sa);
+    }
+    for (int k0 = k_begin; k0 < k_end; k0 += 64) {
+        const bool has_b = k0 + 32 < k_end;
+        if (has_b) load_step(k0 + 32, sb);
+        step_group(k0);
+        compute(sa);
+        if (has_b) {
+            if (k0 + 64 < k_end) load_step(k0 + 64, sa);
+            step_group(k0 + 32);
+            compute(sb);
+        }
     }
 
     // D layout: lane (c, rb = lane / 16) holds rows 4*rb + i, column c of each tile.
@@ -172,18 +222,395 @@ __global__ __launch_bounds__(256) void awq4_mfma_kernel(
             }
         }
     }
-    if (S > 1 && splitk_arrive(counters, blockIdx.z * gridDim.x + blockIdx.x, S)) {
-        const int tile_cols = 512;
-        const int n0 = blockIdx.x * tile_cols;
-        const int rows = min(16 * MT, M - m0);
-        for (int idx = threadIdx.x; idx < rows * tile_cols; idx += 256) {
-            const int m = m0 + idx / tile_cols;
-            const int n = n0 + idx % tile_cols;
-            if (n >= N) continue;
-            float tot = 0.0f;
-            for (int s = 0; s < S; ++s) tot += ws[((size_t)s * M + m) * N + n];
-            if (bias) tot += TT::to_f32(bias[n]);
-            y[(size_t)m * N + n] = TT::from_f32(tot);
+}
+
+// ---------------------------------------------------------------------------
+// Pipelined variant for group sizes >= 128.
+//
+// One workgroup iteration = a K block of 128 rows (4 MFMA steps).  The
+// activation tile of the block is staged in LDS (double buffered, padded rows
+// so the 16 lanes of a fragment read hit distinct banks) and shared by the 4
+// waves; packed weights are prefetched 4 steps ahead into a register ring, so
+// a wave has ~8 KB of weight loads in flight.  With one wave per SIMD (the
+// 64-row tile needs 128 accumulator registers) that ring is what hides HBM
+// latency.
+// ---------------------------------------------------------------------------
+template <typename TT, int MT>
+__global__ __launch_bounds__(256) void awq4_mfma_pipe_kernel(
+    const uint16_t *__restrict__ x, const uint32_t *__restrict__ qw,
+    const uint32_t *__restrict__ qz, const uint16_t *__restrict__ sc,
+    const uint16_t *__restrict__ bias, uint16_t *__restrict__ y, float *__restrict__ ws,
+    int M, int K, int N, int gshift, int kslice, int S) {
+    typedef MfmaOps<TT> Ops;
+    constexpr int KB = 128;                 // K rows per block
+    constexpr int D = KB / 32;              // MFMA steps per block = prefetch depth
+    constexpr int ROWS = 16 * MT;
+    constexpr int RS = KB * 2 + 16;         // padded LDS row stride in bytes
+    constexpr int CHUNKS = ROWS * (KB / 8); // 16-byte chunks per activation block
+    constexpr int CPT = (CHUNKS + 255) / 256;
+    __shared__ __attribute__((aligned(16))) unsigned char lds_a[2][ROWS * RS];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int c = lane & 15, kb = lane >> 4;
+    const int PW = N >> 3;
+    const int rowbytes = PW * 4;
+    const int jw = blockIdx.x * 64 + wave * 16 + c;
+    const bool col_ok = jw < PW;
+    const int jws = col_ok ? jw : PW - 1;
+    const int slice = blockIdx.y;
+    const int m0 = blockIdx.z * ROWS;
+    const int k_begin = slice * kslice;
+    const int k_end = min(K, k_begin + kslice);
+    const int nblk = (k_end - k_begin) / KB;
+    const int gsize = 1 << gshift;
+
+    const __amdgpu_buffer_rsrc_t rs_w = make_rsrc(qw, (uint32_t)K * (uint32_t)rowbytes);
+    const __amdgpu_buffer_rsrc_t rs_x = make_rsrc(x, (uint32_t)M * (uint32_t)K * 2u);
+    const __amdgpu_buffer_rsrc_t rs_z = make_rsrc(qz, (uint32_t)(K >> gshift) * (uint32_t)rowbytes);
+    const __amdgpu_buffer_rsrc_t rs_s = make_rsrc(sc, (uint32_t)(K >> gshift) * (uint32_t)N * 2u);
+    const int voff_w = (kb * 8 * PW + jws) * 4;
+    const int voff_z = jws * 4;
+    const int voff_s = jws * 16;
+    const NibbleMasks nm = nibble_masks();
+
+    // staging map: chunk q of this thread -> (row, 8-k chunk) of the activation block
+    int a_goff[CPT], a_loff[CPT];
+#pragma unroll
+    for (int q = 0; q < CPT; ++q) {
+        const int idx = threadIdx.x + q * 256;
+        const int row = idx / (KB / 8), kc = idx % (KB / 8);
+        int r = m0 + row;
+        r = r < M ? r : M - 1;
+        a_goff[q] = (r * K + kc * 8) * 2;
+        a_loff[q] = (idx < CHUNKS) ? row * RS + kc * 16 : -1;
+    }
+    int a_roff[MT];  // LDS offset of this lane's fragment inside a block, step 0
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) a_roff[mt] = (mt * 16 + c) * RS + kb * 16;
+
+    float4_t acc[MT][8];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int s = 0; s < 8; ++s) acc[mt][s] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    uint32_t ring[D][8];
+    auto load_w = [&](int k0, uint32_t (&w)[8]) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            w[i] = __builtin_amdgcn_raw_buffer_load_b32(rs_w, voff_w, (k0 + i) * rowbytes, 0);
+    };
+    u32x4_t areg[CPT];
+    auto load_a = [&](int k0) {
+#pragma unroll
+        for (int q = 0; q < CPT; ++q)
+            areg[q] = __builtin_amdgcn_raw_buffer_load_b128(rs_x, a_goff[q], k0 * 2, 0);
+    };
+    auto store_a = [&](int buf) {
+#pragma unroll
+        for (int q = 0; q < CPT; ++q)
+            if (a_loff[q] >= 0) *(u32x4_t *)(&lds_a[buf][a_loff[q]]) = areg[q];
+    };
+
+    uint32_t zw_next;
+    u32x4_t sv_next;
+    auto load_group = [&](int g) {
+        zw_next = __builtin_amdgcn_raw_buffer_load_b32(rs_z, voff_z, g * rowbytes, 0);
+        sv_next = __builtin_amdgcn_raw_buffer_load_b128(rs_s, voff_s, g * N * 2, 0);
+    };
+    uint32_t negzb[8], sp[8];
+    auto use_group = [&]() {
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            const int col = awq_slot_col(s);
+            const uint32_t pr = sv_next[col >> 1];
+            const uint32_t sb = (col & 1) ? (pr >> 16) : (pr & 0xFFFFu);
+            sp[s] = sb | (sb << 16);
+            negzb[s] = Ops::splat(-((float)((zw_next >> (4 * s)) & 0xFu) + TT::bias(s)));
+        }
+    };
+
+    if (nblk > 0) {
+        load_group(k_begin >> gshift);
+        load_a(k_begin);
+#pragma unroll
+        for (int d = 0; d < D; ++d) load_w(k_begin + d * 32, ring[d]);
+        store_a(0);
+    }
+    __syncthreads();
+
+    for (int blk = 0; blk < nblk; ++blk) {
+        const int kblk = k_begin + blk * KB;
+        const bool more = blk + 1 < nblk;
+        if (more) load_a(kblk + KB);
+        if ((kblk & (gsize - 1)) == 0 || blk == 0) {  // wave-uniform: entering a new group
+            use_group();
+            const int gn = (kblk >> gshift) + 1;
+            if ((gn << gshift) < k_end) load_group(gn);
+        }
+        const unsigned char *abuf = lds_a[blk & 1];
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+            u32x4_t af[MT];
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) af[mt] = *(const u32x4_t *)(abuf + a_roff[mt] + d * 64);
+            uint32_t tl[4], th[4];
+#pragma unroll
+            for (int pp = 0; pp < 4; ++pp) {
+                tl[pp] = pack_lo16(ring[d][2 * pp], ring[d][2 * pp + 1]);
+                th[pp] = pack_hi16(ring[d][2 * pp], ring[d][2 * pp + 1]);
+            }
+            if (more) load_w(kblk + KB + d * 32, ring[d]);  // refill this ring slot
+#pragma unroll
+            for (int s = 0; s < 8; ++s) {
+                uint32_t b[4];
+#pragma unroll
+                for (int pp = 0; pp < 4; ++pp) {
+                    const uint32_t pr = TT::unpack1(s < 4 ? tl[pp] : th[pp], s & 3, nm);
+                    b[pp] = Ops::dequant_pair(pr, negzb[s], sp[s]);
+                }
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+                    const uint32_t a[4] = {af[mt][0], af[mt][1], af[mt][2], af[mt][3]};
+                    acc[mt][s] = Ops::mfma(a, b, acc[mt][s]);
+                }
+            }
+        }
+        if (more) store_a((blk + 1) & 1);
+        __syncthreads();
+    }
+
+    const int rb = kb;
+    const int nbase = jw * 8;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int m = m0 + mt * 16 + rb * 4 + i;
+            if (m < M && col_ok) {
+                float v[8];
+#pragma unroll
+                for (int s = 0; s < 8; ++s) v[awq_slot_col(s)] = acc[mt][s][i];
+                if (S == 1) {
+                    uint32_t o[4];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        float lo = v[2 * q], hi = v[2 * q + 1];
+                        if (bias) {
+                            lo += TT::to_f32(bias[nbase + 2 * q]);
+                            hi += TT::to_f32(bias[nbase + 2 * q + 1]);
+                        }
+                        o[q] = (uint32_t)TT::from_f32(lo) | ((uint32_t)TT::from_f32(hi) << 16);
+                    }
+                    *(u32x4_t *)(y + (size_t)m * N + nbase) = u32x4_t{o[0], o[1], o[2], o[3]};
+                } else {
+                    float *dst = ws + ((size_t)slice * M + m) * N + nbase;
+                    *(float4_t *)dst = float4_t{v[0], v[1], v[2], v[3]};
+                    *(float4_t *)(dst + 4) = float4_t{v[4], v[5], v[6], v[7]};
+                }
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// K-split-in-workgroup variant: the 4 waves of a workgroup share one
+// 16*MT x 128 output tile and each takes a quarter of the workgroup's K range;
+// their accumulators are combined through LDS.  Compared with four waves side
+// by side this quarters the number of f32 partial tiles that cross workgroups
+// (the dominant cost of the 64-row tile), at the price of 64-byte row segments
+// per wave.  Workgroup ids are remapped so that the two tiles sharing a
+// 128-byte line of every weight row run on the same XCD (shared L2).
+// Activations come straight from L2 into a register double buffer; packed
+// weights are prefetched 4 steps ahead.
+// ---------------------------------------------------------------------------
+template <typename TT, int MT>
+__global__ __launch_bounds__(256) void awq4_mfma_ksplit_kernel(
+    const uint16_t *__restrict__ x, const uint32_t *__restrict__ qw,
+    const uint32_t *__restrict__ qz, const uint16_t *__restrict__ sc,
+    const uint16_t *__restrict__ bias, uint16_t *__restrict__ y, float *__restrict__ ws,
+    int M, int K, int N, int gshift, int kslice, int S, int ctiles) {
+    typedef MfmaOps<TT> Ops;
+    constexpr int D = 4;  // weight prefetch depth in 32-row steps
+    __shared__ __attribute__((aligned(16))) float red[MT * 8 * 64 * 4];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int c = lane & 15, kb = lane >> 4;
+    const int PW = N >> 3;
+    const int rowbytes = PW * 4;
+
+    // XCD-aware id remap: ids b and b+8 (same XCD, dispatched together) get adjacent tiles
+    const int total = ctiles * S;
+    int u = blockIdx.x;
+    if (u < (total / 16) * 16) {
+        const int xcd = u & 7, q = u >> 3;
+        u = (q >> 1) * 16 + xcd * 2 + (q & 1);
+    }
+    const int tile = u % ctiles, slice = u / ctiles;
+
+    const int jw = tile * 16 + c;
+    const bool col_ok = jw < PW;
+    const int jws = col_ok ? jw : PW - 1;
+    const int m0 = blockIdx.z * (16 * MT);
+    const int kq = kslice >> 2;                       // this wave's share of the slice
+    const int k_begin = slice * kslice + wave * kq;
+    const int k_end = min(K, k_begin + kq);
+    const int nsteps = k_end > k_begin ? (k_end - k_begin) >> 5 : 0;
+    const int gsize = 1 << gshift;
+
+    const __amdgpu_buffer_rsrc_t rs_w = make_rsrc(qw, (uint32_t)K * (uint32_t)rowbytes);
+    const __amdgpu_buffer_rsrc_t rs_x = make_rsrc(x, (uint32_t)M * (uint32_t)K * 2u);
+    const __amdgpu_buffer_rsrc_t rs_z = make_rsrc(qz, (uint32_t)(K >> gshift) * (uint32_t)rowbytes);
+    const __amdgpu_buffer_rsrc_t rs_s = make_rsrc(sc, (uint32_t)(K >> gshift) * (uint32_t)N * 2u);
+    const int voff_w = (kb * 8 * PW + jws) * 4;
+    const int voff_z = jws * 4;
+    const int voff_s = jws * 16;
+    int voff_a[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        int r = m0 + mt * 16 + c;
+        r = r < M ? r : M - 1;
+        voff_a[mt] = (r * K + kb * 8) * 2;
+    }
+    const NibbleMasks nm = nibble_masks();
+
+    float4_t acc[MT][8];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int s = 0; s < 8; ++s) acc[mt][s] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    uint32_t ring[D][8];
+    auto load_w = [&](int k0, uint32_t (&w)[8]) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            w[i] = __builtin_amdgcn_raw_buffer_load_b32(rs_w, voff_w, (k0 + i) * rowbytes, 0);
+    };
+    u32x4_t abuf[2][MT];
+    auto load_a = [&](int k0, u32x4_t (&a)[MT]) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+            a[mt] = __builtin_amdgcn_raw_buffer_load_b128(rs_x, voff_a[mt], k0 * 2, 0);
+    };
+    uint32_t zw_next;
+    u32x4_t sv_next;
+    auto load_group = [&](int g) {
+        zw_next = __builtin_amdgcn_raw_buffer_load_b32(rs_z, voff_z, g * rowbytes, 0);
+        sv_next = __builtin_amdgcn_raw_buffer_load_b128(rs_s, voff_s, g * N * 2, 0);
+    };
+    uint32_t negzb[8], sp[8];
+    auto use_group = [&]() {
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            const int col = awq_slot_col(s);
+            const uint32_t pr = sv_next[col >> 1];
+            const uint32_t sb = (col & 1) ? (pr >> 16) : (pr & 0xFFFFu);
+            sp[s] = sb | (sb << 16);
+            negzb[s] = Ops::splat(-((float)((zw_next >> (4 * s)) & 0xFu) + TT::bias(s)));
+        }
+    };
+    auto compute = [&](const uint32_t (&w)[8], const u32x4_t (&a)[MT], uint32_t (&tl)[4], uint32_t (&th)[4]) {
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            uint32_t b[4];
+#pragma unroll
+            for (int pp = 0; pp < 4; ++pp) {
+                const uint32_t pr = TT::unpack1(s < 4 ? tl[pp] : th[pp], s & 3, nm);
+                b[pp] = Ops::dequant_pair(pr, negzb[s], sp[s]);
+            }
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const uint32_t av[4] = {a[mt][0], a[mt][1], a[mt][2], a[mt][3]};
+                acc[mt][s] = Ops::mfma(av, b, acc[mt][s]);
+            }
+        }
+        (void)w;
+    };
+
+    if (nsteps > 0) {
+        load_group(k_begin >> gshift);
+        load_a(k_begin, abuf[0]);
+#pragma unroll
+        for (int d = 0; d < D; ++d)
+            if (d < nsteps) load_w(k_begin + d * 32, ring[d]);
+    }
+    // steps are processed in rounds of D so ring slots are compile-time indices
+    for (int base = 0; base < nsteps; base += D) {
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+            const int si = base + d;
+            if (si < nsteps) {  // wave-uniform
+                const int k0 = k_begin + si * 32;
+                if (si + 1 < nsteps) load_a(k0 + 32, abuf[(d + 1) & 1]);
+                if ((k0 & (gsize - 1)) == 0 || si == 0) {
+                    use_group();
+                    const int gn = (k0 >> gshift) + 1;
+                    if ((gn << gshift) < k_end) load_group(gn);
+                }
+                uint32_t tl[4], th[4];
+#pragma unroll
+                for (int pp = 0; pp < 4; ++pp) {
+                    tl[pp] = pack_lo16(ring[d][2 * pp], ring[d][2 * pp + 1]);
+                    th[pp] = pack_hi16(ring[d][2 * pp], ring[d][2 * pp + 1]);
+                }
+                if (si + D < nsteps) load_w(k0 + D * 32, ring[d]);
+                compute(ring[d], abuf[d & 1], tl, th);
+            }
+        }
+    }
+
+    // combine the four K quarters: waves 1..3 hand their accumulators to wave 0
+    for (int r = 1; r < 4; ++r) {
+        if (wave == r) {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int s = 0; s < 8; ++s)
+                    *(float4_t *)(&red[((mt * 8 + s) * 64 + lane) * 4]) = acc[mt][s];
+        }
+        __syncthreads();
+        if (wave == 0) {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int s = 0; s < 8; ++s)
+                    acc[mt][s] += *(const float4_t *)(&red[((mt * 8 + s) * 64 + lane) * 4]);
+        }
+        __syncthreads();
+    }
+    if (wave != 0) return;
+
+    const int rb = kb;
+    const int nbase = jw * 8;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int m = m0 + mt * 16 + rb * 4 + i;
+            if (m < M && col_ok) {
+                float v[8];
+#pragma unroll
+                for (int s = 0; s < 8; ++s) v[awq_slot_col(s)] = acc[mt][s][i];
+                if (S == 1) {
+                    uint32_t o[4];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        float lo = v[2 * q], hi = v[2 * q + 1];
+                        if (bias) {
+                            lo += TT::to_f32(bias[nbase + 2 * q]);
+                            hi += TT::to_f32(bias[nbase + 2 * q + 1]);
+                        }
+                        o[q] = (uint32_t)TT::from_f32(lo) | ((uint32_t)TT::from_f32(hi) << 16);
+                    }
+                    *(u32x4_t *)(y + (size_t)m * N + nbase) = u32x4_t{o[0], o[1], o[2], o[3]};
+                } else {
+                    float *dst = ws + ((size_t)slice * M + m) * N + nbase;
+                    *(float4_t *)dst = float4_t{v[0], v[1], v[2], v[3]};
+                    *(float4_t *)(dst + 4) = float4_t{v[4], v[5], v[6], v[7]};
+                }
+            }
         }
     }
 }
@@ -196,8 +623,59 @@ static int env_int(const char *name, int dflt) {
 template <typename TT>
 static int launch_awq4_mfma(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p) {
     const int M = (int)p.M, K = (int)p.K, N = (int)p.N;
-    const int mt = M <= 16 ? 1 : (M <= 32 ? 2 : (M <= 48 ? 3 : 4));
+    int mt = M <= 16 ? 1 : (M <= 32 ? 2 : (M <= 48 ? 3 : 4));
+    {
+        const int mt_env = env_int("OXQ_MFMA_MT", 0);
+        if (mt_env >= 1 && mt_env <= 4 && mt_env < mt) mt = mt_env;
+    }
     const int mtiles = (int)ceil_div(M, 16 * mt);
+    const char *dt = TT::DTYPE == 1 ? "f16" : "bf16";
+    char name[64];
+
+    // --- K split inside the workgroup: 128-column tiles, slices of whole 512-row units
+    const int variant = env_int("OXQ_MFMA_VARIANT", 0);  // 0 auto (pipe), 1 ksplit, 2 pipe, 3 simple
+    if (variant == 1 && p.group_size >= 32 && K % 512 == 0 &&
+        (512 % p.group_size == 0 || p.group_size % 512 == 0)) {
+        const int ctiles = (int)ceil_div(N, 128);
+        const int units = K / 512;
+        int S = env_int("OXQ_MFMA_SPLITK", (int)ceil_div(ctx->num_cus, (int64_t)ctiles * mtiles));
+        if (S < 1) S = 1;
+        if (S > units) S = units;
+        int kslice = (int)ceil_div(units, S) * 512;
+        S = (int)ceil_div(K, kslice);
+        while (S > 1 && (uint64_t)S * M * N * 4 > ctx->workspace_bytes) {
+            --S;
+            kslice = (int)ceil_div(units, S) * 512;
+            S = (int)ceil_div(K, kslice);
+        }
+        dim3 grid((unsigned)(ctiles * S), 1, (unsigned)mtiles), block(256);
+        const uint64_t ws_bytes = S > 1 ? (uint64_t)S * M * N * 4 : 0;
+        snprintf(name, sizeof name, "awq4_mfma_ksplit_%s_mt%d", dt, mt);
+        set_plan(ctx, name, grid, block, S, 1, ws_bytes);
+        if (ctx->plan_only) {
+            if (S > 1) add_launch(ctx);
+            return OXQ_OK;
+        }
+#define OXQ_GO(MTv)                                                                                \
+    hipLaunchKernelGGL((awq4_mfma_ksplit_kernel<TT, MTv>), grid, block, 0, s, (const uint16_t *)p.x, \
+                       p.qweight, p.qzeros, (const uint16_t *)p.scales, (const uint16_t *)p.bias,  \
+                       (uint16_t *)p.y, (float *)ctx->workspace, M, K, N, p.group_shift, kslice, S, \
+                       ctiles)
+        switch (mt) {
+        case 1: OXQ_GO(1); break;
+        case 2: OXQ_GO(2); break;
+        case 3: OXQ_GO(3); break;
+        default: OXQ_GO(4); break;
+        }
+#undef OXQ_GO
+        OXQ_HIP_CHECK(hipGetLastError());
+        if (S > 1)
+            return launch_splitk_reduce(ctx, s, (const float *)ctx->workspace, p.bias, p.y, M, N, S,
+                                        p.dtype);
+        return OXQ_OK;
+    }
+
+    // --- four waves side by side: 512-column tiles
     const int ctiles = (int)ceil_div(N, 512);
     // K slices: whole groups (and whole 32-row MFMA steps), about one workgroup per CU
     const int step = (int)(p.group_size > 32 ? p.group_size : 32);
@@ -213,18 +691,27 @@ static int launch_awq4_mfma(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p) 
     S = (int)ceil_div(K, kslice2);
     dim3 grid((unsigned)ctiles, (unsigned)S, (unsigned)mtiles), block(256);
     const uint64_t ws_bytes = S > 1 ? (uint64_t)S * M * N * 4 : 0;
-    char name[64];
-    snprintf(name, sizeof name, "awq4_mfma_%s_mt%d", TT::DTYPE == 1 ? "f16" : "bf16", mt);
+    const bool pipe = variant != 3 && p.group_size >= 128 && kslice2 % 128 == 0 && K % 128 == 0;
+    snprintf(name, sizeof name, "awq4_mfma%s_%s_mt%d", pipe ? "_pipe" : "", dt, mt);
     set_plan(ctx, name, grid, block, S, 1, ws_bytes);
-    if (ctx->plan_only) return OXQ_OK;
-    if (ws_bytes > ctx->workspace_bytes || (size_t)ctiles * mtiles > ctx->n_counters)
+    if (ctx->plan_only) {
+        if (S > 1) add_launch(ctx);
+        return OXQ_OK;
+    }
+    if (ws_bytes > ctx->workspace_bytes)
         return fail(OXQ_ERR_WORKSPACE, "w4a16 tile gemm: needs %llu workspace bytes, ctx holds %zu",
                     (unsigned long long)ws_bytes, ctx->workspace_bytes);
 #define OXQ_GO(MTv)                                                                              \
-    hipLaunchKernelGGL((awq4_mfma_kernel<TT, MTv>), grid, block, 0, s, (const uint16_t *)p.x,    \
-                       p.qweight, p.qzeros, (const uint16_t *)p.scales, (const uint16_t *)p.bias, \
-                       (uint16_t *)p.y, (float *)ctx->workspace, ctx->counters, M, K, N,         \
-                       p.group_shift, kslice2, S)
+    if (pipe)                                                                                    \
+        hipLaunchKernelGGL((awq4_mfma_pipe_kernel<TT, MTv>), grid, block, 0, s,                  \
+                           (const uint16_t *)p.x, p.qweight, p.qzeros, (const uint16_t *)p.scales, \
+                           (const uint16_t *)p.bias, (uint16_t *)p.y, (float *)ctx->workspace, M, K, \
+                           N, p.group_shift, kslice2, S);                                        \
+    else                                                                                         \
+        hipLaunchKernelGGL((awq4_mfma_kernel<TT, MTv>), grid, block, 0, s, (const uint16_t *)p.x, \
+                           p.qweight, p.qzeros, (const uint16_t *)p.scales,                      \
+                           (const uint16_t *)p.bias, (uint16_t *)p.y, (float *)ctx->workspace, M, K, \
+                           N, p.group_shift, kslice2, S)
     switch (mt) {
     case 1: OXQ_GO(1); break;
     case 2: OXQ_GO(2); break;
@@ -233,11 +720,16 @@ static int launch_awq4_mfma(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p) 
     }
 #undef OXQ_GO
     OXQ_HIP_CHECK(hipGetLastError());
+    if (S > 1)
+        return launch_splitk_reduce(ctx, s, (const float *)ctx->workspace, p.bias, p.y, M, N, S, p.dtype);
     return OXQ_OK;
 }
 
 static bool awq4_mfma_ok(const Wna16Problem &p) {
     if (p.bits != 4 || p.pack_dim != OXQ_PACK_OUT) return false;
+    if ((uint64_t)p.K * (uint64_t)(p.N / 2) >= (1ull << 31)) return false;  // 32-bit buffer offsets
+    if ((uint64_t)p.M * (uint64_t)p.K * 2 >= (1ull << 31)) return false;
+    if ((uint64_t)(p.K / p.group_size) * (uint64_t)p.N * 2 >= (1ull << 31)) return false;
     if (p.K % 32 != 0 || p.N % 8 != 0) return false;
     if (p.group_size % 32 != 0) return false;  // a 32-row MFMA step stays inside one group
     if (((uintptr_t)p.x | (uintptr_t)p.scales | (uintptr_t)p.y) & 15) return false;

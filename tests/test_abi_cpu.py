@@ -80,8 +80,10 @@ def test_w4a16_accepts_valid_and_reports_plan(lib, ctx):
                                 C.byref(out)) == 0, err(lib)
     p = plan(lib, ctx)
     assert p.kernel.decode().startswith("awq4_gemv_fast_f16_m1")
-    assert p.block[0] == 256 and p.grid[0] == 14 and p.split_k == p.grid[1] >= 1
+    assert p.block[0] % 64 == 0 and p.split_k == p.grid[1] >= 1
+    assert p.grid[0] * p.grid[1] >= 128          # enough workgroups for 256 CUs
     assert p.workspace_bytes == (p.split_k * 14336 * 4 if p.split_k > 1 else 0)
+    assert p.launches == (2 if p.split_k > 4 else 1)  # many slices -> separate reduce launch
     # odd shape falls to the generic kernel (N not a multiple of 32)
     qw, qz, sc = _awq(192, 104, 64)
     x, out = fake((3, 192), BF16), fake((3, 104), BF16)
@@ -188,9 +190,10 @@ def test_maybe_mpp_declines_like_reference(lib, ctx):
     assert taken.value == 0
     assert call(fake((64, 4096), F16), fake((64, 14336), F16)) == 0 and taken.value == 1
     p = plan(lib, ctx)
-    assert p.kernel.decode() == "awq4_mfma_f16_mt4" and p.grid[0] == 28 and p.grid[2] == 1
+    assert p.kernel.decode() == "awq4_mfma_pipe_f16_mt4" and p.grid[0] == 28 and p.grid[2] == 1
+    assert p.launches == 2 and p.workspace_bytes == p.split_k * 64 * 14336 * 4
     assert call(fake((16, 4096), F16), fake((16, 14336), F16)) == 0 and taken.value == 1
-    assert plan(lib, ctx).kernel.decode() == "awq4_mfma_f16_mt1"
+    assert plan(lib, ctx).kernel.decode() == "awq4_mfma_pipe_f16_mt1"
     # a real error is still an error
     assert call(fake((64, 4000), F16), fake((64, 14336), F16)) == -3 and taken.value == 0
 
@@ -261,7 +264,7 @@ def test_layers_validate_like_reference(lib, ctx):
     assert (k.value, n.value) == (4096, 14336)
     # routing (linear.rs:494-524): m <= 8 -> GEMV kernel, above -> tile GEMM; leading dims flatten
     for shape, kern in [((1, 4096), "awq4_gemv_fast_bf16_m1"), ((2, 3, 4096), "awq4_gemv_fast_bf16_m8"),
-                        ((16, 4096), "awq4_mfma_bf16_mt1"), ((4, 16, 4096), "awq4_mfma_bf16_mt4")]:
+                        ((16, 4096), "awq4_mfma_pipe_bf16_mt1"), ((4, 16, 4096), "awq4_mfma_pipe_bf16_mt4")]:
         x = fake(shape, BF16)
         out = fake(shape[:-1] + (14336,), BF16)
         assert lib.oxq_packed_quant_linear_forward(h, None, C.byref(x), C.byref(out)) == 0, err(lib)
