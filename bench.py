@@ -108,6 +108,9 @@ def main():
     ap.add_argument("--copies", type=int, default=16, help="weight copies rotated to defeat caches")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--all", action="store_true", help="also time GPTQ / GGUF / MXFP4 (stderr)")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="first run a plain 256 MiB device copy 4 times: a kernel of known HBM "
+                         "traffic to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings with")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)")
@@ -121,6 +124,14 @@ def main():
     torch.cuda.set_device(dev)
     ctx = ops.default_context()
     stream = torch.cuda.Stream()
+
+    if args.calib_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(4):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     qw, qz, sc = synth.awq_checkpoint(K, N, G, 4, seed=0x0A0D11E6)
     copies = max(1, args.copies)
@@ -169,13 +180,17 @@ def main():
         print(f"[bench] M={m}: {cases[-1]}", file=sys.stderr, flush=True)
 
     c1 = cases[0]
+    # HBM bytes per launch of the M=1 kernel, measured offline with rocprofv3 --pmc
+    # (FETCH_SIZE, WRITE_SIZE) and recorded in the committed profile summary.
     traffic = None
-    tpath = os.path.join(ROOT, "profiles", "awq4_gemv_m1_traffic.json")
+    tpath = os.path.join(ROOT, "profiles", "awq4_gemv_m1_K4096_N14336_pmc.txt")
     if os.path.exists(tpath):
-        try:
-            traffic = json.load(open(tpath)).get("hbm_bytes_per_launch")
-        except Exception:
-            traffic = None
+        for line in open(tpath):
+            if line.startswith("hbm_bytes_per_launch:"):
+                try:
+                    traffic = int(float(line.split(":", 1)[1].split()[0]))
+                except ValueError:
+                    traffic = None
     result = {
         "metric": "int4 GEMV/GEMM HBM GB/s (% peak) + TFLOPS at M=1/16/64, K=4096 N=14336",
         "value": c1["GB_per_s"],
