@@ -40,17 +40,28 @@ __device__ __forceinline__ void decode_block(const u32x4_t q, float scale, float
         }
 }
 
-__device__ __forceinline__ float dot32_bf16(const uint16_t *__restrict__ xr, const float w[32]) {
+// Block dot product on the gfx950 conversion path: v_cvt_scalef32_pk_bf16_fp4
+// turns one byte (two E2M1 codes, low nibble first) into a bf16 pair - every
+// E2M1 value is exact in bf16 - and v_dot2_f32_bf16 multiplies it with the
+// matching activation pair into an f32 accumulator.  One conversion and one
+// dot per two weights; the E8M0 scale multiplies the block sum once.
+// The activation pair is taken as a by-value uint32_t: bit-casting an element
+// of a vector lvalue directly made the compiler read element 0 every time.
+__device__ __forceinline__ float dot2_fp4(float acc, uint32_t xpair, bf16x2_t wpair) {
+    return __builtin_amdgcn_fdot2_f32_bf16(wpair, __builtin_bit_cast(bf16x2_t, xpair), acc, false);
+}
+
+__device__ __forceinline__ float block_dot_bf16(const u32x4_t q, const uint16_t *__restrict__ xr) {
     const u32x4_t *xp = (const u32x4_t *)xr;
     float acc = 0.0f;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        const u32x4_t v = xp[i];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            acc = fmaf(__builtin_bit_cast(float, v[j] << 16), w[8 * i + 2 * j], acc);
-            acc = fmaf(__builtin_bit_cast(float, v[j] & 0xFFFF0000u), w[8 * i + 2 * j + 1], acc);
-        }
+        const u32x4_t xv = xp[i];
+        const uint32_t w = q[i], x0 = xv[0], x1 = xv[1], x2 = xv[2], x3 = xv[3];
+        acc = dot2_fp4(acc, x0, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, 1.0f, 0));
+        acc = dot2_fp4(acc, x1, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, 1.0f, 1));
+        acc = dot2_fp4(acc, x2, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, 1.0f, 2));
+        acc = dot2_fp4(acc, x3, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, 1.0f, 3));
     }
     return acc;
 }
@@ -92,11 +103,11 @@ __global__ __launch_bounds__(256) void mxfp4_gemv_kernel(
 #pragma unroll
         for (int m = 0; m < MB; ++m) acc[m] = 0.0f;
         for (int b = lane; b < nb; b += 64) {
-            float w[32];
-            decode_block(brow[b], e8m0_to_f32(srow[b]), w);
+            const u32x4_t q = brow[b];
+            const float scale = e8m0_to_f32(srow[b]);
 #pragma unroll
             for (int m = 0; m < MB; ++m)
-                if (m < rows) acc[m] += dot32_bf16(xrow[m] + (size_t)b * 32, w);
+                if (m < rows) acc[m] = fmaf(scale, block_dot_bf16(q, xrow[m] + (size_t)b * 32), acc[m]);
         }
 #pragma unroll
         for (int m = 0; m < MB; ++m) {

@@ -470,6 +470,161 @@ __global__ __launch_bounds__(WPG * GPB * 64) void awq4_gemv_fast(
 }
 
 // ---------------------------------------------------------------------------
+// Fast 4-bit GPTQ kernel.
+//
+// A GPTQ word holds 8 consecutive k of ONE column, so a lane that loads 4 words
+// (one 128-bit load = 4 adjacent columns of a word row) owns 4 output columns
+// outright: no cross-lane reduction.  Masks 0x000F000F / 0x00F000F0 on the word
+// and on word >> 8 give the k pairs (0,4) (1,5) (2,6) (3,7) as exact 16-bit
+// floats (bias 1024 / 64 for f16, 128 for bf16); the matching activation pairs
+// {x[k], x[k+4]} are wave-uniform, built once per workgroup in LDS and read
+// with one 128-bit LDS load per word row.  Per group:
+//     y += s * (acc - bias_even*Xe - bias_odd*Xo - (z+1)*(Xe+Xo)),
+// Xe / Xo = sums of x over even / odd nibble positions of the lane's word rows.
+// One wave owns a whole quantization group (16 word rows at g=128), 8 waves =
+// 8 groups per workgroup, 256 columns per workgroup; K slices go to the workspace.
+// ---------------------------------------------------------------------------
+template <typename TT, int MB>
+__global__ __launch_bounds__(512) void gptq4_gemv_fast(
+    const uint16_t *__restrict__ x, const uint32_t *__restrict__ qw,
+    const uint32_t *__restrict__ qz, const uint16_t *__restrict__ sc,
+    const uint16_t *__restrict__ bias, uint16_t *__restrict__ y, float *__restrict__ ws,
+    unsigned *__restrict__ counters, int M, int K, int N, int gshift, int gpw, int S, int fused) {
+    constexpr int WAVES = 8;
+    constexpr int WR = 16;                 // word rows per chunk (128 k)
+    constexpr int MAXG = 8;                // groups (of >= 128 k) staged per round
+    __shared__ __attribute__((aligned(16))) uint32_t xl[MB][MAXG * WR][4];  // permuted x pairs
+    __shared__ float red[WAVES][256];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int n4 = blockIdx.x * 64 + lane;             // 4-column unit of this lane
+    const int n0 = n4 * 4;
+    const bool valid = n0 < N;
+    const int slice = blockIdx.y;
+    const int G = K >> gshift;
+    const int g0 = slice * gpw, g1 = min(G, g0 + gpw);
+    const int wrows_per_group = (1 << gshift) >> 3;     // word rows per group
+    const int rowbytes = N * 4;
+    const __amdgpu_buffer_rsrc_t rs_w = make_rsrc(qw, (uint32_t)(K >> 3) * (uint32_t)rowbytes);
+    const int voff_w = n0 * 4;
+    const NibbleMasks nm = nibble_masks();
+
+    float yacc[MB][4];
+#pragma unroll
+    for (int m = 0; m < MB; ++m)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) yacc[m][c] = 0.0f;
+
+    // rounds of up to MAXG*128 k: stage permuted x, then each wave walks its share
+    const int k_lo = g0 << gshift, k_hi = g1 << gshift;
+    for (int kr = k_lo; kr < k_hi; kr += MAXG * 128) {
+        const int kr_end = min(k_hi, kr + MAXG * 128);
+        const int nwr = (kr_end - kr) >> 3;            // word rows in this round
+        __syncthreads();
+        for (int idx = threadIdx.x; idx < MB * nwr; idx += WAVES * 64) {
+            const int m = idx / nwr, r = idx % nwr;
+            const int mm = m < M ? m : M - 1;
+            const u32x4_t d = *(const u32x4_t *)(x + (size_t)mm * K + kr + r * 8);
+            u32x4_t o;
+            o[0] = pack_lo16(d[0], d[2]);  // (x0, x4)
+            o[1] = pack_hi16(d[0], d[2]);  // (x1, x5)
+            o[2] = pack_lo16(d[1], d[3]);  // (x2, x6)
+            o[3] = pack_hi16(d[1], d[3]);  // (x3, x7)
+            *(u32x4_t *)(&xl[m][r][0]) = o;
+        }
+        __syncthreads();
+        // chunks of 16 word rows (128 k) are dealt round-robin to the waves
+        const int nchunks = nwr / WR;
+        for (int ch = wave; ch < nchunks; ch += WAVES) {
+            const int kc = kr + ch * 128;
+            const int g = kc >> gshift;
+            u32x4_t w[WR];
+#pragma unroll
+            for (int t = 0; t < WR; ++t)
+                w[t] = __builtin_amdgcn_raw_buffer_load_b128(rs_w, voff_w, ((kc >> 3) + t) * rowbytes, 0);
+            const uint32_t zw = valid ? qz[(size_t)g * (N >> 3) + (n0 >> 3)] : 0u;
+            uint2 sv = valid ? *(const uint2 *)(sc + (size_t)g * N + n0) : uint2{0u, 0u};
+            float acc[MB][4], xe[MB], xo[MB];
+#pragma unroll
+            for (int m = 0; m < MB; ++m) {
+                xe[m] = 0.0f;
+                xo[m] = 0.0f;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) acc[m][c] = 0.0f;
+            }
+#pragma unroll
+            for (int t = 0; t < WR; ++t) {
+                u32x4_t xp[MB];
+#pragma unroll
+                for (int m = 0; m < MB; ++m) xp[m] = *(const u32x4_t *)(&xl[m][ch * WR + t][0]);
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    uint32_t p[4];
+                    TT::unpack4(w[t][c], p, nm);  // pairs (0,4) (1,5) (2,6) (3,7)
+#pragma unroll
+                    for (int m = 0; m < MB; ++m) {
+                        acc[m][c] = TT::dot2(p[0], xp[m][0], acc[m][c]);
+                        acc[m][c] = TT::dot2(p[1], xp[m][1], acc[m][c]);
+                        acc[m][c] = TT::dot2(p[2], xp[m][2], acc[m][c]);
+                        acc[m][c] = TT::dot2(p[3], xp[m][3], acc[m][c]);
+                    }
+                }
+#pragma unroll
+                for (int m = 0; m < MB; ++m) {
+                    xe[m] = TT::dot2(TT::ONES, xp[m][0], xe[m]);
+                    xe[m] = TT::dot2(TT::ONES, xp[m][2], xe[m]);
+                    xo[m] = TT::dot2(TT::ONES, xp[m][1], xo[m]);
+                    xo[m] = TT::dot2(TT::ONES, xp[m][3], xo[m]);
+                }
+            }
+            // a 128-k chunk lies inside one group (group size >= 128): apply scale / zero
+            const int zsh = (n0 & 7) * 4;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const uint32_t spair = c < 2 ? sv.x : sv.y;
+                const float scale = TT::to_f32((c & 1) ? (uint16_t)(spair >> 16) : (uint16_t)(spair & 0xFFFFu));
+                const float zp1 = (float)((zw >> (zsh + 4 * c)) & 0xFu) + 1.0f;
+#pragma unroll
+                for (int m = 0; m < MB; ++m) {
+                    float v = acc[m][c] - TT::bias(0) * xe[m] - TT::bias(1) * xo[m];
+                    v = fmaf(-zp1, xe[m] + xo[m], v);
+                    yacc[m][c] = fmaf(scale, v, yacc[m][c]);
+                }
+            }
+        }
+    }
+
+    const int nbase = blockIdx.x * 256;
+#pragma unroll
+    for (int m = 0; m < MB; ++m) {
+        if (m < M) {
+            __syncthreads();
+            *(float4_t *)(&red[wave][lane * 4]) = float4_t{yacc[m][0], yacc[m][1], yacc[m][2], yacc[m][3]};
+            __syncthreads();
+            for (int col = threadIdx.x; col < 256; col += WAVES * 64) {
+                const int n = nbase + col;
+                if (n < N) {
+                    float tot = 0.0f;
+#pragma unroll
+                    for (int w8 = 0; w8 < WAVES; ++w8) tot += red[w8][col];
+                    if (S == 1) {
+                        const float b = bias ? TT::to_f32(bias[n]) : 0.0f;
+                        y[(size_t)m * N + n] = TT::from_f32(tot + b);
+                    } else if (fused) {
+                        st_agent(ws + ((size_t)slice * M + m) * N + n, tot);
+                    } else {
+                        ws[((size_t)slice * M + m) * N + n] = tot;
+                    }
+                }
+            }
+        }
+    }
+    if (S > 1 && fused && splitk_arrive(counters, blockIdx.x, S))
+        splitk_finish<TT>(ws, bias, y, M, N, S, nbase, 256, WAVES * 64, threadIdx.x);
+}
+
+// ---------------------------------------------------------------------------
 // Host dispatch
 // ---------------------------------------------------------------------------
 static int env_int(const char *name, int dflt) {
@@ -630,8 +785,61 @@ static int launch_generic_t(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p) 
     return OXQ_OK;
 }
 
+static bool gptq4_fast_ok(const Wna16Problem &p) {
+    if (p.bits != 4 || p.pack_dim != OXQ_PACK_IN) return false;
+    if (p.N % 8 != 0 || p.K % 128 != 0 || p.group_size < 128) return false;
+    if (((uintptr_t)p.qweight | (uintptr_t)p.x) & 15) return false;
+    if (((uintptr_t)p.scales) & 7) return false;
+    if ((uint64_t)(p.K / 8) * (uint64_t)p.N * 4 >= (1ull << 31)) return false;
+    return true;
+}
+
+template <typename TT>
+static int launch_gptq4_fast(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p) {
+    const int mb = pick_mb(p.M);
+    const int G = (int)(p.K >> p.group_shift);
+    const int slabs = (int)ceil_div(p.N, 256);
+    int S = (int)ceil_div(ctx->num_cus, slabs);
+    if (S > G) S = G;
+    if (S < 1) S = 1;
+    int gpw = env_int("OXQ_GEMV_GPW", (int)ceil_div(G, S));
+    S = (int)ceil_div(G, gpw);
+    dim3 grid((unsigned)slabs, (unsigned)S), block(512);
+    const uint64_t ws_bytes = S > 1 ? (uint64_t)S * p.M * p.N * 4 : 0;
+    char name[64];
+    snprintf(name, sizeof name, "gptq4_gemv_fast_%s_m%d", TT::DTYPE == 1 ? "f16" : "bf16", mb);
+    set_plan(ctx, name, grid, block, S, 1, ws_bytes);
+    const int fused = splitk_fused(ctx, S);
+    if (ctx->plan_only) {
+        if (S > 1 && !fused) add_launch(ctx);
+        return OXQ_OK;
+    }
+    if (ws_bytes > ctx->workspace_bytes || grid.x > ctx->n_counters)
+        return fail(OXQ_ERR_WORKSPACE, "gptq gemv: needs %llu workspace bytes, ctx holds %zu",
+                    (unsigned long long)ws_bytes, ctx->workspace_bytes);
+#define OXQ_GO(MBv)                                                                               \
+    hipLaunchKernelGGL((gptq4_gemv_fast<TT, MBv>), grid, block, 0, s, (const uint16_t *)p.x,      \
+                       p.qweight, p.qzeros, (const uint16_t *)p.scales, (const uint16_t *)p.bias, \
+                       (uint16_t *)p.y, (float *)ctx->workspace, ctx->counters, (int)p.M, (int)p.K, \
+                       (int)p.N, p.group_shift, gpw, S, fused)
+    switch (mb) {
+    case 1: OXQ_GO(1); break;
+    case 2: OXQ_GO(2); break;
+    case 4: OXQ_GO(4); break;
+    default: OXQ_GO(8); break;
+    }
+#undef OXQ_GO
+    OXQ_HIP_CHECK(hipGetLastError());
+    if (S > 1 && !fused)
+        return launch_splitk_reduce(ctx, s, (const float *)ctx->workspace, p.bias, p.y, p.M, p.N, S,
+                                    p.dtype);
+    return OXQ_OK;
+}
+
 int launch_wna16_gemv(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p) {
     const bool f16 = p.dtype == OXQ_F16;
+    if (gptq4_fast_ok(p) && !env_int("OXQ_FORCE_GENERIC", 0))
+        return f16 ? launch_gptq4_fast<F16Traits>(ctx, s, p) : launch_gptq4_fast<BF16Traits>(ctx, s, p);
     if (awq4_fast_ok(p) && !env_int("OXQ_FORCE_GENERIC", 0))
         return f16 ? launch_awq4_fast<F16Traits>(ctx, s, p) : launch_awq4_fast<BF16Traits>(ctx, s, p);
     if (p.bits == 4)
