@@ -143,47 +143,52 @@ def main():
     x_d = {m: torch.from_numpy(v).to(dev, torch.float16) for m, v in x_host.items()}
     y_d = {m: torch.empty((m, N), dtype=torch.float16, device=dev) for m in (1, 16, 64)}
 
-    cases = []
-    for m in (1, 16, 64):
-        if m <= 8:
-            def step(i, m=m):
-                c = i % copies
-                ops.w4a16_matmul(x_d[m], qw_d[c], qz_d[c], sc_d[c], out=y_d[m], ctx=ctx)
-        else:
-            def step(i, m=m):
-                c = i % copies
-                ops.mpp_quant_matmul(x_d[m], qw_d[c], qz_d[c], sc_d[c], 4, ops.PACK_OUT,
-                                     out=y_d[m], ctx=ctx)
-        step(0)
+    # The hot path as the reference's model code enters it: PackedQuantLinear::forward on a
+    # resident layer (linear.rs:482-533).  The layer repacks its weights tile-major at load.
+    layers = [ops.PackedQuantLinear(4, ops.PACK_OUT, qw_d[c], qz_d[c], sc_d[c], None, torch.float16, ctx=ctx)
+              for c in range(copies)]
+
+    def run_case(m, fn_cold, fn_hot):
+        fn_cold(0)
         plan = ctx.last_plan()
-        wall_ms, ev_ms = time_graph(step, args.steps, args.warmup, stream)
+        wall_ms, ev_ms = time_graph(fn_cold, args.steps, args.warmup, stream)
         # same weights every call: the 30 MB stay in the 256 MB memory-side cache
-        def hot(i, m=m):
-            if m <= 8:
-                ops.w4a16_matmul(x_d[m], qw_d[0], qz_d[0], sc_d[0], out=y_d[m], ctx=ctx)
-            else:
-                ops.mpp_quant_matmul(x_d[m], qw_d[0], qz_d[0], sc_d[0], 4, ops.PACK_OUT,
-                                     out=y_d[m], ctx=ctx)
-        _, hot_ms = time_graph(hot, args.steps, args.warmup, stream)
+        _, hot_ms = time_graph(fn_hot, args.steps, args.warmup, stream)
         us = ev_ms * 1e3 / args.steps
         b = algo_bytes(m)
         flops = 2.0 * m * K * N
-        cases.append({
+        return {
             "M": m, "kernel": plan["kernel"], "grid": list(plan["grid"]), "split_k": plan["split_k"],
+            "launches": plan["launches"],
             "us_per_call": round(us, 3), "us_per_call_wall": round(wall_ms * 1e3 / args.steps, 3),
             "us_per_call_hot_cache": round(hot_ms * 1e3 / args.steps, 3),
             "algorithmic_bytes": b, "GB_per_s": round(b / us / 1e3, 1),
             "hbm_frac": round(b / us / 1e3 / HBM_PEAK_GBS, 4),
             "TFLOP_per_s": round(flops / us / 1e6, 2),
             "mfma_frac": round(flops / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 4),
-        })
-        print(f"[bench] M={m}: {cases[-1]}", file=sys.stderr, flush=True)
+        }
+
+    cases, op_cases = [], []
+    for m in (1, 16, 64):
+        cases.append(run_case(m, lambda i, m=m: layers[i % copies].forward(x_d[m], out=y_d[m]),
+                              lambda i, m=m: layers[0].forward(x_d[m], out=y_d[m])))
+        print(f"[bench] layer M={m}: {cases[-1]}", file=sys.stderr, flush=True)
+    # The stateless ops on the checkpoint layout (metal_ops.rs w4a16_matmul / mpp_quant_matmul).
+    for m in (1, 16, 64):
+        if m <= 8:
+            def op(c, m=m):
+                ops.w4a16_matmul(x_d[m], qw_d[c], qz_d[c], sc_d[c], out=y_d[m], ctx=ctx)
+        else:
+            def op(c, m=m):
+                ops.mpp_quant_matmul(x_d[m], qw_d[c], qz_d[c], sc_d[c], 4, ops.PACK_OUT, out=y_d[m], ctx=ctx)
+        op_cases.append(run_case(m, lambda i, op=op: op(i % copies), lambda i, op=op: op(0)))
+        print(f"[bench] op M={m}: {op_cases[-1]}", file=sys.stderr, flush=True)
 
     c1 = cases[0]
     # HBM bytes per launch of the M=1 kernel, measured offline with rocprofv3 --pmc
     # (FETCH_SIZE, WRITE_SIZE) and recorded in the committed profile summary.
     traffic = None
-    tpath = os.path.join(ROOT, "profiles", "awq4_gemv_m1_K4096_N14336_pmc.txt")
+    tpath = os.path.join(ROOT, "profiles", "pk4_mfma_m1_K4096_N14336_pmc.txt")
     if os.path.exists(tpath):
         for line in open(tpath):
             if line.startswith("hbm_bytes_per_launch:"):
@@ -204,8 +209,10 @@ def main():
         "vs_baseline": None,
         "dtype": "f16",
         "data": "synthetic",
-        "config": {"workload": "AWQ W4A16 GEMV M=1, K=4096 N=14336 g=128, f16 in/out, f32 accumulate "
-                               "(BASELINE configs[1]); M=16/64 tile GEMM in `cases`",
+        "config": {"workload": "AWQ W4A16 M=1, K=4096 N=14336 g=128, f16 in/out, f32 accumulate "
+                               "(BASELINE configs[1]) through PackedQuantLinear.forward on a resident layer; "
+                               "M=16/64 in `cases`; the stateless checkpoint-layout ops in "
+                               "`cases_checkpoint_layout_ops`",
                    "weight_copies_rotated": copies, "timing": "HIP graph of `steps` launches"},
         "roofline": {"bound": "hbm", "achieved": c1["GB_per_s"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(c1["GB_per_s"] / HBM_PEAK_GBS, 4), "traffic": traffic,
@@ -216,6 +223,7 @@ def main():
                          "frac": cases[2]["mfma_frac"], "traffic": None,
                          "kernel": cases[2]["kernel"], "hbm_frac": cases[2]["hbm_frac"]},
         "cases": cases,
+        "cases_checkpoint_layout_ops": op_cases,
     }
     if args.all:
         from oxydllm_amd import bench_extra

@@ -214,7 +214,15 @@ int oxq_mxfp4_moe_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x,
  * routes.  `x` may have any leading dims; m is their product. */
 
 /* linear.rs:403-534 PackedQuantLinear::{new, forward}.  scales must already be
- * in the runtime dtype (`dtype`), as after the cast at linear.rs:437. */
+ * in the runtime dtype (`dtype`), as after the cast at linear.rs:437.
+ *
+ * Like the reference's constructor, `new` is the load-time step: for 4-bit
+ * layers with in_features, out_features and group size all multiples of 64 it
+ * builds a tile-major copy of qweight/qzeros/scales in device memory owned by
+ * the layer (same size as the checkpoint tensors, plus 1.5 bytes per column
+ * and group) and forward never reads the caller's tensors again; it
+ * synchronises the null stream once.  Other layers keep descriptors of the
+ * caller-owned tensors.  OXQ_PREPACK=0 in the environment disables the copy. */
 typedef struct oxq_packed_quant_linear oxq_packed_quant_linear;
 int oxq_packed_quant_linear_new(oxq_ctx *ctx, uint32_t bits, int pack_dim,
                                 const oxq_tensor *qweight, const oxq_tensor *qzeros,
@@ -224,6 +232,12 @@ int oxq_packed_quant_linear_forward(oxq_packed_quant_linear *layer, void *stream
                                     const oxq_tensor *x, const oxq_tensor *out);
 int oxq_packed_quant_linear_in_features(const oxq_packed_quant_linear *layer, int64_t *k);
 int oxq_packed_quant_linear_out_features(const oxq_packed_quant_linear *layer, int64_t *n);
+/* *prepacked = 1 if forward runs on the layer-owned tile-major copy. */
+int oxq_packed_quant_linear_is_prepacked(const oxq_packed_quant_linear *layer, int *prepacked);
+/* linear.rs:510-523: dense dequant of the layer's weights, out = [in, out]
+ * in the layer dtype; element-for-element what forward feeds the matrix cores. */
+int oxq_packed_quant_linear_dequantize(oxq_packed_quant_linear *layer, void *stream,
+                                       const oxq_tensor *out);
 void oxq_packed_quant_linear_free(oxq_packed_quant_linear *layer);
 
 /* linear.rs:179-393 QLinear / GgufFastPath::{build, forward_decode, forward_prefill}. */

@@ -78,6 +78,8 @@ SIGNATURES = {
     "oxq_packed_quant_linear_forward": (C.c_int, [_VP, _VP, _TP, _TP]),
     "oxq_packed_quant_linear_in_features": (C.c_int, [_VP, C.POINTER(C.c_int64)]),
     "oxq_packed_quant_linear_out_features": (C.c_int, [_VP, C.POINTER(C.c_int64)]),
+    "oxq_packed_quant_linear_is_prepacked": (C.c_int, [_VP, C.POINTER(C.c_int)]),
+    "oxq_packed_quant_linear_dequantize": (C.c_int, [_VP, _VP, _TP]),
     "oxq_packed_quant_linear_free": (None, [_VP]),
     "oxq_qlinear_new": (C.c_int, [_VP, C.c_int, _TP, C.c_int64, C.c_int64, _TP, C.c_int,
                                   C.POINTER(_VP)]),

@@ -701,7 +701,55 @@ struct oxq_packed_quant_linear {
     // below m = 64 is a full dense dequant.  Here every m > 8 runs the MFMA tile
     // kernel, which reads the packed weights once.
     int64_t gemv_max_m() const { return 8; }
+    // 4-bit layers with tile-aligned shapes keep a tile-major copy of the
+    // weights made at load (pk4.hip); forward then runs one kernel for every m
+    // and no longer touches the caller's checkpoint tensors.
+    bool prepacked;
+    Pk4Weights pk;
 };
+
+// Load-time repack of an eligible 4-bit layer.  Shapes the repacked kernels do
+// not cover simply keep the checkpoint layout; errors in the tensors themselves
+// surface at forward, where the reference reports them.
+static int prepack_layer(oxq_packed_quant_linear *l) {
+    const char *env = getenv("OXQ_PREPACK");
+    if (env && atoi(env) == 0) return OXQ_OK;
+    oxq_ctx *ctx = l->ctx;
+    oxq_tensor shape_only = l->scales;  // [K, N] descriptor for the shape checks, never written
+    shape_only.rank = 2;
+    shape_only.dims[0] = l->in_features;
+    shape_only.dims[1] = l->out_features;
+    shape_only.contiguous = 1;
+    Wna16Problem src;
+    if (check_wna16(ctx, "PackedQuantLinear", KIND_DEQUANT, nullptr, &l->qweight, &l->qzeros, &l->scales,
+                    l->bits, l->pack_dim, &shape_only, &src) != OXQ_OK)
+        return OXQ_OK;
+    if (!pk4_eligible(src)) return OXQ_OK;
+    l->pk.K = src.K;
+    l->pk.N = src.N;
+    l->pk.group_shift = src.group_shift;
+    l->pk.dtype = l->dtype;
+    if (ctx->plan_only) {
+        l->prepacked = true;
+        return OXQ_OK;
+    }
+    int prev = 0;
+    (void)hipGetDevice(&prev);
+    OXQ_HIP_CHECK(hipSetDevice(ctx->device));
+    int rc = OXQ_OK;
+    hipError_t e = hipMalloc((void **)&l->pk.pw, pk4_weight_bytes(src.K, src.N));
+    if (e == hipSuccess) e = hipMalloc((void **)&l->pk.pzs, pk4_zs_bytes(src.K, src.N, src.group_shift));
+    if (e != hipSuccess) {
+        rc = fail(OXQ_ERR_RUNTIME, "PackedQuantLinear: repack allocation failed: %s", hipGetErrorString(e));
+    } else {
+        rc = launch_pk4_prepack(ctx, nullptr, src, l->pk);
+        if (rc == OXQ_OK && (e = hipStreamSynchronize(nullptr)) != hipSuccess)
+            rc = fail(OXQ_ERR_RUNTIME, "PackedQuantLinear: repack failed: %s", hipGetErrorString(e));
+    }
+    (void)hipSetDevice(prev);
+    if (rc == OXQ_OK) l->prepacked = true;
+    return rc;
+}
 
 struct oxq_qlinear {
     oxq_ctx *ctx;
@@ -769,6 +817,13 @@ int oxq_packed_quant_linear_new(oxq_ctx *ctx, uint32_t bits, int pack_dim,
     l->bits = bits;
     l->pack_dim = pack_dim;
     l->dtype = dtype;
+    l->prepacked = false;
+    l->pk = Pk4Weights{nullptr, nullptr, 0, 0, 0, dtype};
+    int rc = prepack_layer(l);
+    if (rc != OXQ_OK) {
+        oxq_packed_quant_linear_free(l);
+        return rc;
+    }
     *out = l;
     return OXQ_OK;
 }
@@ -782,6 +837,24 @@ int oxq_packed_quant_linear_forward(oxq_packed_quant_linear *l, void *stream, co
     int64_t m;
     OXQ_TRY(flatten_rows(op, x, l->in_features, &x2, &m));
     OXQ_TRY(flatten_out(op, out, m, l->out_features, &o2));
+    if (l->prepacked) {
+        OXQ_TRY(check_tensor(l->ctx, op, "x", &x2));
+        OXQ_TRY(check_tensor(l->ctx, op, "out", &o2));
+        if (x2.dtype != l->dtype)
+            return fail(OXQ_ERR_DTYPE, "%s: scales dtype %s must match x dtype %s", op,
+                        dtype_name(l->dtype), dtype_name(x2.dtype));
+        if (o2.dtype != l->dtype)
+            return fail(OXQ_ERR_DTYPE, "%s: out dtype %s must be %s", op, dtype_name(o2.dtype),
+                        dtype_name(l->dtype));
+        if (m < 1) return fail(OXQ_ERR_SHAPE, "%s: x has no rows", op);
+        Pk4Problem q;
+        q.x = x2.data;
+        q.bias = l->has_bias ? l->bias.data : nullptr;
+        q.y = o2.data;
+        q.M = m;
+        q.w = l->pk;
+        return launch_pk4_forward(l->ctx, (hipStream_t)stream, q);
+    }
     Wna16Problem p;
     const bool gemv = m <= l->gemv_max_m();
     OXQ_TRY(check_wna16(l->ctx, op, gemv ? KIND_GEMV : KIND_TILE, &x2, &l->qweight, &l->qzeros,
@@ -801,7 +874,39 @@ int oxq_packed_quant_linear_out_features(const oxq_packed_quant_linear *l, int64
     *n = l->out_features;
     return OXQ_OK;
 }
-void oxq_packed_quant_linear_free(oxq_packed_quant_linear *l) { delete l; }
+int oxq_packed_quant_linear_is_prepacked(const oxq_packed_quant_linear *l, int *prepacked) {
+    if (!l || !prepacked) return fail(OXQ_ERR_ARG, "PackedQuantLinear: NULL argument");
+    *prepacked = l->prepacked ? 1 : 0;
+    return OXQ_OK;
+}
+
+// linear.rs:510-523: the layer's dense dequant (fallback of forward), [K, N]
+int oxq_packed_quant_linear_dequantize(oxq_packed_quant_linear *l, void *stream, const oxq_tensor *out) {
+    const char *op = "PackedQuantLinear::dequantize";
+    if (!l) return fail(OXQ_ERR_ARG, "%s: layer is NULL", op);
+    if (l->prepacked) {
+        OXQ_TRY(check_tensor(l->ctx, op, "out", out));
+        if (out->rank != 2 || out->dims[0] != l->in_features || out->dims[1] != l->out_features ||
+            !out->contiguous)
+            return fail(OXQ_ERR_SHAPE, "%s: output must be a contiguous [%lld, %lld] tensor", op,
+                        (long long)l->in_features, (long long)l->out_features);
+        if (out->dtype != l->dtype)
+            return fail(OXQ_ERR_DTYPE, "%s: out dtype %s must be %s", op, dtype_name(out->dtype),
+                        dtype_name(l->dtype));
+        return launch_pk4_dequant(l->ctx, (hipStream_t)stream, l->pk, out->data);
+    }
+    Wna16Problem p;
+    OXQ_TRY(check_wna16(l->ctx, op, KIND_DEQUANT, nullptr, &l->qweight, &l->qzeros, &l->scales, l->bits,
+                        l->pack_dim, out, &p));
+    return launch_wna16_dequant(l->ctx, (hipStream_t)stream, p, out->data);
+}
+
+void oxq_packed_quant_linear_free(oxq_packed_quant_linear *l) {
+    if (!l) return;
+    if (l->pk.pw) (void)hipFree(l->pk.pw);
+    if (l->pk.pzs) (void)hipFree(l->pk.pzs);
+    delete l;
+}
 
 // linear.rs:197-247 GgufFastPath::build
 int oxq_qlinear_new(oxq_ctx *ctx, int quant, const oxq_tensor *weight_bytes, int64_t in_features,

@@ -1,0 +1,435 @@
+// Resident 4-bit layers in a tile-major layout: load-time repack + the
+// matmul kernel that runs every batch size on it.
+//
+// Reference semantics: linear.rs:415-448 (PackedQuantLinear::new keeps the
+// checkpoint tensors resident and converts the scales once at load) and
+// linear.rs:482-533 (forward: fused GEMV for small m, staged tile GEMM above,
+// f32 accumulation, result in the activation dtype).  The arithmetic per
+// weight is the tile GEMM's (mpp_gemm.metal:101-266): B = T((q - z) * s)
+// rounded once to the 16-bit activation type, f32 accumulate.
+//
+// Why a repack.  In the checkpoint layouts a [K x 64-column] strip is 32 bytes
+// per row at a row pitch of N/2 bytes; a workgroup that owns such a strip reads
+// narrow column stripes, which this memory system serves at less than half its
+// streaming rate, so the raw-layout kernels give each workgroup a wide slab and
+// split K across workgroups instead - and then pay for the partial sums in
+// HBM.  Stored tile-major, a strip is one contiguous run: one workgroup per
+// 64-column strip streams it with 1 KB wave loads, splits K across its own 8
+// waves and reduces through LDS.  One launch, no workspace, no atomics.
+//
+// Layout (K % 64 == 0, N % 64 == 0, group size a multiple of 64):
+//
+//   pw  [N/64 strips][K/32 steps][64 lanes][4 words]      4 bits per weight
+//   pzs [N/64 strips][K/g groups][16 columns-of-4][4]     one word per column and group
+//
+// Step t of a strip covers 32 rows of K.  Lane l = (ni = l % 16, kb = l / 16)
+// owns the 8 rows  kk = 64*(t/2) + 16*kb + 8*(t%2) .. +7  of the four columns
+// 64*strip + 4*ni + f, f = 0..3: exactly one MFMA B fragment per f.  Word pp
+// (0..3) holds rows kk+2pp (low 16 bits) and kk+2pp+1 (high 16 bits), four
+// nibbles each, nibble f = column f.  Two consecutive steps therefore cover 16
+// consecutive rows per lane group, so the matching activation loads are 32
+// contiguous bytes per row.  One AND-OR per fragment register turns a row pair
+// into two exact 16-bit floats (bias + q).  A pzs word is {-(bias_f + z), s} as
+// two 16-bit floats of the layer's dtype (z already includes GPTQ's +1).
+
+#include "oxq_device.hpp"
+#include "oxq_internal.hpp"
+#include "oxq_mfma.hpp"
+
+namespace oxq {
+
+__device__ __forceinline__ int pk4_kk(int t, int kb) { return ((t >> 1) << 6) + (kb << 4) + ((t & 1) << 3); }
+
+// ---------------------------------------------------------------------------
+// load-time repack
+// ---------------------------------------------------------------------------
+template <bool GPTQ>
+__device__ __forceinline__ uint32_t src_nibble(const uint32_t *__restrict__ qw, int k, int col, int N) {
+    if (GPTQ) return (qw[(size_t)(k >> 3) * N + col] >> (4 * (k & 7))) & 0xFu;
+    const int c = col & 7;
+    const int slot = (c >> 1) | ((c & 1) << 2);  // inverse of the AWQ order [0,2,4,6,1,3,5,7]
+    return (qw[(size_t)k * (N >> 3) + (col >> 3)] >> (4 * slot)) & 0xFu;
+}
+
+template <bool GPTQ>
+__global__ __launch_bounds__(256) void pk4_prepack_weights_kernel(const uint32_t *__restrict__ qw,
+                                                                  uint32_t *__restrict__ pw, int K, int N) {
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const size_t total = (size_t)K * N / 8;
+    if (idx >= total) return;
+    const int NS = K >> 5;
+    const int pp = (int)(idx & 3), l = (int)((idx >> 2) & 63);
+    const size_t st = idx >> 8;
+    const int t = (int)(st % NS), j = (int)(st / NS);
+    const int ni = l & 15, kb = l >> 4;
+    const int k = pk4_kk(t, kb) + 2 * pp;
+    uint32_t w = 0;
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int f = 0; f < 4; ++f)
+            w |= src_nibble<GPTQ>(qw, k + h, 64 * j + 4 * ni + f, N) << (16 * h + 4 * f);
+    pw[idx] = w;
+}
+
+template <typename TT, bool GPTQ>
+__global__ __launch_bounds__(256) void pk4_prepack_zs_kernel(const uint32_t *__restrict__ qz,
+                                                             const uint16_t *__restrict__ sc,
+                                                             uint32_t *__restrict__ pzs, int G, int N) {
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (size_t)G * N) return;
+    const int f = (int)(idx & 3), ni = (int)((idx >> 2) & 15);
+    const size_t jg = idx >> 6;
+    const int g = (int)(jg % G), j = (int)(jg / G);
+    const int col = 64 * j + 4 * ni + f;
+    const int c = col & 7;
+    const int slot = GPTQ ? c : ((c >> 1) | ((c & 1) << 2));
+    const uint32_t z = ((qz[(size_t)g * (N >> 3) + (col >> 3)] >> (4 * slot)) & 0xFu) + (GPTQ ? 1u : 0u);
+    const uint32_t nz = TT::from_f32(-((float)z + TT::bias(f)));
+    pzs[idx] = nz | ((uint32_t)sc[(size_t)g * N + col] << 16);
+}
+
+// ---------------------------------------------------------------------------
+// dense dequant of a resident layer -> [K, N] (linear.rs:510-523 fallback);
+// the same arithmetic as the matmul kernel's B fragments.
+// ---------------------------------------------------------------------------
+template <typename TT>
+__global__ __launch_bounds__(256) void pk4_dequant_kernel(const uint32_t *__restrict__ pw,
+                                                          const uint32_t *__restrict__ pzs,
+                                                          uint16_t *__restrict__ out, int K, int N, int gshift) {
+    typedef MfmaOps<TT> Ops;
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (size_t)K * N / 8) return;
+    const int NS = K >> 5, G = K >> gshift;
+    const int pp = (int)(idx & 3), l = (int)((idx >> 2) & 63);
+    const size_t st = idx >> 8;
+    const int t = (int)(st % NS), j = (int)(st / NS);
+    const int ni = l & 15, kb = l >> 4;
+    const int k = pk4_kk(t, kb) + 2 * pp;
+    const int g = k >> gshift;
+    const uint32_t w = pw[idx];
+    const NibbleMasks nm = nibble_masks();
+#pragma unroll
+    for (int f = 0; f < 4; ++f) {
+        const uint32_t zs = pzs[(((size_t)j * G + g) * 16 + ni) * 4 + f];
+        const uint32_t nz = perm_b32(zs, zs, 0x01000100u), s2 = perm_b32(zs, zs, 0x03020302u);
+        const uint32_t d = Ops::dequant_pair(TT::unpack1(w, f, nm), nz, s2);
+        const int col = 64 * j + 4 * ni + f;
+        out[(size_t)k * N + col] = (uint16_t)(d & 0xFFFFu);
+        out[(size_t)(k + 1) * N + col] = (uint16_t)(d >> 16);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// y[M, N] = x[M, K] . W   on the repacked layout
+//
+// grid.x = strip (64 output columns), grid.z = block of 16*MT rows of x;
+// 8 waves split the groups of K between them.  Per step a wave issues one
+// 1 KB weight load and MT activation loads, D steps ahead of their use (all
+// loads of a wave retire in order, so weights and activations are prefetched
+// at the same distance).  The 8 partial 16*MT x 64 tiles meet in LDS and are
+// added in wave order, which fixes the summation order.
+// ---------------------------------------------------------------------------
+//
+// Two arithmetic forms, both with f32 accumulation:
+//  * GS = false (m > 16, the reference's tile-GEMM range): B = T((q - z) * s),
+//    bit-identical to the dense dequant, fed to the matrix cores.
+//  * GS = true (m <= 16, the reference's fused-GEMV range, which never rounds
+//    the dequantized weight: quant_kernels.metal w4a16 GEMV keeps (q - z) * s in
+//    f32): the matrix cores multiply x by the exact integers bias + q, one
+//    extra MFMA against a fragment of ones yields the row sums of x in the
+//    accumulator layout, and once per group
+//        y += s * (acc_g - (bias + z) * rowsum_g(x))            (all f32).
+// ---------------------------------------------------------------------------
+template <typename TT> struct Pk4Gs;
+template <> struct Pk4Gs<F16Traits> {  // nibble moved to mantissa bits 4..7 of 2^6: 64 + q
+    static constexpr float BIAS = 64.0f;
+    __device__ static __forceinline__ uint32_t unpack(uint32_t w, int f, const NibbleMasks &k) {
+        const uint32_t u = f == 0 ? (w << 4) : f == 1 ? w : f == 2 ? (w >> 4) : (w >> 8);
+        return (u & k.m1) | 0x54005400u;
+    }
+};
+template <> struct Pk4Gs<BF16Traits> {  // 128 + q
+    static constexpr float BIAS = 128.0f;
+    __device__ static __forceinline__ uint32_t unpack(uint32_t w, int f, const NibbleMasks &k) {
+        return BF16Traits::unpack1(w, f, k);
+    }
+};
+
+template <int MT> struct Pk4Depth { static constexpr int D = MT == 1 ? 8 : MT == 2 ? 8 : MT == 3 ? 5 : 4; };
+
+template <typename TT, int MT, bool GS>
+__global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restrict__ x,
+                                                       const uint32_t *__restrict__ pw,
+                                                       const uint32_t *__restrict__ pzs,
+                                                       const uint16_t *__restrict__ bias,
+                                                       uint16_t *__restrict__ y, int M, int K, int N,
+                                                       int gshift, int gpw) {
+    typedef MfmaOps<TT> Ops;
+    constexpr int NW = 8;
+    constexpr int D = Pk4Depth<MT>::D;
+    extern __shared__ __attribute__((aligned(16))) unsigned char pk4_lds[];
+    float4_t *red = (float4_t *)pk4_lds;  // [NW][MT][4 rows-in-quad][64 lanes] of float4 (f = 0..3)
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int ni = lane & 15, kb = lane >> 4;
+    const int j = blockIdx.x;
+    const int m0 = blockIdx.z * (16 * MT);
+    const int NS = K >> 5, G = K >> gshift;
+    const int spg_mask = (1 << (gshift - 5)) - 1;  // steps per group - 1
+    const int g0 = min(G, wave * gpw), g1 = min(G, g0 + gpw);
+    const int t0 = g0 << (gshift - 5), t1 = g1 << (gshift - 5);
+
+    const __amdgpu_buffer_rsrc_t rs_w = make_rsrc(pw + (size_t)j * NS * 256, (uint32_t)NS * 1024u);
+    const __amdgpu_buffer_rsrc_t rs_z = make_rsrc(pzs + (size_t)j * G * 64, (uint32_t)G * 256u);
+    const __amdgpu_buffer_rsrc_t rs_x = make_rsrc(x, (uint32_t)M * (uint32_t)K * 2u);
+    const int voff_w = lane * 16;
+    const int voff_z = ni * 16;
+    int voff_a[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        int r = m0 + mt * 16 + ni;
+        r = r < M ? r : M - 1;  // rows past M are computed and discarded
+        voff_a[mt] = (r * K + kb * 16) * 2;
+    }
+    const NibbleMasks nm = nibble_masks();
+
+    float4_t acc[MT][4];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int f = 0; f < 4; ++f) acc[mt][f] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    u32x4_t wring[D], aring[D][MT];
+    auto load_step = [&](int t, u32x4_t &w, u32x4_t (&a)[MT]) {
+        w = __builtin_amdgcn_raw_buffer_load_b128(rs_w, voff_w, t * 1024, 0);
+        const int ka = ((t >> 1) << 7) + ((t & 1) << 4);  // byte offset of the step inside a row of x
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+            a[mt] = __builtin_amdgcn_raw_buffer_load_b128(rs_x, voff_a[mt], ka, 0);
+    };
+    u32x4_t zs_next;
+    uint32_t negzb[4], sp[4];          // GS = false: splatted -(bias + z) and s
+    float sf[4], nszb[4];              // GS = true: s and -s * (bias + z) in f32
+    float4_t tmp[GS ? MT : 1][4], tmps[GS ? MT : 1];
+    if (GS) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            tmps[mt] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int f = 0; f < 4; ++f) tmp[mt][f] = float4_t{0.f, 0.f, 0.f, 0.f};
+        }
+    }
+    const uint32_t ones[4] = {TT::ONES, TT::ONES, TT::ONES, TT::ONES};
+
+    if (t0 < t1) zs_next = __builtin_amdgcn_raw_buffer_load_b128(rs_z, voff_z, g0 * 256, 0);
+#pragma unroll
+    for (int u = 0; u < D; ++u)
+        if (t0 + u < t1) load_step(t0 + u, wring[u], aring[u]);
+
+    for (int tb = t0; tb < t1; tb += D) {
+#pragma unroll
+        for (int u = 0; u < D; ++u) {
+            const int t = tb + u;
+            if (t < t1) {  // wave-uniform
+                if ((t & spg_mask) == 0) {  // first step of a group
+                    const uint32_t z0 = zs_next[0], z1 = zs_next[1], z2 = zs_next[2], z3 = zs_next[3];
+                    const uint32_t zv[4] = {z0, z1, z2, z3};
+#pragma unroll
+                    for (int f = 0; f < 4; ++f) {
+                        if (GS) {
+                            sf[f] = TT::to_f32((uint16_t)(zv[f] >> 16));
+                            // stored -(bias_f + z)  ->  -(BIAS + z)
+                            const float nzb = TT::to_f32((uint16_t)(zv[f] & 0xFFFFu)) + TT::bias(f) - Pk4Gs<TT>::BIAS;
+                            nszb[f] = sf[f] * nzb;
+                        } else {
+                            negzb[f] = perm_b32(zv[f], zv[f], 0x01000100u);
+                            sp[f] = perm_b32(zv[f], zv[f], 0x03020302u);
+                        }
+                    }
+                    const int gn = (t >> (gshift - 5)) + 1;
+                    if (gn < g1) zs_next = __builtin_amdgcn_raw_buffer_load_b128(rs_z, voff_z, gn * 256, 0);
+                }
+                const u32x4_t wv = wring[u];
+                const uint32_t w0 = wv[0], w1 = wv[1], w2 = wv[2], w3 = wv[3];
+                const uint32_t wp[4] = {w0, w1, w2, w3};
+                uint32_t a[MT][4];
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+                    const u32x4_t av = aring[u][mt];
+                    const uint32_t a0 = av[0], a1 = av[1], a2 = av[2], a3 = av[3];
+                    a[mt][0] = a0, a[mt][1] = a1, a[mt][2] = a2, a[mt][3] = a3;
+                }
+                if (t + D < t1) load_step(t + D, wring[u], aring[u]);  // refill this ring slot
+                if (GS) {
+#pragma unroll
+                    for (int f = 0; f < 4; ++f) {
+                        uint32_t b[4];
+#pragma unroll
+                        for (int pp = 0; pp < 4; ++pp) b[pp] = Pk4Gs<TT>::unpack(wp[pp], f, nm);
+#pragma unroll
+                        for (int mt = 0; mt < MT; ++mt) tmp[mt][f] = Ops::mfma(a[mt], b, tmp[mt][f]);
+                    }
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt) tmps[mt] = Ops::mfma(a[mt], ones, tmps[mt]);
+                    if ((t & spg_mask) == spg_mask) {  // last step of the group: fold it in
+#pragma unroll
+                        for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+                            for (int f = 0; f < 4; ++f) {
+#pragma unroll
+                                for (int i = 0; i < 4; ++i)
+                                    acc[mt][f][i] = fmaf(sf[f], tmp[mt][f][i],
+                                                         fmaf(nszb[f], tmps[mt][i], acc[mt][f][i]));
+                                tmp[mt][f] = float4_t{0.f, 0.f, 0.f, 0.f};
+                            }
+                            tmps[mt] = float4_t{0.f, 0.f, 0.f, 0.f};
+                        }
+                    }
+                } else {
+#pragma unroll
+                    for (int f = 0; f < 4; ++f) {
+                        uint32_t b[4];
+#pragma unroll
+                        for (int pp = 0; pp < 4; ++pp)
+                            b[pp] = Ops::dequant_pair(TT::unpack1(wp[pp], f, nm), negzb[f], sp[f]);
+#pragma unroll
+                        for (int mt = 0; mt < MT; ++mt) acc[mt][f] = Ops::mfma(a[mt], b, acc[mt][f]);
+                    }
+                }
+            }
+        }
+    }
+
+    // the 8 partial tiles -> LDS, float4 = the lane's four columns of one row
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            red[((wave * MT + mt) * 4 + i) * 64 + lane] =
+                float4_t{acc[mt][0][i], acc[mt][1][i], acc[mt][2][i], acc[mt][3][i]};
+    __syncthreads();
+
+    // thread -> (row, 8 consecutive columns); partials added in wave order
+    const int ml = threadIdx.x >> 3, ch = threadIdx.x & 7;
+    if (ml < 16 * MT && m0 + ml < M) {
+        const int mt = ml >> 4, r = ml & 15, rb = r >> 2, i = r & 3;
+        const int l0 = rb * 16 + 2 * ch;
+        float4_t v0 = float4_t{0.f, 0.f, 0.f, 0.f}, v1 = v0;
+#pragma unroll
+        for (int s = 0; s < NW; ++s) {
+            const float4_t *src = red + ((s * MT + mt) * 4 + i) * 64 + l0;
+            v0 += src[0];
+            v1 += src[1];
+        }
+        const int n = 64 * j + 8 * ch;
+        float v[8] = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+        uint32_t o[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            float lo = v[2 * q], hi = v[2 * q + 1];
+            if (bias) {
+                lo += TT::to_f32(bias[n + 2 * q]);
+                hi += TT::to_f32(bias[n + 2 * q + 1]);
+            }
+            o[q] = (uint32_t)TT::from_f32(lo) | ((uint32_t)TT::from_f32(hi) << 16);
+        }
+        *(u32x4_t *)(y + (size_t)(m0 + ml) * N + n) = u32x4_t{o[0], o[1], o[2], o[3]};
+    }
+}
+
+// ---------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------
+bool pk4_eligible(const Wna16Problem &p) {
+    if (p.bits != 4) return false;
+    if (p.K % 64 != 0 || p.N % 64 != 0 || p.group_size % 64 != 0) return false;
+    if ((uint64_t)p.K * (uint64_t)p.N / 2 >= (1ull << 31)) return false;  // 32-bit offsets inside a strip and in x
+    return true;
+}
+
+size_t pk4_weight_bytes(int64_t K, int64_t N) { return (size_t)K * (size_t)N / 2; }
+size_t pk4_zs_bytes(int64_t K, int64_t N, int gshift) { return (size_t)(K >> gshift) * (size_t)N * 4; }
+
+int launch_pk4_prepack(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &src, const Pk4Weights &dst) {
+    const int K = (int)src.K, N = (int)src.N, G = (int)(src.K >> src.group_shift);
+    const size_t words = (size_t)K * N / 8, zsn = (size_t)G * N;
+    const bool gptq = src.pack_dim == OXQ_PACK_IN;
+    dim3 gw((unsigned)ceil_div((int64_t)words, 256)), gz((unsigned)ceil_div((int64_t)zsn, 256)), block(256);
+    set_plan(ctx, gptq ? "pk4_prepack_gptq" : "pk4_prepack_awq", gw, block, 1, 2, 0);
+    if (ctx->plan_only) return OXQ_OK;
+    if (gptq)
+        hipLaunchKernelGGL(pk4_prepack_weights_kernel<true>, gw, block, 0, s, src.qweight, dst.pw, K, N);
+    else
+        hipLaunchKernelGGL(pk4_prepack_weights_kernel<false>, gw, block, 0, s, src.qweight, dst.pw, K, N);
+    OXQ_HIP_CHECK(hipGetLastError());
+#define OXQ_ZS(TTv, GP)                                                                              \
+    hipLaunchKernelGGL((pk4_prepack_zs_kernel<TTv, GP>), gz, block, 0, s, src.qzeros,               \
+                       (const uint16_t *)src.scales, dst.pzs, G, N)
+    if (src.dtype == OXQ_F16) {
+        if (gptq) OXQ_ZS(F16Traits, true); else OXQ_ZS(F16Traits, false);
+    } else {
+        if (gptq) OXQ_ZS(BF16Traits, true); else OXQ_ZS(BF16Traits, false);
+    }
+#undef OXQ_ZS
+    OXQ_HIP_CHECK(hipGetLastError());
+    return OXQ_OK;
+}
+
+int launch_pk4_dequant(oxq_ctx *ctx, hipStream_t s, const Pk4Weights &w, void *out_kn) {
+    const size_t words = (size_t)w.K * w.N / 8;
+    dim3 grid((unsigned)ceil_div((int64_t)words, 256)), block(256);
+    set_plan(ctx, w.dtype == OXQ_F16 ? "pk4_dequant_f16" : "pk4_dequant_bf16", grid, block, 1, 1, 0);
+    if (ctx->plan_only) return OXQ_OK;
+    if (w.dtype == OXQ_F16)
+        hipLaunchKernelGGL(pk4_dequant_kernel<F16Traits>, grid, block, 0, s, w.pw, w.pzs, (uint16_t *)out_kn,
+                           (int)w.K, (int)w.N, w.group_shift);
+    else
+        hipLaunchKernelGGL(pk4_dequant_kernel<BF16Traits>, grid, block, 0, s, w.pw, w.pzs, (uint16_t *)out_kn,
+                           (int)w.K, (int)w.N, w.group_shift);
+    OXQ_HIP_CHECK(hipGetLastError());
+    return OXQ_OK;
+}
+
+template <typename TT, int MT, bool GS>
+static int pk4_go(hipStream_t s, dim3 grid, const Pk4Problem &p, int gpw) {
+    const size_t lds = (size_t)8 * MT * 4 * 64 * 16;
+    static bool attr_set = false;  // one instantiation per (TT, MT)
+    if (!attr_set) {
+        OXQ_HIP_CHECK(hipFuncSetAttribute((const void *)pk4_mfma_kernel<TT, MT, GS>,
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        attr_set = true;
+    }
+    hipLaunchKernelGGL((pk4_mfma_kernel<TT, MT, GS>), grid, dim3(512), lds, s, (const uint16_t *)p.x, p.w.pw,
+                       p.w.pzs, (const uint16_t *)p.bias, (uint16_t *)p.y, (int)p.M, (int)p.w.K, (int)p.w.N,
+                       p.w.group_shift, gpw);
+    OXQ_HIP_CHECK(hipGetLastError());
+    return OXQ_OK;
+}
+
+int launch_pk4_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p) {
+    const int64_t M = p.M;
+    const int mt = M > 48 ? 4 : (int)ceil_div(M, 16);
+    const int G = (int)(p.w.K >> p.w.group_shift);
+    const int gpw = (int)ceil_div(G, 8);
+    dim3 grid((unsigned)(p.w.N / 64), 1, (unsigned)ceil_div(M, 16 * mt));
+    char name[64];
+    snprintf(name, sizeof name, "pk4_mfma_%s_mt%d%s", p.w.dtype == OXQ_F16 ? "f16" : "bf16", mt,
+             mt == 1 ? "_gs" : "");
+    set_plan(ctx, name, grid, dim3(512), 1, 1, 0);
+    if (ctx->plan_only) return OXQ_OK;
+    if ((uint64_t)M * (uint64_t)p.w.K * 2 >= (1ull << 31))
+        return fail(OXQ_ERR_UNSUPPORTED, "pk4 matmul: x larger than 2 GiB");
+    if (((uintptr_t)p.x | (uintptr_t)p.y) & 15)
+        return fail(OXQ_ERR_UNSUPPORTED, "pk4 matmul: x and y must be 16-byte aligned");
+    const bool f16 = p.w.dtype == OXQ_F16;
+    switch (mt) {
+    case 1: return f16 ? pk4_go<F16Traits, 1, true>(s, grid, p, gpw) : pk4_go<BF16Traits, 1, true>(s, grid, p, gpw);
+    case 2: return f16 ? pk4_go<F16Traits, 2, false>(s, grid, p, gpw) : pk4_go<BF16Traits, 2, false>(s, grid, p, gpw);
+    case 3: return f16 ? pk4_go<F16Traits, 3, false>(s, grid, p, gpw) : pk4_go<BF16Traits, 3, false>(s, grid, p, gpw);
+    default: return f16 ? pk4_go<F16Traits, 4, false>(s, grid, p, gpw) : pk4_go<BF16Traits, 4, false>(s, grid, p, gpw);
+    }
+}
+
+}  // namespace oxq

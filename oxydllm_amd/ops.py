@@ -275,6 +275,12 @@ class PackedQuantLinear:
         self.ctx._lib.oxq_packed_quant_linear_in_features(self.handle, C.byref(k))
         self.ctx._lib.oxq_packed_quant_linear_out_features(self.handle, C.byref(n))
         self.in_features, self.out_features = k.value, n.value
+        self.dtype = dtype
+        flag = C.c_int()
+        self.ctx._lib.oxq_packed_quant_linear_is_prepacked(self.handle, C.byref(flag))
+        self.prepacked = bool(flag.value)
+        if self.prepacked:          # the layer owns a tile-major copy; bias is still referenced
+            self._keep = (bias,)
 
     def forward(self, x: torch.Tensor, out=None) -> torch.Tensor:
         if out is None:
@@ -282,6 +288,15 @@ class PackedQuantLinear:
                               device=x.device)
         _lib.check(self.ctx._lib.oxq_packed_quant_linear_forward(self.handle, self.ctx.stream(),
                                                                  desc(x), desc(out)))
+        return out
+
+    def dequantize(self, out=None) -> torch.Tensor:
+        """Dense [in, out] weights in the layer dtype (linear.rs:510-523)."""
+        if out is None:
+            dev = self._keep[0].device if self._keep[0] is not None else torch.device("cuda", self.ctx.device)
+            out = torch.empty((self.in_features, self.out_features), dtype=self.dtype, device=dev)
+        _lib.check(self.ctx._lib.oxq_packed_quant_linear_dequantize(self.handle, self.ctx.stream(),
+                                                                    desc(out)))
         return out
 
     def __del__(self):

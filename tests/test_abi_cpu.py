@@ -265,9 +265,13 @@ def test_layers_validate_like_reference(lib, ctx):
     lib.oxq_packed_quant_linear_in_features(h, C.byref(k))
     lib.oxq_packed_quant_linear_out_features(h, C.byref(n))
     assert (k.value, n.value) == (4096, 14336)
-    # routing (linear.rs:494-524): m <= 8 -> GEMV kernel, above -> tile GEMM; leading dims flatten
-    for shape, kern in [((1, 4096), "awq4_gemv_fast_bf16_m1"), ((2, 3, 4096), "awq4_gemv_fast_bf16_m8"),
-                        ((16, 4096), "awq4_mfma_pipe_bf16_mt1"), ((4, 16, 4096), "awq4_mfma_pipe_bf16_mt4")]:
+    # this layer is tile-aligned, so it is repacked at load and one kernel serves every m
+    # (m <= 16: unrounded-weight form, above: tile-GEMM form); leading dims flatten
+    flag = C.c_int(-1)
+    assert lib.oxq_packed_quant_linear_is_prepacked(h, C.byref(flag)) == 0 and flag.value == 1
+    for shape, kern in [((1, 4096), "pk4_mfma_bf16_mt1_gs"), ((2, 3, 4096), "pk4_mfma_bf16_mt1_gs"),
+                        ((16, 4096), "pk4_mfma_bf16_mt1_gs"), ((17, 4096), "pk4_mfma_bf16_mt2"),
+                        ((4, 16, 4096), "pk4_mfma_bf16_mt4")]:
         x = fake(shape, BF16)
         out = fake(shape[:-1] + (14336,), BF16)
         assert lib.oxq_packed_quant_linear_forward(h, None, C.byref(x), C.byref(out)) == 0, err(lib)

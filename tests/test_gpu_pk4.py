@@ -1,0 +1,187 @@
+"""GPU parity tests for resident 4-bit layers on the tile-major (repacked) path.
+
+The layer constructor repacks AWQ / GPTQ 4-bit checkpoints at load; forward
+then runs one MFMA kernel for every m.  Checked against the CPU oracle:
+  layer.dequantize()  bit-exact against the reference dequant (this pins the
+                      repack: every nibble, zero and scale lands where the
+                      kernel expects it, since forward consumes the same words
+                      with the same arithmetic);
+  layer.forward()     2e-3 relative / 1e-2 absolute of the f32-accumulated
+                      x . dequant(W)^T (+ bias);
+  run-to-run          bitwise identical.
+"""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from oxydllm_amd import synth
+from tests import refgen
+from tests.helpers import TORCH_DT, as_f32, assert_close, bits_of, round_x, to_dev
+
+pytestmark = pytest.mark.gpu
+ops = None
+
+
+def setup_module(module):
+    from oxydllm_amd import ops as _ops
+    module.ops = _ops
+
+
+def say(msg):
+    print(f"[case] {msg}", flush=True)
+    sys.stdout.flush()
+
+
+DT = {"f16": oracle.F16, "bf16": oracle.BF16}
+
+
+def make(kind, K, N, g, seed):
+    if kind == "awq":
+        trip = synth.awq_checkpoint(K, N, g, 4, seed=seed)
+        return trip, ops.PACK_OUT
+    return synth.gptq_checkpoint(K, N, g, 4, seed=seed), ops.PACK_IN
+
+
+def dense(kind, trip, dt):
+    s_r = oracle.round_through(trip[2], dt)
+    if kind == "awq":
+        return oracle.dequantize_awq(trip[0], trip[1], s_r)
+    return oracle.dequantize_gptq(trip[0], trip[1], s_r, 4)
+
+
+def layer_of(trip, pack_dim, dt, bias=None):
+    tdt = TORCH_DT[dt]
+    b = None if bias is None else to_dev(bias, tdt)
+    return ops.PackedQuantLinear(4, pack_dim, to_dev(trip[0]), to_dev(trip[1]), to_dev(trip[2], tdt), b, tdt)
+
+
+@pytest.mark.parametrize("kind", ["awq", "gptq"])
+@pytest.mark.parametrize("dtn,K,N,g", [("f16", 256, 128, 64), ("bf16", 256, 128, 128), ("f16", 512, 192, 128),
+                                       ("bf16", 1280, 64, 128), ("f16", 1024, 320, 256)])
+def test_repacked_dequantize_bit_exact(kind, dtn, K, N, g):
+    dt = DT[dtn]
+    say(f"pk4 dequantize {kind} {dtn} K={K} N={N} g={g}")
+    trip, pack_dim = make(kind, K, N, g, seed=K + N + g)
+    layer = layer_of(trip, pack_dim, dt)
+    assert layer.prepacked
+    want = oracle.transpose_convert(dense(kind, trip, dt), dt)
+    got = layer.dequantize()
+    assert got.shape == (K, N) and got.dtype == TORCH_DT[dt]
+    np.testing.assert_array_equal(bits_of(got), want)
+
+
+def test_repacked_dequantize_reference_generators():
+    """The reference's own closed-form triplets (metal_ops.rs:3668-3716, 4001-4060)."""
+    say("pk4 dequantize reference triplets")
+    for kind, trip, pack_dim in [("awq", refgen.build_awq_triplet(256, 128, 64), ops.PACK_OUT),
+                                 ("gptq", refgen.build_gptq_triplet(4, 256, 128, 64), ops.PACK_IN)]:
+        for dtn in ("f16", "bf16"):
+            dt = DT[dtn]
+            layer = layer_of(trip, pack_dim, dt)
+            assert layer.prepacked
+            want = oracle.transpose_convert(dense(kind, trip, dt), dt)
+            np.testing.assert_array_equal(bits_of(layer.dequantize()), want)
+
+
+@pytest.mark.parametrize("kind", ["awq", "gptq"])
+@pytest.mark.parametrize("dtn", ["f16", "bf16"])
+@pytest.mark.parametrize("K,N,g", [(256, 128, 64), (512, 192, 128), (1280, 64, 128), (2048, 256, 256)])
+def test_repacked_forward_all_m(kind, dtn, K, N, g):
+    """m sweeps every row-tile count (1..4 tiles of 16), partial tiles and m > 64; K/g covers
+    fewer groups than waves (2), a count not divisible by 8 (10) and an even split."""
+    dt = DT[dtn]
+    trip, pack_dim = make(kind, K, N, g, seed=7 * K + N)
+    bias = (np.arange(N, dtype=np.float32) % 11 - 5) * np.float32(0.125)
+    layer = layer_of(trip, pack_dim, dt, bias)
+    assert layer.prepacked
+    w = dense(kind, trip, dt)
+    rng = np.random.default_rng(K + N)
+    for m in (1, 2, 5, 8, 9, 16, 17, 33, 48, 49, 64, 65, 130):
+        say(f"pk4 forward {kind} {dtn} K={K} N={N} g={g} m={m}")
+        x = rng.standard_normal((m, K)).astype(np.float32)
+        ref = oracle.matmul_nt_f32(round_x(x, dt), w, bias)
+        y = layer.forward(to_dev(x, TORCH_DT[dt]))
+        assert y.shape == (m, N)
+        if m <= 16:
+            # the fused-GEMV range: the dequantized weight is never rounded
+            assert_close(y, ref, f"pk4 {kind} {dtn} m{m}")
+        else:
+            # the tile-GEMM range rounds B to the activation type before the matrix unit
+            # (mpp_gemm.metal:115-184): compare with that, and with the reference's own
+            # bound against the unrounded weights (metal_ops.rs:3713-3716)
+            tile = oracle.matmul_nt_f32(round_x(x, dt), oracle.round_through(w, dt), bias)
+            assert_close(y, tile, f"pk4 {kind} {dtn} m{m} vs rounded-tile oracle")
+            assert np.abs(as_f32(y) - ref).max() < 0.06 * np.abs(ref).max() + 1e-2
+
+
+@pytest.mark.parametrize("m", [1, 16, 64])
+@pytest.mark.parametrize("K,N", [(4096, 14336), (14336, 4096)])
+def test_repacked_forward_config1(m, K, N):
+    """Benchmark config 1 (both orientations), f16, and bitwise run-to-run determinism."""
+    dt = oracle.F16
+    say(f"pk4 forward config1 m={m} K={K} N={N}")
+    trip = synth.awq_checkpoint(K, N, 128, 4, seed=0x0A0D11E6)
+    layer = layer_of(trip, ops.PACK_OUT, dt)
+    assert layer.prepacked
+    x = np.random.default_rng(30 + m).standard_normal((m, K)).astype(np.float32)
+    ref = oracle.matmul_nt_f32(round_x(x, dt), dense("awq", trip, dt))
+    xd = to_dev(x, torch.float16)
+    y = layer.forward(xd)
+    assert_close(y, ref, f"pk4 config1 m{m} {K}x{N}")
+    first = bits_of(y)
+    for _ in range(5):
+        np.testing.assert_array_equal(bits_of(layer.forward(xd)), first)
+
+
+def test_repacked_forward_config2_gptq():
+    """Benchmark config 2 (GPTQ 4-bit, K=5120, N=13824, g=128), bf16."""
+    dt = oracle.BF16
+    K, N = 5120, 13824
+    trip = synth.gptq_checkpoint(K, N, 128, 4, seed=0x0A0D11E7)
+    layer = layer_of(trip, ops.PACK_IN, dt)
+    assert layer.prepacked
+    w = dense("gptq", trip, dt)
+    for m in (1, 8, 24):
+        say(f"pk4 forward config2 m={m}")
+        x = np.random.default_rng(40 + m).standard_normal((m, K)).astype(np.float32)
+        wr = w if m <= 16 else oracle.round_through(w, dt)
+        ref = oracle.matmul_nt_f32(round_x(x, dt), wr)
+        assert_close(layer.forward(to_dev(x, torch.bfloat16)), ref, f"pk4 config2 m{m}", bf16_out=True)
+
+
+def test_ineligible_layers_keep_checkpoint_layout():
+    """N not a multiple of 64, g = 32 and 8-bit layers are not repacked and still match."""
+    say("pk4 ineligible shapes")
+    dt = oracle.F16
+    for K, N, g in [(192, 104, 64), (256, 128, 32)]:
+        trip = refgen.build_awq_triplet(K, N, g)
+        layer = layer_of(trip, ops.PACK_OUT, dt)
+        assert not layer.prepacked
+        x = refgen.batch_x(3, K)
+        ref = oracle.matmul_nt_f32(round_x(x, dt), dense("awq", trip, dt))
+        assert_close(layer.forward(to_dev(x, torch.float16)), ref, f"raw layout {K}x{N} g{g}")
+        want = oracle.transpose_convert(dense("awq", trip, dt), dt)
+        np.testing.assert_array_equal(bits_of(layer.dequantize()), want)
+    trip8 = refgen.build_gptq_triplet(8, 256, 128, 64)
+    l8 = ops.PackedQuantLinear(8, ops.PACK_IN, to_dev(trip8[0]), to_dev(trip8[1]),
+                               to_dev(trip8[2], torch.float16), None, torch.float16)
+    assert not l8.prepacked
+
+
+def test_repacked_layer_survives_freed_checkpoint_tensors():
+    """The layer owns its copy: overwrite the caller's tensors after construction."""
+    say("pk4 ownership")
+    dt = oracle.F16
+    K, N, g = 512, 256, 128
+    trip, pack_dim = make("awq", K, N, g, seed=99)
+    qw, qz, sc = to_dev(trip[0]), to_dev(trip[1]), to_dev(trip[2], torch.float16)
+    layer = ops.PackedQuantLinear(4, pack_dim, qw, qz, sc, None, torch.float16)
+    assert layer.prepacked
+    qw.zero_(), qz.zero_(), sc.zero_()
+    torch.cuda.synchronize()
+    x = refgen.batch_x(4, K)
+    ref = oracle.matmul_nt_f32(round_x(x, dt), dense("awq", trip, dt))
+    assert_close(layer.forward(to_dev(x, torch.float16)), ref, "pk4 after source cleared")
