@@ -107,6 +107,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--copies", type=int, default=16, help="weight copies rotated to defeat caches")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--skip-ops", action="store_true", help="skip the checkpoint-layout op cases")
     ap.add_argument("--all", action="store_true", help="also time GPTQ / GGUF / MXFP4 (stderr)")
     ap.add_argument("--calib-copy", action="store_true",
                     help="first run a plain 256 MiB device copy 4 times: a kernel of known HBM "
@@ -174,7 +175,7 @@ def main():
                               lambda i, m=m: layers[0].forward(x_d[m], out=y_d[m])))
         print(f"[bench] layer M={m}: {cases[-1]}", file=sys.stderr, flush=True)
     # The stateless ops on the checkpoint layout (metal_ops.rs w4a16_matmul / mpp_quant_matmul).
-    for m in (1, 16, 64):
+    for m in (() if args.skip_ops else (1, 16, 64)):
         if m <= 8:
             def op(c, m=m):
                 ops.w4a16_matmul(x_d[m], qw_d[c], qz_d[c], sc_d[c], out=y_d[m], ctx=ctx)

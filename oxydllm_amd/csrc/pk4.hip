@@ -17,7 +17,7 @@
 // 64-column strip streams it with 1 KB wave loads, splits K across its own 8
 // waves and reduces through LDS.  One launch, no workspace, no atomics.
 //
-// Layout (K % 64 == 0, N % 64 == 0, group size a multiple of 64):
+// Layout (K % 128 == 0, N % 64 == 0, group size a multiple of 128, at most 128 groups):
 //
 //   pw  [N/64 strips][K/32 steps][64 lanes][4 words]      4 bits per weight
 //   pzs [N/64 strips][K/g groups][16 columns-of-4][4]     one word per column and group
@@ -35,6 +35,8 @@
 #include "oxq_device.hpp"
 #include "oxq_internal.hpp"
 #include "oxq_mfma.hpp"
+
+#include <cstdlib>
 
 namespace oxq {
 
@@ -124,12 +126,25 @@ __global__ __launch_bounds__(256) void pk4_dequant_kernel(const uint32_t *__rest
 // y[M, N] = x[M, K] . W   on the repacked layout
 //
 // grid.x = strip (64 output columns), grid.z = block of 16*MT rows of x;
-// 8 waves split the groups of K between them.  Per step a wave issues one
-// 1 KB weight load and MT activation loads, D steps ahead of their use (all
-// loads of a wave retire in order, so weights and activations are prefetched
-// at the same distance).  The 8 partial 16*MT x 64 tiles meet in LDS and are
-// added in wave order, which fixes the summation order.
-// ---------------------------------------------------------------------------
+// 8 waves split K between them in blocks of 128 rows (4 MFMA steps).
+//
+// Weights: one 1 KB wave load per step, issued two blocks (8 steps) ahead.
+// Activations: the matrix-core fragment pattern (16 rows x 64 bytes per load)
+// is served by L2 at a third of the rate of 256-byte row reads, so a wave
+// fetches its next 16*MT x 128 block of x with 4-rows-x-256-bytes loads one
+// block ahead, parks it in its private LDS slot (16-byte chunks XOR-swizzled by
+// row, so both the row-wise write and the fragment read are conflict-free)
+// and reads fragments from there.  Rows past M are never fetched (out-of-range
+// lane offset: the buffer unit returns zero without touching memory).
+// All vector loads are issued unconditionally - steps past the end of a
+// wave's slice also use the out-of-range offset - so the compiler can count
+// exactly how many loads are younger than the one it waits for; a conditionally
+// issued load makes it wait for all of them, which serialises the pipeline.
+// Activation loads of block b+1 are issued before the weight loads of block
+// b+2: loads retire in order, and this way waiting for the former leaves the
+// latter in flight.  The strip's zeros and scales are staged in LDS once.
+// The 8 partial 16*MT x 64 tiles meet in LDS (each wave's slot is its own
+// activation slot) and are added in wave order, which fixes the summation order.
 //
 // Two arithmetic forms, both with f32 accumulation:
 //  * GS = false (m > 16, the reference's tile-GEMM range): B = T((q - z) * s),
@@ -156,60 +171,84 @@ template <> struct Pk4Gs<BF16Traits> {  // 128 + q
     }
 };
 
-template <int MT> struct Pk4Depth { static constexpr int D = MT == 1 ? 8 : MT == 2 ? 8 : MT == 3 ? 5 : 4; };
-
 template <typename TT, int MT, bool GS>
 __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restrict__ x,
                                                        const uint32_t *__restrict__ pw,
                                                        const uint32_t *__restrict__ pzs,
                                                        const uint16_t *__restrict__ bias,
                                                        uint16_t *__restrict__ y, int M, int K, int N,
-                                                       int gshift, int gpw) {
+                                                       int gshift, int bpw) {
     typedef MfmaOps<TT> Ops;
     constexpr int NW = 8;
-    constexpr int D = Pk4Depth<MT>::D;
+    constexpr int ROWS = 16 * MT;
+    constexpr int AQ = 4 * MT;                 // activation loads per block and lane
+    constexpr int SLOT = ROWS * 256;           // bytes of one wave's LDS slot (= its partial tile)
+    constexpr int OOB = 0x7FFFFF00;
     extern __shared__ __attribute__((aligned(16))) unsigned char pk4_lds[];
-    float4_t *red = (float4_t *)pk4_lds;  // [NW][MT][4 rows-in-quad][64 lanes] of float4 (f = 0..3)
+    u32x4_t *zs_lds = (u32x4_t *)(pk4_lds + NW * SLOT);  // [G][16]: the strip's {-(bias+z), s} words
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int ni = lane & 15, kb = lane >> 4;
     const int j = blockIdx.x;
-    const int m0 = blockIdx.z * (16 * MT);
-    const int NS = K >> 5, G = K >> gshift;
-    const int spg_mask = (1 << (gshift - 5)) - 1;  // steps per group - 1
-    const int g0 = min(G, wave * gpw), g1 = min(G, g0 + gpw);
-    const int t0 = g0 << (gshift - 5), t1 = g1 << (gshift - 5);
+    const int m0 = blockIdx.z * ROWS;
+    const int NS = K >> 5, G = K >> gshift, NB = K >> 7;
+    const int bpg_mask = (1 << (gshift - 7)) - 1;  // blocks per group - 1
+    const int b0 = min(NB, wave * bpw), b1 = min(NB, b0 + bpw);
+    unsigned char *slot = pk4_lds + wave * SLOT;
 
     const __amdgpu_buffer_rsrc_t rs_w = make_rsrc(pw + (size_t)j * NS * 256, (uint32_t)NS * 1024u);
     const __amdgpu_buffer_rsrc_t rs_z = make_rsrc(pzs + (size_t)j * G * 64, (uint32_t)G * 256u);
     const __amdgpu_buffer_rsrc_t rs_x = make_rsrc(x, (uint32_t)M * (uint32_t)K * 2u);
     const int voff_w = lane * 16;
-    const int voff_z = ni * 16;
-    int voff_a[MT];
+    // activation load q of a block: row 4q + lane/16, 16-byte chunk lane%16 of the row's 256 bytes
+    int voff_a[AQ], a_wr[AQ];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-        int r = m0 + mt * 16 + ni;
-        r = r < M ? r : M - 1;  // rows past M are computed and discarded
-        voff_a[mt] = (r * K + kb * 16) * 2;
+    for (int q = 0; q < AQ; ++q) {
+        const int row = 4 * q + kb, r = m0 + row;
+        voff_a[q] = r < M ? (r * K * 2 + ni * 16) : OOB;
+        a_wr[q] = row * 256 + ((ni ^ (row & 15)) << 4);
     }
+    // fragment read of step s (0..3), row tile mt: row 16mt + ni, chunk 8*(s/2) + 2kb + (s%2)
+    int a_rd[4];
+#pragma unroll
+    for (int st = 0; st < 4; ++st) a_rd[st] = ni * 256 + (((8 * (st >> 1) + 2 * kb + (st & 1)) ^ ni) << 4);
     const NibbleMasks nm = nibble_masks();
+
+    constexpr int ZCH = 4;  // 16-byte chunks per thread: 32 KB = 128 groups
+    u32x4_t zstage[ZCH];
+    const int zchunks = G * 16;
+#pragma unroll
+    for (int q = 0; q < ZCH; ++q)
+        if (q * 512 < zchunks)  // block-uniform
+            zstage[q] = __builtin_amdgcn_raw_buffer_load_b128(rs_z, (int)(threadIdx.x + q * 512) * 16, 0, 0);
+
+    u32x4_t areg[AQ], wr[2][4];
+    auto load_a = [&](int blk) {
+        const bool live = blk < b1;  // wave-uniform
+#pragma unroll
+        for (int q = 0; q < AQ; ++q)
+            areg[q] = __builtin_amdgcn_raw_buffer_load_b128(rs_x, live ? voff_a[q] : OOB, blk * 256, 0);
+    };
+    auto load_w = [&](int blk, int st, u32x4_t &w) {
+        w = __builtin_amdgcn_raw_buffer_load_b128(rs_w, blk < b1 ? voff_w : OOB, (blk * 4 + st) * 1024, 0);
+    };
+    auto store_a = [&]() {
+#pragma unroll
+        for (int q = 0; q < AQ; ++q) *(u32x4_t *)(slot + a_wr[q]) = areg[q];
+    };
+
+    load_a(b0);
+#pragma unroll
+    for (int st = 0; st < 4; ++st) load_w(b0, st, wr[0][st]);
+#pragma unroll
+    for (int st = 0; st < 4; ++st) load_w(b0 + 1, st, wr[1][st]);
 
     float4_t acc[MT][4];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
         for (int f = 0; f < 4; ++f) acc[mt][f] = float4_t{0.f, 0.f, 0.f, 0.f};
-
-    u32x4_t wring[D], aring[D][MT];
-    auto load_step = [&](int t, u32x4_t &w, u32x4_t (&a)[MT]) {
-        w = __builtin_amdgcn_raw_buffer_load_b128(rs_w, voff_w, t * 1024, 0);
-        const int ka = ((t >> 1) << 7) + ((t & 1) << 4);  // byte offset of the step inside a row of x
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-            a[mt] = __builtin_amdgcn_raw_buffer_load_b128(rs_x, voff_a[mt], ka, 0);
-    };
-    u32x4_t zs_next;
     uint32_t negzb[4], sp[4];          // GS = false: splatted -(bias + z) and s
     float sf[4], nszb[4];              // GS = true: s and -s * (bias + z) in f32
     float4_t tmp[GS ? MT : 1][4], tmps[GS ? MT : 1];
@@ -223,86 +262,93 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
     }
     const uint32_t ones[4] = {TT::ONES, TT::ONES, TT::ONES, TT::ONES};
 
-    if (t0 < t1) zs_next = __builtin_amdgcn_raw_buffer_load_b128(rs_z, voff_z, g0 * 256, 0);
 #pragma unroll
-    for (int u = 0; u < D; ++u)
-        if (t0 + u < t1) load_step(t0 + u, wring[u], aring[u]);
+    for (int q = 0; q < ZCH; ++q)
+        if ((int)threadIdx.x + q * 512 < zchunks) zs_lds[threadIdx.x + q * 512] = zstage[q];
+    store_a();
+    __syncthreads();
 
-    for (int tb = t0; tb < t1; tb += D) {
+    for (int bb = b0; bb < b1; bb += 2) {
 #pragma unroll
-        for (int u = 0; u < D; ++u) {
-            const int t = tb + u;
-            if (t < t1) {  // wave-uniform
-                if ((t & spg_mask) == 0) {  // first step of a group
-                    const uint32_t z0 = zs_next[0], z1 = zs_next[1], z2 = zs_next[2], z3 = zs_next[3];
-                    const uint32_t zv[4] = {z0, z1, z2, z3};
+        for (int cur = 0; cur < 2; ++cur) {
+            const int blk = bb + cur;
+            load_a(blk + 1);
+            const bool live = blk < b1;  // wave-uniform
+            if (live && (blk & bpg_mask) == 0) {  // first block of a group
+                const u32x4_t zq = zs_lds[(blk >> (gshift - 7)) * 16 + ni];
+                const uint32_t z0 = zq[0], z1 = zq[1], z2 = zq[2], z3 = zq[3];
+                const uint32_t zv[4] = {z0, z1, z2, z3};
 #pragma unroll
-                    for (int f = 0; f < 4; ++f) {
-                        if (GS) {
-                            sf[f] = TT::to_f32((uint16_t)(zv[f] >> 16));
-                            // stored -(bias_f + z)  ->  -(BIAS + z)
-                            const float nzb = TT::to_f32((uint16_t)(zv[f] & 0xFFFFu)) + TT::bias(f) - Pk4Gs<TT>::BIAS;
-                            nszb[f] = sf[f] * nzb;
-                        } else {
-                            negzb[f] = perm_b32(zv[f], zv[f], 0x01000100u);
-                            sp[f] = perm_b32(zv[f], zv[f], 0x03020302u);
-                        }
-                    }
-                    const int gn = (t >> (gshift - 5)) + 1;
-                    if (gn < g1) zs_next = __builtin_amdgcn_raw_buffer_load_b128(rs_z, voff_z, gn * 256, 0);
-                }
-                const u32x4_t wv = wring[u];
-                const uint32_t w0 = wv[0], w1 = wv[1], w2 = wv[2], w3 = wv[3];
-                const uint32_t wp[4] = {w0, w1, w2, w3};
-                uint32_t a[MT][4];
-#pragma unroll
-                for (int mt = 0; mt < MT; ++mt) {
-                    const u32x4_t av = aring[u][mt];
-                    const uint32_t a0 = av[0], a1 = av[1], a2 = av[2], a3 = av[3];
-                    a[mt][0] = a0, a[mt][1] = a1, a[mt][2] = a2, a[mt][3] = a3;
-                }
-                if (t + D < t1) load_step(t + D, wring[u], aring[u]);  // refill this ring slot
-                if (GS) {
-#pragma unroll
-                    for (int f = 0; f < 4; ++f) {
-                        uint32_t b[4];
-#pragma unroll
-                        for (int pp = 0; pp < 4; ++pp) b[pp] = Pk4Gs<TT>::unpack(wp[pp], f, nm);
-#pragma unroll
-                        for (int mt = 0; mt < MT; ++mt) tmp[mt][f] = Ops::mfma(a[mt], b, tmp[mt][f]);
-                    }
-#pragma unroll
-                    for (int mt = 0; mt < MT; ++mt) tmps[mt] = Ops::mfma(a[mt], ones, tmps[mt]);
-                    if ((t & spg_mask) == spg_mask) {  // last step of the group: fold it in
-#pragma unroll
-                        for (int mt = 0; mt < MT; ++mt) {
-#pragma unroll
-                            for (int f = 0; f < 4; ++f) {
-#pragma unroll
-                                for (int i = 0; i < 4; ++i)
-                                    acc[mt][f][i] = fmaf(sf[f], tmp[mt][f][i],
-                                                         fmaf(nszb[f], tmps[mt][i], acc[mt][f][i]));
-                                tmp[mt][f] = float4_t{0.f, 0.f, 0.f, 0.f};
-                            }
-                            tmps[mt] = float4_t{0.f, 0.f, 0.f, 0.f};
-                        }
-                    }
-                } else {
-#pragma unroll
-                    for (int f = 0; f < 4; ++f) {
-                        uint32_t b[4];
-#pragma unroll
-                        for (int pp = 0; pp < 4; ++pp)
-                            b[pp] = Ops::dequant_pair(TT::unpack1(wp[pp], f, nm), negzb[f], sp[f]);
-#pragma unroll
-                        for (int mt = 0; mt < MT; ++mt) acc[mt][f] = Ops::mfma(a[mt], b, acc[mt][f]);
+                for (int f = 0; f < 4; ++f) {
+                    if (GS) {
+                        sf[f] = TT::to_f32((uint16_t)(zv[f] >> 16));
+                        // stored -(bias_f + z)  ->  -(BIAS + z)
+                        const float nzb = TT::to_f32((uint16_t)(zv[f] & 0xFFFFu)) + TT::bias(f) - Pk4Gs<TT>::BIAS;
+                        nszb[f] = sf[f] * nzb;
+                    } else {
+                        negzb[f] = perm_b32(zv[f], zv[f], 0x01000100u);
+                        sp[f] = perm_b32(zv[f], zv[f], 0x03020302u);
                     }
                 }
             }
+#pragma unroll
+            for (int st = 0; st < 4; ++st) {
+                const u32x4_t wv = wr[cur][st];
+                load_w(blk + 2, st, wr[cur][st]);  // refill this ring slot
+                if (live) {
+                    const uint32_t w0 = wv[0], w1 = wv[1], w2 = wv[2], w3 = wv[3];
+                    const uint32_t wp[4] = {w0, w1, w2, w3};
+                    uint32_t a[MT][4];
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt) {
+                        const u32x4_t av = *(const u32x4_t *)(slot + mt * 4096 + a_rd[st]);
+                        const uint32_t a0 = av[0], a1 = av[1], a2 = av[2], a3 = av[3];
+                        a[mt][0] = a0, a[mt][1] = a1, a[mt][2] = a2, a[mt][3] = a3;
+                    }
+                    if (GS) {
+#pragma unroll
+                        for (int f = 0; f < 4; ++f) {
+                            uint32_t b[4];
+#pragma unroll
+                            for (int pp = 0; pp < 4; ++pp) b[pp] = Pk4Gs<TT>::unpack(wp[pp], f, nm);
+#pragma unroll
+                            for (int mt = 0; mt < MT; ++mt) tmp[mt][f] = Ops::mfma(a[mt], b, tmp[mt][f]);
+                        }
+#pragma unroll
+                        for (int mt = 0; mt < MT; ++mt) tmps[mt] = Ops::mfma(a[mt], ones, tmps[mt]);
+                    } else {
+#pragma unroll
+                        for (int f = 0; f < 4; ++f) {
+                            uint32_t b[4];
+#pragma unroll
+                            for (int pp = 0; pp < 4; ++pp)
+                                b[pp] = Ops::dequant_pair(TT::unpack1(wp[pp], f, nm), negzb[f], sp[f]);
+#pragma unroll
+                            for (int mt = 0; mt < MT; ++mt) acc[mt][f] = Ops::mfma(a[mt], b, acc[mt][f]);
+                        }
+                    }
+                }
+            }
+            if (GS && live && (blk & bpg_mask) == bpg_mask) {  // last block of the group: fold it in
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+                    for (int f = 0; f < 4; ++f) {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i)
+                            acc[mt][f][i] = fmaf(sf[f], tmp[mt][f][i], fmaf(nszb[f], tmps[mt][i], acc[mt][f][i]));
+                        tmp[mt][f] = float4_t{0.f, 0.f, 0.f, 0.f};
+                    }
+                    tmps[mt] = float4_t{0.f, 0.f, 0.f, 0.f};
+                }
+            }
+            store_a();  // the next block's activations replace this one's (same wave: in order)
         }
     }
 
-    // the 8 partial tiles -> LDS, float4 = the lane's four columns of one row
+    // the 8 partial tiles -> LDS (each wave into its own slot), float4 = the lane's four
+    // columns of one row
+    float4_t *red = (float4_t *)pk4_lds;  // [NW][MT][4 rows-in-quad][64 lanes] of float4 (f = 0..3)
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -313,7 +359,7 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
 
     // thread -> (row, 8 consecutive columns); partials added in wave order
     const int ml = threadIdx.x >> 3, ch = threadIdx.x & 7;
-    if (ml < 16 * MT && m0 + ml < M) {
+    if (ml < ROWS && m0 + ml < M) {
         const int mt = ml >> 4, r = ml & 15, rb = r >> 2, i = r & 3;
         const int l0 = rb * 16 + 2 * ch;
         float4_t v0 = float4_t{0.f, 0.f, 0.f, 0.f}, v1 = v0;
@@ -344,8 +390,9 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
 // ---------------------------------------------------------------------------
 bool pk4_eligible(const Wna16Problem &p) {
     if (p.bits != 4) return false;
-    if (p.K % 64 != 0 || p.N % 64 != 0 || p.group_size % 64 != 0) return false;
+    if (p.K % 128 != 0 || p.N % 64 != 0 || p.group_size % 128 != 0) return false;
     if ((uint64_t)p.K * (uint64_t)p.N / 2 >= (1ull << 31)) return false;  // 32-bit offsets inside a strip and in x
+    if (p.K / p.group_size > 128) return false;  // a strip's zeros and scales must fit 32 KB of LDS
     return true;
 }
 
@@ -393,17 +440,18 @@ int launch_pk4_dequant(oxq_ctx *ctx, hipStream_t s, const Pk4Weights &w, void *o
 }
 
 template <typename TT, int MT, bool GS>
-static int pk4_go(hipStream_t s, dim3 grid, const Pk4Problem &p, int gpw) {
-    const size_t lds = (size_t)8 * MT * 4 * 64 * 16;
-    static bool attr_set = false;  // one instantiation per (TT, MT)
-    if (!attr_set) {
+static int pk4_go(hipStream_t s, dim3 grid, const Pk4Problem &p, int bpw) {
+    const int G = (int)(p.w.K >> p.w.group_shift);
+    const size_t lds = (size_t)8 * MT * 4096 + (size_t)G * 256;
+    static size_t attr_lds = 0;  // one instantiation per (TT, MT, GS)
+    if (lds > attr_lds) {
         OXQ_HIP_CHECK(hipFuncSetAttribute((const void *)pk4_mfma_kernel<TT, MT, GS>,
                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        attr_set = true;
+        attr_lds = lds;
     }
     hipLaunchKernelGGL((pk4_mfma_kernel<TT, MT, GS>), grid, dim3(512), lds, s, (const uint16_t *)p.x, p.w.pw,
                        p.w.pzs, (const uint16_t *)p.bias, (uint16_t *)p.y, (int)p.M, (int)p.w.K, (int)p.w.N,
-                       p.w.group_shift, gpw);
+                       p.w.group_shift, bpw);
     OXQ_HIP_CHECK(hipGetLastError());
     return OXQ_OK;
 }
@@ -412,7 +460,7 @@ int launch_pk4_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p) {
     const int64_t M = p.M;
     const int mt = M > 48 ? 4 : (int)ceil_div(M, 16);
     const int G = (int)(p.w.K >> p.w.group_shift);
-    const int gpw = (int)ceil_div(G, 8);
+    const int bpw = (int)ceil_div(G, 8) << (p.w.group_shift - 7);  // whole groups per wave, in 128-row blocks
     dim3 grid((unsigned)(p.w.N / 64), 1, (unsigned)ceil_div(M, 16 * mt));
     char name[64];
     snprintf(name, sizeof name, "pk4_mfma_%s_mt%d%s", p.w.dtype == OXQ_F16 ? "f16" : "bf16", mt,
@@ -425,10 +473,10 @@ int launch_pk4_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p) {
         return fail(OXQ_ERR_UNSUPPORTED, "pk4 matmul: x and y must be 16-byte aligned");
     const bool f16 = p.w.dtype == OXQ_F16;
     switch (mt) {
-    case 1: return f16 ? pk4_go<F16Traits, 1, true>(s, grid, p, gpw) : pk4_go<BF16Traits, 1, true>(s, grid, p, gpw);
-    case 2: return f16 ? pk4_go<F16Traits, 2, false>(s, grid, p, gpw) : pk4_go<BF16Traits, 2, false>(s, grid, p, gpw);
-    case 3: return f16 ? pk4_go<F16Traits, 3, false>(s, grid, p, gpw) : pk4_go<BF16Traits, 3, false>(s, grid, p, gpw);
-    default: return f16 ? pk4_go<F16Traits, 4, false>(s, grid, p, gpw) : pk4_go<BF16Traits, 4, false>(s, grid, p, gpw);
+    case 1: return f16 ? pk4_go<F16Traits, 1, true>(s, grid, p, bpw) : pk4_go<BF16Traits, 1, true>(s, grid, p, bpw);
+    case 2: return f16 ? pk4_go<F16Traits, 2, false>(s, grid, p, bpw) : pk4_go<BF16Traits, 2, false>(s, grid, p, bpw);
+    case 3: return f16 ? pk4_go<F16Traits, 3, false>(s, grid, p, bpw) : pk4_go<BF16Traits, 3, false>(s, grid, p, bpw);
+    default: return f16 ? pk4_go<F16Traits, 4, false>(s, grid, p, bpw) : pk4_go<BF16Traits, 4, false>(s, grid, p, bpw);
     }
 }
 

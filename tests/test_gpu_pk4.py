@@ -59,7 +59,7 @@ def layer_of(trip, pack_dim, dt, bias=None):
 
 
 @pytest.mark.parametrize("kind", ["awq", "gptq"])
-@pytest.mark.parametrize("dtn,K,N,g", [("f16", 256, 128, 64), ("bf16", 256, 128, 128), ("f16", 512, 192, 128),
+@pytest.mark.parametrize("dtn,K,N,g", [("f16", 256, 128, 128), ("bf16", 256, 128, 128), ("f16", 512, 192, 128),
                                        ("bf16", 1280, 64, 128), ("f16", 1024, 320, 256)])
 def test_repacked_dequantize_bit_exact(kind, dtn, K, N, g):
     dt = DT[dtn]
@@ -76,8 +76,8 @@ def test_repacked_dequantize_bit_exact(kind, dtn, K, N, g):
 def test_repacked_dequantize_reference_generators():
     """The reference's own closed-form triplets (metal_ops.rs:3668-3716, 4001-4060)."""
     say("pk4 dequantize reference triplets")
-    for kind, trip, pack_dim in [("awq", refgen.build_awq_triplet(256, 128, 64), ops.PACK_OUT),
-                                 ("gptq", refgen.build_gptq_triplet(4, 256, 128, 64), ops.PACK_IN)]:
+    for kind, trip, pack_dim in [("awq", refgen.build_awq_triplet(256, 128, 128), ops.PACK_OUT),
+                                 ("gptq", refgen.build_gptq_triplet(4, 256, 128, 128), ops.PACK_IN)]:
         for dtn in ("f16", "bf16"):
             dt = DT[dtn]
             layer = layer_of(trip, pack_dim, dt)
@@ -88,10 +88,11 @@ def test_repacked_dequantize_reference_generators():
 
 @pytest.mark.parametrize("kind", ["awq", "gptq"])
 @pytest.mark.parametrize("dtn", ["f16", "bf16"])
-@pytest.mark.parametrize("K,N,g", [(256, 128, 64), (512, 192, 128), (1280, 64, 128), (2048, 256, 256)])
+@pytest.mark.parametrize("K,N,g", [(256, 128, 128), (512, 192, 128), (1280, 64, 128), (2048, 256, 256), (1152, 128, 128)])
 def test_repacked_forward_all_m(kind, dtn, K, N, g):
     """m sweeps every row-tile count (1..4 tiles of 16), partial tiles and m > 64; K/g covers
-    fewer groups than waves (2), a count not divisible by 8 (10) and an even split."""
+    fewer groups than waves (2), counts not divisible by 8 (10, 9: an odd number of
+    128-row blocks per wave) and an even split."""
     dt = DT[dtn]
     trip, pack_dim = make(kind, K, N, g, seed=7 * K + N)
     bias = (np.arange(N, dtype=np.float32) % 11 - 5) * np.float32(0.125)
@@ -153,10 +154,10 @@ def test_repacked_forward_config2_gptq():
 
 
 def test_ineligible_layers_keep_checkpoint_layout():
-    """N not a multiple of 64, g = 32 and 8-bit layers are not repacked and still match."""
+    """N not a multiple of 64, g < 128 and 8-bit layers are not repacked and still match."""
     say("pk4 ineligible shapes")
     dt = oracle.F16
-    for K, N, g in [(192, 104, 64), (256, 128, 32)]:
+    for K, N, g in [(192, 104, 64), (256, 128, 32), (256, 128, 64)]:
         trip = refgen.build_awq_triplet(K, N, g)
         layer = layer_of(trip, ops.PACK_OUT, dt)
         assert not layer.prepacked
