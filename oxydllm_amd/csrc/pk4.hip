@@ -156,28 +156,25 @@ __global__ __launch_bounds__(256) void pk4_dequant_kernel(const uint32_t *__rest
 //    accumulator layout, and once per group
 //        y += s * (acc_g - (bias + z) * rowsum_g(x))            (all f32).
 // ---------------------------------------------------------------------------
-template <typename TT> struct Pk4Gs;
-template <> struct Pk4Gs<F16Traits> {  // nibble moved to mantissa bits 4..7 of 2^6: 64 + q
-    static constexpr float BIAS = 64.0f;
-    __device__ static __forceinline__ uint32_t unpack(uint32_t w, int f, const NibbleMasks &k) {
-        const uint32_t u = f == 0 ? (w << 4) : f == 1 ? w : f == 2 ? (w >> 4) : (w >> 8);
-        return (u & k.m1) | 0x54005400u;
-    }
-};
-template <> struct Pk4Gs<BF16Traits> {  // 128 + q
-    static constexpr float BIAS = 128.0f;
-    __device__ static __forceinline__ uint32_t unpack(uint32_t w, int f, const NibbleMasks &k) {
-        return BF16Traits::unpack1(w, f, k);
-    }
+// The integers the GS form feeds the matrix cores: bias_f + q, the same AND-OR unpack as
+// the other form (f16: 1024 + q or 64 + q by nibble position, bf16: 128 + q).
+// Ring depths in 128-row blocks: weights WB, activations AB (registers; the current
+// block's activations live in LDS).  Deeper rings measured no faster: at these sizes the
+// kernel is bound by instruction issue, not by memory latency.
+template <int MT> struct Pk4Ring {
+    static constexpr int AB = 1;
+    static constexpr int WB = 2;
+    static constexpr int U = WB > AB ? WB : AB;  // unroll (both divide it)
 };
 
-template <typename TT, int MT, bool GS>
+// BPG1: group size 128, i.e. every block is one group (no group bookkeeping).
+template <typename TT, int MT, bool GS, bool BPG1, int AB, int WB>
 __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restrict__ x,
                                                        const uint32_t *__restrict__ pw,
                                                        const uint32_t *__restrict__ pzs,
                                                        const uint16_t *__restrict__ bias,
                                                        uint16_t *__restrict__ y, int M, int K, int N,
-                                                       int gshift, int bpw) {
+                                                       int gshift, int bpw, int interleave) {
     typedef MfmaOps<TT> Ops;
     constexpr int NW = 8;
     constexpr int ROWS = 16 * MT;
@@ -194,7 +191,14 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
     const int m0 = blockIdx.z * ROWS;
     const int NS = K >> 5, G = K >> gshift, NB = K >> 7;
     const int bpg_mask = (1 << (gshift - 7)) - 1;  // blocks per group - 1
-    const int b0 = min(NB, wave * bpw), b1 = min(NB, b0 + bpw);
+    // The wave's blocks, by local index i: either one contiguous run of whole groups, or
+    // every 8th group (the 8 waves then sweep the strip together, front to back).
+    const int gs7 = gshift - 7;
+    const int b0 = min(NB, wave * bpw);
+    const int nloc = interleave ? (wave < G ? ((G - wave + 7) >> 3) << gs7 : 0) : min(NB, b0 + bpw) - b0;
+    auto blk_of = [&](int i) {
+        return interleave ? (((((i >> gs7) << 3) + wave) << gs7) | (i & bpg_mask)) : b0 + i;
+    };
     unsigned char *slot = pk4_lds + wave * SLOT;
 
     const __amdgpu_buffer_rsrc_t rs_w = make_rsrc(pw + (size_t)j * NS * 256, (uint32_t)NS * 1024u);
@@ -223,26 +227,34 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
         if (q * 512 < zchunks)  // block-uniform
             zstage[q] = __builtin_amdgcn_raw_buffer_load_b128(rs_z, (int)(threadIdx.x + q * 512) * 16, 0, 0);
 
-    u32x4_t areg[AQ], wr[2][4];
-    auto load_a = [&](int blk) {
-        const bool live = blk < b1;  // wave-uniform
+    constexpr int U = WB > AB ? WB : AB;  // unroll (both divide it)
+    u32x4_t aring[AB][AQ], wring[WB][4];
+    auto load_a = [&](int i, u32x4_t (&a)[AQ]) {
+        const bool live = i < nloc;  // wave-uniform
+        const int blk = blk_of(i);
 #pragma unroll
         for (int q = 0; q < AQ; ++q)
-            areg[q] = __builtin_amdgcn_raw_buffer_load_b128(rs_x, live ? voff_a[q] : OOB, blk * 256, 0);
+            a[q] = __builtin_amdgcn_raw_buffer_load_b128(rs_x, live ? voff_a[q] : OOB, blk * 256, 0);
     };
-    auto load_w = [&](int blk, int st, u32x4_t &w) {
-        w = __builtin_amdgcn_raw_buffer_load_b128(rs_w, blk < b1 ? voff_w : OOB, (blk * 4 + st) * 1024, 0);
+    auto load_w = [&](int i, int st, u32x4_t &w) {
+        w = __builtin_amdgcn_raw_buffer_load_b128(rs_w, i < nloc ? voff_w : OOB, (blk_of(i) * 4 + st) * 1024, 0);
     };
-    auto store_a = [&]() {
+    auto store_a = [&](const u32x4_t (&a)[AQ]) {
 #pragma unroll
-        for (int q = 0; q < AQ; ++q) *(u32x4_t *)(slot + a_wr[q]) = areg[q];
+        for (int q = 0; q < AQ; ++q) *(u32x4_t *)(slot + a_wr[q]) = a[q];
     };
 
-    load_a(b0);
+    // issue order = consumption order: A(b0), W(b0), A(b0+1), W(b0+1), ...
+    u32x4_t afirst[AQ];
+    load_a(0, afirst);
 #pragma unroll
-    for (int st = 0; st < 4; ++st) load_w(b0, st, wr[0][st]);
+    for (int d = 0; d < U; ++d) {
+        if (d < WB) {
 #pragma unroll
-    for (int st = 0; st < 4; ++st) load_w(b0 + 1, st, wr[1][st]);
+            for (int st = 0; st < 4; ++st) load_w(d, st, wring[d][st]);
+        }
+        if (d + 1 <= AB) load_a(d + 1, aring[(d + 1) % AB]);
+    }
 
     float4_t acc[MT][4];
 #pragma unroll
@@ -261,30 +273,31 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
         }
     }
     const uint32_t ones[4] = {TT::ONES, TT::ONES, TT::ONES, TT::ONES};
+    const float4_t zero4 = float4_t{0.f, 0.f, 0.f, 0.f};
 
 #pragma unroll
     for (int q = 0; q < ZCH; ++q)
         if ((int)threadIdx.x + q * 512 < zchunks) zs_lds[threadIdx.x + q * 512] = zstage[q];
-    store_a();
+    store_a(afirst);
     __syncthreads();
 
-    for (int bb = b0; bb < b1; bb += 2) {
+    for (int ib = 0; ib < nloc; ib += U) {
 #pragma unroll
-        for (int cur = 0; cur < 2; ++cur) {
-            const int blk = bb + cur;
-            load_a(blk + 1);
-            const bool live = blk < b1;  // wave-uniform
-            if (live && (blk & bpg_mask) == 0) {  // first block of a group
-                const u32x4_t zq = zs_lds[(blk >> (gshift - 7)) * 16 + ni];
+        for (int u = 0; u < U; ++u) {
+            const int i = ib + u;
+            const bool live = i < nloc;  // wave-uniform
+            const int blk = blk_of(i);
+            const bool gfirst = BPG1 || (blk & bpg_mask) == 0;
+            const bool glast = BPG1 || (blk & bpg_mask) == bpg_mask;
+            if (live && gfirst) {  // first block of a group
+                const u32x4_t zq = zs_lds[(blk >> gs7) * 16 + ni];
                 const uint32_t z0 = zq[0], z1 = zq[1], z2 = zq[2], z3 = zq[3];
                 const uint32_t zv[4] = {z0, z1, z2, z3};
 #pragma unroll
                 for (int f = 0; f < 4; ++f) {
                     if (GS) {
                         sf[f] = TT::to_f32((uint16_t)(zv[f] >> 16));
-                        // stored -(bias_f + z)  ->  -(BIAS + z)
-                        const float nzb = TT::to_f32((uint16_t)(zv[f] & 0xFFFFu)) + TT::bias(f) - Pk4Gs<TT>::BIAS;
-                        nszb[f] = sf[f] * nzb;
+                        nszb[f] = sf[f] * TT::to_f32((uint16_t)(zv[f] & 0xFFFFu));  // -s * (bias_f + z)
                     } else {
                         negzb[f] = perm_b32(zv[f], zv[f], 0x01000100u);
                         sp[f] = perm_b32(zv[f], zv[f], 0x03020302u);
@@ -293,8 +306,8 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
             }
 #pragma unroll
             for (int st = 0; st < 4; ++st) {
-                const u32x4_t wv = wr[cur][st];
-                load_w(blk + 2, st, wr[cur][st]);  // refill this ring slot
+                const u32x4_t wv = wring[u % WB][st];
+                load_w(i + WB, st, wring[u % WB][st]);  // refill this ring slot
                 if (live) {
                     const uint32_t w0 = wv[0], w1 = wv[1], w2 = wv[2], w3 = wv[3];
                     const uint32_t wp[4] = {w0, w1, w2, w3};
@@ -306,16 +319,19 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
                         a[mt][0] = a0, a[mt][1] = a1, a[mt][2] = a2, a[mt][3] = a3;
                     }
                     if (GS) {
+                        // with one block per group the first step starts from zero: no clearing
+                        const bool fresh = BPG1 && st == 0;
 #pragma unroll
                         for (int f = 0; f < 4; ++f) {
                             uint32_t b[4];
 #pragma unroll
-                            for (int pp = 0; pp < 4; ++pp) b[pp] = Pk4Gs<TT>::unpack(wp[pp], f, nm);
+                            for (int pp = 0; pp < 4; ++pp) b[pp] = TT::unpack1(wp[pp], f, nm);
 #pragma unroll
-                            for (int mt = 0; mt < MT; ++mt) tmp[mt][f] = Ops::mfma(a[mt], b, tmp[mt][f]);
+                            for (int mt = 0; mt < MT; ++mt)
+                                tmp[mt][f] = Ops::mfma(a[mt], b, fresh ? zero4 : tmp[mt][f]);
                         }
 #pragma unroll
-                        for (int mt = 0; mt < MT; ++mt) tmps[mt] = Ops::mfma(a[mt], ones, tmps[mt]);
+                        for (int mt = 0; mt < MT; ++mt) tmps[mt] = Ops::mfma(a[mt], ones, fresh ? zero4 : tmps[mt]);
                     } else {
 #pragma unroll
                         for (int f = 0; f < 4; ++f) {
@@ -329,7 +345,7 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
                     }
                 }
             }
-            if (GS && live && (blk & bpg_mask) == bpg_mask) {  // last block of the group: fold it in
+            if (GS && live && glast) {  // last block of the group: fold it in
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt) {
 #pragma unroll
@@ -337,12 +353,14 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
 #pragma unroll
                         for (int i = 0; i < 4; ++i)
                             acc[mt][f][i] = fmaf(sf[f], tmp[mt][f][i], fmaf(nszb[f], tmps[mt][i], acc[mt][f][i]));
-                        tmp[mt][f] = float4_t{0.f, 0.f, 0.f, 0.f};
+                        if (!BPG1) tmp[mt][f] = zero4;
                     }
-                    tmps[mt] = float4_t{0.f, 0.f, 0.f, 0.f};
+                    if (!BPG1) tmps[mt] = zero4;
                 }
             }
-            store_a();  // the next block's activations replace this one's (same wave: in order)
+            // the next block's activations replace this one's (same wave: LDS accesses stay in order)
+            store_a(aring[(u + 1) % AB]);
+            load_a(i + 1 + AB, aring[(u + 1) % AB]);
         }
     }
 
@@ -357,23 +375,36 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
                 float4_t{acc[mt][0][i], acc[mt][1][i], acc[mt][2][i], acc[mt][3][i]};
     __syncthreads();
 
-    // thread -> (row, 8 consecutive columns); partials added in wave order
-    const int ml = threadIdx.x >> 3, ch = threadIdx.x & 7;
+    // thread -> (row, CP consecutive columns), every thread busy where the tile allows;
+    // partials added in wave order.  A row of a partial tile is 64 consecutive floats.
+    constexpr int CP = MT == 1 ? 2 : MT == 2 ? 4 : 8;  // columns per thread
+    constexpr int TPR = 64 / CP;                        // threads per row
+    const int ml = threadIdx.x / TPR, c0 = (threadIdx.x % TPR) * CP;
     if (ml < ROWS && m0 + ml < M) {
         const int mt = ml >> 4, r = ml & 15, rb = r >> 2, i = r & 3;
-        const int l0 = rb * 16 + 2 * ch;
-        float4_t v0 = float4_t{0.f, 0.f, 0.f, 0.f}, v1 = v0;
+        const float *redf = (const float *)pk4_lds;
+        float v[CP];
+#pragma unroll
+        for (int c = 0; c < CP; ++c) v[c] = 0.f;
 #pragma unroll
         for (int s = 0; s < NW; ++s) {
-            const float4_t *src = red + ((s * MT + mt) * 4 + i) * 64 + l0;
-            v0 += src[0];
-            v1 += src[1];
-        }
-        const int n = 64 * j + 8 * ch;
-        float v[8] = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
-        uint32_t o[4];
+            const float *src = redf + ((s * MT + mt) * 4 + i) * 256 + rb * 64 + c0;
+            if (CP == 2) {
+                const float2 t = *(const float2 *)src;
+                v[0] += t.x, v[1] += t.y;
+            } else {
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
+                for (int h = 0; h < CP / 4; ++h) {
+                    const float4_t t = *(const float4_t *)(src + 4 * h);
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) v[4 * h + c] += t[c];
+                }
+            }
+        }
+        const int n = 64 * j + c0;
+        uint32_t o[CP / 2];
+#pragma unroll
+        for (int q = 0; q < CP / 2; ++q) {
             float lo = v[2 * q], hi = v[2 * q + 1];
             if (bias) {
                 lo += TT::to_f32(bias[n + 2 * q]);
@@ -381,7 +412,10 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
             }
             o[q] = (uint32_t)TT::from_f32(lo) | ((uint32_t)TT::from_f32(hi) << 16);
         }
-        *(u32x4_t *)(y + (size_t)(m0 + ml) * N + n) = u32x4_t{o[0], o[1], o[2], o[3]};
+        uint16_t *dst = y + (size_t)(m0 + ml) * N + n;
+        if (CP == 2) *(uint32_t *)dst = o[0];
+        else if (CP == 4) *(uint2 *)dst = uint2{o[0], o[1]};
+        else *(u32x4_t *)dst = u32x4_t{o[0], o[1], o[2], o[3]};
     }
 }
 
@@ -439,21 +473,42 @@ int launch_pk4_dequant(oxq_ctx *ctx, hipStream_t s, const Pk4Weights &w, void *o
     return OXQ_OK;
 }
 
-template <typename TT, int MT, bool GS>
-static int pk4_go(hipStream_t s, dim3 grid, const Pk4Problem &p, int bpw) {
+template <typename TT, int MT, bool GS, bool BPG1, int AB, int WB>
+static int pk4_go3(hipStream_t s, dim3 grid, const Pk4Problem &p, int bpw, int interleave) {
     const int G = (int)(p.w.K >> p.w.group_shift);
     const size_t lds = (size_t)8 * MT * 4096 + (size_t)G * 256;
-    static size_t attr_lds = 0;  // one instantiation per (TT, MT, GS)
+    static size_t attr_lds = 0;  // one per instantiation
     if (lds > attr_lds) {
-        OXQ_HIP_CHECK(hipFuncSetAttribute((const void *)pk4_mfma_kernel<TT, MT, GS>,
+        OXQ_HIP_CHECK(hipFuncSetAttribute((const void *)pk4_mfma_kernel<TT, MT, GS, BPG1, AB, WB>,
                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         attr_lds = lds;
     }
-    hipLaunchKernelGGL((pk4_mfma_kernel<TT, MT, GS>), grid, dim3(512), lds, s, (const uint16_t *)p.x, p.w.pw,
-                       p.w.pzs, (const uint16_t *)p.bias, (uint16_t *)p.y, (int)p.M, (int)p.w.K, (int)p.w.N,
-                       p.w.group_shift, bpw);
+    hipLaunchKernelGGL((pk4_mfma_kernel<TT, MT, GS, BPG1, AB, WB>), grid, dim3(512), lds, s,
+                       (const uint16_t *)p.x, p.w.pw, p.w.pzs, (const uint16_t *)p.bias, (uint16_t *)p.y,
+                       (int)p.M, (int)p.w.K, (int)p.w.N, p.w.group_shift, bpw, interleave);
     OXQ_HIP_CHECK(hipGetLastError());
     return OXQ_OK;
+}
+
+static int pk4_env(const char *name, int dflt) {
+    const char *e = getenv(name);
+    return e ? atoi(e) : dflt;
+}
+
+template <typename TT, int MT, bool GS>
+static int pk4_go(hipStream_t s, dim3 grid, const Pk4Problem &p, int bpw) {
+    const int il = pk4_env("OXQ_PK4_INTERLEAVE", 0);
+    if (MT == 1 && p.w.group_shift == 7 && p.w.dtype == OXQ_F16) {  // measurement aid: ring depth
+        switch (pk4_env("OXQ_PK4_RING", 0)) {
+        case 1: return pk4_go3<F16Traits, 1, true, true, 1, 1>(s, grid, p, bpw, il);
+        case 2: return pk4_go3<F16Traits, 1, true, true, 2, 2>(s, grid, p, bpw, il);
+        case 3: return pk4_go3<F16Traits, 1, true, true, 1, 2>(s, grid, p, bpw, il);
+        default: break;
+        }
+    }
+    return p.w.group_shift == 7
+               ? pk4_go3<TT, MT, GS, true, Pk4Ring<MT>::AB, Pk4Ring<MT>::WB>(s, grid, p, bpw, il)
+               : pk4_go3<TT, MT, GS, false, Pk4Ring<MT>::AB, Pk4Ring<MT>::WB>(s, grid, p, bpw, il);
 }
 
 int launch_pk4_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p) {

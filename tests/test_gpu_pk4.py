@@ -137,6 +137,26 @@ def test_repacked_forward_config1(m, K, N):
         np.testing.assert_array_equal(bits_of(layer.forward(xd)), first)
 
 
+@pytest.mark.parametrize("dtn", ["f16", "bf16"])
+def test_repacked_forward_biased_activations(dtn):
+    """m <= 16 feeds bias + q to the matrix cores and removes the bias with the row sums of x:
+    activations with a large mean and with outliers are where that cancellation is hardest."""
+    dt = DT[dtn]
+    K, N = 4096, 256
+    trip, pack_dim = make("awq", K, N, 128, seed=4242)
+    layer = layer_of(trip, pack_dim, dt)
+    w = dense("awq", trip, dt)
+    rng = np.random.default_rng(77)
+    cases = {"mean 3": 3.0 + 0.1 * rng.standard_normal((4, K)),
+             "positive": np.abs(rng.standard_normal((4, K))) * 2.0,
+             "outliers": rng.standard_normal((4, K)) * np.where(rng.random((4, K)) < 0.01, 60.0, 1.0)}
+    for name, x in cases.items():
+        say(f"pk4 forward {dtn} biased activations: {name}")
+        x = x.astype(np.float32)
+        ref = oracle.matmul_nt_f32(round_x(x, dt), w)
+        assert_close(layer.forward(to_dev(x, TORCH_DT[dt])), ref, f"pk4 {dtn} {name}")
+
+
 def test_repacked_forward_config2_gptq():
     """Benchmark config 2 (GPTQ 4-bit, K=5120, N=13824, g=128), bf16."""
     dt = oracle.BF16
