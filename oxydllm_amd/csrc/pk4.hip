@@ -40,6 +40,38 @@
 
 namespace oxq {
 
+// B = T((q - z) * s) for a pair of weights, from one pzs word {-(bias_f + z), s}.
+// prep() turns the word into two per-group registers, deq() applies them to a pair of
+// (bias_f + q).  f16: packed add (exact) and packed multiply (one rounding).  bf16 has no
+// packed arithmetic here: fma((bias + q), s, -(bias + z) * s) in f32 is exact (both
+// products fit 16 bits, their sum is the 13-bit (q - z) * s), then one hardware
+// round-to-nearest-even conversion of the pair.
+typedef float float2_t __attribute__((ext_vector_type(2)));
+template <typename TT> struct Pk4T;
+template <> struct Pk4T<F16Traits> {
+    __device__ static __forceinline__ void prep(uint32_t zs, uint32_t &c0, uint32_t &c1) {
+        c0 = perm_b32(zs, zs, 0x01000100u);
+        c1 = perm_b32(zs, zs, 0x03020302u);
+    }
+    __device__ static __forceinline__ uint32_t deq(uint32_t p, uint32_t c0, uint32_t c1) {
+        return MfmaOps<F16Traits>::dequant_pair(p, c0, c1);
+    }
+};
+template <> struct Pk4T<BF16Traits> {
+    __device__ static __forceinline__ void prep(uint32_t zs, uint32_t &c0, uint32_t &c1) {
+        const float sf = __builtin_bit_cast(float, zs & 0xFFFF0000u);
+        const float nz = __builtin_bit_cast(float, zs << 16);
+        c0 = __builtin_bit_cast(uint32_t, sf);
+        c1 = __builtin_bit_cast(uint32_t, nz * sf);
+    }
+    __device__ static __forceinline__ uint32_t deq(uint32_t p, uint32_t c0, uint32_t c1) {
+        const float sf = __builtin_bit_cast(float, c0), c = __builtin_bit_cast(float, c1);
+        const float lo = __builtin_fmaf(__builtin_bit_cast(float, p << 16), sf, c);
+        const float hi = __builtin_fmaf(__builtin_bit_cast(float, p & 0xFFFF0000u), sf, c);
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(float2_t{lo, hi}, bf16x2_t));
+    }
+};
+
 __device__ __forceinline__ int pk4_kk(int t, int kb) { return ((t >> 1) << 6) + (kb << 4) + ((t & 1) << 3); }
 
 // ---------------------------------------------------------------------------
@@ -114,8 +146,9 @@ __global__ __launch_bounds__(256) void pk4_dequant_kernel(const uint32_t *__rest
 #pragma unroll
     for (int f = 0; f < 4; ++f) {
         const uint32_t zs = pzs[(((size_t)j * G + g) * 16 + ni) * 4 + f];
-        const uint32_t nz = perm_b32(zs, zs, 0x01000100u), s2 = perm_b32(zs, zs, 0x03020302u);
-        const uint32_t d = Ops::dequant_pair(TT::unpack1(w, f, nm), nz, s2);
+        uint32_t c0, c1;
+        Pk4T<TT>::prep(zs, c0, c1);
+        const uint32_t d = Pk4T<TT>::deq(TT::unpack1(w, f, nm), c0, c1);
         const int col = 64 * j + 4 * ni + f;
         out[(size_t)k * N + col] = (uint16_t)(d & 0xFFFFu);
         out[(size_t)(k + 1) * N + col] = (uint16_t)(d >> 16);
@@ -174,7 +207,7 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
                                                        const uint32_t *__restrict__ pzs,
                                                        const uint16_t *__restrict__ bias,
                                                        uint16_t *__restrict__ y, int M, int K, int N,
-                                                       int gshift, int bpw, int interleave) {
+                                                       int gshift, int bpw, int interleave, int dbg) {
     typedef MfmaOps<TT> Ops;
     constexpr int NW = 8;
     constexpr int ROWS = 16 * MT;
@@ -230,14 +263,14 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
     constexpr int U = WB > AB ? WB : AB;  // unroll (both divide it)
     u32x4_t aring[AB][AQ], wring[WB][4];
     auto load_a = [&](int i, u32x4_t (&a)[AQ]) {
-        const bool live = i < nloc;  // wave-uniform
+        const bool live = i < nloc && !(dbg & 1);  // wave-uniform
         const int blk = blk_of(i);
 #pragma unroll
         for (int q = 0; q < AQ; ++q)
             a[q] = __builtin_amdgcn_raw_buffer_load_b128(rs_x, live ? voff_a[q] : OOB, blk * 256, 0);
     };
     auto load_w = [&](int i, int st, u32x4_t &w) {
-        w = __builtin_amdgcn_raw_buffer_load_b128(rs_w, i < nloc ? voff_w : OOB, (blk_of(i) * 4 + st) * 1024, 0);
+        w = __builtin_amdgcn_raw_buffer_load_b128(rs_w, (i < nloc && !(dbg & 2)) ? voff_w : OOB, (blk_of(i) * 4 + st) * 1024, 0);
     };
     auto store_a = [&](const u32x4_t (&a)[AQ]) {
 #pragma unroll
@@ -261,7 +294,7 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
         for (int f = 0; f < 4; ++f) acc[mt][f] = float4_t{0.f, 0.f, 0.f, 0.f};
-    uint32_t negzb[4], sp[4];          // GS = false: splatted -(bias + z) and s
+    uint32_t negzb[4], sp[4];          // GS = false: the two Pk4T constants per column
     float sf[4], nszb[4];              // GS = true: s and -s * (bias + z) in f32
     float4_t tmp[GS ? MT : 1][4], tmps[GS ? MT : 1];
     if (GS) {
@@ -299,8 +332,7 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
                         sf[f] = TT::to_f32((uint16_t)(zv[f] >> 16));
                         nszb[f] = sf[f] * TT::to_f32((uint16_t)(zv[f] & 0xFFFFu));  // -s * (bias_f + z)
                     } else {
-                        negzb[f] = perm_b32(zv[f], zv[f], 0x01000100u);
-                        sp[f] = perm_b32(zv[f], zv[f], 0x03020302u);
+                        Pk4T<TT>::prep(zv[f], negzb[f], sp[f]);
                     }
                 }
             }
@@ -338,7 +370,7 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
                             uint32_t b[4];
 #pragma unroll
                             for (int pp = 0; pp < 4; ++pp)
-                                b[pp] = Ops::dequant_pair(TT::unpack1(wp[pp], f, nm), negzb[f], sp[f]);
+                                b[pp] = Pk4T<TT>::deq(TT::unpack1(wp[pp], f, nm), negzb[f], sp[f]);
 #pragma unroll
                             for (int mt = 0; mt < MT; ++mt) acc[mt][f] = Ops::mfma(a[mt], b, acc[mt][f]);
                         }
@@ -473,6 +505,11 @@ int launch_pk4_dequant(oxq_ctx *ctx, hipStream_t s, const Pk4Weights &w, void *o
     return OXQ_OK;
 }
 
+static int pk4_env(const char *name, int dflt) {
+    const char *e = getenv(name);
+    return e ? atoi(e) : dflt;
+}
+
 template <typename TT, int MT, bool GS, bool BPG1, int AB, int WB>
 static int pk4_go3(hipStream_t s, dim3 grid, const Pk4Problem &p, int bpw, int interleave) {
     const int G = (int)(p.w.K >> p.w.group_shift);
@@ -485,14 +522,9 @@ static int pk4_go3(hipStream_t s, dim3 grid, const Pk4Problem &p, int bpw, int i
     }
     hipLaunchKernelGGL((pk4_mfma_kernel<TT, MT, GS, BPG1, AB, WB>), grid, dim3(512), lds, s,
                        (const uint16_t *)p.x, p.w.pw, p.w.pzs, (const uint16_t *)p.bias, (uint16_t *)p.y,
-                       (int)p.M, (int)p.w.K, (int)p.w.N, p.w.group_shift, bpw, interleave);
+                       (int)p.M, (int)p.w.K, (int)p.w.N, p.w.group_shift, bpw, interleave, pk4_env("OXQ_PK4_DBG", 0));
     OXQ_HIP_CHECK(hipGetLastError());
     return OXQ_OK;
-}
-
-static int pk4_env(const char *name, int dflt) {
-    const char *e = getenv(name);
-    return e ? atoi(e) : dflt;
 }
 
 template <typename TT, int MT, bool GS>
