@@ -207,7 +207,7 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
                                                        const uint32_t *__restrict__ pzs,
                                                        const uint16_t *__restrict__ bias,
                                                        uint16_t *__restrict__ y, int M, int K, int N,
-                                                       int gshift, int bpw, int interleave, int dbg) {
+                                                       int gshift, int bpw, int interleave) {
     typedef MfmaOps<TT> Ops;
     constexpr int NW = 8;
     constexpr int ROWS = 16 * MT;
@@ -244,7 +244,7 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
     for (int q = 0; q < AQ; ++q) {
         const int row = 4 * q + kb, r = m0 + row;
         voff_a[q] = r < M ? (r * K * 2 + ni * 16) : OOB;
-        a_wr[q] = row * 256 + ((ni ^ (row & 15)) << 4);
+        a_wr[q] = row * 256 + ((ni ^ (row & 15)) << 4);  // = kb*256 + ((ni^kb)<<4), xor (4q&15)<<4, + 1024q
     }
     // fragment read of step s (0..3), row tile mt: row 16mt + ni, chunk 8*(s/2) + 2kb + (s%2)
     int a_rd[4];
@@ -262,15 +262,18 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
 
     constexpr int U = WB > AB ? WB : AB;  // unroll (both divide it)
     u32x4_t aring[AB][AQ], wring[WB][4];
+    // Past the end of the slice the loads go through an empty descriptor: a scalar select,
+    // no vector instruction, and the buffer unit returns zero without touching memory.
+    const __amdgpu_buffer_rsrc_t rs_none = make_rsrc(pw, 0u);
     auto load_a = [&](int i, u32x4_t (&a)[AQ]) {
-        const bool live = i < nloc && !(dbg & 1);  // wave-uniform
+        const __amdgpu_buffer_rsrc_t rs = i < nloc ? rs_x : rs_none;  // wave-uniform
         const int blk = blk_of(i);
 #pragma unroll
-        for (int q = 0; q < AQ; ++q)
-            a[q] = __builtin_amdgcn_raw_buffer_load_b128(rs_x, live ? voff_a[q] : OOB, blk * 256, 0);
+        for (int q = 0; q < AQ; ++q) a[q] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff_a[q], blk * 256, 0);
     };
     auto load_w = [&](int i, int st, u32x4_t &w) {
-        w = __builtin_amdgcn_raw_buffer_load_b128(rs_w, (i < nloc && !(dbg & 2)) ? voff_w : OOB, (blk_of(i) * 4 + st) * 1024, 0);
+        const __amdgpu_buffer_rsrc_t rs = i < nloc ? rs_w : rs_none;
+        w = __builtin_amdgcn_raw_buffer_load_b128(rs, voff_w, (blk_of(i) * 4 + st) * 1024, 0);
     };
     auto store_a = [&](const u32x4_t (&a)[AQ]) {
 #pragma unroll
@@ -522,7 +525,7 @@ static int pk4_go3(hipStream_t s, dim3 grid, const Pk4Problem &p, int bpw, int i
     }
     hipLaunchKernelGGL((pk4_mfma_kernel<TT, MT, GS, BPG1, AB, WB>), grid, dim3(512), lds, s,
                        (const uint16_t *)p.x, p.w.pw, p.w.pzs, (const uint16_t *)p.bias, (uint16_t *)p.y,
-                       (int)p.M, (int)p.w.K, (int)p.w.N, p.w.group_shift, bpw, interleave, pk4_env("OXQ_PK4_DBG", 0));
+                       (int)p.M, (int)p.w.K, (int)p.w.N, p.w.group_shift, bpw, interleave);
     OXQ_HIP_CHECK(hipGetLastError());
     return OXQ_OK;
 }
