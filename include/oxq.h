@@ -216,9 +216,9 @@ int oxq_mxfp4_moe_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x,
 /* linear.rs:403-534 PackedQuantLinear::{new, forward}.  scales must already be
  * in the runtime dtype (`dtype`), as after the cast at linear.rs:437.
  *
- * Like the reference's constructor, `new` is the load-time step: for 4-bit
- * layers with in_features, out_features and group size all multiples of 64 it
- * builds a tile-major copy of qweight/qzeros/scales in device memory owned by
+ * Like the reference's constructor, `new` is the load-time step: for layers
+ * with in_features and group size multiples of 128, out_features a multiple
+ * of 64 and at most 128 groups it builds a tile-major copy of qweight/qzeros/scales in device memory owned by
  * the layer (same size as the checkpoint tensors, plus 1.5 bytes per column
  * and group) and forward never reads the caller's tensors again; it
  * synchronises the null stream once.  Other layers keep descriptors of the

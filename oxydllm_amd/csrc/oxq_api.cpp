@@ -701,14 +701,14 @@ struct oxq_packed_quant_linear {
     // below m = 64 is a full dense dequant.  Here every m > 8 runs the MFMA tile
     // kernel, which reads the packed weights once.
     int64_t gemv_max_m() const { return 8; }
-    // 4-bit layers with tile-aligned shapes keep a tile-major copy of the
+    // 4- and 8-bit layers with tile-aligned shapes keep a tile-major copy of the
     // weights made at load (pk4.hip); forward then runs one kernel for every m
     // and no longer touches the caller's checkpoint tensors.
     bool prepacked;
     Pk4Weights pk;
 };
 
-// Load-time repack of an eligible 4-bit layer.  Shapes the repacked kernels do
+// Load-time repack of an eligible layer.  Shapes the repacked kernels do
 // not cover simply keep the checkpoint layout; errors in the tensors themselves
 // surface at forward, where the reference reports them.
 static int prepack_layer(oxq_packed_quant_linear *l) {
@@ -729,6 +729,7 @@ static int prepack_layer(oxq_packed_quant_linear *l) {
     l->pk.N = src.N;
     l->pk.group_shift = src.group_shift;
     l->pk.dtype = l->dtype;
+    l->pk.bits = src.bits;
     if (ctx->plan_only) {
         l->prepacked = true;
         return OXQ_OK;
@@ -737,7 +738,7 @@ static int prepack_layer(oxq_packed_quant_linear *l) {
     (void)hipGetDevice(&prev);
     OXQ_HIP_CHECK(hipSetDevice(ctx->device));
     int rc = OXQ_OK;
-    hipError_t e = hipMalloc((void **)&l->pk.pw, pk4_weight_bytes(src.K, src.N));
+    hipError_t e = hipMalloc((void **)&l->pk.pw, pk4_weight_bytes(src.K, src.N, src.bits));
     if (e == hipSuccess) e = hipMalloc((void **)&l->pk.pzs, pk4_zs_bytes(src.K, src.N, src.group_shift));
     if (e != hipSuccess) {
         rc = fail(OXQ_ERR_RUNTIME, "PackedQuantLinear: repack allocation failed: %s", hipGetErrorString(e));
@@ -818,7 +819,7 @@ int oxq_packed_quant_linear_new(oxq_ctx *ctx, uint32_t bits, int pack_dim,
     l->pack_dim = pack_dim;
     l->dtype = dtype;
     l->prepacked = false;
-    l->pk = Pk4Weights{nullptr, nullptr, 0, 0, 0, dtype};
+    l->pk = Pk4Weights{nullptr, nullptr, 0, 0, 0, dtype, (int)bits};
     int rc = prepack_layer(l);
     if (rc != OXQ_OK) {
         oxq_packed_quant_linear_free(l);

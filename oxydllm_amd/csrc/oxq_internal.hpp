@@ -103,13 +103,14 @@ struct Mxfp4Problem {
     int64_t n_pairs;
 };
 
-// A resident 4-bit layer repacked tile-major at load (layout: pk4.hip).
+// A resident 4- or 8-bit layer repacked tile-major at load (layout: pk4.hip).
 struct Pk4Weights {
-    uint32_t *pw;           // [N/64][K/32][64][4]
+    uint32_t *pw;           // [N/64][K/32][bits/4][64][4]
     uint32_t *pzs;          // [N/64][K/g][16][4]  {-(bias + z), s} pairs of the layer dtype
     int64_t K, N;
     int group_shift;
     int dtype;              // OXQ_F16 / OXQ_BF16
+    int bits;               // 4 or 8
 };
 
 struct Pk4Problem {
@@ -122,7 +123,7 @@ struct Pk4Problem {
 
 // ---- launchers (defined in the .hip files) ---------------------------------
 bool pk4_eligible(const Wna16Problem &p);
-size_t pk4_weight_bytes(int64_t K, int64_t N);
+size_t pk4_weight_bytes(int64_t K, int64_t N, int bits);
 size_t pk4_zs_bytes(int64_t K, int64_t N, int group_shift);
 int launch_pk4_prepack(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &src, const Pk4Weights &dst);
 int launch_pk4_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p);

@@ -32,6 +32,12 @@
 // into two exact 16-bit floats (bias + q).  A pzs word is {-(bias_f + z), s} as
 // two 16-bit floats of the layer's dtype (z already includes GPTQ's +1).
 
+//
+// 8-bit layers use the same scheme with two 1 KB loads per step: half h (0..1) of a step
+// holds the column pair f = 2h, 2h+1; word pp = {q[kk+2pp][2h], q[kk+2pp][2h+1],
+// q[kk+2pp+1][2h], q[kk+2pp+1][2h+1]} as bytes, so an AND-OR of bytes 0 and 2 (after a
+// shift by 8 for the odd column) again yields a row pair as two exact 16-bit floats.
+
 #include "oxq_device.hpp"
 #include "oxq_internal.hpp"
 #include "oxq_mfma.hpp"
@@ -77,49 +83,63 @@ __device__ __forceinline__ int pk4_kk(int t, int kb) { return ((t >> 1) << 6) + 
 // ---------------------------------------------------------------------------
 // load-time repack
 // ---------------------------------------------------------------------------
-template <bool GPTQ>
-__device__ __forceinline__ uint32_t src_nibble(const uint32_t *__restrict__ qw, int k, int col, int N) {
-    if (GPTQ) return (qw[(size_t)(k >> 3) * N + col] >> (4 * (k & 7))) & 0xFu;
-    const int c = col & 7;
-    const int slot = (c >> 1) | ((c & 1) << 2);  // inverse of the AWQ order [0,2,4,6,1,3,5,7]
-    return (qw[(size_t)k * (N >> 3) + (col >> 3)] >> (4 * slot)) & 0xFu;
+template <bool GPTQ, int BITS>
+__device__ __forceinline__ uint32_t src_q(const uint32_t *__restrict__ qw, int k, int col, int N) {
+    constexpr int PF = 32 / BITS;
+    constexpr uint32_t MASK = (1u << BITS) - 1u;
+    if (GPTQ) return (qw[(size_t)(k / PF) * N + col] >> (BITS * (k % PF))) & MASK;
+    const int c = col % PF;
+    // 4-bit AWQ interleaves the 8 columns of a word ([0,2,4,6,1,3,5,7]); 8-bit is in order
+    const int slot = BITS == 4 ? ((c >> 1) | ((c & 1) << 2)) : c;
+    return (qw[(size_t)k * (N / PF) + col / PF] >> (BITS * slot)) & MASK;
 }
 
-template <bool GPTQ>
+template <bool GPTQ, int BITS>
 __global__ __launch_bounds__(256) void pk4_prepack_weights_kernel(const uint32_t *__restrict__ qw,
                                                                   uint32_t *__restrict__ pw, int K, int N) {
     const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
-    const size_t total = (size_t)K * N / 8;
+    const size_t total = (size_t)K * N * BITS / 32;
     if (idx >= total) return;
     const int NS = K >> 5;
     const int pp = (int)(idx & 3), l = (int)((idx >> 2) & 63);
-    const size_t st = idx >> 8;
+    const int h = BITS == 8 ? (int)((idx >> 8) & 1) : 0;
+    const size_t st = idx >> (BITS == 8 ? 9 : 8);
     const int t = (int)(st % NS), j = (int)(st / NS);
     const int ni = l & 15, kb = l >> 4;
     const int k = pk4_kk(t, kb) + 2 * pp;
     uint32_t w = 0;
+    if (BITS == 4) {
 #pragma unroll
-    for (int h = 0; h < 2; ++h)
+        for (int r = 0; r < 2; ++r)
 #pragma unroll
-        for (int f = 0; f < 4; ++f)
-            w |= src_nibble<GPTQ>(qw, k + h, 64 * j + 4 * ni + f, N) << (16 * h + 4 * f);
+            for (int f = 0; f < 4; ++f)
+                w |= src_q<GPTQ, BITS>(qw, k + r, 64 * j + 4 * ni + f, N) << (16 * r + 4 * f);
+    } else {
+#pragma unroll
+        for (int r = 0; r < 2; ++r)
+#pragma unroll
+            for (int c = 0; c < 2; ++c)
+                w |= src_q<GPTQ, BITS>(qw, k + r, 64 * j + 4 * ni + 2 * h + c, N) << (16 * r + 8 * c);
+    }
     pw[idx] = w;
 }
 
-template <typename TT, bool GPTQ>
+template <typename TT, bool GPTQ, int BITS>
 __global__ __launch_bounds__(256) void pk4_prepack_zs_kernel(const uint32_t *__restrict__ qz,
                                                              const uint16_t *__restrict__ sc,
                                                              uint32_t *__restrict__ pzs, int G, int N) {
+    constexpr int PF = 32 / BITS;
     const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (idx >= (size_t)G * N) return;
     const int f = (int)(idx & 3), ni = (int)((idx >> 2) & 15);
     const size_t jg = idx >> 6;
     const int g = (int)(jg % G), j = (int)(jg / G);
     const int col = 64 * j + 4 * ni + f;
-    const int c = col & 7;
-    const int slot = GPTQ ? c : ((c >> 1) | ((c & 1) << 2));
-    const uint32_t z = ((qz[(size_t)g * (N >> 3) + (col >> 3)] >> (4 * slot)) & 0xFu) + (GPTQ ? 1u : 0u);
-    const uint32_t nz = TT::from_f32(-((float)z + TT::bias(f)));
+    const int c = col % PF;
+    const int slot = (GPTQ || BITS == 8) ? c : ((c >> 1) | ((c & 1) << 2));
+    const uint32_t z = ((qz[(size_t)g * (N / PF) + col / PF] >> (BITS * slot)) & ((1u << BITS) - 1u)) + (GPTQ ? 1u : 0u);
+    const float b = BITS == 4 ? TT::bias(f) : TT::BYTE_BIAS;
+    const uint32_t nz = TT::from_f32(-((float)z + b));
     pzs[idx] = nz | ((uint32_t)sc[(size_t)g * N + col] << 16);
 }
 
@@ -127,16 +147,16 @@ __global__ __launch_bounds__(256) void pk4_prepack_zs_kernel(const uint32_t *__r
 // dense dequant of a resident layer -> [K, N] (linear.rs:510-523 fallback);
 // the same arithmetic as the matmul kernel's B fragments.
 // ---------------------------------------------------------------------------
-template <typename TT>
+template <typename TT, int BITS>
 __global__ __launch_bounds__(256) void pk4_dequant_kernel(const uint32_t *__restrict__ pw,
                                                           const uint32_t *__restrict__ pzs,
                                                           uint16_t *__restrict__ out, int K, int N, int gshift) {
-    typedef MfmaOps<TT> Ops;
     const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= (size_t)K * N / 8) return;
+    if (idx >= (size_t)K * N * BITS / 32) return;
     const int NS = K >> 5, G = K >> gshift;
     const int pp = (int)(idx & 3), l = (int)((idx >> 2) & 63);
-    const size_t st = idx >> 8;
+    const int h = BITS == 8 ? (int)((idx >> 8) & 1) : 0;
+    const size_t st = idx >> (BITS == 8 ? 9 : 8);
     const int t = (int)(st % NS), j = (int)(st / NS);
     const int ni = l & 15, kb = l >> 4;
     const int k = pk4_kk(t, kb) + 2 * pp;
@@ -144,11 +164,13 @@ __global__ __launch_bounds__(256) void pk4_dequant_kernel(const uint32_t *__rest
     const uint32_t w = pw[idx];
     const NibbleMasks nm = nibble_masks();
 #pragma unroll
-    for (int f = 0; f < 4; ++f) {
+    for (int c = 0; c < (BITS == 4 ? 4 : 2); ++c) {
+        const int f = BITS == 4 ? c : 2 * h + c;
         const uint32_t zs = pzs[(((size_t)j * G + g) * 16 + ni) * 4 + f];
         uint32_t c0, c1;
         Pk4T<TT>::prep(zs, c0, c1);
-        const uint32_t d = Pk4T<TT>::deq(TT::unpack1(w, f, nm), c0, c1);
+        const uint32_t pair = BITS == 4 ? TT::unpack1(w, f, nm) : TT::unpack_bytes(c ? (w >> 8) : w);
+        const uint32_t d = Pk4T<TT>::deq(pair, c0, c1);
         const int col = 64 * j + 4 * ni + f;
         out[(size_t)k * N + col] = (uint16_t)(d & 0xFFFFu);
         out[(size_t)(k + 1) * N + col] = (uint16_t)(d >> 16);
@@ -194,14 +216,13 @@ __global__ __launch_bounds__(256) void pk4_dequant_kernel(const uint32_t *__rest
 // Ring depths in 128-row blocks: weights WB, activations AB (registers; the current
 // block's activations live in LDS).  Deeper rings measured no faster: at these sizes the
 // kernel is bound by instruction issue, not by memory latency.
-template <int MT> struct Pk4Ring {
+template <int MT, int BITS> struct Pk4Ring {
     static constexpr int AB = 1;
-    static constexpr int WB = 2;
-    static constexpr int U = WB > AB ? WB : AB;  // unroll (both divide it)
+    static constexpr int WB = (BITS == 8 && MT >= 3) ? 1 : 2;  // 8-bit weights take twice the registers
 };
 
 // BPG1: group size 128, i.e. every block is one group (no group bookkeeping).
-template <typename TT, int MT, bool GS, bool BPG1, int AB, int WB>
+template <typename TT, int BITS, int MT, bool GS, bool BPG1, int AB, int WB>
 __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restrict__ x,
                                                        const uint32_t *__restrict__ pw,
                                                        const uint32_t *__restrict__ pzs,
@@ -214,6 +235,7 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
     constexpr int AQ = 4 * MT;                 // activation loads per block and lane
     constexpr int SLOT = ROWS * 256;           // bytes of one wave's LDS slot (= its partial tile)
     constexpr int OOB = 0x7FFFFF00;
+    constexpr int WL = BITS / 4;               // 1 KB weight loads per step
     extern __shared__ __attribute__((aligned(16))) unsigned char pk4_lds[];
     u32x4_t *zs_lds = (u32x4_t *)(pk4_lds + NW * SLOT);  // [G][16]: the strip's {-(bias+z), s} words
 
@@ -234,7 +256,7 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
     };
     unsigned char *slot = pk4_lds + wave * SLOT;
 
-    const __amdgpu_buffer_rsrc_t rs_w = make_rsrc(pw + (size_t)j * NS * 256, (uint32_t)NS * 1024u);
+    const __amdgpu_buffer_rsrc_t rs_w = make_rsrc(pw + (size_t)j * NS * 256 * WL, (uint32_t)NS * 1024u * WL);
     const __amdgpu_buffer_rsrc_t rs_z = make_rsrc(pzs + (size_t)j * G * 64, (uint32_t)G * 256u);
     const __amdgpu_buffer_rsrc_t rs_x = make_rsrc(x, (uint32_t)M * (uint32_t)K * 2u);
     const int voff_w = lane * 16;
@@ -261,7 +283,7 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
             zstage[q] = __builtin_amdgcn_raw_buffer_load_b128(rs_z, (int)(threadIdx.x + q * 512) * 16, 0, 0);
 
     constexpr int U = WB > AB ? WB : AB;  // unroll (both divide it)
-    u32x4_t aring[AB][AQ], wring[WB][4];
+    u32x4_t aring[AB][AQ], wring[WB][4][WL];
     // Past the end of the slice the loads go through an empty descriptor: a scalar select,
     // no vector instruction, and the buffer unit returns zero without touching memory.
     const __amdgpu_buffer_rsrc_t rs_none = make_rsrc(pw, 0u);
@@ -271,9 +293,11 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
 #pragma unroll
         for (int q = 0; q < AQ; ++q) a[q] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff_a[q], blk * 256, 0);
     };
-    auto load_w = [&](int i, int st, u32x4_t &w) {
+    auto load_w = [&](int i, int st, u32x4_t (&w)[WL]) {
         const __amdgpu_buffer_rsrc_t rs = i < nloc ? rs_w : rs_none;
-        w = __builtin_amdgcn_raw_buffer_load_b128(rs, voff_w, (blk_of(i) * 4 + st) * 1024, 0);
+#pragma unroll
+        for (int h = 0; h < WL; ++h)
+            w[h] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff_w, ((blk_of(i) * 4 + st) * WL + h) * 1024, 0);
     };
     auto store_a = [&](const u32x4_t (&a)[AQ]) {
 #pragma unroll
@@ -341,11 +365,23 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
             }
 #pragma unroll
             for (int st = 0; st < 4; ++st) {
-                const u32x4_t wv = wring[u % WB][st];
+                u32x4_t wv[WL];
+#pragma unroll
+                for (int h = 0; h < WL; ++h) wv[h] = wring[u % WB][st][h];
                 load_w(i + WB, st, wring[u % WB][st]);  // refill this ring slot
                 if (live) {
-                    const uint32_t w0 = wv[0], w1 = wv[1], w2 = wv[2], w3 = wv[3];
-                    const uint32_t wp[4] = {w0, w1, w2, w3};
+                    uint32_t wp[WL][4];
+#pragma unroll
+                    for (int h = 0; h < WL; ++h) {
+                        const uint32_t w0 = wv[h][0], w1 = wv[h][1], w2 = wv[h][2], w3 = wv[h][3];
+                        wp[h][0] = w0, wp[h][1] = w1, wp[h][2] = w2, wp[h][3] = w3;
+                    }
+                    // row pair pp of column f as two exact 16-bit floats bias + q
+                    auto pair = [&](int pp, int f) -> uint32_t {
+                        if (BITS == 4) return TT::unpack1(wp[0][pp], f, nm);
+                        const uint32_t word = wp[(f >> 1) % WL][pp];
+                        return TT::unpack_bytes((f & 1) ? (word >> 8) : word);
+                    };
                     uint32_t a[MT][4];
 #pragma unroll
                     for (int mt = 0; mt < MT; ++mt) {
@@ -360,7 +396,7 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
                         for (int f = 0; f < 4; ++f) {
                             uint32_t b[4];
 #pragma unroll
-                            for (int pp = 0; pp < 4; ++pp) b[pp] = TT::unpack1(wp[pp], f, nm);
+                            for (int pp = 0; pp < 4; ++pp) b[pp] = pair(pp, f);
 #pragma unroll
                             for (int mt = 0; mt < MT; ++mt)
                                 tmp[mt][f] = Ops::mfma(a[mt], b, fresh ? zero4 : tmp[mt][f]);
@@ -373,7 +409,7 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
                             uint32_t b[4];
 #pragma unroll
                             for (int pp = 0; pp < 4; ++pp)
-                                b[pp] = Pk4T<TT>::deq(TT::unpack1(wp[pp], f, nm), negzb[f], sp[f]);
+                                b[pp] = Pk4T<TT>::deq(pair(pp, f), negzb[f], sp[f]);
 #pragma unroll
                             for (int mt = 0; mt < MT; ++mt) acc[mt][f] = Ops::mfma(a[mt], b, acc[mt][f]);
                         }
@@ -458,52 +494,65 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
 // host side
 // ---------------------------------------------------------------------------
 bool pk4_eligible(const Wna16Problem &p) {
-    if (p.bits != 4) return false;
+    if (p.bits != 4 && p.bits != 8) return false;
     if (p.K % 128 != 0 || p.N % 64 != 0 || p.group_size % 128 != 0) return false;
-    if ((uint64_t)p.K * (uint64_t)p.N / 2 >= (1ull << 31)) return false;  // 32-bit offsets inside a strip and in x
+    if ((uint64_t)p.K * (uint64_t)p.N * p.bits / 8 >= (1ull << 31)) return false;  // 32-bit offsets in a strip and in x
     if (p.K / p.group_size > 128) return false;  // a strip's zeros and scales must fit 32 KB of LDS
     return true;
 }
 
-size_t pk4_weight_bytes(int64_t K, int64_t N) { return (size_t)K * (size_t)N / 2; }
+size_t pk4_weight_bytes(int64_t K, int64_t N, int bits) { return (size_t)K * (size_t)N * bits / 8; }
 size_t pk4_zs_bytes(int64_t K, int64_t N, int gshift) { return (size_t)(K >> gshift) * (size_t)N * 4; }
+
+template <bool GPTQ, int BITS>
+static void pk4_prepack_go(hipStream_t s, dim3 gw, dim3 gz, const Wna16Problem &src, const Pk4Weights &dst, int K,
+                           int N, int G) {
+    dim3 block(256);
+    hipLaunchKernelGGL((pk4_prepack_weights_kernel<GPTQ, BITS>), gw, block, 0, s, src.qweight, dst.pw, K, N);
+    if (src.dtype == OXQ_F16)
+        hipLaunchKernelGGL((pk4_prepack_zs_kernel<F16Traits, GPTQ, BITS>), gz, block, 0, s, src.qzeros,
+                           (const uint16_t *)src.scales, dst.pzs, G, N);
+    else
+        hipLaunchKernelGGL((pk4_prepack_zs_kernel<BF16Traits, GPTQ, BITS>), gz, block, 0, s, src.qzeros,
+                           (const uint16_t *)src.scales, dst.pzs, G, N);
+}
 
 int launch_pk4_prepack(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &src, const Pk4Weights &dst) {
     const int K = (int)src.K, N = (int)src.N, G = (int)(src.K >> src.group_shift);
-    const size_t words = (size_t)K * N / 8, zsn = (size_t)G * N;
+    const size_t words = (size_t)K * N * src.bits / 32, zsn = (size_t)G * N;
     const bool gptq = src.pack_dim == OXQ_PACK_IN;
     dim3 gw((unsigned)ceil_div((int64_t)words, 256)), gz((unsigned)ceil_div((int64_t)zsn, 256)), block(256);
-    set_plan(ctx, gptq ? "pk4_prepack_gptq" : "pk4_prepack_awq", gw, block, 1, 2, 0);
+    char name[64];
+    snprintf(name, sizeof name, "pk%d_prepack_%s", src.bits, gptq ? "gptq" : "awq");
+    set_plan(ctx, name, gw, block, 1, 2, 0);
     if (ctx->plan_only) return OXQ_OK;
-    if (gptq)
-        hipLaunchKernelGGL(pk4_prepack_weights_kernel<true>, gw, block, 0, s, src.qweight, dst.pw, K, N);
-    else
-        hipLaunchKernelGGL(pk4_prepack_weights_kernel<false>, gw, block, 0, s, src.qweight, dst.pw, K, N);
-    OXQ_HIP_CHECK(hipGetLastError());
-#define OXQ_ZS(TTv, GP)                                                                              \
-    hipLaunchKernelGGL((pk4_prepack_zs_kernel<TTv, GP>), gz, block, 0, s, src.qzeros,               \
-                       (const uint16_t *)src.scales, dst.pzs, G, N)
-    if (src.dtype == OXQ_F16) {
-        if (gptq) OXQ_ZS(F16Traits, true); else OXQ_ZS(F16Traits, false);
+    if (src.bits == 4) {
+        if (gptq) pk4_prepack_go<true, 4>(s, gw, gz, src, dst, K, N, G);
+        else pk4_prepack_go<false, 4>(s, gw, gz, src, dst, K, N, G);
     } else {
-        if (gptq) OXQ_ZS(BF16Traits, true); else OXQ_ZS(BF16Traits, false);
+        if (gptq) pk4_prepack_go<true, 8>(s, gw, gz, src, dst, K, N, G);
+        else pk4_prepack_go<false, 8>(s, gw, gz, src, dst, K, N, G);
     }
-#undef OXQ_ZS
     OXQ_HIP_CHECK(hipGetLastError());
     return OXQ_OK;
 }
 
 int launch_pk4_dequant(oxq_ctx *ctx, hipStream_t s, const Pk4Weights &w, void *out_kn) {
-    const size_t words = (size_t)w.K * w.N / 8;
+    const size_t words = (size_t)w.K * w.N * w.bits / 32;
     dim3 grid((unsigned)ceil_div((int64_t)words, 256)), block(256);
-    set_plan(ctx, w.dtype == OXQ_F16 ? "pk4_dequant_f16" : "pk4_dequant_bf16", grid, block, 1, 1, 0);
+    char name[64];
+    snprintf(name, sizeof name, "pk%d_dequant_%s", w.bits, w.dtype == OXQ_F16 ? "f16" : "bf16");
+    set_plan(ctx, name, grid, block, 1, 1, 0);
     if (ctx->plan_only) return OXQ_OK;
-    if (w.dtype == OXQ_F16)
-        hipLaunchKernelGGL(pk4_dequant_kernel<F16Traits>, grid, block, 0, s, w.pw, w.pzs, (uint16_t *)out_kn,
-                           (int)w.K, (int)w.N, w.group_shift);
-    else
-        hipLaunchKernelGGL(pk4_dequant_kernel<BF16Traits>, grid, block, 0, s, w.pw, w.pzs, (uint16_t *)out_kn,
-                           (int)w.K, (int)w.N, w.group_shift);
+#define OXQ_DQ(TTv, Bv)                                                                                     \
+    hipLaunchKernelGGL((pk4_dequant_kernel<TTv, Bv>), grid, block, 0, s, w.pw, w.pzs, (uint16_t *)out_kn, \
+                       (int)w.K, (int)w.N, w.group_shift)
+    if (w.dtype == OXQ_F16) {
+        if (w.bits == 4) OXQ_DQ(F16Traits, 4); else OXQ_DQ(F16Traits, 8);
+    } else {
+        if (w.bits == 4) OXQ_DQ(BF16Traits, 4); else OXQ_DQ(BF16Traits, 8);
+    }
+#undef OXQ_DQ
     OXQ_HIP_CHECK(hipGetLastError());
     return OXQ_OK;
 }
@@ -513,37 +562,39 @@ static int pk4_env(const char *name, int dflt) {
     return e ? atoi(e) : dflt;
 }
 
-template <typename TT, int MT, bool GS, bool BPG1, int AB, int WB>
-static int pk4_go3(hipStream_t s, dim3 grid, const Pk4Problem &p, int bpw, int interleave) {
+template <typename TT, int BITS, int MT, bool GS, bool BPG1>
+static int pk4_go3(hipStream_t s, dim3 grid, const Pk4Problem &p, int bpw) {
+    constexpr int AB = Pk4Ring<MT, BITS>::AB, WB = Pk4Ring<MT, BITS>::WB;
     const int G = (int)(p.w.K >> p.w.group_shift);
     const size_t lds = (size_t)8 * MT * 4096 + (size_t)G * 256;
     static size_t attr_lds = 0;  // one per instantiation
     if (lds > attr_lds) {
-        OXQ_HIP_CHECK(hipFuncSetAttribute((const void *)pk4_mfma_kernel<TT, MT, GS, BPG1, AB, WB>,
+        OXQ_HIP_CHECK(hipFuncSetAttribute((const void *)pk4_mfma_kernel<TT, BITS, MT, GS, BPG1, AB, WB>,
                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         attr_lds = lds;
     }
-    hipLaunchKernelGGL((pk4_mfma_kernel<TT, MT, GS, BPG1, AB, WB>), grid, dim3(512), lds, s,
+    hipLaunchKernelGGL((pk4_mfma_kernel<TT, BITS, MT, GS, BPG1, AB, WB>), grid, dim3(512), lds, s,
                        (const uint16_t *)p.x, p.w.pw, p.w.pzs, (const uint16_t *)p.bias, (uint16_t *)p.y,
-                       (int)p.M, (int)p.w.K, (int)p.w.N, p.w.group_shift, bpw, interleave);
+                       (int)p.M, (int)p.w.K, (int)p.w.N, p.w.group_shift, bpw,
+                       pk4_env("OXQ_PK4_INTERLEAVE", 0));
     OXQ_HIP_CHECK(hipGetLastError());
     return OXQ_OK;
 }
 
-template <typename TT, int MT, bool GS>
+template <typename TT, int BITS, int MT, bool GS>
 static int pk4_go(hipStream_t s, dim3 grid, const Pk4Problem &p, int bpw) {
-    const int il = pk4_env("OXQ_PK4_INTERLEAVE", 0);
-    if (MT == 1 && p.w.group_shift == 7 && p.w.dtype == OXQ_F16) {  // measurement aid: ring depth
-        switch (pk4_env("OXQ_PK4_RING", 0)) {
-        case 1: return pk4_go3<F16Traits, 1, true, true, 1, 1>(s, grid, p, bpw, il);
-        case 2: return pk4_go3<F16Traits, 1, true, true, 2, 2>(s, grid, p, bpw, il);
-        case 3: return pk4_go3<F16Traits, 1, true, true, 1, 2>(s, grid, p, bpw, il);
-        default: break;
-        }
+    return p.w.group_shift == 7 ? pk4_go3<TT, BITS, MT, GS, true>(s, grid, p, bpw)
+                                : pk4_go3<TT, BITS, MT, GS, false>(s, grid, p, bpw);
+}
+
+template <typename TT, int BITS>
+static int pk4_by_mt(hipStream_t s, dim3 grid, const Pk4Problem &p, int bpw, int mt) {
+    switch (mt) {
+    case 1: return pk4_go<TT, BITS, 1, true>(s, grid, p, bpw);
+    case 2: return pk4_go<TT, BITS, 2, false>(s, grid, p, bpw);
+    case 3: return pk4_go<TT, BITS, 3, false>(s, grid, p, bpw);
+    default: return pk4_go<TT, BITS, 4, false>(s, grid, p, bpw);
     }
-    return p.w.group_shift == 7
-               ? pk4_go3<TT, MT, GS, true, Pk4Ring<MT>::AB, Pk4Ring<MT>::WB>(s, grid, p, bpw, il)
-               : pk4_go3<TT, MT, GS, false, Pk4Ring<MT>::AB, Pk4Ring<MT>::WB>(s, grid, p, bpw, il);
 }
 
 int launch_pk4_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p) {
@@ -553,21 +604,18 @@ int launch_pk4_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p) {
     const int bpw = (int)ceil_div(G, 8) << (p.w.group_shift - 7);  // whole groups per wave, in 128-row blocks
     dim3 grid((unsigned)(p.w.N / 64), 1, (unsigned)ceil_div(M, 16 * mt));
     char name[64];
-    snprintf(name, sizeof name, "pk4_mfma_%s_mt%d%s", p.w.dtype == OXQ_F16 ? "f16" : "bf16", mt,
+    snprintf(name, sizeof name, "pk%d_mfma_%s_mt%d%s", p.w.bits, p.w.dtype == OXQ_F16 ? "f16" : "bf16", mt,
              mt == 1 ? "_gs" : "");
     set_plan(ctx, name, grid, dim3(512), 1, 1, 0);
     if (ctx->plan_only) return OXQ_OK;
     if ((uint64_t)M * (uint64_t)p.w.K * 2 >= (1ull << 31))
-        return fail(OXQ_ERR_UNSUPPORTED, "pk4 matmul: x larger than 2 GiB");
+        return fail(OXQ_ERR_UNSUPPORTED, "repacked matmul: x larger than 2 GiB");
     if (((uintptr_t)p.x | (uintptr_t)p.y) & 15)
-        return fail(OXQ_ERR_UNSUPPORTED, "pk4 matmul: x and y must be 16-byte aligned");
+        return fail(OXQ_ERR_UNSUPPORTED, "repacked matmul: x and y must be 16-byte aligned");
     const bool f16 = p.w.dtype == OXQ_F16;
-    switch (mt) {
-    case 1: return f16 ? pk4_go<F16Traits, 1, true>(s, grid, p, bpw) : pk4_go<BF16Traits, 1, true>(s, grid, p, bpw);
-    case 2: return f16 ? pk4_go<F16Traits, 2, false>(s, grid, p, bpw) : pk4_go<BF16Traits, 2, false>(s, grid, p, bpw);
-    case 3: return f16 ? pk4_go<F16Traits, 3, false>(s, grid, p, bpw) : pk4_go<BF16Traits, 3, false>(s, grid, p, bpw);
-    default: return f16 ? pk4_go<F16Traits, 4, false>(s, grid, p, bpw) : pk4_go<BF16Traits, 4, false>(s, grid, p, bpw);
-    }
+    if (p.w.bits == 4)
+        return f16 ? pk4_by_mt<F16Traits, 4>(s, grid, p, bpw, mt) : pk4_by_mt<BF16Traits, 4>(s, grid, p, bpw, mt);
+    return f16 ? pk4_by_mt<F16Traits, 8>(s, grid, p, bpw, mt) : pk4_by_mt<BF16Traits, 8>(s, grid, p, bpw, mt);
 }
 
 }  // namespace oxq

@@ -38,34 +38,43 @@ def say(msg):
 DT = {"f16": oracle.F16, "bf16": oracle.BF16}
 
 
+KINDS = ["awq", "gptq", "awq8", "gptq8"]
+
+
+def bits_of_kind(kind):
+    return 8 if kind.endswith("8") else 4
+
+
 def make(kind, K, N, g, seed):
-    if kind == "awq":
-        trip = synth.awq_checkpoint(K, N, g, 4, seed=seed)
-        return trip, ops.PACK_OUT
-    return synth.gptq_checkpoint(K, N, g, 4, seed=seed), ops.PACK_IN
+    bits = bits_of_kind(kind)
+    if kind.startswith("awq"):
+        return synth.awq_checkpoint(K, N, g, bits, seed=seed), ops.PACK_OUT
+    return synth.gptq_checkpoint(K, N, g, bits, seed=seed), ops.PACK_IN
 
 
 def dense(kind, trip, dt):
     s_r = oracle.round_through(trip[2], dt)
     if kind == "awq":
         return oracle.dequantize_awq(trip[0], trip[1], s_r)
-    return oracle.dequantize_gptq(trip[0], trip[1], s_r, 4)
+    if kind == "awq8":
+        return oracle.dequantize_awq8(trip[0], trip[1], s_r)
+    return oracle.dequantize_gptq(trip[0], trip[1], s_r, bits_of_kind(kind))
 
 
-def layer_of(trip, pack_dim, dt, bias=None):
+def layer_of(trip, pack_dim, dt, bias=None, bits=4):
     tdt = TORCH_DT[dt]
     b = None if bias is None else to_dev(bias, tdt)
-    return ops.PackedQuantLinear(4, pack_dim, to_dev(trip[0]), to_dev(trip[1]), to_dev(trip[2], tdt), b, tdt)
+    return ops.PackedQuantLinear(bits, pack_dim, to_dev(trip[0]), to_dev(trip[1]), to_dev(trip[2], tdt), b, tdt)
 
 
-@pytest.mark.parametrize("kind", ["awq", "gptq"])
+@pytest.mark.parametrize("kind", KINDS)
 @pytest.mark.parametrize("dtn,K,N,g", [("f16", 256, 128, 128), ("bf16", 256, 128, 128), ("f16", 512, 192, 128),
                                        ("bf16", 1280, 64, 128), ("f16", 1024, 320, 256)])
 def test_repacked_dequantize_bit_exact(kind, dtn, K, N, g):
     dt = DT[dtn]
     say(f"pk4 dequantize {kind} {dtn} K={K} N={N} g={g}")
     trip, pack_dim = make(kind, K, N, g, seed=K + N + g)
-    layer = layer_of(trip, pack_dim, dt)
+    layer = layer_of(trip, pack_dim, dt, bits=bits_of_kind(kind))
     assert layer.prepacked
     want = oracle.transpose_convert(dense(kind, trip, dt), dt)
     got = layer.dequantize()
@@ -77,16 +86,18 @@ def test_repacked_dequantize_reference_generators():
     """The reference's own closed-form triplets (metal_ops.rs:3668-3716, 4001-4060)."""
     say("pk4 dequantize reference triplets")
     for kind, trip, pack_dim in [("awq", refgen.build_awq_triplet(256, 128, 128), ops.PACK_OUT),
-                                 ("gptq", refgen.build_gptq_triplet(4, 256, 128, 128), ops.PACK_IN)]:
+                                 ("gptq", refgen.build_gptq_triplet(4, 256, 128, 128), ops.PACK_IN),
+                                 ("awq8", refgen.build_w8a16_triplet(256, 128, 128), ops.PACK_OUT),
+                                 ("gptq8", refgen.build_gptq_triplet(8, 256, 128, 128), ops.PACK_IN)]:
         for dtn in ("f16", "bf16"):
             dt = DT[dtn]
-            layer = layer_of(trip, pack_dim, dt)
+            layer = layer_of(trip, pack_dim, dt, bits=bits_of_kind(kind))
             assert layer.prepacked
             want = oracle.transpose_convert(dense(kind, trip, dt), dt)
             np.testing.assert_array_equal(bits_of(layer.dequantize()), want)
 
 
-@pytest.mark.parametrize("kind", ["awq", "gptq"])
+@pytest.mark.parametrize("kind", KINDS)
 @pytest.mark.parametrize("dtn", ["f16", "bf16"])
 @pytest.mark.parametrize("K,N,g", [(256, 128, 128), (512, 192, 128), (1280, 64, 128), (2048, 256, 256), (1152, 128, 128)])
 def test_repacked_forward_all_m(kind, dtn, K, N, g):
@@ -96,7 +107,7 @@ def test_repacked_forward_all_m(kind, dtn, K, N, g):
     dt = DT[dtn]
     trip, pack_dim = make(kind, K, N, g, seed=7 * K + N)
     bias = (np.arange(N, dtype=np.float32) % 11 - 5) * np.float32(0.125)
-    layer = layer_of(trip, pack_dim, dt, bias)
+    layer = layer_of(trip, pack_dim, dt, bias, bits=bits_of_kind(kind))
     assert layer.prepacked
     w = dense(kind, trip, dt)
     rng = np.random.default_rng(K + N)
@@ -137,15 +148,17 @@ def test_repacked_forward_config1(m, K, N):
         np.testing.assert_array_equal(bits_of(layer.forward(xd)), first)
 
 
+@pytest.mark.parametrize("bits", [4, 8])
 @pytest.mark.parametrize("dtn", ["f16", "bf16"])
-def test_repacked_forward_biased_activations(dtn):
+def test_repacked_forward_biased_activations(dtn, bits):
     """m <= 16 feeds bias + q to the matrix cores and removes the bias with the row sums of x:
     activations with a large mean and with outliers are where that cancellation is hardest."""
     dt = DT[dtn]
     K, N = 4096, 256
-    trip, pack_dim = make("awq", K, N, 128, seed=4242)
-    layer = layer_of(trip, pack_dim, dt)
-    w = dense("awq", trip, dt)
+    kind = "awq8" if bits == 8 else "awq"
+    trip, pack_dim = make(kind, K, N, 128, seed=4242)
+    layer = layer_of(trip, pack_dim, dt, bits=bits)
+    w = dense(kind, trip, dt)
     rng = np.random.default_rng(77)
     cases = {"mean 3": 3.0 + 0.1 * rng.standard_normal((4, K)),
              "positive": np.abs(rng.standard_normal((4, K))) * 2.0,
@@ -157,20 +170,21 @@ def test_repacked_forward_biased_activations(dtn):
         assert_close(layer.forward(to_dev(x, TORCH_DT[dt])), ref, f"pk4 {dtn} {name}")
 
 
-def test_repacked_forward_config2_gptq():
-    """Benchmark config 2 (GPTQ 4-bit, K=5120, N=13824, g=128), bf16."""
+@pytest.mark.parametrize("bits", [4, 8])
+def test_repacked_forward_config2_gptq(bits):
+    """Benchmark config 2 (GPTQ 4- and 8-bit, K=5120, N=13824, g=128), bf16."""
     dt = oracle.BF16
     K, N = 5120, 13824
-    trip = synth.gptq_checkpoint(K, N, 128, 4, seed=0x0A0D11E7)
-    layer = layer_of(trip, ops.PACK_IN, dt)
+    trip = synth.gptq_checkpoint(K, N, 128, bits, seed=0x0A0D11E7)
+    layer = layer_of(trip, ops.PACK_IN, dt, bits=bits)
     assert layer.prepacked
-    w = dense("gptq", trip, dt)
+    w = dense("gptq8" if bits == 8 else "gptq", trip, dt)
     for m in (1, 8, 24):
         say(f"pk4 forward config2 m={m}")
         x = np.random.default_rng(40 + m).standard_normal((m, K)).astype(np.float32)
         wr = w if m <= 16 else oracle.round_through(w, dt)
         ref = oracle.matmul_nt_f32(round_x(x, dt), wr)
-        assert_close(layer.forward(to_dev(x, torch.bfloat16)), ref, f"pk4 config2 m{m}", bf16_out=True)
+        assert_close(layer.forward(to_dev(x, torch.bfloat16)), ref, f"pk{bits} config2 m{m}", bf16_out=True)
 
 
 def test_ineligible_layers_keep_checkpoint_layout():
