@@ -51,9 +51,20 @@ def run(ops, ctx, stream, steps, warmup, time_graph):
             def step(i, x=x, y=y, d=d, bits=bits, nc=nc):
                 c = d[i % nc]
                 ops.gptq_matmul(x, c[0], c[1], c[2], bits, out=y, ctx=ctx)
-            out.append(_case(f"gptq{bits} M={m} K={K} N={N}", step, steps, warmup, stream, time_graph,
-                             wbytes + m * K * 2 + m * N * 2, 2.0 * m * K * N, ctx))
-        del d
+            out.append(_case(f"gptq{bits} M={m} K={K} N={N} (gptq_matmul op, checkpoint layout)", step, steps,
+                             warmup, stream, time_graph, wbytes + m * K * 2 + m * N * 2, 2.0 * m * K * N, ctx))
+        # the same weights as resident layers (PackedQuantLinear.forward, repacked at load)
+        layers = [ops.PackedQuantLinear(bits, ops.PACK_IN, c[0], c[1], c[2], None, torch.float16, ctx=ctx)
+                  for c in d]
+        for m in (1, 8, 64):
+            x = torch.randn((m, K), device=dev, dtype=torch.float16)
+            y = torch.empty((m, N), device=dev, dtype=torch.float16)
+
+            def lstep(i, x=x, y=y, layers=layers, nc=nc):
+                layers[i % nc].forward(x, out=y)
+            out.append(_case(f"gptq{bits} M={m} K={K} N={N} (PackedQuantLinear)", lstep, steps, warmup, stream,
+                             time_graph, wbytes + m * K * 2 + m * N * 2, 2.0 * m * K * N, ctx))
+        del d, layers
 
     # ---- config 3: GGUF --------------------------------------------------------
     K = N = 4096

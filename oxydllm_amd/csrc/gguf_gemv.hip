@@ -16,6 +16,8 @@
 #include "oxq_device.hpp"
 #include "oxq_internal.hpp"
 
+#include <cstdlib>
+
 namespace oxq {
 
 __device__ __forceinline__ uint32_t ld16(const uint8_t *p) { return *(const uint16_t *)p; }
@@ -169,6 +171,215 @@ __global__ __launch_bounds__(256) void gguf_gemv_kernel(const void *__restrict__
     }
 }
 
+// ---------------------------------------------------------------------------
+// GEMV with rows and activations staged in LDS.
+//
+// With one wave per row reading global memory directly, every wave re-reads the
+// activations from L2 and fetches its blocks with two-byte loads, and the decode
+// spends about five vector instructions per weight (extract, convert, subtract the
+// offset, scale, multiply-add).  Here a workgroup copies its `rpwg` consecutive rows -
+// one contiguous byte range - and the activations into LDS with 16-byte loads, and the
+// per-unit arithmetic is factored the way the reference's kernels factor it
+// (quant_kernels.metal:1097-1221, 1681-1838): the raw integers are converted once,
+//     y_unit = scale * (sum q_i x_i) - offset * (sum x_i),
+// and the sums of x over 16 elements are computed once per workgroup, not per row.
+// ---------------------------------------------------------------------------
+struct __attribute__((packed, aligned(2))) U32A2 { uint32_t v; };
+__device__ __forceinline__ uint32_t ld32a2(const uint8_t *p) { return ((const U32A2 *)p)->v; }
+
+__device__ __forceinline__ void bytes_to_f32(uint32_t w, float *o) {
+    o[0] = (float)(w & 0xFFu);
+    o[1] = (float)((w >> 8) & 0xFFu);
+    o[2] = (float)((w >> 16) & 0xFFu);
+    o[3] = (float)(w >> 24);
+}
+
+// Unit `u` of a row: q[0..31] = the stored unsigned integers as floats, and the four
+// numbers that turn (dot over elements 0..15, dot over 16..31, sum x over 0..15, sum x
+// over 16..31) into the unit's contribution: a0*dot0 + a1*dot1 - b0*sx0 - b1*sx1.
+template <int FMT>
+__device__ __forceinline__ void unit_ints(const uint8_t *__restrict__ row, int u, float q[32], float &a0,
+                                          float &a1, float &b0, float &b1) {
+    if constexpr (FMT == OXQ_GGUF_Q4_0) {
+        const uint8_t *p = row + (size_t)u * 18;
+        const float d = ld_f16(p);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t w = ld32a2(p + 2 + 4 * i);
+            bytes_to_f32(w & 0x0F0F0F0Fu, q + 4 * i);
+            bytes_to_f32((w >> 4) & 0x0F0F0F0Fu, q + 16 + 4 * i);
+        }
+        a0 = a1 = d;
+        b0 = b1 = 8.0f * d;
+    } else if constexpr (FMT == OXQ_GGUF_Q8_0) {
+        const uint8_t *p = row + (size_t)u * 34;
+        const float d = ld_f16(p);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) bytes_to_f32(ld32a2(p + 2 + 4 * i) ^ 0x80808080u, q + 4 * i);  // q + 128
+        a0 = a1 = d;
+        b0 = b1 = 128.0f * d;
+    } else if constexpr (FMT == OXQ_GGUF_Q4_K) {
+        const int b = u >> 3, sb = u & 7;
+        const uint8_t *p = row + (size_t)b * 144;
+        const float d = ld_f16(p), dmin = ld_f16(p + 2);
+        const uint8_t *sc = p + 4;
+        uint32_t scv, mnv;
+        if (sb < 4) {  // get_scale_min_k4
+            scv = sc[sb] & 63u;
+            mnv = sc[sb + 4] & 63u;
+        } else {
+            scv = (sc[sb + 4] & 0x0Fu) | ((uint32_t)(sc[sb - 4] >> 6) << 4);
+            mnv = ((uint32_t)sc[sb + 4] >> 4) | ((uint32_t)(sc[sb] >> 6) << 4);
+        }
+        const uint8_t *qs = p + 16 + (sb >> 1) * 32;
+        const int sh = (sb & 1) * 4;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) bytes_to_f32((ld32a2(qs + 4 * i) >> sh) & 0x0F0F0F0Fu, q + 4 * i);
+        a0 = a1 = d * (float)scv;
+        b0 = b1 = dmin * (float)mnv;
+    } else {  // Q6_K
+        const int b = u >> 3, sub = u & 7;
+        const int h = sub >> 2, quad = sub & 3;
+        const uint8_t *p = row + (size_t)b * 210;
+        const uint8_t *ql = p + 64 * h + (quad & 1) * 32;
+        const uint8_t *qh = p + 128 + 32 * h;
+        const int8_t *scales = (const int8_t *)(p + 192);
+        const float d = ld_f16(p + 208);
+        const int shl = (quad < 2) ? 0 : 4;
+        const int shh = 2 * quad;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint32_t lo = (ld32a2(ql + 4 * i) >> shl) & 0x0F0F0F0Fu;
+            const uint32_t hi = ((ld32a2(qh + 4 * i) >> shh) & 0x03030303u) << 4;
+            bytes_to_f32(lo | hi, q + 4 * i);  // q + 32
+        }
+        a0 = d * (float)scales[8 * h + 2 * quad];
+        a1 = d * (float)scales[8 * h + 2 * quad + 1];
+        b0 = 32.0f * a0;
+        b1 = 32.0f * a1;
+    }
+}
+
+// Activations sit in LDS as 16-byte chunks, chunk c of unit u at ((c * (units + 1)) + u) * 16:
+// consecutive lanes (units) then read consecutive chunks - with the row-major layout a
+// lane stride of 128 bytes puts a wave's reads on 8 of the 64 banks.
+// 8 consecutive activations (index 8*o .. 8*o+7 of unit u) as f32:
+template <bool BF16X>
+__device__ __forceinline__ void ld_x8(const unsigned char *xrow, int upitch, int u, int o, float out[8]) {
+    if constexpr (BF16X) {
+        const u32x4_t v = *(const u32x4_t *)(xrow + ((size_t)o * upitch + u) * 16);
+        const uint32_t v0 = v[0], v1 = v[1], v2 = v[2], v3 = v[3];
+        const uint32_t vv[4] = {v0, v1, v2, v3};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            out[2 * j] = __builtin_bit_cast(float, vv[j] << 16);
+            out[2 * j + 1] = __builtin_bit_cast(float, vv[j] & 0xFFFF0000u);
+        }
+    } else {
+        const float4_t a = *(const float4_t *)(xrow + ((size_t)(2 * o) * upitch + u) * 16);
+        const float4_t b = *(const float4_t *)(xrow + ((size_t)(2 * o + 1) * upitch + u) * 16);
+        out[0] = a[0], out[1] = a[1], out[2] = a[2], out[3] = a[3];
+        out[4] = b[0], out[5] = b[1], out[6] = b[2], out[7] = b[3];
+    }
+}
+
+template <int FMT, bool BF16X, int MB>
+__global__ __launch_bounds__(256) void gguf_gemv_lds_kernel(const void *__restrict__ x,
+                                                            const uint8_t *__restrict__ w,
+                                                            const void *__restrict__ bias,
+                                                            void *__restrict__ y, int M, int K, int N,
+                                                            int rpwg, size_t total_bytes) {
+    constexpr int XB = BF16X ? 2 : 4;
+    extern __shared__ __attribute__((aligned(16))) unsigned char gg_lds[];
+    constexpr int CPU = 32 * XB / 16;                                 // 16-byte chunks per unit
+    const int upitch = (K >> 5) + 1;                                  // chunk pitch (units + 1)
+    const size_t xrow_bytes = (size_t)CPU * upitch * 16;
+    unsigned char *lds_x = gg_lds;                                   // [MB] chunked activations
+    float *lds_sx = (float *)(gg_lds + (size_t)MB * xrow_bytes);      // [MB][K/16] sums of 16
+    unsigned char *lds_w = (unsigned char *)(lds_sx + (size_t)MB * (K >> 4));
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int n0 = blockIdx.x * rpwg;
+    const int nrows = min(rpwg, N - n0);
+    const int units = K >> 5;
+    const size_t row_bytes = (size_t)(K / GgufFmt<FMT>::BE) * GgufFmt<FMT>::BB;
+    const size_t start = (size_t)n0 * row_bytes, a0 = start & ~(size_t)15;
+    const int head = (int)(start - a0);
+    const int wchunks = (int)((head + (size_t)nrows * row_bytes + 15) >> 4);
+    const int xchunks = (M * K * XB) >> 4;
+    const int cpr = K * XB / 16;  // chunks per activation row
+    for (int c = threadIdx.x; c < xchunks; c += 256) {
+        const int m = c / cpr, g = c - m * cpr;
+        const int u = g / CPU, cc = g - u * CPU;
+        *(u32x4_t *)(lds_x + m * xrow_bytes + ((size_t)cc * upitch + u) * 16) = ((const u32x4_t *)x)[c];
+    }
+    for (int c = threadIdx.x; c < wchunks; c += 256) {
+        const size_t off = a0 + (size_t)c * 16;
+        if (off + 16 <= total_bytes) {
+            ((u32x4_t *)lds_w)[c] = *(const u32x4_t *)(w + off);
+        } else {  // the tensor's last, partial chunk
+            for (int b = 0; b < 16; ++b) lds_w[c * 16 + b] = off + b < total_bytes ? w[off + b] : (uint8_t)0;
+        }
+    }
+    __syncthreads();
+    for (int c = threadIdx.x; c < M * (K >> 4); c += 256) {  // sums of x over 16 elements
+        const int m = c / (K >> 4), h = c - m * (K >> 4);
+        float xa[8], xb[8];
+        ld_x8<BF16X>(lds_x + m * xrow_bytes, upitch, h >> 1, 2 * (h & 1), xa);
+        ld_x8<BF16X>(lds_x + m * xrow_bytes, upitch, h >> 1, 2 * (h & 1) + 1, xb);
+        float sum = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) sum += xa[i];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) sum += xb[i];
+        lds_sx[c] = sum;
+    }
+    __syncthreads();
+    for (int r = wave; r < nrows; r += 4) {
+        const uint8_t *row = lds_w + head + (size_t)r * row_bytes;
+        const int n = n0 + r;
+        float acc[MB];
+#pragma unroll
+        for (int m = 0; m < MB; ++m) acc[m] = 0.0f;
+        for (int u = lane; u < units; u += 64) {
+            float q[32], c0, c1, d0, d1;
+            unit_ints<FMT>(row, u, q, c0, c1, d0, d1);
+#pragma unroll
+            for (int m = 0; m < MB; ++m) {
+                if (m < M) {
+                    float dot0 = 0.0f, dot1 = 0.0f;
+#pragma unroll
+                    for (int o = 0; o < 4; ++o) {
+                        float xv[8];
+                        ld_x8<BF16X>(lds_x + m * xrow_bytes, upitch, u, o, xv);
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) {
+                            if (o < 2) dot0 = fmaf(q[8 * o + i], xv[i], dot0);
+                            else dot1 = fmaf(q[8 * o + i], xv[i], dot1);
+                        }
+                    }
+                    const float *sx = lds_sx + (size_t)m * (K >> 4) + 2 * u;
+                    acc[m] += (c0 * dot0 + c1 * dot1) - (d0 * sx[0] + d1 * sx[1]);
+                }
+            }
+        }
+#pragma unroll
+        for (int m = 0; m < MB; ++m) {
+            if (m < M) {
+                float tot = wave_sum_xor<64>(acc[m]);
+                if (lane == 0) {
+                    if constexpr (BF16X) {
+                        if (bias) tot += BF16Traits::to_f32(((const uint16_t *)bias)[n]);
+                        ((uint16_t *)y)[(size_t)m * N + n] = BF16Traits::from_f32(tot);
+                    } else {
+                        if (bias) tot += ((const float *)bias)[n];
+                        ((float *)y)[(size_t)m * N + n] = tot;
+                    }
+                }
+            }
+        }
+    }
+}
+
 template <int FMT>
 __global__ __launch_bounds__(256) void gguf_dequant_kernel(const uint8_t *__restrict__ w,
                                                            float *__restrict__ out, int K, int N) {
@@ -182,6 +393,15 @@ __global__ __launch_bounds__(256) void gguf_dequant_kernel(const uint8_t *__rest
     float *o = out + (size_t)n * K + (size_t)u * 32;
 #pragma unroll
     for (int i = 0; i < 32; ++i) o[i] = wf[i];
+}
+
+static const char *fmt_name(int q) {
+    switch (q) {
+    case OXQ_GGUF_Q4_0: return "q4_0";
+    case OXQ_GGUF_Q8_0: return "q8_0";
+    case OXQ_GGUF_Q4_K: return "q4k";
+    default: return "q6k";
+    }
 }
 
 template <int FMT, bool BF16X>
@@ -199,32 +419,76 @@ static void launch_rows(hipStream_t s, dim3 grid, const GgufProblem &p, const ui
         hipLaunchKernelGGL((gguf_gemv_kernel<FMT, BF16X, 8>), grid, block, 0, s, x, p.w, p.bias, y, rows, K, N);
 }
 
-static const char *fmt_name(int q) {
-    switch (q) {
-    case OXQ_GGUF_Q4_0: return "q4_0";
-    case OXQ_GGUF_Q8_0: return "q8_0";
-    case OXQ_GGUF_Q4_K: return "q4k";
-    default: return "q6k";
+template <int FMT, bool BF16X, int MB>
+static int launch_rows_lds_mb(hipStream_t s, const GgufProblem &p, const uint8_t *x, uint8_t *y, int rows,
+                              int rpwg, size_t lds) {
+    static size_t attr_lds = 0;
+    if (lds > attr_lds) {
+        OXQ_HIP_CHECK(hipFuncSetAttribute((const void *)gguf_gemv_lds_kernel<FMT, BF16X, MB>,
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        attr_lds = lds;
+    }
+    const int K = (int)p.K, N = (int)p.N;
+    const size_t total = (size_t)N * (size_t)(K / GgufFmt<FMT>::BE) * GgufFmt<FMT>::BB;
+    dim3 grid((unsigned)ceil_div(N, rpwg)), block(256);
+    hipLaunchKernelGGL((gguf_gemv_lds_kernel<FMT, BF16X, MB>), grid, block, lds, s, x, p.w, p.bias, y, rows, K,
+                       N, rpwg, total);
+    return OXQ_OK;
+}
+
+template <int FMT, bool BF16X>
+static int launch_rows_lds(hipStream_t s, const GgufProblem &p, const uint8_t *x, uint8_t *y, int rows,
+                           int rpwg, size_t lds) {
+    if (rows <= 1) return launch_rows_lds_mb<FMT, BF16X, 1>(s, p, x, y, rows, rpwg, lds);
+    if (rows <= 2) return launch_rows_lds_mb<FMT, BF16X, 2>(s, p, x, y, rows, rpwg, lds);
+    if (rows <= 4) return launch_rows_lds_mb<FMT, BF16X, 4>(s, p, x, y, rows, rpwg, lds);
+    return launch_rows_lds_mb<FMT, BF16X, 8>(s, p, x, y, rows, rpwg, lds);
+}
+
+static size_t gguf_row_bytes(int quant, int64_t K) {
+    switch (quant) {
+    case OXQ_GGUF_Q4_0: return (size_t)(K / 32) * 18;
+    case OXQ_GGUF_Q8_0: return (size_t)(K / 32) * 34;
+    case OXQ_GGUF_Q4_K: return (size_t)(K / 256) * 144;
+    default: return (size_t)(K / 256) * 210;
     }
 }
 
 int launch_gguf_gemv(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p) {
-    dim3 grid((unsigned)ceil_div(p.N, 4)), block(256);
     const bool bf = p.act_dtype == OXQ_BF16;
+    const size_t xb = bf ? 2 : 4;
     const uint32_t chunks = (uint32_t)ceil_div(p.M, 8);
+    // LDS variant: activations of one chunk of rows plus `rpwg` weight rows must fit 64 KB
+    const int64_t mrows = p.M < 8 ? p.M : 8;
+    const int mb = mrows <= 1 ? 1 : mrows <= 2 ? 2 : mrows <= 4 ? 4 : 8;
+    const size_t x_lds = (size_t)mb * (32 * xb / 16) * (size_t)((p.K >> 5) + 1) * 16 +
+                         (size_t)mb * (size_t)(p.K >> 4) * 4;
+    const size_t row_bytes = gguf_row_bytes(p.quant, p.K);
+    const char *rp_env = getenv("OXQ_GGUF_RPWG");
+    int rpwg = rp_env ? atoi(rp_env) : 4;
+    if (rpwg < 1) rpwg = 1;
+    while (rpwg > 1 && x_lds + (size_t)rpwg * row_bytes + 32 > 64 * 1024) rpwg >>= 1;
+    const size_t lds = x_lds + (size_t)rpwg * row_bytes + 32;
+    const char *force = getenv("OXQ_FORCE_GENERIC");
+    const bool use_lds = lds <= 64 * 1024 && ((uintptr_t)p.x & 15) == 0 && ((uintptr_t)p.w & 15) == 0 &&
+                         (p.K * xb) % 16 == 0 && !(force && atoi(force));
     char name[64];
-    snprintf(name, sizeof name, "gguf_%s_gemv_%s", fmt_name(p.quant), bf ? "bf16" : "f32");
+    snprintf(name, sizeof name, "gguf_%s_gemv_%s%s", fmt_name(p.quant), bf ? "bf16" : "f32", use_lds ? "_lds" : "");
+    dim3 grid((unsigned)(use_lds ? ceil_div(p.N, rpwg) : ceil_div(p.N, 4))), block(256);
     set_plan(ctx, name, grid, block, 1, chunks, 0);
     if (ctx->plan_only) return OXQ_OK;
-    const size_t xb = bf ? 2 : 4;
     // m > 8: activation rows are processed 8 at a time (the weight is re-read
     // per chunk; a tiled kernel for large m is future work).
     for (int64_t m0 = 0; m0 < p.M; m0 += 8) {
         const int rows = (int)((p.M - m0) < 8 ? (p.M - m0) : 8);
         const uint8_t *x = (const uint8_t *)p.x + (size_t)m0 * p.K * xb;
         uint8_t *y = (uint8_t *)p.y + (size_t)m0 * p.N * xb;
-#define OXQ_FMT(F)                                              \
-    if (bf) launch_rows<F, true>(s, grid, p, x, y, rows);       \
+#define OXQ_FMT(F)                                                                  \
+    if (use_lds) {                                                                  \
+        int rc = bf ? launch_rows_lds<F, true>(s, p, x, y, rows, rpwg, lds)         \
+                    : launch_rows_lds<F, false>(s, p, x, y, rows, rpwg, lds);       \
+        if (rc != OXQ_OK) return rc;                                                \
+    } else if (bf) launch_rows<F, true>(s, grid, p, x, y, rows);                    \
     else launch_rows<F, false>(s, grid, p, x, y, rows)
         switch (p.quant) {
         case OXQ_GGUF_Q4_0: OXQ_FMT(OXQ_GGUF_Q4_0); break;

@@ -12,6 +12,8 @@
 #include "oxq_device.hpp"
 #include "oxq_internal.hpp"
 
+#include <cstdlib>
+
 namespace oxq {
 
 // E2M1 code -> f32: sign | exponent e (2 bits) | mantissa m (1 bit);
@@ -119,6 +121,105 @@ __global__ __launch_bounds__(256) void mxfp4_gemv_kernel(
     }
 }
 
+// Activations in LDS, several rows per wave.  With one wave per output row every wave
+// re-reads its tokens' activations (K * 2 bytes each) from L2, four times the bytes of
+// the weight row itself, and that traffic - not HBM - sets the pace.  Here a workgroup
+// stages the expert's tokens once (up to MB at a time) and its 4 waves then stream RW rows
+// each, all of a row's loads in flight before the first dot product.
+// grid.x = blocks of 4*RW rows, grid.y = expert (1 for the plain form).
+template <int MB, int RW>
+__global__ __launch_bounds__(256) void mxfp4_gemv_lds_kernel(
+    const uint16_t *__restrict__ x, const uint8_t *__restrict__ blocks,
+    const uint8_t *__restrict__ scales, const uint16_t *__restrict__ bias,
+    uint16_t *__restrict__ y, const int32_t *__restrict__ offsets,
+    const int32_t *__restrict__ token_ids, int M, int K, int N) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char mx_lds[];  // [MB][K] bf16
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int e = blockIdx.y;
+    int p0 = 0, p1 = M;
+    if (offsets) {
+        p0 = offsets[e];
+        p1 = offsets[e + 1];
+        if (p1 <= p0) return;  // block-uniform
+    }
+    const int nb = K >> 5;
+    const int n0 = (blockIdx.x * 4 + wave) * RW;
+    const int cpr = K >> 3;  // 16-byte chunks per activation row
+    constexpr int PASSES = 2;  // blocks per lane and row held in registers (K <= 4096)
+
+    for (int pbase = p0; pbase < p1; pbase += MB) {
+        const int rows = min(MB, p1 - pbase);
+        if (pbase > p0) __syncthreads();  // everyone is done with the previous tokens
+        for (int c = threadIdx.x; c < rows * cpr; c += 256) {
+            const int m = c / cpr, cc = c - m * cpr;
+            const int p = pbase + m;
+            const int src = token_ids ? token_ids[p] : p;
+            *(u32x4_t *)(mx_lds + ((size_t)m * K + (size_t)cc * 8) * 2) =
+                *(const u32x4_t *)(x + (size_t)src * K + (size_t)cc * 8);
+        }
+        __syncthreads();
+
+#pragma unroll 1
+        for (int r0 = 0; r0 < RW; r0 += 2) {
+            // two rows at a time: 2 x PASSES weight blocks and scale bytes in flight per lane
+            u32x4_t q[2][PASSES];
+            uint32_t sb[2][PASSES];
+#pragma unroll
+            for (int r = 0; r < 2; ++r) {
+                const int n = n0 + r0 + r;
+                const size_t row = (size_t)e * N + (n < N ? n : N - 1);
+#pragma unroll
+                for (int ps = 0; ps < PASSES; ++ps) {
+                    const int b = lane + 64 * ps;
+                    const int bc = b < nb ? b : nb - 1;
+                    q[r][ps] = ((const u32x4_t *)blocks)[row * nb + bc];
+                    sb[r][ps] = scales[row * nb + bc];
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < 2; ++r) {
+                const int n = n0 + r0 + r;
+                float acc[MB];
+#pragma unroll
+                for (int m = 0; m < MB; ++m) acc[m] = 0.0f;
+#pragma unroll
+                for (int ps = 0; ps < PASSES; ++ps) {
+                    const int b = lane + 64 * ps;
+                    if (b < nb) {
+                        const float scale = e8m0_to_f32(sb[r][ps]);
+#pragma unroll
+                        for (int m = 0; m < MB; ++m)
+                            if (m < rows)
+                                acc[m] = fmaf(scale,
+                                              block_dot_bf16(q[r][ps], (const uint16_t *)(mx_lds + ((size_t)m * K + (size_t)b * 32) * 2)),
+                                              acc[m]);
+                    }
+                }
+                // blocks past 2 x 64 (K > 4096): stream the rest
+                for (int b = lane + 64 * PASSES; b < nb; b += 64) {
+                    const size_t row = (size_t)e * N + (n < N ? n : N - 1);
+                    const u32x4_t qq = ((const u32x4_t *)blocks)[row * nb + b];
+                    const float scale = e8m0_to_f32(scales[row * nb + b]);
+#pragma unroll
+                    for (int m = 0; m < MB; ++m)
+                        if (m < rows)
+                            acc[m] = fmaf(scale, block_dot_bf16(qq, (const uint16_t *)(mx_lds + ((size_t)m * K + (size_t)b * 32) * 2)), acc[m]);
+                }
+                if (n < N) {  // wave-uniform
+                    const float bv = bias ? BF16Traits::to_f32(bias[(size_t)e * N + n]) : 0.0f;
+#pragma unroll
+                    for (int m = 0; m < MB; ++m) {
+                        if (m < rows) {
+                            const float tot = wave_sum_xor<64>(acc[m]);
+                            if (lane == 0) y[(size_t)(pbase + m) * N + n] = BF16Traits::from_f32(tot + bv);
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+
 __global__ __launch_bounds__(256) void mxfp4_dequant_kernel(const uint8_t *__restrict__ blocks,
                                                             const uint8_t *__restrict__ scales,
                                                             float *__restrict__ out, size_t nblocks) {
@@ -131,22 +232,58 @@ __global__ __launch_bounds__(256) void mxfp4_dequant_kernel(const uint8_t *__res
     for (int i = 0; i < 32; ++i) o[i] = w[i];
 }
 
+template <int MB, int RW>
+static int mxfp4_lds_go(hipStream_t s, dim3 grid, const Mxfp4Problem &p, size_t lds) {
+    static size_t attr_lds = 0;
+    if (lds > attr_lds) {
+        OXQ_HIP_CHECK(hipFuncSetAttribute((const void *)mxfp4_gemv_lds_kernel<MB, RW>,
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        attr_lds = lds;
+    }
+    hipLaunchKernelGGL((mxfp4_gemv_lds_kernel<MB, RW>), grid, dim3(256), lds, s, (const uint16_t *)p.x, p.blocks,
+                       p.scales, (const uint16_t *)p.bias, (uint16_t *)p.y, p.expert_offsets, p.token_ids,
+                       (int)p.M, (int)p.K, (int)p.N);
+    OXQ_HIP_CHECK(hipGetLastError());
+    return OXQ_OK;
+}
+
 int launch_mxfp4_gemv(oxq_ctx *ctx, hipStream_t s, const Mxfp4Problem &p) {
     const bool grouped = p.n_experts > 0;
+    const int64_t rows_hint = grouped ? 4 : p.M;  // tokens per expert are few in decode
+    const int mb = rows_hint <= 1 ? 1 : rows_hint <= 2 ? 2 : rows_hint <= 4 ? 4 : 8;
+    constexpr int RW = 8;
+    const size_t lds = (size_t)mb * (size_t)p.K * 2;
+    const char *force = getenv("OXQ_FORCE_GENERIC");
+    const bool use_lds = lds <= 96 * 1024 && !(force && atoi(force));
+    if (use_lds) {
+        dim3 grid((unsigned)ceil_div(p.N, 4 * RW), grouped ? (unsigned)p.n_experts : 1u), block(256);
+        char name[64];
+        snprintf(name, sizeof name, "%s_lds_m%d", grouped ? "mxfp4_moe_gemv_bf16" : "mxfp4_gemv_bf16", mb);
+        set_plan(ctx, name, grid, block, 1, 1, 0);
+        if (ctx->plan_only) return OXQ_OK;
+        if (((uintptr_t)p.blocks & 15) || ((uintptr_t)p.x & 15) || (p.K % 8))
+            return fail(OXQ_ERR_UNSUPPORTED, "mxfp4 gemv: blocks and x must be 16-byte aligned");
+        switch (mb) {
+        case 1: return mxfp4_lds_go<1, RW>(s, grid, p, lds);
+        case 2: return mxfp4_lds_go<2, RW>(s, grid, p, lds);
+        case 4: return mxfp4_lds_go<4, RW>(s, grid, p, lds);
+        default: return mxfp4_lds_go<8, RW>(s, grid, p, lds);
+        }
+    }
     dim3 grid((unsigned)ceil_div(p.N, 4), grouped ? (unsigned)p.n_experts : 1u), block(256);
     set_plan(ctx, grouped ? "mxfp4_moe_gemv_bf16" : "mxfp4_gemv_bf16", grid, block, 1, 1, 0);
     if (ctx->plan_only) return OXQ_OK;
     if (((uintptr_t)p.blocks & 15) || ((uintptr_t)p.x & 15) || (p.K % 8))
         return fail(OXQ_ERR_UNSUPPORTED, "mxfp4 gemv: blocks and x must be 16-byte aligned");
     const int M = (int)p.M, K = (int)p.K, N = (int)p.N;
-    const int64_t rows_hint = grouped ? 8 : p.M;
+    const int64_t rows_hint2 = grouped ? 8 : p.M;
 #define OXQ_GO(MBv)                                                                                   \
     hipLaunchKernelGGL((mxfp4_gemv_kernel<MBv>), grid, block, 0, s, (const uint16_t *)p.x, p.blocks,  \
                        p.scales, (const uint16_t *)p.bias, (uint16_t *)p.y, p.expert_offsets,        \
                        p.token_ids, M, K, N)
-    if (rows_hint <= 1) OXQ_GO(1);
-    else if (rows_hint <= 2) OXQ_GO(2);
-    else if (rows_hint <= 4) OXQ_GO(4);
+    if (rows_hint2 <= 1) OXQ_GO(1);
+    else if (rows_hint2 <= 2) OXQ_GO(2);
+    else if (rows_hint2 <= 4) OXQ_GO(4);
     else OXQ_GO(8);
 #undef OXQ_GO
     OXQ_HIP_CHECK(hipGetLastError());

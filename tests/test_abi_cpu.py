@@ -304,7 +304,7 @@ def test_layers_validate_like_reference(lib, ctx):
         assert lib.oxq_qlinear_forward(q, None, C.byref(fake((m_rows, 4096), BF16)),
                                        C.byref(fake((m_rows, 4096), BF16))) == 0, err(lib)
         p = plan(lib, ctx)
-        assert p.kernel.decode() == kern and p.launches == (m_rows + 7) // 8
+        assert p.kernel.decode().startswith(kern) and p.launches == (m_rows + 7) // 8
     lib.oxq_qlinear_free(q)
     assert lib.oxq_qlinear_new(ctx, _lib.GGUF_Q4_K, C.byref(w), 4096, 4095, None, BF16, C.byref(q)) == -3
 
