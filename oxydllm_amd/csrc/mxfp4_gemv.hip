@@ -68,6 +68,22 @@ __device__ __forceinline__ float block_dot_bf16(const u32x4_t q, const uint16_t 
     return acc;
 }
 
+// Same, with the block's activations stored as four 16-byte chunks `pitch` chunks apart
+// (LDS layout of the staged kernel: consecutive lanes read consecutive chunks, no bank conflicts).
+__device__ __forceinline__ float block_dot_bf16_chunked(const u32x4_t q, const unsigned char *xb, int pitch) {
+    float acc = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const u32x4_t xv = *(const u32x4_t *)(xb + (size_t)i * pitch * 16);
+        const uint32_t w = q[i], x0 = xv[0], x1 = xv[1], x2 = xv[2], x3 = xv[3];
+        acc = dot2_fp4(acc, x0, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, 1.0f, 0));
+        acc = dot2_fp4(acc, x1, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, 1.0f, 1));
+        acc = dot2_fp4(acc, x2, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, 1.0f, 2));
+        acc = dot2_fp4(acc, x3, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, 1.0f, 3));
+    }
+    return acc;
+}
+
 // grid.x = row quads, grid.y = expert (1 for the plain form).
 // offsets == nullptr: plain form, rows 0..M-1 of x / y.
 template <int MB>
@@ -133,7 +149,8 @@ __global__ __launch_bounds__(256) void mxfp4_gemv_lds_kernel(
     const uint8_t *__restrict__ scales, const uint16_t *__restrict__ bias,
     uint16_t *__restrict__ y, const int32_t *__restrict__ offsets,
     const int32_t *__restrict__ token_ids, int M, int K, int N) {
-    extern __shared__ __attribute__((aligned(16))) unsigned char mx_lds[];  // [MB][K] bf16
+    // [MB] token rows; chunk c (0..3) of block b at ((c * (nb + 1)) + b) * 16 bytes
+    extern __shared__ __attribute__((aligned(16))) unsigned char mx_lds[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int e = blockIdx.y;
     int p0 = 0, p1 = M;
@@ -145,6 +162,8 @@ __global__ __launch_bounds__(256) void mxfp4_gemv_lds_kernel(
     const int nb = K >> 5;
     const int n0 = (blockIdx.x * 4 + wave) * RW;
     const int cpr = K >> 3;  // 16-byte chunks per activation row
+    const int pitch = nb + 1;
+    const size_t xrow_bytes = (size_t)4 * pitch * 16;
     constexpr int PASSES = 2;  // blocks per lane and row held in registers (K <= 4096)
 
     for (int pbase = p0; pbase < p1; pbase += MB) {
@@ -154,7 +173,7 @@ __global__ __launch_bounds__(256) void mxfp4_gemv_lds_kernel(
             const int m = c / cpr, cc = c - m * cpr;
             const int p = pbase + m;
             const int src = token_ids ? token_ids[p] : p;
-            *(u32x4_t *)(mx_lds + ((size_t)m * K + (size_t)cc * 8) * 2) =
+            *(u32x4_t *)(mx_lds + m * xrow_bytes + ((size_t)(cc & 3) * pitch + (cc >> 2)) * 16) =
                 *(const u32x4_t *)(x + (size_t)src * K + (size_t)cc * 8);
         }
         __syncthreads();
@@ -191,7 +210,7 @@ __global__ __launch_bounds__(256) void mxfp4_gemv_lds_kernel(
                         for (int m = 0; m < MB; ++m)
                             if (m < rows)
                                 acc[m] = fmaf(scale,
-                                              block_dot_bf16(q[r][ps], (const uint16_t *)(mx_lds + ((size_t)m * K + (size_t)b * 32) * 2)),
+                                              block_dot_bf16_chunked(q[r][ps], mx_lds + m * xrow_bytes + (size_t)b * 16, pitch),
                                               acc[m]);
                     }
                 }
@@ -203,7 +222,7 @@ __global__ __launch_bounds__(256) void mxfp4_gemv_lds_kernel(
 #pragma unroll
                     for (int m = 0; m < MB; ++m)
                         if (m < rows)
-                            acc[m] = fmaf(scale, block_dot_bf16(qq, (const uint16_t *)(mx_lds + ((size_t)m * K + (size_t)b * 32) * 2)), acc[m]);
+                            acc[m] = fmaf(scale, block_dot_bf16_chunked(qq, mx_lds + m * xrow_bytes + (size_t)b * 16, pitch), acc[m]);
                 }
                 if (n < N) {  // wave-uniform
                     const float bv = bias ? BF16Traits::to_f32(bias[(size_t)e * N + n]) : 0.0f;
@@ -252,7 +271,7 @@ int launch_mxfp4_gemv(oxq_ctx *ctx, hipStream_t s, const Mxfp4Problem &p) {
     const int64_t rows_hint = grouped ? 4 : p.M;  // tokens per expert are few in decode
     const int mb = rows_hint <= 1 ? 1 : rows_hint <= 2 ? 2 : rows_hint <= 4 ? 4 : 8;
     constexpr int RW = 8;
-    const size_t lds = (size_t)mb * (size_t)p.K * 2;
+    const size_t lds = (size_t)mb * 4 * (size_t)((p.K >> 5) + 1) * 16;
     const char *force = getenv("OXQ_FORCE_GENERIC");
     const bool use_lds = lds <= 96 * 1024 && !(force && atoi(force));
     if (use_lds) {
