@@ -237,7 +237,10 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
     constexpr int OOB = 0x7FFFFF00;
     constexpr int WL = BITS / 4;               // 1 KB weight loads per step
     extern __shared__ __attribute__((aligned(16))) unsigned char pk4_lds[];
-    u32x4_t *zs_lds = (u32x4_t *)(pk4_lds + NW * SLOT);  // [G][16]: the strip's {-(bias+z), s} words
+    // the strip's zeros and scales, [G][16 column quads]: GS = false the four {-(bias+z), s} words,
+    // GS = true already converted for the group fold: float4 s, float4 -s * (bias + z)
+    u32x4_t *zs_lds = (u32x4_t *)(pk4_lds + NW * SLOT);
+    float4_t *zs_ldsf = (float4_t *)(pk4_lds + NW * SLOT);
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -323,21 +326,40 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
         for (int f = 0; f < 4; ++f) acc[mt][f] = float4_t{0.f, 0.f, 0.f, 0.f};
     uint32_t negzb[4], sp[4];          // GS = false: the two Pk4T constants per column
     float sf[4], nszb[4];              // GS = true: s and -s * (bias + z) in f32
-    float4_t tmp[GS ? MT : 1][4], tmps[GS ? MT : 1];
-    if (GS) {
+    // per-group accumulators of the GS form; with one block per group they live inside one
+    // loop iteration (tmpb below), otherwise across iterations
+    float4_t tmpg[GS ? MT : 1][4], tmpsg[GS ? MT : 1];
+    if (GS && !BPG1) {
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
-            tmps[mt] = float4_t{0.f, 0.f, 0.f, 0.f};
+            tmpsg[mt] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int f = 0; f < 4; ++f) tmp[mt][f] = float4_t{0.f, 0.f, 0.f, 0.f};
+            for (int f = 0; f < 4; ++f) tmpg[mt][f] = float4_t{0.f, 0.f, 0.f, 0.f};
         }
     }
     const uint32_t ones[4] = {TT::ONES, TT::ONES, TT::ONES, TT::ONES};
     const float4_t zero4 = float4_t{0.f, 0.f, 0.f, 0.f};
 
 #pragma unroll
-    for (int q = 0; q < ZCH; ++q)
-        if ((int)threadIdx.x + q * 512 < zchunks) zs_lds[threadIdx.x + q * 512] = zstage[q];
+    for (int q = 0; q < ZCH; ++q) {
+        const int c = (int)threadIdx.x + q * 512;
+        if (c < zchunks) {
+            if (GS) {
+                const uint32_t z0 = zstage[q][0], z1 = zstage[q][1], z2 = zstage[q][2], z3 = zstage[q][3];
+                const uint32_t zv[4] = {z0, z1, z2, z3};
+                float4_t s4, n4;
+#pragma unroll
+                for (int f = 0; f < 4; ++f) {
+                    s4[f] = TT::to_f32((uint16_t)(zv[f] >> 16));
+                    n4[f] = s4[f] * TT::to_f32((uint16_t)(zv[f] & 0xFFFFu));  // -s * (bias_f + z)
+                }
+                zs_ldsf[2 * c] = s4;
+                zs_ldsf[2 * c + 1] = n4;
+            } else {
+                zs_lds[c] = zstage[q];
+            }
+        }
+    }
     store_a(afirst);
     __syncthreads();
 
@@ -349,18 +371,21 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
             const int blk = blk_of(i);
             const bool gfirst = BPG1 || (blk & bpg_mask) == 0;
             const bool glast = BPG1 || (blk & bpg_mask) == bpg_mask;
+            float4_t tmpb[(GS && BPG1) ? MT : 1][4], tmpsb[(GS && BPG1) ? MT : 1];  // written at step 0
+            auto &tmp = *(BPG1 ? &tmpb : &tmpg);
+            auto &tmps = *(BPG1 ? &tmpsb : &tmpsg);
             if (live && gfirst) {  // first block of a group
-                const u32x4_t zq = zs_lds[(blk >> gs7) * 16 + ni];
-                const uint32_t z0 = zq[0], z1 = zq[1], z2 = zq[2], z3 = zq[3];
-                const uint32_t zv[4] = {z0, z1, z2, z3};
+                if (GS) {
+                    const float4_t s4 = zs_ldsf[((blk >> gs7) * 16 + ni) * 2];
+                    const float4_t n4 = zs_ldsf[((blk >> gs7) * 16 + ni) * 2 + 1];
+                    sf[0] = s4[0], sf[1] = s4[1], sf[2] = s4[2], sf[3] = s4[3];
+                    nszb[0] = n4[0], nszb[1] = n4[1], nszb[2] = n4[2], nszb[3] = n4[3];
+                } else {
+                    const u32x4_t zq = zs_lds[(blk >> gs7) * 16 + ni];
+                    const uint32_t z0 = zq[0], z1 = zq[1], z2 = zq[2], z3 = zq[3];
+                    const uint32_t zv[4] = {z0, z1, z2, z3};
 #pragma unroll
-                for (int f = 0; f < 4; ++f) {
-                    if (GS) {
-                        sf[f] = TT::to_f32((uint16_t)(zv[f] >> 16));
-                        nszb[f] = sf[f] * TT::to_f32((uint16_t)(zv[f] & 0xFFFFu));  // -s * (bias_f + z)
-                    } else {
-                        Pk4T<TT>::prep(zv[f], negzb[f], sp[f]);
-                    }
+                    for (int f = 0; f < 4; ++f) Pk4T<TT>::prep(zv[f], negzb[f], sp[f]);
                 }
             }
 #pragma unroll
@@ -566,7 +591,7 @@ template <typename TT, int BITS, int MT, bool GS, bool BPG1>
 static int pk4_go3(hipStream_t s, dim3 grid, const Pk4Problem &p, int bpw) {
     constexpr int AB = Pk4Ring<MT, BITS>::AB, WB = Pk4Ring<MT, BITS>::WB;
     const int G = (int)(p.w.K >> p.w.group_shift);
-    const size_t lds = (size_t)8 * MT * 4096 + (size_t)G * 256;
+    const size_t lds = (size_t)8 * MT * 4096 + (size_t)G * 256 * (GS ? 2 : 1);
     static size_t attr_lds = 0;  // one per instantiation
     if (lds > attr_lds) {
         OXQ_HIP_CHECK(hipFuncSetAttribute((const void *)pk4_mfma_kernel<TT, BITS, MT, GS, BPG1, AB, WB>,
