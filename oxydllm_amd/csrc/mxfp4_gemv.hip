@@ -239,6 +239,138 @@ __global__ __launch_bounds__(256) void mxfp4_gemv_lds_kernel(
     }
 }
 
+// ---------------------------------------------------------------------------
+// Expert GEMV on the matrix cores: the tokens are the M tile (<= 16 rows of
+// v_mfma_f32_16x16x32_bf16), 16 weight rows are one N tile.
+//
+// An MXFP4 block is 32 consecutive k of one row = exactly one MFMA K step for that row, and
+// v_cvt_scalef32_pk_bf16_fp4 converts two E2M1 codes to bf16 *and* applies the block's E8M0
+// scale (a per-lane operand) in one instruction: 4 conversions build a B fragment, exactly.
+// The k index inside an MFMA step only has to agree between A and B, so lane (ni = row,
+// kb = lane / 16) takes four whole consecutive blocks 16T + 4kb + j (j = 0..3, 64 contiguous
+// bytes, four 16-byte loads) and spends them over 16 steps (block j, quarter s = bytes
+// 4s..4s+3); the matching activation fragment is the 16-byte chunk 4*(16T+4kb+j) + s of the
+// token row, read from LDS where the tokens are staged once per workgroup (chunk-major,
+// token fastest).  Rows of the M tile past the expert's token count compute garbage that is
+// never stored (MFMA rows are independent).  One conversion per two weights and one MFMA per
+// 512 weights replace the dot2 chain, the per-row wave reduction and the 70 % lane use of
+// the one-wave-per-row form at 90 blocks per row.
+// grid.x = blocks of 4 waves x FR x 16 rows, grid.y = expert (1 for the plain form).
+// ---------------------------------------------------------------------------
+template <int MTOK, int FR>
+__global__ __launch_bounds__(256) void mxfp4_mfma_kernel(
+    const uint16_t *__restrict__ x, const uint8_t *__restrict__ blocks,
+    const uint8_t *__restrict__ scales, const uint16_t *__restrict__ bias,
+    uint16_t *__restrict__ y, const int32_t *__restrict__ offsets,
+    const int32_t *__restrict__ token_ids, int M, int K, int N) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char mm_lds[];  // [K/8 chunks][MTOK] x 16 B
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int ni = lane & 15, kb = lane >> 4;
+    const int e = blockIdx.y;
+    int p0 = 0, p1 = M;
+    if (offsets) {
+        p0 = offsets[e];
+        p1 = offsets[e + 1];
+        if (p1 <= p0) return;  // block-uniform
+    }
+    const int nb = K >> 5, cpr = K >> 3;
+    const int NT = (nb + 15) >> 4;  // tiles of 16 blocks
+    const int n_base = (blockIdx.x * 4 + wave) * (16 * FR);
+    const u32x4_t *wrow[FR];
+    const uint8_t *srow[FR];
+#pragma unroll
+    for (int f = 0; f < FR; ++f) {
+        const int n = n_base + 16 * f + ni;
+        const size_t row = (size_t)e * N + (n < N ? n : N - 1);
+        wrow[f] = (const u32x4_t *)blocks + row * nb;
+        srow[f] = scales + row * nb;
+    }
+    const int a_tok = (ni & (MTOK - 1)) * 16;
+
+    for (int pbase = p0; pbase < p1; pbase += MTOK) {
+        const int rows = min(MTOK, p1 - pbase);
+        if (pbase > p0) __syncthreads();  // everyone is done with the previous tokens
+        for (int c = threadIdx.x; c < rows * cpr; c += 256) {
+            const int m = c / cpr, cc = c - m * cpr;
+            const int p = pbase + m;
+            const int src = token_ids ? token_ids[p] : p;
+            *(u32x4_t *)(mm_lds + ((size_t)cc * MTOK + m) * 16) = *(const u32x4_t *)(x + (size_t)src * K + (size_t)cc * 8);
+        }
+        __syncthreads();
+
+        float4_t acc[FR];
+#pragma unroll
+        for (int f = 0; f < FR; ++f) acc[f] = float4_t{0.f, 0.f, 0.f, 0.f};
+        u32x4_t wq[2][FR][4];
+        uint32_t sb[2][FR][4];
+        auto load_tile = [&](int T, u32x4_t (&w)[FR][4], uint32_t (&sc)[FR][4]) {
+#pragma unroll
+            for (int f = 0; f < FR; ++f)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int b = 16 * T + 4 * kb + j;
+                    const int bc = b < nb ? b : nb - 1;
+                    w[f][j] = wrow[f][bc];
+                    sc[f][j] = srow[f][bc];
+                }
+        };
+        load_tile(0, wq[0], sb[0]);
+        for (int T0 = 0; T0 < NT; T0 += 2) {
+#pragma unroll
+            for (int par = 0; par < 2; ++par) {
+                const int T = T0 + par;
+                if (T < NT) {  // block-uniform
+                    if (T + 1 < NT) load_tile(T + 1, wq[par ^ 1], sb[par ^ 1]);
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const int b = 16 * T + 4 * kb + j;
+                        const bool valid = b < nb;  // blocks past the row contribute zero
+                        float scf[FR];
+                        uint32_t wj[FR][4];
+#pragma unroll
+                        for (int f = 0; f < FR; ++f) {
+                            scf[f] = e8m0_to_f32(sb[par][f][j]);
+                            const u32x4_t t = wq[par][f][j];
+                            const uint32_t t0 = t[0], t1 = t[1], t2 = t[2], t3 = t[3];
+                            wj[f][0] = valid ? t0 : 0u, wj[f][1] = valid ? t1 : 0u;
+                            wj[f][2] = valid ? t2 : 0u, wj[f][3] = valid ? t3 : 0u;
+                        }
+                        const int bcl = valid ? b : nb - 1;  // a finite activation chunk for padding blocks
+#pragma unroll
+                        for (int sq = 0; sq < 4; ++sq) {
+                            const u32x4_t av = *(const u32x4_t *)(mm_lds + (size_t)(4 * bcl + sq) * MTOK * 16 + a_tok);
+#pragma unroll
+                            for (int f = 0; f < FR; ++f) {
+                                const uint32_t w = wj[f][sq];
+                                u32x4_t bv;
+                                bv[0] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scf[f], 0));
+                                bv[1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scf[f], 1));
+                                bv[2] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scf[f], 2));
+                                bv[3] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scf[f], 3));
+                                acc[f] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av),
+                                                                                __builtin_bit_cast(bf16x8_t, bv), acc[f], 0, 0, 0);
+                            }
+                        }
+                    }
+                }
+            }
+        }
+        // D[m][n]: lane (n = ni, m = 4*kb + i): token 4*kb + i of weight row n_base + 16 f + ni
+#pragma unroll
+        for (int f = 0; f < FR; ++f) {
+            const int n = n_base + 16 * f + ni;
+            if (n < N) {
+                const float bv = bias ? BF16Traits::to_f32(bias[(size_t)e * N + n]) : 0.0f;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int m = 4 * kb + i;
+                    if (m < rows) y[(size_t)(pbase + m) * N + n] = BF16Traits::from_f32(acc[f][i] + bv);
+                }
+            }
+        }
+    }
+}
+
 __global__ __launch_bounds__(256) void mxfp4_dequant_kernel(const uint8_t *__restrict__ blocks,
                                                             const uint8_t *__restrict__ scales,
                                                             float *__restrict__ out, size_t nblocks) {
@@ -266,14 +398,52 @@ static int mxfp4_lds_go(hipStream_t s, dim3 grid, const Mxfp4Problem &p, size_t 
     return OXQ_OK;
 }
 
+template <int MTOK, int FR>
+static int mxfp4_mfma_go(hipStream_t s, dim3 grid, const Mxfp4Problem &p, size_t lds) {
+    static size_t attr_lds = 0;
+    if (lds > attr_lds) {
+        OXQ_HIP_CHECK(hipFuncSetAttribute((const void *)mxfp4_mfma_kernel<MTOK, FR>,
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        attr_lds = lds;
+    }
+    hipLaunchKernelGGL((mxfp4_mfma_kernel<MTOK, FR>), grid, dim3(256), lds, s, (const uint16_t *)p.x, p.blocks,
+                       p.scales, (const uint16_t *)p.bias, (uint16_t *)p.y, p.expert_offsets, p.token_ids,
+                       (int)p.M, (int)p.K, (int)p.N);
+    OXQ_HIP_CHECK(hipGetLastError());
+    return OXQ_OK;
+}
+
 int launch_mxfp4_gemv(oxq_ctx *ctx, hipStream_t s, const Mxfp4Problem &p) {
     const bool grouped = p.n_experts > 0;
+    bool force_rows = false;
+    {
+        // matrix-core form: tokens staged in LDS (MTOK per pass), 4 waves x FR x 16 rows per workgroup
+        const char *v = getenv("OXQ_MXFP4_VARIANT");
+        const int variant = v ? atoi(v) : 0;  // 0 = matrix cores, 1 = dot2 with staged tokens, 2 = one wave per row
+        const int mtok = (grouped || p.M <= 4) ? 4 : 16;
+        const char *frs = getenv("OXQ_MXFP4_FR");
+        const int FR = frs ? atoi(frs) : 1;
+        const size_t lds = (size_t)mtok * (size_t)p.K * 2;
+        if (variant == 0 && lds <= 128 * 1024 && p.K % 32 == 0) {
+            dim3 grid((unsigned)ceil_div(p.N, 4 * 16 * FR), grouped ? (unsigned)p.n_experts : 1u), block(256);
+            char name[64];
+            snprintf(name, sizeof name, "%s_mfma_t%d", grouped ? "mxfp4_moe_gemv_bf16" : "mxfp4_gemv_bf16", mtok);
+            set_plan(ctx, name, grid, block, 1, 1, 0);
+            if (ctx->plan_only) return OXQ_OK;
+            if (((uintptr_t)p.blocks & 15) || ((uintptr_t)p.x & 15))
+                return fail(OXQ_ERR_UNSUPPORTED, "mxfp4 gemv: blocks and x must be 16-byte aligned");
+            if (FR == 1) return mtok == 4 ? mxfp4_mfma_go<4, 1>(s, grid, p, lds) : mxfp4_mfma_go<16, 1>(s, grid, p, lds);
+            if (FR == 4) return mtok == 4 ? mxfp4_mfma_go<4, 4>(s, grid, p, lds) : mxfp4_mfma_go<16, 4>(s, grid, p, lds);
+            return mtok == 4 ? mxfp4_mfma_go<4, 2>(s, grid, p, lds) : mxfp4_mfma_go<16, 2>(s, grid, p, lds);
+        }
+        force_rows = variant == 2;
+    }
     const int64_t rows_hint = grouped ? 4 : p.M;  // tokens per expert are few in decode
     const int mb = rows_hint <= 1 ? 1 : rows_hint <= 2 ? 2 : rows_hint <= 4 ? 4 : 8;
     constexpr int RW = 8;
     const size_t lds = (size_t)mb * 4 * (size_t)((p.K >> 5) + 1) * 16;
     const char *force = getenv("OXQ_FORCE_GENERIC");
-    const bool use_lds = lds <= 96 * 1024 && !(force && atoi(force));
+    const bool use_lds = lds <= 96 * 1024 && !(force && atoi(force)) && !force_rows;
     if (use_lds) {
         dim3 grid((unsigned)ceil_div(p.N, 4 * RW), grouped ? (unsigned)p.n_experts : 1u), block(256);
         char name[64];
