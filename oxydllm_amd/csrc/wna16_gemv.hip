@@ -146,7 +146,18 @@ __global__ __launch_bounds__(256) void awq_gemv_generic(
     if (j < packed_out) {
         int last_g = -1;
         float zf[PF], sf[PF];
-        for (int i = k0 + ty; i < k1; i += 4) {
+        constexpr int UL = 8;  // packed words in flight per lane
+        for (int ib = k0 + ty; ib < k1; ib += 4 * UL) {
+          uint32_t wwb[UL];
+#pragma unroll
+          for (int u = 0; u < UL; ++u) {
+              const int i = ib + 4 * u;
+              wwb[u] = i < k1 ? qw[(size_t)i * packed_out + j] : 0u;
+          }
+#pragma unroll
+          for (int u = 0; u < UL; ++u) {
+            const int i = ib + 4 * u;
+            if (i >= k1) break;
             const int g = i >> gshift;
             if (g != last_g) {
                 const uint32_t zw = qz[(size_t)g * packed_out + j];
@@ -158,7 +169,7 @@ __global__ __launch_bounds__(256) void awq_gemv_generic(
                 }
                 last_g = g;
             }
-            const uint32_t ww = qw[(size_t)i * packed_out + j];
+            const uint32_t ww = wwb[u];
             float w[PF];
 #pragma unroll
             for (int s = 0; s < PF; ++s) w[s] = ((float)((ww >> (BITS * s)) & MASK) - zf[s]) * sf[s];
@@ -170,6 +181,7 @@ __global__ __launch_bounds__(256) void awq_gemv_generic(
                     for (int s = 0; s < PF; ++s) acc[m][s] = fmaf(xv, w[s], acc[m][s]);
                 }
             }
+          }
         }
     }
 
@@ -234,7 +246,18 @@ __global__ __launch_bounds__(256) void gptq_gemv_generic(
         int last_g = -1;
         float zp1 = 0.0f, sv = 0.0f;
         const uint32_t zshift = BITS * (n % PF);
-        for (int iw = w0 + ty; iw < w1; iw += 4) {
+        constexpr int UL = 8;  // packed words in flight per lane
+        for (int ib = w0 + ty; ib < w1; ib += 4 * UL) {
+          uint32_t wwb[UL];
+#pragma unroll
+          for (int u = 0; u < UL; ++u) {
+              const int iw = ib + 4 * u;
+              wwb[u] = iw < w1 ? qw[(size_t)iw * N + n] : 0u;
+          }
+#pragma unroll
+          for (int u = 0; u < UL; ++u) {
+            const int iw = ib + 4 * u;
+            if (iw >= w1) break;
             const int g = (iw * PF) >> gshift;
             if (g != last_g) {
                 const uint32_t zw = qz[(size_t)g * packed_out + n / PF];
@@ -242,7 +265,7 @@ __global__ __launch_bounds__(256) void gptq_gemv_generic(
                 sv = TT::to_f32(sc[(size_t)g * N + n]);
                 last_g = g;
             }
-            const uint32_t ww = qw[(size_t)iw * N + n];
+            const uint32_t ww = wwb[u];
             float w[PF];
 #pragma unroll
             for (int s = 0; s < PF; ++s) w[s] = sv * ((float)((ww >> (BITS * s)) & MASK) - zp1);
@@ -254,6 +277,7 @@ __global__ __launch_bounds__(256) void gptq_gemv_generic(
                     for (int s = 0; s < PF; ++s) acc[m] = fmaf(TT::to_f32(xr[s]), w[s], acc[m]);
                 }
             }
+          }
         }
     }
     const int n0 = blockIdx.x * 64;
