@@ -208,6 +208,42 @@ int oxq_mxfp4_moe_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x,
                          const oxq_tensor *token_ids, int gather_rows, int64_t k, int64_t n,
                          const oxq_tensor *out);
 
+/* ---- mixture-of-experts glue: the steps either side of the expert GEMVs -----
+ * The reference does these on the host / with one launch per expert
+ * (moe.rs:466-607); here they run on the device and feed oxq_mxfp4_moe_matmul. */
+
+/* moe.rs:466-486 + linear.rs:160-171: softmax over experts in f32, stable
+ * descending top-k, optional renormalisation by the sum of the chosen.
+ *  logits    F32 | F16 | BF16 [n_tokens, n_experts]
+ *  top_idx   I32 [n_tokens, top_k] (out)    top_vals  F32 [n_tokens, top_k] (out);  top_k <= 64 */
+int oxq_moe_route(oxq_ctx *ctx, void *stream, const oxq_tensor *logits, int64_t top_k, int norm_topk,
+                  const oxq_tensor *top_idx, const oxq_tensor *top_vals);
+
+/* moe.rs:563-590 dispatch_sparse: (token, slot) pairs grouped by expert, tokens
+ * ascending inside an expert.  P = n_tokens * top_k; n_experts <= 256.
+ *  expert_offsets I32 [n_experts + 1]   token_ids I32 [P]   pair_weights F32 [P]
+ *  pair_pos       I32 [n_tokens, top_k]: where pair (token, slot) went (for the combine) */
+int oxq_moe_group(oxq_ctx *ctx, void *stream, const oxq_tensor *top_idx, const oxq_tensor *top_vals,
+                  int64_t n_experts, const oxq_tensor *expert_offsets, const oxq_tensor *token_ids,
+                  const oxq_tensor *pair_weights, const oxq_tensor *pair_pos);
+
+typedef enum oxq_gated_act {
+    OXQ_ACT_GATED_SILU = 0,      /* [.., gate | up]: silu(gate) * up, ffn_kernels.metal:19-68 */
+    OXQ_ACT_GATED_GELU_TANH = 1, /* [.., gate | up]: gelu_tanh(gate) * up, ffn_kernels.metal:115-160 */
+    OXQ_ACT_GPT_OSS_SWIGLU = 2   /* interleaved (gate, up), clamped, alpha 1.702: moe.rs:152-173 */
+} oxq_gated_act;
+
+/* gate_up [rows, 2*I] -> out [rows, I], same dtype (F32 | F16 | BF16); f32 math, one
+ * rounding.  `limit` is only read by OXQ_ACT_GPT_OSS_SWIGLU. */
+int oxq_gated_activation(oxq_ctx *ctx, void *stream, const oxq_tensor *gate_up, int kind, float limit,
+                         const oxq_tensor *out);
+
+/* moe.rs:592-605: out[token] = sum over slots of top_vals[token, slot] *
+ * expert_out[pair_pos[token, slot]]  (f32 accumulation in slot order, one rounding).
+ *  expert_out T [P, hidden]   out T [n_tokens, hidden] */
+int oxq_moe_combine(oxq_ctx *ctx, void *stream, const oxq_tensor *expert_out, const oxq_tensor *pair_pos,
+                    const oxq_tensor *top_vals, const oxq_tensor *out);
+
 /* ---- layers ----------------------------------------------------------------
  * Host-side mirrors of the reference layer types; they hold descriptors of
  * caller-owned resident weights and route by m exactly where the reference

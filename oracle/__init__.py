@@ -245,3 +245,31 @@ def gpt_oss_swiglu(gu, limit: float) -> np.ndarray:
     h = np.empty((M, two_i // 2), dtype=np.float32)
     lib().orc_gpt_oss_swiglu(_p(gu), C.c_int64(M), C.c_int64(two_i // 2), C.c_float(limit), _p(h))
     return h
+
+
+def gated_silu(gu) -> np.ndarray:
+    gu = _f32(gu)
+    M, two_i = gu.shape
+    out = np.empty((M, two_i // 2), dtype=np.float32)
+    lib().orc_gated_silu(_p(gu), C.c_int64(M), C.c_int64(two_i // 2), _p(out))
+    return out
+
+
+def gated_gelu_tanh(gu) -> np.ndarray:
+    gu = _f32(gu)
+    M, two_i = gu.shape
+    out = np.empty((M, two_i // 2), dtype=np.float32)
+    lib().orc_gated_gelu_tanh(_p(gu), C.c_int64(M), C.c_int64(two_i // 2), _p(out))
+    return out
+
+
+def moe_combine(expert_out, offsets, tokens, weights, n_tokens: int) -> np.ndarray:
+    expert_out = _f32(expert_out)
+    offsets = np.ascontiguousarray(np.asarray(offsets, dtype=np.int64))
+    tokens = np.ascontiguousarray(np.asarray(tokens, dtype=np.uint32))
+    weights = _f32(weights)
+    P, H = expert_out.shape
+    out = np.empty((n_tokens, H), dtype=np.float32)
+    lib().orc_moe_combine(_p(expert_out), _p(offsets), _p(tokens), _p(weights), C.c_int64(len(offsets) - 1),
+                          C.c_int64(n_tokens), C.c_int64(H), _p(out))
+    return out

@@ -22,6 +22,8 @@
  *   orc_moe_route             src/common/moe.rs:466-499 + linear.rs:160-171
  *   orc_moe_group             src/common/moe.rs:563-607  (dispatch_sparse lists)
  *   orc_gpt_oss_swiglu        src/common/moe.rs:152-173
+ *   orc_gated_silu / _gelu_tanh src/common/ffn_kernels.metal:5-17, 23-36, 115-128
+ *   orc_moe_combine           src/common/moe.rs:592-605 (index_add of gate-weighted rows)
  *   orc_f32_to_f16 / bf16     `half` crate from_f32 (IEEE round-to-nearest-even),
  *                             used by awq.rs:421-431
  *
@@ -535,5 +537,38 @@ void orc_gpt_oss_swiglu(const float *gu, int64_t M, int64_t I, float limit, floa
             up = up < -limit ? -limit : (up > limit ? limit : up);
             const float sig = 1.0f / (1.0f + expf(-(gate * 1.702f)));
             h[m * I + k] = (up + 1.0f) * (gate * sig);
+        }
+}
+
+/* Fused gated activations over [.., gate | up]: ffn_kernels.metal:5-17 (scalar functions),
+ * 23-36 and 115-128 (the f32 kernels).  gu [M, 2I] -> out [M, I], f32 math. */
+void orc_gated_silu(const float *gu, int64_t M, int64_t I, float *out) {
+    for (int64_t m = 0; m < M; ++m)
+        for (int64_t k = 0; k < I; ++k) {
+            const float g = gu[m * 2 * I + k], u = gu[m * 2 * I + I + k];
+            out[m * I + k] = (g / (1.0f + expf(-g))) * u;
+        }
+}
+
+void orc_gated_gelu_tanh(const float *gu, int64_t M, int64_t I, float *out) {
+    const float k0 = 0.7978845608028654f, k1 = 0.044715f;
+    for (int64_t m = 0; m < M; ++m)
+        for (int64_t k = 0; k < I; ++k) {
+            const float g = gu[m * 2 * I + k], u = gu[m * 2 * I + I + k];
+            const float inner = k0 * (g + k1 * g * g * g);
+            out[m * I + k] = (0.5f * g * (1.0f + tanhf(inner))) * u;
+        }
+}
+
+/* dispatch_sparse's scatter, moe.rs:592-605: experts in ascending order, each adding
+ * weight * expert_out for its tokens.  Restated in f32 (the reference accumulates in the
+ * activation dtype; the caller rounds as needed).  expert_out is in grouped pair order. */
+void orc_moe_combine(const float *expert_out, const int64_t *offsets, const uint32_t *tokens,
+                     const float *weights, int64_t E, int64_t T, int64_t H, float *out) {
+    for (int64_t i = 0; i < T * H; ++i) out[i] = 0.0f;
+    for (int64_t e = 0; e < E; ++e)
+        for (int64_t p = offsets[e]; p < offsets[e + 1]; ++p) {
+            const int64_t t = tokens[p];
+            for (int64_t h = 0; h < H; ++h) out[t * H + h] += weights[p] * expert_out[p * H + h];
         }
 }

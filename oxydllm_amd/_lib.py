@@ -73,6 +73,10 @@ SIGNATURES = {
     "oxq_mxfp4_dequantize": (C.c_int, [_VP, _VP, _TP, _TP, C.c_int64, C.c_int64, _TP]),
     "oxq_mxfp4_moe_matmul": (C.c_int, [_VP, _VP, _TP, _TP, _TP, _TP, _TP, _TP, C.c_int,
                                        C.c_int64, C.c_int64, _TP]),
+    "oxq_moe_route": (C.c_int, [_VP, _VP, _TP, C.c_int64, C.c_int, _TP, _TP]),
+    "oxq_moe_group": (C.c_int, [_VP, _VP, _TP, _TP, C.c_int64, _TP, _TP, _TP, _TP]),
+    "oxq_gated_activation": (C.c_int, [_VP, _VP, _TP, C.c_int, C.c_float, _TP]),
+    "oxq_moe_combine": (C.c_int, [_VP, _VP, _TP, _TP, _TP, _TP]),
     "oxq_packed_quant_linear_new": (C.c_int, [_VP, C.c_uint32, C.c_int, _TP, _TP, _TP, _TP,
                                               C.c_int, C.POINTER(_VP)]),
     "oxq_packed_quant_linear_forward": (C.c_int, [_VP, _VP, _TP, _TP]),

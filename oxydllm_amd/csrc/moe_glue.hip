@@ -1,0 +1,298 @@
+// The steps either side of the expert GEMVs of a mixture-of-experts layer, on the device:
+// router softmax + top-k, grouping of (token, slot) pairs by expert, the gated activation
+// between the two projections, and the gate-weighted combine.
+//
+// Reference semantics:
+//   route    moe.rs:466-486   logits -> f32, softmax over experts (linear.rs:160-171),
+//                             arg_sort descending (stable: equal scores keep expert order),
+//                             first top_k, optional renormalisation by their sum
+//   group    moe.rs:563-590   dispatch_sparse: per expert the list of its tokens and gate
+//                             weights, tokens ascending, slots in order
+//   activate ffn_kernels.metal:19-242 gated SiLU / GeLU-tanh over [.., gate | up] (f32 math,
+//                             one rounding) and moe.rs:152-173 GPT-OSS clamped SwiGLU over
+//                             interleaved (gate, up) pairs
+//   combine  moe.rs:592-605   output[token] += weight * expert_out[pair]
+//
+// The reference builds the lists on the host after copying the router output back and then
+// launches one set of kernels per active expert; here nothing leaves the device, and the
+// grouped expert GEMV consumes the lists directly (expert_offsets / token_ids).
+// All of it is integer / small elementwise work bound by launch latency; every kernel is
+// deterministic (no atomics on floats, fixed orders).
+
+#include "oxq_device.hpp"
+#include "oxq_internal.hpp"
+
+namespace oxq {
+
+template <typename T> __device__ __forceinline__ float load_f32(const T *p, size_t i);
+template <> __device__ __forceinline__ float load_f32<float>(const float *p, size_t i) { return p[i]; }
+struct F16Tag { uint16_t v; };
+struct BF16Tag { uint16_t v; };
+template <> __device__ __forceinline__ float load_f32<F16Tag>(const F16Tag *p, size_t i) {
+    return F16Traits::to_f32(p[i].v);
+}
+template <> __device__ __forceinline__ float load_f32<BF16Tag>(const BF16Tag *p, size_t i) {
+    return BF16Traits::to_f32(p[i].v);
+}
+template <typename T> __device__ __forceinline__ void store_f32(T *p, size_t i, float v);
+template <> __device__ __forceinline__ void store_f32<float>(float *p, size_t i, float v) { p[i] = v; }
+template <> __device__ __forceinline__ void store_f32<F16Tag>(F16Tag *p, size_t i, float v) {
+    p[i].v = F16Traits::from_f32(v);
+}
+template <> __device__ __forceinline__ void store_f32<BF16Tag>(BF16Tag *p, size_t i, float v) {
+    p[i].v = BF16Traits::from_f32(v);
+}
+
+// ---------------------------------------------------------------------------
+// route: one wave per token, probabilities in LDS
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void moe_route_kernel(const T *__restrict__ logits, int ntok, int E, int top_k,
+                                                        int norm_topk, int32_t *__restrict__ top_idx,
+                                                        float *__restrict__ top_vals) {
+    extern __shared__ float route_lds[];  // [4 waves][E]
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int t = blockIdx.x * 4 + wave;
+    if (t >= ntok) return;  // wave-uniform; no barrier below
+    float *probs = route_lds + (size_t)wave * E;
+    const T *l = logits + (size_t)t * E;
+    float mx = -INFINITY;
+    for (int e = lane; e < E; e += 64) mx = fmaxf(mx, load_f32(l, e));
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+    float sum = 0.0f;
+    for (int e = lane; e < E; e += 64) {
+        const float p = expf(load_f32(l, e) - mx);
+        probs[e] = p;
+        sum += p;
+    }
+    sum = wave_sum_xor<64>(sum);
+    for (int e = lane; e < E; e += 64) probs[e] = probs[e] / sum;
+    // the wave's own LDS writes are visible to its own later reads (same wave, in order)
+    float chosen_sum = 0.0f, my_val = 0.0f;
+    int my_idx = 0;
+    for (int s = 0; s < top_k; ++s) {
+        float bv = -1.0f;
+        int bi = 0x7fffffff;
+        for (int e = lane; e < E; e += 64) {
+            const float p = probs[e];
+            if (p > bv) {  // strict: the lowest index wins among equals within a lane
+                bv = p;
+                bi = e;
+            }
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {  // butterfly: every lane ends with the winner
+            const float ov = __shfl_xor(bv, off, 64);
+            const int oi = __shfl_xor(bi, off, 64);
+            if (ov > bv || (ov == bv && oi < bi)) {
+                bv = ov;
+                bi = oi;
+            }
+        }
+        if (lane == s) {  // slot s is kept by lane s
+            my_val = bv;
+            my_idx = bi;
+        }
+        if (lane == 0) probs[bi] = -2.0f;  // taken
+        chosen_sum += bv;  // slot order, as the reference's sum over the gathered values
+    }
+    if (lane < top_k) {
+        const size_t i = (size_t)t * top_k + lane;
+        top_idx[i] = my_idx;
+        top_vals[i] = norm_topk ? my_val / chosen_sum : my_val;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// group: one wave; thread i owns the contiguous pair range [i*L, (i+1)*L)
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(64) void moe_group_kernel(const int32_t *__restrict__ top_idx,
+                                                       const float *__restrict__ top_vals, int P, int E,
+                                                       int32_t *__restrict__ offsets, int32_t *__restrict__ tokens,
+                                                       float *__restrict__ weights, int32_t *__restrict__ pair_pos,
+                                                       int top_k) {
+    extern __shared__ int32_t group_lds[];  // cnt[E][64], then base[E]
+    int32_t *cnt = group_lds;
+    int32_t *base = group_lds + (size_t)E * 64;
+    const int lane = threadIdx.x;
+    const int L = (P + 63) / 64;
+    const int i0 = min(P, lane * L), i1 = min(P, i0 + L);
+    for (int e = 0; e < E; ++e) cnt[e * 64 + lane] = 0;
+    for (int i = i0; i < i1; ++i) {
+        const int e = top_idx[i];
+        if (e >= 0 && e < E) cnt[e * 64 + lane] += 1;  // ids outside [0, E) are dropped
+    }
+    __syncthreads();
+    // per expert: exclusive prefix over the 64 owners, total in base[e]
+    for (int e = lane; e < E; e += 64) {
+        int run = 0;
+        for (int j = 0; j < 64; ++j) {
+            const int c = cnt[e * 64 + j];
+            cnt[e * 64 + j] = run;
+            run += c;
+        }
+        base[e] = run;
+    }
+    __syncthreads();
+    if (lane == 0) {
+        int run = 0;
+        for (int e = 0; e < E; ++e) {
+            const int c = base[e];
+            offsets[e] = run;
+            base[e] = run;
+            run += c;
+        }
+        offsets[E] = run;
+    }
+    __syncthreads();
+    for (int i = i0; i < i1; ++i) {
+        const int e = top_idx[i];
+        if (e < 0 || e >= E) continue;
+        const int pos = base[e] + cnt[e * 64 + lane];
+        cnt[e * 64 + lane] += 1;
+        tokens[pos] = i / top_k;
+        weights[pos] = top_vals[i];
+        pair_pos[i] = pos;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// gated activation
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ float silu_f32(float x) { return x / (1.0f + expf(-x)); }
+__device__ __forceinline__ float gelu_tanh_f32(float x) {
+    const float k0 = 0.7978845608028654f, k1 = 0.044715f;
+    return 0.5f * x * (1.0f + tanhf(k0 * (x + k1 * x * x * x)));
+}
+
+template <typename T, int KIND>
+__global__ __launch_bounds__(256) void gated_act_kernel(const T *__restrict__ gu, T *__restrict__ out, size_t n_out,
+                                                        int half_n, float limit) {
+    const size_t gid = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (gid >= n_out) return;
+    const size_t row = gid / half_n, col = gid % half_n;
+    float r;
+    if (KIND == OXQ_ACT_GPT_OSS_SWIGLU) {  // interleaved (gate, up), moe.rs:152-173
+        float gate = load_f32(gu, row * 2 * half_n + 2 * col);
+        float up = load_f32(gu, row * 2 * half_n + 2 * col + 1);
+        gate = fminf(gate, limit);
+        up = fminf(fmaxf(up, -limit), limit);
+        const float sig = 1.0f / (1.0f + expf(-(gate * 1.702f)));
+        r = (up + 1.0f) * (gate * sig);
+    } else {  // [gate | up], ffn_kernels.metal:19-242
+        const float g = load_f32(gu, row * 2 * half_n + col);
+        const float u = load_f32(gu, row * 2 * half_n + half_n + col);
+        r = (KIND == OXQ_ACT_GATED_SILU ? silu_f32(g) : gelu_tanh_f32(g)) * u;
+    }
+    store_f32(out, gid, r);
+}
+
+// ---------------------------------------------------------------------------
+// combine: out[t] = sum over slots of w[t, s] * expert_out[pair_pos[t, s]] (f32, slot order)
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void moe_combine_kernel(const T *__restrict__ eo, const int32_t *__restrict__ pair_pos,
+                                                          const float *__restrict__ top_vals, T *__restrict__ out,
+                                                          int ntok, int H, int top_k) {
+    const size_t gid = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (gid >= (size_t)ntok * H) return;
+    const int t = (int)(gid / H), h = (int)(gid % H);
+    float acc = 0.0f;
+    for (int s = 0; s < top_k; ++s) {
+        const int pos = pair_pos[(size_t)t * top_k + s];
+        acc = fmaf(top_vals[(size_t)t * top_k + s], load_f32(eo, (size_t)pos * H + h), acc);
+    }
+    store_f32(out, gid, acc);
+}
+
+// ---------------------------------------------------------------------------
+// launchers
+// ---------------------------------------------------------------------------
+int launch_moe_route(oxq_ctx *ctx, hipStream_t s, const void *logits, int dtype, int64_t T, int64_t E, int64_t top_k,
+                     int norm_topk, int32_t *top_idx, float *top_vals) {
+    dim3 grid((unsigned)ceil_div(T, 4)), block(256);
+    set_plan(ctx, "moe_route", grid, block, 1, 1, 0);
+    if (ctx->plan_only) return OXQ_OK;
+    const size_t lds = (size_t)4 * E * sizeof(float);
+    if (dtype == OXQ_F32)
+        hipLaunchKernelGGL(moe_route_kernel<float>, grid, block, lds, s, (const float *)logits, (int)T, (int)E,
+                           (int)top_k, norm_topk, top_idx, top_vals);
+    else if (dtype == OXQ_F16)
+        hipLaunchKernelGGL(moe_route_kernel<F16Tag>, grid, block, lds, s, (const F16Tag *)logits, (int)T, (int)E,
+                           (int)top_k, norm_topk, top_idx, top_vals);
+    else
+        hipLaunchKernelGGL(moe_route_kernel<BF16Tag>, grid, block, lds, s, (const BF16Tag *)logits, (int)T, (int)E,
+                           (int)top_k, norm_topk, top_idx, top_vals);
+    OXQ_HIP_CHECK(hipGetLastError());
+    return OXQ_OK;
+}
+
+int launch_moe_group(oxq_ctx *ctx, hipStream_t s, const int32_t *top_idx, const float *top_vals, int64_t P, int64_t E,
+                     int64_t top_k, int32_t *offsets, int32_t *tokens, float *weights, int32_t *pair_pos) {
+    dim3 grid(1), block(64);
+    set_plan(ctx, "moe_group", grid, block, 1, 1, 0);
+    if (ctx->plan_only) return OXQ_OK;
+    const size_t lds = ((size_t)E * 64 + (size_t)E) * sizeof(int32_t);
+    static size_t attr_lds = 0;
+    if (lds > attr_lds) {
+        OXQ_HIP_CHECK(hipFuncSetAttribute((const void *)moe_group_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                          (int)lds));
+        attr_lds = lds;
+    }
+    hipLaunchKernelGGL(moe_group_kernel, grid, block, lds, s, top_idx, top_vals, (int)P, (int)E, offsets, tokens,
+                       weights, pair_pos, (int)top_k);
+    OXQ_HIP_CHECK(hipGetLastError());
+    return OXQ_OK;
+}
+
+template <typename T>
+static void gated_go(hipStream_t s, dim3 grid, int kind, const void *gu, void *out, size_t n_out, int half_n,
+                     float limit) {
+    dim3 block(256);
+    if (kind == OXQ_ACT_GATED_SILU)
+        hipLaunchKernelGGL((gated_act_kernel<T, OXQ_ACT_GATED_SILU>), grid, block, 0, s, (const T *)gu, (T *)out, n_out,
+                           half_n, limit);
+    else if (kind == OXQ_ACT_GATED_GELU_TANH)
+        hipLaunchKernelGGL((gated_act_kernel<T, OXQ_ACT_GATED_GELU_TANH>), grid, block, 0, s, (const T *)gu, (T *)out,
+                           n_out, half_n, limit);
+    else
+        hipLaunchKernelGGL((gated_act_kernel<T, OXQ_ACT_GPT_OSS_SWIGLU>), grid, block, 0, s, (const T *)gu, (T *)out,
+                           n_out, half_n, limit);
+}
+
+int launch_gated_activation(oxq_ctx *ctx, hipStream_t s, const void *gu, void *out, int dtype, int64_t rows,
+                            int64_t half_n, int kind, float limit) {
+    const size_t n_out = (size_t)rows * (size_t)half_n;
+    dim3 grid((unsigned)ceil_div((int64_t)n_out, 256)), block(256);
+    set_plan(ctx, kind == OXQ_ACT_GATED_SILU ? "gated_silu" : kind == OXQ_ACT_GATED_GELU_TANH ? "gated_gelu_tanh"
+                                                                                             : "gpt_oss_swiglu",
+             grid, block, 1, 1, 0);
+    if (ctx->plan_only || n_out == 0) return OXQ_OK;
+    if (dtype == OXQ_F32) gated_go<float>(s, grid, kind, gu, out, n_out, (int)half_n, limit);
+    else if (dtype == OXQ_F16) gated_go<F16Tag>(s, grid, kind, gu, out, n_out, (int)half_n, limit);
+    else gated_go<BF16Tag>(s, grid, kind, gu, out, n_out, (int)half_n, limit);
+    OXQ_HIP_CHECK(hipGetLastError());
+    return OXQ_OK;
+}
+
+int launch_moe_combine(oxq_ctx *ctx, hipStream_t s, const void *eo, const int32_t *pair_pos, const float *top_vals,
+                       void *out, int dtype, int64_t T, int64_t H, int64_t top_k) {
+    const size_t n = (size_t)T * (size_t)H;
+    dim3 grid((unsigned)ceil_div((int64_t)n, 256)), block(256);
+    set_plan(ctx, "moe_combine", grid, block, 1, 1, 0);
+    if (ctx->plan_only || n == 0) return OXQ_OK;
+    if (dtype == OXQ_F32)
+        hipLaunchKernelGGL(moe_combine_kernel<float>, grid, block, 0, s, (const float *)eo, pair_pos, top_vals,
+                           (float *)out, (int)T, (int)H, (int)top_k);
+    else if (dtype == OXQ_F16)
+        hipLaunchKernelGGL(moe_combine_kernel<F16Tag>, grid, block, 0, s, (const F16Tag *)eo, pair_pos, top_vals,
+                           (F16Tag *)out, (int)T, (int)H, (int)top_k);
+    else
+        hipLaunchKernelGGL(moe_combine_kernel<BF16Tag>, grid, block, 0, s, (const BF16Tag *)eo, pair_pos, top_vals,
+                           (BF16Tag *)out, (int)T, (int)H, (int)top_k);
+    OXQ_HIP_CHECK(hipGetLastError());
+    return OXQ_OK;
+}
+
+}  // namespace oxq

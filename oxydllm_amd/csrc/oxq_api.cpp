@@ -645,6 +645,124 @@ int oxq_mxfp4_moe_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x,
     return launch_mxfp4_gemv(ctx, (hipStream_t)stream, p);
 }
 
+// ---- mixture-of-experts glue (moe.rs:466-607, ffn_kernels.metal, moe.rs:152-173) --------
+
+static bool is_float_dtype(int d) { return d == OXQ_F32 || d == OXQ_F16 || d == OXQ_BF16; }
+
+int oxq_moe_route(oxq_ctx *ctx, void *stream, const oxq_tensor *logits, int64_t top_k, int norm_topk,
+                  const oxq_tensor *top_idx, const oxq_tensor *top_vals) {
+    const char *op = "MoeRoute";
+    if (!ctx) return fail(OXQ_ERR_ARG, "%s: ctx is NULL", op);
+    OXQ_TRY(check_tensor(ctx, op, "logits", logits));
+    OXQ_TRY(check_tensor(ctx, op, "top_idx", top_idx));
+    OXQ_TRY(check_tensor(ctx, op, "top_vals", top_vals));
+    if (logits->rank != 2 || !logits->contiguous)
+        return fail(OXQ_ERR_SHAPE, "%s: logits must be a contiguous [n_tokens, n_experts]", op);
+    if (!is_float_dtype(logits->dtype))
+        return fail(OXQ_ERR_DTYPE, "%s: logits must be F32, F16 or BF16, got %s", op, dtype_name(logits->dtype));
+    const int64_t T = logits->dims[0], E = logits->dims[1];
+    if (top_k < 1 || top_k > E || top_k > 64)
+        return fail(OXQ_ERR_ARG, "%s: top_k %lld must be in 1..=min(n_experts %lld, 64)", op, (long long)top_k,
+                    (long long)E);
+    if (E > 4096) return fail(OXQ_ERR_UNSUPPORTED, "%s: at most 4096 experts", op);
+    if (top_idx->dtype != OXQ_I32 || top_idx->rank != 2 || top_idx->dims[0] != T || top_idx->dims[1] != top_k ||
+        !top_idx->contiguous)
+        return fail(OXQ_ERR_SHAPE, "%s: top_idx must be a contiguous I32 [%lld, %lld]", op, (long long)T,
+                    (long long)top_k);
+    if (top_vals->dtype != OXQ_F32 || top_vals->rank != 2 || top_vals->dims[0] != T || top_vals->dims[1] != top_k ||
+        !top_vals->contiguous)
+        return fail(OXQ_ERR_SHAPE, "%s: top_vals must be a contiguous F32 [%lld, %lld]", op, (long long)T,
+                    (long long)top_k);
+    return launch_moe_route(ctx, (hipStream_t)stream, logits->data, logits->dtype, T, E, top_k, norm_topk ? 1 : 0,
+                            (int32_t *)top_idx->data, (float *)top_vals->data);
+}
+
+int oxq_moe_group(oxq_ctx *ctx, void *stream, const oxq_tensor *top_idx, const oxq_tensor *top_vals,
+                  int64_t n_experts, const oxq_tensor *expert_offsets, const oxq_tensor *token_ids,
+                  const oxq_tensor *pair_weights, const oxq_tensor *pair_pos) {
+    const char *op = "MoeGroup";
+    if (!ctx) return fail(OXQ_ERR_ARG, "%s: ctx is NULL", op);
+    OXQ_TRY(check_tensor(ctx, op, "top_idx", top_idx));
+    OXQ_TRY(check_tensor(ctx, op, "top_vals", top_vals));
+    OXQ_TRY(check_tensor(ctx, op, "expert_offsets", expert_offsets));
+    OXQ_TRY(check_tensor(ctx, op, "token_ids", token_ids));
+    OXQ_TRY(check_tensor(ctx, op, "pair_weights", pair_weights));
+    OXQ_TRY(check_tensor(ctx, op, "pair_pos", pair_pos));
+    if (top_idx->dtype != OXQ_I32 || top_idx->rank != 2 || !top_idx->contiguous)
+        return fail(OXQ_ERR_SHAPE, "%s: top_idx must be a contiguous I32 [n_tokens, top_k]", op);
+    const int64_t T = top_idx->dims[0], top_k = top_idx->dims[1], P = T * top_k;
+    if (top_vals->dtype != OXQ_F32 || numel(top_vals) != P || !top_vals->contiguous)
+        return fail(OXQ_ERR_SHAPE, "%s: top_vals must be a contiguous F32 [%lld, %lld]", op, (long long)T,
+                    (long long)top_k);
+    if (n_experts < 1 || n_experts > 256)
+        return fail(OXQ_ERR_ARG, "%s: n_experts %lld must be in 1..=256", op, (long long)n_experts);
+    if (top_k < 1) return fail(OXQ_ERR_SHAPE, "%s: top_k must be positive", op);
+    if (expert_offsets->dtype != OXQ_I32 || numel(expert_offsets) != n_experts + 1 || !expert_offsets->contiguous)
+        return fail(OXQ_ERR_SHAPE, "%s: expert_offsets must be a contiguous I32 [%lld]", op,
+                    (long long)(n_experts + 1));
+    if (token_ids->dtype != OXQ_I32 || numel(token_ids) != P || !token_ids->contiguous)
+        return fail(OXQ_ERR_SHAPE, "%s: token_ids must be a contiguous I32 [%lld]", op, (long long)P);
+    if (pair_weights->dtype != OXQ_F32 || numel(pair_weights) != P || !pair_weights->contiguous)
+        return fail(OXQ_ERR_SHAPE, "%s: pair_weights must be a contiguous F32 [%lld]", op, (long long)P);
+    if (pair_pos->dtype != OXQ_I32 || numel(pair_pos) != P || !pair_pos->contiguous)
+        return fail(OXQ_ERR_SHAPE, "%s: pair_pos must be a contiguous I32 [%lld, %lld]", op, (long long)T,
+                    (long long)top_k);
+    if (P > INT32_MAX) return fail(OXQ_ERR_SHAPE, "%s: too many pairs", op);
+    return launch_moe_group(ctx, (hipStream_t)stream, (const int32_t *)top_idx->data, (const float *)top_vals->data,
+                            P, n_experts, top_k, (int32_t *)expert_offsets->data, (int32_t *)token_ids->data,
+                            (float *)pair_weights->data, (int32_t *)pair_pos->data);
+}
+
+int oxq_gated_activation(oxq_ctx *ctx, void *stream, const oxq_tensor *gate_up, int kind, float limit,
+                         const oxq_tensor *out) {
+    const char *op = "GatedActivation";
+    if (!ctx) return fail(OXQ_ERR_ARG, "%s: ctx is NULL", op);
+    OXQ_TRY(check_tensor(ctx, op, "gate_up", gate_up));
+    OXQ_TRY(check_tensor(ctx, op, "out", out));
+    if (kind != OXQ_ACT_GATED_SILU && kind != OXQ_ACT_GATED_GELU_TANH && kind != OXQ_ACT_GPT_OSS_SWIGLU)
+        return fail(OXQ_ERR_ARG, "%s: unknown activation kind %d", op, kind);
+    if (!gate_up->contiguous || !out->contiguous)
+        return fail(OXQ_ERR_CONTIGUOUS, "%s: gate_up and out must be contiguous", op);
+    if (!is_float_dtype(gate_up->dtype) || out->dtype != gate_up->dtype)
+        return fail(OXQ_ERR_DTYPE, "%s: gate_up and out must share a dtype of F32, F16 or BF16", op);
+    const int64_t last = gate_up->dims[gate_up->rank - 1];
+    if (last % 2 != 0)  // metal_ops.rs:1237-1245: last dim must be 2 * intermediate_size
+        return fail(OXQ_ERR_SHAPE, "%s: last dim %lld is not 2 * intermediate_size", op, (long long)last);
+    const int64_t half_n = last / 2;
+    const int64_t rows = half_n > 0 ? numel(gate_up) / last : 0;
+    if (out->rank != gate_up->rank || out->dims[out->rank - 1] != half_n || numel(out) != rows * half_n)
+        return fail(OXQ_ERR_SHAPE, "%s: out must be [.., %lld]", op, (long long)half_n);
+    if (half_n > INT32_MAX) return fail(OXQ_ERR_SHAPE, "%s: dimension exceeds 2^31-1", op);
+    return launch_gated_activation(ctx, (hipStream_t)stream, gate_up->data, out->data, gate_up->dtype, rows, half_n,
+                                   kind, limit);
+}
+
+int oxq_moe_combine(oxq_ctx *ctx, void *stream, const oxq_tensor *expert_out, const oxq_tensor *pair_pos,
+                    const oxq_tensor *top_vals, const oxq_tensor *out) {
+    const char *op = "MoeCombine";
+    if (!ctx) return fail(OXQ_ERR_ARG, "%s: ctx is NULL", op);
+    OXQ_TRY(check_tensor(ctx, op, "expert_out", expert_out));
+    OXQ_TRY(check_tensor(ctx, op, "pair_pos", pair_pos));
+    OXQ_TRY(check_tensor(ctx, op, "top_vals", top_vals));
+    OXQ_TRY(check_tensor(ctx, op, "out", out));
+    if (pair_pos->dtype != OXQ_I32 || pair_pos->rank != 2 || !pair_pos->contiguous)
+        return fail(OXQ_ERR_SHAPE, "%s: pair_pos must be a contiguous I32 [n_tokens, top_k]", op);
+    const int64_t T = pair_pos->dims[0], top_k = pair_pos->dims[1], P = T * top_k;
+    if (top_vals->dtype != OXQ_F32 || numel(top_vals) != P || !top_vals->contiguous)
+        return fail(OXQ_ERR_SHAPE, "%s: top_vals must be a contiguous F32 [%lld, %lld]", op, (long long)T,
+                    (long long)top_k);
+    if (expert_out->rank != 2 || expert_out->dims[0] != P || !expert_out->contiguous)
+        return fail(OXQ_ERR_SHAPE, "%s: expert_out must be a contiguous [%lld, hidden]", op, (long long)P);
+    const int64_t H = expert_out->dims[1];
+    if (!is_float_dtype(expert_out->dtype) || out->dtype != expert_out->dtype)
+        return fail(OXQ_ERR_DTYPE, "%s: expert_out and out must share a dtype of F32, F16 or BF16", op);
+    if (out->rank != 2 || out->dims[0] != T || out->dims[1] != H || !out->contiguous)
+        return fail(OXQ_ERR_SHAPE, "%s: out must be a contiguous [%lld, %lld]", op, (long long)T, (long long)H);
+    if (H > INT32_MAX || T > INT32_MAX) return fail(OXQ_ERR_SHAPE, "%s: dimension exceeds 2^31-1", op);
+    return launch_moe_combine(ctx, (hipStream_t)stream, expert_out->data, (const int32_t *)pair_pos->data,
+                              (const float *)top_vals->data, out->data, out->dtype, T, H, top_k);
+}
+
 }  // extern "C"
 
 // =============================================================================

@@ -135,6 +135,15 @@ int launch_gguf_gemv(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p);
 int launch_gguf_dequant(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p, float *out_nk);
 int launch_mxfp4_gemv(oxq_ctx *ctx, hipStream_t s, const Mxfp4Problem &p);
 int launch_mxfp4_dequant(oxq_ctx *ctx, hipStream_t s, const Mxfp4Problem &p, float *out_nk);
+// mixture-of-experts glue (moe_glue.hip)
+int launch_moe_route(oxq_ctx *ctx, hipStream_t s, const void *logits, int dtype, int64_t T, int64_t E, int64_t top_k,
+                     int norm_topk, int32_t *top_idx, float *top_vals);
+int launch_moe_group(oxq_ctx *ctx, hipStream_t s, const int32_t *top_idx, const float *top_vals, int64_t P, int64_t E,
+                     int64_t top_k, int32_t *offsets, int32_t *tokens, float *weights, int32_t *pair_pos);
+int launch_gated_activation(oxq_ctx *ctx, hipStream_t s, const void *gu, void *out, int dtype, int64_t rows,
+                            int64_t half_n, int kind, float limit);
+int launch_moe_combine(oxq_ctx *ctx, hipStream_t s, const void *eo, const int32_t *pair_pos, const float *top_vals,
+                       void *out, int dtype, int64_t T, int64_t H, int64_t top_k);
 // y[M,N] = sum over S slices of ws[s][M][N] (+ bias), slices added in index order.
 int launch_splitk_reduce(oxq_ctx *ctx, hipStream_t s, const float *ws, const void *bias, void *y,
                          int64_t M, int64_t N, int S, int dtype);

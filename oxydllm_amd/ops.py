@@ -259,6 +259,57 @@ def mxfp4_moe_matmul(x, blocks, scales, bias, expert_offsets, token_ids, k: int,
     return out
 
 
+# ---------------------------------------------------------------- mixture-of-experts glue
+ACT_GATED_SILU, ACT_GATED_GELU_TANH, ACT_GPT_OSS_SWIGLU = 0, 1, 2
+
+
+def moe_route(logits, top_k: int, norm_topk: bool = True, *, ctx: Optional[Context] = None):
+    """moe.rs:466-486: softmax, stable descending top-k, optional renormalisation."""
+    ctx = _ctx(ctx)
+    T = logits.shape[0]
+    idx = torch.empty((T, top_k), dtype=torch.int32, device=logits.device)
+    vals = torch.empty((T, top_k), dtype=torch.float32, device=logits.device)
+    _lib.check(ctx._lib.oxq_moe_route(ctx.handle, ctx.stream(), desc(logits), top_k, 1 if norm_topk else 0,
+                                      desc(idx), desc(vals)))
+    return idx, vals
+
+
+def moe_group(top_idx, top_vals, n_experts: int, *, ctx: Optional[Context] = None):
+    """moe.rs:563-590: (expert_offsets [E+1], token_ids [P], pair_weights [P], pair_pos [T,k])."""
+    ctx = _ctx(ctx)
+    T, k = top_idx.shape
+    dev = top_idx.device
+    offsets = torch.empty((n_experts + 1,), dtype=torch.int32, device=dev)
+    tokens = torch.empty((T * k,), dtype=torch.int32, device=dev)
+    weights = torch.empty((T * k,), dtype=torch.float32, device=dev)
+    pos = torch.empty((T, k), dtype=torch.int32, device=dev)
+    _lib.check(ctx._lib.oxq_moe_group(ctx.handle, ctx.stream(), desc(top_idx), desc(top_vals), n_experts,
+                                      desc(offsets), desc(tokens), desc(weights), desc(pos)))
+    return offsets, tokens, weights, pos
+
+
+def gated_activation(gate_up, kind: int, limit: float = 0.0, *, out=None, ctx: Optional[Context] = None):
+    """ffn_kernels.metal gated SiLU / GeLU-tanh over [.., gate | up]; moe.rs:152-173 GPT-OSS SwiGLU."""
+    ctx = _ctx(ctx)
+    if out is None:
+        out = torch.empty(tuple(gate_up.shape[:-1]) + (gate_up.shape[-1] // 2,), dtype=gate_up.dtype,
+                          device=gate_up.device)
+    _lib.check(ctx._lib.oxq_gated_activation(ctx.handle, ctx.stream(), desc(gate_up), kind, float(limit),
+                                             desc(out)))
+    return out
+
+
+def moe_combine(expert_out, pair_pos, top_vals, *, out=None, ctx: Optional[Context] = None):
+    """moe.rs:592-605: out[t] = sum_s top_vals[t, s] * expert_out[pair_pos[t, s]]."""
+    ctx = _ctx(ctx)
+    if out is None:
+        out = torch.empty((pair_pos.shape[0], expert_out.shape[1]), dtype=expert_out.dtype,
+                          device=expert_out.device)
+    _lib.check(ctx._lib.oxq_moe_combine(ctx.handle, ctx.stream(), desc(expert_out), desc(pair_pos),
+                                        desc(top_vals), desc(out)))
+    return out
+
+
 # ---------------------------------------------------------------- layers
 class PackedQuantLinear:
     """linear.rs:403-534.  Holds resident packed weights; routes by m."""

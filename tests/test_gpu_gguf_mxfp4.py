@@ -16,7 +16,7 @@ import torch
 import oracle
 from oxydllm_amd import synth
 from tests import refgen
-from tests.helpers import as_f32, assert_close, round_x, to_dev
+from tests.helpers import RTOL, ATOL, as_f32, assert_close, round_x, to_dev
 
 pytestmark = pytest.mark.gpu
 ops = None
@@ -205,3 +205,115 @@ def test_mxfp4_moe_config4():
     ys = lay.forward(to_dev(c["x"][tokens[lo:hi]], torch.bfloat16))
     assert_close(ys, ref_gu[lo:hi], "Mxfp4Linear")
     assert torch.equal(ys, y[lo:hi])
+
+
+# ------------------------------------------------------------------ mixture-of-experts glue
+@pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,E,k,norm", [(8, 32, 4, True), (1, 128, 8, True), (70, 64, 2, False), (5, 300, 6, True)])
+def test_moe_route_matches_oracle(dt, T, E, k, norm):
+    """moe.rs:466-486.  Expert ids must agree exactly, gate values to 1e-5 relative (device expf)."""
+    say(f"moe route {dt} T={T} E={E} k={k}")
+    rng = np.random.default_rng(T * E + k)
+    logits = (rng.standard_normal((T, E)) * 2).astype(np.float32)
+    ld = to_dev(logits, dt)
+    lg = ld.float().cpu().numpy()  # what the kernel sees after the dtype cast
+    ridx, rvals = oracle.moe_route(lg, k, norm)
+    idx, vals = ops.moe_route(ld, k, norm)
+    np.testing.assert_array_equal(idx.cpu().numpy().astype(np.uint32), ridx)
+    np.testing.assert_allclose(vals.cpu().numpy(), rvals, rtol=1e-5, atol=1e-7)
+
+
+def test_moe_route_ties_keep_expert_order():
+    """Stable descending sort: equal scores keep ascending expert order (arg_sort_last_dim)."""
+    say("moe route ties")
+    logits = np.zeros((3, 16), np.float32)
+    logits[1, [5, 9, 2]] = 1.0
+    logits[2, :] = np.arange(16) % 4
+    ridx, _ = oracle.moe_route(logits, 4, True)
+    idx, _ = ops.moe_route(to_dev(logits), 4, True)
+    np.testing.assert_array_equal(idx.cpu().numpy().astype(np.uint32), ridx)
+    np.testing.assert_array_equal(ridx[0], [0, 1, 2, 3])
+
+
+@pytest.mark.parametrize("T,E,k", [(8, 32, 4), (1, 32, 4), (257, 16, 2), (1000, 256, 8)])
+def test_moe_group_matches_oracle(T, E, k):
+    """moe.rs:563-590: integer work, compared exactly."""
+    say(f"moe group T={T} E={E} k={k}")
+    rng = np.random.default_rng(T + E)
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    ridx, rvals = oracle.moe_route(logits, k, True)
+    roff, rtok, rw = oracle.moe_group(ridx, rvals, E)
+    off, tok, w, pos = ops.moe_group(to_dev(ridx.astype(np.int32)), to_dev(rvals), E)
+    np.testing.assert_array_equal(off.cpu().numpy(), roff.astype(np.int32))
+    np.testing.assert_array_equal(tok.cpu().numpy(), rtok.astype(np.int32))
+    np.testing.assert_array_equal(w.cpu().numpy(), rw)
+    pos = pos.cpu().numpy()
+    assert sorted(pos.ravel().tolist()) == list(range(T * k))
+    np.testing.assert_array_equal(rtok[pos.ravel()], np.repeat(np.arange(T), k))
+    np.testing.assert_array_equal(rw[pos.ravel()], rvals.ravel())
+
+
+@pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16, torch.float16])
+def test_gated_activations_match_oracle(dt):
+    """ffn_kernels.metal:19-242 and moe.rs:152-173: f32 math, one rounding to the tensor dtype."""
+    say(f"gated activations {dt}")
+    rng = np.random.default_rng(3)
+    gu = (rng.standard_normal((7, 2 * 96)) * 3).astype(np.float32)
+    gd = to_dev(gu, dt)
+    gr = gd.float().cpu().numpy()
+    odt = {torch.float32: None, torch.bfloat16: oracle.BF16, torch.float16: oracle.F16}[dt]
+    for kind, ref in [(ops.ACT_GATED_SILU, oracle.gated_silu(gr)), (ops.ACT_GATED_GELU_TANH, oracle.gated_gelu_tanh(gr)),
+                      (ops.ACT_GPT_OSS_SWIGLU, oracle.gpt_oss_swiglu(gr, 7.0))]:
+        y = ops.gated_activation(gd, kind, 7.0)
+        assert y.shape == (7, 96) and y.dtype == dt
+        assert_close(y, ref, f"gated act {kind} {dt}", rtol=1e-5 if odt is None else RTOL, atol=1e-5 if odt is None else ATOL,
+                     bf16_out=dt == torch.bfloat16)
+    with pytest.raises(ops.OxqError, match="2 \\* intermediate_size"):
+        ops.gated_activation(to_dev(gu[:, :191].copy(), dt), ops.ACT_GATED_SILU)
+
+
+def test_moe_step_config4_end_to_end():
+    """Benchmark config 4 as one device-side pipeline: route -> group -> gate_up -> GPT-OSS SwiGLU ->
+    down -> combine, against the oracle restating moe.rs:466-607 + 152-173 step by step (each
+    intermediate rounded to bf16 where the device stores bf16)."""
+    c = _config4()
+    E, H, I, T, k = c["E"], c["hidden"], c["inter"], c["T"], c["top_k"]
+    say("moe step end to end")
+    nb = H // 32
+    xb = round_x(c["x"], oracle.BF16)
+    gub, dnb = round_x(c["gu_bias"], oracle.BF16), round_x(c["dn_bias"], oracle.BF16)
+    ridx, rvals = oracle.moe_route(c["logits"], k, True)
+    roff, rtok, rw = oracle.moe_group(ridx, rvals, E)
+    P = T * k
+    gu_ref = np.zeros((P, 2 * I), np.float32)
+    for e in range(E):
+        lo, hi = int(roff[e]), int(roff[e + 1])
+        if hi > lo:
+            wg = oracle.dequantize_mxfp4_f32(c["gu_b"][e * 2 * I * nb * 16:(e + 1) * 2 * I * nb * 16],
+                                             c["gu_s"][e * 2 * I * nb:(e + 1) * 2 * I * nb], 2 * I, H)
+            gu_ref[lo:hi] = oracle.matmul_nt_f32(xb[rtok[lo:hi]], wg, gub[e])
+    h_ref = round_x(oracle.gpt_oss_swiglu(round_x(gu_ref, oracle.BF16), 7.0), oracle.BF16)
+    dn_ref = np.zeros((P, H), np.float32)
+    for e in range(E):
+        lo, hi = int(roff[e]), int(roff[e + 1])
+        if hi > lo:
+            wd = oracle.dequantize_mxfp4_f32(c["dn_b"][e * H * nb * 16:(e + 1) * H * nb * 16],
+                                             c["dn_s"][e * H * nb:(e + 1) * H * nb], H, I)
+            dn_ref[lo:hi] = oracle.matmul_nt_f32(h_ref[lo:hi], wd, dnb[e])
+    out_ref = oracle.moe_combine(round_x(dn_ref, oracle.BF16), roff, rtok, rw, T)
+
+    xd = to_dev(c["x"], torch.bfloat16)
+    idx, vals = ops.moe_route(to_dev(c["logits"]), k, True)
+    off, tok, w, pos = ops.moe_group(idx, vals, E)
+    np.testing.assert_array_equal(off.cpu().numpy(), roff.astype(np.int32))
+    gu = ops.mxfp4_moe_matmul(xd, to_dev(c["gu_b"]), to_dev(c["gu_s"]), to_dev(c["gu_bias"], torch.bfloat16),
+                              off, tok, H, 2 * I)
+    h = ops.gated_activation(gu, ops.ACT_GPT_OSS_SWIGLU, 7.0)
+    dn = ops.mxfp4_moe_matmul(h, to_dev(c["dn_b"]), to_dev(c["dn_s"]), to_dev(c["dn_bias"], torch.bfloat16),
+                              off, None, I, H)
+    out = ops.moe_combine(dn, pos, vals)
+    assert out.shape == (T, H) and out.dtype == torch.bfloat16
+    # three bf16 roundings sit between the oracle's and the device's intermediates: compare with the
+    # reference's own end-to-end bound (moe.rs:705-788: 1e-3 * max + 1e-3, widened for bf16 storage)
+    err = np.abs(out.float().cpu().numpy() - out_ref)
+    assert err.max() < 2e-2 * np.abs(out_ref).max() + 1e-2, err.max()

@@ -426,3 +426,37 @@ def test_gpt_oss_expert_scalar_reference():
     expected = dn_bias + wd @ hh
     tol = 1e-3 * np.max(np.abs(expected)) + 1e-3
     assert np.max(np.abs(y - expected)) < tol
+
+
+def test_gated_activations_match_scipy_and_closed_forms():
+    """ffn_kernels.metal:5-17: silu(x) = x / (1 + e^-x); gelu_tanh as the tanh approximation.
+    Checked against scipy's expit / numpy tanh in float64 and on closed forms."""
+    from scipy.special import expit
+    rng = np.random.default_rng(11)
+    gu = (rng.standard_normal((5, 64)) * 4).astype(np.float32)
+    g, u = gu[:, :32].astype(np.float64), gu[:, 32:].astype(np.float64)
+    np.testing.assert_allclose(oracle.gated_silu(gu), g * expit(g) * u, rtol=2e-6, atol=1e-6)
+    gel = 0.5 * g * (1 + np.tanh(0.7978845608028654 * (g + 0.044715 * g ** 3)))
+    np.testing.assert_allclose(oracle.gated_gelu_tanh(gu), gel * u, rtol=2e-6, atol=1e-6)
+    # closed forms: act(0) = 0; large positive gate -> gate * up; large negative -> 0
+    probe = np.array([[0.0, 30.0, -30.0, 1.0, 2.0, 3.0, 4.0, 5.0]], np.float32)  # 4 gates | 4 ups
+    for fn in (oracle.gated_silu, oracle.gated_gelu_tanh):
+        out = fn(probe)[0]
+        assert out[0] == 0.0
+        np.testing.assert_allclose(out[1], 30.0 * 3.0, rtol=1e-6)
+        assert abs(out[2]) < 1e-6
+
+
+def test_moe_combine_matches_dense_gate_matrix():
+    """moe.rs:592-605 restated: the scatter equals out = G . expert_out with the dense
+    [n_tokens, n_pairs] gate matrix (a plain matmul, computed in float64)."""
+    rng = np.random.default_rng(12)
+    T, E, k, H = 9, 16, 3, 24
+    idx, vals = oracle.moe_route(rng.standard_normal((T, E)).astype(np.float32), k, True)
+    offsets, tokens, weights = oracle.moe_group(idx, vals, E)
+    eo = rng.standard_normal((T * k, H)).astype(np.float32)
+    G = np.zeros((T, T * k))
+    for p_, (t, w_) in enumerate(zip(tokens, weights)):
+        G[t, p_] += w_
+    np.testing.assert_allclose(oracle.moe_combine(eo, offsets, tokens, weights, T), G @ eo.astype(np.float64),
+                               rtol=1e-5, atol=1e-6)
