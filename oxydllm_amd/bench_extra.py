@@ -120,4 +120,22 @@ def run(ops, ctx, stream, steps, warmup, time_graph):
     r["note"] = ("expert weights (443 MB total) are read once per step with no copy rotation: "
                  "about 290 MB of active experts exceed the memory-side cache")
     out.append(r)
+
+    # the whole MoE layer step on the device: route -> group -> gate_up -> SwiGLU -> down -> combine
+    logits_d = torch.from_numpy(logits).to(dev)
+    out_d = torch.empty((T, H), device=dev, dtype=torch.bfloat16)
+    h_d = torch.empty((n_pairs, I), device=dev, dtype=torch.bfloat16)
+
+    def full_step(i):
+        idx, vals = ops.moe_route(logits_d, top_k, True, ctx=ctx)
+        off, tok, _, pos = ops.moe_group(idx, vals, E, ctx=ctx)
+        ops.mxfp4_moe_matmul(x, gub[0], gub[1], gu_bias, off, tok, H, 2 * I, out=y_gu, ctx=ctx)
+        ops.gated_activation(y_gu, ops.ACT_GPT_OSS_SWIGLU, 7.0, out=h_d, ctx=ctx)
+        ops.mxfp4_moe_matmul(h_d, dnb[0], dnb[1], dn_bias, off, None, I, H, out=y_dn, ctx=ctx)
+        ops.moe_combine(y_dn, pos, vals, out=out_d, ctx=ctx)
+    r2 = _case(f"mxfp4 moe layer step on device: route + group + gate_up + swiglu + down + combine "
+               f"({E} experts, top-{top_k}, {T} tokens)", full_step, steps, warmup, stream, time_graph, nbytes,
+               2.0 * n_pairs * (2 * I * H + H * I), ctx)
+    r2["launches"] = 6
+    out.append(r2)
     return out
