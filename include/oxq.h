@@ -73,7 +73,13 @@ typedef enum oxq_gguf_quant {
     OXQ_GGUF_Q4_0 = 0,
     OXQ_GGUF_Q8_0 = 1,
     OXQ_GGUF_Q4_K = 2,
-    OXQ_GGUF_Q6_K = 3
+    OXQ_GGUF_Q6_K = 3,
+    OXQ_GGUF_Q4_1 = 4,
+    OXQ_GGUF_Q5_0 = 5,
+    OXQ_GGUF_Q5_1 = 6,
+    OXQ_GGUF_Q2_K = 7,
+    OXQ_GGUF_Q3_K = 8,
+    OXQ_GGUF_Q5_K = 9
 } oxq_gguf_quant;
 
 #define OXQ_MAX_RANK 4

@@ -19,8 +19,10 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "liboxq_oracle.so")
 
 F32, F16, BF16 = 0, 1, 2
-Q4_0, Q8_0, Q4_K, Q6_K = 0, 1, 2, 3
-GGUF_BLOCK_LAYOUT = {Q4_0: (32, 18), Q8_0: (32, 34), Q4_K: (256, 144), Q6_K: (256, 210)}
+Q4_0, Q8_0, Q4_K, Q6_K, Q4_1, Q5_0, Q5_1, Q2_K, Q3_K, Q5_K = range(10)
+GGUF_BLOCK_LAYOUT = {Q4_0: (32, 18), Q8_0: (32, 34), Q4_K: (256, 144), Q6_K: (256, 210),
+                     Q4_1: (32, 20), Q5_0: (32, 22), Q5_1: (32, 24), Q2_K: (256, 84),
+                     Q3_K: (256, 110), Q5_K: (256, 176)}
 
 
 def build(force: bool = False) -> str:

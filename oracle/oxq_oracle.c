@@ -15,9 +15,10 @@
  *                             (AWQ-layout 8-bit, identity slot order)
  *   orc_dequantize_gptq       src/common/awq.rs:442-590            (GPTQ 4/8-bit)
  *   orc_dequantize_mxfp4_f32  src/common/mxfp4.rs:13-64
- *   orc_dequantize_gguf       src/common/quant_kernels.metal:792-795, 1100-1103,
- *                             1228-1233, 1681-1686 (block structs) and
- *                             2342-2384, 2438-2482, 2518-2554 (formulas)
+ *   orc_dequantize_gguf       src/common/quant_kernels.metal:709-713, 792-795, 872-876,
+ *                             954-959, 1100-1103, 1228-1233, 1439-1445, 1681-1686,
+ *                             1841-1846, 2032-2037 (block structs) and 2315-2640
+ *                             (one dequant formula per format)
  *   orc_matmul_nt_f32         src/common/linear.rs:40-79  (x . W^T + bias, f32)
  *   orc_moe_route             src/common/moe.rs:466-499 + linear.rs:160-171
  *   orc_moe_group             src/common/moe.rs:563-607  (dispatch_sparse lists)
@@ -36,7 +37,7 @@
  * independent numpy restatement of the ggml block formats for GGUF.
  * GGUF has no golden vector in the reference (its tests compare against the
  * third-party candle-core 0.11.0 QTensor::dequantize, which is absent here), so
- * bit-level agreement with candle for Q4_0/Q8_0/Q4_K/Q6_K is "parity unpinned"
+ * bit-level agreement with candle for the ten block formats is "parity unpinned"
  * by fixtures; it is pinned by the public ggml block specification, which the
  * reference restates in the cited Metal strips.
  */
@@ -323,10 +324,12 @@ int orc_dequantize_mxfp4_f32(const uint8_t *blocks, size_t blocks_len, const uin
 }
 
 /* ------------------------------------------------------------------ */
-/* GGUF block formats (ggml), formats 0..3 = Q4_0, Q8_0, Q4_K, Q6_K    */
+/* GGUF block formats (ggml): 0..3 = Q4_0, Q8_0, Q4_K, Q6_K,            */
+/* 4..9 = Q4_1, Q5_0, Q5_1, Q2_K, Q3_K, Q5_K                           */
 /* ------------------------------------------------------------------ */
 
-enum { ORC_Q4_0 = 0, ORC_Q8_0 = 1, ORC_Q4_K = 2, ORC_Q6_K = 3 };
+enum { ORC_Q4_0 = 0, ORC_Q8_0 = 1, ORC_Q4_K = 2, ORC_Q6_K = 3,
+       ORC_Q4_1 = 4, ORC_Q5_0 = 5, ORC_Q5_1 = 6, ORC_Q2_K = 7, ORC_Q3_K = 8, ORC_Q5_K = 9 };
 
 int orc_gguf_block_layout(int fmt, int *elems, int *bytes) { /* metal_ops.rs:5228-5241 */
     switch (fmt) {
@@ -334,6 +337,12 @@ int orc_gguf_block_layout(int fmt, int *elems, int *bytes) { /* metal_ops.rs:522
     case ORC_Q8_0: *elems = 32; *bytes = 34; return ORC_OK;
     case ORC_Q4_K: *elems = 256; *bytes = 144; return ORC_OK;
     case ORC_Q6_K: *elems = 256; *bytes = 210; return ORC_OK;
+    case ORC_Q4_1: *elems = 32; *bytes = 20; return ORC_OK;
+    case ORC_Q5_0: *elems = 32; *bytes = 22; return ORC_OK;
+    case ORC_Q5_1: *elems = 32; *bytes = 24; return ORC_OK;
+    case ORC_Q2_K: *elems = 256; *bytes = 84; return ORC_OK;
+    case ORC_Q3_K: *elems = 256; *bytes = 110; return ORC_OK;
+    case ORC_Q5_K: *elems = 256; *bytes = 176; return ORC_OK;
     default: return ORC_ERR_ARG;
     }
 }
@@ -352,6 +361,21 @@ static inline void q4k_scale_min(int j, const uint8_t *q, uint32_t *sc, uint32_t
         *sc = (q[j + 4] & 0x0Fu) | ((uint32_t)(q[j - 4] >> 6) << 4);
         *mn = ((uint32_t)q[j + 4] >> 4) | ((uint32_t)(q[j] >> 6) << 4);
     }
+}
+
+static inline uint32_t rd_u32(const uint8_t *p) {
+    return (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16) | ((uint32_t)p[3] << 24);
+}
+
+/* quant_kernels.metal:2594-2604: signed 6-bit scale of sub-block 0..15, low four bits in
+ * scales[0..7] (nibbles), high two bits in scales[8..11], offset -32. */
+static inline int q3k_scale(int sub, const uint8_t *scales) {
+    const int k = sub % 4, group = sub / 4;
+    const int low_byte = (group < 2) ? (k + 4 * group) : (k + 4 * (group - 2));
+    const int low_shift = (group < 2) ? 0 : 4;
+    const uint32_t low = ((uint32_t)scales[low_byte] >> low_shift) & 0x0Fu;
+    const uint32_t high = ((uint32_t)scales[8 + k] >> (2 * group)) & 0x03u;
+    return (int)(low | (high << 4)) - 32;
 }
 
 static void dequant_block(int fmt, const uint8_t *blk, float *o) {
@@ -398,6 +422,76 @@ static void dequant_block(int fmt, const uint8_t *blk, float *o) {
             const int qv = (int)(nib | (hb << 4)) - 32;
             const float sc_v = d * (float)scales[8 * h + 2 * quad + l / 16];
             o[j] = sc_v * (float)qv;
+        }
+    } break;
+    case ORC_Q4_1: { /* {f16 d, m; u8 qs[16]}  quant_kernels.metal:872-876, 2386-2408 */
+        const float d = rd_f16(blk), m = rd_f16(blk + 2);
+        const uint8_t *qs = blk + 4;
+        for (int j = 0; j < 32; ++j) {
+            const uint32_t qp = (j < 16) ? (qs[j] & 0x0Fu) : (uint32_t)(qs[j - 16] >> 4);
+            o[j] = (float)qp * d + m;
+        }
+    } break;
+    case ORC_Q5_0: { /* {f16 d; u8 qh[4]; u8 qs[16]}  709-713, 2315-2340 */
+        const float d = rd_f16(blk);
+        const uint32_t qh = rd_u32(blk + 2);
+        const uint8_t *qs = blk + 6;
+        for (int j = 0; j < 32; ++j) {
+            const int hi = j / 16, jj = j % 16;
+            const uint32_t xh = ((qh >> (jj + hi * 16)) & 1u) << 4;
+            const uint32_t qp = (hi == 0) ? (qs[jj] & 0x0Fu) : (uint32_t)(qs[jj] >> 4);
+            o[j] = (float)((int)(qp | xh) - 16) * d;
+        }
+    } break;
+    case ORC_Q5_1: { /* {f16 d, m; u8 qh[4]; u8 qs[16]}  954-959, 2410-2436 */
+        const float d = rd_f16(blk), m = rd_f16(blk + 2);
+        const uint32_t qh = rd_u32(blk + 4);
+        const uint8_t *qs = blk + 8;
+        for (int j = 0; j < 32; ++j) {
+            const int hi = j / 16, jj = j % 16;
+            const uint32_t xh = ((qh >> (jj + hi * 16)) & 1u) << 4;
+            const uint32_t qp = (hi == 0) ? (qs[jj] & 0x0Fu) : (uint32_t)(qs[jj] >> 4);
+            o[j] = (float)(qp | xh) * d + m;
+        }
+    } break;
+    case ORC_Q2_K: { /* {u8 scales[16]; u8 qs[64]; f16 d, dmin}  1841-1846, 2556-2592 */
+        const uint8_t *scales = blk, *qs = blk + 16;
+        const float d = rd_f16(blk + 80), dmin = rd_f16(blk + 82);
+        for (int j = 0; j < 256; ++j) {
+            const int half = j / 128, pos = j % 128, sub = pos / 32, in_sub = pos % 32;
+            const int second = in_sub / 16, elem = in_sub % 16;
+            const uint32_t q = ((uint32_t)qs[half * 32 + second * 16 + elem] >> (2 * sub)) & 3u;
+            const uint32_t sc = scales[half * 8 + sub * 2 + second];
+            const float dl = d * (float)(sc & 0x0Fu);
+            const float ml = dmin * (float)((sc >> 4) & 0x0Fu);
+            o[j] = dl * (float)q - ml;
+        }
+    } break;
+    case ORC_Q3_K: { /* {u8 hmask[32]; u8 qs[64]; u8 scales[12]; f16 d}  2032-2037, 2594-2640 */
+        const uint8_t *hmask = blk, *qs = blk + 32, *scales = blk + 96;
+        const float d = rd_f16(blk + 108);
+        for (int j = 0; j < 256; ++j) {
+            const int half = j / 128, shift_idx = (j % 128) / 32, e = j % 32;
+            const uint32_t low2 = ((uint32_t)qs[half * 32 + e] >> (2 * shift_idx)) & 3u;
+            const uint32_t hbit = ((uint32_t)hmask[e] >> (half * 4 + shift_idx)) & 1u;
+            const int q = (int)low2 - (hbit ? 0 : 4);
+            o[j] = d * (float)q3k_scale(j / 16, scales) * (float)q;
+        }
+    } break;
+    case ORC_Q5_K: { /* {f16 d, dmin; u8 scales[12]; u8 qh[32]; u8 qs[128]}  1439-1445, 2484-2516 */
+        const float d = rd_f16(blk), dmin = rd_f16(blk + 2);
+        const uint8_t *scales = blk + 4, *qh = blk + 16, *qs = blk + 48;
+        for (int j = 0; j < 256; ++j) {
+            const int sb = j / 32, elem = j % 32;
+            uint32_t sc, mn;
+            q4k_scale_min(sb, scales, &sc, &mn);
+            const float sc_v = d * (float)sc;
+            const float m_v = dmin * (float)mn;
+            const int iq = sb / 2, lo = sb % 2;
+            const uint32_t low4 =
+                (lo == 0) ? (qs[iq * 32 + elem] & 0x0Fu) : (uint32_t)(qs[iq * 32 + elem] >> 4);
+            const uint32_t hb = ((uint32_t)qh[elem] >> (2 * iq + lo)) & 1u;
+            o[j] = sc_v * (float)(low4 | (hb << 4)) - m_v;
         }
     } break;
     }

@@ -14,7 +14,8 @@ LIB_PATH = os.path.join(HERE, "liboxq_hip.so")
 OXQ_MAX_RANK = 4
 (F32, F16, BF16, U8, I32, U32, I64) = range(7)
 PACK_OUT, PACK_IN = 0, 1
-GGUF_Q4_0, GGUF_Q8_0, GGUF_Q4_K, GGUF_Q6_K = range(4)
+(GGUF_Q4_0, GGUF_Q8_0, GGUF_Q4_K, GGUF_Q6_K, GGUF_Q4_1, GGUF_Q5_0, GGUF_Q5_1, GGUF_Q2_K, GGUF_Q3_K,
+ GGUF_Q5_K) = range(10)
 DEVICE_HOST = -1
 DEVICE_PLAN_ONLY = -1
 MFMA_MIN_M = 9

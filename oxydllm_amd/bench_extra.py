@@ -68,7 +68,7 @@ def run(ops, ctx, stream, steps, warmup, time_graph):
 
     # ---- config 3: GGUF --------------------------------------------------------
     K = N = 4096
-    for fmt in (synth.GGUF_Q4_0, synth.GGUF_Q8_0, synth.GGUF_Q4_K, synth.GGUF_Q6_K):
+    for fmt in sorted(synth.GGUF_NAMES):
         data = synth.gguf_weight(fmt, N, K, seed=0x0A0D11E8 + fmt)
         nc = _copies_for(data.nbytes, cap=48)
         d = [torch.from_numpy(data).to(dev) for _ in range(nc)]

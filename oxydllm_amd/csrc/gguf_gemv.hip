@@ -1,11 +1,10 @@
-// GGUF block-quant GEMV (Q4_0, Q8_0, Q4_K, Q6_K) over the raw ggml block bytes,
-// and the matching dense dequant.
+// GGUF block-quant GEMV (Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q2_K, Q3_K, Q4_K, Q5_K, Q6_K)
+// over the raw ggml block bytes, and the matching dense dequant.
 //
 // Reference semantics: the weight is row n = K/QK consecutive blocks
 // (linear.rs:225-240); element values follow the ggml formats as the reference
-// restates them in quant_kernels.metal:2342-2384 (Q8_0/Q4_0), 2438-2482 (Q4_K)
-// and 2518-2554 (Q6_K); y = x . W^T with f32 accumulation
-// (quant_kernels.metal:792-870, 1097-1221, 1223-1436, 1681-1838).
+// restates them in quant_kernels.metal:2315-2640 (one dequant strip per format);
+// y = x . W^T with f32 accumulation (quant_kernels.metal:709-2300, one gemv per format).
 //
 // Work unit = 32 consecutive elements of one row (a whole Q4_0/Q8_0 block, one
 // of the 8 sub-blocks of a K-quant super-block).  One wave per output row,
@@ -30,6 +29,36 @@ template <> struct GgufFmt<OXQ_GGUF_Q4_0> { static constexpr int BE = 32, BB = 1
 template <> struct GgufFmt<OXQ_GGUF_Q8_0> { static constexpr int BE = 32, BB = 34; };
 template <> struct GgufFmt<OXQ_GGUF_Q4_K> { static constexpr int BE = 256, BB = 144; };
 template <> struct GgufFmt<OXQ_GGUF_Q6_K> { static constexpr int BE = 256, BB = 210; };
+template <> struct GgufFmt<OXQ_GGUF_Q4_1> { static constexpr int BE = 32, BB = 20; };
+template <> struct GgufFmt<OXQ_GGUF_Q5_0> { static constexpr int BE = 32, BB = 22; };
+template <> struct GgufFmt<OXQ_GGUF_Q5_1> { static constexpr int BE = 32, BB = 24; };
+template <> struct GgufFmt<OXQ_GGUF_Q2_K> { static constexpr int BE = 256, BB = 84; };
+template <> struct GgufFmt<OXQ_GGUF_Q3_K> { static constexpr int BE = 256, BB = 110; };
+template <> struct GgufFmt<OXQ_GGUF_Q5_K> { static constexpr int BE = 256, BB = 176; };
+
+// get_scale_min_k4 (quant_kernels.metal:2438-2450): the 6-bit scale and minimum of
+// sub-block sb of a Q4_K / Q5_K super-block.
+__device__ __forceinline__ void k4_scale_min(const uint8_t *sc, int sb, uint32_t &scv, uint32_t &mnv) {
+    if (sb < 4) {
+        scv = sc[sb] & 63u;
+        mnv = sc[sb + 4] & 63u;
+    } else {
+        scv = (sc[sb + 4] & 0x0Fu) | ((uint32_t)(sc[sb - 4] >> 6) << 4);
+        mnv = ((uint32_t)sc[sb + 4] >> 4) | ((uint32_t)(sc[sb] >> 6) << 4);
+    }
+}
+
+// Signed 6-bit scale of sub-block `sub` (0..15) of a Q3_K super-block
+// (quant_kernels.metal:2594-2604).
+__device__ __forceinline__ int q3k_scale(const uint8_t *scales, int sub) {
+    const int k = sub & 3, group = sub >> 2;
+    const uint32_t low = ((uint32_t)scales[k + 4 * (group & 1)] >> (group < 2 ? 0 : 4)) & 0x0Fu;
+    const uint32_t high = ((uint32_t)scales[8 + k] >> (2 * group)) & 3u;
+    return (int)(low | (high << 4)) - 32;
+}
+
+// The four low bits of v, one per byte of the result (bit b -> bit 0 of byte b).
+__device__ __forceinline__ uint32_t spread4(uint32_t v) { return ((v & 0xFu) * 0x00204081u) & 0x01010101u; }
 
 // Decode unit `u` (32 elements) of the row starting at `row` into w[0..31].
 template <int FMT>
@@ -76,6 +105,87 @@ __device__ __forceinline__ void decode_unit(const uint8_t *__restrict__ row, int
             const uint32_t q = ld16(qs + 2 * i);
             w[2 * i] = sc_v * (float)((q >> sh) & 0xF) - m_v;
             w[2 * i + 1] = sc_v * (float)((q >> (8 + sh)) & 0xF) - m_v;
+        }
+    } else if constexpr (FMT == OXQ_GGUF_Q4_1) {
+        const uint8_t *p = row + (size_t)u * 20;
+        const float d = ld_f16(p), m = ld_f16(p + 2);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint32_t q = ld16(p + 4 + 2 * i);
+            w[2 * i] = (float)(q & 0xF) * d + m;
+            w[2 * i + 16] = (float)((q >> 4) & 0xF) * d + m;
+            w[2 * i + 1] = (float)((q >> 8) & 0xF) * d + m;
+            w[2 * i + 17] = (float)((q >> 12) & 0xF) * d + m;
+        }
+    } else if constexpr (FMT == OXQ_GGUF_Q5_0 || FMT == OXQ_GGUF_Q5_1) {
+        constexpr bool MIN = FMT == OXQ_GGUF_Q5_1;
+        const uint8_t *p = row + (size_t)u * (MIN ? 24 : 22);
+        const float d = ld_f16(p), m = MIN ? ld_f16(p + 2) : 0.0f;
+        const uint8_t *hp = p + (MIN ? 4 : 2);
+        const uint32_t qh = ld16(hp) | (ld16(hp + 2) << 16);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint32_t q = ld16(hp + 4 + 2 * i);
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                const int j = 2 * i + e;
+                const uint32_t lo = ((q >> (8 * e)) & 0xF) | (((qh >> j) & 1u) << 4);
+                const uint32_t hi = ((q >> (8 * e + 4)) & 0xF) | (((qh >> (j + 16)) & 1u) << 4);
+                if constexpr (MIN) {
+                    w[j] = (float)lo * d + m;
+                    w[j + 16] = (float)hi * d + m;
+                } else {
+                    w[j] = (float)((int)lo - 16) * d;
+                    w[j + 16] = (float)((int)hi - 16) * d;
+                }
+            }
+        }
+    } else if constexpr (FMT == OXQ_GGUF_Q2_K) {
+        const int b = u >> 3, ub = u & 7;
+        const uint8_t *p = row + (size_t)b * 84;
+        const float d = ld_f16(p + 80), dmin = ld_f16(p + 82);
+        const uint8_t *qs = p + 16 + (ub >> 2) * 32;
+        const int sh = (ub & 3) * 2;
+        const uint32_t sc0 = p[2 * ub], sc1 = p[2 * ub + 1];
+        const float dl0 = d * (float)(sc0 & 0xF), ml0 = dmin * (float)(sc0 >> 4);
+        const float dl1 = d * (float)(sc1 & 0xF), ml1 = dmin * (float)(sc1 >> 4);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const uint32_t q = ld16(qs + 2 * i);
+            const float dl = (i < 8) ? dl0 : dl1, ml = (i < 8) ? ml0 : ml1;
+            w[2 * i] = dl * (float)((q >> sh) & 3) - ml;
+            w[2 * i + 1] = dl * (float)((q >> (8 + sh)) & 3) - ml;
+        }
+    } else if constexpr (FMT == OXQ_GGUF_Q3_K) {
+        const int b = u >> 3, ub = u & 7;
+        const uint8_t *p = row + (size_t)b * 110;
+        const float d = ld_f16(p + 108);
+        const uint8_t *qs = p + 32 + (ub >> 2) * 32;
+        const int sh = (ub & 3) * 2;
+        const float s0 = d * (float)q3k_scale(p + 96, 2 * ub);
+        const float s1 = d * (float)q3k_scale(p + 96, 2 * ub + 1);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const uint32_t q = ld16(qs + 2 * i), hm = ld16(p + 2 * i) >> ub;
+            const float sv = (i < 8) ? s0 : s1;
+            w[2 * i] = sv * (float)((int)((q >> sh) & 3) + (int)((hm & 1) << 2) - 4);
+            w[2 * i + 1] = sv * (float)((int)((q >> (8 + sh)) & 3) + (int)(((hm >> 8) & 1) << 2) - 4);
+        }
+    } else if constexpr (FMT == OXQ_GGUF_Q5_K) {
+        const int b = u >> 3, sb = u & 7;
+        const uint8_t *p = row + (size_t)b * 176;
+        const float d = ld_f16(p), dmin = ld_f16(p + 2);
+        uint32_t scv, mnv;
+        k4_scale_min(p + 4, sb, scv, mnv);
+        const float sc_v = d * (float)scv;
+        const float m_v = dmin * (float)mnv;
+        const uint8_t *qs = p + 48 + (sb >> 1) * 32;
+        const int sh = (sb & 1) * 4;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const uint32_t q = ld16(qs + 2 * i), hb = ld16(p + 16 + 2 * i) >> sb;
+            w[2 * i] = sc_v * (float)(((q >> sh) & 0xF) | ((hb & 1) << 4)) - m_v;
+            w[2 * i + 1] = sc_v * (float)(((q >> (8 + sh)) & 0xF) | (((hb >> 8) & 1) << 4)) - m_v;
         }
     } else {  // Q6_K
         const int b = u >> 3, sub = u & 7;
@@ -235,6 +345,76 @@ __device__ __forceinline__ void unit_ints(const uint8_t *__restrict__ row, int u
         const int sh = (sb & 1) * 4;
 #pragma unroll
         for (int i = 0; i < 8; ++i) bytes_to_f32((ld32a2(qs + 4 * i) >> sh) & 0x0F0F0F0Fu, q + 4 * i);
+        a0 = a1 = d * (float)scv;
+        b0 = b1 = dmin * (float)mnv;
+    } else if constexpr (FMT == OXQ_GGUF_Q4_1) {
+        const uint8_t *p = row + (size_t)u * 20;
+        const float d = ld_f16(p), m = ld_f16(p + 2);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t w = ld32a2(p + 4 + 4 * i);
+            bytes_to_f32(w & 0x0F0F0F0Fu, q + 4 * i);
+            bytes_to_f32((w >> 4) & 0x0F0F0F0Fu, q + 16 + 4 * i);
+        }
+        a0 = a1 = d;
+        b0 = b1 = -m;
+    } else if constexpr (FMT == OXQ_GGUF_Q5_0 || FMT == OXQ_GGUF_Q5_1) {
+        constexpr bool MIN = FMT == OXQ_GGUF_Q5_1;
+        const uint8_t *p = row + (size_t)u * (MIN ? 24 : 22);
+        const float d = ld_f16(p);
+        const uint8_t *hp = p + (MIN ? 4 : 2);
+        const uint32_t qh = ld32a2(hp);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t w = ld32a2(hp + 4 + 4 * i);
+            bytes_to_f32((w & 0x0F0F0F0Fu) | (spread4(qh >> (4 * i)) << 4), q + 4 * i);
+            bytes_to_f32(((w >> 4) & 0x0F0F0F0Fu) | (spread4(qh >> (16 + 4 * i)) << 4), q + 16 + 4 * i);
+        }
+        a0 = a1 = d;
+        b0 = b1 = MIN ? -ld_f16(p + 2) : 16.0f * d;
+    } else if constexpr (FMT == OXQ_GGUF_Q2_K) {
+        const int b = u >> 3, ub = u & 7;
+        const uint8_t *p = row + (size_t)b * 84;
+        const float d = ld_f16(p + 80), dmin = ld_f16(p + 82);
+        const uint8_t *qs = p + 16 + (ub >> 2) * 32;
+        const int sh = (ub & 3) * 2;
+        const uint32_t sc = ld16(p + 2 * ub);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) bytes_to_f32((ld32a2(qs + 4 * i) >> sh) & 0x03030303u, q + 4 * i);
+        a0 = d * (float)(sc & 0xF);
+        b0 = dmin * (float)((sc >> 4) & 0xF);
+        a1 = d * (float)((sc >> 8) & 0xF);
+        b1 = dmin * (float)(sc >> 12);
+    } else if constexpr (FMT == OXQ_GGUF_Q3_K) {
+        const int b = u >> 3, ub = u & 7;
+        const uint8_t *p = row + (size_t)b * 110;
+        const float d = ld_f16(p + 108);
+        const uint8_t *qs = p + 32 + (ub >> 2) * 32;
+        const int sh = (ub & 3) * 2;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint32_t lo = (ld32a2(qs + 4 * i) >> sh) & 0x03030303u;
+            const uint32_t hi = ((ld32a2(p + 4 * i) >> ub) & 0x01010101u) << 2;
+            bytes_to_f32(lo | hi, q + 4 * i);  // q + 4
+        }
+        a0 = d * (float)q3k_scale(p + 96, 2 * ub);
+        a1 = d * (float)q3k_scale(p + 96, 2 * ub + 1);
+        b0 = 4.0f * a0;
+        b1 = 4.0f * a1;
+    } else if constexpr (FMT == OXQ_GGUF_Q5_K) {
+        const int b = u >> 3, sb = u & 7;
+        const uint8_t *p = row + (size_t)b * 176;
+        const float d = ld_f16(p), dmin = ld_f16(p + 2);
+        uint32_t scv, mnv;
+        k4_scale_min(p + 4, sb, scv, mnv);
+        const uint8_t *qs = p + 48 + (sb >> 1) * 32;
+        const int sh = (sb & 1) * 4;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint32_t lo = (ld32a2(qs + 4 * i) >> sh) & 0x0F0F0F0Fu;
+            const uint32_t hi = ((ld32a2(p + 16 + 4 * i) >> sb) & 0x01010101u) << 4;
+            bytes_to_f32(lo | hi, q + 4 * i);
+        }
         a0 = a1 = d * (float)scv;
         b0 = b1 = dmin * (float)mnv;
     } else {  // Q6_K
@@ -400,6 +580,12 @@ static const char *fmt_name(int q) {
     case OXQ_GGUF_Q4_0: return "q4_0";
     case OXQ_GGUF_Q8_0: return "q8_0";
     case OXQ_GGUF_Q4_K: return "q4k";
+    case OXQ_GGUF_Q4_1: return "q4_1";
+    case OXQ_GGUF_Q5_0: return "q5_0";
+    case OXQ_GGUF_Q5_1: return "q5_1";
+    case OXQ_GGUF_Q2_K: return "q2k";
+    case OXQ_GGUF_Q3_K: return "q3k";
+    case OXQ_GGUF_Q5_K: return "q5k";
     default: return "q6k";
     }
 }
@@ -446,12 +632,9 @@ static int launch_rows_lds(hipStream_t s, const GgufProblem &p, const uint8_t *x
 }
 
 static size_t gguf_row_bytes(int quant, int64_t K) {
-    switch (quant) {
-    case OXQ_GGUF_Q4_0: return (size_t)(K / 32) * 18;
-    case OXQ_GGUF_Q8_0: return (size_t)(K / 32) * 34;
-    case OXQ_GGUF_Q4_K: return (size_t)(K / 256) * 144;
-    default: return (size_t)(K / 256) * 210;
-    }
+    int64_t be = 0, bb = 0;
+    oxq_gguf_block_layout(quant, &be, &bb);
+    return (size_t)(K / be) * (size_t)bb;
 }
 
 int launch_gguf_gemv(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p) {
@@ -494,6 +677,12 @@ int launch_gguf_gemv(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p) {
         case OXQ_GGUF_Q4_0: OXQ_FMT(OXQ_GGUF_Q4_0); break;
         case OXQ_GGUF_Q8_0: OXQ_FMT(OXQ_GGUF_Q8_0); break;
         case OXQ_GGUF_Q4_K: OXQ_FMT(OXQ_GGUF_Q4_K); break;
+        case OXQ_GGUF_Q4_1: OXQ_FMT(OXQ_GGUF_Q4_1); break;
+        case OXQ_GGUF_Q5_0: OXQ_FMT(OXQ_GGUF_Q5_0); break;
+        case OXQ_GGUF_Q5_1: OXQ_FMT(OXQ_GGUF_Q5_1); break;
+        case OXQ_GGUF_Q2_K: OXQ_FMT(OXQ_GGUF_Q2_K); break;
+        case OXQ_GGUF_Q3_K: OXQ_FMT(OXQ_GGUF_Q3_K); break;
+        case OXQ_GGUF_Q5_K: OXQ_FMT(OXQ_GGUF_Q5_K); break;
         default: OXQ_FMT(OXQ_GGUF_Q6_K); break;
         }
 #undef OXQ_FMT
@@ -510,12 +699,21 @@ int launch_gguf_dequant(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p, float
     snprintf(name, sizeof name, "gguf_%s_dequant", fmt_name(p.quant));
     set_plan(ctx, name, grid, block, 1, 1, 0);
     if (ctx->plan_only) return OXQ_OK;
+#define OXQ_DQ(F) \
+    case F: hipLaunchKernelGGL((gguf_dequant_kernel<F>), grid, block, 0, s, p.w, out_nk, K, N); break
     switch (p.quant) {
-    case OXQ_GGUF_Q4_0: hipLaunchKernelGGL((gguf_dequant_kernel<OXQ_GGUF_Q4_0>), grid, block, 0, s, p.w, out_nk, K, N); break;
-    case OXQ_GGUF_Q8_0: hipLaunchKernelGGL((gguf_dequant_kernel<OXQ_GGUF_Q8_0>), grid, block, 0, s, p.w, out_nk, K, N); break;
-    case OXQ_GGUF_Q4_K: hipLaunchKernelGGL((gguf_dequant_kernel<OXQ_GGUF_Q4_K>), grid, block, 0, s, p.w, out_nk, K, N); break;
+        OXQ_DQ(OXQ_GGUF_Q4_0);
+        OXQ_DQ(OXQ_GGUF_Q8_0);
+        OXQ_DQ(OXQ_GGUF_Q4_K);
+        OXQ_DQ(OXQ_GGUF_Q4_1);
+        OXQ_DQ(OXQ_GGUF_Q5_0);
+        OXQ_DQ(OXQ_GGUF_Q5_1);
+        OXQ_DQ(OXQ_GGUF_Q2_K);
+        OXQ_DQ(OXQ_GGUF_Q3_K);
+        OXQ_DQ(OXQ_GGUF_Q5_K);
     default: hipLaunchKernelGGL((gguf_dequant_kernel<OXQ_GGUF_Q6_K>), grid, block, 0, s, p.w, out_nk, K, N); break;
     }
+#undef OXQ_DQ
     OXQ_HIP_CHECK(hipGetLastError());
     return OXQ_OK;
 }

@@ -234,6 +234,12 @@ static const char *gguf_name(int q) {
     case OXQ_GGUF_Q8_0: return "Q8_0";
     case OXQ_GGUF_Q4_K: return "Q4K";
     case OXQ_GGUF_Q6_K: return "Q6K";
+    case OXQ_GGUF_Q4_1: return "Q4_1";
+    case OXQ_GGUF_Q5_0: return "Q5_0";
+    case OXQ_GGUF_Q5_1: return "Q5_1";
+    case OXQ_GGUF_Q2_K: return "Q2K";
+    case OXQ_GGUF_Q3_K: return "Q3K";
+    case OXQ_GGUF_Q5_K: return "Q5K";
     default: return "?";
     }
 }
@@ -397,6 +403,12 @@ int oxq_gguf_block_layout(int quant, int64_t *block_elems, int64_t *block_bytes)
     case OXQ_GGUF_Q8_0: e = 32; b = 34; break;
     case OXQ_GGUF_Q4_K: e = 256; b = 144; break;
     case OXQ_GGUF_Q6_K: e = 256; b = 210; break;
+    case OXQ_GGUF_Q4_1: e = 32; b = 20; break;
+    case OXQ_GGUF_Q5_0: e = 32; b = 22; break;
+    case OXQ_GGUF_Q5_1: e = 32; b = 24; break;
+    case OXQ_GGUF_Q2_K: e = 256; b = 84; break;
+    case OXQ_GGUF_Q3_K: e = 256; b = 110; break;
+    case OXQ_GGUF_Q5_K: e = 256; b = 176; break;
     default: return fail(OXQ_ERR_ARG, "unknown GGUF quant %d", quant);
     }
     if (block_elems) *block_elems = e;

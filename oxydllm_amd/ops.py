@@ -15,8 +15,9 @@ from typing import Optional
 import torch
 
 from . import _lib
-from ._lib import (BF16, F16, F32, GGUF_Q4_0, GGUF_Q4_K, GGUF_Q6_K, GGUF_Q8_0, I32, I64, PACK_IN,
-                   PACK_OUT, U8, U32, OxqError, OxqPlan, OxqTensor)
+from ._lib import (BF16, F16, F32, GGUF_Q2_K, GGUF_Q3_K, GGUF_Q4_0, GGUF_Q4_1, GGUF_Q4_K, GGUF_Q5_0,
+                   GGUF_Q5_1, GGUF_Q5_K, GGUF_Q6_K, GGUF_Q8_0, I32, I64, PACK_IN, PACK_OUT, U8, U32,
+                   OxqError, OxqPlan, OxqTensor)
 
 _DTYPES = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16, torch.uint8: U8,
            torch.int32: I32, torch.int64: I64}

@@ -13,9 +13,18 @@ import numpy as np
 AWQ_PACK_ORDER = (0, 2, 4, 6, 1, 3, 5, 7)
 
 GGUF_Q4_0, GGUF_Q8_0, GGUF_Q4_K, GGUF_Q6_K = 0, 1, 2, 3
+GGUF_Q4_1, GGUF_Q5_0, GGUF_Q5_1, GGUF_Q2_K, GGUF_Q3_K, GGUF_Q5_K = 4, 5, 6, 7, 8, 9
 GGUF_BLOCK_LAYOUT = {GGUF_Q4_0: (32, 18), GGUF_Q8_0: (32, 34),
-                     GGUF_Q4_K: (256, 144), GGUF_Q6_K: (256, 210)}
-GGUF_NAMES = {GGUF_Q4_0: "Q4_0", GGUF_Q8_0: "Q8_0", GGUF_Q4_K: "Q4_K", GGUF_Q6_K: "Q6_K"}
+                     GGUF_Q4_K: (256, 144), GGUF_Q6_K: (256, 210),
+                     GGUF_Q4_1: (32, 20), GGUF_Q5_0: (32, 22), GGUF_Q5_1: (32, 24),
+                     GGUF_Q2_K: (256, 84), GGUF_Q3_K: (256, 110), GGUF_Q5_K: (256, 176)}
+GGUF_NAMES = {GGUF_Q4_0: "Q4_0", GGUF_Q8_0: "Q8_0", GGUF_Q4_K: "Q4_K", GGUF_Q6_K: "Q6_K",
+              GGUF_Q4_1: "Q4_1", GGUF_Q5_0: "Q5_0", GGUF_Q5_1: "Q5_1", GGUF_Q2_K: "Q2_K",
+              GGUF_Q3_K: "Q3_K", GGUF_Q5_K: "Q5_K"}
+# byte offsets of the f16 fields (d, then m / dmin where the format has one) in a block
+GGUF_F16_FIELDS = {GGUF_Q4_0: (0,), GGUF_Q8_0: (0,), GGUF_Q4_K: (0, 2), GGUF_Q6_K: (208,),
+                   GGUF_Q4_1: (0, 2), GGUF_Q5_0: (0,), GGUF_Q5_1: (0, 2), GGUF_Q2_K: (80, 82),
+                   GGUF_Q3_K: (108,), GGUF_Q5_K: (0, 2)}
 
 
 # ------------------------------------------------------------------ packers
@@ -113,13 +122,8 @@ def gguf_weight(fmt: int, N: int, K: int, seed: int = 0) -> np.ndarray:
     def f16_bytes(n):
         return r.uniform(1e-3, 2e-2, size=n).astype(np.float16).view(np.uint8).reshape(n, 2)
 
-    if fmt in (GGUF_Q4_0, GGUF_Q8_0):
-        blk[:, 0:2] = f16_bytes(nb)
-    elif fmt == GGUF_Q4_K:
-        blk[:, 0:2] = f16_bytes(nb)
-        blk[:, 2:4] = f16_bytes(nb)
-    else:  # Q6_K: d is the trailing half
-        blk[:, 208:210] = f16_bytes(nb)
+    for off in GGUF_F16_FIELDS[fmt]:
+        blk[:, off:off + 2] = f16_bytes(nb)
     return blk.reshape(-1)
 
 

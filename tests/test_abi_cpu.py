@@ -60,7 +60,9 @@ def test_version_and_status_names(lib):
 def test_gguf_block_layout_matches_reference(lib):
     """metal_ops.rs:5228-5241."""
     want = {_lib.GGUF_Q4_0: (32, 18), _lib.GGUF_Q8_0: (32, 34), _lib.GGUF_Q4_K: (256, 144),
-            _lib.GGUF_Q6_K: (256, 210)}
+            _lib.GGUF_Q6_K: (256, 210), _lib.GGUF_Q4_1: (32, 20), _lib.GGUF_Q5_0: (32, 22),
+            _lib.GGUF_Q5_1: (32, 24), _lib.GGUF_Q2_K: (256, 84), _lib.GGUF_Q3_K: (256, 110),
+            _lib.GGUF_Q5_K: (256, 176)}
     for q, (e, b) in want.items():
         ee, bb = C.c_int64(), C.c_int64()
         assert lib.oxq_gguf_block_layout(q, C.byref(ee), C.byref(bb)) == 0
@@ -203,7 +205,8 @@ def test_maybe_mpp_declines_like_reference(lib, ctx):
 
 def test_gguf_validation(lib, ctx):
     K, N = 4096, 4096
-    for q, (be, bb) in {_lib.GGUF_Q4_0: (32, 18), _lib.GGUF_Q6_K: (256, 210)}.items():
+    for q, (be, bb) in {_lib.GGUF_Q4_0: (32, 18), _lib.GGUF_Q6_K: (256, 210), _lib.GGUF_Q5_1: (32, 24),
+                        _lib.GGUF_Q3_K: (256, 110)}.items():
         w = fake((N * (K // be) * bb,), U8)
         x, out = fake((1, K), BF16), fake((1, N), BF16)
 

@@ -20,7 +20,7 @@ from tests.helpers import RTOL, ATOL, as_f32, assert_close, round_x, to_dev
 
 pytestmark = pytest.mark.gpu
 ops = None
-FMTS = [synth.GGUF_Q4_0, synth.GGUF_Q8_0, synth.GGUF_Q4_K, synth.GGUF_Q6_K]
+FMTS = [pytest.param(f, id=synth.GGUF_NAMES[f]) for f in sorted(synth.GGUF_NAMES)]
 
 
 def setup_module(module):
@@ -79,7 +79,7 @@ def test_gguf_gemv_batch_and_odd_n(fmt):
         assert_close(y, ref, f"gguf batch m{m}")
 
 
-@pytest.mark.parametrize("fmt", [synth.GGUF_Q4_0, synth.GGUF_Q6_K])
+@pytest.mark.parametrize("fmt", FMTS)
 @pytest.mark.parametrize("m", [9, 33, 70])
 def test_gguf_mul_mm(fmt, m):
     """metal_ops.rs:6387-6463: M in {9, 33, 70}."""
@@ -93,6 +93,21 @@ def test_gguf_mul_mm(fmt, m):
     assert_close(y, ref, f"gguf mul_mm m{m}")
     with pytest.raises(ops.OxqError, match=r"out of \[1, 8\]"):
         ops.gguf_quant_matmul(to_dev(x, torch.bfloat16), to_dev(data), K, N, fmt)
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+def test_gguf_gemv_long_rows(fmt):
+    """K = 8192 with 8 activation rows does not fit the staged variant's LDS budget: the
+    direct one-wave-per-row kernel takes over and must agree as well."""
+    N, K, m = 160, 8192, 8
+    say(f"gguf long rows {synth.GGUF_NAMES[fmt]}")
+    data = synth.gguf_weight(fmt, N, K, seed=120 + fmt)
+    w = oracle.dequantize_gguf(fmt, data, N, K)
+    x = np.random.default_rng(121).standard_normal((m, K)).astype(np.float32)
+    ref = oracle.matmul_nt_f32(round_x(x, oracle.BF16), w)
+    y = ops.gguf_quant_matmul(to_dev(x, torch.bfloat16), to_dev(data), K, N, fmt)
+    assert not ops.default_context().last_plan()["kernel"].endswith("_lds")
+    assert_close(y, ref, f"gguf long rows {synth.GGUF_NAMES[fmt]}")
 
 
 def test_qlinear_layer_bias_and_routing():

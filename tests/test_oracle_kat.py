@@ -274,11 +274,114 @@ def _ggml_q6_k(blk):
     return y
 
 
+def _ggml_q4_1(blk):
+    d, m = blk[0:4].view(np.float16).astype(np.float32)
+    qs = blk[4:20].astype(np.int32)
+    y = np.empty(32, np.float32)
+    for j in range(16):  # ggml dequantize_row_q4_1
+        y[j] = np.float32(qs[j] & 0xF) * d + m
+        y[j + 16] = np.float32(qs[j] >> 4) * d + m
+    return y
+
+
+def _ggml_q5(blk, with_min):
+    """ggml dequantize_row_q5_0 / q5_1: the fifth bit of element j is bit j of qh, of
+    element j + 16 bit j + 16 (written there as (qh >> (j + 12)) & 0x10)."""
+    off = 4 if with_min else 2
+    d = blk[0:2].view(np.float16).astype(np.float32)[0]
+    m = blk[2:4].view(np.float16).astype(np.float32)[0] if with_min else np.float32(0)
+    qh = int(blk[off:off + 4].view("<u4")[0])
+    qs = blk[off + 4:off + 20].astype(np.int32)
+    y = np.empty(32, np.float32)
+    for j in range(16):
+        xh0 = ((qh >> j) << 4) & 0x10
+        xh1 = (qh >> (j + 12)) & 0x10
+        x0, x1 = (qs[j] & 0xF) | xh0, (qs[j] >> 4) | xh1
+        if with_min:
+            y[j], y[j + 16] = np.float32(x0) * d + m, np.float32(x1) * d + m
+        else:
+            y[j], y[j + 16] = np.float32(x0 - 16) * d, np.float32(x1 - 16) * d
+    return y
+
+
+def _ggml_q2_k(blk):
+    scales = blk[0:16].astype(np.int32)
+    q = blk[16:80].astype(np.int32)
+    d, dmin = blk[80:84].view(np.float16).astype(np.float32)
+    y = []
+    is_ = 0
+    for n in range(0, 256, 128):  # ggml dequantize_row_q2_K
+        qq = q[(n // 128) * 32:]
+        shift = 0
+        for _ in range(4):
+            for off in (0, 16):
+                sc = scales[is_]
+                is_ += 1
+                dl, ml = d * np.float32(sc & 0xF), dmin * np.float32(sc >> 4)
+                y.extend(dl * ((qq[off:off + 16] >> shift) & 3).astype(np.float32) - ml)
+            shift += 2
+    return np.array(y, np.float32)
+
+
+def _ggml_q3_k(blk):
+    hm = blk[0:32].astype(np.int32)
+    q = blk[32:96].astype(np.int32)
+    d = blk[108:110].view(np.float16).astype(np.float32)[0]
+    # ggml unpacks the 12 scale bytes with three 32-bit words and two masks
+    aux = [int(v) for v in blk[96:108].view("<u4")]
+    k1, k2 = 0x03030303, 0x0F0F0F0F
+    tmp = aux[2]
+    a2 = ((aux[0] >> 4) & k2) | (((tmp >> 4) & k1) << 4)
+    a3 = ((aux[1] >> 4) & k2) | (((tmp >> 6) & k1) << 4)
+    a0 = (aux[0] & k2) | (((tmp >> 0) & k1) << 4)
+    a1 = (aux[1] & k2) | (((tmp >> 2) & k1) << 4)
+    scales = np.array([a0, a1, a2, a3], "<u4").view(np.int8).astype(np.int32)
+    y = []
+    is_, m = 0, 1
+    for n in range(0, 256, 128):  # ggml dequantize_row_q3_K
+        qq = q[(n // 128) * 32:]
+        shift = 0
+        for _ in range(4):
+            for off in (0, 16):
+                dl = d * np.float32(scales[is_] - 32)
+                is_ += 1
+                low = (qq[off:off + 16] >> shift) & 3
+                sub = np.where((hm[off:off + 16] & m) != 0, 0, 4)
+                y.extend(dl * (low - sub).astype(np.float32))
+            shift += 2
+            m <<= 1
+    return np.array(y, np.float32)
+
+
+def _ggml_q5_k(blk):
+    d, dmin = blk[0:4].view(np.float16).astype(np.float32)
+    sc = blk[4:16].astype(np.int32)
+    qh = blk[16:48].astype(np.int32)
+    ql = blk[48:176].astype(np.int32)
+    y = []
+    is_, u1, u2 = 0, 1, 2
+    for j in range(0, 256, 64):  # ggml dequantize_row_q5_K
+        s1, m1 = _k4(is_, sc)
+        s2, m2 = _k4(is_ + 1, sc)
+        d1, mm1 = d * np.float32(s1), dmin * np.float32(m1)
+        d2, mm2 = d * np.float32(s2), dmin * np.float32(m2)
+        qq = ql[(j // 64) * 32:(j // 64) * 32 + 32]
+        y.extend(d1 * ((qq & 0xF) + np.where(qh & u1, 16, 0)).astype(np.float32) - mm1)
+        y.extend(d2 * ((qq >> 4) + np.where(qh & u2, 16, 0)).astype(np.float32) - mm2)
+        is_ += 2
+        u1 <<= 2
+        u2 <<= 2
+    return np.array(y, np.float32)
+
+
 _GGML = {synth.GGUF_Q4_0: _ggml_q4_0, synth.GGUF_Q8_0: _ggml_q8_0,
-         synth.GGUF_Q4_K: _ggml_q4_k, synth.GGUF_Q6_K: _ggml_q6_k}
+         synth.GGUF_Q4_K: _ggml_q4_k, synth.GGUF_Q6_K: _ggml_q6_k,
+         synth.GGUF_Q4_1: _ggml_q4_1, synth.GGUF_Q5_0: lambda b: _ggml_q5(b, False),
+         synth.GGUF_Q5_1: lambda b: _ggml_q5(b, True), synth.GGUF_Q2_K: _ggml_q2_k,
+         synth.GGUF_Q3_K: _ggml_q3_k, synth.GGUF_Q5_K: _ggml_q5_k}
 
 
-@pytest.mark.parametrize("fmt", [synth.GGUF_Q4_0, synth.GGUF_Q8_0, synth.GGUF_Q4_K, synth.GGUF_Q6_K])
+@pytest.mark.parametrize("fmt", sorted(_GGML))
 def test_gguf_dequant_matches_ggml_row_loops(fmt):
     """Block formats per the public ggml spec, walked the way ggml's own
     dequantize_row_* loops walk them (not the per-element index formula)."""
@@ -320,6 +423,84 @@ def test_gguf_closed_forms():
     df = d.astype(np.float32)[0]
     assert np.all(out[0:32] == df * 1 * 1) and np.all(out[32:64] == df * 2 * 2)
     assert np.all(out[64:96] == df * 3 * 1) and np.all(out[96:128] == df * 4 * 2)
+    assert np.all(out[128:] == 0)
+
+
+def test_gguf_closed_forms_more_formats():
+    """One element set at a time: which bit of which byte lands on which element, and the
+    scale that multiplies it, read off the block layouts without the index formulas."""
+    d = np.array([0.5], np.float16)
+    mn = np.array([0.25], np.float16)
+    # Q4_1: byte 3 = 0xA7 -> element 3 = 7 d + m, element 19 = 10 d + m, the rest m
+    blk = np.zeros(20, np.uint8)
+    blk[0:2], blk[2:4], blk[4 + 3] = d.view(np.uint8), mn.view(np.uint8), 0xA7
+    out = oracle.dequantize_gguf(oracle.Q4_1, blk, 1, 32)[0]
+    want = np.full(32, 0.25, np.float32)
+    want[3], want[19] = 3.75, 5.25
+    np.testing.assert_array_equal(out, want)
+    # Q5_0: only qh bit 5 and bit 21 set -> elements 5 and 21 are (16 - 16) d = 0, the rest -16 d
+    blk = np.zeros(22, np.uint8)
+    blk[0:2] = d.view(np.uint8)
+    blk[2:6] = np.array([(1 << 5) | (1 << 21)], "<u4").view(np.uint8)
+    out = oracle.dequantize_gguf(oracle.Q5_0, blk, 1, 32)[0]
+    want = np.full(32, -8.0, np.float32)
+    want[5] = want[21] = 0.0
+    np.testing.assert_array_equal(out, want)
+    # Q5_1: qh bit 31, qs[15] = 0xF0 -> element 31 = 31 d + m
+    blk = np.zeros(24, np.uint8)
+    blk[0:2], blk[2:4] = d.view(np.uint8), mn.view(np.uint8)
+    blk[4:8] = np.array([1 << 31], "<u4").view(np.uint8)
+    blk[8 + 15] = 0xF0
+    out = oracle.dequantize_gguf(oracle.Q5_1, blk, 1, 32)[0]
+    want = np.full(32, 0.25, np.float32)
+    want[31] = 31 * 0.5 + 0.25
+    np.testing.assert_array_equal(out, want)
+    # Q2_K: scales[i] = (i << 4) | (15 - i): sub-block i of 16 elements has dl = d (15 - i),
+    # ml = dmin i; all quants 3 (qs = 0xFF) -> 3 dl - ml
+    blk = np.zeros(84, np.uint8)
+    blk[0:16] = [(i << 4) | (15 - i) for i in range(16)]
+    blk[16:80] = 0xFF
+    blk[80:82], blk[82:84] = d.view(np.uint8), mn.view(np.uint8)
+    out = oracle.dequantize_gguf(oracle.Q2_K, blk, 1, 256)[0]
+    for j in range(256):
+        i = j // 16
+        assert out[j] == np.float32(3 * 0.5 * (15 - i) - 0.25 * i)
+    # Q2_K bit placement: qs[32 + 16 + 2] = 0b01_00_10_11 -> elements 128 + 32 s + 18 = 3, 2, 0, 1
+    blk[0:16] = 1  # dl = d, ml = 0
+    blk[16:80] = 0
+    blk[16 + 32 + 16 + 2] = 0b01001011
+    out = oracle.dequantize_gguf(oracle.Q2_K, blk, 1, 256)[0]
+    want = np.zeros(256, np.float32)
+    want[[128 + 18, 160 + 18, 192 + 18, 224 + 18]] = [1.5, 1.0, 0.0, 0.5]
+    np.testing.assert_array_equal(out, want)
+    # Q3_K: all scale bits zero -> scale -32; hmask all ones, qs = 0 except one byte
+    blk = np.zeros(110, np.uint8)
+    blk[0:32] = 0xFF
+    blk[32 + 32 + 7] = 0b11100100  # second half, element 7: q = 0, 1, 2, 3 at shifts 0, 2, 4, 6
+    blk[108:110] = d.view(np.uint8)
+    out = oracle.dequantize_gguf(oracle.Q3_K, blk, 1, 256)[0]
+    want = np.zeros(256, np.float32)
+    want[[128 + 7, 160 + 7, 192 + 7, 224 + 7]] = np.float32(-16.0) * np.array([0, 1, 2, 3], np.float32)
+    np.testing.assert_array_equal(out, want)
+    # Q3_K: hmask bit clear subtracts 4; six-bit scale assembled from its two places:
+    # sub-block 9 (group 2, k 1): low nibble = scales[1] >> 4, high bits = (scales[9] >> 4) & 3
+    blk = np.zeros(110, np.uint8)
+    blk[96 + 1] = 0x50        # low nibble of sub-blocks 1 (0) and 9 (5)
+    blk[96 + 8 + 1] = 0x20    # high bits of sub-block 9 = 2 -> scale = 5 + 32 - 32 = 5
+    blk[108:110] = d.view(np.uint8)
+    out = oracle.dequantize_gguf(oracle.Q3_K, blk, 1, 256)[0]
+    np.testing.assert_array_equal(out[144:160], np.full(16, 0.5 * 5 * -4, np.float32))
+    np.testing.assert_array_equal(out[16:32], np.full(16, 0.5 * -32 * -4, np.float32))
+    # Q5_K: sc = j + 1 (j < 4), min = 0; qs = 0x21; qh = 0b0110: bit 1 and 2 set ->
+    # sub-block 1 (high nibble 2) gets +16, sub-block 2 (low nibble 1) gets +16
+    blk = np.zeros(176, np.uint8)
+    blk[0:2], blk[2:4] = d.view(np.uint8), d.view(np.uint8)
+    blk[4:8] = [1, 2, 3, 4]
+    blk[16:48] = 0b0110
+    blk[48:176] = 0x21
+    out = oracle.dequantize_gguf(oracle.Q5_K, blk, 1, 256)[0]
+    assert np.all(out[0:32] == 0.5 * 1 * 1) and np.all(out[32:64] == 0.5 * 2 * 18)
+    assert np.all(out[64:96] == 0.5 * 3 * 17) and np.all(out[96:128] == 0.5 * 4 * 2)
     assert np.all(out[128:] == 0)
 
 
