@@ -79,6 +79,16 @@ def run(ops, ctx, stream, steps, warmup, time_graph):
             ops.gguf_quant_matmul(x, d[i % nc], K, N, fmt, out=y, ctx=ctx)
         out.append(_case(f"gguf {synth.GGUF_NAMES[fmt]} M=1 K={K} N={N} f32", step, steps, warmup, stream,
                          time_graph, data.nbytes + K * 4 + N * 4, 2.0 * K * N, ctx))
+        if fmt in (synth.GGUF_Q4_0, synth.GGUF_Q4_K, synth.GGUF_Q6_K, synth.GGUF_Q8_0):
+            for m in (64, 512, 2048):  # prefill: the tile matmul, bf16
+                xb = torch.randn((m, K), device=dev, dtype=torch.bfloat16)
+                yb = torch.empty((m, N), device=dev, dtype=torch.bfloat16)
+
+                def mstep(i, d=d, nc=nc, fmt=fmt, x=xb, y=yb):
+                    ops.gguf_quant_mul_mm(x, d[i % nc], K, N, fmt, out=y, ctx=ctx)
+                out.append(_case(f"gguf {synth.GGUF_NAMES[fmt]} M={m} K={K} N={N} bf16 mul_mm", mstep, steps,
+                                 warmup, stream, time_graph, data.nbytes + m * K * 2 + m * N * 2,
+                                 2.0 * m * K * N, ctx))
         del d
 
     # ---- config 4: MXFP4 MoE -----------------------------------------------------

@@ -1,0 +1,207 @@
+// Decoders of the ggml block formats shared by the GGUF kernels: unit `u` (32 consecutive
+// elements of one weight row) -> 32 floats, each computed exactly as the reference's
+// dequant strips compute it (quant_kernels.metal:2315-2640, one strip per format; block
+// structs at 709-713, 792-795, 872-876, 954-959, 1100-1103, 1228-1233, 1439-1445,
+// 1681-1686, 1841-1846, 2032-2037).  All field offsets inside a block are even, so bytes
+// are fetched as 16-bit words.
+#pragma once
+
+#include "oxq_device.hpp"
+#include "oxq_internal.hpp"
+
+namespace oxq {
+
+__device__ __forceinline__ uint32_t ld16(const uint8_t *p) { return *(const uint16_t *)p; }
+__device__ __forceinline__ float ld_f16(const uint8_t *p) {
+    return (float)__builtin_bit_cast(_Float16, *(const uint16_t *)p);
+}
+
+template <int FMT> struct GgufFmt;
+template <> struct GgufFmt<OXQ_GGUF_Q4_0> { static constexpr int BE = 32, BB = 18; };
+template <> struct GgufFmt<OXQ_GGUF_Q8_0> { static constexpr int BE = 32, BB = 34; };
+template <> struct GgufFmt<OXQ_GGUF_Q4_K> { static constexpr int BE = 256, BB = 144; };
+template <> struct GgufFmt<OXQ_GGUF_Q6_K> { static constexpr int BE = 256, BB = 210; };
+template <> struct GgufFmt<OXQ_GGUF_Q4_1> { static constexpr int BE = 32, BB = 20; };
+template <> struct GgufFmt<OXQ_GGUF_Q5_0> { static constexpr int BE = 32, BB = 22; };
+template <> struct GgufFmt<OXQ_GGUF_Q5_1> { static constexpr int BE = 32, BB = 24; };
+template <> struct GgufFmt<OXQ_GGUF_Q2_K> { static constexpr int BE = 256, BB = 84; };
+template <> struct GgufFmt<OXQ_GGUF_Q3_K> { static constexpr int BE = 256, BB = 110; };
+template <> struct GgufFmt<OXQ_GGUF_Q5_K> { static constexpr int BE = 256, BB = 176; };
+
+// get_scale_min_k4 (quant_kernels.metal:2438-2450): the 6-bit scale and minimum of
+// sub-block sb of a Q4_K / Q5_K super-block.
+__device__ __forceinline__ void k4_scale_min(const uint8_t *sc, int sb, uint32_t &scv, uint32_t &mnv) {
+    if (sb < 4) {
+        scv = sc[sb] & 63u;
+        mnv = sc[sb + 4] & 63u;
+    } else {
+        scv = (sc[sb + 4] & 0x0Fu) | ((uint32_t)(sc[sb - 4] >> 6) << 4);
+        mnv = ((uint32_t)sc[sb + 4] >> 4) | ((uint32_t)(sc[sb] >> 6) << 4);
+    }
+}
+
+// Signed 6-bit scale of sub-block `sub` (0..15) of a Q3_K super-block
+// (quant_kernels.metal:2594-2604).
+__device__ __forceinline__ int q3k_scale(const uint8_t *scales, int sub) {
+    const int k = sub & 3, group = sub >> 2;
+    const uint32_t low = ((uint32_t)scales[k + 4 * (group & 1)] >> (group < 2 ? 0 : 4)) & 0x0Fu;
+    const uint32_t high = ((uint32_t)scales[8 + k] >> (2 * group)) & 3u;
+    return (int)(low | (high << 4)) - 32;
+}
+
+// The four low bits of v, one per byte of the result (bit b -> bit 0 of byte b).
+__device__ __forceinline__ uint32_t spread4(uint32_t v) { return ((v & 0xFu) * 0x00204081u) & 0x01010101u; }
+
+// Decode unit `u` (32 elements) of the row starting at `row` into w[0..31].
+template <int FMT>
+__device__ __forceinline__ void decode_unit(const uint8_t *__restrict__ row, int u, float w[32]) {
+    if constexpr (FMT == OXQ_GGUF_Q4_0) {
+        const uint8_t *p = row + (size_t)u * 18;
+        const float d = ld_f16(p);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint32_t q = ld16(p + 2 + 2 * i);  // bytes 2i, 2i+1
+            w[2 * i] = (float)((int)(q & 0xF) - 8) * d;
+            w[2 * i + 16] = (float)((int)((q >> 4) & 0xF) - 8) * d;
+            w[2 * i + 1] = (float)((int)((q >> 8) & 0xF) - 8) * d;
+            w[2 * i + 17] = (float)((int)((q >> 12) & 0xF) - 8) * d;
+        }
+    } else if constexpr (FMT == OXQ_GGUF_Q8_0) {
+        const uint8_t *p = row + (size_t)u * 34;
+        const float d = ld_f16(p);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const uint32_t q = ld16(p + 2 + 2 * i);
+            w[2 * i] = (float)(int)(int8_t)(q & 0xFF) * d;
+            w[2 * i + 1] = (float)(int)(int8_t)(q >> 8) * d;
+        }
+    } else if constexpr (FMT == OXQ_GGUF_Q4_K) {
+        const int b = u >> 3, sb = u & 7;
+        const uint8_t *p = row + (size_t)b * 144;
+        const float d = ld_f16(p), dmin = ld_f16(p + 2);
+        const uint8_t *sc = p + 4;
+        uint32_t scv, mnv;
+        if (sb < 4) {  // get_scale_min_k4
+            scv = sc[sb] & 63u;
+            mnv = sc[sb + 4] & 63u;
+        } else {
+            scv = (sc[sb + 4] & 0x0Fu) | ((uint32_t)(sc[sb - 4] >> 6) << 4);
+            mnv = ((uint32_t)sc[sb + 4] >> 4) | ((uint32_t)(sc[sb] >> 6) << 4);
+        }
+        const float sc_v = d * (float)scv;
+        const float m_v = dmin * (float)mnv;
+        const uint8_t *qs = p + 16 + (sb >> 1) * 32;
+        const int sh = (sb & 1) * 4;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const uint32_t q = ld16(qs + 2 * i);
+            w[2 * i] = sc_v * (float)((q >> sh) & 0xF) - m_v;
+            w[2 * i + 1] = sc_v * (float)((q >> (8 + sh)) & 0xF) - m_v;
+        }
+    } else if constexpr (FMT == OXQ_GGUF_Q4_1) {
+        const uint8_t *p = row + (size_t)u * 20;
+        const float d = ld_f16(p), m = ld_f16(p + 2);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint32_t q = ld16(p + 4 + 2 * i);
+            w[2 * i] = (float)(q & 0xF) * d + m;
+            w[2 * i + 16] = (float)((q >> 4) & 0xF) * d + m;
+            w[2 * i + 1] = (float)((q >> 8) & 0xF) * d + m;
+            w[2 * i + 17] = (float)((q >> 12) & 0xF) * d + m;
+        }
+    } else if constexpr (FMT == OXQ_GGUF_Q5_0 || FMT == OXQ_GGUF_Q5_1) {
+        constexpr bool MIN = FMT == OXQ_GGUF_Q5_1;
+        const uint8_t *p = row + (size_t)u * (MIN ? 24 : 22);
+        const float d = ld_f16(p), m = MIN ? ld_f16(p + 2) : 0.0f;
+        const uint8_t *hp = p + (MIN ? 4 : 2);
+        const uint32_t qh = ld16(hp) | (ld16(hp + 2) << 16);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint32_t q = ld16(hp + 4 + 2 * i);
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                const int j = 2 * i + e;
+                const uint32_t lo = ((q >> (8 * e)) & 0xF) | (((qh >> j) & 1u) << 4);
+                const uint32_t hi = ((q >> (8 * e + 4)) & 0xF) | (((qh >> (j + 16)) & 1u) << 4);
+                if constexpr (MIN) {
+                    w[j] = (float)lo * d + m;
+                    w[j + 16] = (float)hi * d + m;
+                } else {
+                    w[j] = (float)((int)lo - 16) * d;
+                    w[j + 16] = (float)((int)hi - 16) * d;
+                }
+            }
+        }
+    } else if constexpr (FMT == OXQ_GGUF_Q2_K) {
+        const int b = u >> 3, ub = u & 7;
+        const uint8_t *p = row + (size_t)b * 84;
+        const float d = ld_f16(p + 80), dmin = ld_f16(p + 82);
+        const uint8_t *qs = p + 16 + (ub >> 2) * 32;
+        const int sh = (ub & 3) * 2;
+        const uint32_t sc0 = p[2 * ub], sc1 = p[2 * ub + 1];
+        const float dl0 = d * (float)(sc0 & 0xF), ml0 = dmin * (float)(sc0 >> 4);
+        const float dl1 = d * (float)(sc1 & 0xF), ml1 = dmin * (float)(sc1 >> 4);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const uint32_t q = ld16(qs + 2 * i);
+            const float dl = (i < 8) ? dl0 : dl1, ml = (i < 8) ? ml0 : ml1;
+            w[2 * i] = dl * (float)((q >> sh) & 3) - ml;
+            w[2 * i + 1] = dl * (float)((q >> (8 + sh)) & 3) - ml;
+        }
+    } else if constexpr (FMT == OXQ_GGUF_Q3_K) {
+        const int b = u >> 3, ub = u & 7;
+        const uint8_t *p = row + (size_t)b * 110;
+        const float d = ld_f16(p + 108);
+        const uint8_t *qs = p + 32 + (ub >> 2) * 32;
+        const int sh = (ub & 3) * 2;
+        const float s0 = d * (float)q3k_scale(p + 96, 2 * ub);
+        const float s1 = d * (float)q3k_scale(p + 96, 2 * ub + 1);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const uint32_t q = ld16(qs + 2 * i), hm = ld16(p + 2 * i) >> ub;
+            const float sv = (i < 8) ? s0 : s1;
+            w[2 * i] = sv * (float)((int)((q >> sh) & 3) + (int)((hm & 1) << 2) - 4);
+            w[2 * i + 1] = sv * (float)((int)((q >> (8 + sh)) & 3) + (int)(((hm >> 8) & 1) << 2) - 4);
+        }
+    } else if constexpr (FMT == OXQ_GGUF_Q5_K) {
+        const int b = u >> 3, sb = u & 7;
+        const uint8_t *p = row + (size_t)b * 176;
+        const float d = ld_f16(p), dmin = ld_f16(p + 2);
+        uint32_t scv, mnv;
+        k4_scale_min(p + 4, sb, scv, mnv);
+        const float sc_v = d * (float)scv;
+        const float m_v = dmin * (float)mnv;
+        const uint8_t *qs = p + 48 + (sb >> 1) * 32;
+        const int sh = (sb & 1) * 4;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const uint32_t q = ld16(qs + 2 * i), hb = ld16(p + 16 + 2 * i) >> sb;
+            w[2 * i] = sc_v * (float)(((q >> sh) & 0xF) | ((hb & 1) << 4)) - m_v;
+            w[2 * i + 1] = sc_v * (float)(((q >> (8 + sh)) & 0xF) | (((hb >> 8) & 1) << 4)) - m_v;
+        }
+    } else {  // Q6_K
+        const int b = u >> 3, sub = u & 7;
+        const int h = sub >> 2, quad = sub & 3;
+        const uint8_t *p = row + (size_t)b * 210;
+        const uint8_t *ql = p + 64 * h + (quad & 1) * 32;
+        const uint8_t *qh = p + 128 + 32 * h;
+        const int8_t *scales = (const int8_t *)(p + 192);
+        const float d = ld_f16(p + 208);
+        const float s0 = d * (float)scales[8 * h + 2 * quad];
+        const float s1 = d * (float)scales[8 * h + 2 * quad + 1];
+        const int shl = (quad < 2) ? 0 : 4;
+        const int shh = 2 * quad;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const uint32_t l16 = ld16(ql + 2 * i);
+            const uint32_t h16 = ld16(qh + 2 * i);
+            const int q0 = (int)(((l16 >> shl) & 0xF) | (((h16 >> shh) & 3) << 4)) - 32;
+            const int q1 = (int)(((l16 >> (8 + shl)) & 0xF) | (((h16 >> (8 + shh)) & 3) << 4)) - 32;
+            const float sv = (i < 8) ? s0 : s1;  // elements 0..15 / 16..31
+            w[2 * i] = sv * (float)q0;
+            w[2 * i + 1] = sv * (float)q1;
+        }
+    }
+}
+
+}  // namespace oxq

@@ -582,6 +582,7 @@ int oxq_gguf_quant_mul_mm(oxq_ctx *ctx, void *stream, const oxq_tensor *x,
     GgufProblem p;
     OXQ_TRY(check_gguf(ctx, "GgufQuantMulMM", false, false, x, weight_bytes, in_features,
                        out_features, quant, out, &p));
+    if (gguf_mm_eligible(p)) return launch_gguf_mm(ctx, (hipStream_t)stream, p);
     return launch_gguf_gemv(ctx, (hipStream_t)stream, p);
 }
 
@@ -1091,6 +1092,7 @@ int oxq_qlinear_forward(oxq_qlinear *l, void *stream, const oxq_tensor *x, const
     OXQ_TRY(check_gguf(l->ctx, decode ? "GgufQuantMatmul" : "GgufQuantMulMM", decode, false, &x2,
                        &l->weight_bytes, l->in_features, l->out_features, l->quant, &o2, &p));
     p.bias = l->has_bias ? l->bias.data : nullptr;
+    if (gguf_mm_eligible(p)) return launch_gguf_mm(l->ctx, (hipStream_t)stream, p);
     return launch_gguf_gemv(l->ctx, (hipStream_t)stream, p);
 }
 

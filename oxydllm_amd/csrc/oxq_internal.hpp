@@ -133,6 +133,9 @@ int launch_wna16_mfma(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p);
 int launch_wna16_dequant(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p, void *out_kn);
 int launch_gguf_gemv(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p);
 int launch_gguf_dequant(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p, float *out_nk);
+// m > 8, bf16: tile matmul on the matrix cores (weights rounded to bf16 as the reference's mul_mm does)
+bool gguf_mm_eligible(const GgufProblem &p);
+int launch_gguf_mm(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p);
 int launch_mxfp4_gemv(oxq_ctx *ctx, hipStream_t s, const Mxfp4Problem &p);
 int launch_mxfp4_dequant(oxq_ctx *ctx, hipStream_t s, const Mxfp4Problem &p, float *out_nk);
 // mixture-of-experts glue (moe_glue.hip)

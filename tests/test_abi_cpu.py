@@ -303,11 +303,11 @@ def test_layers_validate_like_reference(lib, ctx):
     q = C.c_void_p()
     w = fake((4096 * 16 * 144,), U8)
     assert lib.oxq_qlinear_new(ctx, _lib.GGUF_Q4_K, C.byref(w), 4096, 4096, None, BF16, C.byref(q)) == 0
-    for m_rows, kern in [(1, "gguf_q4k_gemv_bf16"), (8, "gguf_q4k_gemv_bf16"), (33, "gguf_q4k_gemv_bf16")]:
+    for m_rows, kern in [(1, "gguf_q4k_gemv_bf16"), (8, "gguf_q4k_gemv_bf16"), (33, "gguf_q4k_mul_mm_bf16")]:
         assert lib.oxq_qlinear_forward(q, None, C.byref(fake((m_rows, 4096), BF16)),
                                        C.byref(fake((m_rows, 4096), BF16))) == 0, err(lib)
         p = plan(lib, ctx)
-        assert p.kernel.decode().startswith(kern) and p.launches == (m_rows + 7) // 8
+        assert p.kernel.decode().startswith(kern) and p.launches == (2 if p.split_k > 1 else 1)
     lib.oxq_qlinear_free(q)
     assert lib.oxq_qlinear_new(ctx, _lib.GGUF_Q4_K, C.byref(w), 4096, 4095, None, BF16, C.byref(q)) == -3
 

@@ -79,6 +79,17 @@ def test_gguf_gemv_batch_and_odd_n(fmt):
         assert_close(y, ref, f"gguf batch m{m}")
 
 
+def _check_mul_mm(y, x, w, what, bias=None):
+    """The tile matmul rounds every dequantized weight to bf16 before the matrix unit
+    (quant_kernels.metal:2315-2640 write `(bfloat)` tiles): 2e-3 / 1e-2 against that, and the
+    reference's own bound (metal_ops.rs:6449-6461) against the unrounded weights."""
+    xr = round_x(x, oracle.BF16)
+    tile = oracle.matmul_nt_f32(xr, oracle.round_through(w, oracle.BF16), bias)
+    assert_close(y, tile, what + " vs bf16-tile oracle", bf16_out=True)
+    ref = oracle.matmul_nt_f32(xr, w, bias)
+    assert np.abs(as_f32(y) - ref).max() < 0.06 * np.abs(ref).max() + 1e-2
+
+
 @pytest.mark.parametrize("fmt", FMTS)
 @pytest.mark.parametrize("m", [9, 33, 70])
 def test_gguf_mul_mm(fmt, m):
@@ -88,11 +99,52 @@ def test_gguf_mul_mm(fmt, m):
     data = synth.gguf_weight(fmt, N, K, seed=80 + fmt)
     w = oracle.dequantize_gguf(fmt, data, N, K)
     x = np.random.default_rng(90 + m).standard_normal((m, K)).astype(np.float32)
-    ref = oracle.matmul_nt_f32(round_x(x, oracle.BF16), w)
     y = ops.gguf_quant_mul_mm(to_dev(x, torch.bfloat16), to_dev(data), K, N, fmt)
-    assert_close(y, ref, f"gguf mul_mm m{m}")
+    assert "mul_mm" in ops.default_context().last_plan()["kernel"]
+    _check_mul_mm(y, x, w, f"gguf mul_mm m{m}")
     with pytest.raises(ops.OxqError, match=r"out of \[1, 8\]"):
         ops.gguf_quant_matmul(to_dev(x, torch.bfloat16), to_dev(data), K, N, fmt)
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+@pytest.mark.parametrize("mt,ks", [(4, 1), (1, 1), (2, 1), (4, 3), (2, 5), (1, 2)])
+def test_gguf_mul_mm_ragged(fmt, mt, ks, monkeypatch):
+    """Odd N (1001: partial row tile, unaligned output rows and a tensor whose last 16-byte
+    chunk is partial; 1000 where K is split, which needs N % 4 == 0), m = 150 (token tiles
+    with a partial last one), and for the 32-element formats a K that is not a multiple of the
+    256-element stage.  The launcher picks tokens per tile and K slices from the grid size;
+    every choice is forced over the same ragged shape."""
+    elems, _ = synth.GGUF_BLOCK_LAYOUT[fmt]
+    N, K, m = (1001 if ks == 1 else 1000), (1024 if elems == 256 else 1120), 150
+    say(f"gguf mul_mm ragged {synth.GGUF_NAMES[fmt]} K={K} N={N} mt {mt} ks {ks}")
+    monkeypatch.setenv("OXQ_GGUF_MM_MT", str(mt))
+    monkeypatch.setenv("OXQ_GGUF_MM_KS", str(ks))
+    data = synth.gguf_weight(fmt, N, K, seed=130 + fmt)
+    w = oracle.dequantize_gguf(fmt, data, N, K)
+    x = np.random.default_rng(131).standard_normal((m, K)).astype(np.float32)
+    bias = np.linspace(-2, 2, N).astype(np.float32)
+    layer = ops.QLinear(fmt, to_dev(data), K, N, to_dev(bias, torch.bfloat16), torch.bfloat16)
+    y = layer.forward(to_dev(x, torch.bfloat16))
+    plan = ops.default_context().last_plan()
+    stages = -(-K // 256)
+    per_slice = -(-stages // min(ks, stages))
+    slices = -(-stages // per_slice)
+    assert plan["kernel"].endswith(f"mul_mm_bf16_mt{mt}") and plan["split_k"] == slices
+    assert plan["launches"] == (2 if slices > 1 else 1)
+    _check_mul_mm(y, x, w, f"gguf mul_mm ragged {synth.GGUF_NAMES[fmt]}", round_x(bias, oracle.BF16))
+    y2 = layer.forward(to_dev(x, torch.bfloat16))
+    assert torch.equal(y.view(torch.int16), y2.view(torch.int16))
+
+
+def test_gguf_mul_mm_f32_activations_keep_f32_weights():
+    """f32 activations (the reference's CPU contract) never round the weights."""
+    fmt, N, K, m = synth.GGUF_Q4_K, 96, 512, 20
+    say("gguf mul_mm f32")
+    data = synth.gguf_weight(fmt, N, K, seed=140)
+    w = oracle.dequantize_gguf(fmt, data, N, K)
+    x = np.random.default_rng(141).standard_normal((m, K)).astype(np.float32)
+    y = ops.gguf_quant_mul_mm(to_dev(x), to_dev(data), K, N, fmt)
+    assert_close(y, oracle.matmul_nt_f32(x, w), "gguf mul_mm f32")
 
 
 @pytest.mark.parametrize("fmt", FMTS)
@@ -123,8 +175,11 @@ def test_qlinear_layer_bias_and_routing():
         x = np.random.default_rng(m).standard_normal((m, K)).astype(np.float32)
         y = layer.forward(to_dev(x.reshape(shape), torch.bfloat16))
         assert tuple(y.shape) == shape[:-1] + (N,)
-        ref = oracle.matmul_nt_f32(round_x(x, oracle.BF16), w, round_x(bias, oracle.BF16))
-        assert_close(y.reshape(m, N), ref, f"QLinear {shape}")
+        if m <= 8:
+            ref = oracle.matmul_nt_f32(round_x(x, oracle.BF16), w, round_x(bias, oracle.BF16))
+            assert_close(y.reshape(m, N), ref, f"QLinear {shape}")
+        else:  # prefill: the tile matmul
+            _check_mul_mm(y.reshape(m, N), x, w, f"QLinear {shape}", round_x(bias, oracle.BF16))
 
 
 # ------------------------------------------------------------------ MXFP4
