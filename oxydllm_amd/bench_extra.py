@@ -1,8 +1,9 @@
 """Timings of the other benchmark configurations (`bench.py --all`).
 
 GPTQ 4/8-bit GEMV (K=5120, N=13824, g=128, M in {1, 8}); GGUF Q4_0 / Q8_0 / Q4_K /
-Q6_K GEMV (M=1, K=N=4096, f32 activations); MXFP4 MoE expert GEMV (32 experts,
-top-4, 8 tokens, hidden 2880, gate_up N=5760, down K=2880).  Every case rotates
+Q6_K ... GEMV (M=1, K=N=4096, f32 activations) and tile matmul (M=64..2048, bf16); MXFP4
+MoE expert GEMV (32 experts, top-4, 8 tokens, hidden 2880, gate_up N=5760, down K=2880),
+the same layer at 512 tokens, and one expert's gate_up at prefill sizes.  Every case rotates
 over enough weight copies to exceed the 256 MB memory-side cache and replays a
 HIP graph of `steps` launches.  Returns a list of dicts (GB/s of algorithmic
 bytes, TFLOP/s, fraction of the 8 TB/s HBM peak).
@@ -148,4 +149,36 @@ def run(ops, ctx, stream, steps, warmup, time_graph):
                2.0 * n_pairs * (2 * I * H + H * I), ctx)
     r2["launches"] = 6
     out.append(r2)
+
+    # prefill: one expert's gate_up as a plain layer, and a 512-token MoE layer step
+    for m in (64, 256, 1024):
+        xm = torch.randn((m, H), device=dev, dtype=torch.bfloat16)
+        ym = torch.empty((m, 2 * I), device=dev, dtype=torch.bfloat16)
+        nb1 = 2 * I * (H // 32)
+
+        def pstep(i, xm=xm, ym=ym):
+            ops.mxfp4_matmul(xm, gub[0][:nb1 * 16], gub[1][:nb1], H, 2 * I, out=ym, ctx=ctx)
+        out.append(_case(f"mxfp4 M={m} K={H} N={2 * I} bf16 (mxfp4_matmul, prefill)", pstep, steps, warmup, stream,
+                         time_graph, nb1 * 17 + m * (H + 2 * I) * 2, 2.0 * m * H * 2 * I, ctx))
+    Tp = 512
+    logits_p = torch.randn((Tp, E), device=dev, dtype=torch.float32)
+    xp = torch.randn((Tp, H), device=dev, dtype=torch.bfloat16)
+    np_p = Tp * top_k
+    ygu_p = torch.empty((np_p, 2 * I), device=dev, dtype=torch.bfloat16)
+    h_p = torch.empty((np_p, I), device=dev, dtype=torch.bfloat16)
+    ydn_p = torch.empty((np_p, H), device=dev, dtype=torch.bfloat16)
+    out_p = torch.empty((Tp, H), device=dev, dtype=torch.bfloat16)
+
+    def prefill_step(i):
+        idx, vals = ops.moe_route(logits_p, top_k, True, ctx=ctx)
+        off, tok, _, pos = ops.moe_group(idx, vals, E, ctx=ctx)
+        ops.mxfp4_moe_matmul(xp, gub[0], gub[1], gu_bias, off, tok, H, 2 * I, out=ygu_p, ctx=ctx)
+        ops.gated_activation(ygu_p, ops.ACT_GPT_OSS_SWIGLU, 7.0, out=h_p, ctx=ctx)
+        ops.mxfp4_moe_matmul(h_p, dnb[0], dnb[1], dn_bias, off, None, I, H, out=ydn_p, ctx=ctx)
+        ops.moe_combine(ydn_p, pos, vals, out=out_p, ctx=ctx)
+    r3 = _case(f"mxfp4 moe layer step, prefill: {Tp} tokens, {np_p} pairs over {E} experts", prefill_step, steps,
+               warmup, stream, time_graph, E * per_expert + np_p * (H + 2 * I + I + H) * 2,
+               2.0 * np_p * (2 * I * H + H * I), ctx)
+    r3["launches"] = 6
+    out.append(r3)
     return out

@@ -25,12 +25,6 @@ __device__ __forceinline__ float fp4_to_f32(uint32_t c) {
     return __builtin_bit_cast(float, bits);
 }
 
-// E8M0 -> f32 power of two; 0xFF is NaN (mxfp4.rs:25-31), 0 is the subnormal 2^-127.
-__device__ __forceinline__ float e8m0_to_f32(uint32_t s) {
-    const uint32_t bits = (s == 0xFFu) ? 0x7FC00000u : (s == 0u ? 0x00400000u : (s << 23));
-    return __builtin_bit_cast(float, bits);
-}
-
 __device__ __forceinline__ void decode_block(const u32x4_t q, float scale, float w[32]) {
 #pragma unroll
     for (int i = 0; i < 4; ++i)
@@ -416,6 +410,14 @@ static int mxfp4_mfma_go(hipStream_t s, dim3 grid, const Mxfp4Problem &p, size_t
 int launch_mxfp4_gemv(oxq_ctx *ctx, hipStream_t s, const Mxfp4Problem &p) {
     const bool grouped = p.n_experts > 0;
     bool force_rows = false;
+    {
+        // prefill sizes go to the tile matmul, which converts a weight once per 64 tokens
+        // instead of once per pass of 16 (4 grouped) tokens
+        const char *mm = getenv("OXQ_MXFP4_MM");
+        const int mm_mode = mm ? atoi(mm) : -1;  // 0 = never, 1 = always, default by size
+        const bool big = grouped ? p.n_pairs >= 8 * p.n_experts : p.M > 16;
+        if ((mm_mode == 1 || (mm_mode != 0 && big)) && p.K % 32 == 0) return launch_mxfp4_mm(ctx, s, p);
+    }
     {
         // matrix-core form: tokens staged in LDS (MTOK per pass), 4 waves x FR x 16 rows per workgroup
         const char *v = getenv("OXQ_MXFP4_VARIANT");

@@ -137,6 +137,12 @@ struct BF16Traits {
     }
 };
 
+// E8M0 -> f32 power of two; 0xFF is NaN (mxfp4.rs:25-31), 0 is the subnormal 2^-127.
+__device__ __forceinline__ float e8m0_to_f32(uint32_t s) {
+    const uint32_t bits = (s == 0xFFu) ? 0x7FC00000u : (s == 0u ? 0x00400000u : (s << 23));
+    return __builtin_bit_cast(float, bits);
+}
+
 // ---------------------------------------------------------------------------
 // Reductions
 // ---------------------------------------------------------------------------

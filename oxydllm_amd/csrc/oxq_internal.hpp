@@ -136,6 +136,8 @@ int launch_gguf_dequant(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p, float
 // m > 8, bf16: tile matmul on the matrix cores (weights rounded to bf16 as the reference's mul_mm does)
 bool gguf_mm_eligible(const GgufProblem &p);
 int launch_gguf_mm(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p);
+// MXFP4 prefill (plain m > 16, or grouped with many pairs per expert): same tile matmul
+int launch_mxfp4_mm(oxq_ctx *ctx, hipStream_t s, const Mxfp4Problem &p);
 int launch_mxfp4_gemv(oxq_ctx *ctx, hipStream_t s, const Mxfp4Problem &p);
 int launch_mxfp4_dequant(oxq_ctx *ctx, hipStream_t s, const Mxfp4Problem &p, float *out_nk);
 // mixture-of-experts glue (moe_glue.hip)

@@ -223,6 +223,74 @@ def _config4(seed=0x0A0D11E9):
                 dn_s=dn_s, gu_bias=gu_bias, dn_bias=dn_bias, x=x, logits=logits)
 
 
+@pytest.mark.parametrize("m,n,k", [(17, 10, 64), (33, 100, 96), (150, 1000, 1120), (150, 1001, 2880), (64, 5760, 2880)])
+def test_mxfp4_mul_mm(m, n, k, monkeypatch):
+    """m > 16 runs the tile matmul (metal_ops.rs:6197-6223 switches to mul_mm above 8 rows).
+    E2M1 x E8M0 is exact in bf16, so the tile form matches the unrounded oracle; shapes cover
+    the reference's n = 10, k = 64 case, partial row and token tiles, K that is not a multiple
+    of the 256-element stage, odd N, and split K (forced for the small shapes)."""
+    say(f"mxfp4 mul_mm m={m} n={n} k={k}")
+    blocks, scales = synth.mxfp4_weight(n, k, seed=m + n)
+    w = oracle.dequantize_mxfp4_f32(blocks, scales, n, k)
+    x = np.random.default_rng(m).standard_normal((m, k)).astype(np.float32)
+    ref = oracle.matmul_nt_f32(round_x(x, oracle.BF16), w)
+    bd, sd, xd = to_dev(blocks), to_dev(scales), to_dev(x, torch.bfloat16)
+    y = ops.mxfp4_matmul(xd, bd, sd, k, n)
+    plan = ops.default_context().last_plan()
+    assert plan["kernel"].startswith("mxfp4_mul_mm_bf16")
+    assert_close(y, ref, f"mxfp4 mul_mm {m}x{n}x{k}")
+    if n % 4 == 0 and k >= 512:
+        monkeypatch.setenv("OXQ_MXFP4_MM_KS", "3")
+        y3 = ops.mxfp4_matmul(xd, bd, sd, k, n)
+        assert ops.default_context().last_plan()["split_k"] > 1
+        assert_close(y3, ref, f"mxfp4 mul_mm split {m}x{n}x{k}")
+    # the decode kernel on the same rows agrees within the tolerance as well
+    monkeypatch.setenv("OXQ_MXFP4_MM", "0")
+    y0 = ops.mxfp4_matmul(xd, bd, sd, k, n)
+    assert "gemv" in ops.default_context().last_plan()["kernel"]
+    assert_close(y0, ref, f"mxfp4 gemv form {m}x{n}x{k}")
+
+
+@pytest.mark.parametrize("T,E,top_k,N,K", [(64, 8, 2, 200, 320), (300, 4, 2, 130, 576), (40, 32, 4, 64, 64)])
+def test_mxfp4_moe_prefill_grouped(T, E, top_k, N, K, monkeypatch):
+    """Grouped tile matmul: many routed pairs per expert (prefill).  Experts with no, few and
+    more than one tile of tokens; gathered rows (gate_up) and identity rows (down)."""
+    say(f"mxfp4 moe prefill T={T} E={E} top{top_k} N={N} K={K}")
+    rng = np.random.default_rng(T + E)
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    logits[:, 1] = -30.0  # expert 1 never routed
+    idx, vals = oracle.moe_route(logits, top_k, True)
+    offsets, tokens, _ = oracle.moe_group(idx, vals, E)
+    n_pairs = int(offsets[-1])
+    nb = K // 32
+    blocks, scales = synth.mxfp4_weight(E * N, K, seed=E)
+    bias = rng.standard_normal((E, N)).astype(np.float32) * 0.1
+    x = rng.standard_normal((T, K)).astype(np.float32)
+    xb, bb = round_x(x, oracle.BF16), round_x(bias, oracle.BF16)
+    ref = np.zeros((n_pairs, N), np.float32)
+    for e in range(E):
+        lo, hi = int(offsets[e]), int(offsets[e + 1])
+        if hi > lo:
+            w = oracle.dequantize_mxfp4_f32(blocks[e * N * nb * 16:(e + 1) * N * nb * 16],
+                                            scales[e * N * nb:(e + 1) * N * nb], N, K)
+            ref[lo:hi] = oracle.matmul_nt_f32(xb[tokens[lo:hi]], w, bb[e])
+    off_d, tok_d = to_dev(offsets.astype(np.int32)), to_dev(tokens.astype(np.int32))
+    monkeypatch.setenv("OXQ_MXFP4_MM", "1")
+    y = ops.mxfp4_moe_matmul(to_dev(x, torch.bfloat16), to_dev(blocks), to_dev(scales),
+                             to_dev(bias, torch.bfloat16), off_d, tok_d, K, N)
+    assert ops.default_context().last_plan()["kernel"].startswith("mxfp4_moe_mul_mm_bf16")
+    assert_close(y, ref, "moe prefill gathered")
+    xp = x[tokens]  # identity rows: one activation row per pair
+    y2 = ops.mxfp4_moe_matmul(to_dev(xp, torch.bfloat16), to_dev(blocks), to_dev(scales),
+                              to_dev(bias, torch.bfloat16), off_d, None, K, N)
+    assert_close(y2, ref, "moe prefill identity rows")
+    monkeypatch.setenv("OXQ_MXFP4_MM", "0")
+    y0 = ops.mxfp4_moe_matmul(to_dev(x, torch.bfloat16), to_dev(blocks), to_dev(scales),
+                              to_dev(bias, torch.bfloat16), off_d, tok_d, K, N)
+    assert "gemv" in ops.default_context().last_plan()["kernel"]
+    assert_close(y0, ref, "moe prefill through the decode kernel")
+
+
 def test_mxfp4_moe_config4():
     """Benchmark config 4: 32 experts, top-4, hidden 2880, gate_up N=5760, down K=2880, 8 tokens.
     Routing lists come from the oracle's restatement of moe.rs:466-607."""
