@@ -167,6 +167,34 @@ int oxq_maybe_mpp_quant_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x,
                                const oxq_tensor *scales, uint32_t bits, int pack_dim,
                                const oxq_tensor *out, int *taken);
 
+/* ---- load-time transforms into the AWQ layout ----------------------------
+ * The reference runs these on the CPU while a checkpoint loads; here the
+ * checkpoint tensors are already device-resident.  All outputs are caller
+ * allocated.
+ */
+
+/* awq.rs:187-254 compressed_to_awq: compressed-tensors pack-quantized int4
+ * (weight_packed [out, in/8] I32/U32, nibble i%8 of word (o, i/8) = q + 8;
+ * weight_scale [out, groups]) -> AWQ qweight [in, out/8], qzeros
+ * [groups, out/8] (all 0x88888888), scales [groups, out] of weight_scale's dtype. */
+int oxq_compressed_to_awq(oxq_ctx *ctx, void *stream, const oxq_tensor *weight_packed,
+                          const oxq_tensor *weight_scale, const oxq_tensor *qweight_out,
+                          const oxq_tensor *qzeros_out, const oxq_tensor *scales_out);
+
+/* awq.rs:256-323 concat_awq_along_out: fuses n_parts AWQ weights that share
+ * in_features, group size and bits (QKV, gate|up) into one along the output
+ * dimension.  qweights / qzeros / scales are arrays of n_parts descriptors. */
+int oxq_concat_awq_along_out(oxq_ctx *ctx, void *stream, int bits, int n_parts, const oxq_tensor *qweights,
+                             const oxq_tensor *qzeros, const oxq_tensor *scales, const oxq_tensor *qweight_out,
+                             const oxq_tensor *qzeros_out, const oxq_tensor *scales_out);
+
+/* awq.rs:637-742 rtn_quantize_awq: round-to-nearest 4-bit group quantization of
+ * a dense [out, in] weight (F32, F16 or BF16; tied lm_head, loader.rs:1060-1076)
+ * into AWQ qweight [in, out/8], qzeros [in/g, out/8] and F32 scales [in/g, out]. */
+int oxq_rtn_quantize_awq(oxq_ctx *ctx, void *stream, const oxq_tensor *weight, int64_t group_size,
+                         const oxq_tensor *qweight_out, const oxq_tensor *qzeros_out,
+                         const oxq_tensor *scales_out);
+
 /* ---- GGUF block-quant ops -------------------------------------------------
  * weight_bytes: U8 [N * K/block_elems * block_bytes], row n = consecutive
  * ggml blocks.  x and out: BF16 (the reference's contract) or F32 (the

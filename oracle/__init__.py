@@ -121,6 +121,51 @@ def dequantize_awq(qweight, qzeros, scales) -> np.ndarray:
     return out
 
 
+def compressed_to_awq(weight_packed, weight_scale):
+    """awq.rs:187-254: compressed-tensors int4 [out, in/8] + scales [out, groups] ->
+    AWQ (qweight [in, out/8], qzeros [groups, out/8], scales f32 [groups, out])."""
+    ct, sc = _u32(weight_packed), _f32(weight_scale)
+    out_f, packed_in = ct.shape
+    groups = sc.shape[1]
+    if sc.shape[0] != out_f:
+        raise ValueError("weight_scale dim0 != weight_packed out_features")
+    in_f = packed_in * 8
+    qweight = np.empty((in_f, out_f // 8), np.uint32)
+    qzeros = np.empty((groups, out_f // 8), np.uint32)
+    scales = np.empty((groups, out_f), np.float32)
+    _check(lib().orc_compressed_to_awq(_p(ct), _p(sc), C.c_int64(out_f), C.c_int64(in_f), C.c_int64(groups),
+                                       _p(qweight), _p(qzeros), _p(scales)), "compressed_to_awq")
+    return qweight, qzeros, scales
+
+
+def concat_awq_along_out(parts):
+    """awq.rs:256-323: parts = [(qweight, qzeros, scales), ...] sharing in_features and groups."""
+    if not parts:
+        raise ValueError("concat_awq_along_out: no parts")
+    k, g = parts[0][0].shape[0], parts[0][2].shape[0]
+    for qw, qz, sc in parts[1:]:
+        if qw.shape[0] != k:
+            raise ValueError("AWQ fuse: in_features mismatch")
+        if sc.shape[0] != g:
+            raise ValueError("AWQ fuse: group_size mismatch")
+    return tuple(np.concatenate([p[i] for p in parts], axis=1) for i in range(3))
+
+
+def rtn_quantize_awq(weight, group_size: int):
+    """awq.rs:637-742: dense [out, in] -> AWQ 4-bit (qweight, qzeros, scales f32)."""
+    w = _f32(weight)
+    out_f, in_f = w.shape
+    if out_f % 8 or group_size <= 0 or in_f % group_size:
+        raise ValueError("rtn_quantize_awq: shape not divisible")
+    groups = in_f // group_size
+    qweight = np.empty((in_f, out_f // 8), np.uint32)
+    qzeros = np.empty((groups, out_f // 8), np.uint32)
+    scales = np.empty((groups, out_f), np.float32)
+    _check(lib().orc_rtn_quantize_awq(_p(w), C.c_int64(out_f), C.c_int64(in_f), C.c_int64(group_size),
+                                      _p(qweight), _p(qzeros), _p(scales)), "rtn_quantize_awq")
+    return qweight, qzeros, scales
+
+
 def dequantize_awq8(qweight, qzeros, scales) -> np.ndarray:
     """AWQ-layout 8-bit (identity slot order) -> [N, K] f32."""
     qweight, qzeros, scales = _u32(qweight), _u32(qzeros), _f32(scales)

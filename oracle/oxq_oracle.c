@@ -19,6 +19,8 @@
  *                             954-959, 1100-1103, 1228-1233, 1439-1445, 1681-1686,
  *                             1841-1846, 2032-2037 (block structs) and 2315-2640
  *                             (one dequant formula per format)
+ *   orc_compressed_to_awq     src/common/awq.rs:187-254
+ *   orc_rtn_quantize_awq      src/common/awq.rs:637-742
  *   orc_matmul_nt_f32         src/common/linear.rs:40-79  (x . W^T + bias, f32)
  *   orc_moe_route             src/common/moe.rs:466-499 + linear.rs:160-171
  *   orc_moe_group             src/common/moe.rs:563-607  (dispatch_sparse lists)
@@ -320,6 +322,88 @@ int orc_dequantize_mxfp4_f32(const uint8_t *blocks, size_t blocks_len, const uin
             }
         }
     }
+    return ORC_OK;
+}
+
+/* ------------------------------------------------------------------ */
+/* Load-time transforms into the AWQ layout                            */
+/* ------------------------------------------------------------------ */
+
+static const int ORC_AWQ_ORDER[8] = {0, 2, 4, 6, 1, 3, 5, 7}; /* awq.rs:23 */
+
+/* awq.rs:187-254.  ct [out, in/8]: word (o, c) nibble k = column 8c+k (q+8);
+ * scale_ct [out, groups] f32 -> qweight [in, out/8], qzeros [groups, out/8],
+ * scales [groups, out] f32. */
+int orc_compressed_to_awq(const uint32_t *ct, const float *scale_ct, int64_t out_f, int64_t in_f,
+                          int64_t groups, uint32_t *qweight, uint32_t *qzeros, float *scales) {
+    if (in_f % 8 != 0 || out_f % 8 != 0 || groups == 0 || in_f % groups != 0) return ORC_ERR_SHAPE;
+    const int64_t packed_out = out_f / 8, packed_in = in_f / 8;
+    for (int64_t i = 0; i < in_f; ++i) {
+        const int64_t c = i / 8;
+        const uint32_t sh = 4u * (uint32_t)(i % 8);
+        for (int64_t jw = 0; jw < packed_out; ++jw) {
+            uint32_t w = 0;
+            for (int k = 0; k < 8; ++k) {
+                const int64_t o = jw * 8 + ORC_AWQ_ORDER[k];
+                w |= ((ct[o * packed_in + c] >> sh) & 0xFu) << (4 * k);
+            }
+            qweight[i * packed_out + jw] = w;
+        }
+    }
+    for (int64_t z = 0; z < groups * packed_out; ++z) qzeros[z] = 0x88888888u;
+    for (int64_t o = 0; o < out_f; ++o)
+        for (int64_t g = 0; g < groups; ++g) scales[g * out_f + o] = scale_ct[o * groups + g];
+    return ORC_OK;
+}
+
+/* awq.rs:637-742.  weight [out, in] f32 -> AWQ 4-bit tensors, scales f32 [groups, out]. */
+int orc_rtn_quantize_awq(const float *w, int64_t out_f, int64_t in_f, int64_t group_size,
+                         uint32_t *qweight, uint32_t *qzeros, float *scales) {
+    if (out_f % 8 != 0 || group_size <= 0 || in_f % group_size != 0) return ORC_ERR_SHAPE;
+    const int64_t groups = in_f / group_size, packed_out = out_f / 8;
+    uint8_t *qnib = (uint8_t *)malloc((size_t)(out_f * in_f));
+    uint8_t *znib = (uint8_t *)malloc((size_t)(out_f * groups));
+    if (!qnib || !znib) {
+        free(qnib);
+        free(znib);
+        return ORC_ERR_ARG;
+    }
+    for (int64_t o = 0; o < out_f; ++o) {
+        const float *w_row = w + o * in_f;
+        for (int64_t g = 0; g < groups; ++g) {
+            const float *grp = w_row + g * group_size;
+            float xmin = grp[0], xmax = grp[0];
+            for (int64_t i = 0; i < group_size; ++i) {
+                xmin = fminf(xmin, grp[i]);
+                xmax = fmaxf(xmax, grp[i]);
+            }
+            xmin = fminf(xmin, 0.0f); /* the representable range always spans 0 */
+            xmax = fmaxf(xmax, 0.0f);
+            if (xmax - xmin < 1e-12f) {
+                scales[g * out_f + o] = xmin;
+                znib[o * groups + g] = 0;
+                for (int64_t i = 0; i < group_size; ++i) qnib[o * in_f + g * group_size + i] = 1;
+            } else {
+                const float scale = (xmax - xmin) / 15.0f;
+                const float zero = fminf(fmaxf(roundf(-xmin / scale), 0.0f), 15.0f);
+                scales[g * out_f + o] = scale;
+                znib[o * groups + g] = (uint8_t)zero;
+                for (int64_t i = 0; i < group_size; ++i)
+                    qnib[o * in_f + g * group_size + i] =
+                        (uint8_t)fminf(fmaxf(roundf(grp[i] / scale + zero), 0.0f), 15.0f);
+            }
+        }
+    }
+    memset(qweight, 0, (size_t)(in_f * packed_out) * 4);
+    memset(qzeros, 0, (size_t)(groups * packed_out) * 4);
+    for (int64_t j = 0; j < packed_out; ++j)
+        for (int k = 0; k < 8; ++k) {
+            const int64_t o = j * 8 + ORC_AWQ_ORDER[k];
+            for (int64_t i = 0; i < in_f; ++i) qweight[i * packed_out + j] |= (uint32_t)qnib[o * in_f + i] << (4 * k);
+            for (int64_t g = 0; g < groups; ++g) qzeros[g * packed_out + j] |= (uint32_t)znib[o * groups + g] << (4 * k);
+        }
+    free(qnib);
+    free(znib);
     return ORC_OK;
 }
 

@@ -67,6 +67,9 @@ SIGNATURES = {
     "oxq_mpp_quant_matmul": (C.c_int, [_VP, _VP, _TP, _TP, _TP, _TP, C.c_uint32, C.c_int, _TP]),
     "oxq_maybe_mpp_quant_matmul": (C.c_int, [_VP, _VP, _TP, _TP, _TP, _TP, C.c_uint32, C.c_int,
                                              _TP, C.POINTER(C.c_int)]),
+    "oxq_compressed_to_awq": (C.c_int, [_VP, _VP, _TP, _TP, _TP, _TP, _TP]),
+    "oxq_concat_awq_along_out": (C.c_int, [_VP, _VP, C.c_int, C.c_int, _TP, _TP, _TP, _TP, _TP, _TP]),
+    "oxq_rtn_quantize_awq": (C.c_int, [_VP, _VP, _TP, C.c_int64, _TP, _TP, _TP]),
     "oxq_gguf_quant_matmul": (C.c_int, [_VP, _VP, _TP, _TP, C.c_int64, C.c_int64, C.c_int, _TP]),
     "oxq_gguf_quant_mul_mm": (C.c_int, [_VP, _VP, _TP, _TP, C.c_int64, C.c_int64, C.c_int, _TP]),
     "oxq_gguf_dequantize": (C.c_int, [_VP, _VP, _TP, C.c_int64, C.c_int64, C.c_int, _TP]),

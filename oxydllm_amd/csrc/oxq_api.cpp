@@ -82,6 +82,7 @@ static int check_tensor(const oxq_ctx *ctx, const char *op, const char *what, co
     } while (0)
 
 static bool is_packed_dtype(int dt) { return dt == OXQ_I32 || dt == OXQ_U32; }
+static bool is_float_dtype(int d) { return d == OXQ_F32 || d == OXQ_F16 || d == OXQ_BF16; }
 
 // Validation shared by the AWQ/GPTQ GEMV, dequant and tile-GEMM ops.
 // Order follows W4A16Matmul::metal_fwd (metal_ops.rs:1506-1566),
@@ -595,6 +596,162 @@ int oxq_gguf_dequantize(oxq_ctx *ctx, void *stream, const oxq_tensor *weight_byt
     return launch_gguf_dequant(ctx, (hipStream_t)stream, p, (float *)out->data);
 }
 
+// ---- load-time transforms into the AWQ layout --------------------------------------
+static int check_2d(const char *op, const char *what, const oxq_tensor *t, int64_t d0, int64_t d1) {
+    if (t->rank != 2 || t->dims[0] != d0 || t->dims[1] != d1 || !t->contiguous)
+        return fail(OXQ_ERR_SHAPE, "%s: %s must be a contiguous [%lld, %lld]", op, what, (long long)d0,
+                    (long long)d1);
+    return OXQ_OK;
+}
+
+// awq.rs:187-254
+int oxq_compressed_to_awq(oxq_ctx *ctx, void *stream, const oxq_tensor *weight_packed,
+                          const oxq_tensor *weight_scale, const oxq_tensor *qweight_out,
+                          const oxq_tensor *qzeros_out, const oxq_tensor *scales_out) {
+    const char *op = "compressed_to_awq";
+    if (!ctx) return fail(OXQ_ERR_ARG, "%s: ctx is NULL", op);
+    OXQ_TRY(check_tensor(ctx, op, "weight_packed", weight_packed));
+    OXQ_TRY(check_tensor(ctx, op, "weight_scale", weight_scale));
+    OXQ_TRY(check_tensor(ctx, op, "qweight_out", qweight_out));
+    OXQ_TRY(check_tensor(ctx, op, "qzeros_out", qzeros_out));
+    OXQ_TRY(check_tensor(ctx, op, "scales_out", scales_out));
+    if (weight_packed->rank != 2) return fail(OXQ_ERR_SHAPE, "%s: weight_packed must be 2-D [out, in/8]", op);
+    if (weight_scale->rank != 2) return fail(OXQ_ERR_SHAPE, "%s: weight_scale must be 2-D [out, groups]", op);
+    if (!weight_packed->contiguous || !weight_scale->contiguous)
+        return fail(OXQ_ERR_CONTIGUOUS, "%s: inputs must be contiguous", op);
+    if (!is_packed_dtype(weight_packed->dtype))
+        return fail(OXQ_ERR_DTYPE, "%s: weight_packed must be I32 or U32, got %s", op,
+                    dtype_name(weight_packed->dtype));
+    if (!is_float_dtype(weight_scale->dtype))
+        return fail(OXQ_ERR_DTYPE, "%s: weight_scale must be F32, F16 or BF16", op);
+    const int64_t out_f = weight_packed->dims[0], packed_in = weight_packed->dims[1], in_f = packed_in * 8;
+    const int64_t groups = weight_scale->dims[1];
+    if (weight_scale->dims[0] != out_f)
+        return fail(OXQ_ERR_SHAPE, "%s: weight_scale dim0 %lld != weight_packed out_features %lld", op,
+                    (long long)weight_scale->dims[0], (long long)out_f);
+    if (groups == 0 || in_f % groups != 0)
+        return fail(OXQ_ERR_SHAPE, "%s: in_features %lld not divisible by scale groups %lld", op, (long long)in_f,
+                    (long long)groups);
+    if (out_f % 8 != 0)
+        return fail(OXQ_ERR_SHAPE, "%s: out_features %lld not divisible by pack factor 8", op, (long long)out_f);
+    if (!is_packed_dtype(qweight_out->dtype) || !is_packed_dtype(qzeros_out->dtype) ||
+        scales_out->dtype != weight_scale->dtype)
+        return fail(OXQ_ERR_DTYPE, "%s: outputs must be packed I32/U32 and scales of the checkpoint's dtype", op);
+    OXQ_TRY(check_2d(op, "qweight_out", qweight_out, in_f, out_f / 8));
+    OXQ_TRY(check_2d(op, "qzeros_out", qzeros_out, groups, out_f / 8));
+    OXQ_TRY(check_2d(op, "scales_out", scales_out, groups, out_f));
+    if (out_f > INT32_MAX || in_f > INT32_MAX) return fail(OXQ_ERR_SHAPE, "%s: dimension exceeds 2^31-1", op);
+    return launch_compressed_to_awq(ctx, (hipStream_t)stream, (const uint32_t *)weight_packed->data,
+                                    weight_scale->data, (int)dtype_size(weight_scale->dtype),
+                                    (uint32_t *)qweight_out->data, (uint32_t *)qzeros_out->data, scales_out->data,
+                                    out_f, in_f, groups);
+}
+
+// awq.rs:256-323
+int oxq_concat_awq_along_out(oxq_ctx *ctx, void *stream, int bits, int n_parts, const oxq_tensor *qweights,
+                             const oxq_tensor *qzeros, const oxq_tensor *scales, const oxq_tensor *qweight_out,
+                             const oxq_tensor *qzeros_out, const oxq_tensor *scales_out) {
+    const char *op = "AWQ fuse";
+    if (!ctx) return fail(OXQ_ERR_ARG, "%s: ctx is NULL", op);
+    if (n_parts <= 0 || !qweights || !scales) return fail(OXQ_ERR_ARG, "concat_awq_along_out: no parts");
+    if (!qzeros) return fail(OXQ_ERR_ARG, "%s: qzeros missing on a part, not an AWQ tensor", op);
+    if (bits != 4 && bits != 8) return fail(OXQ_ERR_BITS, "%s: bits must be 4 or 8, got %d", op, bits);
+    const int64_t pf = 32 / bits;
+    int64_t in_f = 0, groups = 0, total_out = 0;
+    for (int i = 0; i < n_parts; ++i) {
+        char what[32];
+        snprintf(what, sizeof what, "part %d qweight", i);
+        OXQ_TRY(check_tensor(ctx, op, what, &qweights[i]));
+        snprintf(what, sizeof what, "part %d qzeros", i);
+        OXQ_TRY(check_tensor(ctx, op, what, &qzeros[i]));
+        snprintf(what, sizeof what, "part %d scales", i);
+        OXQ_TRY(check_tensor(ctx, op, what, &scales[i]));
+        const oxq_tensor &qw = qweights[i], &qz = qzeros[i], &sc = scales[i];
+        if (qw.rank != 2 || qz.rank != 2 || sc.rank != 2 || !qw.contiguous || !qz.contiguous || !sc.contiguous)
+            return fail(OXQ_ERR_SHAPE, "%s: part %d tensors must be contiguous and 2-D", op, i);
+        if (!is_packed_dtype(qw.dtype) || !is_packed_dtype(qz.dtype))
+            return fail(OXQ_ERR_DTYPE, "%s: part %d qweight/qzeros must be I32 or U32", op, i);
+        if (sc.dtype != scales[0].dtype || (sc.dtype != OXQ_F16 && sc.dtype != OXQ_BF16 && sc.dtype != OXQ_F32))
+            return fail(OXQ_ERR_DTYPE, "%s: part %d scales dtype differs from part 0 or is not a float type", op, i);
+        const int64_t out_i = sc.dims[1];
+        if (out_i % pf != 0)
+            return fail(OXQ_ERR_SHAPE, "%s: part %d out_features %lld not divisible by pack_factor %lld", op, i,
+                        (long long)out_i, (long long)pf);
+        if (qw.dims[1] * pf != out_i || qz.dims[1] * pf != out_i || qz.dims[0] != sc.dims[0] || sc.dims[0] == 0 ||
+            qw.dims[0] % sc.dims[0] != 0)
+            return fail(OXQ_ERR_SHAPE, "%s: part %d tensors do not describe one AWQ weight", op, i);
+        if (i == 0) {
+            in_f = qw.dims[0];
+            groups = sc.dims[0];
+        } else {
+            if (qw.dims[0] != in_f)
+                return fail(OXQ_ERR_SHAPE, "%s: in_features mismatch at part %d: expected %lld, got %lld", op, i,
+                            (long long)in_f, (long long)qw.dims[0]);
+            if (sc.dims[0] != groups)
+                return fail(OXQ_ERR_SHAPE, "%s: group_size mismatch at part %d: expected %lld, got %lld", op, i,
+                            (long long)(in_f / groups), (long long)(qw.dims[0] / sc.dims[0]));
+        }
+        total_out += out_i;
+    }
+    OXQ_TRY(check_tensor(ctx, op, "qweight_out", qweight_out));
+    OXQ_TRY(check_tensor(ctx, op, "qzeros_out", qzeros_out));
+    OXQ_TRY(check_tensor(ctx, op, "scales_out", scales_out));
+    if (!is_packed_dtype(qweight_out->dtype) || !is_packed_dtype(qzeros_out->dtype) ||
+        scales_out->dtype != scales[0].dtype)
+        return fail(OXQ_ERR_DTYPE, "%s: outputs must be packed I32/U32 and scales of the parts' dtype", op);
+    OXQ_TRY(check_2d(op, "qweight_out", qweight_out, in_f, total_out / pf));
+    OXQ_TRY(check_2d(op, "qzeros_out", qzeros_out, groups, total_out / pf));
+    OXQ_TRY(check_2d(op, "scales_out", scales_out, groups, total_out));
+    if (total_out > INT32_MAX || in_f > INT32_MAX) return fail(OXQ_ERR_SHAPE, "%s: dimension exceeds 2^31-1", op);
+    const int64_t sb = (int64_t)dtype_size(scales[0].dtype);
+    if ((total_out * sb) % 4 != 0) return fail(OXQ_ERR_SHAPE, "%s: scales rows must be a multiple of 4 bytes", op);
+    set_plan(ctx, "concat_awq_along_out", dim3(1), dim3(256), 1, (uint32_t)(3 * n_parts), 0);
+    int64_t col = 0;
+    for (int i = 0; i < n_parts; ++i) {
+        const int64_t out_i = scales[i].dims[1];
+        // widths in 32-bit words; out_i is a multiple of the pack factor, so 16-bit scale rows are whole words
+        OXQ_TRY(launch_copy2d_u32(ctx, (hipStream_t)stream, qweights[i].data, qweight_out->data, in_f, out_i / pf,
+                                  total_out / pf, col / pf));
+        OXQ_TRY(launch_copy2d_u32(ctx, (hipStream_t)stream, qzeros[i].data, qzeros_out->data, groups, out_i / pf,
+                                  total_out / pf, col / pf));
+        OXQ_TRY(launch_copy2d_u32(ctx, (hipStream_t)stream, scales[i].data, scales_out->data, groups, out_i * sb / 4,
+                                  total_out * sb / 4, col * sb / 4));
+        col += out_i;
+    }
+    return OXQ_OK;
+}
+
+// awq.rs:637-742
+int oxq_rtn_quantize_awq(oxq_ctx *ctx, void *stream, const oxq_tensor *weight, int64_t group_size,
+                         const oxq_tensor *qweight_out, const oxq_tensor *qzeros_out,
+                         const oxq_tensor *scales_out) {
+    const char *op = "rtn_quantize_awq";
+    if (!ctx) return fail(OXQ_ERR_ARG, "%s: ctx is NULL", op);
+    OXQ_TRY(check_tensor(ctx, op, "weight", weight));
+    OXQ_TRY(check_tensor(ctx, op, "qweight_out", qweight_out));
+    OXQ_TRY(check_tensor(ctx, op, "qzeros_out", qzeros_out));
+    OXQ_TRY(check_tensor(ctx, op, "scales_out", scales_out));
+    if (weight->rank != 2) return fail(OXQ_ERR_SHAPE, "%s: weight must be 2-D [out, in]", op);
+    if (!weight->contiguous) return fail(OXQ_ERR_CONTIGUOUS, "%s: weight must be contiguous", op);
+    if (!is_float_dtype(weight->dtype)) return fail(OXQ_ERR_DTYPE, "%s: weight must be F32, F16 or BF16", op);
+    const int64_t out_f = weight->dims[0], in_f = weight->dims[1];
+    if (out_f % 8 != 0)
+        return fail(OXQ_ERR_SHAPE, "%s: out_features (%lld) must be a multiple of 8", op, (long long)out_f);
+    if (group_size <= 0 || in_f % group_size != 0)
+        return fail(OXQ_ERR_GROUP, "%s: in_features (%lld) not divisible by group_size (%lld)", op, (long long)in_f,
+                    (long long)group_size);
+    const int64_t groups = in_f / group_size;
+    if (!is_packed_dtype(qweight_out->dtype) || !is_packed_dtype(qzeros_out->dtype) || scales_out->dtype != OXQ_F32)
+        return fail(OXQ_ERR_DTYPE, "%s: outputs must be packed I32/U32 and F32 scales", op);
+    OXQ_TRY(check_2d(op, "qweight_out", qweight_out, in_f, out_f / 8));
+    OXQ_TRY(check_2d(op, "qzeros_out", qzeros_out, groups, out_f / 8));
+    OXQ_TRY(check_2d(op, "scales_out", scales_out, groups, out_f));
+    if (out_f > INT32_MAX || in_f > INT32_MAX) return fail(OXQ_ERR_SHAPE, "%s: dimension exceeds 2^31-1", op);
+    return launch_rtn_quantize_awq(ctx, (hipStream_t)stream, weight->data, weight->dtype,
+                                   (uint32_t *)qweight_out->data, (uint32_t *)qzeros_out->data,
+                                   (float *)scales_out->data, out_f, in_f, group_size);
+}
+
 // ---- MXFP4 ---------------------------------------------------------------------
 int oxq_mxfp4_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x, const oxq_tensor *blocks,
                      const oxq_tensor *scales, int64_t k, int64_t n, const oxq_tensor *out) {
@@ -660,7 +817,6 @@ int oxq_mxfp4_moe_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x,
 
 // ---- mixture-of-experts glue (moe.rs:466-607, ffn_kernels.metal, moe.rs:152-173) --------
 
-static bool is_float_dtype(int d) { return d == OXQ_F32 || d == OXQ_F16 || d == OXQ_BF16; }
 
 int oxq_moe_route(oxq_ctx *ctx, void *stream, const oxq_tensor *logits, int64_t top_k, int norm_topk,
                   const oxq_tensor *top_idx, const oxq_tensor *top_vals) {

@@ -136,6 +136,14 @@ int launch_gguf_dequant(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p, float
 // m > 8, bf16: tile matmul on the matrix cores (weights rounded to bf16 as the reference's mul_mm does)
 bool gguf_mm_eligible(const GgufProblem &p);
 int launch_gguf_mm(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p);
+// load-time transforms into the AWQ layout (awq_transforms.hip)
+int launch_compressed_to_awq(oxq_ctx *ctx, hipStream_t s, const uint32_t *ct, const void *scale_ct,
+                             int scale_elem_bytes, uint32_t *qweight, uint32_t *qzeros, void *scales,
+                             int64_t out_f, int64_t in_f, int64_t groups);
+int launch_copy2d_u32(oxq_ctx *ctx, hipStream_t s, const void *src, void *dst, int64_t rows, int64_t width,
+                      int64_t dst_pitch, int64_t dst_col);
+int launch_rtn_quantize_awq(oxq_ctx *ctx, hipStream_t s, const void *weight, int dtype, uint32_t *qweight,
+                            uint32_t *qzeros, float *scales, int64_t out_f, int64_t in_f, int64_t group_size);
 // MXFP4 prefill (plain m > 16, or grouped with many pairs per expert): same tile matmul
 int launch_mxfp4_mm(oxq_ctx *ctx, hipStream_t s, const Mxfp4Problem &p);
 int launch_mxfp4_gemv(oxq_ctx *ctx, hipStream_t s, const Mxfp4Problem &p);

@@ -30,8 +30,13 @@ def desc(t: Optional[torch.Tensor]):
     """Tensor -> pointer to an oxq_tensor descriptor (None -> NULL)."""
     if t is None:
         return None
+    return C.byref(desc_struct(t))
+
+
+def desc_struct(t) -> OxqTensor:
+    """Tensor -> oxq_tensor descriptor by value (for arrays of descriptors)."""
     if isinstance(t, OxqTensor):
-        return C.byref(t)
+        return t
     if t.dtype not in _DTYPES:
         raise OxqError(-2, f"unsupported torch dtype {t.dtype}")
     if t.dim() < 1 or t.dim() > _lib.OXQ_MAX_RANK:
@@ -46,7 +51,7 @@ def desc(t: Optional[torch.Tensor]):
     d.device = t.device.index if t.device.type == "cuda" else _lib.DEVICE_HOST
     if t.device.type == "cuda" and d.device is None:
         d.device = torch.cuda.current_device()
-    return C.byref(d)
+    return d
 
 
 class Context:
@@ -190,6 +195,53 @@ def maybe_mpp_quant_matmul(x, qweight, qzeros, scales, bits: int, pack_dim: int,
                                                    desc(qzeros), desc(scales), bits, pack_dim,
                                                    desc(out), C.byref(taken)))
     return out if taken.value else None
+
+
+# ---------------------------------------------------------------- load-time transforms
+def compressed_to_awq(weight_packed, weight_scale, *, ctx: Optional[Context] = None):
+    """awq.rs:187-254: returns AWQ (qweight [in, out/8], qzeros [groups, out/8], scales [groups, out])."""
+    ctx = _ctx(ctx)
+    out_f, packed_in = weight_packed.shape
+    groups = weight_scale.shape[1] if weight_scale.dim() == 2 else 0
+    dev = weight_packed.device
+    qweight = torch.empty((packed_in * 8, out_f // 8), dtype=torch.int32, device=dev)
+    qzeros = torch.empty((groups, out_f // 8), dtype=torch.int32, device=dev)
+    scales = torch.empty((groups, out_f), dtype=weight_scale.dtype, device=dev)
+    _lib.check(ctx._lib.oxq_compressed_to_awq(ctx.handle, ctx.stream(), desc(weight_packed), desc(weight_scale),
+                                              desc(qweight), desc(qzeros), desc(scales)))
+    return qweight, qzeros, scales
+
+
+def concat_awq_along_out(parts, bits: int = 4, *, ctx: Optional[Context] = None):
+    """awq.rs:256-323: parts = [(qweight, qzeros, scales), ...] -> one fused AWQ triplet."""
+    ctx = _ctx(ctx)
+    n = len(parts)
+    if n == 0:
+        raise OxqError(-1, "concat_awq_along_out: no parts")
+    arr = [(OxqTensor * n)(*[desc_struct(p[i]) for p in parts]) for i in range(3)]
+    pf = 32 // bits if bits in (4, 8) else 8
+    total = sum(int(p[2].shape[1]) for p in parts)
+    dev = parts[0][0].device
+    qweight = torch.empty((parts[0][0].shape[0], total // pf), dtype=torch.int32, device=dev)
+    qzeros = torch.empty((parts[0][2].shape[0], total // pf), dtype=torch.int32, device=dev)
+    scales = torch.empty((parts[0][2].shape[0], total), dtype=parts[0][2].dtype, device=dev)
+    _lib.check(ctx._lib.oxq_concat_awq_along_out(ctx.handle, ctx.stream(), bits, n, arr[0], arr[1], arr[2],
+                                                 desc(qweight), desc(qzeros), desc(scales)))
+    return qweight, qzeros, scales
+
+
+def rtn_quantize_awq(weight, group_size: int, *, ctx: Optional[Context] = None):
+    """awq.rs:637-742: dense [out, in] -> AWQ 4-bit (qweight, qzeros, f32 scales)."""
+    ctx = _ctx(ctx)
+    out_f, in_f = weight.shape
+    groups = in_f // group_size if group_size > 0 else 0
+    dev = weight.device
+    qweight = torch.empty((in_f, out_f // 8), dtype=torch.int32, device=dev)
+    qzeros = torch.empty((groups, out_f // 8), dtype=torch.int32, device=dev)
+    scales = torch.empty((groups, out_f), dtype=torch.float32, device=dev)
+    _lib.check(ctx._lib.oxq_rtn_quantize_awq(ctx.handle, ctx.stream(), desc(weight), group_size, desc(qweight),
+                                             desc(qzeros), desc(scales)))
+    return qweight, qzeros, scales
 
 
 # ---------------------------------------------------------------- GGUF

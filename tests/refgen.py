@@ -120,3 +120,37 @@ def mxfp4_x(m, k):
     """metal_ops.rs:6642: ((i % 13) - 6) * 0.05."""
     i = np.arange(m * k)
     return (((i % 13).astype(np.float32) - np.float32(6.0)) * np.float32(0.05)).reshape(m, k)
+
+
+def compressed_tensors_case(out_f=16, in_f=64, group=32):
+    """awq.rs:756-785: signed int4 q = i % 16 - 8, scale = 0.01 + (i % 7) * 0.003, packed as
+    compressed-tensors does (word (o, c) nibble k = q[o][8c + k] + 8)."""
+    groups = in_f // group
+    q = (np.arange(out_f * in_f) % 16 - 8).reshape(out_f, in_f)
+    scale = (np.float32(0.01) + (np.arange(out_f * groups) % 7).astype(np.float32)
+             * np.float32(0.003)).reshape(out_f, groups)
+    packed = np.zeros((out_f, in_f // 8), np.uint32)
+    for k in range(8):
+        packed |= ((q[:, k::8] + 8) & 0xF).astype(np.uint32) << np.uint32(4 * k)
+    return q, scale, packed.view(np.int32)
+
+
+def concat_parts(in_features=8, group_size=4, parts_out=(16, 8, 8)):
+    """awq.rs:1032-1075: three AWQ parts with q = (i + j + 3 idx) & 15, z = (2 g + j + idx) & 15,
+    s = 0.02 (g + 1) + 0.005 (j + 1) + 0.001 idx."""
+    groups = in_features // group_size
+    parts = []
+    for idx, out_f in enumerate(parts_out):
+        i, j = np.meshgrid(np.arange(in_features), np.arange(out_f), indexing="ij")
+        g, jz = np.meshgrid(np.arange(groups), np.arange(out_f), indexing="ij")
+        iw = (i + j + idx * 3) & 0xF
+        iz = (g * 2 + jz + idx) & 0xF
+        sc = (np.float32(0.02) * (g + 1).astype(np.float32) + np.float32(0.005) * (jz + 1).astype(np.float32)
+              + np.float32(0.001) * np.float32(idx)).astype(np.float32)
+        parts.append((synth.pack_awq(iw), synth.pack_awq(iz), sc))
+    return parts
+
+
+def rtn_weight(out_f=16, in_f=64):
+    """awq.rs:803-806: sin(0.013 i)."""
+    return np.sin(np.arange(out_f * in_f, dtype=np.float32) * np.float32(0.013)).astype(np.float32).reshape(out_f, in_f)

@@ -319,3 +319,57 @@ def test_real_context_without_gpu_fails_loudly(lib):
     h = C.c_void_p()
     rc = lib.oxq_ctx_create(0, C.byref(h))
     assert rc == -7 and "no HIP device" in err(lib)
+
+
+def test_awq_load_time_transforms_validate_like_reference(lib, ctx):
+    """awq.rs:188-206 (compressed_to_awq), 257-289 (concat_awq_along_out), 641-654 (rtn_quantize_awq)."""
+    F32 = _lib.F32
+    # compressed-tensors [out=4096, in/8=512], 32 groups -> AWQ [4096, 512] / [32, 512] / [32, 4096]
+    wp, ws = fake((4096, 512), I32), fake((4096, 32), BF16)
+    outs = [fake((4096, 512), I32), fake((32, 512), I32), fake((32, 4096), BF16)]
+
+    def ct(wp=wp, ws=ws, outs=outs):
+        return lib.oxq_compressed_to_awq(ctx, None, C.byref(wp), C.byref(ws), *[C.byref(o) for o in outs])
+    assert ct() == 0, err(lib)
+    assert plan(lib, ctx).kernel.decode() == "compressed_to_awq"
+    assert ct(ws=fake((4000, 32), BF16)) == -3 and "weight_scale dim0 4000 != weight_packed out_features 4096" in err(lib)
+    assert ct(ws=fake((4096, 3), BF16)) == -3 and "not divisible by scale groups" in err(lib)
+    assert ct(wp=fake((4100, 512), I32), ws=fake((4100, 32), BF16)) == -3 and "pack factor" in err(lib)
+    assert ct(wp=fake((4096, 512), F16)) == -2
+    assert ct(outs=[outs[0], outs[1], fake((32, 4096), F16)]) == -2
+    assert ct(outs=[fake((4096, 511), I32), outs[1], outs[2]]) == -3
+
+    # concat: q/k/v-like parts of 4096 + 1024 + 1024 columns
+    parts = [_awq(4096, n, 128, BF16) for n in (4096, 1024, 1024)]
+    arrs = [(_lib.OxqTensor * 3)(*[p[i] for p in parts]) for i in range(3)]
+    fo = _awq(4096, 6144, 128, BF16)
+
+    def cat(n=3, arrs=arrs, fo=fo, bits=4):
+        return lib.oxq_concat_awq_along_out(ctx, None, bits, n, arrs[0], arrs[1], arrs[2], *[C.byref(o) for o in fo])
+    assert cat() == 0, err(lib)
+    p = plan(lib, ctx)
+    assert p.kernel.decode() == "concat_awq_along_out" and p.launches == 9
+    assert cat(n=0) == -1 and "no parts" in err(lib)
+    assert cat(bits=3) == -8
+    assert cat(fo=_awq(4096, 6152, 128, BF16)) == -3
+    bad = [_awq(4096, 4096, 128, BF16), _awq(2048, 1024, 128, BF16), parts[2]]
+    barrs = [(_lib.OxqTensor * 3)(*[q[i] for q in bad]) for i in range(3)]
+    assert cat(arrs=barrs) == -3 and "in_features mismatch at part 1: expected 4096, got 2048" in err(lib)
+    bad = [parts[0], _awq(4096, 1024, 64, BF16), parts[2]]
+    barrs = [(_lib.OxqTensor * 3)(*[q[i] for q in bad]) for i in range(3)]
+    assert cat(arrs=barrs) == -3 and "group_size mismatch at part 1: expected 128, got 64" in err(lib)
+
+    # rtn: tied lm_head [vocab, hidden]
+    w = fake((151936, 4096), BF16)
+    ro = [fake((4096, 151936 // 8), I32), fake((32, 151936 // 8), I32), fake((32, 151936), F32)]
+
+    def rtn(w=w, g=128, ro=ro):
+        return lib.oxq_rtn_quantize_awq(ctx, None, C.byref(w), g, *[C.byref(o) for o in ro])
+    assert rtn() == 0, err(lib)
+    p = plan(lib, ctx)
+    assert p.kernel.decode() == "rtn_quantize_awq" and p.grid[0] == 151936 // 8 and p.block[0] == 512
+    assert rtn(w=fake((151937, 4096), BF16)) == -3 and "must be a multiple of 8" in err(lib)
+    assert rtn(g=96) == -6 and "not divisible by group_size (96)" in err(lib)
+    assert rtn(g=0) == -6
+    assert rtn(w=fake((151936, 4096), I32)) == -2
+    assert rtn(ro=[ro[0], ro[1], fake((32, 151936), BF16)]) == -2

@@ -109,6 +109,80 @@ def test_awq_compressed_tensors_closed_form():
     assert np.max(np.abs(dq - expected)) < 1e-6
 
 
+# ------------------------------------------------------------------ load-time transforms
+def test_compressed_to_awq_matches_direct_dequant():
+    """awq.rs:754-800: dequantizing the converted tensors reproduces q * scale exactly; and the
+    conversion equals unpacking the nibbles and packing them the AWQ way."""
+    q, scale, packed = refgen.compressed_tensors_case()
+    out_f, in_f = q.shape
+    qw, qz, sc = oracle.compressed_to_awq(packed, scale)
+    assert qw.shape == (in_f, out_f // 8) and sc.shape == (scale.shape[1], out_f)
+    dq = oracle.dequantize_awq(qw, qz, sc)
+    expected = q.astype(np.float32) * np.repeat(scale, in_f // scale.shape[1], axis=1)
+    assert np.max(np.abs(dq - expected)) < 1e-6
+    np.testing.assert_array_equal(qw.view(np.int32), synth.pack_awq((q + 8).T))
+    np.testing.assert_array_equal(qz, np.full_like(qz, 0x88888888))
+    np.testing.assert_array_equal(sc, scale.T)
+    with pytest.raises(ValueError):
+        oracle.compressed_to_awq(packed, scale[:8])
+
+
+def test_concat_awq_along_out_matches_separate_dequant():
+    """awq.rs:1032-1093 and 1095-1110."""
+    parts = refgen.concat_parts()
+    fused = oracle.concat_awq_along_out(parts)
+    assert fused[2].shape == (2, 32)
+    separate = np.concatenate([oracle.dequantize_awq(*p) for p in parts], axis=0)
+    np.testing.assert_array_equal(oracle.dequantize_awq(*fused), separate)
+    with pytest.raises(ValueError):
+        oracle.concat_awq_along_out([refgen.concat_parts(4, 4, (8,))[0], refgen.concat_parts(8, 8, (8,))[0]])
+
+
+def _rtn_numpy(w, group):
+    """awq.rs:676-709 with whole-array numpy operations (f32 throughout)."""
+    out_f, in_f = w.shape
+    g = w.reshape(out_f, in_f // group, group)
+    xmin = np.minimum(g.min(axis=2), np.float32(0))
+    xmax = np.maximum(g.max(axis=2), np.float32(0))
+    flat = (xmax - xmin) < np.float32(1e-12)
+    scale = np.where(flat, xmin, (xmax - xmin) / np.float32(15)).astype(np.float32)
+    safe = np.where(flat, np.float32(1), scale)
+
+    def rnd(v):  # round half away from zero, as f32::round
+        return np.copysign(np.floor(np.abs(v) + np.float32(0.5)), v).astype(np.float32)
+    zero = np.where(flat, np.float32(0), np.clip(rnd(-xmin / safe), 0, 15)).astype(np.float32)
+    q = np.clip(rnd(g / safe[:, :, None] + zero[:, :, None]), 0, 15)
+    q = np.where(flat[:, :, None], np.float32(1), q).astype(np.uint8).reshape(out_f, in_f)
+    return q, zero.astype(np.uint8), scale
+
+
+@pytest.mark.parametrize("shape,group", [((16, 64), 32), ((24, 256), 128), ((8, 96), 48)])
+def test_rtn_quantize_awq(shape, group):
+    """awq.rs:802-835 (round trip below 5 % relative error) on the reference's sine weight, and
+    what the arithmetic fixes: the whole-array restatement gives the same integers; every
+    element is reproduced to half a quantization step; an all-zero group stores q = 1, zero = 0,
+    scale = 0 and dequantizes to exactly 0."""
+    w = refgen.rtn_weight(*shape)
+    w[3, :group] = 0.0                       # a flat group
+    w[5, group:2 * group] = np.abs(w[5, group:2 * group]) + 1.0   # a group that does not straddle 0
+    qw, qz, sc = oracle.rtn_quantize_awq(w, group)
+    out_f, in_f = shape
+    assert qw.shape == (in_f, out_f // 8) and qz.shape == (in_f // group, out_f // 8) and sc.shape == (in_f // group, out_f)
+    dq = oracle.dequantize_awq(qw, qz, sc)
+    rel = np.sqrt(((dq - w).astype(np.float64) ** 2).sum() / (w.astype(np.float64) ** 2).sum())
+    assert rel < 0.05
+    q, z, s = _rtn_numpy(w, group)
+    np.testing.assert_array_equal(qw.view(np.int32), synth.pack_awq(q.T))
+    np.testing.assert_array_equal(qz.view(np.int32), synth.pack_awq(z.T))
+    np.testing.assert_array_equal(sc, s.T)
+    step = np.repeat(sc.T, group, axis=1)
+    assert np.all(np.abs(dq - w) <= 0.5 * step * (1 + 1e-5) + 1e-7)
+    assert np.all(dq[3, :group] == 0.0) and sc[0, 3] == 0.0
+    assert np.all((qw[:group, 0] >> 20) & 0xF == 1)   # output row 3 sits in slot 5 (AWQ order[5] = 3)
+    with pytest.raises(ValueError):
+        oracle.rtn_quantize_awq(w[:7], group)
+
+
 @pytest.mark.parametrize("bits", [4, 8])
 def test_gptq_dequant_known_answer(bits):
     """awq.rs:1170-1283, tol 1e-5."""
