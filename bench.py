@@ -152,17 +152,17 @@ def main():
     layers = [ops.PackedQuantLinear(4, ops.PACK_OUT, qw_d[c], qz_d[c], sc_d[c], None, torch.float16, ctx=ctx)
               for c in range(copies)]
 
-    def run_case(m, fn_cold, fn_hot):
+    def run_case(m, fn_cold, fn_hot, k=K, n=N):
         fn_cold(0)
         plan = ctx.last_plan()
         wall_ms, ev_ms = time_graph(fn_cold, args.steps, args.warmup, stream)
         # same weights every call: the 30 MB stay in the 256 MB memory-side cache
         hot_ms = float("nan") if args.no_hot else time_graph(fn_hot, args.steps, args.warmup, stream)[1]
         us = ev_ms * 1e3 / args.steps
-        b = algo_bytes(m)
-        flops = 2.0 * m * K * N
+        b = algo_bytes(m, k, n)
+        flops = 2.0 * m * k * n
         return {
-            "M": m, "kernel": plan["kernel"], "grid": list(plan["grid"]), "split_k": plan["split_k"],
+            "M": m, "K": k, "N": n, "kernel": plan["kernel"], "grid": list(plan["grid"]), "split_k": plan["split_k"],
             "launches": plan["launches"],
             "us_per_call": round(us, 3), "us_per_call_wall": round(wall_ms * 1e3 / args.steps, 3),
             "us_per_call_hot_cache": None if args.no_hot else round(hot_ms * 1e3 / args.steps, 3),
@@ -187,6 +187,24 @@ def main():
                 ops.mpp_quant_matmul(x_d[m], qw_d[c], qz_d[c], sc_d[c], 4, ops.PACK_OUT, out=y_d[m], ctx=ctx)
         op_cases.append(run_case(m, lambda i, op=op: op(i % copies), lambda i, op=op: op(0)))
         print(f"[bench] op M={m}: {op_cases[-1]}", file=sys.stderr, flush=True)
+
+    # The same weight shape the other way round (the MLP's down projection, BASELINE configs[1]
+    # names both orientations): 64 column strips, so K is also cut into slices.
+    down_cases = []
+    if not args.skip_ops:
+        kd, nd = N, K
+        dq = synth.awq_checkpoint(kd, nd, G, 4, seed=0x0A0D11E6 + 1)
+        dlayers = [ops.PackedQuantLinear(4, ops.PACK_OUT, torch.from_numpy(dq[0]).to(dev),
+                                         torch.from_numpy(dq[1]).to(dev),
+                                         torch.from_numpy(dq[2]).to(dev, torch.float16), None, torch.float16,
+                                         ctx=ctx) for _ in range(copies)]
+        for m in (1, 16, 64):
+            xd = torch.randn((m, kd), device=dev, dtype=torch.float16)
+            yd = torch.empty((m, nd), device=dev, dtype=torch.float16)
+            down_cases.append(run_case(m, lambda i, xd=xd, yd=yd: dlayers[i % copies].forward(xd, out=yd),
+                                       lambda i, xd=xd, yd=yd: dlayers[0].forward(xd, out=yd), kd, nd))
+            print(f"[bench] down-projection layer M={m}: {down_cases[-1]}", file=sys.stderr, flush=True)
+        del dlayers
 
     c1 = cases[0]
     # HBM bytes per launch of the M=1 kernel, measured offline with rocprofv3 --pmc
@@ -227,6 +245,7 @@ def main():
                          "frac": cases[2]["mfma_frac"], "traffic": None,
                          "kernel": cases[2]["kernel"], "hbm_frac": cases[2]["hbm_frac"]},
         "cases": cases,
+        "cases_down_projection_K14336_N4096": down_cases,
         "cases_checkpoint_layout_ops": op_cases,
     }
     if args.all:

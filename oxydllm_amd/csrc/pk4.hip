@@ -42,6 +42,7 @@
 #include "oxq_internal.hpp"
 #include "oxq_mfma.hpp"
 
+#include <algorithm>
 #include <cstdlib>
 
 namespace oxq {
@@ -180,8 +181,11 @@ __global__ __launch_bounds__(256) void pk4_dequant_kernel(const uint32_t *__rest
 // ---------------------------------------------------------------------------
 // y[M, N] = x[M, K] . W   on the repacked layout
 //
-// grid.x = strip (64 output columns), grid.z = block of 16*MT rows of x;
-// 8 waves split K between them in blocks of 128 rows (4 MFMA steps).
+// grid.x = strip (64 output columns), grid.z = block of 16*MT rows of x,
+// grid.y = K slice (1 unless the layer has few strips and a long K, see the
+// launcher); 8 waves split the slice between them in blocks of 128 rows (4 MFMA
+// steps).  With more than one slice the workgroup writes its f32 partial tile to
+// the workspace and a second launch adds the slices in order.
 //
 // Weights: one 1 KB wave load per step, issued two blocks (8 steps) ahead.
 // Activations: the matrix-core fragment pattern (16 rows x 64 bytes per load)
@@ -227,8 +231,9 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
                                                        const uint32_t *__restrict__ pw,
                                                        const uint32_t *__restrict__ pzs,
                                                        const uint16_t *__restrict__ bias,
-                                                       uint16_t *__restrict__ y, int M, int K, int N,
-                                                       int gshift, int bpw, int interleave) {
+                                                       uint16_t *__restrict__ y, float *__restrict__ ws,
+                                                       int M, int K, int N, int gshift, int gslice,
+                                                       int interleave) {
     typedef MfmaOps<TT> Ops;
     constexpr int NW = 8;
     constexpr int ROWS = 16 * MT;
@@ -247,15 +252,23 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
     const int ni = lane & 15, kb = lane >> 4;
     const int j = blockIdx.x;
     const int m0 = blockIdx.z * ROWS;
-    const int NS = K >> 5, G = K >> gshift, NB = K >> 7;
+    const int NS = K >> 5, G = K >> gshift;
     const int bpg_mask = (1 << (gshift - 7)) - 1;  // blocks per group - 1
-    // The wave's blocks, by local index i: either one contiguous run of whole groups, or
-    // every 8th group (the 8 waves then sweep the strip together, front to back).
+    // K slice of this workgroup (grid.y slices of `gslice` whole groups; one slice = the
+    // whole strip unless the grid would leave most CUs idle), then the wave's blocks inside
+    // it, by local index i: either one contiguous run of whole groups, the groups dealt out
+    // as evenly as 8 waves allow, or every 8th group (the 8 waves then sweep the slice
+    // together, front to back).
     const int gs7 = gshift - 7;
-    const int b0 = min(NB, wave * bpw);
-    const int nloc = interleave ? (wave < G ? ((G - wave + 7) >> 3) << gs7 : 0) : min(NB, b0 + bpw) - b0;
+    const int sg0 = blockIdx.y * gslice;                 // first group of the slice
+    const int SG = min(G, sg0 + gslice) - sg0;           // groups in the slice (>= 1)
+    const int gbase = SG >> 3, grem = SG & 7;
+    const int wg0 = sg0 + wave * gbase + min(wave, grem);  // the wave's first group
+    const int wgn = gbase + (wave < grem ? 1 : 0);         // and how many
+    const int b0 = wg0 << gs7;
+    const int nloc = interleave ? (wave < SG ? ((SG - wave + 7) >> 3) << gs7 : 0) : wgn << gs7;
     auto blk_of = [&](int i) {
-        return interleave ? (((((i >> gs7) << 3) + wave) << gs7) | (i & bpg_mask)) : b0 + i;
+        return interleave ? ((((((i >> gs7) << 3) + wave) + sg0) << gs7) | (i & bpg_mask)) : b0 + i;
     };
     unsigned char *slot = pk4_lds + wave * SLOT;
 
@@ -279,11 +292,11 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
 
     constexpr int ZCH = 4;  // 16-byte chunks per thread: 32 KB = 128 groups
     u32x4_t zstage[ZCH];
-    const int zchunks = G * 16;
+    const int zchunks = SG * 16;  // the slice's groups only
 #pragma unroll
     for (int q = 0; q < ZCH; ++q)
         if (q * 512 < zchunks)  // block-uniform
-            zstage[q] = __builtin_amdgcn_raw_buffer_load_b128(rs_z, (int)(threadIdx.x + q * 512) * 16, 0, 0);
+            zstage[q] = __builtin_amdgcn_raw_buffer_load_b128(rs_z, (int)(threadIdx.x + q * 512) * 16, sg0 * 256, 0);
 
     constexpr int U = WB > AB ? WB : AB;  // unroll (both divide it)
     u32x4_t aring[AB][AQ], wring[WB][4][WL];
@@ -376,12 +389,12 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
             auto &tmps = *(BPG1 ? &tmpsb : &tmpsg);
             if (live && gfirst) {  // first block of a group
                 if (GS) {
-                    const float4_t s4 = zs_ldsf[((blk >> gs7) * 16 + ni) * 2];
-                    const float4_t n4 = zs_ldsf[((blk >> gs7) * 16 + ni) * 2 + 1];
+                    const float4_t s4 = zs_ldsf[(((blk >> gs7) - sg0) * 16 + ni) * 2];
+                    const float4_t n4 = zs_ldsf[(((blk >> gs7) - sg0) * 16 + ni) * 2 + 1];
                     sf[0] = s4[0], sf[1] = s4[1], sf[2] = s4[2], sf[3] = s4[3];
                     nszb[0] = n4[0], nszb[1] = n4[1], nszb[2] = n4[2], nszb[3] = n4[3];
                 } else {
-                    const u32x4_t zq = zs_lds[(blk >> gs7) * 16 + ni];
+                    const u32x4_t zq = zs_lds[((blk >> gs7) - sg0) * 16 + ni];
                     const uint32_t z0 = zq[0], z1 = zq[1], z2 = zq[2], z3 = zq[3];
                     const uint32_t zv[4] = {z0, z1, z2, z3};
 #pragma unroll
@@ -498,6 +511,17 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
             }
         }
         const int n = 64 * j + c0;
+        if (gridDim.y > 1) {  // this K slice's f32 partial; a second kernel adds the slices in order
+            float *dst = ws + ((size_t)blockIdx.y * M + (m0 + ml)) * N + n;
+            if (CP == 2) {
+                *(float2 *)dst = float2{v[0], v[1]};
+            } else {
+#pragma unroll
+                for (int h = 0; h < CP / 4; ++h)
+                    *(float4_t *)(dst + 4 * h) = float4_t{v[4 * h], v[4 * h + 1], v[4 * h + 2], v[4 * h + 3]};
+            }
+            return;
+        }
         uint32_t o[CP / 2];
 #pragma unroll
         for (int q = 0; q < CP / 2; ++q) {
@@ -588,10 +612,9 @@ static int pk4_env(const char *name, int dflt) {
 }
 
 template <typename TT, int BITS, int MT, bool GS, bool BPG1>
-static int pk4_go3(hipStream_t s, dim3 grid, const Pk4Problem &p, int bpw) {
+static int pk4_go3(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, int gslice) {
     constexpr int AB = Pk4Ring<MT, BITS>::AB, WB = Pk4Ring<MT, BITS>::WB;
-    const int G = (int)(p.w.K >> p.w.group_shift);
-    const size_t lds = (size_t)8 * MT * 4096 + (size_t)G * 256 * (GS ? 2 : 1);
+    const size_t lds = (size_t)8 * MT * 4096 + (size_t)gslice * 256 * (GS ? 2 : 1);
     static size_t attr_lds = 0;  // one per instantiation
     if (lds > attr_lds) {
         OXQ_HIP_CHECK(hipFuncSetAttribute((const void *)pk4_mfma_kernel<TT, BITS, MT, GS, BPG1, AB, WB>,
@@ -600,25 +623,25 @@ static int pk4_go3(hipStream_t s, dim3 grid, const Pk4Problem &p, int bpw) {
     }
     hipLaunchKernelGGL((pk4_mfma_kernel<TT, BITS, MT, GS, BPG1, AB, WB>), grid, dim3(512), lds, s,
                        (const uint16_t *)p.x, p.w.pw, p.w.pzs, (const uint16_t *)p.bias, (uint16_t *)p.y,
-                       (int)p.M, (int)p.w.K, (int)p.w.N, p.w.group_shift, bpw,
+                       (float *)ctx->workspace, (int)p.M, (int)p.w.K, (int)p.w.N, p.w.group_shift, gslice,
                        pk4_env("OXQ_PK4_INTERLEAVE", 0));
     OXQ_HIP_CHECK(hipGetLastError());
     return OXQ_OK;
 }
 
 template <typename TT, int BITS, int MT, bool GS>
-static int pk4_go(hipStream_t s, dim3 grid, const Pk4Problem &p, int bpw) {
-    return p.w.group_shift == 7 ? pk4_go3<TT, BITS, MT, GS, true>(s, grid, p, bpw)
-                                : pk4_go3<TT, BITS, MT, GS, false>(s, grid, p, bpw);
+static int pk4_go(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, int gslice) {
+    return p.w.group_shift == 7 ? pk4_go3<TT, BITS, MT, GS, true>(ctx, s, grid, p, gslice)
+                                : pk4_go3<TT, BITS, MT, GS, false>(ctx, s, grid, p, gslice);
 }
 
 template <typename TT, int BITS>
-static int pk4_by_mt(hipStream_t s, dim3 grid, const Pk4Problem &p, int bpw, int mt) {
+static int pk4_by_mt(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, int gslice, int mt) {
     switch (mt) {
-    case 1: return pk4_go<TT, BITS, 1, true>(s, grid, p, bpw);
-    case 2: return pk4_go<TT, BITS, 2, false>(s, grid, p, bpw);
-    case 3: return pk4_go<TT, BITS, 3, false>(s, grid, p, bpw);
-    default: return pk4_go<TT, BITS, 4, false>(s, grid, p, bpw);
+    case 1: return pk4_go<TT, BITS, 1, true>(ctx, s, grid, p, gslice);
+    case 2: return pk4_go<TT, BITS, 2, false>(ctx, s, grid, p, gslice);
+    case 3: return pk4_go<TT, BITS, 3, false>(ctx, s, grid, p, gslice);
+    default: return pk4_go<TT, BITS, 4, false>(ctx, s, grid, p, gslice);
     }
 }
 
@@ -626,21 +649,43 @@ int launch_pk4_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p) {
     const int64_t M = p.M;
     const int mt = M > 48 ? 4 : (int)ceil_div(M, 16);
     const int G = (int)(p.w.K >> p.w.group_shift);
-    const int bpw = (int)ceil_div(G, 8) << (p.w.group_shift - 7);  // whole groups per wave, in 128-row blocks
-    dim3 grid((unsigned)(p.w.N / 64), 1, (unsigned)ceil_div(M, 16 * mt));
+    // Few column strips and a long K (a down projection: N = 4096 is 64 strips for 256 CUs):
+    // K is also cut into slices of whole groups, at least two groups per wave, so that up to
+    // one workgroup per CU runs; the slices' f32 partial tiles are added in slice order by a
+    // second launch.  Measured (f16, M = 1 / 64): 14336 x 4096 16.6 / 41.1 us unsplit,
+    // 11.2 / 22.5 us in 4 slices, worse again in 5 or 7 (a second round of workgroups); a
+    // 4096 x 4096 layer gains nothing (the extra launch costs what the split saves).
+    const int64_t tiles = (p.w.N / 64) * ceil_div(M, 16 * mt);
+    int ks = 1;
+    if (tiles <= 96 && G >= 64) ks = (int)std::max<int64_t>(1, std::min<int64_t>(256 / tiles, G / 16));
+    ks = pk4_env("OXQ_PK4_KS", ks);
+    ks = std::max(1, std::min(ks, G));
+    while (ks > 1 && (size_t)ks * M * p.w.N * 4 > ctx->workspace_bytes) --ks;
+    const int gslice = (int)ceil_div(G, ks);
+    ks = (int)ceil_div(G, gslice);  // no empty slice
+    dim3 grid((unsigned)(p.w.N / 64), (unsigned)ks, (unsigned)ceil_div(M, 16 * mt));
     char name[64];
     snprintf(name, sizeof name, "pk%d_mfma_%s_mt%d%s", p.w.bits, p.w.dtype == OXQ_F16 ? "f16" : "bf16", mt,
              mt == 1 ? "_gs" : "");
-    set_plan(ctx, name, grid, dim3(512), 1, 1, 0);
-    if (ctx->plan_only) return OXQ_OK;
+    set_plan(ctx, name, grid, dim3(512), ks, 1, ks > 1 ? (size_t)ks * M * p.w.N * 4 : 0);
+    if (ctx->plan_only) {
+        if (ks > 1) add_launch(ctx);
+        return OXQ_OK;
+    }
     if ((uint64_t)M * (uint64_t)p.w.K * 2 >= (1ull << 31))
         return fail(OXQ_ERR_UNSUPPORTED, "repacked matmul: x larger than 2 GiB");
     if (((uintptr_t)p.x | (uintptr_t)p.y) & 15)
         return fail(OXQ_ERR_UNSUPPORTED, "repacked matmul: x and y must be 16-byte aligned");
     const bool f16 = p.w.dtype == OXQ_F16;
+    int rc;
     if (p.w.bits == 4)
-        return f16 ? pk4_by_mt<F16Traits, 4>(s, grid, p, bpw, mt) : pk4_by_mt<BF16Traits, 4>(s, grid, p, bpw, mt);
-    return f16 ? pk4_by_mt<F16Traits, 8>(s, grid, p, bpw, mt) : pk4_by_mt<BF16Traits, 8>(s, grid, p, bpw, mt);
+        rc = f16 ? pk4_by_mt<F16Traits, 4>(ctx, s, grid, p, gslice, mt)
+                 : pk4_by_mt<BF16Traits, 4>(ctx, s, grid, p, gslice, mt);
+    else
+        rc = f16 ? pk4_by_mt<F16Traits, 8>(ctx, s, grid, p, gslice, mt)
+                 : pk4_by_mt<BF16Traits, 8>(ctx, s, grid, p, gslice, mt);
+    if (rc != OXQ_OK || ks == 1) return rc;
+    return launch_splitk_reduce(ctx, s, (const float *)ctx->workspace, p.bias, p.y, M, p.w.N, ks, p.w.dtype);
 }
 
 }  // namespace oxq

@@ -129,6 +129,36 @@ def test_repacked_forward_all_m(kind, dtn, K, N, g):
             assert np.abs(as_f32(y) - ref).max() < 0.06 * np.abs(ref).max() + 1e-2
 
 
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("dtn", ["f16", "bf16"])
+@pytest.mark.parametrize("K,N,g,ks", [(1280, 128, 128, 3), (2048, 64, 256, 2), (1152, 192, 128, 9), (512, 64, 128, 4)])
+def test_repacked_forward_k_slices(kind, dtn, K, N, g, ks, monkeypatch):
+    """Layers with few column strips also cut K into slices (grid.y) whose f32 partial tiles a
+    second launch adds in slice order.  Forced here on small shapes: slices of unequal size
+    (10 groups in 3 slices), fewer groups than waves per slice, one group per slice, bias
+    applied once by the reduction."""
+    dt = DT[dtn]
+    monkeypatch.setenv("OXQ_PK4_KS", str(ks))
+    trip, pack_dim = make(kind, K, N, g, seed=K + N + ks)
+    bias = (np.arange(N, dtype=np.float32) % 7 - 3) * np.float32(0.25)
+    layer = layer_of(trip, pack_dim, dt, bias, bits=bits_of_kind(kind))
+    assert layer.prepacked
+    w = dense(kind, trip, dt)
+    rng = np.random.default_rng(K + ks)
+    groups = K // g
+    per = -(-groups // min(ks, groups))
+    for m in (1, 7, 16, 40, 64, 100):
+        say(f"pk4 k-slices {kind} {dtn} K={K} N={N} g={g} ks={ks} m={m}")
+        x = rng.standard_normal((m, K)).astype(np.float32)
+        xd = to_dev(x, TORCH_DT[dt])
+        y = layer.forward(xd)
+        plan = ops.default_context().last_plan()
+        assert plan["split_k"] == -(-groups // per) and plan["launches"] == 2
+        wr = w if m <= 16 else oracle.round_through(w, dt)
+        assert_close(y, oracle.matmul_nt_f32(round_x(x, dt), wr, bias), f"pk4 k-slices m{m}")
+        np.testing.assert_array_equal(bits_of(layer.forward(xd)), bits_of(y))
+
+
 @pytest.mark.parametrize("m", [1, 16, 64])
 @pytest.mark.parametrize("K,N", [(4096, 14336), (14336, 4096)])
 def test_repacked_forward_config1(m, K, N):
