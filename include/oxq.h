@@ -195,6 +195,28 @@ int oxq_rtn_quantize_awq(oxq_ctx *ctx, void *stream, const oxq_tensor *weight, i
                          const oxq_tensor *qweight_out, const oxq_tensor *qzeros_out,
                          const oxq_tensor *scales_out);
 
+/* ---- block-scaled F8E4M3 (fn variant) ------------------------------------
+ * Weight: U8 [out, in] holding E4M3 encodings (1 sign, 4 exponent bits with
+ * bias 7, 3 mantissa bits; S.1111.111 is NaN, no infinity); scales: F32
+ * [s_rows, s_cols] grid tiling it evenly.  A weight value is
+ * bf16(f32(bf16(f8)) * scale) (quant_kernels.metal:3877-3911).
+ */
+
+/* metal_ops.rs:5562 cast_f8e4m3_to_f32: elementwise widening, any shape. */
+int oxq_cast_f8e4m3_to_f32(oxq_ctx *ctx, void *stream, const oxq_tensor *t, const oxq_tensor *out);
+
+/* metal_ops.rs:5809 f8_block_dequant_bf16: dense BF16 [out, in]. */
+int oxq_f8_block_dequant_bf16(oxq_ctx *ctx, void *stream, const oxq_tensor *bytes,
+                              const oxq_tensor *scales, const oxq_tensor *out);
+
+/* metal_ops.rs:5788 f8_gemv: x BF16 [m, in], 1 <= m <= 8 -> BF16 [m, out]. */
+int oxq_f8_gemv(oxq_ctx *ctx, void *stream, const oxq_tensor *x, const oxq_tensor *bytes,
+                const oxq_tensor *scales, const oxq_tensor *out);
+
+/* moe.rs:106-113 Fp8Cached::forward: any m (GEMV up to 8 rows, tile matmul beyond). */
+int oxq_f8_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x, const oxq_tensor *bytes,
+                  const oxq_tensor *scales, const oxq_tensor *out);
+
 /* ---- GGUF block-quant ops -------------------------------------------------
  * weight_bytes: U8 [N * K/block_elems * block_bytes], row n = consecutive
  * ggml blocks.  x and out: BF16 (the reference's contract) or F32 (the

@@ -121,6 +121,25 @@ def dequantize_awq(qweight, qzeros, scales) -> np.ndarray:
     return out
 
 
+def cast_f8e4m3_to_f32(bytes_) -> np.ndarray:
+    """metal_ops.rs:2942-2955: spec decode of E4M3fn bytes."""
+    b = np.ascontiguousarray(np.asarray(bytes_, dtype=np.uint8))
+    out = np.empty(b.shape, np.float32)
+    lib().orc_cast_f8e4m3_to_f32(_p(b), _p(out), C.c_size_t(b.size))
+    return out
+
+
+def f8_block_dequant_bf16(bytes_, scales) -> np.ndarray:
+    """quant_kernels.metal:3877-3911: bf16 bits [rows, cols] of bf16(f32(bf16(f8)) * scale)."""
+    b = np.ascontiguousarray(np.asarray(bytes_, dtype=np.uint8))
+    sc = _f32(scales)
+    rows, cols = b.shape
+    out = np.empty((rows, cols), np.uint16)
+    _check(lib().orc_f8_block_dequant_bf16(_p(b), _p(sc), C.c_int64(rows), C.c_int64(cols),
+                                           C.c_int64(sc.shape[0]), C.c_int64(sc.shape[1]), _p(out)), "f8_block_dequant")
+    return out
+
+
 def compressed_to_awq(weight_packed, weight_scale):
     """awq.rs:187-254: compressed-tensors int4 [out, in/8] + scales [out, groups] ->
     AWQ (qweight [in, out/8], qzeros [groups, out/8], scales f32 [groups, out])."""

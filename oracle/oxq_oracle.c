@@ -19,6 +19,9 @@
  *                             954-959, 1100-1103, 1228-1233, 1439-1445, 1681-1686,
  *                             1841-1846, 2032-2037 (block structs) and 2315-2640
  *                             (one dequant formula per format)
+ *   orc_f8e4m3_to_f32, orc_f8_block_dequant_bf16
+ *                             src/common/metal_ops.rs:2942-2955 (spec decode),
+ *                             src/common/quant_kernels.metal:3877-3911 (cast chain)
  *   orc_compressed_to_awq     src/common/awq.rs:187-254
  *   orc_rtn_quantize_awq      src/common/awq.rs:637-742
  *   orc_matmul_nt_f32         src/common/linear.rs:40-79  (x . W^T + bias, f32)
@@ -322,6 +325,39 @@ int orc_dequantize_mxfp4_f32(const uint8_t *blocks, size_t blocks_len, const uin
             }
         }
     }
+    return ORC_OK;
+}
+
+/* ------------------------------------------------------------------ */
+/* Block-scaled F8E4M3 (fn variant)                                    */
+/* ------------------------------------------------------------------ */
+
+/* metal_ops.rs:2942-2955 (e4m3_decode): 1 sign, 4 exponent (bias 7), 3 mantissa;
+ * S.1111.111 is NaN, there is no infinity. */
+float orc_f8e4m3_to_f32(uint8_t v) {
+    const uint32_t s = v >> 7, e = (v >> 3) & 0xFu, m = v & 0x7u;
+    float val;
+    if (e == 0) val = ldexpf((float)m * 0.125f, -6);
+    else if (e == 15 && m == 7) val = NAN;
+    else val = ldexpf(1.0f + (float)m * 0.125f, (int)e - 7);
+    return s ? -val : val;
+}
+
+void orc_cast_f8e4m3_to_f32(const uint8_t *in, float *out, size_t n) {
+    for (size_t i = 0; i < n; ++i) out[i] = orc_f8e4m3_to_f32(in[i]);
+}
+
+/* quant_kernels.metal:3877-3911 / metal_ops.rs:4310-4345: F8 -> F32 -> BF16, F32 block
+ * scale fold, -> BF16.  bytes [rows, cols], scales [s_rows, s_cols]; out = bf16 bits. */
+int orc_f8_block_dequant_bf16(const uint8_t *bytes, const float *scales, int64_t rows, int64_t cols,
+                              int64_t s_rows, int64_t s_cols, uint16_t *out) {
+    if (s_rows <= 0 || s_cols <= 0 || rows % s_rows != 0 || cols % s_cols != 0) return ORC_ERR_SHAPE;
+    const int64_t block_r = rows / s_rows, block_c = cols / s_cols;
+    for (int64_t r = 0; r < rows; ++r)
+        for (int64_t c = 0; c < cols; ++c) {
+            const float w = orc_bf16_to_f32(orc_f32_to_bf16(orc_f8e4m3_to_f32(bytes[r * cols + c])));
+            out[r * cols + c] = orc_f32_to_bf16(w * scales[(r / block_r) * s_cols + c / block_c]);
+        }
     return ORC_OK;
 }
 

@@ -92,6 +92,23 @@ def run(ops, ctx, stream, steps, warmup, time_graph):
                                  2.0 * m * K * N, ctx))
         del d
 
+    # ---- block-scaled F8E4M3 (sibling path: streamed FP8 experts) -----------------------
+    for (n8, k8) in ((4096, 4096), (2048, 512)):
+        wb = np.random.default_rng(8).integers(0, 256, size=(n8, k8), dtype=np.uint8)
+        wb = np.where((wb & 0x7F) == 0x7F, wb ^ 0x08, wb).astype(np.uint8)
+        scl = np.random.default_rng(9).uniform(0.01, 1.0, size=(n8 // 128, k8 // 128)).astype(np.float32)
+        nc = _copies_for(wb.nbytes, cap=48)
+        d8 = [(torch.from_numpy(wb).to(dev), torch.from_numpy(scl).to(dev)) for _ in range(nc)]
+        for m in (1, 8, 256):
+            x8 = torch.randn((m, k8), device=dev, dtype=torch.bfloat16)
+            y8 = torch.empty((m, n8), device=dev, dtype=torch.bfloat16)
+
+            def fstep(i, d8=d8, nc=nc, x8=x8, y8=y8):
+                ops.f8_matmul(x8, d8[i % nc][0], d8[i % nc][1], out=y8, ctx=ctx)
+            out.append(_case(f"f8e4m3 block-scaled M={m} K={k8} N={n8} bf16", fstep, steps, warmup, stream,
+                             time_graph, wb.nbytes + scl.nbytes + m * (k8 + n8) * 2, 2.0 * m * k8 * n8, ctx))
+        del d8
+
     # ---- config 4: MXFP4 MoE -----------------------------------------------------
     E, top_k, H, I, T = 32, 4, 2880, 2880, 8
     rng = np.random.default_rng(0x0A0D11E9)

@@ -574,6 +574,7 @@ int oxq_gguf_quant_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x,
     GgufProblem p;
     OXQ_TRY(check_gguf(ctx, "GgufQuantMatmul", true, false, x, weight_bytes, in_features,
                        out_features, quant, out, &p));
+    if (gguf_mm_eligible(p)) return launch_gguf_mm(ctx, (hipStream_t)stream, p);
     return launch_gguf_gemv(ctx, (hipStream_t)stream, p);
 }
 
@@ -750,6 +751,96 @@ int oxq_rtn_quantize_awq(oxq_ctx *ctx, void *stream, const oxq_tensor *weight, i
     return launch_rtn_quantize_awq(ctx, (hipStream_t)stream, weight->data, weight->dtype,
                                    (uint32_t *)qweight_out->data, (uint32_t *)qzeros_out->data,
                                    (float *)scales_out->data, out_f, in_f, group_size);
+}
+
+// ---- block-scaled F8E4M3 -----------------------------------------------------------
+// metal_ops.rs:5562
+int oxq_cast_f8e4m3_to_f32(oxq_ctx *ctx, void *stream, const oxq_tensor *t, const oxq_tensor *out) {
+    const char *op = "cast-f8e4m3-f32";
+    if (!ctx) return fail(OXQ_ERR_ARG, "%s: ctx is NULL", op);
+    OXQ_TRY(check_tensor(ctx, op, "input", t));
+    OXQ_TRY(check_tensor(ctx, op, "out", out));
+    if (t->dtype != OXQ_U8) return fail(OXQ_ERR_DTYPE, "%s: expected F8E4M3 bytes (U8) input, got %s", op, dtype_name(t->dtype));
+    if (!t->contiguous) return fail(OXQ_ERR_CONTIGUOUS, "%s: input must be contiguous", op);
+    if (out->dtype != OXQ_F32 || !out->contiguous || numel(out) != numel(t))
+        return fail(OXQ_ERR_SHAPE, "%s: out must be a contiguous F32 tensor of the input's size", op);
+    return launch_cast_f8e4m3_f32(ctx, (hipStream_t)stream, (const uint8_t *)t->data, (float *)out->data,
+                                  (size_t)numel(t));
+}
+
+// shared checks of F8BlockDequantBf16 (metal_ops.rs:5589-5613) and F8Gemv (5703-5731)
+static int check_f8(oxq_ctx *ctx, const char *op, const oxq_tensor *x, const oxq_tensor *bytes,
+                    const oxq_tensor *scales, const oxq_tensor *out, bool decode, F8Problem *p) {
+    if (!ctx) return fail(OXQ_ERR_ARG, "%s: ctx is NULL", op);
+    if (x) OXQ_TRY(check_tensor(ctx, op, "x", x));
+    OXQ_TRY(check_tensor(ctx, op, "bytes", bytes));
+    OXQ_TRY(check_tensor(ctx, op, "scales", scales));
+    OXQ_TRY(check_tensor(ctx, op, "out", out));
+    if (bytes->dtype != OXQ_U8 || scales->dtype != OXQ_F32)
+        return fail(OXQ_ERR_DTYPE, "%s: expected U8 bytes and F32 scales, got %s/%s", op, dtype_name(bytes->dtype),
+                    dtype_name(scales->dtype));
+    if (!bytes->contiguous || !scales->contiguous) return fail(OXQ_ERR_CONTIGUOUS, "%s: inputs must be contiguous", op);
+    if (bytes->rank != 2 || scales->rank != 2) return fail(OXQ_ERR_SHAPE, "%s: bytes and scales must be 2-D", op);
+    const int64_t rows = bytes->dims[0], cols = bytes->dims[1], s_rows = scales->dims[0], s_cols = scales->dims[1];
+    if (s_rows == 0 || s_cols == 0 || rows % s_rows != 0 || cols % s_cols != 0)
+        return fail(OXQ_ERR_SHAPE, "%s: scale grid [%lld, %lld] does not tile weight [%lld, %lld]", op,
+                    (long long)s_rows, (long long)s_cols, (long long)rows, (long long)cols);
+    if (rows > INT32_MAX || cols > INT32_MAX) return fail(OXQ_ERR_SHAPE, "%s: dimension exceeds 2^31-1", op);
+    int64_t m = 0;
+    if (x) {
+        if (x->dtype != OXQ_BF16) return fail(OXQ_ERR_DTYPE, "%s: x must be BF16, got %s", op, dtype_name(x->dtype));
+        if (!x->contiguous) return fail(OXQ_ERR_CONTIGUOUS, "%s: x must be contiguous", op);
+        if (x->rank != 2 || x->dims[1] != cols || x->dims[0] == 0 || (decode && x->dims[0] > 8)) {
+            char b0[96];
+            dims_str(x, b0, sizeof b0);
+            return fail(decode && x->rank == 2 && x->dims[1] == cols ? OXQ_ERR_M_RANGE : OXQ_ERR_SHAPE,
+                        "%s: x shape %s incompatible with in_features %lld%s", op, b0, (long long)cols,
+                        decode ? " (m must be 1..=8)" : "");
+        }
+        m = x->dims[0];
+        if (out->dtype != OXQ_BF16 || out->rank != 2 || out->dims[0] != m || out->dims[1] != rows || !out->contiguous)
+            return fail(OXQ_ERR_SHAPE, "%s: out must be a contiguous BF16 [%lld, %lld]", op, (long long)m,
+                        (long long)rows);
+        if (m > INT32_MAX) return fail(OXQ_ERR_SHAPE, "%s: dimension exceeds 2^31-1", op);
+    } else if (out->dtype != OXQ_BF16 || out->rank != 2 || out->dims[0] != rows || out->dims[1] != cols ||
+               !out->contiguous) {
+        return fail(OXQ_ERR_SHAPE, "%s: out must be a contiguous BF16 [%lld, %lld]", op, (long long)rows,
+                    (long long)cols);
+    }
+    p->x = x ? x->data : nullptr;
+    p->w = (const uint8_t *)bytes->data;
+    p->scales = (const float *)scales->data;
+    p->y = out->data;
+    p->M = m, p->K = cols, p->N = rows;
+    p->block_r = rows / s_rows, p->block_c = cols / s_cols, p->s_cols = s_cols;
+    return OXQ_OK;
+}
+
+// metal_ops.rs:5809
+int oxq_f8_block_dequant_bf16(oxq_ctx *ctx, void *stream, const oxq_tensor *bytes, const oxq_tensor *scales,
+                              const oxq_tensor *out) {
+    F8Problem p;
+    OXQ_TRY(check_f8(ctx, "f8-block-dequant-bf16", nullptr, bytes, scales, out, false, &p));
+    return launch_f8_block_dequant(ctx, (hipStream_t)stream, p, (uint16_t *)out->data);
+}
+
+// metal_ops.rs:5788 (1 <= m <= 8)
+int oxq_f8_gemv(oxq_ctx *ctx, void *stream, const oxq_tensor *x, const oxq_tensor *bytes,
+                const oxq_tensor *scales, const oxq_tensor *out) {
+    F8Problem p;
+    OXQ_TRY(check_f8(ctx, "f8-gemv", x, bytes, scales, out, true, &p));
+    if (f8_mm_eligible(p)) return launch_f8_mm(ctx, (hipStream_t)stream, p);
+    return launch_f8_gemv(ctx, (hipStream_t)stream, p);
+}
+
+// moe.rs:106-113 Fp8Cached::forward: the GEMV for decode-sized batches, beyond it the
+// dequantized weight times x - here without materializing the dense weight
+int oxq_f8_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x, const oxq_tensor *bytes,
+                  const oxq_tensor *scales, const oxq_tensor *out) {
+    F8Problem p;
+    OXQ_TRY(check_f8(ctx, "f8-matmul", x, bytes, scales, out, false, &p));
+    if (f8_mm_eligible(p)) return launch_f8_mm(ctx, (hipStream_t)stream, p);
+    return launch_f8_gemv(ctx, (hipStream_t)stream, p);
 }
 
 // ---- MXFP4 ---------------------------------------------------------------------

@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdarg>
+#include <algorithm>
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
@@ -103,6 +104,16 @@ struct Mxfp4Problem {
     int64_t n_pairs;
 };
 
+// Block-scaled F8E4M3 weight [N, K] bytes with an F32 scale grid [s_rows, s_cols] tiling it.
+struct F8Problem {
+    const void *x;          // [M, K] bf16 (nullptr for the dequant)
+    const uint8_t *w;       // [N, K]
+    const float *scales;    // [N / block_r, K / block_c]
+    void *y;                // [M, N] bf16
+    int64_t M, K, N;
+    int64_t block_r, block_c, s_cols;
+};
+
 // A resident 4- or 8-bit layer repacked tile-major at load (layout: pk4.hip).
 struct Pk4Weights {
     uint32_t *pw;           // [N/64][K/32][bits/4][64][4]
@@ -144,6 +155,12 @@ int launch_copy2d_u32(oxq_ctx *ctx, hipStream_t s, const void *src, void *dst, i
                       int64_t dst_pitch, int64_t dst_col);
 int launch_rtn_quantize_awq(oxq_ctx *ctx, hipStream_t s, const void *weight, int dtype, uint32_t *qweight,
                             uint32_t *qzeros, float *scales, int64_t out_f, int64_t in_f, int64_t group_size);
+// block-scaled F8E4M3 (f8_block.hip; the tile matmul for m > 8 lives in blockq_mm.hip)
+int launch_cast_f8e4m3_f32(oxq_ctx *ctx, hipStream_t s, const uint8_t *in, float *out, size_t n);
+int launch_f8_block_dequant(oxq_ctx *ctx, hipStream_t s, const F8Problem &p, uint16_t *out);
+int launch_f8_gemv(oxq_ctx *ctx, hipStream_t s, const F8Problem &p);
+bool f8_mm_eligible(const F8Problem &p);
+int launch_f8_mm(oxq_ctx *ctx, hipStream_t s, const F8Problem &p);
 // MXFP4 prefill (plain m > 16, or grouped with many pairs per expert): same tile matmul
 int launch_mxfp4_mm(oxq_ctx *ctx, hipStream_t s, const Mxfp4Problem &p);
 int launch_mxfp4_gemv(oxq_ctx *ctx, hipStream_t s, const Mxfp4Problem &p);

@@ -244,6 +244,39 @@ def rtn_quantize_awq(weight, group_size: int, *, ctx: Optional[Context] = None):
     return qweight, qzeros, scales
 
 
+# ---------------------------------------------------------------- block-scaled F8E4M3
+def cast_f8e4m3_to_f32(t, *, ctx: Optional[Context] = None):
+    """metal_ops.rs:5562: U8 tensor of E4M3 encodings -> F32 of the same shape."""
+    ctx = _ctx(ctx)
+    out = torch.empty(t.shape, dtype=torch.float32, device=t.device)
+    _lib.check(ctx._lib.oxq_cast_f8e4m3_to_f32(ctx.handle, ctx.stream(), desc(t), desc(out)))
+    return out
+
+
+def f8_block_dequant_bf16(bytes_, scales, *, ctx: Optional[Context] = None):
+    """metal_ops.rs:5809: U8 [out, in] + F32 scale grid -> BF16 [out, in]."""
+    ctx = _ctx(ctx)
+    out = torch.empty(tuple(bytes_.shape), dtype=torch.bfloat16, device=bytes_.device)
+    _lib.check(ctx._lib.oxq_f8_block_dequant_bf16(ctx.handle, ctx.stream(), desc(bytes_), desc(scales), desc(out)))
+    return out
+
+
+def f8_gemv(x, bytes_, scales, *, out=None, ctx: Optional[Context] = None):
+    """metal_ops.rs:5788: x BF16 [m <= 8, in] times the block-scaled F8 weight [out, in]."""
+    ctx = _ctx(ctx)
+    out = _out_for(x, bytes_.shape[0], out, ctx)
+    _lib.check(ctx._lib.oxq_f8_gemv(ctx.handle, ctx.stream(), desc(x), desc(bytes_), desc(scales), desc(out)))
+    return out
+
+
+def f8_matmul(x, bytes_, scales, *, out=None, ctx: Optional[Context] = None):
+    """moe.rs:106-113 (Fp8Cached::forward): any m."""
+    ctx = _ctx(ctx)
+    out = _out_for(x, bytes_.shape[0], out, ctx)
+    _lib.check(ctx._lib.oxq_f8_matmul(ctx.handle, ctx.stream(), desc(x), desc(bytes_), desc(scales), desc(out)))
+    return out
+
+
 # ---------------------------------------------------------------- GGUF
 def gguf_block_layout(quant: int):
     e, b = C.c_int64(), C.c_int64()

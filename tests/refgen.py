@@ -154,3 +154,22 @@ def concat_parts(in_features=8, group_size=4, parts_out=(16, 8, 8)):
 def rtn_weight(out_f=16, in_f=64):
     """awq.rs:803-806: sin(0.013 i)."""
     return np.sin(np.arange(out_f * in_f, dtype=np.float32) * np.float32(0.013)).astype(np.float32).reshape(out_f, in_f)
+
+
+def f8_dequant_case(rows=8, cols=256):
+    """metal_ops.rs:4320-4329: bytes (37 i + 11) & 255 with the NaN encodings S.1111.111 moved
+    off (b ^ 0x08), scale grid [2, 2] = 0.5 + 0.75 i."""
+    b = ((np.arange(rows * cols, dtype=np.int64) * 37 + 11) & 0xFF).astype(np.uint8)
+    b = np.where((b & 0x7F) == 0x7F, b ^ 0x08, b).astype(np.uint8)
+    scales = (np.float32(0.5) + np.arange(4, dtype=np.float32) * np.float32(0.75)).reshape(2, 2)
+    return b.reshape(rows, cols), scales
+
+
+def f8_gemv_case(out_f, in_f, s_r, s_c, m):
+    """metal_ops.rs:4388-4396: bytes (29 i + 13) & 255 (NaN encodings moved off),
+    scales 0.2 + (i % 7) * 0.3, x = sin(0.013 i)."""
+    b = ((np.arange(out_f * in_f, dtype=np.int64) * 29 + 13) & 0xFF).astype(np.uint8)
+    b = np.where((b & 0x7F) == 0x7F, b ^ 0x08, b).astype(np.uint8)
+    scales = (np.float32(0.2) + (np.arange(s_r * s_c) % 7).astype(np.float32) * np.float32(0.3)).reshape(s_r, s_c)
+    x = np.sin(np.arange(m * in_f, dtype=np.float32) * np.float32(0.013)).astype(np.float32).reshape(m, in_f)
+    return b.reshape(out_f, in_f), scales, x

@@ -303,7 +303,9 @@ def test_layers_validate_like_reference(lib, ctx):
     q = C.c_void_p()
     w = fake((4096 * 16 * 144,), U8)
     assert lib.oxq_qlinear_new(ctx, _lib.GGUF_Q4_K, C.byref(w), 4096, 4096, None, BF16, C.byref(q)) == 0
-    for m_rows, kern in [(1, "gguf_q4k_gemv_bf16"), (8, "gguf_q4k_gemv_bf16"), (33, "gguf_q4k_mul_mm_bf16")]:
+    # decode rows 1-2: staged GEMV; from 3 rows the tile matmul (up to 8 rows with unrounded weights)
+    for m_rows, kern in [(1, "gguf_q4k_gemv_bf16"), (2, "gguf_q4k_gemv_bf16"), (8, "gguf_q4k_mul_mm_bf16_mt1_f32w"),
+                         (16, "gguf_q4k_mul_mm_bf16_mt1"), (33, "gguf_q4k_mul_mm_bf16_mt4")]:
         assert lib.oxq_qlinear_forward(q, None, C.byref(fake((m_rows, 4096), BF16)),
                                        C.byref(fake((m_rows, 4096), BF16))) == 0, err(lib)
         p = plan(lib, ctx)
@@ -373,3 +375,32 @@ def test_awq_load_time_transforms_validate_like_reference(lib, ctx):
     assert rtn(g=0) == -6
     assert rtn(w=fake((151936, 4096), I32)) == -2
     assert rtn(ro=[ro[0], ro[1], fake((32, 151936), BF16)]) == -2
+
+
+def test_f8_ops_validate_like_reference(lib, ctx):
+    """metal_ops.rs:5589-5613 (dequant), 5703-5731 (gemv), moe.rs:106-113 (any m)."""
+    F32 = _lib.F32
+    b, sc = fake((2048, 512), U8), fake((16, 4), F32)
+    x2, out2 = fake((2, 512), BF16), fake((2, 2048), BF16)
+    assert lib.oxq_f8_gemv(ctx, None, C.byref(x2), C.byref(b), C.byref(sc), C.byref(out2)) == 0, err(lib)
+    p = plan(lib, ctx)
+    assert p.kernel.decode() == "f8_gemv_bf16" and p.grid[0] == 512 and p.launches == 1
+    x, out = fake((4, 512), BF16), fake((4, 2048), BF16)
+    assert lib.oxq_f8_gemv(ctx, None, C.byref(x), C.byref(b), C.byref(sc), C.byref(out)) == 0, err(lib)
+    assert plan(lib, ctx).kernel.decode() == "f8_mul_mm_bf16_mt1"   # from 3 rows: the tile matmul
+    x9, o9 = fake((9, 512), BF16), fake((9, 2048), BF16)
+    assert lib.oxq_f8_gemv(ctx, None, C.byref(x9), C.byref(b), C.byref(sc), C.byref(o9)) == -5
+    assert "m must be 1..=8" in err(lib)
+    assert lib.oxq_f8_matmul(ctx, None, C.byref(x9), C.byref(b), C.byref(sc), C.byref(o9)) == 0, err(lib)
+    assert plan(lib, ctx).kernel.decode().startswith("f8_mul_mm_bf16")
+    assert lib.oxq_f8_gemv(ctx, None, C.byref(fake((4, 512), F16)), C.byref(b), C.byref(sc), C.byref(out)) == -2
+    assert lib.oxq_f8_gemv(ctx, None, C.byref(x), C.byref(b), C.byref(fake((16, 3), F32)), C.byref(out)) == -3
+    assert "scale grid [16, 3] does not tile weight [2048, 512]" in err(lib)
+    assert lib.oxq_f8_gemv(ctx, None, C.byref(x), C.byref(fake((2048, 512), I32)), C.byref(sc), C.byref(out)) == -2
+    dq = fake((2048, 512), BF16)
+    assert lib.oxq_f8_block_dequant_bf16(ctx, None, C.byref(b), C.byref(sc), C.byref(dq)) == 0, err(lib)
+    assert plan(lib, ctx).kernel.decode() == "f8_block_dequant_bf16"
+    assert lib.oxq_f8_block_dequant_bf16(ctx, None, C.byref(b), C.byref(sc), C.byref(fake((2048, 512), F16))) == -3
+    assert lib.oxq_cast_f8e4m3_to_f32(ctx, None, C.byref(b), C.byref(fake((2048, 512), F32))) == 0, err(lib)
+    assert lib.oxq_cast_f8e4m3_to_f32(ctx, None, C.byref(fake((8,), I32)), C.byref(fake((8,), F32))) == -2
+    assert lib.oxq_cast_f8e4m3_to_f32(ctx, None, C.byref(b), C.byref(fake((2048, 511), F32))) == -3

@@ -156,10 +156,19 @@ def test_gguf_gemv_long_rows(fmt):
     data = synth.gguf_weight(fmt, N, K, seed=120 + fmt)
     w = oracle.dequantize_gguf(fmt, data, N, K)
     x = np.random.default_rng(121).standard_normal((m, K)).astype(np.float32)
-    ref = oracle.matmul_nt_f32(round_x(x, oracle.BF16), w)
-    y = ops.gguf_quant_matmul(to_dev(x, torch.bfloat16), to_dev(data), K, N, fmt)
-    assert not ops.default_context().last_plan()["kernel"].endswith("_lds")
+    ref = oracle.matmul_nt_f32(x, w)
+    y = ops.gguf_quant_matmul(to_dev(x), to_dev(data), K, N, fmt)   # f32 activations: always the GEMV kernels
+    kernel = ops.default_context().last_plan()["kernel"]
+    assert kernel.endswith("gemv_f32") and not kernel.endswith("_lds")
     assert_close(y, ref, f"gguf long rows {synth.GGUF_NAMES[fmt]}")
+    # bf16 rows of the decode range take the staged GEMV up to 2 rows and the tile matmul with
+    # unrounded (hi + lo) weights from 3: both are held to the unrounded oracle
+    for mb in (2, 3, 8):
+        xb = x[:mb]
+        yb = ops.gguf_quant_matmul(to_dev(xb, torch.bfloat16), to_dev(data), K, N, fmt)
+        kernel = ops.default_context().last_plan()["kernel"]
+        assert ("gemv" in kernel) if mb <= 2 else kernel.endswith("mul_mm_bf16_mt1_f32w")
+        assert_close(yb, oracle.matmul_nt_f32(round_x(xb, oracle.BF16), w), f"gguf decode rows m={mb}")
 
 
 def test_qlinear_layer_bias_and_routing():

@@ -109,6 +109,40 @@ def test_awq_compressed_tensors_closed_form():
     assert np.max(np.abs(dq - expected)) < 1e-6
 
 
+# ------------------------------------------------------------------ block-scaled F8E4M3
+def test_f8e4m3_decode_every_byte():
+    """metal_ops.rs:2942-2989: the spec decode over all 256 encodings, against torch's own
+    float8_e4m3fn cast (an independent implementation) and against the closed form
+    (-1)^s 2^(e-7) (1 + m/8), subnormals m/8 2^-6, S.1111.111 = NaN, largest finite 448."""
+    import torch
+    b = np.arange(256, dtype=np.uint8)
+    got = oracle.cast_f8e4m3_to_f32(b)
+    ref = torch.from_numpy(b.copy()).view(torch.float8_e4m3fn).to(torch.float32).numpy()
+    nan = np.isnan(ref)
+    assert list(np.nonzero(nan)[0]) == [0x7F, 0xFF] and np.array_equal(np.isnan(got), nan)
+    np.testing.assert_array_equal(got[~nan].view(np.uint32), ref[~nan].view(np.uint32))
+    assert got[0x7E] == 448.0 and got[0xFE] == -448.0 and got[0x01] == 2.0 ** -9 and got[0x38] == 1.0
+    assert got[0x00] == 0.0 and np.signbit(got[0x80]) and got[0x80] == 0.0
+
+
+def test_f8_block_dequant_chain():
+    """metal_ops.rs:4310-4375: F8 -> F32 -> BF16, F32 scale fold, -> BF16, on the reference's
+    bytes and 2 x 2 scale grid, against the same chain written with torch casts."""
+    import torch
+    b, scales = refgen.f8_dequant_case()
+    got = oracle.f8_block_dequant_bf16(b, scales)
+    w = torch.from_numpy(b.copy()).view(torch.float8_e4m3fn).to(torch.float32).to(torch.bfloat16).to(torch.float32)
+    grid = torch.from_numpy(scales).repeat_interleave(b.shape[0] // 2, 0).repeat_interleave(b.shape[1] // 2, 1)
+    want = (w * grid).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    np.testing.assert_array_equal(got, want)
+    # the inner bf16 rounding is the identity on E4M3 values (3 mantissa bits)
+    vals = oracle.cast_f8e4m3_to_f32(np.arange(256, dtype=np.uint8))
+    ok = ~np.isnan(vals)
+    np.testing.assert_array_equal(oracle.round_through(vals[ok], oracle.BF16), vals[ok])
+    with pytest.raises(ValueError):
+        oracle.f8_block_dequant_bf16(b, np.ones((3, 2), np.float32))
+
+
 # ------------------------------------------------------------------ load-time transforms
 def test_compressed_to_awq_matches_direct_dequant():
     """awq.rs:754-800: dequantizing the converted tensors reproduces q * scale exactly; and the
