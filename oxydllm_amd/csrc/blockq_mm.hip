@@ -419,6 +419,9 @@ static int launch_mm_src(oxq_ctx *ctx, hipStream_t s, MmArgs &a, const char *nam
     const size_t lds = (size_t)SRC::LDS_BYTES + (size_t)16 * mt * MM_TP;
     // grouped: sum over experts of ceil(pairs_e / tile) <= pairs / tile + experts
     const int64_t ytiles = grouped ? a.M / (16 * mt) + a.n_experts : ceil_div(a.M, 16 * mt);
+    if (ytiles > 65535)
+        return fail(OXQ_ERR_UNSUPPORTED, "%s mul_mm: %lld token tiles exceed the grid limit of 65535", name_prefix,
+                    (long long)ytiles);
     dim3 grid((unsigned)ceil_div(a.N, MM_BN), (unsigned)ytiles, (unsigned)pl.ks);
     char name[64];
     hilo = hilo && mt == 1 && SRC::HAS_RESIDUE;

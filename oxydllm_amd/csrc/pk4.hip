@@ -663,6 +663,8 @@ int launch_pk4_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p) {
     while (ks > 1 && (size_t)ks * M * p.w.N * 4 > ctx->workspace_bytes) --ks;
     const int gslice = (int)ceil_div(G, ks);
     ks = (int)ceil_div(G, gslice);  // no empty slice
+    if (ceil_div(M, 16 * mt) > 65535)
+        return fail(OXQ_ERR_UNSUPPORTED, "repacked matmul: m = %lld exceeds the grid limit (65535 row tiles)", (long long)M);
     dim3 grid((unsigned)(p.w.N / 64), (unsigned)ks, (unsigned)ceil_div(M, 16 * mt));
     char name[64];
     snprintf(name, sizeof name, "pk%d_mfma_%s_mt%d%s", p.w.bits, p.w.dtype == OXQ_F16 ? "f16" : "bf16", mt,
