@@ -195,6 +195,15 @@ int oxq_rtn_quantize_awq(oxq_ctx *ctx, void *stream, const oxq_tensor *weight, i
                          const oxq_tensor *qweight_out, const oxq_tensor *qzeros_out,
                          const oxq_tensor *scales_out);
 
+/* gguf_weights.rs:255-291 depermute_qk_rows: undoes the per-head row interleave
+ * llama.cpp's converter applies to the q/k projections of Llama-family models
+ * (HF row r of a head is stored at row 2 (r % (head_dim/2)) + r / (head_dim/2));
+ * a row-wise byte shuffle valid for every block format.  `out` must not alias
+ * `weight_bytes`. */
+int oxq_gguf_depermute_qk_rows(oxq_ctx *ctx, void *stream, const oxq_tensor *weight_bytes, int64_t in_features,
+                               int64_t out_features, int quant, int64_t n_heads, int64_t head_dim,
+                               const oxq_tensor *out);
+
 /* ---- block-scaled F8E4M3 (fn variant) ------------------------------------
  * Weight: U8 [out, in] holding E4M3 encodings (1 sign, 4 exponent bits with
  * bias 7, 3 mantissa bits; S.1111.111 is NaN, no infinity); scales: F32

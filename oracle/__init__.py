@@ -121,6 +121,17 @@ def dequantize_awq(qweight, qzeros, scales) -> np.ndarray:
     return out
 
 
+def gguf_depermute_qk_rows(data, row_bytes: int, n_heads: int, head_dim: int) -> np.ndarray:
+    """gguf_weights.rs:255-291: HF row r of a head is read from interleaved row 2 (r % half) + r / half."""
+    rows = np.ascontiguousarray(np.asarray(data, dtype=np.uint8)).reshape(n_heads * head_dim, row_bytes)
+    if head_dim % 2:
+        raise ValueError("depermute_qk_rows: odd head_dim")
+    half = head_dim // 2
+    r = np.arange(head_dim)
+    src = (np.arange(n_heads)[:, None] * head_dim + 2 * (r % half) + r // half).reshape(-1)
+    return rows[src].reshape(-1)
+
+
 def cast_f8e4m3_to_f32(bytes_) -> np.ndarray:
     """metal_ops.rs:2942-2955: spec decode of E4M3fn bytes."""
     b = np.ascontiguousarray(np.asarray(bytes_, dtype=np.uint8))

@@ -70,6 +70,7 @@ SIGNATURES = {
     "oxq_compressed_to_awq": (C.c_int, [_VP, _VP, _TP, _TP, _TP, _TP, _TP]),
     "oxq_concat_awq_along_out": (C.c_int, [_VP, _VP, C.c_int, C.c_int, _TP, _TP, _TP, _TP, _TP, _TP]),
     "oxq_rtn_quantize_awq": (C.c_int, [_VP, _VP, _TP, C.c_int64, _TP, _TP, _TP]),
+    "oxq_gguf_depermute_qk_rows": (C.c_int, [_VP, _VP, _TP, C.c_int64, C.c_int64, C.c_int, C.c_int64, C.c_int64, _TP]),
     "oxq_cast_f8e4m3_to_f32": (C.c_int, [_VP, _VP, _TP, _TP]),
     "oxq_f8_block_dequant_bf16": (C.c_int, [_VP, _VP, _TP, _TP, _TP]),
     "oxq_f8_gemv": (C.c_int, [_VP, _VP, _TP, _TP, _TP, _TP]),

@@ -1,10 +1,11 @@
-// Load-time transforms that produce AWQ-layout tensors on the device:
+// Load-time transforms on the device.  Three produce AWQ-layout tensors:
 //   compressed-tensors int4 (pack-quantized) -> AWQ layout   (awq.rs:187-254 compressed_to_awq)
 //   concatenation of AWQ parts along the output dimension    (awq.rs:256-323 concat_awq_along_out)
 //   round-to-nearest 4-bit group quantization of a dense      (awq.rs:637-742 rtn_quantize_awq)
 //   weight into AWQ tensors
+// and one on GGUF block bytes: the q/k row de-interleave       (gguf_weights.rs:255-291 depermute_qk_rows)
 // The reference runs them on the CPU when a checkpoint is loaded; here the checkpoint tensors
-// are already in HBM, so they are three small kernels.  Integer outputs are bit-exact by
+// are already in HBM, so they are a handful of small kernels.  Integer outputs are bit-exact by
 // construction; the quantizer uses the same f32 operations in the same order as the
 // reference (IEEE division, round half away from zero).
 
@@ -92,6 +93,33 @@ int launch_copy2d_u32(oxq_ctx *ctx, hipStream_t s, const void *src, void *dst, i
     hipLaunchKernelGGL(copy2d_u32_kernel, dim3((unsigned)ceil_div(rows * width, 256)), dim3(256), 0, s,
                        (const uint32_t *)src, (uint32_t *)dst, (int)rows, (int)width, (int)dst_pitch,
                        (int)dst_col);
+    OXQ_HIP_CHECK(hipGetLastError());
+    return OXQ_OK;
+}
+
+// ---- GGUF q/k row de-interleave --------------------------------------------------------
+// gguf_weights.rs:255-291: HF row r of a head sits at interleaved row 2 (r % half) + r / half.
+// Rows are independent runs of blocks, so this is a byte shuffle of whole rows (row lengths
+// are even; copied as 16-bit words).
+__global__ __launch_bounds__(256) void gguf_depermute_rows_kernel(const uint16_t *__restrict__ src,
+                                                                  uint16_t *__restrict__ dst, int head_dim,
+                                                                  int row_words, size_t total_words) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total_words) return;
+    const size_t row = i / row_words, w = i - row * row_words;
+    const int h = (int)(row / head_dim), r = (int)(row % head_dim), half = head_dim >> 1;
+    const size_t srow = (size_t)h * head_dim + 2 * (r % half) + r / half;
+    dst[i] = src[srow * row_words + w];
+}
+
+int launch_gguf_depermute_rows(oxq_ctx *ctx, hipStream_t s, const uint8_t *src, uint8_t *dst, int64_t rows,
+                               int64_t row_bytes, int64_t head_dim) {
+    const size_t words = (size_t)rows * row_bytes / 2;
+    dim3 grid((unsigned)ceil_div((int64_t)words, 256)), block(256);
+    set_plan(ctx, "gguf_depermute_qk_rows", grid, block, 1, 1, 0);
+    if (ctx->plan_only || words == 0) return OXQ_OK;
+    hipLaunchKernelGGL(gguf_depermute_rows_kernel, grid, block, 0, s, (const uint16_t *)src, (uint16_t *)dst,
+                       (int)head_dim, (int)(row_bytes / 2), words);
     OXQ_HIP_CHECK(hipGetLastError());
     return OXQ_OK;
 }

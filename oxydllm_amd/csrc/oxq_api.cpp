@@ -753,6 +753,35 @@ int oxq_rtn_quantize_awq(oxq_ctx *ctx, void *stream, const oxq_tensor *weight, i
                                    (float *)scales_out->data, out_f, in_f, group_size);
 }
 
+// gguf_weights.rs:255-291
+int oxq_gguf_depermute_qk_rows(oxq_ctx *ctx, void *stream, const oxq_tensor *weight_bytes, int64_t in_features,
+                               int64_t out_features, int quant, int64_t n_heads, int64_t head_dim,
+                               const oxq_tensor *out) {
+    const char *op = "depermute_qk_rows";
+    if (!ctx) return fail(OXQ_ERR_ARG, "%s: ctx is NULL", op);
+    int64_t be, bb;
+    if (oxq_gguf_block_layout(quant, &be, &bb) != OXQ_OK) return fail(OXQ_ERR_ARG, "%s: unknown GGUF quant %d", op, quant);
+    OXQ_TRY(check_tensor(ctx, op, "weight_bytes", weight_bytes));
+    OXQ_TRY(check_tensor(ctx, op, "out", out));
+    if (n_heads <= 0 || head_dim <= 0 || out_features != n_heads * head_dim || head_dim % 2 != 0)
+        return fail(OXQ_ERR_SHAPE, "%s: shape [%lld, %lld] incompatible with %lld heads x %lld dims", op,
+                    (long long)out_features, (long long)in_features, (long long)n_heads, (long long)head_dim);
+    if (in_features <= 0 || in_features % be != 0)
+        return fail(OXQ_ERR_SHAPE, "%s: row length %lld not divisible by %s block size %lld", op, (long long)in_features,
+                    gguf_name(quant), (long long)be);
+    const int64_t row_bytes = in_features / be * bb, total = out_features * row_bytes;
+    if (weight_bytes->dtype != OXQ_U8 || out->dtype != OXQ_U8)
+        return fail(OXQ_ERR_DTYPE, "%s: weight_bytes and out must be U8", op);
+    if (!weight_bytes->contiguous || !out->contiguous || numel(weight_bytes) != total || numel(out) != total)
+        return fail(OXQ_ERR_SHAPE, "%s: weight_bytes and out must be contiguous tensors of %lld bytes", op,
+                    (long long)total);
+    if (weight_bytes->data == out->data && total > 0 && !ctx->plan_only)
+        return fail(OXQ_ERR_ARG, "%s: out must not alias weight_bytes", op);
+    if (row_bytes / 2 > INT32_MAX || head_dim > INT32_MAX) return fail(OXQ_ERR_SHAPE, "%s: dimension exceeds 2^31-1", op);
+    return launch_gguf_depermute_rows(ctx, (hipStream_t)stream, (const uint8_t *)weight_bytes->data,
+                                      (uint8_t *)out->data, out_features, row_bytes, head_dim);
+}
+
 // ---- block-scaled F8E4M3 -----------------------------------------------------------
 // metal_ops.rs:5562
 int oxq_cast_f8e4m3_to_f32(oxq_ctx *ctx, void *stream, const oxq_tensor *t, const oxq_tensor *out) {

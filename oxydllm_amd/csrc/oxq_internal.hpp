@@ -153,6 +153,8 @@ int launch_compressed_to_awq(oxq_ctx *ctx, hipStream_t s, const uint32_t *ct, co
                              int64_t out_f, int64_t in_f, int64_t groups);
 int launch_copy2d_u32(oxq_ctx *ctx, hipStream_t s, const void *src, void *dst, int64_t rows, int64_t width,
                       int64_t dst_pitch, int64_t dst_col);
+int launch_gguf_depermute_rows(oxq_ctx *ctx, hipStream_t s, const uint8_t *src, uint8_t *dst, int64_t rows,
+                               int64_t row_bytes, int64_t head_dim);
 int launch_rtn_quantize_awq(oxq_ctx *ctx, hipStream_t s, const void *weight, int dtype, uint32_t *qweight,
                             uint32_t *qzeros, float *scales, int64_t out_f, int64_t in_f, int64_t group_size);
 // block-scaled F8E4M3 (f8_block.hip; the tile matmul for m > 8 lives in blockq_mm.hip)

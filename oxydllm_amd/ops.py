@@ -244,6 +244,16 @@ def rtn_quantize_awq(weight, group_size: int, *, ctx: Optional[Context] = None):
     return qweight, qzeros, scales
 
 
+def gguf_depermute_qk_rows(weight_bytes, in_features: int, out_features: int, quant: int, n_heads: int,
+                           head_dim: int, *, ctx: Optional[Context] = None):
+    """gguf_weights.rs:255-291: block bytes of a q/k projection back in the HF row order."""
+    ctx = _ctx(ctx)
+    out = torch.empty_like(weight_bytes)
+    _lib.check(ctx._lib.oxq_gguf_depermute_qk_rows(ctx.handle, ctx.stream(), desc(weight_bytes), in_features,
+                                                   out_features, quant, n_heads, head_dim, desc(out)))
+    return out
+
+
 # ---------------------------------------------------------------- block-scaled F8E4M3
 def cast_f8e4m3_to_f32(t, *, ctx: Optional[Context] = None):
     """metal_ops.rs:5562: U8 tensor of E4M3 encodings -> F32 of the same shape."""

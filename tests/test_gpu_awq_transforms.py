@@ -179,3 +179,25 @@ def test_rtn_rejects_like_reference():
         ops.rtn_quantize_awq(w, 32)
     with pytest.raises(ops.OxqError, match="not divisible by group_size"):
         ops.rtn_quantize_awq(to_dev(np.zeros((16, 64), np.float32)), 48)
+
+
+@pytest.mark.parametrize("fmt", [synth.GGUF_Q4_K, synth.GGUF_Q8_0, synth.GGUF_Q5_0, synth.GGUF_Q3_K])
+def test_gguf_depermute_qk_rows(fmt):
+    """gguf_weights.rs:255-291, 363-405: bytes equal to the oracle's shuffle; the de-interleaved
+    tensor dequantizes to the HF-ordered rows; bad geometry is rejected as the reference does."""
+    say(f"depermute_qk_rows {synth.GGUF_NAMES[fmt]}")
+    n_heads, head_dim, k = 4, 64, 512
+    n = n_heads * head_dim
+    elems, bbytes = synth.GGUF_BLOCK_LAYOUT[fmt]
+    row_bytes = k // elems * bbytes
+    hf = synth.gguf_weight(fmt, n, k, seed=31 + fmt).reshape(n, row_bytes)
+    permuted = hf.reshape(n_heads, 2, head_dim // 2, row_bytes).swapaxes(1, 2).reshape(-1).copy()
+    got = ops.gguf_depermute_qk_rows(to_dev(permuted), k, n, fmt, n_heads, head_dim)
+    np.testing.assert_array_equal(host(got), oracle.gguf_depermute_qk_rows(permuted, row_bytes, n_heads, head_dim))
+    np.testing.assert_array_equal(host(got).reshape(n, row_bytes), hf)
+    np.testing.assert_array_equal(host(ops.gguf_dequantize(got, k, n, fmt)),
+                                  oracle.dequantize_gguf(fmt, hf.reshape(-1), n, k))
+    with pytest.raises(ops.OxqError, match="incompatible with 3 heads x 64 dims"):
+        ops.gguf_depermute_qk_rows(to_dev(permuted), k, n, fmt, 3, 64)
+    with pytest.raises(ops.OxqError, match="incompatible with 4 heads x 63 dims"):
+        ops.gguf_depermute_qk_rows(to_dev(permuted), k, n, fmt, 4, 63)

@@ -109,6 +109,27 @@ def test_awq_compressed_tensors_closed_form():
     assert np.max(np.abs(dq - expected)) < 1e-6
 
 
+def test_gguf_depermute_qk_rows_inverts_converter_permute():
+    """gguf_weights.rs:363-398: the converter's permute reshape(n_head, 2, hd/2, k).swapaxes(1, 2),
+    applied in HF row space, is undone exactly; here with numpy's own reshape/swapaxes as the
+    independent statement of that permute, on rows of Q4_K blocks."""
+    n_heads, head_dim, k = 2, 8, 512
+    n = n_heads * head_dim
+    row_bytes = k // 256 * 144
+    hf = synth.gguf_weight(synth.GGUF_Q4_K, n, k, seed=77).reshape(n, row_bytes)
+    permuted = hf.reshape(n_heads, 2, head_dim // 2, row_bytes).swapaxes(1, 2).reshape(n, row_bytes)
+    assert not np.array_equal(permuted, hf)
+    restored = oracle.gguf_depermute_qk_rows(permuted.reshape(-1), row_bytes, n_heads, head_dim)
+    np.testing.assert_array_equal(restored.reshape(n, row_bytes), hf)
+    # the reference's loop form of the same permute (gguf_weights.rs:377-386)
+    half = head_dim // 2
+    loop = np.empty_like(hf)
+    for h in range(n_heads):
+        for j in range(head_dim):
+            loop[h * head_dim + j] = hf[h * head_dim + (j % 2) * half + j // 2]
+    np.testing.assert_array_equal(loop, permuted)
+
+
 # ------------------------------------------------------------------ block-scaled F8E4M3
 def test_f8e4m3_decode_every_byte():
     """metal_ops.rs:2942-2989: the spec decode over all 256 encodings, against torch's own
