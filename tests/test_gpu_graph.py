@@ -1,0 +1,98 @@
+"""HIP-graph capture of the hot path: a captured forward must give the eager result on every
+replay, with eager work and synchronizations between replays (captured memset nodes have given
+wrong results on replays after the first on this platform, so nothing here may rely on them;
+the library's launch paths record kernels only).
+"""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from oxydllm_amd import synth
+from tests.helpers import bits_of, to_dev
+
+pytestmark = pytest.mark.gpu
+ops = None
+
+
+def setup_module(module):
+    from oxydllm_amd import ops as _ops
+    module.ops = _ops
+
+
+def say(msg):
+    print(f"[case] {msg}", flush=True)
+    sys.stdout.flush()
+
+
+def replay_matches_eager(name, fn, make_inputs, out):
+    """fn() writes `out` from the current inputs; make_inputs(i) rewrites the inputs in place."""
+    say(f"graph {name}")
+    make_inputs(0)
+    fn()                                  # warm-up: one-time attribute calls happen outside the capture
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        fn()
+    for i in range(1, 5):
+        make_inputs(i)                    # new activations in the same buffers
+        out.zero_()
+        fn()                              # eager reference for these inputs
+        torch.cuda.synchronize()
+        want = bits_of(out).copy()
+        out.zero_()                       # eager work between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(bits_of(out), want, err_msg=f"{name}: replay {i}")
+
+
+@pytest.mark.parametrize("K,N,m", [(4096, 1024, 1), (4096, 1024, 64), (8192, 512, 16)])
+def test_resident_layer_forward_in_a_graph(K, N, m):
+    """(8192, 512): 8 strips, so K is cut into slices and the call is two launches."""
+    trip = synth.awq_checkpoint(K, N, 128, 4, seed=K + N)
+    layer = ops.PackedQuantLinear(4, ops.PACK_OUT, to_dev(trip[0]), to_dev(trip[1]),
+                                  to_dev(trip[2], torch.float16), None, torch.float16)
+    x = torch.empty((m, K), device="cuda", dtype=torch.float16)
+    y = torch.empty((m, N), device="cuda", dtype=torch.float16)
+    gen = torch.Generator(device="cuda")
+
+    def inputs(i):
+        gen.manual_seed(100 + i)
+        x.copy_(torch.randn((m, K), device="cuda", generator=gen).to(torch.float16))
+    replay_matches_eager(f"pk4 {K}x{N} m={m}", lambda: layer.forward(x, out=y), inputs, y)
+    if (K, N) == (8192, 512):
+        assert ops.default_context().last_plan()["launches"] == 2
+
+
+def test_checkpoint_layout_ops_in_a_graph():
+    """The stateless W4A16 op: split-K with the fused last-arriver reduction (counters return to
+    zero by themselves) and with the separate reduction launch."""
+    K, N = 4096, 2048
+    trip = synth.awq_checkpoint(K, N, 128, 4, seed=5)
+    qw, qz, sc = to_dev(trip[0]), to_dev(trip[1]), to_dev(trip[2], torch.float16)
+    for m in (1, 8):
+        x = torch.empty((m, K), device="cuda", dtype=torch.float16)
+        y = torch.empty((m, N), device="cuda", dtype=torch.float16)
+
+        def inputs(i, x=x, m=m):
+            x.copy_(torch.randn((m, K), device="cuda").to(torch.float16) * (1 + i))
+        replay_matches_eager(f"w4a16 op m={m}", lambda: ops.w4a16_matmul(x, qw, qz, sc, out=y), inputs, y)
+
+
+def test_block_quant_paths_in_a_graph():
+    K, N = 2048, 1024
+    data = to_dev(synth.gguf_weight(synth.GGUF_Q4_K, N, K, seed=9))
+    blocks, scales = synth.mxfp4_weight(N, K, seed=10)
+    bd, sd = to_dev(blocks), to_dev(scales)
+    for m in (1, 6, 40):
+        x = torch.empty((m, K), device="cuda", dtype=torch.bfloat16)
+        y = torch.empty((m, N), device="cuda", dtype=torch.bfloat16)
+
+        def inputs(i, x=x, m=m):
+            x.copy_(torch.randn((m, K), device="cuda").to(torch.bfloat16) * (1 + 0.5 * i))
+        layer = ops.QLinear(synth.GGUF_Q4_K, data, K, N, None, torch.bfloat16)
+        replay_matches_eager(f"gguf q4_k m={m}", lambda: layer.forward(x, out=y), inputs, y)
+        replay_matches_eager(f"mxfp4 m={m}", lambda: ops.mxfp4_matmul(x, bd, sd, K, N, out=y), inputs, y)
