@@ -33,6 +33,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 MFMA_F16_PEAK_TFLOPS = 2500.0
 K, N, G = 4096, 14336, 128
+SAMPLES = 11                # timed replays per case; the median is reported
 
 
 def algo_bytes(M: int, k: int = K, n: int = N, g: int = G, bits: int = 4) -> int:
@@ -44,8 +45,9 @@ def algo_bytes(M: int, k: int = K, n: int = N, g: int = G, bits: int = 4) -> int
 
 
 def time_graph(fn_of_step, steps: int, warmup: int, stream):
-    """Capture `steps` consecutive calls into one HIP graph, replay, time with HIP events
-    recorded on the stream the kernels run on.  Returns (wall_ms, event_ms) for `steps` calls."""
+    """Capture `steps` consecutive calls into one HIP graph, replay it SAMPLES times, each
+    replay timed with HIP events recorded on the stream the kernels run on.  Returns the
+    medians (wall_ms, event_ms) for `steps` calls."""
     import torch
     for i in range(warmup):
         fn_of_step(i)
@@ -57,17 +59,20 @@ def time_graph(fn_of_step, steps: int, warmup: int, stream):
     torch.cuda.synchronize()
     graph.replay()          # untimed replay (first replay uploads the graph)
     torch.cuda.synchronize()
-    ev0 = torch.cuda.Event(enable_timing=True)
-    ev1 = torch.cuda.Event(enable_timing=True)
     cur = torch.cuda.current_stream()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    ev0.record(cur)
-    graph.replay()
-    ev1.record(cur)
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3
-    return wall_ms, ev0.elapsed_time(ev1)
+    walls, evs = [], []
+    for _ in range(SAMPLES):   # median of SAMPLES replays of the same `steps` launches
+        ev0 = torch.cuda.Event(enable_timing=True)
+        ev1 = torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        ev0.record(cur)
+        graph.replay()
+        ev1.record(cur)
+        torch.cuda.synchronize()
+        walls.append((time.perf_counter() - t0) * 1e3)
+        evs.append(ev0.elapsed_time(ev1))
+    return float(np.median(walls)), float(np.median(evs))
 
 
 def cpu_baseline(qw, qz, sc, x_f32):
@@ -122,6 +127,10 @@ def main():
     import torch
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
+    from oxydllm_amd import _lib
+    if not os.path.exists(_lib.LIB_PATH):  # load what is built; build only if nothing is
+        from oxydllm_amd import build
+        build.build(force=False)
     from oxydllm_amd import ops, synth
 
     dev = torch.device("cuda:0")
@@ -235,7 +244,7 @@ def main():
                                "(BASELINE configs[1]) through PackedQuantLinear.forward on a resident layer; "
                                "M=16/64 in `cases`; the stateless checkpoint-layout ops in "
                                "`cases_checkpoint_layout_ops`",
-                   "weight_copies_rotated": copies, "timing": "HIP graph of `steps` launches"},
+                   "weight_copies_rotated": copies, "timing": f"HIP graph of `steps` launches, median of {SAMPLES} replays"},
         "roofline": {"bound": "hbm", "achieved": c1["GB_per_s"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(c1["GB_per_s"] / HBM_PEAK_GBS, 4), "traffic": traffic,
                      "kernel": c1["kernel"], "algorithmic_bytes_per_launch": c1["algorithmic_bytes"],
