@@ -52,7 +52,9 @@ typedef enum oxq_status {
     OXQ_ERR_BITS = -8,       /* bits not in {4, 8} */
     OXQ_ERR_RUNTIME = -9,    /* HIP runtime failure */
     OXQ_ERR_WORKSPACE = -10, /* problem needs more split-K workspace than the ctx holds */
-    OXQ_ERR_UNSUPPORTED = -11
+    OXQ_ERR_UNSUPPORTED = -11,
+    OXQ_ERR_IO = -12,    /* a checkpoint file could not be opened or mapped */
+    OXQ_ERR_FORMAT = -13 /* a checkpoint file or JSON text is malformed */
 } oxq_status;
 
 typedef enum oxq_dtype {

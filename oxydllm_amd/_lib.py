@@ -1,4 +1,4 @@
-"""ctypes loader for ``liboxq_hip.so`` (the C ABI declared in ``include/oxq.h``).
+"""ctypes loader for ``liboxq_hip.so`` (the C ABI declared in ``include/oxq.h`` and ``include/oxq_files.h``).
 
 There is no fallback: if the library is missing the import of any op fails with
 an error that says how to build it.
@@ -24,6 +24,7 @@ STATUS = {
     0: "OXQ_OK", -1: "OXQ_ERR_ARG", -2: "OXQ_ERR_DTYPE", -3: "OXQ_ERR_SHAPE",
     -4: "OXQ_ERR_CONTIGUOUS", -5: "OXQ_ERR_M_RANGE", -6: "OXQ_ERR_GROUP", -7: "OXQ_ERR_DEVICE",
     -8: "OXQ_ERR_BITS", -9: "OXQ_ERR_RUNTIME", -10: "OXQ_ERR_WORKSPACE", -11: "OXQ_ERR_UNSUPPORTED",
+    -12: "OXQ_ERR_IO", -13: "OXQ_ERR_FORMAT",
 }
 
 
@@ -37,6 +38,20 @@ class OxqPlan(C.Structure):
     _fields_ = [("kernel", C.c_char * 64), ("grid", C.c_uint32 * 3), ("block", C.c_uint32 * 3),
                 ("split_k", C.c_uint32), ("launches", C.c_uint32),
                 ("workspace_bytes", C.c_uint64)]
+
+
+OXQ_FILE_MAX_RANK = 8
+
+
+class OxqFileTensor(C.Structure):
+    """``oxq_file_tensor`` of include/oxq_files.h."""
+    _fields_ = [("name", C.c_char_p), ("file_dtype", C.c_int32), ("ggml_type", C.c_int32),
+                ("gguf_quant", C.c_int32), ("rank", C.c_int32), ("dims", C.c_int64 * OXQ_FILE_MAX_RANK),
+                ("data", C.c_void_p), ("nbytes", C.c_uint64), ("shard", C.c_int32), ("reserved", C.c_int32)]
+
+
+class OxqQuantScheme(C.Structure):
+    _fields_ = [("kind", C.c_int32), ("bits", C.c_uint32), ("sym", C.c_int32)]
 
 
 class OxqError(RuntimeError):
@@ -101,6 +116,29 @@ SIGNATURES = {
     "oxq_mxfp4_linear_new": (C.c_int, [_VP, _TP, _TP, _TP, C.c_int64, C.c_int64, C.POINTER(_VP)]),
     "oxq_mxfp4_linear_forward": (C.c_int, [_VP, _VP, _TP, _TP]),
     "oxq_mxfp4_linear_free": (None, [_VP]),
+    # include/oxq_files.h
+    "oxq_gguf_open": (C.c_int, [C.POINTER(C.c_char_p), C.c_int, C.POINTER(_VP)]),
+    "oxq_safetensors_open": (C.c_int, [C.POINTER(C.c_char_p), C.c_int, C.POINTER(_VP)]),
+    "oxq_tensor_file_close": (C.c_int, [_VP]),
+    "oxq_tensor_file_count": (C.c_int64, [_VP]),
+    "oxq_tensor_file_at": (C.c_int, [_VP, C.c_int64, C.POINTER(OxqFileTensor)]),
+    "oxq_tensor_file_find": (C.c_int, [_VP, C.c_char_p, C.POINTER(OxqFileTensor), C.POINTER(C.c_int)]),
+    "oxq_tensor_file_total_bytes": (C.c_uint64, [_VP]),
+    "oxq_tensor_file_has_packed_quantized_weights": (C.c_int, [_VP]),
+    "oxq_gguf_metadata_count": (C.c_int64, [_VP]),
+    "oxq_gguf_metadata_at": (C.c_int, [_VP, C.c_int64, C.POINTER(C.c_char_p), C.POINTER(C.c_int),
+                                       C.POINTER(C.c_int), C.POINTER(C.c_uint64)]),
+    "oxq_gguf_metadata_u32": (C.c_int, [_VP, C.c_char_p, C.POINTER(C.c_uint32), C.POINTER(C.c_int)]),
+    "oxq_gguf_metadata_f32": (C.c_int, [_VP, C.c_char_p, C.POINTER(C.c_float), C.POINTER(C.c_int)]),
+    "oxq_gguf_metadata_string": (C.c_int, [_VP, C.c_char_p, C.POINTER(_VP), C.POINTER(C.c_uint64),
+                                           C.POINTER(C.c_int)]),
+    "oxq_gguf_metadata_number": (C.c_int, [_VP, C.c_char_p, C.POINTER(C.c_double), C.POINTER(C.c_int)]),
+    "oxq_gguf_architecture": (C.c_int, [_VP, C.POINTER(_VP), C.POINTER(C.c_uint64), C.POINTER(C.c_int)]),
+    "oxq_gguf_eos_token_ids": (C.c_int, [_VP, C.POINTER(C.c_uint32), C.c_uint64, C.POINTER(C.c_uint64)]),
+    "oxq_validate_quantization_config": (C.c_int, [C.c_char_p, C.c_int, C.POINTER(OxqQuantScheme)]),
+    "oxq_safetensors_try_get_quant": (C.c_int, [_VP, C.POINTER(OxqQuantScheme), C.c_char_p, C.POINTER(OxqFileTensor),
+                                                C.POINTER(OxqFileTensor), C.POINTER(OxqFileTensor), C.POINTER(C.c_int)]),
+    "oxq_upload": (C.c_int, [_VP, _VP, _VP, _VP, C.c_uint64]),
 }
 
 _lib = None

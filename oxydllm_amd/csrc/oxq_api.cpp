@@ -393,6 +393,8 @@ const char *oxq_status_name(int status) {
     case OXQ_ERR_RUNTIME: return "OXQ_ERR_RUNTIME";
     case OXQ_ERR_WORKSPACE: return "OXQ_ERR_WORKSPACE";
     case OXQ_ERR_UNSUPPORTED: return "OXQ_ERR_UNSUPPORTED";
+    case OXQ_ERR_IO: return "OXQ_ERR_IO";
+    case OXQ_ERR_FORMAT: return "OXQ_ERR_FORMAT";
     default: return "OXQ_ERR_?";
     }
 }

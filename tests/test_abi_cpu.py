@@ -40,12 +40,15 @@ def plan(lib, ctx):
 
 
 def test_library_exports_every_declared_symbol(lib):
-    header = open(os.path.join(ROOT, "include", "oxq.h")).read()
-    declared = set(re.findall(r"\b(oxq_[a-z0-9_]+)\s*\(", header))
+    import glob
+    headers = sorted(glob.glob(os.path.join(ROOT, "include", "*.h")))
+    assert [os.path.basename(h) for h in headers] == ["oxq.h", "oxq_files.h"]
+    header = "".join(open(h).read() for h in headers)
+    declared = set(re.findall(r"^(?:int|int64_t|uint64_t|void|const char \*)\s*\*?(oxq_[a-z0-9_]+)\s*\(", header, re.M))
     assert len(declared) >= 30
     missing = [n for n in sorted(declared) if not hasattr(lib, n)]
     assert not missing, f"not exported: {missing}"
-    assert declared == set(_lib.SIGNATURES), "binding table out of sync with include/oxq.h"
+    assert declared == set(_lib.SIGNATURES), "binding table out of sync with include/*.h"
 
 
 def test_version_and_status_names(lib):
