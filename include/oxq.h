@@ -331,6 +331,18 @@ int oxq_packed_quant_linear_new(oxq_ctx *ctx, uint32_t bits, int pack_dim,
                                 const oxq_tensor *qweight, const oxq_tensor *qzeros,
                                 const oxq_tensor *scales, const oxq_tensor *bias_or_null,
                                 int dtype, oxq_packed_quant_linear **out);
+/* ffn.rs:386-400 FeedForward::forward, GateUpProjection::Fused arm: the fused gate|up projection
+ * (qweight etc. of out_features = 2 * intermediate, gate columns first, as concat_awq_along_out builds
+ * it) followed by gated_silu_fused / gated_gelu_tanh_fused (metal_ops.rs, ffn_kernels.metal:19-160),
+ * in one launch.  forward writes act(gate(x)) * up(x), [.., intermediate], and out_features reports
+ * intermediate; both factors are rounded to `dtype` before the activation, so the result equals
+ * oxq_packed_quant_linear_forward followed by oxq_gated_activation bit for bit.  `act` is
+ * OXQ_ACT_GATED_SILU or OXQ_ACT_GATED_GELU_TANH.  Only layers that qualify for the resident copy
+ * (see above) can be built this way; others return OXQ_ERR_UNSUPPORTED and take the two calls. */
+int oxq_packed_quant_linear_new_gate_up(oxq_ctx *ctx, uint32_t bits, int pack_dim, const oxq_tensor *qweight,
+                                        const oxq_tensor *qzeros, const oxq_tensor *scales,
+                                        const oxq_tensor *bias_or_null, int act, int dtype,
+                                        oxq_packed_quant_linear **out);
 int oxq_packed_quant_linear_forward(oxq_packed_quant_linear *layer, void *stream,
                                     const oxq_tensor *x, const oxq_tensor *out);
 int oxq_packed_quant_linear_in_features(const oxq_packed_quant_linear *layer, int64_t *k);

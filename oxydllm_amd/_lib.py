@@ -103,6 +103,8 @@ SIGNATURES = {
     "oxq_moe_combine": (C.c_int, [_VP, _VP, _TP, _TP, _TP, _TP]),
     "oxq_packed_quant_linear_new": (C.c_int, [_VP, C.c_uint32, C.c_int, _TP, _TP, _TP, _TP,
                                               C.c_int, C.POINTER(_VP)]),
+    "oxq_packed_quant_linear_new_gate_up": (C.c_int, [_VP, C.c_uint32, C.c_int, _TP, _TP, _TP, _TP, C.c_int, C.c_int,
+                                                      C.POINTER(_VP)]),
     "oxq_packed_quant_linear_forward": (C.c_int, [_VP, _VP, _TP, _TP]),
     "oxq_packed_quant_linear_in_features": (C.c_int, [_VP, C.POINTER(C.c_int64)]),
     "oxq_packed_quant_linear_out_features": (C.c_int, [_VP, C.POINTER(C.c_int64)]),

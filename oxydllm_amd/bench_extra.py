@@ -67,6 +67,39 @@ def run(ops, ctx, stream, steps, warmup, time_graph):
                              time_graph, wbytes + m * K * 2 + m * N * 2, 2.0 * m * K * N, ctx))
         del d, layers
 
+    # ---- gated FFN entry: fused gate|up projection (config 1's layer twice over) with the activation
+    # in the epilogue, against the projection followed by the activation kernel ------------------------
+    K, I, G = 4096, 14336, 128
+    qw, qz, sc = synth.awq_checkpoint(K, 2 * I, G, 4, seed=0x0A0D11EF)
+    wbytes = qw.nbytes + qz.nbytes + sc.size * 2
+    nc = _copies_for(wbytes, cap=6)
+    plain, fused = [], []
+    for _ in range(nc):
+        t = (torch.from_numpy(qw).to(dev), torch.from_numpy(qz).to(dev), torch.from_numpy(sc).to(dev, torch.float16))
+        plain.append(ops.PackedQuantLinear(4, ops.PACK_OUT, *t, None, torch.float16, ctx=ctx))
+        fused.append(ops.PackedQuantLinear(4, ops.PACK_OUT, *t, None, torch.float16, ctx=ctx,
+                                           gate_up_act=ops.ACT_GATED_SILU))
+        del t
+    for m in (1, 16, 64):
+        x = torch.randn((m, K), device=dev, dtype=torch.float16)
+        y2 = torch.empty((m, 2 * I), device=dev, dtype=torch.float16)
+        y1 = torch.empty((m, I), device=dev, dtype=torch.float16)
+
+        def two(i, x=x, y2=y2, y1=y1):
+            plain[i % nc].forward(x, out=y2)
+            ops.gated_activation(y2, ops.ACT_GATED_SILU, out=y1, ctx=ctx)
+
+        def one(i, x=x, y1=y1):
+            fused[i % nc].forward(x, out=y1)
+        nb = wbytes + m * K * 2 + m * I * 2
+        r = _case(f"awq4 gate|up + SiLU M={m} K={K} I={I} (projection, then activation kernel)", two, steps, warmup,
+                  stream, time_graph, nb + 2 * m * 2 * I * 2, 4.0 * m * K * I, ctx)
+        r["launches"] = 2
+        out.append(r)
+        out.append(_case(f"awq4 gate|up + SiLU M={m} K={K} I={I} (fused epilogue)", one, steps, warmup, stream,
+                         time_graph, nb, 4.0 * m * K * I, ctx))
+    del plain, fused
+
     # ---- config 3: GGUF --------------------------------------------------------
     K = N = 4096
     for fmt in sorted(synth.GGUF_NAMES):

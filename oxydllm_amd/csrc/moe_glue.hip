@@ -160,11 +160,6 @@ __global__ __launch_bounds__(64) void moe_group_kernel(const int32_t *__restrict
 // ---------------------------------------------------------------------------
 // gated activation
 // ---------------------------------------------------------------------------
-__device__ __forceinline__ float silu_f32(float x) { return x / (1.0f + expf(-x)); }
-__device__ __forceinline__ float gelu_tanh_f32(float x) {
-    const float k0 = 0.7978845608028654f, k1 = 0.044715f;
-    return 0.5f * x * (1.0f + tanhf(k0 * (x + k1 * x * x * x)));
-}
 
 template <typename T, int KIND>
 __global__ __launch_bounds__(256) void gated_act_kernel(const T *__restrict__ gu, T *__restrict__ out, size_t n_out,
@@ -179,11 +174,11 @@ __global__ __launch_bounds__(256) void gated_act_kernel(const T *__restrict__ gu
         gate = fminf(gate, limit);
         up = fminf(fmaxf(up, -limit), limit);
         const float sig = 1.0f / (1.0f + expf(-(gate * 1.702f)));
-        r = (up + 1.0f) * (gate * sig);
+        r = mul_f32_rn(up + 1.0f, gate * sig);
     } else {  // [gate | up], ffn_kernels.metal:19-242
         const float g = load_f32(gu, row * 2 * half_n + col);
         const float u = load_f32(gu, row * 2 * half_n + half_n + col);
-        r = (KIND == OXQ_ACT_GATED_SILU ? silu_f32(g) : gelu_tanh_f32(g)) * u;
+        r = mul_f32_rn(KIND == OXQ_ACT_GATED_SILU ? silu_f32(g) : gelu_tanh_f32(g), u);
     }
     store_f32(out, gid, r);
 }

@@ -1115,6 +1115,9 @@ struct oxq_packed_quant_linear {
     // and no longer touches the caller's checkpoint tensors.
     bool prepacked;
     Pk4Weights pk;
+    // 0, or 1 + oxq_gated_act for a fused gate|up layer whose forward applies the gated
+    // activation in the matmul's epilogue: out = act(gate) * up, [.., out_features / 2]
+    int act;
 };
 
 // Load-time repack of an eligible layer.  Shapes the repacked kernels do
@@ -1139,6 +1142,7 @@ static int prepack_layer(oxq_packed_quant_linear *l) {
     l->pk.group_shift = src.group_shift;
     l->pk.dtype = l->dtype;
     l->pk.bits = src.bits;
+    l->pk.gate_half = l->act ? src.N / 2 : 0;
     if (ctx->plan_only) {
         l->prepacked = true;
         return OXQ_OK;
@@ -1179,11 +1183,9 @@ struct oxq_mxfp4_linear {
 
 extern "C" {
 
-int oxq_packed_quant_linear_new(oxq_ctx *ctx, uint32_t bits, int pack_dim,
-                                const oxq_tensor *qweight, const oxq_tensor *qzeros,
-                                const oxq_tensor *scales, const oxq_tensor *bias, int dtype,
-                                oxq_packed_quant_linear **out) {
-    const char *op = "PackedQuantLinear";
+static int new_packed_layer(const char *op, oxq_ctx *ctx, uint32_t bits, int pack_dim, const oxq_tensor *qweight,
+                            const oxq_tensor *qzeros, const oxq_tensor *scales, const oxq_tensor *bias, int dtype,
+                            int act, oxq_packed_quant_linear **out) {
     if (!ctx || !out) return fail(OXQ_ERR_ARG, "%s: NULL argument", op);
     *out = nullptr;
     if (bits != 4 && bits != 8)  // linear.rs:417-419
@@ -1228,14 +1230,37 @@ int oxq_packed_quant_linear_new(oxq_ctx *ctx, uint32_t bits, int pack_dim,
     l->pack_dim = pack_dim;
     l->dtype = dtype;
     l->prepacked = false;
-    l->pk = Pk4Weights{nullptr, nullptr, 0, 0, 0, dtype, (int)bits};
+    l->act = act;
+    l->pk = Pk4Weights{nullptr, nullptr, 0, 0, 0, dtype, (int)bits, 0};
     int rc = prepack_layer(l);
+    if (rc == OXQ_OK && act && !l->prepacked)
+        rc = fail(OXQ_ERR_UNSUPPORTED,
+                  "%s: the fused activation needs a resident layer (in_features and group size multiples of 128, "
+                  "out_features a multiple of 64, at most 128 groups, OXQ_PREPACK not 0); build a plain layer and "
+                  "call oxq_gated_activation on its output instead",
+                  op);
     if (rc != OXQ_OK) {
         oxq_packed_quant_linear_free(l);
         return rc;
     }
     *out = l;
     return OXQ_OK;
+}
+
+int oxq_packed_quant_linear_new(oxq_ctx *ctx, uint32_t bits, int pack_dim,
+                                const oxq_tensor *qweight, const oxq_tensor *qzeros,
+                                const oxq_tensor *scales, const oxq_tensor *bias, int dtype,
+                                oxq_packed_quant_linear **out) {
+    return new_packed_layer("PackedQuantLinear", ctx, bits, pack_dim, qweight, qzeros, scales, bias, dtype, 0, out);
+}
+
+int oxq_packed_quant_linear_new_gate_up(oxq_ctx *ctx, uint32_t bits, int pack_dim, const oxq_tensor *qweight,
+                                        const oxq_tensor *qzeros, const oxq_tensor *scales, const oxq_tensor *bias,
+                                        int act, int dtype, oxq_packed_quant_linear **out) {
+    const char *op = "PackedQuantLinear(gate|up)";
+    if (act != OXQ_ACT_GATED_SILU && act != OXQ_ACT_GATED_GELU_TANH)
+        return fail(OXQ_ERR_ARG, "%s: activation must be OXQ_ACT_GATED_SILU or OXQ_ACT_GATED_GELU_TANH, got %d", op, act);
+    return new_packed_layer(op, ctx, bits, pack_dim, qweight, qzeros, scales, bias, dtype, act + 1, out);
 }
 
 // linear.rs:482-533 PackedQuantLinear::forward
@@ -1246,7 +1271,7 @@ int oxq_packed_quant_linear_forward(oxq_packed_quant_linear *l, void *stream, co
     oxq_tensor x2, o2;
     int64_t m;
     OXQ_TRY(flatten_rows(op, x, l->in_features, &x2, &m));
-    OXQ_TRY(flatten_out(op, out, m, l->out_features, &o2));
+    OXQ_TRY(flatten_out(op, out, m, l->act ? l->out_features / 2 : l->out_features, &o2));
     if (l->prepacked) {
         OXQ_TRY(check_tensor(l->ctx, op, "x", &x2));
         OXQ_TRY(check_tensor(l->ctx, op, "out", &o2));
@@ -1262,6 +1287,7 @@ int oxq_packed_quant_linear_forward(oxq_packed_quant_linear *l, void *stream, co
         q.bias = l->has_bias ? l->bias.data : nullptr;
         q.y = o2.data;
         q.M = m;
+        q.act = l->act;
         q.w = l->pk;
         return launch_pk4_forward(l->ctx, (hipStream_t)stream, q);
     }
@@ -1281,7 +1307,7 @@ int oxq_packed_quant_linear_in_features(const oxq_packed_quant_linear *l, int64_
 }
 int oxq_packed_quant_linear_out_features(const oxq_packed_quant_linear *l, int64_t *n) {
     if (!l || !n) return fail(OXQ_ERR_ARG, "PackedQuantLinear: NULL argument");
-    *n = l->out_features;
+    *n = l->act ? l->out_features / 2 : l->out_features;
     return OXQ_OK;
 }
 int oxq_packed_quant_linear_is_prepacked(const oxq_packed_quant_linear *l, int *prepacked) {

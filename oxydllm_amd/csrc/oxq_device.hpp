@@ -138,6 +138,23 @@ struct BF16Traits {
 };
 
 // E8M0 -> f32 power of two; 0xFF is NaN (mxfp4.rs:25-31), 0 is the subnormal 2^-127.
+// Gate functions of the gated activations (ffn_kernels.metal:5-17), f32 in and out; shared by the
+// stand-alone activation kernel and the fused gate|up epilogue so that both give the same bits.
+// a * b rounded to f32 by one v_mul_f32, kept out of the compiler's sight: otherwise a narrowing
+// conversion that follows may be merged with the multiply into a mixed-precision fma, which rounds
+// once and turns a -0 product into +0, and two kernels finishing the same activation would differ
+// in those bits.  With this the last step is the same everywhere: f32 product, then one narrowing.
+__device__ __forceinline__ float mul_f32_rn(float a, float b) {
+    float r;
+    asm("v_mul_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+__device__ __forceinline__ float silu_f32(float x) { return x / (1.0f + expf(-x)); }
+__device__ __forceinline__ float gelu_tanh_f32(float x) {
+    const float k0 = 0.7978845608028654f, k1 = 0.044715f;
+    return 0.5f * x * (1.0f + tanhf(k0 * (x + k1 * x * x * x)));
+}
+
 __device__ __forceinline__ float e8m0_to_f32(uint32_t s) {
     const uint32_t bits = (s == 0xFFu) ? 0x7FC00000u : (s == 0u ? 0x00400000u : (s << 23));
     return __builtin_bit_cast(float, bits);

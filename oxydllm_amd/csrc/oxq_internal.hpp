@@ -122,13 +122,16 @@ struct Pk4Weights {
     int group_shift;
     int dtype;              // OXQ_F16 / OXQ_BF16
     int bits;               // 4 or 8
+    int64_t gate_half;      // 0, or N/2 for a fused gate|up layer: strip j holds gate columns
+                            // [32j, 32j+32) then up columns [N/2 + 32j, N/2 + 32j + 32)
 };
 
 struct Pk4Problem {
     const void *x;          // [M, K] T
     const void *bias;       // [N] T or nullptr
-    void *y;                // [M, N] T
+    void *y;                // [M, N] T, or [M, N/2] with `act`
     int64_t M;
+    int act;                // 0, or 1 + oxq_gated_act (gate|up layers only): y = act(gate) * up
     Pk4Weights w;
 };
 

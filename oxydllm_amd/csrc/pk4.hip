@@ -81,6 +81,15 @@ template <> struct Pk4T<BF16Traits> {
 
 __device__ __forceinline__ int pk4_kk(int t, int kb) { return ((t >> 1) << 6) + (kb << 4) + ((t & 1) << 3); }
 
+// Resident column -> checkpoint column.  A fused gate|up layer (half = N/2) keeps, in every strip
+// of 64, 32 gate columns followed by the 32 up columns they are multiplied with, so that one
+// workgroup holds both factors of its outputs.
+__device__ __forceinline__ int pk4_src_col(int c, int half) {
+    if (!half) return c;
+    const int j = c >> 6, cc = c & 63;
+    return cc < 32 ? 32 * j + cc : half + 32 * j + (cc - 32);
+}
+
 // ---------------------------------------------------------------------------
 // load-time repack
 // ---------------------------------------------------------------------------
@@ -97,7 +106,8 @@ __device__ __forceinline__ uint32_t src_q(const uint32_t *__restrict__ qw, int k
 
 template <bool GPTQ, int BITS>
 __global__ __launch_bounds__(256) void pk4_prepack_weights_kernel(const uint32_t *__restrict__ qw,
-                                                                  uint32_t *__restrict__ pw, int K, int N) {
+                                                                  uint32_t *__restrict__ pw, int K, int N,
+                                                                  int half) {
     const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
     const size_t total = (size_t)K * N * BITS / 32;
     if (idx >= total) return;
@@ -114,13 +124,13 @@ __global__ __launch_bounds__(256) void pk4_prepack_weights_kernel(const uint32_t
         for (int r = 0; r < 2; ++r)
 #pragma unroll
             for (int f = 0; f < 4; ++f)
-                w |= src_q<GPTQ, BITS>(qw, k + r, 64 * j + 4 * ni + f, N) << (16 * r + 4 * f);
+                w |= src_q<GPTQ, BITS>(qw, k + r, pk4_src_col(64 * j + 4 * ni + f, half), N) << (16 * r + 4 * f);
     } else {
 #pragma unroll
         for (int r = 0; r < 2; ++r)
 #pragma unroll
             for (int c = 0; c < 2; ++c)
-                w |= src_q<GPTQ, BITS>(qw, k + r, 64 * j + 4 * ni + 2 * h + c, N) << (16 * r + 8 * c);
+                w |= src_q<GPTQ, BITS>(qw, k + r, pk4_src_col(64 * j + 4 * ni + 2 * h + c, half), N) << (16 * r + 8 * c);
     }
     pw[idx] = w;
 }
@@ -128,14 +138,14 @@ __global__ __launch_bounds__(256) void pk4_prepack_weights_kernel(const uint32_t
 template <typename TT, bool GPTQ, int BITS>
 __global__ __launch_bounds__(256) void pk4_prepack_zs_kernel(const uint32_t *__restrict__ qz,
                                                              const uint16_t *__restrict__ sc,
-                                                             uint32_t *__restrict__ pzs, int G, int N) {
+                                                             uint32_t *__restrict__ pzs, int G, int N, int half) {
     constexpr int PF = 32 / BITS;
     const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (idx >= (size_t)G * N) return;
     const int f = (int)(idx & 3), ni = (int)((idx >> 2) & 15);
     const size_t jg = idx >> 6;
     const int g = (int)(jg % G), j = (int)(jg / G);
-    const int col = 64 * j + 4 * ni + f;
+    const int col = pk4_src_col(64 * j + 4 * ni + f, half);
     const int c = col % PF;
     const int slot = (GPTQ || BITS == 8) ? c : ((c >> 1) | ((c & 1) << 2));
     const uint32_t z = ((qz[(size_t)g * (N / PF) + col / PF] >> (BITS * slot)) & ((1u << BITS) - 1u)) + (GPTQ ? 1u : 0u);
@@ -151,7 +161,8 @@ __global__ __launch_bounds__(256) void pk4_prepack_zs_kernel(const uint32_t *__r
 template <typename TT, int BITS>
 __global__ __launch_bounds__(256) void pk4_dequant_kernel(const uint32_t *__restrict__ pw,
                                                           const uint32_t *__restrict__ pzs,
-                                                          uint16_t *__restrict__ out, int K, int N, int gshift) {
+                                                          uint16_t *__restrict__ out, int K, int N, int gshift,
+                                                          int half) {
     const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (idx >= (size_t)K * N * BITS / 32) return;
     const int NS = K >> 5, G = K >> gshift;
@@ -172,7 +183,7 @@ __global__ __launch_bounds__(256) void pk4_dequant_kernel(const uint32_t *__rest
         Pk4T<TT>::prep(zs, c0, c1);
         const uint32_t pair = BITS == 4 ? TT::unpack1(w, f, nm) : TT::unpack_bytes(c ? (w >> 8) : w);
         const uint32_t d = Pk4T<TT>::deq(pair, c0, c1);
-        const int col = 64 * j + 4 * ni + f;
+        const int col = pk4_src_col(64 * j + 4 * ni + f, half);
         out[(size_t)k * N + col] = (uint16_t)(d & 0xFFFFu);
         out[(size_t)(k + 1) * N + col] = (uint16_t)(d >> 16);
     }
@@ -233,7 +244,7 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
                                                        const uint16_t *__restrict__ bias,
                                                        uint16_t *__restrict__ y, float *__restrict__ ws,
                                                        int M, int K, int N, int gshift, int gslice,
-                                                       int interleave) {
+                                                       int interleave, int act) {
     typedef MfmaOps<TT> Ops;
     constexpr int NW = 8;
     constexpr int ROWS = 16 * MT;
@@ -484,6 +495,46 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
                 float4_t{acc[mt][0][i], acc[mt][1][i], acc[mt][2][i], acc[mt][3][i]};
     __syncthreads();
 
+    if (act) {
+        // Fused gate|up layer: columns 0..31 of the strip are gate, 32..63 the matching up columns.
+        // thread -> (row, CG gate columns and their up columns); both factors are rounded to the
+        // layer dtype first, as the projection's own output would be (ffn.rs:388-400 runs the
+        // activation on that output), then act(gate) * up in f32 and one rounding.
+        constexpr int CG = MT >= 3 ? 4 : 2;
+        constexpr int TPG = 32 / CG;
+        const int ml = threadIdx.x / TPG, c0 = (threadIdx.x % TPG) * CG;
+        if (ml < ROWS && m0 + ml < M) {
+            const int mt = ml >> 4, r = ml & 15, rb = r >> 2, i = r & 3;
+            const float *redf = (const float *)pk4_lds;
+            float vg[CG], vu[CG];
+#pragma unroll
+            for (int c = 0; c < CG; ++c) vg[c] = vu[c] = 0.f;
+#pragma unroll
+            for (int s = 0; s < NW; ++s) {
+                const float *src = redf + ((s * MT + mt) * 4 + i) * 256 + rb * 64 + c0;
+#pragma unroll
+                for (int c = 0; c < CG; ++c) vg[c] += src[c], vu[c] += src[32 + c];
+            }
+            const int half = N >> 1, n = 32 * j + c0;
+            uint16_t o[CG];
+#pragma unroll
+            for (int c = 0; c < CG; ++c) {
+                float g = vg[c], u = vu[c];
+                if (bias) {
+                    g += TT::to_f32(bias[n + c]);
+                    u += TT::to_f32(bias[half + n + c]);
+                }
+                g = TT::to_f32(TT::from_f32(g));
+                u = TT::to_f32(TT::from_f32(u));
+                o[c] = TT::from_f32(mul_f32_rn(act == 1 ? silu_f32(g) : gelu_tanh_f32(g), u));
+            }
+            uint16_t *dst = y + (size_t)(m0 + ml) * half + n;
+            if (CG == 2) *(uint32_t *)dst = (uint32_t)o[0] | ((uint32_t)o[1] << 16);
+            else *(uint2 *)dst = uint2{(uint32_t)o[0] | ((uint32_t)o[1] << 16), (uint32_t)o[CG - 2] | ((uint32_t)o[CG - 1] << 16)};
+        }
+        return;
+    }
+
     // thread -> (row, CP consecutive columns), every thread busy where the tile allows;
     // partials added in wave order.  A row of a partial tile is 64 consecutive floats.
     constexpr int CP = MT == 1 ? 2 : MT == 2 ? 4 : 8;  // columns per thread
@@ -557,13 +608,14 @@ template <bool GPTQ, int BITS>
 static void pk4_prepack_go(hipStream_t s, dim3 gw, dim3 gz, const Wna16Problem &src, const Pk4Weights &dst, int K,
                            int N, int G) {
     dim3 block(256);
-    hipLaunchKernelGGL((pk4_prepack_weights_kernel<GPTQ, BITS>), gw, block, 0, s, src.qweight, dst.pw, K, N);
+    const int half = (int)dst.gate_half;
+    hipLaunchKernelGGL((pk4_prepack_weights_kernel<GPTQ, BITS>), gw, block, 0, s, src.qweight, dst.pw, K, N, half);
     if (src.dtype == OXQ_F16)
         hipLaunchKernelGGL((pk4_prepack_zs_kernel<F16Traits, GPTQ, BITS>), gz, block, 0, s, src.qzeros,
-                           (const uint16_t *)src.scales, dst.pzs, G, N);
+                           (const uint16_t *)src.scales, dst.pzs, G, N, half);
     else
         hipLaunchKernelGGL((pk4_prepack_zs_kernel<BF16Traits, GPTQ, BITS>), gz, block, 0, s, src.qzeros,
-                           (const uint16_t *)src.scales, dst.pzs, G, N);
+                           (const uint16_t *)src.scales, dst.pzs, G, N, half);
 }
 
 int launch_pk4_prepack(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &src, const Pk4Weights &dst) {
@@ -595,7 +647,7 @@ int launch_pk4_dequant(oxq_ctx *ctx, hipStream_t s, const Pk4Weights &w, void *o
     if (ctx->plan_only) return OXQ_OK;
 #define OXQ_DQ(TTv, Bv)                                                                                     \
     hipLaunchKernelGGL((pk4_dequant_kernel<TTv, Bv>), grid, block, 0, s, w.pw, w.pzs, (uint16_t *)out_kn, \
-                       (int)w.K, (int)w.N, w.group_shift)
+                       (int)w.K, (int)w.N, w.group_shift, (int)w.gate_half)
     if (w.dtype == OXQ_F16) {
         if (w.bits == 4) OXQ_DQ(F16Traits, 4); else OXQ_DQ(F16Traits, 8);
     } else {
@@ -624,7 +676,7 @@ static int pk4_go3(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, 
     hipLaunchKernelGGL((pk4_mfma_kernel<TT, BITS, MT, GS, BPG1, AB, WB>), grid, dim3(512), lds, s,
                        (const uint16_t *)p.x, p.w.pw, p.w.pzs, (const uint16_t *)p.bias, (uint16_t *)p.y,
                        (float *)ctx->workspace, (int)p.M, (int)p.w.K, (int)p.w.N, p.w.group_shift, gslice,
-                       pk4_env("OXQ_PK4_INTERLEAVE", 0));
+                       pk4_env("OXQ_PK4_INTERLEAVE", 0), p.act);
     OXQ_HIP_CHECK(hipGetLastError());
     return OXQ_OK;
 }
@@ -660,6 +712,7 @@ int launch_pk4_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p) {
     if (tiles <= 96 && G >= 64) ks = (int)std::max<int64_t>(1, std::min<int64_t>(256 / tiles, G / 16));
     ks = pk4_env("OXQ_PK4_KS", ks);
     ks = std::max(1, std::min(ks, G));
+    if (p.act) ks = 1;  // the activation needs the whole sum: gate|up layers are wide, one slice fills the chip
     while (ks > 1 && (size_t)ks * M * p.w.N * 4 > ctx->workspace_bytes) --ks;
     const int gslice = (int)ceil_div(G, ks);
     ks = (int)ceil_div(G, gslice);  // no empty slice
@@ -667,8 +720,10 @@ int launch_pk4_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p) {
         return fail(OXQ_ERR_UNSUPPORTED, "repacked matmul: m = %lld exceeds the grid limit (65535 row tiles)", (long long)M);
     dim3 grid((unsigned)(p.w.N / 64), (unsigned)ks, (unsigned)ceil_div(M, 16 * mt));
     char name[64];
-    snprintf(name, sizeof name, "pk%d_mfma_%s_mt%d%s", p.w.bits, p.w.dtype == OXQ_F16 ? "f16" : "bf16", mt,
-             mt == 1 ? "_gs" : "");
+    if (p.act && (!p.w.gate_half || p.act > 2))
+        return fail(OXQ_ERR_ARG, "repacked matmul: activation %d on a layer that is not a fused gate|up layer", p.act);
+    snprintf(name, sizeof name, "pk%d_mfma_%s_mt%d%s%s", p.w.bits, p.w.dtype == OXQ_F16 ? "f16" : "bf16", mt,
+             mt == 1 ? "_gs" : "", p.act == 1 ? "_silu" : p.act == 2 ? "_gelu" : "");
     set_plan(ctx, name, grid, dim3(512), ks, 1, ks > 1 ? (size_t)ks * M * p.w.N * 4 : 0);
     if (ctx->plan_only) {
         if (ks > 1) add_launch(ctx);

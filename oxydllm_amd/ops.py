@@ -411,17 +411,25 @@ class PackedQuantLinear:
     """linear.rs:403-534.  Holds resident packed weights; routes by m."""
 
     def __init__(self, bits: int, pack_dim: int, qweight, qzeros, scales, bias=None,
-                 dtype=torch.float16, ctx: Optional[Context] = None):
+                 dtype=torch.float16, ctx: Optional[Context] = None, gate_up_act: Optional[int] = None):
+        """``gate_up_act`` (ACT_GATED_SILU / ACT_GATED_GELU_TANH) makes this the fused gate|up
+        projection of a gated FFN (ffn.rs:386-400): forward returns act(gate) * up, [.., out/2]."""
         self.ctx = _ctx(ctx)
         self._keep = (qweight, qzeros, scales, bias)
         self.handle = C.c_void_p()
-        _lib.check(self.ctx._lib.oxq_packed_quant_linear_new(
-            self.ctx.handle, bits, pack_dim, desc(qweight), desc(qzeros), desc(scales), desc(bias),
-            _DTYPES[dtype], C.byref(self.handle)))
+        if gate_up_act is None:
+            _lib.check(self.ctx._lib.oxq_packed_quant_linear_new(
+                self.ctx.handle, bits, pack_dim, desc(qweight), desc(qzeros), desc(scales), desc(bias),
+                _DTYPES[dtype], C.byref(self.handle)))
+        else:
+            _lib.check(self.ctx._lib.oxq_packed_quant_linear_new_gate_up(
+                self.ctx.handle, bits, pack_dim, desc(qweight), desc(qzeros), desc(scales), desc(bias),
+                gate_up_act, _DTYPES[dtype], C.byref(self.handle)))
         k, n = C.c_int64(), C.c_int64()
         self.ctx._lib.oxq_packed_quant_linear_in_features(self.handle, C.byref(k))
         self.ctx._lib.oxq_packed_quant_linear_out_features(self.handle, C.byref(n))
         self.in_features, self.out_features = k.value, n.value
+        self.weight_columns = n.value * (2 if gate_up_act is not None else 1)
         self.dtype = dtype
         flag = C.c_int()
         self.ctx._lib.oxq_packed_quant_linear_is_prepacked(self.handle, C.byref(flag))
@@ -441,7 +449,7 @@ class PackedQuantLinear:
         """Dense [in, out] weights in the layer dtype (linear.rs:510-523)."""
         if out is None:
             dev = self._keep[0].device if self._keep[0] is not None else torch.device("cuda", self.ctx.device)
-            out = torch.empty((self.in_features, self.out_features), dtype=self.dtype, device=dev)
+            out = torch.empty((self.in_features, self.weight_columns), dtype=self.dtype, device=dev)
         _lib.check(self.ctx._lib.oxq_packed_quant_linear_dequantize(self.handle, self.ctx.stream(),
                                                                     desc(out)))
         return out

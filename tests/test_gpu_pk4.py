@@ -250,3 +250,71 @@ def test_repacked_layer_survives_freed_checkpoint_tensors():
     x = refgen.batch_x(4, K)
     ref = oracle.matmul_nt_f32(round_x(x, dt), dense("awq", trip, dt))
     assert_close(layer.forward(to_dev(x, torch.float16)), ref, "pk4 after source cleared")
+
+
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("dtn", ["f16", "bf16"])
+@pytest.mark.parametrize("act", ["silu", "gelu"])
+@pytest.mark.parametrize("K,I,g", [(256, 64, 128), (512, 96, 128), (1024, 32, 256)])
+def test_fused_gate_up_activation(kind, dtn, act, K, I, g):
+    """The gate|up layer with the activation in its epilogue (ffn.rs:386-400) against the two-call
+    path it replaces, bit for bit, and against the oracle's gated activation.  Its dense dequant is the plain layer's: the column order of the
+    resident copy is internal."""
+    dt = DT[dtn]
+    N = 2 * I
+    trip, pack_dim = make(kind, K, N, g, seed=3 * K + I)
+    bias = (np.arange(N, dtype=np.float32) % 7 - 3) * np.float32(0.0625)
+    bits = bits_of_kind(kind)
+    tdt = TORCH_DT[dt]
+    kind_id = ops.ACT_GATED_SILU if act == "silu" else ops.ACT_GATED_GELU_TANH
+    for b in (None, bias):
+        plain = layer_of(trip, pack_dim, dt, b, bits=bits)
+        bd = None if b is None else to_dev(b, tdt)
+        fused = ops.PackedQuantLinear(bits, pack_dim, to_dev(trip[0]), to_dev(trip[1]), to_dev(trip[2], tdt), bd, tdt,
+                                      gate_up_act=kind_id)
+        assert fused.prepacked and (fused.in_features, fused.out_features) == (K, I)
+        np.testing.assert_array_equal(bits_of(fused.dequantize()), bits_of(plain.dequantize()))
+        w = dense(kind, trip, dt)
+        rng = np.random.default_rng(K + I)
+        for m in (1, 3, 16, 17, 33, 48, 49, 64, 100):
+            say(f"gate|up {kind} {dtn} {act} K={K} I={I} m={m} bias={b is not None}")
+            x = rng.standard_normal((m, K)).astype(np.float32)
+            xd = to_dev(x, tdt)
+            y = fused.forward(xd)
+            assert y.shape == (m, I)
+            gu = plain.forward(xd)
+            two = ops.gated_activation(gu, kind_id)
+            np.testing.assert_array_equal(bits_of(y), bits_of(two))
+            # the projection itself against the oracle matmul, then the activation on the projection's
+            # own 16-bit output (a last-place difference in a factor would otherwise be amplified by
+            # the gate function's slope: |g|^2 ulp in GeLU's tail)
+            wr = w if m <= 16 else oracle.round_through(w, dt)
+            assert_close(gu, oracle.matmul_nt_f32(round_x(x, dt), wr, b), f"gate|up projection {kind} {dtn} m{m}")
+            ref = oracle.gated_silu(as_f32(gu)) if act == "silu" else oracle.gated_gelu_tanh(as_f32(gu))
+            assert_close(y, ref, f"gate|up {kind} {dtn} {act} m{m}")
+
+
+def test_fused_gate_up_benchmark_shape_and_refusals():
+    K, I, g = 4096, 14336, 128
+    trip = synth.awq_checkpoint(K, 2 * I, g, 4, seed=11)
+    args = (4, ops.PACK_OUT, to_dev(trip[0]), to_dev(trip[1]), to_dev(trip[2], torch.float16), None, torch.float16)
+    plain = ops.PackedQuantLinear(*args)
+    fused = ops.PackedQuantLinear(*args, gate_up_act=ops.ACT_GATED_SILU)
+    rng = np.random.default_rng(2)
+    for m in (1, 16, 64):
+        x = to_dev(rng.standard_normal((m, K)).astype(np.float32), torch.float16)
+        y = fused.forward(x)
+        assert ops.default_context().last_plan()["kernel"].endswith("_silu")
+        assert ops.default_context().last_plan()["launches"] == 1
+        np.testing.assert_array_equal(bits_of(y), bits_of(ops.gated_activation(plain.forward(x), ops.ACT_GATED_SILU)))
+        with pytest.raises(ops.OxqError):
+            fused.forward(x, out=torch.empty((m, 2 * I), dtype=torch.float16, device="cuda"))
+    # a layer that cannot be made resident has no fused form; a non-gated activation kind is refused
+    odd = synth.awq_checkpoint(192, 128, 64, 4, seed=1)
+    with pytest.raises(ops.OxqError) as e:
+        ops.PackedQuantLinear(4, ops.PACK_OUT, to_dev(odd[0]), to_dev(odd[1]), to_dev(odd[2], torch.float16), None,
+                              torch.float16, gate_up_act=ops.ACT_GATED_SILU)
+    assert e.value.status == -11
+    with pytest.raises(ops.OxqError) as e:
+        ops.PackedQuantLinear(*args, gate_up_act=ops.ACT_GPT_OSS_SWIGLU)
+    assert e.value.status == -1
