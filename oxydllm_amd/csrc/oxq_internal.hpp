@@ -143,6 +143,7 @@ int launch_pk4_prepack(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &src, con
 int launch_pk4_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p);
 int launch_pk4_dequant(oxq_ctx *ctx, hipStream_t s, const Pk4Weights &w, void *out_kn);
 int launch_wna16_gemv(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p);
+bool awq4_mfma_ok(const Wna16Problem &p);  // the checkpoint-layout tile kernel takes this problem
 int launch_wna16_mfma(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p);
 int launch_wna16_dequant(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p, void *out_kn);
 int launch_gguf_gemv(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p);

@@ -10,9 +10,9 @@
 // Two kernel families:
 //   *_generic  one packed word per lane per row, f32 math exactly as the
 //              reference writes it; accepts every shape the reference accepts.
-//   awq4_gemv_fast  the bandwidth path for 4-bit AWQ: 128/64/32-bit coalesced
-//              loads, nibbles turned into exact 16-bit floats with one
-//              AND-OR, rows paired so v_dot2_f32_{f16,bf16} does two MACs
+//   awq_gemv_fast / gptq_gemv_fast  the bandwidth path, 4- and 8-bit: 128/64/32-bit
+//              coalesced loads, nibbles or bytes turned into exact 16-bit floats
+//              with one AND-OR, rows paired so v_dot2_f32_{f16,bf16} does two MACs
 //              per lane, zero-point and scale applied once per group.
 //
 // Both split K across workgroups and combine the slices with the
@@ -316,6 +316,10 @@ __global__ __launch_bounds__(256) void gptq_gemv_generic(
 // {x[k], x[k+1]}.  Per group and column the lane then applies
 //     y += s * (acc - (bias + z) * sum_k x[k])
 // which removes both the conversion bias and the zero-point in f32.
+//
+// 8-bit layers run the same kernel with 4 columns per word in identity order: after the
+// same row-pair interleave, bytes 0/2 of a register are one column's pair and bytes 1/3 the next
+// column's (f16: 1024 + q by AND-OR; bf16: through f32).
 // ---------------------------------------------------------------------------
 template <int WPL> struct WordVec;
 template <> struct WordVec<4> {
@@ -339,8 +343,8 @@ template <> struct WordVec<1> {
     }
 };
 
-template <typename TT, int MB, int WPL, int WPG, int GPB, int RPW, int PS>
-__global__ __launch_bounds__(WPG * GPB * 64) void awq4_gemv_fast(
+template <typename TT, int BITS, int MB, int WPL, int WPG, int GPB, int RPW, int PS>
+__global__ __launch_bounds__(WPG * GPB * 64) void awq_gemv_fast(
     const uint16_t *__restrict__ x, const uint32_t *__restrict__ qw,
     const uint32_t *__restrict__ qz, const uint16_t *__restrict__ sc,
     const uint16_t *__restrict__ bias, uint16_t *__restrict__ y, float *__restrict__ ws,
@@ -351,7 +355,8 @@ __global__ __launch_bounds__(WPG * GPB * 64) void awq4_gemv_fast(
     typedef typename WV::type wvec_t;
     constexpr int WAVES = WPG * GPB;
     constexpr int LPR = 64 / RPW;          // lanes per row
-    constexpr int NC = WPL * 8;            // columns per lane
+    constexpr int CPW = 32 / BITS;         // columns per word
+    constexpr int NC = WPL * CPW;          // columns per lane
     constexpr int SLAB_COLS = LPR * NC;
     constexpr int ROWS_PER_CHUNK = 2 * WPG * RPW * PS;
     __shared__ float red[WAVES][SLAB_COLS];
@@ -360,7 +365,7 @@ __global__ __launch_bounds__(WPG * GPB * 64) void awq4_gemv_fast(
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wg = wave / WPG, wr = wave % WPG;  // group slot, row phase (wave-uniform)
     const int cl = lane % LPR, sub = lane / LPR;
-    const int PW = N >> 3;                 // words per row
+    const int PW = N / CPW;                // words per row
     const int rowbytes = PW * 4;
     const int jw = (blockIdx.x * LPR + cl) * WPL;
     const bool valid = jw < PW;
@@ -385,10 +390,20 @@ __global__ __launch_bounds__(WPG * GPB * 64) void awq4_gemv_fast(
     if (valid) {
         for (int g = g0 + wg; g < g1; g += GPB) {
             const wvec_t zw = *(const wvec_t *)(qz + (size_t)g * PW + jw);
-            const uint16_t *srow = sc + (size_t)g * N + (size_t)jw * 8;
-            u32x4_t sv[WPL];
+            const uint16_t *srow = sc + (size_t)g * N + (size_t)jw * CPW;
+            uint32_t sv[WPL][CPW / 2];  // the word's CPW scales, two per register
 #pragma unroll
-            for (int c = 0; c < WPL; ++c) sv[c] = *(const u32x4_t *)(srow + c * 8);  // 8 scales
+            for (int c = 0; c < WPL; ++c) {
+                if constexpr (BITS == 4) {
+                    const u32x4_t v = *(const u32x4_t *)(srow + c * 8);
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) sv[c][q] = v[q];
+                } else {
+                    const uint2 v = *(const uint2 *)(srow + c * 4);
+                    sv[c][0] = v.x;
+                    sv[c][1] = v.y;
+                }
+            }
             float acc[MB][NC];
             float xs[MB];
 #pragma unroll
@@ -416,14 +431,22 @@ __global__ __launch_bounds__(WPG * GPB * 64) void awq4_gemv_fast(
                 for (int t = 0; t < PS; ++t) {
 #pragma unroll
                     for (int c = 0; c < WPL; ++c) {
-                        uint32_t p[8];
-                        TT::unpack4(pack_lo16(wa[t][c], wb[t][c]), p, nm);
-                        TT::unpack4(pack_hi16(wa[t][c], wb[t][c]), p + 4, nm);
+                        uint32_t p[CPW];
+                        const uint32_t lo = pack_lo16(wa[t][c], wb[t][c]), hi = pack_hi16(wa[t][c], wb[t][c]);
+                        if constexpr (BITS == 4) {
+                            TT::unpack4(lo, p, nm);
+                            TT::unpack4(hi, p + 4, nm);
+                        } else {
+                            p[0] = TT::unpack_bytes(lo);
+                            p[1] = TT::unpack_bytes(lo >> 8);
+                            p[2] = TT::unpack_bytes(hi);
+                            p[3] = TT::unpack_bytes(hi >> 8);
+                        }
 #pragma unroll
                         for (int m = 0; m < MB; ++m)
 #pragma unroll
-                            for (int s = 0; s < 8; ++s)
-                                acc[m][c * 8 + s] = TT::dot2(p[s], xp[m][t], acc[m][c * 8 + s]);
+                            for (int s = 0; s < CPW; ++s)
+                                acc[m][c * CPW + s] = TT::dot2(p[s], xp[m][t], acc[m][c * CPW + s]);
                     }
 #pragma unroll
                     for (int m = 0; m < MB; ++m) xs[m] = TT::dot2(TT::ONES, xp[m][t], xs[m]);
@@ -434,16 +457,17 @@ __global__ __launch_bounds__(WPG * GPB * 64) void awq4_gemv_fast(
             for (int c = 0; c < WPL; ++c) {
                 const uint32_t zword = zw[c];
 #pragma unroll
-                for (int s = 0; s < 8; ++s) {
-                    const int col = awq_slot_col(s);
+                for (int s = 0; s < CPW; ++s) {
+                    const int col = BITS == 4 ? awq_slot_col(s) : s;
                     const uint32_t spair = sv[c][col >> 1];
                     const uint16_t sbits = (col & 1) ? (uint16_t)(spair >> 16) : (uint16_t)(spair & 0xFFFFu);
                     const float scale = TT::to_f32(sbits);
-                    const float zb = (float)((zword >> (4 * s)) & 0xFu) + TT::bias(s);
+                    const float zb = (float)((zword >> (BITS * s)) & ((1u << BITS) - 1u)) +
+                                     (BITS == 4 ? TT::bias(s) : TT::BYTE_BIAS);
 #pragma unroll
                     for (int m = 0; m < MB; ++m) {
-                        const float v = fmaf(-zb, xs[m], acc[m][c * 8 + s]);
-                        yacc[m][c * 8 + s] = fmaf(scale, v, yacc[m][c * 8 + s]);
+                        const float v = fmaf(-zb, xs[m], acc[m][c * CPW + s]);
+                        yacc[m][c * CPW + s] = fmaf(scale, v, yacc[m][c * CPW + s]);
                     }
                 }
             }
@@ -466,8 +490,8 @@ __global__ __launch_bounds__(WPG * GPB * 64) void awq4_gemv_fast(
 #pragma unroll
                 for (int c = 0; c < WPL; ++c)
 #pragma unroll
-                    for (int s = 0; s < 8; ++s)
-                        red[wave][cl * NC + c * 8 + awq_slot_col(s)] = yacc[m][c * 8 + s];
+                    for (int s = 0; s < CPW; ++s)
+                        red[wave][cl * NC + c * CPW + (BITS == 4 ? awq_slot_col(s) : s)] = yacc[m][c * CPW + s];
             }
             __syncthreads();
             for (int col = threadIdx.x; col < SLAB_COLS; col += WAVES * 64) {
@@ -508,16 +532,23 @@ __global__ __launch_bounds__(WPG * GPB * 64) void awq4_gemv_fast(
 // One wave owns a whole quantization group (16 word rows at g=128), 8 waves =
 // 8 groups per workgroup, 256 columns per workgroup; K slices go to the workspace.
 // ---------------------------------------------------------------------------
-template <typename TT, int MB>
-__global__ __launch_bounds__(512) void gptq4_gemv_fast(
+//
+// 8-bit layers run the same kernel: a word holds 4 consecutive k, bytes 0/2 and 1/3 become the k
+// pairs (0,2) (1,3) as exact floats (f16: 1024 + q by AND-OR; bf16: through f32), a chunk of 16
+// word rows is 64 k, and the lane's four zeros are one qzeros word.
+template <typename TT, int BITS, int MB>
+__global__ __launch_bounds__(512) void gptq_gemv_fast(
     const uint16_t *__restrict__ x, const uint32_t *__restrict__ qw,
     const uint32_t *__restrict__ qz, const uint16_t *__restrict__ sc,
     const uint16_t *__restrict__ bias, uint16_t *__restrict__ y, float *__restrict__ ws,
     unsigned *__restrict__ counters, int M, int K, int N, int gshift, int gpw, int S, int fused) {
     constexpr int WAVES = 8;
-    constexpr int WR = 16;                 // word rows per chunk (128 k)
-    constexpr int MAXG = 8;                // groups (of >= 128 k) staged per round
-    __shared__ __attribute__((aligned(16))) uint32_t xl[MB][MAXG * WR][4];  // permuted x pairs
+    constexpr int PF = 32 / BITS;          // k per word
+    constexpr int XW = PF / 2;             // x pairs (words) per word row
+    constexpr int WR = 16;                 // word rows per chunk (128 k at 4 bits, 64 k at 8)
+    constexpr int CK = WR * PF;            // k per chunk
+    constexpr int RK = 1024;               // k staged per round
+    __shared__ __attribute__((aligned(16))) uint32_t xl[MB][RK / PF][XW];  // permuted x pairs
     __shared__ float red[WAVES][256];
 
     const int lane = threadIdx.x & 63;
@@ -528,9 +559,8 @@ __global__ __launch_bounds__(512) void gptq4_gemv_fast(
     const int slice = blockIdx.y;
     const int G = K >> gshift;
     const int g0 = slice * gpw, g1 = min(G, g0 + gpw);
-    const int wrows_per_group = (1 << gshift) >> 3;     // word rows per group
     const int rowbytes = N * 4;
-    const __amdgpu_buffer_rsrc_t rs_w = make_rsrc(qw, (uint32_t)(K >> 3) * (uint32_t)rowbytes);
+    const __amdgpu_buffer_rsrc_t rs_w = make_rsrc(qw, (uint32_t)(K / PF) * (uint32_t)rowbytes);
     const int voff_w = n0 * 4;
     const NibbleMasks nm = nibble_masks();
 
@@ -540,34 +570,39 @@ __global__ __launch_bounds__(512) void gptq4_gemv_fast(
 #pragma unroll
         for (int c = 0; c < 4; ++c) yacc[m][c] = 0.0f;
 
-    // rounds of up to MAXG*128 k: stage permuted x, then each wave walks its share
+    // rounds of up to RK k: stage permuted x, then each wave walks its share
     const int k_lo = g0 << gshift, k_hi = g1 << gshift;
-    for (int kr = k_lo; kr < k_hi; kr += MAXG * 128) {
-        const int kr_end = min(k_hi, kr + MAXG * 128);
-        const int nwr = (kr_end - kr) >> 3;            // word rows in this round
+    for (int kr = k_lo; kr < k_hi; kr += RK) {
+        const int kr_end = min(k_hi, kr + RK);
+        const int nwr = (kr_end - kr) / PF;            // word rows in this round
         __syncthreads();
         for (int idx = threadIdx.x; idx < MB * nwr; idx += WAVES * 64) {
             const int m = idx / nwr, r = idx % nwr;
             const int mm = m < M ? m : M - 1;
-            const u32x4_t d = *(const u32x4_t *)(x + (size_t)mm * K + kr + r * 8);
-            u32x4_t o;
-            o[0] = pack_lo16(d[0], d[2]);  // (x0, x4)
-            o[1] = pack_hi16(d[0], d[2]);  // (x1, x5)
-            o[2] = pack_lo16(d[1], d[3]);  // (x2, x6)
-            o[3] = pack_hi16(d[1], d[3]);  // (x3, x7)
-            *(u32x4_t *)(&xl[m][r][0]) = o;
+            if constexpr (BITS == 4) {
+                const u32x4_t d = *(const u32x4_t *)(x + (size_t)mm * K + kr + r * 8);
+                u32x4_t o;
+                o[0] = pack_lo16(d[0], d[2]);  // (x0, x4)
+                o[1] = pack_hi16(d[0], d[2]);  // (x1, x5)
+                o[2] = pack_lo16(d[1], d[3]);  // (x2, x6)
+                o[3] = pack_hi16(d[1], d[3]);  // (x3, x7)
+                *(u32x4_t *)(&xl[m][r][0]) = o;
+            } else {
+                const uint2 d = *(const uint2 *)(x + (size_t)mm * K + kr + r * 4);
+                *(uint2 *)(&xl[m][r][0]) = uint2{pack_lo16(d.x, d.y), pack_hi16(d.x, d.y)};  // (x0, x2) (x1, x3)
+            }
         }
         __syncthreads();
-        // chunks of 16 word rows (128 k) are dealt round-robin to the waves
+        // chunks of 16 word rows are dealt round-robin to the waves
         const int nchunks = nwr / WR;
         for (int ch = wave; ch < nchunks; ch += WAVES) {
-            const int kc = kr + ch * 128;
+            const int kc = kr + ch * CK;
             const int g = kc >> gshift;
             u32x4_t w[WR];
 #pragma unroll
             for (int t = 0; t < WR; ++t)
-                w[t] = __builtin_amdgcn_raw_buffer_load_b128(rs_w, voff_w, ((kc >> 3) + t) * rowbytes, 0);
-            const uint32_t zw = valid ? qz[(size_t)g * (N >> 3) + (n0 >> 3)] : 0u;
+                w[t] = __builtin_amdgcn_raw_buffer_load_b128(rs_w, voff_w, (kc / PF + t) * rowbytes, 0);
+            const uint32_t zw = valid ? qz[(size_t)g * (N / PF) + n0 / PF] : 0u;
             uint2 sv = valid ? *(const uint2 *)(sc + (size_t)g * N + n0) : uint2{0u, 0u};
             float acc[MB][4], xe[MB], xo[MB];
 #pragma unroll
@@ -579,40 +614,62 @@ __global__ __launch_bounds__(512) void gptq4_gemv_fast(
             }
 #pragma unroll
             for (int t = 0; t < WR; ++t) {
-                u32x4_t xp[MB];
+                uint32_t xp[MB][XW];
 #pragma unroll
-                for (int m = 0; m < MB; ++m) xp[m] = *(const u32x4_t *)(&xl[m][ch * WR + t][0]);
+                for (int m = 0; m < MB; ++m) {
+                    if constexpr (BITS == 4) {
+                        const u32x4_t v = *(const u32x4_t *)(&xl[m][ch * WR + t][0]);
 #pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    uint32_t p[4];
-                    TT::unpack4(w[t][c], p, nm);  // pairs (0,4) (1,5) (2,6) (3,7)
-#pragma unroll
-                    for (int m = 0; m < MB; ++m) {
-                        acc[m][c] = TT::dot2(p[0], xp[m][0], acc[m][c]);
-                        acc[m][c] = TT::dot2(p[1], xp[m][1], acc[m][c]);
-                        acc[m][c] = TT::dot2(p[2], xp[m][2], acc[m][c]);
-                        acc[m][c] = TT::dot2(p[3], xp[m][3], acc[m][c]);
+                        for (int q = 0; q < XW; ++q) xp[m][q] = v[q];
+                    } else {
+                        const uint2 v = *(const uint2 *)(&xl[m][ch * WR + t][0]);
+                        xp[m][0] = v.x;
+                        xp[m][1] = v.y;
                     }
                 }
 #pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    uint32_t p[XW];
+                    if constexpr (BITS == 4) {
+                        TT::unpack4(w[t][c], p, nm);  // pairs (0,4) (1,5) (2,6) (3,7)
+                    } else {
+                        p[0] = TT::unpack_bytes(w[t][c]);       // (0,2)
+                        p[1] = TT::unpack_bytes(w[t][c] >> 8);  // (1,3)
+                    }
+#pragma unroll
+                    for (int m = 0; m < MB; ++m)
+#pragma unroll
+                        for (int q = 0; q < XW; ++q) acc[m][c] = TT::dot2(p[q], xp[m][q], acc[m][c]);
+                }
+#pragma unroll
                 for (int m = 0; m < MB; ++m) {
-                    xe[m] = TT::dot2(TT::ONES, xp[m][0], xe[m]);
-                    xe[m] = TT::dot2(TT::ONES, xp[m][2], xe[m]);
-                    xo[m] = TT::dot2(TT::ONES, xp[m][1], xo[m]);
-                    xo[m] = TT::dot2(TT::ONES, xp[m][3], xo[m]);
+                    if constexpr (BITS == 4) {
+                        xe[m] = TT::dot2(TT::ONES, xp[m][0], xe[m]);
+                        xe[m] = TT::dot2(TT::ONES, xp[m][XW - 2], xe[m]);
+                        xo[m] = TT::dot2(TT::ONES, xp[m][1], xo[m]);
+                        xo[m] = TT::dot2(TT::ONES, xp[m][XW - 1], xo[m]);
+                    } else {  // one conversion bias for every byte: a single sum
+                        xe[m] = TT::dot2(TT::ONES, xp[m][0], xe[m]);
+                        xe[m] = TT::dot2(TT::ONES, xp[m][1], xe[m]);
+                    }
                 }
             }
-            // a 128-k chunk lies inside one group (group size >= 128): apply scale / zero
-            const int zsh = (n0 & 7) * 4;
+            // a chunk lies inside one group (group size >= 128): apply scale / zero
+            const int zsh = (n0 % PF) * BITS;
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
                 const uint32_t spair = c < 2 ? sv.x : sv.y;
                 const float scale = TT::to_f32((c & 1) ? (uint16_t)(spair >> 16) : (uint16_t)(spair & 0xFFFFu));
-                const float zp1 = (float)((zw >> (zsh + 4 * c)) & 0xFu) + 1.0f;
+                const float zp1 = (float)((zw >> (zsh + BITS * c)) & ((1u << BITS) - 1u)) + 1.0f;
 #pragma unroll
                 for (int m = 0; m < MB; ++m) {
-                    float v = acc[m][c] - TT::bias(0) * xe[m] - TT::bias(1) * xo[m];
-                    v = fmaf(-zp1, xe[m] + xo[m], v);
+                    float v;
+                    if constexpr (BITS == 4) {
+                        v = acc[m][c] - TT::bias(0) * xe[m] - TT::bias(1) * xo[m];
+                        v = fmaf(-zp1, xe[m] + xo[m], v);
+                    } else {
+                        v = fmaf(-(zp1 + TT::BYTE_BIAS), xe[m], acc[m][c]);
+                    }
                     yacc[m][c] = fmaf(scale, v, yacc[m][c]);
                 }
             }
@@ -668,17 +725,17 @@ static int splitk_fused(const oxq_ctx *ctx, int S) {
 
 static int pick_mb(int64_t M) { return M <= 1 ? 1 : (M <= 2 ? 2 : (M <= 4 ? 4 : 8)); }
 
-template <typename TT, int MB, int WPL, int WPG, int GPB, int RPW, int PS>
-static int launch_awq4_fast_t(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p, int gpw) {
+template <typename TT, int BITS, int MB, int WPL, int WPG, int GPB, int RPW, int PS>
+static int launch_awq_fast_t(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p, int gpw) {
     constexpr int LPR = 64 / RPW;
-    const int PW = (int)(p.N / 8);
+    const int PW = (int)(p.N * BITS / 32);
     const int G = (int)(p.K >> p.group_shift);
     const int S = (int)ceil_div(G, gpw);
     dim3 grid((unsigned)ceil_div(PW, LPR * WPL), (unsigned)S);
     dim3 block(WPG * GPB * 64);
     const uint64_t ws_bytes = S > 1 ? (uint64_t)S * p.M * p.N * 4 : 0;
     char name[64];
-    snprintf(name, sizeof name, "awq4_gemv_fast_%s_m%d_w%d_g%dx%d_r%d_p%d",
+    snprintf(name, sizeof name, "awq%d_gemv_fast_%s_m%d_w%d_g%dx%d_r%d_p%d", BITS,
              TT::DTYPE == 1 ? "f16" : "bf16", MB, WPL, WPG, GPB, RPW, PS);
     set_plan(ctx, name, grid, block, S, 1, ws_bytes);
     if (ctx->plan_only) {
@@ -689,7 +746,7 @@ static int launch_awq4_fast_t(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p
         return fail(OXQ_ERR_WORKSPACE, "w4a16 gemv: needs %llu workspace bytes, ctx holds %zu",
                     (unsigned long long)ws_bytes, ctx->workspace_bytes);
     const int fused = splitk_fused(ctx, S);
-    hipLaunchKernelGGL((awq4_gemv_fast<TT, MB, WPL, WPG, GPB, RPW, PS>), grid, block, 0, s,
+    hipLaunchKernelGGL((awq_gemv_fast<TT, BITS, MB, WPL, WPG, GPB, RPW, PS>), grid, block, 0, s,
                        (const uint16_t *)p.x, p.qweight, p.qzeros, (const uint16_t *)p.scales,
                        (const uint16_t *)p.bias, (uint16_t *)p.y, (float *)ctx->workspace,
                        ctx->counters, (int)p.M, (int)p.K, (int)p.N, p.group_shift, gpw, S, fused);
@@ -701,8 +758,9 @@ static int launch_awq4_fast_t(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p
 }
 
 // Geometry table.  rows per chunk = 2 * WPG * RPW * PS must divide the group size.
-template <typename TT>
-static int launch_awq4_fast(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p) {
+template <typename TT, int BITS>
+static int launch_awq_fast(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p) {
+    constexpr int CPW = 32 / BITS;
     const int mb = pick_mb(p.M);
     const int G = (int)(p.K >> p.group_shift);
     const int gs = (int)p.group_size;
@@ -722,32 +780,32 @@ static int launch_awq4_fast(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p) 
         if (cfg < 0) cfg = gs >= 128 ? 4 : 0;  // measured best on MI355X at K=4096, N=14336
         if (gs >= 128) {
             switch (cfg) {
-            case 1: return launch_awq4_fast_t<TT, 1, 4, 4, 2, 2, 8>(ctx, s, p, gpw_for(1024, 2));
-            case 2: return launch_awq4_fast_t<TT, 1, 4, 4, 4, 4, 4>(ctx, s, p, gpw_for(512, 4));
-            case 4: return launch_awq4_fast_t<TT, 1, 4, 2, 4, 4, 8>(ctx, s, p, gpw_for(512, 4));
-            case 5: return launch_awq4_fast_t<TT, 1, 4, 1, 8, 8, 8>(ctx, s, p, gpw_for(256, 8));
-            case 6: return launch_awq4_fast_t<TT, 1, 4, 1, 4, 8, 8>(ctx, s, p, gpw_for(256, 4));
-            default: return launch_awq4_fast_t<TT, 1, 4, 4, 1, 2, 8>(ctx, s, p, gpw_for(1024, 1));
+            case 1: return launch_awq_fast_t<TT, BITS, 1, 4, 4, 2, 2, 8>(ctx, s, p, gpw_for(1024 * CPW / 8, 2));
+            case 2: return launch_awq_fast_t<TT, BITS, 1, 4, 4, 4, 4, 4>(ctx, s, p, gpw_for(512 * CPW / 8, 4));
+            case 4: return launch_awq_fast_t<TT, BITS, 1, 4, 2, 4, 4, 8>(ctx, s, p, gpw_for(512 * CPW / 8, 4));
+            case 5: return launch_awq_fast_t<TT, BITS, 1, 4, 1, 8, 8, 8>(ctx, s, p, gpw_for(256 * CPW / 8, 8));
+            case 6: return launch_awq_fast_t<TT, BITS, 1, 4, 1, 4, 8, 8>(ctx, s, p, gpw_for(256 * CPW / 8, 4));
+            default: return launch_awq_fast_t<TT, BITS, 1, 4, 4, 1, 2, 8>(ctx, s, p, gpw_for(1024 * CPW / 8, 1));
             }
         }
-        return launch_awq4_fast_t<TT, 1, 4, 4, 1, 2, 4>(ctx, s, p, gpw_for(1024, 1));
+        return launch_awq_fast_t<TT, BITS, 1, 4, 4, 1, 2, 4>(ctx, s, p, gpw_for(1024 * CPW / 8, 1));
     }
     const bool ps8 = gs >= 128;
     if (mb == 2)
-        return ps8 ? launch_awq4_fast_t<TT, 2, 4, 4, 1, 2, 8>(ctx, s, p, gpw_for(1024, 1))
-                   : launch_awq4_fast_t<TT, 2, 4, 4, 1, 2, 4>(ctx, s, p, gpw_for(1024, 1));
+        return ps8 ? launch_awq_fast_t<TT, BITS, 2, 4, 4, 1, 2, 8>(ctx, s, p, gpw_for(1024 * CPW / 8, 1))
+                   : launch_awq_fast_t<TT, BITS, 2, 4, 4, 1, 2, 4>(ctx, s, p, gpw_for(1024 * CPW / 8, 1));
     if (mb == 4)
-        return ps8 ? launch_awq4_fast_t<TT, 4, 2, 4, 1, 2, 8>(ctx, s, p, gpw_for(512, 1))
-                   : launch_awq4_fast_t<TT, 4, 2, 4, 1, 2, 4>(ctx, s, p, gpw_for(512, 1));
-    return ps8 ? launch_awq4_fast_t<TT, 8, 1, 4, 1, 2, 8>(ctx, s, p, gpw_for(256, 1))
-               : launch_awq4_fast_t<TT, 8, 1, 4, 1, 2, 4>(ctx, s, p, gpw_for(256, 1));
+        return ps8 ? launch_awq_fast_t<TT, BITS, 4, 2, 4, 1, 2, 8>(ctx, s, p, gpw_for(512 * CPW / 8, 1))
+                   : launch_awq_fast_t<TT, BITS, 4, 2, 4, 1, 2, 4>(ctx, s, p, gpw_for(512 * CPW / 8, 1));
+    return ps8 ? launch_awq_fast_t<TT, BITS, 8, 1, 4, 1, 2, 8>(ctx, s, p, gpw_for(256 * CPW / 8, 1))
+               : launch_awq_fast_t<TT, BITS, 8, 1, 4, 1, 2, 4>(ctx, s, p, gpw_for(256 * CPW / 8, 1));
 }
 
-static bool awq4_fast_ok(const Wna16Problem &p) {
-    if (p.bits != 4 || p.pack_dim != OXQ_PACK_OUT) return false;
+static bool awq_fast_ok(const Wna16Problem &p) {
+    if ((p.bits != 4 && p.bits != 8) || p.pack_dim != OXQ_PACK_OUT) return false;
     if (p.N % 32 != 0 || p.K % 2 != 0) return false;
     if (p.group_size < 64) return false;  // 2 * WPG * RPW * PS rows per chunk
-    if ((uint64_t)p.K * (uint64_t)(p.N / 2) >= (1ull << 31)) return false;  // 32-bit buffer offsets
+    if ((uint64_t)p.K * (uint64_t)(p.N * p.bits / 8) >= (1ull << 31)) return false;  // 32-bit buffer offsets
     if ((uint64_t)p.M * (uint64_t)p.K * 2 >= (1ull << 31)) return false;
     if (((uintptr_t)p.qweight | (uintptr_t)p.qzeros | (uintptr_t)p.scales) & 15) return false;
     if ((uintptr_t)p.x & 3) return false;
@@ -809,17 +867,17 @@ static int launch_generic_t(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p) 
     return OXQ_OK;
 }
 
-static bool gptq4_fast_ok(const Wna16Problem &p) {
-    if (p.bits != 4 || p.pack_dim != OXQ_PACK_IN) return false;
+static bool gptq_fast_ok(const Wna16Problem &p) {
+    if ((p.bits != 4 && p.bits != 8) || p.pack_dim != OXQ_PACK_IN) return false;
     if (p.N % 8 != 0 || p.K % 128 != 0 || p.group_size < 128) return false;
     if (((uintptr_t)p.qweight | (uintptr_t)p.x) & 15) return false;
     if (((uintptr_t)p.scales) & 7) return false;
-    if ((uint64_t)(p.K / 8) * (uint64_t)p.N * 4 >= (1ull << 31)) return false;
+    if ((uint64_t)(p.K * p.bits / 32) * (uint64_t)p.N * 4 >= (1ull << 31)) return false;
     return true;
 }
 
-template <typename TT>
-static int launch_gptq4_fast(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p) {
+template <typename TT, int BITS>
+static int launch_gptq_fast(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p) {
     const int mb = pick_mb(p.M);
     const int G = (int)(p.K >> p.group_shift);
     const int slabs = (int)ceil_div(p.N, 256);
@@ -831,7 +889,7 @@ static int launch_gptq4_fast(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p)
     dim3 grid((unsigned)slabs, (unsigned)S), block(512);
     const uint64_t ws_bytes = S > 1 ? (uint64_t)S * p.M * p.N * 4 : 0;
     char name[64];
-    snprintf(name, sizeof name, "gptq4_gemv_fast_%s_m%d", TT::DTYPE == 1 ? "f16" : "bf16", mb);
+    snprintf(name, sizeof name, "gptq%d_gemv_fast_%s_m%d", BITS, TT::DTYPE == 1 ? "f16" : "bf16", mb);
     set_plan(ctx, name, grid, block, S, 1, ws_bytes);
     const int fused = splitk_fused(ctx, S);
     if (ctx->plan_only) {
@@ -842,7 +900,7 @@ static int launch_gptq4_fast(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p)
         return fail(OXQ_ERR_WORKSPACE, "gptq gemv: needs %llu workspace bytes, ctx holds %zu",
                     (unsigned long long)ws_bytes, ctx->workspace_bytes);
 #define OXQ_GO(MBv)                                                                               \
-    hipLaunchKernelGGL((gptq4_gemv_fast<TT, MBv>), grid, block, 0, s, (const uint16_t *)p.x,      \
+    hipLaunchKernelGGL((gptq_gemv_fast<TT, BITS, MBv>), grid, block, 0, s, (const uint16_t *)p.x, \
                        p.qweight, p.qzeros, (const uint16_t *)p.scales, (const uint16_t *)p.bias, \
                        (uint16_t *)p.y, (float *)ctx->workspace, ctx->counters, (int)p.M, (int)p.K, \
                        (int)p.N, p.group_shift, gpw, S, fused)
@@ -862,10 +920,22 @@ static int launch_gptq4_fast(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p)
 
 int launch_wna16_gemv(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p) {
     const bool f16 = p.dtype == OXQ_F16;
-    if (gptq4_fast_ok(p) && !env_int("OXQ_FORCE_GENERIC", 0))
-        return f16 ? launch_gptq4_fast<F16Traits>(ctx, s, p) : launch_gptq4_fast<BF16Traits>(ctx, s, p);
-    if (awq4_fast_ok(p) && !env_int("OXQ_FORCE_GENERIC", 0))
-        return f16 ? launch_awq4_fast<F16Traits>(ctx, s, p) : launch_awq4_fast<BF16Traits>(ctx, s, p);
+    // 2..8 rows of f16 on 4-bit AWQ: the matrix-core tile kernel reads the weights once for all
+    // rows (13 - 14 us against 17 - 33 us for the dot2 kernel at 4096 x 14336).  Its B operand is
+    // the dequantized weight rounded to f16, 2^-12 relative: far inside the tolerance; bf16, whose
+    // rounding is 2^-9, keeps the kernel that never rounds the weight.
+    if (p.M >= 2 && f16 && awq4_mfma_ok(p) && env_int("OXQ_GEMV_TILE", 1) && !env_int("OXQ_FORCE_GENERIC", 0))
+        return launch_wna16_mfma(ctx, s, p);
+    if (gptq_fast_ok(p) && !env_int("OXQ_FORCE_GENERIC", 0)) {
+        if (p.bits == 4)
+            return f16 ? launch_gptq_fast<F16Traits, 4>(ctx, s, p) : launch_gptq_fast<BF16Traits, 4>(ctx, s, p);
+        return f16 ? launch_gptq_fast<F16Traits, 8>(ctx, s, p) : launch_gptq_fast<BF16Traits, 8>(ctx, s, p);
+    }
+    if (awq_fast_ok(p) && !env_int("OXQ_FORCE_GENERIC", 0)) {
+        if (p.bits == 4)
+            return f16 ? launch_awq_fast<F16Traits, 4>(ctx, s, p) : launch_awq_fast<BF16Traits, 4>(ctx, s, p);
+        return f16 ? launch_awq_fast<F16Traits, 8>(ctx, s, p) : launch_awq_fast<BF16Traits, 8>(ctx, s, p);
+    }
     if (p.bits == 4)
         return f16 ? launch_generic_t<F16Traits, 4>(ctx, s, p) : launch_generic_t<BF16Traits, 4>(ctx, s, p);
     return f16 ? launch_generic_t<F16Traits, 8>(ctx, s, p) : launch_generic_t<BF16Traits, 8>(ctx, s, p);

@@ -686,7 +686,7 @@ static int launch_awq4_mfma(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p) 
     return OXQ_OK;
 }
 
-static bool awq4_mfma_ok(const Wna16Problem &p) {
+bool awq4_mfma_ok(const Wna16Problem &p) {
     if (p.bits != 4 || p.pack_dim != OXQ_PACK_OUT) return false;
     if ((uint64_t)p.K * (uint64_t)(p.N / 2) >= (1ull << 31)) return false;  // 32-bit buffer offsets
     if ((uint64_t)p.M * (uint64_t)p.K * 2 >= (1ull << 31)) return false;

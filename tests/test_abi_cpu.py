@@ -167,7 +167,7 @@ def test_gptq_validation(lib, ctx):
         name = plan(lib, ctx).kernel.decode()
         assert name.startswith("gptq") and name.endswith("_bf16_m8"), name
         if bits == 8:
-            assert name == "gptq_gemv_generic_w8_bf16_m8"
+            assert name == "gptq8_gemv_fast_bf16_m8"
         bad = fake((K // g, N // pf + 1), I32)
         assert lib.oxq_gptq_matmul(ctx, None, C.byref(x), C.byref(qw), C.byref(bad), C.byref(sc),
                                    bits, C.byref(out)) == -3

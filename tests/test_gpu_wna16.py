@@ -351,3 +351,36 @@ def test_packed_quant_linear_bias_and_leading_dims():
         assert_close(y.reshape(m, N), ref, f"layer bias {shape}")
     with pytest.raises(ops.OxqError, match="input last dim"):
         layer.forward(to_dev(refgen.batch_x(1, K - 32), torch.float16))
+
+
+# ------------------------------------------------------------------ 8-bit fast kernels
+@pytest.mark.parametrize("method", ["awq", "gptq"])
+@pytest.mark.parametrize("dtn", ["f16", "bf16"])
+@pytest.mark.parametrize("K,N,g", [(256, 128, 128), (1024, 96, 256), (1280, 544, 128), (5120, 1024, 128)])
+def test_8bit_fast_gemv(method, dtn, K, N, g, monkeypatch):
+    """The 8-bit stateless ops on the checkpoint layout run the same fast kernels as the 4-bit
+    ones (word = 4 columns / 4 consecutive k); every m of the decode range, ragged column tiles
+    (N = 96, 544), several K slices, and the generic kernel on the same inputs as a second opinion."""
+    dt = DT[dtn]
+    make = synth.awq_checkpoint if method == "awq" else synth.gptq_checkpoint
+    qw, qz, sc = make(K, N, g, 8, seed=K + N)
+    d = dev_triplet(qw, qz, sc, dt)
+    s_r = oracle.round_through(sc, dt)
+    w = oracle.dequantize_awq8(qw, qz, s_r) if method == "awq" else oracle.dequantize_gptq(qw, qz, s_r, 8)
+    op = (lambda x: ops.w8a16_matmul(x, *d)) if method == "awq" else (lambda x: ops.gptq_matmul(x, *d, 8))
+    rng = np.random.default_rng(K * 3 + N)
+    for m in (1, 2, 3, 4, 7, 8):
+        say(f"8-bit fast {method} {dtn} K={K} N={N} g={g} m={m}")
+        x = rng.standard_normal((m, K)).astype(np.float32)
+        xd = to_dev(x, TORCH_DT[dt])
+        monkeypatch.delenv("OXQ_FORCE_GENERIC", raising=False)
+        y = op(xd)
+        kern = ops.default_context().last_plan()["kernel"]
+        assert kern.startswith(f"{method}8_gemv_fast_{dtn}"), kern
+        assert_close(y, oracle.matmul_nt_f32(round_x(x, dt), w), f"{method}8 fast {dtn} m{m}")
+        np.testing.assert_array_equal(bits_of(op(xd)), bits_of(y))          # run-to-run
+        monkeypatch.setenv("OXQ_FORCE_GENERIC", "1")
+        yg = op(xd)
+        assert "generic" in ops.default_context().last_plan()["kernel"]
+        # two roundings of nearly equal sums may land one output ulp apart
+        assert_close(y, as_f32(yg), f"{method}8 fast vs generic {dtn} m{m}", rtol=RTOL + (2.0 ** -7 if dtn == "bf16" else 2.0 ** -10))
