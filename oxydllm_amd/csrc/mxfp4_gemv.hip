@@ -257,7 +257,8 @@ __global__ __launch_bounds__(256) void mxfp4_mfma_kernel(
     const uint8_t *__restrict__ scales, const uint16_t *__restrict__ bias,
     uint16_t *__restrict__ y, const int32_t *__restrict__ offsets,
     const int32_t *__restrict__ token_ids, int M, int K, int N) {
-    extern __shared__ __attribute__((aligned(16))) unsigned char mm_lds[];  // [K/8 chunks][MTOK] x 16 B
+    // [K/8 chunks][MTOK] x 16 B of tokens, then per wave the scale bytes of its 16*FR rows
+    extern __shared__ __attribute__((aligned(16))) unsigned char mm_lds[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int ni = lane & 15, kb = lane >> 4;
     const int e = blockIdx.y;
@@ -270,79 +271,142 @@ __global__ __launch_bounds__(256) void mxfp4_mfma_kernel(
     const int nb = K >> 5, cpr = K >> 3;
     const int NT = (nb + 15) >> 4;  // tiles of 16 blocks
     const int n_base = (blockIdx.x * 4 + wave) * (16 * FR);
+    const int nrows = min(16 * FR, N - n_base);  // rows of this wave inside the matrix (<= 0: none)
+    const bool active = nrows > 0;               // wave-uniform
+    // Loads are issued row-major: lane (lr = lane / 4, lc = lane % 4) fetches block 16T + 4j + lc of
+    // row lr, so four neighbouring lanes read 64 contiguous bytes (16 separate 16-byte requests per
+    // row would reach 4.8 TB/s where this reaches 5.5).  The matrix core wants lane (ni, kb) to hold
+    // row ni: a 4 x 16 lane transpose (ds_bpermute, no LDS memory) at the point of use gives lane
+    // (ni, kb) the block 16T + 4j + kb of row ni.
+    const int lr = lane >> 2, lc = lane & 3;
+    const int tr_src = (4 * ni + kb) * 4;  // byte index of the lane whose register this lane needs
     const u32x4_t *wrow[FR];
-    const uint8_t *srow[FR];
 #pragma unroll
     for (int f = 0; f < FR; ++f) {
-        const int n = n_base + 16 * f + ni;
+        const int n = n_base + 16 * f + lr;
         const size_t row = (size_t)e * N + (n < N ? n : N - 1);
         wrow[f] = (const u32x4_t *)blocks + row * nb;
-        srow[f] = scales + row * nb;
     }
     const int a_tok = (ni & (MTOK - 1)) * 16;
+    // token chunks in LDS: quarter sq (16 bytes of every token) of block b
+    auto tok_chunk = [](int b, int sq) { return (b * 4 + sq) * (MTOK * 16); };
+
+    constexpr int D = 2;  // weight tiles in registers: one in use, D - 1 in flight (3 measured the same)
+    u32x4_t wq[D][FR][4];
+    auto load_tile = [&](int T, u32x4_t (&w)[FR][4]) {
+#pragma unroll
+        for (int f = 0; f < FR; ++f)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int b = 16 * T + 4 * j + lc;
+                w[f][j] = wrow[f][b < nb ? b : nb - 1];
+            }
+    };
+    // the first weight tiles do not depend on the tokens: they are requested before those are staged
+    if (active) {
+#pragma unroll
+        for (int d = 0; d < D - 1; ++d)
+            if (d < NT) load_tile(d, wq[d]);
+    }
+
+    // The wave's scale bytes (rows n_base .. n_base + nrows - 1 are contiguous, nb bytes each): one
+    // coalesced pass of aligned 32-bit loads into LDS instead of four single-byte loads per lane and
+    // tile.  The first and last word may reach up to 3 bytes outside the range; an aligned word that
+    // holds a byte of the tensor lies in the same page as that byte.
+    unsigned char *sc_lds = mm_lds + (size_t)MTOK * K * 2 + (size_t)wave * (16 * FR * nb + 16);
+    int sc_mis = 0;
+    if (active) {
+        const uint8_t *s0 = scales + ((size_t)e * N + n_base) * nb;
+        sc_mis = (int)((uintptr_t)s0 & 3);
+        const uint32_t *s32 = (const uint32_t *)(s0 - sc_mis);
+        const int words = (sc_mis + nrows * nb + 3) >> 2;
+        for (int i = lane; i < words; i += 64) ((uint32_t *)sc_lds)[i] = s32[i];
+    }
+    // per fragment: where this lane's row (clamped to the wave's last valid row) starts in sc_lds
+    int sc_row[FR];
+#pragma unroll
+    for (int f = 0; f < FR; ++f) sc_row[f] = sc_mis + min(16 * f + ni, max(nrows, 1) - 1) * nb;
 
     for (int pbase = p0; pbase < p1; pbase += MTOK) {
         const int rows = min(MTOK, p1 - pbase);
-        if (pbase > p0) __syncthreads();  // everyone is done with the previous tokens
+        if (pbase > p0) {
+            __syncthreads();  // everyone is done with the previous tokens
+            if (active) {
+#pragma unroll
+                for (int d = 0; d < D - 1; ++d)
+                    if (d < NT) load_tile(d, wq[d]);
+            }
+        }
         for (int c = threadIdx.x; c < rows * cpr; c += 256) {
             const int m = c / cpr, cc = c - m * cpr;
             const int p = pbase + m;
             const int src = token_ids ? token_ids[p] : p;
-            *(u32x4_t *)(mm_lds + ((size_t)cc * MTOK + m) * 16) = *(const u32x4_t *)(x + (size_t)src * K + (size_t)cc * 8);
+            *(u32x4_t *)(mm_lds + tok_chunk(cc >> 2, cc & 3) + m * 16) = *(const u32x4_t *)(x + (size_t)src * K + (size_t)cc * 8);
         }
         __syncthreads();
+        if (!active) continue;  // wave-uniform; the barriers above are reached by every wave
 
         float4_t acc[FR];
 #pragma unroll
         for (int f = 0; f < FR; ++f) acc[f] = float4_t{0.f, 0.f, 0.f, 0.f};
-        u32x4_t wq[2][FR][4];
-        uint32_t sb[2][FR][4];
-        auto load_tile = [&](int T, u32x4_t (&w)[FR][4], uint32_t (&sc)[FR][4]) {
+        for (int T0 = 0; T0 < NT; T0 += D) {
 #pragma unroll
-            for (int f = 0; f < FR; ++f)
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int b = 16 * T + 4 * kb + j;
-                    const int bc = b < nb ? b : nb - 1;
-                    w[f][j] = wrow[f][bc];
-                    sc[f][j] = srow[f][bc];
-                }
-        };
-        load_tile(0, wq[0], sb[0]);
-        for (int T0 = 0; T0 < NT; T0 += 2) {
-#pragma unroll
-            for (int par = 0; par < 2; ++par) {
+            for (int par = 0; par < D; ++par) {
                 const int T = T0 + par;
                 if (T < NT) {  // block-uniform
-                    if (T + 1 < NT) load_tile(T + 1, wq[par ^ 1], sb[par ^ 1]);
+                    if (T + D - 1 < NT) load_tile(T + D - 1, wq[(par + D - 1) % D]);
+                    // Lane transposes and scale reads in batches of two blocks, activation reads in batches
+                    // of one block: a wave waits for LDS six times a tile, not once per fragment.
+                    const bool ragged = T == NT - 1 && (nb & 15);  // wave-uniform: only the last tile can be
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        const int b = 16 * T + 4 * kb + j;
-                        const bool valid = b < nb;  // blocks past the row contribute zero
-                        float scf[FR];
-                        uint32_t wj[FR][4];
+                    for (int jh = 0; jh < 4; jh += 2) {
+                        uint32_t wp[FR][2][4];
+                        float scf[FR][2];
+                        int bcl[2];
 #pragma unroll
-                        for (int f = 0; f < FR; ++f) {
-                            scf[f] = e8m0_to_f32(sb[par][f][j]);
-                            const u32x4_t t = wq[par][f][j];
-                            const uint32_t t0 = t[0], t1 = t[1], t2 = t[2], t3 = t[3];
-                            wj[f][0] = valid ? t0 : 0u, wj[f][1] = valid ? t1 : 0u;
-                            wj[f][2] = valid ? t2 : 0u, wj[f][3] = valid ? t3 : 0u;
+                        for (int jj = 0; jj < 2; ++jj) {
+                            const int b = 16 * T + 4 * (jh + jj) + kb;
+                            bcl[jj] = b < nb ? b : nb - 1;  // blocks past the row: a finite chunk, weights zeroed below
                         }
-                        const int bcl = valid ? b : nb - 1;  // a finite activation chunk for padding blocks
 #pragma unroll
-                        for (int sq = 0; sq < 4; ++sq) {
-                            const u32x4_t av = *(const u32x4_t *)(mm_lds + (size_t)(4 * bcl + sq) * MTOK * 16 + a_tok);
+                        for (int f = 0; f < FR; ++f)
 #pragma unroll
-                            for (int f = 0; f < FR; ++f) {
-                                const uint32_t w = wj[f][sq];
-                                u32x4_t bv;
-                                bv[0] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scf[f], 0));
-                                bv[1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scf[f], 1));
-                                bv[2] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scf[f], 2));
-                                bv[3] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scf[f], 3));
-                                acc[f] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av),
-                                                                                __builtin_bit_cast(bf16x8_t, bv), acc[f], 0, 0, 0);
+                            for (int jj = 0; jj < 2; ++jj) {
+                                const u32x4_t t = wq[par][f][jh + jj];
+#pragma unroll
+                                for (int q = 0; q < 4; ++q)
+                                    wp[f][jj][q] = (uint32_t)__builtin_amdgcn_ds_bpermute(tr_src, (int)t[q]);
+                                scf[f][jj] = e8m0_to_f32(sc_lds[sc_row[f] + bcl[jj]]);
+                            }
+                        if (ragged) {
+#pragma unroll
+                            for (int jj = 0; jj < 2; ++jj) {
+                                const bool valid = 16 * T + 4 * (jh + jj) + kb < nb;
+#pragma unroll
+                                for (int f = 0; f < FR; ++f)
+#pragma unroll
+                                    for (int q = 0; q < 4; ++q) wp[f][jj][q] = valid ? wp[f][jj][q] : 0u;
+                            }
+                        }
+#pragma unroll
+                        for (int jj = 0; jj < 2; ++jj) {
+                            u32x4_t av[4];
+#pragma unroll
+                            for (int sq = 0; sq < 4; ++sq)
+                                av[sq] = *(const u32x4_t *)(mm_lds + tok_chunk(bcl[jj], sq) + a_tok);
+#pragma unroll
+                            for (int sq = 0; sq < 4; ++sq) {
+#pragma unroll
+                                for (int f = 0; f < FR; ++f) {
+                                    const uint32_t w = wp[f][jj][sq];
+                                    u32x4_t bv;
+                                    bv[0] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scf[f][jj], 0));
+                                    bv[1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scf[f][jj], 1));
+                                    bv[2] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scf[f][jj], 2));
+                                    bv[3] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scf[f][jj], 3));
+                                    acc[f] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av[sq]),
+                                                                                    __builtin_bit_cast(bf16x8_t, bv), acc[f], 0, 0, 0);
+                                }
                             }
                         }
                     }
@@ -425,8 +489,10 @@ int launch_mxfp4_gemv(oxq_ctx *ctx, hipStream_t s, const Mxfp4Problem &p) {
         const int variant = v ? atoi(v) : 0;  // 0 = matrix cores, 1 = dot2 with staged tokens, 2 = one wave per row
         const int mtok = (grouped || p.M <= 4) ? 4 : 16;
         const char *frs = getenv("OXQ_MXFP4_FR");
-        const int FR = frs ? atoi(frs) : 1;
-        const size_t lds = (size_t)mtok * (size_t)p.K * 2;
+        int FR = frs ? atoi(frs) : 1;
+        FR = FR >= 4 ? 4 : FR >= 2 ? 2 : 1;  // the instantiated fragment counts
+        // tokens, then the four waves' scale bytes (16 * FR rows of K / 32 bytes, + alignment slack)
+        const size_t lds = (size_t)mtok * (size_t)p.K * 2 + 4 * ((size_t)16 * FR * (size_t)(p.K >> 5) + 16);
         if (variant == 0 && lds <= 128 * 1024 && p.K % 32 == 0) {
             dim3 grid((unsigned)ceil_div(p.N, 4 * 16 * FR), grouped ? (unsigned)p.n_experts : 1u), block(256);
             char name[64];
