@@ -281,8 +281,7 @@ __global__ __launch_bounds__(512) void gguf_gemv_lds_kernel(const void *__restri
     const int upitch = (K >> 5) + 1;                                  // chunk pitch (units + 1)
     const size_t xrow_bytes = (size_t)CPU * upitch * 16;
     unsigned char *lds_x = gg_lds;                                   // [MB] chunked activations
-    float *lds_sx = (float *)(gg_lds + (size_t)MB * xrow_bytes);      // [MB][K/16] sums of 16
-    unsigned char *lds_w = (unsigned char *)(lds_sx + (size_t)MB * (K >> 4));
+    unsigned char *lds_w = gg_lds + (size_t)MB * xrow_bytes;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n0 = blockIdx.x * rpwg;
     const int nrows = min(rpwg, N - n0);
@@ -339,19 +338,6 @@ __global__ __launch_bounds__(512) void gguf_gemv_lds_kernel(const void *__restri
         }
     }
     __syncthreads();
-    for (int c = threadIdx.x; c < M * (K >> 4); c += nthr) {  // sums of x over 16 elements
-        const int m = c / (K >> 4), h = c - m * (K >> 4);
-        float xa[8], xb[8];
-        ld_x8<BF16X>(lds_x + m * xrow_bytes, upitch, h >> 1, 2 * (h & 1), xa);
-        ld_x8<BF16X>(lds_x + m * xrow_bytes, upitch, h >> 1, 2 * (h & 1) + 1, xb);
-        float sum = 0.0f;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) sum += xa[i];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) sum += xb[i];
-        lds_sx[c] = sum;
-    }
-    __syncthreads();
     for (int r = wave; r < nrows; r += nwaves) {
         const uint8_t *row = lds_w + head + (size_t)r * row_bytes;
         const int n = n0 + r;
@@ -364,19 +350,20 @@ __global__ __launch_bounds__(512) void gguf_gemv_lds_kernel(const void *__restri
 #pragma unroll
             for (int m = 0; m < MB; ++m) {
                 if (m < M) {
-                    float dot0 = 0.0f, dot1 = 0.0f;
+                    // the sums of x over each half of the unit ride along with the dot products: the
+                    // lane reads these 32 activations anyway, and a separate pass would cost a barrier
+                    float dot0 = 0.0f, dot1 = 0.0f, sx0 = 0.0f, sx1 = 0.0f;
 #pragma unroll
                     for (int o = 0; o < 4; ++o) {
                         float xv[8];
                         ld_x8<BF16X>(lds_x + m * xrow_bytes, upitch, u, o, xv);
 #pragma unroll
                         for (int i = 0; i < 8; ++i) {
-                            if (o < 2) dot0 = fmaf(q[8 * o + i], xv[i], dot0);
-                            else dot1 = fmaf(q[8 * o + i], xv[i], dot1);
+                            if (o < 2) dot0 = fmaf(q[8 * o + i], xv[i], dot0), sx0 += xv[i];
+                            else dot1 = fmaf(q[8 * o + i], xv[i], dot1), sx1 += xv[i];
                         }
                     }
-                    const float *sx = lds_sx + (size_t)m * (K >> 4) + 2 * u;
-                    acc[m] += (c0 * dot0 + c1 * dot1) - (d0 * sx[0] + d1 * sx[1]);
+                    acc[m] += (c0 * dot0 + c1 * dot1) - (d0 * sx0 + d1 * sx1);
                 }
             }
         }
@@ -483,8 +470,7 @@ int launch_gguf_gemv(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p) {
     // LDS variant: activations of one chunk of rows plus `rpwg` weight rows must fit 64 KB
     const int64_t mrows = p.M < 8 ? p.M : 8;
     const int mb = mrows <= 1 ? 1 : mrows <= 2 ? 2 : mrows <= 4 ? 4 : 8;
-    const size_t x_lds = (size_t)mb * (32 * xb / 16) * (size_t)((p.K >> 5) + 1) * 16 +
-                         (size_t)mb * (size_t)(p.K >> 4) * 4;
+    const size_t x_lds = (size_t)mb * (32 * xb / 16) * (size_t)((p.K >> 5) + 1) * 16;
     const size_t row_bytes = gguf_row_bytes(p.quant, p.K);
     const char *rp_env = getenv("OXQ_GGUF_RPWG");
     int rpwg = rp_env ? atoi(rp_env) : 8;  // measured 4096^2, Q4_K: 8 rows x 8 waves 7.5 us, 4 x 4 8.1, 16 x 8 8.8
