@@ -290,50 +290,55 @@ __global__ __launch_bounds__(512) void gguf_gemv_lds_kernel(const void *__restri
     const size_t start = (size_t)n0 * row_bytes, a0 = start & ~(size_t)15;
     const int head = (int)(start - a0);
     const int wchunks = (int)((head + (size_t)nrows * row_bytes + 15) >> 4);
-    const int xchunks = (M * K * XB) >> 4;
     const int cpr = K * XB / 16;  // chunks per activation row
     const int nthr = blockDim.x, nwaves = blockDim.x >> 6;
     // Staging copies in batches of 4 loads per thread: with one load per loop trip every
     // trip pays a full memory round trip before its LDS store.
     constexpr int CB = 4;
-    for (int base = threadIdx.x; base < wchunks; base += nthr * CB) {
+    // chunks that lie wholly inside the tensor; only the tensor's very last chunk can be partial
+    const int full = (int)min((size_t)wchunks, (total_bytes - a0) >> 4);
+    const u32x4_t *wsrc = (const u32x4_t *)(w + a0);
+    for (int base = threadIdx.x; base < full; base += nthr * CB) {
         u32x4_t v[CB];
 #pragma unroll
         for (int b = 0; b < CB; ++b) {
             const int c = base + b * nthr;
-            const size_t off = a0 + (size_t)c * 16;
-            v[b] = u32x4_t{0u, 0u, 0u, 0u};
-            if (c < wchunks) {
-                if (off + 16 <= total_bytes) {
-                    v[b] = *(const u32x4_t *)(w + off);
-                } else {  // the tensor's last, partial chunk
-                    uint32_t t[4] = {0u, 0u, 0u, 0u};
-                    for (int i = 0; i < 16; ++i)
-                        if (off + i < total_bytes) t[i >> 2] |= (uint32_t)w[off + i] << (8 * (i & 3));
-                    v[b] = u32x4_t{t[0], t[1], t[2], t[3]};
-                }
-            }
+            v[b] = c < full ? wsrc[c] : u32x4_t{0u, 0u, 0u, 0u};
         }
 #pragma unroll
         for (int b = 0; b < CB; ++b) {
             const int c = base + b * nthr;
-            if (c < wchunks) ((u32x4_t *)lds_w)[c] = v[b];
+            if (c < full) ((u32x4_t *)lds_w)[c] = v[b];
         }
     }
-    for (int base = threadIdx.x; base < xchunks; base += nthr * CB) {
-        u32x4_t v[CB];
+    if (full < wchunks && threadIdx.x == 0) {  // the tensor's last, partial chunk: byte by byte
+        const size_t off = a0 + (size_t)full * 16;
+        uint32_t t[4] = {0u, 0u, 0u, 0u};
+        for (int i = 0; i < 16; ++i)
+            if (off + i < total_bytes) t[i >> 2] |= (uint32_t)w[off + i] << (8 * (i & 3));
+        ((u32x4_t *)lds_w)[full] = u32x4_t{t[0], t[1], t[2], t[3]};
+    }
+    // activations, row by row (no division per chunk): chunk g of a row holds elements 16 / XB * g ...
 #pragma unroll
-        for (int b = 0; b < CB; ++b) {
-            const int c = base + b * nthr;
-            v[b] = c < xchunks ? ((const u32x4_t *)x)[c] : u32x4_t{0u, 0u, 0u, 0u};
-        }
+    for (int m = 0; m < MB; ++m) {
+        if (m < M) {
+            const u32x4_t *xsrc = (const u32x4_t *)x + (size_t)m * cpr;
+            unsigned char *xdst = lds_x + m * xrow_bytes;
+            for (int base = threadIdx.x; base < cpr; base += nthr * CB) {
+                u32x4_t v[CB];
 #pragma unroll
-        for (int b = 0; b < CB; ++b) {
-            const int c = base + b * nthr;
-            if (c < xchunks) {
-                const int m = c / cpr, g = c - m * cpr;
-                const int u = g / CPU, cc = g - u * CPU;
-                *(u32x4_t *)(lds_x + m * xrow_bytes + ((size_t)cc * upitch + u) * 16) = v[b];
+                for (int b = 0; b < CB; ++b) {
+                    const int g = base + b * nthr;
+                    v[b] = g < cpr ? xsrc[g] : u32x4_t{0u, 0u, 0u, 0u};
+                }
+#pragma unroll
+                for (int b = 0; b < CB; ++b) {
+                    const int g = base + b * nthr;
+                    if (g < cpr) {
+                        const int u = g / CPU, cc = g - u * CPU;  // CPU is a power of two
+                        *(u32x4_t *)(xdst + ((size_t)cc * upitch + u) * 16) = v[b];
+                    }
+                }
             }
         }
     }
