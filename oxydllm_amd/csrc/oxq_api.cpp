@@ -1288,6 +1288,7 @@ int oxq_packed_quant_linear_forward(oxq_packed_quant_linear *l, void *stream, co
         q.y = o2.data;
         q.M = m;
         q.act = l->act;
+        q.no_split = 0;
         q.w = l->pk;
         return launch_pk4_forward(l->ctx, (hipStream_t)stream, q);
     }

@@ -132,6 +132,7 @@ struct Pk4Problem {
     void *y;                // [M, N] T, or [M, N/2] with `act`
     int64_t M;
     int act;                // 0, or 1 + oxq_gated_act (gate|up layers only): y = act(gate) * up
+    int no_split;           // the ctx workspace is taken (it holds the weights): one K slice only
     Pk4Weights w;
 };
 

@@ -713,6 +713,7 @@ int launch_pk4_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p) {
     ks = pk4_env("OXQ_PK4_KS", ks);
     ks = std::max(1, std::min(ks, G));
     if (p.act) ks = 1;  // the activation needs the whole sum: gate|up layers are wide, one slice fills the chip
+    if (p.no_split) ks = 1;
     while (ks > 1 && (size_t)ks * M * p.w.N * 4 > ctx->workspace_bytes) --ks;
     const int gslice = (int)ceil_div(G, ks);
     ks = (int)ceil_div(G, gslice);  // no empty slice

@@ -384,3 +384,42 @@ def test_8bit_fast_gemv(method, dtn, K, N, g, monkeypatch):
         assert "generic" in ops.default_context().last_plan()["kernel"]
         # two roundings of nearly equal sums may land one output ulp apart
         assert_close(y, as_f32(yg), f"{method}8 fast vs generic {dtn} m{m}", rtol=RTOL + (2.0 ** -7 if dtn == "bf16" else 2.0 ** -10))
+
+
+@pytest.mark.parametrize("method,bits", [("gptq", 4), ("gptq", 8), ("awq", 8)])
+@pytest.mark.parametrize("dtn", ["f16", "bf16"])
+def test_stateless_tile_op_on_layouts_without_a_tile_kernel(method, bits, dtn, monkeypatch):
+    """mpp_quant_matmul on GPTQ / 8-bit AWQ checkpoint tensors: the tile-major copy is built in the ctx
+    workspace and the resident-layer kernel runs on it (three launches); with the switch off the call
+    falls back to GEMV passes of 8 rows.  Both against the oracle; a following 4-bit AWQ call on the same
+    ctx (which uses the workspace for K slices) still gives the right answer."""
+    dt = DT[dtn]
+    K, N, g = 1024, 384, 128
+    make = synth.awq_checkpoint if method == "awq" else synth.gptq_checkpoint
+    qw, qz, sc = make(K, N, g, bits, seed=bits + K)
+    d = dev_triplet(qw, qz, sc, dt)
+    s_r = oracle.round_through(sc, dt)
+    w = oracle.dequantize_awq8(qw, qz, s_r) if method == "awq" else oracle.dequantize_gptq(qw, qz, s_r, bits)
+    pd = ops.PACK_OUT if method == "awq" else ops.PACK_IN
+    rng = np.random.default_rng(5)
+    for m in (9, 16, 17, 64, 100):
+        say(f"transient repack {method}{bits} {dtn} m={m}")
+        x = rng.standard_normal((m, K)).astype(np.float32)
+        xd = to_dev(x, TORCH_DT[dt])
+        monkeypatch.delenv("OXQ_TRANSIENT_REPACK", raising=False)
+        y = ops.mpp_quant_matmul(xd, *d, bits, pd)
+        plan = ops.default_context().last_plan()
+        assert plan["kernel"].startswith(f"pk{bits}_mfma_{dtn}") and plan["launches"] == 3, plan
+        wr = w if m <= 16 else oracle.round_through(w, dt)
+        assert_close(y, oracle.matmul_nt_f32(round_x(x, dt), wr), f"{method}{bits} {dtn} m{m} (repacked in the workspace)")
+        monkeypatch.setenv("OXQ_TRANSIENT_REPACK", "0")
+        y2 = ops.mpp_quant_matmul(xd, *d, bits, pd)
+        assert "gemv" in ops.default_context().last_plan()["kernel"]
+        assert_close(y2, oracle.matmul_nt_f32(round_x(x, dt), w), f"{method}{bits} {dtn} m{m} (GEMV passes)")
+    monkeypatch.delenv("OXQ_TRANSIENT_REPACK", raising=False)
+    aw = synth.awq_checkpoint(2048, 128, 128, 4, seed=3)
+    ad = dev_triplet(*aw, dt)
+    wa = oracle.dequantize_awq(aw[0], aw[1], oracle.round_through(aw[2], dt))
+    xa = rng.standard_normal((32, 2048)).astype(np.float32)
+    ya = ops.mpp_quant_matmul(to_dev(xa, TORCH_DT[dt]), *ad, 4, ops.PACK_OUT)
+    assert_close(ya, oracle.matmul_nt_f32(round_x(xa, dt), oracle.round_through(wa, dt)), "awq4 after a repacked call")
