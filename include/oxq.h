@@ -275,6 +275,18 @@ int oxq_mxfp4_moe_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x,
                          const oxq_tensor *token_ids, int gather_rows, int64_t k, int64_t n,
                          const oxq_tensor *out);
 
+/* The gate_up projection of every active GPT-OSS expert followed by the clamped SwiGLU over its
+ * interleaved (gate, up) output rows (moe.rs:152-173: rows 2c and 2c + 1 give output c), in one launch:
+ * arguments as oxq_mxfp4_moe_matmul, out BF16 [n_pairs, n / 2].  Both factors are rounded to BF16 before
+ * the activation, so the result equals oxq_mxfp4_moe_matmul + oxq_gated_activation(OXQ_ACT_GPT_OSS_SWIGLU)
+ * bit for bit.  *fused = 1 when the launch was enqueued; *fused = 0 with OXQ_OK and nothing enqueued when
+ * this problem size runs on a kernel without the fused epilogue (many pairs per expert go to the tile
+ * matmul): make the two calls instead. */
+int oxq_mxfp4_moe_gate_up_swiglu(oxq_ctx *ctx, void *stream, const oxq_tensor *x, const oxq_tensor *blocks,
+                                 const oxq_tensor *scales, const oxq_tensor *bias,
+                                 const oxq_tensor *expert_offsets, const oxq_tensor *token_ids, int gather_rows,
+                                 int64_t k, int64_t n, float limit, const oxq_tensor *out, int *fused);
+
 /* ---- mixture-of-experts glue: the steps either side of the expert GEMVs -----
  * The reference does these on the host / with one launch per expert
  * (moe.rs:466-607); here they run on the device and feed oxq_mxfp4_moe_matmul. */

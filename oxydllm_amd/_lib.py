@@ -97,6 +97,8 @@ SIGNATURES = {
     "oxq_mxfp4_dequantize": (C.c_int, [_VP, _VP, _TP, _TP, C.c_int64, C.c_int64, _TP]),
     "oxq_mxfp4_moe_matmul": (C.c_int, [_VP, _VP, _TP, _TP, _TP, _TP, _TP, _TP, C.c_int,
                                        C.c_int64, C.c_int64, _TP]),
+    "oxq_mxfp4_moe_gate_up_swiglu": (C.c_int, [_VP, _VP, _TP, _TP, _TP, _TP, _TP, _TP, C.c_int,
+                                              C.c_int64, C.c_int64, C.c_float, _TP, C.POINTER(C.c_int)]),
     "oxq_moe_route": (C.c_int, [_VP, _VP, _TP, C.c_int64, C.c_int, _TP, _TP]),
     "oxq_moe_group": (C.c_int, [_VP, _VP, _TP, _TP, C.c_int64, _TP, _TP, _TP, _TP]),
     "oxq_gated_activation": (C.c_int, [_VP, _VP, _TP, C.c_int, C.c_float, _TP]),

@@ -116,6 +116,53 @@ __global__ __launch_bounds__(64) void moe_group_kernel(const int32_t *__restrict
     int32_t *cnt = group_lds;
     int32_t *base = group_lds + (size_t)E * 64;
     const int lane = threadIdx.x;
+    if (P <= 64) {
+        // Decode sizes: one pair per lane, no counting matrix.  The wave peels off one expert at a
+        // time: the first unplaced lane's expert, a ballot of the lanes that share it, rank = the
+        // matching lanes below me (pair order = token order inside an expert), count = the ballot's
+        // population.  At most min(P, E) rounds of scalar work instead of chains of dependent LDS
+        // accesses (E + 64 + E of them in the general path).
+        int32_t *count = group_lds;  // [E], then start[E]
+        int32_t *start = group_lds + E;
+        for (int e = lane; e < E; e += 64) count[e] = 0;
+        const int e = lane < P ? top_idx[lane] : -1;
+        const bool ok = e >= 0 && e < E;  // ids outside [0, E) are dropped
+        int rank = 0;
+        unsigned long long todo = __ballot(ok);
+        while (todo) {  // wave-uniform
+            const int first = __builtin_ctzll(todo);
+            const int e0 = __shfl(e, first, 64);
+            const unsigned long long m = __ballot(ok && e == e0);
+            if (ok && e == e0) rank = __builtin_popcountll(m & ((1ull << lane) - 1ull));
+            if (lane == first) count[e0] = __builtin_popcountll(m);
+            todo &= ~m;
+        }
+        // exclusive scan of the counts in expert order, 64 experts per round
+        int carry = 0;
+        for (int e1 = 0; e1 < E; e1 += 64) {
+            const int ee = e1 + lane;
+            const int c = ee < E ? count[ee] : 0;
+            int incl = c;
+#pragma unroll
+            for (int off = 1; off < 64; off <<= 1) {
+                const int t = __shfl_up(incl, off, 64);
+                if (lane >= off) incl += t;
+            }
+            if (ee < E) {
+                start[ee] = carry + incl - c;
+                offsets[ee] = carry + incl - c;
+            }
+            carry += __shfl(incl, 63, 64);
+        }
+        if (lane == 0) offsets[E] = carry;
+        if (ok) {
+            const int pos = start[e] + rank;
+            tokens[pos] = lane / top_k;
+            weights[pos] = top_vals[lane];
+            pair_pos[lane] = pos;
+        }
+        return;
+    }
     const int L = (P + 63) / 64;
     const int i0 = min(P, lane * L), i1 = min(P, i0 + L);
     for (int e = 0; e < E; ++e) cnt[e * 64 + lane] = 0;
@@ -169,12 +216,7 @@ __global__ __launch_bounds__(256) void gated_act_kernel(const T *__restrict__ gu
     const size_t row = gid / half_n, col = gid % half_n;
     float r;
     if (KIND == OXQ_ACT_GPT_OSS_SWIGLU) {  // interleaved (gate, up), moe.rs:152-173
-        float gate = load_f32(gu, row * 2 * half_n + 2 * col);
-        float up = load_f32(gu, row * 2 * half_n + 2 * col + 1);
-        gate = fminf(gate, limit);
-        up = fminf(fmaxf(up, -limit), limit);
-        const float sig = 1.0f / (1.0f + expf(-(gate * 1.702f)));
-        r = mul_f32_rn(up + 1.0f, gate * sig);
+        r = gpt_oss_swiglu_f32(load_f32(gu, row * 2 * half_n + 2 * col), load_f32(gu, row * 2 * half_n + 2 * col + 1), limit);
     } else {  // [gate | up], ffn_kernels.metal:19-242
         const float g = load_f32(gu, row * 2 * half_n + col);
         const float u = load_f32(gu, row * 2 * half_n + half_n + col);

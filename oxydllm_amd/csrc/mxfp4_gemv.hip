@@ -256,7 +256,7 @@ __global__ __launch_bounds__(256) void mxfp4_mfma_kernel(
     const uint16_t *__restrict__ x, const uint8_t *__restrict__ blocks,
     const uint8_t *__restrict__ scales, const uint16_t *__restrict__ bias,
     uint16_t *__restrict__ y, const int32_t *__restrict__ offsets,
-    const int32_t *__restrict__ token_ids, int M, int K, int N) {
+    const int32_t *__restrict__ token_ids, int M, int K, int N, int swiglu, float limit) {
     // [K/8 chunks][MTOK] x 16 B of tokens, then per wave the scale bytes of its 16*FR rows
     extern __shared__ __attribute__((aligned(16))) unsigned char mm_lds[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -417,8 +417,20 @@ __global__ __launch_bounds__(256) void mxfp4_mfma_kernel(
 #pragma unroll
         for (int f = 0; f < FR; ++f) {
             const int n = n_base + 16 * f + ni;
-            if (n < N) {
-                const float bv = bias ? BF16Traits::to_f32(bias[(size_t)e * N + n]) : 0.0f;
+            const float bv = (bias && n < N) ? BF16Traits::to_f32(bias[(size_t)e * N + n]) : 0.0f;
+            if (swiglu) {
+                // rows 2c / 2c + 1 are the gate / up of output c (moe.rs:152-173) and sit in neighbouring
+                // lanes: each is rounded to bf16 as the projection's own output would be, the even lane
+                // fetches its neighbour's value and stores the activation
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int m = 4 * kb + i;
+                    const float v = BF16Traits::to_f32(BF16Traits::from_f32(acc[f][i] + bv));
+                    const float other = __shfl_xor(v, 1, 64);
+                    if (!(ni & 1) && n + 1 < N && m < rows)
+                        y[(size_t)(pbase + m) * (N >> 1) + (n >> 1)] = BF16Traits::from_f32(gpt_oss_swiglu_f32(v, other, limit));
+                }
+            } else if (n < N) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const int m = 4 * kb + i;
@@ -466,7 +478,7 @@ static int mxfp4_mfma_go(hipStream_t s, dim3 grid, const Mxfp4Problem &p, size_t
     }
     hipLaunchKernelGGL((mxfp4_mfma_kernel<MTOK, FR>), grid, dim3(256), lds, s, (const uint16_t *)p.x, p.blocks,
                        p.scales, (const uint16_t *)p.bias, (uint16_t *)p.y, p.expert_offsets, p.token_ids,
-                       (int)p.M, (int)p.K, (int)p.N);
+                       (int)p.M, (int)p.K, (int)p.N, p.swiglu, p.swiglu_limit);
     OXQ_HIP_CHECK(hipGetLastError());
     return OXQ_OK;
 }
@@ -481,7 +493,8 @@ int launch_mxfp4_gemv(oxq_ctx *ctx, hipStream_t s, const Mxfp4Problem &p) {
         const int mm_mode = mm ? atoi(mm) : -1;  // 0 = never, 1 = always, default by size
         // plain form, measured on one expert's gate_up: m = 8 9.3 / 8.6 us, m = 16 11.8 / 8.7 us
         const bool big = grouped ? p.n_pairs >= 8 * p.n_experts : p.M >= 8;
-        if ((mm_mode == 1 || (mm_mode != 0 && big)) && p.K % 32 == 0) return launch_mxfp4_mm(ctx, s, p);
+        if ((mm_mode == 1 || (mm_mode != 0 && big)) && p.K % 32 == 0)
+            return p.swiglu ? OXQ_DECLINED : launch_mxfp4_mm(ctx, s, p);  // the tile matmul has no fused epilogue
     }
     {
         // matrix-core form: tokens staged in LDS (MTOK per pass), 4 waves x FR x 16 rows per workgroup
@@ -496,7 +509,8 @@ int launch_mxfp4_gemv(oxq_ctx *ctx, hipStream_t s, const Mxfp4Problem &p) {
         if (variant == 0 && lds <= 128 * 1024 && p.K % 32 == 0) {
             dim3 grid((unsigned)ceil_div(p.N, 4 * 16 * FR), grouped ? (unsigned)p.n_experts : 1u), block(256);
             char name[64];
-            snprintf(name, sizeof name, "%s_mfma_t%d", grouped ? "mxfp4_moe_gemv_bf16" : "mxfp4_gemv_bf16", mtok);
+            snprintf(name, sizeof name, "%s_mfma_t%d%s", grouped ? "mxfp4_moe_gemv_bf16" : "mxfp4_gemv_bf16", mtok,
+                     p.swiglu ? "_swiglu" : "");
             set_plan(ctx, name, grid, block, 1, 1, 0);
             if (ctx->plan_only) return OXQ_OK;
             if (((uintptr_t)p.blocks & 15) || ((uintptr_t)p.x & 15))
@@ -507,6 +521,7 @@ int launch_mxfp4_gemv(oxq_ctx *ctx, hipStream_t s, const Mxfp4Problem &p) {
         }
         force_rows = variant == 2;
     }
+    if (p.swiglu) return OXQ_DECLINED;  // only the matrix-core form carries the activation
     const int64_t rows_hint = grouped ? 4 : p.M;  // tokens per expert are few in decode
     const int mb = rows_hint <= 1 ? 1 : rows_hint <= 2 ? 2 : rows_hint <= 4 ? 4 : 8;
     constexpr int RW = 8;

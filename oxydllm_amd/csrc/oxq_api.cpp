@@ -897,13 +897,12 @@ int oxq_mxfp4_dequantize(oxq_ctx *ctx, void *stream, const oxq_tensor *blocks,
     return launch_mxfp4_dequant(ctx, (hipStream_t)stream, p, (float *)out->data);
 }
 
-int oxq_mxfp4_moe_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x,
-                         const oxq_tensor *blocks, const oxq_tensor *scales,
-                         const oxq_tensor *bias, const oxq_tensor *expert_offsets,
-                         const oxq_tensor *token_ids, int gather_rows, int64_t k, int64_t n,
-                         const oxq_tensor *out) {
-    const char *op = "Mxfp4MoeMatmul";
+static int moe_matmul_impl(const char *op, oxq_ctx *ctx, void *stream, const oxq_tensor *x, const oxq_tensor *blocks,
+                           const oxq_tensor *scales, const oxq_tensor *bias, const oxq_tensor *expert_offsets,
+                           const oxq_tensor *token_ids, int gather_rows, int64_t k, int64_t n, bool swiglu, float limit,
+                           const oxq_tensor *out, int *fused) {
     if (!ctx) return fail(OXQ_ERR_ARG, "%s: ctx is NULL", op);
+    if (fused) *fused = 0;
     OXQ_TRY(check_tensor(ctx, op, "expert_offsets", expert_offsets));
     if (expert_offsets->dtype != OXQ_I32 || expert_offsets->rank != 1 || expert_offsets->dims[0] < 2 ||
         !expert_offsets->contiguous)
@@ -911,8 +910,10 @@ int oxq_mxfp4_moe_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x,
     const int64_t n_experts = expert_offsets->dims[0] - 1;
     Mxfp4Problem p;
     OXQ_TRY(check_mxfp4(ctx, op, false, x, blocks, scales, k, n, n_experts, out, &p));
-    if (out->rank != 2 || out->dims[1] != n || !out->contiguous)
-        return fail(OXQ_ERR_SHAPE, "%s: out must be a contiguous [n_pairs, %lld]", op, (long long)n);
+    if (swiglu && (n & 1)) return fail(OXQ_ERR_SHAPE, "%s: interleaved gate / up rows need an even n, got %lld", op, (long long)n);
+    const int64_t out_cols = swiglu ? n / 2 : n;
+    if (out->rank != 2 || out->dims[1] != out_cols || !out->contiguous)
+        return fail(OXQ_ERR_SHAPE, "%s: out must be a contiguous [n_pairs, %lld]", op, (long long)out_cols);
     const int64_t n_pairs = out->dims[0];
     if (gather_rows) {
         OXQ_TRY(check_tensor(ctx, op, "token_ids", token_ids));
@@ -934,7 +935,30 @@ int oxq_mxfp4_moe_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x,
     p.expert_offsets = (const int32_t *)expert_offsets->data;
     p.token_ids = gather_rows ? (const int32_t *)token_ids->data : nullptr;
     p.n_pairs = n_pairs;
-    return launch_mxfp4_gemv(ctx, (hipStream_t)stream, p);
+    p.swiglu = swiglu ? 1 : 0;
+    p.swiglu_limit = limit;
+    const int rc = launch_mxfp4_gemv(ctx, (hipStream_t)stream, p);
+    if (rc == OXQ_DECLINED) return OXQ_OK;  // *fused stays 0, nothing was enqueued
+    if (rc == OXQ_OK && fused) *fused = 1;
+    return rc;
+}
+
+int oxq_mxfp4_moe_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x,
+                         const oxq_tensor *blocks, const oxq_tensor *scales,
+                         const oxq_tensor *bias, const oxq_tensor *expert_offsets,
+                         const oxq_tensor *token_ids, int gather_rows, int64_t k, int64_t n,
+                         const oxq_tensor *out) {
+    return moe_matmul_impl("Mxfp4MoeMatmul", ctx, stream, x, blocks, scales, bias, expert_offsets, token_ids,
+                           gather_rows, k, n, false, 0.0f, out, nullptr);
+}
+
+int oxq_mxfp4_moe_gate_up_swiglu(oxq_ctx *ctx, void *stream, const oxq_tensor *x, const oxq_tensor *blocks,
+                                 const oxq_tensor *scales, const oxq_tensor *bias,
+                                 const oxq_tensor *expert_offsets, const oxq_tensor *token_ids, int gather_rows,
+                                 int64_t k, int64_t n, float limit, const oxq_tensor *out, int *fused) {
+    if (!fused) return fail(OXQ_ERR_ARG, "Mxfp4MoeGateUpSwiglu: fused is NULL");
+    return moe_matmul_impl("Mxfp4MoeGateUpSwiglu", ctx, stream, x, blocks, scales, bias, expert_offsets, token_ids,
+                           gather_rows, k, n, true, limit, out, fused);
 }
 
 // ---- mixture-of-experts glue (moe.rs:466-607, ffn_kernels.metal, moe.rs:152-173) --------

@@ -150,6 +150,13 @@ __device__ __forceinline__ float mul_f32_rn(float a, float b) {
     return r;
 }
 __device__ __forceinline__ float silu_f32(float x) { return x / (1.0f + expf(-x)); }
+// GPT-OSS clamped SwiGLU of one (gate, up) pair, alpha = 1.702 (moe.rs:152-173)
+__device__ __forceinline__ float gpt_oss_swiglu_f32(float gate, float up, float limit) {
+    gate = fminf(gate, limit);
+    up = fminf(fmaxf(up, -limit), limit);
+    const float sig = 1.0f / (1.0f + expf(-(gate * 1.702f)));
+    return mul_f32_rn(up + 1.0f, gate * sig);
+}
 __device__ __forceinline__ float gelu_tanh_f32(float x) {
     const float k0 = 0.7978845608028654f, k1 = 0.044715f;
     return 0.5f * x * (1.0f + tanhf(k0 * (x + k1 * x * x * x)));

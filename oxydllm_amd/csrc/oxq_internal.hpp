@@ -102,7 +102,13 @@ struct Mxfp4Problem {
     const int32_t *expert_offsets;
     const int32_t *token_ids;   // nullptr => identity
     int64_t n_pairs;
+    // fused GPT-OSS SwiGLU over interleaved (gate, up) rows: y is [n_pairs, N / 2]
+    int swiglu = 0;
+    float swiglu_limit = 0.0f;
 };
+// launch_mxfp4_gemv returns this (positive) when p.swiglu is set and the kernel the problem size
+// selects has no fused epilogue; nothing was enqueued
+constexpr int OXQ_DECLINED = 1;
 
 // Block-scaled F8E4M3 weight [N, K] bytes with an F32 scale grid [s_rows, s_cols] tiling it.
 struct F8Problem {

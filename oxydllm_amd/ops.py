@@ -359,6 +359,25 @@ def mxfp4_moe_matmul(x, blocks, scales, bias, expert_offsets, token_ids, k: int,
 ACT_GATED_SILU, ACT_GATED_GELU_TANH, ACT_GPT_OSS_SWIGLU = 0, 1, 2
 
 
+def mxfp4_moe_gate_up_swiglu(x, blocks, scales, bias, expert_offsets, token_ids, k: int, n: int, limit: float, *,
+                             out=None, ctx: Optional[Context] = None):
+    """gate_up projection of the routed pairs + GPT-OSS SwiGLU (moe.rs:152-173) -> [n_pairs, n / 2].  One
+    launch where the decode kernel runs; otherwise the two calls it stands for (same bits either way)."""
+    ctx = _ctx(ctx)
+    gather = token_ids is not None
+    n_pairs = token_ids.numel() if gather else x.shape[0]
+    if out is None:
+        out = torch.empty((n_pairs, n // 2), dtype=x.dtype, device=x.device)
+    fused = C.c_int()
+    _lib.check(ctx._lib.oxq_mxfp4_moe_gate_up_swiglu(ctx.handle, ctx.stream(), desc(x), desc(blocks), desc(scales),
+                                                     desc(bias), desc(expert_offsets), desc(token_ids),
+                                                     1 if gather else 0, k, n, float(limit), desc(out), C.byref(fused)))
+    if not fused.value:
+        gu = mxfp4_moe_matmul(x, blocks, scales, bias, expert_offsets, token_ids, k, n, ctx=ctx)
+        gated_activation(gu, ACT_GPT_OSS_SWIGLU, limit, out=out, ctx=ctx)
+    return out
+
+
 def moe_route(logits, top_k: int, norm_topk: bool = True, *, ctx: Optional[Context] = None):
     """moe.rs:466-486: softmax, stable descending top-k, optional renormalisation."""
     ctx = _ctx(ctx)

@@ -382,7 +382,8 @@ def test_moe_route_ties_keep_expert_order():
     np.testing.assert_array_equal(ridx[0], [0, 1, 2, 3])
 
 
-@pytest.mark.parametrize("T,E,k", [(8, 32, 4), (1, 32, 4), (257, 16, 2), (1000, 256, 8)])
+@pytest.mark.parametrize("T,E,k", [(8, 32, 4), (1, 32, 4), (16, 64, 4), (5, 200, 3), (13, 256, 5), (257, 16, 2),
+                                   (1000, 256, 8)])
 def test_moe_group_matches_oracle(T, E, k):
     """moe.rs:563-590: integer work, compared exactly."""
     say(f"moe group T={T} E={E} k={k}")
@@ -456,6 +457,12 @@ def test_moe_step_config4_end_to_end():
     gu = ops.mxfp4_moe_matmul(xd, to_dev(c["gu_b"]), to_dev(c["gu_s"]), to_dev(c["gu_bias"], torch.bfloat16),
                               off, tok, H, 2 * I)
     h = ops.gated_activation(gu, ops.ACT_GPT_OSS_SWIGLU, 7.0)
+    # the same two steps as one launch: bit-identical
+    h1 = ops.mxfp4_moe_gate_up_swiglu(xd, to_dev(c["gu_b"]), to_dev(c["gu_s"]), to_dev(c["gu_bias"], torch.bfloat16),
+                                      off, tok, H, 2 * I, 7.0)
+    plan = ops.default_context().last_plan()
+    assert plan["kernel"].endswith("_swiglu") and plan["launches"] == 1, plan
+    np.testing.assert_array_equal(h1.view(torch.int16).cpu().numpy(), h.view(torch.int16).cpu().numpy())
     dn = ops.mxfp4_moe_matmul(h, to_dev(c["dn_b"]), to_dev(c["dn_s"]), to_dev(c["dn_bias"], torch.bfloat16),
                               off, None, I, H)
     out = ops.moe_combine(dn, pos, vals)
@@ -464,3 +471,38 @@ def test_moe_step_config4_end_to_end():
     # reference's own end-to-end bound (moe.rs:705-788: 1e-3 * max + 1e-3, widened for bf16 storage)
     err = np.abs(out.float().cpu().numpy() - out_ref)
     assert err.max() < 2e-2 * np.abs(out_ref).max() + 1e-2, err.max()
+
+
+@pytest.mark.parametrize("E,N,K,counts,bias", [(4, 64, 64, (1, 0, 3, 2), True), (3, 38, 96, (5, 1, 0), False),
+                                               (2, 6, 32, (9, 4), True), (5, 130, 160, (0, 0, 2, 0, 1), True)])
+def test_mxfp4_moe_gate_up_swiglu_fused(E, N, K, counts, bias, monkeypatch):
+    """Fused gate_up + GPT-OSS SwiGLU against the two calls it replaces (bit for bit) on ragged shapes:
+    idle experts, more than four pairs per expert (two passes over the tokens), a row count that is not
+    a multiple of 16, with and without bias, gathered and direct rows; and the declined case (tile
+    matmul sizes), where the wrapper makes the two calls."""
+    rng = np.random.default_rng(E * 100 + N)
+    blocks = np.concatenate([synth.mxfp4_weight(N, K, seed=10 + e)[0] for e in range(E)])
+    scales = np.concatenate([synth.mxfp4_weight(N, K, seed=10 + e)[1] for e in range(E)])
+    b = to_dev(rng.standard_normal((E, N)).astype(np.float32), torch.bfloat16) if bias else None
+    offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    P = int(offsets[-1])
+    T = 6
+    tok = rng.integers(0, T, size=P).astype(np.int32)
+    x = to_dev(rng.standard_normal((T, K)).astype(np.float32) * 2.0, torch.bfloat16)
+    bd, sd, od, td = to_dev(blocks), to_dev(scales), to_dev(offsets), to_dev(tok)
+    for gather in (True, False):
+        xs = x if gather else x[torch.from_numpy(tok).long().cuda()].contiguous()
+        tk = td if gather else None
+        say(f"fused swiglu E={E} N={N} K={K} gather={gather}")
+        monkeypatch.setenv("OXQ_MXFP4_MM", "0")
+        two = ops.gated_activation(ops.mxfp4_moe_matmul(xs, bd, sd, b, od, tk, K, N), ops.ACT_GPT_OSS_SWIGLU, 7.0)
+        one = ops.mxfp4_moe_gate_up_swiglu(xs, bd, sd, b, od, tk, K, N, 7.0)
+        assert ops.default_context().last_plan()["kernel"].endswith("_swiglu")
+        assert one.shape == (P, N // 2)
+        np.testing.assert_array_equal(one.view(torch.int16).cpu().numpy(), two.view(torch.int16).cpu().numpy())
+        monkeypatch.setenv("OXQ_MXFP4_MM", "1")      # the tile matmul declines the fused form
+        alt = ops.mxfp4_moe_gate_up_swiglu(xs, bd, sd, b, od, tk, K, N, 7.0)
+        assert ops.default_context().last_plan()["kernel"] == "gpt_oss_swiglu"
+        assert_close(alt, as_f32(two), "declined path", bf16_out=True)
+    with pytest.raises(ops.OxqError):                # odd n cannot be interleaved pairs
+        ops.mxfp4_moe_gate_up_swiglu(x, bd, sd, None, od, td, K, N - 1, 7.0, out=torch.empty((P, N // 2), dtype=torch.bfloat16, device="cuda"))
