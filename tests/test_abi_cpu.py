@@ -7,6 +7,7 @@ import ctypes as C
 import os
 import re
 
+import numpy as np
 import pytest
 
 from oxydllm_amd import _lib
@@ -407,3 +408,117 @@ def test_f8_ops_validate_like_reference(lib, ctx):
     assert lib.oxq_cast_f8e4m3_to_f32(ctx, None, C.byref(b), C.byref(fake((2048, 512), F32))) == 0, err(lib)
     assert lib.oxq_cast_f8e4m3_to_f32(ctx, None, C.byref(fake((8,), I32)), C.byref(fake((8,), F32))) == -2
     assert lib.oxq_cast_f8e4m3_to_f32(ctx, None, C.byref(b), C.byref(fake((2048, 511), F32))) == -3
+
+
+def test_random_descriptors_never_crash_and_always_explain(lib, ctx):
+    """Validation reads descriptors only: whatever a caller passes - wrong ranks, negative or huge dims,
+    unknown dtypes and enums, host or foreign-device tensors, NULL data - every entry point returns a
+    status of the enum and, on failure, a message; nothing is launched (plan-only ctx) and nothing
+    crashes.  Half of the cases start from a valid AWQ / GPTQ problem with one field corrupted."""
+    rng = np.random.default_rng(20240607)
+    DIMS = [0, 1, 2, 3, 7, 8, 16, 31, 32, 33, 64, 100, 128, 256, 1000, 4096, 14336, 2**31 - 1, 2**31, 2**40, 2**62, -1, -5]
+    def rt():
+        t = _lib.OxqTensor()
+        t.data = int(rng.choice([0, 0x1000, 0x1001, 0x7f0000000010]))
+        t.dtype = int(rng.integers(-2, 9))
+        t.rank = int(rng.choice([0, 1, 2, 2, 2, 3, 4, 5, -1]))
+        for i in range(4): t.dims[i] = int(rng.choice(DIMS))
+        t.contiguous = int(rng.integers(0, 2))
+        t.device = int(rng.choice([0, 0, 0, -1, 1, 7]))
+        return t
+    def _mk(shape, d):
+        t = _lib.OxqTensor(); t.data = 0x1000; t.dtype = d; t.rank = len(shape)
+        for i, s in enumerate(shape): t.dims[i] = s
+        t.contiguous = 1; t.device = 0
+        return t
+    names = {}
+    def call(name, *args):
+        fn = getattr(lib, name)
+        rc = fn(*args)
+        assert -13 <= rc <= 0, (name, rc)
+        names.setdefault(name, [0, 0])[0 if rc == 0 else 1] += 1
+        if rc != 0:
+            msg = lib.oxq_last_error()
+            assert msg and len(msg) > 3, name
+    N_IT = 500
+    B = C.byref
+    for it in range(N_IT):
+        ts = [rt() for _ in range(8)]
+        # half of the time start from a valid AWQ/GPTQ problem and corrupt one field
+        if it % 2 == 0:
+            bits = int(rng.choice([4, 8])); pf = 32 // bits
+            K = int(rng.choice([128, 256, 4096])); N = int(rng.choice([64, 128, 14336])); g = int(rng.choice([32, 64, 128]))
+            m = int(rng.choice([1, 4, 8, 9, 64]))
+            dt = int(rng.choice([1, 2]))
+            awq = it % 4 == 0
+            ts[0] = _mk((m, K), dt)
+            ts[1] = _mk((K, N // pf) if awq else (K // pf, N), 4)
+            ts[2] = _mk((K // g, N // pf), 4)
+            ts[3] = _mk((K // g, N), dt)
+            ts[4] = _mk((m, N), dt)
+            ts[5] = _mk((K, N), dt)
+            v = ts[int(rng.integers(0, 6))]
+            f = int(rng.integers(0, 5))
+            if f == 0: v.dtype = int(rng.integers(-2, 9))
+            elif f == 1: v.rank = int(rng.choice([0, 1, 3, 5]))
+            elif f == 2: v.dims[int(rng.integers(0, 2))] = int(rng.choice(DIMS))
+            elif f == 3: v.contiguous = 0
+            else: v.device = int(rng.choice([-1, 1]))
+        bits = int(rng.choice([4, 8, 0, 3, 16, 2**31]))
+        pd = int(rng.choice([0, 1, 2, -1]))
+        i64 = lambda: int(rng.choice(DIMS))
+        q = int(rng.integers(-1, 12))
+        taken = C.c_int()
+        call("oxq_w4a16_matmul", ctx, None, B(ts[0]), B(ts[1]), B(ts[2]), B(ts[3]), B(ts[4]))
+        call("oxq_w8a16_matmul", ctx, None, B(ts[0]), B(ts[1]), B(ts[2]), B(ts[3]), B(ts[4]))
+        call("oxq_gptq_matmul", ctx, None, B(ts[0]), B(ts[1]), B(ts[2]), B(ts[3]), bits & 0xFFFFFFFF, B(ts[4]))
+        call("oxq_dequantize_w4", ctx, None, B(ts[1]), B(ts[2]), B(ts[3]), B(ts[5]))
+        call("oxq_dequantize_w8", ctx, None, B(ts[1]), B(ts[2]), B(ts[3]), B(ts[5]))
+        call("oxq_dequantize_gptq_packed", ctx, None, B(ts[1]), B(ts[2]), B(ts[3]), bits & 0xFFFFFFFF, B(ts[5]))
+        call("oxq_mpp_quant_matmul", ctx, None, B(ts[0]), B(ts[1]), B(ts[2]), B(ts[3]), bits & 0xFFFFFFFF, pd, B(ts[4]))
+        call("oxq_maybe_mpp_quant_matmul", ctx, None, B(ts[0]), B(ts[1]), B(ts[2]), B(ts[3]), bits & 0xFFFFFFFF, pd, B(ts[4]), B(taken))
+        call("oxq_compressed_to_awq", ctx, None, B(ts[0]), B(ts[1]), B(ts[2]), B(ts[3]), B(ts[4]))
+        arr = (_lib.OxqTensor * 3)(ts[0], ts[1], ts[2])
+        call("oxq_concat_awq_along_out", ctx, None, int(rng.choice([4, 8, 3])), int(rng.choice([0, 1, 3, -1])), arr, arr, arr, B(ts[3]), B(ts[4]), B(ts[5]))
+        call("oxq_rtn_quantize_awq", ctx, None, B(ts[0]), i64(), B(ts[1]), B(ts[2]), B(ts[3]))
+        call("oxq_gguf_depermute_qk_rows", ctx, None, B(ts[0]), i64(), i64(), q, i64(), i64(), B(ts[1]))
+        call("oxq_cast_f8e4m3_to_f32", ctx, None, B(ts[0]), B(ts[1]))
+        call("oxq_f8_block_dequant_bf16", ctx, None, B(ts[0]), B(ts[1]), B(ts[2]))
+        call("oxq_f8_gemv", ctx, None, B(ts[0]), B(ts[1]), B(ts[2]), B(ts[3]))
+        call("oxq_f8_matmul", ctx, None, B(ts[0]), B(ts[1]), B(ts[2]), B(ts[3]))
+        call("oxq_gguf_quant_matmul", ctx, None, B(ts[0]), B(ts[1]), i64(), i64(), q, B(ts[2]))
+        call("oxq_gguf_quant_mul_mm", ctx, None, B(ts[0]), B(ts[1]), i64(), i64(), q, B(ts[2]))
+        call("oxq_gguf_dequantize", ctx, None, B(ts[0]), i64(), i64(), q, B(ts[1]))
+        call("oxq_mxfp4_matmul", ctx, None, B(ts[0]), B(ts[1]), B(ts[2]), i64(), i64(), B(ts[3]))
+        call("oxq_mxfp4_dequantize", ctx, None, B(ts[0]), B(ts[1]), i64(), i64(), B(ts[2]))
+        call("oxq_mxfp4_moe_matmul", ctx, None, B(ts[0]), B(ts[1]), B(ts[2]), B(ts[3]), B(ts[4]), B(ts[5]), int(rng.integers(0, 2)), i64(), i64(), B(ts[6]))
+        call("oxq_mxfp4_moe_gate_up_swiglu", ctx, None, B(ts[0]), B(ts[1]), B(ts[2]), B(ts[3]), B(ts[4]), B(ts[5]), int(rng.integers(0, 2)), i64(), i64(), C.c_float(7.0), B(ts[6]), B(taken))
+        call("oxq_moe_route", ctx, None, B(ts[0]), i64(), 1, B(ts[1]), B(ts[2]))
+        call("oxq_moe_group", ctx, None, B(ts[0]), B(ts[1]), i64(), B(ts[2]), B(ts[3]), B(ts[4]), B(ts[5]))
+        call("oxq_gated_activation", ctx, None, B(ts[0]), int(rng.integers(-1, 4)), C.c_float(7.0), B(ts[1]))
+        call("oxq_moe_combine", ctx, None, B(ts[0]), B(ts[1]), B(ts[2]), B(ts[3]))
+        # layers
+        h = C.c_void_p()
+        rc = lib.oxq_packed_quant_linear_new(ctx, bits & 0xFFFFFFFF, pd, B(ts[1]), B(ts[2]), B(ts[3]), None, int(rng.choice([1, 2, 0])), B(h))
+        assert -13 <= rc <= 0
+        if rc == 0:
+            call("oxq_packed_quant_linear_forward", h, None, B(ts[0]), B(ts[4]))
+            call("oxq_packed_quant_linear_dequantize", h, None, B(ts[5]))
+            lib.oxq_packed_quant_linear_free(h)
+        h = C.c_void_p()
+        rc = lib.oxq_packed_quant_linear_new_gate_up(ctx, bits & 0xFFFFFFFF, pd, B(ts[1]), B(ts[2]), B(ts[3]), None, int(rng.integers(-1, 4)), int(rng.choice([1, 2])), B(h))
+        assert -13 <= rc <= 0
+        if rc == 0:
+            call("oxq_packed_quant_linear_forward", h, None, B(ts[0]), B(ts[4]))
+            lib.oxq_packed_quant_linear_free(h)
+        h = C.c_void_p()
+        rc = lib.oxq_qlinear_new(ctx, q, B(ts[0]), i64(), i64(), None, int(rng.choice([0, 2, 1])), B(h))
+        assert -13 <= rc <= 0
+        if rc == 0:
+            call("oxq_qlinear_forward", h, None, B(ts[1]), B(ts[2])); lib.oxq_qlinear_free(h)
+        h = C.c_void_p()
+        rc = lib.oxq_mxfp4_linear_new(ctx, B(ts[0]), B(ts[1]), None, i64(), i64(), B(h))
+        assert -13 <= rc <= 0
+        if rc == 0:
+            call("oxq_mxfp4_linear_forward", h, None, B(ts[2]), B(ts[3])); lib.oxq_mxfp4_linear_free(h)
+    assert names['oxq_w4a16_matmul'][0] > 0 and names['oxq_w4a16_matmul'][1] > 0
