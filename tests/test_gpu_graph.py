@@ -96,3 +96,55 @@ def test_block_quant_paths_in_a_graph():
         layer = ops.QLinear(synth.GGUF_Q4_K, data, K, N, None, torch.bfloat16)
         replay_matches_eager(f"gguf q4_k m={m}", lambda: layer.forward(x, out=y), inputs, y)
         replay_matches_eager(f"mxfp4 m={m}", lambda: ops.mxfp4_matmul(x, bd, sd, K, N, out=y), inputs, y)
+
+
+def test_fused_epilogues_and_workspace_repack_in_a_graph():
+    """The gate|up layer with the activation in its epilogue, the stateless tile op that builds its
+    tile-major copy in the ctx workspace (three kernels, the workspace rewritten on every replay), the
+    8-bit GEMV kernels, and the expert GEMV with the fused SwiGLU."""
+    gen = torch.Generator(device="cuda")
+    K, I = 1024, 256
+    trip = synth.awq_checkpoint(K, 2 * I, 128, 4, seed=3)
+    layer = ops.PackedQuantLinear(4, ops.PACK_OUT, to_dev(trip[0]), to_dev(trip[1]), to_dev(trip[2], torch.float16),
+                                  None, torch.float16, gate_up_act=ops.ACT_GATED_SILU)
+    for m in (1, 40):
+        x = torch.empty((m, K), device="cuda", dtype=torch.float16)
+        y = torch.empty((m, I), device="cuda", dtype=torch.float16)
+
+        def inputs(i, x=x, m=m):
+            gen.manual_seed(300 + i)
+            x.copy_(torch.randn((m, K), device="cuda", generator=gen).to(torch.float16))
+        replay_matches_eager(f"gate|up silu m={m}", lambda: layer.forward(x, out=y), inputs, y)
+
+    for bits in (4, 8):
+        gq = synth.gptq_checkpoint(K, 384, 128, bits, seed=bits)
+        d = (to_dev(gq[0]), to_dev(gq[1]), to_dev(gq[2], torch.float16))
+        for m in (2, 24):
+            x = torch.empty((m, K), device="cuda", dtype=torch.float16)
+            y = torch.empty((m, 384), device="cuda", dtype=torch.float16)
+
+            def inputs(i, x=x, m=m):
+                gen.manual_seed(400 + i)
+                x.copy_(torch.randn((m, K), device="cuda", generator=gen).to(torch.float16))
+            if m <= 8:
+                fn = lambda: ops.gptq_matmul(x, *d, bits, out=y)
+            else:
+                fn = lambda: ops.mpp_quant_matmul(x, *d, bits, ops.PACK_IN, out=y)
+            replay_matches_eager(f"gptq{bits} m={m}", fn, inputs, y)
+            if m > 8:
+                assert ops.default_context().last_plan()["launches"] == 3
+
+    E, N, Kx = 3, 64, 96
+    blocks = torch.from_numpy(np.concatenate([synth.mxfp4_weight(N, Kx, seed=e)[0] for e in range(E)])).cuda()
+    scales = torch.from_numpy(np.concatenate([synth.mxfp4_weight(N, Kx, seed=e)[1] for e in range(E)])).cuda()
+    offsets = to_dev(np.array([0, 2, 2, 5], np.int32))
+    tok = to_dev(np.array([0, 3, 1, 2, 3], np.int32))
+    x = torch.empty((4, Kx), device="cuda", dtype=torch.bfloat16)
+    y = torch.empty((5, N // 2), device="cuda", dtype=torch.bfloat16)
+
+    def inputs(i):
+        gen.manual_seed(500 + i)
+        x.copy_(torch.randn((4, Kx), device="cuda", generator=gen).to(torch.bfloat16))
+    replay_matches_eager("mxfp4 gate_up + swiglu",
+                         lambda: ops.mxfp4_moe_gate_up_swiglu(x, blocks, scales, None, offsets, tok, Kx, N, 7.0, out=y),
+                         inputs, y)
