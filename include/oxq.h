@@ -317,6 +317,13 @@ typedef enum oxq_gated_act {
 int oxq_gated_activation(oxq_ctx *ctx, void *stream, const oxq_tensor *gate_up, int kind, float limit,
                          const oxq_tensor *out);
 
+/* metal_ops.rs:1252 silu_mul_fused and :1271 gelu_tanh_mul_fused (kernels ffn_kernels.metal:72-110 and
+ * 164-200), the GateUpProjection::Separate arm of ffn.rs:386-413: out = act(gate) * up elementwise over
+ * two tensors of one dtype (F32 | F16 | BF16) and one element count; f32 math, one rounding.  `kind` is
+ * OXQ_ACT_GATED_SILU or OXQ_ACT_GATED_GELU_TANH.  Gives the bits of oxq_gated_activation on [gate | up]. */
+int oxq_activation_mul(oxq_ctx *ctx, void *stream, const oxq_tensor *gate, const oxq_tensor *up, int kind,
+                       const oxq_tensor *out);
+
 /* moe.rs:592-605: out[token] = sum over slots of top_vals[token, slot] *
  * expert_out[pair_pos[token, slot]]  (f32 accumulation in slot order, one rounding).
  *  expert_out T [P, hidden]   out T [n_tokens, hidden] */
@@ -384,6 +391,39 @@ int oxq_mxfp4_linear_new(oxq_ctx *ctx, const oxq_tensor *blocks, const oxq_tenso
 int oxq_mxfp4_linear_forward(oxq_mxfp4_linear *layer, void *stream, const oxq_tensor *x,
                              const oxq_tensor *out);
 void oxq_mxfp4_linear_free(oxq_mxfp4_linear *layer);
+
+/* ffn.rs:22-474 FeedForward (the gated MLP) over the quantized arms of AnyLinear (linear.rs:536-542):
+ * down(act(gate(x)) * up(x)).  The MLP borrows its projections: they must outlive it. */
+typedef enum oxq_linear_kind {
+    OXQ_LINEAR_PACKED_QUANT = 0, /* oxq_packed_quant_linear* */
+    OXQ_LINEAR_GGUF = 1,         /* oxq_qlinear* */
+    OXQ_LINEAR_MXFP4 = 2         /* oxq_mxfp4_linear* */
+} oxq_linear_kind;
+typedef struct oxq_any_linear {
+    int kind; /* oxq_linear_kind */
+    void *layer;
+} oxq_any_linear;
+typedef enum oxq_gate_up_kind {
+    OXQ_GATE_UP_FUSED = 0,    /* ffn.rs GateUpProjection::Fused and ::Packed: one projection, [gate | up] columns;
+                               * a layer from oxq_packed_quant_linear_new_gate_up runs the activation in its matmul */
+    OXQ_GATE_UP_SEPARATE = 1, /* ::Separate: gate_proj and up_proj, then silu_mul / gelu_tanh_mul */
+    OXQ_GATE_UP_SIMPLE = 2    /* ::Simple: ungated, act(up(x)) */
+} oxq_gate_up_kind;
+typedef struct oxq_mlp oxq_mlp;
+/* `a` is gate_up_proj (FUSED), gate_proj (SEPARATE) or up_proj (SIMPLE); `b` is up_proj for SEPARATE and NULL
+ * otherwise.  Shape checks as ffn.rs:227-233, 255-261, 270-276, 323-346.  `activation` is
+ * OXQ_ACT_GATED_SILU or OXQ_ACT_GATED_GELU_TANH. */
+int oxq_mlp_new(oxq_ctx *ctx, int gate_up_kind, const oxq_any_linear *a, const oxq_any_linear *b_or_null,
+                const oxq_any_linear *down, int64_t intermediate, int activation, oxq_mlp **out);
+/* Elements (of the projections' output dtype) that forward needs in `scratch` for `rows` rows of x. */
+int oxq_mlp_scratch_elems(const oxq_mlp *mlp, int64_t rows, int64_t *elems);
+/* ffn.rs:386-474 FeedForward::forward.  x [.., in_features] -> out [.., out_features]; the
+ * intermediates live in the caller's `scratch`, nothing is allocated. */
+int oxq_mlp_forward(oxq_mlp *mlp, void *stream, const oxq_tensor *x, const oxq_tensor *scratch,
+                    const oxq_tensor *out);
+int oxq_mlp_in_features(const oxq_mlp *mlp, int64_t *k);
+int oxq_mlp_out_features(const oxq_mlp *mlp, int64_t *n);
+void oxq_mlp_free(oxq_mlp *mlp);
 
 #ifdef __cplusplus
 }

@@ -34,6 +34,10 @@ class OxqTensor(C.Structure):
                 ("device", C.c_int32)]
 
 
+class OxqAnyLinear(C.Structure):
+    _fields_ = [("kind", C.c_int), ("layer", C.c_void_p)]
+
+
 class OxqPlan(C.Structure):
     _fields_ = [("kernel", C.c_char * 64), ("grid", C.c_uint32 * 3), ("block", C.c_uint32 * 3),
                 ("split_k", C.c_uint32), ("launches", C.c_uint32),
@@ -102,6 +106,7 @@ SIGNATURES = {
     "oxq_moe_route": (C.c_int, [_VP, _VP, _TP, C.c_int64, C.c_int, _TP, _TP]),
     "oxq_moe_group": (C.c_int, [_VP, _VP, _TP, _TP, C.c_int64, _TP, _TP, _TP, _TP]),
     "oxq_gated_activation": (C.c_int, [_VP, _VP, _TP, C.c_int, C.c_float, _TP]),
+    "oxq_activation_mul": (C.c_int, [_VP, _VP, _TP, _TP, C.c_int, _TP]),
     "oxq_moe_combine": (C.c_int, [_VP, _VP, _TP, _TP, _TP, _TP]),
     "oxq_packed_quant_linear_new": (C.c_int, [_VP, C.c_uint32, C.c_int, _TP, _TP, _TP, _TP,
                                               C.c_int, C.POINTER(_VP)]),
@@ -120,6 +125,13 @@ SIGNATURES = {
     "oxq_mxfp4_linear_new": (C.c_int, [_VP, _TP, _TP, _TP, C.c_int64, C.c_int64, C.POINTER(_VP)]),
     "oxq_mxfp4_linear_forward": (C.c_int, [_VP, _VP, _TP, _TP]),
     "oxq_mxfp4_linear_free": (None, [_VP]),
+    "oxq_mlp_new": (C.c_int, [_VP, C.c_int, C.POINTER(OxqAnyLinear), C.POINTER(OxqAnyLinear), C.POINTER(OxqAnyLinear),
+                              C.c_int64, C.c_int, C.POINTER(_VP)]),
+    "oxq_mlp_scratch_elems": (C.c_int, [_VP, C.c_int64, C.POINTER(C.c_int64)]),
+    "oxq_mlp_forward": (C.c_int, [_VP, _VP, _TP, _TP, _TP]),
+    "oxq_mlp_in_features": (C.c_int, [_VP, C.POINTER(C.c_int64)]),
+    "oxq_mlp_out_features": (C.c_int, [_VP, C.POINTER(C.c_int64)]),
+    "oxq_mlp_free": (None, [_VP]),
     # include/oxq_files.h
     "oxq_gguf_open": (C.c_int, [C.POINTER(C.c_char_p), C.c_int, C.POINTER(_VP)]),
     "oxq_safetensors_open": (C.c_int, [C.POINTER(C.c_char_p), C.c_int, C.POINTER(_VP)]),

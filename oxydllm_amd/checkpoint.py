@@ -281,6 +281,38 @@ class GgufWeights(TensorFile):
             w = ops.gguf_depermute_qk_rows(w, in_f, out_f, t.gguf_quant, depermute[0], depermute[1], ctx=ctx)
         return ops.QLinear(t.gguf_quant, w, in_f, out_f, bias, out_dtype or torch.bfloat16, ctx=ctx)
 
+    def feed_forward(self, layer_idx: int, intermediate_size: int, activation: Optional[int] = None, out_dtype=None,
+                     ctx=None):
+        """ffn.rs:307-373 FeedForward::load_gguf: ``blk.{i}.ffn_{gate,up,down}.weight`` kept quantized.
+        Separate when ``ffn_gate`` exists, packed when ``ffn_up`` holds gate and up, ungated otherwise."""
+        from . import ops
+        activation = ops.ACT_GATED_SILU if activation is None else activation
+        prefix = f"blk.{layer_idx}"
+        up_t = self.get(f"{prefix}.ffn_up.weight")
+        down_t = self.get(f"{prefix}.ffn_down.weight")
+        up_out = up_t.shape[0]
+        if down_t.shape[1] != intermediate_size:
+            raise OxqError(-3, f"GGUF ffn_down shape mismatch at {prefix}: expected dim1={intermediate_size}, "
+                               f"got {down_t.shape[1]}")
+        gate_t = self.try_get(f"{prefix}.ffn_gate.weight")
+        mk = lambda part: self.qlinear(f"{prefix}.ffn_{part}.weight", out_dtype=out_dtype, ctx=ctx)
+        if gate_t is not None:
+            if gate_t.shape[0] != intermediate_size:
+                raise OxqError(-3, f"GGUF ffn_gate shape mismatch at {prefix}: expected dim0={intermediate_size}, "
+                                   f"got {gate_t.shape[0]}")
+            if up_out != intermediate_size:
+                raise OxqError(-3, f"GGUF ffn_up shape mismatch at {prefix}: expected dim0={intermediate_size}, "
+                                   f"got {up_out}")
+            kind, a, b = ops.GATE_UP_SEPARATE, mk("gate"), mk("up")
+        elif up_out == 2 * intermediate_size:
+            kind, a, b = ops.GATE_UP_FUSED, mk("up"), None
+        elif up_out == intermediate_size:
+            kind, a, b = ops.GATE_UP_SIMPLE, mk("up"), None
+        else:
+            raise OxqError(-3, f"Unsupported GGUF FFN up-proj shape at {prefix}: dim0={up_out} (expected "
+                               f"{intermediate_size} or {2 * intermediate_size})")
+        return ops.FeedForward(kind, a, b, mk("down"), intermediate_size, activation, ctx=ctx)
+
 
 @dataclass
 class QuantWeight:
@@ -384,6 +416,70 @@ class ModelWeights(TensorFile):
             bias = b.to_device(ctx).to(dtype)
         return ops.PackedQuantLinear(raw.bits, raw.pack_dim, raw.qweight, raw.qzeros, raw.scales.to(dtype), bias, dtype,
                                      ctx=ctx)
+
+    def feed_forward(self, layer_idx: int, activation: Optional[int] = None, dtype=None, ctx=None):
+        """ffn.rs:62-68 + 200-285 FeedForward::load, the packed-quant arm: ``model.layers.{i}.mlp`` with
+        down_proj packed.  Separate gate_proj / up_proj tensors whose columns can be joined (out_features a
+        multiple of 8) become one fused gate|up projection, as the reference does for AWQ; here GPTQ is
+        joined too, its tensors concatenate along the same axis.  The fused projection runs the activation in
+        its matmul when the layer qualifies for the tile-major copy; otherwise the activation is a second
+        launch."""
+        import torch
+        from . import ops
+        activation = ops.ACT_GATED_SILU if activation is None else activation
+        dtype = dtype or torch.float16
+        p = f"model.layers.{layer_idx}.mlp"
+        down_raw = self.try_get_quant(f"{p}.down_proj", ctx=ctx)
+        if down_raw is None:
+            raise KeyError(f"no packed-quantized weight at {p}.down_proj")
+
+        def layer(raw, act=None):
+            if raw.qzeros is None:
+                raise OxqError(-1, "PackedQuantLinear: qzeros missing")
+            return ops.PackedQuantLinear(raw.bits, raw.pack_dim, raw.qweight, raw.qzeros, raw.scales.to(dtype), None,
+                                         dtype, ctx=ctx, gate_up_act=act)
+
+        def fused(raw):
+            try:
+                return layer(raw, activation)
+            except OxqError as e:
+                if e.status != -11:     # only "no tile-major copy for this shape" falls back to two launches
+                    raise
+                return layer(raw)
+
+        down = layer(down_raw)
+        inter = down.in_features
+        gate_raw = self.try_get_quant(f"{p}.gate_proj", ctx=ctx)
+        up_raw = self.try_get_quant(f"{p}.up_proj", ctx=ctx)
+        if gate_raw is not None and up_raw is not None:
+            gate_out, up_out = gate_raw.scales.shape[1], up_raw.scales.shape[1]
+            if gate_out != inter or up_out != inter:
+                raise OxqError(-3, f"Packed-quant FFN shape mismatch at {p}: gate/up out_features must both be "
+                                   f"{inter}, got gate={gate_out} up={up_out}")
+            if inter % 8 == 0 and gate_raw.qzeros is not None and up_raw.qzeros is not None:
+                if gate_raw.pack_dim == ops.PACK_OUT:
+                    q, z, sc = ops.concat_awq_along_out([(gate_raw.qweight, gate_raw.qzeros, gate_raw.scales),
+                                                         (up_raw.qweight, up_raw.qzeros, up_raw.scales)],
+                                                        gate_raw.bits, ctx=ctx)
+                else:
+                    q, z, sc = (torch.cat([getattr(gate_raw, f), getattr(up_raw, f)], dim=1).contiguous()
+                                for f in ("qweight", "qzeros", "scales"))
+                both = QuantWeight(gate_raw.bits, gate_raw.pack_dim, gate_raw.sym, q, z, sc)
+                return ops.FeedForward(ops.GATE_UP_FUSED, fused(both), None, down, inter, activation, ctx=ctx)
+            return ops.FeedForward(ops.GATE_UP_SEPARATE, layer(gate_raw), layer(up_raw), down, inter, activation,
+                                   ctx=ctx)
+        gate_up_raw = self.try_get_quant(f"{p}.gate_up_proj", ctx=ctx)
+        if gate_up_raw is not None:
+            packed_out = gate_up_raw.scales.shape[1]
+            if packed_out != 2 * inter:
+                raise OxqError(-3, f"Packed-quant FFN gate_up out_features {packed_out} != 2*{inter}")
+            return ops.FeedForward(ops.GATE_UP_FUSED, fused(gate_up_raw), None, down, inter, activation, ctx=ctx)
+        if up_raw is not None:
+            if up_raw.scales.shape[1] != inter:
+                raise OxqError(-3, f"Packed-quant FFN up_proj out_features {up_raw.scales.shape[1]} != {inter}")
+            return ops.FeedForward(ops.GATE_UP_SIMPLE, layer(up_raw), None, down, inter, activation, ctx=ctx)
+        raise OxqError(-3, f"Mixed quantization at {p}: down_proj is packed but no gate/up tensors are packed. "
+                           "Expected one of: ({gate,up}_proj.qweight) or (gate_up_proj.qweight) or (up_proj.qweight).")
 
     def mxfp4_experts(self, prefix: str, ctx=None) -> dict:
         """The stacked GPT-OSS expert tensors under ``prefix`` (``…mlp``), checked as moe.rs:397-417 checks

@@ -225,6 +225,18 @@ __global__ __launch_bounds__(256) void gated_act_kernel(const T *__restrict__ gu
     store_f32(out, gid, r);
 }
 
+// Two-tensor form (ffn_kernels.metal:72-110 silu_mul, 164-200 gelu_tanh_mul): the gate and the up
+// projection are separate tensors of equal element count.
+template <typename T, int KIND>
+__global__ __launch_bounds__(256) void act_mul_kernel(const T *gate, const T *up, T *out, size_t n) {  // out may be gate
+    const size_t gid = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (gid >= n) return;
+    const float g = load_f32(gate, gid);
+    const float a = KIND == OXQ_ACT_GATED_SILU ? silu_f32(g) : gelu_tanh_f32(g);
+    // up == nullptr: the ungated FFN (ffn.rs:463-468), the activation alone
+    store_f32(out, gid, up ? mul_f32_rn(a, load_f32(up, gid)) : a);
+}
+
 // ---------------------------------------------------------------------------
 // combine: out[t] = sum over slots of w[t, s] * expert_out[pair_pos[t, s]] (f32, slot order)
 // ---------------------------------------------------------------------------
@@ -309,6 +321,30 @@ int launch_gated_activation(oxq_ctx *ctx, hipStream_t s, const void *gu, void *o
     if (dtype == OXQ_F32) gated_go<float>(s, grid, kind, gu, out, n_out, (int)half_n, limit);
     else if (dtype == OXQ_F16) gated_go<F16Tag>(s, grid, kind, gu, out, n_out, (int)half_n, limit);
     else gated_go<BF16Tag>(s, grid, kind, gu, out, n_out, (int)half_n, limit);
+    OXQ_HIP_CHECK(hipGetLastError());
+    return OXQ_OK;
+}
+
+template <typename T>
+static void act_mul_go(hipStream_t s, dim3 grid, int kind, const void *gate, const void *up, void *out, size_t n) {
+    dim3 block(256);
+    if (kind == OXQ_ACT_GATED_SILU)
+        hipLaunchKernelGGL((act_mul_kernel<T, OXQ_ACT_GATED_SILU>), grid, block, 0, s, (const T *)gate, (const T *)up,
+                           (T *)out, n);
+    else
+        hipLaunchKernelGGL((act_mul_kernel<T, OXQ_ACT_GATED_GELU_TANH>), grid, block, 0, s, (const T *)gate,
+                           (const T *)up, (T *)out, n);
+}
+
+int launch_activation_mul(oxq_ctx *ctx, hipStream_t s, const void *gate, const void *up, void *out, int dtype,
+                          int64_t n, int kind) {
+    dim3 grid((unsigned)ceil_div(n, 256)), block(256);
+    set_plan(ctx, kind == OXQ_ACT_GATED_SILU ? (up ? "silu_mul" : "silu") : (up ? "gelu_tanh_mul" : "gelu_tanh"), grid,
+             block, 1, 1, 0);
+    if (ctx->plan_only || n == 0) return OXQ_OK;
+    if (dtype == OXQ_F32) act_mul_go<float>(s, grid, kind, gate, up, out, (size_t)n);
+    else if (dtype == OXQ_F16) act_mul_go<F16Tag>(s, grid, kind, gate, up, out, (size_t)n);
+    else act_mul_go<BF16Tag>(s, grid, kind, gate, up, out, (size_t)n);
     OXQ_HIP_CHECK(hipGetLastError());
     return OXQ_OK;
 }

@@ -1052,6 +1052,29 @@ int oxq_gated_activation(oxq_ctx *ctx, void *stream, const oxq_tensor *gate_up, 
                                    kind, limit);
 }
 
+int oxq_activation_mul(oxq_ctx *ctx, void *stream, const oxq_tensor *gate, const oxq_tensor *up, int kind,
+                       const oxq_tensor *out) {
+    const char *op = kind == OXQ_ACT_GATED_GELU_TANH ? "GeluTanhMulOp" : "SiluMulOp";
+    if (!ctx) return fail(OXQ_ERR_ARG, "%s: ctx is NULL", op);
+    OXQ_TRY(check_tensor(ctx, op, "gate", gate));
+    OXQ_TRY(check_tensor(ctx, op, "up", up));
+    OXQ_TRY(check_tensor(ctx, op, "out", out));
+    if (kind != OXQ_ACT_GATED_SILU && kind != OXQ_ACT_GATED_GELU_TANH)
+        return fail(OXQ_ERR_ARG, "%s: activation kind %d has no two-tensor form", op, kind);
+    if (!gate->contiguous || !up->contiguous)  // metal_ops.rs:649-651
+        return fail(OXQ_ERR_CONTIGUOUS, "%s: both inputs must be contiguous", op);
+    if (!out->contiguous) return fail(OXQ_ERR_CONTIGUOUS, "%s: out must be contiguous", op);
+    if (gate->dtype != up->dtype)  // metal_ops.rs:652-658
+        return fail(OXQ_ERR_DTYPE, "%s: dtype mismatch %s vs %s", op, dtype_name(gate->dtype), dtype_name(up->dtype));
+    if (!is_float_dtype(gate->dtype))
+        return fail(OXQ_ERR_DTYPE, "%s: unsupported dtype %s", op, dtype_name(gate->dtype));
+    if (out->dtype != gate->dtype) return fail(OXQ_ERR_DTYPE, "%s: out must have the inputs' dtype", op);
+    const int64_t n = numel(gate);
+    if (numel(up) != n) return fail(OXQ_ERR_SHAPE, "%s: shape mismatch", op);  // metal_ops.rs:659-662
+    if (numel(out) != n) return fail(OXQ_ERR_SHAPE, "%s: out must have the inputs' shape", op);
+    return launch_activation_mul(ctx, (hipStream_t)stream, gate->data, up->data, out->data, gate->dtype, n, kind);
+}
+
 int oxq_moe_combine(oxq_ctx *ctx, void *stream, const oxq_tensor *expert_out, const oxq_tensor *pair_pos,
                     const oxq_tensor *top_vals, const oxq_tensor *out) {
     const char *op = "MoeCombine";
@@ -1481,5 +1504,211 @@ int oxq_mxfp4_linear_forward(oxq_mxfp4_linear *l, void *stream, const oxq_tensor
 }
 
 void oxq_mxfp4_linear_free(oxq_mxfp4_linear *l) { delete l; }
+
+}  // extern "C"
+
+// ---------------------------------------------------------------------------
+// ffn.rs:22-474 FeedForward over the quantized arms of AnyLinear
+// ---------------------------------------------------------------------------
+struct oxq_mlp {
+    oxq_ctx *ctx;
+    int gate_up_kind;
+    oxq_any_linear a, b, down;
+    int64_t intermediate, in_features, out_features;
+    int activation;
+    int mid_dtype;   // dtype of the projections' outputs, which is what down_proj reads
+    bool epilogue;   // `a` already applies the gated activation in its matmul
+};
+
+namespace oxq {
+
+struct LinearInfo {
+    oxq_ctx *ctx;
+    int64_t in_features, out_features;  // out_features as forward writes them
+    int out_dtype;
+    int act;  // 0, or 1 + oxq_gated_act of a fused gate|up layer
+};
+
+static int linear_info(const char *op, const char *name, const oxq_any_linear *l, LinearInfo *info) {
+    if (!l || !l->layer) return fail(OXQ_ERR_ARG, "%s: %s is NULL", op, name);
+    switch (l->kind) {
+    case OXQ_LINEAR_PACKED_QUANT: {
+        const oxq_packed_quant_linear *q = (const oxq_packed_quant_linear *)l->layer;
+        *info = LinearInfo{q->ctx, q->in_features, q->act ? q->out_features / 2 : q->out_features, q->dtype, q->act};
+        return OXQ_OK;
+    }
+    case OXQ_LINEAR_GGUF: {
+        const oxq_qlinear *q = (const oxq_qlinear *)l->layer;
+        *info = LinearInfo{q->ctx, q->in_features, q->out_features, q->out_dtype, 0};
+        return OXQ_OK;
+    }
+    case OXQ_LINEAR_MXFP4: {
+        const oxq_mxfp4_linear *q = (const oxq_mxfp4_linear *)l->layer;
+        *info = LinearInfo{q->ctx, q->in_features, q->out_features, OXQ_BF16, 0};
+        return OXQ_OK;
+    }
+    default:
+        return fail(OXQ_ERR_ARG, "%s: %s has unknown layer kind %d", op, name, l->kind);
+    }
+}
+
+static int linear_forward(const oxq_any_linear &l, void *stream, const oxq_tensor *x, const oxq_tensor *out) {
+    switch (l.kind) {
+    case OXQ_LINEAR_PACKED_QUANT:
+        return oxq_packed_quant_linear_forward((oxq_packed_quant_linear *)l.layer, stream, x, out);
+    case OXQ_LINEAR_GGUF:
+        return oxq_qlinear_forward((oxq_qlinear *)l.layer, stream, x, out);
+    default:
+        return oxq_mxfp4_linear_forward((oxq_mxfp4_linear *)l.layer, stream, x, out);
+    }
+}
+
+// elements of `mid_dtype` that forward keeps between the projections, per row of x
+static int64_t mlp_scratch_per_row(const oxq_mlp *m) {
+    switch (m->gate_up_kind) {
+    case OXQ_GATE_UP_FUSED: return m->epilogue ? m->intermediate : 3 * m->intermediate;
+    case OXQ_GATE_UP_SEPARATE: return 2 * m->intermediate;
+    default: return m->intermediate;
+    }
+}
+
+static oxq_tensor rows_view(const oxq_tensor *base, int64_t elem_offset, int64_t m, int64_t n) {
+    oxq_tensor t = *base;
+    t.data = (char *)base->data + elem_offset * dtype_size(base->dtype);
+    t.rank = 2;
+    t.dims[0] = m;
+    t.dims[1] = n;
+    t.contiguous = 1;
+    return t;
+}
+
+}  // namespace oxq
+
+extern "C" {
+
+int oxq_mlp_new(oxq_ctx *ctx, int gate_up_kind, const oxq_any_linear *a, const oxq_any_linear *b,
+                const oxq_any_linear *down, int64_t intermediate, int activation, oxq_mlp **out) {
+    const char *op = "FeedForward";
+    if (!ctx || !out) return fail(OXQ_ERR_ARG, "%s: NULL argument", op);
+    *out = nullptr;
+    if (gate_up_kind != OXQ_GATE_UP_FUSED && gate_up_kind != OXQ_GATE_UP_SEPARATE && gate_up_kind != OXQ_GATE_UP_SIMPLE)
+        return fail(OXQ_ERR_ARG, "%s: unknown gate/up layout %d", op, gate_up_kind);
+    if (activation != OXQ_ACT_GATED_SILU && activation != OXQ_ACT_GATED_GELU_TANH)
+        return fail(OXQ_ERR_ARG, "%s: activation must be OXQ_ACT_GATED_SILU or OXQ_ACT_GATED_GELU_TANH, got %d", op,
+                    activation);
+    if (intermediate <= 0) return fail(OXQ_ERR_SHAPE, "%s: intermediate size %lld", op, (long long)intermediate);
+    const bool separate = gate_up_kind == OXQ_GATE_UP_SEPARATE;
+    if (separate != (b != nullptr))
+        return fail(OXQ_ERR_ARG, "%s: the second projection belongs to the separate gate/up layout and to no other", op);
+    LinearInfo ia, ib{}, id;
+    OXQ_TRY(linear_info(op, separate ? "gate_proj" : gate_up_kind == OXQ_GATE_UP_FUSED ? "gate_up_proj" : "up_proj", a, &ia));
+    if (separate) OXQ_TRY(linear_info(op, "up_proj", b, &ib));
+    OXQ_TRY(linear_info(op, "down_proj", down, &id));
+    if (ia.ctx != ctx || id.ctx != ctx || (separate && ib.ctx != ctx))
+        return fail(OXQ_ERR_ARG, "%s: every projection must belong to this context", op);
+    bool epilogue = false;
+    if (gate_up_kind == OXQ_GATE_UP_FUSED) {
+        epilogue = ia.act != 0;
+        if (epilogue && ia.act != activation + 1)
+            return fail(OXQ_ERR_ARG, "%s: gate_up_proj was built with another activation than the layer's", op);
+        // ffn.rs:255-261: a fused projection carries 2 * intermediate columns
+        if (ia.out_features != (epilogue ? intermediate : 2 * intermediate))
+            return fail(OXQ_ERR_SHAPE, "%s: gate_up out_features %lld != 2*%lld", op,
+                        (long long)(epilogue ? 2 * ia.out_features : ia.out_features), (long long)intermediate);
+    } else {
+        if (ia.act || (separate && ib.act))
+            return fail(OXQ_ERR_ARG, "%s: a layer with a fused activation can only be the fused gate_up_proj", op);
+        // ffn.rs:227-233, 270-276
+        if (ia.out_features != intermediate || (separate && ib.out_features != intermediate))
+            return fail(OXQ_ERR_SHAPE, "%s: gate/up out_features must both be %lld, got %lld and %lld", op,
+                        (long long)intermediate, (long long)ia.out_features,
+                        (long long)(separate ? ib.out_features : ia.out_features));
+        if (separate && (ib.in_features != ia.in_features || ib.out_dtype != ia.out_dtype))
+            return fail(OXQ_ERR_SHAPE, "%s: gate_proj and up_proj must share in_features and the output dtype", op);
+    }
+    if (id.act) return fail(OXQ_ERR_ARG, "%s: down_proj cannot carry a fused activation", op);
+    if (id.in_features != intermediate)
+        return fail(OXQ_ERR_SHAPE, "%s: down_proj in_features %lld != intermediate size %lld", op,
+                    (long long)id.in_features, (long long)intermediate);
+    if (!is_float_dtype(ia.out_dtype)) return fail(OXQ_ERR_DTYPE, "%s: projections must write F32, F16 or BF16", op);
+    oxq_mlp *m = new (std::nothrow) oxq_mlp();
+    if (!m) return fail(OXQ_ERR_RUNTIME, "%s: out of host memory", op);
+    m->ctx = ctx;
+    m->gate_up_kind = gate_up_kind;
+    m->a = *a;
+    if (separate) m->b = *b;
+    m->down = *down;
+    m->intermediate = intermediate;
+    m->in_features = ia.in_features;
+    m->out_features = id.out_features;
+    m->activation = activation;
+    m->mid_dtype = ia.out_dtype;
+    m->epilogue = epilogue;
+    *out = m;
+    return OXQ_OK;
+}
+
+int oxq_mlp_scratch_elems(const oxq_mlp *m, int64_t rows, int64_t *elems) {
+    if (!m || !elems || rows < 0) return fail(OXQ_ERR_ARG, "FeedForward: bad argument");
+    *elems = rows * mlp_scratch_per_row(m);
+    return OXQ_OK;
+}
+
+// ffn.rs:386-474 FeedForward::forward
+int oxq_mlp_forward(oxq_mlp *m, void *stream, const oxq_tensor *x, const oxq_tensor *scratch, const oxq_tensor *out) {
+    const char *op = "FeedForward";
+    if (!m) return fail(OXQ_ERR_ARG, "%s: layer is NULL", op);
+    oxq_tensor x2;
+    int64_t rows;
+    OXQ_TRY(flatten_rows(op, x, m->in_features, &x2, &rows));
+    OXQ_TRY(check_tensor(m->ctx, op, "scratch", scratch));
+    const int64_t I = m->intermediate, need = rows * mlp_scratch_per_row(m);
+    if (scratch->dtype != m->mid_dtype || !scratch->contiguous || numel(scratch) < need)
+        return fail(OXQ_ERR_SHAPE, "%s: scratch must be a contiguous %s tensor of at least %lld elements", op,
+                    dtype_name(m->mid_dtype), (long long)need);
+    oxq_tensor h;  // [rows, I]: act(gate) * up, the input of down_proj
+    switch (m->gate_up_kind) {
+    case OXQ_GATE_UP_FUSED:
+        if (m->epilogue) {
+            h = rows_view(scratch, 0, rows, I);
+            OXQ_TRY(linear_forward(m->a, stream, &x2, &h));
+        } else {
+            const oxq_tensor gu = rows_view(scratch, 0, rows, 2 * I);
+            h = rows_view(scratch, rows * 2 * I, rows, I);
+            OXQ_TRY(linear_forward(m->a, stream, &x2, &gu));
+            OXQ_TRY(oxq_gated_activation(m->ctx, stream, &gu, m->activation, 0.0f, &h));
+        }
+        break;
+    case OXQ_GATE_UP_SEPARATE: {
+        h = rows_view(scratch, 0, rows, I);
+        const oxq_tensor u = rows_view(scratch, rows * I, rows, I);
+        OXQ_TRY(linear_forward(m->a, stream, &x2, &h));
+        OXQ_TRY(linear_forward(m->b, stream, &x2, &u));
+        OXQ_TRY(oxq_activation_mul(m->ctx, stream, &h, &u, m->activation, &h));
+        break;
+    }
+    default:
+        h = rows_view(scratch, 0, rows, I);
+        OXQ_TRY(linear_forward(m->a, stream, &x2, &h));
+        if (rows > 0)
+            OXQ_TRY(launch_activation_mul(m->ctx, (hipStream_t)stream, h.data, nullptr, h.data, h.dtype, rows * I,
+                                          m->activation));
+        break;
+    }
+    return linear_forward(m->down, stream, &h, out);
+}
+
+int oxq_mlp_in_features(const oxq_mlp *m, int64_t *k) {
+    if (!m || !k) return fail(OXQ_ERR_ARG, "FeedForward: NULL argument");
+    *k = m->in_features;
+    return OXQ_OK;
+}
+int oxq_mlp_out_features(const oxq_mlp *m, int64_t *n) {
+    if (!m || !n) return fail(OXQ_ERR_ARG, "FeedForward: NULL argument");
+    *n = m->out_features;
+    return OXQ_OK;
+}
+
+void oxq_mlp_free(oxq_mlp *m) { delete m; }
 
 }  // extern "C"

@@ -183,6 +183,8 @@ int launch_moe_route(oxq_ctx *ctx, hipStream_t s, const void *logits, int dtype,
                      int norm_topk, int32_t *top_idx, float *top_vals);
 int launch_moe_group(oxq_ctx *ctx, hipStream_t s, const int32_t *top_idx, const float *top_vals, int64_t P, int64_t E,
                      int64_t top_k, int32_t *offsets, int32_t *tokens, float *weights, int32_t *pair_pos);
+int launch_activation_mul(oxq_ctx *ctx, hipStream_t s, const void *gate, const void *up, void *out, int dtype,
+                          int64_t n, int kind);
 int launch_gated_activation(oxq_ctx *ctx, hipStream_t s, const void *gu, void *out, int dtype, int64_t rows,
                             int64_t half_n, int kind, float limit);
 int launch_moe_combine(oxq_ctx *ctx, hipStream_t s, const void *eo, const int32_t *pair_pos, const float *top_vals,

@@ -414,6 +414,23 @@ def gated_activation(gate_up, kind: int, limit: float = 0.0, *, out=None, ctx: O
     return out
 
 
+def activation_mul(gate, up, kind: int, *, out=None, ctx: Optional[Context] = None):
+    """metal_ops.rs:1252 silu_mul_fused / :1271 gelu_tanh_mul_fused: act(gate) * up over two tensors."""
+    ctx = _ctx(ctx)
+    if out is None:
+        out = torch.empty_like(gate)
+    _lib.check(ctx._lib.oxq_activation_mul(ctx.handle, ctx.stream(), desc(gate), desc(up), kind, desc(out)))
+    return out
+
+
+def silu_mul(gate, up, *, out=None, ctx: Optional[Context] = None):
+    return activation_mul(gate, up, ACT_GATED_SILU, out=out, ctx=ctx)
+
+
+def gelu_tanh_mul(gate, up, *, out=None, ctx: Optional[Context] = None):
+    return activation_mul(gate, up, ACT_GATED_GELU_TANH, out=out, ctx=ctx)
+
+
 def moe_combine(expert_out, pair_pos, top_vals, *, out=None, ctx: Optional[Context] = None):
     """moe.rs:592-605: out[t] = sum_s top_vals[t, s] * expert_out[pair_pos[t, s]]."""
     ctx = _ctx(ctx)
@@ -537,6 +554,62 @@ class Mxfp4Linear:
         try:
             if self.handle:
                 self.ctx._lib.oxq_mxfp4_linear_free(self.handle)
+                self.handle = C.c_void_p()
+        except Exception:
+            pass
+
+
+GATE_UP_FUSED, GATE_UP_SEPARATE, GATE_UP_SIMPLE = 0, 1, 2
+_LINEAR_KINDS = {PackedQuantLinear: 0, QLinear: 1, Mxfp4Linear: 2}
+
+
+class FeedForward:
+    """ffn.rs:22-474 over the quantized projections: down(act(gate(x)) * up(x)).
+
+    ``a`` is the fused gate|up projection (GATE_UP_FUSED; one built with ``gate_up_act=`` runs the
+    activation in its matmul), gate_proj (GATE_UP_SEPARATE, ``b`` = up_proj) or the ungated up_proj
+    (GATE_UP_SIMPLE)."""
+
+    def __init__(self, gate_up_kind: int, a, b, down, intermediate_size: int, activation: int = ACT_GATED_SILU,
+                 ctx: Optional[Context] = None):
+        self.ctx = _ctx(ctx)
+        self._keep = (a, b, down)
+        self.handle = C.c_void_p()
+
+        def any_linear(layer):
+            if layer is None:
+                return None
+            kind = _LINEAR_KINDS.get(type(layer))
+            if kind is None:
+                raise OxqError(-1, f"FeedForward: {type(layer).__name__} is not a quantized projection")
+            return C.byref(_lib.OxqAnyLinear(kind, layer.handle))
+
+        _lib.check(self.ctx._lib.oxq_mlp_new(self.ctx.handle, gate_up_kind, any_linear(a), any_linear(b),
+                                             any_linear(down), intermediate_size, activation, C.byref(self.handle)))
+        k, n = C.c_int64(), C.c_int64()
+        self.ctx._lib.oxq_mlp_in_features(self.handle, C.byref(k))
+        self.ctx._lib.oxq_mlp_out_features(self.handle, C.byref(n))
+        self.in_features, self.out_features = k.value, n.value
+        self.gate_up_kind, self.intermediate_size, self.activation = gate_up_kind, intermediate_size, activation
+
+    def scratch_elems(self, rows: int) -> int:
+        e = C.c_int64()
+        _lib.check(self.ctx._lib.oxq_mlp_scratch_elems(self.handle, rows, C.byref(e)))
+        return e.value
+
+    def forward(self, x: torch.Tensor, out=None, scratch=None) -> torch.Tensor:
+        rows = x.numel() // max(x.shape[-1], 1)
+        if scratch is None:
+            scratch = torch.empty(max(self.scratch_elems(rows), 1), dtype=x.dtype, device=x.device)
+        if out is None:
+            out = torch.empty(tuple(x.shape[:-1]) + (self.out_features,), dtype=x.dtype, device=x.device)
+        _lib.check(self.ctx._lib.oxq_mlp_forward(self.handle, self.ctx.stream(), desc(x), desc(scratch), desc(out)))
+        return out
+
+    def __del__(self):
+        try:
+            if self.handle:
+                self.ctx._lib.oxq_mlp_free(self.handle)
                 self.handle = C.c_void_p()
         except Exception:
             pass

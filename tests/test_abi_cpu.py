@@ -255,6 +255,82 @@ def test_mxfp4_validation(lib, ctx):
     assert call(out=fake((7, N), BF16)) == -3 and "output shape" in err(lib)
 
 
+def test_feed_forward_validates_and_plans(lib, ctx):
+    """ffn.rs:22-474 at the benchmark's layer size: layouts, shape checks, scratch sizes, launch plans."""
+    H, I = 4096, 14336
+
+    def packed(k, n, act=None):
+        h = C.c_void_p()
+        qw, qz, sc = _awq(k, n, 128, BF16)
+        if act is None:
+            rc = lib.oxq_packed_quant_linear_new(ctx, 4, 0, C.byref(qw), C.byref(qz), C.byref(sc), None, BF16, C.byref(h))
+        else:
+            rc = lib.oxq_packed_quant_linear_new_gate_up(ctx, 4, 0, C.byref(qw), C.byref(qz), C.byref(sc), None, act,
+                                                         BF16, C.byref(h))
+        assert rc == 0, err(lib)
+        return h
+
+    def any_(kind, h):
+        return C.byref(_lib.OxqAnyLinear(kind, h)) if h is not None else None
+
+    def new(kind, a, b, down, inter=I, act=0, lk=0):
+        m = C.c_void_p()
+        return lib.oxq_mlp_new(ctx, kind, any_(lk, a), any_(lk, b), any_(lk, down), inter, act, C.byref(m)), m
+
+    gate, up, both, epi, down = packed(H, I), packed(H, I), packed(H, 2 * I), packed(H, 2 * I, 0), packed(I, H)
+    x, out = fake((2, 3, H), BF16), fake((2, 3, H), BF16)
+    for kind, a, b, per_row in [(1, gate, up, 2 * I), (0, both, None, 3 * I), (0, epi, None, I), (2, up, None, I)]:
+        rc, m = new(kind, a, b, down)
+        assert rc == 0, err(lib)
+        e, k, n = C.c_int64(), C.c_int64(), C.c_int64()
+        assert lib.oxq_mlp_scratch_elems(m, 6, C.byref(e)) == 0 and e.value == 6 * per_row
+        assert lib.oxq_mlp_in_features(m, C.byref(k)) == 0 and lib.oxq_mlp_out_features(m, C.byref(n)) == 0
+        assert (k.value, n.value) == (H, H)
+        assert lib.oxq_mlp_forward(m, None, C.byref(x), C.byref(fake((6 * per_row,), BF16)), C.byref(out)) == 0, err(lib)
+        assert plan(lib, ctx).kernel.decode().startswith("pk4_mfma_bf16_mt1_gs")       # the last launch: down_proj
+        assert lib.oxq_mlp_forward(m, None, C.byref(x), C.byref(fake((6 * per_row - 1,), BF16)), C.byref(out)) == -3
+        assert f"at least {6 * per_row} elements" in err(lib)
+        assert lib.oxq_mlp_forward(m, None, C.byref(x), C.byref(fake((6 * per_row,), F16)), C.byref(out)) == -3
+        assert lib.oxq_mlp_forward(m, None, C.byref(fake((6, H + 1), BF16)), C.byref(fake((6 * per_row,), BF16)),
+                                   C.byref(out)) == -3 and "in_features" in err(lib)
+        lib.oxq_mlp_free(m)
+    # refusals, in the reference's words where it has them
+    for args, code, text in [((1, gate, both, down), -3, "gate/up out_features must both be 14336, got 14336 and 28672"),
+                             ((0, gate, None, down), -3, "gate_up out_features 14336 != 2*14336"),
+                             ((1, gate, up, gate), -3, "down_proj in_features 4096 != intermediate size 14336"),
+                             ((0, both, up, down), -1, "second projection"),
+                             ((1, gate, None, down), -1, "second projection"),
+                             ((2, epi, None, down), -1, "only be the fused gate_up_proj"),
+                             ((5, both, None, down), -1, "unknown gate/up layout 5")]:
+        rc, _ = new(*args)
+        assert rc == code and text in err(lib), (args[0], rc, err(lib))
+    rc, _ = new(0, epi, None, down, act=1)
+    assert rc == -1 and "another activation" in err(lib)
+    rc, _ = new(0, both, None, down, act=2)
+    assert rc == -1 and "activation must be" in err(lib)
+    rc, _ = new(0, both, None, down, lk=9)
+    assert rc == -1 and "unknown layer kind 9" in err(lib)
+    assert lib.oxq_mlp_forward(None, None, C.byref(x), C.byref(x), C.byref(out)) == -1
+    lib.oxq_mlp_free(None)
+    # block-quantized projections (ffn.rs:307-373) with the separate layout
+    def gguf(n, k):
+        q = C.c_void_p()
+        assert lib.oxq_qlinear_new(ctx, _lib.GGUF_Q4_K, C.byref(fake((n * (k // 256) * 144,), U8)), k, n, None, BF16,
+                                   C.byref(q)) == 0, err(lib)
+        return q
+    qg, qu, qd = gguf(I, H), gguf(I, H), gguf(H, I)
+    rc, m = new(1, qg, qu, qd, lk=1)
+    assert rc == 0, err(lib)
+    assert lib.oxq_mlp_forward(m, None, C.byref(fake((1, H), BF16)), C.byref(fake((2 * I,), BF16)),
+                               C.byref(fake((1, H), BF16))) == 0, err(lib)
+    assert plan(lib, ctx).kernel.decode().startswith("gguf_q4k_gemv_bf16")
+    lib.oxq_mlp_free(m)
+    for h in (qg, qu, qd):
+        lib.oxq_qlinear_free(h)
+    for h in (gate, up, both, epi, down):
+        lib.oxq_packed_quant_linear_free(h)
+
+
 def test_layers_validate_like_reference(lib, ctx):
     h = C.c_void_p()
     qw, qz, sc = _awq(4096, 14336, 128, BF16)
@@ -496,6 +572,7 @@ def test_random_descriptors_never_crash_and_always_explain(lib, ctx):
         call("oxq_moe_route", ctx, None, B(ts[0]), i64(), 1, B(ts[1]), B(ts[2]))
         call("oxq_moe_group", ctx, None, B(ts[0]), B(ts[1]), i64(), B(ts[2]), B(ts[3]), B(ts[4]), B(ts[5]))
         call("oxq_gated_activation", ctx, None, B(ts[0]), int(rng.integers(-1, 4)), C.c_float(7.0), B(ts[1]))
+        call("oxq_activation_mul", ctx, None, B(ts[0]), B(ts[1]), int(rng.integers(-1, 4)), B(ts[2]))
         call("oxq_moe_combine", ctx, None, B(ts[0]), B(ts[1]), B(ts[2]), B(ts[3]))
         # layers
         h = C.c_void_p()

@@ -420,6 +420,46 @@ def test_gated_activations_match_oracle(dt):
         ops.gated_activation(to_dev(gu[:, :191].copy(), dt), ops.ACT_GATED_SILU)
 
 
+@pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16, torch.float16])
+def test_two_tensor_activations_match_oracle_and_the_fused_tensor_form(dt):
+    """metal_ops.rs:1252/1271 (ffn_kernels.metal:72-110, 164-200): act(gate) * up over separate tensors equals
+    the oracle and, bit for bit, the [gate | up] form on the concatenation; errors as metal_ops.rs:649-662."""
+    say(f"two-tensor activations {dt}")
+    rng = np.random.default_rng(8)
+    for shape in [(5, 96), (3, 2, 77), (1, 1), (0, 8)]:
+        g = (rng.standard_normal(shape) * 3).astype(np.float32)
+        u = (rng.standard_normal(shape) * 3).astype(np.float32)
+        if g.size:
+            g.flat[0] = -90.0  # silu underflows towards -0 here: the sign of the product must survive
+        gd, ud = to_dev(g, dt), to_dev(u, dt)
+        both = torch.cat([gd, ud], dim=-1)
+        br = both.float().cpu().numpy()
+        for fn, kind, ref in [(ops.silu_mul, ops.ACT_GATED_SILU, oracle.gated_silu),
+                              (ops.gelu_tanh_mul, ops.ACT_GATED_GELU_TANH, oracle.gated_gelu_tanh)]:
+            y = fn(gd, ud)
+            assert y.shape == gd.shape and y.dtype == dt
+            if g.size:
+                lo = dt != torch.float32
+                want = ref(br.reshape(-1, br.shape[-1])).reshape(shape)
+                assert_close(y, want, f"{fn.__name__} {dt} {shape}", rtol=RTOL if lo else 1e-5,
+                             atol=ATOL if lo else 1e-5, bf16_out=dt == torch.bfloat16)
+                ints = torch.int32 if dt == torch.float32 else torch.int16
+                same = ops.gated_activation(both, kind)
+                assert torch.equal(y.reshape(-1).view(ints), same.reshape(-1).view(ints))
+            else:
+                assert y.numel() == 0
+    g, u = to_dev(np.ones((2, 8), np.float32), dt), to_dev(np.ones((2, 8), np.float32), dt)
+    with pytest.raises(ops.OxqError, match="shape mismatch"):
+        ops.silu_mul(g, u[:, :4].contiguous())
+    with pytest.raises(ops.OxqError, match="both inputs must be contiguous"):
+        ops.gelu_tanh_mul(g, u.t().contiguous().t())
+    other = torch.float16 if dt != torch.float16 else torch.bfloat16
+    with pytest.raises(ops.OxqError, match="dtype mismatch"):
+        ops.silu_mul(g, u.to(other))
+    with pytest.raises(ops.OxqError, match="no two-tensor form"):
+        ops.activation_mul(g, u, ops.ACT_GPT_OSS_SWIGLU)
+
+
 def test_moe_step_config4_end_to_end():
     """Benchmark config 4 as one device-side pipeline: route -> group -> gate_up -> GPT-OSS SwiGLU ->
     down -> combine, against the oracle restating moe.rs:466-607 + 152-173 step by step (each
