@@ -198,7 +198,7 @@ __global__ __launch_bounds__(256) void pk4_dequant_kernel(const uint32_t *__rest
 // steps).  With more than one slice the workgroup writes its f32 partial tile to
 // the workspace and a second launch adds the slices in order.
 //
-// Weights: one 1 KB wave load per step, issued two blocks (8 steps) ahead.
+// Weights: one 1 KB wave load per step, issued one block (4 steps) ahead.
 // Activations: the matrix-core fragment pattern (16 rows x 64 bytes per load)
 // is served by L2 at a third of the rate of 256-byte row reads, so a wave
 // fetches its next 16*MT x 128 block of x with 4-rows-x-256-bytes loads one
@@ -228,18 +228,22 @@ __global__ __launch_bounds__(256) void pk4_dequant_kernel(const uint32_t *__rest
 // ---------------------------------------------------------------------------
 // The integers the GS form feeds the matrix cores: bias_f + q, the same AND-OR unpack as
 // the other form (f16: 1024 + q or 64 + q by nibble position, bf16: 128 + q).
-// Ring depths in 128-row blocks: weights WB, activations AB (registers; the current
-// block's activations live in LDS).  Deeper rings measured no faster: at these sizes the
-// kernel is bound by instruction issue, not by memory latency.
+// Ring depths: weights WD steps (1 KB wave loads), activations AB 128-row blocks (registers; the
+// current block's activations live in LDS).  One block of weights in flight per wave is the
+// measured optimum (4096 x 14336, f16, M = 1 / 16 / 64): 4 steps 8.8 / 9.2 / 18.1 us, 8 steps
+// 9.0 / 9.7 / 18.0 (8.9 / 9.9 / 18.5 with whole-block slots), 16 steps 9.6 at M = 1, 2 steps
+// equal on this shape and 0.4 us slower on 4096 x 4096; 3 and 6 steps (a three-block loop body)
+// cost 0.5 - 2 us.  A CU takes only so many vector loads in flight: what the first waves issue
+// beyond their next block keeps the other waves' first loads waiting.
 template <int MT, int BITS> struct Pk4Ring {
     static constexpr int AB = 1;
-    static constexpr int WB = (BITS == 8 && MT >= 3) ? 1 : 2;  // 8-bit weights take twice the registers
+    static constexpr int WD = 4;
 };
 
 // BPG1: group size 128, i.e. every block is one group (no group bookkeeping).
 // XQ: activation loads per block and lane that can hold rows below M (4 rows each); the
 // launcher passes 4 * MT, or fewer for a short single tile, whose other rows stay zero in LDS.
-template <typename TT, int BITS, int MT, bool GS, bool BPG1, int AB, int WB, int XQ>
+template <typename TT, int BITS, int MT, bool GS, bool BPG1, int AB, int WD, int XQ>
 __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restrict__ x,
                                                        const uint32_t *__restrict__ pw,
                                                        const uint32_t *__restrict__ pzs,
@@ -317,8 +321,10 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
         if (q * NT < zchunks)  // block-uniform
             zstage[q] = __builtin_amdgcn_raw_buffer_load_b128(rs_z, (int)(threadIdx.x + q * NT) * 16, sg0 * 256, 0);
 
-    constexpr int U = WB > AB ? WB : AB;  // unroll (both divide it)
-    u32x4_t aring[AB][AQ], wring[WB][4][WL];
+    // blocks per unrolled iteration: the ring slot of every step must be a constant, 4 * U % WD == 0
+    constexpr int U = (WD % 4 == 0 ? WD / 4 : (WD % 2 == 0 ? WD / 2 : WD)) * AB;
+    static_assert((4 * U) % WD == 0 && U % AB == 0, "ring slots must repeat with the unrolled loop");
+    u32x4_t aring[AB][AQ], wring[WD][WL];
     // Past the end of the slice the loads go through an empty descriptor: a scalar select,
     // no vector instruction, and the buffer unit returns zero without touching memory.
     const __amdgpu_buffer_rsrc_t rs_none = make_rsrc(pw, 0u);
@@ -343,13 +349,11 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
     u32x4_t afirst[AQ];
     load_a(0, afirst);
 #pragma unroll
-    for (int d = 0; d < U; ++d) {
-        if (d < WB) {
+    for (int g = 0; g < (WD < 4 ? WD : 4); ++g) load_w(g >> 2, g & 3, wring[g]);
 #pragma unroll
-            for (int st = 0; st < 4; ++st) load_w(d, st, wring[d][st]);
-        }
-        if (d + 1 <= AB) load_a(d + 1, aring[(d + 1) % AB]);
-    }
+    for (int d = 1; d <= AB; ++d) load_a(d, aring[d % AB]);
+#pragma unroll
+    for (int g = 4; g < WD; ++g) load_w(g >> 2, g & 3, wring[g]);
 
     float4_t acc[MT][4];
 #pragma unroll
@@ -424,8 +428,8 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
             for (int st = 0; st < 4; ++st) {
                 u32x4_t wv[WL];
 #pragma unroll
-                for (int h = 0; h < WL; ++h) wv[h] = wring[u % WB][st][h];
-                load_w(i + WB, st, wring[u % WB][st]);  // refill this ring slot
+                for (int h = 0; h < WL; ++h) wv[h] = wring[(4 * u + st) % WD][h];
+                load_w(i + (st + WD) / 4, (st + WD) & 3, wring[(4 * u + st) % WD]);  // refill this ring slot
                 if (live) {
                     uint32_t wp[WL][4];
 #pragma unroll
@@ -673,15 +677,15 @@ static int pk4_env(const char *name, int dflt) {
 
 template <typename TT, int BITS, int MT, bool GS, bool BPG1, int XQ>
 static int pk4_go4(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, int gslice) {
-    constexpr int AB = Pk4Ring<MT, BITS>::AB, WB = Pk4Ring<MT, BITS>::WB;
+    constexpr int AB = Pk4Ring<MT, BITS>::AB, WD = Pk4Ring<MT, BITS>::WD;
     const size_t lds = (size_t)8 * MT * 4096 + (size_t)gslice * 256 * (GS ? 2 : 1);
     static size_t attr_lds = 0;  // one per instantiation
     if (lds > attr_lds) {
-        OXQ_HIP_CHECK(hipFuncSetAttribute((const void *)pk4_mfma_kernel<TT, BITS, MT, GS, BPG1, AB, WB, XQ>,
+        OXQ_HIP_CHECK(hipFuncSetAttribute((const void *)pk4_mfma_kernel<TT, BITS, MT, GS, BPG1, AB, WD, XQ>,
                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         attr_lds = lds;
     }
-    hipLaunchKernelGGL((pk4_mfma_kernel<TT, BITS, MT, GS, BPG1, AB, WB, XQ>), grid, dim3(512), lds, s,
+    hipLaunchKernelGGL((pk4_mfma_kernel<TT, BITS, MT, GS, BPG1, AB, WD, XQ>), grid, dim3(512), lds, s,
                        (const uint16_t *)p.x, p.w.pw, p.w.pzs, (const uint16_t *)p.bias, (uint16_t *)p.y,
                        (float *)ctx->workspace, (int)p.M, (int)p.w.K, (int)p.w.N, p.w.group_shift, gslice,
                        pk4_env("OXQ_PK4_INTERLEAVE", 0), p.act);
