@@ -303,7 +303,7 @@ __global__ __launch_bounds__(512) void gguf_gemv_lds_kernel(const void *__restri
 #pragma unroll
         for (int b = 0; b < CB; ++b) {
             const int c = base + b * nthr;
-            v[b] = c < full ? wsrc[c] : u32x4_t{0u, 0u, 0u, 0u};
+            v[b] = c < full ? __builtin_nontemporal_load(wsrc + c) : u32x4_t{0u, 0u, 0u, 0u};  // read once
         }
 #pragma unroll
         for (int b = 0; b < CB; ++b) {

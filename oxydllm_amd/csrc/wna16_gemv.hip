@@ -325,20 +325,20 @@ template <int WPL> struct WordVec;
 template <> struct WordVec<4> {
     typedef uint32_t type __attribute__((ext_vector_type(4)));
     __device__ static __forceinline__ type load(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
-        return __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0);
+        return __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 2);  // weights are read once: nontemporal
     }
 };
 template <> struct WordVec<2> {
     typedef uint32_t type __attribute__((ext_vector_type(2)));
     __device__ static __forceinline__ type load(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
-        return __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, 0);
+        return __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, 2);
     }
 };
 template <> struct WordVec<1> {
     typedef uint32_t type __attribute__((ext_vector_type(1)));
     __device__ static __forceinline__ type load(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
         type v;
-        v[0] = __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0);
+        v[0] = __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 2);
         return v;
     }
 };
@@ -601,7 +601,7 @@ __global__ __launch_bounds__(512) void gptq_gemv_fast(
             u32x4_t w[WR];
 #pragma unroll
             for (int t = 0; t < WR; ++t)
-                w[t] = __builtin_amdgcn_raw_buffer_load_b128(rs_w, voff_w, (kc / PF + t) * rowbytes, 0);
+                w[t] = __builtin_amdgcn_raw_buffer_load_b128(rs_w, voff_w, (kc / PF + t) * rowbytes, 2);  // nontemporal
             const uint32_t zw = valid ? qz[(size_t)g * (N / PF) + n0 / PF] : 0u;
             uint2 sv = valid ? *(const uint2 *)(sc + (size_t)g * N + n0) : uint2{0u, 0u};
             float acc[MB][4], xe[MB], xo[MB];
