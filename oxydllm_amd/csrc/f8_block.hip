@@ -69,7 +69,7 @@ __global__ __launch_bounds__(256) void f8_gemv_kernel(const uint16_t *__restrict
     for (int m = 0; m < MB; ++m) acc[m] = 0.0f;
     if (CHUNKED) {
         for (int c = lane; c < (K >> 4); c += 64) {
-            const u32x4_t q = *(const u32x4_t *)(wrow + (size_t)c * 16);
+            const u32x4_t q = __builtin_nontemporal_load((const u32x4_t *)(wrow + (size_t)c * 16));  // read once
             const float sc = srow[(c * 16) / block_c];
             const uint32_t q0 = q[0], q1 = q[1], q2 = q[2], q3 = q[3];
             const uint32_t qw[4] = {q0, q1, q2, q3};
