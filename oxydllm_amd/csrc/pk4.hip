@@ -212,7 +212,7 @@ __global__ __launch_bounds__(256) void pk4_dequant_kernel(const uint32_t *__rest
 // issued load makes it wait for all of them, which serialises the pipeline.
 // Activation loads of block b+1 are issued before the weight loads of block
 // b+2: loads retire in order, and this way waiting for the former leaves the
-// latter in flight.  The strip's zeros and scales are staged in LDS once.
+// latter in flight.  Zeros and scales are staged in LDS once (below).
 // The 8 partial 16*MT x 64 tiles meet in LDS (each wave's slot is its own
 // activation slot) and are added in wave order, which fixes the summation order.
 //
@@ -278,8 +278,8 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
     // K slice of this workgroup (grid.y slices of `gslice` whole groups; one slice = the
     // whole strip unless the grid would leave most CUs idle), then the wave's blocks inside
     // it, by local index i: either one contiguous run of whole groups, the groups dealt out
-    // as evenly as 8 waves allow, or every 8th group (the 8 waves then sweep the slice
-    // together, front to back).
+    // as evenly as 8 waves allow, or (multi-tile kernels only, a tuning switch that measured
+    // equal) every 8th group, the 8 waves then sweeping the slice together, front to back.
     const int gs7 = gshift - 7;
     const int sg0 = blockIdx.y * gslice;                 // first group of the slice
     const int SG = min(G, sg0 + gslice) - sg0;           // groups in the slice (>= 1)
@@ -317,13 +317,20 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
         *(u32x4_t *)(slot + row * 256 + ((ni ^ (row & 15)) << 4)) = u32x4_t{0u, 0u, 0u, 0u};
     }
 
-    constexpr int ZCH = 2048 / NT;  // 16-byte chunks per thread: 32 KB = 128 groups
+    // Zeros and scales go to LDS, [G][16 column quads].  Single-tile kernels (MT = 1): every wave
+    // stages those of its own groups, so no barrier stands before its loop (7.85 instead of 8.45 us
+    // at M = 1).  The others stage the slice together and meet at a barrier: there the per-wave
+    // form pushes the kernel past its register budget.
+    constexpr bool ZWAVE = MT == 1;
+    constexpr int ZCH = 4;  // 16-byte chunks per lane or thread: 16 groups a wave, 128 a workgroup
     u32x4_t zstage[ZCH];
-    const int zchunks = SG * 16;  // the slice's groups only
+    const int ZT = ZWAVE ? 64 : NT, zt = ZWAVE ? lane : (int)threadIdx.x;
+    const int zc0 = ZWAVE ? (wg0 - sg0) * 16 : 0, zchunks = (ZWAVE ? wgn : SG) * 16;  // within the slice
 #pragma unroll
     for (int q = 0; q < ZCH; ++q)
-        if (q * NT < zchunks)  // block-uniform
-            zstage[q] = __builtin_amdgcn_raw_buffer_load_b128(rs_z, (int)(threadIdx.x + q * NT) * 16, sg0 * 256, 0);
+        if (q * ZT < zchunks)  // uniform
+            zstage[q] = __builtin_amdgcn_raw_buffer_load_b128(
+                rs_z, !ZWAVE || zt + q * ZT < zchunks ? (zc0 + zt + q * ZT) * 16 : OOB, sg0 * 256, 0);
 
     // blocks per unrolled iteration: the ring slot of every step must be a constant, 4 * U % WD == 0
     constexpr int U = (WD % 4 == 0 ? WD / 4 : (WD % 2 == 0 ? WD / 2 : WD)) * AB;
@@ -382,8 +389,8 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
 
 #pragma unroll
     for (int q = 0; q < ZCH; ++q) {
-        const int c = (int)threadIdx.x + q * NT;
-        if (c < zchunks) {
+        const int c = zc0 + zt + q * ZT;
+        if (zt + q * ZT < zchunks) {
             if (GS) {
                 const uint32_t z0 = zstage[q][0], z1 = zstage[q][1], z2 = zstage[q][2], z3 = zstage[q][3];
                 const uint32_t zv[4] = {z0, z1, z2, z3};
@@ -401,7 +408,7 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
         }
     }
     store_a(afirst);
-    __syncthreads();
+    if (!ZWAVE) __syncthreads();
 
     for (int ib = 0; ib < nloc; ib += U) {
 #pragma unroll
@@ -692,7 +699,7 @@ static int pk4_go4(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, 
     hipLaunchKernelGGL((pk4_mfma_kernel<TT, BITS, MT, GS, BPG1, AB, WD, XQ>), grid, dim3(512), lds, s,
                        (const uint16_t *)p.x, p.w.pw, p.w.pzs, (const uint16_t *)p.bias, (uint16_t *)p.y,
                        (float *)ctx->workspace, (int)p.M, (int)p.w.K, (int)p.w.N, p.w.group_shift, gslice,
-                       pk4_env("OXQ_PK4_INTERLEAVE", 0), p.act);
+                       MT == 1 ? 0 : pk4_env("OXQ_PK4_INTERLEAVE", 0), p.act);
     OXQ_HIP_CHECK(hipGetLastError());
     return OXQ_OK;
 }
