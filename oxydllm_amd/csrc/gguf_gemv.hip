@@ -269,7 +269,12 @@ __device__ __forceinline__ void ld_x8(const unsigned char *xrow, int upitch, int
     }
 }
 
-template <int FMT, bool BF16X, int MB>
+// PW (one activation row, one weight row per wave, the launcher checks the sizes): every wave
+// fetches its own weight row and only the activations meet at the barrier.  Staged jointly the
+// kernel is the sum of its parts (4096 x 4096 Q4_K, M = 1: 6.9 us = 2.65 us launch and activations
+// + 1.85 us weights + 2.5 us decode and dot, each measured with the others cut out): nobody
+// computes until the last row of the workgroup has arrived.
+template <int FMT, bool BF16X, int MB, bool PW>
 __global__ __launch_bounds__(512) void gguf_gemv_lds_kernel(const void *__restrict__ x,
                                                             const uint8_t *__restrict__ w,
                                                             const void *__restrict__ bias,
@@ -292,12 +297,54 @@ __global__ __launch_bounds__(512) void gguf_gemv_lds_kernel(const void *__restri
     const int wchunks = (int)((head + (size_t)nrows * row_bytes + 15) >> 4);
     const int cpr = K * XB / 16;  // chunks per activation row
     const int nthr = blockDim.x, nwaves = blockDim.x >> 6;
-    // Staging copies in batches of 4 loads per thread: with one load per loop trip every
-    // trip pays a full memory round trip before its LDS store.
     constexpr int CB = 4;
+    constexpr int WCH = 6;  // 16-byte chunks per lane that hold one weight row (PW)
     // chunks that lie wholly inside the tensor; only the tensor's very last chunk can be partial
     const int full = (int)min((size_t)wchunks, (total_bytes - a0) >> 4);
     const u32x4_t *wsrc = (const u32x4_t *)(w + a0);
+    if constexpr (PW) {
+        // one straight-line batch of activation loads, then the wave's own row: the compiler can count
+        // the younger loads, so storing the activations leaves the weights in flight
+        // (buffer loads: out-of-range lanes need no branch, which would make the count unknowable)
+        constexpr int OOB = 0x7FFFFF00;
+        const __amdgpu_buffer_rsrc_t rs_x = make_rsrc(x, (uint32_t)cpr * 16u);
+        const __amdgpu_buffer_rsrc_t rs_w = make_rsrc(w + a0, (uint32_t)full * 16u);
+        u32x4_t xv[CB], wv[WCH];
+#pragma unroll
+        for (int b = 0; b < CB; ++b)
+            xv[b] = __builtin_amdgcn_raw_buffer_load_b128(rs_x, ((int)threadIdx.x + b * nthr) * 16, 0, 0);
+        const size_t rb = head + (size_t)wave * row_bytes;  // the row's bytes inside the workgroup's span
+        const int wc0 = (int)(rb >> 4);
+        const int wc1 = wave < nrows ? min((int)((rb + row_bytes + 15) >> 4), full) : wc0;
+#pragma unroll
+        for (int q = 0; q < WCH; ++q) {
+            const int c = wc0 + lane + 64 * q;
+            wv[q] = __builtin_amdgcn_raw_buffer_load_b128(rs_w, c < wc1 ? c * 16 : OOB, 0, 2);  // nontemporal
+        }
+        // stores without a branch as well (a load whose only use is conditional gets moved into the
+        // branch): lanes past the row write the unused padding chunk of the layout, unit index `units`
+#pragma unroll
+        for (int b = 0; b < CB; ++b) {
+            const int g = (int)threadIdx.x + b * nthr;
+            const int u = g / CPU, cc = g - u * CPU;
+            *(u32x4_t *)(lds_x + (size_t)(g < cpr ? cc * upitch + u : units) * 16) = xv[b];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int q = 0; q < WCH; ++q) {
+            const int c = wc0 + lane + 64 * q;
+            if (c < wc1) ((u32x4_t *)lds_w)[c] = wv[q];
+        }
+        if (full < wchunks && wave == nrows - 1 && lane == 0) {  // the tensor's last, partial chunk: byte by byte
+            const size_t off = a0 + (size_t)full * 16;
+            uint32_t t[4] = {0u, 0u, 0u, 0u};
+            for (int i = 0; i < 16; ++i)
+                if (off + i < total_bytes) t[i >> 2] |= (uint32_t)w[off + i] << (8 * (i & 3));
+            ((u32x4_t *)lds_w)[full] = u32x4_t{t[0], t[1], t[2], t[3]};
+        }
+    } else {
+    // Staging copies in batches of 4 loads per thread: with one load per loop trip every
+    // trip pays a full memory round trip before its LDS store.
     for (int base = threadIdx.x; base < full; base += nthr * CB) {
         u32x4_t v[CB];
 #pragma unroll
@@ -343,6 +390,7 @@ __global__ __launch_bounds__(512) void gguf_gemv_lds_kernel(const void *__restri
         }
     }
     __syncthreads();
+    }
     for (int r = wave; r < nrows; r += nwaves) {
         const uint8_t *row = lds_w + head + (size_t)r * row_bytes;
         const int n = n0 + r;
@@ -435,12 +483,12 @@ static void launch_rows(hipStream_t s, dim3 grid, const GgufProblem &p, const ui
         hipLaunchKernelGGL((gguf_gemv_kernel<FMT, BF16X, 8>), grid, block, 0, s, x, p.w, p.bias, y, rows, K, N);
 }
 
-template <int FMT, bool BF16X, int MB>
+template <int FMT, bool BF16X, int MB, bool PW = false>
 static int launch_rows_lds_mb(hipStream_t s, const GgufProblem &p, const uint8_t *x, uint8_t *y, int rows,
                               int rpwg, size_t lds) {
     static size_t attr_lds = 0;
     if (lds > attr_lds) {
-        OXQ_HIP_CHECK(hipFuncSetAttribute((const void *)gguf_gemv_lds_kernel<FMT, BF16X, MB>,
+        OXQ_HIP_CHECK(hipFuncSetAttribute((const void *)gguf_gemv_lds_kernel<FMT, BF16X, MB, PW>,
                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         attr_lds = lds;
     }
@@ -448,7 +496,7 @@ static int launch_rows_lds_mb(hipStream_t s, const GgufProblem &p, const uint8_t
     const size_t total = (size_t)N * (size_t)(K / GgufFmt<FMT>::BE) * GgufFmt<FMT>::BB;
     // one wave per row at a time: 8 waves for 8 rows (x is staged once per 8 rows), else 4
     dim3 grid((unsigned)ceil_div(N, rpwg)), block(rpwg >= 8 ? 512 : 256);
-    hipLaunchKernelGGL((gguf_gemv_lds_kernel<FMT, BF16X, MB>), grid, block, lds, s, x, p.w, p.bias, y, rows, K,
+    hipLaunchKernelGGL((gguf_gemv_lds_kernel<FMT, BF16X, MB, PW>), grid, block, lds, s, x, p.w, p.bias, y, rows, K,
                        N, rpwg, total);
     return OXQ_OK;
 }
@@ -456,7 +504,15 @@ static int launch_rows_lds_mb(hipStream_t s, const GgufProblem &p, const uint8_t
 template <int FMT, bool BF16X>
 static int launch_rows_lds(hipStream_t s, const GgufProblem &p, const uint8_t *x, uint8_t *y, int rows,
                            int rpwg, size_t lds) {
-    if (rows <= 1) return launch_rows_lds_mb<FMT, BF16X, 1>(s, p, x, y, rows, rpwg, lds);
+    if (rows <= 1) {
+        // a wave per weight row needs: 8 waves for the 8 rows, the row in 6 chunks a lane, x in one batch
+        const size_t row_bytes = (size_t)(p.K / GgufFmt<FMT>::BE) * GgufFmt<FMT>::BB;
+        const char *pw_env = getenv("OXQ_GGUF_PW");
+        if (rpwg == 8 && row_bytes + 30 <= 6 * 64 * 16 && p.K * (BF16X ? 2 : 4) / 16 <= 4 * 512 &&
+            !(pw_env && atoi(pw_env) == 0))
+            return launch_rows_lds_mb<FMT, BF16X, 1, true>(s, p, x, y, rows, rpwg, lds);
+        return launch_rows_lds_mb<FMT, BF16X, 1>(s, p, x, y, rows, rpwg, lds);
+    }
     if (rows <= 2) return launch_rows_lds_mb<FMT, BF16X, 2>(s, p, x, y, rows, rpwg, lds);
     if (rows <= 4) return launch_rows_lds_mb<FMT, BF16X, 4>(s, p, x, y, rows, rpwg, lds);
     return launch_rows_lds_mb<FMT, BF16X, 8>(s, p, x, y, rows, rpwg, lds);
