@@ -16,7 +16,7 @@ import torch
 import oracle
 from oxydllm_amd import synth
 from tests import refgen
-from tests.helpers import RTOL, ATOL, as_f32, assert_close, round_x, to_dev
+from tests.helpers import RTOL, ATOL, as_f32, assert_close, bits_of, round_x, to_dev
 
 pytestmark = pytest.mark.gpu
 ops = None
@@ -145,6 +145,34 @@ def test_gguf_mul_mm_f32_activations_keep_f32_weights():
     x = np.random.default_rng(141).standard_normal((m, K)).astype(np.float32)
     y = ops.gguf_quant_mul_mm(to_dev(x), to_dev(data), K, N, fmt)
     assert_close(y, oracle.matmul_nt_f32(x, w), "gguf mul_mm f32")
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+def test_gguf_gemv_single_row_wave_per_weight_row(fmt, monkeypatch):
+    """One activation row: every wave fetches its own weight row (six 16-byte chunks a lane at most, the
+    activations in one batch of four).  Shapes at and past those limits, a last workgroup with fewer rows
+    than waves, rows that start off 16-byte boundaries and a tensor whose size is no multiple of 16; the
+    result must equal the jointly staged kernel's bit for bit (same arithmetic in the same order) and the
+    oracle within tolerance."""
+    elems, bbytes = synth.GGUF_BLOCK_LAYOUT[fmt]
+    shapes = [(13, 256), (8, 2 * elems if elems == 256 else 96), (37, 4096), (21, 5632), (9, 8192)]
+    for N, K in shapes:
+        if K % elems:
+            continue
+        for dt in (torch.float32, torch.bfloat16):
+            say(f"gguf wave-per-row {synth.GGUF_NAMES[fmt]} N={N} K={K} {dt}")
+            data = synth.gguf_weight(fmt, N, K, seed=N + K + fmt)
+            w = oracle.dequantize_gguf(fmt, data, N, K)
+            x = np.random.default_rng(N * 7 + K).standard_normal((1, K)).astype(np.float32)
+            xd, wd = to_dev(x, dt), to_dev(data)
+            xr = x if dt == torch.float32 else round_x(x, oracle.BF16)
+            monkeypatch.setenv("OXQ_GGUF_PW", "1")
+            y = ops.gguf_quant_matmul(xd, wd, K, N, fmt)
+            assert_close(y, oracle.matmul_nt_f32(xr, w), f"gguf wave-per-row {synth.GGUF_NAMES[fmt]} {N}x{K}")
+            monkeypatch.setenv("OXQ_GGUF_PW", "0")
+            joint = ops.gguf_quant_matmul(xd, wd, K, N, fmt)
+            np.testing.assert_array_equal(bits_of(y), bits_of(joint))
+    monkeypatch.delenv("OXQ_GGUF_PW")
 
 
 @pytest.mark.parametrize("fmt", FMTS)
