@@ -278,7 +278,7 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
     // K slice of this workgroup (grid.y slices of `gslice` whole groups; one slice = the
     // whole strip unless the grid would leave most CUs idle), then the wave's blocks inside
     // it, by local index i: either one contiguous run of whole groups, the groups dealt out
-    // as evenly as 8 waves allow, or (multi-tile kernels only, a tuning switch that measured
+    // as evenly as 8 waves allow, or (four-tile kernels only, a tuning switch that measured
     // equal) every 8th group, the 8 waves then sweeping the slice together, front to back.
     const int gs7 = gshift - 7;
     const int sg0 = blockIdx.y * gslice;                 // first group of the slice
@@ -317,11 +317,11 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
         *(u32x4_t *)(slot + row * 256 + ((ni ^ (row & 15)) << 4)) = u32x4_t{0u, 0u, 0u, 0u};
     }
 
-    // Zeros and scales go to LDS, [G][16 column quads].  Single-tile kernels (MT = 1): every wave
-    // stages those of its own groups, so no barrier stands before its loop (7.85 instead of 8.45 us
-    // at M = 1).  The others stage the slice together and meet at a barrier: there the per-wave
-    // form pushes the kernel past its register budget.
-    constexpr bool ZWAVE = MT == 1;
+    // Zeros and scales go to LDS, [G][16 column quads].  Up to three row tiles every wave stages
+    // those of its own groups, so no barrier stands before its loop (7.85 instead of 8.45 us at
+    // M = 1, 5 % at M = 33..48).  The four-tile kernels stage the slice together and meet at a
+    // barrier: there the per-wave form pushes the kernel past its register budget.
+    constexpr bool ZWAVE = MT <= 3;
     constexpr int ZCH = 4;  // 16-byte chunks per lane or thread: 16 groups a wave, 128 a workgroup
     u32x4_t zstage[ZCH];
     const int ZT = ZWAVE ? 64 : NT, zt = ZWAVE ? lane : (int)threadIdx.x;
@@ -699,7 +699,7 @@ static int pk4_go4(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, 
     hipLaunchKernelGGL((pk4_mfma_kernel<TT, BITS, MT, GS, BPG1, AB, WD, XQ>), grid, dim3(512), lds, s,
                        (const uint16_t *)p.x, p.w.pw, p.w.pzs, (const uint16_t *)p.bias, (uint16_t *)p.y,
                        (float *)ctx->workspace, (int)p.M, (int)p.w.K, (int)p.w.N, p.w.group_shift, gslice,
-                       MT == 1 ? 0 : pk4_env("OXQ_PK4_INTERLEAVE", 0), p.act);
+                       MT <= 3 ? 0 : pk4_env("OXQ_PK4_INTERLEAVE", 0), p.act);
     OXQ_HIP_CHECK(hipGetLastError());
     return OXQ_OK;
 }
