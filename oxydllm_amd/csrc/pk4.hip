@@ -243,7 +243,8 @@ template <int MT, int BITS> struct Pk4Ring {
 // BPG1: group size 128, i.e. every block is one group (no group bookkeeping).
 // XQ: activation loads per block and lane that can hold rows below M (4 rows each); the
 // launcher passes 4 * MT, or fewer for a short single tile, whose other rows stay zero in LDS.
-template <typename TT, int BITS, int MT, bool GS, bool BPG1, int AB, int WD, int XQ>
+// ZW: every wave stages the zeros and scales of its own groups (no barrier before the loop).
+template <typename TT, int BITS, int MT, bool GS, bool BPG1, int AB, int WD, int XQ, bool ZW>
 __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restrict__ x,
                                                        const uint32_t *__restrict__ pw,
                                                        const uint32_t *__restrict__ pzs,
@@ -278,7 +279,7 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
     // K slice of this workgroup (grid.y slices of `gslice` whole groups; one slice = the
     // whole strip unless the grid would leave most CUs idle), then the wave's blocks inside
     // it, by local index i: either one contiguous run of whole groups, the groups dealt out
-    // as evenly as 8 waves allow, or (four-tile kernels only, a tuning switch that measured
+    // as evenly as 8 waves allow, or (jointly staged kernels only, a tuning switch that measured
     // equal) every 8th group, the 8 waves then sweeping the slice together, front to back.
     const int gs7 = gshift - 7;
     const int sg0 = blockIdx.y * gslice;                 // first group of the slice
@@ -317,12 +318,13 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
         *(u32x4_t *)(slot + row * 256 + ((ni ^ (row & 15)) << 4)) = u32x4_t{0u, 0u, 0u, 0u};
     }
 
-    // Zeros and scales go to LDS, [G][16 column quads].  Up to three row tiles every wave stages
-    // those of its own groups, so no barrier stands before its loop (7.85 instead of 8.45 us at
-    // M = 1, 5 % at M = 33..48).  The four-tile kernels stage the slice together and meet at a
-    // barrier: there the per-wave form pushes the kernel past its register budget.
-    constexpr bool ZWAVE = MT <= 3;
-    constexpr int ZCH = 4;  // 16-byte chunks per lane or thread: 16 groups a wave, 128 a workgroup
+    // Zeros and scales go to LDS, [G][16 column quads].  ZW: every wave stages those of its own
+    // groups, so no barrier stands before its loop (7.85 instead of 8.45 us at M = 1, 5 % at
+    // M = 33..48 and at 256).  The four-tile kernels are at their register budget: they do so with
+    // one 16-byte chunk per lane, i.e. up to four groups a wave, and otherwise stage the slice
+    // together and meet at a barrier.
+    constexpr bool ZWAVE = ZW;
+    constexpr int ZCH = ZW && MT == 4 ? 1 : 4;  // 16-byte chunks per lane (4 groups each) or thread
     u32x4_t zstage[ZCH];
     const int ZT = ZWAVE ? 64 : NT, zt = ZWAVE ? lane : (int)threadIdx.x;
     const int zc0 = ZWAVE ? (wg0 - sg0) * 16 : 0, zchunks = (ZWAVE ? wgn : SG) * 16;  // within the slice
@@ -686,20 +688,20 @@ static int pk4_env(const char *name, int dflt) {
     return e ? atoi(e) : dflt;
 }
 
-template <typename TT, int BITS, int MT, bool GS, bool BPG1, int XQ>
+template <typename TT, int BITS, int MT, bool GS, bool BPG1, int XQ, bool ZW = (MT <= 3)>
 static int pk4_go4(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, int gslice) {
     constexpr int AB = Pk4Ring<MT, BITS>::AB, WD = Pk4Ring<MT, BITS>::WD;
     const size_t lds = (size_t)8 * MT * 4096 + (size_t)gslice * 256 * (GS ? 2 : 1);
     static size_t attr_lds = 0;  // one per instantiation
     if (lds > attr_lds) {
-        OXQ_HIP_CHECK(hipFuncSetAttribute((const void *)pk4_mfma_kernel<TT, BITS, MT, GS, BPG1, AB, WD, XQ>,
+        OXQ_HIP_CHECK(hipFuncSetAttribute((const void *)pk4_mfma_kernel<TT, BITS, MT, GS, BPG1, AB, WD, XQ, ZW>,
                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         attr_lds = lds;
     }
-    hipLaunchKernelGGL((pk4_mfma_kernel<TT, BITS, MT, GS, BPG1, AB, WD, XQ>), grid, dim3(512), lds, s,
+    hipLaunchKernelGGL((pk4_mfma_kernel<TT, BITS, MT, GS, BPG1, AB, WD, XQ, ZW>), grid, dim3(512), lds, s,
                        (const uint16_t *)p.x, p.w.pw, p.w.pzs, (const uint16_t *)p.bias, (uint16_t *)p.y,
                        (float *)ctx->workspace, (int)p.M, (int)p.w.K, (int)p.w.N, p.w.group_shift, gslice,
-                       MT <= 3 ? 0 : pk4_env("OXQ_PK4_INTERLEAVE", 0), p.act);
+                       ZW ? 0 : pk4_env("OXQ_PK4_INTERLEAVE", 0), p.act);
     OXQ_HIP_CHECK(hipGetLastError());
     return OXQ_OK;
 }
@@ -712,6 +714,10 @@ static int pk4_go3(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, 
         const int xq = pk4_env("OXQ_PK4_XQ", 1) ? (int)ceil_div(p.M, 4) : 4;
         if (xq == 1) return pk4_go4<TT, BITS, MT, GS, BPG1, 1>(ctx, s, grid, p, gslice);
         if (xq == 2) return pk4_go4<TT, BITS, MT, GS, BPG1, 2>(ctx, s, grid, p, gslice);
+    }
+    if constexpr (MT == 4) {  // at most four groups a wave: the single-chunk per-wave staging
+        if (gslice <= 32 && pk4_env("OXQ_PK4_INTERLEAVE", 0) == 0)
+            return pk4_go4<TT, BITS, MT, GS, BPG1, 4 * MT, true>(ctx, s, grid, p, gslice);
     }
     return pk4_go4<TT, BITS, MT, GS, BPG1, 4 * MT>(ctx, s, grid, p, gslice);
 }
