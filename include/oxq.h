@@ -306,6 +306,12 @@ int oxq_moe_group(oxq_ctx *ctx, void *stream, const oxq_tensor *top_idx, const o
                   int64_t n_experts, const oxq_tensor *expert_offsets, const oxq_tensor *token_ids,
                   const oxq_tensor *pair_weights, const oxq_tensor *pair_pos);
 
+/* oxq_moe_route followed by oxq_moe_group (n_experts = logits' second dim) as one call, same arguments and
+ * outputs; up to 64 (token, slot) pairs and 256 experts, i.e. decode, it is one launch instead of two. */
+int oxq_moe_route_group(oxq_ctx *ctx, void *stream, const oxq_tensor *logits, int64_t top_k, int norm_topk,
+                        const oxq_tensor *top_idx, const oxq_tensor *top_vals, const oxq_tensor *expert_offsets,
+                        const oxq_tensor *token_ids, const oxq_tensor *pair_weights, const oxq_tensor *pair_pos);
+
 typedef enum oxq_gated_act {
     OXQ_ACT_GATED_SILU = 0,      /* [.., gate | up]: silu(gate) * up, ffn_kernels.metal:19-68 */
     OXQ_ACT_GATED_GELU_TANH = 1, /* [.., gate | up]: gelu_tanh(gate) * up, ffn_kernels.metal:115-160 */

@@ -105,6 +105,7 @@ SIGNATURES = {
                                               C.c_int64, C.c_int64, C.c_float, _TP, C.POINTER(C.c_int)]),
     "oxq_moe_route": (C.c_int, [_VP, _VP, _TP, C.c_int64, C.c_int, _TP, _TP]),
     "oxq_moe_group": (C.c_int, [_VP, _VP, _TP, _TP, C.c_int64, _TP, _TP, _TP, _TP]),
+    "oxq_moe_route_group": (C.c_int, [_VP, _VP, _TP, C.c_int64, C.c_int, _TP, _TP, _TP, _TP, _TP, _TP]),
     "oxq_gated_activation": (C.c_int, [_VP, _VP, _TP, C.c_int, C.c_float, _TP]),
     "oxq_activation_mul": (C.c_int, [_VP, _VP, _TP, _TP, C.c_int, _TP]),
     "oxq_moe_combine": (C.c_int, [_VP, _VP, _TP, _TP, _TP, _TP]),

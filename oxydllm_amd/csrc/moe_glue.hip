@@ -46,16 +46,10 @@ template <> __device__ __forceinline__ void store_f32<BF16Tag>(BF16Tag *p, size_
 // ---------------------------------------------------------------------------
 // route: one wave per token, probabilities in LDS
 // ---------------------------------------------------------------------------
+// one token, one wave: lane s < top_k ends with slot s in (my_idx, my_val); probs = E floats of LDS
 template <typename T>
-__global__ __launch_bounds__(256) void moe_route_kernel(const T *__restrict__ logits, int ntok, int E, int top_k,
-                                                        int norm_topk, int32_t *__restrict__ top_idx,
-                                                        float *__restrict__ top_vals) {
-    extern __shared__ float route_lds[];  // [4 waves][E]
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int t = blockIdx.x * 4 + wave;
-    if (t >= ntok) return;  // wave-uniform; no barrier below
-    float *probs = route_lds + (size_t)wave * E;
-    const T *l = logits + (size_t)t * E;
+__device__ __forceinline__ void route_token(const T *__restrict__ l, int E, int top_k, int norm_topk, float *probs,
+                                            int lane, int &out_idx, float &out_val) {
     float mx = -INFINITY;
     for (int e = lane; e < E; e += 64) mx = fmaxf(mx, load_f32(l, e));
 #pragma unroll
@@ -97,10 +91,76 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T *__restrict__ lo
         if (lane == 0) probs[bi] = -2.0f;  // taken
         chosen_sum += bv;  // slot order, as the reference's sum over the gathered values
     }
+    out_idx = my_idx;
+    out_val = norm_topk ? my_val / chosen_sum : my_val;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void moe_route_kernel(const T *__restrict__ logits, int ntok, int E, int top_k,
+                                                        int norm_topk, int32_t *__restrict__ top_idx,
+                                                        float *__restrict__ top_vals) {
+    extern __shared__ float route_lds[];  // [4 waves][E]
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int t = blockIdx.x * 4 + wave;
+    if (t >= ntok) return;  // wave-uniform; no barrier below
+    int my_idx;
+    float my_val;
+    route_token(logits + (size_t)t * E, E, top_k, norm_topk, route_lds + (size_t)wave * E, lane, my_idx, my_val);
     if (lane < top_k) {
         const size_t i = (size_t)t * top_k + lane;
         top_idx[i] = my_idx;
-        top_vals[i] = norm_topk ? my_val / chosen_sum : my_val;
+        top_vals[i] = my_val;
+    }
+}
+
+// Decode sizes (P <= 64), one wave: the pairs of (top_idx, top_vals) grouped by expert.  `scratch` = 2 E ints of LDS.
+__device__ __forceinline__ void group_pairs_small(const int32_t *top_idx, const float *top_vals, int P, int E, int top_k,
+                                                  int32_t *scratch, int lane, int32_t *__restrict__ offsets,
+                                                  int32_t *__restrict__ tokens, float *__restrict__ weights,
+                                                  int32_t *__restrict__ pair_pos) {
+    // Decode sizes: one pair per lane, no counting matrix.  The wave peels off one expert at a
+    // time: the first unplaced lane's expert, a ballot of the lanes that share it, rank = the
+    // matching lanes below me (pair order = token order inside an expert), count = the ballot's
+    // population.  At most min(P, E) rounds of scalar work instead of chains of dependent LDS
+    // accesses (E + 64 + E of them in the general path).
+    int32_t *count = scratch;  // [E], then start[E]
+    int32_t *start = scratch + E;
+    for (int e = lane; e < E; e += 64) count[e] = 0;
+    const int e = lane < P ? top_idx[lane] : -1;
+    const bool ok = e >= 0 && e < E;  // ids outside [0, E) are dropped
+    int rank = 0;
+    unsigned long long todo = __ballot(ok);
+    while (todo) {  // wave-uniform
+        const int first = __builtin_ctzll(todo);
+        const int e0 = __shfl(e, first, 64);
+        const unsigned long long m = __ballot(ok && e == e0);
+        if (ok && e == e0) rank = __builtin_popcountll(m & ((1ull << lane) - 1ull));
+        if (lane == first) count[e0] = __builtin_popcountll(m);
+        todo &= ~m;
+    }
+    // exclusive scan of the counts in expert order, 64 experts per round
+    int carry = 0;
+    for (int e1 = 0; e1 < E; e1 += 64) {
+        const int ee = e1 + lane;
+        const int c = ee < E ? count[ee] : 0;
+        int incl = c;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const int t = __shfl_up(incl, off, 64);
+            if (lane >= off) incl += t;
+        }
+        if (ee < E) {
+            start[ee] = carry + incl - c;
+            offsets[ee] = carry + incl - c;
+        }
+        carry += __shfl(incl, 63, 64);
+    }
+    if (lane == 0) offsets[E] = carry;
+    if (ok) {
+        const int pos = start[e] + rank;
+        tokens[pos] = lane / top_k;
+        weights[pos] = top_vals[lane];
+        pair_pos[lane] = pos;
     }
 }
 
@@ -117,50 +177,7 @@ __global__ __launch_bounds__(64) void moe_group_kernel(const int32_t *__restrict
     int32_t *base = group_lds + (size_t)E * 64;
     const int lane = threadIdx.x;
     if (P <= 64) {
-        // Decode sizes: one pair per lane, no counting matrix.  The wave peels off one expert at a
-        // time: the first unplaced lane's expert, a ballot of the lanes that share it, rank = the
-        // matching lanes below me (pair order = token order inside an expert), count = the ballot's
-        // population.  At most min(P, E) rounds of scalar work instead of chains of dependent LDS
-        // accesses (E + 64 + E of them in the general path).
-        int32_t *count = group_lds;  // [E], then start[E]
-        int32_t *start = group_lds + E;
-        for (int e = lane; e < E; e += 64) count[e] = 0;
-        const int e = lane < P ? top_idx[lane] : -1;
-        const bool ok = e >= 0 && e < E;  // ids outside [0, E) are dropped
-        int rank = 0;
-        unsigned long long todo = __ballot(ok);
-        while (todo) {  // wave-uniform
-            const int first = __builtin_ctzll(todo);
-            const int e0 = __shfl(e, first, 64);
-            const unsigned long long m = __ballot(ok && e == e0);
-            if (ok && e == e0) rank = __builtin_popcountll(m & ((1ull << lane) - 1ull));
-            if (lane == first) count[e0] = __builtin_popcountll(m);
-            todo &= ~m;
-        }
-        // exclusive scan of the counts in expert order, 64 experts per round
-        int carry = 0;
-        for (int e1 = 0; e1 < E; e1 += 64) {
-            const int ee = e1 + lane;
-            const int c = ee < E ? count[ee] : 0;
-            int incl = c;
-#pragma unroll
-            for (int off = 1; off < 64; off <<= 1) {
-                const int t = __shfl_up(incl, off, 64);
-                if (lane >= off) incl += t;
-            }
-            if (ee < E) {
-                start[ee] = carry + incl - c;
-                offsets[ee] = carry + incl - c;
-            }
-            carry += __shfl(incl, 63, 64);
-        }
-        if (lane == 0) offsets[E] = carry;
-        if (ok) {
-            const int pos = start[e] + rank;
-            tokens[pos] = lane / top_k;
-            weights[pos] = top_vals[lane];
-            pair_pos[lane] = pos;
-        }
+        group_pairs_small(top_idx, top_vals, P, E, top_k, group_lds, lane, offsets, tokens, weights, pair_pos);
         return;
     }
     const int L = (P + 63) / 64;
@@ -202,6 +219,39 @@ __global__ __launch_bounds__(64) void moe_group_kernel(const int32_t *__restrict
         weights[pos] = top_vals[i];
         pair_pos[i] = pos;
     }
+}
+
+// ---------------------------------------------------------------------------
+// route + group in one launch for decode sizes (n_tokens * top_k <= 64): the waves route the tokens
+// between them, the choices stay in LDS, and after one barrier wave 0 groups them.  Same arithmetic
+// and the same outputs as the two kernels above, one launch period less.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(1024) void moe_route_group_kernel(const T *__restrict__ logits, int ntok, int E, int top_k,
+                                                               int norm_topk, int32_t *__restrict__ top_idx,
+                                                               float *__restrict__ top_vals, int32_t *__restrict__ offsets,
+                                                               int32_t *__restrict__ tokens, float *__restrict__ weights,
+                                                               int32_t *__restrict__ pair_pos) {
+    extern __shared__ float rg_lds[];  // [waves][E] probabilities, [64] chosen experts, [64] their weights, [2 E] group scratch
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    int32_t *s_idx = (int32_t *)(rg_lds + (size_t)nw * E);
+    float *s_val = (float *)(s_idx + 64);
+    int32_t *scratch = (int32_t *)(s_val + 64);
+    for (int t = wave; t < ntok; t += nw) {
+        int my_idx;
+        float my_val;
+        route_token(logits + (size_t)t * E, E, top_k, norm_topk, rg_lds + (size_t)wave * E, lane, my_idx, my_val);
+        if (lane < top_k) {
+            const int i = t * top_k + lane;
+            top_idx[i] = my_idx;
+            top_vals[i] = my_val;
+            s_idx[i] = my_idx;
+            s_val[i] = my_val;
+        }
+    }
+    __syncthreads();
+    if (wave == 0)
+        group_pairs_small(s_idx, s_val, ntok * top_k, E, top_k, scratch, lane, offsets, tokens, weights, pair_pos);
 }
 
 // ---------------------------------------------------------------------------
@@ -291,6 +341,33 @@ int launch_moe_group(oxq_ctx *ctx, hipStream_t s, const int32_t *top_idx, const 
     }
     hipLaunchKernelGGL(moe_group_kernel, grid, block, lds, s, top_idx, top_vals, (int)P, (int)E, offsets, tokens,
                        weights, pair_pos, (int)top_k);
+    OXQ_HIP_CHECK(hipGetLastError());
+    return OXQ_OK;
+}
+
+int launch_moe_route_group(oxq_ctx *ctx, hipStream_t s, const void *logits, int dtype, int64_t T, int64_t E,
+                           int64_t top_k, int norm_topk, int32_t *top_idx, float *top_vals, int32_t *offsets,
+                           int32_t *tokens, float *weights, int32_t *pair_pos) {
+    const int nw = (int)std::min<int64_t>(T, 16);
+    dim3 grid(1), block((unsigned)nw * 64);
+    set_plan(ctx, "moe_route_group", grid, block, 1, 1, 0);
+    if (ctx->plan_only) return OXQ_OK;
+    const size_t lds = ((size_t)nw * E + 128 + 2 * (size_t)E) * sizeof(float);
+#define OXQ_RG(TY)                                                                                                   \
+    do {                                                                                                             \
+        static size_t attr_lds = 0;                                                                                  \
+        if (lds > attr_lds) {                                                                                        \
+            OXQ_HIP_CHECK(hipFuncSetAttribute((const void *)moe_route_group_kernel<TY>,                              \
+                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));                \
+            attr_lds = lds;                                                                                          \
+        }                                                                                                            \
+        hipLaunchKernelGGL(moe_route_group_kernel<TY>, grid, block, lds, s, (const TY *)logits, (int)T, (int)E,      \
+                           (int)top_k, norm_topk, top_idx, top_vals, offsets, tokens, weights, pair_pos);            \
+    } while (0)
+    if (dtype == OXQ_F32) OXQ_RG(float);
+    else if (dtype == OXQ_F16) OXQ_RG(F16Tag);
+    else OXQ_RG(BF16Tag);
+#undef OXQ_RG
     OXQ_HIP_CHECK(hipGetLastError());
     return OXQ_OK;
 }

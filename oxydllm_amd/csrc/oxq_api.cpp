@@ -964,8 +964,8 @@ int oxq_mxfp4_moe_gate_up_swiglu(oxq_ctx *ctx, void *stream, const oxq_tensor *x
 // ---- mixture-of-experts glue (moe.rs:466-607, ffn_kernels.metal, moe.rs:152-173) --------
 
 
-int oxq_moe_route(oxq_ctx *ctx, void *stream, const oxq_tensor *logits, int64_t top_k, int norm_topk,
-                  const oxq_tensor *top_idx, const oxq_tensor *top_vals) {
+static int check_moe_route(oxq_ctx *ctx, const oxq_tensor *logits, int64_t top_k, const oxq_tensor *top_idx,
+                           const oxq_tensor *top_vals) {
     const char *op = "MoeRoute";
     if (!ctx) return fail(OXQ_ERR_ARG, "%s: ctx is NULL", op);
     OXQ_TRY(check_tensor(ctx, op, "logits", logits));
@@ -988,13 +988,19 @@ int oxq_moe_route(oxq_ctx *ctx, void *stream, const oxq_tensor *logits, int64_t 
         !top_vals->contiguous)
         return fail(OXQ_ERR_SHAPE, "%s: top_vals must be a contiguous F32 [%lld, %lld]", op, (long long)T,
                     (long long)top_k);
-    return launch_moe_route(ctx, (hipStream_t)stream, logits->data, logits->dtype, T, E, top_k, norm_topk ? 1 : 0,
-                            (int32_t *)top_idx->data, (float *)top_vals->data);
+    return OXQ_OK;
 }
 
-int oxq_moe_group(oxq_ctx *ctx, void *stream, const oxq_tensor *top_idx, const oxq_tensor *top_vals,
-                  int64_t n_experts, const oxq_tensor *expert_offsets, const oxq_tensor *token_ids,
-                  const oxq_tensor *pair_weights, const oxq_tensor *pair_pos) {
+int oxq_moe_route(oxq_ctx *ctx, void *stream, const oxq_tensor *logits, int64_t top_k, int norm_topk,
+                  const oxq_tensor *top_idx, const oxq_tensor *top_vals) {
+    OXQ_TRY(check_moe_route(ctx, logits, top_k, top_idx, top_vals));
+    return launch_moe_route(ctx, (hipStream_t)stream, logits->data, logits->dtype, logits->dims[0], logits->dims[1],
+                            top_k, norm_topk ? 1 : 0, (int32_t *)top_idx->data, (float *)top_vals->data);
+}
+
+static int check_moe_group(oxq_ctx *ctx, const oxq_tensor *top_idx, const oxq_tensor *top_vals, int64_t n_experts,
+                           const oxq_tensor *expert_offsets, const oxq_tensor *token_ids,
+                           const oxq_tensor *pair_weights, const oxq_tensor *pair_pos) {
     const char *op = "MoeGroup";
     if (!ctx) return fail(OXQ_ERR_ARG, "%s: ctx is NULL", op);
     OXQ_TRY(check_tensor(ctx, op, "top_idx", top_idx));
@@ -1023,8 +1029,34 @@ int oxq_moe_group(oxq_ctx *ctx, void *stream, const oxq_tensor *top_idx, const o
         return fail(OXQ_ERR_SHAPE, "%s: pair_pos must be a contiguous I32 [%lld, %lld]", op, (long long)T,
                     (long long)top_k);
     if (P > INT32_MAX) return fail(OXQ_ERR_SHAPE, "%s: too many pairs", op);
+    return OXQ_OK;
+}
+
+int oxq_moe_group(oxq_ctx *ctx, void *stream, const oxq_tensor *top_idx, const oxq_tensor *top_vals,
+                  int64_t n_experts, const oxq_tensor *expert_offsets, const oxq_tensor *token_ids,
+                  const oxq_tensor *pair_weights, const oxq_tensor *pair_pos) {
+    OXQ_TRY(check_moe_group(ctx, top_idx, top_vals, n_experts, expert_offsets, token_ids, pair_weights, pair_pos));
     return launch_moe_group(ctx, (hipStream_t)stream, (const int32_t *)top_idx->data, (const float *)top_vals->data,
-                            P, n_experts, top_k, (int32_t *)expert_offsets->data, (int32_t *)token_ids->data,
+                            numel(top_idx), n_experts, top_idx->dims[1], (int32_t *)expert_offsets->data,
+                            (int32_t *)token_ids->data, (float *)pair_weights->data, (int32_t *)pair_pos->data);
+}
+
+// moe.rs:466-486 followed by 563-590, as one call
+int oxq_moe_route_group(oxq_ctx *ctx, void *stream, const oxq_tensor *logits, int64_t top_k, int norm_topk,
+                        const oxq_tensor *top_idx, const oxq_tensor *top_vals, const oxq_tensor *expert_offsets,
+                        const oxq_tensor *token_ids, const oxq_tensor *pair_weights, const oxq_tensor *pair_pos) {
+    OXQ_TRY(check_moe_route(ctx, logits, top_k, top_idx, top_vals));
+    const int64_t T = logits->dims[0], E = logits->dims[1];
+    OXQ_TRY(check_moe_group(ctx, top_idx, top_vals, E, expert_offsets, token_ids, pair_weights, pair_pos));
+    if (T >= 1 && T * top_k <= 64)  // decode sizes: one launch
+        return launch_moe_route_group(ctx, (hipStream_t)stream, logits->data, logits->dtype, T, E, top_k,
+                                      norm_topk ? 1 : 0, (int32_t *)top_idx->data, (float *)top_vals->data,
+                                      (int32_t *)expert_offsets->data, (int32_t *)token_ids->data,
+                                      (float *)pair_weights->data, (int32_t *)pair_pos->data);
+    OXQ_TRY(launch_moe_route(ctx, (hipStream_t)stream, logits->data, logits->dtype, T, E, top_k, norm_topk ? 1 : 0,
+                             (int32_t *)top_idx->data, (float *)top_vals->data));
+    return launch_moe_group(ctx, (hipStream_t)stream, (const int32_t *)top_idx->data, (const float *)top_vals->data,
+                            T * top_k, E, top_k, (int32_t *)expert_offsets->data, (int32_t *)token_ids->data,
                             (float *)pair_weights->data, (int32_t *)pair_pos->data);
 }
 

@@ -181,6 +181,9 @@ int launch_mxfp4_dequant(oxq_ctx *ctx, hipStream_t s, const Mxfp4Problem &p, flo
 // mixture-of-experts glue (moe_glue.hip)
 int launch_moe_route(oxq_ctx *ctx, hipStream_t s, const void *logits, int dtype, int64_t T, int64_t E, int64_t top_k,
                      int norm_topk, int32_t *top_idx, float *top_vals);
+int launch_moe_route_group(oxq_ctx *ctx, hipStream_t s, const void *logits, int dtype, int64_t T, int64_t E,
+                           int64_t top_k, int norm_topk, int32_t *top_idx, float *top_vals, int32_t *offsets,
+                           int32_t *tokens, float *weights, int32_t *pair_pos);
 int launch_moe_group(oxq_ctx *ctx, hipStream_t s, const int32_t *top_idx, const float *top_vals, int64_t P, int64_t E,
                      int64_t top_k, int32_t *offsets, int32_t *tokens, float *weights, int32_t *pair_pos);
 int launch_activation_mul(oxq_ctx *ctx, hipStream_t s, const void *gate, const void *up, void *out, int dtype,

@@ -403,6 +403,24 @@ def moe_group(top_idx, top_vals, n_experts: int, *, ctx: Optional[Context] = Non
     return offsets, tokens, weights, pos
 
 
+def moe_route_group(logits, top_k: int, norm_topk: bool = True, *, ctx: Optional[Context] = None):
+    """moe_route + moe_group in one call (one launch for decode sizes): returns (top_idx, top_vals,
+    expert_offsets, token_ids, pair_weights, pair_pos)."""
+    ctx = _ctx(ctx)
+    T, E = logits.shape
+    dev = logits.device
+    idx = torch.empty((T, top_k), dtype=torch.int32, device=dev)
+    vals = torch.empty((T, top_k), dtype=torch.float32, device=dev)
+    offsets = torch.empty((E + 1,), dtype=torch.int32, device=dev)
+    tokens = torch.empty((T * top_k,), dtype=torch.int32, device=dev)
+    weights = torch.empty((T * top_k,), dtype=torch.float32, device=dev)
+    pos = torch.empty((T, top_k), dtype=torch.int32, device=dev)
+    _lib.check(ctx._lib.oxq_moe_route_group(ctx.handle, ctx.stream(), desc(logits), top_k, 1 if norm_topk else 0,
+                                            desc(idx), desc(vals), desc(offsets), desc(tokens), desc(weights),
+                                            desc(pos)))
+    return idx, vals, offsets, tokens, weights, pos
+
+
 def gated_activation(gate_up, kind: int, limit: float = 0.0, *, out=None, ctx: Optional[Context] = None):
     """ffn_kernels.metal gated SiLU / GeLU-tanh over [.., gate | up]; moe.rs:152-173 GPT-OSS SwiGLU."""
     ctx = _ctx(ctx)

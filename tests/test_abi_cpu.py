@@ -571,6 +571,7 @@ def test_random_descriptors_never_crash_and_always_explain(lib, ctx):
         call("oxq_mxfp4_moe_gate_up_swiglu", ctx, None, B(ts[0]), B(ts[1]), B(ts[2]), B(ts[3]), B(ts[4]), B(ts[5]), int(rng.integers(0, 2)), i64(), i64(), C.c_float(7.0), B(ts[6]), B(taken))
         call("oxq_moe_route", ctx, None, B(ts[0]), i64(), 1, B(ts[1]), B(ts[2]))
         call("oxq_moe_group", ctx, None, B(ts[0]), B(ts[1]), i64(), B(ts[2]), B(ts[3]), B(ts[4]), B(ts[5]))
+        call("oxq_moe_route_group", ctx, None, B(ts[0]), i64(), 1, B(ts[1]), B(ts[2]), B(ts[3]), B(ts[4]), B(ts[5]), B(ts[6]))
         call("oxq_gated_activation", ctx, None, B(ts[0]), int(rng.integers(-1, 4)), C.c_float(7.0), B(ts[1]))
         call("oxq_activation_mul", ctx, None, B(ts[0]), B(ts[1]), int(rng.integers(-1, 4)), B(ts[2]))
         call("oxq_moe_combine", ctx, None, B(ts[0]), B(ts[1]), B(ts[2]), B(ts[3]))

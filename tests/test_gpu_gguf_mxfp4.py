@@ -429,6 +429,26 @@ def test_moe_group_matches_oracle(T, E, k):
     np.testing.assert_array_equal(rw[pos.ravel()], rvals.ravel())
 
 
+@pytest.mark.parametrize("T,E,k,norm", [(8, 32, 4, True), (1, 32, 4, True), (16, 64, 4, False), (5, 200, 3, True),
+                                         (64, 16, 1, True), (13, 256, 5, True), (17, 32, 4, True), (300, 8, 2, False)])
+def test_moe_route_group_equals_the_two_calls(T, E, k, norm):
+    """moe.rs:466-486 + 563-590 in one call: identical outputs to route followed by group, as one launch up to
+    64 pairs and as the two launches beyond."""
+    say(f"moe_route_group T={T} E={E} k={k}")
+    logits = torch.from_numpy(np.random.default_rng(T * E + k).standard_normal((T, E)).astype(np.float32)).cuda()
+    for dt in (torch.float32, torch.bfloat16):
+        lg = logits.to(dt)
+        idx, vals = ops.moe_route(lg, k, norm)
+        want = (idx, vals) + tuple(ops.moe_group(idx, vals, E))
+        got = ops.moe_route_group(lg, k, norm)
+        assert ops.default_context().last_plan()["kernel"] == ("moe_route_group" if T * k <= 64 else "moe_group")
+        for a, b, name in zip(got, want, ("top_idx", "top_vals", "expert_offsets", "token_ids", "pair_weights", "pair_pos")):
+            assert a.dtype == b.dtype and a.shape == b.shape, name
+            assert torch.equal(a.view(torch.int32), b.view(torch.int32)), name
+    with pytest.raises(ops.OxqError, match="top_k"):
+        ops.moe_route_group(logits, E + 1)
+
+
 @pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16, torch.float16])
 def test_gated_activations_match_oracle(dt):
     """ffn_kernels.metal:19-242 and moe.rs:152-173: f32 math, one rounding to the tensor dtype."""
