@@ -46,21 +46,40 @@ template <> __device__ __forceinline__ void store_f32<BF16Tag>(BF16Tag *p, size_
 // ---------------------------------------------------------------------------
 // route: one wave per token, probabilities in LDS
 // ---------------------------------------------------------------------------
+// Whole-wave reductions that leave the result in every lane, on the DPP lane permutes (pairs, quads,
+// halves of 8 and rows of 16) and four lane reads for the rows: about twenty instructions, where the
+// same butterfly through ds_bpermute is six trips through the LDS crossbar.  All 64 lanes must be active.
+template <typename V, typename F>
+__device__ __forceinline__ V wave_all_reduce(V v, F op) {
+    static_assert(sizeof(V) == 4, "32-bit values");
+    auto dpp = [](V x, auto ctrl) {
+        return __builtin_bit_cast(V, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), decltype(ctrl)::value,
+                                                                0xF, 0xF, false));
+    };
+    v = op(v, dpp(v, std::integral_constant<int, 0xB1>{}));   // quad_perm [1,0,3,2]: lane ^ 1
+    v = op(v, dpp(v, std::integral_constant<int, 0x4E>{}));   // quad_perm [2,3,0,1]: lane ^ 2
+    v = op(v, dpp(v, std::integral_constant<int, 0x141>{}));  // row_half_mirror: the other quad of 8
+    v = op(v, dpp(v, std::integral_constant<int, 0x140>{}));  // row_mirror: the other half of 16
+    const int b = __builtin_bit_cast(int, v);
+    const V r0 = __builtin_bit_cast(V, __builtin_amdgcn_readlane(b, 0)), r1 = __builtin_bit_cast(V, __builtin_amdgcn_readlane(b, 16));
+    const V r2 = __builtin_bit_cast(V, __builtin_amdgcn_readlane(b, 32)), r3 = __builtin_bit_cast(V, __builtin_amdgcn_readlane(b, 48));
+    return op(op(r0, r1), op(r2, r3));
+}
+
 // one token, one wave: lane s < top_k ends with slot s in (my_idx, my_val); probs = E floats of LDS
 template <typename T>
 __device__ __forceinline__ void route_token(const T *__restrict__ l, int E, int top_k, int norm_topk, float *probs,
                                             int lane, int &out_idx, float &out_val) {
     float mx = -INFINITY;
     for (int e = lane; e < E; e += 64) mx = fmaxf(mx, load_f32(l, e));
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+    mx = wave_all_reduce(mx, [](float a, float b) { return fmaxf(a, b); });
     float sum = 0.0f;
     for (int e = lane; e < E; e += 64) {
         const float p = expf(load_f32(l, e) - mx);
         probs[e] = p;
         sum += p;
     }
-    sum = wave_sum_xor<64>(sum);
+    sum = wave_all_reduce(sum, [](float a, float b) { return a + b; });
     for (int e = lane; e < E; e += 64) probs[e] = probs[e] / sum;
     // the wave's own LDS writes are visible to its own later reads (same wave, in order)
     float chosen_sum = 0.0f, my_val = 0.0f;
@@ -75,15 +94,10 @@ __device__ __forceinline__ void route_token(const T *__restrict__ l, int E, int 
                 bi = e;
             }
         }
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) {  // butterfly: every lane ends with the winner
-            const float ov = __shfl_xor(bv, off, 64);
-            const int oi = __shfl_xor(bi, off, 64);
-            if (ov > bv || (ov == bv && oi < bi)) {
-                bv = ov;
-                bi = oi;
-            }
-        }
+        // the largest value, then the lowest index among the lanes that hold it
+        const float best = wave_all_reduce(bv, [](float a, float b) { return fmaxf(a, b); });
+        bi = wave_all_reduce(bv == best ? bi : 0x7fffffff, [](int a, int b) { return a < b ? a : b; });
+        bv = best;
         if (lane == s) {  // slot s is kept by lane s
             my_val = bv;
             my_idx = bi;
@@ -132,7 +146,7 @@ __device__ __forceinline__ void group_pairs_small(const int32_t *top_idx, const 
     unsigned long long todo = __ballot(ok);
     while (todo) {  // wave-uniform
         const int first = __builtin_ctzll(todo);
-        const int e0 = __shfl(e, first, 64);
+        const int e0 = __builtin_amdgcn_readlane(e, first);
         const unsigned long long m = __ballot(ok && e == e0);
         if (ok && e == e0) rank = __builtin_popcountll(m & ((1ull << lane) - 1ull));
         if (lane == first) count[e0] = __builtin_popcountll(m);
