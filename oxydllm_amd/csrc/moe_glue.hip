@@ -46,26 +46,6 @@ template <> __device__ __forceinline__ void store_f32<BF16Tag>(BF16Tag *p, size_
 // ---------------------------------------------------------------------------
 // route: one wave per token, probabilities in LDS
 // ---------------------------------------------------------------------------
-// Whole-wave reductions that leave the result in every lane, on the DPP lane permutes (pairs, quads,
-// halves of 8 and rows of 16) and four lane reads for the rows: about twenty instructions, where the
-// same butterfly through ds_bpermute is six trips through the LDS crossbar.  All 64 lanes must be active.
-template <typename V, typename F>
-__device__ __forceinline__ V wave_all_reduce(V v, F op) {
-    static_assert(sizeof(V) == 4, "32-bit values");
-    auto dpp = [](V x, auto ctrl) {
-        return __builtin_bit_cast(V, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), decltype(ctrl)::value,
-                                                                0xF, 0xF, false));
-    };
-    v = op(v, dpp(v, std::integral_constant<int, 0xB1>{}));   // quad_perm [1,0,3,2]: lane ^ 1
-    v = op(v, dpp(v, std::integral_constant<int, 0x4E>{}));   // quad_perm [2,3,0,1]: lane ^ 2
-    v = op(v, dpp(v, std::integral_constant<int, 0x141>{}));  // row_half_mirror: the other quad of 8
-    v = op(v, dpp(v, std::integral_constant<int, 0x140>{}));  // row_mirror: the other half of 16
-    const int b = __builtin_bit_cast(int, v);
-    const V r0 = __builtin_bit_cast(V, __builtin_amdgcn_readlane(b, 0)), r1 = __builtin_bit_cast(V, __builtin_amdgcn_readlane(b, 16));
-    const V r2 = __builtin_bit_cast(V, __builtin_amdgcn_readlane(b, 32)), r3 = __builtin_bit_cast(V, __builtin_amdgcn_readlane(b, 48));
-    return op(op(r0, r1), op(r2, r3));
-}
-
 // one token, one wave: lane s < top_k ends with slot s in (my_idx, my_val); probs = E floats of LDS
 template <typename T>
 __device__ __forceinline__ void route_token(const T *__restrict__ l, int E, int top_k, int norm_topk, float *probs,

@@ -6,6 +6,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
+#include <type_traits>
 
 namespace oxq {
 
@@ -170,11 +171,35 @@ __device__ __forceinline__ float e8m0_to_f32(uint32_t s) {
 // ---------------------------------------------------------------------------
 // Reductions
 // ---------------------------------------------------------------------------
+// Whole-wave reductions that leave the result in every lane, on the DPP lane permutes (pairs, quads,
+// halves of 8 and rows of 16) and four lane reads for the rows: about twenty instructions, where the
+// same butterfly through ds_bpermute is six trips through the LDS crossbar.  All 64 lanes must be active.
+template <typename V, typename F>
+__device__ __forceinline__ V wave_all_reduce(V v, F op) {
+    static_assert(sizeof(V) == 4, "32-bit values");
+    auto dpp = [](V x, auto ctrl) {
+        return __builtin_bit_cast(V, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), decltype(ctrl)::value,
+                                                                0xF, 0xF, false));
+    };
+    v = op(v, dpp(v, std::integral_constant<int, 0xB1>{}));   // quad_perm [1,0,3,2]: lane ^ 1
+    v = op(v, dpp(v, std::integral_constant<int, 0x4E>{}));   // quad_perm [2,3,0,1]: lane ^ 2
+    v = op(v, dpp(v, std::integral_constant<int, 0x141>{}));  // row_half_mirror: the other quad of 8
+    v = op(v, dpp(v, std::integral_constant<int, 0x140>{}));  // row_mirror: the other half of 16
+    const int b = __builtin_bit_cast(int, v);
+    const V r0 = __builtin_bit_cast(V, __builtin_amdgcn_readlane(b, 0)), r1 = __builtin_bit_cast(V, __builtin_amdgcn_readlane(b, 16));
+    const V r2 = __builtin_bit_cast(V, __builtin_amdgcn_readlane(b, 32)), r3 = __builtin_bit_cast(V, __builtin_amdgcn_readlane(b, 48));
+    return op(op(r0, r1), op(r2, r3));
+}
+
 template <int WIDTH>
 __device__ __forceinline__ float wave_sum_xor(float v) {  // butterfly over WIDTH lanes
+    if constexpr (WIDTH == 64) {
+        return wave_all_reduce(v, [](float a, float b) { return a + b; });
+    } else {
 #pragma unroll
-    for (int off = WIDTH / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, WAVE);
-    return v;
+        for (int off = WIDTH / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, WAVE);
+        return v;
+    }
 }
 
 // ---------------------------------------------------------------------------
