@@ -107,31 +107,34 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T *__restrict__ lo
     }
 }
 
+// The lanes of the wave that hold the same expert id as this lane (itself included), for lanes with
+// `ok`: one ballot per bit of the id, no loop over experts.
+__device__ __forceinline__ unsigned long long lanes_with_my_expert(int e, bool ok, int id_bits) {
+    unsigned long long m = __ballot(ok);
+    for (int j = 0; j < id_bits; ++j) {  // wave-uniform trip count
+        const bool bit = (e >> j) & 1;
+        const unsigned long long b = __ballot(ok && bit);
+        m &= bit ? b : ~b;
+    }
+    return m;
+}
+__device__ __forceinline__ int expert_id_bits(int E) { return E > 1 ? 32 - __builtin_clz(E - 1) : 0; }
+
 // Decode sizes (P <= 64), one wave: the pairs of (top_idx, top_vals) grouped by expert.  `scratch` = 2 E ints of LDS.
 __device__ __forceinline__ void group_pairs_small(const int32_t *top_idx, const float *top_vals, int P, int E, int top_k,
                                                   int32_t *scratch, int lane, int32_t *__restrict__ offsets,
                                                   int32_t *__restrict__ tokens, float *__restrict__ weights,
                                                   int32_t *__restrict__ pair_pos) {
-    // Decode sizes: one pair per lane, no counting matrix.  The wave peels off one expert at a
-    // time: the first unplaced lane's expert, a ballot of the lanes that share it, rank = the
-    // matching lanes below me (pair order = token order inside an expert), count = the ballot's
-    // population.  At most min(P, E) rounds of scalar work instead of chains of dependent LDS
-    // accesses (E + 64 + E of them in the general path).
+    // Decode sizes: one pair per lane, no counting matrix.  rank = the lanes below me with my expert
+    // (pair order = token order inside an expert), count = all of them; the lowest such lane records it.
     int32_t *count = scratch;  // [E], then start[E]
     int32_t *start = scratch + E;
     for (int e = lane; e < E; e += 64) count[e] = 0;
     const int e = lane < P ? top_idx[lane] : -1;
     const bool ok = e >= 0 && e < E;  // ids outside [0, E) are dropped
-    int rank = 0;
-    unsigned long long todo = __ballot(ok);
-    while (todo) {  // wave-uniform
-        const int first = __builtin_ctzll(todo);
-        const int e0 = __builtin_amdgcn_readlane(e, first);
-        const unsigned long long m = __ballot(ok && e == e0);
-        if (ok && e == e0) rank = __builtin_popcountll(m & ((1ull << lane) - 1ull));
-        if (lane == first) count[e0] = __builtin_popcountll(m);
-        todo &= ~m;
-    }
+    const unsigned long long mine = lanes_with_my_expert(e, ok, expert_id_bits(E));
+    const int rank = __builtin_popcountll(mine & ((1ull << lane) - 1ull));
+    if (ok && rank == 0) count[e] = __builtin_popcountll(mine);
     // exclusive scan of the counts in expert order, 64 experts per round
     int carry = 0;
     for (int e1 = 0; e1 < E; e1 += 64) {
@@ -159,56 +162,87 @@ __device__ __forceinline__ void group_pairs_small(const int32_t *top_idx, const 
 }
 
 // ---------------------------------------------------------------------------
-// group: one wave; thread i owns the contiguous pair range [i*L, (i+1)*L)
+// group.  Up to 64 pairs: one wave, one pair per lane (group_pairs_small).  Above: 16 waves, wave w
+// owns the pairs [w C, (w + 1) C) and takes them 64 at a time, ranking the lanes that share an expert
+// with ballots exactly as the small form does; its running count per expert lives in its own row of LDS,
+// and the rank inside (wave, expert) is parked in pair_pos.  A scan over (expert, wave) then gives every
+// wave its first position per expert, and a second pass over the pairs writes the lists.  Pair order
+// inside an expert is pair order, whatever the scheduling: every sum here is over integers.
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(64) void moe_group_kernel(const int32_t *__restrict__ top_idx,
                                                        const float *__restrict__ top_vals, int P, int E,
                                                        int32_t *__restrict__ offsets, int32_t *__restrict__ tokens,
                                                        float *__restrict__ weights, int32_t *__restrict__ pair_pos,
                                                        int top_k) {
-    extern __shared__ int32_t group_lds[];  // cnt[E][64], then base[E]
-    int32_t *cnt = group_lds;
-    int32_t *base = group_lds + (size_t)E * 64;
-    const int lane = threadIdx.x;
-    if (P <= 64) {
-        group_pairs_small(top_idx, top_vals, P, E, top_k, group_lds, lane, offsets, tokens, weights, pair_pos);
-        return;
-    }
-    const int L = (P + 63) / 64;
-    const int i0 = min(P, lane * L), i1 = min(P, i0 + L);
-    for (int e = 0; e < E; ++e) cnt[e * 64 + lane] = 0;
-    for (int i = i0; i < i1; ++i) {
-        const int e = top_idx[i];
-        if (e >= 0 && e < E) cnt[e * 64 + lane] += 1;  // ids outside [0, E) are dropped
+    extern __shared__ int32_t group_lds[];  // count[E], start[E]
+    group_pairs_small(top_idx, top_vals, P, E, top_k, group_lds, (int)threadIdx.x, offsets, tokens, weights, pair_pos);
+}
+
+constexpr int GROUP_WAVES = 16;
+__global__ __launch_bounds__(GROUP_WAVES * 64) void moe_group_waves_kernel(
+    const int32_t *__restrict__ top_idx, const float *__restrict__ top_vals, int P, int E,
+    int32_t *__restrict__ offsets, int32_t *__restrict__ tokens, float *__restrict__ weights,
+    int32_t *__restrict__ pair_pos, int top_k) {
+    extern __shared__ int32_t group_lds[];  // cnt[GROUP_WAVES][E], then start[E]
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int32_t *cnt = group_lds + (size_t)wave * E;
+    int32_t *start = group_lds + (size_t)GROUP_WAVES * E;
+    for (int e = lane; e < E; e += 64) cnt[e] = 0;  // the wave's own row: its LDS accesses stay in order
+    const int C = ((P + GROUP_WAVES * 64 - 1) / (GROUP_WAVES * 64)) * 64;  // pairs per wave, whole batches of 64
+    const int i0 = min(P, wave * C), i1 = min(P, i0 + C);
+    const unsigned long long below = (1ull << lane) - 1ull;
+    const int id_bits = expert_id_bits(E);
+    for (int b = i0; b < i1; b += 64) {
+        const int i = b + lane;
+        const int e = i < i1 ? top_idx[i] : -1;
+        const bool ok = e >= 0 && e < E;  // ids outside [0, E) are dropped
+        const unsigned long long mine = lanes_with_my_expert(e, ok, id_bits);
+        const int r = __builtin_popcountll(mine & below);
+        const int before = ok ? cnt[e] : 0;  // every lane reads before the lowest lane of each expert adds
+        if (ok && r == 0) cnt[e] = before + __builtin_popcountll(mine);
+        const int rank = before + r;
+        if (ok) pair_pos[i] = rank;  // within (wave, expert); made absolute below
     }
     __syncthreads();
-    // per expert: exclusive prefix over the 64 owners, total in base[e]
-    for (int e = lane; e < E; e += 64) {
-        int run = 0;
-        for (int j = 0; j < 64; ++j) {
-            const int c = cnt[e * 64 + j];
-            cnt[e * 64 + j] = run;
-            run += c;
+    // per expert: exclusive prefix over the waves, total in start[e]
+    for (int e = threadIdx.x; e < E; e += GROUP_WAVES * 64) {
+        int c[GROUP_WAVES], run = 0;
+#pragma unroll
+        for (int w = 0; w < GROUP_WAVES; ++w) c[w] = group_lds[(size_t)w * E + e];  // independent reads first
+#pragma unroll
+        for (int w = 0; w < GROUP_WAVES; ++w) {
+            group_lds[(size_t)w * E + e] = run;
+            run += c[w];
         }
-        base[e] = run;
+        start[e] = run;
     }
     __syncthreads();
-    if (lane == 0) {
-        int run = 0;
-        for (int e = 0; e < E; ++e) {
-            const int c = base[e];
-            offsets[e] = run;
-            base[e] = run;
-            run += c;
+    if (wave == 0) {  // exclusive scan of the totals in expert order, 64 experts per round
+        int carry = 0;
+        for (int e1 = 0; e1 < E; e1 += 64) {
+            const int ee = e1 + lane;
+            const int c = ee < E ? start[ee] : 0;
+            int incl = c;
+#pragma unroll
+            for (int off = 1; off < 64; off <<= 1) {
+                const int t = __shfl_up(incl, off, 64);
+                if (lane >= off) incl += t;
+            }
+            if (ee < E) {
+                start[ee] = carry + incl - c;
+                offsets[ee] = carry + incl - c;
+            }
+            carry += __shfl(incl, 63, 64);
         }
-        offsets[E] = run;
+        if (lane == 0) offsets[E] = carry;
     }
     __syncthreads();
-    for (int i = i0; i < i1; ++i) {
+    for (int b = i0; b < i1; b += 64) {
+        const int i = b + lane;
+        if (i >= i1) continue;
         const int e = top_idx[i];
         if (e < 0 || e >= E) continue;
-        const int pos = base[e] + cnt[e * 64 + lane];
-        cnt[e * 64 + lane] += 1;
+        const int pos = start[e] + cnt[e] + pair_pos[i];
         tokens[pos] = i / top_k;
         weights[pos] = top_vals[i];
         pair_pos[i] = pos;
@@ -323,18 +357,18 @@ int launch_moe_route(oxq_ctx *ctx, hipStream_t s, const void *logits, int dtype,
 
 int launch_moe_group(oxq_ctx *ctx, hipStream_t s, const int32_t *top_idx, const float *top_vals, int64_t P, int64_t E,
                      int64_t top_k, int32_t *offsets, int32_t *tokens, float *weights, int32_t *pair_pos) {
-    dim3 grid(1), block(64);
+    const bool small = P <= 64;
+    dim3 grid(1), block(small ? 64 : GROUP_WAVES * 64);
     set_plan(ctx, "moe_group", grid, block, 1, 1, 0);
     if (ctx->plan_only) return OXQ_OK;
-    const size_t lds = ((size_t)E * 64 + (size_t)E) * sizeof(int32_t);
-    static size_t attr_lds = 0;
-    if (lds > attr_lds) {
-        OXQ_HIP_CHECK(hipFuncSetAttribute((const void *)moe_group_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                          (int)lds));
-        attr_lds = lds;
+    if (small) {
+        hipLaunchKernelGGL(moe_group_kernel, grid, block, 2 * (size_t)E * sizeof(int32_t), s, top_idx, top_vals, (int)P,
+                           (int)E, offsets, tokens, weights, pair_pos, (int)top_k);
+    } else {
+        const size_t lds = ((size_t)GROUP_WAVES + 1) * (size_t)E * sizeof(int32_t);  // at most 17 KB (256 experts)
+        hipLaunchKernelGGL(moe_group_waves_kernel, grid, block, lds, s, top_idx, top_vals, (int)P, (int)E, offsets,
+                           tokens, weights, pair_pos, (int)top_k);
     }
-    hipLaunchKernelGGL(moe_group_kernel, grid, block, lds, s, top_idx, top_vals, (int)P, (int)E, offsets, tokens,
-                       weights, pair_pos, (int)top_k);
     OXQ_HIP_CHECK(hipGetLastError());
     return OXQ_OK;
 }
