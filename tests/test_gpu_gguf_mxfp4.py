@@ -450,20 +450,33 @@ def test_moe_route_group_equals_the_two_calls(T, E, k, norm):
 
 
 @pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16, torch.float16])
-def test_gated_activations_match_oracle(dt):
+def test_gated_activations_match_oracle(dt, monkeypatch):
+    monkeypatch.setenv("OXQ_ACT_VEC", "1")      # the 8-outputs-a-thread kernel at test sizes too
     """ffn_kernels.metal:19-242 and moe.rs:152-173: f32 math, one rounding to the tensor dtype."""
     say(f"gated activations {dt}")
     rng = np.random.default_rng(3)
-    gu = (rng.standard_normal((7, 2 * 96)) * 3).astype(np.float32)
-    gd = to_dev(gu, dt)
-    gr = gd.float().cpu().numpy()
     odt = {torch.float32: None, torch.bfloat16: oracle.BF16, torch.float16: oracle.F16}[dt]
-    for kind, ref in [(ops.ACT_GATED_SILU, oracle.gated_silu(gr)), (ops.ACT_GATED_GELU_TANH, oracle.gated_gelu_tanh(gr)),
-                      (ops.ACT_GPT_OSS_SWIGLU, oracle.gpt_oss_swiglu(gr, 7.0))]:
-        y = ops.gated_activation(gd, kind, 7.0)
-        assert y.shape == (7, 96) and y.dtype == dt
-        assert_close(y, ref, f"gated act {kind} {dt}", rtol=1e-5 if odt is None else RTOL, atol=1e-5 if odt is None else ATOL,
-                     bf16_out=dt == torch.bfloat16)
+    for rows, half in [(7, 96), (5, 37), (3, 8), (2, 20)]:   # whole 16-byte pieces per half (8 outputs a thread) and not
+        gu = (rng.standard_normal((rows, 2 * half)) * 3).astype(np.float32)
+        gd = to_dev(gu, dt)
+        gr = gd.float().cpu().numpy()
+        for kind, ref in [(ops.ACT_GATED_SILU, oracle.gated_silu(gr)), (ops.ACT_GATED_GELU_TANH, oracle.gated_gelu_tanh(gr)),
+                          (ops.ACT_GPT_OSS_SWIGLU, oracle.gpt_oss_swiglu(gr, 7.0))]:
+            y = ops.gated_activation(gd, kind, 7.0)
+            assert y.shape == (rows, half) and y.dtype == dt
+            assert_close(y, ref, f"gated act {kind} {dt} {rows}x{half}", rtol=1e-5 if odt is None else RTOL,
+                         atol=1e-5 if odt is None else ATOL, bf16_out=dt == torch.bfloat16)
+            if half % 8 == 0 and dt != torch.float32:
+                # the same rows inside a wider, odd-width tensor take the one-output-a-thread kernel: same bits
+                wide = torch.zeros((rows, 2 * (half + 1)), dtype=dt, device="cuda")
+                if kind == ops.ACT_GPT_OSS_SWIGLU:
+                    wide[:, :2 * half] = gd
+                else:
+                    wide[:, :half] = gd[:, :half]
+                    wide[:, half + 1:2 * half + 1] = gd[:, half:]
+                y1 = ops.gated_activation(wide, kind, 7.0)[:, :half]
+                assert torch.equal(y.view(torch.int16), y1.contiguous().view(torch.int16))
+    gu = (rng.standard_normal((7, 2 * 96)) * 3).astype(np.float32)
     with pytest.raises(ops.OxqError, match="2 \\* intermediate_size"):
         ops.gated_activation(to_dev(gu[:, :191].copy(), dt), ops.ACT_GATED_SILU)
 
