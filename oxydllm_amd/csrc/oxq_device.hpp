@@ -191,6 +191,22 @@ __device__ __forceinline__ V wave_all_reduce(V v, F op) {
     return op(op(r0, r1), op(r2, r3));
 }
 
+// v[l] + v[l ^ 16] and v[l] + v[l ^ 32] in every lane: v_permlane16_swap / v_permlane32_swap exchange
+// the odd rows (upper half) of one register with the even rows (lower half) of the other, so with the
+// value in both, the two results hold the two partners of every lane.  Vector ALU, no LDS crossbar.
+__device__ __forceinline__ float add_lane_xor16(float v) {
+    const uint32_t b = __builtin_bit_cast(uint32_t, v);
+    const auto r = __builtin_amdgcn_permlane16_swap(b, b, false, false);
+    const uint32_t r0 = r[0], r1 = r[1];
+    return __builtin_bit_cast(float, r0) + __builtin_bit_cast(float, r1);
+}
+__device__ __forceinline__ float add_lane_xor32(float v) {
+    const uint32_t b = __builtin_bit_cast(uint32_t, v);
+    const auto r = __builtin_amdgcn_permlane32_swap(b, b, false, false);
+    const uint32_t r0 = r[0], r1 = r[1];
+    return __builtin_bit_cast(float, r0) + __builtin_bit_cast(float, r1);
+}
+
 template <int WIDTH>
 __device__ __forceinline__ float wave_sum_xor(float v) {  // butterfly over WIDTH lanes
     if constexpr (WIDTH == 64) {

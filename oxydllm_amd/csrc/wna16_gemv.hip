@@ -482,8 +482,13 @@ __global__ __launch_bounds__(WPG * GPB * 64) void awq_gemv_fast(
 #pragma unroll
             for (int c = 0; c < NC; ++c) {
                 float v = yacc[m][c];
+                if constexpr (LPR == 16) {  // lanes l, l ^ 16, l ^ 32, l ^ 48 on the gfx950 lane-swap instructions
+                    v = add_lane_xor16(v);
+                    v = add_lane_xor32(v);
+                } else {
 #pragma unroll
-                for (int off = LPR; off < 64; off <<= 1) v += __shfl_xor(v, off, WAVE);
+                    for (int off = LPR; off < 64; off <<= 1) v += __shfl_xor(v, off, WAVE);
+                }
                 yacc[m][c] = v;
             }
             if (sub == 0) {
