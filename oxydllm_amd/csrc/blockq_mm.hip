@@ -372,12 +372,8 @@ struct MmPlan {
 
 template <class SRC, int MT, bool HILO = false>
 static int launch_mm_go(hipStream_t s, const MmArgs &a, dim3 grid, size_t lds) {
-    static bool attr_set = false;
-    if (!attr_set) {
-        OXQ_HIP_CHECK(hipFuncSetAttribute((const void *)blockq_mm_kernel<SRC, MT, HILO>,
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        attr_set = true;
-    }
+    static LdsGrant lds_grant;  // one per instantiation
+    OXQ_HIP_CHECK(lds_grant.ensure((const void *)blockq_mm_kernel<SRC, MT, HILO>, lds));
     hipLaunchKernelGGL((blockq_mm_kernel<SRC, MT, HILO>), grid, dim3(256), lds, s, a);
     OXQ_HIP_CHECK(hipGetLastError());
     return OXQ_OK;

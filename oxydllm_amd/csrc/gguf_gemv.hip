@@ -486,12 +486,8 @@ static void launch_rows(hipStream_t s, dim3 grid, const GgufProblem &p, const ui
 template <int FMT, bool BF16X, int MB, bool PW = false>
 static int launch_rows_lds_mb(hipStream_t s, const GgufProblem &p, const uint8_t *x, uint8_t *y, int rows,
                               int rpwg, size_t lds) {
-    static size_t attr_lds = 0;
-    if (lds > attr_lds) {
-        OXQ_HIP_CHECK(hipFuncSetAttribute((const void *)gguf_gemv_lds_kernel<FMT, BF16X, MB, PW>,
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        attr_lds = lds;
-    }
+    static LdsGrant lds_grant;  // one per instantiation
+    OXQ_HIP_CHECK(lds_grant.ensure((const void *)gguf_gemv_lds_kernel<FMT, BF16X, MB, PW>, lds));
     const int K = (int)p.K, N = (int)p.N;
     const size_t total = (size_t)N * (size_t)(K / GgufFmt<FMT>::BE) * GgufFmt<FMT>::BB;
     // one wave per row at a time: 8 waves for 8 rows (x is staged once per 8 rows), else 4

@@ -426,12 +426,8 @@ int launch_moe_route_group(oxq_ctx *ctx, hipStream_t s, const void *logits, int 
     const size_t lds = ((size_t)nw * E + 128 + 2 * (size_t)E) * sizeof(float);
 #define OXQ_RG(TY)                                                                                                   \
     do {                                                                                                             \
-        static size_t attr_lds = 0;                                                                                  \
-        if (lds > attr_lds) {                                                                                        \
-            OXQ_HIP_CHECK(hipFuncSetAttribute((const void *)moe_route_group_kernel<TY>,                              \
-                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));                \
-            attr_lds = lds;                                                                                          \
-        }                                                                                                            \
+        static LdsGrant lds_grant;                                                                                   \
+        OXQ_HIP_CHECK(lds_grant.ensure((const void *)moe_route_group_kernel<TY>, lds));                              \
         hipLaunchKernelGGL(moe_route_group_kernel<TY>, grid, block, lds, s, (const TY *)logits, (int)T, (int)E,      \
                            (int)top_k, norm_topk, top_idx, top_vals, offsets, tokens, weights, pair_pos);            \
     } while (0)

@@ -455,12 +455,8 @@ __global__ __launch_bounds__(256) void mxfp4_dequant_kernel(const uint8_t *__res
 
 template <int MB, int RW>
 static int mxfp4_lds_go(hipStream_t s, dim3 grid, const Mxfp4Problem &p, size_t lds) {
-    static size_t attr_lds = 0;
-    if (lds > attr_lds) {
-        OXQ_HIP_CHECK(hipFuncSetAttribute((const void *)mxfp4_gemv_lds_kernel<MB, RW>,
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        attr_lds = lds;
-    }
+    static LdsGrant lds_grant;  // one per instantiation
+    OXQ_HIP_CHECK(lds_grant.ensure((const void *)mxfp4_gemv_lds_kernel<MB, RW>, lds));
     hipLaunchKernelGGL((mxfp4_gemv_lds_kernel<MB, RW>), grid, dim3(256), lds, s, (const uint16_t *)p.x, p.blocks,
                        p.scales, (const uint16_t *)p.bias, (uint16_t *)p.y, p.expert_offsets, p.token_ids,
                        (int)p.M, (int)p.K, (int)p.N);
@@ -470,12 +466,8 @@ static int mxfp4_lds_go(hipStream_t s, dim3 grid, const Mxfp4Problem &p, size_t 
 
 template <int MTOK, int FR>
 static int mxfp4_mfma_go(hipStream_t s, dim3 grid, const Mxfp4Problem &p, size_t lds) {
-    static size_t attr_lds = 0;
-    if (lds > attr_lds) {
-        OXQ_HIP_CHECK(hipFuncSetAttribute((const void *)mxfp4_mfma_kernel<MTOK, FR>,
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        attr_lds = lds;
-    }
+    static LdsGrant lds_grant;  // one per instantiation
+    OXQ_HIP_CHECK(lds_grant.ensure((const void *)mxfp4_mfma_kernel<MTOK, FR>, lds));
     hipLaunchKernelGGL((mxfp4_mfma_kernel<MTOK, FR>), grid, dim3(256), lds, s, (const uint16_t *)p.x, p.blocks,
                        p.scales, (const uint16_t *)p.bias, (uint16_t *)p.y, p.expert_offsets, p.token_ids,
                        (int)p.M, (int)p.K, (int)p.N, p.swiglu, p.swiglu_limit);

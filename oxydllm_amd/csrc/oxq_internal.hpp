@@ -5,6 +5,8 @@
 
 #include <cstdarg>
 #include <algorithm>
+#include <atomic>
+#include <mutex>
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
@@ -62,6 +64,29 @@ void add_launch(oxq_ctx *ctx);
         if (_e != hipSuccess)                                                                 \
             return ::oxq::fail(OXQ_ERR_RUNTIME, "%s failed: %s", #expr, hipGetErrorString(_e)); \
     } while (0)
+
+// A kernel's dynamic-LDS limit (hipFuncAttributeMaxDynamicSharedMemorySize) belongs to the pair
+// (function, device).  One LdsGrant per kernel instantiation remembers what each device has been
+// granted; the usual path is one atomic load, the raise happens under a lock so that a smaller
+// request from another engine thread cannot overwrite a larger one.
+struct LdsGrant {
+    static constexpr int MAX_DEVICES = 64;
+    std::atomic<size_t> granted[MAX_DEVICES] = {};
+    hipError_t ensure(const void *fn, size_t lds) {
+        int dev = 0;
+        hipError_t e = hipGetDevice(&dev);
+        if (e != hipSuccess) return e;
+        if (dev < 0 || dev >= MAX_DEVICES)  // not remembered: ask every time
+            return hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (lds <= granted[dev].load(std::memory_order_acquire)) return hipSuccess;
+        static std::mutex mu;
+        std::lock_guard<std::mutex> lock(mu);
+        if (lds <= granted[dev].load(std::memory_order_relaxed)) return hipSuccess;
+        e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e == hipSuccess) granted[dev].store(lds, std::memory_order_release);
+        return e;
+    }
+};
 
 // ---- problem descriptors handed to the launchers (all validated) ----------
 

@@ -692,12 +692,8 @@ template <typename TT, int BITS, int MT, bool GS, bool BPG1, int XQ, bool ZW = (
 static int pk4_go4(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, int gslice) {
     constexpr int AB = Pk4Ring<MT, BITS>::AB, WD = Pk4Ring<MT, BITS>::WD;
     const size_t lds = (size_t)8 * MT * 4096 + (size_t)gslice * 256 * (GS ? 2 : 1);
-    static size_t attr_lds = 0;  // one per instantiation
-    if (lds > attr_lds) {
-        OXQ_HIP_CHECK(hipFuncSetAttribute((const void *)pk4_mfma_kernel<TT, BITS, MT, GS, BPG1, AB, WD, XQ, ZW>,
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        attr_lds = lds;
-    }
+    static LdsGrant lds_grant;  // one per instantiation
+    OXQ_HIP_CHECK(lds_grant.ensure((const void *)pk4_mfma_kernel<TT, BITS, MT, GS, BPG1, AB, WD, XQ, ZW>, lds));
     hipLaunchKernelGGL((pk4_mfma_kernel<TT, BITS, MT, GS, BPG1, AB, WD, XQ, ZW>), grid, dim3(512), lds, s,
                        (const uint16_t *)p.x, p.w.pw, p.w.pzs, (const uint16_t *)p.bias, (uint16_t *)p.y,
                        (float *)ctx->workspace, (int)p.M, (int)p.w.K, (int)p.w.N, p.w.group_shift, gslice,
