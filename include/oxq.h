@@ -130,6 +130,17 @@ int oxq_gguf_block_layout(int quant, int64_t *block_elems, int64_t *block_bytes)
 int oxq_w4a16_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x, const oxq_tensor *qweight,
                      const oxq_tensor *qzeros, const oxq_tensor *scales, const oxq_tensor *out);
 
+/* No counterpart in the reference.  oxq_w4a16_matmul for callers that cannot allocate device
+ * memory (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc):
+ * same arguments, checks, kernels and result bits, but the split-K partial sums go to a static
+ * device array inside the library (16 MiB on every GPU the library runs on, held until the process
+ * ends) instead of the ctx workspace, the K slices are always added by a second launch, and the
+ * call makes no allocation of any kind.  A call whose partial sums (slices * m * N * 4 bytes) exceed
+ * 16 MiB fails with OXQ_ERR_WORKSPACE and enqueues nothing.  Every call on a GPU shares that GPU's
+ * array: calls that overlap on one GPU (two streams, two threads) race; serialise them. */
+int oxq_w4a16_matmul_static(oxq_ctx *ctx, void *stream, const oxq_tensor *x, const oxq_tensor *qweight,
+                            const oxq_tensor *qzeros, const oxq_tensor *scales, const oxq_tensor *out);
+
 /* metal_ops.rs:1835 w8a16_matmul: qweight [K, N/4] identity slot order. */
 int oxq_w8a16_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x, const oxq_tensor *qweight,
                      const oxq_tensor *qzeros, const oxq_tensor *scales, const oxq_tensor *out);

@@ -78,6 +78,7 @@ SIGNATURES = {
     "oxq_version": (None, [C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     "oxq_gguf_block_layout": (C.c_int, [C.c_int, C.POINTER(C.c_int64), C.POINTER(C.c_int64)]),
     "oxq_w4a16_matmul": (C.c_int, [_VP, _VP, _TP, _TP, _TP, _TP, _TP]),
+    "oxq_w4a16_matmul_static": (C.c_int, [_VP, _VP, _TP, _TP, _TP, _TP, _TP]),
     "oxq_w8a16_matmul": (C.c_int, [_VP, _VP, _TP, _TP, _TP, _TP, _TP]),
     "oxq_gptq_matmul": (C.c_int, [_VP, _VP, _TP, _TP, _TP, _TP, C.c_uint32, _TP]),
     "oxq_dequantize_w4": (C.c_int, [_VP, _VP, _TP, _TP, _TP, _TP]),

@@ -367,6 +367,41 @@ static int check_mxfp4(oxq_ctx *ctx, const char *op, bool dequant, const oxq_ten
 
 using namespace oxq;
 
+// -----------------------------------------------------------------------------
+// Split-K partial sums for the allocation-free entry point (oxq_w4a16_matmul_static): a device
+// array that exists from the moment the code object is loaded, one copy per GPU, each at its own
+// address.  In host code the name `scratch` is only a handle for hipGetSymbolAddress; the address
+// it returns (per device, taken once with that device current) is what kernels and copies use.
+// -----------------------------------------------------------------------------
+#define OXQ_STATIC_SCRATCH_BYTES (16u << 20)
+static __device__ __align__(256) unsigned char scratch[OXQ_STATIC_SCRATCH_BYTES];
+
+namespace oxq {
+static constexpr int SCRATCH_MAX_DEVICES = 64;
+static std::atomic<void *> g_scratch_ptr[SCRATCH_MAX_DEVICES] = {};
+static std::mutex g_scratch_mu;
+
+// The calling thread must have `device` current.
+static int scratch_lookup(int device, void **out) {
+    if (device < 0 || device >= SCRATCH_MAX_DEVICES)
+        return fail(OXQ_ERR_DEVICE, "static scratch: device ordinal %d outside 0..%d", device, SCRATCH_MAX_DEVICES - 1);
+    void *ptr = g_scratch_ptr[device].load(std::memory_order_acquire);
+    if (!ptr) {
+        std::lock_guard<std::mutex> lock(g_scratch_mu);
+        ptr = g_scratch_ptr[device].load(std::memory_order_relaxed);
+        if (!ptr) {
+            hipError_t e = hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch));
+            if (e != hipSuccess || !ptr)
+                return fail(OXQ_ERR_RUNTIME, "static scratch: hipGetSymbolAddress on device %d failed: %s", device,
+                            hipGetErrorString(e));
+            g_scratch_ptr[device].store(ptr, std::memory_order_release);
+        }
+    }
+    *out = ptr;
+    return OXQ_OK;
+}
+}  // namespace oxq
+
 // =============================================================================
 // C ABI
 // =============================================================================
@@ -461,8 +496,17 @@ int oxq_ctx_create(int device, oxq_ctx **out) {
             break;
         if ((e = hipMemset(ctx->counters, 0, ctx->n_counters * sizeof(unsigned))) != hipSuccess) break;
         e = hipDeviceSynchronize();
+        // this device's address of the static scratch array, looked up once while it is current
+        void *sp = nullptr;
+        if (e == hipSuccess && scratch_lookup(device, &sp) != OXQ_OK) rc = OXQ_ERR_RUNTIME;
     } while (0);
     (void)hipSetDevice(prev);
+    if (e == hipSuccess && rc != OXQ_OK) {  // scratch_lookup has set the message
+        (void)hipFree(ctx->workspace);
+        (void)hipFree(ctx->counters);
+        delete ctx;
+        return rc;
+    }
     if (e != hipSuccess) {
         rc = fail(OXQ_ERR_RUNTIME, "oxq_ctx_create: %s", hipGetErrorString(e));
         if (ctx->workspace) (void)hipFree(ctx->workspace);
@@ -499,6 +543,46 @@ int oxq_w4a16_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x, const oxq_
     OXQ_TRY(check_wna16(ctx, "W4A16Matmul", KIND_GEMV, x, qweight, qzeros, scales, 4, OXQ_PACK_OUT,
                         out, &p));
     return launch_wna16_gemv(ctx, (hipStream_t)stream, p);
+}
+
+// oxq_w4a16_matmul for callers that cannot allocate: same validation, same kernels, same bits, but
+// the split-K partial sums live in this device's copy of the static `scratch` array instead of the
+// ctx workspace, and the slices are always added by the second launch (plain stores, no arrival
+// counters: nothing in the array has to start at zero).  Calls no allocator.
+int oxq_w4a16_matmul_static(oxq_ctx *ctx, void *stream, const oxq_tensor *x, const oxq_tensor *qweight,
+                            const oxq_tensor *qzeros, const oxq_tensor *scales, const oxq_tensor *out) {
+    Wna16Problem p;
+    OXQ_TRY(check_wna16(ctx, "W4A16MatmulStatic", KIND_GEMV, x, qweight, qzeros, scales, 4, OXQ_PACK_OUT,
+                        out, &p));
+    oxq_ctx shadow = *ctx;  // the launchers read workspace, its size and the reduction mode from a ctx
+    shadow.workspace = nullptr;
+    shadow.workspace_bytes = ~(size_t)0;
+    shadow.counters = nullptr;
+    shadow.n_counters = 0xFFFFFFFFu;
+    shadow.splitk_mode = 2;
+    shadow.plan_only = true;  // first pass: what would this call need?
+    OXQ_TRY(launch_wna16_gemv(&shadow, (hipStream_t)stream, p));
+    if (shadow.plan.workspace_bytes > OXQ_STATIC_SCRATCH_BYTES)
+        return fail(OXQ_ERR_WORKSPACE,
+                    "W4A16MatmulStatic: the call needs %llu bytes of split-K partial sums, the static scratch "
+                    "array holds %u (m = %lld, n = %lld, %u slices): use oxq_w4a16_matmul",
+                    (unsigned long long)shadow.plan.workspace_bytes, OXQ_STATIC_SCRATCH_BYTES, (long long)p.M,
+                    (long long)p.N, shadow.plan.split_k);
+    if (shadow.plan.split_k > 1 && shadow.plan.launches < 2)
+        return fail(OXQ_ERR_UNSUPPORTED, "W4A16MatmulStatic: this shape sums its K slices with arrival counters");
+    if (ctx->plan_only) {
+        ctx->plan = shadow.plan;
+        return OXQ_OK;
+    }
+    void *sp = g_scratch_ptr[ctx->device >= 0 && ctx->device < SCRATCH_MAX_DEVICES ? ctx->device : 0].load(
+        std::memory_order_acquire);
+    if (!sp) return fail(OXQ_ERR_RUNTIME, "W4A16MatmulStatic: no static scratch address for device %d", ctx->device);
+    shadow.plan_only = false;
+    shadow.workspace = sp;
+    shadow.workspace_bytes = OXQ_STATIC_SCRATCH_BYTES;
+    const int rc = launch_wna16_gemv(&shadow, (hipStream_t)stream, p);
+    if (rc == OXQ_OK) ctx->plan = shadow.plan;
+    return rc;
 }
 
 int oxq_w8a16_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x, const oxq_tensor *qweight,

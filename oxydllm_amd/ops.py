@@ -121,6 +121,16 @@ def w4a16_matmul(x, qweight, qzeros, scales, *, out=None, ctx: Optional[Context]
     return out
 
 
+def w4a16_matmul_static(x, qweight, qzeros, scales, *, out, ctx: Optional[Context] = None):
+    """``w4a16_matmul`` through the entry point that allocates nothing: the split-K partial sums go to
+    the library's static device array (16 MiB per GPU) instead of the ctx workspace.  ``out`` is
+    mandatory (this binding allocates nothing either); calls that overlap on one GPU race."""
+    ctx = _ctx(ctx)
+    _lib.check(ctx._lib.oxq_w4a16_matmul_static(ctx.handle, ctx.stream(), desc(x), desc(qweight),
+                                                desc(qzeros), desc(scales), desc(out)))
+    return out
+
+
 def w8a16_matmul(x, qweight, qzeros, scales, *, out=None, ctx: Optional[Context] = None):
     """metal_ops.rs:1835."""
     ctx = _ctx(ctx)
