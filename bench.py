@@ -16,6 +16,10 @@ results, in GB/s and TFLOP/s, ride along in `cases`.  `roofline` describes the
 dominant kernel (the M=1 GEMV, HBM-bound); `cpu_baseline` times the CPU oracle's
 restatement of the reference's CPU path (dequantize at load, then a dense f32
 x.W^T per call, linear.rs:40-79, 597-600) on this machine's cores.
+`roofline.bare_read_us` / `bare_read_nt_us` are a plain read of the same packed
+weights with the same launch shape and no arithmetic (plain / nontemporal loads).
+`other_configs` holds one compact row per case of BASELINE configs 0, 2, 3 and 4,
+each with its own roofline fraction and a CPU baseline per configuration.
 """
 from __future__ import annotations
 
@@ -116,7 +120,12 @@ def main():
     ap.add_argument("--no-hot", action="store_true",
                     help="skip the same-weights-every-call (cache-resident) timings, so that a profiler "
                          "run sees only the launches `value` is computed from plus the warm-up")
-    ap.add_argument("--all", action="store_true", help="also time GPTQ / GGUF / MXFP4 (stderr)")
+    ap.add_argument("--no-others", action="store_true",
+                    help="skip the compact rows for BASELINE configs 0, 2, 3 and 4 (`other_configs`)")
+    ap.add_argument("--no-bare-read", action="store_true",
+                    help="skip the plain-read calibration (`roofline.bare_read_us`)")
+    ap.add_argument("--all", action="store_true",
+                    help="also the long list: prefill sizes, fused FFN entry, F8, all ten GGUF formats (`extra_configs`)")
     ap.add_argument("--calib-copy", action="store_true",
                     help="first run a plain 256 MiB device copy 4 times: a kernel of known HBM "
                          "traffic to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings with")
@@ -215,6 +224,24 @@ def main():
             print(f"[bench] down-projection layer M={m}: {down_cases[-1]}", file=sys.stderr, flush=True)
         del dlayers
 
+    # What a kernel with no arithmetic takes to read the same packed weights once: 224 workgroups of 512
+    # threads, 128 KB each (the resident-layer kernel's launch shape), plain and nontemporal loads, cold.
+    bare = {}
+    if not args.no_bare_read:
+        nbytes_w = K * N // 2
+        pool = torch.empty(copies * nbytes_w, dtype=torch.uint8, device=dev).random_(0, 256)
+        sums = torch.empty(256, dtype=torch.int32, device=dev)
+        for nt in (0, 1):
+            def rd(i, nt=nt):
+                c = i % copies
+                ops.calib_read(pool[c * nbytes_w:(c + 1) * nbytes_w], N // 64, bool(nt), sums, ctx=ctx)
+            _, ev = time_graph(rd, args.steps, args.warmup, stream)
+            bare["bare_read_nt_us" if nt else "bare_read_us"] = round(ev * 1e3 / args.steps, 3)
+        bare["bare_read_bytes"] = nbytes_w
+        bare["bare_read_workgroups"] = N // 64
+        print(f"[bench] plain read of {nbytes_w} B by {N // 64} workgroups: {bare}", file=sys.stderr, flush=True)
+        del pool
+
     c1 = cases[0]
     # HBM bytes per launch of the M=1 kernel, measured offline with rocprofv3 --pmc
     # (FETCH_SIZE, WRITE_SIZE) and recorded in the committed profile summary.
@@ -248,7 +275,7 @@ def main():
         "roofline": {"bound": "hbm", "achieved": c1["GB_per_s"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(c1["GB_per_s"] / HBM_PEAK_GBS, 4), "traffic": traffic,
                      "kernel": c1["kernel"], "algorithmic_bytes_per_launch": c1["algorithmic_bytes"],
-                     "us_per_launch": c1["us_per_call"]},
+                     "us_per_launch": c1["us_per_call"], **bare},
         "roofline_m64": {"bound": "mfma", "achieved": cases[2]["TFLOP_per_s"],
                          "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                          "frac": cases[2]["mfma_frac"], "traffic": None,
@@ -257,9 +284,18 @@ def main():
         "cases_down_projection_K14336_N4096": down_cases,
         "cases_checkpoint_layout_ops": op_cases,
     }
+    del layers, qw_d, qz_d, sc_d
+    torch.cuda.empty_cache()
+    if not args.no_others:
+        from oxydllm_amd import bench_configs
+        result["other_configs"] = bench_configs.run(ops, ctx, stream, args.steps, args.warmup, time_graph,
+                                                    with_cpu=not args.no_cpu)
+        for r in result["other_configs"]:
+            print(f"[bench] {r['config']}: {r['case']}: {r['us_per_call']} us, {r['GB_per_s']} GB/s "
+                  f"({r['roofline']['frac']:.3f} of HBM peak), {r['kernel']}", file=sys.stderr, flush=True)
     if args.all:
         from oxydllm_amd import bench_extra
-        result["other_configs"] = bench_extra.run(ops, ctx, stream, args.steps, args.warmup, time_graph)
+        result["extra_configs"] = bench_extra.run(ops, ctx, stream, args.steps, args.warmup, time_graph)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(qw, qz, sc, x_host[1])
     else:

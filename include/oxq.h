@@ -121,6 +121,16 @@ void oxq_version(int *major, int *minor);
 /* Block layout of a GGUF format: metal_ops.rs:5228-5241 (block_layout). */
 int oxq_gguf_block_layout(int quant, int64_t *block_elems, int64_t *block_bytes);
 
+/* ---- measurement aid ---------------------------------------------------------
+ * No counterpart in the reference.  A plain streaming read of `src` (U8, contiguous, 16-byte
+ * aligned; its size a multiple of workgroups * 64 KiB) by `workgroups` workgroups of 512 threads,
+ * each reading one contiguous span with 16-byte loads, eight in flight per lane - the launch shape of
+ * the resident-layer GEMV with the arithmetic taken out.  `checksums` (U32 [>= workgroups]) receives
+ * an xor of every span, which keeps the loads alive and lets a test check the read.  bench.py times
+ * it beside the GEMV kernels: it is what a read-once kernel can reach on the machine at hand. */
+int oxq_calib_read(oxq_ctx *ctx, void *stream, const oxq_tensor *src, int workgroups, int nontemporal,
+                   const oxq_tensor *checksums);
+
 /* ---- decode GEMV ops (1 <= m <= 8) ---------------------------------------
  * y[m,N] = x[m,K] . dequant(W), f32 accumulate, result in x's dtype.
  * x, scales: F16 or BF16 (same type); qweight/qzeros: I32 or U32. */

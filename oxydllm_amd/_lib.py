@@ -9,7 +9,8 @@ import ctypes as C
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "liboxq_hip.so")
+# OXQ_LIB_PATH names another build of the same library (a tuning variant); the default is the in-tree one
+LIB_PATH = os.environ.get("OXQ_LIB_PATH") or os.path.join(HERE, "liboxq_hip.so")
 
 OXQ_MAX_RANK = 4
 (F32, F16, BF16, U8, I32, U32, I64) = range(7)
@@ -77,6 +78,7 @@ SIGNATURES = {
     "oxq_status_name": (C.c_char_p, [C.c_int]),
     "oxq_version": (None, [C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     "oxq_gguf_block_layout": (C.c_int, [C.c_int, C.POINTER(C.c_int64), C.POINTER(C.c_int64)]),
+    "oxq_calib_read": (C.c_int, [_VP, _VP, _TP, C.c_int, C.c_int, _TP]),
     "oxq_w4a16_matmul": (C.c_int, [_VP, _VP, _TP, _TP, _TP, _TP, _TP]),
     "oxq_w4a16_matmul_static": (C.c_int, [_VP, _VP, _TP, _TP, _TP, _TP, _TP]),
     "oxq_w8a16_matmul": (C.c_int, [_VP, _VP, _TP, _TP, _TP, _TP, _TP]),

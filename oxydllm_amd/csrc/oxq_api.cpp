@@ -536,6 +536,31 @@ int oxq_ctx_last_plan(const oxq_ctx *ctx, oxq_plan *out) {
     return OXQ_OK;
 }
 
+// ---- measurement aid ----------------------------------------------------------
+int oxq_calib_read(oxq_ctx *ctx, void *stream, const oxq_tensor *src, int workgroups, int nontemporal,
+                   const oxq_tensor *checksums) {
+    if (!ctx || !src || !checksums) return fail(OXQ_ERR_ARG, "CalibRead: NULL argument");
+    OXQ_TRY(check_tensor(ctx, "CalibRead", "src", src));
+    OXQ_TRY(check_tensor(ctx, "CalibRead", "checksums", checksums));
+    if (src->dtype != OXQ_U8 || !src->contiguous)
+        return fail(OXQ_ERR_DTYPE, "CalibRead: src must be a contiguous U8 tensor, got %s", dtype_name(src->dtype));
+    if ((checksums->dtype != OXQ_U32 && checksums->dtype != OXQ_I32) || !checksums->contiguous)
+        return fail(OXQ_ERR_DTYPE, "CalibRead: checksums must be a contiguous U32/I32 tensor, got %s",
+                    dtype_name(checksums->dtype));
+    const int64_t bytes = numel(src);
+    if (workgroups < 1 || workgroups > 65535 || numel(checksums) < workgroups)
+        return fail(OXQ_ERR_SHAPE, "CalibRead: %d workgroups need 1..65535 and one checksum word each (got %lld)",
+                    workgroups, (long long)numel(checksums));
+    if (bytes <= 0 || bytes % ((int64_t)workgroups * 65536) != 0 || bytes / workgroups >= (int64_t(1) << 31))
+        return fail(OXQ_ERR_SHAPE,
+                    "CalibRead: %lld bytes over %d workgroups: every workgroup reads a span that is a multiple "
+                    "of 64 KiB and below 2 GiB", (long long)bytes, workgroups);
+    if (!ctx->plan_only && ((uintptr_t)src->data & 15))
+        return fail(OXQ_ERR_UNSUPPORTED, "CalibRead: src must be 16-byte aligned");
+    return launch_calib_read(ctx, (hipStream_t)stream, (const uint8_t *)src->data, (uint64_t)bytes, workgroups,
+                             nontemporal, (uint32_t *)checksums->data);
+}
+
 // ---- AWQ / GPTQ -------------------------------------------------------------
 int oxq_w4a16_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x, const oxq_tensor *qweight,
                      const oxq_tensor *qzeros, const oxq_tensor *scales, const oxq_tensor *out) {

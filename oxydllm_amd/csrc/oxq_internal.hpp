@@ -217,6 +217,9 @@ int launch_gated_activation(oxq_ctx *ctx, hipStream_t s, const void *gu, void *o
                             int64_t half_n, int kind, float limit);
 int launch_moe_combine(oxq_ctx *ctx, hipStream_t s, const void *eo, const int32_t *pair_pos, const float *top_vals,
                        void *out, int dtype, int64_t T, int64_t H, int64_t top_k);
+// plain streaming read (calib.hip): bytes = workgroups * span, span a multiple of 64 KiB
+int launch_calib_read(oxq_ctx *ctx, hipStream_t s, const uint8_t *src, uint64_t bytes, int workgroups, int nontemporal,
+                      uint32_t *out);
 // y[M,N] = sum over S slices of ws[s][M][N] (+ bias), slices added in index order.
 int launch_splitk_reduce(oxq_ctx *ctx, hipStream_t s, const float *ws, const void *bias, void *y,
                          int64_t M, int64_t N, int S, int dtype);

@@ -112,6 +112,15 @@ def _out_for(x: torch.Tensor, n: int, out, ctx):
 
 
 # ---------------------------------------------------------------- AWQ / GPTQ ops
+def calib_read(src, workgroups: int, nontemporal: bool, checksums, *, ctx: Optional[Context] = None):
+    """Plain streaming read of ``src`` (uint8) by ``workgroups`` workgroups; ``checksums`` (int32/uint32,
+    one word per workgroup) receives the xor of every span.  A measurement aid (see include/oxq.h)."""
+    ctx = _ctx(ctx)
+    _lib.check(ctx._lib.oxq_calib_read(ctx.handle, ctx.stream(), desc(src), int(workgroups), int(bool(nontemporal)),
+                                       desc(checksums)))
+    return checksums
+
+
 def w4a16_matmul(x, qweight, qzeros, scales, *, out=None, ctx: Optional[Context] = None):
     """metal_ops.rs:1821.  x [m,K] (m in 1..=8) -> [m,N] in x's dtype."""
     ctx = _ctx(ctx)
