@@ -38,6 +38,8 @@ HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 MFMA_F16_PEAK_TFLOPS = 2500.0
 K, N, G = 4096, 14336, 128
 SAMPLES = 11                # timed replays per case; the median is reported
+MIN_TIMED_STEPS = 200       # launches inside one event pair (short graphs are replayed back to back)
+SPINUP_MS = 30.0            # untimed replays ahead of the samples of every case
 
 
 def algo_bytes(M: int, k: int = K, n: int = N, g: int = G, bits: int = 4) -> int:
@@ -63,19 +65,40 @@ def time_graph(fn_of_step, steps: int, warmup: int, stream):
     torch.cuda.synchronize()
     graph.replay()          # untimed replay (first replay uploads the graph)
     torch.cuda.synchronize()
+    # Untimed: keep the GPU busy for SPINUP_MS before sampling.  A replay of 20 steps lasts 0.2 ms; from
+    # idle, that is over before the clocks have come up, and a short run would time the ramp.
+    t_spin = time.perf_counter()
+    while (time.perf_counter() - t_spin) * 1e3 < SPINUP_MS:
+        for _ in range(8):
+            graph.replay()
+        torch.cuda.synchronize()
     cur = torch.cuda.current_stream()
+    reps = max(1, -(-MIN_TIMED_STEPS // steps))
     walls, evs = [], []
     for _ in range(SAMPLES):   # median of SAMPLES replays of the same `steps` launches
         ev0 = torch.cuda.Event(enable_timing=True)
         ev1 = torch.cuda.Event(enable_timing=True)
+        # (a) the host's clock around one replay, synchronized on both sides: `steps` launches plus
+        # the host's graph-launch latency (about 12 us, a large share of a 20-step replay)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        ev0.record(cur)
         graph.replay()
-        ev1.record(cur)
         torch.cuda.synchronize()
         walls.append((time.perf_counter() - t0) * 1e3)
-        evs.append(ev0.elapsed_time(ev1))
+        # (b) HIP events on the launch stream, with untimed replays directly ahead: the timed replays
+        # are enqueued while the GPU is still busy, so the first kernel starts when the event before it
+        # completes and the launch latency is not counted as kernel time.  The event pair itself costs a
+        # few microseconds, which a 20-step replay would carry as +0.4 us per step: short graphs are
+        # replayed `reps` times back to back inside one pair (at least MIN_TIMED_STEPS launches) and the
+        # pair's time is divided by `reps`, i.e. each sample is the mean time of `steps` launches.
+        graph.replay()
+        graph.replay()
+        ev0.record(cur)
+        for _ in range(reps):
+            graph.replay()
+        ev1.record(cur)
+        torch.cuda.synchronize()
+        evs.append(ev0.elapsed_time(ev1) / reps)
     return float(np.median(walls)), float(np.median(evs))
 
 
@@ -271,7 +294,8 @@ def main():
                                "(BASELINE configs[1]) through PackedQuantLinear.forward on a resident layer; "
                                "M=16/64 in `cases`; the stateless checkpoint-layout ops in "
                                "`cases_checkpoint_layout_ops`",
-                   "weight_copies_rotated": copies, "timing": f"HIP graph of `steps` launches, median of {SAMPLES} replays"},
+                   "weight_copies_rotated": copies, "timing": f"HIP graph of `steps` launches; {SAMPLES} samples, each one HIP-event pair around "
+                             f"max(1, ceil({MIN_TIMED_STEPS}/steps)) back-to-back replays divided by that count; median"},
         "roofline": {"bound": "hbm", "achieved": c1["GB_per_s"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(c1["GB_per_s"] / HBM_PEAK_GBS, 4), "traffic": traffic,
                      "kernel": c1["kernel"], "algorithmic_bytes_per_launch": c1["algorithmic_bytes"],
