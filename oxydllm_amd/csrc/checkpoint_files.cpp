@@ -18,6 +18,8 @@
 #include <cmath>
 #include <cstdlib>
 #include <map>
+#include <new>
+#include <exception>
 #include <string>
 #include <unordered_map>
 #include <utility>
@@ -437,6 +439,10 @@ int load_gguf_shard(oxq_tensor_file *f, int shard) {
     uint64_t n_tensors = r.count(version);
     uint64_t n_meta = r.count(version);
     if (!r.ok) return fail(OXQ_ERR_FORMAT, "%s: truncated GGUF header", path);
+    // a tensor record is at least 24 bytes (name length, rank, type, offset), a metadata record at least 12
+    if (n_tensors > m.len / 24 || n_meta > m.len / 12)
+        return fail(OXQ_ERR_FORMAT, "%s: truncated or damaged GGUF header: %llu tensors and %llu metadata records cannot fit in %zu bytes", path,
+                    (unsigned long long)n_tensors, (unsigned long long)n_meta, m.len);
 
     uint64_t alignment = 32;
     for (uint64_t i = 0; i < n_meta; ++i) {
@@ -511,7 +517,11 @@ int load_gguf_shard(oxq_tensor_file *f, int shard) {
         if (elems % uint64_t(info.type->block_elems) != 0)
             return fail(OXQ_ERR_FORMAT, "%s: tensor '%s': tensor elements %llu not divisible by block size %lld", path,
                         info.name.c_str(), (unsigned long long)elems, (long long)info.type->block_elems);
-        uint64_t nbytes = elems / uint64_t(info.type->block_elems) * uint64_t(info.type->block_bytes);
+        const uint64_t blocks = elems / uint64_t(info.type->block_elems);
+        if (blocks > UINT64_MAX / uint64_t(info.type->block_bytes))  // one-element "blocks" (F32, F16 ...) can wrap
+            return fail(OXQ_ERR_FORMAT, "%s: tensor '%s': byte count of %llu elements overflows", path,
+                        info.name.c_str(), (unsigned long long)elems);
+        uint64_t nbytes = blocks * uint64_t(info.type->block_bytes);
         uint64_t start = data_offset + info.offset;
         if (start < data_offset || start + nbytes < start)
             return fail(OXQ_ERR_FORMAT, "%s: tensor '%s': tensor offset overflow", path, info.name.c_str());
@@ -666,40 +676,65 @@ bool ieq(const char *a, const char *b) {
     return *a == *b;
 }
 
+// No exception may cross the C ABI (a Rust caller would abort or worse): every entry point below runs
+// inside this guard, which turns std::bad_alloc and anything else thrown by the containers into a status.
+template <typename F>
+static int guarded(const char *op, F &&f) noexcept {
+    try {
+        return f();
+    } catch (const std::bad_alloc &) {
+        return fail(OXQ_ERR_RUNTIME, "%s: out of host memory", op);
+    } catch (const std::exception &e) {
+        return fail(OXQ_ERR_RUNTIME, "%s: %s", op, e.what());
+    } catch (...) {
+        return fail(OXQ_ERR_RUNTIME, "%s: unexpected exception", op);
+    }
+}
+
 }  // namespace
 
 extern "C" {
 
 int oxq_gguf_open(const char *const *paths, int n_paths, oxq_tensor_file **out) {
-    return open_files("oxq_gguf_open", paths, n_paths, true, out);
+    return guarded("oxq_gguf_open", [&]() -> int {
+        return open_files("oxq_gguf_open", paths, n_paths, true, out);
+    });
 }
 
 int oxq_safetensors_open(const char *const *paths, int n_paths, oxq_tensor_file **out) {
-    return open_files("oxq_safetensors_open", paths, n_paths, false, out);
+    return guarded("oxq_safetensors_open", [&]() -> int {
+        return open_files("oxq_safetensors_open", paths, n_paths, false, out);
+    });
 }
 
 int oxq_tensor_file_close(oxq_tensor_file *f) {
-    delete f;
-    return OXQ_OK;
+    return guarded("oxq_tensor_file_close", [&]() -> int {
+        delete f;
+        return OXQ_OK;
+    });
 }
 
 int64_t oxq_tensor_file_count(const oxq_tensor_file *f) { return f ? int64_t(f->order.size()) : 0; }
 
 int oxq_tensor_file_at(const oxq_tensor_file *f, int64_t index, oxq_file_tensor *out) {
-    if (!f || !out) return fail(OXQ_ERR_ARG, "oxq_tensor_file_at: NULL argument");
-    if (index < 0 || index >= int64_t(f->order.size()))
-        return fail(OXQ_ERR_ARG, "oxq_tensor_file_at: index %lld out of [0, %zu)", (long long)index, f->order.size());
-    fill(*f->order[size_t(index)], out);
-    return OXQ_OK;
+    return guarded("oxq_tensor_file_at", [&]() -> int {
+        if (!f || !out) return fail(OXQ_ERR_ARG, "oxq_tensor_file_at: NULL argument");
+        if (index < 0 || index >= int64_t(f->order.size()))
+            return fail(OXQ_ERR_ARG, "oxq_tensor_file_at: index %lld out of [0, %zu)", (long long)index, f->order.size());
+        fill(*f->order[size_t(index)], out);
+        return OXQ_OK;
+    });
 }
 
 int oxq_tensor_file_find(const oxq_tensor_file *f, const char *name, oxq_file_tensor *out, int *found) {
-    if (!f || !name || !out || !found) return fail(OXQ_ERR_ARG, "oxq_tensor_file_find: NULL argument");
-    const TensorEntry *e = resolve(f, name);
-    *found = e != nullptr;
-    if (e) fill(*e, out);
-    else memset(out, 0, sizeof *out);
-    return OXQ_OK;
+    return guarded("oxq_tensor_file_find", [&]() -> int {
+        if (!f || !name || !out || !found) return fail(OXQ_ERR_ARG, "oxq_tensor_file_find: NULL argument");
+        const TensorEntry *e = resolve(f, name);
+        *found = e != nullptr;
+        if (e) fill(*e, out);
+        else memset(out, 0, sizeof *out);
+        return OXQ_OK;
+    });
 }
 
 uint64_t oxq_tensor_file_total_bytes(const oxq_tensor_file *f) {
@@ -710,245 +745,267 @@ uint64_t oxq_tensor_file_total_bytes(const oxq_tensor_file *f) {
 }
 
 int oxq_tensor_file_has_packed_quantized_weights(const oxq_tensor_file *f) {
-    if (!f) return 0;
-    auto ends_with = [](const std::string &s, const char *suffix) {
-        size_t n = strlen(suffix);
-        return s.size() >= n && s.compare(s.size() - n, n, suffix) == 0;
-    };
-    for (const TensorEntry *e : f->order)
-        if (ends_with(e->name, ".qweight") || ends_with(e->name, ".weight_packed")) return 1;
-    return 0;
+    return guarded("oxq_tensor_file_has_packed_quantized_weights", [&]() -> int {
+        if (!f) return 0;
+        auto ends_with = [](const std::string &s, const char *suffix) {
+            size_t n = strlen(suffix);
+            return s.size() >= n && s.compare(s.size() - n, n, suffix) == 0;
+        };
+        for (const TensorEntry *e : f->order)
+            if (ends_with(e->name, ".qweight") || ends_with(e->name, ".weight_packed")) return 1;
+        return 0;
+    });
 }
 
 int64_t oxq_gguf_metadata_count(const oxq_tensor_file *f) { return f ? int64_t(f->meta.size()) : 0; }
 
 int oxq_gguf_metadata_at(const oxq_tensor_file *f, int64_t index, const char **key, int *value_type, int *elem_type,
                          uint64_t *elem_count) {
-    if (!f || !key || !value_type) return fail(OXQ_ERR_ARG, "oxq_gguf_metadata_at: NULL argument");
-    if (index < 0 || index >= int64_t(f->meta.size()))
-        return fail(OXQ_ERR_ARG, "oxq_gguf_metadata_at: index %lld out of [0, %zu)", (long long)index, f->meta.size());
-    const auto &kv = f->meta[size_t(index)];
-    *key = kv.first.c_str();
-    *value_type = kv.second.type;
-    if (elem_type) *elem_type = kv.second.type == OXQ_GGUF_ARRAY ? kv.second.elem_type : -1;
-    if (elem_count) *elem_count = kv.second.type == OXQ_GGUF_ARRAY ? kv.second.elem_count : 0;
-    return OXQ_OK;
+    return guarded("oxq_gguf_metadata_at", [&]() -> int {
+        if (!f || !key || !value_type) return fail(OXQ_ERR_ARG, "oxq_gguf_metadata_at: NULL argument");
+        if (index < 0 || index >= int64_t(f->meta.size()))
+            return fail(OXQ_ERR_ARG, "oxq_gguf_metadata_at: index %lld out of [0, %zu)", (long long)index, f->meta.size());
+        const auto &kv = f->meta[size_t(index)];
+        *key = kv.first.c_str();
+        *value_type = kv.second.type;
+        if (elem_type) *elem_type = kv.second.type == OXQ_GGUF_ARRAY ? kv.second.elem_type : -1;
+        if (elem_count) *elem_count = kv.second.type == OXQ_GGUF_ARRAY ? kv.second.elem_count : 0;
+        return OXQ_OK;
+    });
 }
 
 int oxq_gguf_metadata_u32(const oxq_tensor_file *f, const char *key, uint32_t *value, int *found) {
-    if (!f || !key || !value || !found) return fail(OXQ_ERR_ARG, "oxq_gguf_metadata_u32: NULL argument");
-    const MetaValue *v = meta(f, key);
-    *found = v && v->type == OXQ_GGUF_U32;
-    if (*found) *value = uint32_t(v->bits);
-    return OXQ_OK;
+    return guarded("oxq_gguf_metadata_u32", [&]() -> int {
+        if (!f || !key || !value || !found) return fail(OXQ_ERR_ARG, "oxq_gguf_metadata_u32: NULL argument");
+        const MetaValue *v = meta(f, key);
+        *found = v && v->type == OXQ_GGUF_U32;
+        if (*found) *value = uint32_t(v->bits);
+        return OXQ_OK;
+    });
 }
 
 int oxq_gguf_metadata_f32(const oxq_tensor_file *f, const char *key, float *value, int *found) {
-    if (!f || !key || !value || !found) return fail(OXQ_ERR_ARG, "oxq_gguf_metadata_f32: NULL argument");
-    const MetaValue *v = meta(f, key);
-    *found = v && v->type == OXQ_GGUF_F32;
-    if (*found) {
-        uint32_t b = uint32_t(v->bits);
-        memcpy(value, &b, 4);
-    }
-    return OXQ_OK;
+    return guarded("oxq_gguf_metadata_f32", [&]() -> int {
+        if (!f || !key || !value || !found) return fail(OXQ_ERR_ARG, "oxq_gguf_metadata_f32: NULL argument");
+        const MetaValue *v = meta(f, key);
+        *found = v && v->type == OXQ_GGUF_F32;
+        if (*found) {
+            uint32_t b = uint32_t(v->bits);
+            memcpy(value, &b, 4);
+        }
+        return OXQ_OK;
+    });
 }
 
 int oxq_gguf_metadata_string(const oxq_tensor_file *f, const char *key, const char **value, uint64_t *len, int *found) {
-    if (!f || !key || !value || !found) return fail(OXQ_ERR_ARG, "oxq_gguf_metadata_string: NULL argument");
-    const MetaValue *v = meta(f, key);
-    *found = v && v->type == OXQ_GGUF_STRING;
-    if (*found) {
-        *value = v->str.c_str();
-        if (len) *len = v->str.size();
-    }
-    return OXQ_OK;
+    return guarded("oxq_gguf_metadata_string", [&]() -> int {
+        if (!f || !key || !value || !found) return fail(OXQ_ERR_ARG, "oxq_gguf_metadata_string: NULL argument");
+        const MetaValue *v = meta(f, key);
+        *found = v && v->type == OXQ_GGUF_STRING;
+        if (*found) {
+            *value = v->str.c_str();
+            if (len) *len = v->str.size();
+        }
+        return OXQ_OK;
+    });
 }
 
 int oxq_gguf_metadata_number(const oxq_tensor_file *f, const char *key, double *value, int *found) {
-    if (!f || !key || !value || !found) return fail(OXQ_ERR_ARG, "oxq_gguf_metadata_number: NULL argument");
-    const MetaValue *v = meta(f, key);
-    *found = 0;
-    if (!v) return OXQ_OK;
-    uint64_t b = v->bits;
-    switch (v->type) {
-    case OXQ_GGUF_U8: case OXQ_GGUF_U16: case OXQ_GGUF_U32: case OXQ_GGUF_U64: *value = double(b); break;
-    case OXQ_GGUF_BOOL: *value = b ? 1.0 : 0.0; break;
-    case OXQ_GGUF_I8: *value = double(int8_t(b)); break;
-    case OXQ_GGUF_I16: *value = double(int16_t(b)); break;
-    case OXQ_GGUF_I32: *value = double(int32_t(b)); break;
-    case OXQ_GGUF_I64: *value = double(int64_t(b)); break;
-    case OXQ_GGUF_F32: { uint32_t w = uint32_t(b); float x; memcpy(&x, &w, 4); *value = x; break; }
-    case OXQ_GGUF_F64: { double x; memcpy(&x, &b, 8); *value = x; break; }
-    default: return OXQ_OK;
-    }
-    *found = 1;
-    return OXQ_OK;
+    return guarded("oxq_gguf_metadata_number", [&]() -> int {
+        if (!f || !key || !value || !found) return fail(OXQ_ERR_ARG, "oxq_gguf_metadata_number: NULL argument");
+        const MetaValue *v = meta(f, key);
+        *found = 0;
+        if (!v) return OXQ_OK;
+        uint64_t b = v->bits;
+        switch (v->type) {
+        case OXQ_GGUF_U8: case OXQ_GGUF_U16: case OXQ_GGUF_U32: case OXQ_GGUF_U64: *value = double(b); break;
+        case OXQ_GGUF_BOOL: *value = b ? 1.0 : 0.0; break;
+        case OXQ_GGUF_I8: *value = double(int8_t(b)); break;
+        case OXQ_GGUF_I16: *value = double(int16_t(b)); break;
+        case OXQ_GGUF_I32: *value = double(int32_t(b)); break;
+        case OXQ_GGUF_I64: *value = double(int64_t(b)); break;
+        case OXQ_GGUF_F32: { uint32_t w = uint32_t(b); float x; memcpy(&x, &w, 4); *value = x; break; }
+        case OXQ_GGUF_F64: { double x; memcpy(&x, &b, 8); *value = x; break; }
+        default: return OXQ_OK;
+        }
+        *found = 1;
+        return OXQ_OK;
+    });
 }
 
 int oxq_gguf_architecture(const oxq_tensor_file *f, const char **value, uint64_t *len, int *found) {
-    return oxq_gguf_metadata_string(f, "general.architecture", value, len, found);
+    return guarded("oxq_gguf_architecture", [&]() -> int {
+        return oxq_gguf_metadata_string(f, "general.architecture", value, len, found);
+    });
 }
 
 int oxq_gguf_eos_token_ids(const oxq_tensor_file *f, uint32_t *ids, uint64_t cap, uint64_t *count) {
-    if (!f || !count || (!ids && cap)) return fail(OXQ_ERR_ARG, "oxq_gguf_eos_token_ids: NULL argument");
-    std::vector<uint32_t> all;
-    if (const MetaValue *v = meta(f, "tokenizer.ggml.eos_token_id"))
-        if (v->type == OXQ_GGUF_U32) all.push_back(uint32_t(v->bits));
-    if (const MetaValue *v = meta(f, "tokenizer.ggml.eos_token_ids"))
-        if (v->type == OXQ_GGUF_ARRAY && v->elem_type == OXQ_GGUF_U32)
-            for (uint64_t i = 0; i < v->elem_count; ++i) {
-                uint32_t id;
-                memcpy(&id, v->elems + 4 * i, 4);
-                if (std::find(all.begin(), all.end(), id) == all.end()) all.push_back(id);
-            }
-    *count = all.size();
-    for (uint64_t i = 0; i < all.size() && i < cap; ++i) ids[i] = all[i];
-    return OXQ_OK;
+    return guarded("oxq_gguf_eos_token_ids", [&]() -> int {
+        if (!f || !count || (!ids && cap)) return fail(OXQ_ERR_ARG, "oxq_gguf_eos_token_ids: NULL argument");
+        std::vector<uint32_t> all;
+        if (const MetaValue *v = meta(f, "tokenizer.ggml.eos_token_id"))
+            if (v->type == OXQ_GGUF_U32) all.push_back(uint32_t(v->bits));
+        if (const MetaValue *v = meta(f, "tokenizer.ggml.eos_token_ids"))
+            if (v->type == OXQ_GGUF_ARRAY && v->elem_type == OXQ_GGUF_U32)
+                for (uint64_t i = 0; i < v->elem_count; ++i) {
+                    uint32_t id;
+                    memcpy(&id, v->elems + 4 * i, 4);
+                    if (std::find(all.begin(), all.end(), id) == all.end()) all.push_back(id);
+                }
+        *count = all.size();
+        for (uint64_t i = 0; i < all.size() && i < cap; ++i) ids[i] = all[i];
+        return OXQ_OK;
+    });
 }
 
 int oxq_validate_quantization_config(const char *json, int whole_config, oxq_quant_scheme *out) {
-    const char *op = "oxq_validate_quantization_config";
-    if (!json || !out) return fail(OXQ_ERR_ARG, "%s: NULL argument", op);
-    out->kind = OXQ_SCHEME_NONE;
-    out->bits = 0;
-    out->sym = 0;
-    Json doc;
-    JsonParser jp(json, strlen(json));
-    if (!jp.document(doc)) return fail(OXQ_ERR_FORMAT, "%s: %s", op, jp.err.c_str());
-    const Json &v = whole_config ? doc.at("quantization_config") : doc;
-    if (v.is_null()) return OXQ_OK;
+    return guarded("oxq_validate_quantization_config", [&]() -> int {
+        const char *op = "oxq_validate_quantization_config";
+        if (!json || !out) return fail(OXQ_ERR_ARG, "%s: NULL argument", op);
+        out->kind = OXQ_SCHEME_NONE;
+        out->bits = 0;
+        out->sym = 0;
+        Json doc;
+        JsonParser jp(json, strlen(json));
+        if (!jp.document(doc)) return fail(OXQ_ERR_FORMAT, "%s: %s", op, jp.err.c_str());
+        const Json &v = whole_config ? doc.at("quantization_config") : doc;
+        if (v.is_null()) return OXQ_OK;
 
-    std::string method = v.at("quant_method").as_str("");
-    for (char &c : method) c = char(tolower((unsigned char)c));
-    const Json &bits = v.at("bits");
-    const char *version = v.at("version").as_str("gemm");
+        std::string method = v.at("quant_method").as_str("");
+        for (char &c : method) c = char(tolower((unsigned char)c));
+        const Json &bits = v.at("bits");
+        const char *version = v.at("version").as_str("gemm");
 
-    if (method == "awq") {
-        if (!bits.is_u64)
-            return fail(OXQ_ERR_UNSUPPORTED, "AWQ checkpoint missing required 'bits' field in quantization_config");
-        uint32_t b = uint32_t(bits.u64);
-        if (b != 4 && b != 8)
-            return fail(OXQ_ERR_UNSUPPORTED, "AWQ checkpoint bits=%u not supported. Only 4 and 8 bits are recognised.", b);
-        if (!ieq(version, "gemm"))
-            return fail(OXQ_ERR_UNSUPPORTED, "AWQ version '%s' is not supported (only 'gemm' has a runtime path).", version);
-        out->kind = OXQ_SCHEME_AWQ;
-        out->bits = b;
-        return OXQ_OK;
-    }
-    if (method == "fp8" || method == "mxfp4" || method.empty()) return OXQ_OK;
-    if (method == "gptq") {
-        if (!bits.is_u64)
-            return fail(OXQ_ERR_UNSUPPORTED, "GPTQ checkpoint missing required 'bits' field in quantization_config");
-        if (bits.u64 != 4 && bits.u64 != 8)
-            return fail(OXQ_ERR_UNSUPPORTED, "GPTQ checkpoint bits=%llu not supported. Only 4 and 8 bits are recognised.",
-                        (unsigned long long)bits.u64);
-        const Json &sym = v.at("sym"), &desc = v.at("desc_act");
-        bool s = sym.kind == Json::Bool ? sym.b : true;
-        bool d = desc.kind == Json::Bool ? desc.b : false;
-        if (d)
-            return fail(OXQ_ERR_UNSUPPORTED, "GPTQ checkpoint has desc_act=true (act-order). Only desc_act=false "
-                                             "(sequential g_idx) is supported.");
-        const char *fmt = v.at("checkpoint_format").as_str("gptq");
-        if (!ieq(fmt, "gptq"))
-            return fail(OXQ_ERR_UNSUPPORTED, "GPTQ checkpoint_format='%s' not supported (only the canonical 'gptq' format).",
-                        fmt);
-        out->kind = OXQ_SCHEME_GPTQ;
-        out->bits = uint32_t(bits.u64);
-        out->sym = s;
-        return OXQ_OK;
-    }
-    if (method == "compressed-tensors") {
-        const char *format = v.at("format").as_str("");
-        if (strcmp(format, "pack-quantized") != 0)
-            return fail(OXQ_ERR_UNSUPPORTED, "compressed-tensors format '%s' not supported (only 'pack-quantized')", format);
-        const Json &groups = v.at("config_groups");
-        size_t n_groups = 0;
-        if (groups.kind == Json::Object) {
-            // distinct keys (a JSON map keeps one value per key)
-            std::vector<const std::string *> seen;
-            for (const auto &kv : groups.obj) {
-                bool dup = false;
-                for (const std::string *s : seen) dup = dup || *s == kv.first;
-                if (!dup) seen.push_back(&kv.first);
-            }
-            n_groups = seen.size();
+        if (method == "awq") {
+            if (!bits.is_u64)
+                return fail(OXQ_ERR_UNSUPPORTED, "AWQ checkpoint missing required 'bits' field in quantization_config");
+            uint32_t b = uint32_t(bits.u64);
+            if (b != 4 && b != 8)
+                return fail(OXQ_ERR_UNSUPPORTED, "AWQ checkpoint bits=%u not supported. Only 4 and 8 bits are recognised.", b);
+            if (!ieq(version, "gemm"))
+                return fail(OXQ_ERR_UNSUPPORTED, "AWQ version '%s' is not supported (only 'gemm' has a runtime path).", version);
+            out->kind = OXQ_SCHEME_AWQ;
+            out->bits = b;
+            return OXQ_OK;
         }
-        const Json &w = groups.at("group_0").at("weights");
-        const Json &nb = w.at("num_bits"), &symm = w.at("symmetric");
-        uint64_t num_bits = nb.is_u64 ? nb.u64 : 0;
-        bool symmetric = symm.kind == Json::Bool ? symm.b : false;
-        const char *wtype = w.at("type").as_str("");
-        const char *strategy = w.at("strategy").as_str("");
-        bool actorder = w.at("actorder").kind == Json::String;
-        if (n_groups != 1 || num_bits != 4 || !symmetric || strcmp(wtype, "int") != 0 || strcmp(strategy, "group") != 0 ||
-            actorder)
-            return fail(OXQ_ERR_UNSUPPORTED,
-                        "compressed-tensors config not supported: requires a single group with int4 symmetric "
-                        "group-strategy weights, no actorder (got groups=%zu, bits=%llu, sym=%s, type='%s', strategy='%s', "
-                        "actorder=%s)",
-                        n_groups, (unsigned long long)num_bits, symmetric ? "true" : "false", wtype, strategy,
-                        actorder ? "set" : "none");
-        out->kind = OXQ_SCHEME_COMPRESSED_TENSORS4;
-        out->bits = 4;
-        out->sym = 1;
-        return OXQ_OK;
-    }
-    return fail(OXQ_ERR_UNSUPPORTED,
-                "Unknown quantization method '%s' in quantization_config. Supported: awq (gemm, 4/8-bit), gptq (4/8-bit, "
-                "desc_act=false), compressed-tensors (pack-quantized int4), fp8, mxfp4.",
-                method.c_str());
+        if (method == "fp8" || method == "mxfp4" || method.empty()) return OXQ_OK;
+        if (method == "gptq") {
+            if (!bits.is_u64)
+                return fail(OXQ_ERR_UNSUPPORTED, "GPTQ checkpoint missing required 'bits' field in quantization_config");
+            if (bits.u64 != 4 && bits.u64 != 8)
+                return fail(OXQ_ERR_UNSUPPORTED, "GPTQ checkpoint bits=%llu not supported. Only 4 and 8 bits are recognised.",
+                            (unsigned long long)bits.u64);
+            const Json &sym = v.at("sym"), &desc = v.at("desc_act");
+            bool s = sym.kind == Json::Bool ? sym.b : true;
+            bool d = desc.kind == Json::Bool ? desc.b : false;
+            if (d)
+                return fail(OXQ_ERR_UNSUPPORTED, "GPTQ checkpoint has desc_act=true (act-order). Only desc_act=false "
+                                                 "(sequential g_idx) is supported.");
+            const char *fmt = v.at("checkpoint_format").as_str("gptq");
+            if (!ieq(fmt, "gptq"))
+                return fail(OXQ_ERR_UNSUPPORTED, "GPTQ checkpoint_format='%s' not supported (only the canonical 'gptq' format).",
+                            fmt);
+            out->kind = OXQ_SCHEME_GPTQ;
+            out->bits = uint32_t(bits.u64);
+            out->sym = s;
+            return OXQ_OK;
+        }
+        if (method == "compressed-tensors") {
+            const char *format = v.at("format").as_str("");
+            if (strcmp(format, "pack-quantized") != 0)
+                return fail(OXQ_ERR_UNSUPPORTED, "compressed-tensors format '%s' not supported (only 'pack-quantized')", format);
+            const Json &groups = v.at("config_groups");
+            size_t n_groups = 0;
+            if (groups.kind == Json::Object) {
+                // distinct keys (a JSON map keeps one value per key)
+                std::vector<const std::string *> seen;
+                for (const auto &kv : groups.obj) {
+                    bool dup = false;
+                    for (const std::string *s : seen) dup = dup || *s == kv.first;
+                    if (!dup) seen.push_back(&kv.first);
+                }
+                n_groups = seen.size();
+            }
+            const Json &w = groups.at("group_0").at("weights");
+            const Json &nb = w.at("num_bits"), &symm = w.at("symmetric");
+            uint64_t num_bits = nb.is_u64 ? nb.u64 : 0;
+            bool symmetric = symm.kind == Json::Bool ? symm.b : false;
+            const char *wtype = w.at("type").as_str("");
+            const char *strategy = w.at("strategy").as_str("");
+            bool actorder = w.at("actorder").kind == Json::String;
+            if (n_groups != 1 || num_bits != 4 || !symmetric || strcmp(wtype, "int") != 0 || strcmp(strategy, "group") != 0 ||
+                actorder)
+                return fail(OXQ_ERR_UNSUPPORTED,
+                            "compressed-tensors config not supported: requires a single group with int4 symmetric "
+                            "group-strategy weights, no actorder (got groups=%zu, bits=%llu, sym=%s, type='%s', strategy='%s', "
+                            "actorder=%s)",
+                            n_groups, (unsigned long long)num_bits, symmetric ? "true" : "false", wtype, strategy,
+                            actorder ? "set" : "none");
+            out->kind = OXQ_SCHEME_COMPRESSED_TENSORS4;
+            out->bits = 4;
+            out->sym = 1;
+            return OXQ_OK;
+        }
+        return fail(OXQ_ERR_UNSUPPORTED,
+                    "Unknown quantization method '%s' in quantization_config. Supported: awq (gemm, 4/8-bit), gptq (4/8-bit, "
+                    "desc_act=false), compressed-tensors (pack-quantized int4), fp8, mxfp4.",
+                    method.c_str());
+    });
 }
 
 int oxq_safetensors_try_get_quant(const oxq_tensor_file *f, const oxq_quant_scheme *scheme, const char *prefix,
                                   oxq_file_tensor *qweight, oxq_file_tensor *qzeros, oxq_file_tensor *scales, int *found) {
-    if (!f || !scheme || !prefix || !qweight || !qzeros || !scales || !found)
-        return fail(OXQ_ERR_ARG, "oxq_safetensors_try_get_quant: NULL argument");
-    *found = 0;
-    memset(qweight, 0, sizeof *qweight);
-    memset(qzeros, 0, sizeof *qzeros);
-    memset(scales, 0, sizeof *scales);
-    std::string p(prefix);
-    const TensorEntry *w = nullptr, *z = nullptr, *s = nullptr;
-    switch (scheme->kind) {
-    case OXQ_SCHEME_NONE: return OXQ_OK;
-    case OXQ_SCHEME_AWQ:
-        w = resolve(f, p + ".qweight");
-        z = resolve(f, p + ".qzeros");
-        s = resolve(f, p + ".scales");
-        if (!w || !z || !s) return OXQ_OK;
-        break;
-    case OXQ_SCHEME_GPTQ:
-        w = resolve(f, p + ".qweight");
-        s = resolve(f, p + ".scales");
-        z = resolve(f, p + ".qzeros");
-        if (!w || !s) return OXQ_OK;
-        break;
-    case OXQ_SCHEME_COMPRESSED_TENSORS4:
-        w = resolve(f, p + ".weight_packed");
-        s = resolve(f, p + ".weight_scale");
-        if (!w || !s) return OXQ_OK;
-        break;
-    default: return fail(OXQ_ERR_ARG, "oxq_safetensors_try_get_quant: bad scheme kind %d", scheme->kind);
-    }
-    fill(*w, qweight);
-    fill(*s, scales);
-    if (z) fill(*z, qzeros);
-    *found = 1;
-    return OXQ_OK;
+    return guarded("oxq_safetensors_try_get_quant", [&]() -> int {
+        if (!f || !scheme || !prefix || !qweight || !qzeros || !scales || !found)
+            return fail(OXQ_ERR_ARG, "oxq_safetensors_try_get_quant: NULL argument");
+        *found = 0;
+        memset(qweight, 0, sizeof *qweight);
+        memset(qzeros, 0, sizeof *qzeros);
+        memset(scales, 0, sizeof *scales);
+        std::string p(prefix);
+        const TensorEntry *w = nullptr, *z = nullptr, *s = nullptr;
+        switch (scheme->kind) {
+        case OXQ_SCHEME_NONE: return OXQ_OK;
+        case OXQ_SCHEME_AWQ:
+            w = resolve(f, p + ".qweight");
+            z = resolve(f, p + ".qzeros");
+            s = resolve(f, p + ".scales");
+            if (!w || !z || !s) return OXQ_OK;
+            break;
+        case OXQ_SCHEME_GPTQ:
+            w = resolve(f, p + ".qweight");
+            s = resolve(f, p + ".scales");
+            z = resolve(f, p + ".qzeros");
+            if (!w || !s) return OXQ_OK;
+            break;
+        case OXQ_SCHEME_COMPRESSED_TENSORS4:
+            w = resolve(f, p + ".weight_packed");
+            s = resolve(f, p + ".weight_scale");
+            if (!w || !s) return OXQ_OK;
+            break;
+        default: return fail(OXQ_ERR_ARG, "oxq_safetensors_try_get_quant: bad scheme kind %d", scheme->kind);
+        }
+        fill(*w, qweight);
+        fill(*s, scales);
+        if (z) fill(*z, qzeros);
+        *found = 1;
+        return OXQ_OK;
+    });
 }
 
 int oxq_upload(oxq_ctx *ctx, void *stream, void *dst_device, const void *src_host, uint64_t nbytes) {
-    if (!ctx) return fail(OXQ_ERR_ARG, "oxq_upload: ctx is NULL");
-    if (ctx->plan_only) return fail(OXQ_ERR_DEVICE, "oxq_upload: a plan-only ctx has no device");
-    if (nbytes == 0) return OXQ_OK;
-    if (!dst_device || !src_host) return fail(OXQ_ERR_ARG, "oxq_upload: NULL pointer");
-    OXQ_HIP_CHECK(hipSetDevice(ctx->device));
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    OXQ_HIP_CHECK(hipMemcpyAsync(dst_device, src_host, size_t(nbytes), hipMemcpyHostToDevice, s));
-    // pageable source: the runtime stages it, but the mapping may be closed right after the call
-    OXQ_HIP_CHECK(hipStreamSynchronize(s));
-    return OXQ_OK;
+    return guarded("oxq_upload", [&]() -> int {
+        if (!ctx) return fail(OXQ_ERR_ARG, "oxq_upload: ctx is NULL");
+        if (ctx->plan_only) return fail(OXQ_ERR_DEVICE, "oxq_upload: a plan-only ctx has no device");
+        if (nbytes == 0) return OXQ_OK;
+        if (!dst_device || !src_host) return fail(OXQ_ERR_ARG, "oxq_upload: NULL pointer");
+        OXQ_HIP_CHECK(hipSetDevice(ctx->device));
+        hipStream_t s = static_cast<hipStream_t>(stream);
+        OXQ_HIP_CHECK(hipMemcpyAsync(dst_device, src_host, size_t(nbytes), hipMemcpyHostToDevice, s));
+        // pageable source: the runtime stages it, but the mapping may be closed right after the call
+        OXQ_HIP_CHECK(hipStreamSynchronize(s));
+        return OXQ_OK;
+    });
 }
 
 }  // extern "C"

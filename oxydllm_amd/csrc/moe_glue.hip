@@ -80,11 +80,21 @@ __device__ __forceinline__ void route_token(const T *__restrict__ l, int E, int 
         const float best = wave_all_reduce(bv, [](float a, float b) { return fmaxf(a, b); });
         bi = wave_all_reduce(bv == best ? bi : 0x7fffffff, [](int a, int b) { return a < b ? a : b; });
         bv = best;
+        if (bi >= E) {
+            // Nothing compared greater: the probabilities are NaN (a NaN or +inf logit makes the whole row
+            // NaN).  A stable sort leaves such a row in index order, so the slot takes the lowest index not
+            // taken yet and its (NaN) value: top_idx always stays inside [0, E).
+            int fi = 0x7fffffff;
+            for (int e = lane; e < E; e += 64)
+                if (!(probs[e] == -2.0f) && e < fi) fi = e;
+            bi = wave_all_reduce(fi, [](int a, int b) { return a < b ? a : b; });
+            bv = probs[bi < E ? bi : 0];
+        }
         if (lane == s) {  // slot s is kept by lane s
             my_val = bv;
             my_idx = bi;
         }
-        if (lane == 0) probs[bi] = -2.0f;  // taken
+        if (lane == 0 && bi < E) probs[bi] = -2.0f;  // taken
         chosen_sum += bv;  // slot order, as the reference's sum over the gathered values
     }
     out_idx = my_idx;

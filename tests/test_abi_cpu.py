@@ -6,6 +6,7 @@ metal_ops.rs:3943-3958) before anything would be launched.
 import ctypes as C
 import os
 import re
+import subprocess
 
 import numpy as np
 import pytest
@@ -600,3 +601,78 @@ def test_random_descriptors_never_crash_and_always_explain(lib, ctx):
         if rc == 0:
             call("oxq_mxfp4_linear_forward", h, None, B(ts[2]), B(ts[3])); lib.oxq_mxfp4_linear_free(h)
     assert names['oxq_w4a16_matmul'][0] > 0 and names['oxq_w4a16_matmul'][1] > 0
+
+
+# ------------------------------------------------------------------ the headers as a C99 consumer sees them
+def _c_declarations():
+    """(return type, name, [parameter declarations]) of every function include/*.h declares."""
+    import glob
+    text = "".join(open(h).read() for h in sorted(glob.glob(os.path.join(ROOT, "include", "*.h"))))
+    text = re.sub(r"/\*.*?\*/", " ", text, flags=re.S)
+    out = []
+    for m in re.finditer(r"^(int|int64_t|uint64_t|void|const char \*)\s*(oxq_[a-z0-9_]+)\s*\(([^;{]*)\)\s*;", text, re.M):
+        params = [p.strip() for p in re.sub(r"\s+", " ", m.group(3)).split(",")]
+        out.append((m.group(1).strip(), m.group(2), [] if params == ["void"] else params))
+    return out
+
+
+def _c_argument(param: str) -> str:
+    ptype = re.sub(r"\b[a-z_0-9]+$", "", param).strip()  # drop the parameter name
+    if ptype in ("oxq_ctx *", "const oxq_ctx *"):
+        return "ctx"
+    if ptype == "const oxq_tensor *":
+        return "&t"
+    if ptype == "const char *":
+        return '"x"'
+    if "*" in ptype:
+        return "NULL"
+    if ptype == "float":
+        return "1.0f"
+    return "1"
+
+
+def test_headers_compile_as_c99_and_every_entry_point_answers(tmp_path):
+    """A C99 translation unit (gcc -std=c99 -pedantic -Wall -Wextra -Werror) includes both headers and calls
+    every declared function on a plan-only ctx with a small valid descriptor or NULL per parameter: the
+    headers are plain C (what bindgen or a hand-written `extern "C"` block needs), every symbol links, and
+    no entry point crashes on arguments it must refuse."""
+    decls = _c_declarations()
+    assert len(decls) >= 70 and {d[1] for d in decls} == set(_lib.SIGNATURES)
+    lines = ['#include <stdio.h>', '#include <string.h>', '#include "oxq.h"', '#include "oxq_files.h"', '',
+             'int main(void) {', '    oxq_ctx *ctx = NULL;', '    oxq_tensor t;', '    oxq_plan plan;', '    int calls = 0;',
+             '    memset(&t, 0, sizeof t);', '    t.dtype = OXQ_F16; t.rank = 2; t.dims[0] = 1; t.dims[1] = 256; t.contiguous = 1;',
+             '    if (oxq_ctx_create(OXQ_DEVICE_PLAN_ONLY, &ctx) != OXQ_OK || !ctx) return 2;']
+    skip = {"oxq_ctx_create", "oxq_ctx_destroy"}
+    for ret, name, params in decls:
+        if name in skip:
+            continue
+        args = ", ".join(_c_argument(p) for p in params)
+        lines.append(f"    (void){name}({args}); ++calls;")
+    lines += [
+        '    {   /* one call that must succeed: the plan of a 4-bit AWQ GEMV */',
+        '        oxq_tensor x = t, qw = t, qz = t, sc = t, y = t;',
+        '        x.dims[1] = 4096;',
+        '        qw.dtype = OXQ_I32; qw.dims[0] = 4096; qw.dims[1] = 512;',
+        '        qz.dtype = OXQ_I32; qz.dims[0] = 32; qz.dims[1] = 512;',
+        '        sc.dims[0] = 32; sc.dims[1] = 4096;',
+        '        y.dims[1] = 4096;',
+        '        if (oxq_w4a16_matmul(ctx, NULL, &x, &qw, &qz, &sc, &y) != OXQ_OK) { printf("%s\\n", oxq_last_error()); return 3; }',
+        '        if (oxq_ctx_last_plan(ctx, &plan) != OXQ_OK || plan.kernel[0] == 0 || plan.launches < 1) return 4;',
+        '        if (oxq_w4a16_matmul_static(ctx, NULL, &x, &qw, &qz, &sc, &y) != OXQ_OK) return 5;',
+        '        x.dtype = OXQ_F32;',
+        '        if (oxq_w4a16_matmul(ctx, NULL, &x, &qw, &qz, &sc, &y) != OXQ_ERR_DTYPE) return 6;',
+        '    }',
+        '    if (oxq_ctx_destroy(ctx) != OXQ_OK) return 7;',
+        '    printf("%d calls, last kernel %s\\n", calls, plan.kernel);',
+        '    return 0;', '}', '']
+    src = tmp_path / "abi_c99.c"
+    src.write_text("\n".join(lines))
+    exe = tmp_path / "abi_c99"
+    libdir = os.path.dirname(_lib.LIB_PATH)
+    cc = subprocess.run(["gcc", "-std=c99", "-pedantic", "-Wall", "-Wextra", "-Werror", f"-I{os.path.join(ROOT, 'include')}",
+                         str(src), "-o", str(exe), f"-L{libdir}", "-loxq_hip", f"-Wl,-rpath,{libdir}",
+                         "-Wl,-rpath,/opt/rocm/lib"], capture_output=True, text=True)
+    assert cc.returncode == 0, cc.stderr
+    run = subprocess.run([str(exe)], capture_output=True, text=True, timeout=120)
+    assert run.returncode == 0, (run.returncode, run.stdout, run.stderr)
+    assert f"{len(decls) - len(skip)} calls" in run.stdout and "awq4" in run.stdout, run.stdout

@@ -163,6 +163,19 @@ def test_gguf_rejects_malformed_files(tmp_path):
     i = data.index(b"k") + 1
     data[i:i + 4] = struct.pack("<I", 13)
     expect(bytes(data), -13, "unknown value type 13")
+    # Byte counts that wrap 64 bits: one F32 tensor of 2^62 elements (2^62 * 4 = 0 mod 2^64) and one of
+    # 2^31 x 2^31.  Without a check the slice has "0 bytes", lies inside the map and carries dims that do
+    # not match it; a caller that sizes a read from the dims would run past the mapping.
+    for dims in ((1 << 62,), (1 << 31, 1 << 31)):
+        G.write_gguf(path, [], [("w", dims, 0, b"\0" * 32)])
+        with pytest.raises(OxqError) as e:
+            ck.GgufWeights.load(path)
+        assert _status(e) == -13 and "overflows" in e.value.message, e.value.message
+    # more tensor / metadata records than the file has bytes for: refused before anything is reserved
+    G.write_gguf(path, [], [])
+    data = bytearray(open(path, "rb").read())
+    data[8:16] = struct.pack("<Q", 1 << 40)
+    expect(bytes(data), -13, "cannot fit")
     with pytest.raises(OxqError) as e:
         ck.GgufWeights.load(str(tmp_path / "nope.gguf"))
     assert _status(e) == -12

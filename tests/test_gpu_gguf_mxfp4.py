@@ -410,6 +410,35 @@ def test_moe_route_ties_keep_expert_order():
     np.testing.assert_array_equal(ridx[0], [0, 1, 2, 3])
 
 
+@pytest.mark.parametrize("E,k", [(32, 4), (200, 6)])
+def test_moe_route_rows_without_an_order_stay_in_range(E, k):
+    """A NaN or +inf logit makes every probability of its row NaN.  A stable sort leaves such a row in index
+    order (the oracle, like arg_sort_last_dim, then returns experts 0..k-1 with NaN weights); the device must
+    do the same: ids inside [0, E), so that grouping still places every pair."""
+    say(f"moe route NaN rows E={E} k={k}")
+    rng = np.random.default_rng(E)
+    logits = rng.standard_normal((6, E)).astype(np.float32)
+    logits[1, E // 2] = np.nan
+    logits[3, 0] = np.nan
+    logits[4, E - 1] = np.inf
+    ridx, rvals = oracle.moe_route(logits, k, True)
+    for r in (1, 3, 4):
+        np.testing.assert_array_equal(ridx[r], np.arange(k))
+        assert np.isnan(rvals[r]).all()
+    for fn in (lambda: ops.moe_route(to_dev(logits), k, True), lambda: ops.moe_route_group(to_dev(logits), k, True)[:2]):
+        idx, vals = fn()
+        idx, vals = idx.cpu().numpy(), vals.cpu().numpy()
+        np.testing.assert_array_equal(idx.astype(np.uint32), ridx)
+        np.testing.assert_array_equal(np.isnan(vals), np.isnan(rvals))
+        ok = ~np.isnan(rvals)
+        np.testing.assert_allclose(vals[ok], rvals[ok], rtol=1e-5, atol=1e-7)
+    _, _, off, tok, _, pos = ops.moe_route_group(to_dev(logits), k, True)
+    roff, rtok, _ = oracle.moe_group(ridx, rvals, E)
+    np.testing.assert_array_equal(off.cpu().numpy(), roff.astype(np.int32))
+    np.testing.assert_array_equal(tok.cpu().numpy(), rtok.astype(np.int32))
+    assert sorted(pos.cpu().numpy().ravel().tolist()) == list(range(6 * k))
+
+
 @pytest.mark.parametrize("T,E,k", [(8, 32, 4), (1, 32, 4), (16, 64, 4), (5, 200, 3), (13, 256, 5), (257, 16, 2),
                                    (1000, 256, 8)])
 def test_moe_group_matches_oracle(T, E, k):

@@ -423,3 +423,48 @@ def test_stateless_tile_op_on_layouts_without_a_tile_kernel(method, bits, dtn, m
     xa = rng.standard_normal((32, 2048)).astype(np.float32)
     ya = ops.mpp_quant_matmul(to_dev(xa, TORCH_DT[dt]), *ad, 4, ops.PACK_OUT)
     assert_close(ya, oracle.matmul_nt_f32(round_x(xa, dt), oracle.round_through(wa, dt)), "awq4 after a repacked call")
+
+
+# ------------------------------------------------------------------ split-K: fused sum against the second launch
+@pytest.mark.parametrize("route", ["awq4", "awq8", "gptq4", "gptq8", "awq4_generic", "gptq4_generic"])
+@pytest.mark.parametrize("dtn", ["f16", "bf16"])
+def test_splitk_fused_and_two_launch_sums_give_the_same_bits(route, dtn, monkeypatch):
+    """The K slices' partial sums are added in slice order either by the last workgroup to arrive (mode 1,
+    relaxed device-scope accesses and an arrival counter) or by a second launch (mode 2, plain stores and a
+    kernel boundary).  Both must give the same bits on every GEMV route, for every row count."""
+    dt = DT[dtn]
+    bits = 8 if route.endswith("8") else 4
+    gptq = route.startswith("gptq")
+    generic = route.endswith("generic")
+    K, N, g = (2048, 1024, 128) if not generic else (1024, 328, 32)
+    qw, qz, sc = (synth.gptq_checkpoint if gptq else synth.awq_checkpoint)(K, N, g, bits, seed=77)
+    d = dev_triplet(qw, qz, sc, dt)
+    ctxs = {}
+    for mode in (1, 2):
+        monkeypatch.setenv("OXQ_SPLITK_MODE", str(mode))
+        ctxs[mode] = ops.Context()
+    monkeypatch.delenv("OXQ_SPLITK_MODE")
+    for m in (1, 3, 8):
+        if m > 1 and dtn == "f16" and bits == 4 and not gptq:
+            continue  # f16 batches on 4-bit AWQ run the tile kernel, which always sums with the second launch
+        say(f"split-K modes {route} {dtn} m={m}")
+        x = np.random.default_rng(m).standard_normal((m, K)).astype(np.float32)
+        xd = to_dev(x, TORCH_DT[dt])
+        outs, plans = {}, {}
+        for mode in (1, 2):
+            if gptq:
+                outs[mode] = ops.gptq_matmul(xd, *d, bits, ctx=ctxs[mode])
+            elif bits == 8:
+                outs[mode] = ops.w8a16_matmul(xd, *d, ctx=ctxs[mode])
+            else:
+                outs[mode] = ops.w4a16_matmul(xd, *d, ctx=ctxs[mode])
+            plans[mode] = ctxs[mode].last_plan()
+        torch.cuda.synchronize()
+        assert plans[1]["kernel"] == plans[2]["kernel"] and plans[1]["split_k"] == plans[2]["split_k"] > 1, plans
+        assert ("generic" in plans[1]["kernel"]) == generic, plans[1]
+        assert plans[1]["launches"] == 1 and plans[2]["launches"] == 2, plans
+        assert np.array_equal(bits_of(outs[1]), bits_of(outs[2])), f"{route} {dtn} m={m}: fused and two-launch sums differ"
+        ref = (gptq_ref(qw, qz, sc, x, dt, bits) if gptq else awq_ref(qw, qz, sc, x, dt, bits))[0]
+        assert_close(outs[1], ref, f"split-K {route} {dtn} m={m}")
+    for c in ctxs.values():
+        c.close()

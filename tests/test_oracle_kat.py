@@ -668,6 +668,18 @@ def test_linear_from_awq_matches_dense():
     np.testing.assert_allclose(oracle.matmul_nt_f32(x, w, bias), want, rtol=1e-5, atol=1e-5)
 
 
+def test_moe_route_nan_row_keeps_index_order():
+    """A row whose probabilities are all NaN has no order: numpy's stable argsort, like the oracle's stable
+    insertion sort, leaves it as it is, so the chosen experts are 0..k-1 (in range) with NaN weights."""
+    logits = np.random.default_rng(3).standard_normal((3, 16)).astype(np.float32)
+    logits[1, 7] = np.nan
+    idx, vals = oracle.moe_route(logits, 4, True)
+    np.testing.assert_array_equal(idx[1], [0, 1, 2, 3])
+    assert np.isnan(vals[1]).all() and not np.isnan(vals[[0, 2]]).any()
+    offsets, tokens, _ = oracle.moe_group(idx, vals, 16)
+    assert offsets[-1] == 12 and sorted(tokens.tolist()) == sorted([0, 1, 2] * 4)
+
+
 def test_moe_route_matches_numpy():
     rng = np.random.default_rng(7)
     logits = rng.standard_normal((8, 32)).astype(np.float32)
