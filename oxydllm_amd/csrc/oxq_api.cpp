@@ -1340,7 +1340,7 @@ static int prepack_layer(oxq_packed_quant_linear *l) {
     OXQ_HIP_CHECK(hipSetDevice(ctx->device));
     int rc = OXQ_OK;
     hipError_t e = hipMalloc((void **)&l->pk.pw, pk4_weight_bytes(src.K, src.N, src.bits));
-    if (e == hipSuccess) e = hipMalloc((void **)&l->pk.pzs, pk4_zs_bytes(src.K, src.N, src.group_shift));
+    l->pk.pzs = nullptr;  // the zero/scale pairs live inside the blocks of pw
     if (e != hipSuccess) {
         rc = fail(OXQ_ERR_RUNTIME, "PackedQuantLinear: repack allocation failed: %s", hipGetErrorString(e));
     } else {

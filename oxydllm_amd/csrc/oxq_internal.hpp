@@ -147,8 +147,8 @@ struct F8Problem {
 
 // A resident 4- or 8-bit layer repacked tile-major at load (layout: pk4.hip).
 struct Pk4Weights {
-    uint32_t *pw;           // [N/64][K/32][bits/4][64][4]
-    uint32_t *pzs;          // [N/64][K/g][16][4]  {-(bias + z), s} pairs of the layer dtype
+    uint32_t *pw;           // [N/64][K/128]{[4][bits/4][64][4] weights, [16][4] {-(bias + z), s} pairs}
+    uint32_t *pzs;          // unused (the pairs live inside the blocks of pw); kept null
     int64_t K, N;
     int group_shift;
     int dtype;              // OXQ_F16 / OXQ_BF16

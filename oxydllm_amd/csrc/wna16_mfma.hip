@@ -703,16 +703,14 @@ int launch_wna16_mfma(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p) {
                                   : launch_awq4_mfma<BF16Traits>(ctx, s, p);
     // Layouts without a tile kernel of their own on the checkpoint layout (GPTQ, 8-bit AWQ): when the
     // tile-major copy fits the ctx workspace, build it there and run the resident-layer kernel on it.
-    // Two launches more (about 45 us at 5120 x 13824, 4-bit) instead of one GEMV pass over the weights
+    // One launch more (about 45 us at 5120 x 13824, 4-bit) instead of one GEMV pass over the weights
     // per 8 rows (35 - 45 us each): ahead from m = 9.  A caller that holds the layer should hold a
     // PackedQuantLinear, which repacks once.
     if (p.M > 8 && pk4_eligible(p) && !ctx->plan_only && env_int("OXQ_TRANSIENT_REPACK", 1) &&
         !env_int("OXQ_FORCE_GENERIC", 0)) {
         const size_t wb = (pk4_weight_bytes(p.K, p.N, p.bits) + 255) & ~(size_t)255;
-        const size_t zb = pk4_zs_bytes(p.K, p.N, p.group_shift);
-        if (wb + zb <= ctx->workspace_bytes) {
-            Pk4Weights w{(uint32_t *)ctx->workspace, (uint32_t *)((uint8_t *)ctx->workspace + wb), p.K, p.N,
-                         p.group_shift, p.dtype, p.bits, 0};
+        if (wb <= ctx->workspace_bytes) {
+            Pk4Weights w{(uint32_t *)ctx->workspace, nullptr, p.K, p.N, p.group_shift, p.dtype, p.bits, 0};
             int rc = launch_pk4_prepack(ctx, s, p, w);
             if (rc != OXQ_OK) return rc;
             Pk4Problem q;
@@ -724,7 +722,7 @@ int launch_wna16_mfma(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p) {
             q.no_split = 1;
             q.w = w;
             rc = launch_pk4_forward(ctx, s, q);
-            ctx->plan.launches = 3;
+            ctx->plan.launches = 2;
             return rc;
         }
     }

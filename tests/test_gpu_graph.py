@@ -132,7 +132,7 @@ def test_fused_epilogues_and_workspace_repack_in_a_graph():
                 fn = lambda: ops.mpp_quant_matmul(x, *d, bits, ops.PACK_IN, out=y)
             replay_matches_eager(f"gptq{bits} m={m}", fn, inputs, y)
             if m > 8:
-                assert ops.default_context().last_plan()["launches"] == 3
+                assert ops.default_context().last_plan()["launches"] == 2
 
     E, N, Kx = 3, 64, 96
     blocks = torch.from_numpy(np.concatenate([synth.mxfp4_weight(N, Kx, seed=e)[0] for e in range(E)])).cuda()

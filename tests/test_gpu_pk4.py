@@ -145,7 +145,7 @@ def test_repacked_forward_k_slices(kind, dtn, K, N, g, ks, monkeypatch):
     assert layer.prepacked
     w = dense(kind, trip, dt)
     rng = np.random.default_rng(K + ks)
-    groups = K // g
+    groups = K // 128  # slices are cut in blocks of 128 rows of K
     per = -(-groups // min(ks, groups))
     for m in (1, 7, 16, 40, 64, 100):
         say(f"pk4 k-slices {kind} {dtn} K={K} N={N} g={g} ks={ks} m={m}")
