@@ -394,15 +394,29 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
     const __amdgpu_buffer_rsrc_t rs_w = make_rsrc(pw + (size_t)j * NB * (BB / 4), (uint32_t)NB * (uint32_t)BB);
     const __amdgpu_buffer_rsrc_t rs_x = make_rsrc(x, (uint32_t)M * (uint32_t)K * 2u);
     const int voff_w = lane * 16;
-    const int voff_z = 1024 * WL * 4 + ni * 16;  // the block's zero/scale pairs of this lane's four columns
-    // activation load q of a block: row 4q + lane/16, 16-byte chunk lane%16 of the row's 256 bytes
-    int voff_a[AQ], a_wr[AQ];
+    // The block's zero/scale pairs: lane (ni, kb) fetches word kb of column quad ni (one 4-byte load a lane,
+    // 256 contiguous bytes a wave: a quarter of what a 16-byte load costs the address unit, which is the
+    // busiest unit from 32 rows on) and the four lane groups then exchange their words (zs_words).
+    const int voff_z = 1024 * WL * 4 + (ni * 4 + kb) * 4;
+    // activation load q of a block: row 4q + lane/16, 16-byte chunk lane%16 of the row's 256 bytes; rows
+    // past M get an offset beyond any buffer, for which the buffer unit returns zeros without touching
+    // memory (the scalar offset of a buffer load is not part of its bounds check, so the lane offset
+    // has to carry the row)
+    // Up to two row tiles every load keeps its own offset register; the larger kernels are at their
+    // register budget and derives them from the first one (a row past M then lies beyond the end of x by
+    // its lane offset alone, which the bounds check does cover).
+    constexpr bool VA1 = MT >= 3;
+    int voff_a[VA1 ? 1 : AQ];
 #pragma unroll
-    for (int q = 0; q < AQ; ++q) {
-        const int row = 4 * q + kb, r = m0 + row;
+    for (int q = 0; q < (VA1 ? 1 : AQ); ++q) {
+        const int r = m0 + 4 * q + kb;
         voff_a[q] = r < M ? (r * K * 2 + ni * 16) : OOB;
-        a_wr[q] = row * 256 + ((ni ^ (row & 15)) << 4);  // = kb*256 + ((ni^kb)<<4), xor (4q&15)<<4, + 1024q
     }
+    uint32_t rowstep = 4u * (uint32_t)K * 2u;
+    // LDS position of (row = 4q + kb, chunk ni): chunk index XORed with row % 16 = kb | (q % 4) << 2
+    int a_wr[4];
+#pragma unroll
+    for (int qq = 0; qq < 4; ++qq) a_wr[qq] = kb * 256 + (((ni ^ kb) ^ (qq << 2)) << 4);  // + 1024 q
     // fragment read of step s (0..3), row tile mt: row 16mt + ni, chunk 8*(s/2) + 2kb + (s%2)
     int a_rd[4];
 #pragma unroll
@@ -416,7 +430,8 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
     }
 
     static_assert(WD == 4, "the ring holds exactly one block");
-    u32x4_t aring[AQ], wring[WD][WL], zring;
+    u32x4_t aring[AQ], wring[WD][WL];
+    uint32_t zring;
     // Past the end of the wave's share the loads go through an empty descriptor: a scalar select,
     // no vector instruction, and the buffer unit returns zero without touching memory.
     const __amdgpu_buffer_rsrc_t rs_none = make_rsrc(pw, 0u);
@@ -424,7 +439,15 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
         const __amdgpu_buffer_rsrc_t rs = i < nloc ? rs_x : rs_none;  // wave-uniform
         const int blk = blk_of(i);
 #pragma unroll
-        for (int q = 0; q < AQ; ++q) a[q] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff_a[q], blk * 256, 0);
+        for (int q = 0; q < AQ; ++q) {
+            if (VA1) {
+                if (q == 0) asm volatile("" : "+s"(rowstep));  // recomputed per block: 15 registers less to hold
+                const uint32_t v = (uint32_t)voff_a[0] + (uint32_t)q * rowstep;
+                a[q] = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)(v < (uint32_t)voff_a[0] ? (uint32_t)OOB : v), blk * 256, 0);
+            } else {
+                a[q] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff_a[q], blk * 256, 0);
+            }
+        }
     };
     auto load_w = [&](int i, int st, u32x4_t (&w)[WL]) {
         const __amdgpu_buffer_rsrc_t rs = i < nloc ? rs_w : rs_none;
@@ -434,11 +457,21 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
     };
     auto load_z = [&](int i) {
         const __amdgpu_buffer_rsrc_t rs = i < nloc ? rs_w : rs_none;
-        zring = __builtin_amdgcn_raw_buffer_load_b128(rs, voff_z, blk_of(i) * BB, WNT);
+        zring = __builtin_amdgcn_raw_buffer_load_b32(rs, voff_z, blk_of(i) * BB, WNT);
+    };
+    // zv[f] = the word that lane group f fetched, in every lane group: the lane-swap instructions
+    // exchange 16-lane rows between two registers (odd rows of one with even rows of the other, then
+    // the upper half of one with the lower half of the other).
+    auto zs_words = [&](uint32_t z, uint32_t (&zv)[4]) {
+        const auto p16 = __builtin_amdgcn_permlane16_swap(z, z, false, false);  // {r0 r0 r2 r2}, {r1 r1 r3 r3}
+        const uint32_t even = p16[0], odd = p16[1];
+        const auto pe = __builtin_amdgcn_permlane32_swap(even, even, false, false);  // {r0 x4}, {r2 x4}
+        const auto po = __builtin_amdgcn_permlane32_swap(odd, odd, false, false);    // {r1 x4}, {r3 x4}
+        zv[0] = pe[0], zv[2] = pe[1], zv[1] = po[0], zv[3] = po[1];
     };
     auto store_a = [&](const u32x4_t (&a)[AQ]) {
 #pragma unroll
-        for (int q = 0; q < AQ; ++q) *(u32x4_t *)(slot + a_wr[q]) = a[q];
+        for (int q = 0; q < AQ; ++q) *(u32x4_t *)(slot + q * 1024 + a_wr[q & 3]) = a[q];
     };
 
     // issue order = consumption order.  The tile form needs the pairs before its first B fragment,
@@ -465,8 +498,8 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
     for (int i = 0; i < nloc; ++i) {
         float4_t tmp[GS ? MT : 1][4], tmps[GS ? MT : 1];  // per-block integer sums of the GS form
         if (!GS) {
-            const uint32_t z0 = zring[0], z1 = zring[1], z2 = zring[2], z3 = zring[3];
-            const uint32_t zv[4] = {z0, z1, z2, z3};
+            uint32_t zv[4];
+            zs_words(zring, zv);
 #pragma unroll
             for (int f = 0; f < 4; ++f) Pk4T<TT>::prep(zv[f], negzb[f], sp[f]);
             load_z(i + 1);
@@ -521,8 +554,8 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
             }
         }
         if (GS) {  // fold the block in: y += s * (sum - (bias + z) * rowsum), all f32
-            const uint32_t z0 = zring[0], z1 = zring[1], z2 = zring[2], z3 = zring[3];
-            const uint32_t zv[4] = {z0, z1, z2, z3};
+            uint32_t zv[4];
+            zs_words(zring, zv);
             load_z(i + 1);
 #pragma unroll
             for (int f = 0; f < 4; ++f) {
@@ -618,7 +651,7 @@ static int pk4_go4(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, 
     OXQ_HIP_CHECK(lds_grant.ensure((const void *)pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ>, lds));
     hipLaunchKernelGGL((pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ>), grid, dim3(512), lds, s, (const uint16_t *)p.x,
                        p.w.pw, (const uint16_t *)p.bias, (uint16_t *)p.y, (float *)ctx->workspace, (int)p.M,
-                       (int)p.w.K, (int)p.w.N, bslice, pk4_env("OXQ_PK4_CONTIGUOUS", 0), p.act);
+                       (int)p.w.K, (int)p.w.N, bslice, pk4_env("OXQ_PK4_CONTIGUOUS", 1), p.act);
     OXQ_HIP_CHECK(hipGetLastError());
     return OXQ_OK;
 }
