@@ -308,6 +308,33 @@ int oxq_mxfp4_moe_gate_up_swiglu(oxq_ctx *ctx, void *stream, const oxq_tensor *x
                                  const oxq_tensor *expert_offsets, const oxq_tensor *token_ids, int gather_rows,
                                  int64_t k, int64_t n, float limit, const oxq_tensor *out, int *fused);
 
+/* ---- resident MXFP4 experts ---------------------------------------------------
+ * moe.rs:366-417 (load_gpt_oss keeps the stacked tensors of a projection, [E, n, k/32, 16] blocks and
+ * [E, n, k/32] scales, for the life of the model) and moe.rs:563-607 (dispatch_sparse runs them).
+ * `new` is the load-time step: when n is a multiple of 16 it builds a tile-major copy in device memory
+ * owned by the handle (matrix-core operand order, one contiguous run per 16 rows; the checkpoint tensors'
+ * size plus at most one block in four per row) and synchronises the null stream once; decode sizes then
+ * stream that copy.  The caller's tensors are borrowed and must outlive the handle: many pairs per expert
+ * (n_pairs >= 8 * n_experts) and shapes that do not qualify run on them, with the stateless ops' kernels.
+ * OXQ_PREPACK=0 in the environment disables the copy. */
+typedef struct oxq_mxfp4_experts oxq_mxfp4_experts;
+int oxq_mxfp4_experts_new(oxq_ctx *ctx, const oxq_tensor *blocks, const oxq_tensor *scales,
+                          const oxq_tensor *bias_or_null, int64_t n_experts, int64_t k, int64_t n,
+                          oxq_mxfp4_experts **out);
+/* Arguments and result of oxq_mxfp4_moe_matmul without the weight tensors. */
+int oxq_mxfp4_experts_matmul(oxq_mxfp4_experts *experts, void *stream, const oxq_tensor *x,
+                             const oxq_tensor *expert_offsets, const oxq_tensor *token_ids, int gather_rows,
+                             const oxq_tensor *out);
+/* Arguments and result of oxq_mxfp4_moe_gate_up_swiglu without the weight tensors. */
+int oxq_mxfp4_experts_gate_up_swiglu(oxq_mxfp4_experts *experts, void *stream, const oxq_tensor *x,
+                                     const oxq_tensor *expert_offsets, const oxq_tensor *token_ids,
+                                     int gather_rows, float limit, const oxq_tensor *out, int *fused);
+/* *resident = 1 if decode sizes run on the handle's own tile-major copy. */
+int oxq_mxfp4_experts_is_resident(const oxq_mxfp4_experts *experts, int *resident);
+/* Dense dequant [n, k] F32 of one expert, read back from what the GEMV streams (the copy, if there is one). */
+int oxq_mxfp4_experts_dequantize(oxq_mxfp4_experts *experts, void *stream, int64_t expert, const oxq_tensor *out);
+void oxq_mxfp4_experts_free(oxq_mxfp4_experts *experts);
+
 /* ---- mixture-of-experts glue: the steps either side of the expert GEMVs -----
  * The reference does these on the host / with one launch per expert
  * (moe.rs:466-607); here they run on the device and feed oxq_mxfp4_moe_matmul. */

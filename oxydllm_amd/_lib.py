@@ -106,6 +106,12 @@ SIGNATURES = {
                                        C.c_int64, C.c_int64, _TP]),
     "oxq_mxfp4_moe_gate_up_swiglu": (C.c_int, [_VP, _VP, _TP, _TP, _TP, _TP, _TP, _TP, C.c_int,
                                               C.c_int64, C.c_int64, C.c_float, _TP, C.POINTER(C.c_int)]),
+    "oxq_mxfp4_experts_new": (C.c_int, [_VP, _TP, _TP, _TP, C.c_int64, C.c_int64, C.c_int64, C.POINTER(_VP)]),
+    "oxq_mxfp4_experts_matmul": (C.c_int, [_VP, _VP, _TP, _TP, _TP, C.c_int, _TP]),
+    "oxq_mxfp4_experts_gate_up_swiglu": (C.c_int, [_VP, _VP, _TP, _TP, _TP, C.c_int, C.c_float, _TP, C.POINTER(C.c_int)]),
+    "oxq_mxfp4_experts_is_resident": (C.c_int, [_VP, C.POINTER(C.c_int)]),
+    "oxq_mxfp4_experts_dequantize": (C.c_int, [_VP, _VP, C.c_int64, _TP]),
+    "oxq_mxfp4_experts_free": (None, [_VP]),
     "oxq_moe_route": (C.c_int, [_VP, _VP, _TP, C.c_int64, C.c_int, _TP, _TP]),
     "oxq_moe_group": (C.c_int, [_VP, _VP, _TP, _TP, C.c_int64, _TP, _TP, _TP, _TP]),
     "oxq_moe_route_group": (C.c_int, [_VP, _VP, _TP, C.c_int64, C.c_int, _TP, _TP, _TP, _TP, _TP, _TP]),

@@ -453,6 +453,237 @@ __global__ __launch_bounds__(256) void mxfp4_dequant_kernel(const uint8_t *__res
     for (int i = 0; i < 32; ++i) o[i] = w[i];
 }
 
+// ---------------------------------------------------------------------------
+// Resident experts (moe.rs:366-417 keeps the stacked expert tensors of a projection for the life of
+// the model): a tile-major copy built once at load, read by the decode GEMV below.
+//
+// In the checkpoint layout the 16 weight rows a wave feeds the matrix cores with are 16 runs of
+// K/2 bytes, and a wave load is sixteen 64-byte pieces, most of them split over two cache lines.
+// The copy stores, per expert and tile of 16 rows, chunks of 1 KB in operand order:
+//
+//   pw [E][N/16 tiles][NC chunks][64 lanes][16 bytes]     NC = ceil(K/32 / 4)
+//   ps [E][N/16 tiles][ceil(NC/4)][64 lanes][4 bytes]     the E8M0 bytes, byte c % 4 = chunk c
+//
+// Chunk c, lane (ni = lane % 16, kb = lane / 16) holds block 4c + kb of row 16 tile + ni (blocks past
+// the row are zero weights with scale 1).  A wave's weights are one contiguous run read front to back
+// with 1 KB loads - nontemporal, nothing is read twice - and land in matrix-core operand order: no
+// lane transpose, no scale staging.  The four 4-byte words of a lane's block serve four MFMA steps.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void mxfp4_repack_kernel(const uint8_t *__restrict__ blocks,
+                                                           const uint8_t *__restrict__ scales,
+                                                           u32x4_t *__restrict__ pw, uint8_t *__restrict__ ps,
+                                                           int E, int N, int nb, int NC, int NG) {
+    // one thread per (expert, tile, chunk, lane)
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const int ntiles = N >> 4;
+    if (idx >= (size_t)E * ntiles * NC * 64) return;
+    const int lane = (int)(idx & 63);
+    const int c = (int)((idx >> 6) % NC);
+    const size_t et = (idx >> 6) / NC;  // expert * ntiles + tile
+    const int ni = lane & 15, kb = lane >> 4;
+    const int b = 4 * c + kb;
+    const size_t row = et * 16 + ni;  // = expert * N + 16 tile + ni
+    const bool valid = b < nb;
+    pw[idx] = valid ? ((const u32x4_t *)blocks)[row * nb + b] : u32x4_t{0u, 0u, 0u, 0u};
+    ps[((et * NG + (c >> 2)) * 64 + lane) * 4 + (c & 3)] = valid ? scales[row * nb + b] : (uint8_t)127;
+    // the tail of the last scale word (chunks past NC) is never read as a scale of a real block; keep it defined
+    if (c == NC - 1)
+        for (int cc = (c & 3) + 1; cc < 4; ++cc) ps[((et * NG + (c >> 2)) * 64 + lane) * 4 + cc] = 127;
+}
+
+// dense [N, K] f32 of one expert, from the resident copy (pins the repack bit for bit)
+__global__ __launch_bounds__(256) void mxfp4_res_dequant_kernel(const u32x4_t *__restrict__ pw,
+                                                                const uint8_t *__restrict__ ps,
+                                                                float *__restrict__ out, int N, int nb, int NC,
+                                                                int NG) {
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;  // (tile, chunk, lane) of this expert
+    const int ntiles = N >> 4;
+    if (idx >= (size_t)ntiles * NC * 64) return;
+    const int lane = (int)(idx & 63), c = (int)((idx >> 6) % NC), tile = (int)((idx >> 6) / NC);
+    const int ni = lane & 15, kb = lane >> 4;
+    const int b = 4 * c + kb;
+    if (b >= nb) return;
+    float w[32];
+    decode_block(pw[idx], e8m0_to_f32(ps[(((size_t)tile * NG + (c >> 2)) * 64 + lane) * 4 + (c & 3)]), w);
+    float *o = out + ((size_t)(16 * tile + ni) * nb + b) * 32;
+#pragma unroll
+    for (int i = 0; i < 32; ++i) o[i] = w[i];
+}
+
+// Decode GEMV on the resident copy.  grid.x = groups of 4 tiles (one wave each), grid.y = expert.
+// The expert's tokens (MTOK per pass) are staged in LDS once per workgroup; every wave then streams its
+// tile: WR chunks in flight, one scale word per four chunks, four MFMA steps per chunk with the tokens
+// as the M tile.  Token chunks of one block lie 64 bytes further apart than they are long, which
+// spreads the four lane groups (four consecutive blocks) over all banks.
+template <int MTOK, int WR, int NWV>
+__global__ __launch_bounds__(NWV * 64) void mxfp4_res_kernel(const uint16_t *__restrict__ x,
+                                                        const u32x4_t *__restrict__ pw,
+                                                        const uint8_t *__restrict__ ps,
+                                                        const uint16_t *__restrict__ bias, uint16_t *__restrict__ y,
+                                                        const int32_t *__restrict__ offsets,
+                                                        const int32_t *__restrict__ token_ids, int K, int N, int NC,
+                                                        int NG, int swiglu, float limit) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char mr_lds[];
+    // WR: weight chunks in flight per wave (1 KB each); NWV: waves (tiles of 16 rows) per workgroup
+    constexpr int BSTR = 4 * MTOK * 16 + 64;    // bytes of one block's token chunks, padded
+    constexpr int OOB = 0x7FFFFF00;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int ni = lane & 15, kb = lane >> 4;
+    const int e = blockIdx.y;
+    const int p0 = offsets[e], p1 = offsets[e + 1];
+    if (p1 <= p0) return;  // block-uniform: an expert without tokens
+    const int nb = K >> 5, cpr = K >> 3;
+    const int ntiles = N >> 4;
+    const int tile = blockIdx.x * NWV + wave;
+    const bool active = tile < ntiles;  // wave-uniform
+    const size_t et = (size_t)e * ntiles + (active ? tile : 0);
+    const __amdgpu_buffer_rsrc_t rs_w = make_rsrc(pw + et * NC * 64, active ? (uint32_t)NC * 1024u : 0u);
+    const __amdgpu_buffer_rsrc_t rs_s = make_rsrc(ps + et * NG * 256, active ? (uint32_t)NG * 256u : 0u);
+    const int voff_w = lane * 16, voff_s = lane * 4;
+    const int a_tok = (ni & (MTOK - 1)) * 16;
+
+    u32x4_t wring[WR];
+    uint32_t sring[WR / 4];
+    auto load_w = [&](int c) {  // chunks past the tile fall beyond the descriptor: zeros, no memory access
+        return __builtin_amdgcn_raw_buffer_load_b128(rs_w, c < NC ? voff_w : OOB, c * 1024, 2);
+    };
+    auto load_s = [&](int g) { return __builtin_amdgcn_raw_buffer_load_b32(rs_s, g < NG ? voff_s : OOB, g * 256, 2); };
+
+    for (int pbase = p0; pbase < p1; pbase += MTOK) {
+        const int rows = min(MTOK, p1 - pbase);
+        // the first weights do not depend on the tokens: they are requested before those are staged
+#pragma unroll
+        for (int u = 0; u < WR; ++u) {
+            if ((u & 3) == 0) sring[u >> 2] = load_s(u >> 2);
+            wring[u] = load_w(u);
+        }
+        if (pbase > p0) __syncthreads();  // everyone is done with the previous tokens
+        for (int c = threadIdx.x; c < rows * cpr; c += NWV * 64) {
+            const int m = c / cpr, cc = c - m * cpr;
+            const int p = pbase + m;
+            const int src = token_ids ? token_ids[p] : p;
+            *(u32x4_t *)(mr_lds + (cc >> 2) * BSTR + (cc & 3) * (MTOK * 16) + m * 16) =
+                *(const u32x4_t *)(x + (size_t)src * K + (size_t)cc * 8);
+        }
+        __syncthreads();
+        if (!active) continue;  // wave-uniform; the barriers above are reached by every wave
+
+        float4_t acc = float4_t{0.f, 0.f, 0.f, 0.f};
+        for (int c0 = 0; c0 < NC; c0 += WR) {
+#pragma unroll
+            for (int u = 0; u < WR; ++u) {
+                const int c = c0 + u;
+                const u32x4_t w = wring[u];
+                const uint32_t sw = sring[u >> 2];
+                wring[u] = load_w(c + WR);
+                if ((u & 3) == 3) sring[u >> 2] = load_s((c + WR) >> 2);
+                if (c < NC) {  // wave-uniform
+                    const float scale = e8m0_to_f32((sw >> (8 * (u & 3))) & 0xFFu);
+                    const int b = min(4 * c + kb, nb - 1);  // blocks past the row: a finite chunk times zero weights
+                    const unsigned char *xb = mr_lds + b * BSTR + a_tok;
+                    const uint32_t w0 = w[0], w1 = w[1], w2 = w[2], w3 = w[3];
+                    const uint32_t wq[4] = {w0, w1, w2, w3};
+#pragma unroll
+                    for (int sq = 0; sq < 4; ++sq) {
+                        const u32x4_t av = *(const u32x4_t *)(xb + sq * (MTOK * 16));
+                        u32x4_t bv;
+                        bv[0] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(wq[sq], scale, 0));
+                        bv[1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(wq[sq], scale, 1));
+                        bv[2] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(wq[sq], scale, 2));
+                        bv[3] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(wq[sq], scale, 3));
+                        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av),
+                                                                     __builtin_bit_cast(bf16x8_t, bv), acc, 0, 0, 0);
+                    }
+                }
+            }
+        }
+        // D[m][n]: lane (n = ni, m = 4*kb + i): token 4*kb + i of weight row 16 tile + ni
+        const int n = 16 * tile + ni;
+        const float bvv = bias ? BF16Traits::to_f32(bias[(size_t)e * N + n]) : 0.0f;
+        if (swiglu) {
+            // rows 2c / 2c + 1 are the gate / up of output c (moe.rs:152-173) and sit in neighbouring lanes:
+            // each is rounded to bf16 as the projection's own output would be, the even lane fetches its
+            // neighbour's value and stores the activation
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int m = 4 * kb + i;
+                const float v = BF16Traits::to_f32(BF16Traits::from_f32(acc[i] + bvv));
+                const float other = __shfl_xor(v, 1, 64);
+                if (!(ni & 1) && m < rows)
+                    y[(size_t)(pbase + m) * (N >> 1) + (n >> 1)] = BF16Traits::from_f32(gpt_oss_swiglu_f32(v, other, limit));
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int m = 4 * kb + i;
+                if (m < rows) y[(size_t)(pbase + m) * N + n] = BF16Traits::from_f32(acc[i] + bvv);
+            }
+        }
+    }
+}
+
+bool mxfp4_res_eligible(int64_t K, int64_t N) {
+    // whole tiles of 16 rows; the staged tokens (4 per pass) must fit LDS; 32-bit offsets inside a tile
+    return K % 32 == 0 && N % 16 == 0 && N > 0 && (K / 32) * (4 * 4 * 16 + 64) <= 96 * 1024 && K <= (1 << 24);
+}
+size_t mxfp4_res_weight_bytes(int64_t E, int64_t K, int64_t N) {
+    return (size_t)E * (size_t)(N / 16) * (size_t)ceil_div(K / 32, 4) * 1024;
+}
+size_t mxfp4_res_scale_bytes(int64_t E, int64_t K, int64_t N) {
+    return (size_t)E * (size_t)(N / 16) * (size_t)ceil_div(ceil_div(K / 32, 4), 4) * 256;
+}
+
+int launch_mxfp4_repack(oxq_ctx *ctx, hipStream_t s, const uint8_t *blocks, const uint8_t *scales, void *pw, void *ps,
+                        int64_t E, int64_t K, int64_t N) {
+    const int nb = (int)(K / 32), NC = (int)ceil_div(nb, 4), NG = (int)ceil_div(NC, 4);
+    const size_t threads = (size_t)E * (N / 16) * NC * 64;
+    dim3 grid((unsigned)ceil_div((int64_t)threads, 256)), block(256);
+    set_plan(ctx, "mxfp4_repack", grid, block, 1, 1, 0);
+    if (ctx->plan_only) return OXQ_OK;
+    if ((uintptr_t)blocks & 15) return fail(OXQ_ERR_UNSUPPORTED, "mxfp4 repack: blocks must be 16-byte aligned");
+    hipLaunchKernelGGL(mxfp4_repack_kernel, grid, block, 0, s, blocks, scales, (u32x4_t *)pw, (uint8_t *)ps, (int)E,
+                       (int)N, nb, NC, NG);
+    OXQ_HIP_CHECK(hipGetLastError());
+    return OXQ_OK;
+}
+
+int launch_mxfp4_res_dequant(oxq_ctx *ctx, hipStream_t s, const void *pw, const void *ps, int64_t expert, int64_t K,
+                             int64_t N, float *out_nk) {
+    const int nb = (int)(K / 32), NC = (int)ceil_div(nb, 4), NG = (int)ceil_div(NC, 4);
+    const size_t threads = (size_t)(N / 16) * NC * 64;
+    dim3 grid((unsigned)ceil_div((int64_t)threads, 256)), block(256);
+    set_plan(ctx, "mxfp4_res_dequant", grid, block, 1, 1, 0);
+    if (ctx->plan_only) return OXQ_OK;
+    const u32x4_t *w = (const u32x4_t *)pw + (size_t)expert * (N / 16) * NC * 64;
+    const uint8_t *sc = (const uint8_t *)ps + (size_t)expert * (N / 16) * NG * 256;
+    hipLaunchKernelGGL(mxfp4_res_dequant_kernel, grid, block, 0, s, w, sc, out_nk, (int)N, nb, NC, NG);
+    OXQ_HIP_CHECK(hipGetLastError());
+    return OXQ_OK;
+}
+
+// p.blocks / p.scales hold the resident copy; grouped form only
+int launch_mxfp4_res_gemv(oxq_ctx *ctx, hipStream_t s, const Mxfp4Problem &p) {
+    const int nb = (int)(p.K / 32), NC = (int)ceil_div(nb, 4), NG = (int)ceil_div(NC, 4);
+    constexpr int MTOK = 4;
+    const size_t lds = (size_t)nb * (4 * MTOK * 16 + 64);
+    // 8 chunks in flight per wave and 4 waves per workgroup measured best on 32 experts x (5760 + 2880) x 2880
+    // (47.5 us a decode step; 4 / 16 chunks: 49.5 / 58.7 us; 8 / 2 waves: 50.9 / 58.3 us)
+    constexpr int WR = 8, NWV = 4;
+    dim3 grid((unsigned)ceil_div(p.N / 16, NWV), (unsigned)p.n_experts), block(NWV * 64);
+    char name[64];
+    snprintf(name, sizeof name, "mxfp4_experts_gemv_bf16_t%d%s", MTOK, p.swiglu ? "_swiglu" : "");
+    set_plan(ctx, name, grid, block, 1, 1, 0);
+    if (ctx->plan_only) return OXQ_OK;
+    if ((uintptr_t)p.x & 15) return fail(OXQ_ERR_UNSUPPORTED, "mxfp4 experts: x must be 16-byte aligned");
+    static LdsGrant lds_grant;
+    OXQ_HIP_CHECK(lds_grant.ensure((const void *)mxfp4_res_kernel<MTOK, WR, NWV>, lds));
+    hipLaunchKernelGGL((mxfp4_res_kernel<MTOK, WR, NWV>), grid, block, lds, s, (const uint16_t *)p.x,
+                       (const u32x4_t *)p.blocks, p.scales, (const uint16_t *)p.bias, (uint16_t *)p.y, p.expert_offsets,
+                       p.token_ids, (int)p.K, (int)p.N, NC, NG, p.swiglu, p.swiglu_limit);
+    OXQ_HIP_CHECK(hipGetLastError());
+    return OXQ_OK;
+}
+
 template <int MB, int RW>
 static int mxfp4_lds_go(hipStream_t s, dim3 grid, const Mxfp4Problem &p, size_t lds) {
     static LdsGrant lds_grant;  // one per instantiation

@@ -402,6 +402,14 @@ static int scratch_lookup(int device, void **out) {
 }
 }  // namespace oxq
 
+struct oxq_mxfp4_experts {
+    oxq_ctx *ctx;
+    oxq_tensor blocks, scales, bias;  // the caller's tensors (prefill sizes and ineligible shapes run on them)
+    bool has_bias;
+    int64_t n_experts, k, n;
+    void *pw, *ps;                    // resident tile-major copy, owned; null when the shape does not qualify
+};
+
 // =============================================================================
 // C ABI
 // =============================================================================
@@ -1068,6 +1076,169 @@ int oxq_mxfp4_moe_gate_up_swiglu(oxq_ctx *ctx, void *stream, const oxq_tensor *x
     if (!fused) return fail(OXQ_ERR_ARG, "Mxfp4MoeGateUpSwiglu: fused is NULL");
     return moe_matmul_impl("Mxfp4MoeGateUpSwiglu", ctx, stream, x, blocks, scales, bias, expert_offsets, token_ids,
                            gather_rows, k, n, true, limit, out, fused);
+}
+
+// ---- resident MXFP4 experts (moe.rs:366-417 load_gpt_oss keeps the stacked tensors for the model's life) ----
+int oxq_mxfp4_experts_new(oxq_ctx *ctx, const oxq_tensor *blocks, const oxq_tensor *scales, const oxq_tensor *bias,
+                          int64_t n_experts, int64_t k, int64_t n, oxq_mxfp4_experts **out) {
+    const char *op = "Mxfp4Experts";
+    if (!ctx || !out) return fail(OXQ_ERR_ARG, "%s: NULL argument", op);
+    *out = nullptr;
+    OXQ_TRY(check_tensor(ctx, op, "blocks", blocks));
+    OXQ_TRY(check_tensor(ctx, op, "scales", scales));
+    if (blocks->dtype != OXQ_U8 || scales->dtype != OXQ_U8)
+        return fail(OXQ_ERR_DTYPE, "%s: blocks/scales must be U8, got %s/%s", op, dtype_name(blocks->dtype),
+                    dtype_name(scales->dtype));
+    if (n_experts <= 0 || k <= 0 || n <= 0 || k % 32 != 0)
+        return fail(OXQ_ERR_SHAPE, "%s: %lld experts of [%lld, %lld]: K must be a positive multiple of 32", op,
+                    (long long)n_experts, (long long)n, (long long)k);
+    if (k > INT32_MAX || n > INT32_MAX || n_experts > 65535)
+        return fail(OXQ_ERR_SHAPE, "%s: dimension out of range", op);
+    const int64_t nb = k / 32;
+    if (numel(blocks) != n_experts * n * nb * 16 || numel(scales) != n_experts * n * nb || !blocks->contiguous ||
+        !scales->contiguous)
+        return fail(OXQ_ERR_SHAPE, "%s: blocks %lld / scales %lld elements don't match %lld x [%lld, %lld]", op,
+                    (long long)numel(blocks), (long long)numel(scales), (long long)n_experts, (long long)n,
+                    (long long)k);
+    if (bias) {
+        OXQ_TRY(check_tensor(ctx, op, "bias", bias));
+        if (bias->dtype != OXQ_BF16 || numel(bias) != n_experts * n || !bias->contiguous)
+            return fail(OXQ_ERR_SHAPE, "%s: bias must be a contiguous BF16 [%lld, %lld]", op, (long long)n_experts,
+                        (long long)n);
+    }
+    oxq_mxfp4_experts *h = new (std::nothrow) oxq_mxfp4_experts();
+    if (!h) return fail(OXQ_ERR_RUNTIME, "%s: out of host memory", op);
+    h->ctx = ctx;
+    h->blocks = *blocks;
+    h->scales = *scales;
+    h->has_bias = bias != nullptr;
+    if (bias) h->bias = *bias;
+    h->n_experts = n_experts;
+    h->k = k;
+    h->n = n;
+    h->pw = h->ps = nullptr;
+    const char *env = getenv("OXQ_PREPACK");
+    const bool want = !(env && atoi(env) == 0) && mxfp4_res_eligible(k, n) && !((uintptr_t)blocks->data & 15);
+    if (want && !ctx->plan_only) {
+        int prev = 0;
+        (void)hipGetDevice(&prev);
+        hipError_t e = hipSetDevice(ctx->device);
+        int rc = OXQ_OK;
+        if (e == hipSuccess) e = hipMalloc(&h->pw, mxfp4_res_weight_bytes(n_experts, k, n));
+        if (e == hipSuccess) e = hipMalloc(&h->ps, mxfp4_res_scale_bytes(n_experts, k, n));
+        if (e != hipSuccess) {
+            rc = fail(OXQ_ERR_RUNTIME, "%s: repack allocation failed: %s", op, hipGetErrorString(e));
+        } else {
+            rc = launch_mxfp4_repack(ctx, nullptr, (const uint8_t *)blocks->data, (const uint8_t *)scales->data, h->pw,
+                                     h->ps, n_experts, k, n);
+            if (rc == OXQ_OK && (e = hipStreamSynchronize(nullptr)) != hipSuccess)
+                rc = fail(OXQ_ERR_RUNTIME, "%s: repack failed: %s", op, hipGetErrorString(e));
+        }
+        (void)hipSetDevice(prev);
+        if (rc != OXQ_OK) {
+            if (h->pw) (void)hipFree(h->pw);
+            if (h->ps) (void)hipFree(h->ps);
+            delete h;
+            return rc;
+        }
+    } else if (want) {
+        h->pw = h->ps = (void *)16;  // plan-only: routes as a resident copy would, nothing is dereferenced
+    }
+    *out = h;
+    return OXQ_OK;
+}
+
+static int experts_forward(oxq_mxfp4_experts *h, void *stream, const oxq_tensor *x, const oxq_tensor *expert_offsets,
+                           const oxq_tensor *token_ids, int gather_rows, bool swiglu, float limit, const oxq_tensor *out,
+                           int *fused) {
+    const char *op = swiglu ? "Mxfp4ExpertsGateUpSwiglu" : "Mxfp4ExpertsMatmul";
+    if (!h) return fail(OXQ_ERR_ARG, "%s: handle is NULL", op);
+    // same checks and, for the sizes the resident kernel does not take, the same kernels as the stateless op
+    oxq_ctx *ctx = h->ctx;
+    if (fused) *fused = 0;
+    OXQ_TRY(check_tensor(ctx, op, "expert_offsets", expert_offsets));
+    if (expert_offsets->dtype != OXQ_I32 || expert_offsets->rank != 1 || expert_offsets->dims[0] != h->n_experts + 1 ||
+        !expert_offsets->contiguous)
+        return fail(OXQ_ERR_SHAPE, "%s: expert_offsets must be a contiguous I32 [%lld]", op, (long long)h->n_experts + 1);
+    const bool resident = h->pw != nullptr;
+    const int64_t n_pairs = (out && out->rank == 2) ? out->dims[0] : 0;
+    // many pairs per expert (prefill) convert a weight once per 64 tokens in the tile matmul, which reads the
+    // checkpoint layout
+    if (!resident || n_pairs >= 8 * h->n_experts)
+        return moe_matmul_impl(op, ctx, stream, x, &h->blocks, &h->scales, h->has_bias ? &h->bias : nullptr, expert_offsets,
+                               token_ids, gather_rows, h->k, h->n, swiglu, limit, out, fused);
+    Mxfp4Problem p;
+    OXQ_TRY(check_mxfp4(ctx, op, false, x, &h->blocks, &h->scales, h->k, h->n, h->n_experts, out, &p));
+    if (swiglu && (h->n & 1)) return fail(OXQ_ERR_SHAPE, "%s: interleaved gate / up rows need an even n", op);
+    const int64_t out_cols = swiglu ? h->n / 2 : h->n;
+    if (out->rank != 2 || out->dims[1] != out_cols || !out->contiguous)
+        return fail(OXQ_ERR_SHAPE, "%s: out must be a contiguous [n_pairs, %lld]", op, (long long)out_cols);
+    if (gather_rows) {
+        OXQ_TRY(check_tensor(ctx, op, "token_ids", token_ids));
+        if (token_ids->dtype != OXQ_I32 || numel(token_ids) != n_pairs || !token_ids->contiguous)
+            return fail(OXQ_ERR_SHAPE, "%s: token_ids must be a contiguous I32 [%lld]", op, (long long)n_pairs);
+    } else if (x->dims[0] != n_pairs) {
+        return fail(OXQ_ERR_SHAPE, "%s: x has %lld rows, out has %lld", op, (long long)x->dims[0], (long long)n_pairs);
+    }
+    p.blocks = (const uint8_t *)h->pw;
+    p.scales = (const uint8_t *)h->ps;
+    p.bias = h->has_bias ? h->bias.data : nullptr;
+    p.n_experts = h->n_experts;
+    p.expert_offsets = (const int32_t *)expert_offsets->data;
+    p.token_ids = gather_rows ? (const int32_t *)token_ids->data : nullptr;
+    p.n_pairs = n_pairs;
+    p.swiglu = swiglu ? 1 : 0;
+    p.swiglu_limit = limit;
+    const int rc = launch_mxfp4_res_gemv(ctx, (hipStream_t)stream, p);
+    if (rc == OXQ_OK && fused) *fused = 1;
+    return rc;
+}
+
+int oxq_mxfp4_experts_matmul(oxq_mxfp4_experts *h, void *stream, const oxq_tensor *x, const oxq_tensor *expert_offsets,
+                             const oxq_tensor *token_ids, int gather_rows, const oxq_tensor *out) {
+    return experts_forward(h, stream, x, expert_offsets, token_ids, gather_rows, false, 0.0f, out, nullptr);
+}
+
+int oxq_mxfp4_experts_gate_up_swiglu(oxq_mxfp4_experts *h, void *stream, const oxq_tensor *x,
+                                     const oxq_tensor *expert_offsets, const oxq_tensor *token_ids, int gather_rows,
+                                     float limit, const oxq_tensor *out, int *fused) {
+    if (!fused) return fail(OXQ_ERR_ARG, "Mxfp4ExpertsGateUpSwiglu: fused is NULL");
+    return experts_forward(h, stream, x, expert_offsets, token_ids, gather_rows, true, limit, out, fused);
+}
+
+int oxq_mxfp4_experts_is_resident(const oxq_mxfp4_experts *h, int *resident) {
+    if (!h || !resident) return fail(OXQ_ERR_ARG, "Mxfp4Experts: NULL argument");
+    *resident = h->pw != nullptr;
+    return OXQ_OK;
+}
+
+int oxq_mxfp4_experts_dequantize(oxq_mxfp4_experts *h, void *stream, int64_t expert, const oxq_tensor *out) {
+    const char *op = "Mxfp4ExpertsDequantize";
+    if (!h || !out) return fail(OXQ_ERR_ARG, "%s: NULL argument", op);
+    if (expert < 0 || expert >= h->n_experts)
+        return fail(OXQ_ERR_ARG, "%s: expert %lld outside 0..%lld", op, (long long)expert, (long long)h->n_experts - 1);
+    OXQ_TRY(check_tensor(h->ctx, op, "out", out));
+    if (out->dtype != OXQ_F32 || out->rank != 2 || out->dims[0] != h->n || out->dims[1] != h->k || !out->contiguous)
+        return fail(OXQ_ERR_SHAPE, "%s: out must be a contiguous F32 [%lld, %lld]", op, (long long)h->n, (long long)h->k);
+    if (h->pw)
+        return launch_mxfp4_res_dequant(h->ctx, (hipStream_t)stream, h->pw, h->ps, expert, h->k, h->n, (float *)out->data);
+    Mxfp4Problem p;
+    memset(&p, 0, sizeof p);
+    const int64_t nb = h->k / 32;
+    p.blocks = (const uint8_t *)h->blocks.data + (size_t)expert * h->n * nb * 16;
+    p.scales = (const uint8_t *)h->scales.data + (size_t)expert * h->n * nb;
+    p.K = h->k;
+    p.N = h->n;
+    return launch_mxfp4_dequant(h->ctx, (hipStream_t)stream, p, (float *)out->data);
+}
+
+void oxq_mxfp4_experts_free(oxq_mxfp4_experts *h) {
+    if (!h) return;
+    if (!h->ctx->plan_only) {
+        if (h->pw) (void)hipFree(h->pw);
+        if (h->ps) (void)hipFree(h->ps);
+    }
+    delete h;
 }
 
 // ---- mixture-of-experts glue (moe.rs:466-607, ffn_kernels.metal, moe.rs:152-173) --------

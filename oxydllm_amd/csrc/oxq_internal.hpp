@@ -203,6 +203,15 @@ int launch_f8_mm(oxq_ctx *ctx, hipStream_t s, const F8Problem &p);
 int launch_mxfp4_mm(oxq_ctx *ctx, hipStream_t s, const Mxfp4Problem &p);
 int launch_mxfp4_gemv(oxq_ctx *ctx, hipStream_t s, const Mxfp4Problem &p);
 int launch_mxfp4_dequant(oxq_ctx *ctx, hipStream_t s, const Mxfp4Problem &p, float *out_nk);
+// resident experts: tile-major copy (layout: mxfp4_gemv.hip) and the decode GEMV on it
+bool mxfp4_res_eligible(int64_t K, int64_t N);
+size_t mxfp4_res_weight_bytes(int64_t E, int64_t K, int64_t N);
+size_t mxfp4_res_scale_bytes(int64_t E, int64_t K, int64_t N);
+int launch_mxfp4_repack(oxq_ctx *ctx, hipStream_t s, const uint8_t *blocks, const uint8_t *scales, void *pw, void *ps,
+                        int64_t E, int64_t K, int64_t N);
+int launch_mxfp4_res_dequant(oxq_ctx *ctx, hipStream_t s, const void *pw, const void *ps, int64_t expert, int64_t K,
+                             int64_t N, float *out_nk);
+int launch_mxfp4_res_gemv(oxq_ctx *ctx, hipStream_t s, const Mxfp4Problem &p);
 // mixture-of-experts glue (moe_glue.hip)
 int launch_moe_route(oxq_ctx *ctx, hipStream_t s, const void *logits, int dtype, int64_t T, int64_t E, int64_t top_k,
                      int norm_topk, int32_t *top_idx, float *top_vals);

@@ -683,14 +683,13 @@ int launch_pk4_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p) {
     const int mt = M > 48 ? 4 : (int)ceil_div(M, 16);
     const int NB = (int)(p.w.K / 128);
     // Few column strips and a long K (a down projection: N = 4096 is 64 strips for 256 CUs):
-    // K is also cut into slices, at least two blocks per wave, so that up to one workgroup per CU
+    // K is also cut into slices, at least one block per wave, so that up to one workgroup per CU
     // runs; the slices' f32 partial tiles are added in slice order by a second launch.  Measured
-    // (f16, M = 1 / 64): 14336 x 4096 16.6 / 41.1 us unsplit, 11.2 / 22.5 us in 4 slices, worse again
-    // in 5 or 7 (a second round of workgroups); a 4096 x 4096 layer gains nothing (the extra launch
-    // costs what the split saves).
+    // (f16, M = 1 / 16): 14336 x 4096 16.9 / 19.1 us unsplit, 9.0 / 10.0 us in 4 slices, 9.5 - 10.2 /
+    // 11.4 - 12.1 us in 3, 6 or 8; a 4096 x 4096 layer 6.4 / 7.4 us unsplit, 5.7 / 6.6 us in 4 slices.
     const int64_t tiles = (p.w.N / 64) * ceil_div(M, 16 * mt);
     int ks = 1;
-    if (tiles <= 96 && NB >= 64) ks = (int)std::max<int64_t>(1, std::min<int64_t>(256 / tiles, NB / 16));
+    if (tiles <= 96 && NB >= 32) ks = (int)std::max<int64_t>(1, std::min<int64_t>(256 / tiles, NB / 8));
     ks = pk4_env("OXQ_PK4_KS", ks);
     ks = std::max(1, std::min(ks, NB));
     if (p.act) ks = 1;  // the activation needs the whole sum: gate|up layers are wide, one slice fills the chip

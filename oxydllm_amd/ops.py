@@ -397,6 +397,66 @@ def mxfp4_moe_gate_up_swiglu(x, blocks, scales, bias, expert_offsets, token_ids,
     return out
 
 
+class Mxfp4Experts:
+    """The stacked MXFP4 expert tensors of one MoE projection, kept resident (moe.rs:366-417): ``blocks`` u8
+    [E * n * k/32 * 16], ``scales`` u8 [E * n * k/32], ``bias`` bf16 [E, n] or None.  Construction builds the
+    tile-major copy that decode sizes stream; the caller's tensors are borrowed (prefill sizes run on them)."""
+
+    def __init__(self, blocks, scales, bias, n_experts: int, k: int, n: int, *, ctx: Optional[Context] = None):
+        self.ctx = _ctx(ctx)
+        self._keep = (blocks, scales, bias)
+        self.n_experts, self.k, self.n = n_experts, k, n
+        self.handle = C.c_void_p()
+        _lib.check(self.ctx._lib.oxq_mxfp4_experts_new(self.ctx.handle, desc(blocks), desc(scales), desc(bias),
+                                                       n_experts, k, n, C.byref(self.handle)))
+
+    @property
+    def resident(self) -> bool:
+        r = C.c_int()
+        _lib.check(self.ctx._lib.oxq_mxfp4_experts_is_resident(self.handle, C.byref(r)))
+        return bool(r.value)
+
+    def matmul(self, x, expert_offsets, token_ids, *, out=None):
+        gather = token_ids is not None
+        n_pairs = token_ids.numel() if gather else x.shape[0]
+        if out is None:
+            out = torch.empty((n_pairs, self.n), dtype=x.dtype, device=x.device)
+        _lib.check(self.ctx._lib.oxq_mxfp4_experts_matmul(self.handle, self.ctx.stream(), desc(x), desc(expert_offsets),
+                                                          desc(token_ids), 1 if gather else 0, desc(out)))
+        return out
+
+    def gate_up_swiglu(self, x, expert_offsets, token_ids, limit: float, *, out=None):
+        gather = token_ids is not None
+        n_pairs = token_ids.numel() if gather else x.shape[0]
+        if out is None:
+            out = torch.empty((n_pairs, self.n // 2), dtype=x.dtype, device=x.device)
+        fused = C.c_int()
+        _lib.check(self.ctx._lib.oxq_mxfp4_experts_gate_up_swiglu(self.handle, self.ctx.stream(), desc(x),
+                                                                  desc(expert_offsets), desc(token_ids),
+                                                                  1 if gather else 0, float(limit), desc(out),
+                                                                  C.byref(fused)))
+        if not fused.value:
+            gu = self.matmul(x, expert_offsets, token_ids)
+            gated_activation(gu, ACT_GPT_OSS_SWIGLU, limit, out=out, ctx=self.ctx)
+        return out
+
+    def dequantize(self, expert: int):
+        out = torch.empty((self.n, self.k), dtype=torch.float32, device=self._keep[0].device)
+        _lib.check(self.ctx._lib.oxq_mxfp4_experts_dequantize(self.handle, self.ctx.stream(), expert, desc(out)))
+        return out
+
+    def close(self):
+        if self.handle:
+            self.ctx._lib.oxq_mxfp4_experts_free(self.handle)
+            self.handle = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
 def moe_route(logits, top_k: int, norm_topk: bool = True, *, ctx: Optional[Context] = None):
     """moe.rs:466-486: softmax, stable descending top-k, optional renormalisation."""
     ctx = _ctx(ctx)
