@@ -139,6 +139,13 @@ def run(ops, ctx, stream, steps, warmup, time_graph, with_cpu=True):
         r = _row("cfg3", f"gguf {synth.GGUF_NAMES[fmt]} M=1 K={K} N={N} f32 activations, gguf_quant_matmul op",
                  lambda i, d=d, nc=nc, fmt=fmt: ops.gguf_quant_matmul(x, d[i % nc], K, N, fmt, out=y, ctx=ctx),
                  steps, warmup, stream, time_graph, nb, 2.0 * K * N, ctx)
+        # what reading the same block bytes costs when nothing else is done (64 KiB per workgroup)
+        wgs = data.nbytes // 65536
+        sums = torch.zeros(wgs, device=dev, dtype=torch.int32)
+        _, ev = time_graph(lambda i, d=d, nc=nc: ops.calib_read(d[i % nc].view(torch.uint8).reshape(-1)[:wgs * 65536],
+                                                               wgs, True, sums, ctx=ctx), steps, warmup, stream)
+        r["bare_read_nt_us"] = round(ev * 1e3 / steps, 3)
+        r["bare_read_workgroups"] = wgs
         if with_cpu:
             def cpu_call(fmt=fmt, data=data):
                 oracle.matmul_nt_f32(xh, oracle.dequantize_gguf(fmt, data, N, K))
