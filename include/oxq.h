@@ -118,6 +118,25 @@ const char *oxq_last_error(void);
 const char *oxq_status_name(int status);
 void oxq_version(int *major, int *minor);
 
+/* ---- opt-in weight cache behind the stateless ops -----------------------------
+ * The reference's layers call the op functions with the same resident tensors on every forward
+ * (linear.rs:482-533).  With this cache on, oxq_w4a16_matmul / oxq_w8a16_matmul / oxq_gptq_matmul /
+ * oxq_mpp_quant_matmul remember a (qweight, qzeros, scales) triple by its device addresses: the first
+ * call builds the tile-major copy that oxq_packed_quant_linear_new builds (one extra launch and a
+ * hipMalloc; skipped while the stream is being captured, where the call takes its usual path) and
+ * later calls run the resident-layer kernel on it, with that layer's arithmetic (m <= 16: unrounded
+ * weights, f32 fold; above: tile GEMM on weights rounded to the activation type).  Shapes the
+ * resident layout does not cover take the usual path.  The copy costs the packed tensors' size
+ * again; least recently used copies go when max_bytes is reached.
+ *
+ * Contract: while a triple is cached its tensors must neither change nor be freed and reused - the
+ * ctx cannot see that.  Call oxq_ctx_forget_weights(ctx, qweight->data) before doing so (NULL drops
+ * every copy).  Off by default (max_bytes = 0, or OXQ_WEIGHT_CACHE_MB in the environment).
+ * No counterpart in the reference, whose ops read the checkpoint layout directly. */
+int oxq_ctx_set_weight_cache(oxq_ctx *ctx, int64_t max_bytes);
+int oxq_ctx_forget_weights(oxq_ctx *ctx, const void *qweight_data);
+int oxq_ctx_weight_cache_bytes(const oxq_ctx *ctx, int64_t *bytes, int64_t *entries);
+
 /* Block layout of a GGUF format: metal_ops.rs:5228-5241 (block_layout). */
 int oxq_gguf_block_layout(int quant, int64_t *block_elems, int64_t *block_bytes);
 

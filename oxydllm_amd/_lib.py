@@ -77,6 +77,9 @@ SIGNATURES = {
     "oxq_last_error": (C.c_char_p, []),
     "oxq_status_name": (C.c_char_p, [C.c_int]),
     "oxq_version": (None, [C.POINTER(C.c_int), C.POINTER(C.c_int)]),
+    "oxq_ctx_set_weight_cache": (C.c_int, [_VP, C.c_int64]),
+    "oxq_ctx_forget_weights": (C.c_int, [_VP, _VP]),
+    "oxq_ctx_weight_cache_bytes": (C.c_int, [_VP, C.POINTER(C.c_int64), C.POINTER(C.c_int64)]),
     "oxq_gguf_block_layout": (C.c_int, [C.c_int, C.POINTER(C.c_int64), C.POINTER(C.c_int64)]),
     "oxq_calib_read": (C.c_int, [_VP, _VP, _TP, C.c_int, C.c_int, _TP]),
     "oxq_w4a16_matmul": (C.c_int, [_VP, _VP, _TP, _TP, _TP, _TP, _TP]),

@@ -40,6 +40,19 @@ def _row(config, case, fn_of_step, steps, warmup, stream, time_graph, nbytes, fl
                          "frac": round(gbs / HBM_PEAK_GBS, 4)}}
 
 
+def _cached_row(config, case, call, nc, steps, warmup, stream, time_graph, nbytes, flops, ctx):
+    """`call(c)` on weight copy c with the ctx's opt-in weight cache on: every copy is seen once
+    outside the timed region (that call builds its tile-major copy), the timed calls find it."""
+    ctx.set_weight_cache(2 << 30)
+    try:
+        for c in range(nc):
+            call(c)
+        torch.cuda.synchronize()
+        return _row(config, case, lambda i: call(i % nc), steps, warmup, stream, time_graph, nbytes, flops, ctx)
+    finally:
+        ctx.set_weight_cache(0)
+
+
 def _time_cpu(fn, budget_s: float, max_calls: int):
     fn()  # warm
     calls, total = 0, 0.0
@@ -94,6 +107,9 @@ def run(ops, ctx, stream, steps, warmup, time_graph, with_cpu=True):
     rows.append(_row("cfg0", f"awq4 M=1 K={K} N={N} g={G} f16, w4a16_matmul op (checkpoint layout)",
                      lambda i: ops.w4a16_matmul(x, *d[i % nc], out=y, ctx=ctx), steps, warmup, stream, time_graph,
                      nb, 2.0 * K * N, ctx))
+    rows.append(_cached_row("cfg0", f"awq4 M=1 K={K} N={N} g={G} f16, w4a16_matmul op with the ctx weight cache on",
+                            lambda c: ops.w4a16_matmul(x, *d[c], out=y, ctx=ctx), nc, steps, warmup, stream,
+                            time_graph, nb, 2.0 * K * N, ctx))
     del d, layers
 
     # ---- config 2 --------------------------------------------------------------------------------------
@@ -124,6 +140,10 @@ def run(ops, ctx, stream, steps, warmup, time_graph, with_cpu=True):
             rows.append(_row("cfg2", f"gptq{bits} M={m} K={K} N={N} g={G} f16, gptq_matmul op (checkpoint layout)",
                              lambda i, x=x, y=y, bits=bits: ops.gptq_matmul(x, *d[i % nc], bits, out=y, ctx=ctx),
                              steps, warmup, stream, time_graph, nb, 2.0 * m * K * N, ctx))
+            rows.append(_cached_row("cfg2", f"gptq{bits} M={m} K={K} N={N} g={G} f16, gptq_matmul op with the ctx "
+                                            "weight cache on",
+                                    lambda c, x=x, y=y, bits=bits: ops.gptq_matmul(x, *d[c], bits, out=y, ctx=ctx),
+                                    nc, steps, warmup, stream, time_graph, nb, 2.0 * m * K * N, ctx))
         del d, layers
 
     # ---- config 3 --------------------------------------------------------------------------------------

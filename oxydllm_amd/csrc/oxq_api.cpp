@@ -6,6 +6,7 @@
 
 #include <cstdlib>
 #include <new>
+#include <vector>
 
 namespace oxq {
 
@@ -479,6 +480,10 @@ int oxq_ctx_create(int device, oxq_ctx **out) {
         const char *m = getenv("OXQ_SPLITK_MODE");
         ctx->splitk_mode = (m && *m) ? atoi(m) : 0;
     }
+    {
+        const char *m = getenv("OXQ_WEIGHT_CACHE_MB");
+        ctx->wcache_limit = (m && atoi(m) > 0) ? (size_t)atoi(m) << 20 : 0;
+    }
     if (ctx->plan_only) {
         *out = ctx;
         return OXQ_OK;
@@ -526,9 +531,12 @@ int oxq_ctx_create(int device, oxq_ctx **out) {
     return OXQ_OK;
 }
 
+static void wcache_destroy(oxq_ctx *ctx);  // frees every cached weight copy and the cache itself
+
 int oxq_ctx_destroy(oxq_ctx *ctx) {
     if (!ctx) return OXQ_OK;
     if (!ctx->plan_only) {
+        wcache_destroy(ctx);
         if (ctx->workspace) (void)hipFree(ctx->workspace);
         if (ctx->counters) (void)hipFree(ctx->counters);
     }
@@ -569,12 +577,166 @@ int oxq_calib_read(oxq_ctx *ctx, void *stream, const oxq_tensor *src, int workgr
                              nontemporal, (uint32_t *)checksums->data);
 }
 
+// ---- opt-in cache of tile-major weight copies behind the stateless ops ---------------------------
+// The reference's ops are called with the same resident tensors on every forward (linear.rs:482-533
+// passes the layer's own qweight / qzeros / scales).  A caller that swaps in only the op functions,
+// not the layer types, can let the ctx remember those tensors by address: the first call on a
+// (qweight, qzeros, scales) triple builds the resident layers' tile-major copy, later calls run the
+// resident-layer kernel on it.  Off unless oxq_ctx_set_weight_cache (or OXQ_WEIGHT_CACHE_MB) gives
+// it room: the ctx cannot see a caller overwrite or free those tensors, so the caller has to say
+// so (oxq_ctx_forget_weights).
+struct oxq_weight_cache {
+    struct Entry {
+        const void *qw, *qz, *sc;
+        int64_t K, N;
+        int group_shift, dtype, bits, pack_dim;
+        Pk4Weights w;
+        size_t bytes;
+        uint64_t last_use;
+    };
+    std::vector<Entry> entries;
+    size_t bytes = 0;
+    uint64_t tick = 0;
+};
+
+static void wcache_drop(oxq_ctx *ctx, size_t i) {
+    oxq_weight_cache *c = ctx->wcache;
+    (void)hipFree(c->entries[i].w.pw);  // waits for the device: no kernel still reads the copy
+    c->bytes -= c->entries[i].bytes;
+    c->entries.erase(c->entries.begin() + (long)i);
+}
+
+static void wcache_clear(oxq_ctx *ctx) {
+    if (!ctx->wcache) return;
+    while (!ctx->wcache->entries.empty()) wcache_drop(ctx, ctx->wcache->entries.size() - 1);
+}
+
+static void wcache_destroy(oxq_ctx *ctx) {
+    if (!ctx->wcache) return;
+    int prev = 0;
+    (void)hipGetDevice(&prev);
+    (void)hipSetDevice(ctx->device);
+    wcache_clear(ctx);
+    (void)hipSetDevice(prev);
+    delete ctx->wcache;
+    ctx->wcache = nullptr;
+}
+
+// true: the call was served (rc holds its status).  false: take the checkpoint-layout path.
+static bool wcache_forward(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p, int *rc) {
+    if (!ctx->wcache_limit || ctx->plan_only || !pk4_eligible(p)) return false;
+    if (((uintptr_t)p.x | (uintptr_t)p.y) & 15) return false;
+    if (!ctx->wcache) {
+        ctx->wcache = new (std::nothrow) oxq_weight_cache();
+        if (!ctx->wcache) return false;
+    }
+    oxq_weight_cache *c = ctx->wcache;
+    oxq_weight_cache::Entry *hit = nullptr;
+    for (auto &e : c->entries)
+        if (e.qw == p.qweight && e.qz == p.qzeros && e.sc == p.scales && e.K == p.K && e.N == p.N &&
+            e.group_shift == p.group_shift && e.dtype == p.dtype && e.bits == p.bits && e.pack_dim == p.pack_dim) {
+            hit = &e;
+            break;
+        }
+    if (!hit) {
+        // building a copy allocates: not while the stream is being captured into a graph
+        hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(s, &cs) != hipSuccess || cs != hipStreamCaptureStatusNone) {
+            (void)hipGetLastError();
+            return false;
+        }
+        const size_t bytes = (pk4_weight_bytes(p.K, p.N, p.bits) + 255) & ~(size_t)255;
+        if (bytes > ctx->wcache_limit) return false;
+        while (c->bytes + bytes > ctx->wcache_limit && !c->entries.empty()) {  // least recently used first
+            size_t lru = 0;
+            for (size_t i = 1; i < c->entries.size(); ++i)
+                if (c->entries[i].last_use < c->entries[lru].last_use) lru = i;
+            wcache_drop(ctx, lru);
+        }
+        void *mem = nullptr;
+        if (hipMalloc(&mem, bytes) != hipSuccess) {
+            (void)hipGetLastError();
+            return false;
+        }
+        oxq_weight_cache::Entry e{p.qweight, p.qzeros, p.scales, p.K, p.N, p.group_shift, p.dtype, p.bits, p.pack_dim,
+                                  Pk4Weights{(uint32_t *)mem, nullptr, p.K, p.N, p.group_shift, p.dtype, p.bits, 0},
+                                  bytes, 0};
+        const int prc = launch_pk4_prepack(ctx, s, p, e.w);  // on the caller's stream, ahead of the matmul
+        if (prc != OXQ_OK) {
+            (void)hipFree(mem);
+            *rc = prc;
+            return true;
+        }
+        try {
+            c->entries.push_back(e);
+        } catch (...) {
+            (void)hipFree(mem);
+            return false;
+        }
+        c->bytes += bytes;
+        hit = &c->entries.back();
+    }
+    hit->last_use = ++c->tick;
+    Pk4Problem q;
+    q.x = p.x;
+    q.bias = p.bias;
+    q.y = p.y;
+    q.M = p.M;
+    q.act = 0;
+    q.no_split = 0;
+    q.w = hit->w;
+    *rc = launch_pk4_forward(ctx, s, q);
+    return true;
+}
+
+int oxq_ctx_set_weight_cache(oxq_ctx *ctx, int64_t max_bytes) {
+    if (!ctx) return fail(OXQ_ERR_ARG, "oxq_ctx_set_weight_cache: ctx is NULL");
+    if (max_bytes < 0) return fail(OXQ_ERR_ARG, "oxq_ctx_set_weight_cache: max_bytes %lld is negative", (long long)max_bytes);
+    ctx->wcache_limit = (size_t)max_bytes;
+    if (ctx->wcache) {
+        int prev = 0;
+        (void)hipGetDevice(&prev);
+        (void)hipSetDevice(ctx->device);
+        while (ctx->wcache->bytes > ctx->wcache_limit && !ctx->wcache->entries.empty()) {
+            size_t lru = 0;
+            for (size_t i = 1; i < ctx->wcache->entries.size(); ++i)
+                if (ctx->wcache->entries[i].last_use < ctx->wcache->entries[lru].last_use) lru = i;
+            wcache_drop(ctx, lru);
+        }
+        (void)hipSetDevice(prev);
+    }
+    return OXQ_OK;
+}
+
+int oxq_ctx_forget_weights(oxq_ctx *ctx, const void *qweight_data) {
+    if (!ctx) return fail(OXQ_ERR_ARG, "oxq_ctx_forget_weights: ctx is NULL");
+    if (!ctx->wcache) return OXQ_OK;
+    int prev = 0;
+    (void)hipGetDevice(&prev);
+    (void)hipSetDevice(ctx->device);
+    if (!qweight_data) wcache_clear(ctx);
+    else
+        for (size_t i = ctx->wcache->entries.size(); i-- > 0;)
+            if (ctx->wcache->entries[i].qw == qweight_data) wcache_drop(ctx, i);
+    (void)hipSetDevice(prev);
+    return OXQ_OK;
+}
+
+int oxq_ctx_weight_cache_bytes(const oxq_ctx *ctx, int64_t *bytes, int64_t *entries) {
+    if (!ctx) return fail(OXQ_ERR_ARG, "oxq_ctx_weight_cache_bytes: ctx is NULL");
+    if (bytes) *bytes = ctx->wcache ? (int64_t)ctx->wcache->bytes : 0;
+    if (entries) *entries = ctx->wcache ? (int64_t)ctx->wcache->entries.size() : 0;
+    return OXQ_OK;
+}
+
 // ---- AWQ / GPTQ -------------------------------------------------------------
 int oxq_w4a16_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x, const oxq_tensor *qweight,
                      const oxq_tensor *qzeros, const oxq_tensor *scales, const oxq_tensor *out) {
     Wna16Problem p;
     OXQ_TRY(check_wna16(ctx, "W4A16Matmul", KIND_GEMV, x, qweight, qzeros, scales, 4, OXQ_PACK_OUT,
                         out, &p));
+    int crc;
+    if (wcache_forward(ctx, (hipStream_t)stream, p, &crc)) return crc;
     return launch_wna16_gemv(ctx, (hipStream_t)stream, p);
 }
 
@@ -593,6 +755,8 @@ int oxq_w4a16_matmul_static(oxq_ctx *ctx, void *stream, const oxq_tensor *x, con
     shadow.counters = nullptr;
     shadow.n_counters = 0xFFFFFFFFu;
     shadow.splitk_mode = 2;
+    shadow.wcache = nullptr;
+    shadow.wcache_limit = 0;
     shadow.plan_only = true;  // first pass: what would this call need?
     OXQ_TRY(launch_wna16_gemv(&shadow, (hipStream_t)stream, p));
     if (shadow.plan.workspace_bytes > OXQ_STATIC_SCRATCH_BYTES)
@@ -623,6 +787,8 @@ int oxq_w8a16_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x, const oxq_
     Wna16Problem p;
     OXQ_TRY(check_wna16(ctx, "W8A16Matmul", KIND_GEMV, x, qweight, qzeros, scales, 8, OXQ_PACK_OUT,
                         out, &p));
+    int crc;
+    if (wcache_forward(ctx, (hipStream_t)stream, p, &crc)) return crc;
     return launch_wna16_gemv(ctx, (hipStream_t)stream, p);
 }
 
@@ -632,6 +798,8 @@ int oxq_gptq_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x, const oxq_t
     Wna16Problem p;
     OXQ_TRY(check_wna16(ctx, "GptqMatmul", KIND_GEMV, x, qweight, qzeros, scales, bits, OXQ_PACK_IN,
                         out, &p));
+    int crc;
+    if (wcache_forward(ctx, (hipStream_t)stream, p, &crc)) return crc;
     return launch_wna16_gemv(ctx, (hipStream_t)stream, p);
 }
 
@@ -667,6 +835,8 @@ int oxq_mpp_quant_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x,
     Wna16Problem p;
     OXQ_TRY(check_wna16(ctx, "MppQuantMatmul", KIND_TILE, x, qweight, qzeros, scales, bits, pack_dim,
                         out, &p));
+    int crc;
+    if (wcache_forward(ctx, (hipStream_t)stream, p, &crc)) return crc;
     return launch_wna16_mfma(ctx, (hipStream_t)stream, p);
 }
 

@@ -23,6 +23,8 @@ struct oxq_ctx {
     int num_cus;
     int splitk_mode;        // 0 auto, 1 fused last-arriver, 2 separate reduce kernel
     oxq_plan plan;
+    struct oxq_weight_cache *wcache;  // tile-major copies the stateless ops made (opt-in), or null
+    size_t wcache_limit;              // bytes the cache may hold; 0 = off
 };
 
 namespace oxq {

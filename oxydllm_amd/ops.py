@@ -90,6 +90,19 @@ class Context:
             return 0
         return torch.cuda.current_stream().cuda_stream
 
+    # opt-in cache of tile-major weight copies behind the stateless ops (see include/oxq.h)
+    def set_weight_cache(self, max_bytes: int) -> None:
+        _lib.check(self._lib.oxq_ctx_set_weight_cache(self.handle, int(max_bytes)))
+
+    def forget_weights(self, qweight: Optional[torch.Tensor] = None) -> None:
+        ptr = C.c_void_p(qweight.data_ptr()) if qweight is not None else C.c_void_p()
+        _lib.check(self._lib.oxq_ctx_forget_weights(self.handle, ptr))
+
+    def weight_cache_usage(self) -> tuple:
+        b, n = C.c_int64(), C.c_int64()
+        _lib.check(self._lib.oxq_ctx_weight_cache_bytes(self.handle, C.byref(b), C.byref(n)))
+        return b.value, n.value
+
 
 _default_ctx: dict = {}
 

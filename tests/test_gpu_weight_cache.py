@@ -1,0 +1,210 @@
+"""GPU tests of the opt-in weight cache behind the stateless ops.
+
+With the cache on, w4a16_matmul / w8a16_matmul / gptq_matmul / mpp_quant_matmul remember their weight
+tensors by address, build the resident layers' tile-major copy on the first call and run the
+resident-layer kernel afterwards.  Checked here:
+  * the result is bit for bit what PackedQuantLinear.forward gives on the same tensors, and within
+    2e-3 relative / 1e-2 absolute of the f32-accumulated oracle;
+  * forgetting, eviction by size and shapes the resident layout does not cover fall back to the
+    checkpoint-layout kernels;
+  * a first call inside a graph capture allocates nothing (it takes the usual path), a warmed call
+    is captured and replays with the eager bits.
+"""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from oxydllm_amd import synth
+from tests.helpers import TORCH_DT, as_f32, assert_close, bits_of, round_x, to_dev
+
+pytestmark = pytest.mark.gpu
+ops = None
+
+
+def setup_module(module):
+    from oxydllm_amd import ops as _ops
+    module.ops = _ops
+
+
+def say(msg):
+    print(f"[case] {msg}", flush=True)
+    sys.stdout.flush()
+
+
+def _trip(kind, K, N, g, seed):
+    bits = 8 if kind.endswith("8") else 4
+    if kind.startswith("awq"):
+        return synth.awq_checkpoint(K, N, g, bits, seed=seed), ops.PACK_OUT, bits
+    return synth.gptq_checkpoint(K, N, g, bits, seed=seed), ops.PACK_IN, bits
+
+
+def _dense(kind, trip, dt):
+    s_r = oracle.round_through(trip[2], dt)
+    if kind == "awq":
+        return oracle.dequantize_awq(trip[0], trip[1], s_r)
+    if kind == "awq8":
+        return oracle.dequantize_awq8(trip[0], trip[1], s_r)
+    return oracle.dequantize_gptq(trip[0], trip[1], s_r, 8 if kind.endswith("8") else 4)
+
+
+def _op(kind, ctx, x, dev, bits, pack_dim, out, tile=False):
+    if tile:
+        return ops.mpp_quant_matmul(x, dev[0], dev[1], dev[2], bits, pack_dim, out=out, ctx=ctx)
+    if kind == "awq":
+        return ops.w4a16_matmul(x, dev[0], dev[1], dev[2], out=out, ctx=ctx)
+    if kind == "awq8":
+        return ops.w8a16_matmul(x, dev[0], dev[1], dev[2], out=out, ctx=ctx)
+    return ops.gptq_matmul(x, dev[0], dev[1], dev[2], bits, out=out, ctx=ctx)
+
+
+@pytest.mark.parametrize("kind", ["awq", "awq8", "gptq", "gptq8"])
+@pytest.mark.parametrize("dtn", ["f16", "bf16"])
+def test_cached_op_equals_resident_layer_and_oracle(kind, dtn):
+    dt = {"f16": oracle.F16, "bf16": oracle.BF16}[dtn]
+    tdt = TORCH_DT[dt]
+    K, N, g = 1024, 512, 128
+    trip, pack_dim, bits = _trip(kind, K, N, g, seed=77)
+    dev = (to_dev(trip[0]), to_dev(trip[1]), to_dev(trip[2], tdt))
+    ctx = ops.Context()
+    layer = ops.PackedQuantLinear(bits, pack_dim, dev[0], dev[1], dev[2], None, tdt, ctx=ctx)
+    assert layer.prepacked
+    w = _dense(kind, trip, dt)
+    try:
+        for m, tile in [(1, False), (5, False), (8, False), (33, True), (64, True)]:
+            say(f"weight cache {kind} {dtn} m={m} tile={tile}")
+            xh = round_x(np.random.default_rng(m).standard_normal((m, K)).astype(np.float32), dt)
+            x = to_dev(xh, tdt)
+            y0 = torch.empty((m, N), device="cuda", dtype=tdt)
+            ctx.set_weight_cache(0)
+            _op(kind, ctx, x, dev, bits, pack_dim, y0, tile)
+            plain = ctx.last_plan()["kernel"]
+            ctx.set_weight_cache(64 << 20)
+            y1 = torch.empty_like(y0)
+            _op(kind, ctx, x, dev, bits, pack_dim, y1, tile)           # builds the copy (or finds it)
+            assert ctx.last_plan()["kernel"].startswith(f"pk{bits}_mfma"), ctx.last_plan()
+            y2 = torch.empty_like(y0)
+            _op(kind, ctx, x, dev, bits, pack_dim, y2, tile)           # served from the copy
+            assert ctx.last_plan()["kernel"].startswith(f"pk{bits}_mfma")
+            assert ctx.last_plan()["launches"] <= 2
+            yl = layer.forward(x)
+            torch.cuda.synchronize()
+            np.testing.assert_array_equal(bits_of(y1), bits_of(yl))
+            np.testing.assert_array_equal(bits_of(y2), bits_of(yl))
+            wk = oracle.round_through(w, dt) if m > 16 else w           # the tile range rounds B once
+            assert_close(y1, oracle.matmul_nt_f32(xh, wk), f"{kind} {dtn} cached m={m} (uncached: {plain})")
+        nbytes, entries = ctx.weight_cache_usage()
+        assert entries == 1 and nbytes >= K * N * bits // 8
+    finally:
+        ctx.close()
+
+
+def test_forget_evict_and_ineligible_shapes():
+    K, N, g = 512, 256, 128
+    tdt = torch.float16
+    ctx = ops.Context()
+    try:
+        trips = [synth.awq_checkpoint(K, N, g, 4, seed=s) for s in (1, 2)]
+        devs = [(to_dev(t[0]), to_dev(t[1]), to_dev(t[2], tdt)) for t in trips]
+        x = torch.randn((2, K), device="cuda", dtype=tdt)
+        y = torch.empty((2, N), device="cuda", dtype=tdt)
+        ref = []
+        for d in devs:
+            ops.w4a16_matmul(x, *d, out=y, ctx=ctx)
+            torch.cuda.synchronize()
+            ref.append(as_f32(y).copy())
+        assert not ctx.last_plan()["kernel"].startswith("pk4")
+
+        one = (K // 128) * (N // 64) * (1024 + 64) * 4          # bytes of one copy
+        say("weight cache: room for one copy, two weights in turn")
+        ctx.set_weight_cache(one + 256)
+        for rnd in range(3):
+            for d, r in zip(devs, ref):
+                ops.w4a16_matmul(x, *d, out=y, ctx=ctx)
+                assert ctx.last_plan()["kernel"].startswith("pk4")
+                torch.cuda.synchronize()
+                np.testing.assert_allclose(as_f32(y), r, rtol=2e-3, atol=1e-2)
+                assert ctx.weight_cache_usage()[1] == 1
+
+        say("weight cache: forget one, forget all")
+        ctx.set_weight_cache(8 * one)
+        for d in devs:
+            ops.w4a16_matmul(x, *d, out=y, ctx=ctx)
+        assert ctx.weight_cache_usage()[1] == 2
+        ctx.forget_weights(devs[0][0])
+        assert ctx.weight_cache_usage()[1] == 1
+        ctx.forget_weights(None)
+        assert ctx.weight_cache_usage() == (0, 0)
+
+        say("weight cache: a new weight at a forgotten address is rebuilt")
+        devs[0][0].copy_(devs[1][0]), devs[0][1].copy_(devs[1][1]), devs[0][2].copy_(devs[1][2])
+        ops.w4a16_matmul(x, *devs[0], out=y, ctx=ctx)
+        torch.cuda.synchronize()
+        np.testing.assert_allclose(as_f32(y), ref[1], rtol=2e-3, atol=1e-2)
+
+        say("weight cache: a shape outside the resident layout keeps its kernel")
+        t3 = synth.awq_checkpoint(256, 96, 64, 4, seed=3)      # group 64, N % 64 != 0
+        d3 = (to_dev(t3[0]), to_dev(t3[1]), to_dev(t3[2], tdt))
+        x3 = torch.randn((1, 256), device="cuda", dtype=tdt)
+        y3 = torch.empty((1, 96), device="cuda", dtype=tdt)
+        before = ctx.weight_cache_usage()
+        ops.w4a16_matmul(x3, *d3, out=y3, ctx=ctx)
+        assert not ctx.last_plan()["kernel"].startswith("pk4")
+        assert ctx.weight_cache_usage() == before
+
+        say("weight cache: a copy larger than the limit is not made")
+        ctx.forget_weights(None)
+        ctx.set_weight_cache(one - 256)
+        ops.w4a16_matmul(x, *devs[1], out=y, ctx=ctx)
+        assert not ctx.last_plan()["kernel"].startswith("pk4")
+        assert ctx.weight_cache_usage() == (0, 0)
+    finally:
+        ctx.close()
+
+
+def test_capture_allocates_nothing_and_replays_the_cached_kernel():
+    K, N, g, m = 2048, 512, 128, 4
+    tdt = torch.float16
+    trip = synth.awq_checkpoint(K, N, g, 4, seed=9)
+    dev = (to_dev(trip[0]), to_dev(trip[1]), to_dev(trip[2], tdt))
+    x = torch.randn((m, K), device="cuda", dtype=tdt)
+    y = torch.empty((m, N), device="cuda", dtype=tdt)
+    ctx = ops.Context()
+    try:
+        ctx.set_weight_cache(64 << 20)
+        ops.w4a16_matmul(x, *dev, out=y, ctx=ctx)                # warm the kernels' one-time set-up
+        ctx.forget_weights(None)
+        stream = torch.cuda.Stream()
+        say("weight cache: first sight of a weight during capture")
+        g1 = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g1, stream=stream):
+            ops.w4a16_matmul(x, *dev, out=y, ctx=ctx)
+            missed = ctx.last_plan()["kernel"]
+        assert not missed.startswith("pk4"), missed
+        assert ctx.weight_cache_usage() == (0, 0)
+
+        ops.w4a16_matmul(x, *dev, out=y, ctx=ctx)                # eager: builds the copy
+        torch.cuda.synchronize()
+        assert ctx.weight_cache_usage()[1] == 1
+        say("weight cache: warmed call captured and replayed")
+        g2 = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g2, stream=stream):
+            ops.w4a16_matmul(x, *dev, out=y, ctx=ctx)
+            assert ctx.last_plan()["kernel"].startswith("pk4")
+        gen = torch.Generator(device="cuda")
+        for i in range(1, 5):
+            gen.manual_seed(i)
+            x.copy_(torch.randn((m, K), device="cuda", dtype=tdt, generator=gen))
+            y.zero_()
+            ops.w4a16_matmul(x, *dev, out=y, ctx=ctx)
+            torch.cuda.synchronize()
+            want = bits_of(y).copy()
+            y.zero_()
+            torch.cuda.synchronize()
+            g2.replay()
+            torch.cuda.synchronize()
+            np.testing.assert_array_equal(bits_of(y), want, err_msg=f"replay {i}")
+    finally:
+        ctx.close()
