@@ -62,6 +62,20 @@ def test_version_and_status_names(lib):
         assert lib.oxq_status_name(code).decode() == name
 
 
+def test_weight_cache_controls_answer_without_a_gpu(lib, ctx):
+    """A plan-only ctx never builds a copy: the controls accept, report an empty cache, and reject
+    what cannot be a size."""
+    assert lib.oxq_ctx_set_weight_cache(ctx, 1 << 30) == 0
+    b, n = C.c_int64(-1), C.c_int64(-1)
+    assert lib.oxq_ctx_weight_cache_bytes(ctx, C.byref(b), C.byref(n)) == 0
+    assert (b.value, n.value) == (0, 0)
+    assert lib.oxq_ctx_forget_weights(ctx, None) == 0
+    assert lib.oxq_ctx_forget_weights(ctx, C.c_void_p(0x1000)) == 0
+    assert lib.oxq_ctx_set_weight_cache(ctx, -1) == -1 and "negative" in err(lib)
+    assert lib.oxq_ctx_set_weight_cache(None, 0) == -1
+    assert lib.oxq_ctx_set_weight_cache(ctx, 0) == 0
+
+
 def test_gguf_block_layout_matches_reference(lib):
     """metal_ops.rs:5228-5241."""
     want = {_lib.GGUF_Q4_0: (32, 18), _lib.GGUF_Q8_0: (32, 34), _lib.GGUF_Q4_K: (256, 144),
