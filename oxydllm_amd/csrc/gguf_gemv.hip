@@ -103,6 +103,22 @@ __global__ __launch_bounds__(256) void gguf_gemv_kernel(const void *__restrict__
 struct __attribute__((packed, aligned(2))) U32A2 { uint32_t v; };
 __device__ __forceinline__ uint32_t ld32a2(const uint8_t *p) { return ((const U32A2 *)p)->v; }
 
+// NDW consecutive dwords from an even address.  Blocks of 18, 22, 34, 110 or 210 bytes put every other
+// block at an address that is 2 mod 4; a 16-byte LDS read from such an address is served in short
+// pieces (Q6_K, four such reads per unit: waves spent a third of their time waiting on LDS).  Aligned
+// dword reads and one funnel shift per dword cost the same LDS cycles as an aligned wide read.
+// Reads one dword past the span when the address is aligned (its value is shifted out).
+template <int NDW>
+__device__ __forceinline__ void ld_span(const uint8_t *p, uint32_t (&out)[NDW]) {
+    const uint32_t mis = (uint32_t)(uintptr_t)p & 2u;
+    const uint32_t *q = (const uint32_t *)(p - mis);
+    uint32_t d[NDW + 1];
+#pragma unroll
+    for (int i = 0; i <= NDW; ++i) d[i] = q[i];
+#pragma unroll
+    for (int i = 0; i < NDW; ++i) out[i] = __builtin_amdgcn_alignbit(d[i + 1], d[i], mis * 8u);
+}
+
 __device__ __forceinline__ void bytes_to_f32(uint32_t w, float *o) {
     o[0] = (float)(w & 0xFFu);
     o[1] = (float)((w >> 8) & 0xFFu);
@@ -119,9 +135,11 @@ __device__ __forceinline__ void unit_ints(const uint8_t *__restrict__ row, int u
     if constexpr (FMT == OXQ_GGUF_Q4_0) {
         const uint8_t *p = row + (size_t)u * 18;
         const float d = ld_f16(p);
+        uint32_t qs[4];
+        ld_span<4>(p + 2, qs);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const uint32_t w = ld32a2(p + 2 + 4 * i);
+            const uint32_t w = qs[i];
             bytes_to_f32(w & 0x0F0F0F0Fu, q + 4 * i);
             bytes_to_f32((w >> 4) & 0x0F0F0F0Fu, q + 16 + 4 * i);
         }
@@ -130,8 +148,10 @@ __device__ __forceinline__ void unit_ints(const uint8_t *__restrict__ row, int u
     } else if constexpr (FMT == OXQ_GGUF_Q8_0) {
         const uint8_t *p = row + (size_t)u * 34;
         const float d = ld_f16(p);
+        uint32_t qs[8];
+        ld_span<8>(p + 2, qs);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) bytes_to_f32(ld32a2(p + 2 + 4 * i) ^ 0x80808080u, q + 4 * i);  // q + 128
+        for (int i = 0; i < 8; ++i) bytes_to_f32(qs[i] ^ 0x80808080u, q + 4 * i);  // q + 128
         a0 = a1 = d;
         b0 = b1 = 128.0f * d;
     } else if constexpr (FMT == OXQ_GGUF_Q4_K) {
@@ -169,10 +189,12 @@ __device__ __forceinline__ void unit_ints(const uint8_t *__restrict__ row, int u
         const uint8_t *p = row + (size_t)u * (MIN ? 24 : 22);
         const float d = ld_f16(p);
         const uint8_t *hp = p + (MIN ? 4 : 2);
-        const uint32_t qh = ld32a2(hp);
+        uint32_t hq[5];
+        ld_span<5>(hp, hq);
+        const uint32_t qh = hq[0];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const uint32_t w = ld32a2(hp + 4 + 4 * i);
+            const uint32_t w = hq[1 + i];
             bytes_to_f32((w & 0x0F0F0F0Fu) | (spread4(qh >> (4 * i)) << 4), q + 4 * i);
             bytes_to_f32(((w >> 4) & 0x0F0F0F0Fu) | (spread4(qh >> (16 + 4 * i)) << 4), q + 16 + 4 * i);
         }
@@ -197,10 +219,13 @@ __device__ __forceinline__ void unit_ints(const uint8_t *__restrict__ row, int u
         const float d = ld_f16(p + 108);
         const uint8_t *qs = p + 32 + (ub >> 2) * 32;
         const int sh = (ub & 3) * 2;
+        uint32_t lw[8], hw[8];
+        ld_span<8>(qs, lw);
+        ld_span<8>(p, hw);
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            const uint32_t lo = (ld32a2(qs + 4 * i) >> sh) & 0x03030303u;
-            const uint32_t hi = ((ld32a2(p + 4 * i) >> ub) & 0x01010101u) << 2;
+            const uint32_t lo = (lw[i] >> sh) & 0x03030303u;
+            const uint32_t hi = ((hw[i] >> ub) & 0x01010101u) << 2;
             bytes_to_f32(lo | hi, q + 4 * i);  // q + 4
         }
         a0 = d * (float)q3k_scale(p + 96, 2 * ub);
@@ -233,10 +258,13 @@ __device__ __forceinline__ void unit_ints(const uint8_t *__restrict__ row, int u
         const float d = ld_f16(p + 208);
         const int shl = (quad < 2) ? 0 : 4;
         const int shh = 2 * quad;
+        uint32_t lw[8], hw[8];
+        ld_span<8>(ql, lw);
+        ld_span<8>(qh, hw);
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            const uint32_t lo = (ld32a2(ql + 4 * i) >> shl) & 0x0F0F0F0Fu;
-            const uint32_t hi = ((ld32a2(qh + 4 * i) >> shh) & 0x03030303u) << 4;
+            const uint32_t lo = (lw[i] >> shl) & 0x0F0F0F0Fu;
+            const uint32_t hi = ((hw[i] >> shh) & 0x03030303u) << 4;
             bytes_to_f32(lo | hi, q + 4 * i);  // q + 32
         }
         a0 = d * (float)scales[8 * h + 2 * quad];
