@@ -31,13 +31,13 @@ template <> struct GgufFmt<OXQ_GGUF_Q5_K> { static constexpr int BE = 256, BB = 
 // get_scale_min_k4 (quant_kernels.metal:2438-2450): the 6-bit scale and minimum of
 // sub-block sb of a Q4_K / Q5_K super-block.
 __device__ __forceinline__ void k4_scale_min(const uint8_t *sc, int sb, uint32_t &scv, uint32_t &mnv) {
-    if (sb < 4) {
-        scv = sc[sb] & 63u;
-        mnv = sc[sb + 4] & 63u;
-    } else {
-        scv = (sc[sb + 4] & 0x0Fu) | ((uint32_t)(sc[sb - 4] >> 6) << 4);
-        mnv = ((uint32_t)sc[sb + 4] >> 4) | ((uint32_t)(sc[sb] >> 6) << 4);
-    }
+    // three byte reads and selects for every sub-block: lanes of one wave hold both kinds, and a
+    // branch would run both sides one after the other
+    const int j = sb & 3;
+    const uint32_t a = sc[j], b = sc[j + 4], c = sc[j + 8];
+    const uint32_t low = sb < 4 ? 0xFFFFFFFFu : 0u;  // bit select, so that no branch comes back
+    scv = ((a & 63u) & low) | (((c & 0x0Fu) | ((a >> 6) << 4)) & ~low);
+    mnv = ((b & 63u) & low) | (((c >> 4) | ((b >> 6) << 4)) & ~low);
 }
 
 // Signed 6-bit scale of sub-block `sub` (0..15) of a Q3_K super-block

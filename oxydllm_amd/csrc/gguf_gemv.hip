@@ -119,7 +119,11 @@ __device__ __forceinline__ void ld_span(const uint8_t *p, uint32_t (&out)[NDW]) 
     for (int i = 0; i < NDW; ++i) out[i] = __builtin_amdgcn_alignbit(d[i + 1], d[i], mis * 8u);
 }
 
+// The empty asm keeps the caller's shift-and-mask of the whole dword apart from the four conversions:
+// merged, the compiler extracts every byte by itself (v_bfe + v_cvt_f32_ubyte0, two instructions a
+// weight); apart, each conversion is one v_cvt_f32_ubyteN.
 __device__ __forceinline__ void bytes_to_f32(uint32_t w, float *o) {
+    asm volatile("" : "+v"(w));
     o[0] = (float)(w & 0xFFu);
     o[1] = (float)((w >> 8) & 0xFFu);
     o[2] = (float)((w >> 16) & 0xFFu);
@@ -158,19 +162,15 @@ __device__ __forceinline__ void unit_ints(const uint8_t *__restrict__ row, int u
         const int b = u >> 3, sb = u & 7;
         const uint8_t *p = row + (size_t)b * 144;
         const float d = ld_f16(p), dmin = ld_f16(p + 2);
-        const uint8_t *sc = p + 4;
         uint32_t scv, mnv;
-        if (sb < 4) {  // get_scale_min_k4
-            scv = sc[sb] & 63u;
-            mnv = sc[sb + 4] & 63u;
-        } else {
-            scv = (sc[sb + 4] & 0x0Fu) | ((uint32_t)(sc[sb - 4] >> 6) << 4);
-            mnv = ((uint32_t)sc[sb + 4] >> 4) | ((uint32_t)(sc[sb] >> 6) << 4);
-        }
-        const uint8_t *qs = p + 16 + (sb >> 1) * 32;
+        k4_scale_min(p + 4, sb, scv, mnv);
+        // 144-byte blocks in rows that start at a multiple of 16: the 32 bytes are two aligned chunks
+        const u32x4_t *qs = (const u32x4_t *)(p + 16 + (sb >> 1) * 32);
+        const u32x4_t q0 = qs[0], q1 = qs[1];
+        const uint32_t qw[8] = {q0[0], q0[1], q0[2], q0[3], q1[0], q1[1], q1[2], q1[3]};
         const int sh = (sb & 1) * 4;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) bytes_to_f32((ld32a2(qs + 4 * i) >> sh) & 0x0F0F0F0Fu, q + 4 * i);
+        for (int i = 0; i < 8; ++i) bytes_to_f32((qw[i] >> sh) & 0x0F0F0F0Fu, q + 4 * i);
         a0 = a1 = d * (float)scv;
         b0 = b1 = dmin * (float)mnv;
     } else if constexpr (FMT == OXQ_GGUF_Q4_1) {
@@ -274,14 +274,16 @@ __device__ __forceinline__ void unit_ints(const uint8_t *__restrict__ row, int u
     }
 }
 
-// Activations sit in LDS as 16-byte chunks, chunk c of unit u at ((c * (units + 1)) + u) * 16:
-// consecutive lanes (units) then read consecutive chunks - with the row-major layout a
-// lane stride of 128 bytes puts a wave's reads on 8 of the 64 banks.
-// 8 consecutive activations (index 8*o .. 8*o+7 of unit u) as f32:
+// Activations sit in LDS unit by unit: the CPU 16-byte chunks of unit u at u * (CPU + 1) * 16, one
+// pad chunk after each unit.  Consecutive lanes (units) then read at a pitch of 144 (f32) or 80 (bf16)
+// bytes, which puts every 8 neighbouring lanes on the 8 different 16-byte bank groups, and a chunk's
+// offset inside its unit is an immediate of the load (one address register a unit).  Behind the
+// activations: the sums of x over every 16 elements (two floats a unit), computed once per workgroup.
+// 8 consecutive activations (index 8*o .. 8*o+7 of the unit at `xu`) as f32:
 template <bool BF16X>
-__device__ __forceinline__ void ld_x8(const unsigned char *xrow, int upitch, int u, int o, float out[8]) {
+__device__ __forceinline__ void ld_x8(const unsigned char *xu, int o, float out[8]) {
     if constexpr (BF16X) {
-        const u32x4_t v = *(const u32x4_t *)(xrow + ((size_t)o * upitch + u) * 16);
+        const u32x4_t v = *(const u32x4_t *)(xu + o * 16);
         const uint32_t v0 = v[0], v1 = v[1], v2 = v[2], v3 = v[3];
         const uint32_t vv[4] = {v0, v1, v2, v3};
 #pragma unroll
@@ -290,8 +292,8 @@ __device__ __forceinline__ void ld_x8(const unsigned char *xrow, int upitch, int
             out[2 * j + 1] = __builtin_bit_cast(float, vv[j] & 0xFFFF0000u);
         }
     } else {
-        const float4_t a = *(const float4_t *)(xrow + ((size_t)(2 * o) * upitch + u) * 16);
-        const float4_t b = *(const float4_t *)(xrow + ((size_t)(2 * o + 1) * upitch + u) * 16);
+        const float4_t a = *(const float4_t *)(xu + (2 * o) * 16);
+        const float4_t b = *(const float4_t *)(xu + (2 * o + 1) * 16);
         out[0] = a[0], out[1] = a[1], out[2] = a[2], out[3] = a[3];
         out[4] = b[0], out[5] = b[1], out[6] = b[2], out[7] = b[3];
     }
@@ -303,7 +305,7 @@ __device__ __forceinline__ void ld_x8(const unsigned char *xrow, int upitch, int
 // + 1.85 us weights + 2.5 us decode and dot, each measured with the others cut out): nobody
 // computes until the last row of the workgroup has arrived.
 template <int FMT, bool BF16X, int MB, bool PW>
-__global__ __launch_bounds__(512) void gguf_gemv_lds_kernel(const void *__restrict__ x,
+__global__ __launch_bounds__(PW ? 1024 : 512) void gguf_gemv_lds_kernel(const void *__restrict__ x,
                                                             const uint8_t *__restrict__ w,
                                                             const void *__restrict__ bias,
                                                             void *__restrict__ y, int M, int K, int N,
@@ -311,8 +313,8 @@ __global__ __launch_bounds__(512) void gguf_gemv_lds_kernel(const void *__restri
     constexpr int XB = BF16X ? 2 : 4;
     extern __shared__ __attribute__((aligned(16))) unsigned char gg_lds[];
     constexpr int CPU = 32 * XB / 16;                                 // 16-byte chunks per unit
-    const int upitch = (K >> 5) + 1;                                  // chunk pitch (units + 1)
-    const size_t xrow_bytes = (size_t)CPU * upitch * 16;
+    constexpr int XP = (CPU + 1) * 16;                                // bytes of one unit's activations + pad
+    const size_t xrow_bytes = ((size_t)(K >> 5) * (XP + 8) + 15) & ~(size_t)15;  // units, then 2 sums a unit
     unsigned char *lds_x = gg_lds;                                   // [MB] chunked activations
     unsigned char *lds_w = gg_lds + (size_t)MB * xrow_bytes;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -330,6 +332,25 @@ __global__ __launch_bounds__(512) void gguf_gemv_lds_kernel(const void *__restri
     // chunks that lie wholly inside the tensor; only the tensor's very last chunk can be partial
     const int full = (int)min((size_t)wchunks, (total_bytes - a0) >> 4);
     const u32x4_t *wsrc = (const u32x4_t *)(w + a0);
+    // sums of x over every 16 elements, once per workgroup (every row's decode needs them: the
+    // offset terms of the formats multiply them); summed in element order
+    auto stage_sums = [&]() {
+        for (int t = threadIdx.x; t < MB * 2 * units; t += nthr) {
+            const int m = MB == 1 ? 0 : t / (2 * units), hu = t - m * 2 * units;
+            if (m < M) {
+                unsigned char *xr = lds_x + m * xrow_bytes;
+                float sx = 0.0f;
+#pragma unroll
+                for (int o = 0; o < 2; ++o) {
+                    float xv[8];
+                    ld_x8<BF16X>(xr + (hu >> 1) * XP, 2 * (hu & 1) + o, xv);
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) sx += xv[i];
+                }
+                ((float *)(xr + (size_t)units * XP))[hu] = sx;
+            }
+        }
+    };
     if constexpr (PW) {
         // one straight-line batch of activation loads, then the wave's own row: the compiler can count
         // the younger loads, so storing the activations leaves the weights in flight
@@ -355,9 +376,11 @@ __global__ __launch_bounds__(512) void gguf_gemv_lds_kernel(const void *__restri
         for (int b = 0; b < CB; ++b) {
             const int g = (int)threadIdx.x + b * nthr;
             const int u = g / CPU, cc = g - u * CPU;
-            *(u32x4_t *)(lds_x + (size_t)(g < cpr ? cc * upitch + u : units) * 16) = xv[b];
+            *(u32x4_t *)(lds_x + (g < cpr ? u * XP + cc * 16 : CPU * 16)) = xv[b];  // else: unit 0's pad
         }
         __syncthreads();
+        stage_sums();
+        __syncthreads();  // both barriers come before the wait for the wave's own weight row
 #pragma unroll
         for (int q = 0; q < WCH; ++q) {
             const int c = wc0 + lane + 64 * q;
@@ -411,12 +434,14 @@ __global__ __launch_bounds__(512) void gguf_gemv_lds_kernel(const void *__restri
                     const int g = base + b * nthr;
                     if (g < cpr) {
                         const int u = g / CPU, cc = g - u * CPU;  // CPU is a power of two
-                        *(u32x4_t *)(xdst + ((size_t)cc * upitch + u) * 16) = v[b];
+                        *(u32x4_t *)(xdst + (size_t)u * XP + cc * 16) = v[b];
                     }
                 }
             }
         }
     }
+    __syncthreads();
+    stage_sums();
     __syncthreads();
     }
     for (int r = wave; r < nrows; r += nwaves) {
@@ -425,29 +450,32 @@ __global__ __launch_bounds__(512) void gguf_gemv_lds_kernel(const void *__restri
         float acc[MB];
 #pragma unroll
         for (int m = 0; m < MB; ++m) acc[m] = 0.0f;
-        for (int u = lane; u < units; u += 64) {
+        // unit `u` of the row against every activation row
+        auto add_unit = [&](int u) {
             float q[32], c0, c1, d0, d1;
             unit_ints<FMT>(row, u, q, c0, c1, d0, d1);
 #pragma unroll
             for (int m = 0; m < MB; ++m) {
                 if (m < M) {
-                    // the sums of x over each half of the unit ride along with the dot products: the
-                    // lane reads these 32 activations anyway, and a separate pass would cost a barrier
-                    float dot0 = 0.0f, dot1 = 0.0f, sx0 = 0.0f, sx1 = 0.0f;
+                    const unsigned char *xr = lds_x + m * xrow_bytes;
+                    const unsigned char *xu = xr + u * XP;
+                    const float2 sx = *(const float2 *)(xr + (size_t)units * XP + u * 8);
+                    float dot0 = 0.0f, dot1 = 0.0f;
 #pragma unroll
                     for (int o = 0; o < 4; ++o) {
                         float xv[8];
-                        ld_x8<BF16X>(lds_x + m * xrow_bytes, upitch, u, o, xv);
+                        ld_x8<BF16X>(xu, o, xv);
 #pragma unroll
                         for (int i = 0; i < 8; ++i) {
-                            if (o < 2) dot0 = fmaf(q[8 * o + i], xv[i], dot0), sx0 += xv[i];
-                            else dot1 = fmaf(q[8 * o + i], xv[i], dot1), sx1 += xv[i];
+                            if (o < 2) dot0 = fmaf(q[8 * o + i], xv[i], dot0);
+                            else dot1 = fmaf(q[8 * o + i], xv[i], dot1);
                         }
                     }
-                    acc[m] += (c0 * dot0 + c1 * dot1) - (d0 * sx0 + d1 * sx1);
+                    acc[m] += (c0 * dot0 + c1 * dot1) - (d0 * sx.x + d1 * sx.y);
                 }
             }
-        }
+        };
+        for (int u = lane; u < units; u += 64) add_unit(u);
 #pragma unroll
         for (int m = 0; m < MB; ++m) {
             if (m < M) {
@@ -518,8 +546,9 @@ static int launch_rows_lds_mb(hipStream_t s, const GgufProblem &p, const uint8_t
     OXQ_HIP_CHECK(lds_grant.ensure((const void *)gguf_gemv_lds_kernel<FMT, BF16X, MB, PW>, lds));
     const int K = (int)p.K, N = (int)p.N;
     const size_t total = (size_t)N * (size_t)(K / GgufFmt<FMT>::BE) * GgufFmt<FMT>::BB;
-    // one wave per row at a time: 8 waves for 8 rows (x is staged once per 8 rows), else 4
-    dim3 grid((unsigned)ceil_div(N, rpwg)), block(rpwg >= 8 ? 512 : 256);
+    // one wave per row at a time: 8 waves for 8 rows (x is staged once per 8 rows), else 4; the
+    // wave-per-row form also runs 16 rows on 16 waves
+    dim3 grid((unsigned)ceil_div(N, rpwg)), block(PW && rpwg >= 16 ? 1024 : rpwg >= 8 ? 512 : 256);
     hipLaunchKernelGGL((gguf_gemv_lds_kernel<FMT, BF16X, MB, PW>), grid, block, lds, s, x, p.w, p.bias, y, rows, K,
                        N, rpwg, total);
     return OXQ_OK;
@@ -532,8 +561,8 @@ static int launch_rows_lds(hipStream_t s, const GgufProblem &p, const uint8_t *x
         // a wave per weight row needs: 8 waves for the 8 rows, the row in 6 chunks a lane, x in one batch
         const size_t row_bytes = (size_t)(p.K / GgufFmt<FMT>::BE) * GgufFmt<FMT>::BB;
         const char *pw_env = getenv("OXQ_GGUF_PW");
-        if (rpwg == 8 && row_bytes + 30 <= 6 * 64 * 16 && p.K * (BF16X ? 2 : 4) / 16 <= 4 * 512 &&
-            !(pw_env && atoi(pw_env) == 0))
+        if ((rpwg == 8 || rpwg == 16) && row_bytes + 30 <= 6 * 64 * 16 &&
+            p.K * (BF16X ? 2 : 4) / 16 <= 4 * 64 * rpwg && !(pw_env && atoi(pw_env) == 0))
             return launch_rows_lds_mb<FMT, BF16X, 1, true>(s, p, x, y, rows, rpwg, lds);
         return launch_rows_lds_mb<FMT, BF16X, 1>(s, p, x, y, rows, rpwg, lds);
     }
@@ -555,19 +584,27 @@ int launch_gguf_gemv(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p) {
     // LDS variant: activations of one chunk of rows plus `rpwg` weight rows must fit 64 KB
     const int64_t mrows = p.M < 8 ? p.M : 8;
     const int mb = mrows <= 1 ? 1 : mrows <= 2 ? 2 : mrows <= 4 ? 4 : 8;
-    const size_t x_lds = (size_t)mb * (32 * xb / 16) * (size_t)((p.K >> 5) + 1) * 16;
+    // per activation row: K/32 units of 32 elements + one 16-byte pad each, then two sums a unit
+    const size_t x_lds = (size_t)mb * ((((size_t)(p.K >> 5) * ((32 * xb / 16 + 1) * 16 + 8)) + 15) & ~(size_t)15);
     const size_t row_bytes = gguf_row_bytes(p.quant, p.K);
     const char *rp_env = getenv("OXQ_GGUF_RPWG");
-    int rpwg = rp_env ? atoi(rp_env) : 8;  // measured 4096^2, Q4_K: 8 rows x 8 waves 7.5 us, 4 x 4 8.1, 16 x 8 8.8
+    // 8 rows on 8 waves.  For one activation row OXQ_GGUF_RPWG=16 runs 16 rows on 16 waves, which halves
+    // the activation traffic (every workgroup stages all of x); measured slower on 4096 x 4096 (Q4_0 5.5
+    // against 5.1 us, Q6_K 6.8 against 6.0 us): one workgroup per CU starts its weight loads later.
+    const char *pw_env = getenv("OXQ_GGUF_PW");
+    const bool wave_per_row = p.M == 1 && row_bytes + 30 <= 6 * 64 * 16 && !(pw_env && atoi(pw_env) == 0);
+    int rpwg = rp_env ? atoi(rp_env) : 8;
     if (rpwg < 1) rpwg = 1;
-    while (rpwg > 1 && x_lds + (size_t)rpwg * row_bytes + 32 > 64 * 1024) rpwg >>= 1;
-    const size_t lds = x_lds + (size_t)rpwg * row_bytes + 32;
+    if (rpwg > 8 && !(wave_per_row && rpwg == 16 && p.K * (int64_t)xb / 16 <= 4 * 64 * 16)) rpwg = 8;
+    auto lds_cap_of = [](int r) { return (size_t)(r == 16 ? 128 : 64) * 1024; };
+    while (rpwg > 1 && x_lds + (size_t)rpwg * row_bytes + 32 > lds_cap_of(rpwg)) rpwg >>= 1;
+    const size_t lds = x_lds + (size_t)rpwg * row_bytes + 32, lds_cap = lds_cap_of(rpwg);
     const char *force = getenv("OXQ_FORCE_GENERIC");
-    const bool use_lds = lds <= 64 * 1024 && ((uintptr_t)p.x & 15) == 0 && ((uintptr_t)p.w & 15) == 0 &&
+    const bool use_lds = lds <= lds_cap && ((uintptr_t)p.x & 15) == 0 && ((uintptr_t)p.w & 15) == 0 &&
                          (p.K * xb) % 16 == 0 && !(force && atoi(force));
     char name[64];
     snprintf(name, sizeof name, "gguf_%s_gemv_%s%s", fmt_name(p.quant), bf ? "bf16" : "f32", use_lds ? "_lds" : "");
-    dim3 grid((unsigned)(use_lds ? ceil_div(p.N, rpwg) : ceil_div(p.N, 4))), block(use_lds && rpwg >= 8 ? 512 : 256);
+    dim3 grid((unsigned)(use_lds ? ceil_div(p.N, rpwg) : ceil_div(p.N, 4))), block(use_lds && rpwg >= 16 ? 1024 : use_lds && rpwg >= 8 ? 512 : 256);
     set_plan(ctx, name, grid, block, 1, chunks, 0);
     if (ctx->plan_only) return OXQ_OK;
     // m > 8: activation rows are processed 8 at a time (the weight is re-read
