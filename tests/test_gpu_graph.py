@@ -148,3 +148,34 @@ def test_fused_epilogues_and_workspace_repack_in_a_graph():
     replay_matches_eager("mxfp4 gate_up + swiglu",
                          lambda: ops.mxfp4_moe_gate_up_swiglu(x, blocks, scales, None, offsets, tok, Kx, N, 7.0, out=y),
                          inputs, y)
+
+
+def test_resident_experts_in_a_graph():
+    """The MoE decode step on resident experts: gate_up with the SwiGLU in its epilogue, then down,
+    captured together; the token lists stay, the activations change between replays."""
+    gen = torch.Generator(device="cuda")
+    E, H, I = 4, 128, 96
+    gu = [synth.mxfp4_weight(2 * I, H, seed=10 + e) for e in range(E)]
+    dn = [synth.mxfp4_weight(H, I, seed=20 + e) for e in range(E)]
+    gub = torch.from_numpy(np.concatenate([g[0] for g in gu])).cuda(), torch.from_numpy(np.concatenate([g[1] for g in gu])).cuda()
+    dnb = torch.from_numpy(np.concatenate([d[0] for d in dn])).cuda(), torch.from_numpy(np.concatenate([d[1] for d in dn])).cuda()
+    gu_bias = (torch.randn((E, 2 * I), device="cuda") * 0.1).to(torch.bfloat16)
+    dn_bias = (torch.randn((E, H), device="cuda") * 0.1).to(torch.bfloat16)
+    gu_ex = ops.Mxfp4Experts(gub[0], gub[1], gu_bias, E, H, 2 * I)
+    dn_ex = ops.Mxfp4Experts(dnb[0], dnb[1], dn_bias, E, I, H)
+    assert gu_ex.resident and dn_ex.resident
+    offsets = to_dev(np.array([0, 3, 3, 4, 6], np.int32))
+    tok = to_dev(np.array([0, 1, 2, 1, 0, 2], np.int32))
+    x = torch.empty((3, H), device="cuda", dtype=torch.bfloat16)
+    h = torch.empty((6, I), device="cuda", dtype=torch.bfloat16)
+    y = torch.empty((6, H), device="cuda", dtype=torch.bfloat16)
+
+    def inputs(i):
+        gen.manual_seed(600 + i)
+        x.copy_(torch.randn((3, H), device="cuda", generator=gen).to(torch.bfloat16))
+
+    def step():
+        gu_ex.gate_up_swiglu(x, offsets, tok, 7.0, out=h)
+        assert ops.default_context().last_plan()["kernel"].startswith("mxfp4_experts_gemv")
+        dn_ex.matmul(h, offsets, None, out=y)
+    replay_matches_eager("resident experts: gate_up + swiglu, down", step, inputs, y)
