@@ -590,7 +590,7 @@ int launch_gguf_gemv(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p) {
     const char *rp_env = getenv("OXQ_GGUF_RPWG");
     // 8 rows on 8 waves.  For one activation row OXQ_GGUF_RPWG=16 runs 16 rows on 16 waves, which halves
     // the activation traffic (every workgroup stages all of x); measured slower on 4096 x 4096 (Q4_0 5.5
-    // against 5.1 us, Q6_K 6.8 against 6.0 us): one workgroup per CU starts its weight loads later.
+    // against 5.1 us, Q6_K 6.8 against 6.0 us); 16 rows on 8 waves of two rows each: 6.0 and 7.5 us.
     const char *pw_env = getenv("OXQ_GGUF_PW");
     const bool wave_per_row = p.M == 1 && row_bytes + 30 <= 6 * 64 * 16 && !(pw_env && atoi(pw_env) == 0);
     int rpwg = rp_env ? atoi(rp_env) : 8;
