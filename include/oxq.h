@@ -124,7 +124,7 @@ void oxq_version(int *major, int *minor);
  * oxq_mpp_quant_matmul remember a (qweight, qzeros, scales) triple by its device addresses: the first
  * call builds the tile-major copy that oxq_packed_quant_linear_new builds (one extra launch and a
  * hipMalloc; skipped while the stream is being captured, where the call takes its usual path) and
- * later calls run the resident-layer kernel on it, with that layer's arithmetic (m <= 16: unrounded
+ * later calls run the resident-layer kernel on it, with that layer's arithmetic (few rows: unrounded
  * weights, f32 fold; above: tile GEMM on weights rounded to the activation type).  Shapes the
  * resident layout does not cover take the usual path.  The copy costs the packed tensors' size
  * again; least recently used copies go when max_bytes is reached.

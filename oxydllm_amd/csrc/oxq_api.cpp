@@ -659,7 +659,8 @@ static bool wcache_forward(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p, i
             return false;
         }
         oxq_weight_cache::Entry e{p.qweight, p.qzeros, p.scales, p.K, p.N, p.group_shift, p.dtype, p.bits, p.pack_dim,
-                                  Pk4Weights{(uint32_t *)mem, nullptr, p.K, p.N, p.group_shift, p.dtype, p.bits, 0},
+                                  Pk4Weights{(uint32_t *)mem, nullptr, p.K, p.N, p.group_shift, p.dtype, p.bits, 0,
+                                             p.pack_dim == OXQ_PACK_IN ? 32 : 16},
                                   bytes, 0};
         const int prc = launch_pk4_prepack(ctx, s, p, e.w);  // on the caller's stream, ahead of the matmul
         if (prc != OXQ_OK) {
@@ -1672,6 +1673,7 @@ static int prepack_layer(oxq_packed_quant_linear *l) {
     l->pk.dtype = l->dtype;
     l->pk.bits = src.bits;
     l->pk.gate_half = l->act ? src.N / 2 : 0;
+    l->pk.gemv_rows = src.pack_dim == OXQ_PACK_IN ? 32 : 16;
     if (ctx->plan_only) {
         l->prepacked = true;
         return OXQ_OK;

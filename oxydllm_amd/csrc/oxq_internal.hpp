@@ -157,6 +157,8 @@ struct Pk4Weights {
     int bits;               // 4 or 8
     int64_t gate_half;      // 0, or N/2 for a fused gate|up layer: strip j holds gate columns
                             // [32j, 32j+32) then up columns [N/2 + 32j, N/2 + 32j + 32)
+    int gemv_rows;          // rows up to which the reference runs its fused GEMV, which never rounds the
+                            // dequantized weight (linear.rs:450-480: 16 AWQ, 32 GPTQ); 0 = 16
 };
 
 struct Pk4Problem {

@@ -668,12 +668,29 @@ static int pk4_go(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, i
     return pk4_go4<TT, BITS, MT, GS, 4 * MT>(ctx, s, grid, p, bslice);
 }
 
+// Which form multiplies.  The folded form (exact integers through the matrix cores, scale and
+// zero applied per block in f32: the weight is never rounded) is what the reference's fused GEMV
+// computes, so it serves that kernel's range of m: 16 rows for AWQ, 32 for GPTQ (gemv_rows).
+// Above, the reference's tile GEMM rounds the dequantized weight to the activation type: bf16
+// layers keep that (tile form); for f16 the rounding is 2^-12 of a weight, far inside the
+// tolerance either way, and the folded form is the faster one up to three row tiles
+// (4096 x 14336 f16: 17 rows 10.8 -> 9.9 us, 48 rows 14.3 -> 13.5 us; bf16 GPTQ 17 rows 13.3 -> 10.1 us).
+// At four row tiles the fold costs what the dequant costs and its extra accumulators do not fit.
+static bool pk4_folds(const Pk4Problem &p, int mt) {
+    if (mt == 1) return true;
+    if (mt > 3 || !pk4_env("OXQ_PK4_FOLD", 1)) return false;
+    const int gemv_rows = p.w.gemv_rows ? p.w.gemv_rows : 16;
+    if (p.w.dtype == OXQ_F16) return true;
+    return mt == 2 && p.M <= gemv_rows;
+}
+
 template <typename TT, int BITS>
 static int pk4_by_mt(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, int bslice, int mt) {
+    const bool fold = pk4_folds(p, mt);
     switch (mt) {
     case 1: return pk4_go<TT, BITS, 1, true>(ctx, s, grid, p, bslice);
-    case 2: return pk4_go<TT, BITS, 2, false>(ctx, s, grid, p, bslice);
-    case 3: return pk4_go<TT, BITS, 3, false>(ctx, s, grid, p, bslice);
+    case 2: return fold ? pk4_go<TT, BITS, 2, true>(ctx, s, grid, p, bslice) : pk4_go<TT, BITS, 2, false>(ctx, s, grid, p, bslice);
+    case 3: return fold ? pk4_go<TT, BITS, 3, true>(ctx, s, grid, p, bslice) : pk4_go<TT, BITS, 3, false>(ctx, s, grid, p, bslice);
     default: return pk4_go<TT, BITS, 4, false>(ctx, s, grid, p, bslice);
     }
 }
@@ -704,7 +721,7 @@ int launch_pk4_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p) {
     if (p.act && (!p.w.gate_half || p.act > 2))
         return fail(OXQ_ERR_ARG, "repacked matmul: activation %d on a layer that is not a fused gate|up layer", p.act);
     snprintf(name, sizeof name, "pk%d_mfma_%s_mt%d%s%s", p.w.bits, p.w.dtype == OXQ_F16 ? "f16" : "bf16", mt,
-             mt == 1 ? "_gs" : "", p.act == 1 ? "_silu" : p.act == 2 ? "_gelu" : "");
+             pk4_folds(p, mt) ? "_gs" : "", p.act == 1 ? "_silu" : p.act == 2 ? "_gelu" : "");
     set_plan(ctx, name, grid, dim3(512), ks, 1, ks > 1 ? (size_t)ks * M * p.w.N * 4 : 0);
     if (ctx->plan_only) {
         if (ks > 1) add_launch(ctx);

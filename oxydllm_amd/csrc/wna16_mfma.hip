@@ -710,7 +710,8 @@ int launch_wna16_mfma(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p) {
         !env_int("OXQ_FORCE_GENERIC", 0)) {
         const size_t wb = (pk4_weight_bytes(p.K, p.N, p.bits) + 255) & ~(size_t)255;
         if (wb <= ctx->workspace_bytes) {
-            Pk4Weights w{(uint32_t *)ctx->workspace, nullptr, p.K, p.N, p.group_shift, p.dtype, p.bits, 0};
+            Pk4Weights w{(uint32_t *)ctx->workspace, nullptr, p.K, p.N, p.group_shift, p.dtype, p.bits, 0,
+                           p.pack_dim == OXQ_PACK_IN ? 32 : 16};
             int rc = launch_pk4_prepack(ctx, s, p, w);
             if (rc != OXQ_OK) return rc;
             Pk4Problem q;

@@ -68,6 +68,19 @@ def assert_close(got, ref: np.ndarray, what="", rtol=RTOL, atol=ATOL, bf16_out=N
                            f"max err {err.max():.3e} at ref {ref.flat[err.argmax()]:.4f}")
 
 
+def resident_rounds_weights(m: int, dt: int, gptq: bool) -> bool:
+    """Whether a resident layer multiplies the dequantized weight rounded to the activation type at m
+    rows (the reference's tile GEMM stages it so, mpp_gemm.metal:115-184) or unrounded (its fused GEMV,
+    which serves up to 16 rows for AWQ and 32 for GPTQ, linear.rs:450-480).  f16 layers keep the
+    unrounded form up to 48 rows: rounding to f16 moves a weight by 2^-12, inside the tolerance."""
+    import oracle
+    if m <= 16:
+        return False
+    if dt == oracle.F16:
+        return m > 48
+    return not (gptq and m <= 32)
+
+
 def round_x(x_f32: np.ndarray, dt: int) -> np.ndarray:
     """The activation values the kernel actually sees (x rounded to its 16-bit dtype)."""
     return oracle.round_through(x_f32, dt)

@@ -13,7 +13,7 @@ from oxydllm_amd import checkpoint as ck
 from oxydllm_amd import ops, synth
 from tests import ggufio as G
 from tests import refgen
-from tests.helpers import as_f32, assert_close, round_x, to_dev
+from tests.helpers import as_f32, assert_close, round_x, to_dev, resident_rounds_weights
 
 pytestmark = pytest.mark.gpu
 
@@ -81,7 +81,7 @@ def test_safetensors_file_to_packed_linear(tmp_path, method, bits):
         for m in (1, 7, 40):
             x = _x(m, K, seed=m)
             y = layer.forward(to_dev(x, torch.float16))
-            wr = wt if m <= 16 else oracle.round_through(wt, oracle.F16)
+            wr = oracle.round_through(wt, oracle.F16) if resident_rounds_weights(m, oracle.F16, method == "gptq") else wt
             ref = oracle.matmul_nt_f32(round_x(x, oracle.F16), wr, bias.astype(np.float32))
             assert_close(y, ref, f"{method}{bits} m={m}")
         assert w.try_get_quant("model.layers.1.mlp.gate_proj") is None

@@ -19,7 +19,7 @@ import torch
 import oracle
 from oxydllm_amd import synth
 from tests import refgen
-from tests.helpers import TORCH_DT, as_f32, assert_close, bits_of, round_x, to_dev
+from tests.helpers import TORCH_DT, as_f32, assert_close, bits_of, resident_rounds_weights, round_x, to_dev
 
 pytestmark = pytest.mark.gpu
 ops = None
@@ -117,7 +117,7 @@ def test_repacked_forward_all_m(kind, dtn, K, N, g):
         ref = oracle.matmul_nt_f32(round_x(x, dt), w, bias)
         y = layer.forward(to_dev(x, TORCH_DT[dt]))
         assert y.shape == (m, N)
-        if m <= 16:
+        if not resident_rounds_weights(m, dt, kind.startswith("gptq")):
             # the fused-GEMV range: the dequantized weight is never rounded
             assert_close(y, ref, f"pk4 {kind} {dtn} m{m}")
         else:
@@ -154,7 +154,7 @@ def test_repacked_forward_k_slices(kind, dtn, K, N, g, ks, monkeypatch):
         y = layer.forward(xd)
         plan = ops.default_context().last_plan()
         assert plan["split_k"] == -(-groups // per) and plan["launches"] == 2
-        wr = w if m <= 16 else oracle.round_through(w, dt)
+        wr = oracle.round_through(w, dt) if resident_rounds_weights(m, dt, kind.startswith("gptq")) else w
         assert_close(y, oracle.matmul_nt_f32(round_x(x, dt), wr, bias), f"pk4 k-slices m{m}")
         np.testing.assert_array_equal(bits_of(layer.forward(xd)), bits_of(y))
 
@@ -212,7 +212,7 @@ def test_repacked_forward_config2_gptq(bits):
     for m in (1, 8, 24):
         say(f"pk4 forward config2 m={m}")
         x = np.random.default_rng(40 + m).standard_normal((m, K)).astype(np.float32)
-        wr = w if m <= 16 else oracle.round_through(w, dt)
+        wr = oracle.round_through(w, dt) if resident_rounds_weights(m, dt, True) else w
         ref = oracle.matmul_nt_f32(round_x(x, dt), wr)
         assert_close(layer.forward(to_dev(x, torch.bfloat16)), ref, f"pk{bits} config2 m{m}", bf16_out=True)
 
@@ -288,7 +288,7 @@ def test_fused_gate_up_activation(kind, dtn, act, K, I, g):
             # the projection itself against the oracle matmul, then the activation on the projection's
             # own 16-bit output (a last-place difference in a factor would otherwise be amplified by
             # the gate function's slope: |g|^2 ulp in GeLU's tail)
-            wr = w if m <= 16 else oracle.round_through(w, dt)
+            wr = oracle.round_through(w, dt) if resident_rounds_weights(m, dt, kind.startswith("gptq")) else w
             assert_close(gu, oracle.matmul_nt_f32(round_x(x, dt), wr, b), f"gate|up projection {kind} {dtn} m{m}")
             ref = oracle.gated_silu(as_f32(gu)) if act == "silu" else oracle.gated_gelu_tanh(as_f32(gu))
             assert_close(y, ref, f"gate|up {kind} {dtn} {act} m{m}")

@@ -12,7 +12,7 @@ import torch
 
 import oracle
 from oxydllm_amd import ops, synth
-from tests.helpers import assert_close, round_x, to_dev
+from tests.helpers import assert_close, round_x, to_dev, resident_rounds_weights
 
 pytestmark = pytest.mark.gpu
 
@@ -101,6 +101,6 @@ def test_resident_layer_random_shapes(monkeypatch):
         x = rng.standard_normal((M, K)).astype(np.float32)
         y = layer.forward(to_dev(x, tdt))
         plan = ops.default_context().last_plan()
-        wr = w if M <= 16 else oracle.round_through(w, dt)
+        wr = oracle.round_through(w, dt) if resident_rounds_weights(M, dt, bool(gptq)) else w
         ref = oracle.matmul_nt_f32(round_x(x, dt), wr)
         assert_close(y, ref, f"pk{bits} gptq={gptq} M{M} N{N} K{K} g{g} ks{plan['split_k']} {plan['kernel']}")

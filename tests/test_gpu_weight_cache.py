@@ -18,7 +18,7 @@ import torch
 
 import oracle
 from oxydllm_amd import synth
-from tests.helpers import TORCH_DT, as_f32, assert_close, bits_of, round_x, to_dev
+from tests.helpers import TORCH_DT, as_f32, assert_close, bits_of, resident_rounds_weights, round_x, to_dev
 
 pytestmark = pytest.mark.gpu
 ops = None
@@ -93,7 +93,7 @@ def test_cached_op_equals_resident_layer_and_oracle(kind, dtn):
             torch.cuda.synchronize()
             np.testing.assert_array_equal(bits_of(y1), bits_of(yl))
             np.testing.assert_array_equal(bits_of(y2), bits_of(yl))
-            wk = oracle.round_through(w, dt) if m > 16 else w           # the tile range rounds B once
+            wk = oracle.round_through(w, dt) if resident_rounds_weights(m, dt, kind.startswith("gptq")) else w
             assert_close(y1, oracle.matmul_nt_f32(xh, wk), f"{kind} {dtn} cached m={m} (uncached: {plain})")
         nbytes, entries = ctx.weight_cache_usage()
         assert entries == 1 and nbytes >= K * N * bits // 8

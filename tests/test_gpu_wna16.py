@@ -18,7 +18,7 @@ import torch
 import oracle
 from oxydllm_amd import synth
 from tests import refgen
-from tests.helpers import RTOL, ATOL, TORCH_DT, as_f32, assert_close, bits_of, round_x, to_dev
+from tests.helpers import RTOL, ATOL, TORCH_DT, as_f32, assert_close, bits_of, round_x, to_dev, resident_rounds_weights
 
 pytestmark = pytest.mark.gpu
 ops = None
@@ -410,7 +410,7 @@ def test_stateless_tile_op_on_layouts_without_a_tile_kernel(method, bits, dtn, m
         y = ops.mpp_quant_matmul(xd, *d, bits, pd)
         plan = ops.default_context().last_plan()
         assert plan["kernel"].startswith(f"pk{bits}_mfma_{dtn}") and plan["launches"] == 2, plan
-        wr = w if m <= 16 else oracle.round_through(w, dt)
+        wr = oracle.round_through(w, dt) if resident_rounds_weights(m, dt, method == "gptq") else w
         assert_close(y, oracle.matmul_nt_f32(round_x(x, dt), wr), f"{method}{bits} {dtn} m{m} (repacked in the workspace)")
         monkeypatch.setenv("OXQ_TRANSIENT_REPACK", "0")
         y2 = ops.mpp_quant_matmul(xd, *d, bits, pd)
