@@ -133,7 +133,7 @@ template <int FMT> struct GgufSource {
         uint32_t o[16], ol[16];
         if (s * 8 + u < units) {
             float wf[32];
-            decode_unit<FMT>(raw + dr * RAWP + head, u, wf);
+            decode_unit<FMT, true>(raw + dr * RAWP + head, u, wf);  // LDS: block bytes as aligned dwords
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 o[i] = pack_bf16(wf[2 * i], wf[2 * i + 1]);

@@ -28,6 +28,36 @@ template <> struct GgufFmt<OXQ_GGUF_Q2_K> { static constexpr int BE = 256, BB = 
 template <> struct GgufFmt<OXQ_GGUF_Q3_K> { static constexpr int BE = 256, BB = 110; };
 template <> struct GgufFmt<OXQ_GGUF_Q5_K> { static constexpr int BE = 256, BB = 176; };
 
+// NDW consecutive dwords from an even address.  Blocks of 18, 22, 34, 110 or 210 bytes put every other
+// block at an address that is 2 mod 4; a 16-byte LDS read from such an address is served in short
+// pieces (Q6_K, four such reads per unit: waves spent a third of their time waiting on LDS).  Aligned
+// dword reads and one funnel shift per dword cost the same LDS cycles as an aligned wide read.
+// Reads one dword past the span when the address is aligned (its value is shifted out).
+template <int NDW>
+__device__ __forceinline__ void ld_span(const uint8_t *p, uint32_t (&out)[NDW]) {
+    const uint32_t mis = (uint32_t)(uintptr_t)p & 2u;
+    const uint32_t *q = (const uint32_t *)(p - mis);
+    uint32_t d[NDW + 1];
+#pragma unroll
+    for (int i = 0; i <= NDW; ++i) d[i] = q[i];
+#pragma unroll
+    for (int i = 0; i < NDW; ++i) out[i] = __builtin_amdgcn_alignbit(d[i + 1], d[i], mis * 8u);
+}
+
+// 16-bit pieces of a span of NDW dwords that starts at an even address: read one by one (any memory),
+// or - SPAN, LDS only, since it reads up to four bytes past the span - fetched at once with ld_span.
+template <int NDW, bool SPAN> struct Halves {
+    uint32_t d[SPAN ? NDW : 1];
+    const uint8_t *p;
+    __device__ __forceinline__ explicit Halves(const uint8_t *p_) : p(p_) {
+        if constexpr (SPAN) ld_span<NDW>(p_, d);
+    }
+    __device__ __forceinline__ uint32_t h(int i) const {
+        if constexpr (SPAN) return (d[i >> 1] >> (16 * (i & 1))) & 0xFFFFu;
+        else return ld16(p + 2 * i);
+    }
+};
+
 // get_scale_min_k4 (quant_kernels.metal:2438-2450): the 6-bit scale and minimum of
 // sub-block sb of a Q4_K / Q5_K super-block.
 __device__ __forceinline__ void k4_scale_min(const uint8_t *sc, int sb, uint32_t &scv, uint32_t &mnv) {
@@ -53,14 +83,15 @@ __device__ __forceinline__ int q3k_scale(const uint8_t *scales, int sub) {
 __device__ __forceinline__ uint32_t spread4(uint32_t v) { return ((v & 0xFu) * 0x00204081u) & 0x01010101u; }
 
 // Decode unit `u` (32 elements) of the row starting at `row` into w[0..31].
-template <int FMT>
+template <int FMT, bool SPAN = false>
 __device__ __forceinline__ void decode_unit(const uint8_t *__restrict__ row, int u, float w[32]) {
     if constexpr (FMT == OXQ_GGUF_Q4_0) {
         const uint8_t *p = row + (size_t)u * 18;
         const float d = ld_f16(p);
+        const Halves<4, SPAN> qs(p + 2);
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            const uint32_t q = ld16(p + 2 + 2 * i);  // bytes 2i, 2i+1
+            const uint32_t q = qs.h(i);  // bytes 2i, 2i+1
             w[2 * i] = (float)((int)(q & 0xF) - 8) * d;
             w[2 * i + 16] = (float)((int)((q >> 4) & 0xF) - 8) * d;
             w[2 * i + 1] = (float)((int)((q >> 8) & 0xF) - 8) * d;
@@ -69,9 +100,10 @@ __device__ __forceinline__ void decode_unit(const uint8_t *__restrict__ row, int
     } else if constexpr (FMT == OXQ_GGUF_Q8_0) {
         const uint8_t *p = row + (size_t)u * 34;
         const float d = ld_f16(p);
+        const Halves<8, SPAN> qs(p + 2);
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            const uint32_t q = ld16(p + 2 + 2 * i);
+            const uint32_t q = qs.h(i);
             w[2 * i] = (float)(int)(int8_t)(q & 0xFF) * d;
             w[2 * i + 1] = (float)(int)(int8_t)(q >> 8) * d;
         }
@@ -114,10 +146,11 @@ __device__ __forceinline__ void decode_unit(const uint8_t *__restrict__ row, int
         const uint8_t *p = row + (size_t)u * (MIN ? 24 : 22);
         const float d = ld_f16(p), m = MIN ? ld_f16(p + 2) : 0.0f;
         const uint8_t *hp = p + (MIN ? 4 : 2);
-        const uint32_t qh = ld16(hp) | (ld16(hp + 2) << 16);
+        const Halves<5, SPAN> hq(hp);
+        const uint32_t qh = hq.h(0) | (hq.h(1) << 16);
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            const uint32_t q = ld16(hp + 4 + 2 * i);
+            const uint32_t q = hq.h(2 + i);
 #pragma unroll
             for (int e = 0; e < 2; ++e) {
                 const int j = 2 * i + e;
@@ -156,9 +189,10 @@ __device__ __forceinline__ void decode_unit(const uint8_t *__restrict__ row, int
         const int sh = (ub & 3) * 2;
         const float s0 = d * (float)q3k_scale(p + 96, 2 * ub);
         const float s1 = d * (float)q3k_scale(p + 96, 2 * ub + 1);
+        const Halves<8, SPAN> lq(qs), hq(p);
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            const uint32_t q = ld16(qs + 2 * i), hm = ld16(p + 2 * i) >> ub;
+            const uint32_t q = lq.h(i), hm = hq.h(i) >> ub;
             const float sv = (i < 8) ? s0 : s1;
             w[2 * i] = sv * (float)((int)((q >> sh) & 3) + (int)((hm & 1) << 2) - 4);
             w[2 * i + 1] = sv * (float)((int)((q >> (8 + sh)) & 3) + (int)(((hm >> 8) & 1) << 2) - 4);
@@ -191,10 +225,11 @@ __device__ __forceinline__ void decode_unit(const uint8_t *__restrict__ row, int
         const float s1 = d * (float)scales[8 * h + 2 * quad + 1];
         const int shl = (quad < 2) ? 0 : 4;
         const int shh = 2 * quad;
+        const Halves<8, SPAN> lq(ql), hq(qh);
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            const uint32_t l16 = ld16(ql + 2 * i);
-            const uint32_t h16 = ld16(qh + 2 * i);
+            const uint32_t l16 = lq.h(i);
+            const uint32_t h16 = hq.h(i);
             const int q0 = (int)(((l16 >> shl) & 0xF) | (((h16 >> shh) & 3) << 4)) - 32;
             const int q1 = (int)(((l16 >> (8 + shl)) & 0xF) | (((h16 >> (8 + shh)) & 3) << 4)) - 32;
             const float sv = (i < 8) ? s0 : s1;  // elements 0..15 / 16..31

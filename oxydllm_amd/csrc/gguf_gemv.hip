@@ -103,22 +103,6 @@ __global__ __launch_bounds__(256) void gguf_gemv_kernel(const void *__restrict__
 struct __attribute__((packed, aligned(2))) U32A2 { uint32_t v; };
 __device__ __forceinline__ uint32_t ld32a2(const uint8_t *p) { return ((const U32A2 *)p)->v; }
 
-// NDW consecutive dwords from an even address.  Blocks of 18, 22, 34, 110 or 210 bytes put every other
-// block at an address that is 2 mod 4; a 16-byte LDS read from such an address is served in short
-// pieces (Q6_K, four such reads per unit: waves spent a third of their time waiting on LDS).  Aligned
-// dword reads and one funnel shift per dword cost the same LDS cycles as an aligned wide read.
-// Reads one dword past the span when the address is aligned (its value is shifted out).
-template <int NDW>
-__device__ __forceinline__ void ld_span(const uint8_t *p, uint32_t (&out)[NDW]) {
-    const uint32_t mis = (uint32_t)(uintptr_t)p & 2u;
-    const uint32_t *q = (const uint32_t *)(p - mis);
-    uint32_t d[NDW + 1];
-#pragma unroll
-    for (int i = 0; i <= NDW; ++i) d[i] = q[i];
-#pragma unroll
-    for (int i = 0; i < NDW; ++i) out[i] = __builtin_amdgcn_alignbit(d[i + 1], d[i], mis * 8u);
-}
-
 // The empty asm keeps the caller's shift-and-mask of the whole dword apart from the four conversions:
 // merged, the compiler extracts every byte by itself (v_bfe + v_cvt_f32_ubyte0, two instructions a
 // weight); apart, each conversion is one v_cvt_f32_ubyteN.
