@@ -132,8 +132,12 @@ template <int FMT> struct GgufSource {
         const int head = (int)(((size_t)dn * row_bytes + (size_t)s * SEG) & 15);
         uint32_t o[16], ol[16];
         if (s * 8 + u < units) {
-            float wf[32];
-            decode_unit<FMT, true>(raw + dr * RAWP + head, u, wf);  // LDS: block bytes as aligned dwords
+            // stored integers converted once, then one fma a weight: scale * q - offset, the value
+            // of the format's dequant (both products exact in f32 or rounded the same single time)
+            float wf[32], c0, c1, d0, d1;
+            unit_ints<FMT>(raw + dr * RAWP + head, u, wf, c0, c1, d0, d1);
+#pragma unroll
+            for (int i = 0; i < 32; ++i) wf[i] = fmaf(i < 16 ? c0 : c1, wf[i], -(i < 16 ? d0 : d1));
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 o[i] = pack_bf16(wf[2 * i], wf[2 * i + 1]);

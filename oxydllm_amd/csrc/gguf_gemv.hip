@@ -100,164 +100,6 @@ __global__ __launch_bounds__(256) void gguf_gemv_kernel(const void *__restrict__
 //     y_unit = scale * (sum q_i x_i) - offset * (sum x_i),
 // and the sums of x over 16 elements are computed once per workgroup, not per row.
 // ---------------------------------------------------------------------------
-struct __attribute__((packed, aligned(2))) U32A2 { uint32_t v; };
-__device__ __forceinline__ uint32_t ld32a2(const uint8_t *p) { return ((const U32A2 *)p)->v; }
-
-// The empty asm keeps the caller's shift-and-mask of the whole dword apart from the four conversions:
-// merged, the compiler extracts every byte by itself (v_bfe + v_cvt_f32_ubyte0, two instructions a
-// weight); apart, each conversion is one v_cvt_f32_ubyteN.
-__device__ __forceinline__ void bytes_to_f32(uint32_t w, float *o) {
-    asm volatile("" : "+v"(w));
-    o[0] = (float)(w & 0xFFu);
-    o[1] = (float)((w >> 8) & 0xFFu);
-    o[2] = (float)((w >> 16) & 0xFFu);
-    o[3] = (float)(w >> 24);
-}
-
-// Unit `u` of a row: q[0..31] = the stored unsigned integers as floats, and the four
-// numbers that turn (dot over elements 0..15, dot over 16..31, sum x over 0..15, sum x
-// over 16..31) into the unit's contribution: a0*dot0 + a1*dot1 - b0*sx0 - b1*sx1.
-template <int FMT>
-__device__ __forceinline__ void unit_ints(const uint8_t *__restrict__ row, int u, float q[32], float &a0,
-                                          float &a1, float &b0, float &b1) {
-    if constexpr (FMT == OXQ_GGUF_Q4_0) {
-        const uint8_t *p = row + (size_t)u * 18;
-        const float d = ld_f16(p);
-        uint32_t qs[4];
-        ld_span<4>(p + 2, qs);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const uint32_t w = qs[i];
-            bytes_to_f32(w & 0x0F0F0F0Fu, q + 4 * i);
-            bytes_to_f32((w >> 4) & 0x0F0F0F0Fu, q + 16 + 4 * i);
-        }
-        a0 = a1 = d;
-        b0 = b1 = 8.0f * d;
-    } else if constexpr (FMT == OXQ_GGUF_Q8_0) {
-        const uint8_t *p = row + (size_t)u * 34;
-        const float d = ld_f16(p);
-        uint32_t qs[8];
-        ld_span<8>(p + 2, qs);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) bytes_to_f32(qs[i] ^ 0x80808080u, q + 4 * i);  // q + 128
-        a0 = a1 = d;
-        b0 = b1 = 128.0f * d;
-    } else if constexpr (FMT == OXQ_GGUF_Q4_K) {
-        const int b = u >> 3, sb = u & 7;
-        const uint8_t *p = row + (size_t)b * 144;
-        const float d = ld_f16(p), dmin = ld_f16(p + 2);
-        uint32_t scv, mnv;
-        k4_scale_min(p + 4, sb, scv, mnv);
-        // 144-byte blocks in rows that start at a multiple of 16: the 32 bytes are two aligned chunks
-        const u32x4_t *qs = (const u32x4_t *)(p + 16 + (sb >> 1) * 32);
-        const u32x4_t q0 = qs[0], q1 = qs[1];
-        const uint32_t qw[8] = {q0[0], q0[1], q0[2], q0[3], q1[0], q1[1], q1[2], q1[3]};
-        const int sh = (sb & 1) * 4;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) bytes_to_f32((qw[i] >> sh) & 0x0F0F0F0Fu, q + 4 * i);
-        a0 = a1 = d * (float)scv;
-        b0 = b1 = dmin * (float)mnv;
-    } else if constexpr (FMT == OXQ_GGUF_Q4_1) {
-        const uint8_t *p = row + (size_t)u * 20;
-        const float d = ld_f16(p), m = ld_f16(p + 2);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const uint32_t w = ld32a2(p + 4 + 4 * i);
-            bytes_to_f32(w & 0x0F0F0F0Fu, q + 4 * i);
-            bytes_to_f32((w >> 4) & 0x0F0F0F0Fu, q + 16 + 4 * i);
-        }
-        a0 = a1 = d;
-        b0 = b1 = -m;
-    } else if constexpr (FMT == OXQ_GGUF_Q5_0 || FMT == OXQ_GGUF_Q5_1) {
-        constexpr bool MIN = FMT == OXQ_GGUF_Q5_1;
-        const uint8_t *p = row + (size_t)u * (MIN ? 24 : 22);
-        const float d = ld_f16(p);
-        const uint8_t *hp = p + (MIN ? 4 : 2);
-        uint32_t hq[5];
-        ld_span<5>(hp, hq);
-        const uint32_t qh = hq[0];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const uint32_t w = hq[1 + i];
-            bytes_to_f32((w & 0x0F0F0F0Fu) | (spread4(qh >> (4 * i)) << 4), q + 4 * i);
-            bytes_to_f32(((w >> 4) & 0x0F0F0F0Fu) | (spread4(qh >> (16 + 4 * i)) << 4), q + 16 + 4 * i);
-        }
-        a0 = a1 = d;
-        b0 = b1 = MIN ? -ld_f16(p + 2) : 16.0f * d;
-    } else if constexpr (FMT == OXQ_GGUF_Q2_K) {
-        const int b = u >> 3, ub = u & 7;
-        const uint8_t *p = row + (size_t)b * 84;
-        const float d = ld_f16(p + 80), dmin = ld_f16(p + 82);
-        const uint8_t *qs = p + 16 + (ub >> 2) * 32;
-        const int sh = (ub & 3) * 2;
-        const uint32_t sc = ld16(p + 2 * ub);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) bytes_to_f32((ld32a2(qs + 4 * i) >> sh) & 0x03030303u, q + 4 * i);
-        a0 = d * (float)(sc & 0xF);
-        b0 = dmin * (float)((sc >> 4) & 0xF);
-        a1 = d * (float)((sc >> 8) & 0xF);
-        b1 = dmin * (float)(sc >> 12);
-    } else if constexpr (FMT == OXQ_GGUF_Q3_K) {
-        const int b = u >> 3, ub = u & 7;
-        const uint8_t *p = row + (size_t)b * 110;
-        const float d = ld_f16(p + 108);
-        const uint8_t *qs = p + 32 + (ub >> 2) * 32;
-        const int sh = (ub & 3) * 2;
-        uint32_t lw[8], hw[8];
-        ld_span<8>(qs, lw);
-        ld_span<8>(p, hw);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const uint32_t lo = (lw[i] >> sh) & 0x03030303u;
-            const uint32_t hi = ((hw[i] >> ub) & 0x01010101u) << 2;
-            bytes_to_f32(lo | hi, q + 4 * i);  // q + 4
-        }
-        a0 = d * (float)q3k_scale(p + 96, 2 * ub);
-        a1 = d * (float)q3k_scale(p + 96, 2 * ub + 1);
-        b0 = 4.0f * a0;
-        b1 = 4.0f * a1;
-    } else if constexpr (FMT == OXQ_GGUF_Q5_K) {
-        const int b = u >> 3, sb = u & 7;
-        const uint8_t *p = row + (size_t)b * 176;
-        const float d = ld_f16(p), dmin = ld_f16(p + 2);
-        uint32_t scv, mnv;
-        k4_scale_min(p + 4, sb, scv, mnv);
-        const uint8_t *qs = p + 48 + (sb >> 1) * 32;
-        const int sh = (sb & 1) * 4;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const uint32_t lo = (ld32a2(qs + 4 * i) >> sh) & 0x0F0F0F0Fu;
-            const uint32_t hi = ((ld32a2(p + 16 + 4 * i) >> sb) & 0x01010101u) << 4;
-            bytes_to_f32(lo | hi, q + 4 * i);
-        }
-        a0 = a1 = d * (float)scv;
-        b0 = b1 = dmin * (float)mnv;
-    } else {  // Q6_K
-        const int b = u >> 3, sub = u & 7;
-        const int h = sub >> 2, quad = sub & 3;
-        const uint8_t *p = row + (size_t)b * 210;
-        const uint8_t *ql = p + 64 * h + (quad & 1) * 32;
-        const uint8_t *qh = p + 128 + 32 * h;
-        const int8_t *scales = (const int8_t *)(p + 192);
-        const float d = ld_f16(p + 208);
-        const int shl = (quad < 2) ? 0 : 4;
-        const int shh = 2 * quad;
-        uint32_t lw[8], hw[8];
-        ld_span<8>(ql, lw);
-        ld_span<8>(qh, hw);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const uint32_t lo = (lw[i] >> shl) & 0x0F0F0F0Fu;
-            const uint32_t hi = ((hw[i] >> shh) & 0x03030303u) << 4;
-            bytes_to_f32(lo | hi, q + 4 * i);  // q + 32
-        }
-        a0 = d * (float)scales[8 * h + 2 * quad];
-        a1 = d * (float)scales[8 * h + 2 * quad + 1];
-        b0 = 32.0f * a0;
-        b1 = 32.0f * a1;
-    }
-}
-
 // Activations sit in LDS unit by unit: the CPU 16-byte chunks of unit u at u * (CPU + 1) * 16, one
 // pad chunk after each unit.  Consecutive lanes (units) then read at a pitch of 144 (f32) or 80 (bf16)
 // bytes, which puts every 8 neighbouring lanes on the 8 different 16-byte bank groups, and a chunk's
