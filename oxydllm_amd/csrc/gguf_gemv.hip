@@ -158,21 +158,32 @@ __global__ __launch_bounds__(PW ? 1024 : 512) void gguf_gemv_lds_kernel(const vo
     // chunks that lie wholly inside the tensor; only the tensor's very last chunk can be partial
     const int full = (int)min((size_t)wchunks, (total_bytes - a0) >> 4);
     const u32x4_t *wsrc = (const u32x4_t *)(w + a0);
-    // sums of x over every 16 elements, once per workgroup (every row's decode needs them: the
-    // offset terms of the formats multiply them); summed in element order
+    // sums of x over every 16 elements, once per workgroup (every row's decode needs them: the offset
+    // terms of the formats multiply them).  Association: the elements of a 16-byte chunk in order, then
+    // the chunks of the half unit pairwise - what the wave-per-row form gets from lane exchanges.
+    auto chunk_sum = [](const u32x4_t v) {
+        float sx = 0.0f;
+        if constexpr (BF16X) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t e = v[j];
+                sx += __builtin_bit_cast(float, e << 16) + __builtin_bit_cast(float, e & 0xFFFF0000u);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) sx += __builtin_bit_cast(float, (uint32_t)v[j]);
+        }
+        return sx;
+    };
     auto stage_sums = [&]() {
+        constexpr int HC = CPU / 2;
         for (int t = threadIdx.x; t < MB * 2 * units; t += nthr) {
             const int m = MB == 1 ? 0 : t / (2 * units), hu = t - m * 2 * units;
             if (m < M) {
                 unsigned char *xr = lds_x + m * xrow_bytes;
-                float sx = 0.0f;
-#pragma unroll
-                for (int o = 0; o < 2; ++o) {
-                    float xv[8];
-                    ld_x8<BF16X>(xr + (hu >> 1) * XP, 2 * (hu & 1) + o, xv);
-#pragma unroll
-                    for (int i = 0; i < 8; ++i) sx += xv[i];
-                }
+                const u32x4_t *c = (const u32x4_t *)(xr + (hu >> 1) * XP + (hu & 1) * HC * 16);
+                float sx = chunk_sum(c[0]) + chunk_sum(c[1]);
+                if constexpr (HC == 4) sx += chunk_sum(c[2]) + chunk_sum(c[3]);
                 ((float *)(xr + (size_t)units * XP))[hu] = sx;
             }
         }
@@ -203,10 +214,16 @@ __global__ __launch_bounds__(PW ? 1024 : 512) void gguf_gemv_lds_kernel(const vo
             const int g = (int)threadIdx.x + b * nthr;
             const int u = g / CPU, cc = g - u * CPU;
             *(u32x4_t *)(lds_x + (g < cpr ? u * XP + cc * 16 : CPU * 16)) = xv[b];  // else: unit 0's pad
+            // the sums of x over 16 elements, from the registers that carry x: a chunk's own elements,
+            // then the HC chunks of a half unit, which neighbouring lanes hold (lane ^ 1, lane ^ 2)
+            constexpr int HC = CPU / 2;
+            float sx = chunk_sum(xv[b]);
+            sx += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, sx), 0xB1, 0xF, 0xF, false));
+            if constexpr (HC == 4)
+                sx += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, sx), 0x4E, 0xF, 0xF, false));
+            if (g < cpr && (cc & (HC - 1)) == 0) ((float *)(lds_x + (size_t)units * XP))[2 * u + cc / HC] = sx;
         }
-        __syncthreads();
-        stage_sums();
-        __syncthreads();  // both barriers come before the wait for the wave's own weight row
+        __syncthreads();  // the one barrier comes before the wait for the wave's own weight row
 #pragma unroll
         for (int q = 0; q < WCH; ++q) {
             const int c = wc0 + lane + 64 * q;
