@@ -660,7 +660,7 @@ static bool wcache_forward(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p, i
         }
         oxq_weight_cache::Entry e{p.qweight, p.qzeros, p.scales, p.K, p.N, p.group_shift, p.dtype, p.bits, p.pack_dim,
                                   Pk4Weights{(uint32_t *)mem, nullptr, p.K, p.N, p.group_shift, p.dtype, p.bits, 0,
-                                             p.pack_dim == OXQ_PACK_IN ? 32 : 16},
+                                             p.pack_dim == OXQ_PACK_IN ? 32 : 16, pk4_choose_strip(p.K, p.N, p.bits, 0)},
                                   bytes, 0};
         const int prc = launch_pk4_prepack(ctx, s, p, e.w);  // on the caller's stream, ahead of the matmul
         if (prc != OXQ_OK) {
@@ -1674,6 +1674,7 @@ static int prepack_layer(oxq_packed_quant_linear *l) {
     l->pk.bits = src.bits;
     l->pk.gate_half = l->act ? src.N / 2 : 0;
     l->pk.gemv_rows = src.pack_dim == OXQ_PACK_IN ? 32 : 16;
+    l->pk.strip = pk4_choose_strip(src.K, src.N, src.bits, l->pk.gate_half);
     if (ctx->plan_only) {
         l->prepacked = true;
         return OXQ_OK;

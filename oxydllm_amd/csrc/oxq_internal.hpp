@@ -159,6 +159,7 @@ struct Pk4Weights {
                             // [32j, 32j+32) then up columns [N/2 + 32j, N/2 + 32j + 32)
     int gemv_rows;          // rows up to which the reference runs its fused GEMV, which never rounds the
                             // dequantized weight (linear.rs:450-480: 16 AWQ, 32 GPTQ); 0 = 16
+    int strip;              // columns of a strip of pw: 64 (or 0), or 16 (narrow 4-bit layers, see pk4.hip)
 };
 
 struct Pk4Problem {
@@ -174,6 +175,7 @@ struct Pk4Problem {
 // ---- launchers (defined in the .hip files) ---------------------------------
 bool pk4_eligible(const Wna16Problem &p);
 size_t pk4_weight_bytes(int64_t K, int64_t N, int bits);
+int pk4_choose_strip(int64_t K, int64_t N, int bits, int64_t gate_half);
 size_t pk4_zs_bytes(int64_t K, int64_t N, int group_shift);
 int launch_pk4_prepack(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &src, const Pk4Weights &dst);
 int launch_pk4_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p);

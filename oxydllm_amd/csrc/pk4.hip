@@ -50,6 +50,7 @@
 #include "oxq_mfma.hpp"
 
 #include <algorithm>
+#include <type_traits>
 #include <cstdlib>
 
 namespace oxq {
@@ -577,6 +578,341 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
 }
 
 // ---------------------------------------------------------------------------
+// Narrow layers: strips of 16 columns (4-bit).
+//
+// A layer with few 64-column strips (a down projection, an attention projection) fills the chip
+// only when K is also cut into slices, whose partial tiles a second launch has to add.  Stored in
+// strips of 16 columns the same layer has four times as many strips, so that at one to four rows of x
+// a workgroup per strip fills the chip with K inside the workgroup: one launch.  With more rows a
+// workgroup takes four neighbouring strips (every strip re-reads x, which then outweighs the weights)
+// and the launch has the shape of the 64-column form.
+//
+//   pw  [N/16 strips][K/128 blocks]{ [64 lanes][4 words] , [16 columns] {-z, s} pairs }     1088 bytes a block
+//
+// Lane l = (ni = l % 16, kb = l / 16) of a block holds, in word t (= MFMA step t of the block), the 8 rows
+// 128*b + 64*(t/2) + 16*kb + 8*(t%2) .. +7 (the wide form's order) of column 16*strip + ni: row 2pp in nibble pp of the low half, row 2pp+1 in
+// nibble pp of the high half, so the same AND-OR as in the wide form yields row pair pp as two exact
+// 16-bit floats.  One 1 KB wave load is a block: a strip's words span the block's four steps, so the ring
+// holds whole blocks and a block is requested when an earlier one starts.
+// The conversion bias now goes with the row pair, not with the column (f16: 1024 for even pp, 64 for
+// odd pp; bf16: 128): the pairs hold -z alone, the folded form takes the biases out with a second row
+// sum (x against a fragment of the biases), the tile form keeps one constant per bias and column.
+// ---------------------------------------------------------------------------
+constexpr int PK4N_BW = 272;  // words of one block: 256 of weights, 16 of pairs
+
+template <typename TT, bool GPTQ>
+__global__ __launch_bounds__(256) void pk4n_prepack_kernel(const uint32_t *__restrict__ qw,
+                                                           const uint32_t *__restrict__ qz,
+                                                           const uint16_t *__restrict__ sc,
+                                                           uint32_t *__restrict__ pw, int K, int N, int gshift) {
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const int NB = K >> 7;
+    if (idx >= (size_t)(N >> 4) * NB * PK4N_BW) return;
+    const int w = (int)(idx % PK4N_BW);
+    const int b = (int)((idx / PK4N_BW) % NB), j = (int)(idx / ((size_t)PK4N_BW * NB));
+    if (w < 256) {
+        const int t = w & 3, l = w >> 2, ni = l & 15, kb = l >> 4;
+        const int k = pk4_kk(4 * b + t, kb), col = 16 * j + ni;  // the wide form's step -> row order
+        uint32_t v = 0;
+#pragma unroll
+        for (int r = 0; r < 8; ++r) v |= src_q<GPTQ, 4>(qw, k + r, col, N) << (4 * (r >> 1) + 16 * (r & 1));
+        pw[idx] = v;
+    } else {
+        const int col = 16 * j + (w - 256);
+        const int g = (b << 7) >> gshift;
+        const int c = col % 8;
+        const int slot = GPTQ ? c : ((c >> 1) | ((c & 1) << 2));
+        const uint32_t z = ((qz[(size_t)g * (N / 8) + col / 8] >> (4 * slot)) & 15u) + (GPTQ ? 1u : 0u);
+        pw[idx] = (uint32_t)TT::from_f32(-(float)z) | ((uint32_t)sc[(size_t)g * N + col] << 16);
+    }
+}
+
+// The constants of one column and block from its pair word {-z, s}; deq() = T((q - z) * s) of a row pair.
+template <typename TT> struct Pk4N;
+template <> struct Pk4N<F16Traits> {
+    uint32_t ce, co, sp;  // -(1024 + z), -(64 + z), s, each in both halves
+    __device__ __forceinline__ void prep(uint32_t zw) {
+        const uint32_t nz = perm_b32(zw, zw, 0x01000100u);
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        ce = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, nz) + __builtin_bit_cast(h2, 0xE400E400u));
+        co = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, nz) + __builtin_bit_cast(h2, 0xD400D400u));
+        sp = perm_b32(zw, zw, 0x03020302u);
+    }
+    __device__ __forceinline__ uint32_t deq(uint32_t p, int pp) const {
+        return MfmaOps<F16Traits>::dequant_pair(p, (pp & 1) ? co : ce, sp);
+    }
+};
+template <> struct Pk4N<BF16Traits> {
+    uint32_t c0, c1;
+    __device__ __forceinline__ void prep(uint32_t zw) {
+        const float sf = __builtin_bit_cast(float, zw & 0xFFFF0000u);
+        const float nz = __builtin_bit_cast(float, zw << 16);
+        c0 = __builtin_bit_cast(uint32_t, sf);
+        c1 = __builtin_bit_cast(uint32_t, (nz - 128.0f) * sf);
+    }
+    __device__ __forceinline__ uint32_t deq(uint32_t p, int) const { return Pk4T<BF16Traits>::deq(p, c0, c1); }
+};
+
+template <typename TT>
+__global__ __launch_bounds__(256) void pk4n_dequant_kernel(const uint32_t *__restrict__ pw,
+                                                           uint16_t *__restrict__ out, int K, int N) {
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;  // over the weight words only
+    const int NB = K >> 7;
+    if (idx >= (size_t)(N >> 4) * NB * 256) return;
+    const int w = (int)(idx % 256);
+    const int b = (int)((idx / 256) % NB), j = (int)(idx / ((size_t)256 * NB));
+    const uint32_t *blk = pw + ((size_t)j * NB + b) * PK4N_BW;
+    const int t = w & 3, l = w >> 2, ni = l & 15, kb = l >> 4;
+    const int k = pk4_kk(4 * b + t, kb), col = 16 * j + ni;
+    const uint32_t wd = blk[w];
+    const NibbleMasks nm = nibble_masks();
+    Pk4N<TT> c;
+    c.prep(blk[256 + ni]);
+#pragma unroll
+    for (int pp = 0; pp < 4; ++pp) {
+        const uint32_t d = c.deq(TT::unpack1(wd, pp, nm), pp);
+        out[(size_t)(k + 2 * pp) * N + col] = (uint16_t)(d & 0xFFFFu);
+        out[(size_t)(k + 2 * pp + 1) * N + col] = (uint16_t)(d >> 16);
+    }
+}
+
+// The waves' partial tiles meet in LDS as in the wide form; a thread then owns (row, column ni of every
+// strip of the workgroup) and adds the waves in order.
+template <typename TT, int MT, int NS>
+__device__ __forceinline__ void pk4n_epilogue(const float4_t (&acc)[MT][NS], const uint16_t *__restrict__ bias,
+                                              uint16_t *__restrict__ y, float *__restrict__ ws, int M, int N, int j,
+                                              int m0, int wave, int lane) {
+    constexpr int NW = 8, NT = NW * 64, ROWS = 16 * MT;
+    extern __shared__ __attribute__((aligned(16))) unsigned char pk4_lds[];
+    // every wave into its own activation slot (other waves may still be reading theirs): [MT][4 e][64 lanes][NS]
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            float *dst = (float *)(pk4_lds + (size_t)wave * MT * 4096) + ((mt * 4 + e) * 64 + lane) * NS;
+            if constexpr (NS == 4) *(float4_t *)dst = float4_t{acc[mt][0][e], acc[mt][1][e], acc[mt][2][e], acc[mt][3][e]};
+            else dst[0] = acc[mt][0][e];
+        }
+    __syncthreads();
+    for (int t = threadIdx.x; t < ROWS * 16; t += NT) {
+        const int ml = t >> 4, ni = t & 15;
+        if (m0 + ml >= M) continue;
+        const int mt = ml >> 4, r = ml & 15, kb = r >> 2, e = r & 3;
+        float v[NS];
+#pragma unroll
+        for (int f = 0; f < NS; ++f) v[f] = 0.f;
+#pragma unroll
+        for (int s = 0; s < NW; ++s) {
+            const float *src = (const float *)(pk4_lds + (size_t)s * MT * 4096) + ((mt * 4 + e) * 64 + kb * 16 + ni) * NS;
+            if constexpr (NS == 4) {
+                const float4_t q = *(const float4_t *)src;
+                v[0] += q[0], v[1] += q[1], v[2] += q[2], v[3] += q[3];
+            } else {
+                v[0] += src[0];
+            }
+        }
+#pragma unroll
+        for (int f = 0; f < NS; ++f) {
+            const int n = 16 * (NS * j + f) + ni;
+            if (gridDim.y > 1) {  // this K slice's f32 partial; a second kernel adds the slices in order
+                ws[((size_t)blockIdx.y * M + (m0 + ml)) * N + n] = v[f];
+            } else {
+                float o = v[f];
+                if (bias) o += TT::to_f32(bias[n]);
+                y[(size_t)(m0 + ml) * N + n] = TT::from_f32(o);
+            }
+        }
+    }
+}
+
+template <typename TT, int MT, bool GS, int NS, int XQ>
+__global__ __launch_bounds__(512) void pk4n_mfma_kernel(const uint16_t *__restrict__ x,
+                                                        const uint32_t *__restrict__ pw,
+                                                        const uint16_t *__restrict__ bias,
+                                                        uint16_t *__restrict__ y, float *__restrict__ ws,
+                                                        int M, int K, int N, int bslice) {
+    typedef MfmaOps<TT> Ops;
+    constexpr bool DUAL = TT::DTYPE == F16Traits::DTYPE;  // two conversion biases (see the layout note)
+    constexpr int NW = 8, ROWS = 16 * MT, AQ = XQ, SLOT = ROWS * 256, OOB = 0x7FFFFF00, BB = PK4N_BW * 4;
+    constexpr int WNT = MT < 4 ? 2 : 0;
+    extern __shared__ __attribute__((aligned(16))) unsigned char pk4_lds[];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int ni = lane & 15, kb = lane >> 4;
+    const int j = blockIdx.x;
+    const int m0 = blockIdx.z * ROWS;
+    const int NB = K >> 7;
+    const int sb0 = blockIdx.y * bslice;
+    const int SB = min(NB, sb0 + bslice) - sb0;
+    const int cbase = SB / NW, crem = SB % NW;
+    const int nloc = cbase + (wave < crem ? 1 : 0);
+    const int cb0 = sb0 + wave * cbase + min(wave, crem);
+    unsigned char *slot = pk4_lds + wave * SLOT;
+
+    const __amdgpu_buffer_rsrc_t rs_w =
+        make_rsrc(pw + (size_t)j * NS * NB * PK4N_BW, (uint32_t)NS * (uint32_t)NB * (uint32_t)BB);
+    const __amdgpu_buffer_rsrc_t rs_x = make_rsrc(x, (uint32_t)M * (uint32_t)K * 2u);
+    const __amdgpu_buffer_rsrc_t rs_none = make_rsrc(pw, 0u);
+    const int voff_w = lane * 16, voff_z = 1024 + ni * 4;
+    constexpr bool VA1 = MT >= 3;
+    int voff_a[VA1 ? 1 : AQ];
+#pragma unroll
+    for (int q = 0; q < (VA1 ? 1 : AQ); ++q) {
+        const int r = m0 + 4 * q + kb;
+        voff_a[q] = r < M ? (r * K * 2 + ni * 16) : OOB;
+    }
+    uint32_t rowstep = 4u * (uint32_t)K * 2u;
+    int a_wr[4];
+#pragma unroll
+    for (int qq = 0; qq < 4; ++qq) a_wr[qq] = kb * 256 + (((ni ^ kb) ^ (qq << 2)) << 4);
+    int a_rd[4];
+#pragma unroll
+    for (int st = 0; st < 4; ++st) a_rd[st] = ni * 256 + (((8 * (st >> 1) + 2 * kb + (st & 1)) ^ ni) << 4);
+    const NibbleMasks nm = nibble_masks();
+#pragma unroll
+    for (int q = AQ; q < 4 * MT; ++q) {
+        const int row = 4 * q + kb;
+        *(u32x4_t *)(slot + row * 256 + ((ni ^ (row & 15)) << 4)) = u32x4_t{0u, 0u, 0u, 0u};
+    }
+
+    // ring of RD blocks: a workgroup of four strips keeps one block ahead (4 KB a wave in flight, as the
+    // wide form), a single strip two (its blocks are 1 KB; measured 4096 x 4096 / 4096 x 6144 / 8192 x 4096
+    // at one row: one ahead 4.11 / 4.82 / 6.19 us, two 3.89 / 4.84 / 5.78, three 3.93 / 5.13 / 5.97)
+    constexpr int RD = NS == 1 ? 3 : 2;
+    u32x4_t aring[AQ], wr[RD][NS];
+    uint32_t zr[RD][NS];
+    auto load_a = [&](int i, u32x4_t (&a)[AQ]) {
+        const __amdgpu_buffer_rsrc_t rs = i < nloc ? rs_x : rs_none;
+        const int blk = cb0 + i;
+#pragma unroll
+        for (int q = 0; q < AQ; ++q) {
+            if (VA1) {
+                if (q == 0) asm volatile("" : "+s"(rowstep));
+                const uint32_t v = (uint32_t)voff_a[0] + (uint32_t)q * rowstep;
+                a[q] = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)(v < (uint32_t)voff_a[0] ? (uint32_t)OOB : v), blk * 256, 0);
+            } else {
+                a[q] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff_a[q], blk * 256, 0);
+            }
+        }
+    };
+    auto load_w = [&](int i, u32x4_t (&w)[NS], uint32_t (&z)[NS]) {
+        const __amdgpu_buffer_rsrc_t rs = i < nloc ? rs_w : rs_none;
+#pragma unroll
+        for (int f = 0; f < NS; ++f) {
+            const int so = (f * NB + cb0 + i) * BB;
+            w[f] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff_w, so, WNT);
+            z[f] = __builtin_amdgcn_raw_buffer_load_b32(rs, voff_z, so, WNT);
+        }
+    };
+    auto store_a = [&](const u32x4_t (&a)[AQ]) {
+#pragma unroll
+        for (int q = 0; q < AQ; ++q) *(u32x4_t *)(slot + q * 1024 + a_wr[q & 3]) = a[q];
+    };
+
+    u32x4_t afirst[AQ];
+    load_a(0, afirst);
+#pragma unroll
+    for (int d = 0; d + 1 < RD; ++d) load_w(d, wr[d], zr[d]);
+    load_a(1, aring);
+
+    float4_t acc[MT][NS];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int f = 0; f < NS; ++f) acc[mt][f] = float4_t{0.f, 0.f, 0.f, 0.f};
+    const uint32_t ones[4] = {TT::ONES, TT::ONES, TT::ONES, TT::ONES};
+    // the biases of row pairs 0..3 as a B fragment (f16: 1024, 64, 1024, 64)
+    const uint32_t biases[4] = {0x64006400u, 0x54005400u, 0x64006400u, 0x54005400u};
+    const float4_t zero4 = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    store_a(afirst);
+
+    // one block: its weights are in ring half CUR; the next block is requested into the other half first
+    auto block = [&](int i, auto cur_c) {
+        constexpr int CUR = decltype(cur_c)::value, NXT = (CUR + RD - 1) % RD;
+        load_w(i + RD - 1, wr[NXT], zr[NXT]);
+        float4_t tmp[GS ? MT : 1][NS], tmp1[GS ? MT : 1], tmpb[(GS && DUAL) ? MT : 1];
+        Pk4N<TT> cst[GS ? 1 : NS];
+        if (!GS) {
+#pragma unroll
+            for (int f = 0; f < NS; ++f) cst[f].prep(zr[CUR][f]);
+        }
+#pragma unroll
+        for (int st = 0; st < 4; ++st) {
+            uint32_t a[MT][4];
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const u32x4_t av = *(const u32x4_t *)(slot + mt * 4096 + a_rd[st]);
+                const uint32_t a0 = av[0], a1 = av[1], a2 = av[2], a3 = av[3];
+                a[mt][0] = a0, a[mt][1] = a1, a[mt][2] = a2, a[mt][3] = a3;
+            }
+            const bool fresh = st == 0;
+#pragma unroll
+            for (int f = 0; f < NS; ++f) {
+                const uint32_t w = wr[CUR][f][st];
+                uint32_t b[4];
+#pragma unroll
+                for (int pp = 0; pp < 4; ++pp) {
+                    const uint32_t pr = TT::unpack1(w, pp, nm);
+                    b[pp] = GS ? pr : cst[f].deq(pr, pp);
+                }
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+                    if (GS) tmp[mt][f] = Ops::mfma(a[mt], b, fresh ? zero4 : tmp[mt][f]);
+                    else acc[mt][f] = Ops::mfma(a[mt], b, acc[mt][f]);
+                }
+            }
+            if (GS) {
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+                    tmp1[mt] = Ops::mfma(a[mt], ones, fresh ? zero4 : tmp1[mt]);
+                    if (DUAL) tmpb[mt] = Ops::mfma(a[mt], biases, fresh ? zero4 : tmpb[mt]);
+                }
+            }
+        }
+        if (GS) {  // y += s * ((sum - biased row sum) - z * row sum), all f32
+#pragma unroll
+            for (int f = 0; f < NS; ++f) {
+                const uint32_t zw = zr[CUR][f];
+                const float sf = TT::to_f32((uint16_t)(zw >> 16));
+                const float nz = TT::to_f32((uint16_t)(zw & 0xFFFFu)) - (DUAL ? 0.0f : 128.0f);
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const float d = DUAL ? tmp[mt][f][e] - tmpb[mt][e] : tmp[mt][f][e];
+                        acc[mt][f][e] = fmaf(sf, fmaf(nz, tmp1[mt][e], d), acc[mt][f][e]);
+                    }
+            }
+        }
+        store_a(aring);
+        load_a(i + 2, aring);
+    };
+    {
+        int i = 0;
+        if constexpr (RD == 2) {
+            for (; i + 1 < nloc; i += 2) {
+                block(i, std::integral_constant<int, 0>{});
+                block(i + 1, std::integral_constant<int, 1>{});
+            }
+            if (i < nloc) block(i, std::integral_constant<int, 0>{});
+        } else {
+            static_assert(RD == 3, "the loop below is unrolled for a ring of three");
+            for (; i + 2 < nloc; i += 3) {
+                block(i, std::integral_constant<int, 0>{});
+                block(i + 1, std::integral_constant<int, 1>{});
+                block(i + 2, std::integral_constant<int, 2>{});
+            }
+            if (i < nloc) block(i, std::integral_constant<int, 0>{});
+            if (i + 1 < nloc) block(i + 1, std::integral_constant<int, 1>{});
+        }
+    }
+
+    pk4n_epilogue<TT, MT, NS>(acc, bias, y, ws, M, N, j, m0, wave, lane);
+}
+
+// ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
 size_t pk4_weight_bytes(int64_t K, int64_t N, int bits) {
@@ -599,9 +935,19 @@ int launch_pk4_prepack(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &src, con
     const bool gptq = src.pack_dim == OXQ_PACK_IN;
     dim3 grid((unsigned)ceil_div((int64_t)words, 256)), block(256);
     char name[64];
-    snprintf(name, sizeof name, "pk%d_prepack_%s", src.bits, gptq ? "gptq" : "awq");
+    snprintf(name, sizeof name, "pk%d_prepack_%s%s", src.bits, gptq ? "gptq" : "awq", dst.strip == 16 ? "_n16" : "");
     set_plan(ctx, name, grid, block, 1, 1, 0);
     if (ctx->plan_only) return OXQ_OK;
+    if (dst.strip == 16) {
+#define OXQ_PPN(TTv, Gv)                                                                                  \
+    hipLaunchKernelGGL((pk4n_prepack_kernel<TTv, Gv>), grid, block, 0, s, src.qweight, src.qzeros,        \
+                       (const uint16_t *)src.scales, dst.pw, K, N, src.group_shift)
+        if (src.dtype == OXQ_F16) { if (gptq) OXQ_PPN(F16Traits, true); else OXQ_PPN(F16Traits, false); }
+        else { if (gptq) OXQ_PPN(BF16Traits, true); else OXQ_PPN(BF16Traits, false); }
+#undef OXQ_PPN
+        OXQ_HIP_CHECK(hipGetLastError());
+        return OXQ_OK;
+    }
     const int half = (int)dst.gate_half;
 #define OXQ_PP(TTv, Gv, Bv)                                                                                     \
     hipLaunchKernelGGL((pk4_prepack_kernel<TTv, Gv, Bv>), grid, block, 0, s, src.qweight, src.qzeros,           \
@@ -625,6 +971,14 @@ int launch_pk4_dequant(oxq_ctx *ctx, hipStream_t s, const Pk4Weights &w, void *o
     snprintf(name, sizeof name, "pk%d_dequant_%s", w.bits, w.dtype == OXQ_F16 ? "f16" : "bf16");
     set_plan(ctx, name, grid, block, 1, 1, 0);
     if (ctx->plan_only) return OXQ_OK;
+    if (w.strip == 16) {
+        if (w.dtype == OXQ_F16)
+            hipLaunchKernelGGL((pk4n_dequant_kernel<F16Traits>), grid, block, 0, s, w.pw, (uint16_t *)out_kn, (int)w.K, (int)w.N);
+        else
+            hipLaunchKernelGGL((pk4n_dequant_kernel<BF16Traits>), grid, block, 0, s, w.pw, (uint16_t *)out_kn, (int)w.K, (int)w.N);
+        OXQ_HIP_CHECK(hipGetLastError());
+        return OXQ_OK;
+    }
 #define OXQ_DQ(TTv, Bv)                                                                           \
     hipLaunchKernelGGL((pk4_dequant_kernel<TTv, Bv>), grid, block, 0, s, w.pw, (uint16_t *)out_kn, \
                        (int)w.K, (int)w.N, (int)w.gate_half)
@@ -695,7 +1049,91 @@ static int pk4_by_mt(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p
     }
 }
 
+// Strip width of a layer's resident copy: 16 columns for 4-bit layers with few 64-column strips and a
+// long K (the shapes that otherwise need K slices and a second launch), 64 otherwise.
+int pk4_choose_strip(int64_t K, int64_t N, int bits, int64_t gate_half) {
+    // Measured (f16, one row of x; 64-column strips with K slices -> 16-column strips, one launch):
+    // 4096 x 4096 5.85 -> 3.89 us, 4096 x 6144 6.80 -> 4.84 us, 8192 x 4096 5.78 us; at 8 rows and more four
+    // strips share a workgroup and the layer runs within 3 % of the wide form.  A single strip does the
+    // per-block work on x (fragment reads, row sums, fold) for 1 KB of weights instead of 4 KB, so beyond
+    // K = 8192 it stops paying: 14336 x 4096 8.95 us against 8.99, and that layer keeps the wide form.
+    const int mode = pk4_env("OXQ_PK4_STRIP16", 1);  // 0 never, 1 by shape, 2 wherever the layout applies
+    if (!mode || bits != 4 || gate_half || N % 64 != 0) return 64;
+    if (mode == 2) return 16;
+    return (N / 64 <= 96 && N / 16 >= 128 && K / 128 >= 32 && K / 128 <= 64) ? 16 : 64;
+}
+
+template <typename TT, int MT, bool GS, int NS, int XQ>
+static int pk4n_go4(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, int bslice) {
+    const size_t lds = (size_t)8 * MT * 4096;
+    static LdsGrant lds_grant;  // one per instantiation
+    OXQ_HIP_CHECK(lds_grant.ensure((const void *)pk4n_mfma_kernel<TT, MT, GS, NS, XQ>, lds));
+    hipLaunchKernelGGL((pk4n_mfma_kernel<TT, MT, GS, NS, XQ>), grid, dim3(512), lds, s, (const uint16_t *)p.x, p.w.pw,
+                       (const uint16_t *)p.bias, (uint16_t *)p.y, (float *)ctx->workspace, (int)p.M, (int)p.w.K,
+                       (int)p.w.N, bslice);
+    OXQ_HIP_CHECK(hipGetLastError());
+    return OXQ_OK;
+}
+
+template <typename TT>
+static int pk4n_by_shape(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, int bslice, int mt, int ns,
+                         bool fold) {
+    if (ns == 1) return pk4n_go4<TT, 1, true, 1, 1>(ctx, s, grid, p, bslice);
+    switch (mt) {
+    case 1: {
+        const int xq = pk4_env("OXQ_PK4_XQ", 1) ? (int)ceil_div(p.M, 4) : 4;
+        if (xq == 1) return pk4n_go4<TT, 1, true, 4, 1>(ctx, s, grid, p, bslice);
+        if (xq == 2) return pk4n_go4<TT, 1, true, 4, 2>(ctx, s, grid, p, bslice);
+        return pk4n_go4<TT, 1, true, 4, 4>(ctx, s, grid, p, bslice);
+    }
+    case 2: return fold ? pk4n_go4<TT, 2, true, 4, 8>(ctx, s, grid, p, bslice) : pk4n_go4<TT, 2, false, 4, 8>(ctx, s, grid, p, bslice);
+    case 3: return pk4n_go4<TT, 3, false, 4, 12>(ctx, s, grid, p, bslice);
+    default: return pk4n_go4<TT, 4, false, 4, 16>(ctx, s, grid, p, bslice);
+    }
+}
+
+// forward on a layer stored in 16-column strips
+static int launch_pk4n_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p) {
+    const int64_t M = p.M, N = p.w.N;
+    const int mt = M > 48 ? 4 : (int)ceil_div(M, 16);
+    const int NB = (int)(p.w.K / 128);
+    // up to four rows a workgroup per strip (x is re-read by every strip: four rows of x against a
+    // strip's 16 columns is what 16 rows are against 64), when that gives the chip enough workgroups
+    const int ns = (M <= 4 && N / 16 >= 128 && pk4_env("OXQ_PK4N_NS1", 1)) ? 1 : 4;
+    const int64_t tiles = (N / (16 * ns)) * ceil_div(M, 16 * mt);
+    int ks = 1;
+    if (tiles <= 96 && NB >= 32) ks = (int)std::max<int64_t>(1, std::min<int64_t>(256 / tiles, NB / 8));
+    ks = pk4_env("OXQ_PK4_KS", ks);
+    ks = std::max(1, std::min(ks, NB));
+    if (p.no_split) ks = 1;
+    while (ks > 1 && (size_t)ks * M * N * 4 > ctx->workspace_bytes) --ks;
+    const int bslice = (int)ceil_div(NB, ks);
+    ks = (int)ceil_div(NB, bslice);
+    if (ceil_div(M, 16 * mt) > 65535)
+        return fail(OXQ_ERR_UNSUPPORTED, "repacked matmul: m = %lld exceeds the grid limit (65535 row tiles)", (long long)M);
+    if (p.act) return fail(OXQ_ERR_ARG, "repacked matmul: a fused activation on a layer in 16-column strips");
+    const bool fold = mt <= 2 && pk4_folds(p, mt);  // three row tiles of folded sums do not fit beside the two-block ring
+    dim3 grid((unsigned)(N / (16 * ns)), (unsigned)ks, (unsigned)ceil_div(M, 16 * mt));
+    char name[64];
+    snprintf(name, sizeof name, "pk4_mfma_%s_mt%d%s_n16x%d", p.w.dtype == OXQ_F16 ? "f16" : "bf16", mt,
+             (fold || ns == 1) ? "_gs" : "", ns);
+    set_plan(ctx, name, grid, dim3(512), ks, 1, ks > 1 ? (size_t)ks * M * N * 4 : 0);
+    if (ctx->plan_only) {
+        if (ks > 1) add_launch(ctx);
+        return OXQ_OK;
+    }
+    if ((uint64_t)M * (uint64_t)p.w.K * 2 >= (1ull << 31))
+        return fail(OXQ_ERR_UNSUPPORTED, "repacked matmul: x larger than 2 GiB");
+    if (((uintptr_t)p.x | (uintptr_t)p.y) & 15)
+        return fail(OXQ_ERR_UNSUPPORTED, "repacked matmul: x and y must be 16-byte aligned");
+    const int rc = p.w.dtype == OXQ_F16 ? pk4n_by_shape<F16Traits>(ctx, s, grid, p, bslice, mt, ns, fold)
+                                        : pk4n_by_shape<BF16Traits>(ctx, s, grid, p, bslice, mt, ns, fold);
+    if (rc != OXQ_OK || ks == 1) return rc;
+    return launch_splitk_reduce(ctx, s, (const float *)ctx->workspace, p.bias, p.y, M, N, ks, p.w.dtype);
+}
+
 int launch_pk4_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p) {
+    if (p.w.strip == 16) return launch_pk4n_forward(ctx, s, p);
     const int64_t M = p.M;
     const int mt = M > 48 ? 4 : (int)ceil_div(M, 16);
     const int NB = (int)(p.w.K / 128);

@@ -711,7 +711,7 @@ int launch_wna16_mfma(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p) {
         const size_t wb = (pk4_weight_bytes(p.K, p.N, p.bits) + 255) & ~(size_t)255;
         if (wb <= ctx->workspace_bytes) {
             Pk4Weights w{(uint32_t *)ctx->workspace, nullptr, p.K, p.N, p.group_shift, p.dtype, p.bits, 0,
-                           p.pack_dim == OXQ_PACK_IN ? 32 : 16};
+                           p.pack_dim == OXQ_PACK_IN ? 32 : 16, 64};
             int rc = launch_pk4_prepack(ctx, s, p, w);
             if (rc != OXQ_OK) return rc;
             Pk4Problem q;
