@@ -641,6 +641,11 @@ template <> struct Pk4N<F16Traits> {
     __device__ __forceinline__ uint32_t deq(uint32_t p, int pp) const {
         return MfmaOps<F16Traits>::dequant_pair(p, (pp & 1) ? co : ce, sp);
     }
+    // (bias + q) - (bias + z): the exact integers q - z as a pair of f16
+    __device__ __forceinline__ uint32_t minus_zero(uint32_t p, int pp) const {
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        return __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, p) + __builtin_bit_cast(h2, (pp & 1) ? co : ce));
+    }
 };
 template <> struct Pk4N<BF16Traits> {
     uint32_t c0, c1;
@@ -651,6 +656,7 @@ template <> struct Pk4N<BF16Traits> {
         c1 = __builtin_bit_cast(uint32_t, (nz - 128.0f) * sf);
     }
     __device__ __forceinline__ uint32_t deq(uint32_t p, int) const { return Pk4T<BF16Traits>::deq(p, c0, c1); }
+    __device__ __forceinline__ uint32_t minus_zero(uint32_t p, int) const { return p; }  // f16 only
 };
 
 template <typename TT>
@@ -733,6 +739,10 @@ __global__ __launch_bounds__(512) void pk4n_mfma_kernel(const uint16_t *__restri
                                                         int M, int K, int N, int bslice) {
     typedef MfmaOps<TT> Ops;
     constexpr bool DUAL = TT::DTYPE == F16Traits::DTYPE;  // two conversion biases (see the layout note)
+    // A single f16 strip: the row sums would be two MFMAs a step beside the strip's one, so the zero and
+    // the conversion bias are taken off the weights instead - (bias + q) - (bias + z) is an exact packed
+    // f16 add - and the block folds in with its scale alone.
+    constexpr bool EXACT = GS && DUAL && NS == 1;
     constexpr int NW = 8, ROWS = 16 * MT, AQ = XQ, SLOT = ROWS * 256, OOB = 0x7FFFFF00, BB = PK4N_BW * 4;
     constexpr int WNT = MT < 4 ? 2 : 0;
     extern __shared__ __attribute__((aligned(16))) unsigned char pk4_lds[];
@@ -833,8 +843,8 @@ __global__ __launch_bounds__(512) void pk4n_mfma_kernel(const uint16_t *__restri
         constexpr int CUR = decltype(cur_c)::value, NXT = (CUR + RD - 1) % RD;
         load_w(i + RD - 1, wr[NXT], zr[NXT]);
         float4_t tmp[GS ? MT : 1][NS], tmp1[GS ? MT : 1], tmpb[(GS && DUAL) ? MT : 1];
-        Pk4N<TT> cst[GS ? 1 : NS];
-        if (!GS) {
+        Pk4N<TT> cst[(GS && !EXACT) ? 1 : NS];
+        if (!GS || EXACT) {
 #pragma unroll
             for (int f = 0; f < NS; ++f) cst[f].prep(zr[CUR][f]);
         }
@@ -855,7 +865,8 @@ __global__ __launch_bounds__(512) void pk4n_mfma_kernel(const uint16_t *__restri
 #pragma unroll
                 for (int pp = 0; pp < 4; ++pp) {
                     const uint32_t pr = TT::unpack1(w, pp, nm);
-                    b[pp] = GS ? pr : cst[f].deq(pr, pp);
+                    if constexpr (EXACT) b[pp] = cst[f].minus_zero(pr, pp);
+                    else b[pp] = GS ? pr : cst[f].deq(pr, pp);
                 }
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt) {
@@ -863,7 +874,7 @@ __global__ __launch_bounds__(512) void pk4n_mfma_kernel(const uint16_t *__restri
                     else acc[mt][f] = Ops::mfma(a[mt], b, acc[mt][f]);
                 }
             }
-            if (GS) {
+            if (GS && !EXACT) {
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt) {
                     tmp1[mt] = Ops::mfma(a[mt], ones, fresh ? zero4 : tmp1[mt]);
@@ -881,8 +892,12 @@ __global__ __launch_bounds__(512) void pk4n_mfma_kernel(const uint16_t *__restri
                 for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
-                        const float d = DUAL ? tmp[mt][f][e] - tmpb[mt][e] : tmp[mt][f][e];
-                        acc[mt][f][e] = fmaf(sf, fmaf(nz, tmp1[mt][e], d), acc[mt][f][e]);
+                        if constexpr (EXACT) {
+                            acc[mt][f][e] = fmaf(sf, tmp[mt][f][e], acc[mt][f][e]);
+                        } else {
+                            const float d = DUAL ? tmp[mt][f][e] - tmpb[mt][e] : tmp[mt][f][e];
+                            acc[mt][f][e] = fmaf(sf, fmaf(nz, tmp1[mt][e], d), acc[mt][f][e]);
+                        }
                     }
             }
         }
