@@ -1068,10 +1068,11 @@ static int pk4_by_mt(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p
 // long K (the shapes that otherwise need K slices and a second launch), 64 otherwise.
 int pk4_choose_strip(int64_t K, int64_t N, int bits, int64_t gate_half) {
     // Measured (f16, one row of x; 64-column strips with K slices -> 16-column strips, one launch):
-    // 4096 x 4096 5.85 -> 3.89 us, 4096 x 6144 6.80 -> 4.84 us, 8192 x 4096 5.78 us; at 8 rows and more four
+    // 4096 x 4096 5.85 -> 3.74 us, 4096 x 6144 6.80 -> 4.69 us, 8192 x 4096 5.72 us; at 8 rows and more four
     // strips share a workgroup and the layer runs within 3 % of the wide form.  A single strip does the
-    // per-block work on x (fragment reads, row sums, fold) for 1 KB of weights instead of 4 KB, so beyond
-    // K = 8192 it stops paying: 14336 x 4096 8.95 us against 8.99, and that layer keeps the wide form.
+    // per-block work on x (fragment reads, fold) for 1 KB of weights instead of 4 KB, so on long K it pays
+    // less: 14336 x 4096 8.54 us against 8.99 at one row but 1 - 5 % more from 8 rows on; that layer keeps
+    // the wide form.
     const int mode = pk4_env("OXQ_PK4_STRIP16", 1);  // 0 never, 1 by shape, 2 wherever the layout applies
     if (!mode || bits != 4 || gate_half || N % 64 != 0) return 64;
     if (mode == 2) return 16;
