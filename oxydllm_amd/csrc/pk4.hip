@@ -1094,7 +1094,11 @@ static int pk4n_go4(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p,
 template <typename TT>
 static int pk4n_by_shape(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, int bslice, int mt, int ns,
                          bool fold) {
-    if (ns == 1) return pk4n_go4<TT, 1, true, 1, 1>(ctx, s, grid, p, bslice);
+    if (ns == 1) {
+        if (p.M <= 4) return pk4n_go4<TT, 1, true, 1, 1>(ctx, s, grid, p, bslice);
+        if (p.M <= 8) return pk4n_go4<TT, 1, true, 1, 2>(ctx, s, grid, p, bslice);
+        return pk4n_go4<TT, 1, true, 1, 4>(ctx, s, grid, p, bslice);
+    }
     switch (mt) {
     case 1: {
         const int xq = pk4_env("OXQ_PK4_XQ", 1) ? (int)ceil_div(p.M, 4) : 4;
@@ -1113,9 +1117,13 @@ static int launch_pk4n_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p)
     const int64_t M = p.M, N = p.w.N;
     const int mt = M > 48 ? 4 : (int)ceil_div(M, 16);
     const int NB = (int)(p.w.K / 128);
-    // up to four rows a workgroup per strip (x is re-read by every strip: four rows of x against a
-    // strip's 16 columns is what 16 rows are against 64), when that gives the chip enough workgroups
-    const int ns = (M <= 4 && N / 16 >= 128 && pk4_env("OXQ_PK4N_NS1", 1)) ? 1 : 4;
+    // One workgroup per strip when that gives the chip enough workgroups and x is small: every strip
+    // re-reads x (four rows against a strip's 16 columns are what 16 rows are against 64).  Measured, f16,
+    // single strip against four strips with K slices: 4096 x 4096 at 8 / 16 rows 4.32 / 5.27 against 6.11 /
+    // 6.47 us; 8192 x 4096 6.38 / 8.24 against 7.47 / 8.32; 4096 x 6144 (384 strips, more than one round of
+    // workgroups) 6.21 / 8.04 against 7.11 / 7.80: up to 8 rows always, up to 16 on a single round and short K.
+    const int ns1_rows = pk4_env("OXQ_PK4N_NS1_ROWS", (N / 16 <= 256 && NB <= 32) ? 16 : 8);
+    const int ns = (M <= ns1_rows && M <= 16 && N / 16 >= 128) ? 1 : 4;
     const int64_t tiles = (N / (16 * ns)) * ceil_div(M, 16 * mt);
     int ks = 1;
     if (tiles <= 96 && NB >= 32) ks = (int)std::max<int64_t>(1, std::min<int64_t>(256 / tiles, NB / 8));

@@ -1,7 +1,7 @@
 """GPU parity tests for resident 4-bit layers stored in strips of 16 columns.
 
 Layers with few 64-column strips and a long K (attention projections) are kept in 16-column strips: up
-to four rows of x run one workgroup per strip (one launch, K inside the workgroup), more rows run four
+to 8 (or 16) rows of x run one workgroup per strip (one launch, K inside the workgroup), more rows run four
 strips a workgroup.  Checked against the CPU oracle on shapes that take the layout by themselves and,
 with the layout forced, on small ragged ones:
   layer.dequantize()  bit-exact (pins the repack of this layout);
@@ -61,8 +61,8 @@ def kernel_of_last_call():
 @pytest.mark.parametrize("dtn", ["f16", "bf16"])
 @pytest.mark.parametrize("K,N,g", [(256, 2048, 128), (384, 2112, 128), (1024, 64, 256), (640, 192, 128)])
 def test_narrow_layout_forced_on_small_shapes(kind, dtn, K, N, g, monkeypatch):
-    """N >= 2048 takes the single-strip form up to four rows; the narrower ones always run four strips
-    a workgroup.  K/128 = 2, 3, 5, 8 blocks over 8 waves: empty waves, odd shares, ring tails."""
+    """N >= 2048 takes the single-strip form for its first 8 or 16 rows; the narrower ones always run
+    four strips a workgroup.  K/128 = 2, 3, 5, 8 blocks over 8 waves: empty waves, odd shares, ring tails."""
     monkeypatch.setenv("OXQ_PK4_STRIP16", "2")
     dt = DT[dtn]
     trip, pack_dim = make(kind, K, N, g, seed=K + N)
@@ -80,7 +80,8 @@ def test_narrow_layout_forced_on_small_shapes(kind, dtn, K, N, g, monkeypatch):
         y = layer.forward(xd)
         plan = kernel_of_last_call()
         assert "_n16x" in plan["kernel"], plan
-        assert plan["kernel"].endswith("x1") == (m <= 4 and N >= 2048), plan
+        single = N >= 2048 and m <= (16 if N // 16 <= 256 and K // 128 <= 32 else 8)
+        assert plan["kernel"].endswith("x1") == single, plan
         # three row tiles keep the tile form in this layout: the fold's sums do not fit beside the ring
         rounded = resident_rounds_weights(m, dt, kind == "gptq") or (dt == oracle.F16 and 32 < m <= 48)
         assert ("_gs" in plan["kernel"]) == (not rounded), plan
@@ -112,7 +113,7 @@ def test_narrow_layout_k_slices(ks, monkeypatch):
 
 @pytest.mark.parametrize("K,N", [(4096, 4096), (4096, 6144), (8192, 2048)])
 def test_attention_projection_shapes_take_the_narrow_layout(K, N, monkeypatch):
-    """By shape alone (no switch): one launch up to four rows, the wide layout's answer within tolerance."""
+    """By shape alone (no switch): one launch up to eight rows, the wide layout's answer within tolerance."""
     dt = oracle.F16
     trip, pack_dim = make("awq", K, N, 128, seed=N)
     layer = layer_of(trip, pack_dim, dt)
@@ -121,14 +122,14 @@ def test_attention_projection_shapes_take_the_narrow_layout(K, N, monkeypatch):
     monkeypatch.delenv("OXQ_PK4_STRIP16")
     w = dense("awq", trip, dt)
     np.testing.assert_array_equal(bits_of(layer.dequantize()), bits_of(wide.dequantize()))
-    for m in (1, 4, 16, 64):
+    for m in (1, 4, 8, 16, 64):
         say(f"narrow by shape K={K} N={N} m={m}")
         x = np.random.default_rng(m).standard_normal((m, K)).astype(np.float32)
         xd = to_dev(x, torch.float16)
         y = layer.forward(xd)
         plan = kernel_of_last_call()
         assert "_n16x" in plan["kernel"], plan
-        if m <= 4:
+        if m <= 8:
             assert plan["launches"] == 1 and plan["split_k"] == 1 and plan["grid"][0] == N // 16, plan
         yw = wide.forward(xd)
         assert "_n16x" not in kernel_of_last_call()["kernel"]
