@@ -1169,6 +1169,11 @@ int launch_pk4_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p) {
     const int64_t tiles = (p.w.N / 64) * ceil_div(M, 16 * mt);
     int ks = 1;
     if (tiles <= 96 && NB >= 32) ks = (int)std::max<int64_t>(1, std::min<int64_t>(256 / tiles, NB / 8));
+    // Half a round of workgroups and a long K: two slices.  Measured (f16, 1 / 16 / 64 rows): 8192 x 8192
+    // 11.3 / 12.9 / 26.3 us unsplit, 9.9 / 10.9 / 20.0 us in two slices; 28672 x 8192 32.5 / 37.6 / 78.2
+    // against 23.3 / 25.9 / 49.4 us (four slices: 23.4 / 26.8 / 54.2).  At K = 4096 or 5120 the second
+    // launch costs more than the slices save (4096 x 8192: 6.7 / 7.8 / 13.5 against 7.0 / 8.0 / 14.9 us).
+    else if (tiles <= 128 && NB >= 64) ks = 2;
     ks = pk4_env("OXQ_PK4_KS", ks);
     ks = std::max(1, std::min(ks, NB));
     if (p.act) ks = 1;  // the activation needs the whole sum: gate|up layers are wide, one slice fills the chip
