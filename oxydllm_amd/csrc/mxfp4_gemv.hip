@@ -461,11 +461,13 @@ __global__ __launch_bounds__(256) void mxfp4_dequant_kernel(const uint8_t *__res
 // K/2 bytes, and a wave load is sixteen 64-byte pieces, most of them split over two cache lines.
 // The copy stores, per expert and tile of 16 rows, chunks of 1 KB in operand order:
 //
-//   pw [E][N/16 tiles][NC chunks][64 lanes][16 bytes]     NC = ceil(K/32 / 4)
+//   pw [E][N/16 tiles][K/32 blocks][16 rows][16 bytes]    = NC chunks of [64 lanes][16 bytes], NC = ceil(K/32 / 4),
+//                                                           the last one cut off after the row's last block
 //   ps [E][N/16 tiles][ceil(NC/4)][64 lanes][4 bytes]     the E8M0 bytes, byte c % 4 = chunk c
 //
-// Chunk c, lane (ni = lane % 16, kb = lane / 16) holds block 4c + kb of row 16 tile + ni (blocks past
-// the row are zero weights with scale 1).  A wave's weights are one contiguous run read front to back
+// Chunk c, lane (ni = lane % 16, kb = lane / 16) holds block 4c + kb of row 16 tile + ni.  Blocks past
+// the row are not stored: their lanes load from beyond the tile's buffer descriptor, which returns
+// zero weights without touching memory (K = 2880 is 22.5 chunks: 2.2 % of the bytes).  A wave's weights are one contiguous run read front to back
 // with 1 KB loads - nontemporal, nothing is read twice - and land in matrix-core operand order: no
 // lane transpose, no scale staging.  The four 4-byte words of a lane's block serve four MFMA steps.
 // ---------------------------------------------------------------------------
@@ -484,7 +486,7 @@ __global__ __launch_bounds__(256) void mxfp4_repack_kernel(const uint8_t *__rest
     const int b = 4 * c + kb;
     const size_t row = et * 16 + ni;  // = expert * N + 16 tile + ni
     const bool valid = b < nb;
-    pw[idx] = valid ? ((const u32x4_t *)blocks)[row * nb + b] : u32x4_t{0u, 0u, 0u, 0u};
+    if (valid) pw[et * nb * 16 + c * 64 + lane] = ((const u32x4_t *)blocks)[row * nb + b];
     ps[((et * NG + (c >> 2)) * 64 + lane) * 4 + (c & 3)] = valid ? scales[row * nb + b] : (uint8_t)127;
     // the tail of the last scale word (chunks past NC) is never read as a scale of a real block; keep it defined
     if (c == NC - 1)
@@ -504,7 +506,7 @@ __global__ __launch_bounds__(256) void mxfp4_res_dequant_kernel(const u32x4_t *_
     const int b = 4 * c + kb;
     if (b >= nb) return;
     float w[32];
-    decode_block(pw[idx], e8m0_to_f32(ps[(((size_t)tile * NG + (c >> 2)) * 64 + lane) * 4 + (c & 3)]), w);
+    decode_block(pw[(size_t)tile * nb * 16 + c * 64 + lane], e8m0_to_f32(ps[(((size_t)tile * NG + (c >> 2)) * 64 + lane) * 4 + (c & 3)]), w);
     float *o = out + ((size_t)(16 * tile + ni) * nb + b) * 32;
 #pragma unroll
     for (int i = 0; i < 32; ++i) o[i] = w[i];
@@ -537,15 +539,17 @@ __global__ __launch_bounds__(NWV * 64) void mxfp4_res_kernel(const uint16_t *__r
     const int tile = blockIdx.x * NWV + wave;
     const bool active = tile < ntiles;  // wave-uniform
     const size_t et = (size_t)e * ntiles + (active ? tile : 0);
-    const __amdgpu_buffer_rsrc_t rs_w = make_rsrc(pw + et * NC * 64, active ? (uint32_t)NC * 1024u : 0u);
+    const __amdgpu_buffer_rsrc_t rs_w = make_rsrc(pw + et * nb * 16, active ? (uint32_t)nb * 256u : 0u);
     const __amdgpu_buffer_rsrc_t rs_s = make_rsrc(ps + et * NG * 256, active ? (uint32_t)NG * 256u : 0u);
     const int voff_w = lane * 16, voff_s = lane * 4;
     const int a_tok = (ni & (MTOK - 1)) * 16;
 
     u32x4_t wring[WR];
     uint32_t sring[WR / 4];
-    auto load_w = [&](int c) {  // chunks past the tile fall beyond the descriptor: zeros, no memory access
-        return __builtin_amdgcn_raw_buffer_load_b128(rs_w, c < NC ? voff_w : OOB, c * 1024, 2);
+    // blocks past the row get an offset beyond the descriptor: zeros, no memory access (the range check
+    // looks at the lane's offset only, not at the scalar one, so the lane has to carry it)
+    auto load_w = [&](int c) {
+        return __builtin_amdgcn_raw_buffer_load_b128(rs_w, 4 * c + kb < nb ? voff_w : OOB, c * 1024, 2);
     };
     auto load_s = [&](int g) { return __builtin_amdgcn_raw_buffer_load_b32(rs_s, g < NG ? voff_s : OOB, g * 256, 2); };
 
@@ -627,7 +631,7 @@ bool mxfp4_res_eligible(int64_t K, int64_t N) {
     return K % 32 == 0 && N % 16 == 0 && N > 0 && (K / 32) * (4 * 4 * 16 + 64) <= 96 * 1024 && K <= (1 << 24);
 }
 size_t mxfp4_res_weight_bytes(int64_t E, int64_t K, int64_t N) {
-    return (size_t)E * (size_t)(N / 16) * (size_t)ceil_div(K / 32, 4) * 1024;
+    return (size_t)E * (size_t)(N / 16) * (size_t)(K / 32) * 256;
 }
 size_t mxfp4_res_scale_bytes(int64_t E, int64_t K, int64_t N) {
     return (size_t)E * (size_t)(N / 16) * (size_t)ceil_div(ceil_div(K / 32, 4), 4) * 256;
@@ -654,7 +658,7 @@ int launch_mxfp4_res_dequant(oxq_ctx *ctx, hipStream_t s, const void *pw, const 
     dim3 grid((unsigned)ceil_div((int64_t)threads, 256)), block(256);
     set_plan(ctx, "mxfp4_res_dequant", grid, block, 1, 1, 0);
     if (ctx->plan_only) return OXQ_OK;
-    const u32x4_t *w = (const u32x4_t *)pw + (size_t)expert * (N / 16) * NC * 64;
+    const u32x4_t *w = (const u32x4_t *)pw + (size_t)expert * (N / 16) * nb * 16;
     const uint8_t *sc = (const uint8_t *)ps + (size_t)expert * (N / 16) * NG * 256;
     hipLaunchKernelGGL(mxfp4_res_dequant_kernel, grid, block, 0, s, w, sc, out_nk, (int)N, nb, NC, NG);
     OXQ_HIP_CHECK(hipGetLastError());
