@@ -1071,12 +1071,13 @@ int pk4_choose_strip(int64_t K, int64_t N, int bits, int64_t gate_half) {
     // 4096 x 4096 5.85 -> 3.74 us, 4096 x 6144 6.80 -> 4.69 us, 8192 x 4096 5.72 us; at 8 rows and more four
     // strips share a workgroup and the layer runs within 3 % of the wide form.  A single strip does the
     // per-block work on x (fragment reads, fold) for 1 KB of weights instead of 4 KB, so on long K it pays
-    // less: 14336 x 4096 8.54 us against 8.99 at one row but 1 - 5 % more from 8 rows on; that layer keeps
-    // the wide form.
+    // less: 11008 x 4096 7.16 / 7.92 us against 8.31 / 8.79 at 1 / 8 rows (9.61 against 9.29 at 16), but
+    // 14336 x 4096 8.58 us against 8.82 at one row and 2 - 3 % more from 8 rows on; that layer keeps the
+    // wide form.
     const int mode = pk4_env("OXQ_PK4_STRIP16", 1);  // 0 never, 1 by shape, 2 wherever the layout applies
     if (!mode || bits != 4 || gate_half || N % 64 != 0) return 64;
     if (mode == 2) return 16;
-    return (N / 64 <= 96 && N / 16 >= 128 && K / 128 >= 32 && K / 128 <= 64) ? 16 : 64;
+    return (N / 64 <= 96 && N / 16 >= 128 && K / 128 >= 32 && K / 128 <= 96) ? 16 : 64;
 }
 
 template <typename TT, int MT, bool GS, int NS, int XQ>
@@ -1127,6 +1128,8 @@ static int launch_pk4n_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p)
     const int64_t tiles = (N / (16 * ns)) * ceil_div(M, 16 * mt);
     int ks = 1;
     if (tiles <= 96 && NB >= 32) ks = (int)std::max<int64_t>(1, std::min<int64_t>(256 / tiles, NB / 8));
+    else if (ns == 4 && tiles <= 128 && NB >= 64) ks = 2;  // as in the wide form; 128 single strips are faster whole
+                                                           // (8192 x 2048 at one row: 5.20 against 5.65 us)
     ks = pk4_env("OXQ_PK4_KS", ks);
     ks = std::max(1, std::min(ks, NB));
     if (p.no_split) ks = 1;
