@@ -443,8 +443,9 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
         for (int q = 0; q < AQ; ++q) {
             if (VA1) {
                 if (q == 0) asm volatile("" : "+s"(rowstep));  // recomputed per block: 15 registers less to hold
-                const uint32_t v = (uint32_t)voff_a[0] + (uint32_t)q * rowstep;
-                a[q] = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)(v < (uint32_t)voff_a[0] ? (uint32_t)OOB : v), blk * 256, 0);
+                // no wrap-around: 15 row steps stay below 2^31 (K <= 2^24, checked on the host), so a row
+                // past M - from the first offset or by the steps - lies beyond x (< 2 GiB) and reads zeros
+                a[q] = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)((uint32_t)voff_a[0] + (uint32_t)q * rowstep), blk * 256, 0);
             } else {
                 a[q] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff_a[q], blk * 256, 0);
             }
@@ -799,8 +800,9 @@ __global__ __launch_bounds__(512) void pk4n_mfma_kernel(const uint16_t *__restri
         for (int q = 0; q < AQ; ++q) {
             if (VA1) {
                 if (q == 0) asm volatile("" : "+s"(rowstep));
-                const uint32_t v = (uint32_t)voff_a[0] + (uint32_t)q * rowstep;
-                a[q] = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)(v < (uint32_t)voff_a[0] ? (uint32_t)OOB : v), blk * 256, 0);
+                // no wrap-around: 15 row steps stay below 2^31 (K <= 2^24, checked on the host), so a row
+                // past M - from the first offset or by the steps - lies beyond x (< 2 GiB) and reads zeros
+                a[q] = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)((uint32_t)voff_a[0] + (uint32_t)q * rowstep), blk * 256, 0);
             } else {
                 a[q] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff_a[q], blk * 256, 0);
             }
@@ -939,7 +941,7 @@ bool pk4_eligible(const Wna16Problem &p) {
     if (p.bits != 4 && p.bits != 8) return false;
     if (p.K % 128 != 0 || p.N % 64 != 0 || p.group_size % 128 != 0) return false;
     // 32-bit offsets inside a strip and in x; one launch of the repack covers the copy
-    if ((uint64_t)(p.K / 128) * pk4_block_words(p.bits) * 4 >= (1ull << 31)) return false;
+    if ((uint64_t)(p.K / 128) * pk4_block_words(p.bits) * 4 >= (1ull << 31) || p.K > (1 << 24)) return false;
     if (pk4_weight_bytes(p.K, p.N, p.bits) / 4 >= (1ull << 31) * 256) return false;
     return true;
 }
