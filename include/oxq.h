@@ -455,6 +455,16 @@ int oxq_qlinear_new(oxq_ctx *ctx, int quant, const oxq_tensor *weight_bytes, int
                     oxq_qlinear **out);
 int oxq_qlinear_forward(oxq_qlinear *layer, void *stream, const oxq_tensor *x,
                         const oxq_tensor *out);
+/* linear.rs:225-240 (the fast path's own copy of the block bytes).  For Q4_0, Q8_0, Q4_K and Q6_K layers
+ * with out_features % 16 == 0 and in_features a multiple of 128 (256 for the K-quants) oxq_qlinear_new
+ * builds a layer-owned copy of the blocks in strips of 16 rows (the file's bytes per weight, so twice the
+ * layer's bytes while the caller keeps weight_bytes); forward then runs 1 - 4 rows of x on that copy and
+ * everything else on weight_bytes as before.  OXQ_PREPACK=0 in the environment turns the copy off.
+ * *resident = 1 if the layer holds the copy. */
+int oxq_qlinear_is_resident(const oxq_qlinear *layer, int *resident);
+/* Dense f32 [out_features, in_features] of the layer's weights, read from the copy when there is one:
+ * bit for bit what oxq_gguf_dequantize returns for weight_bytes. */
+int oxq_qlinear_dequantize(oxq_qlinear *layer, void *stream, const oxq_tensor *out);
 void oxq_qlinear_free(oxq_qlinear *layer);
 
 /* mxfp4.rs:67-169 Mxfp4Linear::{new, forward}. */

@@ -174,8 +174,15 @@ def run(ops, ctx, stream, steps, warmup, time_graph, with_cpu=True):
                                  "ms_per_call": round(per * 1e3, 3),
                                  "sample": f"{calls} calls of block dequant + f32 dot per row (restatement; candle's "
                                            "QMatMul, which the reference calls on the CPU, is not available here)"}
+        layers = [ops.QLinear(fmt, d[i], K, N, None, torch.float32, ctx=ctx) for i in range(nc)]
+        rr = _row("cfg3", f"gguf {synth.GGUF_NAMES[fmt]} M=1 K={K} N={N} f32 activations, QLinear.forward (resident "
+                          "strip-major copy of the blocks)",
+                  lambda i, layers=layers, nc=nc: layers[i % nc].forward(x, out=y), steps, warmup, stream, time_graph,
+                  nb, 2.0 * K * N, ctx)
+        rr["bare_read_nt_us"] = r["bare_read_nt_us"]
+        rows.append(rr)
         rows.append(r)
-        del d
+        del d, layers
 
     # ---- config 4 --------------------------------------------------------------------------------------
     E, top_k, H, I, T = 32, 4, 2880, 2880, 8

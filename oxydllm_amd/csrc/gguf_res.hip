@@ -1,0 +1,577 @@
+// Resident GGUF layers (linear.rs:197-247 GgufFastPath::build keeps a copy of the block bytes for the
+// life of the layer): a strip-major copy built once at load, and the decode GEMV that reads it.
+//
+// In the file layout a weight row is one run of blocks, so a kernel that gives a wave a row has to
+// stage all of x for every workgroup behind a barrier and fetches blocks of 18, 34, 144 or 210 bytes
+// that straddle every alignment.  The copy cuts the matrix into strips of 16 rows (output columns)
+// and chunks of 128 elements of K; lane (col = l % 16, kq = l / 16) of a chunk owns unit kq (32
+// consecutive elements) of row 16 strip + col:
+//
+//   block (CH chunks) = CH x { planes [64 lanes][16 B] (+ [64 lanes][8 B]) of quant bits,
+//                              [64 lanes][2 B] unit header (if the format has one) }
+//                       + [16 rows] block header (K-quants: the super-block's d / dmin / scales)
+//
+//   Q4_0  CH 1  16 B quants (the block's 16 bytes as stored), unit header d                    1152 B
+//   Q8_0  CH 1  32 B quants (as stored), unit header d                                         2176 B
+//   Q4_K  CH 2  16 B quants (element e in the low nibble of byte e, e + 16 in the high one),
+//               block header = the super-block's first 16 bytes (d, dmin, 12 scale bytes)      2304 B
+//   Q6_K  CH 2  16 B low nibbles (as Q4_K) + 8 B high bit pairs (element 16 h + 4 s + b in bits
+//               2s of byte b of word h), unit header = the unit's two int8 scales,
+//               block header = d                                                               3360 B
+//
+// Exactly the file's bytes per weight.  A wave's load of a plane is one contiguous 1 KB run; the 8
+// waves of a workgroup split the strip's chunks, each stages only its own part of x in its own LDS
+// slot (no workgroup barrier before the arithmetic), and the partial sums meet in LDS at the end in
+// a fixed order.  The arithmetic is the staged GEMV's: raw integers converted once,
+// y += a0 dot0 + a1 dot1 - b0 sum0 - b1 sum1 per unit (quant_kernels.metal:1097-1221, 1681-1838).
+#include "gguf_decode.hpp"
+
+namespace oxq {
+
+template <int FMT> struct GgrFmt;
+template <> struct GgrFmt<OXQ_GGUF_Q4_0> { static constexpr int CH = 1, QW = 4, UH = 2, BH = 0; };
+template <> struct GgrFmt<OXQ_GGUF_Q8_0> { static constexpr int CH = 1, QW = 8, UH = 2, BH = 0; };
+template <> struct GgrFmt<OXQ_GGUF_Q4_K> { static constexpr int CH = 2, QW = 4, UH = 0, BH = 16; };
+template <> struct GgrFmt<OXQ_GGUF_Q6_K> { static constexpr int CH = 2, QW = 6, UH = 2, BH = 2; };
+
+template <int FMT> struct GgrLayout {
+    typedef GgrFmt<FMT> F;
+    static constexpr int P128 = F::QW / 4, P64 = (F::QW % 4) / 2;
+    static constexpr int UH_OFF = 64 * F::QW * 4;            // unit headers behind the planes
+    static constexpr int CHB = 64 * (F::QW * 4 + F::UH);     // bytes of a chunk
+    static constexpr int BH_OFF = F::CH * CHB;               // block header behind the chunks
+    static constexpr int BLKB = F::CH * CHB + 16 * F::BH;    // bytes of a block
+    static_assert(BLKB == 16 * (128 * F::CH / GgufFmt<FMT>::BE) * GgufFmt<FMT>::BB, "the copy has the file's size");
+};
+
+// ---------------------------------------------------------------------------
+// repack: one thread per (strip, chunk, lane) = one unit of one row
+// ---------------------------------------------------------------------------
+template <int FMT>
+__global__ __launch_bounds__(256) void ggr_repack_kernel(const uint8_t *__restrict__ w, uint8_t *__restrict__ pw,
+                                                         int K, int N) {
+    typedef GgrFmt<FMT> F;
+    typedef GgrLayout<FMT> L;
+    const int nch = K >> 7;
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (size_t)(N >> 4) * nch * 64) return;
+    const int lane = (int)(idx & 63), c = (int)((idx >> 6) % nch), strip = (int)((idx >> 6) / nch);
+    const int col = lane & 15, kq = lane >> 4;
+    const int u = 4 * c + kq;
+    const size_t row_bytes = (size_t)(K / GgufFmt<FMT>::BE) * GgufFmt<FMT>::BB;
+    const uint8_t *row = w + (size_t)(16 * strip + col) * row_bytes;
+    uint8_t *blk = pw + ((size_t)strip * (nch / F::CH) + c / F::CH) * L::BLKB;
+    uint8_t *chunk = blk + (c % F::CH) * L::CHB;
+
+    uint32_t qw[F::QW];
+    uint32_t uh = 0;
+    if constexpr (FMT == OXQ_GGUF_Q4_0 || FMT == OXQ_GGUF_Q8_0) {
+        const uint8_t *p = row + (size_t)u * GgufFmt<FMT>::BB;
+        uh = ld16(p);
+#pragma unroll
+        for (int i = 0; i < F::QW; ++i) qw[i] = ld16(p + 2 + 4 * i) | (ld16(p + 4 + 4 * i) << 16);
+    } else if constexpr (FMT == OXQ_GGUF_Q4_K) {
+        const int b = u >> 3, sb = u & 7;
+        const uint8_t *p = row + (size_t)b * 144;
+        const uint8_t *qs = p + 16 + (sb >> 1) * 32;
+        const int sh = (sb & 1) * 4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            uint32_t v = 0;
+#pragma unroll
+            for (int bb = 0; bb < 4; ++bb) {
+                const uint32_t lo = ((uint32_t)qs[4 * i + bb] >> sh) & 0xFu, hi = ((uint32_t)qs[16 + 4 * i + bb] >> sh) & 0xFu;
+                v |= (lo | (hi << 4)) << (8 * bb);
+            }
+            qw[i] = v;
+        }
+        if (sb == 0) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) *(uint16_t *)(blk + L::BH_OFF + col * 16 + 2 * i) = (uint16_t)ld16(p + 2 * i);
+        }
+    } else {  // Q6_K
+        const int b = u >> 3, sub = u & 7;
+        const int h = sub >> 2, quad = sub & 3;
+        const uint8_t *p = row + (size_t)b * 210;
+        const uint8_t *ql = p + 64 * h + (quad & 1) * 32;
+        const uint8_t *qh = p + 128 + 32 * h;
+        const int shl = (quad < 2) ? 0 : 4, shh = 2 * quad;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            uint32_t v = 0;
+#pragma unroll
+            for (int bb = 0; bb < 4; ++bb) {
+                const uint32_t lo = ((uint32_t)ql[4 * i + bb] >> shl) & 0xFu, hi = ((uint32_t)ql[16 + 4 * i + bb] >> shl) & 0xFu;
+                v |= (lo | (hi << 4)) << (8 * bb);
+            }
+            qw[i] = v;
+        }
+#pragma unroll
+        for (int hs = 0; hs < 2; ++hs) {
+            uint32_t v = 0;
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+#pragma unroll
+                for (int bb = 0; bb < 4; ++bb)
+                    v |= (((uint32_t)qh[16 * hs + 4 * s + bb] >> shh) & 3u) << (8 * bb + 2 * s);
+            qw[4 + hs] = v;
+        }
+        uh = (uint32_t)p[192 + 2 * sub] | ((uint32_t)p[192 + 2 * sub + 1] << 8);
+        if (sub == 0) *(uint16_t *)(blk + L::BH_OFF + col * 2) = (uint16_t)ld16(p + 208);
+    }
+#pragma unroll
+    for (int pl = 0; pl < L::P128; ++pl)
+        *(u32x4_t *)(chunk + pl * 1024 + lane * 16) = u32x4_t{qw[4 * pl], qw[4 * pl + 1], qw[4 * pl + 2], qw[4 * pl + 3]};
+    if constexpr (L::P64) {
+        uint32_t *d = (uint32_t *)(chunk + L::P128 * 1024 + lane * 8);
+        d[0] = qw[4 * L::P128], d[1] = qw[4 * L::P128 + 1];
+    }
+    if constexpr (F::UH) *(uint16_t *)(chunk + L::UH_OFF + lane * 2) = (uint16_t)uh;
+}
+
+// ---------------------------------------------------------------------------
+// A unit from the copy: the stored unsigned integers as floats and the four factors of
+// a0*dot0 + a1*dot1 - b0*sum0 - b1*sum1 (as unit_ints does from the file layout).
+//   qw: the unit's quant words; uh: its header; bh: the block header words of its row; sb: index of
+//   the unit inside its block (K-quants).
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t v) { return (float)__builtin_bit_cast(_Float16, (uint16_t)v); }
+
+template <int FMT>
+__device__ __forceinline__ void ggr_factors(uint32_t uh, const uint32_t (&bh)[4], int sb, float &a0, float &a1,
+                                            float &b0, float &b1) {
+    if constexpr (FMT == OXQ_GGUF_Q4_0) {
+        const float d = f16_bits_to_f32(uh);
+        a0 = a1 = d, b0 = b1 = 8.0f * d;
+    } else if constexpr (FMT == OXQ_GGUF_Q8_0) {
+        const float d = f16_bits_to_f32(uh);
+        a0 = a1 = d, b0 = b1 = 128.0f * d;
+    } else if constexpr (FMT == OXQ_GGUF_Q4_K) {
+        const float d = f16_bits_to_f32(bh[0] & 0xFFFFu), dmin = f16_bits_to_f32(bh[0] >> 16);
+        // get_scale_min_k4 (quant_kernels.metal:2438-2450) on the 12 scale bytes in bh[1..3]
+        const uint32_t sft = 8u * (uint32_t)(sb & 3);
+        const uint32_t a = (bh[1] >> sft) & 0xFFu, b = (bh[2] >> sft) & 0xFFu, c = (bh[3] >> sft) & 0xFFu;
+        const uint32_t low = sb < 4 ? 0xFFFFFFFFu : 0u;
+        const uint32_t scv = ((a & 63u) & low) | (((c & 0x0Fu) | ((a >> 6) << 4)) & ~low);
+        const uint32_t mnv = ((b & 63u) & low) | (((c >> 4) | ((b >> 6) << 4)) & ~low);
+        a0 = a1 = d * (float)scv;
+        b0 = b1 = dmin * (float)mnv;
+    } else {  // Q6_K
+        const float d = f16_bits_to_f32(bh[0] & 0xFFFFu);
+        a0 = d * (float)(int)(int8_t)(uh & 0xFFu);
+        a1 = d * (float)(int)(int8_t)((uh >> 8) & 0xFFu);
+        b0 = 32.0f * a0, b1 = 32.0f * a1;
+    }
+}
+
+template <int FMT>
+__device__ __forceinline__ void ggr_ints(const uint32_t (&qw)[GgrFmt<FMT>::QW], float q[32]) {
+    if constexpr (FMT == OXQ_GGUF_Q8_0) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) bytes_to_f32(qw[i] ^ 0x80808080u, q + 4 * i);  // q + 128
+    } else if constexpr (FMT == OXQ_GGUF_Q6_K) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            bytes_to_f32((qw[i] & 0x0F0F0F0Fu) | (((qw[4] >> (2 * i)) & 0x03030303u) << 4), q + 4 * i);  // q + 32
+            bytes_to_f32(((qw[i] >> 4) & 0x0F0F0F0Fu) | (((qw[5] >> (2 * i)) & 0x03030303u) << 4), q + 16 + 4 * i);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            bytes_to_f32(qw[i] & 0x0F0F0F0Fu, q + 4 * i);
+            bytes_to_f32((qw[i] >> 4) & 0x0F0F0F0Fu, q + 16 + 4 * i);
+        }
+    }
+}
+
+// dense [N, K] f32 from the copy, with the arithmetic of decode_unit (pins the repack bit for bit)
+template <int FMT>
+__global__ __launch_bounds__(256) void ggr_dequant_kernel(const uint8_t *__restrict__ pw, float *__restrict__ out,
+                                                          int K, int N) {
+    typedef GgrFmt<FMT> F;
+    typedef GgrLayout<FMT> L;
+    const int nch = K >> 7;
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (size_t)(N >> 4) * nch * 64) return;
+    const int lane = (int)(idx & 63), c = (int)((idx >> 6) % nch), strip = (int)((idx >> 6) / nch);
+    const int col = lane & 15, kq = lane >> 4;
+    const uint8_t *blk = pw + ((size_t)strip * (nch / F::CH) + c / F::CH) * L::BLKB;
+    const uint8_t *chunk = blk + (c % F::CH) * L::CHB;
+    uint32_t qw[F::QW];
+#pragma unroll
+    for (int pl = 0; pl < L::P128; ++pl) {
+        const u32x4_t v = *(const u32x4_t *)(chunk + pl * 1024 + lane * 16);
+        qw[4 * pl] = v[0], qw[4 * pl + 1] = v[1], qw[4 * pl + 2] = v[2], qw[4 * pl + 3] = v[3];
+    }
+    if constexpr (L::P64) {
+        const uint32_t *d = (const uint32_t *)(chunk + L::P128 * 1024 + lane * 8);
+        qw[4 * L::P128] = d[0], qw[4 * L::P128 + 1] = d[1];
+    }
+    uint32_t uh = 0, bh[4] = {0u, 0u, 0u, 0u};
+    if constexpr (F::UH) uh = *(const uint16_t *)(chunk + L::UH_OFF + lane * 2);
+    if constexpr (F::BH == 16) {
+        const u32x4_t v = *(const u32x4_t *)(blk + L::BH_OFF + col * 16);
+        bh[0] = v[0], bh[1] = v[1], bh[2] = v[2], bh[3] = v[3];
+    } else if constexpr (F::BH == 2) {
+        bh[0] = *(const uint16_t *)(blk + L::BH_OFF + col * 2);
+    }
+    const int sb = 4 * (c % F::CH) + kq;
+    float wf[32];
+    if constexpr (FMT == OXQ_GGUF_Q4_0) {
+        const float d = f16_bits_to_f32(uh);
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const uint32_t byte = (qw[e >> 2] >> (8 * (e & 3))) & 0xFFu;
+            wf[e] = (float)((int)(byte & 0xF) - 8) * d;
+            wf[e + 16] = (float)((int)(byte >> 4) - 8) * d;
+        }
+    } else if constexpr (FMT == OXQ_GGUF_Q8_0) {
+        const float d = f16_bits_to_f32(uh);
+#pragma unroll
+        for (int e = 0; e < 32; ++e) wf[e] = (float)(int)(int8_t)((qw[e >> 2] >> (8 * (e & 3))) & 0xFFu) * d;
+    } else if constexpr (FMT == OXQ_GGUF_Q4_K) {
+        float sc_v, m_v, t0, t1;
+        ggr_factors<FMT>(uh, bh, sb, sc_v, t0, m_v, t1);
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const uint32_t byte = (qw[e >> 2] >> (8 * (e & 3))) & 0xFFu;
+            wf[e] = sc_v * (float)(byte & 0xF) - m_v;
+            wf[e + 16] = sc_v * (float)(byte >> 4) - m_v;
+        }
+    } else {
+        float s0, s1, t0, t1;
+        ggr_factors<FMT>(uh, bh, sb, s0, s1, t0, t1);
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const uint32_t byte = (qw[e >> 2] >> (8 * (e & 3))) & 0xFFu;
+            const uint32_t h0 = (qw[4] >> (8 * (e & 3) + 2 * (e >> 2))) & 3u, h1 = (qw[5] >> (8 * (e & 3) + 2 * (e >> 2))) & 3u;
+            wf[e] = s0 * (float)((int)((byte & 0xF) | (h0 << 4)) - 32);
+            wf[e + 16] = s1 * (float)((int)((byte >> 4) | (h1 << 4)) - 32);
+        }
+    }
+    float *o = out + (size_t)(16 * strip + col) * K + (size_t)(4 * c + kq) * 32;
+#pragma unroll
+    for (int i = 0; i < 32; ++i) o[i] = wf[i];
+}
+
+// ---------------------------------------------------------------------------
+// Decode GEMV on the copy.  grid.x = strips, 8 waves; wave w takes a contiguous run of the strip's
+// chunks, stages its own part of the MB activation rows in its own LDS slot (as f32, unit by unit
+// with one 16-byte pad a unit, then the sums of x over every 16 elements) and walks its chunks with
+// RD chunks of weights in flight.
+// ---------------------------------------------------------------------------
+template <int FMT, bool BF16X, int MB, int NW>
+__global__ __launch_bounds__(NW * 64) void ggr_gemv_kernel(const void *__restrict__ x, const uint8_t *__restrict__ pw,
+                                                       const void *__restrict__ bias, void *__restrict__ y, int M,
+                                                       int K, int N, int nmax) {
+    typedef GgrFmt<FMT> F;
+    typedef GgrLayout<FMT> L;
+    constexpr int RD = NW == 8 ? 4 : 2, OOB = 0x7FFFFF00;
+    constexpr int XP = 144;                                    // bytes of a unit's 32 floats + one pad chunk
+    extern __shared__ __attribute__((aligned(16))) unsigned char gr_lds[];
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int col = lane & 15, kq = lane >> 4;
+    const int strip = blockIdx.x;
+    const int nch = K >> 7;
+    const int cbase = nch / NW, crem = nch % NW;
+    const int n = cbase + (wave < crem ? 1 : 0);               // this wave's chunks: [c0, c0 + n)
+    const int c0 = wave * cbase + min(wave, crem);
+    const size_t xrow = (size_t)nmax * 4 * (XP + 8);           // a row's units, then two sums a unit (multiple of 16)
+    unsigned char *slot = gr_lds + (size_t)wave * MB * xrow;
+    float *red = (float *)(gr_lds + (size_t)NW * MB * xrow);   // [MB][16][NW] partial sums
+
+    const __amdgpu_buffer_rsrc_t rs_w =
+        make_rsrc(pw + (size_t)strip * (nch / F::CH) * L::BLKB, (uint32_t)(nch / F::CH) * (uint32_t)L::BLKB);
+    const __amdgpu_buffer_rsrc_t rs_none = make_rsrc(pw, 0u);
+
+    struct Stage {
+        uint32_t qw[F::QW];
+        uint32_t uh;
+        uint32_t bh[4];
+    };
+    Stage ring[RD];
+    auto load = [&](int i, Stage &st) {  // chunk i of the wave; past its share through an empty descriptor
+        const __amdgpu_buffer_rsrc_t rs = i < n ? rs_w : rs_none;
+        const int c = c0 + i;
+        const int boff = (c / F::CH) * L::BLKB, coff = boff + (c % F::CH) * L::CHB;
+#pragma unroll
+        for (int pl = 0; pl < L::P128; ++pl) {
+            const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(rs, lane * 16, coff + pl * 1024, 2);
+            st.qw[4 * pl] = v[0], st.qw[4 * pl + 1] = v[1], st.qw[4 * pl + 2] = v[2], st.qw[4 * pl + 3] = v[3];
+        }
+        if constexpr (L::P64) {
+            typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+            const u32x2_t v = __builtin_amdgcn_raw_buffer_load_b64(rs, lane * 8, coff + L::P128 * 1024, 2);
+            st.qw[4 * L::P128] = v[0], st.qw[4 * L::P128 + 1] = v[1];
+        }
+        st.uh = 0;
+        if constexpr (F::UH) st.uh = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(rs, lane * 2, coff + L::UH_OFF, 2);
+        st.bh[0] = st.bh[1] = st.bh[2] = st.bh[3] = 0;
+        if constexpr (F::BH == 16) {
+            const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(rs, col * 16, boff + L::BH_OFF, 0);
+            st.bh[0] = v[0], st.bh[1] = v[1], st.bh[2] = v[2], st.bh[3] = v[3];
+        } else if constexpr (F::BH == 2) {
+            st.bh[0] = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(rs, col * 2, boff + L::BH_OFF, 0);
+        }
+    };
+    // this wave's part of x: elements [128 c0, 128 (c0 + n)) of every row, staged as f32 in 16-byte
+    // pieces of the source; with them the sums of x over every 16 elements, from the registers that
+    // carry x: the piece's own elements, then the 4 (bf16: 2) pieces of a half unit, which
+    // neighbouring lanes hold.  The first batch of row 0 is requested before the first weights (both are
+    // needed to start; x is the smaller), its stores come after the weights' requests.
+    constexpr int XB = BF16X ? 2 : 4, EPP = 16 / XB;       // elements a 16-byte piece of x
+    const int pieces = n * 128 / EPP;
+    const __amdgpu_buffer_rsrc_t rs_x = make_rsrc(x, (uint32_t)M * (uint32_t)K * (uint32_t)XB);
+    auto x_load = [&](int m, int base, u32x4_t (&v)[4]) {
+        const int rowoff = m < M ? m * K * XB + c0 * 128 * XB : OOB;
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            const int p = base + b * 64 + lane;
+            v[b] = __builtin_amdgcn_raw_buffer_load_b128(rs_x, p < pieces ? rowoff + p * 16 : OOB, 0, 0);
+        }
+    };
+    auto x_store = [&](int m, int base, const u32x4_t (&v)[4]) {
+        unsigned char *xr = slot + m * xrow;
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            const int p = base + b * 64 + lane;
+            float sx;
+            if constexpr (BF16X) {
+                sx = 0.0f;
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    sx += __builtin_bit_cast(float, (uint32_t)v[b][j] << 16) +
+                          __builtin_bit_cast(float, (uint32_t)v[b][j] & 0xFFFF0000u);
+                sx += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, sx), 0xB1, 0xF, 0xF, false));
+            } else {
+                sx = (__builtin_bit_cast(float, (uint32_t)v[b][0]) + __builtin_bit_cast(float, (uint32_t)v[b][1])) +
+                     (__builtin_bit_cast(float, (uint32_t)v[b][2]) + __builtin_bit_cast(float, (uint32_t)v[b][3]));
+                sx += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, sx), 0xB1, 0xF, 0xF, false));
+                sx += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, sx), 0x4E, 0xF, 0xF, false));
+            }
+            if (p < pieces) {
+                constexpr int PPH = BF16X ? 2 : 4;  // pieces a half unit
+                if ((p & (PPH - 1)) == 0) ((float *)(xr + (size_t)nmax * 4 * XP))[p / PPH] = sx;
+                if constexpr (BF16X) {
+                    const int u = p >> 2, cc = (p & 3) * 2;
+                    float4_t lo, hi;
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) {
+                        lo[2 * j] = __builtin_bit_cast(float, (uint32_t)v[b][j] << 16);
+                        lo[2 * j + 1] = __builtin_bit_cast(float, (uint32_t)v[b][j] & 0xFFFF0000u);
+                        hi[2 * j] = __builtin_bit_cast(float, (uint32_t)v[b][2 + j] << 16);
+                        hi[2 * j + 1] = __builtin_bit_cast(float, (uint32_t)v[b][2 + j] & 0xFFFF0000u);
+                    }
+                    *(float4_t *)(xr + u * XP + cc * 16) = lo;
+                    *(float4_t *)(xr + u * XP + cc * 16 + 16) = hi;
+                } else {
+                    *(u32x4_t *)(xr + (p >> 3) * XP + (p & 7) * 16) = v[b];
+                }
+            }
+        }
+    };
+    {
+        u32x4_t v0[4];
+        x_load(0, 0, v0);
+#pragma unroll
+        for (int d = 0; d < RD; ++d) load(d, ring[d]);
+        x_store(0, 0, v0);
+#pragma unroll
+        for (int m = 0; m < MB; ++m)
+            for (int base = m ? 0 : 256; base < pieces; base += 256) {
+                u32x4_t v[4];
+                x_load(m, base, v);
+                x_store(m, base, v);
+            }
+    }
+
+    float acc[MB];
+#pragma unroll
+    for (int m = 0; m < MB; ++m) acc[m] = 0.0f;
+    const int nround = (n + RD - 1) / RD * RD;
+    for (int i0 = 0; i0 < nround; i0 += RD) {
+#pragma unroll
+        for (int d = 0; d < RD; ++d) {
+            const int i = i0 + d;
+            const Stage st = ring[d];
+            load(i + RD, ring[d]);
+            float q[32], a0, a1, b0, b1;
+            ggr_ints<FMT>(st.qw, q);
+            ggr_factors<FMT>(st.uh, st.bh, 4 * ((c0 + i) % F::CH) + kq, a0, a1, b0, b1);
+            // chunks past the share hold zeros (a = b = 0); their x comes from the share's last chunk
+            const int uw = 4 * min(i, n - 1) + kq;
+#pragma unroll
+            for (int m = 0; m < MB; ++m) {
+                const unsigned char *xr = slot + m * xrow;
+                const float4_t *xu = (const float4_t *)(xr + uw * XP);
+                const float2 sx = *(const float2 *)(xr + (size_t)nmax * 4 * XP + uw * 8);
+                float dot0 = 0.0f, dot1 = 0.0f;
+#pragma unroll
+                for (int o = 0; o < 8; ++o) {
+                    const float4_t xv = xu[o];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        if (o < 4) dot0 = fmaf(q[4 * o + e], xv[e], dot0);
+                        else dot1 = fmaf(q[4 * o + e], xv[e], dot1);
+                    }
+                }
+                acc[m] += (a0 * dot0 + a1 * dot1) - (b0 * sx.x + b1 * sx.y);
+            }
+        }
+    }
+    // the four units of a column inside the wave (lanes l, l + 16, l + 32, l + 48), then the waves through LDS:
+    // red [MB][16 columns][NW waves]
+#pragma unroll
+    for (int m = 0; m < MB; ++m) {
+        float v = acc[m];
+        v += __shfl_xor(v, 16, 64);
+        v += __shfl_xor(v, 32, 64);
+        if (lane < 16) red[(m * 16 + lane) * NW + wave] = v;
+    }
+    __syncthreads();
+    if (threadIdx.x < 16 * MB) {
+        const int m = threadIdx.x >> 4, c = threadIdx.x & 15;
+        if (m < M) {
+            const float4_t *r4 = (const float4_t *)(red + (m * 16 + c) * NW);
+            float tot = 0.0f;
+#pragma unroll
+            for (int w = 0; w < NW / 4; ++w) {
+                const float4_t t = r4[w];
+                tot += (t[0] + t[1]) + (t[2] + t[3]);
+            }
+            const int nn = 16 * strip + c;
+            if constexpr (BF16X) {
+                if (bias) tot += BF16Traits::to_f32(((const uint16_t *)bias)[nn]);
+                ((uint16_t *)y)[(size_t)m * N + nn] = BF16Traits::from_f32(tot);
+            } else {
+                if (bias) tot += ((const float *)bias)[nn];
+                ((float *)y)[(size_t)m * N + nn] = tot;
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------
+static bool ggr_format(int quant) {
+    return quant == OXQ_GGUF_Q4_0 || quant == OXQ_GGUF_Q8_0 || quant == OXQ_GGUF_Q4_K || quant == OXQ_GGUF_Q6_K;
+}
+static int ggr_chunks_per_block(int quant) { return (quant == OXQ_GGUF_Q4_K || quant == OXQ_GGUF_Q6_K) ? 2 : 1; }
+
+bool gguf_res_eligible(int quant, int64_t K, int64_t N) {
+    if (!ggr_format(quant) || N <= 0 || N % 16 != 0 || K <= 0 || K % (128 * ggr_chunks_per_block(quant)) != 0) return false;
+    int64_t be = 0, bb = 0;
+    oxq_gguf_block_layout(quant, &be, &bb);
+    // 32-bit offsets inside a strip and in x
+    return (uint64_t)(K / be) * (uint64_t)bb * 16 < (1ull << 31) && K <= (1 << 22);
+}
+size_t gguf_res_bytes(int quant, int64_t K, int64_t N) {
+    int64_t be = 0, bb = 0;
+    oxq_gguf_block_layout(quant, &be, &bb);
+    return (size_t)N * (size_t)(K / be) * (size_t)bb;
+}
+
+static int ggr_waves(int64_t K) {
+    const char *e = getenv("OXQ_GGR_WAVES");
+    const int w = e ? atoi(e) : 16;
+    return (w == 8 || K / 128 < 16) ? 8 : 16;
+}
+static size_t ggr_lds_bytes(int64_t K, int mb) {
+    const int nw = ggr_waves(K);
+    const int64_t nmax = ceil_div(K / 128, nw);
+    return (size_t)nw * mb * (size_t)nmax * 4 * (144 + 8) + (size_t)nw * mb * 64 * 4;
+}
+// rows of x one launch of the resident GEMV takes (more go to the kernels on the file layout)
+bool gguf_res_takes(int64_t K, int64_t M) {
+    if (M < 1 || M > 4) return false;
+    return ggr_lds_bytes(K, M <= 1 ? 1 : M <= 2 ? 2 : 4) <= 144 * 1024;
+}
+
+static const char *ggr_name(int q) {
+    return q == OXQ_GGUF_Q4_0 ? "q4_0" : q == OXQ_GGUF_Q8_0 ? "q8_0" : q == OXQ_GGUF_Q4_K ? "q4k" : "q6k";
+}
+
+int launch_gguf_res_repack(oxq_ctx *ctx, hipStream_t s, int quant, const uint8_t *w, void *pw, int64_t K, int64_t N) {
+    const size_t threads = (size_t)(N / 16) * (K / 128) * 64;
+    dim3 grid((unsigned)ceil_div((int64_t)threads, 256)), block(256);
+    char name[64];
+    snprintf(name, sizeof name, "gguf_%s_repack", ggr_name(quant));
+    set_plan(ctx, name, grid, block, 1, 1, 0);
+    if (ctx->plan_only) return OXQ_OK;
+#define OXQ_GR(F) \
+    case F: hipLaunchKernelGGL((ggr_repack_kernel<F>), grid, block, 0, s, w, (uint8_t *)pw, (int)K, (int)N); break
+    switch (quant) {
+        OXQ_GR(OXQ_GGUF_Q4_0);
+        OXQ_GR(OXQ_GGUF_Q8_0);
+        OXQ_GR(OXQ_GGUF_Q4_K);
+        OXQ_GR(OXQ_GGUF_Q6_K);
+    default: return fail(OXQ_ERR_UNSUPPORTED, "gguf repack: format %d has no resident layout", quant);
+    }
+#undef OXQ_GR
+    OXQ_HIP_CHECK(hipGetLastError());
+    return OXQ_OK;
+}
+
+int launch_gguf_res_dequant(oxq_ctx *ctx, hipStream_t s, int quant, const void *pw, int64_t K, int64_t N, float *out_nk) {
+    const size_t threads = (size_t)(N / 16) * (K / 128) * 64;
+    dim3 grid((unsigned)ceil_div((int64_t)threads, 256)), block(256);
+    char name[64];
+    snprintf(name, sizeof name, "gguf_%s_res_dequant", ggr_name(quant));
+    set_plan(ctx, name, grid, block, 1, 1, 0);
+    if (ctx->plan_only) return OXQ_OK;
+#define OXQ_GR(F) \
+    case F: hipLaunchKernelGGL((ggr_dequant_kernel<F>), grid, block, 0, s, (const uint8_t *)pw, out_nk, (int)K, (int)N); break
+    switch (quant) {
+        OXQ_GR(OXQ_GGUF_Q4_0);
+        OXQ_GR(OXQ_GGUF_Q8_0);
+        OXQ_GR(OXQ_GGUF_Q4_K);
+        OXQ_GR(OXQ_GGUF_Q6_K);
+    default: return fail(OXQ_ERR_UNSUPPORTED, "gguf dequant: format %d has no resident layout", quant);
+    }
+#undef OXQ_GR
+    OXQ_HIP_CHECK(hipGetLastError());
+    return OXQ_OK;
+}
+
+template <int FMT, bool BF16X, int MB, int NW>
+static int ggr_go(hipStream_t s, dim3 grid, const GgufProblem &p, size_t lds, int nmax) {
+    static LdsGrant lds_grant;  // one per instantiation
+    OXQ_HIP_CHECK(lds_grant.ensure((const void *)ggr_gemv_kernel<FMT, BF16X, MB, NW>, lds));
+    hipLaunchKernelGGL((ggr_gemv_kernel<FMT, BF16X, MB, NW>), grid, dim3(NW * 64), lds, s, p.x, p.w, p.bias, p.y,
+                       (int)p.M, (int)p.K, (int)p.N, nmax);
+    OXQ_HIP_CHECK(hipGetLastError());
+    return OXQ_OK;
+}
+template <int FMT, int NW>
+static int ggr_by_rows(hipStream_t s, dim3 grid, const GgufProblem &p, size_t lds, int nmax, int mb) {
+    const bool bf = p.act_dtype == OXQ_BF16;
+    if (mb == 1) return bf ? ggr_go<FMT, true, 1, NW>(s, grid, p, lds, nmax) : ggr_go<FMT, false, 1, NW>(s, grid, p, lds, nmax);
+    if (mb == 2) return bf ? ggr_go<FMT, true, 2, NW>(s, grid, p, lds, nmax) : ggr_go<FMT, false, 2, NW>(s, grid, p, lds, nmax);
+    return bf ? ggr_go<FMT, true, 4, NW>(s, grid, p, lds, nmax) : ggr_go<FMT, false, 4, NW>(s, grid, p, lds, nmax);
+}
+
+// p.w is the resident copy
+int launch_gguf_res_gemv(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p) {
+    const int mb = p.M <= 1 ? 1 : p.M <= 2 ? 2 : 4;
+    const int nw = ggr_waves(p.K);
+    const int nmax = (int)ceil_div(p.K / 128, nw);
+    const size_t lds = ggr_lds_bytes(p.K, mb);
+    dim3 grid((unsigned)(p.N / 16));
+    char name[64];
+    snprintf(name, sizeof name, "gguf_%s_res_gemv_%s_m%d", ggr_name(p.quant), p.act_dtype == OXQ_BF16 ? "bf16" : "f32", mb);
+    set_plan(ctx, name, grid, dim3(nw * 64), 1, 1, 0);
+    if (ctx->plan_only) return OXQ_OK;
+    if (!gguf_res_takes(p.K, p.M)) return fail(OXQ_ERR_UNSUPPORTED, "gguf resident gemv: m = %lld", (long long)p.M);
+    if ((uintptr_t)p.x & 15) return fail(OXQ_ERR_UNSUPPORTED, "gguf resident gemv: x must be 16-byte aligned");
+    if ((uint64_t)p.M * (uint64_t)p.K * 4 >= (1ull << 31)) return fail(OXQ_ERR_UNSUPPORTED, "gguf resident gemv: x larger than 2 GiB");
+    switch (p.quant) {
+    case OXQ_GGUF_Q4_0: return nw == 8 ? ggr_by_rows<OXQ_GGUF_Q4_0, 8>(s, grid, p, lds, nmax, mb) : ggr_by_rows<OXQ_GGUF_Q4_0, 16>(s, grid, p, lds, nmax, mb);
+    case OXQ_GGUF_Q8_0: return nw == 8 ? ggr_by_rows<OXQ_GGUF_Q8_0, 8>(s, grid, p, lds, nmax, mb) : ggr_by_rows<OXQ_GGUF_Q8_0, 16>(s, grid, p, lds, nmax, mb);
+    case OXQ_GGUF_Q4_K: return nw == 8 ? ggr_by_rows<OXQ_GGUF_Q4_K, 8>(s, grid, p, lds, nmax, mb) : ggr_by_rows<OXQ_GGUF_Q4_K, 16>(s, grid, p, lds, nmax, mb);
+    case OXQ_GGUF_Q6_K: return nw == 8 ? ggr_by_rows<OXQ_GGUF_Q6_K, 8>(s, grid, p, lds, nmax, mb) : ggr_by_rows<OXQ_GGUF_Q6_K, 16>(s, grid, p, lds, nmax, mb);
+    default: return fail(OXQ_ERR_UNSUPPORTED, "gguf resident gemv: format %d", p.quant);
+    }
+}
+
+}  // namespace oxq

@@ -1704,7 +1704,39 @@ struct oxq_qlinear {
     int64_t in_features, out_features;
     int quant;
     int out_dtype;
+    void *res = nullptr;    // layer-owned strip-major copy of the blocks (decode GEMV)
+    bool resident = false;
 };
+
+// linear.rs:225-240: the fast path copies the block bytes at build; here the copy is strip-major
+static int build_resident_gguf(oxq_qlinear *l) {
+    const char *env = getenv("OXQ_PREPACK");
+    if (env && atoi(env) == 0) return OXQ_OK;
+    if (!gguf_res_eligible(l->quant, l->in_features, l->out_features)) return OXQ_OK;
+    if (((uintptr_t)l->weight_bytes.data & 1) != 0) return OXQ_OK;
+    oxq_ctx *ctx = l->ctx;
+    if (ctx->plan_only) {
+        l->resident = true;
+        return OXQ_OK;
+    }
+    int prev = 0;
+    (void)hipGetDevice(&prev);
+    OXQ_HIP_CHECK(hipSetDevice(ctx->device));
+    int rc = OXQ_OK;
+    hipError_t e = hipMalloc(&l->res, gguf_res_bytes(l->quant, l->in_features, l->out_features));
+    if (e != hipSuccess) {
+        l->res = nullptr;
+        rc = fail(OXQ_ERR_RUNTIME, "QLinear: repack allocation failed: %s", hipGetErrorString(e));
+    } else {
+        rc = launch_gguf_res_repack(ctx, nullptr, l->quant, (const uint8_t *)l->weight_bytes.data, l->res, l->in_features,
+                                    l->out_features);
+        if (rc == OXQ_OK && (e = hipStreamSynchronize(nullptr)) != hipSuccess)
+            rc = fail(OXQ_ERR_RUNTIME, "QLinear: repack failed: %s", hipGetErrorString(e));
+    }
+    (void)hipSetDevice(prev);
+    if (rc == OXQ_OK) l->resident = true;
+    return rc;
+}
 
 struct oxq_mxfp4_linear {
     oxq_ctx *ctx;
@@ -1909,6 +1941,11 @@ int oxq_qlinear_new(oxq_ctx *ctx, int quant, const oxq_tensor *weight_bytes, int
     l->out_features = out_features;
     l->quant = quant;
     l->out_dtype = out_dtype;
+    const int rc = build_resident_gguf(l);
+    if (rc != OXQ_OK) {
+        oxq_qlinear_free(l);
+        return rc;
+    }
     *out = l;
     return OXQ_OK;
 }
@@ -1929,11 +1966,47 @@ int oxq_qlinear_forward(oxq_qlinear *l, void *stream, const oxq_tensor *x, const
     OXQ_TRY(check_gguf(l->ctx, decode ? "GgufQuantMatmul" : "GgufQuantMulMM", decode, false, &x2,
                        &l->weight_bytes, l->in_features, l->out_features, l->quant, &o2, &p));
     p.bias = l->has_bias ? l->bias.data : nullptr;
+    if (l->resident && gguf_res_takes(p.K, p.M) && ((uintptr_t)p.x & 15) == 0) {
+        p.w = (const uint8_t *)l->res;
+        return launch_gguf_res_gemv(l->ctx, (hipStream_t)stream, p);
+    }
     if (gguf_mm_eligible(p)) return launch_gguf_mm(l->ctx, (hipStream_t)stream, p);
     return launch_gguf_gemv(l->ctx, (hipStream_t)stream, p);
 }
 
-void oxq_qlinear_free(oxq_qlinear *l) { delete l; }
+int oxq_qlinear_is_resident(const oxq_qlinear *l, int *resident) {
+    if (!l || !resident) return fail(OXQ_ERR_ARG, "QLinear: NULL argument");
+    *resident = l->resident ? 1 : 0;
+    return OXQ_OK;
+}
+
+int oxq_qlinear_dequantize(oxq_qlinear *l, void *stream, const oxq_tensor *out) {
+    const char *op = "QLinear dequantize";
+    if (!l) return fail(OXQ_ERR_ARG, "%s: layer is NULL", op);
+    OXQ_TRY(check_tensor(l->ctx, op, "out", out));
+    if (out->dtype != OXQ_F32 || out->rank != 2 || out->dims[0] != l->out_features || out->dims[1] != l->in_features)
+        return fail(OXQ_ERR_SHAPE, "%s: out must be F32 [%lld, %lld]", op, (long long)l->out_features,
+                    (long long)l->in_features);
+    if (l->resident)
+        return launch_gguf_res_dequant(l->ctx, (hipStream_t)stream, l->quant, l->res, l->in_features, l->out_features,
+                                       (float *)out->data);
+    GgufProblem p{};
+    p.w = (const uint8_t *)l->weight_bytes.data;
+    p.K = l->in_features, p.N = l->out_features, p.quant = l->quant, p.act_dtype = OXQ_F32;
+    return launch_gguf_dequant(l->ctx, (hipStream_t)stream, p, (float *)out->data);
+}
+
+void oxq_qlinear_free(oxq_qlinear *l) {
+    if (!l) return;
+    if (l->res) {
+        int prev = 0;
+        (void)hipGetDevice(&prev);
+        (void)hipSetDevice(l->ctx->device);
+        (void)hipFree(l->res);
+        (void)hipSetDevice(prev);
+    }
+    delete l;
+}
 
 // mxfp4.rs:78-116 Mxfp4Linear::new
 int oxq_mxfp4_linear_new(oxq_ctx *ctx, const oxq_tensor *blocks, const oxq_tensor *scales,

@@ -617,6 +617,7 @@ class QLinear:
         self.ctx = _ctx(ctx)
         self._keep = (weight_bytes, bias)
         self.handle = C.c_void_p()
+        self.in_features = in_features
         self.out_features = out_features
         _lib.check(self.ctx._lib.oxq_qlinear_new(
             self.ctx.handle, quant, desc(weight_bytes), in_features, out_features, desc(bias),
@@ -628,6 +629,20 @@ class QLinear:
                               device=x.device)
         _lib.check(self.ctx._lib.oxq_qlinear_forward(self.handle, self.ctx.stream(), desc(x),
                                                      desc(out)))
+        return out
+
+    @property
+    def resident(self) -> bool:
+        """True if the layer holds the strip-major copy that 1 - 4 rows of x run on."""
+        r = C.c_int(0)
+        _lib.check(self.ctx._lib.oxq_qlinear_is_resident(self.handle, C.byref(r)))
+        return bool(r.value)
+
+    def dequantize(self) -> torch.Tensor:
+        """Dense f32 [out_features, in_features], read from the layer's copy when it holds one."""
+        out = torch.empty((self.out_features, self.in_features), dtype=torch.float32,
+                          device=self._keep[0].device)
+        _lib.check(self.ctx._lib.oxq_qlinear_dequantize(self.handle, self.ctx.stream(), desc(out)))
         return out
 
     def __del__(self):
