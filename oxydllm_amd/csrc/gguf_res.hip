@@ -267,21 +267,23 @@ __global__ __launch_bounds__(NW * 64) void ggr_gemv_kernel(const void *__restric
     typedef GgrFmt<FMT> F;
     typedef GgrLayout<FMT> L;
     constexpr int RD = NW == 8 ? 4 : 2, OOB = 0x7FFFFF00;
+    constexpr int GR = 4;                                      // strips between two meetings of the workgroup
     constexpr int XP = 144;                                    // bytes of a unit's 32 floats + one pad chunk
     extern __shared__ __attribute__((aligned(16))) unsigned char gr_lds[];
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int col = lane & 15, kq = lane >> 4;
-    const int strip = blockIdx.x;
+    int strip = blockIdx.x;
+    const int nstrips = N >> 4;
     const int nch = K >> 7;
     const int cbase = nch / NW, crem = nch % NW;
     const int n = cbase + (wave < crem ? 1 : 0);               // this wave's chunks: [c0, c0 + n)
     const int c0 = wave * cbase + min(wave, crem);
     const size_t xrow = (size_t)nmax * 4 * (XP + 8);           // a row's units, then two sums a unit (multiple of 16)
     unsigned char *slot = gr_lds + (size_t)wave * MB * xrow;
-    float *red = (float *)(gr_lds + (size_t)NW * MB * xrow);   // [MB][16][NW] partial sums
+    float *red0 = (float *)(gr_lds + (size_t)NW * MB * xrow);  // 2 x GR x [MB][16][NW] partial sums
 
-    const __amdgpu_buffer_rsrc_t rs_w =
-        make_rsrc(pw + (size_t)strip * (nch / F::CH) * L::BLKB, (uint32_t)(nch / F::CH) * (uint32_t)L::BLKB);
+    const size_t strip_bytes = (size_t)(nch / F::CH) * L::BLKB;
+    __amdgpu_buffer_rsrc_t rs_w = make_rsrc(pw + (size_t)strip * strip_bytes, (uint32_t)strip_bytes);
     const __amdgpu_buffer_rsrc_t rs_none = make_rsrc(pw, 0u);
 
     struct Stage {
@@ -385,6 +387,10 @@ __global__ __launch_bounds__(NW * 64) void ggr_gemv_kernel(const void *__restric
             }
     }
 
+    // a workgroup walks the strips blockIdx.x, + gridDim.x, ...: x is staged once
+    for (int it = 0;; ++it) {
+    const int r = it % GR, half = (it / GR) & 1;
+    float *red = red0 + (half * GR + r) * (MB * 16 * NW);
     float acc[MB];
 #pragma unroll
     for (int m = 0; m < MB; ++m) acc[m] = 0.0f;
@@ -419,8 +425,18 @@ __global__ __launch_bounds__(NW * 64) void ggr_gemv_kernel(const void *__restric
             }
         }
     }
-    // the four units of a column inside the wave (lanes l, l + 16, l + 32, l + 48), then the waves through LDS:
-    // red [MB][16 columns][NW waves]
+    // the next strip's first weights are requested before this strip's sums meet
+    const int strip_done = strip;
+    strip += gridDim.x;
+    if (strip < nstrips) {
+        rs_w = make_rsrc(pw + (size_t)strip * strip_bytes, (uint32_t)strip_bytes);
+#pragma unroll
+        for (int d = 0; d < RD; ++d) load(d, ring[d]);
+    }
+    // The four units of a column inside the wave (lanes l, l + 16, l + 32, l + 48), then the waves through
+    // LDS: red [GR strips][MB][16 columns][NW waves], two such groups in turn.  The workgroup meets once a
+    // group of GR strips (or at its last strip): a barrier a strip would stall the 2 - 7 chunks a wave
+    // has per strip; the next group writes the other half, so one barrier a group is enough.
 #pragma unroll
     for (int m = 0; m < MB; ++m) {
         float v = acc[m];
@@ -428,26 +444,31 @@ __global__ __launch_bounds__(NW * 64) void ggr_gemv_kernel(const void *__restric
         v += __shfl_xor(v, 32, 64);
         if (lane < 16) red[(m * 16 + lane) * NW + wave] = v;
     }
-    __syncthreads();
-    if (threadIdx.x < 16 * MB) {
-        const int m = threadIdx.x >> 4, c = threadIdx.x & 15;
-        if (m < M) {
-            const float4_t *r4 = (const float4_t *)(red + (m * 16 + c) * NW);
-            float tot = 0.0f;
+    const bool last = strip >= nstrips;
+    if (r == GR - 1 || last) {
+        __syncthreads();
+        if (threadIdx.x < (r + 1) * 16 * MB) {
+            const int rr = threadIdx.x / (16 * MB), m = (threadIdx.x >> 4) % MB, c = threadIdx.x & 15;
+            if (m < M) {
+                const float4_t *r4 = (const float4_t *)(red0 + (half * GR + rr) * (MB * 16 * NW) + (m * 16 + c) * NW);
+                float tot = 0.0f;
 #pragma unroll
-            for (int w = 0; w < NW / 4; ++w) {
-                const float4_t t = r4[w];
-                tot += (t[0] + t[1]) + (t[2] + t[3]);
-            }
-            const int nn = 16 * strip + c;
-            if constexpr (BF16X) {
-                if (bias) tot += BF16Traits::to_f32(((const uint16_t *)bias)[nn]);
-                ((uint16_t *)y)[(size_t)m * N + nn] = BF16Traits::from_f32(tot);
-            } else {
-                if (bias) tot += ((const float *)bias)[nn];
-                ((float *)y)[(size_t)m * N + nn] = tot;
+                for (int w = 0; w < NW / 4; ++w) {
+                    const float4_t t = r4[w];
+                    tot += (t[0] + t[1]) + (t[2] + t[3]);
+                }
+                const int nn = 16 * (strip_done - (r - rr) * (int)gridDim.x) + c;
+                if constexpr (BF16X) {
+                    if (bias) tot += BF16Traits::to_f32(((const uint16_t *)bias)[nn]);
+                    ((uint16_t *)y)[(size_t)m * N + nn] = BF16Traits::from_f32(tot);
+                } else {
+                    if (bias) tot += ((const float *)bias)[nn];
+                    ((float *)y)[(size_t)m * N + nn] = tot;
+                }
             }
         }
+    }
+    if (last) break;
     }
 }
 
@@ -480,7 +501,7 @@ static int ggr_waves(int64_t K) {
 static size_t ggr_lds_bytes(int64_t K, int mb) {
     const int nw = ggr_waves(K);
     const int64_t nmax = ceil_div(K / 128, nw);
-    return (size_t)nw * mb * (size_t)nmax * 4 * (144 + 8) + (size_t)nw * mb * 64 * 4;
+    return (size_t)nw * mb * (size_t)nmax * 4 * (144 + 8) + (size_t)2 * 4 * nw * mb * 16 * 4;
 }
 // rows of x one launch of the resident GEMV takes (more go to the kernels on the file layout)
 bool gguf_res_takes(int64_t K, int64_t M) {
@@ -557,7 +578,9 @@ int launch_gguf_res_gemv(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p) {
     const int nw = ggr_waves(p.K);
     const int nmax = (int)ceil_div(p.K / 128, nw);
     const size_t lds = ggr_lds_bytes(p.K, mb);
-    dim3 grid((unsigned)(p.N / 16));
+    const char *ge = getenv("OXQ_GGR_GRID");
+    const int64_t cap = ge ? atoi(ge) : (nw == 8 ? 512 : 256);
+    dim3 grid((unsigned)std::min<int64_t>(p.N / 16, cap > 0 ? cap : p.N / 16));
     char name[64];
     snprintf(name, sizeof name, "gguf_%s_res_gemv_%s_m%d", ggr_name(p.quant), p.act_dtype == OXQ_BF16 ? "bf16" : "f32", mb);
     set_plan(ctx, name, grid, dim3(nw * 64), 1, 1, 0);
