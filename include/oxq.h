@@ -127,11 +127,13 @@ void oxq_version(int *major, int *minor);
  * later calls run the resident-layer kernel on it, with that layer's arithmetic (few rows: unrounded
  * weights, f32 fold; above: tile GEMM on weights rounded to the activation type).  Shapes the
  * resident layout does not cover take the usual path.  The copy costs the packed tensors' size
- * again; least recently used copies go when max_bytes is reached.
+ * again; least recently used copies go when max_bytes is reached.  oxq_gguf_quant_matmul does the
+ * same for Q4_0 / Q8_0 / Q4_K / Q6_K weights at 1 - 4 rows of x, keyed by the address of the block
+ * bytes, with the strip-major copy that oxq_qlinear_new builds.
  *
  * Contract: while a triple is cached its tensors must neither change nor be freed and reused - the
- * ctx cannot see that.  Call oxq_ctx_forget_weights(ctx, qweight->data) before doing so (NULL drops
- * every copy).  Off by default (max_bytes = 0, or OXQ_WEIGHT_CACHE_MB in the environment).
+ * ctx cannot see that.  Call oxq_ctx_forget_weights(ctx, qweight->data) (for a GGUF weight: the
+ * address of its block bytes) before doing so (NULL drops every copy).  Off by default (max_bytes = 0, or OXQ_WEIGHT_CACHE_MB in the environment).
  * No counterpart in the reference, whose ops read the checkpoint layout directly. */
 int oxq_ctx_set_weight_cache(oxq_ctx *ctx, int64_t max_bytes);
 int oxq_ctx_forget_weights(oxq_ctx *ctx, const void *qweight_data);

@@ -182,7 +182,15 @@ def run(ops, ctx, stream, steps, warmup, time_graph, with_cpu=True):
         rr["bare_read_nt_us"] = r["bare_read_nt_us"]
         rows.append(rr)
         rows.append(r)
-        del d, layers
+        del layers
+        rc = _cached_row("cfg3", f"gguf {synth.GGUF_NAMES[fmt]} M=1 K={K} N={N} f32 activations, gguf_quant_matmul op "
+                                 "with the ctx weight cache on",
+                         lambda c, d=d, fmt=fmt: ops.gguf_quant_matmul(x, d[c], K, N, fmt, out=y, ctx=ctx),
+                         nc, steps, warmup, stream, time_graph, nb, 2.0 * K * N, ctx)
+        rc["bare_read_nt_us"] = r["bare_read_nt_us"]
+        rows.append(rc)
+        ctx.forget_weights(None)
+        del d
 
     # ---- config 4 --------------------------------------------------------------------------------------
     E, top_k, H, I, T = 32, 4, 2880, 2880, 8

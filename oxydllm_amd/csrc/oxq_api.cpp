@@ -690,6 +690,67 @@ static bool wcache_forward(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p, i
     return true;
 }
 
+// The same for a GGUF weight (Q4_0 / Q8_0 / Q4_K / Q6_K, 1 - 4 rows of x): the copy is the strip-major
+// one of the QLinear layers.  Entry fields: qw = the block bytes, bits = the ggml format, w.pw = the copy.
+static bool wcache_forward_gguf(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p, int *rc) {
+    if (!ctx->wcache_limit || ctx->plan_only || !gguf_res_eligible(p.quant, p.K, p.N) || !gguf_res_takes(p.K, p.M))
+        return false;
+    if (((uintptr_t)p.x & 15) || ((uintptr_t)p.w & 1)) return false;
+    if (!ctx->wcache) {
+        ctx->wcache = new (std::nothrow) oxq_weight_cache();
+        if (!ctx->wcache) return false;
+    }
+    oxq_weight_cache *c = ctx->wcache;
+    oxq_weight_cache::Entry *hit = nullptr;
+    for (auto &e : c->entries)
+        if (e.qw == p.w && e.qz == nullptr && e.sc == nullptr && e.K == p.K && e.N == p.N && e.bits == p.quant &&
+            e.pack_dim == -1) {
+            hit = &e;
+            break;
+        }
+    if (!hit) {
+        hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(s, &cs) != hipSuccess || cs != hipStreamCaptureStatusNone) {
+            (void)hipGetLastError();
+            return false;
+        }
+        const size_t bytes = (gguf_res_bytes(p.quant, p.K, p.N) + 255) & ~(size_t)255;
+        if (bytes > ctx->wcache_limit) return false;
+        while (c->bytes + bytes > ctx->wcache_limit && !c->entries.empty()) {
+            size_t lru = 0;
+            for (size_t i = 1; i < c->entries.size(); ++i)
+                if (c->entries[i].last_use < c->entries[lru].last_use) lru = i;
+            wcache_drop(ctx, lru);
+        }
+        void *mem = nullptr;
+        if (hipMalloc(&mem, bytes) != hipSuccess) {
+            (void)hipGetLastError();
+            return false;
+        }
+        oxq_weight_cache::Entry e{p.w, nullptr, nullptr, p.K, p.N, 0, 0, p.quant, -1,
+                                  Pk4Weights{(uint32_t *)mem, nullptr, p.K, p.N, 0, 0, 0, 0, 0, 0}, bytes, 0};
+        const int prc = launch_gguf_res_repack(ctx, s, p.quant, p.w, mem, p.K, p.N);
+        if (prc != OXQ_OK) {
+            (void)hipFree(mem);
+            *rc = prc;
+            return true;
+        }
+        try {
+            c->entries.push_back(e);
+        } catch (...) {
+            (void)hipFree(mem);
+            return false;
+        }
+        c->bytes += bytes;
+        hit = &c->entries.back();
+    }
+    hit->last_use = ++c->tick;
+    GgufProblem q = p;
+    q.w = (const uint8_t *)hit->w.pw;
+    *rc = launch_gguf_res_gemv(ctx, s, q);
+    return true;
+}
+
 int oxq_ctx_set_weight_cache(oxq_ctx *ctx, int64_t max_bytes) {
     if (!ctx) return fail(OXQ_ERR_ARG, "oxq_ctx_set_weight_cache: ctx is NULL");
     if (max_bytes < 0) return fail(OXQ_ERR_ARG, "oxq_ctx_set_weight_cache: max_bytes %lld is negative", (long long)max_bytes);
@@ -864,6 +925,8 @@ int oxq_gguf_quant_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x,
     GgufProblem p;
     OXQ_TRY(check_gguf(ctx, "GgufQuantMatmul", true, false, x, weight_bytes, in_features,
                        out_features, quant, out, &p));
+    int rc = OXQ_OK;
+    if (wcache_forward_gguf(ctx, (hipStream_t)stream, p, &rc)) return rc;
     if (gguf_mm_eligible(p)) return launch_gguf_mm(ctx, (hipStream_t)stream, p);
     return launch_gguf_gemv(ctx, (hipStream_t)stream, p);
 }
@@ -1998,13 +2061,7 @@ int oxq_qlinear_dequantize(oxq_qlinear *l, void *stream, const oxq_tensor *out) 
 
 void oxq_qlinear_free(oxq_qlinear *l) {
     if (!l) return;
-    if (l->res) {
-        int prev = 0;
-        (void)hipGetDevice(&prev);
-        (void)hipSetDevice(l->ctx->device);
-        (void)hipFree(l->res);
-        (void)hipSetDevice(prev);
-    }
+    if (l->res) (void)hipFree(l->res);  // by address: the layer may outlive its ctx
     delete l;
 }
 

@@ -164,6 +164,43 @@ def test_forget_evict_and_ineligible_shapes():
         ctx.close()
 
 
+@pytest.mark.parametrize("fmt", [synth.GGUF_Q4_0, synth.GGUF_Q8_0, synth.GGUF_Q4_K, synth.GGUF_Q6_K])
+def test_cached_gguf_op_equals_the_resident_layer(fmt):
+    N, K = 256, 2048
+    data = synth.gguf_weight(fmt, N, K, seed=90 + fmt)
+    wd = to_dev(data)
+    w = oracle.dequantize_gguf(fmt, data, N, K)
+    ctx = ops.Context()
+    layer = ops.QLinear(fmt, wd, K, N, None, torch.float32, ctx=ctx)
+    assert layer.resident
+    try:
+        for m in (1, 3, 6):
+            say(f"weight cache gguf {synth.GGUF_NAMES[fmt]} m={m}")
+            x = np.random.default_rng(m).standard_normal((m, K)).astype(np.float32)
+            xd = to_dev(x)
+            ctx.set_weight_cache(0)
+            ops.gguf_quant_matmul(xd, wd, K, N, fmt, ctx=ctx)
+            assert "_res_" not in ctx.last_plan()["kernel"]
+            ctx.set_weight_cache(64 << 20)
+            y1 = ops.gguf_quant_matmul(xd, wd, K, N, fmt, ctx=ctx)
+            y2 = ops.gguf_quant_matmul(xd, wd, K, N, fmt, ctx=ctx)
+            assert ("_res_gemv_" in ctx.last_plan()["kernel"]) == (m <= 4), ctx.last_plan()
+            yl = layer.forward(xd)
+            torch.cuda.synchronize()
+            if m <= 4:
+                np.testing.assert_array_equal(bits_of(y1), bits_of(yl))
+            np.testing.assert_array_equal(bits_of(y2), bits_of(y1))
+            assert_close(y1, oracle.matmul_nt_f32(x, w), f"cached gguf op m={m}")
+            nbytes, entries = ctx.weight_cache_usage()   # setting the limit to 0 above dropped the copy
+            assert (entries, nbytes >= data.nbytes) == ((1, True) if m <= 4 else (0, False))
+        ops.gguf_quant_matmul(to_dev(x[:1]), wd, K, N, fmt, ctx=ctx)
+        assert ctx.weight_cache_usage()[1] == 1
+        ctx.forget_weights(wd)
+        assert ctx.weight_cache_usage() == (0, 0)
+    finally:
+        ctx.close()
+
+
 def test_capture_allocates_nothing_and_replays_the_cached_kernel():
     K, N, g, m = 2048, 512, 128, 4
     tdt = torch.float16
