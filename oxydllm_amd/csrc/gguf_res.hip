@@ -11,18 +11,25 @@
 //                              [64 lanes][2 B] unit header (if the format has one) }
 //                       + [16 rows] block header (K-quants: the super-block's d / dmin / scales)
 //
-//   Q4_0  CH 1  16 B quants (the block's 16 bytes as stored), unit header d                    1152 B
-//   Q8_0  CH 1  32 B quants (as stored), unit header d                                         2176 B
-//   Q4_K  CH 2  16 B quants (element e in the low nibble of byte e, e + 16 in the high one),
-//               block header = the super-block's first 16 bytes (d, dmin, 12 scale bytes)      2304 B
-//   Q6_K  CH 2  16 B low nibbles (as Q4_K) + 8 B high bit pairs (element 16 h + 4 s + b in bits
-//               2s of byte b of word h), unit header = the unit's two int8 scales,
-//               block header = d                                                               3360 B
+//   Q4_0  CH 1  16 B quants, unit header d                                                     1152 B
+//   Q8_0  CH 1  32 B quants, unit header d                                                     2176 B
+//   Q4_K  CH 2  16 B quants, block header = the super-block's first 16 bytes (d, dmin, 12
+//               scale bytes)                                                                   2304 B
+//   Q6_K  CH 2  16 B low nibbles + 8 B high bit pairs, unit header = the unit's two int8
+//               scales, block header = d                                                       3360 B
 //
-// Exactly the file's bytes per weight.  A wave's load of a plane is one contiguous 1 KB run; the 8
-// waves of a workgroup split the strip's chunks, each stages only its own part of x in its own LDS
-// slot (no workgroup barrier before the arithmetic), and the partial sums meet in LDS at the end in
-// a fixed order.  The arithmetic is the staged GEMV's: raw integers converted once,
+// Exactly the file's bytes per weight.  Inside a unit the 16 elements of each half are stored ROTATED
+// by the lane's column: position n (0..15) of half h holds element 16 h + (col - n) mod 16 (4-bit
+// formats: half 0 in the low nibbles of the 16 bytes, half 1 in the high ones, byte n = position n;
+// Q8_0: byte 16 h + n; Q6_K: low nibbles likewise, the bit pair of position 16 h + 4 s + b in bits 2s
+// of byte b of word h).  That is what lets the activations stay in registers: lane col loads
+// x[16 h + col] of its unit (two 4-byte loads, 64 contiguous bytes per 16 lanes), and a rotation of
+// that register by n lanes inside the row of 16 (a DPP operand of the multiply-add, no instruction of
+// its own) hands every lane the element its position n multiplies.  No LDS, no staging, no barrier
+// before the arithmetic; the sums of x over 16 elements are four rotate-adds of the same register.
+//
+// The 16 (8) waves of a workgroup split the strip's chunks, the partial sums meet in LDS at the end
+// in a fixed order.  The arithmetic is the staged GEMV's: raw integers converted once,
 // y += a0 dot0 + a1 dot1 - b0 sum0 - b1 sum1 per unit (quant_kernels.metal:1097-1221, 1681-1838).
 #include "gguf_decode.hpp"
 
@@ -65,11 +72,28 @@ __global__ __launch_bounds__(256) void ggr_repack_kernel(const uint8_t *__restri
 
     uint32_t qw[F::QW];
     uint32_t uh = 0;
-    if constexpr (FMT == OXQ_GGUF_Q4_0 || FMT == OXQ_GGUF_Q8_0) {
-        const uint8_t *p = row + (size_t)u * GgufFmt<FMT>::BB;
+    // position n of a half holds element (col - n) mod 16 of that half
+    auto el = [&](int n) { return (col - n) & 15; };
+    if constexpr (FMT == OXQ_GGUF_Q4_0) {
+        const uint8_t *p = row + (size_t)u * 18;
         uh = ld16(p);
 #pragma unroll
-        for (int i = 0; i < F::QW; ++i) qw[i] = ld16(p + 2 + 4 * i) | (ld16(p + 4 + 4 * i) << 16);
+        for (int i = 0; i < 4; ++i) {
+            uint32_t v = 0;
+#pragma unroll
+            for (int bb = 0; bb < 4; ++bb) v |= (uint32_t)p[2 + el(4 * i + bb)] << (8 * bb);  // byte e: elements e, e + 16
+            qw[i] = v;
+        }
+    } else if constexpr (FMT == OXQ_GGUF_Q8_0) {
+        const uint8_t *p = row + (size_t)u * 34;
+        uh = ld16(p);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            uint32_t v = 0;
+#pragma unroll
+            for (int bb = 0; bb < 4; ++bb) v |= (uint32_t)p[2 + 16 * (i >> 2) + el(4 * (i & 3) + bb)] << (8 * bb);
+            qw[i] = v;
+        }
     } else if constexpr (FMT == OXQ_GGUF_Q4_K) {
         const int b = u >> 3, sb = u & 7;
         const uint8_t *p = row + (size_t)b * 144;
@@ -80,7 +104,8 @@ __global__ __launch_bounds__(256) void ggr_repack_kernel(const uint8_t *__restri
             uint32_t v = 0;
 #pragma unroll
             for (int bb = 0; bb < 4; ++bb) {
-                const uint32_t lo = ((uint32_t)qs[4 * i + bb] >> sh) & 0xFu, hi = ((uint32_t)qs[16 + 4 * i + bb] >> sh) & 0xFu;
+                const int e = el(4 * i + bb);
+                const uint32_t lo = ((uint32_t)qs[e] >> sh) & 0xFu, hi = ((uint32_t)qs[16 + e] >> sh) & 0xFu;
                 v |= (lo | (hi << 4)) << (8 * bb);
             }
             qw[i] = v;
@@ -101,7 +126,8 @@ __global__ __launch_bounds__(256) void ggr_repack_kernel(const uint8_t *__restri
             uint32_t v = 0;
 #pragma unroll
             for (int bb = 0; bb < 4; ++bb) {
-                const uint32_t lo = ((uint32_t)ql[4 * i + bb] >> shl) & 0xFu, hi = ((uint32_t)ql[16 + 4 * i + bb] >> shl) & 0xFu;
+                const int e = el(4 * i + bb);
+                const uint32_t lo = ((uint32_t)ql[e] >> shl) & 0xFu, hi = ((uint32_t)ql[16 + e] >> shl) & 0xFu;
                 v |= (lo | (hi << 4)) << (8 * bb);
             }
             qw[i] = v;
@@ -113,7 +139,7 @@ __global__ __launch_bounds__(256) void ggr_repack_kernel(const uint8_t *__restri
             for (int s = 0; s < 4; ++s)
 #pragma unroll
                 for (int bb = 0; bb < 4; ++bb)
-                    v |= (((uint32_t)qh[16 * hs + 4 * s + bb] >> shh) & 3u) << (8 * bb + 2 * s);
+                    v |= (((uint32_t)qh[16 * hs + el(4 * s + bb)] >> shh) & 3u) << (8 * bb + 2 * s);
             qw[4 + hs] = v;
         }
         uh = (uint32_t)p[192 + 2 * sub] | ((uint32_t)p[192 + 2 * sub + 1] << 8);
@@ -249,26 +275,68 @@ __global__ __launch_bounds__(256) void ggr_dequant_kernel(const uint8_t *__restr
             wf[e + 16] = s1 * (float)((int)((byte >> 4) | (h1 << 4)) - 32);
         }
     }
+    // wf is in stored order: position n of half h is element (col - n) mod 16 of that half
     float *o = out + (size_t)(16 * strip + col) * K + (size_t)(4 * c + kq) * 32;
 #pragma unroll
-    for (int i = 0; i < 32; ++i) o[i] = wf[i];
+    for (int i = 0; i < 32; ++i) o[(i & 16) + ((col - i) & 15)] = wf[i];
 }
 
 // ---------------------------------------------------------------------------
-// Decode GEMV on the copy.  grid.x = strips, 8 waves; wave w takes a contiguous run of the strip's
-// chunks, stages its own part of the MB activation rows in its own LDS slot (as f32, unit by unit
-// with one 16-byte pad a unit, then the sums of x over every 16 elements) and walks its chunks with
-// RD chunks of weights in flight.
+// Decode GEMV on the copy.  grid.x = workgroups that walk the strips; wave w takes a contiguous run
+// of a strip's chunks with RD chunks (weights, headers and its lanes' two activations per row) in
+// flight.  Nothing goes through LDS but the partial sums at the end.
 // ---------------------------------------------------------------------------
+// value of lane (l - n) mod 16 of the caller's row of 16 lanes (DPP row_ror: the compiler folds the
+// move into the multiply-add that uses it)
+template <int NROT>
+__device__ __forceinline__ float row_ror(float v) {
+    if constexpr (NROT == 0) return v;
+    else return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x120 + NROT, 0xF, 0xF, true));
+}
+// dot += sum over n of q[n] * (xv of lane (l - n) mod 16).  Written out as v_fmac_f32 with a DPP source
+// (the compiler keeps the rotation as a move of its own in front of every multiply-add otherwise).  A
+// DPP source written by a vector instruction less than two wait states earlier reads stale data on this
+// target, and the hazard pass does not look inside an asm block: hence the leading s_nop.
+__device__ __forceinline__ void ggr_dot16(const float *q, float xv, float &dot) {
+    asm("s_nop 1\n\t"
+        "v_fmac_f32_e32 %0, %1, %2\n\t"
+        "v_fmac_f32_dpp %0, %1, %3 row_ror:1 row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "v_fmac_f32_dpp %0, %1, %4 row_ror:2 row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "v_fmac_f32_dpp %0, %1, %5 row_ror:3 row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "v_fmac_f32_dpp %0, %1, %6 row_ror:4 row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "v_fmac_f32_dpp %0, %1, %7 row_ror:5 row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "v_fmac_f32_dpp %0, %1, %8 row_ror:6 row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "v_fmac_f32_dpp %0, %1, %9 row_ror:7 row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "v_fmac_f32_dpp %0, %1, %10 row_ror:8 row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "v_fmac_f32_dpp %0, %1, %11 row_ror:9 row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "v_fmac_f32_dpp %0, %1, %12 row_ror:10 row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "v_fmac_f32_dpp %0, %1, %13 row_ror:11 row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "v_fmac_f32_dpp %0, %1, %14 row_ror:12 row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "v_fmac_f32_dpp %0, %1, %15 row_ror:13 row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "v_fmac_f32_dpp %0, %1, %16 row_ror:14 row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "v_fmac_f32_dpp %0, %1, %17 row_ror:15 row_mask:0xf bank_mask:0xf bound_ctrl:1"
+        : "+v"(dot)
+        : "v"(xv), "v"(q[0]), "v"(q[1]), "v"(q[2]), "v"(q[3]), "v"(q[4]), "v"(q[5]), "v"(q[6]), "v"(q[7]), "v"(q[8]),
+          "v"(q[9]), "v"(q[10]), "v"(q[11]), "v"(q[12]), "v"(q[13]), "v"(q[14]), "v"(q[15]));
+}
+// sum of the 16 lanes of a row, in every lane
+__device__ __forceinline__ float row_sum16(float v) {
+    v += row_ror<8>(v);
+    v += row_ror<4>(v);
+    v += row_ror<2>(v);
+    v += row_ror<1>(v);
+    return v;
+}
+
 template <int FMT, bool BF16X, int MB, int NW>
 __global__ __launch_bounds__(NW * 64) void ggr_gemv_kernel(const void *__restrict__ x, const uint8_t *__restrict__ pw,
                                                        const void *__restrict__ bias, void *__restrict__ y, int M,
-                                                       int K, int N, int nmax) {
+                                                       int K, int N) {
     typedef GgrFmt<FMT> F;
     typedef GgrLayout<FMT> L;
     constexpr int RD = NW == 8 ? 4 : 2, OOB = 0x7FFFFF00;
     constexpr int GR = 4;                                      // strips between two meetings of the workgroup
-    constexpr int XP = 144;                                    // bytes of a unit's 32 floats + one pad chunk
+    constexpr int XB = BF16X ? 2 : 4;
     extern __shared__ __attribute__((aligned(16))) unsigned char gr_lds[];
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int col = lane & 15, kq = lane >> 4;
@@ -278,21 +346,40 @@ __global__ __launch_bounds__(NW * 64) void ggr_gemv_kernel(const void *__restric
     const int cbase = nch / NW, crem = nch % NW;
     const int n = cbase + (wave < crem ? 1 : 0);               // this wave's chunks: [c0, c0 + n)
     const int c0 = wave * cbase + min(wave, crem);
-    const size_t xrow = (size_t)nmax * 4 * (XP + 8);           // a row's units, then two sums a unit (multiple of 16)
-    unsigned char *slot = gr_lds + (size_t)wave * MB * xrow;
-    float *red0 = (float *)(gr_lds + (size_t)NW * MB * xrow);  // 2 x GR x [MB][16][NW] partial sums
+    float *red0 = (float *)gr_lds;                             // 2 x GR x [MB][16][NW] partial sums
 
     const size_t strip_bytes = (size_t)(nch / F::CH) * L::BLKB;
     __amdgpu_buffer_rsrc_t rs_w = make_rsrc(pw + (size_t)strip * strip_bytes, (uint32_t)strip_bytes);
+    const __amdgpu_buffer_rsrc_t rs_x = make_rsrc(x, (uint32_t)M * (uint32_t)K * (uint32_t)XB);
     const __amdgpu_buffer_rsrc_t rs_none = make_rsrc(pw, 0u);
+    // lane (col, kq) holds x[16 h + col] of unit kq of a chunk, h = 0, 1; rows past M read nothing
+    int voff_x[MB];
+#pragma unroll
+    for (int m = 0; m < MB; ++m) voff_x[m] = m < M ? (m * K + kq * 32 + col) * XB : OOB;
 
     struct Stage {
         uint32_t qw[F::QW];
         uint32_t uh;
         uint32_t bh[4];
+        float xr[MB][2];
     };
     Stage ring[RD];
-    auto load = [&](int i, Stage &st) {  // chunk i of the wave; past its share through an empty descriptor
+    auto load_x = [&](int i, Stage &st) {
+        const __amdgpu_buffer_rsrc_t rs = i < n ? rs_x : rs_none;
+        const int soff = (c0 + i) * 128 * XB;
+#pragma unroll
+        for (int m = 0; m < MB; ++m)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                if constexpr (BF16X) {
+                    const uint32_t v = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(rs, voff_x[m] + h * 16 * XB, soff, 0);
+                    st.xr[m][h] = __builtin_bit_cast(float, v << 16);
+                } else {
+                    st.xr[m][h] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs, voff_x[m] + h * 16 * XB, soff, 0));
+                }
+            }
+    };
+    auto load_w = [&](int i, Stage &st) {  // chunk i of the wave; past its share through an empty descriptor
         const __amdgpu_buffer_rsrc_t rs = i < n ? rs_w : rs_none;
         const int c = c0 + i;
         const int boff = (c / F::CH) * L::BLKB, coff = boff + (c % F::CH) * L::CHB;
@@ -316,159 +403,87 @@ __global__ __launch_bounds__(NW * 64) void ggr_gemv_kernel(const void *__restric
             st.bh[0] = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(rs, col * 2, boff + L::BH_OFF, 0);
         }
     };
-    // this wave's part of x: elements [128 c0, 128 (c0 + n)) of every row, staged as f32 in 16-byte
-    // pieces of the source; with them the sums of x over every 16 elements, from the registers that
-    // carry x: the piece's own elements, then the 4 (bf16: 2) pieces of a half unit, which
-    // neighbouring lanes hold.  The first batch of row 0 is requested before the first weights (both are
-    // needed to start; x is the smaller), its stores come after the weights' requests.
-    constexpr int XB = BF16X ? 2 : 4, EPP = 16 / XB;       // elements a 16-byte piece of x
-    const int pieces = n * 128 / EPP;
-    const __amdgpu_buffer_rsrc_t rs_x = make_rsrc(x, (uint32_t)M * (uint32_t)K * (uint32_t)XB);
-    auto x_load = [&](int m, int base, u32x4_t (&v)[4]) {
-        const int rowoff = m < M ? m * K * XB + c0 * 128 * XB : OOB;
 #pragma unroll
-        for (int b = 0; b < 4; ++b) {
-            const int p = base + b * 64 + lane;
-            v[b] = __builtin_amdgcn_raw_buffer_load_b128(rs_x, p < pieces ? rowoff + p * 16 : OOB, 0, 0);
-        }
-    };
-    auto x_store = [&](int m, int base, const u32x4_t (&v)[4]) {
-        unsigned char *xr = slot + m * xrow;
-#pragma unroll
-        for (int b = 0; b < 4; ++b) {
-            const int p = base + b * 64 + lane;
-            float sx;
-            if constexpr (BF16X) {
-                sx = 0.0f;
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    sx += __builtin_bit_cast(float, (uint32_t)v[b][j] << 16) +
-                          __builtin_bit_cast(float, (uint32_t)v[b][j] & 0xFFFF0000u);
-                sx += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, sx), 0xB1, 0xF, 0xF, false));
-            } else {
-                sx = (__builtin_bit_cast(float, (uint32_t)v[b][0]) + __builtin_bit_cast(float, (uint32_t)v[b][1])) +
-                     (__builtin_bit_cast(float, (uint32_t)v[b][2]) + __builtin_bit_cast(float, (uint32_t)v[b][3]));
-                sx += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, sx), 0xB1, 0xF, 0xF, false));
-                sx += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, sx), 0x4E, 0xF, 0xF, false));
-            }
-            if (p < pieces) {
-                constexpr int PPH = BF16X ? 2 : 4;  // pieces a half unit
-                if ((p & (PPH - 1)) == 0) ((float *)(xr + (size_t)nmax * 4 * XP))[p / PPH] = sx;
-                if constexpr (BF16X) {
-                    const int u = p >> 2, cc = (p & 3) * 2;
-                    float4_t lo, hi;
-#pragma unroll
-                    for (int j = 0; j < 2; ++j) {
-                        lo[2 * j] = __builtin_bit_cast(float, (uint32_t)v[b][j] << 16);
-                        lo[2 * j + 1] = __builtin_bit_cast(float, (uint32_t)v[b][j] & 0xFFFF0000u);
-                        hi[2 * j] = __builtin_bit_cast(float, (uint32_t)v[b][2 + j] << 16);
-                        hi[2 * j + 1] = __builtin_bit_cast(float, (uint32_t)v[b][2 + j] & 0xFFFF0000u);
-                    }
-                    *(float4_t *)(xr + u * XP + cc * 16) = lo;
-                    *(float4_t *)(xr + u * XP + cc * 16 + 16) = hi;
-                } else {
-                    *(u32x4_t *)(xr + (p >> 3) * XP + (p & 7) * 16) = v[b];
-                }
-            }
-        }
-    };
-    {
-        u32x4_t v0[4];
-        x_load(0, 0, v0);
-#pragma unroll
-        for (int d = 0; d < RD; ++d) load(d, ring[d]);
-        x_store(0, 0, v0);
-#pragma unroll
-        for (int m = 0; m < MB; ++m)
-            for (int base = m ? 0 : 256; base < pieces; base += 256) {
-                u32x4_t v[4];
-                x_load(m, base, v);
-                x_store(m, base, v);
-            }
+    for (int d = 0; d < RD; ++d) {
+        load_x(d, ring[d]);
+        load_w(d, ring[d]);
     }
 
-    // a workgroup walks the strips blockIdx.x, + gridDim.x, ...: x is staged once
+    // a workgroup walks the strips blockIdx.x, + gridDim.x, ...
     for (int it = 0;; ++it) {
-    const int r = it % GR, half = (it / GR) & 1;
-    float *red = red0 + (half * GR + r) * (MB * 16 * NW);
-    float acc[MB];
+        const int r = it % GR, half = (it / GR) & 1;
+        float *red = red0 + (half * GR + r) * (MB * 16 * NW);
+        float acc[MB];
 #pragma unroll
-    for (int m = 0; m < MB; ++m) acc[m] = 0.0f;
-    const int nround = (n + RD - 1) / RD * RD;
-    for (int i0 = 0; i0 < nround; i0 += RD) {
+        for (int m = 0; m < MB; ++m) acc[m] = 0.0f;
+        const int nround = (n + RD - 1) / RD * RD;
+        const int strip_done = strip;
+        strip += gridDim.x;
+        const bool last = strip >= nstrips;
+        for (int i0 = 0; i0 < nround; i0 += RD) {
 #pragma unroll
-        for (int d = 0; d < RD; ++d) {
-            const int i = i0 + d;
-            const Stage st = ring[d];
-            load(i + RD, ring[d]);
-            float q[32], a0, a1, b0, b1;
-            ggr_ints<FMT>(st.qw, q);
-            ggr_factors<FMT>(st.uh, st.bh, 4 * ((c0 + i) % F::CH) + kq, a0, a1, b0, b1);
-            // chunks past the share hold zeros (a = b = 0); their x comes from the share's last chunk
-            const int uw = 4 * min(i, n - 1) + kq;
+            for (int d = 0; d < RD; ++d) {
+                const int i = i0 + d;
+                const Stage st = ring[d];
+                // the ring runs on into the next strip (same chunks of x, the next strip's weights)
+                if (i + RD < nround) {
+                    load_x(i + RD, ring[d]);
+                    load_w(i + RD, ring[d]);
+                } else if (!last) {
+                    if (d == 0 && i + RD == nround)
+                        rs_w = make_rsrc(pw + (size_t)strip * strip_bytes, (uint32_t)strip_bytes);
+                    load_x(i + RD - nround, ring[d]);
+                    load_w(i + RD - nround, ring[d]);
+                }
+                float q[32], a0, a1, b0, b1;
+                ggr_ints<FMT>(st.qw, q);
+                ggr_factors<FMT>(st.uh, st.bh, 4 * ((c0 + i) % F::CH) + kq, a0, a1, b0, b1);
+                // chunks past the share hold zeros (weights, headers and x alike)
 #pragma unroll
-            for (int m = 0; m < MB; ++m) {
-                const unsigned char *xr = slot + m * xrow;
-                const float4_t *xu = (const float4_t *)(xr + uw * XP);
-                const float2 sx = *(const float2 *)(xr + (size_t)nmax * 4 * XP + uw * 8);
-                float dot0 = 0.0f, dot1 = 0.0f;
+                for (int m = 0; m < MB; ++m) {
+                    float dot0 = 0.0f, dot1 = 0.0f;
+                    ggr_dot16(q, st.xr[m][0], dot0);
+                    ggr_dot16(q + 16, st.xr[m][1], dot1);
+                    const float sx0 = row_sum16(st.xr[m][0]), sx1 = row_sum16(st.xr[m][1]);
+                    acc[m] += (a0 * dot0 + a1 * dot1) - (b0 * sx0 + b1 * sx1);
+                }
+            }
+        }
+        // The four units of a column inside the wave (lanes l, l + 16, l + 32, l + 48), then the waves
+        // through LDS: red [GR strips][MB][16 columns][NW waves], two such groups in turn.  The workgroup
+        // meets once a group of GR strips (or at its last strip); the next group writes the other half, so
+        // one barrier a group is enough.
 #pragma unroll
-                for (int o = 0; o < 8; ++o) {
-                    const float4_t xv = xu[o];
+        for (int m = 0; m < MB; ++m) {
+            float v = acc[m];
+            v += __shfl_xor(v, 16, 64);
+            v += __shfl_xor(v, 32, 64);
+            if (lane < 16) red[(m * 16 + lane) * NW + wave] = v;
+        }
+        if (r == GR - 1 || last) {
+            __syncthreads();
+            if (threadIdx.x < (r + 1) * 16 * MB) {
+                const int rr = threadIdx.x / (16 * MB), m = (threadIdx.x >> 4) % MB, c = threadIdx.x & 15;
+                if (m < M) {
+                    const float4_t *r4 = (const float4_t *)(red0 + (half * GR + rr) * (MB * 16 * NW) + (m * 16 + c) * NW);
+                    float tot = 0.0f;
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        if (o < 4) dot0 = fmaf(q[4 * o + e], xv[e], dot0);
-                        else dot1 = fmaf(q[4 * o + e], xv[e], dot1);
+                    for (int w = 0; w < NW / 4; ++w) {
+                        const float4_t t = r4[w];
+                        tot += (t[0] + t[1]) + (t[2] + t[3]);
+                    }
+                    const int nn = 16 * (strip_done - (r - rr) * (int)gridDim.x) + c;
+                    if constexpr (BF16X) {
+                        if (bias) tot += BF16Traits::to_f32(((const uint16_t *)bias)[nn]);
+                        ((uint16_t *)y)[(size_t)m * N + nn] = BF16Traits::from_f32(tot);
+                    } else {
+                        if (bias) tot += ((const float *)bias)[nn];
+                        ((float *)y)[(size_t)m * N + nn] = tot;
                     }
                 }
-                acc[m] += (a0 * dot0 + a1 * dot1) - (b0 * sx.x + b1 * sx.y);
             }
         }
-    }
-    // the next strip's first weights are requested before this strip's sums meet
-    const int strip_done = strip;
-    strip += gridDim.x;
-    if (strip < nstrips) {
-        rs_w = make_rsrc(pw + (size_t)strip * strip_bytes, (uint32_t)strip_bytes);
-#pragma unroll
-        for (int d = 0; d < RD; ++d) load(d, ring[d]);
-    }
-    // The four units of a column inside the wave (lanes l, l + 16, l + 32, l + 48), then the waves through
-    // LDS: red [GR strips][MB][16 columns][NW waves], two such groups in turn.  The workgroup meets once a
-    // group of GR strips (or at its last strip): a barrier a strip would stall the 2 - 7 chunks a wave
-    // has per strip; the next group writes the other half, so one barrier a group is enough.
-#pragma unroll
-    for (int m = 0; m < MB; ++m) {
-        float v = acc[m];
-        v += __shfl_xor(v, 16, 64);
-        v += __shfl_xor(v, 32, 64);
-        if (lane < 16) red[(m * 16 + lane) * NW + wave] = v;
-    }
-    const bool last = strip >= nstrips;
-    if (r == GR - 1 || last) {
-        __syncthreads();
-        if (threadIdx.x < (r + 1) * 16 * MB) {
-            const int rr = threadIdx.x / (16 * MB), m = (threadIdx.x >> 4) % MB, c = threadIdx.x & 15;
-            if (m < M) {
-                const float4_t *r4 = (const float4_t *)(red0 + (half * GR + rr) * (MB * 16 * NW) + (m * 16 + c) * NW);
-                float tot = 0.0f;
-#pragma unroll
-                for (int w = 0; w < NW / 4; ++w) {
-                    const float4_t t = r4[w];
-                    tot += (t[0] + t[1]) + (t[2] + t[3]);
-                }
-                const int nn = 16 * (strip_done - (r - rr) * (int)gridDim.x) + c;
-                if constexpr (BF16X) {
-                    if (bias) tot += BF16Traits::to_f32(((const uint16_t *)bias)[nn]);
-                    ((uint16_t *)y)[(size_t)m * N + nn] = BF16Traits::from_f32(tot);
-                } else {
-                    if (bias) tot += ((const float *)bias)[nn];
-                    ((float *)y)[(size_t)m * N + nn] = tot;
-                }
-            }
-        }
-    }
-    if (last) break;
+        if (last) break;
     }
 }
 
@@ -498,16 +513,11 @@ static int ggr_waves(int64_t K) {
     const int w = e ? atoi(e) : 16;
     return (w == 8 || K / 128 < 16) ? 8 : 16;
 }
-static size_t ggr_lds_bytes(int64_t K, int mb) {
-    const int nw = ggr_waves(K);
-    const int64_t nmax = ceil_div(K / 128, nw);
-    return (size_t)nw * mb * (size_t)nmax * 4 * (144 + 8) + (size_t)2 * 4 * nw * mb * 16 * 4;
-}
+static size_t ggr_lds_bytes(int64_t K, int mb) { return (size_t)2 * 4 * ggr_waves(K) * mb * 16 * 4; }
 // rows of x one launch of the resident GEMV takes (more go to the kernels on the file layout)
-bool gguf_res_takes(int64_t K, int64_t M) {
-    if (M < 1 || M > 4) return false;
-    return ggr_lds_bytes(K, M <= 1 ? 1 : M <= 2 ? 2 : 4) <= 144 * 1024;
-}
+// (8 rows in one pass need more registers than a wave of a 16-wave workgroup has: measured 14.8 us on
+// 4096 x 4096 Q4_0 against 6.3 us at 4 rows)
+bool gguf_res_takes(int64_t, int64_t M) { return M >= 1 && M <= 4; }
 
 static const char *ggr_name(int q) {
     return q == OXQ_GGUF_Q4_0 ? "q4_0" : q == OXQ_GGUF_Q8_0 ? "q8_0" : q == OXQ_GGUF_Q4_K ? "q4k" : "q6k";
@@ -556,27 +566,26 @@ int launch_gguf_res_dequant(oxq_ctx *ctx, hipStream_t s, int quant, const void *
 }
 
 template <int FMT, bool BF16X, int MB, int NW>
-static int ggr_go(hipStream_t s, dim3 grid, const GgufProblem &p, size_t lds, int nmax) {
+static int ggr_go(hipStream_t s, dim3 grid, const GgufProblem &p, size_t lds) {
     static LdsGrant lds_grant;  // one per instantiation
     OXQ_HIP_CHECK(lds_grant.ensure((const void *)ggr_gemv_kernel<FMT, BF16X, MB, NW>, lds));
     hipLaunchKernelGGL((ggr_gemv_kernel<FMT, BF16X, MB, NW>), grid, dim3(NW * 64), lds, s, p.x, p.w, p.bias, p.y,
-                       (int)p.M, (int)p.K, (int)p.N, nmax);
+                       (int)p.M, (int)p.K, (int)p.N);
     OXQ_HIP_CHECK(hipGetLastError());
     return OXQ_OK;
 }
 template <int FMT, int NW>
-static int ggr_by_rows(hipStream_t s, dim3 grid, const GgufProblem &p, size_t lds, int nmax, int mb) {
+static int ggr_by_rows(hipStream_t s, dim3 grid, const GgufProblem &p, size_t lds, int mb) {
     const bool bf = p.act_dtype == OXQ_BF16;
-    if (mb == 1) return bf ? ggr_go<FMT, true, 1, NW>(s, grid, p, lds, nmax) : ggr_go<FMT, false, 1, NW>(s, grid, p, lds, nmax);
-    if (mb == 2) return bf ? ggr_go<FMT, true, 2, NW>(s, grid, p, lds, nmax) : ggr_go<FMT, false, 2, NW>(s, grid, p, lds, nmax);
-    return bf ? ggr_go<FMT, true, 4, NW>(s, grid, p, lds, nmax) : ggr_go<FMT, false, 4, NW>(s, grid, p, lds, nmax);
+    if (mb == 1) return bf ? ggr_go<FMT, true, 1, NW>(s, grid, p, lds) : ggr_go<FMT, false, 1, NW>(s, grid, p, lds);
+    if (mb == 2) return bf ? ggr_go<FMT, true, 2, NW>(s, grid, p, lds) : ggr_go<FMT, false, 2, NW>(s, grid, p, lds);
+    return bf ? ggr_go<FMT, true, 4, NW>(s, grid, p, lds) : ggr_go<FMT, false, 4, NW>(s, grid, p, lds);
 }
 
 // p.w is the resident copy
 int launch_gguf_res_gemv(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p) {
     const int mb = p.M <= 1 ? 1 : p.M <= 2 ? 2 : 4;
     const int nw = ggr_waves(p.K);
-    const int nmax = (int)ceil_div(p.K / 128, nw);
     const size_t lds = ggr_lds_bytes(p.K, mb);
     const char *ge = getenv("OXQ_GGR_GRID");
     const int64_t cap = ge ? atoi(ge) : (nw == 8 ? 512 : 256);
@@ -586,13 +595,13 @@ int launch_gguf_res_gemv(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p) {
     set_plan(ctx, name, grid, dim3(nw * 64), 1, 1, 0);
     if (ctx->plan_only) return OXQ_OK;
     if (!gguf_res_takes(p.K, p.M)) return fail(OXQ_ERR_UNSUPPORTED, "gguf resident gemv: m = %lld", (long long)p.M);
-    if ((uintptr_t)p.x & 15) return fail(OXQ_ERR_UNSUPPORTED, "gguf resident gemv: x must be 16-byte aligned");
+    if ((uintptr_t)p.x & 3) return fail(OXQ_ERR_UNSUPPORTED, "gguf resident gemv: x must be 4-byte aligned");
     if ((uint64_t)p.M * (uint64_t)p.K * 4 >= (1ull << 31)) return fail(OXQ_ERR_UNSUPPORTED, "gguf resident gemv: x larger than 2 GiB");
     switch (p.quant) {
-    case OXQ_GGUF_Q4_0: return nw == 8 ? ggr_by_rows<OXQ_GGUF_Q4_0, 8>(s, grid, p, lds, nmax, mb) : ggr_by_rows<OXQ_GGUF_Q4_0, 16>(s, grid, p, lds, nmax, mb);
-    case OXQ_GGUF_Q8_0: return nw == 8 ? ggr_by_rows<OXQ_GGUF_Q8_0, 8>(s, grid, p, lds, nmax, mb) : ggr_by_rows<OXQ_GGUF_Q8_0, 16>(s, grid, p, lds, nmax, mb);
-    case OXQ_GGUF_Q4_K: return nw == 8 ? ggr_by_rows<OXQ_GGUF_Q4_K, 8>(s, grid, p, lds, nmax, mb) : ggr_by_rows<OXQ_GGUF_Q4_K, 16>(s, grid, p, lds, nmax, mb);
-    case OXQ_GGUF_Q6_K: return nw == 8 ? ggr_by_rows<OXQ_GGUF_Q6_K, 8>(s, grid, p, lds, nmax, mb) : ggr_by_rows<OXQ_GGUF_Q6_K, 16>(s, grid, p, lds, nmax, mb);
+    case OXQ_GGUF_Q4_0: return nw == 8 ? ggr_by_rows<OXQ_GGUF_Q4_0, 8>(s, grid, p, lds, mb) : ggr_by_rows<OXQ_GGUF_Q4_0, 16>(s, grid, p, lds, mb);
+    case OXQ_GGUF_Q8_0: return nw == 8 ? ggr_by_rows<OXQ_GGUF_Q8_0, 8>(s, grid, p, lds, mb) : ggr_by_rows<OXQ_GGUF_Q8_0, 16>(s, grid, p, lds, mb);
+    case OXQ_GGUF_Q4_K: return nw == 8 ? ggr_by_rows<OXQ_GGUF_Q4_K, 8>(s, grid, p, lds, mb) : ggr_by_rows<OXQ_GGUF_Q4_K, 16>(s, grid, p, lds, mb);
+    case OXQ_GGUF_Q6_K: return nw == 8 ? ggr_by_rows<OXQ_GGUF_Q6_K, 8>(s, grid, p, lds, mb) : ggr_by_rows<OXQ_GGUF_Q6_K, 16>(s, grid, p, lds, mb);
     default: return fail(OXQ_ERR_UNSUPPORTED, "gguf resident gemv: format %d", p.quant);
     }
 }
