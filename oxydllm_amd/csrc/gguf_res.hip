@@ -424,7 +424,13 @@ __global__ __launch_bounds__(NW * 64) void ggr_gemv_kernel(const void *__restric
 #pragma unroll
             for (int d = 0; d < RD; ++d) {
                 const int i = i0 + d;
-                const Stage st = ring[d];
+                // The stage is unpacked before its slot is requested again: converting first delays the
+                // request by a few dozen instructions and saves a register copy of the whole stage.
+                float q[32], a0, a1, b0, b1, xr[MB][2];
+                ggr_ints<FMT>(ring[d].qw, q);
+                ggr_factors<FMT>(ring[d].uh, ring[d].bh, 4 * ((c0 + i) % F::CH) + kq, a0, a1, b0, b1);
+#pragma unroll
+                for (int m = 0; m < MB; ++m) xr[m][0] = ring[d].xr[m][0], xr[m][1] = ring[d].xr[m][1];
                 // the ring runs on into the next strip (same chunks of x, the next strip's weights)
                 if (i + RD < nround) {
                     load_x(i + RD, ring[d]);
@@ -435,17 +441,21 @@ __global__ __launch_bounds__(NW * 64) void ggr_gemv_kernel(const void *__restric
                     load_x(i + RD - nround, ring[d]);
                     load_w(i + RD - nround, ring[d]);
                 }
-                float q[32], a0, a1, b0, b1;
-                ggr_ints<FMT>(st.qw, q);
-                ggr_factors<FMT>(st.uh, st.bh, 4 * ((c0 + i) % F::CH) + kq, a0, a1, b0, b1);
                 // chunks past the share hold zeros (weights, headers and x alike)
 #pragma unroll
                 for (int m = 0; m < MB; ++m) {
-                    float dot0 = 0.0f, dot1 = 0.0f;
-                    ggr_dot16(q, st.xr[m][0], dot0);
-                    ggr_dot16(q + 16, st.xr[m][1], dot1);
-                    const float sx0 = row_sum16(st.xr[m][0]), sx1 = row_sum16(st.xr[m][1]);
-                    acc[m] += (a0 * dot0 + a1 * dot1) - (b0 * sx0 + b1 * sx1);
+                    if constexpr (FMT == OXQ_GGUF_Q6_K) {  // a scale per half unit
+                        float dot0 = 0.0f, dot1 = 0.0f;
+                        ggr_dot16(q, xr[m][0], dot0);
+                        ggr_dot16(q + 16, xr[m][1], dot1);
+                        const float sx0 = row_sum16(xr[m][0]), sx1 = row_sum16(xr[m][1]);
+                        acc[m] += (a0 * dot0 + a1 * dot1) - (b0 * sx0 + b1 * sx1);
+                    } else {                               // one scale a unit: one chain, one sum
+                        float dot = 0.0f;
+                        ggr_dot16(q, xr[m][0], dot);
+                        ggr_dot16(q + 16, xr[m][1], dot);
+                        acc[m] += a0 * dot - b0 * row_sum16(xr[m][0] + xr[m][1]);
+                    }
                 }
             }
         }
