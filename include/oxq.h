@@ -144,7 +144,7 @@ int oxq_gguf_block_layout(int quant, int64_t *block_elems, int64_t *block_bytes)
 
 /* ---- measurement aid ---------------------------------------------------------
  * No counterpart in the reference.  A plain streaming read of `src` (U8, contiguous, 16-byte
- * aligned; its size a multiple of workgroups * 64 KiB) by `workgroups` workgroups of 512 threads,
+ * aligned; its size a multiple of workgroups * 8 KiB) by `workgroups` workgroups of 512 threads,
  * each reading one contiguous span with 16-byte loads, eight in flight per lane - the launch shape of
  * the resident-layer GEMV with the arithmetic taken out.  `checksums` (U32 [>= workgroups]) receives
  * an xor of every span, which keeps the loads alive and lets a test check the read.  bench.py times

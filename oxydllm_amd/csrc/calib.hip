@@ -11,14 +11,16 @@ namespace oxq {
 template <int POLICY>
 __global__ __launch_bounds__(512) void calib_read_kernel(const uint8_t *__restrict__ src, uint32_t *__restrict__ out,
                                                          uint32_t span) {
-    // span: bytes per workgroup, a multiple of 64 KiB (8 loads x 512 lanes x 16 bytes)
+    // span: bytes per workgroup, a multiple of 8 KiB (512 lanes x 16 bytes); up to 8 loads a lane in flight
+    // (loads past the span get an offset beyond the descriptor: no memory access)
     const __amdgpu_buffer_rsrc_t rs = make_rsrc(src + (size_t)blockIdx.x * span, span);
     const int voff = threadIdx.x * 16;
     u32x4_t acc = {0u, 0u, 0u, 0u};
     for (uint32_t base = 0; base < span; base += 65536u) {
         u32x4_t v[8];
 #pragma unroll
-        for (int q = 0; q < 8; ++q) v[q] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff, (int)(base + q * 8192u), POLICY);
+        for (int q = 0; q < 8; ++q)
+            v[q] = __builtin_amdgcn_raw_buffer_load_b128(rs, base + q * 8192u < span ? voff : 0x7FFFFF00, (int)(base + q * 8192u), POLICY);
 #pragma unroll
         for (int q = 0; q < 8; ++q) acc ^= v[q];
     }

@@ -567,10 +567,10 @@ int oxq_calib_read(oxq_ctx *ctx, void *stream, const oxq_tensor *src, int workgr
     if (workgroups < 1 || workgroups > 65535 || numel(checksums) < workgroups)
         return fail(OXQ_ERR_SHAPE, "CalibRead: %d workgroups need 1..65535 and one checksum word each (got %lld)",
                     workgroups, (long long)numel(checksums));
-    if (bytes <= 0 || bytes % ((int64_t)workgroups * 65536) != 0 || bytes / workgroups >= (int64_t(1) << 31))
+    if (bytes <= 0 || bytes % ((int64_t)workgroups * 8192) != 0 || bytes / workgroups >= (int64_t(1) << 31))
         return fail(OXQ_ERR_SHAPE,
                     "CalibRead: %lld bytes over %d workgroups: every workgroup reads a span that is a multiple "
-                    "of 64 KiB and below 2 GiB", (long long)bytes, workgroups);
+                    "of 8 KiB and below 2 GiB", (long long)bytes, workgroups);
     if (!ctx->plan_only && ((uintptr_t)src->data & 15))
         return fail(OXQ_ERR_UNSUPPORTED, "CalibRead: src must be 16-byte aligned");
     return launch_calib_read(ctx, (hipStream_t)stream, (const uint8_t *)src->data, (uint64_t)bytes, workgroups,
