@@ -527,7 +527,9 @@ static size_t ggr_lds_bytes(int64_t K, int mb) { return (size_t)2 * 4 * ggr_wave
 // rows of x one launch of the resident GEMV takes (more go to the kernels on the file layout)
 // (8 rows in one pass need more registers than a wave of a 16-wave workgroup has: measured 14.8 us on
 // 4096 x 4096 Q4_0 against 6.3 us at 4 rows)
-bool gguf_res_takes(int64_t, int64_t M) { return M >= 1 && M <= 4; }
+// f32 activations at 5 - 8 rows take two passes of four: the file layout has no staged kernel for them
+// (4096 x 4096: 31 us), while bf16 rows go to the tile matmul there, which two passes only equal.
+bool gguf_res_takes(int64_t, int64_t M, int act_dtype) { return M >= 1 && (M <= 4 || (M <= 8 && act_dtype == OXQ_F32)); }
 
 static const char *ggr_name(int q) {
     return q == OXQ_GGUF_Q4_0 ? "q4_0" : q == OXQ_GGUF_Q8_0 ? "q8_0" : q == OXQ_GGUF_Q4_K ? "q4k" : "q6k";
@@ -593,27 +595,38 @@ static int ggr_by_rows(hipStream_t s, dim3 grid, const GgufProblem &p, size_t ld
 }
 
 // p.w is the resident copy
-int launch_gguf_res_gemv(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p) {
-    const int mb = p.M <= 1 ? 1 : p.M <= 2 ? 2 : 4;
-    const int nw = ggr_waves(p.K);
-    const size_t lds = ggr_lds_bytes(p.K, mb);
+int launch_gguf_res_gemv(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p0) {
+    const int64_t rows0 = std::min<int64_t>(p0.M, 4);
+    const int mb = rows0 <= 1 ? 1 : rows0 <= 2 ? 2 : 4;
+    const int nw = ggr_waves(p0.K);
+    const size_t lds = ggr_lds_bytes(p0.K, mb);
     const char *ge = getenv("OXQ_GGR_GRID");
     const int64_t cap = ge ? atoi(ge) : (nw == 8 ? 512 : 256);
-    dim3 grid((unsigned)std::min<int64_t>(p.N / 16, cap > 0 ? cap : p.N / 16));
+    dim3 grid((unsigned)std::min<int64_t>(p0.N / 16, cap > 0 ? cap : p0.N / 16));
     char name[64];
-    snprintf(name, sizeof name, "gguf_%s_res_gemv_%s_m%d", ggr_name(p.quant), p.act_dtype == OXQ_BF16 ? "bf16" : "f32", mb);
-    set_plan(ctx, name, grid, dim3(nw * 64), 1, 1, 0);
+    snprintf(name, sizeof name, "gguf_%s_res_gemv_%s_m%d", ggr_name(p0.quant), p0.act_dtype == OXQ_BF16 ? "bf16" : "f32", mb);
+    set_plan(ctx, name, grid, dim3(nw * 64), 1, (uint32_t)ceil_div(p0.M, 4), 0);
     if (ctx->plan_only) return OXQ_OK;
-    if (!gguf_res_takes(p.K, p.M)) return fail(OXQ_ERR_UNSUPPORTED, "gguf resident gemv: m = %lld", (long long)p.M);
-    if ((uintptr_t)p.x & 3) return fail(OXQ_ERR_UNSUPPORTED, "gguf resident gemv: x must be 4-byte aligned");
-    if ((uint64_t)p.M * (uint64_t)p.K * 4 >= (1ull << 31)) return fail(OXQ_ERR_UNSUPPORTED, "gguf resident gemv: x larger than 2 GiB");
-    switch (p.quant) {
-    case OXQ_GGUF_Q4_0: return nw == 8 ? ggr_by_rows<OXQ_GGUF_Q4_0, 8>(s, grid, p, lds, mb) : ggr_by_rows<OXQ_GGUF_Q4_0, 16>(s, grid, p, lds, mb);
-    case OXQ_GGUF_Q8_0: return nw == 8 ? ggr_by_rows<OXQ_GGUF_Q8_0, 8>(s, grid, p, lds, mb) : ggr_by_rows<OXQ_GGUF_Q8_0, 16>(s, grid, p, lds, mb);
-    case OXQ_GGUF_Q4_K: return nw == 8 ? ggr_by_rows<OXQ_GGUF_Q4_K, 8>(s, grid, p, lds, mb) : ggr_by_rows<OXQ_GGUF_Q4_K, 16>(s, grid, p, lds, mb);
-    case OXQ_GGUF_Q6_K: return nw == 8 ? ggr_by_rows<OXQ_GGUF_Q6_K, 8>(s, grid, p, lds, mb) : ggr_by_rows<OXQ_GGUF_Q6_K, 16>(s, grid, p, lds, mb);
-    default: return fail(OXQ_ERR_UNSUPPORTED, "gguf resident gemv: format %d", p.quant);
+    if (!gguf_res_takes(p0.K, p0.M, p0.act_dtype)) return fail(OXQ_ERR_UNSUPPORTED, "gguf resident gemv: m = %lld", (long long)p0.M);
+    if ((uintptr_t)p0.x & 3) return fail(OXQ_ERR_UNSUPPORTED, "gguf resident gemv: x must be 4-byte aligned");
+    const size_t xb = p0.act_dtype == OXQ_BF16 ? 2 : 4;
+    if ((uint64_t)p0.M * (uint64_t)p0.K * 4 >= (1ull << 31)) return fail(OXQ_ERR_UNSUPPORTED, "gguf resident gemv: x larger than 2 GiB");
+    for (int64_t m0 = 0; m0 < p0.M; m0 += 4) {  // rows of x four at a time
+        GgufProblem p = p0;
+        p.M = std::min<int64_t>(4, p0.M - m0);
+        p.x = (const uint8_t *)p0.x + (size_t)m0 * p0.K * xb;
+        p.y = (uint8_t *)p0.y + (size_t)m0 * p0.N * xb;
+        int rc;
+        switch (p.quant) {
+        case OXQ_GGUF_Q4_0: rc = nw == 8 ? ggr_by_rows<OXQ_GGUF_Q4_0, 8>(s, grid, p, lds, mb) : ggr_by_rows<OXQ_GGUF_Q4_0, 16>(s, grid, p, lds, mb); break;
+        case OXQ_GGUF_Q8_0: rc = nw == 8 ? ggr_by_rows<OXQ_GGUF_Q8_0, 8>(s, grid, p, lds, mb) : ggr_by_rows<OXQ_GGUF_Q8_0, 16>(s, grid, p, lds, mb); break;
+        case OXQ_GGUF_Q4_K: rc = nw == 8 ? ggr_by_rows<OXQ_GGUF_Q4_K, 8>(s, grid, p, lds, mb) : ggr_by_rows<OXQ_GGUF_Q4_K, 16>(s, grid, p, lds, mb); break;
+        case OXQ_GGUF_Q6_K: rc = nw == 8 ? ggr_by_rows<OXQ_GGUF_Q6_K, 8>(s, grid, p, lds, mb) : ggr_by_rows<OXQ_GGUF_Q6_K, 16>(s, grid, p, lds, mb); break;
+        default: return fail(OXQ_ERR_UNSUPPORTED, "gguf resident gemv: format %d", p.quant);
+        }
+        if (rc != OXQ_OK) return rc;
     }
+    return OXQ_OK;
 }
 
 }  // namespace oxq

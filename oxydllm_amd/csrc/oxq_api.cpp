@@ -693,7 +693,7 @@ static bool wcache_forward(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p, i
 // The same for a GGUF weight (Q4_0 / Q8_0 / Q4_K / Q6_K, 1 - 4 rows of x): the copy is the strip-major
 // one of the QLinear layers.  Entry fields: qw = the block bytes, bits = the ggml format, w.pw = the copy.
 static bool wcache_forward_gguf(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p, int *rc) {
-    if (!ctx->wcache_limit || ctx->plan_only || !gguf_res_eligible(p.quant, p.K, p.N) || !gguf_res_takes(p.K, p.M))
+    if (!ctx->wcache_limit || ctx->plan_only || !gguf_res_eligible(p.quant, p.K, p.N) || !gguf_res_takes(p.K, p.M, p.act_dtype))
         return false;
     if (((uintptr_t)p.x & 15) || ((uintptr_t)p.w & 1)) return false;
     if (!ctx->wcache) {
@@ -2029,7 +2029,7 @@ int oxq_qlinear_forward(oxq_qlinear *l, void *stream, const oxq_tensor *x, const
     OXQ_TRY(check_gguf(l->ctx, decode ? "GgufQuantMatmul" : "GgufQuantMulMM", decode, false, &x2,
                        &l->weight_bytes, l->in_features, l->out_features, l->quant, &o2, &p));
     p.bias = l->has_bias ? l->bias.data : nullptr;
-    if (l->resident && gguf_res_takes(p.K, p.M) && ((uintptr_t)p.x & 15) == 0) {
+    if (l->resident && gguf_res_takes(p.K, p.M, p.act_dtype) && ((uintptr_t)p.x & 15) == 0) {
         p.w = (const uint8_t *)l->res;
         return launch_gguf_res_gemv(l->ctx, (hipStream_t)stream, p);
     }

@@ -190,7 +190,7 @@ int launch_gguf_dequant(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p, float
 // resident (strip-major) copy of a GGUF weight and its decode GEMV (gguf_res.hip)
 bool gguf_res_eligible(int quant, int64_t K, int64_t N);
 size_t gguf_res_bytes(int quant, int64_t K, int64_t N);
-bool gguf_res_takes(int64_t K, int64_t M);
+bool gguf_res_takes(int64_t K, int64_t M, int act_dtype);
 int launch_gguf_res_repack(oxq_ctx *ctx, hipStream_t s, int quant, const uint8_t *w, void *pw, int64_t K, int64_t N);
 int launch_gguf_res_dequant(oxq_ctx *ctx, hipStream_t s, int quant, const void *pw, int64_t K, int64_t N, float *out_nk);
 int launch_gguf_res_gemv(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p);  // p.w = the copy

@@ -21,7 +21,7 @@ from tests.helpers import assert_close, bits_of, round_x, to_dev
 pytestmark = pytest.mark.gpu
 ops = None
 RES = [synth.GGUF_Q4_0, synth.GGUF_Q8_0, synth.GGUF_Q4_K, synth.GGUF_Q6_K]
-ROWS = 4   # rows of x that run on the copy; up to 8 (the reference's GEMV range) the file layout serves
+ROWS = 4   # rows of x one pass on the copy takes; f32 rows up to 8 (the reference's GEMV range) take two passes
 FMTS = [pytest.param(f, id=synth.GGUF_NAMES[f]) for f in RES]
 
 
@@ -91,7 +91,7 @@ def test_resident_gemv_rows_bias_and_shapes(fmt):
                 y = layer.forward(to_dev(x, tdt))
                 kernel = ops.default_context().last_plan()["kernel"]
                 on_copy = "_res_gemv_" in kernel
-                assert on_copy == (m <= ROWS), (kernel, m, K)
+                assert on_copy == (m <= ROWS or (m <= 8 and dt is None)), (kernel, m, K)
                 assert_close(y, oracle.matmul_nt_f32(xr, w, br), f"resident {name} N={N} K={K} m={m}",
                              bf16_out=dt is not None)
 
