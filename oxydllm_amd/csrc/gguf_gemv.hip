@@ -423,37 +423,64 @@ static size_t gguf_row_bytes(int quant, int64_t K) {
 int launch_gguf_gemv(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p) {
     const bool bf = p.act_dtype == OXQ_BF16;
     const size_t xb = bf ? 2 : 4;
-    const uint32_t chunks = (uint32_t)ceil_div(p.M, 8);
-    // LDS variant: activations of one chunk of rows plus `rpwg` weight rows must fit 64 KB
-    const int64_t mrows = p.M < 8 ? p.M : 8;
-    const int mb = mrows <= 1 ? 1 : mrows <= 2 ? 2 : mrows <= 4 ? 4 : 8;
-    // per activation row: K/32 units of 32 elements + one 16-byte pad each, then two sums a unit
-    const size_t x_lds = (size_t)mb * ((((size_t)(p.K >> 5) * ((32 * xb / 16 + 1) * 16 + 8)) + 15) & ~(size_t)15);
     const size_t row_bytes = gguf_row_bytes(p.quant, p.K);
     const char *rp_env = getenv("OXQ_GGUF_RPWG");
-    // 8 rows on 8 waves.  For one activation row OXQ_GGUF_RPWG=16 runs 16 rows on 16 waves, which halves
-    // the activation traffic (every workgroup stages all of x); measured slower on 4096 x 4096 (Q4_0 5.5
-    // against 5.1 us, Q6_K 6.8 against 6.0 us); 16 rows on 8 waves of two rows each: 6.0 and 7.5 us.
     const char *pw_env = getenv("OXQ_GGUF_PW");
-    const bool wave_per_row = p.M == 1 && row_bytes + 30 <= 6 * 64 * 16 && !(pw_env && atoi(pw_env) == 0);
-    int rpwg = rp_env ? atoi(rp_env) : 8;
-    if (rpwg < 1) rpwg = 1;
-    if (rpwg > 8 && !(wave_per_row && rpwg == 16 && p.K * (int64_t)xb / 16 <= 4 * 64 * 16)) rpwg = 8;
-    auto lds_cap_of = [](int r) { return (size_t)(r == 16 ? 128 : 64) * 1024; };
-    while (rpwg > 1 && x_lds + (size_t)rpwg * row_bytes + 32 > lds_cap_of(rpwg)) rpwg >>= 1;
-    const size_t lds = x_lds + (size_t)rpwg * row_bytes + 32, lds_cap = lds_cap_of(rpwg);
+    const char *big_env = getenv("OXQ_GGUF_BIG_LDS");
     const char *force = getenv("OXQ_FORCE_GENERIC");
-    const bool use_lds = lds <= lds_cap && ((uintptr_t)p.x & 15) == 0 && ((uintptr_t)p.w & 15) == 0 &&
-                         (p.K * xb) % 16 == 0 && !(force && atoi(force));
+    const bool aligned = ((uintptr_t)p.x & 15) == 0 && ((uintptr_t)p.w & 15) == 0 && (p.K * xb) % 16 == 0 &&
+                         !(force && atoi(force));
+    // The staged kernel for `mb` activation rows a pass: x (per row K/32 units of 32 elements + one 16-byte
+    // pad each, then two sums a unit) and `rpwg` weight rows in LDS.  8 rows on 8 waves; for one activation
+    // row OXQ_GGUF_RPWG=16 runs 16 rows on 16 waves, which halves the activation traffic (every workgroup
+    // stages all of x): measured slower on 4096 x 4096 (Q4_0 5.5 against 5.1 us, Q6_K 6.8 against 6.0 us); 16
+    // rows on 8 waves of two rows each: 6.0 and 7.5 us.  64 KB of LDS a workgroup (two or more per CU) while
+    // at least 4 weight rows fit beside x; otherwise up to 150 KB, one workgroup per CU, if 8 rows fit then
+    // (a down projection: K = 14336 is 68 KB of f32 x alone; Q4_1 14336 x 4096 at one row 31 -> 17 us; with
+    // 4 rows a workgroup the staged kernel is no faster than a wave per row from global memory).
+    struct Staged {
+        bool ok;
+        int rpwg;
+        size_t lds;
+    };
+    auto staged = [&](int mb) -> Staged {
+        const size_t x_lds = (size_t)mb * ((((size_t)(p.K >> 5) * ((32 * xb / 16 + 1) * 16 + 8)) + 15) & ~(size_t)15);
+        const bool wave_per_row = mb == 1 && row_bytes + 30 <= 6 * 64 * 16 && !(pw_env && atoi(pw_env) == 0);
+        int rpwg = rp_env ? atoi(rp_env) : 8;
+        if (rpwg < 1) rpwg = 1;
+        if (rpwg > 8 && !(wave_per_row && rpwg == 16 && p.K * (int64_t)xb / 16 <= 4 * 64 * 16)) rpwg = 8;
+        const int rp0 = rpwg;
+        auto lds_cap_of = [](int r) { return (size_t)(r == 16 ? 128 : 64) * 1024; };
+        while (rpwg > 1 && x_lds + (size_t)rpwg * row_bytes + 32 > lds_cap_of(rpwg)) rpwg >>= 1;
+        size_t cap = lds_cap_of(rpwg);
+        if ((rpwg < 4 || x_lds + (size_t)rpwg * row_bytes + 32 > cap) && rp0 >= 8 && !(big_env && atoi(big_env) == 0) &&
+            x_lds + (size_t)8 * row_bytes + 32 <= (size_t)150 * 1024)
+            rpwg = 8, cap = (size_t)150 * 1024;
+        const size_t lds = x_lds + (size_t)rpwg * row_bytes + 32;
+        return Staged{aligned && lds <= cap, rpwg, lds};
+    };
+    // rows of x a pass: as many of the 8 the kernels take as still leave a staged kernel (the weight is re-read
+    // per pass, which costs less than the unstaged kernel: 4096 x 4096 f32 at 8 rows 59 -> 26 us in two passes)
+    const int64_t mrows = p.M < 8 ? p.M : 8;
+    int mb = mrows <= 1 ? 1 : mrows <= 2 ? 2 : mrows <= 4 ? 4 : 8;
+    Staged st = staged(mb);
+    while (!st.ok && mb > 1) {
+        mb >>= 1;
+        st = staged(mb);
+    }
+    const bool use_lds = st.ok;
+    const int rpwg = st.rpwg;
+    const size_t lds = st.lds;
+    const int pass = use_lds ? mb : 8;  // rows of x a launch
+    const uint32_t chunks = (uint32_t)ceil_div(p.M, pass);
     char name[64];
     snprintf(name, sizeof name, "gguf_%s_gemv_%s%s", fmt_name(p.quant), bf ? "bf16" : "f32", use_lds ? "_lds" : "");
     dim3 grid((unsigned)(use_lds ? ceil_div(p.N, rpwg) : ceil_div(p.N, 4))), block(use_lds && rpwg >= 16 ? 1024 : use_lds && rpwg >= 8 ? 512 : 256);
     set_plan(ctx, name, grid, block, 1, chunks, 0);
     if (ctx->plan_only) return OXQ_OK;
-    // m > 8: activation rows are processed 8 at a time (the weight is re-read
-    // per chunk; a tiled kernel for large m is future work).
-    for (int64_t m0 = 0; m0 < p.M; m0 += 8) {
-        const int rows = (int)((p.M - m0) < 8 ? (p.M - m0) : 8);
+    // more rows than a pass takes: the weight is re-read per pass (beyond 8 rows the tile matmul serves)
+    for (int64_t m0 = 0; m0 < p.M; m0 += pass) {
+        const int rows = (int)((p.M - m0) < pass ? (p.M - m0) : pass);
         const uint8_t *x = (const uint8_t *)p.x + (size_t)m0 * p.K * xb;
         uint8_t *y = (uint8_t *)p.y + (size_t)m0 * p.N * xb;
 #define OXQ_FMT(F)                                                                  \

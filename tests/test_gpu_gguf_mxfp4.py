@@ -176,9 +176,10 @@ def test_gguf_gemv_single_row_wave_per_weight_row(fmt, monkeypatch):
 
 
 @pytest.mark.parametrize("fmt", FMTS)
-def test_gguf_gemv_long_rows(fmt):
-    """K = 8192 with 8 activation rows does not fit the staged variant's LDS budget: the
-    direct one-wave-per-row kernel takes over and must agree as well."""
+def test_gguf_gemv_long_rows(fmt, monkeypatch):
+    """K = 8192 with 8 activation rows does not fit the staged variant's LDS budget in one pass: the rows go
+    through it in passes of as many as fit; the direct one-wave-per-row kernel (shapes that never fit, here
+    forced) must agree as well."""
     N, K, m = 160, 8192, 8
     say(f"gguf long rows {synth.GGUF_NAMES[fmt]}")
     data = synth.gguf_weight(fmt, N, K, seed=120 + fmt)
@@ -186,9 +187,15 @@ def test_gguf_gemv_long_rows(fmt):
     x = np.random.default_rng(121).standard_normal((m, K)).astype(np.float32)
     ref = oracle.matmul_nt_f32(x, w)
     y = ops.gguf_quant_matmul(to_dev(x), to_dev(data), K, N, fmt)   # f32 activations: always the GEMV kernels
+    plan = ops.default_context().last_plan()
+    assert plan["kernel"].endswith("gemv_f32_lds") and plan["launches"] in (2, 4, 8), plan
+    assert_close(y, ref, f"gguf long rows {synth.GGUF_NAMES[fmt]}")
+    monkeypatch.setenv("OXQ_FORCE_GENERIC", "1")
+    y = ops.gguf_quant_matmul(to_dev(x), to_dev(data), K, N, fmt)
     kernel = ops.default_context().last_plan()["kernel"]
     assert kernel.endswith("gemv_f32") and not kernel.endswith("_lds")
-    assert_close(y, ref, f"gguf long rows {synth.GGUF_NAMES[fmt]}")
+    assert_close(y, ref, f"gguf long rows, wave per row {synth.GGUF_NAMES[fmt]}")
+    monkeypatch.delenv("OXQ_FORCE_GENERIC")
     # bf16 rows of the decode range take the staged GEMV up to 2 rows and the tile matmul with
     # unrounded (hi + lo) weights from 3: both are held to the unrounded oracle
     for mb in (2, 3, 8):
