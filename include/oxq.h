@@ -128,7 +128,8 @@ void oxq_version(int *major, int *minor);
  * weights, f32 fold; above: tile GEMM on weights rounded to the activation type).  Shapes the
  * resident layout does not cover take the usual path.  The copy costs the packed tensors' size
  * again; least recently used copies go when max_bytes is reached.  oxq_gguf_quant_matmul does the
- * same for Q4_0 / Q8_0 / Q4_K / Q6_K weights at 1 - 4 rows of x (f32: 1 - 8), keyed by the address of the block
+ * same for the GGUF formats that have a strip-major form (see oxq_qlinear_new) at 1 - 4 rows of x (f32: 1 - 8),
+ * keyed by the address of the block
  * bytes, with the strip-major copy that oxq_qlinear_new builds.
  *
  * Contract: while a triple is cached its tensors must neither change nor be freed and reused - the
@@ -457,8 +458,9 @@ int oxq_qlinear_new(oxq_ctx *ctx, int quant, const oxq_tensor *weight_bytes, int
                     oxq_qlinear **out);
 int oxq_qlinear_forward(oxq_qlinear *layer, void *stream, const oxq_tensor *x,
                         const oxq_tensor *out);
-/* linear.rs:225-240 (the fast path's own copy of the block bytes).  For Q4_0, Q8_0, Q4_K and Q6_K layers
- * with out_features % 16 == 0 and in_features a multiple of 128 (256 for the K-quants) oxq_qlinear_new
+/* linear.rs:225-240 (the fast path's own copy of the block bytes).  For Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q4_K,
+ * Q5_K and Q6_K layers with out_features % 16 == 0 and in_features a multiple of 128 (256 for the K-quants)
+ * oxq_qlinear_new
  * builds a layer-owned copy of the blocks in strips of 16 rows (the file's bytes per weight, so twice the
  * layer's bytes while the caller keeps weight_bytes); forward then runs 1 - 4 rows of x on that copy (f32
  * rows up to 8, in two passes of four) and everything else on weight_bytes as before.  OXQ_PREPACK=0 in the environment turns the copy off.

@@ -17,12 +17,17 @@
 //               scale bytes)                                                                   2304 B
 //   Q6_K  CH 2  16 B low nibbles + 8 B high bit pairs, unit header = the unit's two int8
 //               scales, block header = d                                                       3360 B
+//   Q4_1  CH 1  16 B quants, unit header d, m (4 B)                                            1280 B
+//   Q5_0  CH 1  16 B low nibbles + 4 B high bits, unit header d                                1408 B
+//   Q5_1  CH 1  16 B low nibbles + 4 B high bits, unit header d, m (4 B)                       1536 B
+//   Q5_K  CH 2  16 B low nibbles + 4 B high bits, block header as Q4_K                         2816 B
 //
 // Exactly the file's bytes per weight.  Inside a unit the 16 elements of each half are stored ROTATED
 // by the lane's column: position n (0..15) of half h holds element 16 h + (col - n) mod 16 (4-bit
 // formats: half 0 in the low nibbles of the 16 bytes, half 1 in the high ones, byte n = position n;
 // Q8_0: byte 16 h + n; Q6_K: low nibbles likewise, the bit pair of position 16 h + 4 s + b in bits 2s
-// of byte b of word h).  That is what lets the activations stay in registers: lane col loads
+// of byte b of word h; 5-bit formats: low nibbles likewise, the high bit of position 16 h + n in bit
+// 16 h + n of the fifth word).  That is what lets the activations stay in registers: lane col loads
 // x[16 h + col] of its unit (two 4-byte loads, 64 contiguous bytes per 16 lanes), and a rotation of
 // that register by n lanes inside the row of 16 (a DPP operand of the multiply-add, no instruction of
 // its own) hands every lane the element its position n multiplies.  No LDS, no staging, no barrier
@@ -40,10 +45,14 @@ template <> struct GgrFmt<OXQ_GGUF_Q4_0> { static constexpr int CH = 1, QW = 4, 
 template <> struct GgrFmt<OXQ_GGUF_Q8_0> { static constexpr int CH = 1, QW = 8, UH = 2, BH = 0; };
 template <> struct GgrFmt<OXQ_GGUF_Q4_K> { static constexpr int CH = 2, QW = 4, UH = 0, BH = 16; };
 template <> struct GgrFmt<OXQ_GGUF_Q6_K> { static constexpr int CH = 2, QW = 6, UH = 2, BH = 2; };
+template <> struct GgrFmt<OXQ_GGUF_Q4_1> { static constexpr int CH = 1, QW = 4, UH = 4, BH = 0; };
+template <> struct GgrFmt<OXQ_GGUF_Q5_0> { static constexpr int CH = 1, QW = 5, UH = 2, BH = 0; };
+template <> struct GgrFmt<OXQ_GGUF_Q5_1> { static constexpr int CH = 1, QW = 5, UH = 4, BH = 0; };
+template <> struct GgrFmt<OXQ_GGUF_Q5_K> { static constexpr int CH = 2, QW = 5, UH = 0, BH = 16; };
 
 template <int FMT> struct GgrLayout {
     typedef GgrFmt<FMT> F;
-    static constexpr int P128 = F::QW / 4, P64 = (F::QW % 4) / 2;
+    static constexpr int P128 = F::QW / 4, P64 = (F::QW % 4) / 2, P32 = F::QW % 2;  // planes of 16, 8 and 4 bytes a lane
     static constexpr int UH_OFF = 64 * F::QW * 4;            // unit headers behind the planes
     static constexpr int CHB = 64 * (F::QW * 4 + F::UH);     // bytes of a chunk
     static constexpr int BH_OFF = F::CH * CHB;               // block header behind the chunks
@@ -94,11 +103,38 @@ __global__ __launch_bounds__(256) void ggr_repack_kernel(const uint8_t *__restri
             for (int bb = 0; bb < 4; ++bb) v |= (uint32_t)p[2 + 16 * (i >> 2) + el(4 * (i & 3) + bb)] << (8 * bb);
             qw[i] = v;
         }
-    } else if constexpr (FMT == OXQ_GGUF_Q4_K) {
+    } else if constexpr (FMT == OXQ_GGUF_Q4_1 || FMT == OXQ_GGUF_Q5_0 || FMT == OXQ_GGUF_Q5_1) {
+        constexpr bool MIN = FMT != OXQ_GGUF_Q5_0, FIVE = FMT != OXQ_GGUF_Q4_1;
+        const uint8_t *p = row + (size_t)u * GgufFmt<FMT>::BB;
+        uh = ld16(p) | (MIN ? ld16(p + 2) << 16 : 0u);
+        const uint8_t *hp = p + (MIN ? 4 : 2), *qs = hp + (FIVE ? 4 : 0);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            uint32_t v = 0;
+#pragma unroll
+            for (int bb = 0; bb < 4; ++bb) v |= (uint32_t)qs[el(4 * i + bb)] << (8 * bb);  // byte e: elements e, e + 16
+            qw[i] = v;
+        }
+        if constexpr (FIVE) {
+            const uint32_t qh = ld16(hp) | (ld16(hp + 2) << 16);  // bit e: element e
+            uint32_t v = 0;
+#pragma unroll
+            for (int nn = 0; nn < 16; ++nn) v |= (((qh >> el(nn)) & 1u) << nn) | (((qh >> (16 + el(nn))) & 1u) << (16 + nn));
+            qw[4] = v;
+        }
+    } else if constexpr (FMT == OXQ_GGUF_Q4_K || FMT == OXQ_GGUF_Q5_K) {
+        constexpr bool FIVE = FMT == OXQ_GGUF_Q5_K;
         const int b = u >> 3, sb = u & 7;
-        const uint8_t *p = row + (size_t)b * 144;
-        const uint8_t *qs = p + 16 + (sb >> 1) * 32;
+        const uint8_t *p = row + (size_t)b * (FIVE ? 176 : 144);
+        const uint8_t *qs = p + (FIVE ? 48 : 16) + (sb >> 1) * 32;
         const int sh = (sb & 1) * 4;
+        if constexpr (FIVE) {  // bit sb of byte e of qh (p + 16): element e of unit sb
+            uint32_t v = 0;
+#pragma unroll
+            for (int nn = 0; nn < 16; ++nn)
+                v |= ((((uint32_t)p[16 + el(nn)] >> sb) & 1u) << nn) | ((((uint32_t)p[32 + el(nn)] >> sb) & 1u) << (16 + nn));
+            qw[4] = v;
+        }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             uint32_t v = 0;
@@ -152,7 +188,9 @@ __global__ __launch_bounds__(256) void ggr_repack_kernel(const uint8_t *__restri
         uint32_t *d = (uint32_t *)(chunk + L::P128 * 1024 + lane * 8);
         d[0] = qw[4 * L::P128], d[1] = qw[4 * L::P128 + 1];
     }
-    if constexpr (F::UH) *(uint16_t *)(chunk + L::UH_OFF + lane * 2) = (uint16_t)uh;
+    if constexpr (L::P32) *(uint32_t *)(chunk + L::P128 * 1024 + L::P64 * 512 + lane * 4) = qw[F::QW - 1];
+    if constexpr (F::UH == 2) *(uint16_t *)(chunk + L::UH_OFF + lane * 2) = (uint16_t)uh;
+    if constexpr (F::UH == 4) *(uint32_t *)(chunk + L::UH_OFF + lane * 4) = uh;
 }
 
 // ---------------------------------------------------------------------------
@@ -172,7 +210,13 @@ __device__ __forceinline__ void ggr_factors(uint32_t uh, const uint32_t (&bh)[4]
     } else if constexpr (FMT == OXQ_GGUF_Q8_0) {
         const float d = f16_bits_to_f32(uh);
         a0 = a1 = d, b0 = b1 = 128.0f * d;
-    } else if constexpr (FMT == OXQ_GGUF_Q4_K) {
+    } else if constexpr (FMT == OXQ_GGUF_Q4_1 || FMT == OXQ_GGUF_Q5_1) {
+        a0 = a1 = f16_bits_to_f32(uh & 0xFFFFu);
+        b0 = b1 = -f16_bits_to_f32(uh >> 16);
+    } else if constexpr (FMT == OXQ_GGUF_Q5_0) {
+        const float d = f16_bits_to_f32(uh);
+        a0 = a1 = d, b0 = b1 = 16.0f * d;
+    } else if constexpr (FMT == OXQ_GGUF_Q4_K || FMT == OXQ_GGUF_Q5_K) {
         const float d = f16_bits_to_f32(bh[0] & 0xFFFFu), dmin = f16_bits_to_f32(bh[0] >> 16);
         // get_scale_min_k4 (quant_kernels.metal:2438-2450) on the 12 scale bytes in bh[1..3]
         const uint32_t sft = 8u * (uint32_t)(sb & 3);
@@ -200,6 +244,12 @@ __device__ __forceinline__ void ggr_ints(const uint32_t (&qw)[GgrFmt<FMT>::QW], 
         for (int i = 0; i < 4; ++i) {
             bytes_to_f32((qw[i] & 0x0F0F0F0Fu) | (((qw[4] >> (2 * i)) & 0x03030303u) << 4), q + 4 * i);  // q + 32
             bytes_to_f32(((qw[i] >> 4) & 0x0F0F0F0Fu) | (((qw[5] >> (2 * i)) & 0x03030303u) << 4), q + 16 + 4 * i);
+        }
+    } else if constexpr (GgrFmt<FMT>::QW == 5) {  // a fifth bit from word 4: bit 16 h + n for position n of half h
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            bytes_to_f32((qw[i] & 0x0F0F0F0Fu) | (spread4(qw[4] >> (4 * i)) << 4), q + 4 * i);
+            bytes_to_f32(((qw[i] >> 4) & 0x0F0F0F0Fu) | (spread4(qw[4] >> (16 + 4 * i)) << 4), q + 16 + 4 * i);
         }
     } else {
 #pragma unroll
@@ -233,8 +283,10 @@ __global__ __launch_bounds__(256) void ggr_dequant_kernel(const uint8_t *__restr
         const uint32_t *d = (const uint32_t *)(chunk + L::P128 * 1024 + lane * 8);
         qw[4 * L::P128] = d[0], qw[4 * L::P128 + 1] = d[1];
     }
+    if constexpr (L::P32) qw[F::QW - 1] = *(const uint32_t *)(chunk + L::P128 * 1024 + L::P64 * 512 + lane * 4);
     uint32_t uh = 0, bh[4] = {0u, 0u, 0u, 0u};
-    if constexpr (F::UH) uh = *(const uint16_t *)(chunk + L::UH_OFF + lane * 2);
+    if constexpr (F::UH == 2) uh = *(const uint16_t *)(chunk + L::UH_OFF + lane * 2);
+    if constexpr (F::UH == 4) uh = *(const uint32_t *)(chunk + L::UH_OFF + lane * 4);
     if constexpr (F::BH == 16) {
         const u32x4_t v = *(const u32x4_t *)(blk + L::BH_OFF + col * 16);
         bh[0] = v[0], bh[1] = v[1], bh[2] = v[2], bh[3] = v[3];
@@ -255,14 +307,35 @@ __global__ __launch_bounds__(256) void ggr_dequant_kernel(const uint8_t *__restr
         const float d = f16_bits_to_f32(uh);
 #pragma unroll
         for (int e = 0; e < 32; ++e) wf[e] = (float)(int)(int8_t)((qw[e >> 2] >> (8 * (e & 3))) & 0xFFu) * d;
-    } else if constexpr (FMT == OXQ_GGUF_Q4_K) {
+    } else if constexpr (FMT == OXQ_GGUF_Q4_K || FMT == OXQ_GGUF_Q5_K) {
         float sc_v, m_v, t0, t1;
         ggr_factors<FMT>(uh, bh, sb, sc_v, t0, m_v, t1);
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
             const uint32_t byte = (qw[e >> 2] >> (8 * (e & 3))) & 0xFFu;
-            wf[e] = sc_v * (float)(byte & 0xF) - m_v;
-            wf[e + 16] = sc_v * (float)(byte >> 4) - m_v;
+            uint32_t lo = byte & 0xF, hi = byte >> 4;
+            if constexpr (FMT == OXQ_GGUF_Q5_K) lo |= ((qw[4] >> e) & 1u) << 4, hi |= ((qw[4] >> (16 + e)) & 1u) << 4;
+            wf[e] = sc_v * (float)lo - m_v;
+            wf[e + 16] = sc_v * (float)hi - m_v;
+        }
+    } else if constexpr (FMT == OXQ_GGUF_Q4_1 || FMT == OXQ_GGUF_Q5_1) {
+        const float d = f16_bits_to_f32(uh & 0xFFFFu), m = f16_bits_to_f32(uh >> 16);
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const uint32_t byte = (qw[e >> 2] >> (8 * (e & 3))) & 0xFFu;
+            uint32_t lo = byte & 0xF, hi = byte >> 4;
+            if constexpr (FMT == OXQ_GGUF_Q5_1) lo |= ((qw[4] >> e) & 1u) << 4, hi |= ((qw[4] >> (16 + e)) & 1u) << 4;
+            wf[e] = (float)lo * d + m;
+            wf[e + 16] = (float)hi * d + m;
+        }
+    } else if constexpr (FMT == OXQ_GGUF_Q5_0) {
+        const float d = f16_bits_to_f32(uh);
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const uint32_t byte = (qw[e >> 2] >> (8 * (e & 3))) & 0xFFu;
+            const uint32_t lo = (byte & 0xF) | (((qw[4] >> e) & 1u) << 4), hi = (byte >> 4) | (((qw[4] >> (16 + e)) & 1u) << 4);
+            wf[e] = (float)((int)lo - 16) * d;
+            wf[e + 16] = (float)((int)hi - 16) * d;
         }
     } else {
         float s0, s1, t0, t1;
@@ -393,8 +466,11 @@ __global__ __launch_bounds__(NW * 64) void ggr_gemv_kernel(const void *__restric
             const u32x2_t v = __builtin_amdgcn_raw_buffer_load_b64(rs, lane * 8, coff + L::P128 * 1024, 2);
             st.qw[4 * L::P128] = v[0], st.qw[4 * L::P128 + 1] = v[1];
         }
+        if constexpr (L::P32)
+            st.qw[F::QW - 1] = __builtin_amdgcn_raw_buffer_load_b32(rs, lane * 4, coff + L::P128 * 1024 + L::P64 * 512, 2);
         st.uh = 0;
-        if constexpr (F::UH) st.uh = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(rs, lane * 2, coff + L::UH_OFF, 2);
+        if constexpr (F::UH == 2) st.uh = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(rs, lane * 2, coff + L::UH_OFF, 2);
+        if constexpr (F::UH == 4) st.uh = __builtin_amdgcn_raw_buffer_load_b32(rs, lane * 4, coff + L::UH_OFF, 2);
         st.bh[0] = st.bh[1] = st.bh[2] = st.bh[3] = 0;
         if constexpr (F::BH == 16) {
             const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(rs, col * 16, boff + L::BH_OFF, 0);
@@ -501,9 +577,12 @@ __global__ __launch_bounds__(NW * 64) void ggr_gemv_kernel(const void *__restric
 // host side
 // ---------------------------------------------------------------------------
 static bool ggr_format(int quant) {
-    return quant == OXQ_GGUF_Q4_0 || quant == OXQ_GGUF_Q8_0 || quant == OXQ_GGUF_Q4_K || quant == OXQ_GGUF_Q6_K;
+    return quant == OXQ_GGUF_Q4_0 || quant == OXQ_GGUF_Q8_0 || quant == OXQ_GGUF_Q4_K || quant == OXQ_GGUF_Q6_K ||
+           quant == OXQ_GGUF_Q4_1 || quant == OXQ_GGUF_Q5_0 || quant == OXQ_GGUF_Q5_1 || quant == OXQ_GGUF_Q5_K;
 }
-static int ggr_chunks_per_block(int quant) { return (quant == OXQ_GGUF_Q4_K || quant == OXQ_GGUF_Q6_K) ? 2 : 1; }
+static int ggr_chunks_per_block(int quant) {
+    return (quant == OXQ_GGUF_Q4_K || quant == OXQ_GGUF_Q6_K || quant == OXQ_GGUF_Q5_K) ? 2 : 1;
+}
 
 bool gguf_res_eligible(int quant, int64_t K, int64_t N) {
     if (!ggr_format(quant) || N <= 0 || N % 16 != 0 || K <= 0 || K % (128 * ggr_chunks_per_block(quant)) != 0) return false;
@@ -532,7 +611,16 @@ static size_t ggr_lds_bytes(int64_t K, int mb) { return (size_t)2 * 4 * ggr_wave
 bool gguf_res_takes(int64_t, int64_t M, int act_dtype) { return M >= 1 && (M <= 4 || (M <= 8 && act_dtype == OXQ_F32)); }
 
 static const char *ggr_name(int q) {
-    return q == OXQ_GGUF_Q4_0 ? "q4_0" : q == OXQ_GGUF_Q8_0 ? "q8_0" : q == OXQ_GGUF_Q4_K ? "q4k" : "q6k";
+    switch (q) {
+    case OXQ_GGUF_Q4_0: return "q4_0";
+    case OXQ_GGUF_Q8_0: return "q8_0";
+    case OXQ_GGUF_Q4_K: return "q4k";
+    case OXQ_GGUF_Q4_1: return "q4_1";
+    case OXQ_GGUF_Q5_0: return "q5_0";
+    case OXQ_GGUF_Q5_1: return "q5_1";
+    case OXQ_GGUF_Q5_K: return "q5k";
+    default: return "q6k";
+    }
 }
 
 int launch_gguf_res_repack(oxq_ctx *ctx, hipStream_t s, int quant, const uint8_t *w, void *pw, int64_t K, int64_t N) {
@@ -549,6 +637,10 @@ int launch_gguf_res_repack(oxq_ctx *ctx, hipStream_t s, int quant, const uint8_t
         OXQ_GR(OXQ_GGUF_Q8_0);
         OXQ_GR(OXQ_GGUF_Q4_K);
         OXQ_GR(OXQ_GGUF_Q6_K);
+        OXQ_GR(OXQ_GGUF_Q4_1);
+        OXQ_GR(OXQ_GGUF_Q5_0);
+        OXQ_GR(OXQ_GGUF_Q5_1);
+        OXQ_GR(OXQ_GGUF_Q5_K);
     default: return fail(OXQ_ERR_UNSUPPORTED, "gguf repack: format %d has no resident layout", quant);
     }
 #undef OXQ_GR
@@ -570,6 +662,10 @@ int launch_gguf_res_dequant(oxq_ctx *ctx, hipStream_t s, int quant, const void *
         OXQ_GR(OXQ_GGUF_Q8_0);
         OXQ_GR(OXQ_GGUF_Q4_K);
         OXQ_GR(OXQ_GGUF_Q6_K);
+        OXQ_GR(OXQ_GGUF_Q4_1);
+        OXQ_GR(OXQ_GGUF_Q5_0);
+        OXQ_GR(OXQ_GGUF_Q5_1);
+        OXQ_GR(OXQ_GGUF_Q5_K);
     default: return fail(OXQ_ERR_UNSUPPORTED, "gguf dequant: format %d has no resident layout", quant);
     }
 #undef OXQ_GR
@@ -622,6 +718,10 @@ int launch_gguf_res_gemv(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p0) {
         case OXQ_GGUF_Q8_0: rc = nw == 8 ? ggr_by_rows<OXQ_GGUF_Q8_0, 8>(s, grid, p, lds, mb) : ggr_by_rows<OXQ_GGUF_Q8_0, 16>(s, grid, p, lds, mb); break;
         case OXQ_GGUF_Q4_K: rc = nw == 8 ? ggr_by_rows<OXQ_GGUF_Q4_K, 8>(s, grid, p, lds, mb) : ggr_by_rows<OXQ_GGUF_Q4_K, 16>(s, grid, p, lds, mb); break;
         case OXQ_GGUF_Q6_K: rc = nw == 8 ? ggr_by_rows<OXQ_GGUF_Q6_K, 8>(s, grid, p, lds, mb) : ggr_by_rows<OXQ_GGUF_Q6_K, 16>(s, grid, p, lds, mb); break;
+        case OXQ_GGUF_Q4_1: rc = nw == 8 ? ggr_by_rows<OXQ_GGUF_Q4_1, 8>(s, grid, p, lds, mb) : ggr_by_rows<OXQ_GGUF_Q4_1, 16>(s, grid, p, lds, mb); break;
+        case OXQ_GGUF_Q5_0: rc = nw == 8 ? ggr_by_rows<OXQ_GGUF_Q5_0, 8>(s, grid, p, lds, mb) : ggr_by_rows<OXQ_GGUF_Q5_0, 16>(s, grid, p, lds, mb); break;
+        case OXQ_GGUF_Q5_1: rc = nw == 8 ? ggr_by_rows<OXQ_GGUF_Q5_1, 8>(s, grid, p, lds, mb) : ggr_by_rows<OXQ_GGUF_Q5_1, 16>(s, grid, p, lds, mb); break;
+        case OXQ_GGUF_Q5_K: rc = nw == 8 ? ggr_by_rows<OXQ_GGUF_Q5_K, 8>(s, grid, p, lds, mb) : ggr_by_rows<OXQ_GGUF_Q5_K, 16>(s, grid, p, lds, mb); break;
         default: return fail(OXQ_ERR_UNSUPPORTED, "gguf resident gemv: format %d", p.quant);
         }
         if (rc != OXQ_OK) return rc;

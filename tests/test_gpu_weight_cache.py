@@ -164,7 +164,8 @@ def test_forget_evict_and_ineligible_shapes():
         ctx.close()
 
 
-@pytest.mark.parametrize("fmt", [synth.GGUF_Q4_0, synth.GGUF_Q8_0, synth.GGUF_Q4_K, synth.GGUF_Q6_K])
+@pytest.mark.parametrize("fmt", [synth.GGUF_Q4_0, synth.GGUF_Q8_0, synth.GGUF_Q4_K, synth.GGUF_Q6_K, synth.GGUF_Q5_0,
+                                 synth.GGUF_Q5_K])
 def test_cached_gguf_op_equals_the_resident_layer(fmt):
     N, K = 256, 2048
     data = synth.gguf_weight(fmt, N, K, seed=90 + fmt)
