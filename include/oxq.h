@@ -458,10 +458,10 @@ int oxq_qlinear_new(oxq_ctx *ctx, int quant, const oxq_tensor *weight_bytes, int
                     oxq_qlinear **out);
 int oxq_qlinear_forward(oxq_qlinear *layer, void *stream, const oxq_tensor *x,
                         const oxq_tensor *out);
-/* linear.rs:225-240 (the fast path's own copy of the block bytes).  For Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q4_K,
- * Q5_K and Q6_K layers with out_features % 16 == 0 and in_features a multiple of 128 (256 for the K-quants)
- * oxq_qlinear_new
- * builds a layer-owned copy of the blocks in strips of 16 rows (the file's bytes per weight, so twice the
+/* linear.rs:225-240 (the fast path's own copy of the block bytes).  For layers of any of the ten formats
+ * with out_features % 16 == 0 and in_features a multiple of 128 (256 for the K-quants) oxq_qlinear_new
+ * builds a layer-owned copy of the blocks in strips of 16 rows (the file's bytes per weight; Q3_K: 112 for
+ * 110 bytes a super-block; so twice the
  * layer's bytes while the caller keeps weight_bytes); forward then runs 1 - 4 rows of x on that copy (f32
  * rows up to 8, in two passes of four) and everything else on weight_bytes as before.  OXQ_PREPACK=0 in the environment turns the copy off.
  * *resident = 1 if the layer holds the copy. */

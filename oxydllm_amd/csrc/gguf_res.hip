@@ -21,13 +21,17 @@
 //   Q5_0  CH 1  16 B low nibbles + 4 B high bits, unit header d                                1408 B
 //   Q5_1  CH 1  16 B low nibbles + 4 B high bits, unit header d, m (4 B)                       1536 B
 //   Q5_K  CH 2  16 B low nibbles + 4 B high bits, block header as Q4_K                         2816 B
+//   Q2_K  CH 2  8 B bit pairs, unit header = the unit's two scale bytes, block header d, dmin  1344 B
+//   Q3_K  CH 2  8 B low bit pairs + 4 B high bits, block header = the 12 scale bytes, d, 2 B
+//               unused (the one format two bytes a super-block larger than the file)           1792 B
 //
 // Exactly the file's bytes per weight.  Inside a unit the 16 elements of each half are stored ROTATED
 // by the lane's column: position n (0..15) of half h holds element 16 h + (col - n) mod 16 (4-bit
 // formats: half 0 in the low nibbles of the 16 bytes, half 1 in the high ones, byte n = position n;
 // Q8_0: byte 16 h + n; Q6_K: low nibbles likewise, the bit pair of position 16 h + 4 s + b in bits 2s
 // of byte b of word h; 5-bit formats: low nibbles likewise, the high bit of position 16 h + n in bit
-// 16 h + n of the fifth word).  That is what lets the activations stay in registers: lane col loads
+// 16 h + n of the fifth word; Q2_K / Q3_K: the bit pair of position 16 h + 4 s + b in bits 2s of byte b of
+// word h, Q3_K's third bit as the fifth of the 5-bit formats).  That is what lets the activations stay in registers: lane col loads
 // x[16 h + col] of its unit (two 4-byte loads, 64 contiguous bytes per 16 lanes), and a rotation of
 // that register by n lanes inside the row of 16 (a DPP operand of the multiply-add, no instruction of
 // its own) hands every lane the element its position n multiplies.  No LDS, no staging, no barrier
@@ -49,6 +53,10 @@ template <> struct GgrFmt<OXQ_GGUF_Q4_1> { static constexpr int CH = 1, QW = 4, 
 template <> struct GgrFmt<OXQ_GGUF_Q5_0> { static constexpr int CH = 1, QW = 5, UH = 2, BH = 0; };
 template <> struct GgrFmt<OXQ_GGUF_Q5_1> { static constexpr int CH = 1, QW = 5, UH = 4, BH = 0; };
 template <> struct GgrFmt<OXQ_GGUF_Q5_K> { static constexpr int CH = 2, QW = 5, UH = 0, BH = 16; };
+template <> struct GgrFmt<OXQ_GGUF_Q2_K> { static constexpr int CH = 2, QW = 2, UH = 2, BH = 4; };
+template <> struct GgrFmt<OXQ_GGUF_Q3_K> { static constexpr int CH = 2, QW = 3, UH = 0, BH = 16; };
+// formats with a scale per 16 elements: two multiply-add chains and two sums a unit
+template <int FMT> constexpr bool ggr_two_scales = FMT == OXQ_GGUF_Q6_K || FMT == OXQ_GGUF_Q2_K || FMT == OXQ_GGUF_Q3_K;
 
 template <int FMT> struct GgrLayout {
     typedef GgrFmt<FMT> F;
@@ -57,7 +65,9 @@ template <int FMT> struct GgrLayout {
     static constexpr int CHB = 64 * (F::QW * 4 + F::UH);     // bytes of a chunk
     static constexpr int BH_OFF = F::CH * CHB;               // block header behind the chunks
     static constexpr int BLKB = F::CH * CHB + 16 * F::BH;    // bytes of a block
-    static_assert(BLKB == 16 * (128 * F::CH / GgufFmt<FMT>::BE) * GgufFmt<FMT>::BB, "the copy has the file's size");
+    // the file's bytes per weight, except Q3_K: its 12 scale bytes and d share one 16-byte header (112 for 110)
+    static_assert(BLKB == 16 * (128 * F::CH / GgufFmt<FMT>::BE) * (GgufFmt<FMT>::BB + (FMT == OXQ_GGUF_Q3_K ? 2 : 0)),
+                  "the copy has the file's size");
 };
 
 // ---------------------------------------------------------------------------
@@ -150,6 +160,39 @@ __global__ __launch_bounds__(256) void ggr_repack_kernel(const uint8_t *__restri
 #pragma unroll
             for (int i = 0; i < 8; ++i) *(uint16_t *)(blk + L::BH_OFF + col * 16 + 2 * i) = (uint16_t)ld16(p + 2 * i);
         }
+    } else if constexpr (FMT == OXQ_GGUF_Q2_K || FMT == OXQ_GGUF_Q3_K) {
+        constexpr bool THREE = FMT == OXQ_GGUF_Q3_K;
+        const int b = u >> 3, ub = u & 7;
+        const uint8_t *p = row + (size_t)b * (THREE ? 110 : 84);
+        const uint8_t *qs = p + (THREE ? 32 : 16) + (ub >> 2) * 32;  // element e: bits sh, sh + 1 of byte e
+        const int sh = (ub & 3) * 2;
+#pragma unroll
+        for (int hs = 0; hs < 2; ++hs) {
+            uint32_t v = 0;
+#pragma unroll
+            for (int s2 = 0; s2 < 4; ++s2)
+#pragma unroll
+                for (int bb = 0; bb < 4; ++bb)
+                    v |= (((uint32_t)qs[16 * hs + el(4 * s2 + bb)] >> sh) & 3u) << (8 * bb + 2 * s2);
+            qw[hs] = v;
+        }
+        if constexpr (THREE) {  // bit ub of byte e of hmask (p): the third bit of element e of unit ub
+            uint32_t v = 0;
+#pragma unroll
+            for (int nn = 0; nn < 16; ++nn)
+                v |= ((((uint32_t)p[el(nn)] >> ub) & 1u) << nn) | ((((uint32_t)p[16 + el(nn)] >> ub) & 1u) << (16 + nn));
+            qw[2] = v;
+            if (ub == 0) {
+                uint16_t *h = (uint16_t *)(blk + L::BH_OFF + col * 16);
+#pragma unroll
+                for (int i = 0; i < 6; ++i) h[i] = (uint16_t)ld16(p + 96 + 2 * i);
+                h[6] = (uint16_t)ld16(p + 108);
+                h[7] = 0;
+            }
+        } else {
+            uh = (uint32_t)p[2 * ub] | ((uint32_t)p[2 * ub + 1] << 8);
+            if (ub == 0) *(uint32_t *)(blk + L::BH_OFF + col * 4) = ld16(p + 80) | (ld16(p + 82) << 16);
+        }
     } else {  // Q6_K
         const int b = u >> 3, sub = u & 7;
         const int h = sub >> 2, quad = sub & 3;
@@ -226,6 +269,24 @@ __device__ __forceinline__ void ggr_factors(uint32_t uh, const uint32_t (&bh)[4]
         const uint32_t mnv = ((b & 63u) & low) | (((c >> 4) | ((b >> 6) << 4)) & ~low);
         a0 = a1 = d * (float)scv;
         b0 = b1 = dmin * (float)mnv;
+    } else if constexpr (FMT == OXQ_GGUF_Q2_K) {
+        const float d = f16_bits_to_f32(bh[0] & 0xFFFFu), dmin = f16_bits_to_f32(bh[0] >> 16);
+        a0 = d * (float)(uh & 0xFu);
+        b0 = dmin * (float)((uh >> 4) & 0xFu);
+        a1 = d * (float)((uh >> 8) & 0xFu);
+        b1 = dmin * (float)(uh >> 12);
+    } else if constexpr (FMT == OXQ_GGUF_Q3_K) {
+        // q3k_scale (quant_kernels.metal:2594-2604) of sub-blocks 2 sb and 2 sb + 1 on the 12 scale bytes in bh[0..2]
+        // (sub-blocks 2 sb and 2 sb + 1 share their group sb / 2 and sit in bytes k = 2 (sb % 2) and k + 1)
+        const float d = f16_bits_to_f32(bh[3] & 0xFFFFu);
+        const uint32_t group = (uint32_t)sb >> 1, k8 = 16u * ((uint32_t)sb & 1u);
+        const uint32_t b0w = bh[0], b1w = bh[1], b2w = bh[2];
+        const uint32_t lw = ((group & 1u) ? b1w : b0w) >> k8 >> (group < 2u ? 0u : 4u);  // bytes k, k + 1 in bits 0.., 8..
+        const uint32_t hw = b2w >> k8 >> (2u * group);
+        const int s0 = (int)((lw & 0xFu) | ((hw & 3u) << 4)) - 32;
+        const int s1 = (int)(((lw >> 8) & 0xFu) | (((hw >> 8) & 3u) << 4)) - 32;
+        a0 = d * (float)s0, a1 = d * (float)s1;
+        b0 = 4.0f * a0, b1 = 4.0f * a1;
     } else {  // Q6_K
         const float d = f16_bits_to_f32(bh[0] & 0xFFFFu);
         a0 = d * (float)(int)(int8_t)(uh & 0xFFu);
@@ -245,6 +306,15 @@ __device__ __forceinline__ void ggr_ints(const uint32_t (&qw)[GgrFmt<FMT>::QW], 
             bytes_to_f32((qw[i] & 0x0F0F0F0Fu) | (((qw[4] >> (2 * i)) & 0x03030303u) << 4), q + 4 * i);  // q + 32
             bytes_to_f32(((qw[i] >> 4) & 0x0F0F0F0Fu) | (((qw[5] >> (2 * i)) & 0x03030303u) << 4), q + 16 + 4 * i);
         }
+    } else if constexpr (FMT == OXQ_GGUF_Q2_K || FMT == OXQ_GGUF_Q3_K) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int s2 = 0; s2 < 4; ++s2) {
+                uint32_t v = (qw[h] >> (2 * s2)) & 0x03030303u;
+                if constexpr (FMT == OXQ_GGUF_Q3_K) v |= spread4(qw[2] >> (16 * h + 4 * s2)) << 2;  // q + 4
+                bytes_to_f32(v, q + 16 * h + 4 * s2);
+            }
     } else if constexpr (GgrFmt<FMT>::QW == 5) {  // a fifth bit from word 4: bit 16 h + n for position n of half h
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -290,6 +360,8 @@ __global__ __launch_bounds__(256) void ggr_dequant_kernel(const uint8_t *__restr
     if constexpr (F::BH == 16) {
         const u32x4_t v = *(const u32x4_t *)(blk + L::BH_OFF + col * 16);
         bh[0] = v[0], bh[1] = v[1], bh[2] = v[2], bh[3] = v[3];
+    } else if constexpr (F::BH == 4) {
+        bh[0] = *(const uint32_t *)(blk + L::BH_OFF + col * 4);
     } else if constexpr (F::BH == 2) {
         bh[0] = *(const uint16_t *)(blk + L::BH_OFF + col * 2);
     }
@@ -327,6 +399,21 @@ __global__ __launch_bounds__(256) void ggr_dequant_kernel(const uint8_t *__restr
             if constexpr (FMT == OXQ_GGUF_Q5_1) lo |= ((qw[4] >> e) & 1u) << 4, hi |= ((qw[4] >> (16 + e)) & 1u) << 4;
             wf[e] = (float)lo * d + m;
             wf[e + 16] = (float)hi * d + m;
+        }
+    } else if constexpr (FMT == OXQ_GGUF_Q2_K || FMT == OXQ_GGUF_Q3_K) {
+        float s0, s1, m0, m1;
+        ggr_factors<FMT>(uh, bh, sb, s0, s1, m0, m1);
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const int sft = 8 * (e & 3) + 2 * (e >> 2);
+            const uint32_t lo = (qw[0] >> sft) & 3u, hi = (qw[1] >> sft) & 3u;
+            if constexpr (FMT == OXQ_GGUF_Q2_K) {
+                wf[e] = s0 * (float)lo - m0;
+                wf[e + 16] = s1 * (float)hi - m1;
+            } else {
+                wf[e] = s0 * (float)((int)lo + (int)(((qw[2] >> e) & 1u) << 2) - 4);
+                wf[e + 16] = s1 * (float)((int)hi + (int)(((qw[2] >> (16 + e)) & 1u) << 2) - 4);
+            }
         }
     } else if constexpr (FMT == OXQ_GGUF_Q5_0) {
         const float d = f16_bits_to_f32(uh);
@@ -475,6 +562,8 @@ __global__ __launch_bounds__(NW * 64) void ggr_gemv_kernel(const void *__restric
         if constexpr (F::BH == 16) {
             const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(rs, col * 16, boff + L::BH_OFF, 0);
             st.bh[0] = v[0], st.bh[1] = v[1], st.bh[2] = v[2], st.bh[3] = v[3];
+        } else if constexpr (F::BH == 4) {
+            st.bh[0] = __builtin_amdgcn_raw_buffer_load_b32(rs, col * 4, boff + L::BH_OFF, 0);
         } else if constexpr (F::BH == 2) {
             st.bh[0] = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(rs, col * 2, boff + L::BH_OFF, 0);
         }
@@ -520,7 +609,7 @@ __global__ __launch_bounds__(NW * 64) void ggr_gemv_kernel(const void *__restric
                 // chunks past the share hold zeros (weights, headers and x alike)
 #pragma unroll
                 for (int m = 0; m < MB; ++m) {
-                    if constexpr (FMT == OXQ_GGUF_Q6_K) {  // a scale per half unit
+                    if constexpr (ggr_two_scales<FMT>) {  // a scale per half unit
                         float dot0 = 0.0f, dot1 = 0.0f;
                         ggr_dot16(q, xr[m][0], dot0);
                         ggr_dot16(q + 16, xr[m][1], dot1);
@@ -578,10 +667,12 @@ __global__ __launch_bounds__(NW * 64) void ggr_gemv_kernel(const void *__restric
 // ---------------------------------------------------------------------------
 static bool ggr_format(int quant) {
     return quant == OXQ_GGUF_Q4_0 || quant == OXQ_GGUF_Q8_0 || quant == OXQ_GGUF_Q4_K || quant == OXQ_GGUF_Q6_K ||
-           quant == OXQ_GGUF_Q4_1 || quant == OXQ_GGUF_Q5_0 || quant == OXQ_GGUF_Q5_1 || quant == OXQ_GGUF_Q5_K;
+           quant == OXQ_GGUF_Q4_1 || quant == OXQ_GGUF_Q5_0 || quant == OXQ_GGUF_Q5_1 || quant == OXQ_GGUF_Q5_K ||
+           quant == OXQ_GGUF_Q2_K || quant == OXQ_GGUF_Q3_K;
 }
 static int ggr_chunks_per_block(int quant) {
-    return (quant == OXQ_GGUF_Q4_K || quant == OXQ_GGUF_Q6_K || quant == OXQ_GGUF_Q5_K) ? 2 : 1;
+    return (quant == OXQ_GGUF_Q4_K || quant == OXQ_GGUF_Q6_K || quant == OXQ_GGUF_Q5_K || quant == OXQ_GGUF_Q2_K ||
+            quant == OXQ_GGUF_Q3_K) ? 2 : 1;
 }
 
 bool gguf_res_eligible(int quant, int64_t K, int64_t N) {
@@ -594,6 +685,7 @@ bool gguf_res_eligible(int quant, int64_t K, int64_t N) {
 size_t gguf_res_bytes(int quant, int64_t K, int64_t N) {
     int64_t be = 0, bb = 0;
     oxq_gguf_block_layout(quant, &be, &bb);
+    if (quant == OXQ_GGUF_Q3_K) bb += 2;  // the 16-byte header of the copy's super-block
     return (size_t)N * (size_t)(K / be) * (size_t)bb;
 }
 
@@ -619,6 +711,8 @@ static const char *ggr_name(int q) {
     case OXQ_GGUF_Q5_0: return "q5_0";
     case OXQ_GGUF_Q5_1: return "q5_1";
     case OXQ_GGUF_Q5_K: return "q5k";
+    case OXQ_GGUF_Q2_K: return "q2k";
+    case OXQ_GGUF_Q3_K: return "q3k";
     default: return "q6k";
     }
 }
@@ -641,6 +735,8 @@ int launch_gguf_res_repack(oxq_ctx *ctx, hipStream_t s, int quant, const uint8_t
         OXQ_GR(OXQ_GGUF_Q5_0);
         OXQ_GR(OXQ_GGUF_Q5_1);
         OXQ_GR(OXQ_GGUF_Q5_K);
+        OXQ_GR(OXQ_GGUF_Q2_K);
+        OXQ_GR(OXQ_GGUF_Q3_K);
     default: return fail(OXQ_ERR_UNSUPPORTED, "gguf repack: format %d has no resident layout", quant);
     }
 #undef OXQ_GR
@@ -666,6 +762,8 @@ int launch_gguf_res_dequant(oxq_ctx *ctx, hipStream_t s, int quant, const void *
         OXQ_GR(OXQ_GGUF_Q5_0);
         OXQ_GR(OXQ_GGUF_Q5_1);
         OXQ_GR(OXQ_GGUF_Q5_K);
+        OXQ_GR(OXQ_GGUF_Q2_K);
+        OXQ_GR(OXQ_GGUF_Q3_K);
     default: return fail(OXQ_ERR_UNSUPPORTED, "gguf dequant: format %d has no resident layout", quant);
     }
 #undef OXQ_GR
@@ -722,6 +820,8 @@ int launch_gguf_res_gemv(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p0) {
         case OXQ_GGUF_Q5_0: rc = nw == 8 ? ggr_by_rows<OXQ_GGUF_Q5_0, 8>(s, grid, p, lds, mb) : ggr_by_rows<OXQ_GGUF_Q5_0, 16>(s, grid, p, lds, mb); break;
         case OXQ_GGUF_Q5_1: rc = nw == 8 ? ggr_by_rows<OXQ_GGUF_Q5_1, 8>(s, grid, p, lds, mb) : ggr_by_rows<OXQ_GGUF_Q5_1, 16>(s, grid, p, lds, mb); break;
         case OXQ_GGUF_Q5_K: rc = nw == 8 ? ggr_by_rows<OXQ_GGUF_Q5_K, 8>(s, grid, p, lds, mb) : ggr_by_rows<OXQ_GGUF_Q5_K, 16>(s, grid, p, lds, mb); break;
+        case OXQ_GGUF_Q2_K: rc = nw == 8 ? ggr_by_rows<OXQ_GGUF_Q2_K, 8>(s, grid, p, lds, mb) : ggr_by_rows<OXQ_GGUF_Q2_K, 16>(s, grid, p, lds, mb); break;
+        case OXQ_GGUF_Q3_K: rc = nw == 8 ? ggr_by_rows<OXQ_GGUF_Q3_K, 8>(s, grid, p, lds, mb) : ggr_by_rows<OXQ_GGUF_Q3_K, 16>(s, grid, p, lds, mb); break;
         default: return fail(OXQ_ERR_UNSUPPORTED, "gguf resident gemv: format %d", p.quant);
         }
         if (rc != OXQ_OK) return rc;

@@ -412,11 +412,11 @@ def test_layers_validate_like_reference(lib, ctx):
     assert plan(lib, ctx).kernel.decode() == "gguf_q4k_res_dequant"
     assert lib.oxq_qlinear_dequantize(q, None, C.byref(fake((4096, 4095), F32))) == -3
     lib.oxq_qlinear_free(q)
-    # a format without a strip-major form keeps the file layout
-    w2k = fake((4096 * 16 * 84,), U8)
-    assert lib.oxq_qlinear_new(ctx, _lib.GGUF_Q2_K, C.byref(w2k), 4096, 4096, None, BF16, C.byref(q)) == 0
+    # a layer whose rows are not whole strips of 16 keeps the file layout
+    w2k = fake((4104 * 16 * 84,), U8)
+    assert lib.oxq_qlinear_new(ctx, _lib.GGUF_Q2_K, C.byref(w2k), 4096, 4104, None, BF16, C.byref(q)) == 0
     assert lib.oxq_qlinear_is_resident(q, C.byref(res)) == 0 and res.value == 0
-    assert lib.oxq_qlinear_forward(q, None, C.byref(fake((1, 4096), BF16)), C.byref(fake((1, 4096), BF16))) == 0
+    assert lib.oxq_qlinear_forward(q, None, C.byref(fake((1, 4096), BF16)), C.byref(fake((1, 4104), BF16))) == 0
     assert plan(lib, ctx).kernel.decode().startswith("gguf_q2k_gemv_bf16")
     lib.oxq_qlinear_free(q)
     assert lib.oxq_qlinear_new(ctx, _lib.GGUF_Q4_K, C.byref(w), 4096, 4095, None, BF16, C.byref(q)) == -3

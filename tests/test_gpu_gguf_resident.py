@@ -1,6 +1,6 @@
 """Resident GGUF layers (QLinear's strip-major copy of the block bytes) through the C ABI.
 
-oxq_qlinear_new repacks Q4_0 / Q4_1 / Q5_0 / Q5_1 / Q8_0 / Q4_K / Q5_K / Q6_K weights into strips of 16 rows at load
+oxq_qlinear_new repacks the weights of all ten block formats into strips of 16 rows at load
 (linear.rs:225-240 copies the bytes at build); 1 - 4 rows of x then run on that copy.  The repack is
 pinned bit for bit: the dense dequant read back from the copy must equal the oracle's dequantize_gguf
 of the file's bytes.  The GEMV on the copy is held to the f32-accumulated oracle within 2e-3 relative /
@@ -21,8 +21,8 @@ from tests.helpers import assert_close, bits_of, round_x, to_dev
 pytestmark = pytest.mark.gpu
 ops = None
 RES = [synth.GGUF_Q4_0, synth.GGUF_Q8_0, synth.GGUF_Q4_K, synth.GGUF_Q6_K,
-       synth.GGUF_Q4_1, synth.GGUF_Q5_0, synth.GGUF_Q5_1, synth.GGUF_Q5_K]
-KQ = (synth.GGUF_Q4_K, synth.GGUF_Q6_K, synth.GGUF_Q5_K)   # super-blocks of 256
+       synth.GGUF_Q4_1, synth.GGUF_Q5_0, synth.GGUF_Q5_1, synth.GGUF_Q5_K, synth.GGUF_Q2_K, synth.GGUF_Q3_K]
+KQ = (synth.GGUF_Q4_K, synth.GGUF_Q6_K, synth.GGUF_Q5_K, synth.GGUF_Q2_K, synth.GGUF_Q3_K)   # super-blocks of 256
 ROWS = 4   # rows of x one pass on the copy takes; f32 rows up to 8 (the reference's GEMV range) take two passes
 FMTS = [pytest.param(f, id=synth.GGUF_NAMES[f]) for f in RES]
 
@@ -125,7 +125,7 @@ def test_workgroups_that_walk_several_strips(cap, monkeypatch):
 def test_layers_outside_the_copys_reach_keep_the_file_layout(monkeypatch):
     say("resident gguf: ineligible layers")
     K, N = 512, 96
-    for fmt, n, k in [(synth.GGUF_Q2_K, N, K), (synth.GGUF_Q3_K, N, K), (synth.GGUF_Q4_0, 100, K),
+    for fmt, n, k in [(synth.GGUF_Q2_K, 104, K), (synth.GGUF_Q3_K, N, K), (synth.GGUF_Q4_0, 100, K),
                       (synth.GGUF_Q4_0, N, 416), (synth.GGUF_Q5_1, N, 96), (synth.GGUF_Q6_K, N, 768)]:
         data = synth.gguf_weight(fmt, n, k, seed=5)
         layer = ops.QLinear(fmt, to_dev(data), k, n, None, torch.float32)
