@@ -639,6 +639,13 @@ template <> struct Pk4N<F16Traits> {
         co = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, nz) + __builtin_bit_cast(h2, 0xD400D400u));
         sp = perm_b32(zw, zw, 0x03020302u);
     }
+    // the odd pairs' constant from the even pairs': -(1024 + z) + 960 (exact); for kernels short of registers
+    __device__ __forceinline__ void odd_from_even() {
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        uint32_t e = ce;
+        asm volatile("" : "+v"(e));
+        co = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, e) + __builtin_bit_cast(h2, 0x63806380u));
+    }
     __device__ __forceinline__ uint32_t deq(uint32_t p, int pp) const {
         return MfmaOps<F16Traits>::dequant_pair(p, (pp & 1) ? co : ce, sp);
     }
@@ -658,6 +665,7 @@ template <> struct Pk4N<BF16Traits> {
     }
     __device__ __forceinline__ uint32_t deq(uint32_t p, int) const { return Pk4T<BF16Traits>::deq(p, c0, c1); }
     __device__ __forceinline__ uint32_t minus_zero(uint32_t p, int) const { return p; }  // f16 only
+    __device__ __forceinline__ void odd_from_even() {}
 };
 
 template <typename TT>
@@ -685,11 +693,11 @@ __global__ __launch_bounds__(256) void pk4n_dequant_kernel(const uint32_t *__res
 
 // The waves' partial tiles meet in LDS as in the wide form; a thread then owns (row, column ni of every
 // strip of the workgroup) and adds the waves in order.
-template <typename TT, int MT, int NS>
+template <typename TT, int MT, int NS, int NW>
 __device__ __forceinline__ void pk4n_epilogue(const float4_t (&acc)[MT][NS], const uint16_t *__restrict__ bias,
                                               uint16_t *__restrict__ y, float *__restrict__ ws, int M, int N, int j,
                                               int m0, int wave, int lane) {
-    constexpr int NW = 8, NT = NW * 64, ROWS = 16 * MT;
+    constexpr int NT = NW * 64, ROWS = 16 * MT;
     extern __shared__ __attribute__((aligned(16))) unsigned char pk4_lds[];
     // every wave into its own activation slot (other waves may still be reading theirs): [MT][4 e][64 lanes][NS]
 #pragma unroll
@@ -732,8 +740,8 @@ __device__ __forceinline__ void pk4n_epilogue(const float4_t (&acc)[MT][NS], con
     }
 }
 
-template <typename TT, int MT, bool GS, int NS, int XQ>
-__global__ __launch_bounds__(512) void pk4n_mfma_kernel(const uint16_t *__restrict__ x,
+template <typename TT, int MT, bool GS, int NS, int XQ, int NW>
+__global__ __launch_bounds__(NW * 64) void pk4n_mfma_kernel(const uint16_t *__restrict__ x,
                                                         const uint32_t *__restrict__ pw,
                                                         const uint16_t *__restrict__ bias,
                                                         uint16_t *__restrict__ y, float *__restrict__ ws,
@@ -744,7 +752,7 @@ __global__ __launch_bounds__(512) void pk4n_mfma_kernel(const uint16_t *__restri
     // the conversion bias are taken off the weights instead - (bias + q) - (bias + z) is an exact packed
     // f16 add - and the block folds in with its scale alone.
     constexpr bool EXACT = GS && DUAL && NS == 1;
-    constexpr int NW = 8, ROWS = 16 * MT, AQ = XQ, SLOT = ROWS * 256, OOB = 0x7FFFFF00, BB = PK4N_BW * 4;
+    constexpr int ROWS = 16 * MT, AQ = XQ, SLOT = ROWS * 256, OOB = 0x7FFFFF00, BB = PK4N_BW * 4;
     constexpr int WNT = MT < 4 ? 2 : 0;
     extern __shared__ __attribute__((aligned(16))) unsigned char pk4_lds[];
 
@@ -791,8 +799,11 @@ __global__ __launch_bounds__(512) void pk4n_mfma_kernel(const uint16_t *__restri
     // wide form), a single strip two (its blocks are 1 KB; measured 4096 x 4096 / 4096 x 6144 / 8192 x 4096
     // at one row: one ahead 4.11 / 4.82 / 6.19 us, two 3.89 / 4.84 / 5.78, three 3.93 / 5.13 / 5.97)
     constexpr int RD = NS == 1 ? 3 : 2;
+    // The tile form turns a block's pairs into its constants at the block's start, so one set of pair
+    // registers serves every block; the folded forms need the pairs at the block's end and ring them too.
+    constexpr int ZD = (GS || EXACT) ? RD : 1;
     u32x4_t aring[AQ], wr[RD][NS];
-    uint32_t zr[RD][NS];
+    uint32_t zr[ZD][NS];
     auto load_a = [&](int i, u32x4_t (&a)[AQ]) {
         const __amdgpu_buffer_rsrc_t rs = i < nloc ? rs_x : rs_none;
         const int blk = cb0 + i;
@@ -808,13 +819,19 @@ __global__ __launch_bounds__(512) void pk4n_mfma_kernel(const uint16_t *__restri
             }
         }
     };
+    auto load_z = [&](int i, uint32_t (&z)[NS]) {
+        const __amdgpu_buffer_rsrc_t rs = i < nloc ? rs_w : rs_none;
+#pragma unroll
+        for (int f = 0; f < NS; ++f)
+            z[f] = __builtin_amdgcn_raw_buffer_load_b32(rs, voff_z, (f * NB + cb0 + i) * BB, WNT);
+    };
     auto load_w = [&](int i, u32x4_t (&w)[NS], uint32_t (&z)[NS]) {
         const __amdgpu_buffer_rsrc_t rs = i < nloc ? rs_w : rs_none;
 #pragma unroll
         for (int f = 0; f < NS; ++f) {
             const int so = (f * NB + cb0 + i) * BB;
             w[f] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff_w, so, WNT);
-            z[f] = __builtin_amdgcn_raw_buffer_load_b32(rs, voff_z, so, WNT);
+            if constexpr (ZD == RD) z[f] = __builtin_amdgcn_raw_buffer_load_b32(rs, voff_z, so, WNT);
         }
     };
     auto store_a = [&](const u32x4_t (&a)[AQ]) {
@@ -825,7 +842,8 @@ __global__ __launch_bounds__(512) void pk4n_mfma_kernel(const uint16_t *__restri
     u32x4_t afirst[AQ];
     load_a(0, afirst);
 #pragma unroll
-    for (int d = 0; d + 1 < RD; ++d) load_w(d, wr[d], zr[d]);
+    for (int d = 0; d + 1 < RD; ++d) load_w(d, wr[d], zr[d % ZD]);
+    if constexpr (ZD == 1) load_z(0, zr[0]);
     load_a(1, aring);
 
     float4_t acc[MT][NS];
@@ -843,13 +861,15 @@ __global__ __launch_bounds__(512) void pk4n_mfma_kernel(const uint16_t *__restri
     // one block: its weights are in ring half CUR; the next block is requested into the other half first
     auto block = [&](int i, auto cur_c) {
         constexpr int CUR = decltype(cur_c)::value, NXT = (CUR + RD - 1) % RD;
-        load_w(i + RD - 1, wr[NXT], zr[NXT]);
+        constexpr int ZC = CUR % ZD, ZN = NXT % ZD;
+        load_w(i + RD - 1, wr[NXT], zr[ZN]);
         float4_t tmp[GS ? MT : 1][NS], tmp1[GS ? MT : 1], tmpb[(GS && DUAL) ? MT : 1];
         Pk4N<TT> cst[(GS && !EXACT) ? 1 : NS];
         if (!GS || EXACT) {
 #pragma unroll
-            for (int f = 0; f < NS; ++f) cst[f].prep(zr[CUR][f]);
+            for (int f = 0; f < NS; ++f) cst[f].prep(zr[ZC][f]);
         }
+        if constexpr (ZD == 1) load_z(i + 1, zr[0]);
 #pragma unroll
         for (int st = 0; st < 4; ++st) {
             uint32_t a[MT][4];
@@ -864,6 +884,7 @@ __global__ __launch_bounds__(512) void pk4n_mfma_kernel(const uint16_t *__restri
             for (int f = 0; f < NS; ++f) {
                 const uint32_t w = wr[CUR][f][st];
                 uint32_t b[4];
+                if constexpr (!GS && MT == 4) cst[f].odd_from_even();
 #pragma unroll
                 for (int pp = 0; pp < 4; ++pp) {
                     const uint32_t pr = TT::unpack1(w, pp, nm);
@@ -887,7 +908,7 @@ __global__ __launch_bounds__(512) void pk4n_mfma_kernel(const uint16_t *__restri
         if (GS) {  // y += s * ((sum - biased row sum) - z * row sum), all f32
 #pragma unroll
             for (int f = 0; f < NS; ++f) {
-                const uint32_t zw = zr[CUR][f];
+                const uint32_t zw = zr[ZC][f];
                 const float sf = TT::to_f32((uint16_t)(zw >> 16));
                 const float nz = TT::to_f32((uint16_t)(zw & 0xFFFFu)) - (DUAL ? 0.0f : 128.0f);
 #pragma unroll
@@ -905,6 +926,10 @@ __global__ __launch_bounds__(512) void pk4n_mfma_kernel(const uint16_t *__restri
         }
         store_a(aring);
         load_a(i + 2, aring);
+        // the requests for the block after next stay here: sunk to their use in the next block (which the
+        // scheduler does in some single-tile instantiations to save registers) they would be waited for at
+        // once (bf16, 16 rows, 14336 x 4096: 13.0 -> 10.7 us).  The larger tiles schedule better without.
+        if constexpr (MT == 1) __builtin_amdgcn_sched_barrier(0);
     };
     {
         int i = 0;
@@ -926,7 +951,7 @@ __global__ __launch_bounds__(512) void pk4n_mfma_kernel(const uint16_t *__restri
         }
     }
 
-    pk4n_epilogue<TT, MT, NS>(acc, bias, y, ws, M, N, j, m0, wave, lane);
+    pk4n_epilogue<TT, MT, NS, NW>(acc, bias, y, ws, M, N, j, m0, wave, lane);
 }
 
 // ---------------------------------------------------------------------------
@@ -1066,28 +1091,34 @@ static int pk4_by_mt(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p
     }
 }
 
-// Strip width of a layer's resident copy: 16 columns for 4-bit layers with few 64-column strips and a
-// long K (the shapes that otherwise need K slices and a second launch), 64 otherwise.
+// Strip width of a layer's resident copy: 16 columns for 4-bit layers of at most 128 64-column strips and a
+// K of 32 - 112 blocks (the shapes that otherwise leave CUs idle or need K slices and a second launch),
+// 64 otherwise.
 int pk4_choose_strip(int64_t K, int64_t N, int bits, int64_t gate_half) {
-    // Measured (f16, one row of x; 64-column strips with K slices -> 16-column strips, one launch):
-    // 4096 x 4096 5.85 -> 3.74 us, 4096 x 6144 6.80 -> 4.69 us, 8192 x 4096 5.72 us; at 8 rows and more four
-    // strips share a workgroup and the layer runs within 3 % of the wide form.  A single strip does the
-    // per-block work on x (fragment reads, fold) for 1 KB of weights instead of 4 KB, so on long K it pays
-    // less: 11008 x 4096 7.16 / 7.92 us against 8.31 / 8.79 at 1 / 8 rows (9.61 against 9.29 at 16), but
-    // 14336 x 4096 8.58 us against 8.82 at one row and 2 - 3 % more from 8 rows on; that layer keeps the
-    // wide form.
+    // Measured (f16; 64-column strips, with K slices where few -> 16-column strips, one launch up to 8 rows),
+    // at 1 / 4 / 16 / 64 rows of x:
+    //    4096 x  4096   5.85 / -    / -     / -      ->  3.64 /  3.95 /  5.24 / 11.5 us
+    //    4096 x  8192   6.69 / 6.87 /  7.74 / 13.83  ->  5.01 /  5.53 /  8.29 / 14.13
+    //    8192 x  8192   9.99 / 10.1 / 10.98 / 19.86  ->  7.82 /  8.77 / 11.58 / 20.27
+    //   11008 x  4096   8.39 / 8.43 /  9.17 / 16.53  ->  5.94 /  6.62 /  9.44 / 16.86
+    //   14336 x  4096   8.92 / 9.12 / 10.06 / 18.20  ->  7.00 /  7.75 / 10.47 / 18.73
+    // one to eight rows gain 12 - 30 %, 16 rows and more lose 2 - 8 % (four strips share a workgroup there and
+    // a strip's 1 KB blocks cost more per-block work than the wide form's 4 KB).  Layers that fill the chip
+    // with 64-column strips gain nothing (4096 x 14336: 7.49 / 7.50 / 8.40 / 16.3 against 7.45 / 8.23 / 9.11 /
+    // 16.4; 5120 x 13824 and 8192 x 28672 alike), and on a very long K every strip's pass over x outweighs
+    // the saved launch from 4 rows on (28672 x 8192: 23.2 / 23.4 us wide, 21.3 / 26.6 narrow).
     const int mode = pk4_env("OXQ_PK4_STRIP16", 1);  // 0 never, 1 by shape, 2 wherever the layout applies
     if (!mode || bits != 4 || gate_half || N % 64 != 0) return 64;
     if (mode == 2) return 16;
-    return (N / 64 <= 96 && N / 16 >= 128 && K / 128 >= 32 && K / 128 <= 96) ? 16 : 64;
+    return (N / 64 <= 128 && N / 16 >= 128 && K / 128 >= 32 && K / 128 <= 112) ? 16 : 64;
 }
 
-template <typename TT, int MT, bool GS, int NS, int XQ>
+template <typename TT, int MT, bool GS, int NS, int XQ, int NW = 8>
 static int pk4n_go4(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, int bslice) {
-    const size_t lds = (size_t)8 * MT * 4096;
+    const size_t lds = (size_t)NW * MT * 4096;
     static LdsGrant lds_grant;  // one per instantiation
-    OXQ_HIP_CHECK(lds_grant.ensure((const void *)pk4n_mfma_kernel<TT, MT, GS, NS, XQ>, lds));
-    hipLaunchKernelGGL((pk4n_mfma_kernel<TT, MT, GS, NS, XQ>), grid, dim3(512), lds, s, (const uint16_t *)p.x, p.w.pw,
+    OXQ_HIP_CHECK(lds_grant.ensure((const void *)pk4n_mfma_kernel<TT, MT, GS, NS, XQ, NW>, lds));
+    hipLaunchKernelGGL((pk4n_mfma_kernel<TT, MT, GS, NS, XQ, NW>), grid, dim3(NW * 64), lds, s, (const uint16_t *)p.x, p.w.pw,
                        (const uint16_t *)p.bias, (uint16_t *)p.y, (float *)ctx->workspace, (int)p.M, (int)p.w.K,
                        (int)p.w.N, bslice);
     OXQ_HIP_CHECK(hipGetLastError());
@@ -1096,8 +1127,9 @@ static int pk4n_go4(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p,
 
 template <typename TT>
 static int pk4n_by_shape(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, int bslice, int mt, int ns,
-                         bool fold) {
+                         bool fold, bool w16) {
     if (ns == 1) {
+        if (w16) return pk4n_go4<TT, 1, true, 1, 1, 16>(ctx, s, grid, p, bslice);
         if (p.M <= 4) return pk4n_go4<TT, 1, true, 1, 1>(ctx, s, grid, p, bslice);
         if (p.M <= 8) return pk4n_go4<TT, 1, true, 1, 2>(ctx, s, grid, p, bslice);
         return pk4n_go4<TT, 1, true, 1, 4>(ctx, s, grid, p, bslice);
@@ -1143,10 +1175,14 @@ static int launch_pk4n_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p)
     if (p.act) return fail(OXQ_ERR_ARG, "repacked matmul: a fused activation on a layer in 16-column strips");
     const bool fold = mt <= 2 && pk4_folds(p, mt);  // three row tiles of folded sums do not fit beside the two-block ring
     dim3 grid((unsigned)(N / (16 * ns)), (unsigned)ks, (unsigned)ceil_div(M, 16 * mt));
+    // One or two rows of a single strip on a long K: 16 waves, so that a wave's chain of blocks is half as
+    // long (f16, one / two rows, 8 -> 16 waves: 14336 x 4096 7.44 / 7.55 -> 7.00 / 7.37 us, 8192 x 2048 at one
+    // row 4.75 -> 4.39; from three rows on, and at K = 4096, 8 waves are as fast or faster).
+    const bool w16 = ns == 1 && M <= 2 && pk4_env("OXQ_PK4N_W16", NB >= 64);
     char name[64];
     snprintf(name, sizeof name, "pk4_mfma_%s_mt%d%s_n16x%d", p.w.dtype == OXQ_F16 ? "f16" : "bf16", mt,
              (fold || ns == 1) ? "_gs" : "", ns);
-    set_plan(ctx, name, grid, dim3(512), ks, 1, ks > 1 ? (size_t)ks * M * N * 4 : 0);
+    set_plan(ctx, name, grid, dim3(w16 ? 1024 : 512), ks, 1, ks > 1 ? (size_t)ks * M * N * 4 : 0);
     if (ctx->plan_only) {
         if (ks > 1) add_launch(ctx);
         return OXQ_OK;
@@ -1155,8 +1191,8 @@ static int launch_pk4n_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p)
         return fail(OXQ_ERR_UNSUPPORTED, "repacked matmul: x larger than 2 GiB");
     if (((uintptr_t)p.x | (uintptr_t)p.y) & 15)
         return fail(OXQ_ERR_UNSUPPORTED, "repacked matmul: x and y must be 16-byte aligned");
-    const int rc = p.w.dtype == OXQ_F16 ? pk4n_by_shape<F16Traits>(ctx, s, grid, p, bslice, mt, ns, fold)
-                                        : pk4n_by_shape<BF16Traits>(ctx, s, grid, p, bslice, mt, ns, fold);
+    const int rc = p.w.dtype == OXQ_F16 ? pk4n_by_shape<F16Traits>(ctx, s, grid, p, bslice, mt, ns, fold, w16)
+                                        : pk4n_by_shape<BF16Traits>(ctx, s, grid, p, bslice, mt, ns, fold, w16);
     if (rc != OXQ_OK || ks == 1) return rc;
     return launch_splitk_reduce(ctx, s, (const float *)ctx->workspace, p.bias, p.y, M, N, ks, p.w.dtype);
 }

@@ -111,9 +111,10 @@ def test_narrow_layout_k_slices(ks, monkeypatch):
         assert_close(y, oracle.matmul_nt_f32(round_x(x, dt), wr, bias), f"narrow k-slices m{m}")
 
 
-@pytest.mark.parametrize("K,N", [(4096, 4096), (4096, 6144), (8192, 2048)])
-def test_attention_projection_shapes_take_the_narrow_layout(K, N, monkeypatch):
-    """By shape alone (no switch): one launch up to eight rows, the wide layout's answer within tolerance."""
+@pytest.mark.parametrize("K,N", [(4096, 4096), (4096, 6144), (8192, 2048), (14336, 4096), (4096, 8192)])
+def test_attention_and_down_projection_shapes_take_the_narrow_layout(K, N, monkeypatch):
+    """By shape alone (no switch): one launch up to eight rows (16 waves a workgroup for one or two rows on a
+    long K), the wide layout's answer within tolerance."""
     dt = oracle.F16
     trip, pack_dim = make("awq", K, N, 128, seed=N)
     layer = layer_of(trip, pack_dim, dt)
@@ -122,7 +123,7 @@ def test_attention_projection_shapes_take_the_narrow_layout(K, N, monkeypatch):
     monkeypatch.delenv("OXQ_PK4_STRIP16")
     w = dense("awq", trip, dt)
     np.testing.assert_array_equal(bits_of(layer.dequantize()), bits_of(wide.dequantize()))
-    for m in (1, 4, 8, 16, 64):
+    for m in (1, 2, 4, 8, 16, 64):
         say(f"narrow by shape K={K} N={N} m={m}")
         x = np.random.default_rng(m).standard_normal((m, K)).astype(np.float32)
         xd = to_dev(x, torch.float16)
@@ -131,6 +132,7 @@ def test_attention_projection_shapes_take_the_narrow_layout(K, N, monkeypatch):
         assert "_n16x" in plan["kernel"], plan
         if m <= 8:
             assert plan["launches"] == 1 and plan["split_k"] == 1 and plan["grid"][0] == N // 16, plan
+            assert plan["block"][0] == (1024 if m <= 2 and K >= 8192 else 512), plan
         yw = wide.forward(xd)
         assert "_n16x" not in kernel_of_last_call()["kernel"]
         wr = oracle.round_through(w, dt) if resident_rounds_weights(m, dt, False) else w
@@ -140,7 +142,7 @@ def test_attention_projection_shapes_take_the_narrow_layout(K, N, monkeypatch):
 
 
 def test_shapes_outside_the_rule_keep_the_wide_layout():
-    for K, N in [(14336, 4096), (4096, 1024), (4096, 14336), (2048, 4096)]:
+    for K, N in [(14464, 2048), (4096, 1024), (4096, 14336), (2048, 4096)]:
         trip, pack_dim = make("awq", K, N, 128, seed=1)
         layer = layer_of(trip, pack_dim, oracle.F16)
         layer.forward(torch.zeros((1, K), device="cuda", dtype=torch.float16))
