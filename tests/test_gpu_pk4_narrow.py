@@ -141,6 +141,30 @@ def test_attention_and_down_projection_shapes_take_the_narrow_layout(K, N, monke
         assert_close(yw, ref, f"wide twin m{m}")
 
 
+@pytest.mark.parametrize("kind", ["awq", "gptq"])
+@pytest.mark.parametrize("dtn", ["f16", "bf16"])
+def test_sixteen_wave_workgroups_on_a_long_k(kind, dtn):
+    """One or two rows on K >= 8192 run 16 waves a workgroup; 65 blocks leave them uneven shares (4 or 5)."""
+    dt = DT[dtn]
+    K, N, g = 8192 + 128, 2048, 128
+    trip, pack_dim = make(kind, K, N, g, seed=K)
+    bias = (np.arange(N, dtype=np.float32) % 11 - 5) * np.float32(0.25)
+    layer = layer_of(trip, pack_dim, dt, bias)
+    w = dense(kind, trip, dt)
+    np.testing.assert_array_equal(bits_of(layer.dequantize()), oracle.transpose_convert(w, dt))
+    rng = np.random.default_rng(K)
+    for m in (1, 2, 3):
+        say(f"narrow 16 waves {kind} {dtn} m={m}")
+        x = rng.standard_normal((m, K)).astype(np.float32)
+        xd = to_dev(x, TORCH_DT[dt])
+        y = layer.forward(xd)
+        plan = kernel_of_last_call()
+        assert plan["kernel"].endswith("_n16x1") and plan["launches"] == 1 and plan["grid"][0] == N // 16, plan
+        assert plan["block"][0] == (1024 if m <= 2 else 512), plan
+        assert_close(y, oracle.matmul_nt_f32(round_x(x, dt), w, bias), f"narrow 16 waves {kind} {dtn} m{m}")
+        np.testing.assert_array_equal(bits_of(layer.forward(xd)), bits_of(y))
+
+
 def test_shapes_outside_the_rule_keep_the_wide_layout():
     for K, N in [(14464, 2048), (4096, 1024), (4096, 14336), (2048, 4096)]:
         trip, pack_dim = make("awq", K, N, 128, seed=1)
