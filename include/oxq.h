@@ -418,8 +418,8 @@ int oxq_moe_combine(oxq_ctx *ctx, void *stream, const oxq_tensor *expert_out, co
  * with in_features and group size multiples of 128, out_features a multiple
  * of 64 and at most 128 groups it builds a tile-major copy of qweight/qzeros/scales in device memory owned by
  * the layer (same size as the checkpoint tensors, plus 1.5 bytes per column
- * and 128 rows; strips of 64 output columns, or of 16 for narrow 4-bit layers
- * such as attention projections) and forward never reads the caller's tensors again; it
+ * and 128 rows; strips of 64 output columns, or of 16 for 4-bit layers of at
+ * most 8192 columns and 4096 - 14336 rows, such as attention and down projections) and forward never reads the caller's tensors again; it
  * synchronises the null stream once.  Other layers keep descriptors of the
  * caller-owned tensors.  OXQ_PREPACK=0 in the environment disables the copy. */
 typedef struct oxq_packed_quant_linear oxq_packed_quant_linear;
