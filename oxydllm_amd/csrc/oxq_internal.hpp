@@ -170,6 +170,7 @@ struct Pk4Problem {
     int act;                // 0, or 1 + oxq_gated_act (gate|up layers only): y = act(gate) * up
     int no_split;           // the ctx workspace is taken (it holds the weights): one K slice only
     Pk4Weights w;
+    void *ws = nullptr;     // filled in by the launcher: the ctx workspace for K-slice partials
 };
 
 // ---- launchers (defined in the .hip files) ---------------------------------

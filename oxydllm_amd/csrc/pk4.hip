@@ -242,11 +242,11 @@ template <int MT, int BITS> struct Pk4Ring {
 
 // The 8 waves' partial 16*MT x 64 tiles meet in LDS and are added in wave order; then either the
 // fused gate|up activation, the K slice's f32 partial, or the result in the layer dtype.
-template <typename TT, int MT>
+template <typename TT, int MT, int NW = 8>
 __device__ __forceinline__ void pk4_epilogue(const float4_t (&acc)[MT][4], const uint16_t *__restrict__ bias,
                                              uint16_t *__restrict__ y, float *__restrict__ ws, int M, int N, int j,
                                              int m0, int act, int wave, int lane) {
-    constexpr int NW = 8, NT = NW * 64, ROWS = 16 * MT;
+    constexpr int NT = NW * 64, ROWS = 16 * MT;
     extern __shared__ __attribute__((aligned(16))) unsigned char pk4_lds[];
     // each wave into its own slot, float4 = the lane's four columns of one row
     float4_t *red = (float4_t *)pk4_lds;  // [NW][MT][4 rows-in-quad][64 lanes] of float4 (f = 0..3)
@@ -576,6 +576,140 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
     }
 
     pk4_epilogue<TT, MT>(acc, bias, y, ws, M, N, j, m0, act, wave, lane);
+}
+
+// ---------------------------------------------------------------------------
+// One row tile, a wave's whole share requested up front (folded form).
+//
+// With at most NBLK blocks a wave (K = 4096: 4) there is nothing to ring: every load of the wave - x, weights
+// and pairs of all its blocks - is issued before the first one is waited for, in the order of use, and the
+// blocks are then worked off as they arrive.  No loop, so no loop-carried ring registers for the compiler to
+// copy (a copy waits for the load behind it) and no request that can sink below a use.
+// ---------------------------------------------------------------------------
+template <typename TT, int BITS, int NBLK, int XQ, int NW>
+__global__ __launch_bounds__(NW * 64) void pk4_front_kernel(const uint16_t *__restrict__ x,
+                                                        const uint32_t *__restrict__ pw,
+                                                        const uint16_t *__restrict__ bias,
+                                                        uint16_t *__restrict__ y, float *__restrict__ ws,
+                                                        int M, int K, int N, int bslice, int act) {
+    typedef MfmaOps<TT> Ops;
+    constexpr int MT = 1, AQ = XQ, SLOT = 16 * 256, OOB = 0x7FFFFF00, WL = BITS / 4;
+    constexpr int BB = pk4_block_words(BITS) * 4;
+    extern __shared__ __attribute__((aligned(16))) unsigned char pk4_lds[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int ni = lane & 15, kb = lane >> 4;
+    const int j = blockIdx.x;
+    const int NB = K >> 7;
+    const int sb0 = blockIdx.y * bslice;
+    const int SB = min(NB, sb0 + bslice) - sb0;
+    const int cbase = SB / NW, crem = SB % NW;
+    const int nloc = cbase + (wave < crem ? 1 : 0);
+    const int cb0 = sb0 + wave * cbase + min(wave, crem);
+    unsigned char *slot = pk4_lds + wave * SLOT;
+
+    const __amdgpu_buffer_rsrc_t rs_w = make_rsrc(pw + (size_t)j * NB * (BB / 4), (uint32_t)NB * (uint32_t)BB);
+    const __amdgpu_buffer_rsrc_t rs_x = make_rsrc(x, (uint32_t)M * (uint32_t)K * 2u);
+    const __amdgpu_buffer_rsrc_t rs_none = make_rsrc(pw, 0u);
+    const int voff_w = lane * 16;
+    const int voff_z = 1024 * WL * 4 + (ni * 4 + kb) * 4;
+    int voff_a[AQ];
+#pragma unroll
+    for (int q = 0; q < AQ; ++q) {
+        const int r = 4 * q + kb;
+        voff_a[q] = r < M ? (r * K * 2 + ni * 16) : OOB;
+    }
+    int a_wr[4];
+#pragma unroll
+    for (int qq = 0; qq < 4; ++qq) a_wr[qq] = kb * 256 + (((ni ^ kb) ^ (qq << 2)) << 4);
+    int a_rd[4];
+#pragma unroll
+    for (int st = 0; st < 4; ++st) a_rd[st] = ni * 256 + (((8 * (st >> 1) + 2 * kb + (st & 1)) ^ ni) << 4);
+    const NibbleMasks nm = nibble_masks();
+
+    u32x4_t av[NBLK][AQ], wv[NBLK][4][WL];
+    uint32_t zv[NBLK];
+#pragma unroll
+    for (int b = 0; b < NBLK; ++b) {
+        const bool live = b < nloc;  // wave-uniform
+        const __amdgpu_buffer_rsrc_t rx = live ? rs_x : rs_none, rw = live ? rs_w : rs_none;
+        const int blk = cb0 + b;
+#pragma unroll
+        for (int q = 0; q < AQ; ++q) av[b][q] = __builtin_amdgcn_raw_buffer_load_b128(rx, voff_a[q], blk * 256, 0);
+#pragma unroll
+        for (int st = 0; st < 4; ++st)
+#pragma unroll
+            for (int h = 0; h < WL; ++h)
+                wv[b][st][h] = __builtin_amdgcn_raw_buffer_load_b128(rw, voff_w, blk * BB + (st * WL + h) * 1024, 2);
+        zv[b] = __builtin_amdgcn_raw_buffer_load_b32(rw, voff_z, blk * BB, 2);
+        __builtin_amdgcn_sched_barrier(0);  // blocks are requested in the order they are used
+    }
+    // rows no load covers: zero once
+#pragma unroll
+    for (int q = AQ; q < 4; ++q) {
+        const int row = 4 * q + kb;
+        *(u32x4_t *)(slot + row * 256 + ((ni ^ (row & 15)) << 4)) = u32x4_t{0u, 0u, 0u, 0u};
+    }
+    __builtin_amdgcn_sched_barrier(0);  // every request above, before anything below
+
+    float4_t acc[MT][4];
+#pragma unroll
+    for (int f = 0; f < 4; ++f) acc[0][f] = float4_t{0.f, 0.f, 0.f, 0.f};
+    const uint32_t ones[4] = {TT::ONES, TT::ONES, TT::ONES, TT::ONES};
+    const float4_t zero4 = float4_t{0.f, 0.f, 0.f, 0.f};
+
+#pragma unroll
+    for (int b = 0; b < NBLK; ++b) {
+        // No branch around a block past the wave's share (zeros times zeros): behind a branch the compiler
+        // sinks the block's requests to their use.
+        {
+#pragma unroll
+            for (int q = 0; q < AQ; ++q) *(u32x4_t *)(slot + q * 1024 + a_wr[q & 3]) = av[b][q];
+            float4_t tmp[4], tmps;
+#pragma unroll
+            for (int st = 0; st < 4; ++st) {
+                uint32_t wp[WL][4];
+#pragma unroll
+                for (int h = 0; h < WL; ++h) {
+                    const u32x4_t t = wv[b][st][h];
+                    wp[h][0] = t[0], wp[h][1] = t[1], wp[h][2] = t[2], wp[h][3] = t[3];
+                }
+                auto pair = [&](int pp, int f) -> uint32_t {
+                    if (BITS == 4) return TT::unpack1(wp[0][pp], f, nm);
+                    const uint32_t word = wp[(f >> 1) % WL][pp];
+                    return TT::unpack_bytes((f & 1) ? (word >> 8) : word);
+                };
+                uint32_t a[4];
+                {
+                    const u32x4_t t = *(const u32x4_t *)(slot + a_rd[st]);
+                    a[0] = t[0], a[1] = t[1], a[2] = t[2], a[3] = t[3];
+                }
+                const bool fresh = st == 0;
+#pragma unroll
+                for (int f = 0; f < 4; ++f) {
+                    uint32_t bq[4];
+#pragma unroll
+                    for (int pp = 0; pp < 4; ++pp) bq[pp] = pair(pp, f);
+                    tmp[f] = Ops::mfma(a, bq, fresh ? zero4 : tmp[f]);
+                }
+                tmps = Ops::mfma(a, ones, fresh ? zero4 : tmps);
+            }
+            // the pairs of the four columns: the four lane groups fetched one word each
+            const auto p16 = __builtin_amdgcn_permlane16_swap(zv[b], zv[b], false, false);
+            const uint32_t even = p16[0], odd = p16[1];
+            const auto pe = __builtin_amdgcn_permlane32_swap(even, even, false, false);
+            const auto po = __builtin_amdgcn_permlane32_swap(odd, odd, false, false);
+            const uint32_t zq[4] = {pe[0], po[0], pe[1], po[1]};
+#pragma unroll
+            for (int f = 0; f < 4; ++f) {
+                const float sf = TT::to_f32((uint16_t)(zq[f] >> 16));
+                const float nszb = sf * TT::to_f32((uint16_t)(zq[f] & 0xFFFFu));
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[0][f][e] = fmaf(sf, tmp[f][e], fmaf(nszb, tmps[e], acc[0][f][e]));
+            }
+        }
+    }
+    pk4_epilogue<TT, MT, NW>(acc, bias, y, ws, M, N, j, 0, act, wave, lane);
 }
 
 // ---------------------------------------------------------------------------
@@ -954,6 +1088,113 @@ __global__ __launch_bounds__(NW * 64) void pk4n_mfma_kernel(const uint16_t *__re
     pk4n_epilogue<TT, MT, NS, NW>(acc, bias, y, ws, M, N, j, m0, wave, lane);
 }
 
+// A single strip, up to 8 rows, a wave's whole share (at most NBLK blocks of 1 KB) requested up front: the
+// 16-column counterpart of pk4_front_kernel, 16 waves.
+template <typename TT, int NBLK, int XQ>
+__global__ __launch_bounds__(1024) void pk4n_front_kernel(const uint16_t *__restrict__ x,
+                                                          const uint32_t *__restrict__ pw,
+                                                          const uint16_t *__restrict__ bias,
+                                                          uint16_t *__restrict__ y, float *__restrict__ ws,
+                                                          int M, int K, int N, int bslice) {
+    typedef MfmaOps<TT> Ops;
+    constexpr bool DUAL = TT::DTYPE == F16Traits::DTYPE;  // f16: zero and bias come off the weights exactly
+    constexpr int NW = 16, MT = 1, AQ = XQ, SLOT = 16 * 256, OOB = 0x7FFFFF00, BB = PK4N_BW * 4;
+    extern __shared__ __attribute__((aligned(16))) unsigned char pk4_lds[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int ni = lane & 15, kb = lane >> 4;
+    const int j = blockIdx.x;
+    const int NB = K >> 7;
+    const int sb0 = blockIdx.y * bslice;
+    const int SB = min(NB, sb0 + bslice) - sb0;
+    const int cbase = SB / NW, crem = SB % NW;
+    const int nloc = cbase + (wave < crem ? 1 : 0);
+    const int cb0 = sb0 + wave * cbase + min(wave, crem);
+    unsigned char *slot = pk4_lds + wave * SLOT;
+
+    const __amdgpu_buffer_rsrc_t rs_w = make_rsrc(pw + (size_t)j * NB * PK4N_BW, (uint32_t)NB * (uint32_t)BB);
+    const __amdgpu_buffer_rsrc_t rs_x = make_rsrc(x, (uint32_t)M * (uint32_t)K * 2u);
+    const __amdgpu_buffer_rsrc_t rs_none = make_rsrc(pw, 0u);
+    const int voff_w = lane * 16, voff_z = 1024 + ni * 4;
+    int voff_a[AQ];
+#pragma unroll
+    for (int q = 0; q < AQ; ++q) {
+        const int r = 4 * q + kb;
+        voff_a[q] = r < M ? (r * K * 2 + ni * 16) : OOB;
+    }
+    int a_wr[4];
+#pragma unroll
+    for (int qq = 0; qq < 4; ++qq) a_wr[qq] = kb * 256 + (((ni ^ kb) ^ (qq << 2)) << 4);
+    int a_rd[4];
+#pragma unroll
+    for (int st = 0; st < 4; ++st) a_rd[st] = ni * 256 + (((8 * (st >> 1) + 2 * kb + (st & 1)) ^ ni) << 4);
+    const NibbleMasks nm = nibble_masks();
+
+    u32x4_t av[NBLK][AQ], wv[NBLK];
+    uint32_t zv[NBLK];
+#pragma unroll
+    for (int b = 0; b < NBLK; ++b) {
+        const bool live = b < nloc;  // wave-uniform
+        const __amdgpu_buffer_rsrc_t rx = live ? rs_x : rs_none, rw = live ? rs_w : rs_none;
+        const int blk = cb0 + b;
+#pragma unroll
+        for (int q = 0; q < AQ; ++q) av[b][q] = __builtin_amdgcn_raw_buffer_load_b128(rx, voff_a[q], blk * 256, 0);
+        wv[b] = __builtin_amdgcn_raw_buffer_load_b128(rw, voff_w, blk * BB, 2);
+        zv[b] = __builtin_amdgcn_raw_buffer_load_b32(rw, voff_z, blk * BB, 2);
+        __builtin_amdgcn_sched_barrier(0);  // blocks are requested in the order they are used
+    }
+#pragma unroll
+    for (int q = AQ; q < 4; ++q) {
+        const int row = 4 * q + kb;
+        *(u32x4_t *)(slot + row * 256 + ((ni ^ (row & 15)) << 4)) = u32x4_t{0u, 0u, 0u, 0u};
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    float4_t acc[MT][1];
+    acc[0][0] = float4_t{0.f, 0.f, 0.f, 0.f};
+    const uint32_t ones[4] = {TT::ONES, TT::ONES, TT::ONES, TT::ONES};
+    const float4_t zero4 = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int b = 0; b < NBLK; ++b) {
+        // no branch around a block past the wave's share (zeros times zeros): behind one the compiler sinks
+        // the block's requests to their use
+#pragma unroll
+        for (int q = 0; q < AQ; ++q) *(u32x4_t *)(slot + q * 1024 + a_wr[q & 3]) = av[b][q];
+        Pk4N<TT> cst;
+        if constexpr (DUAL) cst.prep(zv[b]);
+        float4_t tmp, tmp1;
+#pragma unroll
+        for (int st = 0; st < 4; ++st) {
+            uint32_t a[4];
+            {
+                const u32x4_t t = *(const u32x4_t *)(slot + a_rd[st]);
+                a[0] = t[0], a[1] = t[1], a[2] = t[2], a[3] = t[3];
+            }
+            const uint32_t w = wv[b][st];
+            uint32_t bq[4];
+#pragma unroll
+            for (int pp = 0; pp < 4; ++pp) {
+                const uint32_t pr = TT::unpack1(w, pp, nm);
+                bq[pp] = DUAL ? cst.minus_zero(pr, pp) : pr;
+            }
+            const bool fresh = st == 0;
+            tmp = Ops::mfma(a, bq, fresh ? zero4 : tmp);
+            if constexpr (!DUAL) tmp1 = Ops::mfma(a, ones, fresh ? zero4 : tmp1);
+        }
+        const uint32_t zw = zv[b];
+        const float sf = TT::to_f32((uint16_t)(zw >> 16));
+        if constexpr (DUAL) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[0][0][e] = fmaf(sf, tmp[e], acc[0][0][e]);
+        } else {
+            const float nz = TT::to_f32((uint16_t)(zw & 0xFFFFu)) - 128.0f;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[0][0][e] = fmaf(sf, fmaf(nz, tmp1[e], tmp[e]), acc[0][0][e]);
+        }
+    }
+    pk4n_epilogue<TT, MT, 1, NW>(acc, bias, y, ws, M, N, j, 0, wave, lane);
+}
+
 // ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
@@ -1039,8 +1280,32 @@ static int pk4_env(const char *name, int dflt) {
     return e ? atoi(e) : dflt;
 }
 
+template <typename TT, int BITS, int NBLK, int XQ, int NW>
+static int pk4_front_go(hipStream_t s, dim3 grid, const Pk4Problem &p, int bslice) {
+    const size_t lds = (size_t)NW * 4096;
+    static LdsGrant lds_grant;
+    OXQ_HIP_CHECK(lds_grant.ensure((const void *)pk4_front_kernel<TT, BITS, NBLK, XQ, NW>, lds));
+    hipLaunchKernelGGL((pk4_front_kernel<TT, BITS, NBLK, XQ, NW>), grid, dim3(NW * 64), lds, s, (const uint16_t *)p.x, p.w.pw,
+                       (const uint16_t *)p.bias, (uint16_t *)p.y, (float *)p.ws, (int)p.M, (int)p.w.K, (int)p.w.N,
+                       bslice, p.act);
+    OXQ_HIP_CHECK(hipGetLastError());
+    return OXQ_OK;
+}
+
 template <typename TT, int BITS, int MT, bool GS, int XQ>
-static int pk4_go4(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, int bslice) {
+static int pk4_go4(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, int bslice, bool front) {
+    if constexpr (MT == 1 && GS && BITS == 4) {
+        if (front) {
+            Pk4Problem q = p;
+            q.ws = ctx->workspace;
+            const int share = (bslice + 15) / 16;  // blocks a wave, 16 waves (the launcher's rule: pk4_front_ok)
+            if (share <= 1) return pk4_front_go<TT, BITS, 1, XQ, 16>(s, grid, q, bslice);
+            if constexpr (XQ <= 2)
+                if (share <= 2) return pk4_front_go<TT, BITS, 2, XQ, 16>(s, grid, q, bslice);
+            if constexpr (XQ == 1)
+                if (share <= 3) return pk4_front_go<TT, BITS, 3, XQ, 16>(s, grid, q, bslice);
+        }
+    }
     constexpr int WD = Pk4Ring<MT, BITS>::WD;
     const size_t lds = (size_t)8 * MT * 4096;
     static LdsGrant lds_grant;  // one per instantiation
@@ -1053,15 +1318,15 @@ static int pk4_go4(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, 
 }
 
 template <typename TT, int BITS, int MT, bool GS>
-static int pk4_go(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, int bslice) {
+static int pk4_go(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, int bslice, bool front) {
     // A single short tile: rows past M are known at launch, so the loads that would only fetch them
     // are left out (M = 1: 8.8 instead of 9.1 us on 4096 x 14336).
     if constexpr (MT == 1) {
         const int xq = pk4_env("OXQ_PK4_XQ", 1) ? (int)ceil_div(p.M, 4) : 4;
-        if (xq == 1) return pk4_go4<TT, BITS, MT, GS, 1>(ctx, s, grid, p, bslice);
-        if (xq == 2) return pk4_go4<TT, BITS, MT, GS, 2>(ctx, s, grid, p, bslice);
+        if (xq == 1) return pk4_go4<TT, BITS, MT, GS, 1>(ctx, s, grid, p, bslice, front);
+        if (xq == 2) return pk4_go4<TT, BITS, MT, GS, 2>(ctx, s, grid, p, bslice, front);
     }
-    return pk4_go4<TT, BITS, MT, GS, 4 * MT>(ctx, s, grid, p, bslice);
+    return pk4_go4<TT, BITS, MT, GS, 4 * MT>(ctx, s, grid, p, bslice, front);
 }
 
 // Which form multiplies.  The folded form (exact integers through the matrix cores, scale and
@@ -1081,13 +1346,13 @@ static bool pk4_folds(const Pk4Problem &p, int mt) {
 }
 
 template <typename TT, int BITS>
-static int pk4_by_mt(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, int bslice, int mt) {
+static int pk4_by_mt(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, int bslice, int mt, bool front) {
     const bool fold = pk4_folds(p, mt);
     switch (mt) {
-    case 1: return pk4_go<TT, BITS, 1, true>(ctx, s, grid, p, bslice);
-    case 2: return fold ? pk4_go<TT, BITS, 2, true>(ctx, s, grid, p, bslice) : pk4_go<TT, BITS, 2, false>(ctx, s, grid, p, bslice);
-    case 3: return fold ? pk4_go<TT, BITS, 3, true>(ctx, s, grid, p, bslice) : pk4_go<TT, BITS, 3, false>(ctx, s, grid, p, bslice);
-    default: return pk4_go<TT, BITS, 4, false>(ctx, s, grid, p, bslice);
+    case 1: return pk4_go<TT, BITS, 1, true>(ctx, s, grid, p, bslice, front);
+    case 2: return fold ? pk4_go<TT, BITS, 2, true>(ctx, s, grid, p, bslice, false) : pk4_go<TT, BITS, 2, false>(ctx, s, grid, p, bslice, false);
+    case 3: return fold ? pk4_go<TT, BITS, 3, true>(ctx, s, grid, p, bslice, false) : pk4_go<TT, BITS, 3, false>(ctx, s, grid, p, bslice, false);
+    default: return pk4_go<TT, BITS, 4, false>(ctx, s, grid, p, bslice, false);
     }
 }
 
@@ -1125,10 +1390,34 @@ static int pk4n_go4(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p,
     return OXQ_OK;
 }
 
+template <typename TT, int NBLK, int XQ>
+static int pk4n_front_go(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, int bslice) {
+    const size_t lds = (size_t)16 * 4096;
+    static LdsGrant lds_grant;
+    OXQ_HIP_CHECK(lds_grant.ensure((const void *)pk4n_front_kernel<TT, NBLK, XQ>, lds));
+    hipLaunchKernelGGL((pk4n_front_kernel<TT, NBLK, XQ>), grid, dim3(1024), lds, s, (const uint16_t *)p.x, p.w.pw,
+                       (const uint16_t *)p.bias, (uint16_t *)p.y, (float *)ctx->workspace, (int)p.M, (int)p.w.K,
+                       (int)p.w.N, bslice);
+    OXQ_HIP_CHECK(hipGetLastError());
+    return OXQ_OK;
+}
+
 template <typename TT>
 static int pk4n_by_shape(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, int bslice, int mt, int ns,
-                         bool fold, bool w16) {
+                         bool fold, bool w16, bool nfront) {
     if (ns == 1) {
+        const int share = (bslice + 15) / 16;
+        if (nfront && p.M <= 4 && share <= 8) {
+            switch (share) {
+            case 1: case 2: return pk4n_front_go<TT, 2, 1>(ctx, s, grid, p, bslice);
+            case 3: return pk4n_front_go<TT, 3, 1>(ctx, s, grid, p, bslice);
+            case 4: return pk4n_front_go<TT, 4, 1>(ctx, s, grid, p, bslice);
+            case 5: return pk4n_front_go<TT, 5, 1>(ctx, s, grid, p, bslice);
+            case 6: return pk4n_front_go<TT, 6, 1>(ctx, s, grid, p, bslice);
+            case 7: return pk4n_front_go<TT, 7, 1>(ctx, s, grid, p, bslice);
+            default: return pk4n_front_go<TT, 8, 1>(ctx, s, grid, p, bslice);
+            }
+        }
         if (w16) return pk4n_go4<TT, 1, true, 1, 1, 16>(ctx, s, grid, p, bslice);
         if (p.M <= 4) return pk4n_go4<TT, 1, true, 1, 1>(ctx, s, grid, p, bslice);
         if (p.M <= 8) return pk4n_go4<TT, 1, true, 1, 2>(ctx, s, grid, p, bslice);
@@ -1178,7 +1467,12 @@ static int launch_pk4n_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p)
     // One or two rows of a single strip on a long K: 16 waves, so that a wave's chain of blocks is half as
     // long (f16, one / two rows, 8 -> 16 waves: 14336 x 4096 7.44 / 7.55 -> 7.00 / 7.37 us, 8192 x 2048 at one
     // row 4.75 -> 4.39; from three rows on, and at K = 4096, 8 waves are as fast or faster).
-    const bool w16 = ns == 1 && M <= 2 && pk4_env("OXQ_PK4N_W16", NB >= 64);
+    // Up to four rows of a single strip whose K slice is at most 128 blocks: 16 waves that request their whole
+    // share (at most 8 blocks of 1 KB) before waiting for anything (pk4n_front_kernel).  Measured, f16, one /
+    // four rows, against the ring: 4096 x 4096 3.48 / 3.84 against 3.70 / 3.89 us, 8192 x 4096 4.78 / 5.38 against
+    // 5.02 / 5.40, 14336 x 4096 6.76 / 7.57 against 6.96 / 7.70, 8192 x 8192 7.24 / 8.22 against 7.80 / 8.73.
+    const bool nfront = ns == 1 && M <= 4 && ceil_div(bslice, 16) <= 8 && pk4_env("OXQ_PK4_FRONT", 1);
+    const bool w16 = nfront || (ns == 1 && M <= 2 && pk4_env("OXQ_PK4N_W16", NB >= 64));
     char name[64];
     snprintf(name, sizeof name, "pk4_mfma_%s_mt%d%s_n16x%d", p.w.dtype == OXQ_F16 ? "f16" : "bf16", mt,
              (fold || ns == 1) ? "_gs" : "", ns);
@@ -1191,8 +1485,8 @@ static int launch_pk4n_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p)
         return fail(OXQ_ERR_UNSUPPORTED, "repacked matmul: x larger than 2 GiB");
     if (((uintptr_t)p.x | (uintptr_t)p.y) & 15)
         return fail(OXQ_ERR_UNSUPPORTED, "repacked matmul: x and y must be 16-byte aligned");
-    const int rc = p.w.dtype == OXQ_F16 ? pk4n_by_shape<F16Traits>(ctx, s, grid, p, bslice, mt, ns, fold, w16)
-                                        : pk4n_by_shape<BF16Traits>(ctx, s, grid, p, bslice, mt, ns, fold, w16);
+    const int rc = p.w.dtype == OXQ_F16 ? pk4n_by_shape<F16Traits>(ctx, s, grid, p, bslice, mt, ns, fold, w16, nfront)
+                                        : pk4n_by_shape<BF16Traits>(ctx, s, grid, p, bslice, mt, ns, fold, w16, nfront);
     if (rc != OXQ_OK || ks == 1) return rc;
     return launch_splitk_reduce(ctx, s, (const float *)ctx->workspace, p.bias, p.y, M, N, ks, p.w.dtype);
 }
@@ -1228,9 +1522,22 @@ int launch_pk4_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p) {
     char name[64];
     if (p.act && (!p.w.gate_half || p.act > 2))
         return fail(OXQ_ERR_ARG, "repacked matmul: activation %d on a layer that is not a fused gate|up layer", p.act);
+    // A single row tile of a 4-bit layer with a short K slice: 16 waves, each requesting its whole share (one to
+    // three blocks) before it waits for anything (pk4_front_kernel).  Measured, f16, up-front against ring:
+    //   2048 x 16384 (1 block a wave)   1 / 4 / 16 rows      4.88 / 4.99 / 5.54   against  5.13 / 5.25 / 5.87 us
+    //   4096 x 14336 (2 blocks)         1 / 4 / 8 / 16 rows  6.88 / 7.10 / 7.42 / 8.34     7.49 / 7.54 / 7.72 / 8.40
+    //   5120 x 13824 (3 blocks)         1 / 4 / 8 / 16 rows  8.51 / 8.80 / 9.52 / 10.73    8.83 / 8.93 / 9.19 / 10.17
+    //   6144 x 16384 (3 blocks)         1 / 4 / 8 rows       10.23 / 10.42 / 10.56         10.45 / 10.58 / 10.95
+    // The more x a wave requests with its weights, and the more blocks, the less it gains: taken for one block at
+    // any row count, two blocks up to 8 rows, three up to 4.  8-bit layers have twice the bytes in flight and
+    // lose by it (5120 x 13824 at one row: 14.5 - 16.9 against 12.9 us): they keep the ring.
+    const int front_xq = pk4_env("OXQ_PK4_XQ", 1) ? (int)ceil_div(M, 4) : 4;
+    const int front_share = (bslice + 15) / 16;
+    const bool front = mt == 1 && p.w.bits == 4 && pk4_env("OXQ_PK4_FRONT", 1) &&
+                       (front_share <= 1 || (front_share == 2 && front_xq <= 2) || (front_share == 3 && front_xq == 1));
     snprintf(name, sizeof name, "pk%d_mfma_%s_mt%d%s%s", p.w.bits, p.w.dtype == OXQ_F16 ? "f16" : "bf16", mt,
              pk4_folds(p, mt) ? "_gs" : "", p.act == 1 ? "_silu" : p.act == 2 ? "_gelu" : "");
-    set_plan(ctx, name, grid, dim3(512), ks, 1, ks > 1 ? (size_t)ks * M * p.w.N * 4 : 0);
+    set_plan(ctx, name, grid, dim3(front ? 1024 : 512), ks, 1, ks > 1 ? (size_t)ks * M * p.w.N * 4 : 0);
     if (ctx->plan_only) {
         if (ks > 1) add_launch(ctx);
         return OXQ_OK;
@@ -1242,11 +1549,11 @@ int launch_pk4_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p) {
     const bool f16 = p.w.dtype == OXQ_F16;
     int rc;
     if (p.w.bits == 4)
-        rc = f16 ? pk4_by_mt<F16Traits, 4>(ctx, s, grid, p, bslice, mt)
-                 : pk4_by_mt<BF16Traits, 4>(ctx, s, grid, p, bslice, mt);
+        rc = f16 ? pk4_by_mt<F16Traits, 4>(ctx, s, grid, p, bslice, mt, front)
+                 : pk4_by_mt<BF16Traits, 4>(ctx, s, grid, p, bslice, mt, front);
     else
-        rc = f16 ? pk4_by_mt<F16Traits, 8>(ctx, s, grid, p, bslice, mt)
-                 : pk4_by_mt<BF16Traits, 8>(ctx, s, grid, p, bslice, mt);
+        rc = f16 ? pk4_by_mt<F16Traits, 8>(ctx, s, grid, p, bslice, mt, false)
+                 : pk4_by_mt<BF16Traits, 8>(ctx, s, grid, p, bslice, mt, false);
     if (rc != OXQ_OK || ks == 1) return rc;
     return launch_splitk_reduce(ctx, s, (const float *)ctx->workspace, p.bias, p.y, M, p.w.N, ks, p.w.dtype);
 }

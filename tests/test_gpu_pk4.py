@@ -129,6 +129,47 @@ def test_repacked_forward_all_m(kind, dtn, K, N, g):
             assert np.abs(as_f32(y) - ref).max() < 0.06 * np.abs(ref).max() + 1e-2
 
 
+def front_rule(K, ks, m):
+    """The launcher's rule for the kernel that requests a wave's whole share up front (16 waves)."""
+    bslice = -(-(K // 128) // ks)
+    share, xq = -(-bslice // 16), -(-m // 4)
+    return m <= 16 and (share <= 1 or (share == 2 and xq <= 2) or (share == 3 and xq == 1))
+
+
+@pytest.mark.parametrize("kind", ["awq", "gptq"])
+@pytest.mark.parametrize("dtn", ["f16", "bf16"])
+@pytest.mark.parametrize("K,N,g,ks", [(2048, 256, 128, 1), (4096 + 640, 128, 128, 1), (6144, 64, 128, 1),
+                                      (4096, 192, 256, 1), (128 * 21, 64, 128, 1), (4096, 128, 128, 3)])
+def test_whole_share_requested_up_front(kind, dtn, K, N, g, ks, monkeypatch):
+    """A single row tile of a 4-bit layer with at most three blocks a wave: 16 waves request everything first.
+    16, 37, 48, 32 and 21 blocks over 16 waves (even shares, 2 or 3, 3, 2, 1 or 2) and three K slices of 11;
+    against the oracle, against the ring kernel within the tolerance, run to run bitwise."""
+    monkeypatch.setenv("OXQ_PK4_STRIP16", "0")   # these small N would take the 16-column layout
+    monkeypatch.setenv("OXQ_PK4_KS", str(ks))    # and few strips would cut K by themselves
+    dt = DT[dtn]
+    trip, pack_dim = make(kind, K, N, g, seed=K + 3 * N)
+    bias = (np.arange(N, dtype=np.float32) % 9 - 4) * np.float32(0.25)
+    layer = layer_of(trip, pack_dim, dt, bias)
+    w = dense(kind, trip, dt)
+    rng = np.random.default_rng(K)
+    for m in (1, 2, 4, 5, 8, 9, 16):
+        say(f"pk4 up-front {kind} {dtn} K={K} N={N} ks={ks} m={m}")
+        x = rng.standard_normal((m, K)).astype(np.float32)
+        xd = to_dev(x, TORCH_DT[dt])
+        ref = oracle.matmul_nt_f32(round_x(x, dt), w, bias)
+        y = layer.forward(xd)
+        plan = ops.default_context().last_plan()
+        assert "_n16x" not in plan["kernel"] and plan["split_k"] == ks, plan
+        assert plan["block"][0] == (1024 if front_rule(K, ks, m) else 512), (plan, m)
+        assert_close(y, ref, f"pk4 up-front {kind} {dtn} m{m}")
+        np.testing.assert_array_equal(bits_of(layer.forward(xd)), bits_of(y))
+        monkeypatch.setenv("OXQ_PK4_FRONT", "0")
+        y0 = layer.forward(xd)
+        assert ops.default_context().last_plan()["block"][0] == 512
+        monkeypatch.delenv("OXQ_PK4_FRONT")
+        assert_close(y0, ref, f"pk4 ring {kind} {dtn} m{m}")
+
+
 @pytest.mark.parametrize("kind", KINDS)
 @pytest.mark.parametrize("dtn", ["f16", "bf16"])
 @pytest.mark.parametrize("K,N,g,ks", [(1280, 128, 128, 3), (2048, 64, 256, 2), (1152, 192, 128, 9), (512, 64, 128, 4)])
