@@ -373,6 +373,12 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
     // loads (cache policy bit 1), which a bare read of the same 30 MB also gains 7 % from.
     // From 49 rows on several row tiles may share a strip through L2, so those keep the default.
     constexpr int WNT = MT < 4 ? 2 : 0;
+    // Hand-placed memory operations (the three places marked PLACED below) instead of the compiler's own order,
+    // where that measured faster - same box, 48 / 64 / 128 rows: 8-bit f16 5120 x 13824 21.8 / 27.3 / 42.5 ->
+    // 20.6 / 24.3 / 41.0 us; 4-bit bf16 4096 x 14336 at 33 / 48 rows 16.4 / 16.7 -> 15.2 / 15.9 us.  The 4-bit f16
+    // kernels and bf16 at four row tiles are as fast or faster as the compiler orders them (f16 at 64 / 128
+    // rows 16.9 / 29.4 against 16.6 / 30.8; bf16 19.6 / 33.8 against 18.7 / 34.3).
+    constexpr bool PLACED = MT >= 3 && (BITS == 8 || (TT::DTYPE == BF16Traits::DTYPE && MT == 3));
     extern __shared__ __attribute__((aligned(16))) unsigned char pk4_lds[];
 
     const int lane = threadIdx.x & 63;
@@ -497,7 +503,27 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
 
     store_a(afirst);
 
-    for (int i = 0; i < nloc; ++i) {
+    // PLACED (1).  The counter a wave waits on counts its loads in issue order, and what the loop waits for at
+    // its top is the stricter of what its two entries require.  From three row tiles on the compiler requests
+    // the second x block before the first pairs and weights here, but after them inside the loop: coming from
+    // here the pairs have 4 younger loads, so the loop would wait with "at most 4 outstanding" - that is, for
+    // 12 of the 16 x loads it has just issued - in every iteration.  With block 0's pairs and weights
+    // complete before the loop, only the loop's own order counts.
+    if constexpr (PLACED) {
+        asm volatile("" ::"v"(zring));
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+#pragma unroll
+            for (int h = 0; h < WL; ++h) asm volatile("" ::"v"(wring[g][h]));
+    }
+    // Two blocks an iteration where placed by hand: the ring registers a block loads are copied to the ones
+    // the loop carries at the loop's end, which waits for those loads; twice as rarely this way.
+    constexpr int UF = PLACED ? 2 : 1;
+    for (int i0 = 0; i0 < nloc; i0 += UF)
+#pragma unroll
+    for (int u = 0; u < UF; ++u) {
+        const int i = i0 + u;
+        if (u > 0 && i >= nloc) break;
         float4_t tmp[GS ? MT : 1][4], tmps[GS ? MT : 1];  // per-block integer sums of the GS form
         if (!GS) {
             uint32_t zv[4];
@@ -554,6 +580,10 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
                     for (int mt = 0; mt < MT; ++mt) acc[mt][f] = Ops::mfma(a[mt], b, acc[mt][f]);
                 }
             }
+            // PLACED (2).  Vector-memory requests, LDS writes and MFMAs stay inside their step (vector and
+            // scalar arithmetic and LDS reads may move across): the ring refill above is then issued a block
+            // ahead of its use, as written, instead of at the block's end with the other three.
+            if constexpr (PLACED) __builtin_amdgcn_sched_barrier(0x106);
         }
         if (GS) {  // fold the block in: y += s * (sum - (bias + z) * rowsum), all f32
             uint32_t zv[4];
@@ -571,6 +601,10 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
             }
         }
         // the next block's activations replace this one's (same wave: LDS accesses stay in order)
+        // PLACED (3).  The x block stays in its registers until here: hoisted to the block's start (with all 16
+        // fragments of the current block held in registers instead), its reload comes late in the block and
+        // is waited for at the next block's start.
+        if constexpr (PLACED) __builtin_amdgcn_sched_barrier(0);
         store_a(aring);
         load_a(i + 2, aring);
     }
@@ -1418,6 +1452,18 @@ static int pk4n_by_shape(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Proble
             default: return pk4n_front_go<TT, 8, 1>(ctx, s, grid, p, bslice);
             }
         }
+        if (nfront && p.M > 8 && share <= 2) return pk4n_front_go<TT, 2, 4>(ctx, s, grid, p, bslice);
+        if (nfront && p.M <= 8 && share <= 8) {
+            switch (share) {
+            case 1: case 2: return pk4n_front_go<TT, 2, 2>(ctx, s, grid, p, bslice);
+            case 3: return pk4n_front_go<TT, 3, 2>(ctx, s, grid, p, bslice);
+            case 4: return pk4n_front_go<TT, 4, 2>(ctx, s, grid, p, bslice);
+            case 5: return pk4n_front_go<TT, 5, 2>(ctx, s, grid, p, bslice);
+            case 6: return pk4n_front_go<TT, 6, 2>(ctx, s, grid, p, bslice);
+            case 7: return pk4n_front_go<TT, 7, 2>(ctx, s, grid, p, bslice);
+            default: return pk4n_front_go<TT, 8, 2>(ctx, s, grid, p, bslice);
+            }
+        }
         if (w16) return pk4n_go4<TT, 1, true, 1, 1, 16>(ctx, s, grid, p, bslice);
         if (p.M <= 4) return pk4n_go4<TT, 1, true, 1, 1>(ctx, s, grid, p, bslice);
         if (p.M <= 8) return pk4n_go4<TT, 1, true, 1, 2>(ctx, s, grid, p, bslice);
@@ -1467,11 +1513,14 @@ static int launch_pk4n_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p)
     // One or two rows of a single strip on a long K: 16 waves, so that a wave's chain of blocks is half as
     // long (f16, one / two rows, 8 -> 16 waves: 14336 x 4096 7.44 / 7.55 -> 7.00 / 7.37 us, 8192 x 2048 at one
     // row 4.75 -> 4.39; from three rows on, and at K = 4096, 8 waves are as fast or faster).
-    // Up to four rows of a single strip whose K slice is at most 128 blocks: 16 waves that request their whole
-    // share (at most 8 blocks of 1 KB) before waiting for anything (pk4n_front_kernel).  Measured, f16, one /
-    // four rows, against the ring: 4096 x 4096 3.48 / 3.84 against 3.70 / 3.89 us, 8192 x 4096 4.78 / 5.38 against
-    // 5.02 / 5.40, 14336 x 4096 6.76 / 7.57 against 6.96 / 7.70, 8192 x 8192 7.24 / 8.22 against 7.80 / 8.73.
-    const bool nfront = ns == 1 && M <= 4 && ceil_div(bslice, 16) <= 8 && pk4_env("OXQ_PK4_FRONT", 1);
+    // Up to eight rows of a single strip whose K slice is at most 128 blocks: 16 waves that request their whole
+    // share (at most 8 blocks of 1 KB) before waiting for anything (pk4n_front_kernel).  Measured, f16, 1 / 4 /
+    // 8 rows, against the ring: 4096 x 4096 3.48 / 3.84 / 4.21 against 3.70 / 3.89 / 4.36 us, 8192 x 4096 4.78 /
+    // 5.38 / 6.21 against 5.02 / 5.40 / 6.44, 14336 x 4096 6.76 / 7.57 / 9.33 against 6.96 / 7.70 / 9.49,
+    // 4096 x 8192 4.72 / 5.26 / 6.10 against 5.02 / 5.53 / 6.56.  With at most two blocks a wave (K <= 4096) also
+    // the 9 - 16 rows that a single strip takes there: 4096 x 4096 at 9 / 16 rows 4.37 / 5.12 against 4.71 / 5.28.
+    const bool nfront = ns == 1 && ceil_div(bslice, 16) <= 8 && pk4_env("OXQ_PK4_FRONT", 1) &&
+                        (M <= 8 || (M <= 16 && ceil_div(bslice, 16) <= 2));
     const bool w16 = nfront || (ns == 1 && M <= 2 && pk4_env("OXQ_PK4N_W16", NB >= 64));
     char name[64];
     snprintf(name, sizeof name, "pk4_mfma_%s_mt%d%s_n16x%d", p.w.dtype == OXQ_F16 ? "f16" : "bf16", mt,

@@ -132,7 +132,7 @@ def test_attention_and_down_projection_shapes_take_the_narrow_layout(K, N, monke
         assert "_n16x" in plan["kernel"], plan
         if m <= 8:
             assert plan["launches"] == 1 and plan["split_k"] == 1 and plan["grid"][0] == N // 16, plan
-            assert plan["block"][0] == (1024 if m <= 4 else 512), plan   # up to 4 rows: 16 waves, all requests first
+            assert plan["block"][0] == 1024, plan   # up to 8 rows: 16 waves, all requests first
         yw = wide.forward(xd)
         assert "_n16x" not in kernel_of_last_call()["kernel"]
         wr = oracle.round_through(w, dt) if resident_rounds_weights(m, dt, False) else w
@@ -145,7 +145,7 @@ def test_attention_and_down_projection_shapes_take_the_narrow_layout(K, N, monke
 @pytest.mark.parametrize("dtn", ["f16", "bf16"])
 def test_sixteen_wave_workgroups_on_a_long_k(kind, dtn, monkeypatch):
     """One or two rows on K >= 8192 run 16 waves a workgroup; 65 blocks leave them uneven shares (4 or 5).
-    Up to 4 rows and 8 blocks a wave the waves request their whole share first (a kernel of its own); with
+    Up to 8 rows and 8 blocks a wave the waves request their whole share first (a kernel of its own); with
     that switched off the ring kernel takes the same calls."""
     dt = DT[dtn]
     K, N, g = 8192 + 128, 2048, 128
@@ -157,14 +157,14 @@ def test_sixteen_wave_workgroups_on_a_long_k(kind, dtn, monkeypatch):
     rng = np.random.default_rng(K)
     for front in (1, 0):
         monkeypatch.setenv("OXQ_PK4_FRONT", str(front))
-        for m in (1, 2, 3, 4, 5):
+        for m in (1, 2, 3, 4, 5, 8):
             say(f"narrow 16 waves {kind} {dtn} m={m} up-front={front}")
             x = rng.standard_normal((m, K)).astype(np.float32)
             xd = to_dev(x, TORCH_DT[dt])
             y = layer.forward(xd)
             plan = kernel_of_last_call()
             assert plan["kernel"].endswith("_n16x1") and plan["launches"] == 1 and plan["grid"][0] == N // 16, plan
-            assert plan["block"][0] == (1024 if m <= (4 if front else 2) else 512), plan
+            assert plan["block"][0] == (1024 if m <= (8 if front else 2) else 512), plan
             assert_close(y, oracle.matmul_nt_f32(round_x(x, dt), w, bias), f"narrow 16 waves {kind} {dtn} m{m}")
             np.testing.assert_array_equal(bits_of(layer.forward(xd)), bits_of(y))
 
