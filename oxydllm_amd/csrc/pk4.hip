@@ -17,6 +17,11 @@
 // 64-column strip streams it with 1 KB wave loads, splits K across its own 8
 // waves and reduces through LDS.  One launch, no workspace, no atomics.
 //
+// Kernels in this file: pk4_mfma_kernel (every row count; a wave rings one block of weights ahead),
+// pk4_front_kernel (one row tile of a 4-bit layer with a short K slice: 16 waves, each requesting its
+// whole share before it waits), pk4n_mfma_kernel / pk4n_front_kernel (the same pair for layers stored in
+// 16-column strips), the load-time repacks and the dense dequants that pin them.
+//
 // Layout (K % 128 == 0, N % 64 == 0, group size a multiple of 128).  A strip is a run of
 // K/128 self-contained blocks; a block covers 128 rows of K and holds its weights followed by the
 // zeros and scales that apply to them:
