@@ -360,7 +360,7 @@ __device__ __forceinline__ void pk4_epilogue(const float4_t (&acc)[MT][4], const
 
 // XQ: activation loads per block and lane that can hold rows below M (4 rows each); the
 // launcher passes 4 * MT, or fewer for a short single tile, whose other rows stay zero in LDS.
-template <typename TT, int BITS, int MT, bool GS, int WD, int XQ>
+template <typename TT, int BITS, int MT, bool GS, int WD, int XQ, bool PLZ = false>
 __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restrict__ x,
                                                        const uint32_t *__restrict__ pw,
                                                        const uint16_t *__restrict__ bias,
@@ -383,7 +383,11 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
     // 20.6 / 24.3 / 41.0 us; 4-bit bf16 4096 x 14336 at 33 / 48 rows 16.4 / 16.7 -> 15.2 / 15.9 us.  The 4-bit f16
     // kernels and bf16 at four row tiles are as fast or faster as the compiler orders them (f16 at 64 / 128
     // rows 16.9 / 29.4 against 16.6 / 30.8; bf16 19.6 / 33.8 against 18.7 / 34.3).
-    constexpr bool PLACED = MT >= 3 && (BITS == 8 || (TT::DTYPE == BF16Traits::DTYPE && MT == 3));
+    // PLZ: the 4-bit kernel at four row tiles when a strip has one row-tile workgroup and the tile is (nearly)
+    // full, 57 - 64 rows: placed it is 1.5 - 5 % faster there (same box, 64 rows: f16 16.48 -> 16.24, bf16 19.39 ->
+    // 18.43, 5120 x 13824 f16 20.3 -> 19.9 us), slower at 49 rows (f16 15.33 -> 15.71) and when two or more
+    // row-tile workgroups share a strip's weights through L2 (128 rows: f16 29.4 -> 30.8).
+    constexpr bool PLACED = PLZ || (MT >= 3 && (BITS == 8 || (TT::DTYPE == BF16Traits::DTYPE && MT == 3)));
     extern __shared__ __attribute__((aligned(16))) unsigned char pk4_lds[];
 
     const int lane = threadIdx.x & 63;
@@ -1347,6 +1351,18 @@ static int pk4_go4(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, 
     }
     constexpr int WD = Pk4Ring<MT, BITS>::WD;
     const size_t lds = (size_t)8 * MT * 4096;
+    if constexpr (MT == 4 && BITS == 4) {
+        if (grid.z == 1 && p.M > 56 && pk4_env("OXQ_PK4_PLACE64", 1)) {
+            static LdsGrant lds_grant_p;
+            OXQ_HIP_CHECK(lds_grant_p.ensure((const void *)pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ, true>, lds));
+            hipLaunchKernelGGL((pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ, true>), grid, dim3(512), lds, s,
+                               (const uint16_t *)p.x, p.w.pw, (const uint16_t *)p.bias, (uint16_t *)p.y,
+                               (float *)ctx->workspace, (int)p.M, (int)p.w.K, (int)p.w.N, bslice,
+                               pk4_env("OXQ_PK4_CONTIGUOUS", 1), p.act);
+            OXQ_HIP_CHECK(hipGetLastError());
+            return OXQ_OK;
+        }
+    }
     static LdsGrant lds_grant;  // one per instantiation
     OXQ_HIP_CHECK(lds_grant.ensure((const void *)pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ>, lds));
     hipLaunchKernelGGL((pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ>), grid, dim3(512), lds, s, (const uint16_t *)p.x,
