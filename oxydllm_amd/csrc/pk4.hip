@@ -629,7 +629,7 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
 // blocks are then worked off as they arrive.  No loop, so no loop-carried ring registers for the compiler to
 // copy (a copy waits for the load behind it) and no request that can sink below a use.
 // ---------------------------------------------------------------------------
-template <typename TT, int BITS, int NBLK, int XQ, int NW>
+template <typename TT, int BITS, int NBLK, int XQ, int NW, int WIN = NBLK>
 __global__ __launch_bounds__(NW * 64) void pk4_front_kernel(const uint16_t *__restrict__ x,
                                                         const uint32_t *__restrict__ pw,
                                                         const uint16_t *__restrict__ bias,
@@ -670,23 +670,24 @@ __global__ __launch_bounds__(NW * 64) void pk4_front_kernel(const uint16_t *__re
     for (int st = 0; st < 4; ++st) a_rd[st] = ni * 256 + (((8 * (st >> 1) + 2 * kb + (st & 1)) ^ ni) << 4);
     const NibbleMasks nm = nibble_masks();
 
-    u32x4_t av[NBLK][AQ], wv[NBLK][4][WL];
-    uint32_t zv[NBLK];
-#pragma unroll
-    for (int b = 0; b < NBLK; ++b) {
+    u32x4_t av[WIN][AQ], wv[WIN][4][WL];
+    uint32_t zv[WIN];
+    auto request = [&](int b, u32x4_t (&a)[AQ], u32x4_t (&w)[4][WL], uint32_t &z) {
         const bool live = b < nloc;  // wave-uniform
         const __amdgpu_buffer_rsrc_t rx = live ? rs_x : rs_none, rw = live ? rs_w : rs_none;
         const int blk = cb0 + b;
 #pragma unroll
-        for (int q = 0; q < AQ; ++q) av[b][q] = __builtin_amdgcn_raw_buffer_load_b128(rx, voff_a[q], blk * 256, 0);
+        for (int q = 0; q < AQ; ++q) a[q] = __builtin_amdgcn_raw_buffer_load_b128(rx, voff_a[q], blk * 256, 0);
 #pragma unroll
         for (int st = 0; st < 4; ++st)
 #pragma unroll
             for (int h = 0; h < WL; ++h)
-                wv[b][st][h] = __builtin_amdgcn_raw_buffer_load_b128(rw, voff_w, blk * BB + (st * WL + h) * 1024, 2);
-        zv[b] = __builtin_amdgcn_raw_buffer_load_b32(rw, voff_z, blk * BB, 2);
+                w[st][h] = __builtin_amdgcn_raw_buffer_load_b128(rw, voff_w, blk * BB + (st * WL + h) * 1024, 2);
+        z = __builtin_amdgcn_raw_buffer_load_b32(rw, voff_z, blk * BB, 2);
         __builtin_amdgcn_sched_barrier(0);  // blocks are requested in the order they are used
-    }
+    };
+#pragma unroll
+    for (int b = 0; b < WIN; ++b) request(b, av[b], wv[b], zv[b]);
     // rows no load covers: zero once
 #pragma unroll
     for (int q = AQ; q < 4; ++q) {
@@ -707,14 +708,14 @@ __global__ __launch_bounds__(NW * 64) void pk4_front_kernel(const uint16_t *__re
         // sinks the block's requests to their use.
         {
 #pragma unroll
-            for (int q = 0; q < AQ; ++q) *(u32x4_t *)(slot + q * 1024 + a_wr[q & 3]) = av[b][q];
+            for (int q = 0; q < AQ; ++q) *(u32x4_t *)(slot + q * 1024 + a_wr[q & 3]) = av[b % WIN][q];
             float4_t tmp[4], tmps;
 #pragma unroll
             for (int st = 0; st < 4; ++st) {
                 uint32_t wp[WL][4];
 #pragma unroll
                 for (int h = 0; h < WL; ++h) {
-                    const u32x4_t t = wv[b][st][h];
+                    const u32x4_t t = wv[b % WIN][st][h];
                     wp[h][0] = t[0], wp[h][1] = t[1], wp[h][2] = t[2], wp[h][3] = t[3];
                 }
                 auto pair = [&](int pp, int f) -> uint32_t {
@@ -738,7 +739,7 @@ __global__ __launch_bounds__(NW * 64) void pk4_front_kernel(const uint16_t *__re
                 tmps = Ops::mfma(a, ones, fresh ? zero4 : tmps);
             }
             // the pairs of the four columns: the four lane groups fetched one word each
-            const auto p16 = __builtin_amdgcn_permlane16_swap(zv[b], zv[b], false, false);
+            const auto p16 = __builtin_amdgcn_permlane16_swap(zv[b % WIN], zv[b % WIN], false, false);
             const uint32_t even = p16[0], odd = p16[1];
             const auto pe = __builtin_amdgcn_permlane32_swap(even, even, false, false);
             const auto po = __builtin_amdgcn_permlane32_swap(odd, odd, false, false);
@@ -750,6 +751,10 @@ __global__ __launch_bounds__(NW * 64) void pk4_front_kernel(const uint16_t *__re
 #pragma unroll
                 for (int e = 0; e < 4; ++e) acc[0][f][e] = fmaf(sf, tmp[f][e], fmaf(nszb, tmps[e], acc[0][f][e]));
             }
+        }
+        if constexpr (WIN < NBLK) {
+            // a window of WIN blocks in flight: the next one goes into the registers this block has left
+            if (b + WIN < NBLK) request(b + WIN, av[b % WIN], wv[b % WIN], zv[b % WIN]);
         }
     }
     pk4_epilogue<TT, MT, NW>(acc, bias, y, ws, M, N, j, 0, act, wave, lane);
@@ -1323,12 +1328,12 @@ static int pk4_env(const char *name, int dflt) {
     return e ? atoi(e) : dflt;
 }
 
-template <typename TT, int BITS, int NBLK, int XQ, int NW>
+template <typename TT, int BITS, int NBLK, int XQ, int NW, int WIN = NBLK>
 static int pk4_front_go(hipStream_t s, dim3 grid, const Pk4Problem &p, int bslice) {
     const size_t lds = (size_t)NW * 4096;
     static LdsGrant lds_grant;
-    OXQ_HIP_CHECK(lds_grant.ensure((const void *)pk4_front_kernel<TT, BITS, NBLK, XQ, NW>, lds));
-    hipLaunchKernelGGL((pk4_front_kernel<TT, BITS, NBLK, XQ, NW>), grid, dim3(NW * 64), lds, s, (const uint16_t *)p.x, p.w.pw,
+    OXQ_HIP_CHECK(lds_grant.ensure((const void *)pk4_front_kernel<TT, BITS, NBLK, XQ, NW, WIN>, lds));
+    hipLaunchKernelGGL((pk4_front_kernel<TT, BITS, NBLK, XQ, NW, WIN>), grid, dim3(NW * 64), lds, s, (const uint16_t *)p.x, p.w.pw,
                        (const uint16_t *)p.bias, (uint16_t *)p.y, (float *)p.ws, (int)p.M, (int)p.w.K, (int)p.w.N,
                        bslice, p.act);
     OXQ_HIP_CHECK(hipGetLastError());
@@ -1345,8 +1350,10 @@ static int pk4_go4(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, 
             if (share <= 1) return pk4_front_go<TT, BITS, 1, XQ, 16>(s, grid, q, bslice);
             if constexpr (XQ <= 2)
                 if (share <= 2) return pk4_front_go<TT, BITS, 2, XQ, 16>(s, grid, q, bslice);
-            if constexpr (XQ == 1)
+            if constexpr (XQ == 1) {
                 if (share <= 3) return pk4_front_go<TT, BITS, 3, XQ, 16>(s, grid, q, bslice);
+                if (share <= 4) return pk4_front_go<TT, BITS, 4, XQ, 16, 3>(s, grid, q, bslice);  // three in flight
+            }
         }
     }
     constexpr int WD = Pk4Ring<MT, BITS>::WD;
@@ -1599,12 +1606,18 @@ int launch_pk4_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p) {
     //   5120 x 13824 (3 blocks)         1 / 4 / 8 / 16 rows  8.51 / 8.80 / 9.52 / 10.73    8.83 / 8.93 / 9.19 / 10.17
     //   6144 x 16384 (3 blocks)         1 / 4 / 8 rows       10.23 / 10.42 / 10.56         10.45 / 10.58 / 10.95
     // The more x a wave requests with its weights, and the more blocks, the less it gains: taken for one block at
-    // any row count, two blocks up to 8 rows, three up to 4.  8-bit layers have twice the bytes in flight and
-    // lose by it (5120 x 13824 at one row: 14.5 - 16.9 against 12.9 us): they keep the ring.
+    // any row count, two blocks up to 8 rows, three up to 4.  Four blocks a wave (K = 8192), up to 4 rows, with a
+    // window of three blocks in flight - the fourth is requested into the first's registers once that is worked
+    // off, still in straight-line code: 8192 x 28672 at 1 / 4 rows 21.57 / 22.02 against 22.59 / 22.94 us (windows
+    // of two and four: 21.69, 21.68).  8-bit layers have twice the bytes in flight and lose by it (5120 x 13824
+    // at one row: 14.5 - 16.9 against 12.9 us); a window of one block with 8 waves gains 4 % there when the
+    // wave's share is exactly the kernel's block count and loses as much when a block of zeros is multiplied
+    // through (4096 x 14336: 12.1 against 11.8): they keep the ring.
     const int front_xq = pk4_env("OXQ_PK4_XQ", 1) ? (int)ceil_div(M, 4) : 4;
     const int front_share = (bslice + 15) / 16;
     const bool front = mt == 1 && p.w.bits == 4 && pk4_env("OXQ_PK4_FRONT", 1) &&
-                       (front_share <= 1 || (front_share == 2 && front_xq <= 2) || (front_share == 3 && front_xq == 1));
+                       (front_share <= 1 || (front_share == 2 && front_xq <= 2) ||
+                        ((front_share == 3 || front_share == 4) && front_xq == 1));
     snprintf(name, sizeof name, "pk%d_mfma_%s_mt%d%s%s", p.w.bits, p.w.dtype == OXQ_F16 ? "f16" : "bf16", mt,
              pk4_folds(p, mt) ? "_gs" : "", p.act == 1 ? "_silu" : p.act == 2 ? "_gelu" : "");
     set_plan(ctx, name, grid, dim3(front ? 1024 : 512), ks, 1, ks > 1 ? (size_t)ks * M * p.w.N * 4 : 0);

@@ -133,17 +133,20 @@ def front_rule(K, ks, m):
     """The launcher's rule for the kernel that requests a wave's whole share up front (16 waves)."""
     bslice = -(-(K // 128) // ks)
     share, xq = -(-bslice // 16), -(-m // 4)
-    return m <= 16 and (share <= 1 or (share == 2 and xq <= 2) or (share == 3 and xq == 1))
+    return m <= 16 and (share <= 1 or (share == 2 and xq <= 2) or (share in (3, 4) and xq == 1))
 
 
 @pytest.mark.parametrize("kind", ["awq", "gptq"])
 @pytest.mark.parametrize("dtn", ["f16", "bf16"])
 @pytest.mark.parametrize("K,N,g,ks", [(2048, 256, 128, 1), (4096 + 640, 128, 128, 1), (6144, 64, 128, 1),
-                                      (4096, 192, 256, 1), (128 * 21, 64, 128, 1), (4096, 128, 128, 3)])
+                                      (4096, 192, 256, 1), (128 * 21, 64, 128, 1), (4096, 128, 128, 3),
+                                      (8192, 64, 128, 1), (8192 - 384, 128, 128, 1)])
 def test_whole_share_requested_up_front(kind, dtn, K, N, g, ks, monkeypatch):
-    """A single row tile of a 4-bit layer with at most three blocks a wave: 16 waves request everything first.
-    16, 37, 48, 32 and 21 blocks over 16 waves (even shares, 2 or 3, 3, 2, 1 or 2) and three K slices of 11;
-    against the oracle, against the ring kernel within the tolerance, run to run bitwise."""
+    """A single row tile of a 4-bit layer with at most four blocks a wave: 16 waves request everything first
+    (four blocks: three, the fourth once the first is worked off).
+    16, 37, 48, 32 and 21 blocks over 16 waves (even shares, 2 or 3, 3, 2, 1 or 2), three K slices of 11,
+    64 blocks (4 each) and 61 (3 or 4); against the oracle, against the ring kernel within the tolerance,
+    run to run bitwise."""
     monkeypatch.setenv("OXQ_PK4_STRIP16", "0")   # these small N would take the 16-column layout
     monkeypatch.setenv("OXQ_PK4_KS", str(ks))    # and few strips would cut K by themselves
     dt = DT[dtn]
