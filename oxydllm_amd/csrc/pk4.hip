@@ -1341,18 +1341,35 @@ static int pk4_front_go(hipStream_t s, dim3 grid, const Pk4Problem &p, int bslic
 }
 
 template <typename TT, int BITS, int MT, bool GS, int XQ>
-static int pk4_go4(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, int bslice, bool front) {
-    if constexpr (MT == 1 && GS && BITS == 4) {
-        if (front) {
-            Pk4Problem q = p;
-            q.ws = ctx->workspace;
-            const int share = (bslice + 15) / 16;  // blocks a wave, 16 waves (the launcher's rule: pk4_front_ok)
-            if (share <= 1) return pk4_front_go<TT, BITS, 1, XQ, 16>(s, grid, q, bslice);
-            if constexpr (XQ <= 2)
-                if (share <= 2) return pk4_front_go<TT, BITS, 2, XQ, 16>(s, grid, q, bslice);
-            if constexpr (XQ == 1) {
-                if (share <= 3) return pk4_front_go<TT, BITS, 3, XQ, 16>(s, grid, q, bslice);
-                if (share <= 4) return pk4_front_go<TT, BITS, 4, XQ, 16, 3>(s, grid, q, bslice);  // three in flight
+static int pk4_go4(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, int bslice, int front) {
+    if constexpr (MT == 1 && GS) {
+        Pk4Problem q = p;
+        q.ws = ctx->workspace;
+        const int share8 = (bslice + 7) / 8;
+        if (front == 2) {  // 8 waves, one or two blocks in flight: the ring, unrolled
+            if constexpr (BITS == 4) {
+                // two blocks in flight pay on a long chain: from 5 blocks a wave on at up to 4 rows, from 7 at any
+                if constexpr (XQ == 1) {
+                    if (share8 == 5) return pk4_front_go<TT, BITS, 5, XQ, 8, 2>(s, grid, q, bslice);
+                    if (share8 == 6) return pk4_front_go<TT, BITS, 6, XQ, 8, 2>(s, grid, q, bslice);
+                }
+                if (share8 >= 7) return pk4_front_go<TT, BITS, 8, XQ, 8, 2>(s, grid, q, bslice);
+            }
+            switch (share8) {
+            case 1: return pk4_front_go<TT, BITS, 1, XQ, 8, 1>(s, grid, q, bslice);
+            case 2: return pk4_front_go<TT, BITS, 2, XQ, 8, 1>(s, grid, q, bslice);
+            case 3: return pk4_front_go<TT, BITS, 3, XQ, 8, 1>(s, grid, q, bslice);
+            case 4: return pk4_front_go<TT, BITS, 4, XQ, 8, 1>(s, grid, q, bslice);
+            case 5: return pk4_front_go<TT, BITS, 5, XQ, 8, 1>(s, grid, q, bslice);
+            case 6: return pk4_front_go<TT, BITS, 6, XQ, 8, 1>(s, grid, q, bslice);
+            default: return pk4_front_go<TT, BITS, 8, XQ, 8, 1>(s, grid, q, bslice);
+            }
+        }
+        if (front == 1) {  // 16 waves, two blocks each: all of it requested first (4-bit), one at a time (8-bit)
+            if constexpr (BITS == 4) {
+                if constexpr (XQ <= 2) return pk4_front_go<TT, BITS, 2, XQ, 16>(s, grid, q, bslice);
+            } else {
+                return pk4_front_go<TT, BITS, 2, XQ, 16, 1>(s, grid, q, bslice);
             }
         }
     }
@@ -1380,7 +1397,7 @@ static int pk4_go4(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, 
 }
 
 template <typename TT, int BITS, int MT, bool GS>
-static int pk4_go(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, int bslice, bool front) {
+static int pk4_go(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, int bslice, int front) {
     // A single short tile: rows past M are known at launch, so the loads that would only fetch them
     // are left out (M = 1: 8.8 instead of 9.1 us on 4096 x 14336).
     if constexpr (MT == 1) {
@@ -1408,13 +1425,13 @@ static bool pk4_folds(const Pk4Problem &p, int mt) {
 }
 
 template <typename TT, int BITS>
-static int pk4_by_mt(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, int bslice, int mt, bool front) {
+static int pk4_by_mt(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, int bslice, int mt, int front) {
     const bool fold = pk4_folds(p, mt);
     switch (mt) {
     case 1: return pk4_go<TT, BITS, 1, true>(ctx, s, grid, p, bslice, front);
-    case 2: return fold ? pk4_go<TT, BITS, 2, true>(ctx, s, grid, p, bslice, false) : pk4_go<TT, BITS, 2, false>(ctx, s, grid, p, bslice, false);
-    case 3: return fold ? pk4_go<TT, BITS, 3, true>(ctx, s, grid, p, bslice, false) : pk4_go<TT, BITS, 3, false>(ctx, s, grid, p, bslice, false);
-    default: return pk4_go<TT, BITS, 4, false>(ctx, s, grid, p, bslice, false);
+    case 2: return fold ? pk4_go<TT, BITS, 2, true>(ctx, s, grid, p, bslice, 0) : pk4_go<TT, BITS, 2, false>(ctx, s, grid, p, bslice, 0);
+    case 3: return fold ? pk4_go<TT, BITS, 3, true>(ctx, s, grid, p, bslice, 0) : pk4_go<TT, BITS, 3, false>(ctx, s, grid, p, bslice, 0);
+    default: return pk4_go<TT, BITS, 4, false>(ctx, s, grid, p, bslice, 0);
     }
 }
 
@@ -1599,28 +1616,42 @@ int launch_pk4_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p) {
     char name[64];
     if (p.act && (!p.w.gate_half || p.act > 2))
         return fail(OXQ_ERR_ARG, "repacked matmul: activation %d on a layer that is not a fused gate|up layer", p.act);
-    // A single row tile of a 4-bit layer with a short K slice: 16 waves, each requesting its whole share (one to
-    // three blocks) before it waits for anything (pk4_front_kernel).  Measured, f16, up-front against ring:
-    //   2048 x 16384 (1 block a wave)   1 / 4 / 16 rows      4.88 / 4.99 / 5.54   against  5.13 / 5.25 / 5.87 us
-    //   4096 x 14336 (2 blocks)         1 / 4 / 8 / 16 rows  6.88 / 7.10 / 7.42 / 8.34     7.49 / 7.54 / 7.72 / 8.40
-    //   5120 x 13824 (3 blocks)         1 / 4 / 8 / 16 rows  8.51 / 8.80 / 9.52 / 10.73    8.83 / 8.93 / 9.19 / 10.17
-    //   6144 x 16384 (3 blocks)         1 / 4 / 8 rows       10.23 / 10.42 / 10.56         10.45 / 10.58 / 10.95
-    // The more x a wave requests with its weights, and the more blocks, the less it gains: taken for one block at
-    // any row count, two blocks up to 8 rows, three up to 4.  Four blocks a wave (K = 8192), up to 4 rows, with a
-    // window of three blocks in flight - the fourth is requested into the first's registers once that is worked
-    // off, still in straight-line code: 8192 x 28672 at 1 / 4 rows 21.57 / 22.02 against 22.59 / 22.94 us (windows
-    // of two and four: 21.69, 21.68).  8-bit layers have twice the bytes in flight and lose by it (5120 x 13824
-    // at one row: 14.5 - 16.9 against 12.9 us); a window of one block with 8 waves gains 4 % there when the
-    // wave's share is exactly the kernel's block count and loses as much when a block of zeros is multiplied
-    // through (4096 x 14336: 12.1 against 11.8): they keep the ring.
+    // A single row tile (up to 16 rows) runs straight-line kernels (pk4_front_kernel) where one exists for the
+    // slice: no loop, so no loop-carried ring registers to copy (and wait for) at its end, and every request
+    // placed where the source puts it.  Which form, measured side by side on one box (f16, us; "ring" is
+    // pk4_mfma_kernel, "16w" 16 waves that request their whole share first, "8w1" / "8w2" 8 waves with one / two
+    // blocks in flight, the next requested into a block's registers when it is worked off):
+    //   4-bit          rows             ring                        16w                         8w1                         8w2
+    //   2048 x 16384   1 / 4 / 16       5.15 / 5.25 / 5.96          5.00 / 5.08 / 5.55          4.91 / 5.04 / 5.36          4.93 / 5.12 / 5.64
+    //   4096 x 14336   1 / 4 / 8 / 16   7.54 / 7.55 / 7.93 / 8.66   6.86 / 7.06 / 7.45 / 8.29   7.11 / 7.40 / 7.50 / 7.92   6.99 / 7.11 / 7.77 / 8.32
+    //   5120 x 13824   1 / 4 / 8 / 16   8.90 / 8.96 / 9.31 / 10.4   8.51 / 8.76 / - / -         8.35 / 8.43 / 8.72 / 9.84   7.93 / 8.26 / 8.79 / 10.2
+    //   6144 x 16384   1 / 4 / 8 / 16   10.5 / 10.6 / 11.0 / 12.3   10.2 / 10.3 / - / -         10.1 / 10.3 / 10.3 / 11.3   10.1 / 10.2 / 10.6 / 11.9
+    //   8192 x 28672   1 / 4 / 8 / 16   22.7 / 23.2 / 24.8 / 27.3   21.6 / 22.2 / - / -         22.4 / 23.0 / 23.9 / 25.7   21.1 / 21.5 / 22.4 / 25.4
+    //   8-bit                                                       (16 waves, one in flight)
+    //   4096 x 14336   1 / 4 / 16       11.8 / 12.2 / 13.1          10.75 / 11.00 / 11.70       11.14 / 11.49 / 12.19       10.99 / 11.34 / 12.33
+    //   5120 x 13824   1 / 4 / 16       12.96 / 13.3 / 15.0         -                           12.38 / 12.81 / 14.57       12.80 / 13.14 / 15.20
+    //   6144 x 16384   1 / 4 / 16       17.75 / 17.95 / 18.65       17.20 / 17.40 / 18.26       17.29 / 17.49 / 18.00       17.32 / 17.53 / 19.03
+    // (16 waves that request a whole 8-bit share first have twice the bytes in flight and lose: 5120 x 13824 at one
+    // row 14.5 - 16.9 us.)  A wave whose share is short of the kernel's block count multiplies a block of zeros
+    // through: 40 blocks over 16 waves (2 or 3 each) lose what 5 each over 8 waves do not.  The rule:
+    //   4-bit  32 blocks, up to 8 rows: 16w.  Otherwise 8 waves for up to 8 blocks a wave (K <= 8192 unsliced), two
+    //          in flight from 5 blocks a wave on at up to 4 rows and from 7 on at any, else one.
+    //   8-bit  32 blocks in a single slice: 16 waves, one block in flight.  Otherwise 8w1 where every wave's share is
+    //          whole and the kernel exists for it (1 - 6, 8).
     const int front_xq = pk4_env("OXQ_PK4_XQ", 1) ? (int)ceil_div(M, 4) : 4;
-    const int front_share = (bslice + 15) / 16;
-    const bool front = mt == 1 && p.w.bits == 4 && pk4_env("OXQ_PK4_FRONT", 1) &&
-                       (front_share <= 1 || (front_share == 2 && front_xq <= 2) ||
-                        ((front_share == 3 || front_share == 4) && front_xq == 1));
-    snprintf(name, sizeof name, "pk%d_mfma_%s_mt%d%s%s", p.w.bits, p.w.dtype == OXQ_F16 ? "f16" : "bf16", mt,
-             pk4_folds(p, mt) ? "_gs" : "", p.act == 1 ? "_silu" : p.act == 2 ? "_gelu" : "");
-    set_plan(ctx, name, grid, dim3(front ? 1024 : 512), ks, 1, ks > 1 ? (size_t)ks * M * p.w.N * 4 : 0);
+    const int front_mode = pk4_env("OXQ_PK4_FRONT", 1);  // 0: the ring kernel, 2: never 16 waves
+    const int share8 = (bslice + 7) / 8;
+    int front = 0;
+    if (mt == 1 && front_mode != 0) {
+        if (p.w.bits == 4)
+            front = (front_mode != 2 && bslice == 32 && front_xq <= 2) ? 1 : share8 <= 8 ? 2 : 0;
+        else
+            front = (front_mode != 2 && bslice == 32 && ks == 1) ? 1 : (bslice % 8 == 0 && share8 <= 8 && share8 != 7) ? 2 : 0;
+    }
+    snprintf(name, sizeof name, "pk%d_mfma_%s_mt%d%s%s%s", p.w.bits, p.w.dtype == OXQ_F16 ? "f16" : "bf16", mt,
+             pk4_folds(p, mt) ? "_gs" : "", front == 1 ? "_front" : front == 2 ? "_line" : "",
+             p.act == 1 ? "_silu" : p.act == 2 ? "_gelu" : "");
+    set_plan(ctx, name, grid, dim3(front == 1 ? 1024 : 512), ks, 1, ks > 1 ? (size_t)ks * M * p.w.N * 4 : 0);
     if (ctx->plan_only) {
         if (ks > 1) add_launch(ctx);
         return OXQ_OK;
@@ -1635,8 +1666,8 @@ int launch_pk4_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p) {
         rc = f16 ? pk4_by_mt<F16Traits, 4>(ctx, s, grid, p, bslice, mt, front)
                  : pk4_by_mt<BF16Traits, 4>(ctx, s, grid, p, bslice, mt, front);
     else
-        rc = f16 ? pk4_by_mt<F16Traits, 8>(ctx, s, grid, p, bslice, mt, false)
-                 : pk4_by_mt<BF16Traits, 8>(ctx, s, grid, p, bslice, mt, false);
+        rc = f16 ? pk4_by_mt<F16Traits, 8>(ctx, s, grid, p, bslice, mt, front)
+                 : pk4_by_mt<BF16Traits, 8>(ctx, s, grid, p, bslice, mt, front);
     if (rc != OXQ_OK || ks == 1) return rc;
     return launch_splitk_reduce(ctx, s, (const float *)ctx->workspace, p.bias, p.y, M, p.w.N, ks, p.w.dtype);
 }

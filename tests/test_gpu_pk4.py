@@ -129,24 +129,33 @@ def test_repacked_forward_all_m(kind, dtn, K, N, g):
             assert np.abs(as_f32(y) - ref).max() < 0.06 * np.abs(ref).max() + 1e-2
 
 
-def front_rule(K, ks, m):
-    """The launcher's rule for the kernel that requests a wave's whole share up front (16 waves)."""
+def front_rule(K, ks, m, bits=4):
+    """The launcher's rule for a single row tile: "front" = 16 waves (4-bit: the whole share of two blocks
+    requested up front, 8-bit: one block at a time), "line" = 8 waves, the ring as straight-line code (up to
+    8 blocks a wave), "" = the ring kernel."""
     bslice = -(-(K // 128) // ks)
-    share, xq = -(-bslice // 16), -(-m // 4)
-    return m <= 16 and (share <= 1 or (share == 2 and xq <= 2) or (share in (3, 4) and xq == 1))
+    share8, xq = -(-bslice // 8), -(-m // 4)
+    if m > 16:
+        return ""
+    if bits == 4:
+        return "front" if bslice == 32 and xq <= 2 else "line" if share8 <= 8 else ""
+    if bslice == 32 and ks == 1:
+        return "front"
+    return "line" if bslice % 8 == 0 and share8 in (1, 2, 3, 4, 5, 6, 8) else ""
 
 
 @pytest.mark.parametrize("kind", ["awq", "gptq"])
 @pytest.mark.parametrize("dtn", ["f16", "bf16"])
 @pytest.mark.parametrize("K,N,g,ks", [(2048, 256, 128, 1), (4096 + 640, 128, 128, 1), (6144, 64, 128, 1),
                                       (4096, 192, 256, 1), (128 * 21, 64, 128, 1), (4096, 128, 128, 3),
-                                      (8192, 64, 128, 1), (8192 - 384, 128, 128, 1)])
+                                      (8192, 64, 128, 1), (8192 - 384, 128, 128, 1), (5120, 128, 128, 1),
+                                      (7168, 64, 128, 1), (9216, 64, 128, 1), (1024, 128, 128, 1), (768, 64, 128, 1)])
 def test_whole_share_requested_up_front(kind, dtn, K, N, g, ks, monkeypatch):
-    """A single row tile of a 4-bit layer with at most four blocks a wave: 16 waves request everything first
-    (four blocks: three, the fourth once the first is worked off).
-    16, 37, 48, 32 and 21 blocks over 16 waves (even shares, 2 or 3, 3, 2, 1 or 2), three K slices of 11,
-    64 blocks (4 each) and 61 (3 or 4); against the oracle, against the ring kernel within the tolerance,
-    run to run bitwise."""
+    """A single row tile of a 4-bit layer runs straight-line kernels: 16 waves that request everything first
+    for 32 blocks and up to 8 rows, otherwise 8 waves with one or two blocks in flight for up to 8 blocks a wave.
+    16, 37, 48, 32 and 21 blocks (2, 4 or 5, 6, 4 or 2 each, 2 or 3), three K slices of 11, 64 blocks (8 each),
+    61 (7 or 8), 40 (5 each), 56 (7: the kernel for 8 with a block of zeros), 8 and 6 blocks (one or none) and
+    72 (9: the ring); against the oracle, against the ring kernel within the tolerance, run to run bitwise."""
     monkeypatch.setenv("OXQ_PK4_STRIP16", "0")   # these small N would take the 16-column layout
     monkeypatch.setenv("OXQ_PK4_KS", str(ks))    # and few strips would cut K by themselves
     dt = DT[dtn]
@@ -163,14 +172,54 @@ def test_whole_share_requested_up_front(kind, dtn, K, N, g, ks, monkeypatch):
         y = layer.forward(xd)
         plan = ops.default_context().last_plan()
         assert "_n16x" not in plan["kernel"] and plan["split_k"] == ks, plan
-        assert plan["block"][0] == (1024 if front_rule(K, ks, m) else 512), (plan, m)
+        form = front_rule(K, ks, m)
+        assert plan["block"][0] == (1024 if form == "front" else 512), (plan, m)
+        assert plan["kernel"].endswith("_gs" + ("_" + form if form else "")), (plan, m, form)
         assert_close(y, ref, f"pk4 up-front {kind} {dtn} m{m}")
         np.testing.assert_array_equal(bits_of(layer.forward(xd)), bits_of(y))
         monkeypatch.setenv("OXQ_PK4_FRONT", "0")
         y0 = layer.forward(xd)
-        assert ops.default_context().last_plan()["block"][0] == 512
+        plan = ops.default_context().last_plan()
+        assert plan["block"][0] == 512 and plan["kernel"].endswith("_gs"), plan
         monkeypatch.delenv("OXQ_PK4_FRONT")
         assert_close(y0, ref, f"pk4 ring {kind} {dtn} m{m}")
+
+
+@pytest.mark.parametrize("kind", ["awq8", "gptq8"])
+@pytest.mark.parametrize("dtn", ["f16", "bf16"])
+@pytest.mark.parametrize("K,N,g,ks", [(1024, 128, 128, 1), (2048, 64, 128, 1), (5120, 64, 128, 1), (8192, 64, 128, 1),
+                                      (4096, 128, 256, 2), (7168, 64, 128, 1), (4096 + 640, 64, 128, 1),
+                                      (9216, 64, 128, 1), (4096, 64, 128, 1), (8192, 128, 128, 2)])
+def test_eight_bit_single_row_tile_in_straight_line_code(kind, dtn, K, N, g, ks, monkeypatch):
+    """8-bit layers take the 8-wave straight-line kernel where every wave's share is whole and the kernel exists
+    for it (1 - 6 or 8 blocks): 8, 16, 40 and 64 blocks and two K slices of 16; 32 blocks in one slice run 16
+    waves; 56 (7 each), 37 (uneven) and 72 (9 each) keep the ring.  Against the oracle, run to run bitwise, and
+    the ring kernel on the same calls."""
+    monkeypatch.setenv("OXQ_PK4_KS", str(ks))
+    dt = DT[dtn]
+    trip, pack_dim = make(kind, K, N, g, seed=K + 5 * N)
+    bias = (np.arange(N, dtype=np.float32) % 9 - 4) * np.float32(0.25)
+    layer = layer_of(trip, pack_dim, dt, bias, bits=8)
+    w = dense(kind, trip, dt)
+    rng = np.random.default_rng(K + 1)
+    for m in (1, 3, 4, 7, 8, 12, 16):
+        say(f"pk8 straight-line {kind} {dtn} K={K} N={N} ks={ks} m={m}")
+        x = rng.standard_normal((m, K)).astype(np.float32)
+        xd = to_dev(x, TORCH_DT[dt])
+        ref = oracle.matmul_nt_f32(round_x(x, dt), w, bias)
+        y = layer.forward(xd)
+        plan = ops.default_context().last_plan()
+        form = front_rule(K, ks, m, bits=8)
+        assert plan["kernel"].startswith("pk8_mfma") and plan["split_k"] == ks, plan
+        assert plan["block"][0] == (1024 if form == "front" else 512), (plan, m)
+        assert plan["kernel"].endswith("_gs" + ("_" + form if form else "")), (plan, m, form)
+        assert_close(y, ref, f"pk8 straight-line {kind} {dtn} m{m}")
+        np.testing.assert_array_equal(bits_of(layer.forward(xd)), bits_of(y))
+        monkeypatch.setenv("OXQ_PK4_FRONT", "0")
+        y0 = layer.forward(xd)
+        assert ops.default_context().last_plan()["kernel"].endswith("_gs")
+        monkeypatch.delenv("OXQ_PK4_FRONT")
+        assert_close(y0, ref, f"pk8 ring {kind} {dtn} m{m}")
 
 
 @pytest.mark.parametrize("kind", KINDS)
