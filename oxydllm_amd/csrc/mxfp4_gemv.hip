@@ -259,7 +259,7 @@ __global__ __launch_bounds__(256) void mxfp4_mfma_kernel(
     const int32_t *__restrict__ token_ids, int M, int K, int N, int swiglu, float limit) {
     // [K/8 chunks][MTOK] x 16 B of tokens, then per wave the scale bytes of its 16*FR rows
     extern __shared__ __attribute__((aligned(16))) unsigned char mm_lds[];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int ni = lane & 15, kb = lane >> 4;
     const int e = blockIdx.y;
     int p0 = 0, p1 = M;
@@ -280,13 +280,15 @@ __global__ __launch_bounds__(256) void mxfp4_mfma_kernel(
     // (ni, kb) the block 16T + 4j + kb of row ni.
     const int lr = lane >> 2, lc = lane & 3;
     const int tr_src = (4 * ni + kb) * 4;  // byte index of the lane whose register this lane needs
-    const u32x4_t *wrow[FR];
+    // Buffer loads relative to the wave's first row: a tile past the row's end is requested from beyond the
+    // descriptor (zeros, no memory access), so that every request is unconditional - behind a condition the
+    // compiler joins the paths with and without new requests and waits as if there were none, i.e. for the
+    // tile just requested.
+    const __amdgpu_buffer_rsrc_t rs_w = make_rsrc((const u32x4_t *)blocks + ((size_t)e * N + (active ? n_base : 0)) * nb,
+                                                  active ? (uint32_t)nrows * (uint32_t)nb * 16u : 0u);
+    int wrow[FR];  // byte offset of the lane's row (clamped to the wave's last valid row)
 #pragma unroll
-    for (int f = 0; f < FR; ++f) {
-        const int n = n_base + 16 * f + lr;
-        const size_t row = (size_t)e * N + (n < N ? n : N - 1);
-        wrow[f] = (const u32x4_t *)blocks + row * nb;
-    }
+    for (int f = 0; f < FR; ++f) wrow[f] = min(16 * f + lr, max(nrows, 1) - 1) * nb * 16;
     const int a_tok = (ni & (MTOK - 1)) * 16;
     // token chunks in LDS: quarter sq (16 bytes of every token) of block b
     auto tok_chunk = [](int b, int sq) { return (b * 4 + sq) * (MTOK * 16); };
@@ -299,14 +301,13 @@ __global__ __launch_bounds__(256) void mxfp4_mfma_kernel(
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const int b = 16 * T + 4 * j + lc;
-                w[f][j] = wrow[f][b < nb ? b : nb - 1];
+                w[f][j] = __builtin_amdgcn_raw_buffer_load_b128(rs_w, T < NT ? wrow[f] + (b < nb ? b : nb - 1) * 16 : 0x7FFFFF00, 0, 0);
             }
     };
     // the first weight tiles do not depend on the tokens: they are requested before those are staged
     if (active) {
 #pragma unroll
-        for (int d = 0; d < D - 1; ++d)
-            if (d < NT) load_tile(d, wq[d]);
+        for (int d = 0; d < D - 1; ++d) load_tile(d, wq[d]);
     }
 
     // The wave's scale bytes (rows n_base .. n_base + nrows - 1 are contiguous, nb bytes each): one
@@ -333,8 +334,7 @@ __global__ __launch_bounds__(256) void mxfp4_mfma_kernel(
             __syncthreads();  // everyone is done with the previous tokens
             if (active) {
 #pragma unroll
-                for (int d = 0; d < D - 1; ++d)
-                    if (d < NT) load_tile(d, wq[d]);
+                for (int d = 0; d < D - 1; ++d) load_tile(d, wq[d]);
             }
         }
         for (int c = threadIdx.x; c < rows * cpr; c += 256) {
@@ -349,69 +349,69 @@ __global__ __launch_bounds__(256) void mxfp4_mfma_kernel(
         float4_t acc[FR];
 #pragma unroll
         for (int f = 0; f < FR; ++f) acc[f] = float4_t{0.f, 0.f, 0.f, 0.f};
-        for (int T0 = 0; T0 < NT; T0 += D) {
+        auto tile = [&](int T, int par) {
+            load_tile(T + D - 1, wq[(par + D - 1) % D]);  // past the end: zeros, no memory access
+            // Lane transposes and scale reads in batches of two blocks, activation reads in batches
+            // of one block: a wave waits for LDS six times a tile, not once per fragment.
+            const bool ragged = T == NT - 1 && (nb & 15);  // wave-uniform: only the last tile can be
 #pragma unroll
-            for (int par = 0; par < D; ++par) {
-                const int T = T0 + par;
-                if (T < NT) {  // block-uniform
-                    if (T + D - 1 < NT) load_tile(T + D - 1, wq[(par + D - 1) % D]);
-                    // Lane transposes and scale reads in batches of two blocks, activation reads in batches
-                    // of one block: a wave waits for LDS six times a tile, not once per fragment.
-                    const bool ragged = T == NT - 1 && (nb & 15);  // wave-uniform: only the last tile can be
+            for (int jh = 0; jh < 4; jh += 2) {
+                uint32_t wp[FR][2][4];
+                float scf[FR][2];
+                int bcl[2];
 #pragma unroll
-                    for (int jh = 0; jh < 4; jh += 2) {
-                        uint32_t wp[FR][2][4];
-                        float scf[FR][2];
-                        int bcl[2];
+                for (int jj = 0; jj < 2; ++jj) {
+                    const int b = 16 * T + 4 * (jh + jj) + kb;
+                    bcl[jj] = b < nb ? b : nb - 1;  // blocks past the row: a finite chunk, weights zeroed below
+                }
 #pragma unroll
-                        for (int jj = 0; jj < 2; ++jj) {
-                            const int b = 16 * T + 4 * (jh + jj) + kb;
-                            bcl[jj] = b < nb ? b : nb - 1;  // blocks past the row: a finite chunk, weights zeroed below
-                        }
+                for (int f = 0; f < FR; ++f)
+#pragma unroll
+                    for (int jj = 0; jj < 2; ++jj) {
+                        const u32x4_t t = wq[par][f][jh + jj];
+#pragma unroll
+                        for (int q = 0; q < 4; ++q)
+                            wp[f][jj][q] = (uint32_t)__builtin_amdgcn_ds_bpermute(tr_src, (int)t[q]);
+                        scf[f][jj] = e8m0_to_f32(sc_lds[sc_row[f] + bcl[jj]]);
+                    }
+                if (ragged) {
+#pragma unroll
+                    for (int jj = 0; jj < 2; ++jj) {
+                        const bool valid = 16 * T + 4 * (jh + jj) + kb < nb;
 #pragma unroll
                         for (int f = 0; f < FR; ++f)
 #pragma unroll
-                            for (int jj = 0; jj < 2; ++jj) {
-                                const u32x4_t t = wq[par][f][jh + jj];
+                            for (int q = 0; q < 4; ++q) wp[f][jj][q] = valid ? wp[f][jj][q] : 0u;
+                    }
+                }
 #pragma unroll
-                                for (int q = 0; q < 4; ++q)
-                                    wp[f][jj][q] = (uint32_t)__builtin_amdgcn_ds_bpermute(tr_src, (int)t[q]);
-                                scf[f][jj] = e8m0_to_f32(sc_lds[sc_row[f] + bcl[jj]]);
-                            }
-                        if (ragged) {
+                for (int jj = 0; jj < 2; ++jj) {
+                    u32x4_t av[4];
 #pragma unroll
-                            for (int jj = 0; jj < 2; ++jj) {
-                                const bool valid = 16 * T + 4 * (jh + jj) + kb < nb;
+                    for (int sq = 0; sq < 4; ++sq)
+                        av[sq] = *(const u32x4_t *)(mm_lds + tok_chunk(bcl[jj], sq) + a_tok);
 #pragma unroll
-                                for (int f = 0; f < FR; ++f)
+                    for (int sq = 0; sq < 4; ++sq) {
 #pragma unroll
-                                    for (int q = 0; q < 4; ++q) wp[f][jj][q] = valid ? wp[f][jj][q] : 0u;
-                            }
-                        }
-#pragma unroll
-                        for (int jj = 0; jj < 2; ++jj) {
-                            u32x4_t av[4];
-#pragma unroll
-                            for (int sq = 0; sq < 4; ++sq)
-                                av[sq] = *(const u32x4_t *)(mm_lds + tok_chunk(bcl[jj], sq) + a_tok);
-#pragma unroll
-                            for (int sq = 0; sq < 4; ++sq) {
-#pragma unroll
-                                for (int f = 0; f < FR; ++f) {
-                                    const uint32_t w = wp[f][jj][sq];
-                                    u32x4_t bv;
-                                    bv[0] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scf[f][jj], 0));
-                                    bv[1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scf[f][jj], 1));
-                                    bv[2] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scf[f][jj], 2));
-                                    bv[3] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scf[f][jj], 3));
-                                    acc[f] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av[sq]),
-                                                                                    __builtin_bit_cast(bf16x8_t, bv), acc[f], 0, 0, 0);
-                                }
-                            }
+                        for (int f = 0; f < FR; ++f) {
+                            const uint32_t w = wp[f][jj][sq];
+                            u32x4_t bv;
+                            bv[0] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scf[f][jj], 0));
+                            bv[1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scf[f][jj], 1));
+                            bv[2] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scf[f][jj], 2));
+                            bv[3] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scf[f][jj], 3));
+                            acc[f] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av[sq]),
+                                                                            __builtin_bit_cast(bf16x8_t, bv), acc[f], 0, 0, 0);
                         }
                     }
                 }
             }
+        };
+        // (as straight-line code for a known tile count this kernel is slower: 59.7 against 53.5 us a decode step)
+        for (int T0 = 0; T0 < NT; T0 += D) {
+#pragma unroll
+            for (int par = 0; par < D; ++par)
+                if (T0 + par < NT) tile(T0 + par, par);  // block-uniform
         }
         // D[m][n]: lane (n = ni, m = 4*kb + i): token 4*kb + i of weight row n_base + 16 f + ni
 #pragma unroll
@@ -517,7 +517,7 @@ __global__ __launch_bounds__(256) void mxfp4_res_dequant_kernel(const u32x4_t *_
 // tile: WR chunks in flight, one scale word per four chunks, four MFMA steps per chunk with the tokens
 // as the M tile.  Token chunks of one block lie 64 bytes further apart than they are long, which
 // spreads the four lane groups (four consecutive blocks) over all banks.
-template <int MTOK, int WR, int NWV>
+template <int MTOK, int WR, int NWV, int NCT>
 __global__ __launch_bounds__(NWV * 64) void mxfp4_res_kernel(const uint16_t *__restrict__ x,
                                                         const u32x4_t *__restrict__ pw,
                                                         const uint8_t *__restrict__ ps,
@@ -573,31 +573,45 @@ __global__ __launch_bounds__(NWV * 64) void mxfp4_res_kernel(const uint16_t *__r
         if (!active) continue;  // wave-uniform; the barriers above are reached by every wave
 
         float4_t acc = float4_t{0.f, 0.f, 0.f, 0.f};
-        for (int c0 = 0; c0 < NC; c0 += WR) {
+        auto chunk = [&](int c, int u, const u32x4_t w, const uint32_t sw) {
+            const float scale = e8m0_to_f32((sw >> (8 * (u & 3))) & 0xFFu);
+            const int b = min(4 * c + kb, nb - 1);  // blocks past the row: a finite chunk times zero weights
+            const unsigned char *xb = mr_lds + b * BSTR + a_tok;
+            const uint32_t w0 = w[0], w1 = w[1], w2 = w[2], w3 = w[3];
+            const uint32_t wq[4] = {w0, w1, w2, w3};
 #pragma unroll
-            for (int u = 0; u < WR; ++u) {
-                const int c = c0 + u;
-                const u32x4_t w = wring[u];
-                const uint32_t sw = sring[u >> 2];
-                wring[u] = load_w(c + WR);
-                if ((u & 3) == 3) sring[u >> 2] = load_s((c + WR) >> 2);
-                if (c < NC) {  // wave-uniform
-                    const float scale = e8m0_to_f32((sw >> (8 * (u & 3))) & 0xFFu);
-                    const int b = min(4 * c + kb, nb - 1);  // blocks past the row: a finite chunk times zero weights
-                    const unsigned char *xb = mr_lds + b * BSTR + a_tok;
-                    const uint32_t w0 = w[0], w1 = w[1], w2 = w[2], w3 = w[3];
-                    const uint32_t wq[4] = {w0, w1, w2, w3};
+            for (int sq = 0; sq < 4; ++sq) {
+                const u32x4_t av = *(const u32x4_t *)(xb + sq * (MTOK * 16));
+                u32x4_t bv;
+                bv[0] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(wq[sq], scale, 0));
+                bv[1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(wq[sq], scale, 1));
+                bv[2] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(wq[sq], scale, 2));
+                bv[3] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(wq[sq], scale, 3));
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av),
+                                                             __builtin_bit_cast(bf16x8_t, bv), acc, 0, 0, 0);
+            }
+        };
+        // A slot is requested again only after its last use, so that the new chunk can land in the same registers:
+        // requested before (while the old value is still live) it lands in others, and the copies into the loop's
+        // registers at the loop's end wait for every request just made - the ring drained once a round.
+        if constexpr (NCT > 0) {
+            // the chunk count is known: straight-line code, every request a value of its own
 #pragma unroll
-                    for (int sq = 0; sq < 4; ++sq) {
-                        const u32x4_t av = *(const u32x4_t *)(xb + sq * (MTOK * 16));
-                        u32x4_t bv;
-                        bv[0] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(wq[sq], scale, 0));
-                        bv[1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(wq[sq], scale, 1));
-                        bv[2] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(wq[sq], scale, 2));
-                        bv[3] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(wq[sq], scale, 3));
-                        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av),
-                                                                     __builtin_bit_cast(bf16x8_t, bv), acc, 0, 0, 0);
-                    }
+            for (int c = 0; c < NCT; ++c) {
+                const int u = c % WR;
+                chunk(c, u, wring[u], sring[u >> 2]);
+                if (c + WR < NCT) wring[u] = load_w(c + WR);
+                if ((u & 3) == 3 && c + WR - 3 < NCT) sring[u >> 2] = load_s((c + WR) >> 2);  // chunks c + WR - 3 .. c + WR
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        } else {
+            for (int c0 = 0; c0 < NC; c0 += WR) {
+#pragma unroll
+                for (int u = 0; u < WR; ++u) {
+                    const int c = c0 + u;
+                    if (c < NC) chunk(c, u, wring[u], sring[u >> 2]);  // wave-uniform
+                    wring[u] = load_w(c + WR);
+                    if ((u & 3) == 3) sring[u >> 2] = load_s((c + WR) >> 2);
                 }
             }
         }
@@ -665,13 +679,25 @@ int launch_mxfp4_res_dequant(oxq_ctx *ctx, hipStream_t s, const void *pw, const 
     return OXQ_OK;
 }
 
+template <int MTOK, int WR, int NWV, int NCT>
+static int mxfp4_res_go(hipStream_t s, dim3 grid, dim3 block, size_t lds, const Mxfp4Problem &p, int NC, int NG) {
+    static LdsGrant lds_grant;  // one per instantiation
+    OXQ_HIP_CHECK(lds_grant.ensure((const void *)mxfp4_res_kernel<MTOK, WR, NWV, NCT>, lds));
+    hipLaunchKernelGGL((mxfp4_res_kernel<MTOK, WR, NWV, NCT>), grid, block, lds, s, (const uint16_t *)p.x,
+                       (const u32x4_t *)p.blocks, p.scales, (const uint16_t *)p.bias, (uint16_t *)p.y, p.expert_offsets,
+                       p.token_ids, (int)p.K, (int)p.N, NC, NG, p.swiglu, p.swiglu_limit);
+    OXQ_HIP_CHECK(hipGetLastError());
+    return OXQ_OK;
+}
+
 // p.blocks / p.scales hold the resident copy; grouped form only
 int launch_mxfp4_res_gemv(oxq_ctx *ctx, hipStream_t s, const Mxfp4Problem &p) {
     const int nb = (int)(p.K / 32), NC = (int)ceil_div(nb, 4), NG = (int)ceil_div(NC, 4);
     constexpr int MTOK = 4;
     const size_t lds = (size_t)nb * (4 * MTOK * 16 + 64);
     // 8 chunks in flight per wave and 4 waves per workgroup measured best on 32 experts x (5760 + 2880) x 2880
-    // (47.5 us a decode step; 4 / 16 chunks: 49.5 / 58.7 us; 8 / 2 waves: 50.9 / 58.3 us)
+    // (44.7 us a decode step; 4 / 12 / 16 chunks: 45.8 / 48.7 / 51.6 us; 8 / 2 waves: 46.5 / 54.2 us).  The same
+    // step with the chunk loop kept as a loop: 45.6 us; with its slots requested before their last use: 47.7)
     constexpr int WR = 8, NWV = 4;
     dim3 grid((unsigned)ceil_div(p.N / 16, NWV), (unsigned)p.n_experts), block(NWV * 64);
     char name[64];
@@ -679,13 +705,13 @@ int launch_mxfp4_res_gemv(oxq_ctx *ctx, hipStream_t s, const Mxfp4Problem &p) {
     set_plan(ctx, name, grid, block, 1, 1, 0);
     if (ctx->plan_only) return OXQ_OK;
     if ((uintptr_t)p.x & 15) return fail(OXQ_ERR_UNSUPPORTED, "mxfp4 experts: x must be 16-byte aligned");
-    static LdsGrant lds_grant;
-    OXQ_HIP_CHECK(lds_grant.ensure((const void *)mxfp4_res_kernel<MTOK, WR, NWV>, lds));
-    hipLaunchKernelGGL((mxfp4_res_kernel<MTOK, WR, NWV>), grid, block, lds, s, (const uint16_t *)p.x,
-                       (const u32x4_t *)p.blocks, p.scales, (const uint16_t *)p.bias, (uint16_t *)p.y, p.expert_offsets,
-                       p.token_ids, (int)p.K, (int)p.N, NC, NG, p.swiglu, p.swiglu_limit);
-    OXQ_HIP_CHECK(hipGetLastError());
-    return OXQ_OK;
+    switch (NC) {  // K = 2048, 2880, 3072, 4096: the chunk loop as straight-line code
+    case 16: return mxfp4_res_go<MTOK, WR, NWV, 16>(s, grid, block, lds, p, NC, NG);
+    case 23: return mxfp4_res_go<MTOK, WR, NWV, 23>(s, grid, block, lds, p, NC, NG);
+    case 24: return mxfp4_res_go<MTOK, WR, NWV, 24>(s, grid, block, lds, p, NC, NG);
+    case 32: return mxfp4_res_go<MTOK, WR, NWV, 32>(s, grid, block, lds, p, NC, NG);
+    default: return mxfp4_res_go<MTOK, WR, NWV, 0>(s, grid, block, lds, p, NC, NG);
+    }
 }
 
 template <int MB, int RW>

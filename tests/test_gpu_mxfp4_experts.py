@@ -68,6 +68,14 @@ def test_experts_dequantize_is_bit_exact(E, N, K):
     (5, 80, 160, [0, 0, 5, 9, 1]),        # more pairs than one pass of 4 takes
     (2, 64, 2880, [2, 3]),
     (6, 128, 512, [0, 0, 0, 0, 0, 1]),
+    # chunk counts with a straight-line kernel of their own (16, 23, 24, 32 chunks of four blocks), a ragged
+    # last chunk beside them (2848 = 89 blocks) and the looping kernel on either side (22 and 25 chunks)
+    (2, 32, 2048, [1, 5]),
+    (2, 48, 3072, [3, 2]),
+    (1, 32, 4096, [6]),
+    (2, 32, 2848, [4, 1]),
+    (2, 32, 2816, [1, 2]),
+    (2, 32, 3200, [2, 4]),
 ])
 @pytest.mark.parametrize("gather", [True, False])
 def test_experts_matmul_matches_oracle_and_the_stateless_op(E, N, K, counts, gather):
