@@ -360,7 +360,8 @@ __device__ __forceinline__ void pk4_epilogue(const float4_t (&acc)[MT][4], const
 
 // XQ: activation loads per block and lane that can hold rows below M (4 rows each); the
 // launcher passes 4 * MT, or fewer for a short single tile, whose other rows stay zero in LDS.
-template <typename TT, int BITS, int MT, bool GS, int WD, int XQ, bool PLZ = false>
+// NBLK > 0: every wave has exactly NBLK blocks and the block loop is straight-line code.
+template <typename TT, int BITS, int MT, bool GS, int WD, int XQ, bool PLZ = false, int NBLK = 0>
 __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restrict__ x,
                                                        const uint32_t *__restrict__ pw,
                                                        const uint16_t *__restrict__ bias,
@@ -527,8 +528,11 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
     }
     // Two blocks an iteration where placed by hand: the ring registers a block loads are copied to the ones
     // the loop carries at the loop's end, which waits for those loads; twice as rarely this way.
-    constexpr int UF = PLACED ? 2 : 1;
-    for (int i0 = 0; i0 < nloc; i0 += UF)
+    // With the block count known (NBLK) there is no loop at all (figures where it is launched).
+    constexpr int UF = NBLK > 0 ? 1 : PLACED ? 2 : 1;
+    const int trip = NBLK > 0 ? NBLK : nloc;
+#pragma unroll(NBLK > 0 ? NBLK : 1)
+    for (int i0 = 0; i0 < trip; i0 += UF)
 #pragma unroll
     for (int u = 0; u < UF; ++u) {
         const int i = i0 + u;
@@ -546,7 +550,6 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
             u32x4_t wv[WL];
 #pragma unroll
             for (int h = 0; h < WL; ++h) wv[h] = wring[st][h];
-            load_w(i + 1, st, wring[st]);  // refill this ring slot
             uint32_t wp[WL][4];
 #pragma unroll
             for (int h = 0; h < WL; ++h) {
@@ -592,6 +595,10 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
             // PLACED (2).  Vector-memory requests, LDS writes and MFMAs stay inside their step (vector and
             // scalar arithmetic and LDS reads may move across): the ring refill above is then issued a block
             // ahead of its use, as written, instead of at the block's end with the other three.
+            // Refill this ring slot after its last use, so that the new block can land in the same registers
+            // (requested while the old value is live it lands in others, copied at the loop's end behind a wait
+            // for the request): 17 / 33 / 48 rows f16 9.96 / 12.76 / 13.57 -> 9.85 / 12.57 / 13.44 us.
+            load_w(i + 1, st, wring[st]);
             if constexpr (PLACED) __builtin_amdgcn_sched_barrier(0x106);
         }
         if (GS) {  // fold the block in: y += s * (sum - (bias + z) * rowsum), all f32
@@ -1375,6 +1382,31 @@ static int pk4_go4(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, 
     }
     constexpr int WD = Pk4Ring<MT, BITS>::WD;
     const size_t lds = (size_t)8 * MT * 4096;
+    if constexpr (MT >= 3) {
+        // Four or five blocks a wave (K = 4096, 5120 unsliced) and one row-tile workgroup a strip: the block loop as
+        // straight-line code.  Same box, loop -> straight line, 48 / 64 rows: 4-bit f16 4096 x 14336 13.66 / 16.40 ->
+        // 13.06 / 16.29 us, bf16 15.74 / 18.70 -> 15.23 / 17.91; 5120 x 13824 f16 16.6 / 20.39 -> 16.05 / 20.1, bf16
+        // 18.9 / 22.12 -> 18.16 / 21.82; 8-bit f16 4096 x 14336 17.09 / 20.4 -> 16.65 / 19.85.  (Two row tiles lose by
+        // it: 4-bit f16 at 17 / 32 rows 9.86 / 11.07 -> 12.15 / 13.12.)
+        if (grid.z == 1 && (bslice == 32 || bslice == 40) && pk4_env("OXQ_PK4_FRONT", 1)) {
+            static LdsGrant lg4, lg5;
+            if (bslice == 32) {
+                OXQ_HIP_CHECK(lg4.ensure((const void *)pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ, false, 4>, lds));
+                hipLaunchKernelGGL((pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ, false, 4>), grid, dim3(512), lds, s,
+                                   (const uint16_t *)p.x, p.w.pw, (const uint16_t *)p.bias, (uint16_t *)p.y,
+                                   (float *)ctx->workspace, (int)p.M, (int)p.w.K, (int)p.w.N, bslice,
+                                   pk4_env("OXQ_PK4_CONTIGUOUS", 1), p.act);
+            } else {
+                OXQ_HIP_CHECK(lg5.ensure((const void *)pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ, false, 5>, lds));
+                hipLaunchKernelGGL((pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ, false, 5>), grid, dim3(512), lds, s,
+                                   (const uint16_t *)p.x, p.w.pw, (const uint16_t *)p.bias, (uint16_t *)p.y,
+                                   (float *)ctx->workspace, (int)p.M, (int)p.w.K, (int)p.w.N, bslice,
+                                   pk4_env("OXQ_PK4_CONTIGUOUS", 1), p.act);
+            }
+            OXQ_HIP_CHECK(hipGetLastError());
+            return OXQ_OK;
+        }
+    }
     if constexpr (MT == 4 && BITS == 4) {
         if (grid.z == 1 && p.M > 56 && pk4_env("OXQ_PK4_PLACE64", 1)) {
             static LdsGrant lds_grant_p;
