@@ -1143,9 +1143,10 @@ __global__ __launch_bounds__(NW * 64) void pk4n_mfma_kernel(const uint16_t *__re
     pk4n_epilogue<TT, MT, NS, NW>(acc, bias, y, ws, M, N, j, m0, wave, lane);
 }
 
-// A single strip, up to 8 rows, a wave's whole share (at most NBLK blocks of 1 KB) requested up front: the
-// 16-column counterpart of pk4_front_kernel, 16 waves.
-template <typename TT, int NBLK, int XQ>
+// A single strip, up to 16 rows, a wave's whole share (at most NBLK blocks of 1 KB) requested up front, or WIN
+// blocks of it with the next requested into a block's registers when it is worked off: the 16-column
+// counterpart of pk4_front_kernel, 16 waves.
+template <typename TT, int NBLK, int XQ, int WIN = NBLK>
 __global__ __launch_bounds__(1024) void pk4n_front_kernel(const uint16_t *__restrict__ x,
                                                           const uint32_t *__restrict__ pw,
                                                           const uint16_t *__restrict__ bias,
@@ -1185,19 +1186,20 @@ __global__ __launch_bounds__(1024) void pk4n_front_kernel(const uint16_t *__rest
     for (int st = 0; st < 4; ++st) a_rd[st] = ni * 256 + (((8 * (st >> 1) + 2 * kb + (st & 1)) ^ ni) << 4);
     const NibbleMasks nm = nibble_masks();
 
-    u32x4_t av[NBLK][AQ], wv[NBLK];
-    uint32_t zv[NBLK];
-#pragma unroll
-    for (int b = 0; b < NBLK; ++b) {
+    u32x4_t av[WIN][AQ], wv[WIN];
+    uint32_t zv[WIN];
+    auto request = [&](int b, u32x4_t (&a)[AQ], u32x4_t &w, uint32_t &z) {
         const bool live = b < nloc;  // wave-uniform
         const __amdgpu_buffer_rsrc_t rx = live ? rs_x : rs_none, rw = live ? rs_w : rs_none;
         const int blk = cb0 + b;
 #pragma unroll
-        for (int q = 0; q < AQ; ++q) av[b][q] = __builtin_amdgcn_raw_buffer_load_b128(rx, voff_a[q], blk * 256, 0);
-        wv[b] = __builtin_amdgcn_raw_buffer_load_b128(rw, voff_w, blk * BB, 2);
-        zv[b] = __builtin_amdgcn_raw_buffer_load_b32(rw, voff_z, blk * BB, 2);
+        for (int q = 0; q < AQ; ++q) a[q] = __builtin_amdgcn_raw_buffer_load_b128(rx, voff_a[q], blk * 256, 0);
+        w = __builtin_amdgcn_raw_buffer_load_b128(rw, voff_w, blk * BB, 2);
+        z = __builtin_amdgcn_raw_buffer_load_b32(rw, voff_z, blk * BB, 2);
         __builtin_amdgcn_sched_barrier(0);  // blocks are requested in the order they are used
-    }
+    };
+#pragma unroll
+    for (int b = 0; b < WIN; ++b) request(b, av[b], wv[b], zv[b]);
 #pragma unroll
     for (int q = AQ; q < 4; ++q) {
         const int row = 4 * q + kb;
@@ -1214,9 +1216,9 @@ __global__ __launch_bounds__(1024) void pk4n_front_kernel(const uint16_t *__rest
         // no branch around a block past the wave's share (zeros times zeros): behind one the compiler sinks
         // the block's requests to their use
 #pragma unroll
-        for (int q = 0; q < AQ; ++q) *(u32x4_t *)(slot + q * 1024 + a_wr[q & 3]) = av[b][q];
+        for (int q = 0; q < AQ; ++q) *(u32x4_t *)(slot + q * 1024 + a_wr[q & 3]) = av[b % WIN][q];
         Pk4N<TT> cst;
-        if constexpr (DUAL) cst.prep(zv[b]);
+        if constexpr (DUAL) cst.prep(zv[b % WIN]);
         float4_t tmp, tmp1;
 #pragma unroll
         for (int st = 0; st < 4; ++st) {
@@ -1225,7 +1227,7 @@ __global__ __launch_bounds__(1024) void pk4n_front_kernel(const uint16_t *__rest
                 const u32x4_t t = *(const u32x4_t *)(slot + a_rd[st]);
                 a[0] = t[0], a[1] = t[1], a[2] = t[2], a[3] = t[3];
             }
-            const uint32_t w = wv[b][st];
+            const uint32_t w = wv[b % WIN][st];
             uint32_t bq[4];
 #pragma unroll
             for (int pp = 0; pp < 4; ++pp) {
@@ -1236,7 +1238,7 @@ __global__ __launch_bounds__(1024) void pk4n_front_kernel(const uint16_t *__rest
             tmp = Ops::mfma(a, bq, fresh ? zero4 : tmp);
             if constexpr (!DUAL) tmp1 = Ops::mfma(a, ones, fresh ? zero4 : tmp1);
         }
-        const uint32_t zw = zv[b];
+        const uint32_t zw = zv[b % WIN];
         const float sf = TT::to_f32((uint16_t)(zw >> 16));
         if constexpr (DUAL) {
 #pragma unroll
@@ -1246,6 +1248,8 @@ __global__ __launch_bounds__(1024) void pk4n_front_kernel(const uint16_t *__rest
 #pragma unroll
             for (int e = 0; e < 4; ++e) acc[0][0][e] = fmaf(sf, fmaf(nz, tmp1[e], tmp[e]), acc[0][0][e]);
         }
+        if constexpr (WIN < NBLK)
+            if (b + WIN < NBLK) request(b + WIN, av[b % WIN], wv[b % WIN], zv[b % WIN]);
     }
     pk4n_epilogue<TT, MT, 1, NW>(acc, bias, y, ws, M, N, j, 0, wave, lane);
 }
@@ -1501,12 +1505,12 @@ static int pk4n_go4(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p,
     return OXQ_OK;
 }
 
-template <typename TT, int NBLK, int XQ>
+template <typename TT, int NBLK, int XQ, int WIN = NBLK>
 static int pk4n_front_go(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, int bslice) {
     const size_t lds = (size_t)16 * 4096;
     static LdsGrant lds_grant;
-    OXQ_HIP_CHECK(lds_grant.ensure((const void *)pk4n_front_kernel<TT, NBLK, XQ>, lds));
-    hipLaunchKernelGGL((pk4n_front_kernel<TT, NBLK, XQ>), grid, dim3(1024), lds, s, (const uint16_t *)p.x, p.w.pw,
+    OXQ_HIP_CHECK(lds_grant.ensure((const void *)pk4n_front_kernel<TT, NBLK, XQ, WIN>, lds));
+    hipLaunchKernelGGL((pk4n_front_kernel<TT, NBLK, XQ, WIN>), grid, dim3(1024), lds, s, (const uint16_t *)p.x, p.w.pw,
                        (const uint16_t *)p.bias, (uint16_t *)p.y, (float *)ctx->workspace, (int)p.M, (int)p.w.K,
                        (int)p.w.N, bslice);
     OXQ_HIP_CHECK(hipGetLastError());
@@ -1530,6 +1534,8 @@ static int pk4n_by_shape(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Proble
             }
         }
         if (nfront && p.M > 8 && share <= 2) return pk4n_front_go<TT, 2, 4>(ctx, s, grid, p, bslice);
+        if (nfront && p.M > 8 && share == 3) return pk4n_front_go<TT, 3, 4, 2>(ctx, s, grid, p, bslice);  // two in flight
+        if (nfront && p.M > 8 && share == 4) return pk4n_front_go<TT, 4, 4, 2>(ctx, s, grid, p, bslice);
         if (nfront && p.M <= 8 && share <= 8) {
             switch (share) {
             case 1: case 2: return pk4n_front_go<TT, 2, 2>(ctx, s, grid, p, bslice);
@@ -1569,7 +1575,10 @@ static int launch_pk4n_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p)
     // single strip against four strips with K slices: 4096 x 4096 at 8 / 16 rows 4.32 / 5.27 against 6.11 /
     // 6.47 us; 8192 x 4096 6.38 / 8.24 against 7.47 / 8.32; 4096 x 6144 (384 strips, more than one round of
     // workgroups) 6.21 / 8.04 against 7.11 / 7.80: up to 8 rows always, up to 16 on a single round and short K.
-    const int ns1_rows = pk4_env("OXQ_PK4N_NS1_ROWS", (N / 16 <= 256 && NB <= 32) ? 16 : 8);
+    // Also up to 16 on whole rounds of 256 strips and K <= 8192 (9 / 16 rows: 8192 x 4096 6.90 / 8.07 against
+    // 7.87 / 8.31, 4096 x 8192 6.49 / 7.81 against 7.53 / 8.31); not beyond (14336 x 4096 at 12 / 16 rows 11.2 / 12.4
+    // against 10.3 / 10.7) and not on half a round (8192 x 2048 at 16 rows 7.52 against 6.63).
+    const int ns1_rows = pk4_env("OXQ_PK4N_NS1_ROWS", ((N / 16 <= 256 && NB <= 32) || ((N / 16) % 256 == 0 && NB <= 64)) ? 16 : 8);
     const int ns = (M <= ns1_rows && M <= 16 && N / 16 >= 128) ? 1 : 4;
     const int64_t tiles = (N / (16 * ns)) * ceil_div(M, 16 * mt);
     int ks = 1;
@@ -1595,9 +1604,11 @@ static int launch_pk4n_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p)
     // 8 rows, against the ring: 4096 x 4096 3.48 / 3.84 / 4.21 against 3.70 / 3.89 / 4.36 us, 8192 x 4096 4.78 /
     // 5.38 / 6.21 against 5.02 / 5.40 / 6.44, 14336 x 4096 6.76 / 7.57 / 9.33 against 6.96 / 7.70 / 9.49,
     // 4096 x 8192 4.72 / 5.26 / 6.10 against 5.02 / 5.53 / 6.56.  With at most two blocks a wave (K <= 4096) also
-    // the 9 - 16 rows that a single strip takes there: 4096 x 4096 at 9 / 16 rows 4.37 / 5.12 against 4.71 / 5.28.
+    // the 9 - 16 rows that a single strip takes there: 4096 x 4096 at 9 / 16 rows 4.37 / 5.12 against 4.71 / 5.28;
+    // with three or four blocks a wave (K <= 8192) two of them in flight: 8192 x 4096 at 9 / 12 / 16 rows 6.90 /
+    // 7.41 / 8.07 -> 6.67 / 7.16 / 7.96.
     const bool nfront = ns == 1 && ceil_div(bslice, 16) <= 8 && pk4_env("OXQ_PK4_FRONT", 1) &&
-                        (M <= 8 || (M <= 16 && ceil_div(bslice, 16) <= 2));
+                        (M <= 8 || (M <= 16 && ceil_div(bslice, 16) <= 4));
     const bool w16 = nfront || (ns == 1 && M <= 2 && pk4_env("OXQ_PK4N_W16", NB >= 64));
     char name[64];
     snprintf(name, sizeof name, "pk4_mfma_%s_mt%d%s_n16x%d", p.w.dtype == OXQ_F16 ? "f16" : "bf16", mt,

@@ -80,7 +80,8 @@ def test_narrow_layout_forced_on_small_shapes(kind, dtn, K, N, g, monkeypatch):
         y = layer.forward(xd)
         plan = kernel_of_last_call()
         assert "_n16x" in plan["kernel"], plan
-        single = N >= 2048 and m <= (16 if N // 16 <= 256 and K // 128 <= 32 else 8)
+        wide16 = (N // 16 <= 256 and K // 128 <= 32) or ((N // 16) % 256 == 0 and K // 128 <= 64)
+        single = N >= 2048 and m <= (16 if wide16 else 8)
         assert plan["kernel"].endswith("x1") == single, plan
         # three row tiles keep the tile form in this layout: the fold's sums do not fit beside the ring
         rounded = resident_rounds_weights(m, dt, kind == "gptq") or (dt == oracle.F16 and 32 < m <= 48)
@@ -111,10 +112,11 @@ def test_narrow_layout_k_slices(ks, monkeypatch):
         assert_close(y, oracle.matmul_nt_f32(round_x(x, dt), wr, bias), f"narrow k-slices m{m}")
 
 
-@pytest.mark.parametrize("K,N", [(4096, 4096), (4096, 6144), (8192, 2048), (14336, 4096), (4096, 8192)])
+@pytest.mark.parametrize("K,N", [(4096, 4096), (4096, 6144), (8192, 2048), (14336, 4096), (4096, 8192), (8192, 4096),
+                                 (6144, 4096)])
 def test_attention_and_down_projection_shapes_take_the_narrow_layout(K, N, monkeypatch):
-    """By shape alone (no switch): one launch up to eight rows (16 waves a workgroup for one or two rows on a
-    long K), the wide layout's answer within tolerance."""
+    """By shape alone (no switch): one launch up to eight rows, up to 16 on whole rounds of strips and K <= 8192
+    (16 waves a workgroup), the wide layout's answer within tolerance."""
     dt = oracle.F16
     trip, pack_dim = make("awq", K, N, 128, seed=N)
     layer = layer_of(trip, pack_dim, dt)
@@ -123,7 +125,8 @@ def test_attention_and_down_projection_shapes_take_the_narrow_layout(K, N, monke
     monkeypatch.delenv("OXQ_PK4_STRIP16")
     w = dense("awq", trip, dt)
     np.testing.assert_array_equal(bits_of(layer.dequantize()), bits_of(wide.dequantize()))
-    for m in (1, 2, 4, 8, 16, 64):
+    wide16 = (N // 16 <= 256 and K // 128 <= 32) or ((N // 16) % 256 == 0 and K // 128 <= 64)
+    for m in (1, 2, 4, 8, 9, 12, 16, 64):
         say(f"narrow by shape K={K} N={N} m={m}")
         x = np.random.default_rng(m).standard_normal((m, K)).astype(np.float32)
         xd = to_dev(x, torch.float16)
@@ -133,6 +136,11 @@ def test_attention_and_down_projection_shapes_take_the_narrow_layout(K, N, monke
         if m <= 8:
             assert plan["launches"] == 1 and plan["split_k"] == 1 and plan["grid"][0] == N // 16, plan
             assert plan["block"][0] == 1024, plan   # up to 8 rows: 16 waves, all requests first
+        elif m <= 16:
+            # 9 - 16 rows: one strip a workgroup on whole rounds of strips and K <= 8192 (16 waves there)
+            assert plan["kernel"].endswith("x1") == wide16, plan
+            if wide16:
+                assert plan["launches"] == 1 and plan["block"][0] == 1024, plan
         yw = wide.forward(xd)
         assert "_n16x" not in kernel_of_last_call()["kernel"]
         wr = oracle.round_through(w, dt) if resident_rounds_weights(m, dt, False) else w
