@@ -623,6 +623,8 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
         if constexpr (PLACED) __builtin_amdgcn_sched_barrier(0);
         store_a(aring);
         load_a(i + 2, aring);
+        // two row tiles as straight-line code: the requests for the block after next stay at the block's end
+        if constexpr (NBLK > 0 && MT == 2) __builtin_amdgcn_sched_barrier(0);
     }
 
     pk4_epilogue<TT, MT>(acc, bias, y, ws, M, N, j, m0, act, wave, lane);
@@ -1386,12 +1388,36 @@ static int pk4_go4(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, 
     }
     constexpr int WD = Pk4Ring<MT, BITS>::WD;
     const size_t lds = (size_t)8 * MT * 4096;
+    if constexpr (MT == 2) {
+        // Two row tiles, four or five blocks a wave, one row-tile workgroup a strip: straight-line code with the
+        // memory operations placed by hand and the block-end requests pinned.  Same box, loop -> straight line,
+        // 4096 x 14336 at 17 / 32 rows: f16 9.85 / 11.04 -> 9.66 / 10.45 us, bf16 14.37 / 14.55 -> 12.04 / 12.48, 8-bit
+        // f16 14.00 / 14.71 -> 13.26 / 14.14.  (Unrolled without the pins it is slower than the loop: f16 12.15 /
+        // 13.12; with the block-end pin alone 9.70 / 10.91.)
+        if (grid.z == 1 && (bslice == 32 || bslice == 40) && pk4_env("OXQ_PK4_FRONT", 1)) {
+            static LdsGrant lg4, lg5;
+            if (bslice == 32) {
+                OXQ_HIP_CHECK(lg4.ensure((const void *)pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ, true, 4>, lds));
+                hipLaunchKernelGGL((pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ, true, 4>), grid, dim3(512), lds, s,
+                                   (const uint16_t *)p.x, p.w.pw, (const uint16_t *)p.bias, (uint16_t *)p.y,
+                                   (float *)ctx->workspace, (int)p.M, (int)p.w.K, (int)p.w.N, bslice,
+                                   pk4_env("OXQ_PK4_CONTIGUOUS", 1), p.act);
+            } else {
+                OXQ_HIP_CHECK(lg5.ensure((const void *)pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ, true, 5>, lds));
+                hipLaunchKernelGGL((pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ, true, 5>), grid, dim3(512), lds, s,
+                                   (const uint16_t *)p.x, p.w.pw, (const uint16_t *)p.bias, (uint16_t *)p.y,
+                                   (float *)ctx->workspace, (int)p.M, (int)p.w.K, (int)p.w.N, bslice,
+                                   pk4_env("OXQ_PK4_CONTIGUOUS", 1), p.act);
+            }
+            OXQ_HIP_CHECK(hipGetLastError());
+            return OXQ_OK;
+        }
+    }
     if constexpr (MT >= 3) {
         // Four or five blocks a wave (K = 4096, 5120 unsliced) and one row-tile workgroup a strip: the block loop as
         // straight-line code.  Same box, loop -> straight line, 48 / 64 rows: 4-bit f16 4096 x 14336 13.66 / 16.40 ->
         // 13.06 / 16.29 us, bf16 15.74 / 18.70 -> 15.23 / 17.91; 5120 x 13824 f16 16.6 / 20.39 -> 16.05 / 20.1, bf16
-        // 18.9 / 22.12 -> 18.16 / 21.82; 8-bit f16 4096 x 14336 17.09 / 20.4 -> 16.65 / 19.85.  (Two row tiles lose by
-        // it: 4-bit f16 at 17 / 32 rows 9.86 / 11.07 -> 12.15 / 13.12.)
+        // 18.9 / 22.12 -> 18.16 / 21.82; 8-bit f16 4096 x 14336 17.09 / 20.4 -> 16.65 / 19.85.
         if (grid.z == 1 && (bslice == 32 || bslice == 40) && pk4_env("OXQ_PK4_FRONT", 1)) {
             static LdsGrant lg4, lg5;
             if (bslice == 32) {
