@@ -1391,16 +1391,30 @@ static int pk4_go4(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, 
     constexpr int WD = Pk4Ring<MT, BITS>::WD;
     const size_t lds = (size_t)8 * MT * 4096;
     if constexpr (MT == 2) {
-        // Two row tiles, four or five blocks a wave, one row-tile workgroup a strip: straight-line code with the
+        // Two row tiles, four or five blocks a wave (4-bit: also six or eight, K = 6144, 8192 - 32 rows f16 15.69 / 35.45
+        // -> 14.88 / 33.73 us, bf16 20.54 / 49.01 -> 17.24 / 39.82 on 6144 x 16384 / 8192 x 28672), one row-tile workgroup
+        // a strip: straight-line code with the
         // memory operations placed by hand and the block-end requests pinned.  Same box, loop -> straight line,
         // 4096 x 14336 at 17 / 32 rows: f16 9.85 / 11.04 -> 9.66 / 10.45 us, bf16 14.37 / 14.55 -> 12.04 / 12.48, 8-bit
         // f16 14.00 / 14.71 -> 13.26 / 14.14.  (Unrolled without the pins it is slower than the loop: f16 12.15 /
         // 13.12; with the block-end pin alone 9.70 / 10.91.)
-        if (grid.z == 1 && (bslice == 32 || bslice == 40) && pk4_env("OXQ_PK4_FRONT", 1)) {
-            static LdsGrant lg4, lg5;
+        if (grid.z == 1 && (bslice == 32 || bslice == 40 || ((bslice == 48 || bslice == 64) && BITS == 4)) && pk4_env("OXQ_PK4_FRONT", 1)) {
+            static LdsGrant lg4, lg5, lg6, lg8;
             if (bslice == 32) {
                 OXQ_HIP_CHECK(lg4.ensure((const void *)pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ, true, 4>, lds));
                 hipLaunchKernelGGL((pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ, true, 4>), grid, dim3(512), lds, s,
+                                   (const uint16_t *)p.x, p.w.pw, (const uint16_t *)p.bias, (uint16_t *)p.y,
+                                   (float *)ctx->workspace, (int)p.M, (int)p.w.K, (int)p.w.N, bslice,
+                                   pk4_env("OXQ_PK4_CONTIGUOUS", 1), p.act);
+            } else if (bslice == 48) {
+                OXQ_HIP_CHECK(lg6.ensure((const void *)pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ, true, 6>, lds));
+                hipLaunchKernelGGL((pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ, true, 6>), grid, dim3(512), lds, s,
+                                   (const uint16_t *)p.x, p.w.pw, (const uint16_t *)p.bias, (uint16_t *)p.y,
+                                   (float *)ctx->workspace, (int)p.M, (int)p.w.K, (int)p.w.N, bslice,
+                                   pk4_env("OXQ_PK4_CONTIGUOUS", 1), p.act);
+            } else if (bslice == 64) {
+                OXQ_HIP_CHECK(lg8.ensure((const void *)pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ, true, 8>, lds));
+                hipLaunchKernelGGL((pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ, true, 8>), grid, dim3(512), lds, s,
                                    (const uint16_t *)p.x, p.w.pw, (const uint16_t *)p.bias, (uint16_t *)p.y,
                                    (float *)ctx->workspace, (int)p.M, (int)p.w.K, (int)p.w.N, bslice,
                                    pk4_env("OXQ_PK4_CONTIGUOUS", 1), p.act);
@@ -1420,11 +1434,23 @@ static int pk4_go4(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, 
         // straight-line code.  Same box, loop -> straight line, 48 / 64 rows: 4-bit f16 4096 x 14336 13.66 / 16.40 ->
         // 13.06 / 16.29 us, bf16 15.74 / 18.70 -> 15.23 / 17.91; 5120 x 13824 f16 16.6 / 20.39 -> 16.05 / 20.1, bf16
         // 18.9 / 22.12 -> 18.16 / 21.82; 8-bit f16 4096 x 14336 17.09 / 20.4 -> 16.65 / 19.85.
-        if (grid.z == 1 && (bslice == 32 || bslice == 40) && pk4_env("OXQ_PK4_FRONT", 1)) {
-            static LdsGrant lg4, lg5;
+        if (grid.z == 1 && (bslice == 32 || bslice == 40 || ((bslice == 48 || bslice == 64) && BITS == 4)) && pk4_env("OXQ_PK4_FRONT", 1)) {
+            static LdsGrant lg4, lg5, lg6, lg8;
             if (bslice == 32) {
                 OXQ_HIP_CHECK(lg4.ensure((const void *)pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ, false, 4>, lds));
                 hipLaunchKernelGGL((pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ, false, 4>), grid, dim3(512), lds, s,
+                                   (const uint16_t *)p.x, p.w.pw, (const uint16_t *)p.bias, (uint16_t *)p.y,
+                                   (float *)ctx->workspace, (int)p.M, (int)p.w.K, (int)p.w.N, bslice,
+                                   pk4_env("OXQ_PK4_CONTIGUOUS", 1), p.act);
+            } else if (bslice == 48) {
+                OXQ_HIP_CHECK(lg6.ensure((const void *)pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ, false, 6>, lds));
+                hipLaunchKernelGGL((pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ, false, 6>), grid, dim3(512), lds, s,
+                                   (const uint16_t *)p.x, p.w.pw, (const uint16_t *)p.bias, (uint16_t *)p.y,
+                                   (float *)ctx->workspace, (int)p.M, (int)p.w.K, (int)p.w.N, bslice,
+                                   pk4_env("OXQ_PK4_CONTIGUOUS", 1), p.act);
+            } else if (bslice == 64) {
+                OXQ_HIP_CHECK(lg8.ensure((const void *)pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ, false, 8>, lds));
+                hipLaunchKernelGGL((pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ, false, 8>), grid, dim3(512), lds, s,
                                    (const uint16_t *)p.x, p.w.pw, (const uint16_t *)p.bias, (uint16_t *)p.y,
                                    (float *)ctx->workspace, (int)p.M, (int)p.w.K, (int)p.w.N, bslice,
                                    pk4_env("OXQ_PK4_CONTIGUOUS", 1), p.act);

@@ -224,10 +224,11 @@ def test_eight_bit_single_row_tile_in_straight_line_code(kind, dtn, K, N, g, ks,
 
 @pytest.mark.parametrize("kind", ["awq", "gptq", "gptq8"])
 @pytest.mark.parametrize("dtn", ["f16", "bf16"])
-@pytest.mark.parametrize("K,N,g,ks", [(4096, 128, 128, 1), (8192, 64, 128, 2), (8064, 64, 128, 2), (5120, 64, 128, 1)])
+@pytest.mark.parametrize("K,N,g,ks", [(4096, 128, 128, 1), (8192, 64, 128, 2), (8064, 64, 128, 2), (5120, 64, 128, 1),
+                                      (6144, 64, 128, 1), (8192, 64, 128, 1)])
 def test_two_to_four_row_tiles_in_straight_line_code(kind, dtn, K, N, g, ks, monkeypatch):
-    """17 - 64 rows on K slices of 32 or 40 blocks run the block loop as straight-line code (four or five
-    blocks a wave); 63 blocks in two slices leave one wave of the second slice a block short.  Against the
+    """17 - 64 rows on K slices of 32 or 40 blocks (4-bit: also 48 and 64) run the block loop as straight-line
+    code (four to eight blocks a wave); 63 blocks in two slices leave one wave of the second slice a block short.  Against the
     oracle of the form the row count takes, run to run bitwise, and against the looping kernel."""
     monkeypatch.setenv("OXQ_PK4_STRIP16", "0")
     monkeypatch.setenv("OXQ_PK4_KS", str(ks))
