@@ -531,7 +531,8 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
     // With the block count known (NBLK) there is no loop at all (figures where it is launched).
     constexpr int UF = NBLK > 0 ? 1 : PLACED ? 2 : 1;
     const int trip = NBLK > 0 ? NBLK : nloc;
-#pragma unroll(NBLK > 0 ? NBLK : 1)
+    constexpr int UNROLL = NBLK > 0 ? NBLK : 1;
+#pragma unroll UNROLL
     for (int i0 = 0; i0 < trip; i0 += UF)
 #pragma unroll
     for (int u = 0; u < UF; ++u) {
