@@ -377,8 +377,12 @@ __global__ __launch_bounds__(512) void pk4_mfma_kernel(const uint16_t *__restric
     constexpr int BB = pk4_block_words(BITS) * 4;  // bytes of one block: weights, then the zero/scale pairs
     // Up to 48 rows there is one row tile, so every weight is read once per launch: nontemporal
     // loads (cache policy bit 1), which a bare read of the same 30 MB also gains 7 % from.
-    // From 49 rows on several row tiles may share a strip through L2, so those keep the default.
-    constexpr int WNT = MT < 4 ? 2 : 0;
+    // From 49 rows on several row tiles may share a strip through L2, so those keep the default - except the
+    // forms that are only launched with one row-tile workgroup a strip (NBLK, PLZ).  64 rows, same box, default ->
+    // nontemporal: 4096 x 14336 f16 15.93 -> 15.45 us, bf16 17.48 -> 17.02; 5120 x 13824 f16 19.33 -> 18.54, 8-bit 24.14 ->
+    // 22.60; 8192 x 28672 51.7 -> 50.8.  (4096 x 11008 measures 14.44 -> 14.60: its 12 rotated copies, 270 MB, are
+    // partly still in the 256 MB memory-side cache when their turn comes again, which a decoder's layers are not.)
+    constexpr int WNT = (MT < 4 || NBLK > 0 || PLZ) ? 2 : 0;
     // Hand-placed memory operations (the three places marked PLACED below) instead of the compiler's own order,
     // where that measured faster - same box, 48 / 64 / 128 rows: 8-bit f16 5120 x 13824 21.8 / 27.3 / 42.5 ->
     // 20.6 / 24.3 / 41.0 us; 4-bit bf16 4096 x 14336 at 33 / 48 rows 16.4 / 16.7 -> 15.2 / 15.9 us.  The 4-bit f16
@@ -947,7 +951,7 @@ __global__ __launch_bounds__(NW * 64) void pk4n_mfma_kernel(const uint16_t *__re
     // f16 add - and the block folds in with its scale alone.
     constexpr bool EXACT = GS && DUAL && NS == 1;
     constexpr int ROWS = 16 * MT, AQ = XQ, SLOT = ROWS * 256, OOB = 0x7FFFFF00, BB = PK4N_BW * 4;
-    constexpr int WNT = MT < 4 ? 2 : 0;
+    constexpr int WNT = MT < 4 ? 2 : 0;  // (nontemporal at 49 - 64 rows measured slower here: 4096 x 4096 11.90 against 11.51 us)
     extern __shared__ __attribute__((aligned(16))) unsigned char pk4_lds[];
 
     const int lane = threadIdx.x & 63;
