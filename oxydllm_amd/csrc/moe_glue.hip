@@ -379,9 +379,29 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const T *__restrict__ 
     if (gid >= (size_t)ntok * H) return;
     const int t = (int)(gid / H), h = (int)(gid % H);
     float acc = 0.0f;
-    for (int s = 0; s < top_k; ++s) {
-        const int pos = pair_pos[(size_t)t * top_k + s];
-        acc = fmaf(top_vals[(size_t)t * top_k + s], load_f32(eo, (size_t)pos * H + h), acc);
+    constexpr int MAXK = 8;
+    if (top_k <= MAXK) {
+        // all positions first, then all expert outputs, then the sum in slot order: two dependent loads deep
+        // instead of two per slot
+        int pos[MAXK];
+        float w[MAXK], v[MAXK];
+#pragma unroll
+        for (int s = 0; s < MAXK; ++s)
+            if (s < top_k) {
+                pos[s] = pair_pos[(size_t)t * top_k + s];
+                w[s] = top_vals[(size_t)t * top_k + s];
+            }
+#pragma unroll
+        for (int s = 0; s < MAXK; ++s)
+            if (s < top_k) v[s] = load_f32(eo, (size_t)pos[s] * H + h);
+#pragma unroll
+        for (int s = 0; s < MAXK; ++s)
+            if (s < top_k) acc = fmaf(w[s], v[s], acc);
+    } else {
+        for (int s = 0; s < top_k; ++s) {
+            const int pos = pair_pos[(size_t)t * top_k + s];
+            acc = fmaf(top_vals[(size_t)t * top_k + s], load_f32(eo, (size_t)pos * H + h), acc);
+        }
     }
     store_f32(out, gid, acc);
 }
