@@ -181,6 +181,9 @@ size_t pk4_zs_bytes(int64_t K, int64_t N, int group_shift);
 int launch_pk4_prepack(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &src, const Pk4Weights &dst);
 int launch_pk4_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p);
 int launch_pk4_dequant(oxq_ctx *ctx, hipStream_t s, const Pk4Weights &w, void *out_kn);
+// 49 - 64 rows on a 4-bit layer in 64-column strips (pk4_tile.hip)
+bool pk4_tile64_takes(const Pk4Problem &p, int ks);
+int launch_pk4_tile64(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p);
 int launch_wna16_gemv(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p);
 bool awq4_mfma_ok(const Wna16Problem &p);  // the checkpoint-layout tile kernel takes this problem
 int launch_wna16_mfma(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p);
