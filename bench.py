@@ -16,8 +16,9 @@ results, in GB/s and TFLOP/s, ride along in `cases`.  `roofline` describes the
 dominant kernel (the M=1 GEMV, HBM-bound); `cpu_baseline` times the CPU oracle's
 restatement of the reference's CPU path (dequantize at load, then a dense f32
 x.W^T per call, linear.rs:40-79, 597-600) on this machine's cores.
-`roofline.bare_read_us` / `bare_read_nt_us` are a plain read of the same packed
-weights with the same launch shape and no arithmetic (plain / nontemporal loads).
+`roofline.bare_read_us` / `bare_read_nt_us` / `bare_read_best_us` are plain reads of the same
+packed weights with no arithmetic (in passes, plain / nontemporal; everything requested first),
+`roofline.empty_launch_us` an empty kernel of the same launch shape.
 `other_configs` holds one compact row per case of BASELINE configs 0, 2, 3 and 4,
 each with its own roofline fraction and a CPU baseline per configuration.
 """
@@ -267,28 +268,47 @@ def main():
             print(f"[bench] down-projection layer M={m}: {down_cases[-1]}", file=sys.stderr, flush=True)
         del dlayers
 
-    # What a kernel with no arithmetic takes to read the same packed weights once: 224 workgroups of 512
-    # threads, 128 KB each (the resident-layer kernel's launch shape), plain and nontemporal loads, cold.
+    # What the machine does with the same bytes and launch shape when there is no arithmetic (include/oxq_bench.h):
+    #  * empty_launch_us: an empty kernel of the M = 1 kernel's launch shape - the period of back-to-back launches;
+    #  * bare_read_us / bare_read_nt_us: 224 workgroups of 512 threads read the packed weights in passes, eight loads
+    #    in flight a lane (plain / nontemporal);
+    #  * bare_read_best_us: the same bytes with every lane's whole share requested before the first wait, as the
+    #    M <= 16 kernels request their weights - the best of 8 and 16 waves a workgroup, nontemporal.
     bare = {}
     if not args.no_bare_read:
         nbytes_w = K * N // 2
         pool = torch.empty(copies * nbytes_w, dtype=torch.uint8, device=dev).random_(0, 256)
         sums = torch.empty(256, dtype=torch.int32, device=dev)
+        m1 = cases[0]
+        _, ev = time_graph(lambda i: ops.empty_launch(m1["grid"][0], 1024 if "front" in m1["kernel"] else 512, 65536, ctx=ctx),
+                           args.steps, args.warmup, stream)
+        bare["empty_launch_us"] = round(ev * 1e3 / args.steps, 3)
         for nt in (0, 1):
             def rd(i, nt=nt):
                 c = i % copies
                 ops.calib_read(pool[c * nbytes_w:(c + 1) * nbytes_w], N // 64, bool(nt), sums, ctx=ctx)
             _, ev = time_graph(rd, args.steps, args.warmup, stream)
             bare["bare_read_nt_us" if nt else "bare_read_us"] = round(ev * 1e3 / args.steps, 3)
+        best = {}
+        for waves in (8, 16):
+            def rd(i, waves=waves):
+                c = i % copies
+                ops.read_upfront(pool[c * nbytes_w:(c + 1) * nbytes_w], N // 64, waves, True, sums, ctx=ctx)
+            _, ev = time_graph(rd, args.steps, args.warmup, stream)
+            best[waves] = round(ev * 1e3 / args.steps, 3)
+        bare["bare_read_best_us"] = min(best.values())
+        bare["bare_read_best_waves"] = min(best, key=best.get)
+        bare["bare_read_upfront_us_by_waves"] = best
         bare["bare_read_bytes"] = nbytes_w
         bare["bare_read_workgroups"] = N // 64
         print(f"[bench] plain read of {nbytes_w} B by {N // 64} workgroups: {bare}", file=sys.stderr, flush=True)
         del pool
 
     c1 = cases[0]
-    # HBM bytes per launch of the M=1 kernel, measured offline with rocprofv3 --pmc
-    # (FETCH_SIZE, WRITE_SIZE) and recorded in the committed profile summary.
-    traffic = None
+    # HBM bytes per launch of the M=1 kernel, measured offline with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE) and
+    # recorded in the committed profile summary - which names the kernel it measured: a summary of another
+    # kernel than the one this run timed gives no traffic figure.
+    traffic, traffic_kernel = None, None
     tpath = os.path.join(ROOT, "profiles", "pk4_mfma_m1_K4096_N14336_pmc.txt")
     if os.path.exists(tpath):
         for line in open(tpath):
@@ -297,6 +317,10 @@ def main():
                     traffic = int(float(line.split(":", 1)[1].split()[0]))
                 except ValueError:
                     traffic = None
+            elif line.startswith("kernel_of_traffic:"):
+                traffic_kernel = line.split(":", 1)[1].strip()
+    if traffic_kernel != c1["kernel"]:
+        traffic = None
     result = {
         "metric": "int4 GEMV/GEMM HBM GB/s (% peak) + TFLOPS at M=1/16/64, K=4096 N=14336",
         "value": c1["GB_per_s"],

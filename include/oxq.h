@@ -118,6 +118,16 @@ const char *oxq_last_error(void);
 const char *oxq_status_name(int status);
 void oxq_version(int *major, int *minor);
 
+/* ---- tuning switches -----------------------------------------------------------
+ * No counterpart in the reference.  Every switch that selects between kernels or launch shapes
+ * (OXQ_PK4_FRONT, OXQ_PK4_KS, OXQ_FORCE_GENERIC, ...: the list is OXQ_TUNE_LIST in the library's
+ * sources) lives in the ctx.  oxq_ctx_create reads each once from the environment variable of the
+ * same name; oxq_ctx_set_tuning overrides one for this ctx, oxq_ctx_reset_tuning(ctx, name) returns it
+ * to the environment's value (name = NULL: all of them).  The op functions never read the
+ * environment.  An unknown name is OXQ_ERR_ARG.  Meant for tests and for tuning runs. */
+int oxq_ctx_set_tuning(oxq_ctx *ctx, const char *name, int value);
+int oxq_ctx_reset_tuning(oxq_ctx *ctx, const char *name);
+
 /* ---- opt-in weight cache behind the stateless ops -----------------------------
  * The reference's layers call the op functions with the same resident tensors on every forward
  * (linear.rs:482-533).  With this cache on, oxq_w4a16_matmul / oxq_w8a16_matmul / oxq_gptq_matmul /
@@ -132,6 +142,14 @@ void oxq_version(int *major, int *minor);
  * keyed by the address of the block
  * bytes, with the strip-major copy that oxq_qlinear_new builds.
  *
+ * A copy that served a call while the stream was being captured is part of that graph: it stays, and
+ * counts against max_bytes, until oxq_ctx_forget_weights or oxq_ctx_destroy frees it - either of which
+ * invalidates every graph captured with it.  Dropping a copy (eviction, a smaller max_bytes, forget)
+ * calls hipFree, which waits for the device: the one place where these op functions can synchronise.
+ * When the weights in use need more room than max_bytes, the copies that were used within the last
+ * (copies + 1) calls stay and the others run on the checkpoint layout, rather than every call rebuilding
+ * a copy.
+ *
  * Contract: while a triple is cached its tensors must neither change nor be freed and reused - the
  * ctx cannot see that.  Call oxq_ctx_forget_weights(ctx, qweight->data) (for a GGUF weight: the
  * address of its block bytes) before doing so (NULL drops every copy).  Off by default (max_bytes = 0, or OXQ_WEIGHT_CACHE_MB in the environment).
@@ -142,16 +160,6 @@ int oxq_ctx_weight_cache_bytes(const oxq_ctx *ctx, int64_t *bytes, int64_t *entr
 
 /* Block layout of a GGUF format: metal_ops.rs:5228-5241 (block_layout). */
 int oxq_gguf_block_layout(int quant, int64_t *block_elems, int64_t *block_bytes);
-
-/* ---- measurement aid ---------------------------------------------------------
- * No counterpart in the reference.  A plain streaming read of `src` (U8, contiguous, 16-byte
- * aligned; its size a multiple of workgroups * 8 KiB) by `workgroups` workgroups of 512 threads,
- * each reading one contiguous span with 16-byte loads, eight in flight per lane - the launch shape of
- * the resident-layer GEMV with the arithmetic taken out.  `checksums` (U32 [>= workgroups]) receives
- * an xor of every span, which keeps the loads alive and lets a test check the read.  bench.py times
- * it beside the GEMV kernels: it is what a read-once kernel can reach on the machine at hand. */
-int oxq_calib_read(oxq_ctx *ctx, void *stream, const oxq_tensor *src, int workgroups, int nontemporal,
-                   const oxq_tensor *checksums);
 
 /* ---- decode GEMV ops (1 <= m <= 8) ---------------------------------------
  * y[m,N] = x[m,K] . dequant(W), f32 accumulate, result in x's dtype.
@@ -168,7 +176,9 @@ int oxq_w4a16_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x, const oxq_
  * device array inside the library (16 MiB on every GPU the library runs on, held until the process
  * ends) instead of the ctx workspace, the K slices are always added by a second launch, and the
  * call makes no allocation of any kind.  A call whose partial sums (slices * m * N * 4 bytes) exceed
- * 16 MiB fails with OXQ_ERR_WORKSPACE and enqueues nothing.  Every call on a GPU shares that GPU's
+ * 16 MiB fails with OXQ_ERR_WORKSPACE and enqueues nothing; a shape whose K slices the generic kernel
+ * can only add with arrival counters (N not a multiple of 4 and more than one slice) fails with
+ * OXQ_ERR_UNSUPPORTED, likewise before anything is enqueued.  Every call on a GPU shares that GPU's
  * array: calls that overlap on one GPU (two streams, two threads) race; serialise them. */
 int oxq_w4a16_matmul_static(oxq_ctx *ctx, void *stream, const oxq_tensor *x, const oxq_tensor *qweight,
                             const oxq_tensor *qzeros, const oxq_tensor *scales, const oxq_tensor *out);

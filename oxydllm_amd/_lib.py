@@ -66,7 +66,7 @@ class OxqError(RuntimeError):
         self.message = message
 
 
-# Every symbol include/oxq.h declares, with its argument types.
+# Every symbol include/*.h declares, with its argument types.
 _TP = C.POINTER(OxqTensor)
 _VP = C.c_void_p
 SIGNATURES = {
@@ -81,7 +81,11 @@ SIGNATURES = {
     "oxq_ctx_forget_weights": (C.c_int, [_VP, _VP]),
     "oxq_ctx_weight_cache_bytes": (C.c_int, [_VP, C.POINTER(C.c_int64), C.POINTER(C.c_int64)]),
     "oxq_gguf_block_layout": (C.c_int, [C.c_int, C.POINTER(C.c_int64), C.POINTER(C.c_int64)]),
+    "oxq_ctx_set_tuning": (C.c_int, [_VP, C.c_char_p, C.c_int]),
+    "oxq_ctx_reset_tuning": (C.c_int, [_VP, C.c_char_p]),
     "oxq_calib_read": (C.c_int, [_VP, _VP, _TP, C.c_int, C.c_int, _TP]),
+    "oxq_bench_read_upfront": (C.c_int, [_VP, _VP, _TP, C.c_int, C.c_int, C.c_int, _TP]),
+    "oxq_bench_empty_launch": (C.c_int, [_VP, _VP, C.c_int, C.c_int, C.c_int]),
     "oxq_w4a16_matmul": (C.c_int, [_VP, _VP, _TP, _TP, _TP, _TP, _TP]),
     "oxq_w4a16_matmul_static": (C.c_int, [_VP, _VP, _TP, _TP, _TP, _TP, _TP]),
     "oxq_w8a16_matmul": (C.c_int, [_VP, _VP, _TP, _TP, _TP, _TP, _TP]),

@@ -387,18 +387,16 @@ static int launch_mm_go(hipStream_t s, const MmArgs &a, dim3 grid, size_t lds) {
 // for the 4-bit formats, slower for the others, whose kernels then need > 256 registers).
 // When that grid cannot fill the 256 CUs, K is split over up to 8 slices of at least two
 // stages.  `rows` = tokens (plain) or routed pairs (grouped, never split).
-static MmPlan plan_mm(const oxq_ctx *ctx, int64_t rows, int64_t K, int64_t N, bool grouped, const char *env_prefix) {
+static MmPlan plan_mm(const oxq_ctx *ctx, int64_t rows, int64_t K, int64_t N, bool grouped, oxq_tune_key mt_key,
+                      oxq_tune_key ks_key) {
     MmPlan pl;
     pl.mt = rows > 32 ? 4 : rows > 16 ? 2 : 1;
-    char key[48];
-    snprintf(key, sizeof key, "%s_MT", env_prefix);
-    if (const char *e = getenv(key)) pl.mt = atoi(e) == 1 ? 1 : atoi(e) == 2 ? 2 : 4;
+    if (tune_given(ctx, mt_key)) pl.mt = tune(ctx, mt_key, 4) == 1 ? 1 : tune(ctx, mt_key, 4) == 2 ? 2 : 4;
     const int stages = (int)ceil_div(K, MM_BK);
     const int64_t tiles = ceil_div(N, MM_BN) * ceil_div(rows, 16 * pl.mt);
     pl.ks = 1;
     if (tiles < 192) pl.ks = (int)std::min<int64_t>({ceil_div(256, tiles), 8, std::max(1, stages / 2)});
-    snprintf(key, sizeof key, "%s_KS", env_prefix);
-    if (const char *e = getenv(key)) pl.ks = std::max(1, std::min(atoi(e), stages));
+    if (tune_given(ctx, ks_key)) pl.ks = std::max(1, std::min(tune(ctx, ks_key, 1), stages));
     // the reduction kernel works on groups of 4 columns; the workspace bounds the split
     if (N % 4 != 0 || grouped) pl.ks = 1;
     while (pl.ks > 1 && (size_t)pl.ks * rows * N * 4 > ctx->workspace_bytes) --pl.ks;
@@ -409,10 +407,10 @@ static MmPlan plan_mm(const oxq_ctx *ctx, int64_t rows, int64_t K, int64_t N, bo
 
 // hilo: (GGUF, m <= 8) keep the rounding residue of every weight, see GgufSource::decode
 template <class SRC>
-static int launch_mm_src(oxq_ctx *ctx, hipStream_t s, MmArgs &a, const char *name_prefix, const char *env_prefix,
+static int launch_mm_src(oxq_ctx *ctx, hipStream_t s, MmArgs &a, const char *name_prefix, oxq_tune_key mt_key, oxq_tune_key ks_key,
                          bool hilo = false) {
     const bool grouped = a.offsets != nullptr;
-    const MmPlan pl = plan_mm(ctx, a.M, a.K, a.N, grouped, env_prefix);
+    const MmPlan pl = plan_mm(ctx, a.M, a.K, a.N, grouped, mt_key, ks_key);
     const int mt = pl.mt;
     a.ws = (float *)ctx->workspace;
     a.stages_per_slice = pl.stages_per_slice;
@@ -449,9 +447,8 @@ static int launch_mm_src(oxq_ctx *ctx, hipStream_t s, MmArgs &a, const char *nam
     return launch_splitk_reduce(ctx, s, (const float *)ctx->workspace, a.bias, a.y, a.M, a.N, pl.ks, OXQ_BF16);
 }
 
-bool gguf_mm_eligible(const GgufProblem &p) {
-    const char *e = getenv("OXQ_GGUF_MM_MIN_M");
-    const int min_m = e ? atoi(e) : 3;  // measured 4096^2: m = 2 GEMV 9.1 / tile 10.6 us, m = 4 16.0 / 10.5
+bool gguf_mm_eligible(const oxq_ctx *ctx, const GgufProblem &p) {
+    const int min_m = tune(ctx, OXQ_TUNE_GGUF_MM_MIN_M, 3);  // measured 4096^2: m = 2 GEMV 9.1 / tile 10.6 us, m = 4 16.0 / 10.5
     return p.act_dtype == OXQ_BF16 && p.M >= min_m && ((uintptr_t)p.x & 15) == 0 && ((uintptr_t)p.w & 15) == 0 &&
            (p.K % 8) == 0;
 }
@@ -463,10 +460,9 @@ int launch_gguf_mm(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p) {
     a.x = (const uint16_t *)p.x, a.w = p.w, a.bias = (const uint16_t *)p.bias, a.y = (uint16_t *)p.y;
     a.M = (int)p.M, a.K = (int)p.K, a.N = (int)p.N;
     a.total_bytes = (size_t)p.N * (size_t)(p.K / be) * (size_t)bb;
-    const char *env = "OXQ_GGUF_MM";
     const bool hilo = p.M <= 8;  // the decode range (GgufQuantMatmul): weights are not rounded to bf16
 #define OXQ_GG(F, NAME) \
-    case F: return launch_mm_src<GgufSource<F>>(ctx, s, a, NAME, env, hilo)
+    case F: return launch_mm_src<GgufSource<F>>(ctx, s, a, NAME, OXQ_TUNE_GGUF_MM_MT, OXQ_TUNE_GGUF_MM_KS, hilo)
     switch (p.quant) {
         OXQ_GG(OXQ_GGUF_Q4_0, "gguf_q4_0");
         OXQ_GG(OXQ_GGUF_Q8_0, "gguf_q8_0");
@@ -495,12 +491,11 @@ int launch_mxfp4_mm(oxq_ctx *ctx, hipStream_t s, const Mxfp4Problem &p) {
     }
     if (!ctx->plan_only && (((uintptr_t)p.blocks & 15) || ((uintptr_t)p.x & 15)))
         return fail(OXQ_ERR_UNSUPPORTED, "mxfp4 mul_mm: blocks and x must be 16-byte aligned");
-    return launch_mm_src<Mxfp4Source>(ctx, s, a, grouped ? "mxfp4_moe" : "mxfp4", "OXQ_MXFP4_MM");
+    return launch_mm_src<Mxfp4Source>(ctx, s, a, grouped ? "mxfp4_moe" : "mxfp4", OXQ_TUNE_MXFP4_MM_MT, OXQ_TUNE_MXFP4_MM_KS);
 }
 
-bool f8_mm_eligible(const F8Problem &p) {
-    const char *e = getenv("OXQ_F8_MM_MIN_M");
-    const int min_m = e ? atoi(e) : 3;  // measured 4096^2 at m = 8: GEMV 19.9 us, tile matmul 11.5 us
+bool f8_mm_eligible(const oxq_ctx *ctx, const F8Problem &p) {
+    const int min_m = tune(ctx, OXQ_TUNE_F8_MM_MIN_M, 3);  // measured 4096^2 at m = 8: GEMV 19.9 us, tile matmul 11.5 us
     return p.M >= min_m && p.K % 32 == 0 && p.block_c % 32 == 0 && ((uintptr_t)p.x & 15) == 0 &&
            ((uintptr_t)p.w & 15) == 0;
 }
@@ -511,7 +506,7 @@ int launch_f8_mm(oxq_ctx *ctx, hipStream_t s, const F8Problem &p) {
     a.M = (int)p.M, a.K = (int)p.K, a.N = (int)p.N;
     a.f8_scales = p.scales, a.f8_block_r = (int)p.block_r, a.f8_block_c = (int)p.block_c;
     a.f8_s_cols = (int)p.s_cols;
-    return launch_mm_src<F8Source>(ctx, s, a, "f8", "OXQ_F8_MM");
+    return launch_mm_src<F8Source>(ctx, s, a, "f8", OXQ_TUNE_F8_MM_MT, OXQ_TUNE_F8_MM_KS);
 }
 
 }  // namespace oxq

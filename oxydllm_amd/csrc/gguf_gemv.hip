@@ -398,14 +398,13 @@ static int launch_rows_lds_mb(hipStream_t s, const GgufProblem &p, const uint8_t
 }
 
 template <int FMT, bool BF16X>
-static int launch_rows_lds(hipStream_t s, const GgufProblem &p, const uint8_t *x, uint8_t *y, int rows,
-                           int rpwg, size_t lds) {
+static int launch_rows_lds(const oxq_ctx *ctx, hipStream_t s, const GgufProblem &p, const uint8_t *x, uint8_t *y,
+                           int rows, int rpwg, size_t lds) {
     if (rows <= 1) {
         // a wave per weight row needs: 8 waves for the 8 rows, the row in 6 chunks a lane, x in one batch
         const size_t row_bytes = (size_t)(p.K / GgufFmt<FMT>::BE) * GgufFmt<FMT>::BB;
-        const char *pw_env = getenv("OXQ_GGUF_PW");
         if ((rpwg == 8 || rpwg == 16) && row_bytes + 30 <= 6 * 64 * 16 &&
-            p.K * (BF16X ? 2 : 4) / 16 <= 4 * 64 * rpwg && !(pw_env && atoi(pw_env) == 0))
+            p.K * (BF16X ? 2 : 4) / 16 <= 4 * 64 * rpwg && tune(ctx, OXQ_TUNE_GGUF_PW, 1) != 0)
             return launch_rows_lds_mb<FMT, BF16X, 1, true>(s, p, x, y, rows, rpwg, lds);
         return launch_rows_lds_mb<FMT, BF16X, 1>(s, p, x, y, rows, rpwg, lds);
     }
@@ -424,12 +423,8 @@ int launch_gguf_gemv(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p) {
     const bool bf = p.act_dtype == OXQ_BF16;
     const size_t xb = bf ? 2 : 4;
     const size_t row_bytes = gguf_row_bytes(p.quant, p.K);
-    const char *rp_env = getenv("OXQ_GGUF_RPWG");
-    const char *pw_env = getenv("OXQ_GGUF_PW");
-    const char *big_env = getenv("OXQ_GGUF_BIG_LDS");
-    const char *force = getenv("OXQ_FORCE_GENERIC");
     const bool aligned = ((uintptr_t)p.x & 15) == 0 && ((uintptr_t)p.w & 15) == 0 && (p.K * xb) % 16 == 0 &&
-                         !(force && atoi(force));
+                         !tune(ctx, OXQ_TUNE_FORCE_GENERIC, 0);
     // The staged kernel for `mb` activation rows a pass: x (per row K/32 units of 32 elements + one 16-byte
     // pad each, then two sums a unit) and `rpwg` weight rows in LDS.  8 rows on 8 waves; for one activation
     // row OXQ_GGUF_RPWG=16 runs 16 rows on 16 waves, which halves the activation traffic (every workgroup
@@ -445,15 +440,15 @@ int launch_gguf_gemv(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p) {
     };
     auto staged = [&](int mb) -> Staged {
         const size_t x_lds = (size_t)mb * ((((size_t)(p.K >> 5) * ((32 * xb / 16 + 1) * 16 + 8)) + 15) & ~(size_t)15);
-        const bool wave_per_row = mb == 1 && row_bytes + 30 <= 6 * 64 * 16 && !(pw_env && atoi(pw_env) == 0);
-        int rpwg = rp_env ? atoi(rp_env) : 8;
+        const bool wave_per_row = mb == 1 && row_bytes + 30 <= 6 * 64 * 16 && tune(ctx, OXQ_TUNE_GGUF_PW, 1) != 0;
+        int rpwg = tune(ctx, OXQ_TUNE_GGUF_RPWG, 8);
         if (rpwg < 1) rpwg = 1;
         if (rpwg > 8 && !(wave_per_row && rpwg == 16 && p.K * (int64_t)xb / 16 <= 4 * 64 * 16)) rpwg = 8;
         const int rp0 = rpwg;
         auto lds_cap_of = [](int r) { return (size_t)(r == 16 ? 128 : 64) * 1024; };
         while (rpwg > 1 && x_lds + (size_t)rpwg * row_bytes + 32 > lds_cap_of(rpwg)) rpwg >>= 1;
         size_t cap = lds_cap_of(rpwg);
-        if ((rpwg < 4 || x_lds + (size_t)rpwg * row_bytes + 32 > cap) && rp0 >= 8 && !(big_env && atoi(big_env) == 0) &&
+        if ((rpwg < 4 || x_lds + (size_t)rpwg * row_bytes + 32 > cap) && rp0 >= 8 && tune(ctx, OXQ_TUNE_GGUF_BIG_LDS, 1) != 0 &&
             x_lds + (size_t)8 * row_bytes + 32 <= (size_t)150 * 1024)
             rpwg = 8, cap = (size_t)150 * 1024;
         const size_t lds = x_lds + (size_t)rpwg * row_bytes + 32;
@@ -485,8 +480,8 @@ int launch_gguf_gemv(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p) {
         uint8_t *y = (uint8_t *)p.y + (size_t)m0 * p.N * xb;
 #define OXQ_FMT(F)                                                                  \
     if (use_lds) {                                                                  \
-        int rc = bf ? launch_rows_lds<F, true>(s, p, x, y, rows, rpwg, lds)         \
-                    : launch_rows_lds<F, false>(s, p, x, y, rows, rpwg, lds);       \
+        int rc = bf ? launch_rows_lds<F, true>(ctx, s, p, x, y, rows, rpwg, lds)         \
+                    : launch_rows_lds<F, false>(ctx, s, p, x, y, rows, rpwg, lds);       \
         if (rc != OXQ_OK) return rc;                                                \
     } else if (bf) launch_rows<F, true>(s, grid, p, x, y, rows);                    \
     else launch_rows<F, false>(s, grid, p, x, y, rows)

@@ -689,12 +689,11 @@ size_t gguf_res_bytes(int quant, int64_t K, int64_t N) {
     return (size_t)N * (size_t)(K / be) * (size_t)bb;
 }
 
-static int ggr_waves(int64_t K) {
-    const char *e = getenv("OXQ_GGR_WAVES");
-    const int w = e ? atoi(e) : 16;
+static int ggr_waves(const oxq_ctx *ctx, int64_t K) {
+    const int w = tune(ctx, OXQ_TUNE_GGR_WAVES, 16);
     return (w == 8 || K / 128 < 16) ? 8 : 16;
 }
-static size_t ggr_lds_bytes(int64_t K, int mb) { return (size_t)2 * 4 * ggr_waves(K) * mb * 16 * 4; }
+static size_t ggr_lds_bytes(const oxq_ctx *ctx, int64_t K, int mb) { return (size_t)2 * 4 * ggr_waves(ctx, K) * mb * 16 * 4; }
 // rows of x one launch of the resident GEMV takes (more go to the kernels on the file layout)
 // (8 rows in one pass need more registers than a wave of a 16-wave workgroup has: measured 14.8 us on
 // 4096 x 4096 Q4_0 against 6.3 us at 4 rows)
@@ -792,10 +791,9 @@ static int ggr_by_rows(hipStream_t s, dim3 grid, const GgufProblem &p, size_t ld
 int launch_gguf_res_gemv(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p0) {
     const int64_t rows0 = std::min<int64_t>(p0.M, 4);
     const int mb = rows0 <= 1 ? 1 : rows0 <= 2 ? 2 : 4;
-    const int nw = ggr_waves(p0.K);
-    const size_t lds = ggr_lds_bytes(p0.K, mb);
-    const char *ge = getenv("OXQ_GGR_GRID");
-    const int64_t cap = ge ? atoi(ge) : (nw == 8 ? 512 : 256);
+    const int nw = ggr_waves(ctx, p0.K);
+    const size_t lds = ggr_lds_bytes(ctx, p0.K, mb);
+    const int64_t cap = tune(ctx, OXQ_TUNE_GGR_GRID, nw == 8 ? 512 : 256);
     dim3 grid((unsigned)std::min<int64_t>(p0.N / 16, cap > 0 ? cap : p0.N / 16));
     char name[64];
     snprintf(name, sizeof name, "gguf_%s_res_gemv_%s_m%d", ggr_name(p0.quant), p0.act_dtype == OXQ_BF16 ? "bf16" : "f32", mb);

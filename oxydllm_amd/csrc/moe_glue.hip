@@ -494,8 +494,7 @@ int launch_gated_activation(oxq_ctx *ctx, hipStream_t s, const void *gu, void *o
     if (ctx->plan_only || n_out == 0) return OXQ_OK;
     // from 64 K vectors on (two workgroups a CU): below, one output a thread spreads the work wider and
     // is faster (decode: 2.0 against 2.5 us; 2048 x 2880 outputs: 13.1 against 10.2 us)
-    const char *vec_env = getenv("OXQ_ACT_VEC");
-    const size_t vec_min = vec_env ? (size_t)atoll(vec_env) : (size_t)65536;
+    const size_t vec_min = (size_t)std::max(0, tune(ctx, OXQ_TUNE_ACT_VEC, 65536));
     if (dtype != OXQ_F32 && half_n % 8 == 0 && (((uintptr_t)gu | (uintptr_t)out) & 15) == 0 && n_out / 8 >= vec_min) {
         const size_t n_vec = n_out / 8;
         dim3 vgrid((unsigned)ceil_div((int64_t)n_vec, 256));

@@ -742,8 +742,7 @@ int launch_mxfp4_gemv(oxq_ctx *ctx, hipStream_t s, const Mxfp4Problem &p) {
     {
         // prefill sizes go to the tile matmul, which converts a weight once per 64 tokens
         // instead of once per pass of 16 (4 grouped) tokens
-        const char *mm = getenv("OXQ_MXFP4_MM");
-        const int mm_mode = mm ? atoi(mm) : -1;  // 0 = never, 1 = always, default by size
+        const int mm_mode = tune(ctx, OXQ_TUNE_MXFP4_MM, -1);  // 0 = never, 1 = always, default by size
         // plain form, measured on one expert's gate_up: m = 8 9.3 / 8.6 us, m = 16 11.8 / 8.7 us
         const bool big = grouped ? p.n_pairs >= 8 * p.n_experts : p.M >= 8;
         if ((mm_mode == 1 || (mm_mode != 0 && big)) && p.K % 32 == 0)
@@ -751,11 +750,9 @@ int launch_mxfp4_gemv(oxq_ctx *ctx, hipStream_t s, const Mxfp4Problem &p) {
     }
     {
         // matrix-core form: tokens staged in LDS (MTOK per pass), 4 waves x FR x 16 rows per workgroup
-        const char *v = getenv("OXQ_MXFP4_VARIANT");
-        const int variant = v ? atoi(v) : 0;  // 0 = matrix cores, 1 = dot2 with staged tokens, 2 = one wave per row
+        const int variant = tune(ctx, OXQ_TUNE_MXFP4_VARIANT, 0);  // 0 = matrix cores, 1 = dot2 with staged tokens, 2 = one wave per row
         const int mtok = (grouped || p.M <= 4) ? 4 : 16;
-        const char *frs = getenv("OXQ_MXFP4_FR");
-        int FR = frs ? atoi(frs) : 1;
+        int FR = tune(ctx, OXQ_TUNE_MXFP4_FR, 1);
         FR = FR >= 4 ? 4 : FR >= 2 ? 2 : 1;  // the instantiated fragment counts
         // tokens, then the four waves' scale bytes (16 * FR rows of K / 32 bytes, + alignment slack)
         const size_t lds = (size_t)mtok * (size_t)p.K * 2 + 4 * ((size_t)16 * FR * (size_t)(p.K >> 5) + 16);
@@ -779,8 +776,7 @@ int launch_mxfp4_gemv(oxq_ctx *ctx, hipStream_t s, const Mxfp4Problem &p) {
     const int mb = rows_hint <= 1 ? 1 : rows_hint <= 2 ? 2 : rows_hint <= 4 ? 4 : 8;
     constexpr int RW = 8;
     const size_t lds = (size_t)mb * 4 * (size_t)((p.K >> 5) + 1) * 16;
-    const char *force = getenv("OXQ_FORCE_GENERIC");
-    const bool use_lds = lds <= 96 * 1024 && !(force && atoi(force)) && !force_rows;
+    const bool use_lds = lds <= 96 * 1024 && !tune(ctx, OXQ_TUNE_FORCE_GENERIC, 0) && !force_rows;
     if (use_lds) {
         dim3 grid((unsigned)ceil_div(p.N, 4 * RW), grouped ? (unsigned)p.n_experts : 1u), block(256);
         char name[64];

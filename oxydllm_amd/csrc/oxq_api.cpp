@@ -3,6 +3,7 @@
 // routing to the kernel launchers.
 
 #include "oxq_internal.hpp"
+#include "oxq_bench.h"
 
 #include <cstdlib>
 #include <new>
@@ -408,7 +409,8 @@ struct oxq_mxfp4_experts {
     oxq_tensor blocks, scales, bias;  // the caller's tensors (prefill sizes and ineligible shapes run on them)
     bool has_bias;
     int64_t n_experts, k, n;
-    void *pw, *ps;                    // resident tile-major copy, owned; null when the shape does not qualify
+    void *pw, *ps;                    // resident tile-major copy; null when the shape does not qualify
+    bool owns;                        // pw / ps are device allocations of this handle (not a plan-only ctx's stand-ins)
 };
 
 // =============================================================================
@@ -463,6 +465,47 @@ int oxq_gguf_block_layout(int quant, int64_t *block_elems, int64_t *block_bytes)
     return OXQ_OK;
 }
 
+// Names of the tuning switches: OXQ_<name> as an environment variable and as the key of oxq_ctx_set_tuning.
+static const char *const kTuneNames[OXQ_TUNE_COUNT] = {
+#define OXQ_TUNE_NAME(n) "OXQ_" #n,
+    OXQ_TUNE_LIST(OXQ_TUNE_NAME)
+#undef OXQ_TUNE_NAME
+};
+
+static int tune_from_env(int key) {
+    const char *v = getenv(kTuneNames[key]);
+    return (v && *v) ? atoi(v) : OXQ_TUNE_UNSET;
+}
+
+static int tune_key_of(const char *name) {
+    if (!name) return -1;
+    for (int k = 0; k < OXQ_TUNE_COUNT; ++k)
+        if (strcmp(name, kTuneNames[k]) == 0) return k;
+    return -1;
+}
+
+int oxq_ctx_set_tuning(oxq_ctx *ctx, const char *name, int value) {
+    if (!ctx) return fail(OXQ_ERR_ARG, "oxq_ctx_set_tuning: ctx is NULL");
+    const int k = tune_key_of(name);
+    if (k < 0) return fail(OXQ_ERR_ARG, "oxq_ctx_set_tuning: unknown switch '%s'", name ? name : "(null)");
+    ctx->tuning[k] = value;
+    if (k == OXQ_TUNE_SPLITK_MODE) ctx->splitk_mode = value;
+    return OXQ_OK;
+}
+
+int oxq_ctx_reset_tuning(oxq_ctx *ctx, const char *name) {
+    if (!ctx) return fail(OXQ_ERR_ARG, "oxq_ctx_reset_tuning: ctx is NULL");
+    if (name) {
+        const int k = tune_key_of(name);
+        if (k < 0) return fail(OXQ_ERR_ARG, "oxq_ctx_reset_tuning: unknown switch '%s'", name);
+        ctx->tuning[k] = tune_from_env(k);
+    } else {
+        for (int k = 0; k < OXQ_TUNE_COUNT; ++k) ctx->tuning[k] = tune_from_env(k);
+    }
+    ctx->splitk_mode = tune(ctx, OXQ_TUNE_SPLITK_MODE, 0);
+    return OXQ_OK;
+}
+
 int oxq_ctx_create(int device, oxq_ctx **out) {
     if (!out) return fail(OXQ_ERR_ARG, "oxq_ctx_create: out is NULL");
     *out = nullptr;
@@ -476,10 +519,8 @@ int oxq_ctx_create(int device, oxq_ctx **out) {
     const size_t ws_mb = (ws_env && atoi(ws_env) > 0) ? (size_t)atoi(ws_env) : 64;
     ctx->workspace_bytes = ws_mb << 20;
     ctx->n_counters = 16384;
-    {
-        const char *m = getenv("OXQ_SPLITK_MODE");
-        ctx->splitk_mode = (m && *m) ? atoi(m) : 0;
-    }
+    for (int k = 0; k < OXQ_TUNE_COUNT; ++k) ctx->tuning[k] = tune_from_env(k);
+    ctx->splitk_mode = tune(ctx, OXQ_TUNE_SPLITK_MODE, 0);
     {
         const char *m = getenv("OXQ_WEIGHT_CACHE_MB");
         ctx->wcache_limit = (m && atoi(m) > 0) ? (size_t)atoi(m) << 20 : 0;
@@ -577,6 +618,40 @@ int oxq_calib_read(oxq_ctx *ctx, void *stream, const oxq_tensor *src, int workgr
                              nontemporal, (uint32_t *)checksums->data);
 }
 
+int oxq_bench_read_upfront(oxq_ctx *ctx, void *stream, const oxq_tensor *src, int workgroups, int waves,
+                           int nontemporal, const oxq_tensor *checksums) {
+    if (!ctx || !src || !checksums) return fail(OXQ_ERR_ARG, "ReadUpfront: NULL argument");
+    OXQ_TRY(check_tensor(ctx, "ReadUpfront", "src", src));
+    OXQ_TRY(check_tensor(ctx, "ReadUpfront", "checksums", checksums));
+    if (src->dtype != OXQ_U8 || !src->contiguous)
+        return fail(OXQ_ERR_DTYPE, "ReadUpfront: src must be a contiguous U8 tensor, got %s", dtype_name(src->dtype));
+    if ((checksums->dtype != OXQ_U32 && checksums->dtype != OXQ_I32) || !checksums->contiguous)
+        return fail(OXQ_ERR_DTYPE, "ReadUpfront: checksums must be a contiguous U32/I32 tensor, got %s",
+                    dtype_name(checksums->dtype));
+    const int64_t bytes = numel(src);
+    if (waves != 8 && waves != 16) return fail(OXQ_ERR_ARG, "ReadUpfront: %d waves a workgroup (8 or 16)", waves);
+    if (workgroups < 1 || workgroups > 65535 || numel(checksums) < workgroups)
+        return fail(OXQ_ERR_SHAPE, "ReadUpfront: %d workgroups need 1..65535 and one checksum word each (got %lld)",
+                    workgroups, (long long)numel(checksums));
+    const int64_t per_wave = (int64_t)workgroups * waves * 1024;
+    if (bytes <= 0 || bytes % per_wave != 0 || bytes / per_wave > 32)
+        return fail(OXQ_ERR_SHAPE, "ReadUpfront: %lld bytes over %d workgroups of %d waves: every wave reads 1 .. 32 KiB "
+                    "in whole KiB", (long long)bytes, workgroups, waves);
+    if (!ctx->plan_only && ((uintptr_t)src->data & 15))
+        return fail(OXQ_ERR_UNSUPPORTED, "ReadUpfront: src must be 16-byte aligned");
+    return launch_calib_upfront(ctx, (hipStream_t)stream, (const uint8_t *)src->data, (uint64_t)bytes, workgroups, waves,
+                                nontemporal, (uint32_t *)checksums->data);
+}
+
+int oxq_bench_empty_launch(oxq_ctx *ctx, void *stream, int workgroups, int threads, int lds_bytes) {
+    if (!ctx) return fail(OXQ_ERR_ARG, "EmptyLaunch: ctx is NULL");
+    if (workgroups < 1 || workgroups > 65535 || threads < 64 || threads > 1024 || threads % 64 != 0 || lds_bytes < 0 ||
+        lds_bytes > 160 * 1024)
+        return fail(OXQ_ERR_ARG, "EmptyLaunch: %d workgroups of %d threads with %d bytes of LDS", workgroups, threads,
+                    lds_bytes);
+    return launch_empty(ctx, (hipStream_t)stream, workgroups, threads, lds_bytes);
+}
+
 // ---- opt-in cache of tile-major weight copies behind the stateless ops ---------------------------
 // The reference's ops are called with the same resident tensors on every forward (linear.rs:482-533
 // passes the layer's own qweight / qzeros / scales).  A caller that swaps in only the op functions,
@@ -593,6 +668,7 @@ struct oxq_weight_cache {
         Pk4Weights w;
         size_t bytes;
         uint64_t last_use;
+        bool pinned;  // a captured graph holds this copy's address: only forget / destroy may free it
     };
     std::vector<Entry> entries;
     size_t bytes = 0;
@@ -622,6 +698,36 @@ static void wcache_destroy(oxq_ctx *ctx) {
     ctx->wcache = nullptr;
 }
 
+// Makes room for `bytes` more.  Least recently used copies go first, except those a captured graph may hold
+// (pinned) and those used within the last entries + 1 calls: when the working set is larger than the limit,
+// evicting what the next calls will ask for again would rebuild a copy on every call - far slower than the
+// checkpoint-layout kernel the copy replaces - so the newcomer takes that kernel instead and the copies stay.
+// False: no room.  (hipFree, which a dropped copy costs, waits for the device.)
+static bool wcache_make_room(oxq_ctx *ctx, size_t bytes) {
+    oxq_weight_cache *c = ctx->wcache;
+    if (bytes > ctx->wcache_limit) return false;
+    while (c->bytes + bytes > ctx->wcache_limit) {
+        size_t lru = c->entries.size();
+        for (size_t i = 0; i < c->entries.size(); ++i)
+            if (!c->entries[i].pinned && (lru == c->entries.size() || c->entries[i].last_use < c->entries[lru].last_use)) lru = i;
+        if (lru == c->entries.size()) return false;
+        if (c->tick - c->entries[lru].last_use <= c->entries.size() + 1) return false;
+        wcache_drop(ctx, lru);
+    }
+    return true;
+}
+
+// A hit while the stream is being captured puts the copy's address into the graph: from then on the copy stays
+// until the caller forgets the weight or destroys the ctx (either of which invalidates that graph).
+static void wcache_pin_if_capturing(hipStream_t s, oxq_weight_cache::Entry *e) {
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &cs) != hipSuccess) {
+        (void)hipGetLastError();
+        return;
+    }
+    if (cs != hipStreamCaptureStatusNone) e->pinned = true;
+}
+
 // true: the call was served (rc holds its status).  false: take the checkpoint-layout path.
 static bool wcache_forward(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p, int *rc) {
     if (!ctx->wcache_limit || ctx->plan_only || !pk4_eligible(p)) return false;
@@ -631,6 +737,7 @@ static bool wcache_forward(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p, i
         if (!ctx->wcache) return false;
     }
     oxq_weight_cache *c = ctx->wcache;
+    ++c->tick;  // one tick a call, hit or not: an entry's age is counted in calls
     oxq_weight_cache::Entry *hit = nullptr;
     for (auto &e : c->entries)
         if (e.qw == p.qweight && e.qz == p.qzeros && e.sc == p.scales && e.K == p.K && e.N == p.N &&
@@ -646,13 +753,7 @@ static bool wcache_forward(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p, i
             return false;
         }
         const size_t bytes = (pk4_weight_bytes(p.K, p.N, p.bits) + 255) & ~(size_t)255;
-        if (bytes > ctx->wcache_limit) return false;
-        while (c->bytes + bytes > ctx->wcache_limit && !c->entries.empty()) {  // least recently used first
-            size_t lru = 0;
-            for (size_t i = 1; i < c->entries.size(); ++i)
-                if (c->entries[i].last_use < c->entries[lru].last_use) lru = i;
-            wcache_drop(ctx, lru);
-        }
+        if (!wcache_make_room(ctx, bytes)) return false;
         void *mem = nullptr;
         if (hipMalloc(&mem, bytes) != hipSuccess) {
             (void)hipGetLastError();
@@ -660,8 +761,8 @@ static bool wcache_forward(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p, i
         }
         oxq_weight_cache::Entry e{p.qweight, p.qzeros, p.scales, p.K, p.N, p.group_shift, p.dtype, p.bits, p.pack_dim,
                                   Pk4Weights{(uint32_t *)mem, nullptr, p.K, p.N, p.group_shift, p.dtype, p.bits, 0,
-                                             p.pack_dim == OXQ_PACK_IN ? 32 : 16, pk4_choose_strip(p.K, p.N, p.bits, 0)},
-                                  bytes, 0};
+                                             p.pack_dim == OXQ_PACK_IN ? 32 : 16, pk4_choose_strip(ctx, p.K, p.N, p.bits, 0)},
+                                  bytes, 0, false};
         const int prc = launch_pk4_prepack(ctx, s, p, e.w);  // on the caller's stream, ahead of the matmul
         if (prc != OXQ_OK) {
             (void)hipFree(mem);
@@ -677,7 +778,8 @@ static bool wcache_forward(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p, i
         c->bytes += bytes;
         hit = &c->entries.back();
     }
-    hit->last_use = ++c->tick;
+    hit->last_use = c->tick;
+    wcache_pin_if_capturing(s, hit);
     Pk4Problem q;
     q.x = p.x;
     q.bias = p.bias;
@@ -701,6 +803,7 @@ static bool wcache_forward_gguf(oxq_ctx *ctx, hipStream_t s, const GgufProblem &
         if (!ctx->wcache) return false;
     }
     oxq_weight_cache *c = ctx->wcache;
+    ++c->tick;
     oxq_weight_cache::Entry *hit = nullptr;
     for (auto &e : c->entries)
         if (e.qw == p.w && e.qz == nullptr && e.sc == nullptr && e.K == p.K && e.N == p.N && e.bits == p.quant &&
@@ -715,20 +818,14 @@ static bool wcache_forward_gguf(oxq_ctx *ctx, hipStream_t s, const GgufProblem &
             return false;
         }
         const size_t bytes = (gguf_res_bytes(p.quant, p.K, p.N) + 255) & ~(size_t)255;
-        if (bytes > ctx->wcache_limit) return false;
-        while (c->bytes + bytes > ctx->wcache_limit && !c->entries.empty()) {
-            size_t lru = 0;
-            for (size_t i = 1; i < c->entries.size(); ++i)
-                if (c->entries[i].last_use < c->entries[lru].last_use) lru = i;
-            wcache_drop(ctx, lru);
-        }
+        if (!wcache_make_room(ctx, bytes)) return false;
         void *mem = nullptr;
         if (hipMalloc(&mem, bytes) != hipSuccess) {
             (void)hipGetLastError();
             return false;
         }
         oxq_weight_cache::Entry e{p.w, nullptr, nullptr, p.K, p.N, 0, 0, p.quant, -1,
-                                  Pk4Weights{(uint32_t *)mem, nullptr, p.K, p.N, 0, 0, 0, 0, 0, 0}, bytes, 0};
+                                  Pk4Weights{(uint32_t *)mem, nullptr, p.K, p.N, 0, 0, 0, 0, 0, 0}, bytes, 0, false};
         const int prc = launch_gguf_res_repack(ctx, s, p.quant, p.w, mem, p.K, p.N);
         if (prc != OXQ_OK) {
             (void)hipFree(mem);
@@ -744,7 +841,8 @@ static bool wcache_forward_gguf(oxq_ctx *ctx, hipStream_t s, const GgufProblem &
         c->bytes += bytes;
         hit = &c->entries.back();
     }
-    hit->last_use = ++c->tick;
+    hit->last_use = c->tick;
+    wcache_pin_if_capturing(s, hit);
     GgufProblem q = p;
     q.w = (const uint8_t *)hit->w.pw;
     *rc = launch_gguf_res_gemv(ctx, s, q);
@@ -759,10 +857,14 @@ int oxq_ctx_set_weight_cache(oxq_ctx *ctx, int64_t max_bytes) {
         int prev = 0;
         (void)hipGetDevice(&prev);
         (void)hipSetDevice(ctx->device);
-        while (ctx->wcache->bytes > ctx->wcache_limit && !ctx->wcache->entries.empty()) {
-            size_t lru = 0;
-            for (size_t i = 1; i < ctx->wcache->entries.size(); ++i)
-                if (ctx->wcache->entries[i].last_use < ctx->wcache->entries[lru].last_use) lru = i;
+        // copies a captured graph may hold stay (and count against the limit) until they are forgotten
+        while (ctx->wcache->bytes > ctx->wcache_limit) {
+            const size_t n = ctx->wcache->entries.size();
+            size_t lru = n;
+            for (size_t i = 0; i < n; ++i)
+                if (!ctx->wcache->entries[i].pinned &&
+                    (lru == n || ctx->wcache->entries[i].last_use < ctx->wcache->entries[lru].last_use)) lru = i;
+            if (lru == n) break;
             wcache_drop(ctx, lru);
         }
         (void)hipSetDevice(prev);
@@ -927,7 +1029,7 @@ int oxq_gguf_quant_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x,
                        out_features, quant, out, &p));
     int rc = OXQ_OK;
     if (wcache_forward_gguf(ctx, (hipStream_t)stream, p, &rc)) return rc;
-    if (gguf_mm_eligible(p)) return launch_gguf_mm(ctx, (hipStream_t)stream, p);
+    if (gguf_mm_eligible(ctx, p)) return launch_gguf_mm(ctx, (hipStream_t)stream, p);
     return launch_gguf_gemv(ctx, (hipStream_t)stream, p);
 }
 
@@ -937,7 +1039,7 @@ int oxq_gguf_quant_mul_mm(oxq_ctx *ctx, void *stream, const oxq_tensor *x,
     GgufProblem p;
     OXQ_TRY(check_gguf(ctx, "GgufQuantMulMM", false, false, x, weight_bytes, in_features,
                        out_features, quant, out, &p));
-    if (gguf_mm_eligible(p)) return launch_gguf_mm(ctx, (hipStream_t)stream, p);
+    if (gguf_mm_eligible(ctx, p)) return launch_gguf_mm(ctx, (hipStream_t)stream, p);
     return launch_gguf_gemv(ctx, (hipStream_t)stream, p);
 }
 
@@ -1211,7 +1313,7 @@ int oxq_f8_gemv(oxq_ctx *ctx, void *stream, const oxq_tensor *x, const oxq_tenso
                 const oxq_tensor *scales, const oxq_tensor *out) {
     F8Problem p;
     OXQ_TRY(check_f8(ctx, "f8-gemv", x, bytes, scales, out, true, &p));
-    if (f8_mm_eligible(p)) return launch_f8_mm(ctx, (hipStream_t)stream, p);
+    if (f8_mm_eligible(ctx, p)) return launch_f8_mm(ctx, (hipStream_t)stream, p);
     return launch_f8_gemv(ctx, (hipStream_t)stream, p);
 }
 
@@ -1221,7 +1323,7 @@ int oxq_f8_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x, const oxq_ten
                   const oxq_tensor *scales, const oxq_tensor *out) {
     F8Problem p;
     OXQ_TRY(check_f8(ctx, "f8-matmul", x, bytes, scales, out, false, &p));
-    if (f8_mm_eligible(p)) return launch_f8_mm(ctx, (hipStream_t)stream, p);
+    if (f8_mm_eligible(ctx, p)) return launch_f8_mm(ctx, (hipStream_t)stream, p);
     return launch_f8_gemv(ctx, (hipStream_t)stream, p);
 }
 
@@ -1351,8 +1453,8 @@ int oxq_mxfp4_experts_new(oxq_ctx *ctx, const oxq_tensor *blocks, const oxq_tens
     h->k = k;
     h->n = n;
     h->pw = h->ps = nullptr;
-    const char *env = getenv("OXQ_PREPACK");
-    const bool want = !(env && atoi(env) == 0) && mxfp4_res_eligible(k, n) && !((uintptr_t)blocks->data & 15);
+    h->owns = false;
+    const bool want = tune(ctx, OXQ_TUNE_PREPACK, 1) != 0 && mxfp4_res_eligible(k, n) && !((uintptr_t)blocks->data & 15);
     if (want && !ctx->plan_only) {
         int prev = 0;
         (void)hipGetDevice(&prev);
@@ -1375,6 +1477,7 @@ int oxq_mxfp4_experts_new(oxq_ctx *ctx, const oxq_tensor *blocks, const oxq_tens
             delete h;
             return rc;
         }
+        h->owns = true;
     } else if (want) {
         h->pw = h->ps = (void *)16;  // plan-only: routes as a resident copy would, nothing is dereferenced
     }
@@ -1468,7 +1571,7 @@ int oxq_mxfp4_experts_dequantize(oxq_mxfp4_experts *h, void *stream, int64_t exp
 
 void oxq_mxfp4_experts_free(oxq_mxfp4_experts *h) {
     if (!h) return;
-    if (!h->ctx->plan_only) {
+    if (h->owns) {  // by the handle's own flag: the experts may outlive their ctx
         if (h->pw) (void)hipFree(h->pw);
         if (h->ps) (void)hipFree(h->ps);
     }
@@ -1717,9 +1820,8 @@ struct oxq_packed_quant_linear {
 // not cover simply keep the checkpoint layout; errors in the tensors themselves
 // surface at forward, where the reference reports them.
 static int prepack_layer(oxq_packed_quant_linear *l) {
-    const char *env = getenv("OXQ_PREPACK");
-    if (env && atoi(env) == 0) return OXQ_OK;
     oxq_ctx *ctx = l->ctx;
+    if (tune(ctx, OXQ_TUNE_PREPACK, 1) == 0) return OXQ_OK;
     oxq_tensor shape_only = l->scales;  // [K, N] descriptor for the shape checks, never written
     shape_only.rank = 2;
     shape_only.dims[0] = l->in_features;
@@ -1737,7 +1839,7 @@ static int prepack_layer(oxq_packed_quant_linear *l) {
     l->pk.bits = src.bits;
     l->pk.gate_half = l->act ? src.N / 2 : 0;
     l->pk.gemv_rows = src.pack_dim == OXQ_PACK_IN ? 32 : 16;
-    l->pk.strip = pk4_choose_strip(src.K, src.N, src.bits, l->pk.gate_half);
+    l->pk.strip = pk4_choose_strip(l->ctx, src.K, src.N, src.bits, l->pk.gate_half);
     if (ctx->plan_only) {
         l->prepacked = true;
         return OXQ_OK;
@@ -1773,8 +1875,7 @@ struct oxq_qlinear {
 
 // linear.rs:225-240: the fast path copies the block bytes at build; here the copy is strip-major
 static int build_resident_gguf(oxq_qlinear *l) {
-    const char *env = getenv("OXQ_PREPACK");
-    if (env && atoi(env) == 0) return OXQ_OK;
+    if (tune(l->ctx, OXQ_TUNE_PREPACK, 1) == 0) return OXQ_OK;
     if (!gguf_res_eligible(l->quant, l->in_features, l->out_features)) return OXQ_OK;
     if (((uintptr_t)l->weight_bytes.data & 1) != 0) return OXQ_OK;
     oxq_ctx *ctx = l->ctx;
@@ -2033,7 +2134,7 @@ int oxq_qlinear_forward(oxq_qlinear *l, void *stream, const oxq_tensor *x, const
         p.w = (const uint8_t *)l->res;
         return launch_gguf_res_gemv(l->ctx, (hipStream_t)stream, p);
     }
-    if (gguf_mm_eligible(p)) return launch_gguf_mm(l->ctx, (hipStream_t)stream, p);
+    if (gguf_mm_eligible(l->ctx, p)) return launch_gguf_mm(l->ctx, (hipStream_t)stream, p);
     return launch_gguf_gemv(l->ctx, (hipStream_t)stream, p);
 }
 
@@ -2050,6 +2151,7 @@ int oxq_qlinear_dequantize(oxq_qlinear *l, void *stream, const oxq_tensor *out) 
     if (out->dtype != OXQ_F32 || out->rank != 2 || out->dims[0] != l->out_features || out->dims[1] != l->in_features)
         return fail(OXQ_ERR_SHAPE, "%s: out must be F32 [%lld, %lld]", op, (long long)l->out_features,
                     (long long)l->in_features);
+    if (!out->contiguous) return fail(OXQ_ERR_CONTIGUOUS, "%s: out must be contiguous", op);
     if (l->resident)
         return launch_gguf_res_dequant(l->ctx, (hipStream_t)stream, l->quant, l->res, l->in_features, l->out_features,
                                        (float *)out->data);

@@ -13,6 +13,23 @@
 
 #include "oxq.h"
 
+// Tuning switches.  Each is read from the environment variable OXQ_<name> once, when a ctx is created,
+// and can be set per ctx with oxq_ctx_set_tuning; the launchers only ever look at the ctx, so a forward
+// call costs no getenv and two engine threads cannot race on the process environment.
+#define OXQ_TUNE_LIST(X)                                                                                      \
+    X(ACT_VEC) X(F8_MM_KS) X(F8_MM_MIN_M) X(F8_MM_MT) X(FORCE_GENERIC) X(GEMV_CFG) X(GEMV_GPW) X(GEMV_TILE)   \
+    X(GGR_GRID) X(GGR_WAVES) X(GGUF_BIG_LDS) X(GGUF_MM_KS) X(GGUF_MM_MIN_M) X(GGUF_MM_MT) X(GGUF_PW)          \
+    X(GGUF_RPWG) X(MFMA_MT) X(MFMA_SPLITK) X(MFMA_VARIANT) X(MXFP4_FR) X(MXFP4_MM) X(MXFP4_MM_KS)             \
+    X(MXFP4_MM_MT) X(MXFP4_VARIANT) X(PK4N_NS1_ROWS) X(PK4N_W16) X(PK4_CONTIGUOUS) X(PK4_FOLD) X(PK4_FRONT)   \
+    X(PK4_KS) X(PK4_PLACE64) X(PK4_STRIP16) X(PK4_T64) X(PK4_XQ) X(PREPACK) X(SPLITK_MODE) X(TRANSIENT_REPACK)
+enum oxq_tune_key {
+#define OXQ_TUNE_ENUM(n) OXQ_TUNE_##n,
+    OXQ_TUNE_LIST(OXQ_TUNE_ENUM)
+#undef OXQ_TUNE_ENUM
+    OXQ_TUNE_COUNT
+};
+constexpr int OXQ_TUNE_UNSET = -2147483647 - 1;
+
 struct oxq_ctx {
     int device;             // HIP ordinal, or OXQ_DEVICE_PLAN_ONLY
     bool plan_only;
@@ -25,6 +42,7 @@ struct oxq_ctx {
     oxq_plan plan;
     struct oxq_weight_cache *wcache;  // tile-major copies the stateless ops made (opt-in), or null
     size_t wcache_limit;              // bytes the cache may hold; 0 = off
+    int tuning[OXQ_TUNE_COUNT];       // tuning switches (OXQ_TUNE_UNSET = the launcher's own default)
 };
 
 namespace oxq {
@@ -55,6 +73,13 @@ inline int ilog2(int64_t v) {
     return s;
 }
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// a tuning switch of this ctx, or `dflt` where neither the environment nor the caller set it
+inline int tune(const oxq_ctx *ctx, oxq_tune_key key, int dflt) {
+    const int v = ctx->tuning[key];
+    return v == OXQ_TUNE_UNSET ? dflt : v;
+}
+inline bool tune_given(const oxq_ctx *ctx, oxq_tune_key key) { return ctx->tuning[key] != OXQ_TUNE_UNSET; }
 
 void set_plan(oxq_ctx *ctx, const char *kernel, dim3 grid, dim3 block, uint32_t split_k,
               uint32_t launches, uint64_t ws_bytes);
@@ -176,7 +201,7 @@ struct Pk4Problem {
 // ---- launchers (defined in the .hip files) ---------------------------------
 bool pk4_eligible(const Wna16Problem &p);
 size_t pk4_weight_bytes(int64_t K, int64_t N, int bits);
-int pk4_choose_strip(int64_t K, int64_t N, int bits, int64_t gate_half);
+int pk4_choose_strip(const oxq_ctx *ctx, int64_t K, int64_t N, int bits, int64_t gate_half);
 size_t pk4_zs_bytes(int64_t K, int64_t N, int group_shift);
 int launch_pk4_prepack(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &src, const Pk4Weights &dst);
 int launch_pk4_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p);
@@ -198,7 +223,7 @@ bool gguf_res_takes(int64_t K, int64_t M, int act_dtype);
 int launch_gguf_res_repack(oxq_ctx *ctx, hipStream_t s, int quant, const uint8_t *w, void *pw, int64_t K, int64_t N);
 int launch_gguf_res_dequant(oxq_ctx *ctx, hipStream_t s, int quant, const void *pw, int64_t K, int64_t N, float *out_nk);
 int launch_gguf_res_gemv(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p);  // p.w = the copy
-bool gguf_mm_eligible(const GgufProblem &p);
+bool gguf_mm_eligible(const oxq_ctx *ctx, const GgufProblem &p);
 int launch_gguf_mm(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p);
 // load-time transforms into the AWQ layout (awq_transforms.hip)
 int launch_compressed_to_awq(oxq_ctx *ctx, hipStream_t s, const uint32_t *ct, const void *scale_ct,
@@ -214,7 +239,7 @@ int launch_rtn_quantize_awq(oxq_ctx *ctx, hipStream_t s, const void *weight, int
 int launch_cast_f8e4m3_f32(oxq_ctx *ctx, hipStream_t s, const uint8_t *in, float *out, size_t n);
 int launch_f8_block_dequant(oxq_ctx *ctx, hipStream_t s, const F8Problem &p, uint16_t *out);
 int launch_f8_gemv(oxq_ctx *ctx, hipStream_t s, const F8Problem &p);
-bool f8_mm_eligible(const F8Problem &p);
+bool f8_mm_eligible(const oxq_ctx *ctx, const F8Problem &p);
 int launch_f8_mm(oxq_ctx *ctx, hipStream_t s, const F8Problem &p);
 // MXFP4 prefill (plain m > 16, or grouped with many pairs per expert): same tile matmul
 int launch_mxfp4_mm(oxq_ctx *ctx, hipStream_t s, const Mxfp4Problem &p);
@@ -246,6 +271,10 @@ int launch_moe_combine(oxq_ctx *ctx, hipStream_t s, const void *eo, const int32_
 // plain streaming read (calib.hip): bytes = workgroups * span, span a multiple of 64 KiB
 int launch_calib_read(oxq_ctx *ctx, hipStream_t s, const uint8_t *src, uint64_t bytes, int workgroups, int nontemporal,
                       uint32_t *out);
+// the same read with every lane's share requested up front; an empty launch (calib.hip)
+int launch_calib_upfront(oxq_ctx *ctx, hipStream_t s, const uint8_t *src, uint64_t bytes, int workgroups, int waves,
+                         int nontemporal, uint32_t *out);
+int launch_empty(oxq_ctx *ctx, hipStream_t s, int workgroups, int threads, int lds_bytes);
 // y[M,N] = sum over S slices of ws[s][M][N] (+ bias), slices added in index order.
 int launch_splitk_reduce(oxq_ctx *ctx, hipStream_t s, const float *ws, const void *bias, void *y,
                          int64_t M, int64_t N, int S, int dtype);

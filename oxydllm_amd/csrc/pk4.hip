@@ -1185,11 +1185,6 @@ int launch_pk4_dequant(oxq_ctx *ctx, hipStream_t s, const Pk4Weights &w, void *o
     return OXQ_OK;
 }
 
-static int pk4_env(const char *name, int dflt) {
-    const char *e = getenv(name);
-    return e ? atoi(e) : dflt;
-}
-
 template <typename TT, int BITS, int NBLK, int XQ, int NW, int WIN = NBLK>
 static int pk4_front_go(hipStream_t s, dim3 grid, const Pk4Problem &p, int bslice) {
     const size_t lds = (size_t)NW * 4096;
@@ -1198,6 +1193,19 @@ static int pk4_front_go(hipStream_t s, dim3 grid, const Pk4Problem &p, int bslic
     hipLaunchKernelGGL((pk4_front_kernel<TT, BITS, NBLK, XQ, NW, WIN>), grid, dim3(NW * 64), lds, s, (const uint16_t *)p.x, p.w.pw,
                        (const uint16_t *)p.bias, (uint16_t *)p.y, (float *)p.ws, (int)p.M, (int)p.w.K, (int)p.w.N,
                        bslice, p.act);
+    OXQ_HIP_CHECK(hipGetLastError());
+    return OXQ_OK;
+}
+
+// one instantiation of pk4_mfma_kernel: its LDS grant, the launch, the error check
+template <typename TT, int BITS, int MT, bool GS, int WD, int XQ, bool PLZ = false, int NBLK = 0>
+static int pk4_mfma_go(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, int bslice) {
+    const size_t lds = (size_t)8 * MT * 4096;
+    static LdsGrant lds_grant;
+    OXQ_HIP_CHECK(lds_grant.ensure((const void *)pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ, PLZ, NBLK>, lds));
+    hipLaunchKernelGGL((pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ, PLZ, NBLK>), grid, dim3(512), lds, s,
+                       (const uint16_t *)p.x, p.w.pw, (const uint16_t *)p.bias, (uint16_t *)p.y, (float *)ctx->workspace,
+                       (int)p.M, (int)p.w.K, (int)p.w.N, bslice, tune(ctx, OXQ_TUNE_PK4_CONTIGUOUS, 1), p.act);
     OXQ_HIP_CHECK(hipGetLastError());
     return OXQ_OK;
 }
@@ -1236,101 +1244,31 @@ static int pk4_go4(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, 
         }
     }
     constexpr int WD = Pk4Ring<MT, BITS>::WD;
-    const size_t lds = (size_t)8 * MT * 4096;
-    if constexpr (MT == 2) {
-        // Two row tiles, four or five blocks a wave (4-bit: also six or eight, K = 6144, 8192 - 32 rows f16 15.69 / 35.45
-        // -> 14.88 / 33.73 us, bf16 20.54 / 49.01 -> 17.24 / 39.82 on 6144 x 16384 / 8192 x 28672), one row-tile workgroup
-        // a strip: straight-line code with the
-        // memory operations placed by hand and the block-end requests pinned.  Same box, loop -> straight line,
-        // 4096 x 14336 at 17 / 32 rows: f16 9.85 / 11.04 -> 9.66 / 10.45 us, bf16 14.37 / 14.55 -> 12.04 / 12.48, 8-bit
-        // f16 14.00 / 14.71 -> 13.26 / 14.14.  (Unrolled without the pins it is slower than the loop: f16 12.15 /
-        // 13.12; with the block-end pin alone 9.70 / 10.91.)
-        if (grid.z == 1 && (bslice == 32 || bslice == 40 || ((bslice == 48 || bslice == 64) && BITS == 4)) && pk4_env("OXQ_PK4_FRONT", 1)) {
-            static LdsGrant lg4, lg5, lg6, lg8;
-            if (bslice == 32) {
-                OXQ_HIP_CHECK(lg4.ensure((const void *)pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ, true, 4>, lds));
-                hipLaunchKernelGGL((pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ, true, 4>), grid, dim3(512), lds, s,
-                                   (const uint16_t *)p.x, p.w.pw, (const uint16_t *)p.bias, (uint16_t *)p.y,
-                                   (float *)ctx->workspace, (int)p.M, (int)p.w.K, (int)p.w.N, bslice,
-                                   pk4_env("OXQ_PK4_CONTIGUOUS", 1), p.act);
-            } else if (bslice == 48) {
-                OXQ_HIP_CHECK(lg6.ensure((const void *)pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ, true, 6>, lds));
-                hipLaunchKernelGGL((pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ, true, 6>), grid, dim3(512), lds, s,
-                                   (const uint16_t *)p.x, p.w.pw, (const uint16_t *)p.bias, (uint16_t *)p.y,
-                                   (float *)ctx->workspace, (int)p.M, (int)p.w.K, (int)p.w.N, bslice,
-                                   pk4_env("OXQ_PK4_CONTIGUOUS", 1), p.act);
-            } else if (bslice == 64) {
-                OXQ_HIP_CHECK(lg8.ensure((const void *)pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ, true, 8>, lds));
-                hipLaunchKernelGGL((pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ, true, 8>), grid, dim3(512), lds, s,
-                                   (const uint16_t *)p.x, p.w.pw, (const uint16_t *)p.bias, (uint16_t *)p.y,
-                                   (float *)ctx->workspace, (int)p.M, (int)p.w.K, (int)p.w.N, bslice,
-                                   pk4_env("OXQ_PK4_CONTIGUOUS", 1), p.act);
-            } else {
-                OXQ_HIP_CHECK(lg5.ensure((const void *)pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ, true, 5>, lds));
-                hipLaunchKernelGGL((pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ, true, 5>), grid, dim3(512), lds, s,
-                                   (const uint16_t *)p.x, p.w.pw, (const uint16_t *)p.bias, (uint16_t *)p.y,
-                                   (float *)ctx->workspace, (int)p.M, (int)p.w.K, (int)p.w.N, bslice,
-                                   pk4_env("OXQ_PK4_CONTIGUOUS", 1), p.act);
+    // Two to four row tiles whose K slice is four or five blocks a wave (K = 4096, 5120 unsliced; 4-bit layers also six
+    // and eight, K = 6144, 8192) with one row-tile workgroup a strip: the block loop as straight-line code.  Two row
+    // tiles with the memory operations placed by hand and the block-end requests pinned (PLZ) - unrolled without the
+    // pins they are slower than the loop.  Same box, loop -> straight line, 4096 x 14336: 17 / 32 rows f16 9.85 / 11.04 ->
+    // 9.66 / 10.45 us, bf16 14.37 / 14.55 -> 12.04 / 12.48, 8-bit f16 14.00 / 14.71 -> 13.26 / 14.14; 48 / 64 rows 4-bit f16
+    // 13.66 / 16.40 -> 13.06 / 16.29, bf16 15.74 / 18.70 -> 15.23 / 17.91, 8-bit f16 17.09 / 20.4 -> 16.65 / 19.85; 32 rows on
+    // 6144 x 16384 / 8192 x 28672 f16 15.69 / 35.45 -> 14.88 / 33.73, bf16 20.54 / 49.01 -> 17.24 / 39.82.
+    if constexpr (MT >= 2) {
+        constexpr bool PLZ = MT == 2;
+        if (grid.z == 1 && bslice % 8 == 0 && tune(ctx, OXQ_TUNE_PK4_FRONT, 1)) {
+            switch (bslice / 8) {
+            case 4: return pk4_mfma_go<TT, BITS, MT, GS, WD, XQ, PLZ, 4>(ctx, s, grid, p, bslice);
+            case 5: return pk4_mfma_go<TT, BITS, MT, GS, WD, XQ, PLZ, 5>(ctx, s, grid, p, bslice);
+            case 6: if constexpr (BITS == 4) return pk4_mfma_go<TT, BITS, MT, GS, WD, XQ, PLZ, 6>(ctx, s, grid, p, bslice); break;
+            case 8: if constexpr (BITS == 4) return pk4_mfma_go<TT, BITS, MT, GS, WD, XQ, PLZ, 8>(ctx, s, grid, p, bslice); break;
+            default: break;
             }
-            OXQ_HIP_CHECK(hipGetLastError());
-            return OXQ_OK;
         }
     }
-    if constexpr (MT >= 3) {
-        // Four or five blocks a wave (K = 4096, 5120 unsliced) and one row-tile workgroup a strip: the block loop as
-        // straight-line code.  Same box, loop -> straight line, 48 / 64 rows: 4-bit f16 4096 x 14336 13.66 / 16.40 ->
-        // 13.06 / 16.29 us, bf16 15.74 / 18.70 -> 15.23 / 17.91; 5120 x 13824 f16 16.6 / 20.39 -> 16.05 / 20.1, bf16
-        // 18.9 / 22.12 -> 18.16 / 21.82; 8-bit f16 4096 x 14336 17.09 / 20.4 -> 16.65 / 19.85.
-        if (grid.z == 1 && (bslice == 32 || bslice == 40 || ((bslice == 48 || bslice == 64) && BITS == 4)) && pk4_env("OXQ_PK4_FRONT", 1)) {
-            static LdsGrant lg4, lg5, lg6, lg8;
-            if (bslice == 32) {
-                OXQ_HIP_CHECK(lg4.ensure((const void *)pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ, false, 4>, lds));
-                hipLaunchKernelGGL((pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ, false, 4>), grid, dim3(512), lds, s,
-                                   (const uint16_t *)p.x, p.w.pw, (const uint16_t *)p.bias, (uint16_t *)p.y,
-                                   (float *)ctx->workspace, (int)p.M, (int)p.w.K, (int)p.w.N, bslice,
-                                   pk4_env("OXQ_PK4_CONTIGUOUS", 1), p.act);
-            } else if (bslice == 48) {
-                OXQ_HIP_CHECK(lg6.ensure((const void *)pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ, false, 6>, lds));
-                hipLaunchKernelGGL((pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ, false, 6>), grid, dim3(512), lds, s,
-                                   (const uint16_t *)p.x, p.w.pw, (const uint16_t *)p.bias, (uint16_t *)p.y,
-                                   (float *)ctx->workspace, (int)p.M, (int)p.w.K, (int)p.w.N, bslice,
-                                   pk4_env("OXQ_PK4_CONTIGUOUS", 1), p.act);
-            } else if (bslice == 64) {
-                OXQ_HIP_CHECK(lg8.ensure((const void *)pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ, false, 8>, lds));
-                hipLaunchKernelGGL((pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ, false, 8>), grid, dim3(512), lds, s,
-                                   (const uint16_t *)p.x, p.w.pw, (const uint16_t *)p.bias, (uint16_t *)p.y,
-                                   (float *)ctx->workspace, (int)p.M, (int)p.w.K, (int)p.w.N, bslice,
-                                   pk4_env("OXQ_PK4_CONTIGUOUS", 1), p.act);
-            } else {
-                OXQ_HIP_CHECK(lg5.ensure((const void *)pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ, false, 5>, lds));
-                hipLaunchKernelGGL((pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ, false, 5>), grid, dim3(512), lds, s,
-                                   (const uint16_t *)p.x, p.w.pw, (const uint16_t *)p.bias, (uint16_t *)p.y,
-                                   (float *)ctx->workspace, (int)p.M, (int)p.w.K, (int)p.w.N, bslice,
-                                   pk4_env("OXQ_PK4_CONTIGUOUS", 1), p.act);
-            }
-            OXQ_HIP_CHECK(hipGetLastError());
-            return OXQ_OK;
-        }
-    }
+    // a (nearly) full fourth row tile of a 4-bit layer on its own strip: the loop with hand-placed memory operations
     if constexpr (MT == 4 && BITS == 4) {
-        if (grid.z == 1 && p.M > 56 && pk4_env("OXQ_PK4_PLACE64", 1)) {
-            static LdsGrant lds_grant_p;
-            OXQ_HIP_CHECK(lds_grant_p.ensure((const void *)pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ, true>, lds));
-            hipLaunchKernelGGL((pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ, true>), grid, dim3(512), lds, s,
-                               (const uint16_t *)p.x, p.w.pw, (const uint16_t *)p.bias, (uint16_t *)p.y,
-                               (float *)ctx->workspace, (int)p.M, (int)p.w.K, (int)p.w.N, bslice,
-                               pk4_env("OXQ_PK4_CONTIGUOUS", 1), p.act);
-            OXQ_HIP_CHECK(hipGetLastError());
-            return OXQ_OK;
-        }
+        if (grid.z == 1 && p.M > 56 && tune(ctx, OXQ_TUNE_PK4_PLACE64, 1))
+            return pk4_mfma_go<TT, BITS, MT, GS, WD, XQ, true>(ctx, s, grid, p, bslice);
     }
-    static LdsGrant lds_grant;  // one per instantiation
-    OXQ_HIP_CHECK(lds_grant.ensure((const void *)pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ>, lds));
-    hipLaunchKernelGGL((pk4_mfma_kernel<TT, BITS, MT, GS, WD, XQ>), grid, dim3(512), lds, s, (const uint16_t *)p.x,
-                       p.w.pw, (const uint16_t *)p.bias, (uint16_t *)p.y, (float *)ctx->workspace, (int)p.M,
-                       (int)p.w.K, (int)p.w.N, bslice, pk4_env("OXQ_PK4_CONTIGUOUS", 1), p.act);
-    OXQ_HIP_CHECK(hipGetLastError());
-    return OXQ_OK;
+    return pk4_mfma_go<TT, BITS, MT, GS, WD, XQ>(ctx, s, grid, p, bslice);
 }
 
 template <typename TT, int BITS, int MT, bool GS>
@@ -1338,7 +1276,7 @@ static int pk4_go(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, i
     // A single short tile: rows past M are known at launch, so the loads that would only fetch them
     // are left out (M = 1: 8.8 instead of 9.1 us on 4096 x 14336).
     if constexpr (MT == 1) {
-        const int xq = pk4_env("OXQ_PK4_XQ", 1) ? (int)ceil_div(p.M, 4) : 4;
+        const int xq = tune(ctx, OXQ_TUNE_PK4_XQ, 1) ? (int)ceil_div(p.M, 4) : 4;
         if (xq == 1) return pk4_go4<TT, BITS, MT, GS, 1>(ctx, s, grid, p, bslice, front);
         if (xq == 2) return pk4_go4<TT, BITS, MT, GS, 2>(ctx, s, grid, p, bslice, front);
     }
@@ -1353,9 +1291,9 @@ static int pk4_go(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, i
 // tolerance either way, and the folded form is the faster one up to three row tiles
 // (4096 x 14336 f16: 17 rows 10.8 -> 9.9 us, 48 rows 14.3 -> 13.5 us; bf16 GPTQ 17 rows 13.3 -> 10.1 us).
 // At four row tiles the fold costs what the dequant costs and its extra accumulators do not fit.
-static bool pk4_folds(const Pk4Problem &p, int mt) {
+static bool pk4_folds(const oxq_ctx *ctx, const Pk4Problem &p, int mt) {
     if (mt == 1) return true;
-    if (mt > 3 || !pk4_env("OXQ_PK4_FOLD", 1)) return false;
+    if (mt > 3 || !tune(ctx, OXQ_TUNE_PK4_FOLD, 1)) return false;
     const int gemv_rows = p.w.gemv_rows ? p.w.gemv_rows : 16;
     if (p.w.dtype == OXQ_F16) return true;
     return mt == 2 && p.M <= gemv_rows;
@@ -1363,7 +1301,7 @@ static bool pk4_folds(const Pk4Problem &p, int mt) {
 
 template <typename TT, int BITS>
 static int pk4_by_mt(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p, int bslice, int mt, int front) {
-    const bool fold = pk4_folds(p, mt);
+    const bool fold = pk4_folds(ctx, p, mt);
     switch (mt) {
     case 1: return pk4_go<TT, BITS, 1, true>(ctx, s, grid, p, bslice, front);
     case 2: return fold ? pk4_go<TT, BITS, 2, true>(ctx, s, grid, p, bslice, 0) : pk4_go<TT, BITS, 2, false>(ctx, s, grid, p, bslice, 0);
@@ -1375,7 +1313,7 @@ static int pk4_by_mt(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p
 // Strip width of a layer's resident copy: 16 columns for 4-bit layers of at most 128 64-column strips and a
 // K of 32 - 112 blocks (the shapes that otherwise leave CUs idle or need K slices and a second launch),
 // 64 otherwise.
-int pk4_choose_strip(int64_t K, int64_t N, int bits, int64_t gate_half) {
+int pk4_choose_strip(const oxq_ctx *ctx, int64_t K, int64_t N, int bits, int64_t gate_half) {
     // Measured (f16; 64-column strips, with K slices where few -> 16-column strips, one launch up to 8 rows),
     // at 1 / 4 / 16 / 64 rows of x:
     //    4096 x  4096   5.85 / -    / -     / -      ->  3.64 /  3.95 /  5.24 / 11.5 us
@@ -1388,7 +1326,7 @@ int pk4_choose_strip(int64_t K, int64_t N, int bits, int64_t gate_half) {
     // with 64-column strips gain nothing (4096 x 14336: 7.49 / 7.50 / 8.40 / 16.3 against 7.45 / 8.23 / 9.11 /
     // 16.4; 5120 x 13824 and 8192 x 28672 alike), and on a very long K every strip's pass over x outweighs
     // the saved launch from 4 rows on (28672 x 8192: 23.2 / 23.4 us wide, 21.3 / 26.6 narrow).
-    const int mode = pk4_env("OXQ_PK4_STRIP16", 1);  // 0 never, 1 by shape, 2 wherever the layout applies
+    const int mode = tune(ctx, OXQ_TUNE_PK4_STRIP16, 1);  // 0 never, 1 by shape, 2 wherever the layout applies
     if (!mode || bits != 4 || gate_half || N % 64 != 0) return 64;
     if (mode == 2) return 16;
     return (N / 64 <= 128 && N / 16 >= 128 && K / 128 >= 32 && K / 128 <= 112) ? 16 : 64;
@@ -1455,7 +1393,7 @@ static int pk4n_by_shape(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Proble
     }
     switch (mt) {
     case 1: {
-        const int xq = pk4_env("OXQ_PK4_XQ", 1) ? (int)ceil_div(p.M, 4) : 4;
+        const int xq = tune(ctx, OXQ_TUNE_PK4_XQ, 1) ? (int)ceil_div(p.M, 4) : 4;
         if (xq == 1) return pk4n_go4<TT, 1, true, 4, 1>(ctx, s, grid, p, bslice);
         if (xq == 2) return pk4n_go4<TT, 1, true, 4, 2>(ctx, s, grid, p, bslice);
         return pk4n_go4<TT, 1, true, 4, 4>(ctx, s, grid, p, bslice);
@@ -1479,14 +1417,14 @@ static int launch_pk4n_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p)
     // Also up to 16 on whole rounds of 256 strips and K <= 8192 (9 / 16 rows: 8192 x 4096 6.90 / 8.07 against
     // 7.87 / 8.31, 4096 x 8192 6.49 / 7.81 against 7.53 / 8.31); not beyond (14336 x 4096 at 12 / 16 rows 11.2 / 12.4
     // against 10.3 / 10.7) and not on half a round (8192 x 2048 at 16 rows 7.52 against 6.63).
-    const int ns1_rows = pk4_env("OXQ_PK4N_NS1_ROWS", ((N / 16 <= 256 && NB <= 32) || ((N / 16) % 256 == 0 && NB <= 64)) ? 16 : 8);
+    const int ns1_rows = tune(ctx, OXQ_TUNE_PK4N_NS1_ROWS, ((N / 16 <= 256 && NB <= 32) || ((N / 16) % 256 == 0 && NB <= 64)) ? 16 : 8);
     const int ns = (M <= ns1_rows && M <= 16 && N / 16 >= 128) ? 1 : 4;
     const int64_t tiles = (N / (16 * ns)) * ceil_div(M, 16 * mt);
     int ks = 1;
     if (tiles <= 96 && NB >= 32) ks = (int)std::max<int64_t>(1, std::min<int64_t>(256 / tiles, NB / 8));
     else if (ns == 4 && tiles <= 128 && NB >= 64) ks = 2;  // as in the wide form; 128 single strips are faster whole
                                                            // (8192 x 2048 at one row: 5.20 against 5.65 us)
-    ks = pk4_env("OXQ_PK4_KS", ks);
+    ks = tune(ctx, OXQ_TUNE_PK4_KS, ks);
     ks = std::max(1, std::min(ks, NB));
     if (p.no_split) ks = 1;
     while (ks > 1 && (size_t)ks * M * N * 4 > ctx->workspace_bytes) --ks;
@@ -1495,7 +1433,7 @@ static int launch_pk4n_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p)
     if (ceil_div(M, 16 * mt) > 65535)
         return fail(OXQ_ERR_UNSUPPORTED, "repacked matmul: m = %lld exceeds the grid limit (65535 row tiles)", (long long)M);
     if (p.act) return fail(OXQ_ERR_ARG, "repacked matmul: a fused activation on a layer in 16-column strips");
-    const bool fold = mt <= 2 && pk4_folds(p, mt);  // three row tiles of folded sums do not fit beside the two-block ring
+    const bool fold = mt <= 2 && pk4_folds(ctx, p, mt);  // three row tiles of folded sums do not fit beside the two-block ring
     dim3 grid((unsigned)(N / (16 * ns)), (unsigned)ks, (unsigned)ceil_div(M, 16 * mt));
     // One or two rows of a single strip on a long K: 16 waves, so that a wave's chain of blocks is half as
     // long (f16, one / two rows, 8 -> 16 waves: 14336 x 4096 7.44 / 7.55 -> 7.00 / 7.37 us, 8192 x 2048 at one
@@ -1508,9 +1446,9 @@ static int launch_pk4n_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p)
     // the 9 - 16 rows that a single strip takes there: 4096 x 4096 at 9 / 16 rows 4.37 / 5.12 against 4.71 / 5.28;
     // with three or four blocks a wave (K <= 8192) two of them in flight: 8192 x 4096 at 9 / 12 / 16 rows 6.90 /
     // 7.41 / 8.07 -> 6.67 / 7.16 / 7.96.
-    const bool nfront = ns == 1 && ceil_div(bslice, 16) <= 8 && pk4_env("OXQ_PK4_FRONT", 1) &&
+    const bool nfront = ns == 1 && ceil_div(bslice, 16) <= 8 && tune(ctx, OXQ_TUNE_PK4_FRONT, 1) &&
                         (M <= 8 || (M <= 16 && ceil_div(bslice, 16) <= 4));
-    const bool w16 = nfront || (ns == 1 && M <= 2 && pk4_env("OXQ_PK4N_W16", NB >= 64));
+    const bool w16 = nfront || (ns == 1 && M <= 2 && tune(ctx, OXQ_TUNE_PK4N_W16, NB >= 64));
     char name[64];
     snprintf(name, sizeof name, "pk4_mfma_%s_mt%d%s_n16x%d", p.w.dtype == OXQ_F16 ? "f16" : "bf16", mt,
              (fold || ns == 1) ? "_gs" : "", ns);
@@ -1547,7 +1485,7 @@ int launch_pk4_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p) {
     // against 23.3 / 25.9 / 49.4 us (four slices: 23.4 / 26.8 / 54.2).  At K = 4096 or 5120 the second
     // launch costs more than the slices save (4096 x 8192: 6.7 / 7.8 / 13.5 against 7.0 / 8.0 / 14.9 us).
     else if (tiles <= 128 && NB >= 64) ks = 2;
-    ks = pk4_env("OXQ_PK4_KS", ks);
+    ks = tune(ctx, OXQ_TUNE_PK4_KS, ks);
     ks = std::max(1, std::min(ks, NB));
     if (p.act) ks = 1;  // the activation needs the whole sum: gate|up layers are wide, one slice fills the chip
     if (p.no_split) ks = 1;
@@ -1582,8 +1520,8 @@ int launch_pk4_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p) {
     //          in flight from 5 blocks a wave on at up to 4 rows and from 7 on at any, else one.
     //   8-bit  32 blocks in a single slice: 16 waves, one block in flight.  Otherwise 8w1 where every wave's share is
     //          whole and the kernel exists for it (1 - 6, 8).
-    const int front_xq = pk4_env("OXQ_PK4_XQ", 1) ? (int)ceil_div(M, 4) : 4;
-    const int front_mode = pk4_env("OXQ_PK4_FRONT", 1);  // 0: the ring kernel, 2: never 16 waves
+    const int front_xq = tune(ctx, OXQ_TUNE_PK4_XQ, 1) ? (int)ceil_div(M, 4) : 4;
+    const int front_mode = tune(ctx, OXQ_TUNE_PK4_FRONT, 1);  // 0: the ring kernel, 2: never 16 waves
     const int share8 = (bslice + 7) / 8;
     int front = 0;
     if (mt == 1 && front_mode != 0) {
@@ -1593,7 +1531,7 @@ int launch_pk4_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p) {
             front = (front_mode != 2 && bslice == 32 && ks == 1) ? 1 : (bslice % 8 == 0 && share8 <= 8 && share8 != 7) ? 2 : 0;
     }
     snprintf(name, sizeof name, "pk%d_mfma_%s_mt%d%s%s%s", p.w.bits, p.w.dtype == OXQ_F16 ? "f16" : "bf16", mt,
-             pk4_folds(p, mt) ? "_gs" : "", front == 1 ? "_front" : front == 2 ? "_line" : "",
+             pk4_folds(ctx, p, mt) ? "_gs" : "", front == 1 ? "_front" : front == 2 ? "_line" : "",
              p.act == 1 ? "_silu" : p.act == 2 ? "_gelu" : "");
     set_plan(ctx, name, grid, dim3(front == 1 ? 1024 : 512), ks, 1, ks > 1 ? (size_t)ks * M * p.w.N * 4 : 0);
     if (ctx->plan_only) {
@@ -1606,7 +1544,7 @@ int launch_pk4_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p) {
         return fail(OXQ_ERR_UNSUPPORTED, "repacked matmul: x and y must be 16-byte aligned");
     const bool f16 = p.w.dtype == OXQ_F16;
     int rc;
-    if (pk4_env("OXQ_PK4_T64", 1) && pk4_tile64_takes(p, ks)) {
+    if (tune(ctx, OXQ_TUNE_PK4_T64, 1) && pk4_tile64_takes(p, ks)) {
         Pk4Problem q = p;
         q.ws = ctx->workspace;
         return launch_pk4_tile64(ctx, s, q);

@@ -713,11 +713,6 @@ __global__ __launch_bounds__(512) void gptq_gemv_fast(
 // ---------------------------------------------------------------------------
 // Host dispatch
 // ---------------------------------------------------------------------------
-static int env_int(const char *name, int dflt) {
-    const char *v = getenv(name);
-    return (v && *v) ? atoi(v) : dflt;
-}
-
 // 1: the last workgroup of a tile sums the slices; 0: a second launch does.
 // The fused form saves a launch but its sum runs on one workgroup per tile, so
 // it only pays for few slices.
@@ -769,8 +764,8 @@ static int launch_awq_fast(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p) {
     const int mb = pick_mb(p.M);
     const int G = (int)(p.K >> p.group_shift);
     const int gs = (int)p.group_size;
-    int cfg = env_int("OXQ_GEMV_CFG", -1);
-    int gpw_env = env_int("OXQ_GEMV_GPW", 0);
+    int cfg = tune(ctx, OXQ_TUNE_GEMV_CFG, -1);
+    int gpw_env = tune(ctx, OXQ_TUNE_GEMV_GPW, 0);
     auto gpw_for = [&](int slab_cols, int gpb) {
         if (gpw_env > 0) return gpw_env;
         const int slabs = (int)ceil_div(p.N, slab_cols);
@@ -889,7 +884,7 @@ static int launch_gptq_fast(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p) 
     int S = (int)ceil_div(ctx->num_cus, slabs);
     if (S > G) S = G;
     if (S < 1) S = 1;
-    int gpw = env_int("OXQ_GEMV_GPW", (int)ceil_div(G, S));
+    int gpw = tune(ctx, OXQ_TUNE_GEMV_GPW, (int)ceil_div(G, S));
     S = (int)ceil_div(G, gpw);
     dim3 grid((unsigned)slabs, (unsigned)S), block(512);
     const uint64_t ws_bytes = S > 1 ? (uint64_t)S * p.M * p.N * 4 : 0;
@@ -929,14 +924,14 @@ int launch_wna16_gemv(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p) {
     // rows (13 - 14 us against 17 - 33 us for the dot2 kernel at 4096 x 14336).  Its B operand is
     // the dequantized weight rounded to f16, 2^-12 relative: far inside the tolerance; bf16, whose
     // rounding is 2^-9, keeps the kernel that never rounds the weight.
-    if (p.M >= 2 && f16 && awq4_mfma_ok(p) && env_int("OXQ_GEMV_TILE", 1) && !env_int("OXQ_FORCE_GENERIC", 0))
+    if (p.M >= 2 && f16 && awq4_mfma_ok(p) && tune(ctx, OXQ_TUNE_GEMV_TILE, 1) && !tune(ctx, OXQ_TUNE_FORCE_GENERIC, 0))
         return launch_wna16_mfma(ctx, s, p);
-    if (gptq_fast_ok(p) && !env_int("OXQ_FORCE_GENERIC", 0)) {
+    if (gptq_fast_ok(p) && !tune(ctx, OXQ_TUNE_FORCE_GENERIC, 0)) {
         if (p.bits == 4)
             return f16 ? launch_gptq_fast<F16Traits, 4>(ctx, s, p) : launch_gptq_fast<BF16Traits, 4>(ctx, s, p);
         return f16 ? launch_gptq_fast<F16Traits, 8>(ctx, s, p) : launch_gptq_fast<BF16Traits, 8>(ctx, s, p);
     }
-    if (awq_fast_ok(p) && !env_int("OXQ_FORCE_GENERIC", 0)) {
+    if (awq_fast_ok(p) && !tune(ctx, OXQ_TUNE_FORCE_GENERIC, 0)) {
         if (p.bits == 4)
             return f16 ? launch_awq_fast<F16Traits, 4>(ctx, s, p) : launch_awq_fast<BF16Traits, 4>(ctx, s, p);
         return f16 ? launch_awq_fast<F16Traits, 8>(ctx, s, p) : launch_awq_fast<BF16Traits, 8>(ctx, s, p);

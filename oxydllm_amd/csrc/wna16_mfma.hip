@@ -576,17 +576,12 @@ __global__ __launch_bounds__(256) void awq4_mfma_ksplit_kernel(
     }
 }
 
-static int env_int(const char *name, int dflt) {
-    const char *v = getenv(name);
-    return (v && *v) ? atoi(v) : dflt;
-}
-
 template <typename TT>
 static int launch_awq4_mfma(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p) {
     const int M = (int)p.M, K = (int)p.K, N = (int)p.N;
     int mt = M <= 16 ? 1 : (M <= 32 ? 2 : (M <= 48 ? 3 : 4));
     {
-        const int mt_env = env_int("OXQ_MFMA_MT", 0);
+        const int mt_env = tune(ctx, OXQ_TUNE_MFMA_MT, 0);
         if (mt_env >= 1 && mt_env <= 4 && mt_env < mt) mt = mt_env;
     }
     const int mtiles = (int)ceil_div(M, 16 * mt);
@@ -594,12 +589,12 @@ static int launch_awq4_mfma(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p) 
     char name[64];
 
     // --- K split inside the workgroup: 128-column tiles, slices of whole 512-row units
-    const int variant = env_int("OXQ_MFMA_VARIANT", 0);  // 0 auto (pipe), 1 ksplit, 2 pipe, 3 simple
+    const int variant = tune(ctx, OXQ_TUNE_MFMA_VARIANT, 0);  // 0 auto (pipe), 1 ksplit, 2 pipe, 3 simple
     if (variant == 1 && p.group_size >= 32 && K % 512 == 0 &&
         (512 % p.group_size == 0 || p.group_size % 512 == 0)) {
         const int ctiles = (int)ceil_div(N, 128);
         const int units = K / 512;
-        int S = env_int("OXQ_MFMA_SPLITK", (int)ceil_div(ctx->num_cus, (int64_t)ctiles * mtiles));
+        int S = tune(ctx, OXQ_TUNE_MFMA_SPLITK, (int)ceil_div(ctx->num_cus, (int64_t)ctiles * mtiles));
         if (S < 1) S = 1;
         if (S > units) S = units;
         int kslice = (int)ceil_div(units, S) * 512;
@@ -641,7 +636,7 @@ static int launch_awq4_mfma(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p) 
     // K slices: whole groups (and whole 32-row MFMA steps), about one workgroup per CU
     const int step = (int)(p.group_size > 32 ? p.group_size : 32);
     const int units = K / step;
-    int S = env_int("OXQ_MFMA_SPLITK", ctx->num_cus / (mtiles * ctiles));
+    int S = tune(ctx, OXQ_TUNE_MFMA_SPLITK, ctx->num_cus / (mtiles * ctiles));
     if (S < 1) S = 1;
     if (S > units) S = units;
     const int kslice = (int)ceil_div(units, S) * step;
@@ -698,7 +693,7 @@ bool awq4_mfma_ok(const Wna16Problem &p) {
 }
 
 int launch_wna16_mfma(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p) {
-    if (awq4_mfma_ok(p) && !env_int("OXQ_FORCE_GENERIC", 0))
+    if (awq4_mfma_ok(p) && !tune(ctx, OXQ_TUNE_FORCE_GENERIC, 0))
         return p.dtype == OXQ_F16 ? launch_awq4_mfma<F16Traits>(ctx, s, p)
                                   : launch_awq4_mfma<BF16Traits>(ctx, s, p);
     // Layouts without a tile kernel of their own on the checkpoint layout (GPTQ, 8-bit AWQ): when the
@@ -706,8 +701,8 @@ int launch_wna16_mfma(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p) {
     // One launch more (about 45 us at 5120 x 13824, 4-bit) instead of one GEMV pass over the weights
     // per 8 rows (35 - 45 us each): ahead from m = 9.  A caller that holds the layer should hold a
     // PackedQuantLinear, which repacks once.
-    if (p.M > 8 && pk4_eligible(p) && !ctx->plan_only && env_int("OXQ_TRANSIENT_REPACK", 1) &&
-        !env_int("OXQ_FORCE_GENERIC", 0)) {
+    if (p.M > 8 && pk4_eligible(p) && !ctx->plan_only && tune(ctx, OXQ_TUNE_TRANSIENT_REPACK, 1) &&
+        !tune(ctx, OXQ_TUNE_FORCE_GENERIC, 0)) {
         const size_t wb = (pk4_weight_bytes(p.K, p.N, p.bits) + 255) & ~(size_t)255;
         if (wb <= ctx->workspace_bytes) {
             Pk4Weights w{(uint32_t *)ctx->workspace, nullptr, p.K, p.N, p.group_shift, p.dtype, p.bits, 0,

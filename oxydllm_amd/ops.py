@@ -90,6 +90,17 @@ class Context:
             return 0
         return torch.cuda.current_stream().cuda_stream
 
+    def set_tuning(self, name: str, value: Optional[int]) -> None:
+        """One tuning switch of this context (see include/oxq.h); ``None`` returns it to the
+        environment's value, or to the launcher's default."""
+        if value is None:
+            _lib.check(self._lib.oxq_ctx_reset_tuning(self.handle, name.encode()))
+        else:
+            _lib.check(self._lib.oxq_ctx_set_tuning(self.handle, name.encode(), int(value)))
+
+    def reset_tuning(self) -> None:
+        _lib.check(self._lib.oxq_ctx_reset_tuning(self.handle, None))
+
     # opt-in cache of tile-major weight copies behind the stateless ops (see include/oxq.h)
     def set_weight_cache(self, max_bytes: int) -> None:
         _lib.check(self._lib.oxq_ctx_set_weight_cache(self.handle, int(max_bytes)))
@@ -127,11 +138,25 @@ def _out_for(x: torch.Tensor, n: int, out, ctx):
 # ---------------------------------------------------------------- AWQ / GPTQ ops
 def calib_read(src, workgroups: int, nontemporal: bool, checksums, *, ctx: Optional[Context] = None):
     """Plain streaming read of ``src`` (uint8) by ``workgroups`` workgroups; ``checksums`` (int32/uint32,
-    one word per workgroup) receives the xor of every span.  A measurement aid (see include/oxq.h)."""
+    one word per workgroup) receives the xor of every span.  A measurement aid (see include/oxq_bench.h)."""
     ctx = _ctx(ctx)
     _lib.check(ctx._lib.oxq_calib_read(ctx.handle, ctx.stream(), desc(src), int(workgroups), int(bool(nontemporal)),
                                        desc(checksums)))
     return checksums
+
+
+def read_upfront(src, workgroups: int, waves: int, nontemporal: bool, checksums, *, ctx: Optional[Context] = None):
+    """The same read with every lane's share requested before the first wait (include/oxq_bench.h)."""
+    ctx = _ctx(ctx)
+    _lib.check(ctx._lib.oxq_bench_read_upfront(ctx.handle, ctx.stream(), desc(src), int(workgroups), int(waves),
+                                               int(bool(nontemporal)), desc(checksums)))
+    return checksums
+
+
+def empty_launch(workgroups: int, threads: int, lds_bytes: int = 0, *, ctx: Optional[Context] = None):
+    """An empty kernel of the given launch shape (include/oxq_bench.h)."""
+    ctx = _ctx(ctx)
+    _lib.check(ctx._lib.oxq_bench_empty_launch(ctx.handle, ctx.stream(), int(workgroups), int(threads), int(lds_bytes)))
 
 
 def w4a16_matmul(x, qweight, qzeros, scales, *, out=None, ctx: Optional[Context] = None):

@@ -34,3 +34,20 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+@pytest.fixture(autouse=True)
+def _tuning_back_to_defaults(request):
+    """Tests flip tuning switches on the default context (helpers.tune); every test starts from the defaults."""
+    yield
+    if "gpu" not in request.keywords:
+        return
+    try:
+        import torch
+        if not torch.cuda.is_available():
+            return
+        from oxydllm_amd import ops
+        for ctx in list(ops._default_ctx.values()):
+            ctx.reset_tuning()
+    except Exception:
+        pass

@@ -84,3 +84,10 @@ def resident_rounds_weights(m: int, dt: int, gptq: bool) -> bool:
 def round_x(x_f32: np.ndarray, dt: int) -> np.ndarray:
     """The activation values the kernel actually sees (x rounded to its 16-bit dtype)."""
     return oracle.round_through(x_f32, dt)
+
+
+def tune(name, value, ctx=None):
+    """Sets one tuning switch (``None``: back to its default) on ``ctx`` or the default context; conftest's
+    autouse fixture returns the default context's switches to their defaults after every test."""
+    from oxydllm_amd import ops
+    (ctx if ctx is not None else ops.default_context()).set_tuning(name, value)

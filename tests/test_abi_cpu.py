@@ -44,7 +44,7 @@ def plan(lib, ctx):
 def test_library_exports_every_declared_symbol(lib):
     import glob
     headers = sorted(glob.glob(os.path.join(ROOT, "include", "*.h")))
-    assert [os.path.basename(h) for h in headers] == ["oxq.h", "oxq_files.h"]
+    assert [os.path.basename(h) for h in headers] == ["oxq.h", "oxq_bench.h", "oxq_files.h"]
     header = "".join(open(h).read() for h in headers)
     declared = set(re.findall(r"^(?:int|int64_t|uint64_t|void|const char \*)\s*\*?(oxq_[a-z0-9_]+)\s*\(", header, re.M))
     assert len(declared) >= 30
@@ -411,6 +411,8 @@ def test_layers_validate_like_reference(lib, ctx):
     assert lib.oxq_qlinear_dequantize(q, None, C.byref(fake((4096, 4096), F32))) == 0, err(lib)
     assert plan(lib, ctx).kernel.decode() == "gguf_q4k_res_dequant"
     assert lib.oxq_qlinear_dequantize(q, None, C.byref(fake((4096, 4095), F32))) == -3
+    # a strided view of the right shape would be written past its storage: refused
+    assert lib.oxq_qlinear_dequantize(q, None, C.byref(fake((4096, 4096), F32, contiguous=False))) == -4
     lib.oxq_qlinear_free(q)
     # a layer whose rows are not whole strips of 16 keeps the file layout
     w2k = fake((4104 * 16 * 84,), U8)
@@ -665,7 +667,7 @@ def test_headers_compile_as_c99_and_every_entry_point_answers(tmp_path):
     no entry point crashes on arguments it must refuse."""
     decls = _c_declarations()
     assert len(decls) >= 70 and {d[1] for d in decls} == set(_lib.SIGNATURES)
-    lines = ['#include <stdio.h>', '#include <string.h>', '#include "oxq.h"', '#include "oxq_files.h"', '',
+    lines = ['#include <stdio.h>', '#include <string.h>', '#include "oxq.h"', '#include "oxq_bench.h"', '#include "oxq_files.h"', '',
              'int main(void) {', '    oxq_ctx *ctx = NULL;', '    oxq_tensor t;', '    oxq_plan plan;', '    int calls = 0;',
              '    memset(&t, 0, sizeof t);', '    t.dtype = OXQ_F16; t.rank = 2; t.dims[0] = 1; t.dims[1] = 256; t.contiguous = 1;',
              '    if (oxq_ctx_create(OXQ_DEVICE_PLAN_ONLY, &ctx) != OXQ_OK || !ctx) return 2;']

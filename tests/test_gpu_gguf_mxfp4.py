@@ -16,7 +16,7 @@ import torch
 import oracle
 from oxydllm_amd import synth
 from tests import refgen
-from tests.helpers import RTOL, ATOL, as_f32, assert_close, bits_of, round_x, to_dev
+from tests.helpers import RTOL, ATOL, as_f32, assert_close, bits_of, round_x, to_dev, tune
 
 pytestmark = pytest.mark.gpu
 ops = None
@@ -117,8 +117,8 @@ def test_gguf_mul_mm_ragged(fmt, mt, ks, monkeypatch):
     elems, _ = synth.GGUF_BLOCK_LAYOUT[fmt]
     N, K, m = (1001 if ks == 1 else 1000), (1024 if elems == 256 else 1120), 150
     say(f"gguf mul_mm ragged {synth.GGUF_NAMES[fmt]} K={K} N={N} mt {mt} ks {ks}")
-    monkeypatch.setenv("OXQ_GGUF_MM_MT", str(mt))
-    monkeypatch.setenv("OXQ_GGUF_MM_KS", str(ks))
+    tune("OXQ_GGUF_MM_MT", mt)
+    tune("OXQ_GGUF_MM_KS", ks)
     data = synth.gguf_weight(fmt, N, K, seed=130 + fmt)
     w = oracle.dequantize_gguf(fmt, data, N, K)
     x = np.random.default_rng(131).standard_normal((m, K)).astype(np.float32)
@@ -166,13 +166,13 @@ def test_gguf_gemv_single_row_wave_per_weight_row(fmt, monkeypatch):
             x = np.random.default_rng(N * 7 + K).standard_normal((1, K)).astype(np.float32)
             xd, wd = to_dev(x, dt), to_dev(data)
             xr = x if dt == torch.float32 else round_x(x, oracle.BF16)
-            monkeypatch.setenv("OXQ_GGUF_PW", "1")
+            tune("OXQ_GGUF_PW", 1)
             y = ops.gguf_quant_matmul(xd, wd, K, N, fmt)
             assert_close(y, oracle.matmul_nt_f32(xr, w), f"gguf wave-per-row {synth.GGUF_NAMES[fmt]} {N}x{K}")
-            monkeypatch.setenv("OXQ_GGUF_PW", "0")
+            tune("OXQ_GGUF_PW", 0)
             joint = ops.gguf_quant_matmul(xd, wd, K, N, fmt)
             np.testing.assert_array_equal(bits_of(y), bits_of(joint))
-    monkeypatch.delenv("OXQ_GGUF_PW")
+    tune("OXQ_GGUF_PW", None)
 
 
 @pytest.mark.parametrize("fmt", FMTS)
@@ -190,12 +190,12 @@ def test_gguf_gemv_long_rows(fmt, monkeypatch):
     plan = ops.default_context().last_plan()
     assert plan["kernel"].endswith("gemv_f32_lds") and plan["launches"] in (2, 4, 8), plan
     assert_close(y, ref, f"gguf long rows {synth.GGUF_NAMES[fmt]}")
-    monkeypatch.setenv("OXQ_FORCE_GENERIC", "1")
+    tune("OXQ_FORCE_GENERIC", 1)
     y = ops.gguf_quant_matmul(to_dev(x), to_dev(data), K, N, fmt)
     kernel = ops.default_context().last_plan()["kernel"]
     assert kernel.endswith("gemv_f32") and not kernel.endswith("_lds")
     assert_close(y, ref, f"gguf long rows, wave per row {synth.GGUF_NAMES[fmt]}")
-    monkeypatch.delenv("OXQ_FORCE_GENERIC")
+    tune("OXQ_FORCE_GENERIC", None)
     # bf16 rows of the decode range take the staged GEMV up to 2 rows and the tile matmul with
     # unrounded (hi + lo) weights from 3: both are held to the unrounded oracle
     for mb in (2, 3, 8):
@@ -284,12 +284,12 @@ def test_mxfp4_mul_mm(m, n, k, monkeypatch):
     assert plan["kernel"].startswith("mxfp4_mul_mm_bf16")
     assert_close(y, ref, f"mxfp4 mul_mm {m}x{n}x{k}")
     if n % 4 == 0 and k >= 512:
-        monkeypatch.setenv("OXQ_MXFP4_MM_KS", "3")
+        tune("OXQ_MXFP4_MM_KS", 3)
         y3 = ops.mxfp4_matmul(xd, bd, sd, k, n)
         assert ops.default_context().last_plan()["split_k"] > 1
         assert_close(y3, ref, f"mxfp4 mul_mm split {m}x{n}x{k}")
     # the decode kernel on the same rows agrees within the tolerance as well
-    monkeypatch.setenv("OXQ_MXFP4_MM", "0")
+    tune("OXQ_MXFP4_MM", 0)
     y0 = ops.mxfp4_matmul(xd, bd, sd, k, n)
     assert "gemv" in ops.default_context().last_plan()["kernel"]
     assert_close(y0, ref, f"mxfp4 gemv form {m}x{n}x{k}")
@@ -319,7 +319,7 @@ def test_mxfp4_moe_prefill_grouped(T, E, top_k, N, K, monkeypatch):
                                             scales[e * N * nb:(e + 1) * N * nb], N, K)
             ref[lo:hi] = oracle.matmul_nt_f32(xb[tokens[lo:hi]], w, bb[e])
     off_d, tok_d = to_dev(offsets.astype(np.int32)), to_dev(tokens.astype(np.int32))
-    monkeypatch.setenv("OXQ_MXFP4_MM", "1")
+    tune("OXQ_MXFP4_MM", 1)
     y = ops.mxfp4_moe_matmul(to_dev(x, torch.bfloat16), to_dev(blocks), to_dev(scales),
                              to_dev(bias, torch.bfloat16), off_d, tok_d, K, N)
     assert ops.default_context().last_plan()["kernel"].startswith("mxfp4_moe_mul_mm_bf16")
@@ -328,7 +328,7 @@ def test_mxfp4_moe_prefill_grouped(T, E, top_k, N, K, monkeypatch):
     y2 = ops.mxfp4_moe_matmul(to_dev(xp, torch.bfloat16), to_dev(blocks), to_dev(scales),
                               to_dev(bias, torch.bfloat16), off_d, None, K, N)
     assert_close(y2, ref, "moe prefill identity rows")
-    monkeypatch.setenv("OXQ_MXFP4_MM", "0")
+    tune("OXQ_MXFP4_MM", 0)
     y0 = ops.mxfp4_moe_matmul(to_dev(x, torch.bfloat16), to_dev(blocks), to_dev(scales),
                               to_dev(bias, torch.bfloat16), off_d, tok_d, K, N)
     assert "gemv" in ops.default_context().last_plan()["kernel"]
@@ -487,7 +487,7 @@ def test_moe_route_group_equals_the_two_calls(T, E, k, norm):
 
 @pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16, torch.float16])
 def test_gated_activations_match_oracle(dt, monkeypatch):
-    monkeypatch.setenv("OXQ_ACT_VEC", "1")      # the 8-outputs-a-thread kernel at test sizes too
+    tune("OXQ_ACT_VEC", 1)      # the 8-outputs-a-thread kernel at test sizes too
     """ffn_kernels.metal:19-242 and moe.rs:152-173: f32 math, one rounding to the tensor dtype."""
     say(f"gated activations {dt}")
     rng = np.random.default_rng(3)
@@ -631,13 +631,13 @@ def test_mxfp4_moe_gate_up_swiglu_fused(E, N, K, counts, bias, monkeypatch):
         xs = x if gather else x[torch.from_numpy(tok).long().cuda()].contiguous()
         tk = td if gather else None
         say(f"fused swiglu E={E} N={N} K={K} gather={gather}")
-        monkeypatch.setenv("OXQ_MXFP4_MM", "0")
+        tune("OXQ_MXFP4_MM", 0)
         two = ops.gated_activation(ops.mxfp4_moe_matmul(xs, bd, sd, b, od, tk, K, N), ops.ACT_GPT_OSS_SWIGLU, 7.0)
         one = ops.mxfp4_moe_gate_up_swiglu(xs, bd, sd, b, od, tk, K, N, 7.0)
         assert ops.default_context().last_plan()["kernel"].endswith("_swiglu")
         assert one.shape == (P, N // 2)
         np.testing.assert_array_equal(one.view(torch.int16).cpu().numpy(), two.view(torch.int16).cpu().numpy())
-        monkeypatch.setenv("OXQ_MXFP4_MM", "1")      # the tile matmul declines the fused form
+        tune("OXQ_MXFP4_MM", 1)      # the tile matmul declines the fused form
         alt = ops.mxfp4_moe_gate_up_swiglu(xs, bd, sd, b, od, tk, K, N, 7.0)
         assert ops.default_context().last_plan()["kernel"] == "gpt_oss_swiglu"
         assert_close(alt, as_f32(two), "declined path", bf16_out=True)

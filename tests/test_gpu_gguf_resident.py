@@ -16,7 +16,7 @@ import torch
 
 import oracle
 from oxydllm_amd import synth
-from tests.helpers import assert_close, bits_of, round_x, to_dev
+from tests.helpers import assert_close, bits_of, round_x, to_dev, tune
 
 pytestmark = pytest.mark.gpu
 ops = None
@@ -102,7 +102,7 @@ def test_resident_gemv_rows_bias_and_shapes(fmt):
 def test_workgroups_that_walk_several_strips(cap, monkeypatch):
     """More strips than workgroups (a wide layer; forced here by capping the grid): a workgroup stages x
     once, walks its strips and meets once per group of four - full groups, a partial last group, a single strip."""
-    monkeypatch.setenv("OXQ_GGR_GRID", str(cap))
+    tune("OXQ_GGR_GRID", cap)
     N, K = 16 * 11, 2048
     for fmt in RES:
         data = synth.gguf_weight(fmt, N, K, seed=cap + fmt)
@@ -116,7 +116,7 @@ def test_workgroups_that_walk_several_strips(cap, monkeypatch):
             plan = ops.default_context().last_plan()
             assert "_res_gemv_" in plan["kernel"] and plan["grid"][0] == cap, plan
             assert_close(y, oracle.matmul_nt_f32(x, w, bias), f"cap {cap} fmt {fmt} m={m}")
-    monkeypatch.delenv("OXQ_GGR_GRID")
+    tune("OXQ_GGR_GRID", None)
     y1 = layer.forward(to_dev(x))
     assert ops.default_context().last_plan()["grid"][0] == N // 16
     assert np.array_equal(bits_of(y1), bits_of(y)), "the walk does not change a column's sum order"
@@ -136,7 +136,7 @@ def test_layers_outside_the_copys_reach_keep_the_file_layout(monkeypatch):
         assert_close(y, oracle.matmul_nt_f32(x, oracle.dequantize_gguf(fmt, data, n, k)), f"fmt {fmt} N={n} K={k}")
         want = oracle.dequantize_gguf(fmt, data, n, k)
         assert np.array_equal(layer.dequantize().cpu().numpy().view(np.uint32), want.view(np.uint32))
-    monkeypatch.setenv("OXQ_PREPACK", "0")
+    tune("OXQ_PREPACK", 0)
     data = synth.gguf_weight(synth.GGUF_Q4_0, N, K, seed=6)
     assert not ops.QLinear(synth.GGUF_Q4_0, to_dev(data), K, N, None, torch.float32).resident
 

@@ -15,7 +15,7 @@ import torch
 
 import oracle
 from oxydllm_amd import synth
-from tests.helpers import assert_close, bits_of, round_x, to_dev
+from tests.helpers import assert_close, bits_of, round_x, to_dev, tune
 
 pytestmark = pytest.mark.gpu
 
@@ -152,7 +152,7 @@ def test_experts_fall_back_where_the_copy_does_not_apply(monkeypatch):
     assert "mul_mm" in ops.default_context().last_plan()["kernel"]
     y0 = ops.mxfp4_moe_matmul(to_dev(x, torch.bfloat16), bd, sd, biasd, to_dev(offsets), to_dev(tokens), K, N)
     assert np.array_equal(bits_of(y), bits_of(y0))
-    monkeypatch.setenv("OXQ_PREPACK", "0")
+    tune("OXQ_PREPACK", 0)
     assert not ops.Mxfp4Experts(bd, sd, biasd, E, K, N).resident
 
 

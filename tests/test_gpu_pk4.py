@@ -19,7 +19,7 @@ import torch
 import oracle
 from oxydllm_amd import synth
 from tests import refgen
-from tests.helpers import TORCH_DT, as_f32, assert_close, bits_of, resident_rounds_weights, round_x, to_dev
+from tests.helpers import TORCH_DT, as_f32, assert_close, bits_of, resident_rounds_weights, round_x, to_dev, tune
 
 pytestmark = pytest.mark.gpu
 ops = None
@@ -156,8 +156,8 @@ def test_whole_share_requested_up_front(kind, dtn, K, N, g, ks, monkeypatch):
     16, 37, 48, 32 and 21 blocks (2, 4 or 5, 6, 4 or 2 each, 2 or 3), three K slices of 11, 64 blocks (8 each),
     61 (7 or 8), 40 (5 each), 56 (7: the kernel for 8 with a block of zeros), 8 and 6 blocks (one or none) and
     72 (9: the ring); against the oracle, against the ring kernel within the tolerance, run to run bitwise."""
-    monkeypatch.setenv("OXQ_PK4_STRIP16", "0")   # these small N would take the 16-column layout
-    monkeypatch.setenv("OXQ_PK4_KS", str(ks))    # and few strips would cut K by themselves
+    tune("OXQ_PK4_STRIP16", 0)   # these small N would take the 16-column layout
+    tune("OXQ_PK4_KS", ks)    # and few strips would cut K by themselves
     dt = DT[dtn]
     trip, pack_dim = make(kind, K, N, g, seed=K + 3 * N)
     bias = (np.arange(N, dtype=np.float32) % 9 - 4) * np.float32(0.25)
@@ -177,11 +177,11 @@ def test_whole_share_requested_up_front(kind, dtn, K, N, g, ks, monkeypatch):
         assert plan["kernel"].endswith("_gs" + ("_" + form if form else "")), (plan, m, form)
         assert_close(y, ref, f"pk4 up-front {kind} {dtn} m{m}")
         np.testing.assert_array_equal(bits_of(layer.forward(xd)), bits_of(y))
-        monkeypatch.setenv("OXQ_PK4_FRONT", "0")
+        tune("OXQ_PK4_FRONT", 0)
         y0 = layer.forward(xd)
         plan = ops.default_context().last_plan()
         assert plan["block"][0] == 512 and plan["kernel"].endswith("_gs"), plan
-        monkeypatch.delenv("OXQ_PK4_FRONT")
+        tune("OXQ_PK4_FRONT", None)
         assert_close(y0, ref, f"pk4 ring {kind} {dtn} m{m}")
 
 
@@ -195,7 +195,7 @@ def test_eight_bit_single_row_tile_in_straight_line_code(kind, dtn, K, N, g, ks,
     for it (1 - 6 or 8 blocks): 8, 16, 40 and 64 blocks and two K slices of 16; 32 blocks in one slice run 16
     waves; 56 (7 each), 37 (uneven) and 72 (9 each) keep the ring.  Against the oracle, run to run bitwise, and
     the ring kernel on the same calls."""
-    monkeypatch.setenv("OXQ_PK4_KS", str(ks))
+    tune("OXQ_PK4_KS", ks)
     dt = DT[dtn]
     trip, pack_dim = make(kind, K, N, g, seed=K + 5 * N)
     bias = (np.arange(N, dtype=np.float32) % 9 - 4) * np.float32(0.25)
@@ -215,10 +215,10 @@ def test_eight_bit_single_row_tile_in_straight_line_code(kind, dtn, K, N, g, ks,
         assert plan["kernel"].endswith("_gs" + ("_" + form if form else "")), (plan, m, form)
         assert_close(y, ref, f"pk8 straight-line {kind} {dtn} m{m}")
         np.testing.assert_array_equal(bits_of(layer.forward(xd)), bits_of(y))
-        monkeypatch.setenv("OXQ_PK4_FRONT", "0")
+        tune("OXQ_PK4_FRONT", 0)
         y0 = layer.forward(xd)
         assert ops.default_context().last_plan()["kernel"].endswith("_gs")
-        monkeypatch.delenv("OXQ_PK4_FRONT")
+        tune("OXQ_PK4_FRONT", None)
         assert_close(y0, ref, f"pk8 ring {kind} {dtn} m{m}")
 
 
@@ -230,8 +230,8 @@ def test_two_to_four_row_tiles_in_straight_line_code(kind, dtn, K, N, g, ks, mon
     """17 - 64 rows on K slices of 32 or 40 blocks (4-bit: also 48 and 64) run the block loop as straight-line
     code (four to eight blocks a wave); 63 blocks in two slices leave one wave of the second slice a block short.  Against the
     oracle of the form the row count takes, run to run bitwise, and against the looping kernel."""
-    monkeypatch.setenv("OXQ_PK4_STRIP16", "0")
-    monkeypatch.setenv("OXQ_PK4_KS", str(ks))
+    tune("OXQ_PK4_STRIP16", 0)
+    tune("OXQ_PK4_KS", ks)
     dt = DT[dtn]
     trip, pack_dim = make(kind, K, N, g, seed=K + N)
     bias = (np.arange(N, dtype=np.float32) % 9 - 4) * np.float32(0.25)
@@ -250,9 +250,9 @@ def test_two_to_four_row_tiles_in_straight_line_code(kind, dtn, K, N, g, ks, mon
         ref = oracle.matmul_nt_f32(round_x(x, dt), w, bias)
         assert_close(y, ref, f"pk4 four tiles {kind} {dtn} m{m}")
         np.testing.assert_array_equal(bits_of(layer.forward(xd)), bits_of(y))
-        monkeypatch.setenv("OXQ_PK4_FRONT", "0")
+        tune("OXQ_PK4_FRONT", 0)
         y0 = layer.forward(xd)
-        monkeypatch.delenv("OXQ_PK4_FRONT")
+        tune("OXQ_PK4_FRONT", None)
         assert_close(y0, ref, f"pk4 four tiles, loop {kind} {dtn} m{m}")
 
 
@@ -265,7 +265,7 @@ def test_repacked_forward_k_slices(kind, dtn, K, N, g, ks, monkeypatch):
     (10 groups in 3 slices), fewer groups than waves per slice, one group per slice, bias
     applied once by the reduction."""
     dt = DT[dtn]
-    monkeypatch.setenv("OXQ_PK4_KS", str(ks))
+    tune("OXQ_PK4_KS", ks)
     trip, pack_dim = make(kind, K, N, g, seed=K + N + ks)
     bias = (np.arange(N, dtype=np.float32) % 7 - 3) * np.float32(0.25)
     layer = layer_of(trip, pack_dim, dt, bias, bits=bits_of_kind(kind))

@@ -17,7 +17,7 @@ import torch
 
 import oracle
 from oxydllm_amd import synth
-from tests.helpers import TORCH_DT, as_f32, assert_close, bits_of, resident_rounds_weights, round_x, to_dev
+from tests.helpers import TORCH_DT, as_f32, assert_close, bits_of, resident_rounds_weights, round_x, to_dev, tune
 
 pytestmark = pytest.mark.gpu
 ops = None
@@ -63,7 +63,7 @@ def kernel_of_last_call():
 def test_narrow_layout_forced_on_small_shapes(kind, dtn, K, N, g, monkeypatch):
     """N >= 2048 takes the single-strip form for its first 8 or 16 rows; the narrower ones always run
     four strips a workgroup.  K/128 = 2, 3, 5, 8 blocks over 8 waves: empty waves, odd shares, ring tails."""
-    monkeypatch.setenv("OXQ_PK4_STRIP16", "2")
+    tune("OXQ_PK4_STRIP16", 2)
     dt = DT[dtn]
     trip, pack_dim = make(kind, K, N, g, seed=K + N)
     bias = (np.arange(N, dtype=np.float32) % 13 - 6) * np.float32(0.125)
@@ -93,8 +93,8 @@ def test_narrow_layout_forced_on_small_shapes(kind, dtn, K, N, g, monkeypatch):
 
 @pytest.mark.parametrize("ks", [2, 3])
 def test_narrow_layout_k_slices(ks, monkeypatch):
-    monkeypatch.setenv("OXQ_PK4_STRIP16", "2")
-    monkeypatch.setenv("OXQ_PK4_KS", str(ks))
+    tune("OXQ_PK4_STRIP16", 2)
+    tune("OXQ_PK4_KS", ks)
     dt = oracle.F16
     K, N = 1152, 128
     trip, pack_dim = make("awq", K, N, 128, seed=ks)
@@ -120,9 +120,9 @@ def test_attention_and_down_projection_shapes_take_the_narrow_layout(K, N, monke
     dt = oracle.F16
     trip, pack_dim = make("awq", K, N, 128, seed=N)
     layer = layer_of(trip, pack_dim, dt)
-    monkeypatch.setenv("OXQ_PK4_STRIP16", "0")
+    tune("OXQ_PK4_STRIP16", 0)
     wide = layer_of(trip, pack_dim, dt)
-    monkeypatch.delenv("OXQ_PK4_STRIP16")
+    tune("OXQ_PK4_STRIP16", None)
     w = dense("awq", trip, dt)
     np.testing.assert_array_equal(bits_of(layer.dequantize()), bits_of(wide.dequantize()))
     wide16 = (N // 16 <= 256 and K // 128 <= 32) or ((N // 16) % 256 == 0 and K // 128 <= 64)
@@ -164,7 +164,7 @@ def test_sixteen_wave_workgroups_on_a_long_k(kind, dtn, monkeypatch):
     np.testing.assert_array_equal(bits_of(layer.dequantize()), oracle.transpose_convert(w, dt))
     rng = np.random.default_rng(K)
     for front in (1, 0):
-        monkeypatch.setenv("OXQ_PK4_FRONT", str(front))
+        tune("OXQ_PK4_FRONT", front)
         for m in (1, 2, 3, 4, 5, 8):
             say(f"narrow 16 waves {kind} {dtn} m={m} up-front={front}")
             x = rng.standard_normal((m, K)).astype(np.float32)

@@ -12,7 +12,7 @@ import torch
 
 import oracle
 from oxydllm_amd import ops, synth
-from tests.helpers import assert_close, round_x, to_dev, resident_rounds_weights
+from tests.helpers import assert_close, round_x, to_dev, resident_rounds_weights, tune
 
 pytestmark = pytest.mark.gpu
 
@@ -92,9 +92,9 @@ def test_resident_layer_random_shapes(monkeypatch):
         else:
             w = oracle.dequantize_awq8(qw, qz, s_r)
         if rng.integers(0, 2):
-            monkeypatch.setenv("OXQ_PK4_KS", str(int(rng.integers(2, 6))))
+            tune("OXQ_PK4_KS", int(rng.integers(2, 6)))
         else:
-            monkeypatch.delenv("OXQ_PK4_KS", raising=False)
+            tune("OXQ_PK4_KS", None)
         layer = ops.PackedQuantLinear(bits, ops.PACK_IN if gptq else ops.PACK_OUT, to_dev(qw), to_dev(qz),
                                       to_dev(sc, tdt), None, tdt)
         assert layer.prepacked

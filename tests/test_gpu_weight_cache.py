@@ -118,15 +118,23 @@ def test_forget_evict_and_ineligible_shapes():
         assert not ctx.last_plan()["kernel"].startswith("pk4")
 
         one = (K // 128) * (N // 64) * (1024 + 64) * 4          # bytes of one copy
-        say("weight cache: room for one copy, two weights in turn")
+        say("weight cache: room for one copy, two weights in turn: the first stays, the second keeps its own kernel")
         ctx.set_weight_cache(one + 256)
         for rnd in range(3):
-            for d, r in zip(devs, ref):
+            for i, (d, r) in enumerate(zip(devs, ref)):
                 ops.w4a16_matmul(x, *d, out=y, ctx=ctx)
-                assert ctx.last_plan()["kernel"].startswith("pk4")
+                # evicting the copy the next call asks for would rebuild one on every call
+                assert ctx.last_plan()["kernel"].startswith("pk4") == (i == 0), (rnd, i, ctx.last_plan()["kernel"])
                 torch.cuda.synchronize()
                 np.testing.assert_allclose(as_f32(y), r, rtol=2e-3, atol=1e-2)
                 assert ctx.weight_cache_usage()[1] == 1
+        say("weight cache: a weight that keeps coming alone takes the room")
+        for _ in range(4):
+            ops.w4a16_matmul(x, *devs[1], out=y, ctx=ctx)
+        assert ctx.last_plan()["kernel"].startswith("pk4")
+        torch.cuda.synchronize()
+        np.testing.assert_allclose(as_f32(y), ref[1], rtol=2e-3, atol=1e-2)
+        assert ctx.weight_cache_usage()[1] == 1
 
         say("weight cache: forget one, forget all")
         ctx.set_weight_cache(8 * one)
@@ -243,5 +251,30 @@ def test_capture_allocates_nothing_and_replays_the_cached_kernel():
             g2.replay()
             torch.cuda.synchronize()
             np.testing.assert_array_equal(bits_of(y), want, err_msg=f"replay {i}")
+
+        say("weight cache: the copy a captured graph holds survives a smaller limit and other weights")
+        one = ctx.weight_cache_usage()[0]
+        ctx.set_weight_cache(256)                                  # would drop every copy that is not held
+        assert ctx.weight_cache_usage() == (one, 1)
+        ctx.set_weight_cache(one + 256)                            # room for one: a second weight would evict it
+        trip2 = synth.awq_checkpoint(K, N, g, 4, seed=10)
+        dev2 = (to_dev(trip2[0]), to_dev(trip2[1]), to_dev(trip2[2], tdt))
+        y2 = torch.empty((m, N), device="cuda", dtype=tdt)
+        for _ in range(5):
+            ops.w4a16_matmul(x, *dev2, out=y2, ctx=ctx)
+            assert not ctx.last_plan()["kernel"].startswith("pk4")
+        assert ctx.weight_cache_usage() == (one, 1)
+        y.zero_()
+        ops.w4a16_matmul(x, *dev, out=y, ctx=ctx)
+        torch.cuda.synchronize()
+        want = bits_of(y).copy()
+        y.zero_()
+        torch.cuda.synchronize()
+        g2.replay()
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(bits_of(y), want, err_msg="replay after the limit shrank")
+        del g2                                                     # forgetting the weight invalidates the graph
+        ctx.forget_weights(dev[0])
+        assert ctx.weight_cache_usage() == (0, 0)
     finally:
         ctx.close()

@@ -18,7 +18,7 @@ import torch
 import oracle
 from oxydllm_amd import synth
 from tests import refgen
-from tests.helpers import RTOL, ATOL, TORCH_DT, as_f32, assert_close, bits_of, round_x, to_dev, resident_rounds_weights
+from tests.helpers import RTOL, ATOL, TORCH_DT, as_f32, assert_close, bits_of, round_x, to_dev, resident_rounds_weights, tune
 
 pytestmark = pytest.mark.gpu
 ops = None
@@ -373,13 +373,13 @@ def test_8bit_fast_gemv(method, dtn, K, N, g, monkeypatch):
         say(f"8-bit fast {method} {dtn} K={K} N={N} g={g} m={m}")
         x = rng.standard_normal((m, K)).astype(np.float32)
         xd = to_dev(x, TORCH_DT[dt])
-        monkeypatch.delenv("OXQ_FORCE_GENERIC", raising=False)
+        tune("OXQ_FORCE_GENERIC", None)
         y = op(xd)
         kern = ops.default_context().last_plan()["kernel"]
         assert kern.startswith(f"{method}8_gemv_fast_{dtn}"), kern
         assert_close(y, oracle.matmul_nt_f32(round_x(x, dt), w), f"{method}8 fast {dtn} m{m}")
         np.testing.assert_array_equal(bits_of(op(xd)), bits_of(y))          # run-to-run
-        monkeypatch.setenv("OXQ_FORCE_GENERIC", "1")
+        tune("OXQ_FORCE_GENERIC", 1)
         yg = op(xd)
         assert "generic" in ops.default_context().last_plan()["kernel"]
         # two roundings of nearly equal sums may land one output ulp apart
@@ -406,17 +406,17 @@ def test_stateless_tile_op_on_layouts_without_a_tile_kernel(method, bits, dtn, m
         say(f"transient repack {method}{bits} {dtn} m={m}")
         x = rng.standard_normal((m, K)).astype(np.float32)
         xd = to_dev(x, TORCH_DT[dt])
-        monkeypatch.delenv("OXQ_TRANSIENT_REPACK", raising=False)
+        tune("OXQ_TRANSIENT_REPACK", None)
         y = ops.mpp_quant_matmul(xd, *d, bits, pd)
         plan = ops.default_context().last_plan()
         assert plan["kernel"].startswith(f"pk{bits}_mfma_{dtn}") and plan["launches"] == 2, plan
         wr = oracle.round_through(w, dt) if resident_rounds_weights(m, dt, method == "gptq") else w
         assert_close(y, oracle.matmul_nt_f32(round_x(x, dt), wr), f"{method}{bits} {dtn} m{m} (repacked in the workspace)")
-        monkeypatch.setenv("OXQ_TRANSIENT_REPACK", "0")
+        tune("OXQ_TRANSIENT_REPACK", 0)
         y2 = ops.mpp_quant_matmul(xd, *d, bits, pd)
         assert "gemv" in ops.default_context().last_plan()["kernel"]
         assert_close(y2, oracle.matmul_nt_f32(round_x(x, dt), w), f"{method}{bits} {dtn} m{m} (GEMV passes)")
-    monkeypatch.delenv("OXQ_TRANSIENT_REPACK", raising=False)
+    tune("OXQ_TRANSIENT_REPACK", None)
     aw = synth.awq_checkpoint(2048, 128, 128, 4, seed=3)
     ad = dev_triplet(*aw, dt)
     wa = oracle.dequantize_awq(aw[0], aw[1], oracle.round_through(aw[2], dt))
@@ -441,9 +441,8 @@ def test_splitk_fused_and_two_launch_sums_give_the_same_bits(route, dtn, monkeyp
     d = dev_triplet(qw, qz, sc, dt)
     ctxs = {}
     for mode in (1, 2):
-        monkeypatch.setenv("OXQ_SPLITK_MODE", str(mode))
         ctxs[mode] = ops.Context()
-    monkeypatch.delenv("OXQ_SPLITK_MODE")
+        tune("OXQ_SPLITK_MODE", mode, ctx=ctxs[mode])
     for m in (1, 3, 8):
         if m > 1 and dtn == "f16" and bits == 4 and not gptq:
             continue  # f16 batches on 4-bit AWQ run the tile kernel, which always sums with the second launch

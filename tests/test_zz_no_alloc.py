@@ -14,7 +14,7 @@ import torch
 
 import oracle
 from oxydllm_amd import _lib, synth
-from tests.helpers import TORCH_DT, assert_close, bits_of, fake, round_x, to_dev
+from tests.helpers import TORCH_DT, assert_close, bits_of, fake, round_x, to_dev, tune
 
 pytestmark = pytest.mark.gpu
 
@@ -54,6 +54,20 @@ def test_static_scratch_matches_workspace_entry_point_two_calls(dtn):
         assert plan_st["kernel"] == plan_ws["kernel"] and plan_st["split_k"] == plan_ws["split_k"]
         assert np.array_equal(bits_of(got), bits_of(want)), f"{dtn} m={m} {K}x{N}: bits differ from oxq_w4a16_matmul"
         assert_close(got, ref, f"static {dtn} m={m} {K}x{N}")
+        # what the entry point is for: it runs under stream capture (an allocation there fails the capture) and
+        # leaves the device's free memory as it found it; every replay gives the eager bits
+        free0 = torch.cuda.mem_get_info()[0]
+        graph, stream = torch.cuda.CUDAGraph(), torch.cuda.Stream()
+        with torch.cuda.graph(graph, stream=stream):
+            ops.w4a16_matmul_static(xd, *d, out=out, ctx=ctx)
+        for rep in range(3):
+            out.fill_(float("nan"))
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert np.array_equal(bits_of(out), bits_of(want)), f"{dtn} m={m} {K}x{N}: replay {rep} differs"
+        assert torch.cuda.mem_get_info()[0] >= free0 - (1 << 20), "device memory was allocated"  # (graph objects: < 1 MiB)
+        del graph
 
 
 def test_static_scratch_rejects_oversize_and_plans_without_gpu_memory(monkeypatch):
@@ -63,7 +77,7 @@ def test_static_scratch_rejects_oversize_and_plans_without_gpu_memory(monkeypatc
     # The library's own slicing keeps the partial sums of any shape within a few MiB; one K slice per
     # group (a tuning switch) on 8 rows x 131072 columns asks for 32 x 8 x 131072 x 4 bytes = 128 MiB,
     # which the 16 MiB array cannot hold: refused on the host, nothing is enqueued.
-    monkeypatch.setenv("OXQ_GEMV_GPW", "1")
+    tune("OXQ_GEMV_GPW", 1, ctx=plan)
     K, N, g, m = 4096, 131072, 128, 8
     args = (fake((m, K), _lib.BF16), fake((K, N // 8), _lib.I32), fake((K // g, N // 8), _lib.I32),
             fake((K // g, N), _lib.BF16), fake((m, N), _lib.BF16))
@@ -71,7 +85,7 @@ def test_static_scratch_rejects_oversize_and_plans_without_gpu_memory(monkeypatc
     msg = lib.oxq_last_error().decode()
     assert rc == -10, (rc, msg)  # OXQ_ERR_WORKSPACE
     assert "static scratch" in msg and "16777216" in msg, msg
-    monkeypatch.delenv("OXQ_GEMV_GPW")
+    tune("OXQ_GEMV_GPW", None, ctx=plan)
     # a plan-only ctx answers without a device
     small = (fake((1, 4096), _lib.F16, device=0), fake((4096, 512), _lib.I32, device=0), fake((32, 512), _lib.I32, device=0),
              fake((32, 4096), _lib.F16, device=0), fake((1, 4096), _lib.F16, device=0))
