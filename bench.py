@@ -274,7 +274,7 @@ def main():
     #    in flight a lane (plain / nontemporal);
     #  * bare_read_best_us: the same bytes with every lane's whole share requested before the first wait, as the
     #    M <= 16 kernels request their weights - the best of 8 and 16 waves a workgroup, nontemporal.
-    bare = {}
+    bare, streams = {}, None
     if not args.no_bare_read:
         nbytes_w = K * N // 2
         pool = torch.empty(copies * nbytes_w, dtype=torch.uint8, device=dev).random_(0, 256)
@@ -299,10 +299,21 @@ def main():
         bare["bare_read_best_us"] = min(best.values())
         bare["bare_read_best_waves"] = min(best, key=best.get)
         bare["bare_read_upfront_us_by_waves"] = best
+        # the M = 64 kernel's two request streams, alone and together: the strip's weights (cold) and the 64 rows of x
+        # that every workgroup reads whole (512 KB, L2 hits), the latter straight into LDS as that kernel does it
+        xs = torch.empty(64 * K * 2, dtype=torch.uint8, device=dev).random_(0, 256)
+        streams = {}
+        for which, key in ((1, "weights_us"), (2, "x_64_rows_us"), (3, "both_us")):
+            def rd(i, which=which):
+                c = i % copies
+                ops.two_streams(pool[c * nbytes_w:(c + 1) * nbytes_w], xs, N // 64, which, sums, ctx=ctx)
+            _, ev = time_graph(rd, args.steps, args.warmup, stream)
+            streams[key] = round(ev * 1e3 / args.steps, 3)
         bare["bare_read_bytes"] = nbytes_w
         bare["bare_read_workgroups"] = N // 64
         print(f"[bench] plain read of {nbytes_w} B by {N // 64} workgroups: {bare}", file=sys.stderr, flush=True)
-        del pool
+        print(f"[bench] two request streams a compute unit (M = 64): {streams}", file=sys.stderr, flush=True)
+        del pool, xs
 
     c1 = cases[0]
     # HBM bytes per launch of the M=1 kernel, measured offline with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE) and
@@ -347,7 +358,8 @@ def main():
         "roofline_m64": {"bound": "mfma", "achieved": cases[2]["TFLOP_per_s"],
                          "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                          "frac": cases[2]["mfma_frac"], "traffic": None,
-                         "kernel": cases[2]["kernel"], "hbm_frac": cases[2]["hbm_frac"]},
+                         "kernel": cases[2]["kernel"], "hbm_frac": cases[2]["hbm_frac"],
+                         "us_per_launch": cases[2]["us_per_call"], "request_streams_us": streams},
         "cases": cases,
         "cases_down_projection_K14336_N4096": down_cases,
         "cases_checkpoint_layout_ops": op_cases,
@@ -356,14 +368,14 @@ def main():
     del layers, qw_d, qz_d, sc_d
     torch.cuda.empty_cache()
     if not args.no_others:
-        from oxydllm_amd import bench_configs
+        import bench_configs
         result["other_configs"] = bench_configs.run(ops, ctx, stream, args.steps, args.warmup, time_graph,
                                                     with_cpu=not args.no_cpu)
         for r in result["other_configs"]:
             print(f"[bench] {r['config']}: {r['case']}: {r['us_per_call']} us, {r['GB_per_s']} GB/s "
                   f"({r['roofline']['frac']:.3f} of HBM peak), {r['kernel']}", file=sys.stderr, flush=True)
     if args.all:
-        from oxydllm_amd import bench_extra
+        import bench_extra
         result["extra_configs"] = bench_extra.run(ops, ctx, stream, args.steps, args.warmup, time_graph)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(qw, qz, sc, x_host[1])

@@ -18,7 +18,7 @@ import time
 import numpy as np
 import torch
 
-from . import synth
+from oxydllm_amd import synth
 
 HBM_PEAK_GBS = 8000.0
 

@@ -13,7 +13,7 @@ from __future__ import annotations
 import numpy as np
 import torch
 
-from . import synth
+from oxydllm_amd import synth
 
 HBM_PEAK_GBS = 8000.0
 

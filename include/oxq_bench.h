@@ -27,6 +27,15 @@ int oxq_calib_read(oxq_ctx *ctx, void *stream, const oxq_tensor *src, int workgr
 int oxq_bench_read_upfront(oxq_ctx *ctx, void *stream, const oxq_tensor *src, int workgroups, int waves,
                            int nontemporal, const oxq_tensor *checksums);
 
+/* Two request streams from every compute unit.  Workgroups of 12 waves: waves 0 - 7 read the workgroup's
+ * span of `w` (U8; workgroups x 64, 128 or 136 KiB; cold, so from HBM) with everything requested first, waves
+ * 8 - 11 read all of `x` (U8, a multiple of 32 KiB; the same bytes in every workgroup, so L2 hits) straight
+ * into LDS, as a tile kernel stages its activations.  which = 1: only w, 2: only x, 3: both at once.  On
+ * this machine "both" takes about the sum of the two, not the larger (a compute unit serves its vector-memory
+ * requests in issue order): that is the price of the activation rows a tile kernel re-reads per strip. */
+int oxq_bench_two_streams(oxq_ctx *ctx, void *stream, const oxq_tensor *w, const oxq_tensor *x, int workgroups,
+                          int which, const oxq_tensor *checksums);
+
 /* An empty kernel with the given launch shape (threads a multiple of 64, up to 1024; lds_bytes of
  * dynamic LDS, up to 160 KiB): what one launch costs when it does nothing. */
 int oxq_bench_empty_launch(oxq_ctx *ctx, void *stream, int workgroups, int threads, int lds_bytes);

@@ -643,6 +643,31 @@ int oxq_bench_read_upfront(oxq_ctx *ctx, void *stream, const oxq_tensor *src, in
                                 nontemporal, (uint32_t *)checksums->data);
 }
 
+int oxq_bench_two_streams(oxq_ctx *ctx, void *stream, const oxq_tensor *w, const oxq_tensor *x, int workgroups,
+                          int which, const oxq_tensor *checksums) {
+    if (!ctx || !w || !x || !checksums) return fail(OXQ_ERR_ARG, "TwoStreams: NULL argument");
+    OXQ_TRY(check_tensor(ctx, "TwoStreams", "w", w));
+    OXQ_TRY(check_tensor(ctx, "TwoStreams", "x", x));
+    OXQ_TRY(check_tensor(ctx, "TwoStreams", "checksums", checksums));
+    if (w->dtype != OXQ_U8 || !w->contiguous || x->dtype != OXQ_U8 || !x->contiguous)
+        return fail(OXQ_ERR_DTYPE, "TwoStreams: w and x must be contiguous U8 tensors");
+    if ((checksums->dtype != OXQ_U32 && checksums->dtype != OXQ_I32) || !checksums->contiguous)
+        return fail(OXQ_ERR_DTYPE, "TwoStreams: checksums must be a contiguous U32/I32 tensor");
+    if (which < 1 || which > 3) return fail(OXQ_ERR_ARG, "TwoStreams: which = %d (1 w, 2 x, 3 both)", which);
+    const int64_t wb = numel(w), xb = numel(x);
+    if (workgroups < 1 || workgroups > 65535 || numel(checksums) < workgroups)
+        return fail(OXQ_ERR_SHAPE, "TwoStreams: %d workgroups need 1..65535 and one checksum word each", workgroups);
+    const int64_t span = wb / workgroups;
+    if (wb <= 0 || wb % workgroups != 0 || (span != 8 * 8192 && span != 16 * 8192 && span != 17 * 8192))
+        return fail(OXQ_ERR_SHAPE, "TwoStreams: w must be workgroups x 64, 128 or 136 KiB (got %lld bytes)", (long long)wb);
+    if (xb <= 0 || xb % (4 * 8192) != 0 || xb >= (int64_t(1) << 31))
+        return fail(OXQ_ERR_SHAPE, "TwoStreams: x must be a multiple of 32 KiB below 2 GiB (got %lld bytes)", (long long)xb);
+    if (!ctx->plan_only && (((uintptr_t)w->data | (uintptr_t)x->data) & 15))
+        return fail(OXQ_ERR_UNSUPPORTED, "TwoStreams: w and x must be 16-byte aligned");
+    return launch_calib_two_streams(ctx, (hipStream_t)stream, (const uint8_t *)w->data, (uint64_t)wb, (const uint8_t *)x->data,
+                                    (uint64_t)xb, workgroups, which, (uint32_t *)checksums->data);
+}
+
 int oxq_bench_empty_launch(oxq_ctx *ctx, void *stream, int workgroups, int threads, int lds_bytes) {
     if (!ctx) return fail(OXQ_ERR_ARG, "EmptyLaunch: ctx is NULL");
     if (workgroups < 1 || workgroups > 65535 || threads < 64 || threads > 1024 || threads % 64 != 0 || lds_bytes < 0 ||

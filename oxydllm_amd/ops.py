@@ -153,6 +153,14 @@ def read_upfront(src, workgroups: int, waves: int, nontemporal: bool, checksums,
     return checksums
 
 
+def two_streams(w, x, workgroups: int, which: int, checksums, *, ctx: Optional[Context] = None):
+    """Cold weight stream and L2-resident activation stream from every compute unit, alone (which = 1, 2) or
+    together (3) (include/oxq_bench.h)."""
+    ctx = _ctx(ctx)
+    _lib.check(ctx._lib.oxq_bench_two_streams(ctx.handle, ctx.stream(), desc(w), desc(x), int(workgroups), int(which),
+                                              desc(checksums)))
+
+
 def empty_launch(workgroups: int, threads: int, lds_bytes: int = 0, *, ctx: Optional[Context] = None):
     """An empty kernel of the given launch shape (include/oxq_bench.h)."""
     ctx = _ctx(ctx)
