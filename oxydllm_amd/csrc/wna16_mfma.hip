@@ -696,7 +696,9 @@ int launch_wna16_mfma(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p) {
     if (awq4_mfma_ok(p) && !tune(ctx, OXQ_TUNE_FORCE_GENERIC, 0))
         return p.dtype == OXQ_F16 ? launch_awq4_mfma<F16Traits>(ctx, s, p)
                                   : launch_awq4_mfma<BF16Traits>(ctx, s, p);
-    // Layouts without a tile kernel of their own on the checkpoint layout (GPTQ, 8-bit AWQ): when the
+    if (gptq_tile_ok(p) && tune(ctx, OXQ_TUNE_GPTQ_TILE, 1) && !tune(ctx, OXQ_TUNE_FORCE_GENERIC, 0))
+        return launch_gptq_tile(ctx, s, p);
+    // Layouts without a tile kernel of their own on the checkpoint layout (8-bit AWQ, unaligned GPTQ): when the
     // tile-major copy fits the ctx workspace, build it there and run the resident-layer kernel on it.
     // One launch more (about 45 us at 5120 x 13824, 4-bit) instead of one GEMV pass over the weights
     // per 8 rows (35 - 45 us each): ahead from m = 9.  A caller that holds the layer should hold a

@@ -99,9 +99,9 @@ def test_block_quant_paths_in_a_graph():
 
 
 def test_fused_epilogues_and_workspace_repack_in_a_graph():
-    """The gate|up layer with the activation in its epilogue, the stateless tile op that builds its
-    tile-major copy in the ctx workspace (three kernels, the workspace rewritten on every replay), the
-    8-bit GEMV kernels, and the expert GEMV with the fused SwiGLU."""
+    """The gate|up layer with the activation in its epilogue, the GPTQ tile kernel on the checkpoint layout,
+    the stateless tile op that builds its tile-major copy in the ctx workspace (the workspace rewritten on
+    every replay), and the expert GEMV with the fused SwiGLU."""
     gen = torch.Generator(device="cuda")
     K, I = 1024, 256
     trip = synth.awq_checkpoint(K, 2 * I, 128, 4, seed=3)
@@ -132,7 +132,23 @@ def test_fused_epilogues_and_workspace_repack_in_a_graph():
                 fn = lambda: ops.mpp_quant_matmul(x, *d, bits, ops.PACK_IN, out=y)
             replay_matches_eager(f"gptq{bits} m={m}", fn, inputs, y)
             if m > 8:
-                assert ops.default_context().last_plan()["launches"] == 2
+                plan = ops.default_context().last_plan()
+                assert plan["kernel"].startswith(f"gptq{bits}_tile") and plan["launches"] == 1, plan
+
+    # 8-bit AWQ above 8 rows has no tile kernel on the checkpoint layout: the op repacks into the ctx
+    # workspace and runs the resident-layer kernel on the copy (two launches, the workspace rewritten on
+    # every replay)
+    aq = synth.awq_checkpoint(K, 384, 128, 8, seed=11)
+    d = (to_dev(aq[0]), to_dev(aq[1]), to_dev(aq[2], torch.float16))
+    m = 24
+    x = torch.empty((m, K), device="cuda", dtype=torch.float16)
+    y = torch.empty((m, 384), device="cuda", dtype=torch.float16)
+
+    def inputs(i):
+        gen.manual_seed(500 + i)
+        x.copy_(torch.randn((m, K), device="cuda", generator=gen).to(torch.float16))
+    replay_matches_eager(f"awq8 m={m}", lambda: ops.mpp_quant_matmul(x, *d, 8, ops.PACK_OUT, out=y), inputs, y)
+    assert ops.default_context().last_plan()["launches"] == 2
 
     E, N, Kx = 3, 64, 96
     blocks = torch.from_numpy(np.concatenate([synth.mxfp4_weight(N, Kx, seed=e)[0] for e in range(E)])).cuda()

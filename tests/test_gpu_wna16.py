@@ -369,6 +369,7 @@ def test_8bit_fast_gemv(method, dtn, K, N, g, monkeypatch):
     w = oracle.dequantize_awq8(qw, qz, s_r) if method == "awq" else oracle.dequantize_gptq(qw, qz, s_r, 8)
     op = (lambda x: ops.w8a16_matmul(x, *d)) if method == "awq" else (lambda x: ops.gptq_matmul(x, *d, 8))
     rng = np.random.default_rng(K * 3 + N)
+    tune("OXQ_GPTQ_TILE", 0)  # this test is about the dot-product kernels (the tile kernel: test_gpu_gptq_tile.py)
     for m in (1, 2, 3, 4, 7, 8):
         say(f"8-bit fast {method} {dtn} K={K} N={N} g={g} m={m}")
         x = rng.standard_normal((m, K)).astype(np.float32)
@@ -389,10 +390,11 @@ def test_8bit_fast_gemv(method, dtn, K, N, g, monkeypatch):
 @pytest.mark.parametrize("method,bits", [("gptq", 4), ("gptq", 8), ("awq", 8)])
 @pytest.mark.parametrize("dtn", ["f16", "bf16"])
 def test_stateless_tile_op_on_layouts_without_a_tile_kernel(method, bits, dtn, monkeypatch):
-    """mpp_quant_matmul on GPTQ / 8-bit AWQ checkpoint tensors: the tile-major copy is built in the ctx
-    workspace and the resident-layer kernel runs on it (two launches); with the switch off the call
-    falls back to GEMV passes of 8 rows.  Both against the oracle; a following 4-bit AWQ call on the same
-    ctx (which uses the workspace for K slices) still gives the right answer."""
+    """mpp_quant_matmul on GPTQ / 8-bit AWQ checkpoint tensors.  GPTQ runs its own tile kernel on the
+    checkpoint layout (one launch); with that switched off, and for 8-bit AWQ, the tile-major copy is built
+    in the ctx workspace and the resident-layer kernel runs on it (two launches); with that switch off too
+    the call falls back to GEMV passes of 8 rows.  All against the oracle; a following 4-bit AWQ call on the
+    same ctx (which uses the workspace for K slices) still gives the right answer."""
     dt = DT[dtn]
     K, N, g = 1024, 384, 128
     make = synth.awq_checkpoint if method == "awq" else synth.gptq_checkpoint
@@ -407,6 +409,15 @@ def test_stateless_tile_op_on_layouts_without_a_tile_kernel(method, bits, dtn, m
         x = rng.standard_normal((m, K)).astype(np.float32)
         xd = to_dev(x, TORCH_DT[dt])
         tune("OXQ_TRANSIENT_REPACK", None)
+        if method == "gptq":
+            tune("OXQ_GPTQ_TILE", None)
+            y = ops.mpp_quant_matmul(xd, *d, bits, pd)
+            plan = ops.default_context().last_plan()
+            assert plan["kernel"].startswith(f"gptq{bits}_tile_{dtn}") and plan["launches"] == 1, plan
+            # the tile kernel keeps the unrounded weight up to 32 rows (the reach of the reference's GEMV)
+            wr = oracle.round_through(w, dt) if m > 32 else w
+            assert_close(y, oracle.matmul_nt_f32(round_x(x, dt), wr), f"{method}{bits} {dtn} m{m} (tile kernel on the checkpoint layout)")
+            tune("OXQ_GPTQ_TILE", 0)
         y = ops.mpp_quant_matmul(xd, *d, bits, pd)
         plan = ops.default_context().last_plan()
         assert plan["kernel"].startswith(f"pk{bits}_mfma_{dtn}") and plan["launches"] == 2, plan
@@ -443,6 +454,7 @@ def test_splitk_fused_and_two_launch_sums_give_the_same_bits(route, dtn, monkeyp
     for mode in (1, 2):
         ctxs[mode] = ops.Context()
         tune("OXQ_SPLITK_MODE", mode, ctx=ctxs[mode])
+        tune("OXQ_GPTQ_TILE", 0, ctx=ctxs[mode])  # the GPTQ tile kernel keeps K inside the workgroup: nothing to sum
     for m in (1, 3, 8):
         if m > 1 and dtn == "f16" and bits == 4 and not gptq:
             continue  # f16 batches on 4-bit AWQ run the tile kernel, which always sums with the second launch

@@ -66,7 +66,9 @@ def test_static_scratch_matches_workspace_entry_point_two_calls(dtn):
             graph.replay()
             torch.cuda.synchronize()
             assert np.array_equal(bits_of(out), bits_of(want)), f"{dtn} m={m} {K}x{N}: replay {rep} differs"
-        assert torch.cuda.mem_get_info()[0] >= free0 - (1 << 20), "device memory was allocated"  # (graph objects: < 1 MiB)
+        # an instantiated graph may take a 2 MiB chunk of device memory for its own bookkeeping; the workspace the
+        # other entry point would allocate for these shapes is 64 MiB
+        assert torch.cuda.mem_get_info()[0] >= free0 - (8 << 20), "device memory was allocated"
         del graph
 
 
