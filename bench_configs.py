@@ -27,20 +27,27 @@ def _copies_for(nbytes: int, want_total: int = 400 << 20, cap: int = 24) -> int:
     return int(max(2, min(cap, -(-want_total // max(1, nbytes)))))
 
 
-def _row(config, case, fn_of_step, steps, warmup, stream, time_graph, nbytes, flops, ctx):
+MFMA_PEAK_TFLOPS = 2500.0  # dense f16 / bf16
+
+
+def _row(config, case, fn_of_step, steps, warmup, stream, time_graph, nbytes, flops, ctx, mfma=False):
+    """mfma: price the row against the dense 16-bit MFMA peak (tile GEMMs at 64 rows) instead of HBM."""
     fn_of_step(0)
     plan = ctx.last_plan()
     _, ev_ms = time_graph(fn_of_step, steps, warmup, stream)
     us = ev_ms * 1e3 / steps
     gbs = nbytes / us / 1e3
+    tf = flops / us / 1e6
+    roof = ({"bound": "mfma", "achieved": round(tf, 2), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+             "frac": round(tf / MFMA_PEAK_TFLOPS, 4)} if mfma else
+            {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+             "frac": round(gbs / HBM_PEAK_GBS, 4)})
     return {"config": config, "case": case, "kernel": plan["kernel"], "launches": plan["launches"],
             "us_per_call": round(us, 3), "algorithmic_bytes": int(nbytes), "GB_per_s": round(gbs, 1),
-            "TFLOP_per_s": round(flops / us / 1e6, 3),
-            "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": round(gbs / HBM_PEAK_GBS, 4)}}
+            "TFLOP_per_s": round(tf, 3), "roofline": roof}
 
 
-def _cached_row(config, case, call, nc, steps, warmup, stream, time_graph, nbytes, flops, ctx):
+def _cached_row(config, case, call, nc, steps, warmup, stream, time_graph, nbytes, flops, ctx, mfma=False):
     """`call(c)` on weight copy c with the ctx's opt-in weight cache on: every copy is seen once
     outside the timed region (that call builds its tile-major copy), the timed calls find it."""
     ctx.set_weight_cache(2 << 30)
@@ -48,7 +55,7 @@ def _cached_row(config, case, call, nc, steps, warmup, stream, time_graph, nbyte
         for c in range(nc):
             call(c)
         torch.cuda.synchronize()
-        return _row(config, case, lambda i: call(i % nc), steps, warmup, stream, time_graph, nbytes, flops, ctx)
+        return _row(config, case, lambda i: call(i % nc), steps, warmup, stream, time_graph, nbytes, flops, ctx, mfma)
     finally:
         ctx.set_weight_cache(0)
 
@@ -122,14 +129,14 @@ def run(ops, ctx, stream, steps, warmup, time_graph, with_cpu=True):
              for _ in range(nc)]
         layers = [ops.PackedQuantLinear(bits, ops.PACK_IN, *c, None, torch.float16, ctx=ctx) for c in d]
         first = True
-        for m in (1, 8):
+        for m in (1, 8, 64):  # 64 rows: the prefill tile op on the same tensors (mpp_quant_matmul)
             xh = np.random.default_rng(20 + m).standard_normal((m, K)).astype(np.float32)
             x = torch.from_numpy(xh).to(dev, torch.float16)
             y = torch.empty((m, N), device=dev, dtype=torch.float16)
             nb = wbytes + m * K * 2 + m * N * 2
             r = _row("cfg2", f"gptq{bits} M={m} K={K} N={N} g={G} f16, PackedQuantLinear.forward (resident layer)",
                      lambda i, x=x, y=y: layers[i % nc].forward(x, out=y), steps, warmup, stream, time_graph, nb,
-                     2.0 * m * K * N, ctx)
+                     2.0 * m * K * N, ctx, m >= 64)
             if with_cpu and first and bits == 4:
                 w = oracle.dequantize_gptq(qw, qz, oracle.round_through(sc, oracle.F16), bits)
                 r["cpu_baseline"] = _cpu_dense(w, oracle.round_through(xh, oracle.F16), nb,
@@ -137,13 +144,18 @@ def run(ops, ctx, stream, steps, warmup, time_graph, with_cpu=True):
                 del w
             first = False
             rows.append(r)
-            rows.append(_row("cfg2", f"gptq{bits} M={m} K={K} N={N} g={G} f16, gptq_matmul op (checkpoint layout)",
-                             lambda i, x=x, y=y, bits=bits: ops.gptq_matmul(x, *d[i % nc], bits, out=y, ctx=ctx),
-                             steps, warmup, stream, time_graph, nb, 2.0 * m * K * N, ctx))
-            rows.append(_cached_row("cfg2", f"gptq{bits} M={m} K={K} N={N} g={G} f16, gptq_matmul op with the ctx "
+            if m <= 8:
+                opn, op = "gptq_matmul", (lambda t, x=x, y=y, bits=bits: ops.gptq_matmul(x, *t, bits, out=y, ctx=ctx))
+            else:
+                opn, op = "mpp_quant_matmul", (lambda t, x=x, y=y, bits=bits: ops.mpp_quant_matmul(x, *t, bits, ops.PACK_IN,
+                                                                                                 out=y, ctx=ctx))
+            rows.append(_row("cfg2", f"gptq{bits} M={m} K={K} N={N} g={G} f16, {opn} op (checkpoint layout)",
+                             lambda i, op=op: op(d[i % nc]), steps, warmup, stream, time_graph, nb, 2.0 * m * K * N, ctx,
+                             m >= 64))
+            rows.append(_cached_row("cfg2", f"gptq{bits} M={m} K={K} N={N} g={G} f16, {opn} op with the ctx "
                                             "weight cache on",
-                                    lambda c, x=x, y=y, bits=bits: ops.gptq_matmul(x, *d[c], bits, out=y, ctx=ctx),
-                                    nc, steps, warmup, stream, time_graph, nb, 2.0 * m * K * N, ctx))
+                                    lambda c, op=op: op(d[c]), nc, steps, warmup, stream, time_graph, nb,
+                                    2.0 * m * K * N, ctx, m >= 64))
         del d, layers
 
     # ---- config 3 --------------------------------------------------------------------------------------

@@ -62,7 +62,13 @@ __global__ __launch_bounds__(512) void gptq_tile_kernel(const uint16_t *__restri
     constexpr int WL = BITS / 4;      // 16-byte loads a lane and MFMA step
     constexpr int XL = 2 * MT;        // 16-byte loads a lane and half block of x (64 rows of K)
     constexpr int STAGE = 16 * MT * 128;
+    // One row tile in straight-line code: the wave's whole share of x is put into LDS before the first block
+    // (2 PER stages a wave), requested ahead of the weights.  Otherwise x travels by half blocks through two
+    // stages a wave, and every request for it queues behind the weights requested before it.
+    constexpr bool XFRONT = MT == 1 && PER > 0;
+    constexpr int NSTAGE = XFRONT ? 2 * PER : 2;
     constexpr uint32_t OOB = 0x80000000u;
+    constexpr int WAUX = MT <= 2 ? 2 : 0;  // up to 32 rows one workgroup reads a strip's weights, once: nontemporal
     extern __shared__ __attribute__((aligned(16))) unsigned char pk4_lds[];
 
     const int lane = threadIdx.x & 63;
@@ -73,7 +79,7 @@ __global__ __launch_bounds__(512) void gptq_tile_kernel(const uint16_t *__restri
     const int per = PER ? PER : (NB + 7) >> 3;  // PER: K / 128 = 8 PER (launcher)
     const int b0 = wave * per;
     const int b1 = b0 + per < NB ? b0 + per : NB;
-    unsigned char *slot = pk4_lds + wave * 2 * STAGE;
+    unsigned char *slot = pk4_lds + wave * NSTAGE * STAGE;
 
     const int wrow = N * 4;  // bytes a word row
     const __amdgpu_buffer_rsrc_t rs_w = make_rsrc(qw, (uint32_t)(K / PF) * (uint32_t)wrow);
@@ -108,7 +114,7 @@ __global__ __launch_bounds__(512) void gptq_tile_kernel(const uint16_t *__restri
 #pragma unroll
             for (int u = 0; u < WL; ++u)
                 w.q[t][u] = __builtin_amdgcn_raw_buffer_load_b128(rs_w, (int)(voff_w + live + (uint32_t)u * wrow),
-                                                                 ((b * 4 + t) * 4 * WL) * wrow, 0);
+                                                                 ((b * 4 + t) * 4 * WL) * wrow, WAUX);
         w.z = __builtin_amdgcn_raw_buffer_load_b32(rs_z, (int)(voff_z + live), g * (N / PF) * 4, 0);
         const auto sv = __builtin_amdgcn_raw_buffer_load_b64(rs_s, (int)(voff_s + live), g * N * 2, 0);
         w.s[0] = sv[0], w.s[1] = sv[1];
@@ -120,7 +126,7 @@ __global__ __launch_bounds__(512) void gptq_tile_kernel(const uint16_t *__restri
         for (int i = 0; i < XL; ++i)
             xr[i] = __builtin_amdgcn_raw_buffer_load_b128(rs_x, (int)(xo0 + (uint32_t)i * xstep + live), b * 256 + h * 128, 0);
     };
-    auto stage_x = [&](int h) {
+    auto stage_x = [&](int h) {  // h: LDS stage
 #pragma unroll
         for (int i = 0; i < XL; ++i) {
             const u32x4_t n = xr[i];
@@ -165,14 +171,14 @@ __global__ __launch_bounds__(512) void gptq_tile_kernel(const uint16_t *__restri
             }
         }
     };
-    auto half = [&](const WB &w, int h) {
+    auto half = [&](const WB &w, int h, int st) {  // half h of the block, in LDS stage st
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
             const int t = 2 * h + u;
             uint32_t a[MT][4];
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
-                const u32x4_t av = *(const u32x4_t *)(slot + h * STAGE + mt * 2048 + a_rd + ((((4 * u + kb) ^ (ni >> 1)) & 7) << 4));
+                const u32x4_t av = *(const u32x4_t *)(slot + st * STAGE + mt * 2048 + a_rd + ((((4 * u + kb) ^ (ni >> 1)) & 7) << 4));
                 a[mt][0] = av[0], a[mt][1] = av[1], a[mt][2] = av[2], a[mt][3] = av[3];
             }
             if (FOLD) {
@@ -229,17 +235,47 @@ __global__ __launch_bounds__(512) void gptq_tile_kernel(const uint16_t *__restri
         if (more) load_w(bn, wn);
         __builtin_amdgcn_sched_barrier(0);  // requests stay where they are written (the scheduler sinks them to their use)
         pairs(w);
-        half(w, 0);
+        half(w, 0, 0);
         stage_x(1);
         load_x(b + 1, 0);
         __builtin_amdgcn_sched_barrier(0);
-        half(w, 1);
+        half(w, 1, 1);
+        fold();
+    };
+    // the same with x already in LDS: block i of the wave's share sits in stages 2 i and 2 i + 1
+    auto block_xfront = [&](int i, const WB &w, int bn, WB &wn, bool more) {
+        if (more) load_w(bn, wn);
+        __builtin_amdgcn_sched_barrier(0);
+        pairs(w);
+        half(w, 0, 2 * i);
+        half(w, 1, 2 * i + 1);
         fold();
     };
 
     // D register sets of weights in a ring, D - 1 blocks requested ahead.
     WB w[D];
-    if (PER) {
+    if (XFRONT) {
+        // x of the whole share first (the vector-memory counter runs in issue order: what is needed first is
+        // requested first), then the weights; x is in LDS by the time the first block's weights arrive
+        u32x4_t xa[NSTAGE][XL];
+#pragma unroll
+        for (int st = 0; st < NSTAGE; ++st)
+#pragma unroll
+            for (int i = 0; i < XL; ++i)
+                xa[st][i] = __builtin_amdgcn_raw_buffer_load_b128(rs_x, (int)(xo0 + (uint32_t)i * xstep), (b0 * 2 + st) * 128, 0);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < D - 1 && i < PER; ++i) load_w(b0 + i, w[i]);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int st = 0; st < NSTAGE; ++st) {
+#pragma unroll
+            for (int i = 0; i < XL; ++i) xr[i] = xa[st][i];
+            stage_x(st);
+        }
+#pragma unroll
+        for (int i = 0; i < PER; ++i) block_xfront(i, w[i % D], b0 + i + D - 1, w[(i + D - 1) % D], i + D - 1 < PER);
+    } else if (PER) {
         // K = 8 PER blocks: straight-line code, every wave PER blocks; D = PER requests a wave's whole share
         // before it waits for any of it
         load_x(b0, 0);
@@ -278,7 +314,8 @@ bool gptq_tile_ok(const Wna16Problem &p) {
 template <typename TT, int BITS, int MT, int PER, int D>
 static int gptq_tile_go(hipStream_t s, dim3 grid, const Wna16Problem &p) {
     constexpr bool FOLD = MT <= 2;
-    const size_t lds = (size_t)8 * MT * 4096;  // 8 partial tiles of 16 MT x 64 f32 (the x slots are as large)
+    // 8 partial tiles of 16 MT x 64 f32; the x stages are as large, or 2 PER stages of 2 KB a wave when x goes first
+    const size_t lds = MT == 1 && PER > 2 ? (size_t)8 * 2 * PER * 2048 : (size_t)8 * MT * 4096;
     static LdsGrant lds_grant;
     OXQ_HIP_CHECK(lds_grant.ensure((const void *)gptq_tile_kernel<TT, BITS, MT, PER, D, FOLD>, lds));
     hipLaunchKernelGGL((gptq_tile_kernel<TT, BITS, MT, PER, D, FOLD>), grid, dim3(512), lds, s, (const uint16_t *)p.x, p.qweight,
