@@ -85,7 +85,9 @@ __global__ __launch_bounds__(512) void gptq_tile_kernel(const uint16_t *__restri
     const __amdgpu_buffer_rsrc_t rs_w = make_rsrc(qw, (uint32_t)(K / PF) * (uint32_t)wrow);
     const __amdgpu_buffer_rsrc_t rs_z = make_rsrc(qz, (uint32_t)(K >> gshift) * (uint32_t)(N / PF) * 4u);
     const __amdgpu_buffer_rsrc_t rs_s = make_rsrc(sc, (uint32_t)(K >> gshift) * (uint32_t)N * 2u);
-    const __amdgpu_buffer_rsrc_t rs_x = make_rsrc(x + (size_t)m0 * K, (uint32_t)(M - m0) * (uint32_t)K * 2u);
+    // this workgroup's rows only: the descriptor's 32-bit size holds them whatever M is
+    const int rows = M - m0 < 16 * MT ? M - m0 : 16 * MT;
+    const __amdgpu_buffer_rsrc_t rs_x = make_rsrc(x + (size_t)m0 * K, (uint32_t)rows * (uint32_t)K * 2u);
     const uint32_t voff_w = (uint32_t)(kb * WL) * (uint32_t)wrow + (uint32_t)(64 * j + 4 * ni) * 4u;
     const uint32_t voff_s = (uint32_t)(64 * j + 4 * ni) * 2u;
     // the zero points of the lane's four columns lie in one word

@@ -81,3 +81,30 @@ def test_gptq_tile_rows_do_not_depend_on_the_batch(bits):
     y100 = bits_of(_run(ops, xd, d, bits, 100))
     y40 = bits_of(_run(ops, xd[:40].contiguous(), d, bits, 40))
     np.testing.assert_array_equal(y40, y100[:40])
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_gptq_tile_many_row_tiles_and_bias(bits):
+    """300 rows are five row-tile workgroups a strip, the last one ragged; the bias is added once, after the
+    waves' sum."""
+    from oxydllm_amd import ops
+    dt = oracle.BF16
+    K, N, g, m = 1024, 128, 128, 300
+    qw, qz, sc = synth.gptq_checkpoint(K, N, g, bits, seed=5 + bits)
+    bias = ((np.arange(N, dtype=np.float32) % 11) - 5) * np.float32(0.125)
+    layer = ops.PackedQuantLinear(bits, ops.PACK_IN, to_dev(qw), to_dev(qz), to_dev(sc, torch.bfloat16),
+                                  to_dev(bias, torch.bfloat16), torch.bfloat16)
+    tune("OXQ_PREPACK", 0)  # a layer that keeps the checkpoint layout forwards through the stateless ops
+    plain = ops.PackedQuantLinear(bits, ops.PACK_IN, to_dev(qw), to_dev(qz), to_dev(sc, torch.bfloat16),
+                                  to_dev(bias, torch.bfloat16), torch.bfloat16)
+    x = np.random.default_rng(17).standard_normal((m, K)).astype(np.float32)
+    xd = to_dev(x, torch.bfloat16)
+    say(f"gptq tile bits={bits} m={m} with bias, through a layer on the checkpoint layout")
+    y = plain.forward(xd)
+    plan = ops.default_context().last_plan()
+    assert plan["kernel"] == f"gptq{bits}_tile_bf16_mt4" and plan["grid"] == (N // 64, 5, 1), plan
+    w = oracle.round_through(oracle.dequantize_gptq(qw, qz, oracle.round_through(sc, dt), bits), dt)
+    assert_close(y, oracle.matmul_nt_f32(round_x(x, dt), w, oracle.round_through(bias, dt)), f"gptq{bits} tile m{m} bias")
+    # the resident layer's tile form is the same arithmetic in the same order of K blocks per wave only when the
+    # waves' shares agree; its result stays within the tolerance of this one
+    assert_close(y, layer.forward(xd).float().cpu().numpy(), f"gptq{bits} tile vs resident m{m}")
