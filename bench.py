@@ -39,7 +39,7 @@ HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 MFMA_F16_PEAK_TFLOPS = 2500.0
 K, N, G = 4096, 14336, 128
 SAMPLES = 11                # timed replays per case; the median is reported
-MIN_TIMED_STEPS = 200       # launches inside one event pair (short graphs are replayed back to back)
+MIN_TIMED_STEPS = 200       # launches inside one event pair (short runs are timed as one longer graph)
 SPINUP_MS = 30.0            # untimed replays ahead of the samples of every case
 
 
@@ -75,6 +75,18 @@ def time_graph(fn_of_step, steps: int, warmup: int, stream):
         torch.cuda.synchronize()
     cur = torch.cuda.current_stream()
     reps = max(1, -(-MIN_TIMED_STEPS // steps))
+    # Short graphs: the event pair times one graph of reps * steps launches (the same calls, the step index
+    # running on), so that the gap between two graph launches (several microseconds: 0.2 - 0.4 us a step at 20
+    # steps) is not booked as kernel time.  The host-clock figure stays one replay of `steps` launches.
+    timed = graph
+    if reps > 1:
+        timed = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(timed, stream=stream):
+            for i in range(reps * steps):
+                fn_of_step(i)
+        torch.cuda.synchronize()
+        timed.replay()
+        torch.cuda.synchronize()
     walls, evs = [], []
     for _ in range(SAMPLES):   # median of SAMPLES replays of the same `steps` launches
         ev0 = torch.cuda.Event(enable_timing=True)
@@ -86,17 +98,16 @@ def time_graph(fn_of_step, steps: int, warmup: int, stream):
         graph.replay()
         torch.cuda.synchronize()
         walls.append((time.perf_counter() - t0) * 1e3)
-        # (b) HIP events on the launch stream, with untimed replays directly ahead: the timed replays
-        # are enqueued while the GPU is still busy, so the first kernel starts when the event before it
+        # (b) HIP events on the launch stream, with untimed replays directly ahead: the timed replay
+        # is enqueued while the GPU is still busy, so the first kernel starts when the event before it
         # completes and the launch latency is not counted as kernel time.  The event pair itself costs a
-        # few microseconds, which a 20-step replay would carry as +0.4 us per step: short graphs are
-        # replayed `reps` times back to back inside one pair (at least MIN_TIMED_STEPS launches) and the
-        # pair's time is divided by `reps`, i.e. each sample is the mean time of `steps` launches.
+        # few microseconds, which 20 steps would carry as +0.4 us per step: the pair spans at least
+        # MIN_TIMED_STEPS launches (`reps` times `steps`) and its time is divided by `reps`, i.e. each sample
+        # is the mean time of `steps` launches.
         graph.replay()
         graph.replay()
         ev0.record(cur)
-        for _ in range(reps):
-            graph.replay()
+        timed.replay()
         ev1.record(cur)
         torch.cuda.synchronize()
         evs.append(ev0.elapsed_time(ev1) / reps)
@@ -349,8 +360,8 @@ def main():
                                "(BASELINE configs[1]) through PackedQuantLinear.forward on a resident layer; "
                                "M=16/64 in `cases`; the stateless checkpoint-layout ops in "
                                "`cases_checkpoint_layout_ops`",
-                   "weight_copies_rotated": copies, "timing": f"HIP graph of `steps` launches; {SAMPLES} samples, each one HIP-event pair around "
-                             f"max(1, ceil({MIN_TIMED_STEPS}/steps)) back-to-back replays divided by that count; median"},
+                   "weight_copies_rotated": copies, "timing": f"HIP graph of max(1, ceil({MIN_TIMED_STEPS}/steps)) x `steps` launches; {SAMPLES} samples, each one "
+                             f"HIP-event pair around one replay, divided by that factor; median"},
         "roofline": {"bound": "hbm", "achieved": c1["GB_per_s"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(c1["GB_per_s"] / HBM_PEAK_GBS, 4), "traffic": traffic,
                      "kernel": c1["kernel"], "algorithmic_bytes_per_launch": c1["algorithmic_bytes"],
