@@ -294,6 +294,12 @@ def main():
         _, ev = time_graph(lambda i: ops.empty_launch(m1["grid"][0], 1024 if "front" in m1["kernel"] else 512, 65536, ctx=ctx),
                            args.steps, args.warmup, stream)
         bare["empty_launch_us"] = round(ev * 1e3 / args.steps, 3)
+        # the same launch shape with one grid barrier in it (bounded spin): what a persistent kernel would pay per
+        # layer boundary instead of a launch
+        bar_state = torch.zeros(2, dtype=torch.int32, device=dev)
+        _, ev = time_graph(lambda i: ops.grid_barrier(m1["grid"][0], 1024 if "front" in m1["kernel"] else 512, bar_state,
+                                                      ctx=ctx), args.steps, args.warmup, stream)
+        bare["grid_barrier_launch_us"] = round(ev * 1e3 / args.steps, 3) if int(bar_state[1].item()) == 0 else None
         for nt in (0, 1):
             def rd(i, nt=nt):
                 c = i % copies

@@ -40,6 +40,15 @@ int oxq_bench_two_streams(oxq_ctx *ctx, void *stream, const oxq_tensor *w, const
  * dynamic LDS, up to 160 KiB): what one launch costs when it does nothing. */
 int oxq_bench_empty_launch(oxq_ctx *ctx, void *stream, int workgroups, int threads, int lds_bytes);
 
+/* A launch that does nothing but one grid barrier: thread 0 of every workgroup takes a ticket from the
+ * device-scope counter state[0] and polls it until its round is complete; after spin_limit polls
+ * (1 .. 4194304) it gives up, sets state[1] to 1 and leaves, so every wave exits.  `state`: two zeroed
+ * 32-bit words on the device, never reset between launches.  workgroups must all be resident at once (at
+ * most one per compute unit at more than 512 threads, two below).  Against oxq_bench_empty_launch: what a
+ * persistent kernel would pay to make one layer's outputs visible to the next inside one launch. */
+int oxq_bench_grid_barrier(oxq_ctx *ctx, void *stream, int workgroups, int threads, const oxq_tensor *state,
+                           uint32_t spin_limit);
+
 #ifdef __cplusplus
 }
 #endif

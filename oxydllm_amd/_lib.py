@@ -86,6 +86,7 @@ SIGNATURES = {
     "oxq_calib_read": (C.c_int, [_VP, _VP, _TP, C.c_int, C.c_int, _TP]),
     "oxq_bench_read_upfront": (C.c_int, [_VP, _VP, _TP, C.c_int, C.c_int, C.c_int, _TP]),
     "oxq_bench_empty_launch": (C.c_int, [_VP, _VP, C.c_int, C.c_int, C.c_int]),
+    "oxq_bench_grid_barrier": (C.c_int, [_VP, _VP, C.c_int, C.c_int, _TP, C.c_uint32]),
     "oxq_bench_two_streams": (C.c_int, [_VP, _VP, _TP, _TP, C.c_int, C.c_int, _TP]),
     "oxq_w4a16_matmul": (C.c_int, [_VP, _VP, _TP, _TP, _TP, _TP, _TP]),
     "oxq_w4a16_matmul_static": (C.c_int, [_VP, _VP, _TP, _TP, _TP, _TP, _TP]),

@@ -86,6 +86,42 @@ int launch_empty(oxq_ctx *ctx, hipStream_t s, int workgroups, int threads, int l
     return OXQ_OK;
 }
 
+// A launch whose workgroups meet at one grid barrier: thread 0 of every workgroup takes a ticket from a
+// device-scope counter and waits until the counter has reached the end of its ticket's round (the counter
+// is never reset: round r ends at (r + 1) * workgroups, so replays need no clearing).  The wait is bounded:
+// after `spin_limit` polls a workgroup gives up, raises the error word and leaves, so every wave exits
+// whatever happens.  The caller must launch no more workgroups than are resident at once.
+template <int NW>
+__global__ __launch_bounds__(NW * 64) void grid_barrier_kernel(unsigned *counter, unsigned *err, unsigned workgroups,
+                                                               unsigned spin_limit) {
+    if (threadIdx.x == 0) {
+        const unsigned t = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const unsigned target = (t / workgroups + 1u) * workgroups;
+        unsigned polls = 0;
+        while ((int)(__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - target) < 0) {
+            if (++polls > spin_limit) {
+                __hip_atomic_store(err, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                break;
+            }
+            __builtin_amdgcn_s_sleep(1);
+        }
+    }
+    __syncthreads();
+}
+
+int launch_grid_barrier(oxq_ctx *ctx, hipStream_t s, int workgroups, int threads, unsigned *counter, unsigned *err,
+                        unsigned spin_limit) {
+    dim3 grid((unsigned)workgroups), block((unsigned)threads);
+    set_plan(ctx, "grid_barrier", grid, block, 1, 1, 0);
+    if (ctx->plan_only) return OXQ_OK;
+    if (threads <= 512)
+        hipLaunchKernelGGL(grid_barrier_kernel<8>, grid, block, 0, s, counter, err, (unsigned)workgroups, spin_limit);
+    else
+        hipLaunchKernelGGL(grid_barrier_kernel<16>, grid, block, 0, s, counter, err, (unsigned)workgroups, spin_limit);
+    OXQ_HIP_CHECK(hipGetLastError());
+    return OXQ_OK;
+}
+
 int launch_calib_upfront(oxq_ctx *ctx, hipStream_t s, const uint8_t *src, uint64_t bytes, int workgroups, int waves,
                          int nontemporal, uint32_t *out) {
     const uint64_t span = bytes / (uint64_t)workgroups;

@@ -677,6 +677,25 @@ int oxq_bench_empty_launch(oxq_ctx *ctx, void *stream, int workgroups, int threa
     return launch_empty(ctx, (hipStream_t)stream, workgroups, threads, lds_bytes);
 }
 
+int oxq_bench_grid_barrier(oxq_ctx *ctx, void *stream, int workgroups, int threads, const oxq_tensor *state,
+                           uint32_t spin_limit) {
+    if (!ctx || !state) return fail(OXQ_ERR_ARG, "GridBarrier: NULL argument");
+    if (workgroups < 1 || threads < 64 || threads > 1024 || threads % 64 != 0)
+        return fail(OXQ_ERR_ARG, "GridBarrier: %d workgroups of %d threads", workgroups, threads);
+    // every workgroup must be resident at once, or the ones that are would wait for ones that cannot start
+    const int resident = (ctx->num_cus > 0 ? ctx->num_cus : 256) * (threads <= 512 ? 2 : 1);
+    if (workgroups > resident)
+        return fail(OXQ_ERR_ARG, "GridBarrier: %d workgroups of %d threads are not resident at once on %d compute units",
+                    workgroups, threads, ctx->num_cus);
+    if ((state->dtype != OXQ_I32 && state->dtype != OXQ_U32) || state->rank != 1 || state->dims[0] < 2 || !state->contiguous)
+        return fail(OXQ_ERR_SHAPE, "GridBarrier: state must be two contiguous 32-bit words {counter, error}");
+    if (!ctx->plan_only && (state->device == OXQ_DEVICE_HOST || !state->data))
+        return fail(OXQ_ERR_DEVICE, "GridBarrier: state must be a device tensor");
+    if (spin_limit == 0 || spin_limit > (1u << 22)) return fail(OXQ_ERR_ARG, "GridBarrier: spin limit %u", spin_limit);
+    return launch_grid_barrier(ctx, (hipStream_t)stream, workgroups, threads, (unsigned *)state->data,
+                               (unsigned *)state->data + 1, spin_limit);
+}
+
 // ---- opt-in cache of tile-major weight copies behind the stateless ops ---------------------------
 // The reference's ops are called with the same resident tensors on every forward (linear.rs:482-533
 // passes the layer's own qweight / qzeros / scales).  A caller that swaps in only the op functions,

@@ -277,6 +277,8 @@ int launch_calib_read(oxq_ctx *ctx, hipStream_t s, const uint8_t *src, uint64_t 
 int launch_calib_upfront(oxq_ctx *ctx, hipStream_t s, const uint8_t *src, uint64_t bytes, int workgroups, int waves,
                          int nontemporal, uint32_t *out);
 int launch_empty(oxq_ctx *ctx, hipStream_t s, int workgroups, int threads, int lds_bytes);
+int launch_grid_barrier(oxq_ctx *ctx, hipStream_t s, int workgroups, int threads, unsigned *counter, unsigned *err,
+                        unsigned spin_limit);
 int launch_calib_two_streams(oxq_ctx *ctx, hipStream_t s, const uint8_t *w, uint64_t w_bytes, const uint8_t *x,
                              uint64_t x_bytes, int workgroups, int which, uint32_t *out);
 // y[M,N] = sum over S slices of ws[s][M][N] (+ bias), slices added in index order.

@@ -167,6 +167,14 @@ def empty_launch(workgroups: int, threads: int, lds_bytes: int = 0, *, ctx: Opti
     _lib.check(ctx._lib.oxq_bench_empty_launch(ctx.handle, ctx.stream(), int(workgroups), int(threads), int(lds_bytes)))
 
 
+def grid_barrier(workgroups: int, threads: int, state, spin_limit: int = 1 << 18, *, ctx: Optional[Context] = None):
+    """A launch that is one bounded grid barrier (include/oxq_bench.h); state: two zeroed int32 words
+    {counter, error}, the error word is 1 afterwards if a workgroup gave up."""
+    ctx = _ctx(ctx)
+    _lib.check(ctx._lib.oxq_bench_grid_barrier(ctx.handle, ctx.stream(), int(workgroups), int(threads), desc(state),
+                                               int(spin_limit)))
+
+
 def w4a16_matmul(x, qweight, qzeros, scales, *, out=None, ctx: Optional[Context] = None):
     """metal_ops.rs:1821.  x [m,K] (m in 1..=8) -> [m,N] in x's dtype."""
     ctx = _ctx(ctx)
