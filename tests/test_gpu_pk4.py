@@ -254,6 +254,13 @@ def test_two_to_four_row_tiles_in_straight_line_code(kind, dtn, K, N, g, ks, mon
         y0 = layer.forward(xd)
         tune("OXQ_PK4_FRONT", None)
         assert_close(y0, ref, f"pk4 four tiles, loop {kind} {dtn} m{m}")
+        if m > 48 and bits == 4 and ks == 1 and K in (4096, 5120):
+            # the 49 - 64-row kernel (x straight into LDS, weights up front) shares the ring kernel's arithmetic, K
+            # split and summation order: the same bits
+            tune("OXQ_PK4_T64", 0)
+            y1 = layer.forward(xd)
+            tune("OXQ_PK4_T64", None)
+            np.testing.assert_array_equal(bits_of(y1), bits_of(y))
 
 
 @pytest.mark.parametrize("kind", KINDS)
