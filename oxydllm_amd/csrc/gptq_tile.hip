@@ -18,8 +18,9 @@
 // form, which never rounds a dequantized weight; above it B = T((q - (z + 1)) * s), bit-identical to the
 // dense dequant (f16: exact packed add, one rounding in the packed multiply; bf16: exact f32 fma, one
 // conversion), as the reference's staged GEMM rounds B.  f32 accumulation, the 8 waves' partial tiles
-// added in wave order.  One workgroup a 64-column strip and 16 MT rows, the
-// waves split K in contiguous runs of 128-row blocks: one launch, no workspace, deterministic.
+// added in wave order.  One workgroup a 64-column strip and 16 MT rows, the waves split K in contiguous
+// runs of 128-row blocks: one launch, no workspace, deterministic.  Layers of few strips are also cut into
+// K slices (grid.z), whose f32 partial tiles a second launch adds in slice order.
 
 #include "pk4_common.hpp"
 
@@ -56,7 +57,7 @@ __global__ __launch_bounds__(512) void gptq_tile_kernel(const uint16_t *__restri
                                                         const uint32_t *__restrict__ qz,
                                                         const uint16_t *__restrict__ sc,
                                                         const uint16_t *__restrict__ bias, uint16_t *__restrict__ y,
-                                                        int M, int K, int N, int gshift) {
+                                                        float *__restrict__ ws, int M, int K, int N, int gshift) {
     typedef MfmaOps<TT> Ops;
     constexpr int PF = 32 / BITS;     // rows of K a word
     constexpr int WL = BITS / 4;      // 16-byte loads a lane and MFMA step
@@ -75,10 +76,14 @@ __global__ __launch_bounds__(512) void gptq_tile_kernel(const uint16_t *__restri
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int ni = lane & 15, kb = lane >> 4;
     const int j = blockIdx.x, m0 = blockIdx.y * 16 * MT;
-    const int NB = K >> 7;
-    const int per = PER ? PER : (NB + 7) >> 3;  // PER: K / 128 = 8 PER (launcher)
-    const int b0 = wave * per;
-    const int b1 = b0 + per < NB ? b0 + per : NB;
+    // K slices (grid.z; narrow layers): slice z owns blocks [z * NBS, (z + 1) * NBS) and writes an f32 partial tile
+    const int NBT = K >> 7;
+    const int NBS = (NBT + (int)gridDim.z - 1) / (int)gridDim.z;
+    const int s0 = blockIdx.z * NBS;
+    const int NB = s0 + NBS < NBT ? NBS : NBT - s0;   // blocks of this slice
+    const int per = PER ? PER : (NB + 7) >> 3;  // PER: K / 128 = 8 PER, one slice (launcher)
+    const int b0 = s0 + wave * per;
+    const int b1 = b0 + per < s0 + NB ? b0 + per : s0 + NB;
     unsigned char *slot = pk4_lds + wave * NSTAGE * STAGE;
 
     const int wrow = N * 4;  // bytes a word row
@@ -299,7 +304,8 @@ __global__ __launch_bounds__(512) void gptq_tile_kernel(const uint16_t *__restri
         }
     }
     __syncthreads();  // the partial tiles go where other waves' x stages were
-    pk4_epilogue_lanes<TT, MT>(acc, bias, y, M, N, j, m0, wave, lane);
+    pk4_epilogue_lanes<TT, MT>(acc, bias, y, M, N, j, m0, wave, lane,
+                               gridDim.z > 1 ? ws + (size_t)blockIdx.z * M * N : nullptr);
 }
 
 // 128-row blocks inside one quantization group, 64-column strips, 32-bit buffer offsets, 16-byte rows
@@ -314,14 +320,14 @@ bool gptq_tile_ok(const Wna16Problem &p) {
 }
 
 template <typename TT, int BITS, int MT, int PER, int D>
-static int gptq_tile_go(hipStream_t s, dim3 grid, const Wna16Problem &p) {
+static int gptq_tile_go(hipStream_t s, dim3 grid, const Wna16Problem &p, float *ws) {
     constexpr bool FOLD = MT <= 2;
     // 8 partial tiles of 16 MT x 64 f32; the x stages are as large, or 2 PER stages of 2 KB a wave when x goes first
     const size_t lds = MT == 1 && PER > 2 ? (size_t)8 * 2 * PER * 2048 : (size_t)8 * MT * 4096;
     static LdsGrant lds_grant;
     OXQ_HIP_CHECK(lds_grant.ensure((const void *)gptq_tile_kernel<TT, BITS, MT, PER, D, FOLD>, lds));
     hipLaunchKernelGGL((gptq_tile_kernel<TT, BITS, MT, PER, D, FOLD>), grid, dim3(512), lds, s, (const uint16_t *)p.x, p.qweight,
-                       p.qzeros, (const uint16_t *)p.scales, (const uint16_t *)p.bias, (uint16_t *)p.y, (int)p.M,
+                       p.qzeros, (const uint16_t *)p.scales, (const uint16_t *)p.bias, (uint16_t *)p.y, ws, (int)p.M,
                        (int)p.K, (int)p.N, p.group_shift);
     OXQ_HIP_CHECK(hipGetLastError());
     return OXQ_OK;
@@ -330,35 +336,59 @@ static int gptq_tile_go(hipStream_t s, dim3 grid, const Wna16Problem &p) {
 // Weight ring: as deep as the registers beside the accumulators and the x half block allow.  K = 4096 and
 // 5120 (4 or 5 blocks a wave) run as straight-line code.
 template <typename TT, int BITS, int MT>
-static int gptq_tile_per(hipStream_t s, dim3 grid, int per, const Wna16Problem &p) {
+static int gptq_tile_per(hipStream_t s, dim3 grid, int per, const Wna16Problem &p, float *ws) {
     constexpr bool f16 = TT::DTYPE == 1;
     constexpr int DMAX = BITS == 4 ? (MT == 1 ? 5 : MT == 2 ? 4 : 2) : (MT == 1 ? (f16 ? 4 : 3) : MT == 2 ? 3 : 2);
-    if (per == 4) return gptq_tile_go<TT, BITS, MT, 4, (DMAX < 4 ? DMAX : 4)>(s, grid, p);
-    if (per == 5) return gptq_tile_go<TT, BITS, MT, 5, (DMAX < 5 ? DMAX : 5)>(s, grid, p);
-    return gptq_tile_go<TT, BITS, MT, 0, 2>(s, grid, p);
+    if (per == 4) return gptq_tile_go<TT, BITS, MT, 4, (DMAX < 4 ? DMAX : 4)>(s, grid, p, ws);
+    if (per == 5) return gptq_tile_go<TT, BITS, MT, 5, (DMAX < 5 ? DMAX : 5)>(s, grid, p, ws);
+    return gptq_tile_go<TT, BITS, MT, 0, 2>(s, grid, p, ws);
 }
 
 template <typename TT, int BITS>
-static int gptq_tile_mt(hipStream_t s, dim3 grid, int mt, const Wna16Problem &p) {
+static int gptq_tile_mt(hipStream_t s, dim3 grid, int mt, const Wna16Problem &p, float *ws) {
     const int64_t NB = p.K / 128;
-    const int per = NB % 8 == 0 ? (int)(NB / 8) : 0;
+    const int per = grid.z == 1 && NB % 8 == 0 ? (int)(NB / 8) : 0;  // straight-line code: one slice of 32 or 40 blocks
     switch (mt) {
-    case 1: return gptq_tile_per<TT, BITS, 1>(s, grid, per, p);
-    case 2: return gptq_tile_per<TT, BITS, 2>(s, grid, per, p);
-    default: return gptq_tile_per<TT, BITS, 4>(s, grid, per, p);
+    case 1: return gptq_tile_per<TT, BITS, 1>(s, grid, per, p, ws);
+    case 2: return gptq_tile_per<TT, BITS, 2>(s, grid, per, p, ws);
+    default: return gptq_tile_per<TT, BITS, 4>(s, grid, per, p, ws);
     }
+}
+
+// K slices for a layer of few strips: as many as bring the launch to about one workgroup a CU, at least
+// 8 blocks (one a wave) each; their f32 partial tiles are added in slice order by a second launch.
+int gptq_tile_slices(const oxq_ctx *ctx, const Wna16Problem &p) {
+    const int mt = p.M > 32 ? 4 : (int)((p.M + 15) / 16);
+    const int64_t tiles = (p.N / 64) * ceil_div(p.M, 16 * mt), NB = p.K / 128;
+    int ks = 1;
+    if (tiles <= 96 && NB >= 32) ks = (int)std::max<int64_t>(1, std::min<int64_t>(256 / tiles, NB / 8));
+    else if (tiles <= 128 && NB >= 64) ks = 2;  // half a round of workgroups and a long K
+    ks = tune(ctx, OXQ_TUNE_GPTQ_TILE_KS, ks);
+    return (int)std::max<int64_t>(1, std::min<int64_t>(ks, NB));
 }
 
 int launch_gptq_tile(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p) {
     const int mt = p.M > 32 ? 4 : (int)((p.M + 15) / 16);  // three row tiles run as four (their sum divides over 8 waves)
-    dim3 grid((unsigned)(p.N / 64), (unsigned)ceil_div(p.M, 16 * mt));
+    const int ks = gptq_tile_slices(ctx, p);
+    dim3 grid((unsigned)(p.N / 64), (unsigned)ceil_div(p.M, 16 * mt), (unsigned)ks);
+    const size_t ws_bytes = ks > 1 ? (size_t)ks * p.M * p.N * 4 : 0;
     char name[64];
     snprintf(name, sizeof name, "gptq%d_tile_%s_mt%d", p.bits, p.dtype == OXQ_F16 ? "f16" : "bf16", mt);
-    set_plan(ctx, name, grid, dim3(512), 1, 1, 0);
-    if (ctx->plan_only) return OXQ_OK;
+    set_plan(ctx, name, grid, dim3(512), ks, 1, ws_bytes);
+    if (ctx->plan_only) {
+        if (ks > 1) add_launch(ctx);
+        return OXQ_OK;
+    }
+    if (ws_bytes > ctx->workspace_bytes)
+        return fail(OXQ_ERR_WORKSPACE, "gptq tile: %d K slices need %zu workspace bytes, ctx holds %zu", ks, ws_bytes,
+                    ctx->workspace_bytes);
+    float *ws = (float *)ctx->workspace;
     const bool f16 = p.dtype == OXQ_F16;
-    if (p.bits == 4) return f16 ? gptq_tile_mt<F16Traits, 4>(s, grid, mt, p) : gptq_tile_mt<BF16Traits, 4>(s, grid, mt, p);
-    return f16 ? gptq_tile_mt<F16Traits, 8>(s, grid, mt, p) : gptq_tile_mt<BF16Traits, 8>(s, grid, mt, p);
+    int rc;
+    if (p.bits == 4) rc = f16 ? gptq_tile_mt<F16Traits, 4>(s, grid, mt, p, ws) : gptq_tile_mt<BF16Traits, 4>(s, grid, mt, p, ws);
+    else rc = f16 ? gptq_tile_mt<F16Traits, 8>(s, grid, mt, p, ws) : gptq_tile_mt<BF16Traits, 8>(s, grid, mt, p, ws);
+    if (rc != OXQ_OK || ks == 1) return rc;
+    return launch_splitk_reduce(ctx, s, ws, p.bias, p.y, p.M, p.N, ks, p.dtype);
 }
 
 }  // namespace oxq

@@ -174,10 +174,12 @@ __device__ __forceinline__ void pk4_epilogue(const float4_t (&acc)[MT][4], const
 // wave order (the same order and so the same bits as pk4_epilogue), every LDS access a lane-linear
 // 16-byte one (no bank conflicts; in pk4_epilogue's row-major read two rows of a 16-lane group share
 // their banks).  Lane (ni, kb) ends up with row 16 mt + 4 kb + e, columns 4 ni .. 4 ni + 3: 8 bytes of y.
+// ws != nullptr: this workgroup is one K slice of several; its f32 partial tile goes to ws[M][N] (the slice's
+// plane) and a second kernel adds the planes in slice order and applies the bias.
 template <typename TT, int MT, int NW = 8>
 __device__ __forceinline__ void pk4_epilogue_lanes(const float4_t (&acc)[MT][4], const uint16_t *__restrict__ bias,
                                                    uint16_t *__restrict__ y, int M, int N, int j, int m0, int wave,
-                                                   int lane) {
+                                                   int lane, float *__restrict__ ws = nullptr) {
     static_assert((4 * MT) % NW == 0 || NW % (4 * MT) == 0, "planes divide over the waves");
     extern __shared__ __attribute__((aligned(16))) unsigned char pk4_lds[];
     float4_t *red = (float4_t *)pk4_lds;  // [NW][MT][4 e][64 lanes]
@@ -204,7 +206,9 @@ __device__ __forceinline__ void pk4_epilogue_lanes(const float4_t (&acc)[MT][4],
 #pragma unroll
         for (int s = 0; s < NW; ++s) v += red[((s * MT + mt) * 4 + e) * 64 + lane];
         const int row = m0 + 16 * mt + 4 * kb + e;
-        if (row < M) {
+        if (row < M && ws) {
+            *(float4_t *)(ws + (size_t)row * N + 64 * j + 4 * ni) = v;
+        } else if (row < M) {
             if (bias) v += bv;
             const uint2 o = uint2{(uint32_t)TT::from_f32(v[0]) | ((uint32_t)TT::from_f32(v[1]) << 16),
                                   (uint32_t)TT::from_f32(v[2]) | ((uint32_t)TT::from_f32(v[3]) << 16)};

@@ -926,15 +926,16 @@ int launch_wna16_gemv(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p) {
     // rounding is 2^-9, keeps the kernel that never rounds the weight.
     if (p.M >= 2 && f16 && awq4_mfma_ok(p) && tune(ctx, OXQ_TUNE_GEMV_TILE, 1) && !tune(ctx, OXQ_TUNE_FORCE_GENERIC, 0))
         return launch_wna16_mfma(ctx, s, p);
-    // GPTQ words feed the matrix cores as they are stored (gptq_tile.hip): one launch over 64-column
-    // strips, K inside the workgroup, the same time for 1 - 16 rows where the dot-product kernel's
-    // arithmetic grows with the rows.  Like that kernel it never rounds a dequantized weight at these row
-    // counts.  Below 96 strips most CUs have no workgroup: there the sliced kernel keeps one to three rows,
-    // and every row count up to 8 when K is long.
+    // GPTQ words feed the matrix cores as they are stored (gptq_tile.hip): 64-column strips, K inside the
+    // workgroup (layers of few strips: K slices and the slice-ordered sum), the same time for 1 - 16 rows where
+    // the dot-product kernel's arithmetic grows with the rows.  Like that kernel it never rounds a dequantized
+    // weight at these row counts.  A single row of a layer of few strips stays with the dot-product kernel
+    // (4096 x 4096: 7.1 against 7.3 us; 8-bit also two rows: 8.4 against 9.0); from there on the tile kernel
+    // is ahead (14336 x 4096 at 2 / 8 rows: 10.5 / 10.7 against 11.2 / 21.0 us).
     if (gptq_tile_ok(p) && !tune(ctx, OXQ_TUNE_FORCE_GENERIC, 0)) {
         const int v = tune(ctx, OXQ_TUNE_GPTQ_TILE, 1);
         const bool wide = p.N >= 96 * 64;
-        if (v == 2 || (v == 1 && (wide || (p.M >= 4 && p.K <= 8192)))) return launch_gptq_tile(ctx, s, p);
+        if (v == 2 || (v == 1 && (wide || p.M >= (p.bits == 4 ? 2 : 4)))) return launch_gptq_tile(ctx, s, p);
     }
     if (gptq_fast_ok(p) && !tune(ctx, OXQ_TUNE_FORCE_GENERIC, 0)) {
         if (p.bits == 4)

@@ -5,8 +5,9 @@ Against the oracle's dense dequant (awq.rs:442-590) and f32 matmul: with the unr
 (the reach of the reference's fused GEMV, linear.rs:450-480), with the weight rounded to the activation type
 above (the reference's staged GEMM, mpp_gemm.metal:115-184).  Shapes cover every code path of the kernel:
 K = 4096 and 5120 (4 and 5 blocks a wave, straight-line code), other K through the block loop with one block a
-wave, uneven shares, waves without a block and an odd number of blocks a wave; one, two and four row tiles with
-ragged last tiles and several row-tile workgroups; groups larger than a block; bias; both bit widths and types.
+wave, uneven shares, waves without a block and an odd number of blocks a wave; K slices (few strips and 32 blocks
+or more) with and without them forced off; one, two and four row tiles with ragged last tiles and several row-tile
+workgroups; groups larger than a block; bias; both bit widths and types.
 """
 import sys
 
@@ -54,8 +55,11 @@ def test_gptq_tile_against_oracle(bits, dtn, K, N, g):
         plan = ops.default_context().last_plan()
         mt = 4 if m > 32 else (m + 15) // 16
         assert plan["kernel"] == f"gptq{bits}_tile_{dtn}_mt{mt}", plan
-        assert plan["launches"] == 1 and plan["split_k"] == 1, plan
-        assert plan["grid"] == (N // 64, -(-m // (16 * mt)), 1), plan
+        # these layers have few strips: from 32 blocks of K on they are cut into K slices, added by a second launch
+        tiles = (N // 64) * -(-m // (16 * mt))
+        ks = max(1, min(256 // tiles, K // 128 // 8)) if K // 128 >= 32 and tiles <= 96 else 1
+        assert plan["split_k"] == ks and plan["launches"] == (2 if ks > 1 else 1), plan
+        assert plan["grid"] == (N // 64, -(-m // (16 * mt)), ks), plan
         ref = oracle.matmul_nt_f32(round_x(x, dt), w_r if m > 32 else w)
         assert_close(y, ref, f"gptq{bits} tile {dtn} {K}x{N} g{g} m{m}")
         np.testing.assert_array_equal(bits_of(_run(ops, xd, d, bits, m)), bits_of(y))  # run to run
@@ -108,3 +112,34 @@ def test_gptq_tile_many_row_tiles_and_bias(bits):
     # the resident layer's tile form is the same arithmetic in the same order of K blocks per wave only when the
     # waves' shares agree; its result stays within the tolerance of this one
     assert_close(y, layer.forward(xd).float().cpu().numpy(), f"gptq{bits} tile vs resident m{m}")
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("dtn", ["f16", "bf16"])
+def test_gptq_tile_k_slices_and_straight_line_code_agree(bits, dtn):
+    """K = 4096 and 5120 on a layer of few strips: by default K slices (the block loop, partial tiles added by the
+    second launch); with one slice forced the straight-line kernels.  Both against the oracle, and the sliced sum
+    run to run bitwise."""
+    from oxydllm_amd import ops
+    dt = DT[dtn]
+    for K in (4096, 5120):
+        N, g = 128, 128
+        qw, qz, sc = synth.gptq_checkpoint(K, N, g, bits, seed=K + bits)
+        d = (to_dev(qw), to_dev(qz), to_dev(sc, TORCH_DT[dt]))
+        w = oracle.dequantize_gptq(qw, qz, oracle.round_through(sc, dt), bits)
+        rng = np.random.default_rng(K)
+        tune("OXQ_GPTQ_TILE", 2)
+        for m in (1, 8, 16, 32, 64):
+            x = rng.standard_normal((m, K)).astype(np.float32)
+            xd = to_dev(x, TORCH_DT[dt])
+            ref = oracle.matmul_nt_f32(round_x(x, dt), oracle.round_through(w, dt) if m > 32 else w)
+            for ks in (None, 1, 3):
+                say(f"gptq tile bits={bits} {dtn} K={K} m={m} slices={ks}")
+                tune("OXQ_GPTQ_TILE_KS", ks)
+                y = _run(ops, xd, d, bits, m)
+                plan = ops.default_context().last_plan()
+                want_ks = {None: min(256 // 2, K // 128 // 8), 1: 1, 3: 3}[ks]
+                assert plan["split_k"] == want_ks and plan["launches"] == (2 if want_ks > 1 else 1), plan
+                assert_close(y, ref, f"gptq{bits} tile {dtn} K{K} m{m} ks{ks}")
+                np.testing.assert_array_equal(bits_of(_run(ops, xd, d, bits, m)), bits_of(y))
+            tune("OXQ_GPTQ_TILE_KS", None)
