@@ -58,7 +58,19 @@ def build(force: bool = False, jobs: int = 6) -> str:
         res = subprocess.run(cmd, capture_output=True, text=True)
         if res.returncode != 0:
             raise RuntimeError(f"link failed:\n{res.stderr}")
+    _check_no_missing_kernels(LIB)
     return LIB
+
+
+def _check_no_missing_kernels(lib: str) -> None:
+    """A shared library links with undefined symbols.  One of the library's own (a kernel whose host stub the
+    compiler did not emit) would only show at load time on the GPU box: refuse it here."""
+    res = subprocess.run(["nm", "-D", "--undefined-only", lib], capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"nm failed on {lib}:\n{res.stderr}")
+    own = [l.split()[-1] for l in res.stdout.splitlines() if "_ZN3oxq" in l or " oxq_" in l]
+    if own:
+        raise RuntimeError(f"{lib} has undefined symbols of its own (first of {len(own)}): {own[0]}")
 
 
 if __name__ == "__main__":
