@@ -1,0 +1,594 @@
+// Resident GGUF layers for 16-bit activations: a copy of the blocks laid out for the matrix cores, and the
+// matmul that reads it at any number of rows (linear.rs:197-284 GgufFastPath: forward_decode up to 8 rows,
+// forward_prefill above; kernels quant_kernels.metal:792-870, 1097-1221 and the mul_mm strips).
+//
+// The rotated copy of gguf_res.hip gives a lane one unit of 32 elements and multiplies on the vector ALU: the
+// work grows with every row of x.  Here a strip of 16 output columns and a unit of 32 elements of K are one
+// v_mfma_f32_16x16x32_bf16 whose 16 rows are rows of x, so 1 to 16 rows cost the same instructions:
+//
+//   strip j (16 columns), chunk c (128 elements of K = 4 units), lane l = (ni = l % 16, kb = l / 16):
+//   word t of the lane's quants = elements 8 kb .. 8 kb + 7 of unit 4 c + t of column 16 j + ni, which is the B
+//   operand of the unit's MFMA once the integers are 16-bit floats; A = the same 8 elements of row ni of x.
+//
+//   Q4_0  chunk = [64 lanes][16 B] nibbles (element 2 pp in nibble pp, 2 pp + 1 in nibble pp + 4 of word t, so
+//                 that one AND-OR per pair yields 128 + q as two bf16) + [16 columns][4 units] f16 d    1152 B
+//   Q8_0  chunk = 2 x [64 lanes][16 B] (plane h = units 2 h, 2 h + 1; bytes of a word: elements 0, 2, 1, 3 of
+//                 its four, stored as q + 128) + [16 columns][4 units] f16 d                             2176 B
+//   Q4_K  block = 2 chunks of [64 lanes][16 B] nibbles as Q4_0 + [16 columns] the super-block's first 16
+//                 bytes (d, dmin, 12 scale bytes)                                                        2304 B
+//   Q6_K  block = 2 chunks of { [64 lanes][16 B] low nibbles, [64 lanes][8 B] high bit pairs, [16 columns][8]
+//                 int8 scales } + [16 columns] f16 d.  A scale covers 16 elements, so a step is a sub-block of 16
+//                 and v_mfma_f32_16x16x16_bf16: step s of the chunk takes elements 16 s + 4 kb .. + 3; their
+//                 nibbles sit in word s / 2 as Q4_0's pairs 2 (s % 2) and 2 (s % 2) + 1, their bit pairs in
+//                 word s / 4 of the second plane, field 2 (s % 4) + pair of each 16-bit half              3360 B
+//
+// Exactly the file's bytes per weight.  The integers stay integers: the MFMA accumulates x * (bias + q) in f32
+// (products of 8-bit significands are exact), a second MFMA against the constant -(bias + offset) takes the
+// bias and the format's offset out in the same accumulator, and the unit's scale multiplies the sum once per
+// output, in f32, as the reference's GEMV does (d * sum of q * x, quant_kernels.metal:1097-1221).
+//
+// A workgroup is one strip; its 16 (8) waves split the strip's chunks and stage their own rows of x through
+// LDS (no barrier before the epilogue); the partial tiles meet in LDS in wave order.
+#include "gguf_decode.hpp"
+#include "pk4_common.hpp"
+
+namespace oxq {
+
+template <int FMT> struct GgmFmt;
+// WQ: 16-byte quant planes a chunk; CH: chunks a block; UH: bytes of unit headers a chunk and column;
+// BH: bytes of block header a column; NEG: the constant that takes bias and offset out (as a bf16 pair)
+template <> struct GgmFmt<OXQ_GGUF_Q4_0> { static constexpr int WQ = 1, CH = 1, UH = 8, BH = 0; static constexpr uint32_t NEG = 0xC308C308u; };  // -136
+template <> struct GgmFmt<OXQ_GGUF_Q8_0> { static constexpr int WQ = 2, CH = 1, UH = 8, BH = 0; static constexpr uint32_t NEG = 0xC300C300u; };  // -128
+template <> struct GgmFmt<OXQ_GGUF_Q4_K> { static constexpr int WQ = 1, CH = 2, UH = 0, BH = 16; static constexpr uint32_t NEG = 0xC300C300u; };  // -128
+template <> struct GgmFmt<OXQ_GGUF_Q6_K> { static constexpr int WQ = 1, CH = 2, UH = 8, BH = 2; static constexpr uint32_t NEG = 0xC320C320u; };  // -160
+
+template <int FMT> struct GgmLayout {
+    typedef GgmFmt<FMT> F;
+    static constexpr int H_OFF = F::WQ * 1024;                                  // Q6_K: the plane of bit pairs
+    static constexpr int UH_OFF = F::WQ * 1024 + (FMT == OXQ_GGUF_Q6_K ? 512 : 0);
+    static constexpr int CHB = UH_OFF + 16 * F::UH;
+    static constexpr int BH_OFF = F::CH * CHB;
+    static constexpr int BLKB = F::CH * CHB + 16 * F::BH;
+    static_assert(BLKB == 16 * (128 * F::CH / GgufFmt<FMT>::BE) * GgufFmt<FMT>::BB, "the copy has the file's size");
+};
+
+// ---------------------------------------------------------------------------
+// repack: one thread per (strip, chunk, lane)
+// ---------------------------------------------------------------------------
+template <int FMT>
+__global__ __launch_bounds__(256) void ggm_repack_kernel(const uint8_t *__restrict__ w, uint8_t *__restrict__ pw, int K,
+                                                         int N) {
+    typedef GgmFmt<FMT> F;
+    typedef GgmLayout<FMT> L;
+    const int nch = K >> 7;
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (size_t)(N >> 4) * nch * 64) return;
+    const int lane = (int)(idx & 63), c = (int)((idx >> 6) % nch), strip = (int)((idx >> 6) / nch);
+    const int ni = lane & 15, kb = lane >> 4;
+    const size_t row_bytes = (size_t)(K / GgufFmt<FMT>::BE) * GgufFmt<FMT>::BB;
+    const uint8_t *row = w + (size_t)(16 * strip + ni) * row_bytes;
+    uint8_t *blk = pw + ((size_t)strip * (nch / F::CH) + c / F::CH) * L::BLKB;
+    uint8_t *chunk = blk + (c % F::CH) * L::CHB;
+    if constexpr (FMT == OXQ_GGUF_Q4_0) {
+        uint32_t q[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const uint8_t *p = row + (size_t)(4 * c + t) * 18;
+            uint32_t v = 0;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int e = 8 * kb + i;  // element e of the unit: low nibble of byte e (e < 16), high of byte e - 16
+                const uint32_t nib = e < 16 ? (p[2 + e] & 0xFu) : (p[2 + e - 16] >> 4);
+                v |= nib << (4 * (i >> 1) + 16 * (i & 1));
+            }
+            q[t] = v;
+            if (t == kb) *(uint16_t *)(chunk + L::UH_OFF + ni * 8 + t * 2) = ld16(p);
+        }
+        *(u32x4_t *)(chunk + lane * 16) = u32x4_t{q[0], q[1], q[2], q[3]};
+    } else if constexpr (FMT == OXQ_GGUF_Q8_0) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            uint32_t q[4];
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt) {
+                const int t = 2 * h + tt;
+                const uint8_t *p = row + (size_t)(4 * c + t) * 34;
+#pragma unroll
+                for (int d = 0; d < 2; ++d) {  // word d of the step: elements 4 d .. 4 d + 3 of the lane's 8
+                    const uint8_t *e = p + 2 + 8 * kb + 4 * d;
+                    q[2 * tt + d] = ((uint32_t)(e[0] ^ 0x80u)) | ((uint32_t)(e[2] ^ 0x80u) << 8) |
+                                    ((uint32_t)(e[1] ^ 0x80u) << 16) | ((uint32_t)(e[3] ^ 0x80u) << 24);
+                }
+                if (t == kb) *(uint16_t *)(chunk + L::UH_OFF + ni * 8 + t * 2) = ld16(p);
+            }
+            *(u32x4_t *)(chunk + h * 1024 + lane * 16) = u32x4_t{q[0], q[1], q[2], q[3]};
+        }
+    } else if constexpr (FMT == OXQ_GGUF_Q4_K) {
+        // quant_kernels.metal:2438-2482: sub-block sb of the super-block reads byte (sb / 2) * 32 + e of qs, low
+        // nibble if sb is even
+        const uint8_t *p = row + (size_t)(c >> 1) * 144;
+        uint32_t q[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const int sb = 4 * (c & 1) + t;
+            uint32_t v = 0;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const uint32_t byte = p[16 + (sb >> 1) * 32 + 8 * kb + i];
+                v |= ((sb & 1) ? (byte >> 4) : (byte & 0xFu)) << (4 * (i >> 1) + 16 * (i & 1));
+            }
+            q[t] = v;
+        }
+        *(u32x4_t *)(chunk + lane * 16) = u32x4_t{q[0], q[1], q[2], q[3]};
+        if ((c & 1) == 0 && kb < 4) *(uint32_t *)(blk + L::BH_OFF + ni * 16 + kb * 4) = ld32a2(p + 4 * kb);
+    } else if constexpr (FMT == OXQ_GGUF_Q6_K) {
+        // quant_kernels.metal:2518-2554: element j of the super-block, h = j / 128, q = (j % 128) / 32, l = j % 32:
+        // low nibble from ql[64 h + (q & 1) * 32 + l] (high nibble of the byte if q >= 2), bit pair 2 q of qh[32 h + l]
+        const uint8_t *p = row + (size_t)(c >> 1) * 210;
+        const int h = c & 1;
+        uint32_t lw[4] = {0u, 0u, 0u, 0u}, hw[2] = {0u, 0u};
+#pragma unroll
+        for (int s2 = 0; s2 < 8; ++s2)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int jj = 16 * s2 + 4 * kb + i;  // element of this half of the super-block
+                const int qq = jj >> 5, l = jj & 31;
+                const uint32_t lb = p[64 * h + (qq & 1) * 32 + l];
+                const uint32_t lo = qq < 2 ? (lb & 0xFu) : (lb >> 4);
+                const uint32_t hi = (p[128 + 32 * h + l] >> (2 * qq)) & 3u;
+                const int pair = i >> 1, half = i & 1;
+                lw[s2 >> 1] |= lo << (4 * (2 * (s2 & 1) + pair) + 16 * half);
+                hw[s2 >> 2] |= hi << (2 * (2 * (s2 & 3) + pair) + 16 * half);
+            }
+        *(u32x4_t *)(chunk + lane * 16) = u32x4_t{lw[0], lw[1], lw[2], lw[3]};
+        *(uint2 *)(chunk + L::H_OFF + lane * 8) = uint2{hw[0], hw[1]};
+        if (kb < 2) *(uint32_t *)(chunk + L::UH_OFF + ni * 8 + kb * 4) = ld32a2(p + 192 + 8 * h + 4 * kb);
+        if (h == 0 && kb == 0) *(uint16_t *)(blk + L::BH_OFF + ni * 2) = ld16(p + 208);
+    }
+}
+
+// dense [N, K] f32 from the copy, with the arithmetic of the file-layout dequant (pins the repack bit for bit)
+template <int FMT>
+__global__ __launch_bounds__(256) void ggm_dequant_kernel(const uint8_t *__restrict__ pw, float *__restrict__ out, int K,
+                                                          int N) {
+    typedef GgmFmt<FMT> F;
+    typedef GgmLayout<FMT> L;
+    const int nch = K >> 7;
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (size_t)(N >> 4) * nch * 64) return;
+    const int lane = (int)(idx & 63), c = (int)((idx >> 6) % nch), strip = (int)((idx >> 6) / nch);
+    const int ni = lane & 15, kb = lane >> 4;
+    const uint8_t *blk = pw + ((size_t)strip * (nch / F::CH) + c / F::CH) * L::BLKB;
+    const uint8_t *chunk = blk + (c % F::CH) * L::CHB;
+    float *o = out + (size_t)(16 * strip + ni) * K + (size_t)c * 128 + 8 * kb;
+    if constexpr (FMT == OXQ_GGUF_Q4_0) {
+        const u32x4_t q = *(const u32x4_t *)(chunk + lane * 16);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const float d = (float)__builtin_bit_cast(_Float16, *(const uint16_t *)(chunk + L::UH_OFF + ni * 8 + t * 2));
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                o[32 * t + i] = (float)((int)((q[t] >> (4 * (i >> 1) + 16 * (i & 1))) & 0xFu) - 8) * d;
+        }
+    } else if constexpr (FMT == OXQ_GGUF_Q8_0) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const u32x4_t q = *(const u32x4_t *)(chunk + h * 1024 + lane * 16);
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt) {
+                const int t = 2 * h + tt;
+                const float d = (float)__builtin_bit_cast(_Float16, *(const uint16_t *)(chunk + L::UH_OFF + ni * 8 + t * 2));
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const int byte = ((i & 3) >> 1) | ((i & 1) << 1);  // elements 0, 2, 1, 3 in bytes 0 .. 3
+                    o[32 * t + i] = (float)((int)((q[2 * tt + (i >> 2)] >> (8 * byte)) & 0xFFu) - 128) * d;
+                }
+            }
+        }
+    } else if constexpr (FMT == OXQ_GGUF_Q4_K) {
+        const u32x4_t q = *(const u32x4_t *)(chunk + lane * 16);
+        const uint8_t *hd = blk + L::BH_OFF + ni * 16;
+        const float d = (float)__builtin_bit_cast(_Float16, *(const uint16_t *)hd);
+        const float dmin = (float)__builtin_bit_cast(_Float16, *(const uint16_t *)(hd + 2));
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            uint32_t scv, mnv;
+            k4_scale_min(hd + 4, 4 * (c & 1) + t, scv, mnv);
+            const float d1 = d * (float)scv, m1 = dmin * (float)mnv;
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                o[32 * t + i] = d1 * (float)((q[t] >> (4 * (i >> 1) + 16 * (i & 1))) & 0xFu) - m1;
+        }
+    } else if constexpr (FMT == OXQ_GGUF_Q6_K) {
+        const u32x4_t lw = *(const u32x4_t *)(chunk + lane * 16);
+        const uint2 hw = *(const uint2 *)(chunk + L::H_OFF + lane * 8);
+        const float d = (float)__builtin_bit_cast(_Float16, *(const uint16_t *)(blk + L::BH_OFF + ni * 2));
+        float *o6 = out + (size_t)(16 * strip + ni) * K + (size_t)c * 128 + 4 * kb;
+#pragma unroll
+        for (int s2 = 0; s2 < 8; ++s2) {
+            const float ds = d * (float)(int)*(const int8_t *)(chunk + L::UH_OFF + ni * 8 + s2);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int pair = i >> 1, half = i & 1;
+                const uint32_t lo = (lw[s2 >> 1] >> (4 * (2 * (s2 & 1) + pair) + 16 * half)) & 0xFu;
+                const uint32_t hi = ((s2 < 4 ? hw.x : hw.y) >> (2 * (2 * (s2 & 3) + pair) + 16 * half)) & 3u;
+                o6[16 * s2 + i] = ds * (float)((int)(lo | (hi << 4)) - 32);
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// the matmul
+// ---------------------------------------------------------------------------
+// bytes 0 and 2 (1 and 3) of a word as a pair of bf16: through f32, exact for 0 .. 255
+__device__ __forceinline__ uint32_t ggm_bytes02(uint32_t w) {
+    const float lo = (float)(w & 0xFFu), hi = (float)((w >> 16) & 0xFFu);
+    return pack_hi16(__builtin_bit_cast(uint32_t, lo), __builtin_bit_cast(uint32_t, hi));
+}
+__device__ __forceinline__ uint32_t ggm_bytes13(uint32_t w) {
+    const float lo = (float)((w >> 8) & 0xFFu), hi = (float)(w >> 24);
+    return pack_hi16(__builtin_bit_cast(uint32_t, lo), __builtin_bit_cast(uint32_t, hi));
+}
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float ggm_f16(uint32_t bits) { return (float)__builtin_bit_cast(_Float16, (uint16_t)bits); }
+
+// The registers of one chunk: its quants and headers as requested, and what turns them into MFMA operands and
+// the factors of a step.  A step's sum t = sum over the step's elements of x * q', q' = q minus the format's
+// offset (exact integers); y += f0(step) * t + f1(step) * (sum of x) where the format has a minimum.
+template <int FMT> struct GgmChunk {
+    typedef GgmFmt<FMT> F;
+    typedef GgmLayout<FMT> L;
+    static constexpr int NSTEP = FMT == OXQ_GGUF_Q6_K ? 8 : 4;
+    static constexpr bool HAS_MIN = FMT == OXQ_GGUF_Q4_K;
+    u32x4_t q[F::WQ];
+    uint32_t qh[FMT == OXQ_GGUF_Q6_K ? 2 : 1];
+    uint32_t uh[F::UH ? 2 : 1];   // unit headers of the column: four f16 d (Q4_0, Q8_0), eight int8 scales (Q6_K)
+    uint32_t bh[F::BH == 16 ? 4 : 1];  // block header of the column
+
+    // c: the chunk's index in its strip
+    template <typename RS>
+    __device__ __forceinline__ void request(const RS &rs, int lane, int ni, int c) {
+        const int blk = (c / F::CH) * L::BLKB, soff = blk + (c % F::CH) * L::CHB;
+        // headers first: the factors and the minimum's term are worked out while the quants are on their way
+        if constexpr (F::UH == 8) {
+            const u32x2_t v = __builtin_amdgcn_raw_buffer_load_b64(rs, ni * 8, soff + L::UH_OFF, 2);
+            uh[0] = v[0], uh[1] = v[1];
+        }
+        if constexpr (F::BH == 16) {
+            const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(rs, ni * 16, blk + L::BH_OFF, 0);
+            bh[0] = v[0], bh[1] = v[1], bh[2] = v[2], bh[3] = v[3];
+        } else if constexpr (F::BH == 2) {
+            bh[0] = __builtin_amdgcn_raw_buffer_load_b32(rs, (ni >> 1) * 4, blk + L::BH_OFF, 0);
+        }
+#pragma unroll
+        for (int pl = 0; pl < F::WQ; ++pl) q[pl] = __builtin_amdgcn_raw_buffer_load_b128(rs, lane * 16, soff + pl * 1024, 2);
+        if constexpr (FMT == OXQ_GGUF_Q6_K) {
+            const u32x2_t v = __builtin_amdgcn_raw_buffer_load_b64(rs, lane * 8, soff + L::H_OFF, 2);
+            qh[0] = v[0], qh[1] = v[1];
+        }
+    }
+    // The factors of the chunk's steps, once per chunk when its registers have arrived; half = c % 2 (wave-uniform).
+    // f0[st] multiplies the step's sum, f1[st] (formats with a minimum) the bias term -128 sum(x).
+    __device__ __forceinline__ void factors(int half, int ni, float (&f0)[NSTEP], float (&f1)[NSTEP]) const {
+        if constexpr (FMT == OXQ_GGUF_Q4_K) {
+            // get_scale_min_k4 (quant_kernels.metal:2438-2450) for the chunk's four sub-blocks at once, a byte each
+            const uint32_t sc4 = half ? ((bh[3] & 0x0F0F0F0Fu) | ((bh[1] >> 2) & 0x30303030u)) : (bh[1] & 0x3F3F3F3Fu);
+            const uint32_t mn4 = half ? (((bh[3] >> 4) & 0x0F0F0F0Fu) | ((bh[2] >> 2) & 0x30303030u)) : (bh[2] & 0x3F3F3F3Fu);
+            const float d = ggm_f16(bh[0] & 0xFFFFu), dm = ggm_f16(bh[0] >> 16) * 0.0078125f;  // dmin / 128
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                f0[t] = d * (float)((sc4 >> (8 * t)) & 0xFFu);
+                f1[t] = dm * (float)((mn4 >> (8 * t)) & 0xFFu);
+            }
+        } else if constexpr (FMT == OXQ_GGUF_Q6_K) {
+            const float d = ggm_f16((ni & 1) ? (bh[0] >> 16) : (bh[0] & 0xFFFFu));
+#pragma unroll
+            for (int st = 0; st < 8; ++st) f0[st] = d * (float)(int)(int8_t)((uh[st >> 2] >> (8 * (st & 3))) & 0xFFu), f1[st] = 0.f;
+        } else {
+#pragma unroll
+            for (int st = 0; st < 4; ++st) f0[st] = ggm_f16((st & 1) ? (uh[st >> 1] >> 16) : (uh[st >> 1] & 0xFFFFu)), f1[st] = 0.f;
+        }
+    }
+    // B operand of step st: bias + q as bf16 pairs (four for a step of 32 elements, two for one of 16)
+    __device__ __forceinline__ void operand(int st, uint32_t (&b)[4], const NibbleMasks &nm) const {
+        if constexpr (FMT == OXQ_GGUF_Q4_0 || FMT == OXQ_GGUF_Q4_K) {
+#pragma unroll
+            for (int pp = 0; pp < 4; ++pp) b[pp] = BF16Traits::unpack1(q[0][st], pp, nm);
+        } else if constexpr (FMT == OXQ_GGUF_Q8_0) {
+            const uint32_t w0 = q[st >> 1][2 * (st & 1)], w1 = q[st >> 1][2 * (st & 1) + 1];
+            b[0] = ggm_bytes02(w0), b[1] = ggm_bytes13(w0), b[2] = ggm_bytes02(w1), b[3] = ggm_bytes13(w1);
+        } else {  // Q6_K: nibble | bit pair << 4, 128 + (0 .. 63) is exact in bf16
+            const uint32_t lw = q[0][st >> 1], hw = qh[st >> 2];
+#pragma unroll
+            for (int pr = 0; pr < 2; ++pr) {
+                const int f = 2 * (st & 3) + pr;
+                const uint32_t hs = f < 2 ? (hw << (4 - 2 * f)) : (hw >> (2 * f - 4));
+                b[pr] = (hs & nm.m1) | BF16Traits::unpack1(lw, 2 * (st & 1) + pr, nm);  // m1: the bit pairs' mask, in a register
+            }
+            b[2] = b[3] = 0u;
+        }
+    }
+};
+
+typedef short short4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float4_t ggm_mfma16(uint32_t a0, uint32_t a1, uint32_t b0, uint32_t b1, float4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4_t, u32x2_t{a0, a1}),
+                                                     __builtin_bit_cast(short4_t, u32x2_t{b0, b1}), c, 0, 0, 0);
+}
+
+template <int FMT, int MT, int XQ, int NW>
+__global__ __launch_bounds__(NW * 64) void ggm_kernel(const uint16_t *__restrict__ x, const uint8_t *__restrict__ pw,
+                                                      const uint16_t *__restrict__ bias, uint16_t *__restrict__ y,
+                                                      float *__restrict__ ws, int M, int K, int N, int cslice) {
+    typedef BF16Traits TT;
+    typedef MfmaOps<TT> Ops;
+    typedef GgmFmt<FMT> F;
+    typedef GgmLayout<FMT> L;
+    typedef GgmChunk<FMT> C;
+    constexpr int ROWS = 16 * MT, AQ = XQ, SLOT = ROWS * 256, OOB = 0x7FFFFF00, NSTEP = C::NSTEP;
+    // chunks in flight a wave: three, two where block headers and factors take the registers (measured on
+    // 4096 x 4096 at one row, Q8_0: 5.06 us with three, 5.87 with two)
+    constexpr int RD = FMT == OXQ_GGUF_Q4_K ? 2 : 3;
+    constexpr bool K16 = NSTEP == 8;  // steps of 16 elements
+    extern __shared__ __attribute__((aligned(16))) unsigned char pk4_lds[];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int ni = lane & 15, kb = lane >> 4;
+    const int j = blockIdx.x;
+    const int m0 = blockIdx.z * ROWS;
+    const int NC = K >> 7;
+    const int sc0 = blockIdx.y * cslice;
+    const int SC = min(NC, sc0 + cslice) - sc0;
+    const int cbase = SC / NW, crem = SC % NW;
+    const int nloc = cbase + (wave < crem ? 1 : 0);
+    const int cc0 = sc0 + wave * cbase + min(wave, crem);
+    unsigned char *slot = pk4_lds + wave * SLOT;
+
+    const uint32_t strip_bytes = (uint32_t)(NC / F::CH) * (uint32_t)L::BLKB;
+    const __amdgpu_buffer_rsrc_t rs_w = make_rsrc(pw + (size_t)j * strip_bytes, strip_bytes);
+    const int xrows = min(M - m0, ROWS);
+    const __amdgpu_buffer_rsrc_t rs_x = make_rsrc(x + (size_t)m0 * K, (uint32_t)xrows * (uint32_t)K * 2u);
+    const __amdgpu_buffer_rsrc_t rs_none = make_rsrc(pw, 0u);
+    int voff_a[AQ];
+#pragma unroll
+    for (int q = 0; q < AQ; ++q) {
+        const int r = 4 * q + kb;
+        voff_a[q] = r < xrows ? (r * K * 2 + ni * 16) : OOB;
+    }
+    // x in LDS: row r of the tile at r * 256, its sixteen 16-byte pieces XOR-swizzled by the row
+    int a_wr[4];
+#pragma unroll
+    for (int qq = 0; qq < 4; ++qq) a_wr[qq] = kb * 256 + (((ni ^ kb) ^ (qq << 2)) << 4);
+    // step st of the chunk: elements 32 st + 8 kb .. + 7 of row ni (16 st + 4 kb .. + 3 for steps of 16)
+    int a_rd[NSTEP];
+#pragma unroll
+    for (int st = 0; st < NSTEP; ++st)
+        a_rd[st] = K16 ? ni * 256 + (((2 * st + (kb >> 1)) ^ ni) << 4) + (kb & 1) * 8 : ni * 256 + (((4 * st + kb) ^ ni) << 4);
+    // both masks in registers: v_and_or_b32 takes one literal, and the exponent pattern is it
+    const NibbleMasks nm = FMT == OXQ_GGUF_Q6_K ? NibbleMasks{vgpr_const(0x000F000Fu), vgpr_const(0x00300030u)} : nibble_masks();
+#pragma unroll
+    for (int q = AQ; q < 4 * MT; ++q) {  // rows no call of this instantiation brings stay zero
+        const int row = 4 * q + kb;
+        *(u32x4_t *)(slot + row * 256 + ((ni ^ (row & 15)) << 4)) = u32x4_t{0u, 0u, 0u, 0u};
+    }
+
+    C wr[RD];
+    u32x4_t ar[RD][AQ];
+    auto request = [&](int i, C &w, u32x4_t (&a)[AQ]) {
+        const bool live = i < nloc;  // wave-uniform
+        const __amdgpu_buffer_rsrc_t rx = live ? rs_x : rs_none, rw = live ? rs_w : rs_none;
+        const int c = cc0 + i;
+#pragma unroll
+        for (int q = 0; q < AQ; ++q) a[q] = __builtin_amdgcn_raw_buffer_load_b128(rx, voff_a[q], c * 256, 0);
+        w.request(rw, lane, ni, c);
+        __builtin_amdgcn_sched_barrier(0);  // chunks are requested in the order they are used
+    };
+#pragma unroll
+    for (int d = 0; d < RD; ++d) request(d, wr[d], ar[d]);
+
+    float4_t acc[MT][1];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[mt][0] = float4_t{0.f, 0.f, 0.f, 0.f};
+    const uint32_t neg[4] = {F::NEG, F::NEG, F::NEG, F::NEG};
+    const float4_t zero4 = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    // A operand of step st, row tile mt
+    auto load_a = [&](int st, int mt, uint32_t (&a)[4]) {
+        if constexpr (K16) {
+            const uint2 av = *(const uint2 *)(slot + mt * 4096 + a_rd[st]);
+            a[0] = av.x, a[1] = av.y, a[2] = 0u, a[3] = 0u;
+        } else {
+            const u32x4_t av = *(const u32x4_t *)(slot + mt * 4096 + a_rd[st]);
+            a[0] = av[0], a[1] = av[1], a[2] = av[2], a[3] = av[3];
+        }
+    };
+    auto mma = [&](const uint32_t (&a)[4], const uint32_t (&b)[4], float4_t c) -> float4_t {
+        if constexpr (K16) return ggm_mfma16(a[0], a[1], b[0], b[1], c);
+        else return Ops::mfma(a, b, c);
+    };
+
+    auto chunk = [&](int i, auto cur_c, bool more) {
+        constexpr int CUR = decltype(cur_c)::value;
+        C &w = wr[CUR];
+#pragma unroll
+        for (int q = 0; q < AQ; ++q) *(u32x4_t *)(slot + q * 1024 + a_wr[q & 3]) = ar[CUR][q];
+        float f0[NSTEP], f1[NSTEP];
+        if constexpr (MT == 1) {
+            // what depends on x alone first (x is requested ahead of the chunk's quants): the operands and the
+            // bias term of four steps, so that one MFMA a step is left when the quants arrive
+#pragma unroll
+            for (int g = 0; g < NSTEP; g += 4) {
+                uint32_t a[4][4];
+                float4_t tn[4];
+#pragma unroll
+                for (int s4 = 0; s4 < 4; ++s4) {
+                    load_a(g + s4, 0, a[s4]);
+                    tn[s4] = mma(a[s4], neg, zero4);
+                }
+                if (g == 0) w.factors((cc0 + i) & 1, ni, f0, f1);
+                if constexpr (C::HAS_MIN) {
+#pragma unroll
+                    for (int s4 = 0; s4 < 4; ++s4)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) acc[0][0][e] = fmaf(f1[g + s4], tn[s4][e], acc[0][0][e]);
+                }
+#pragma unroll
+                for (int s4 = 0; s4 < 4; ++s4) {
+                    uint32_t b[4];
+                    w.operand(g + s4, b, nm);
+                    const float4_t t = mma(a[s4], b, tn[s4]);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) acc[0][0][e] = fmaf(f0[g + s4], t[e], acc[0][0][e]);
+                }
+            }
+        } else {  // more row tiles: step by step, the registers do not hold a chunk's operands
+            w.factors((cc0 + i) & 1, ni, f0, f1);
+#pragma unroll
+            for (int st = 0; st < NSTEP; ++st) {
+                uint32_t b[4];
+                w.operand(st, b, nm);
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+                    uint32_t a[4];
+                    load_a(st, mt, a);
+                    const float4_t tn = mma(a, neg, zero4);
+                    const float4_t t = mma(a, b, tn);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        acc[mt][0][e] = fmaf(f0[st], t[e], acc[mt][0][e]);
+                        if constexpr (C::HAS_MIN) acc[mt][0][e] = fmaf(f1[st], tn[e], acc[mt][0][e]);
+                    }
+                }
+            }
+        }
+        if (more) request(i + RD, wr[CUR], ar[CUR]);
+        __builtin_amdgcn_sched_barrier(0);  // one chunk's operands in the registers at a time
+    };
+    {
+        int i = 0;
+        if constexpr (RD == 2) {
+            for (; i + 1 < nloc; i += 2) {
+                chunk(i, std::integral_constant<int, 0>{}, true);
+                chunk(i + 1, std::integral_constant<int, 1>{}, true);
+            }
+            if (i < nloc) chunk(i, std::integral_constant<int, 0>{}, false);
+        } else {
+            for (; i + 2 < nloc; i += 3) {
+                chunk(i, std::integral_constant<int, 0>{}, true);
+                chunk(i + 1, std::integral_constant<int, 1>{}, true);
+                chunk(i + 2, std::integral_constant<int, 2>{}, true);
+            }
+            if (i < nloc) chunk(i, std::integral_constant<int, 0>{}, false);
+            if (i + 1 < nloc) chunk(i + 1, std::integral_constant<int, 1>{}, false);
+        }
+    }
+    pk4n_epilogue<TT, MT, 1, NW>(acc, bias, y, ws, M, N, j, m0, wave, lane);
+}
+
+// ---------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------
+static bool ggm_format(int quant) {
+    return quant == OXQ_GGUF_Q4_0 || quant == OXQ_GGUF_Q8_0 || quant == OXQ_GGUF_Q4_K || quant == OXQ_GGUF_Q6_K;
+}
+static const char *ggm_name(int q) {
+    switch (q) {
+    case OXQ_GGUF_Q4_0: return "q4_0";
+    case OXQ_GGUF_Q8_0: return "q8_0";
+    case OXQ_GGUF_Q4_K: return "q4k";
+    default: return "q6k";
+    }
+}
+
+bool gguf_mfma_eligible(const oxq_ctx *ctx, int quant, int64_t K, int64_t N) {
+    if (!ggm_format(quant) || tune(ctx, OXQ_TUNE_GGUF_MFMA, 1) == 0) return false;
+    return gguf_res_eligible(quant, K, N);  // the same strips, chunks and 32-bit offsets
+}
+
+int launch_gguf_mfma_repack(oxq_ctx *ctx, hipStream_t s, int quant, const uint8_t *w, void *pw, int64_t K, int64_t N) {
+    const size_t threads = (size_t)(N / 16) * (K / 128) * 64;
+    dim3 grid((unsigned)ceil_div((int64_t)threads, 256)), block(256);
+    char name[64];
+    snprintf(name, sizeof name, "gguf_%s_mfma_repack", ggm_name(quant));
+    set_plan(ctx, name, grid, block, 1, 1, 0);
+    if (ctx->plan_only) return OXQ_OK;
+    switch (quant) {
+    case OXQ_GGUF_Q4_0: hipLaunchKernelGGL((ggm_repack_kernel<OXQ_GGUF_Q4_0>), grid, block, 0, s, w, (uint8_t *)pw, (int)K, (int)N); break;
+    case OXQ_GGUF_Q8_0: hipLaunchKernelGGL((ggm_repack_kernel<OXQ_GGUF_Q8_0>), grid, block, 0, s, w, (uint8_t *)pw, (int)K, (int)N); break;
+    case OXQ_GGUF_Q4_K: hipLaunchKernelGGL((ggm_repack_kernel<OXQ_GGUF_Q4_K>), grid, block, 0, s, w, (uint8_t *)pw, (int)K, (int)N); break;
+    case OXQ_GGUF_Q6_K: hipLaunchKernelGGL((ggm_repack_kernel<OXQ_GGUF_Q6_K>), grid, block, 0, s, w, (uint8_t *)pw, (int)K, (int)N); break;
+    default: return fail(OXQ_ERR_UNSUPPORTED, "gguf repack: format %d has no matrix-core layout", quant);
+    }
+    OXQ_HIP_CHECK(hipGetLastError());
+    return OXQ_OK;
+}
+
+int launch_gguf_mfma_dequant(oxq_ctx *ctx, hipStream_t s, int quant, const void *pw, int64_t K, int64_t N, float *out_nk) {
+    const size_t threads = (size_t)(N / 16) * (K / 128) * 64;
+    dim3 grid((unsigned)ceil_div((int64_t)threads, 256)), block(256);
+    char name[64];
+    snprintf(name, sizeof name, "gguf_%s_mfma_dequant", ggm_name(quant));
+    set_plan(ctx, name, grid, block, 1, 1, 0);
+    if (ctx->plan_only) return OXQ_OK;
+    switch (quant) {
+    case OXQ_GGUF_Q4_0: hipLaunchKernelGGL((ggm_dequant_kernel<OXQ_GGUF_Q4_0>), grid, block, 0, s, (const uint8_t *)pw, out_nk, (int)K, (int)N); break;
+    case OXQ_GGUF_Q8_0: hipLaunchKernelGGL((ggm_dequant_kernel<OXQ_GGUF_Q8_0>), grid, block, 0, s, (const uint8_t *)pw, out_nk, (int)K, (int)N); break;
+    case OXQ_GGUF_Q4_K: hipLaunchKernelGGL((ggm_dequant_kernel<OXQ_GGUF_Q4_K>), grid, block, 0, s, (const uint8_t *)pw, out_nk, (int)K, (int)N); break;
+    case OXQ_GGUF_Q6_K: hipLaunchKernelGGL((ggm_dequant_kernel<OXQ_GGUF_Q6_K>), grid, block, 0, s, (const uint8_t *)pw, out_nk, (int)K, (int)N); break;
+    default: return fail(OXQ_ERR_UNSUPPORTED, "gguf dequant: format %d has no matrix-core layout", quant);
+    }
+    OXQ_HIP_CHECK(hipGetLastError());
+    return OXQ_OK;
+}
+
+template <int FMT, int MT, int XQ, int NW>
+static int ggm_go(hipStream_t s, dim3 grid, const GgufProblem &p, float *ws, int cslice) {
+    static LdsGrant lds_grant;  // one per instantiation
+    const size_t lds = (size_t)NW * MT * 4096;
+    OXQ_HIP_CHECK(lds_grant.ensure((const void *)ggm_kernel<FMT, MT, XQ, NW>, lds));
+    hipLaunchKernelGGL((ggm_kernel<FMT, MT, XQ, NW>), grid, dim3(NW * 64), lds, s, (const uint16_t *)p.x, p.w,
+                       (const uint16_t *)p.bias, (uint16_t *)p.y, ws, (int)p.M, (int)p.K, (int)p.N, cslice);
+    OXQ_HIP_CHECK(hipGetLastError());
+    return OXQ_OK;
+}
+template <int FMT, int NW>
+static int ggm_by_rows(hipStream_t s, dim3 grid, const GgufProblem &p, float *ws, int cslice, int mt, int xq) {
+    if (mt == 2) return ggm_go<FMT, 2, 8, NW>(s, grid, p, ws, cslice);
+    if (xq == 1) return ggm_go<FMT, 1, 1, NW>(s, grid, p, ws, cslice);
+    if (xq == 2) return ggm_go<FMT, 1, 2, NW>(s, grid, p, ws, cslice);
+    return ggm_go<FMT, 1, 4, NW>(s, grid, p, ws, cslice);
+}
+
+// rows of x a launch of the matrix-core kernel takes (more go to the tile matmul on the file layout)
+bool gguf_mfma_takes(const oxq_ctx *ctx, int64_t M, int act_dtype) {
+    return act_dtype == OXQ_BF16 && M >= 1 && M <= tune(ctx, OXQ_TUNE_GGUF_MFMA_MAX_M, 32);
+}
+
+// p.w is the matrix-core copy
+int launch_gguf_mfma(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p) {
+    const int mt = p.M > 16 ? 2 : 1;
+    const int rows = (int)std::min<int64_t>(p.M, 16 * mt);
+    const int xq = rows <= 4 ? 1 : rows <= 8 ? 2 : 4;
+    // two row tiles need more than the 128 registers a wave of a 16-wave workgroup has
+    const int nw = (p.K / 128 < 16 || mt == 2) ? 8 : 16;
+    dim3 grid((unsigned)(p.N / 16), 1, (unsigned)ceil_div(p.M, (int64_t)16 * mt));
+    char name[64];
+    snprintf(name, sizeof name, "gguf_%s_mfma_bf16_mt%d", ggm_name(p.quant), mt);
+    set_plan(ctx, name, grid, dim3(nw * 64), 1, 1, 0);
+    if (ctx->plan_only) return OXQ_OK;
+    if (p.act_dtype != OXQ_BF16) return fail(OXQ_ERR_UNSUPPORTED, "gguf matrix-core matmul: activations must be BF16");
+    if ((uintptr_t)p.x & 15) return fail(OXQ_ERR_UNSUPPORTED, "gguf matrix-core matmul: x must be 16-byte aligned");
+    if ((uint64_t)16 * mt * (uint64_t)p.K * 2 >= (1ull << 31)) return fail(OXQ_ERR_UNSUPPORTED, "gguf matrix-core matmul: K too large");
+    const int cslice = (int)(p.K / 128);
+    switch (p.quant) {
+    case OXQ_GGUF_Q4_0: return nw == 8 ? ggm_by_rows<OXQ_GGUF_Q4_0, 8>(s, grid, p, nullptr, cslice, mt, xq) : ggm_by_rows<OXQ_GGUF_Q4_0, 16>(s, grid, p, nullptr, cslice, mt, xq);
+    case OXQ_GGUF_Q8_0: return nw == 8 ? ggm_by_rows<OXQ_GGUF_Q8_0, 8>(s, grid, p, nullptr, cslice, mt, xq) : ggm_by_rows<OXQ_GGUF_Q8_0, 16>(s, grid, p, nullptr, cslice, mt, xq);
+    case OXQ_GGUF_Q4_K: return nw == 8 ? ggm_by_rows<OXQ_GGUF_Q4_K, 8>(s, grid, p, nullptr, cslice, mt, xq) : ggm_by_rows<OXQ_GGUF_Q4_K, 16>(s, grid, p, nullptr, cslice, mt, xq);
+    case OXQ_GGUF_Q6_K: return nw == 8 ? ggm_by_rows<OXQ_GGUF_Q6_K, 8>(s, grid, p, nullptr, cslice, mt, xq) : ggm_by_rows<OXQ_GGUF_Q6_K, 16>(s, grid, p, nullptr, cslice, mt, xq);
+    default: return fail(OXQ_ERR_UNSUPPORTED, "gguf matrix-core matmul: format %d", p.quant);
+    }
+}
+
+}  // namespace oxq

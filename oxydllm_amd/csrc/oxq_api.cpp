@@ -836,11 +836,15 @@ static bool wcache_forward(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p, i
     return true;
 }
 
-// The same for a GGUF weight (Q4_0 / Q8_0 / Q4_K / Q6_K, 1 - 4 rows of x): the copy is the strip-major
-// one of the QLinear layers.  Entry fields: qw = the block bytes, bits = the ggml format, w.pw = the copy.
+// The same for a GGUF weight: the copy is the strip-major one of the QLinear layers - the matrix-core layout
+// for bf16 activations (up to the rows its kernel takes), the rotated one of the vector GEMV for f32 (1 - 8
+// rows).  Entry fields: qw = the block bytes, bits = the ggml format, pack_dim = -1 (rotated) or -2
+// (matrix-core), w.pw = the copy.
 static bool wcache_forward_gguf(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p, int *rc) {
-    if (!ctx->wcache_limit || ctx->plan_only || !gguf_res_eligible(p.quant, p.K, p.N) || !gguf_res_takes(p.K, p.M, p.act_dtype))
-        return false;
+    if (!ctx->wcache_limit || ctx->plan_only || !gguf_res_eligible(p.quant, p.K, p.N)) return false;
+    const bool mfma = p.act_dtype == OXQ_BF16 && gguf_mfma_eligible(ctx, p.quant, p.K, p.N);
+    if (!(mfma ? gguf_mfma_takes(ctx, p.M, p.act_dtype) : gguf_res_takes(p.K, p.M, p.act_dtype))) return false;
+    const int kind = mfma ? -2 : -1;
     if (((uintptr_t)p.x & 15) || ((uintptr_t)p.w & 1)) return false;
     if (!ctx->wcache) {
         ctx->wcache = new (std::nothrow) oxq_weight_cache();
@@ -851,7 +855,7 @@ static bool wcache_forward_gguf(oxq_ctx *ctx, hipStream_t s, const GgufProblem &
     oxq_weight_cache::Entry *hit = nullptr;
     for (auto &e : c->entries)
         if (e.qw == p.w && e.qz == nullptr && e.sc == nullptr && e.K == p.K && e.N == p.N && e.bits == p.quant &&
-            e.pack_dim == -1) {
+            e.pack_dim == kind) {
             hit = &e;
             break;
         }
@@ -868,9 +872,9 @@ static bool wcache_forward_gguf(oxq_ctx *ctx, hipStream_t s, const GgufProblem &
             (void)hipGetLastError();
             return false;
         }
-        oxq_weight_cache::Entry e{p.w, nullptr, nullptr, p.K, p.N, 0, 0, p.quant, -1,
+        oxq_weight_cache::Entry e{p.w, nullptr, nullptr, p.K, p.N, 0, 0, p.quant, kind,
                                   Pk4Weights{(uint32_t *)mem, nullptr, p.K, p.N, 0, 0, 0, 0, 0, 0}, bytes, 0, false};
-        const int prc = launch_gguf_res_repack(ctx, s, p.quant, p.w, mem, p.K, p.N);
+        const int prc = (mfma ? launch_gguf_mfma_repack : launch_gguf_res_repack)(ctx, s, p.quant, p.w, mem, p.K, p.N);
         if (prc != OXQ_OK) {
             (void)hipFree(mem);
             *rc = prc;
@@ -889,7 +893,7 @@ static bool wcache_forward_gguf(oxq_ctx *ctx, hipStream_t s, const GgufProblem &
     wcache_pin_if_capturing(s, hit);
     GgufProblem q = p;
     q.w = (const uint8_t *)hit->w.pw;
-    *rc = launch_gguf_res_gemv(ctx, s, q);
+    *rc = mfma ? launch_gguf_mfma(ctx, s, q) : launch_gguf_res_gemv(ctx, s, q);
     return true;
 }
 
@@ -1083,6 +1087,8 @@ int oxq_gguf_quant_mul_mm(oxq_ctx *ctx, void *stream, const oxq_tensor *x,
     GgufProblem p;
     OXQ_TRY(check_gguf(ctx, "GgufQuantMulMM", false, false, x, weight_bytes, in_features,
                        out_features, quant, out, &p));
+    int rc = OXQ_OK;
+    if (wcache_forward_gguf(ctx, (hipStream_t)stream, p, &rc)) return rc;
     if (gguf_mm_eligible(ctx, p)) return launch_gguf_mm(ctx, (hipStream_t)stream, p);
     return launch_gguf_gemv(ctx, (hipStream_t)stream, p);
 }
@@ -1913,8 +1919,9 @@ struct oxq_qlinear {
     int64_t in_features, out_features;
     int quant;
     int out_dtype;
-    void *res = nullptr;    // layer-owned strip-major copy of the blocks (decode GEMV)
+    void *res = nullptr;    // layer-owned strip-major copy of the blocks
     bool resident = false;
+    bool mfma = false;      // the copy is the matrix-core layout (bf16 layers), else the rotated one of the vector GEMV
 };
 
 // linear.rs:225-240: the fast path copies the block bytes at build; here the copy is strip-major
@@ -1923,6 +1930,8 @@ static int build_resident_gguf(oxq_qlinear *l) {
     if (!gguf_res_eligible(l->quant, l->in_features, l->out_features)) return OXQ_OK;
     if (((uintptr_t)l->weight_bytes.data & 1) != 0) return OXQ_OK;
     oxq_ctx *ctx = l->ctx;
+    // a bf16 layer (the reference's GPU path: bf16 x and y) of a format that has it takes the matrix-core layout
+    l->mfma = l->out_dtype == OXQ_BF16 && gguf_mfma_eligible(ctx, l->quant, l->in_features, l->out_features);
     if (ctx->plan_only) {
         l->resident = true;
         return OXQ_OK;
@@ -1936,8 +1945,8 @@ static int build_resident_gguf(oxq_qlinear *l) {
         l->res = nullptr;
         rc = fail(OXQ_ERR_RUNTIME, "QLinear: repack allocation failed: %s", hipGetErrorString(e));
     } else {
-        rc = launch_gguf_res_repack(ctx, nullptr, l->quant, (const uint8_t *)l->weight_bytes.data, l->res, l->in_features,
-                                    l->out_features);
+        rc = (l->mfma ? launch_gguf_mfma_repack : launch_gguf_res_repack)(
+            ctx, nullptr, l->quant, (const uint8_t *)l->weight_bytes.data, l->res, l->in_features, l->out_features);
         if (rc == OXQ_OK && (e = hipStreamSynchronize(nullptr)) != hipSuccess)
             rc = fail(OXQ_ERR_RUNTIME, "QLinear: repack failed: %s", hipGetErrorString(e));
     }
@@ -2174,7 +2183,12 @@ int oxq_qlinear_forward(oxq_qlinear *l, void *stream, const oxq_tensor *x, const
     OXQ_TRY(check_gguf(l->ctx, decode ? "GgufQuantMatmul" : "GgufQuantMulMM", decode, false, &x2,
                        &l->weight_bytes, l->in_features, l->out_features, l->quant, &o2, &p));
     p.bias = l->has_bias ? l->bias.data : nullptr;
-    if (l->resident && gguf_res_takes(p.K, p.M, p.act_dtype) && ((uintptr_t)p.x & 15) == 0) {
+    if (l->resident && l->mfma) {
+        if (gguf_mfma_takes(l->ctx, p.M, p.act_dtype) && ((uintptr_t)p.x & 15) == 0) {
+            p.w = (const uint8_t *)l->res;
+            return launch_gguf_mfma(l->ctx, (hipStream_t)stream, p);
+        }
+    } else if (l->resident && gguf_res_takes(p.K, p.M, p.act_dtype) && ((uintptr_t)p.x & 15) == 0) {
         p.w = (const uint8_t *)l->res;
         return launch_gguf_res_gemv(l->ctx, (hipStream_t)stream, p);
     }
@@ -2197,8 +2211,8 @@ int oxq_qlinear_dequantize(oxq_qlinear *l, void *stream, const oxq_tensor *out) 
                     (long long)l->in_features);
     if (!out->contiguous) return fail(OXQ_ERR_CONTIGUOUS, "%s: out must be contiguous", op);
     if (l->resident)
-        return launch_gguf_res_dequant(l->ctx, (hipStream_t)stream, l->quant, l->res, l->in_features, l->out_features,
-                                       (float *)out->data);
+        return (l->mfma ? launch_gguf_mfma_dequant : launch_gguf_res_dequant)(
+            l->ctx, (hipStream_t)stream, l->quant, l->res, l->in_features, l->out_features, (float *)out->data);
     GgufProblem p{};
     p.w = (const uint8_t *)l->weight_bytes.data;
     p.K = l->in_features, p.N = l->out_features, p.quant = l->quant, p.act_dtype = OXQ_F32;

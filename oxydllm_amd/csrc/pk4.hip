@@ -731,55 +731,6 @@ __global__ __launch_bounds__(256) void pk4n_dequant_kernel(const uint32_t *__res
     }
 }
 
-// The waves' partial tiles meet in LDS as in the wide form; a thread then owns (row, column ni of every
-// strip of the workgroup) and adds the waves in order.
-template <typename TT, int MT, int NS, int NW>
-__device__ __forceinline__ void pk4n_epilogue(const float4_t (&acc)[MT][NS], const uint16_t *__restrict__ bias,
-                                              uint16_t *__restrict__ y, float *__restrict__ ws, int M, int N, int j,
-                                              int m0, int wave, int lane) {
-    constexpr int NT = NW * 64, ROWS = 16 * MT;
-    extern __shared__ __attribute__((aligned(16))) unsigned char pk4_lds[];
-    // every wave into its own activation slot (other waves may still be reading theirs): [MT][4 e][64 lanes][NS]
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            float *dst = (float *)(pk4_lds + (size_t)wave * MT * 4096) + ((mt * 4 + e) * 64 + lane) * NS;
-            if constexpr (NS == 4) *(float4_t *)dst = float4_t{acc[mt][0][e], acc[mt][1][e], acc[mt][2][e], acc[mt][3][e]};
-            else dst[0] = acc[mt][0][e];
-        }
-    __syncthreads();
-    for (int t = threadIdx.x; t < ROWS * 16; t += NT) {
-        const int ml = t >> 4, ni = t & 15;
-        if (m0 + ml >= M) continue;
-        const int mt = ml >> 4, r = ml & 15, kb = r >> 2, e = r & 3;
-        float v[NS];
-#pragma unroll
-        for (int f = 0; f < NS; ++f) v[f] = 0.f;
-#pragma unroll
-        for (int s = 0; s < NW; ++s) {
-            const float *src = (const float *)(pk4_lds + (size_t)s * MT * 4096) + ((mt * 4 + e) * 64 + kb * 16 + ni) * NS;
-            if constexpr (NS == 4) {
-                const float4_t q = *(const float4_t *)src;
-                v[0] += q[0], v[1] += q[1], v[2] += q[2], v[3] += q[3];
-            } else {
-                v[0] += src[0];
-            }
-        }
-#pragma unroll
-        for (int f = 0; f < NS; ++f) {
-            const int n = 16 * (NS * j + f) + ni;
-            if (gridDim.y > 1) {  // this K slice's f32 partial; a second kernel adds the slices in order
-                ws[((size_t)blockIdx.y * M + (m0 + ml)) * N + n] = v[f];
-            } else {
-                float o = v[f];
-                if (bias) o += TT::to_f32(bias[n]);
-                y[(size_t)(m0 + ml) * N + n] = TT::from_f32(o);
-            }
-        }
-    }
-}
-
 template <typename TT, int MT, bool GS, int NS, int XQ, int NW>
 __global__ __launch_bounds__(NW * 64) void pk4n_mfma_kernel(const uint16_t *__restrict__ x,
                                                         const uint32_t *__restrict__ pw,

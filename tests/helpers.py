@@ -81,6 +81,20 @@ def resident_rounds_weights(m: int, dt: int, gptq: bool) -> bool:
     return not (gptq and m <= 32)
 
 
+GGUF_MATRIX_CORE_ROWS = 32
+
+
+def gguf_on_matrix_cores(fmt: int, n: int, k: int, m: int, bf16: bool = True) -> bool:
+    """Whether a resident bf16 QLinear of this format and shape runs m rows on its matrix-core copy: then the
+    weights stay unrounded (the GEMV's arithmetic) also above 8 rows, where the reference's prefill tiles round
+    them to bf16."""
+    from oxydllm_amd import synth
+    if not bf16 or fmt not in (synth.GGUF_Q4_0, synth.GGUF_Q8_0, synth.GGUF_Q4_K, synth.GGUF_Q6_K):
+        return False
+    kq = fmt in (synth.GGUF_Q4_K, synth.GGUF_Q6_K)
+    return n % 16 == 0 and k % (256 if kq else 128) == 0 and 1 <= m <= GGUF_MATRIX_CORE_ROWS
+
+
 def round_x(x_f32: np.ndarray, dt: int) -> np.ndarray:
     """The activation values the kernel actually sees (x rounded to its 16-bit dtype)."""
     return oracle.round_through(x_f32, dt)

@@ -335,7 +335,7 @@ def test_feed_forward_validates_and_plans(lib, ctx):
     assert rc == 0, err(lib)
     assert lib.oxq_mlp_forward(m, None, C.byref(fake((1, H), BF16)), C.byref(fake((2 * I,), BF16)),
                                C.byref(fake((1, H), BF16))) == 0, err(lib)
-    assert plan(lib, ctx).kernel.decode().startswith("gguf_q4k_res_gemv_bf16")
+    assert plan(lib, ctx).kernel.decode().startswith("gguf_q4k_mfma_bf16_mt1")  # a bf16 layer: the matrix-core copy
     lib.oxq_mlp_free(m)
     for h in (qg, qu, qd):
         lib.oxq_qlinear_free(h)
@@ -396,9 +396,9 @@ def test_layers_validate_like_reference(lib, ctx):
     w = fake((4096 * 16 * 144,), U8)
     assert lib.oxq_qlinear_new(ctx, _lib.GGUF_Q4_K, C.byref(w), 4096, 4096, None, BF16, C.byref(q)) == 0
     # rows 1-4: the GEMV on the layer's strip-major copy; 5-8 the tile matmul with unrounded weights
-    for m_rows, kern in [(1, "gguf_q4k_res_gemv_bf16_m1"), (2, "gguf_q4k_res_gemv_bf16_m2"),
-                         (4, "gguf_q4k_res_gemv_bf16_m4"), (8, "gguf_q4k_mul_mm_bf16_mt1_f32w"),
-                         (16, "gguf_q4k_mul_mm_bf16_mt1"), (33, "gguf_q4k_mul_mm_bf16_mt4")]:
+    for m_rows, kern in [(1, "gguf_q4k_mfma_bf16_mt1"), (2, "gguf_q4k_mfma_bf16_mt1"),
+                         (4, "gguf_q4k_mfma_bf16_mt1"), (8, "gguf_q4k_mfma_bf16_mt1"),
+                         (16, "gguf_q4k_mfma_bf16_mt1"), (32, "gguf_q4k_mfma_bf16_mt2"), (33, "gguf_q4k_mul_mm_bf16_mt4")]:
         assert lib.oxq_qlinear_forward(q, None, C.byref(fake((m_rows, 4096), BF16)),
                                        C.byref(fake((m_rows, 4096), BF16))) == 0, err(lib)
         p = plan(lib, ctx)
@@ -406,7 +406,7 @@ def test_layers_validate_like_reference(lib, ctx):
     res = C.c_int(-1)
     assert lib.oxq_qlinear_is_resident(q, C.byref(res)) == 0 and res.value == 1
     assert lib.oxq_qlinear_dequantize(q, None, C.byref(fake((4096, 4096), F32))) == 0, err(lib)
-    assert plan(lib, ctx).kernel.decode() == "gguf_q4k_res_dequant"
+    assert plan(lib, ctx).kernel.decode() == "gguf_q4k_mfma_dequant"
     assert lib.oxq_qlinear_dequantize(q, None, C.byref(fake((4096, 4095), F32))) == -3
     # a strided view of the right shape would be written past its storage: refused
     assert lib.oxq_qlinear_dequantize(q, None, C.byref(fake((4096, 4096), F32, contiguous=False))) == -4

@@ -13,7 +13,7 @@ from oxydllm_amd import checkpoint as ck
 from oxydllm_amd import ops, synth
 from tests import ggufio as G
 from tests import refgen
-from tests.helpers import as_f32, assert_close, round_x, to_dev, resident_rounds_weights
+from tests.helpers import as_f32, assert_close, gguf_on_matrix_cores, round_x, to_dev, resident_rounds_weights
 
 pytestmark = pytest.mark.gpu
 
@@ -36,7 +36,8 @@ def test_gguf_file_to_qlinear(tmp_path):
                 x = _x(m, K, seed=m)
                 y = layer.forward(to_dev(x, torch.bfloat16))
                 wt = oracle.dequantize_gguf(fmt, data[name], N, K)
-                ref = oracle.matmul_nt_f32(round_x(x, oracle.BF16), wt if m <= 8 else oracle.round_through(wt, oracle.BF16))
+                unrounded = m <= 8 or gguf_on_matrix_cores(fmt, N, K, m)
+                ref = oracle.matmul_nt_f32(round_x(x, oracle.BF16), wt if unrounded else oracle.round_through(wt, oracle.BF16))
                 assert_close(y, ref, f"{name} m={m}", bf16_out=True)
         # q projection with the converter's row interleave undone on the device
         fmt, N, K = shapes["blk.0.attn_q.weight"]

@@ -1,0 +1,167 @@
+"""Resident bf16 GGUF layers on the matrix-core layout (csrc/gguf_mfma.hip), through the C ABI.
+
+A bf16 QLinear (linear.rs:197-284, the reference's GPU contract: bf16 x and y) of Q4_0, Q8_0, Q4_K or Q6_K keeps
+a copy of its blocks in which a strip of 16 columns and a step of 32 (Q6_K: 16) elements of K are one MFMA whose
+rows are rows of x; 1 - 32 rows run on it in one launch.  The arithmetic is the GEMV's at every row count
+(quant_kernels.metal:1097-1221, 1681-1838: integer sums, one f32 scale per sub-block): the weights are never
+rounded to bf16, which the reference's prefill tiles do above 8 rows (quant_kernels.metal:2315-2640).  Hence
+the oracle here is the f32 dequant with an f32 matmul at 2e-3 relative / 1e-2 absolute (plus half a bf16 ulp of
+the output) for all rows, and for 9 - 32 rows also the tile oracle within the reference's own bound
+(metal_ops.rs:6449-6461).
+
+Shapes cover: the benchmark's 4096 x 4096 (two chunks a wave); one chunk a wave and waves without one
+(K = 256 .. 1024, 8-wave workgroups); long K (7 and 14 chunks a wave: the ring's loop with every tail); odd
+numbers of super-blocks, so that a wave's share starts in the middle of one; one to four row quads, two row
+tiles, ragged rows; bias.  The repack itself is pinned bit for bit in test_gpu_gguf_resident.py.
+"""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from oxydllm_amd import synth
+from tests.helpers import as_f32, assert_close, bits_of, gguf_on_matrix_cores, round_x, to_dev, tune
+
+pytestmark = pytest.mark.gpu
+ops = None
+MC = [synth.GGUF_Q4_0, synth.GGUF_Q8_0, synth.GGUF_Q4_K, synth.GGUF_Q6_K]
+FMTS = [pytest.param(f, id=synth.GGUF_NAMES[f]) for f in MC]
+TAG = {synth.GGUF_Q4_0: "q4_0", synth.GGUF_Q8_0: "q8_0", synth.GGUF_Q4_K: "q4k", synth.GGUF_Q6_K: "q6k"}
+
+
+def setup_module(module):
+    from oxydllm_amd import ops as _ops
+    module.ops = _ops
+
+
+def say(msg):
+    print(f"[case] {msg}", flush=True)
+    sys.stdout.flush()
+
+
+def _layer(fmt, N, K, seed, bias=None):
+    data = synth.gguf_weight(fmt, N, K, seed=seed)
+    layer = ops.QLinear(fmt, to_dev(data), K, N, None if bias is None else to_dev(bias, torch.bfloat16), torch.bfloat16)
+    assert layer.resident
+    return data, layer
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+@pytest.mark.parametrize("N,K", [(4096, 4096), (16, 256), (48, 768), (64, 1792), (32, 14336), (16, 28672), (112, 2304 + 256)])
+def test_matrix_core_layer_against_oracle(fmt, N, K):
+    name = synth.GGUF_NAMES[fmt]
+    bias = ((np.arange(N, dtype=np.float32) % 13) - 6) * np.float32(0.25)
+    data, layer = _layer(fmt, N, K, seed=N + K + fmt, bias=bias)
+    w = oracle.dequantize_gguf(fmt, data, N, K)
+    br = round_x(bias, oracle.BF16)
+    rows = (1, 4, 8, 9, 16, 32) if N == 4096 else (1, 2, 3, 4, 5, 7, 8, 9, 12, 13, 16, 17, 31, 32)
+    for m in rows:
+        say(f"gguf matrix-core {name} N={N} K={K} m={m}")
+        x = np.random.default_rng(K + 3 * m).standard_normal((m, K)).astype(np.float32)
+        xd = to_dev(x, torch.bfloat16)
+        y = layer.forward(xd)
+        plan = ops.default_context().last_plan()
+        mt = 2 if m > 16 else 1
+        assert plan["kernel"] == f"gguf_{TAG[fmt]}_mfma_bf16_mt{mt}" and plan["launches"] == 1, plan
+        assert plan["grid"] == (N // 16, 1, 1), plan
+        assert plan["block"][0] == (512 if (K // 128 < 16 or mt == 2) else 1024), plan
+        xr = round_x(x, oracle.BF16)
+        ref = oracle.matmul_nt_f32(xr, w, br)
+        assert_close(y, ref, f"matrix-core {name} N={N} K={K} m={m}", bf16_out=True)
+        if m > 8:  # what the reference's prefill tiles would give, within the reference's own bound
+            tile = oracle.matmul_nt_f32(xr, oracle.round_through(w, oracle.BF16), br)
+            assert np.abs(as_f32(y) - tile).max() < 0.06 * np.abs(tile).max() + 1e-2
+        assert np.array_equal(bits_of(layer.forward(xd)), bits_of(y)), "run to run"
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+def test_rows_do_not_depend_on_the_batch(fmt):
+    """A row's result is the same bits at every row count up to 32: alone, among 8, among 16 (one row tile), among
+    32 (two row tiles; the same chunks per wave only where the workgroup has as many waves, so K is short here)."""
+    N, K = 64, 1024
+    data, layer = _layer(fmt, N, K, seed=21 + fmt)
+    x = np.random.default_rng(22).standard_normal((32, K)).astype(np.float32)
+    xd = to_dev(x, torch.bfloat16)
+    y32 = bits_of(layer.forward(xd))
+    y16 = bits_of(layer.forward(xd[:16].contiguous()))
+    y8 = bits_of(layer.forward(xd[:8].contiguous()))
+    np.testing.assert_array_equal(y16, y32[:16])
+    np.testing.assert_array_equal(y8, y32[:8])
+    for r in (0, 3, 7, 15, 31):
+        say(f"gguf matrix-core {synth.GGUF_NAMES[fmt]} row {r} alone")
+        y1 = bits_of(layer.forward(xd[r:r + 1].contiguous()))
+        np.testing.assert_array_equal(y1[0], y32[r])
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+def test_switches_and_rows_beyond_the_kernel(fmt):
+    """More than 32 rows go to the tile matmul on the file layout; OXQ_GGUF_MFMA_MAX_M moves that bound;
+    OXQ_GGUF_MFMA = 0 builds the rotated copy of the vector GEMV instead (1 - 4 rows)."""
+    from tests.test_gpu_gguf_mxfp4 import _check_mul_mm
+    N, K = 96, 512
+    data, layer = _layer(fmt, N, K, seed=31 + fmt)
+    w = oracle.dequantize_gguf(fmt, data, N, K)
+    x = np.random.default_rng(32).standard_normal((40, K)).astype(np.float32)
+    say(f"gguf matrix-core {synth.GGUF_NAMES[fmt]}: 40 rows")
+    y = layer.forward(to_dev(x, torch.bfloat16))
+    assert "_mul_mm_" in ops.default_context().last_plan()["kernel"]
+    _check_mul_mm(y, x, w, "40 rows")
+    tune("OXQ_GGUF_MFMA_MAX_M", 8)
+    say(f"gguf matrix-core {synth.GGUF_NAMES[fmt]}: bound moved to 8")
+    y = layer.forward(to_dev(x[:9], torch.bfloat16))
+    assert "_mul_mm_" in ops.default_context().last_plan()["kernel"]
+    _check_mul_mm(y, x[:9], w, "9 rows with the bound at 8")
+    y = layer.forward(to_dev(x[:8], torch.bfloat16))
+    assert "_mfma_bf16_mt1" in ops.default_context().last_plan()["kernel"]
+    tune("OXQ_GGUF_MFMA_MAX_M", None)
+    tune("OXQ_GGUF_MFMA", 0)
+    say(f"gguf matrix-core {synth.GGUF_NAMES[fmt]}: switched off")
+    rot = ops.QLinear(fmt, to_dev(data), K, N, None, torch.bfloat16)
+    tune("OXQ_GGUF_MFMA", None)
+    assert rot.resident
+    y4 = rot.forward(to_dev(x[:4], torch.bfloat16))
+    assert "_res_gemv_bf16" in ops.default_context().last_plan()["kernel"]
+    ref = oracle.matmul_nt_f32(round_x(x[:4], oracle.BF16), w)
+    assert_close(y4, ref, "rotated copy of a bf16 layer", bf16_out=True)
+    assert_close(layer.forward(to_dev(x[:4], torch.bfloat16)), ref, "matrix-core copy, the same rows", bf16_out=True)
+    assert np.array_equal(rot.dequantize().cpu().numpy().view(np.uint32), layer.dequantize().cpu().numpy().view(np.uint32))
+
+
+def test_f32_layers_keep_the_rotated_copy():
+    """f32 activations are the reference's CPU contract (linear.rs:357-372): exact f32 arithmetic on the vector ALU."""
+    fmt, N, K = synth.GGUF_Q4_K, 64, 512
+    data = synth.gguf_weight(fmt, N, K, seed=41)
+    layer = ops.QLinear(fmt, to_dev(data), K, N, None, torch.float32)
+    x = np.random.default_rng(42).standard_normal((2, K)).astype(np.float32)
+    y = layer.forward(to_dev(x))
+    assert "_res_gemv_f32" in ops.default_context().last_plan()["kernel"]
+    assert not gguf_on_matrix_cores(fmt, N, K, 2, bf16=False)
+    assert_close(y, oracle.matmul_nt_f32(x, oracle.dequantize_gguf(fmt, data, N, K)), "f32 layer")
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+def test_matrix_core_layer_replays_in_a_graph(fmt):
+    N, K = 256, 2048
+    say(f"gguf matrix-core graph replay {synth.GGUF_NAMES[fmt]}")
+    data, layer = _layer(fmt, N, K, seed=51 + fmt)
+    x = torch.randn((6, K), device="cuda", dtype=torch.bfloat16)
+    y = torch.empty((6, N), device="cuda", dtype=torch.bfloat16)
+    layer.forward(x, out=y)
+    stream = torch.cuda.Stream()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=stream):
+        layer.forward(x, out=y)
+    gen = torch.Generator(device="cuda")
+    for i in range(1, 4):
+        gen.manual_seed(i)
+        x.copy_(torch.randn((6, K), device="cuda", generator=gen).to(torch.bfloat16))
+        layer.forward(x, out=y)
+        torch.cuda.synchronize()
+        want = bits_of(y).copy()
+        y.zero_()
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(bits_of(y), want), f"replay {i}"

@@ -16,7 +16,7 @@ import torch
 import oracle
 from oxydllm_amd import synth
 from tests import refgen
-from tests.helpers import RTOL, ATOL, as_f32, assert_close, bits_of, round_x, to_dev, tune
+from tests.helpers import RTOL, ATOL, as_f32, assert_close, bits_of, gguf_on_matrix_cores, round_x, to_dev, tune
 
 pytestmark = pytest.mark.gpu
 ops = None
@@ -214,12 +214,12 @@ def test_qlinear_layer_bias_and_routing():
     w = oracle.dequantize_gguf(fmt, data, N, K)
     bias = np.linspace(-1, 1, N).astype(np.float32)
     layer = ops.QLinear(fmt, to_dev(data), K, N, to_dev(bias, torch.bfloat16), torch.bfloat16)
-    for shape in [(1, K), (2, 4, K), (3, 5, K)]:
+    for shape in [(1, K), (2, 4, K), (3, 5, K), (5, 8, K)]:
         m = int(np.prod(shape[:-1]))
         x = np.random.default_rng(m).standard_normal((m, K)).astype(np.float32)
         y = layer.forward(to_dev(x.reshape(shape), torch.bfloat16))
         assert tuple(y.shape) == shape[:-1] + (N,)
-        if m <= 8:
+        if m <= 8 or gguf_on_matrix_cores(fmt, N, K, m):  # the matrix-core copy keeps the GEMV's unrounded weights
             ref = oracle.matmul_nt_f32(round_x(x, oracle.BF16), w, round_x(bias, oracle.BF16))
             assert_close(y.reshape(m, N), ref, f"QLinear {shape}")
         else:  # prefill: the tile matmul

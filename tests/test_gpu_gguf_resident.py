@@ -1,9 +1,10 @@
 """Resident GGUF layers (QLinear's strip-major copy of the block bytes) through the C ABI.
 
 oxq_qlinear_new repacks the weights of all ten block formats into strips of 16 rows at load
-(linear.rs:225-240 copies the bytes at build); 1 - 4 rows of x then run on that copy.  The repack is
-pinned bit for bit: the dense dequant read back from the copy must equal the oracle's dequantize_gguf
-of the file's bytes.  The GEMV on the copy is held to the f32-accumulated oracle within 2e-3 relative /
+(linear.rs:225-240 copies the bytes at build); 1 - 4 rows of x then run on that copy.  A bf16 layer of
+Q4_0, Q8_0, Q4_K or Q6_K takes the matrix-core layout instead (tests/test_gpu_gguf_mfma.py), on which up
+to 32 rows run.  Either repack is pinned bit for bit: the dense dequant read back from the copy must equal
+the oracle's dequantize_gguf of the file's bytes.  The GEMV on the copy is held to the f32-accumulated oracle within 2e-3 relative /
 1e-2 absolute (plus half a bf16 ulp for bf16 outputs), with f32 and bf16 activations, with and without
 bias, on the benchmark's configuration 3, on long and ragged K, and is compared with the kernels on the
 file layout; shapes outside the copy's reach and more than 4 rows keep those kernels.
@@ -16,7 +17,7 @@ import torch
 
 import oracle
 from oxydllm_amd import synth
-from tests.helpers import assert_close, bits_of, round_x, to_dev, tune
+from tests.helpers import assert_close, bits_of, gguf_on_matrix_cores, round_x, to_dev, tune
 
 pytestmark = pytest.mark.gpu
 ops = None
@@ -38,14 +39,17 @@ def say(msg):
 
 
 @pytest.mark.parametrize("fmt", FMTS)
+@pytest.mark.parametrize("tdt", [torch.float32, torch.bfloat16], ids=["rotated", "bf16-layer"])
 @pytest.mark.parametrize("N,K", [(16, 256), (48, 1024), (160, 2304), (32, 4096)])
-def test_resident_copy_dequantizes_bit_exact(fmt, N, K):
-    say(f"resident gguf dequant {synth.GGUF_NAMES[fmt]} N={N} K={K}")
+def test_resident_copy_dequantizes_bit_exact(fmt, tdt, N, K):
+    say(f"resident gguf dequant {synth.GGUF_NAMES[fmt]} N={N} K={K} {tdt}")
     data = synth.gguf_weight(fmt, N, K, seed=7 * N + K + fmt)
-    layer = ops.QLinear(fmt, to_dev(data), K, N, None, torch.float32)
+    layer = ops.QLinear(fmt, to_dev(data), K, N, None, tdt)
     assert layer.resident
     want = oracle.dequantize_gguf(fmt, data, N, K)
     got = layer.dequantize().cpu().numpy()
+    kernel = ops.default_context().last_plan()["kernel"]
+    assert ("_mfma_dequant" in kernel) == gguf_on_matrix_cores(fmt, N, K, 1, tdt == torch.bfloat16), kernel
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), "repack changed a weight"
 
 
@@ -66,7 +70,8 @@ def test_resident_gemv_config3(fmt, act):
     assert layer.resident
     y = layer.forward(xd)
     plan = ops.default_context().last_plan()
-    assert "_res_gemv_" in plan["kernel"] and plan["launches"] == 1 and plan["grid"][0] == N // 16, plan
+    tag = "_mfma_bf16_mt1" if gguf_on_matrix_cores(fmt, N, K, 1, act == "bf16") else "_res_gemv_"
+    assert tag in plan["kernel"] and plan["launches"] == 1 and plan["grid"][0] == N // 16, plan
     assert y.shape == (1, N) and y.dtype == tdt
     assert_close(y, oracle.matmul_nt_f32(xr, w), f"resident {synth.GGUF_NAMES[fmt]} {act}", bf16_out=act == "bf16")
     y0 = ops.gguf_quant_matmul(xd, wd, K, N, fmt)
@@ -92,8 +97,11 @@ def test_resident_gemv_rows_bias_and_shapes(fmt):
                 xr = round_x(x, dt) if dt is not None else x
                 y = layer.forward(to_dev(x, tdt))
                 kernel = ops.default_context().last_plan()["kernel"]
-                on_copy = "_res_gemv_" in kernel
-                assert on_copy == (m <= ROWS or (m <= 8 and dt is None)), (kernel, m, K)
+                if gguf_on_matrix_cores(fmt, N, K, m, dt is not None):
+                    assert "_mfma_bf16_mt1" in kernel, (kernel, m, K)
+                else:
+                    on_copy = "_res_gemv_" in kernel
+                    assert on_copy == (m <= ROWS or (m <= 8 and dt is None)), (kernel, m, K)
                 assert_close(y, oracle.matmul_nt_f32(xr, w, br), f"resident {name} N={N} K={K} m={m}",
                              bf16_out=dt is not None)
 
