@@ -248,8 +248,8 @@ template <int FMT> struct GgmChunk {
 
     // c: the chunk's index in its strip
     template <typename RS>
-    __device__ __forceinline__ void request(const RS &rs, int lane, int ni, int c) {
-        const int blk = (c / F::CH) * L::BLKB, soff = blk + (c % F::CH) * L::CHB;
+    __device__ __forceinline__ void request(const RS &rs, int lane, int ni, int c, int strip_off) {
+        const int blk = strip_off + (c / F::CH) * L::BLKB, soff = blk + (c % F::CH) * L::CHB;
         // headers first: the factors and the minimum's term are worked out while the quants are on their way
         if constexpr (F::UH == 8) {
             const u32x2_t v = __builtin_amdgcn_raw_buffer_load_b64(rs, ni * 8, soff + L::UH_OFF, 2);
@@ -273,8 +273,10 @@ template <int FMT> struct GgmChunk {
     __device__ __forceinline__ void factors(int half, int ni, float (&f0)[NSTEP], float (&f1)[NSTEP]) const {
         if constexpr (FMT == OXQ_GGUF_Q4_K) {
             // get_scale_min_k4 (quant_kernels.metal:2438-2450) for the chunk's four sub-blocks at once, a byte each
-            const uint32_t sc4 = half ? ((bh[3] & 0x0F0F0F0Fu) | ((bh[1] >> 2) & 0x30303030u)) : (bh[1] & 0x3F3F3F3Fu);
-            const uint32_t mn4 = half ? (((bh[3] >> 4) & 0x0F0F0F0Fu) | ((bh[2] >> 2) & 0x30303030u)) : (bh[2] & 0x3F3F3F3Fu);
+            // (selected by mask: as a branch on the chunk's parity the two sides kept twice the registers alive)
+            const uint32_t hm = half ? 0xFFFFFFFFu : 0u;
+            const uint32_t sc4 = (((bh[3] & 0x0F0F0F0Fu) | ((bh[1] >> 2) & 0x30303030u)) & hm) | (bh[1] & 0x3F3F3F3Fu & ~hm);
+            const uint32_t mn4 = ((((bh[3] >> 4) & 0x0F0F0F0Fu) | ((bh[2] >> 2) & 0x30303030u)) & hm) | (bh[2] & 0x3F3F3F3Fu & ~hm);
             const float d = ggm_f16(bh[0] & 0xFFFFu), dm = ggm_f16(bh[0] >> 16) * 0.0078125f;  // dmin / 128
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
@@ -317,7 +319,7 @@ __device__ __forceinline__ float4_t ggm_mfma16(uint32_t a0, uint32_t a1, uint32_
                                                      __builtin_bit_cast(short4_t, u32x2_t{b0, b1}), c, 0, 0, 0);
 }
 
-template <int FMT, int MT, int XQ, int NW>
+template <int FMT, int MT, int XQ, int NW, int NS>
 __global__ __launch_bounds__(NW * 64) void ggm_kernel(const uint16_t *__restrict__ x, const uint8_t *__restrict__ pw,
                                                       const uint16_t *__restrict__ bias, uint16_t *__restrict__ y,
                                                       float *__restrict__ ws, int M, int K, int N, int cslice) {
@@ -329,7 +331,7 @@ __global__ __launch_bounds__(NW * 64) void ggm_kernel(const uint16_t *__restrict
     constexpr int ROWS = 16 * MT, AQ = XQ, SLOT = ROWS * 256, OOB = 0x7FFFFF00, NSTEP = C::NSTEP;
     // chunks in flight a wave: three, two where block headers and factors take the registers (measured on
     // 4096 x 4096 at one row, Q8_0: 5.06 us with three, 5.87 with two)
-    constexpr int RD = FMT == OXQ_GGUF_Q4_K ? 2 : 3;
+    constexpr int RD = NS > 1 ? 2 : 3;
     constexpr bool K16 = NSTEP == 8;  // steps of 16 elements
     extern __shared__ __attribute__((aligned(16))) unsigned char pk4_lds[];
 
@@ -346,8 +348,9 @@ __global__ __launch_bounds__(NW * 64) void ggm_kernel(const uint16_t *__restrict
     const int cc0 = sc0 + wave * cbase + min(wave, crem);
     unsigned char *slot = pk4_lds + wave * SLOT;
 
+    // the workgroup's NS neighbouring strips behind one descriptor (NS * strip_bytes < 2^31: checked on the host)
     const uint32_t strip_bytes = (uint32_t)(NC / F::CH) * (uint32_t)L::BLKB;
-    const __amdgpu_buffer_rsrc_t rs_w = make_rsrc(pw + (size_t)j * strip_bytes, strip_bytes);
+    const __amdgpu_buffer_rsrc_t rs_w = make_rsrc(pw + (size_t)j * NS * strip_bytes, NS * strip_bytes);
     const int xrows = min(M - m0, ROWS);
     const __amdgpu_buffer_rsrc_t rs_x = make_rsrc(x + (size_t)m0 * K, (uint32_t)xrows * (uint32_t)K * 2u);
     const __amdgpu_buffer_rsrc_t rs_none = make_rsrc(pw, 0u);
@@ -374,23 +377,26 @@ __global__ __launch_bounds__(NW * 64) void ggm_kernel(const uint16_t *__restrict
         *(u32x4_t *)(slot + row * 256 + ((ni ^ (row & 15)) << 4)) = u32x4_t{0u, 0u, 0u, 0u};
     }
 
-    C wr[RD];
+    C wr[RD][NS];
     u32x4_t ar[RD][AQ];
-    auto request = [&](int i, C &w, u32x4_t (&a)[AQ]) {
+    auto request = [&](int i, C (&w)[NS], u32x4_t (&a)[AQ]) {
         const bool live = i < nloc;  // wave-uniform
         const __amdgpu_buffer_rsrc_t rx = live ? rs_x : rs_none, rw = live ? rs_w : rs_none;
         const int c = cc0 + i;
 #pragma unroll
         for (int q = 0; q < AQ; ++q) a[q] = __builtin_amdgcn_raw_buffer_load_b128(rx, voff_a[q], c * 256, 0);
-        w.request(rw, lane, ni, c);
+#pragma unroll
+        for (int f = 0; f < NS; ++f) w[f].request(rw, lane, ni, c, (int)(f * strip_bytes));
         __builtin_amdgcn_sched_barrier(0);  // chunks are requested in the order they are used
     };
 #pragma unroll
     for (int d = 0; d < RD; ++d) request(d, wr[d], ar[d]);
 
-    float4_t acc[MT][1];
+    float4_t acc[MT][NS];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) acc[mt][0] = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int f = 0; f < NS; ++f) acc[mt][f] = float4_t{0.f, 0.f, 0.f, 0.f};
     const uint32_t neg[4] = {F::NEG, F::NEG, F::NEG, F::NEG};
     const float4_t zero4 = float4_t{0.f, 0.f, 0.f, 0.f};
 
@@ -411,13 +417,12 @@ __global__ __launch_bounds__(NW * 64) void ggm_kernel(const uint16_t *__restrict
 
     auto chunk = [&](int i, auto cur_c, bool more) {
         constexpr int CUR = decltype(cur_c)::value;
-        C &w = wr[CUR];
 #pragma unroll
         for (int q = 0; q < AQ; ++q) *(u32x4_t *)(slot + q * 1024 + a_wr[q & 3]) = ar[CUR][q];
         float f0[NSTEP], f1[NSTEP];
         if constexpr (MT == 1) {
             // what depends on x alone first (x is requested ahead of the chunk's quants): the operands and the
-            // bias term of four steps, so that one MFMA a step is left when the quants arrive
+            // bias term of four steps, so that one MFMA a step and strip is left when the quants arrive
 #pragma unroll
             for (int g = 0; g < NSTEP; g += 4) {
                 uint32_t a[4][4];
@@ -427,23 +432,30 @@ __global__ __launch_bounds__(NW * 64) void ggm_kernel(const uint16_t *__restrict
                     load_a(g + s4, 0, a[s4]);
                     tn[s4] = mma(a[s4], neg, zero4);
                 }
-                if (g == 0) w.factors((cc0 + i) & 1, ni, f0, f1);
-                if constexpr (C::HAS_MIN) {
 #pragma unroll
-                    for (int s4 = 0; s4 < 4; ++s4)
+                for (int f = 0; f < NS; ++f) {
+                    const C &w = wr[CUR][f];
+                    if (g == 0 || NS > 1) w.factors((cc0 + i) & 1, ni, f0, f1);
+                    if constexpr (C::HAS_MIN) {
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) acc[0][0][e] = fmaf(f1[g + s4], tn[s4][e], acc[0][0][e]);
-                }
+                        for (int s4 = 0; s4 < 4; ++s4)
 #pragma unroll
-                for (int s4 = 0; s4 < 4; ++s4) {
-                    uint32_t b[4];
-                    w.operand(g + s4, b, nm);
-                    const float4_t t = mma(a[s4], b, tn[s4]);
+                            for (int e = 0; e < 4; ++e) acc[0][f][e] = fmaf(f1[g + s4], tn[s4][e], acc[0][f][e]);
+                    }
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) acc[0][0][e] = fmaf(f0[g + s4], t[e], acc[0][0][e]);
+                    for (int s4 = 0; s4 < 4; ++s4) {
+                        uint32_t b[4];
+                        w.operand(g + s4, b, nm);
+                        const float4_t t = mma(a[s4], b, tn[s4]);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) acc[0][f][e] = fmaf(f0[g + s4], t[e], acc[0][f][e]);
+                    }
+                    if constexpr (NS > 1) __builtin_amdgcn_sched_barrier(0);  // one strip's operands at a time
                 }
             }
         } else {  // more row tiles: step by step, the registers do not hold a chunk's operands
+            static_assert(MT == 1 || NS == 1, "two row tiles take one strip");
+            const C &w = wr[CUR][0];
             w.factors((cc0 + i) & 1, ni, f0, f1);
 #pragma unroll
             for (int st = 0; st < NSTEP; ++st) {
@@ -484,7 +496,7 @@ __global__ __launch_bounds__(NW * 64) void ggm_kernel(const uint16_t *__restrict
             if (i + 1 < nloc) chunk(i + 1, std::integral_constant<int, 1>{}, false);
         }
     }
-    pk4n_epilogue<TT, MT, 1, NW>(acc, bias, y, ws, M, N, j, m0, wave, lane);
+    pk4n_epilogue<TT, MT, NS, NW>(acc, bias, y, ws, M, N, j, m0, wave, lane);
 }
 
 // ---------------------------------------------------------------------------
@@ -543,50 +555,73 @@ int launch_gguf_mfma_dequant(oxq_ctx *ctx, hipStream_t s, int quant, const void 
     return OXQ_OK;
 }
 
-template <int FMT, int MT, int XQ, int NW>
+template <int FMT, int MT, int XQ, int NW, int NS>
 static int ggm_go(hipStream_t s, dim3 grid, const GgufProblem &p, float *ws, int cslice) {
     static LdsGrant lds_grant;  // one per instantiation
     const size_t lds = (size_t)NW * MT * 4096;
-    OXQ_HIP_CHECK(lds_grant.ensure((const void *)ggm_kernel<FMT, MT, XQ, NW>, lds));
-    hipLaunchKernelGGL((ggm_kernel<FMT, MT, XQ, NW>), grid, dim3(NW * 64), lds, s, (const uint16_t *)p.x, p.w,
+    OXQ_HIP_CHECK(lds_grant.ensure((const void *)ggm_kernel<FMT, MT, XQ, NW, NS>, lds));
+    hipLaunchKernelGGL((ggm_kernel<FMT, MT, XQ, NW, NS>), grid, dim3(NW * 64), lds, s, (const uint16_t *)p.x, p.w,
                        (const uint16_t *)p.bias, (uint16_t *)p.y, ws, (int)p.M, (int)p.K, (int)p.N, cslice);
     OXQ_HIP_CHECK(hipGetLastError());
     return OXQ_OK;
 }
-template <int FMT, int NW>
-static int ggm_by_rows(hipStream_t s, dim3 grid, const GgufProblem &p, float *ws, int cslice, int mt, int xq) {
-    if (mt == 2) return ggm_go<FMT, 2, 8, NW>(s, grid, p, ws, cslice);
-    if (xq == 1) return ggm_go<FMT, 1, 1, NW>(s, grid, p, ws, cslice);
-    if (xq == 2) return ggm_go<FMT, 1, 2, NW>(s, grid, p, ws, cslice);
-    return ggm_go<FMT, 1, 4, NW>(s, grid, p, ws, cslice);
+template <int FMT>
+static int ggm_by_shape(hipStream_t s, dim3 grid, const GgufProblem &p, float *ws, int cslice, int mt, int xq, int nw, int ns) {
+    if (ns == 4) {  // 8 waves: four strips' quants in flight take the registers of two waves of a 16-wave workgroup
+        if (xq == 1) return ggm_go<FMT, 1, 1, 8, 4>(s, grid, p, ws, cslice);
+        if (xq == 2) return ggm_go<FMT, 1, 2, 8, 4>(s, grid, p, ws, cslice);
+        return ggm_go<FMT, 1, 4, 8, 4>(s, grid, p, ws, cslice);
+    }
+    if (mt == 2) return ggm_go<FMT, 2, 8, 8, 1>(s, grid, p, ws, cslice);
+    if (nw == 8) {
+        if (xq == 1) return ggm_go<FMT, 1, 1, 8, 1>(s, grid, p, ws, cslice);
+        if (xq == 2) return ggm_go<FMT, 1, 2, 8, 1>(s, grid, p, ws, cslice);
+        return ggm_go<FMT, 1, 4, 8, 1>(s, grid, p, ws, cslice);
+    }
+    if (xq == 1) return ggm_go<FMT, 1, 1, 16, 1>(s, grid, p, ws, cslice);
+    if (xq == 2) return ggm_go<FMT, 1, 2, 16, 1>(s, grid, p, ws, cslice);
+    return ggm_go<FMT, 1, 4, 16, 1>(s, grid, p, ws, cslice);
 }
 
-// rows of x a launch of the matrix-core kernel takes (more go to the tile matmul on the file layout)
-bool gguf_mfma_takes(const oxq_ctx *ctx, int64_t M, int act_dtype) {
-    return act_dtype == OXQ_BF16 && M >= 1 && M <= tune(ctx, OXQ_TUNE_GGUF_MFMA_MAX_M, 32);
+// A wide layer (768 strips or more) gives a workgroup four neighbouring strips: every strip of a workgroup re-reads
+// the rows of x, which outweighs the weights from a few rows on, and 224 workgroups of 64 columns fill the chip
+// as 896 of 16 do not (three and a half rounds).
+static int ggm_strips(const oxq_ctx *ctx, int64_t N) {
+    const int v = tune(ctx, OXQ_TUNE_GGUF_MFMA_NS, 0);
+    if (v == 1 || v == 4) return (N / 16) % v == 0 ? v : 1;
+    return (N / 16 >= 768 && (N / 16) % 4 == 0) ? 4 : 1;
+}
+
+// rows of x a launch of the matrix-core kernel takes (more go to the tile matmul on the file layout): 32, 16 where
+// a workgroup takes four strips (two row tiles of four strips do not fit the registers)
+bool gguf_mfma_takes(const oxq_ctx *ctx, int64_t M, int64_t N, int act_dtype) {
+    const int64_t cap = ggm_strips(ctx, N) == 4 ? 16 : 32;
+    return act_dtype == OXQ_BF16 && M >= 1 && M <= std::min<int64_t>(cap, tune(ctx, OXQ_TUNE_GGUF_MFMA_MAX_M, 32));
 }
 
 // p.w is the matrix-core copy
 int launch_gguf_mfma(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p) {
+    const int ns = p.M <= 16 ? ggm_strips(ctx, p.N) : 1;
     const int mt = p.M > 16 ? 2 : 1;
     const int rows = (int)std::min<int64_t>(p.M, 16 * mt);
     const int xq = rows <= 4 ? 1 : rows <= 8 ? 2 : 4;
     // two row tiles need more than the 128 registers a wave of a 16-wave workgroup has
-    const int nw = (p.K / 128 < 16 || mt == 2) ? 8 : 16;
-    dim3 grid((unsigned)(p.N / 16), 1, (unsigned)ceil_div(p.M, (int64_t)16 * mt));
+    const int nw = (p.K / 128 < 16 || mt == 2 || ns == 4) ? 8 : 16;
+    dim3 grid((unsigned)(p.N / (16 * ns)), 1, (unsigned)ceil_div(p.M, (int64_t)16 * mt));
     char name[64];
-    snprintf(name, sizeof name, "gguf_%s_mfma_bf16_mt%d", ggm_name(p.quant), mt);
+    snprintf(name, sizeof name, "gguf_%s_mfma_bf16_mt%d%s", ggm_name(p.quant), mt, ns == 4 ? "_n64" : "");
     set_plan(ctx, name, grid, dim3(nw * 64), 1, 1, 0);
     if (ctx->plan_only) return OXQ_OK;
     if (p.act_dtype != OXQ_BF16) return fail(OXQ_ERR_UNSUPPORTED, "gguf matrix-core matmul: activations must be BF16");
     if ((uintptr_t)p.x & 15) return fail(OXQ_ERR_UNSUPPORTED, "gguf matrix-core matmul: x must be 16-byte aligned");
     if ((uint64_t)16 * mt * (uint64_t)p.K * 2 >= (1ull << 31)) return fail(OXQ_ERR_UNSUPPORTED, "gguf matrix-core matmul: K too large");
+    if (gguf_res_bytes(p.quant, p.K, 16) * (uint64_t)ns >= (1ull << 31)) return fail(OXQ_ERR_UNSUPPORTED, "gguf matrix-core matmul: K too large");
     const int cslice = (int)(p.K / 128);
     switch (p.quant) {
-    case OXQ_GGUF_Q4_0: return nw == 8 ? ggm_by_rows<OXQ_GGUF_Q4_0, 8>(s, grid, p, nullptr, cslice, mt, xq) : ggm_by_rows<OXQ_GGUF_Q4_0, 16>(s, grid, p, nullptr, cslice, mt, xq);
-    case OXQ_GGUF_Q8_0: return nw == 8 ? ggm_by_rows<OXQ_GGUF_Q8_0, 8>(s, grid, p, nullptr, cslice, mt, xq) : ggm_by_rows<OXQ_GGUF_Q8_0, 16>(s, grid, p, nullptr, cslice, mt, xq);
-    case OXQ_GGUF_Q4_K: return nw == 8 ? ggm_by_rows<OXQ_GGUF_Q4_K, 8>(s, grid, p, nullptr, cslice, mt, xq) : ggm_by_rows<OXQ_GGUF_Q4_K, 16>(s, grid, p, nullptr, cslice, mt, xq);
-    case OXQ_GGUF_Q6_K: return nw == 8 ? ggm_by_rows<OXQ_GGUF_Q6_K, 8>(s, grid, p, nullptr, cslice, mt, xq) : ggm_by_rows<OXQ_GGUF_Q6_K, 16>(s, grid, p, nullptr, cslice, mt, xq);
+    case OXQ_GGUF_Q4_0: return ggm_by_shape<OXQ_GGUF_Q4_0>(s, grid, p, nullptr, cslice, mt, xq, nw, ns);
+    case OXQ_GGUF_Q8_0: return ggm_by_shape<OXQ_GGUF_Q8_0>(s, grid, p, nullptr, cslice, mt, xq, nw, ns);
+    case OXQ_GGUF_Q4_K: return ggm_by_shape<OXQ_GGUF_Q4_K>(s, grid, p, nullptr, cslice, mt, xq, nw, ns);
+    case OXQ_GGUF_Q6_K: return ggm_by_shape<OXQ_GGUF_Q6_K>(s, grid, p, nullptr, cslice, mt, xq, nw, ns);
     default: return fail(OXQ_ERR_UNSUPPORTED, "gguf matrix-core matmul: format %d", p.quant);
     }
 }

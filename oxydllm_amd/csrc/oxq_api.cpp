@@ -843,7 +843,7 @@ static bool wcache_forward(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p, i
 static bool wcache_forward_gguf(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p, int *rc) {
     if (!ctx->wcache_limit || ctx->plan_only || !gguf_res_eligible(p.quant, p.K, p.N)) return false;
     const bool mfma = p.act_dtype == OXQ_BF16 && gguf_mfma_eligible(ctx, p.quant, p.K, p.N);
-    if (!(mfma ? gguf_mfma_takes(ctx, p.M, p.act_dtype) : gguf_res_takes(p.K, p.M, p.act_dtype))) return false;
+    if (!(mfma ? gguf_mfma_takes(ctx, p.M, p.N, p.act_dtype) : gguf_res_takes(p.K, p.M, p.act_dtype))) return false;
     const int kind = mfma ? -2 : -1;
     if (((uintptr_t)p.x & 15) || ((uintptr_t)p.w & 1)) return false;
     if (!ctx->wcache) {
@@ -2184,7 +2184,7 @@ int oxq_qlinear_forward(oxq_qlinear *l, void *stream, const oxq_tensor *x, const
                        &l->weight_bytes, l->in_features, l->out_features, l->quant, &o2, &p));
     p.bias = l->has_bias ? l->bias.data : nullptr;
     if (l->resident && l->mfma) {
-        if (gguf_mfma_takes(l->ctx, p.M, p.act_dtype) && ((uintptr_t)p.x & 15) == 0) {
+        if (gguf_mfma_takes(l->ctx, p.M, p.N, p.act_dtype) && ((uintptr_t)p.x & 15) == 0) {
             p.w = (const uint8_t *)l->res;
             return launch_gguf_mfma(l->ctx, (hipStream_t)stream, p);
         }
