@@ -195,6 +195,19 @@ def run(ops, ctx, stream, steps, warmup, time_graph, with_cpu=True):
         rows.append(rr)
         rows.append(r)
         del layers
+        # bf16 activations (the reference's GPU contract, linear.rs:250-284): a bf16 layer keeps the matrix-core
+        # copy of the four formats; 1, 8 (the decode op's limit) and 16 rows
+        layers = [ops.QLinear(fmt, d[i], K, N, None, torch.bfloat16, ctx=ctx) for i in range(nc)]
+        for m in (1, 8, 16):
+            xb = torch.randn((m, K), device=dev, dtype=torch.bfloat16)
+            yb = torch.empty((m, N), device=dev, dtype=torch.bfloat16)
+            rb = _row("cfg3", f"gguf {synth.GGUF_NAMES[fmt]} M={m} K={K} N={N} bf16 activations, QLinear.forward (resident "
+                              "matrix-core copy of the blocks)",
+                      lambda i, layers=layers, nc=nc, xb=xb, yb=yb: layers[i % nc].forward(xb, out=yb), steps, warmup, stream,
+                      time_graph, data.nbytes + m * (K + N) * 2, 2.0 * m * K * N, ctx)
+            rb["bare_read_nt_us"] = r["bare_read_nt_us"]
+            rows.append(rb)
+        del layers
         rc = _cached_row("cfg3", f"gguf {synth.GGUF_NAMES[fmt]} M=1 K={K} N={N} f32 activations, gguf_quant_matmul op "
                                  "with the ctx weight cache on",
                          lambda c, d=d, fmt=fmt: ops.gguf_quant_matmul(x, d[c], K, N, fmt, out=y, ctx=ctx),

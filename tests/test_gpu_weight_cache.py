@@ -209,6 +209,38 @@ def test_cached_gguf_op_equals_the_resident_layer(fmt):
         ctx.close()
 
 
+@pytest.mark.parametrize("fmt", [synth.GGUF_Q4_0, synth.GGUF_Q8_0, synth.GGUF_Q4_K, synth.GGUF_Q6_K])
+def test_cached_gguf_op_with_bf16_activations_runs_on_the_matrix_core_copy(fmt):
+    """bf16 activations: the cache holds the matrix-core copy of a bf16 QLinear; the decode op (1 - 8 rows) and the
+    prefill op (up to 32 rows) run on it with the layer's bits.  f32 calls on the same bytes keep the rotated copy:
+    two entries."""
+    N, K = 64, 1024
+    data = synth.gguf_weight(fmt, N, K, seed=95 + fmt)
+    wd = to_dev(data)
+    w = oracle.dequantize_gguf(fmt, data, N, K)
+    layer = ops.QLinear(fmt, wd, K, N, None, torch.bfloat16)
+    nbytes = (data.size + 255) // 256 * 256
+    ctx = ops.Context()
+    try:
+        ctx.set_weight_cache(1 << 22)
+        for m, op in [(1, ops.gguf_quant_matmul), (8, ops.gguf_quant_matmul), (9, ops.gguf_quant_mul_mm), (32, ops.gguf_quant_mul_mm)]:
+            say(f"weight cache gguf bf16 {synth.GGUF_NAMES[fmt]} m={m}")
+            x = np.random.default_rng(m).standard_normal((m, K)).astype(np.float32)
+            xd = to_dev(x, torch.bfloat16)
+            y = op(xd, wd, K, N, fmt, ctx=ctx)
+            assert "_mfma_bf16_mt" in ctx.last_plan()["kernel"], ctx.last_plan()
+            np.testing.assert_array_equal(bits_of(y), bits_of(layer.forward(xd)))
+            assert_close(y, oracle.matmul_nt_f32(round_x(x, oracle.BF16), w), f"cached gguf bf16 op m={m}", bf16_out=True)
+        assert ctx.weight_cache_usage() == (nbytes, 1)
+        ops.gguf_quant_mul_mm(to_dev(x[:1].repeat(33, 0), torch.bfloat16), wd, K, N, fmt, ctx=ctx)
+        assert "_mul_mm_" in ctx.last_plan()["kernel"]  # more rows than the kernel takes: the file layout
+        ops.gguf_quant_matmul(to_dev(x[:2]), wd, K, N, fmt, ctx=ctx)
+        assert "_res_gemv_f32" in ctx.last_plan()["kernel"]
+        assert ctx.weight_cache_usage() == (2 * nbytes, 2)
+    finally:
+        ctx.close()
+
+
 def test_capture_allocates_nothing_and_replays_the_cached_kernel():
     K, N, g, m = 2048, 512, 128, 4
     tdt = torch.float16
