@@ -14,6 +14,11 @@
 //                 that one AND-OR per pair yields 128 + q as two bf16) + [16 columns][4 units] f16 d    1152 B
 //   Q8_0  chunk = 2 x [64 lanes][16 B] (plane h = units 2 h, 2 h + 1; bytes of a word: elements 0, 2, 1, 3 of
 //                 its four, stored as q + 128) + [16 columns][4 units] f16 d                             2176 B
+//   Q4_1  as Q4_0, the unit headers are {d, m} pairs                                                     1280 B
+//   Q5_0  as Q4_0 + [64 lanes][4 B] of fifth bits: the bit of element 2 pp (2 pp + 1) of unit t in bit
+//         4 t + pp (16 + 4 t + pp), so that one shift puts a pair's bits at positions 4 and 20           1408 B
+//   Q5_1  as Q5_0 with {d, m} pairs                                                                      1536 B
+//   Q5_K  as Q4_K with the plane of fifth bits in every chunk                                            2816 B
 //   Q4_K  block = 2 chunks of [64 lanes][16 B] nibbles as Q4_0 + [16 columns] the super-block's first 16
 //                 bytes (d, dmin, 12 scale bytes)                                                        2304 B
 //   Q6_K  block = 2 chunks of { [64 lanes][16 B] low nibbles, [64 lanes][8 B] high bit pairs, [16 columns][8]
@@ -39,13 +44,21 @@ template <int FMT> struct GgmFmt;
 // BH: bytes of block header a column; NEG: the constant that takes bias and offset out (as a bf16 pair)
 template <> struct GgmFmt<OXQ_GGUF_Q4_0> { static constexpr int WQ = 1, CH = 1, UH = 8, BH = 0; static constexpr uint32_t NEG = 0xC308C308u; };  // -136
 template <> struct GgmFmt<OXQ_GGUF_Q8_0> { static constexpr int WQ = 2, CH = 1, UH = 8, BH = 0; static constexpr uint32_t NEG = 0xC300C300u; };  // -128
+template <> struct GgmFmt<OXQ_GGUF_Q4_1> { static constexpr int WQ = 1, CH = 1, UH = 16, BH = 0; static constexpr uint32_t NEG = 0xC300C300u; };  // -128
+template <> struct GgmFmt<OXQ_GGUF_Q5_0> { static constexpr int WQ = 1, CH = 1, UH = 8, BH = 0; static constexpr uint32_t NEG = 0xC310C310u; };  // -144
+template <> struct GgmFmt<OXQ_GGUF_Q5_1> { static constexpr int WQ = 1, CH = 1, UH = 16, BH = 0; static constexpr uint32_t NEG = 0xC300C300u; };  // -128
+template <> struct GgmFmt<OXQ_GGUF_Q5_K> { static constexpr int WQ = 1, CH = 2, UH = 0, BH = 16; static constexpr uint32_t NEG = 0xC300C300u; };  // -128
 template <> struct GgmFmt<OXQ_GGUF_Q4_K> { static constexpr int WQ = 1, CH = 2, UH = 0, BH = 16; static constexpr uint32_t NEG = 0xC300C300u; };  // -128
 template <> struct GgmFmt<OXQ_GGUF_Q6_K> { static constexpr int WQ = 1, CH = 2, UH = 8, BH = 2; static constexpr uint32_t NEG = 0xC320C320u; };  // -160
 
+// formats with a fifth bit; with a minimum beside the scale
+template <int FMT> constexpr bool ggm_fifth_bit = FMT == OXQ_GGUF_Q5_0 || FMT == OXQ_GGUF_Q5_1 || FMT == OXQ_GGUF_Q5_K;
+template <int FMT> constexpr bool ggm_has_min = FMT == OXQ_GGUF_Q4_K || FMT == OXQ_GGUF_Q5_K || FMT == OXQ_GGUF_Q4_1 || FMT == OXQ_GGUF_Q5_1;
+
 template <int FMT> struct GgmLayout {
     typedef GgmFmt<FMT> F;
-    static constexpr int H_OFF = F::WQ * 1024;                                  // Q6_K: the plane of bit pairs
-    static constexpr int UH_OFF = F::WQ * 1024 + (FMT == OXQ_GGUF_Q6_K ? 512 : 0);
+    static constexpr int H_OFF = F::WQ * 1024;                                  // Q6_K: the plane of bit pairs; fifth bits
+    static constexpr int UH_OFF = F::WQ * 1024 + (FMT == OXQ_GGUF_Q6_K ? 512 : ggm_fifth_bit<FMT> ? 256 : 0);
     static constexpr int CHB = UH_OFF + 16 * F::UH;
     static constexpr int BH_OFF = F::CH * CHB;
     static constexpr int BLKB = F::CH * CHB + 16 * F::BH;
@@ -103,23 +116,52 @@ __global__ __launch_bounds__(256) void ggm_repack_kernel(const uint8_t *__restri
             }
             *(u32x4_t *)(chunk + h * 1024 + lane * 16) = u32x4_t{q[0], q[1], q[2], q[3]};
         }
-    } else if constexpr (FMT == OXQ_GGUF_Q4_K) {
+    } else if constexpr (FMT == OXQ_GGUF_Q4_1 || FMT == OXQ_GGUF_Q5_0 || FMT == OXQ_GGUF_Q5_1) {
+        // quant_kernels.metal:709-790, 872-1036: {d (, m)} (, 32 fifth bits), 16 bytes of nibbles as Q4_0
+        constexpr bool MIN = FMT != OXQ_GGUF_Q5_0, FIFTH = FMT != OXQ_GGUF_Q4_1;
+        constexpr int BB = GgufFmt<FMT>::BB, QS = (MIN ? 4 : 2) + (FIFTH ? 4 : 0);
+        uint32_t q[4], hb = 0;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const uint8_t *p = row + (size_t)(4 * c + t) * BB;
+            const uint32_t qh = FIFTH ? (ld16(p + QS - 4) | (ld16(p + QS - 2) << 16)) : 0u;
+            uint32_t v = 0;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int e = 8 * kb + i;
+                const uint32_t nib = e < 16 ? (p[QS + e] & 0xFu) : (p[QS + e - 16] >> 4);
+                v |= nib << (4 * (i >> 1) + 16 * (i & 1));
+                hb |= ((qh >> e) & 1u) << (4 * t + (i >> 1) + 16 * (i & 1));
+            }
+            q[t] = v;
+            if (t == kb) {
+                if constexpr (MIN) *(uint32_t *)(chunk + L::UH_OFF + ni * 16 + t * 4) = ld16(p) | (ld16(p + 2) << 16);
+                else *(uint16_t *)(chunk + L::UH_OFF + ni * 8 + t * 2) = ld16(p);
+            }
+        }
+        *(u32x4_t *)(chunk + lane * 16) = u32x4_t{q[0], q[1], q[2], q[3]};
+        if constexpr (FIFTH) *(uint32_t *)(chunk + L::H_OFF + lane * 4) = hb;
+    } else if constexpr (FMT == OXQ_GGUF_Q4_K || FMT == OXQ_GGUF_Q5_K) {
         // quant_kernels.metal:2438-2482: sub-block sb of the super-block reads byte (sb / 2) * 32 + e of qs, low
-        // nibble if sb is even
-        const uint8_t *p = row + (size_t)(c >> 1) * 144;
-        uint32_t q[4];
+        // nibble if sb is even; Q5_K (1438-1680): its fifth bit is bit sb of byte e of qh
+        constexpr bool FIFTH = FMT == OXQ_GGUF_Q5_K;
+        const uint8_t *p = row + (size_t)(c >> 1) * GgufFmt<FMT>::BB;
+        const uint8_t *qs = p + (FIFTH ? 48 : 16);
+        uint32_t q[4], hb = 0;
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
             const int sb = 4 * (c & 1) + t;
             uint32_t v = 0;
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                const uint32_t byte = p[16 + (sb >> 1) * 32 + 8 * kb + i];
+                const uint32_t byte = qs[(sb >> 1) * 32 + 8 * kb + i];
                 v |= ((sb & 1) ? (byte >> 4) : (byte & 0xFu)) << (4 * (i >> 1) + 16 * (i & 1));
+                if constexpr (FIFTH) hb |= (((uint32_t)p[16 + 8 * kb + i] >> sb) & 1u) << (4 * t + (i >> 1) + 16 * (i & 1));
             }
             q[t] = v;
         }
         *(u32x4_t *)(chunk + lane * 16) = u32x4_t{q[0], q[1], q[2], q[3]};
+        if constexpr (FIFTH) *(uint32_t *)(chunk + L::H_OFF + lane * 4) = hb;
         if ((c & 1) == 0 && kb < 4) *(uint32_t *)(blk + L::BH_OFF + ni * 16 + kb * 4) = ld32a2(p + 4 * kb);
     } else if constexpr (FMT == OXQ_GGUF_Q6_K) {
         // quant_kernels.metal:2518-2554: element j of the super-block, h = j / 128, q = (j % 128) / 32, l = j % 32:
@@ -185,8 +227,25 @@ __global__ __launch_bounds__(256) void ggm_dequant_kernel(const uint8_t *__restr
                 }
             }
         }
-    } else if constexpr (FMT == OXQ_GGUF_Q4_K) {
+    } else if constexpr (FMT == OXQ_GGUF_Q4_1 || FMT == OXQ_GGUF_Q5_0 || FMT == OXQ_GGUF_Q5_1) {
+        constexpr bool MIN = FMT != OXQ_GGUF_Q5_0, FIFTH = FMT != OXQ_GGUF_Q4_1;
         const u32x4_t q = *(const u32x4_t *)(chunk + lane * 16);
+        const uint32_t hb = FIFTH ? *(const uint32_t *)(chunk + L::H_OFF + lane * 4) : 0u;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const uint8_t *uh = chunk + L::UH_OFF + ni * (MIN ? 16 : 8) + t * (MIN ? 4 : 2);
+            const float d = (float)__builtin_bit_cast(_Float16, *(const uint16_t *)uh);
+            const float m = MIN ? (float)__builtin_bit_cast(_Float16, *(const uint16_t *)(uh + 2)) : 0.0f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const uint32_t v = ((q[t] >> (4 * (i >> 1) + 16 * (i & 1))) & 0xFu) |
+                                   (((hb >> (4 * t + (i >> 1) + 16 * (i & 1))) & 1u) << 4);
+                o[32 * t + i] = MIN ? (float)v * d + m : (float)((int)v - 16) * d;
+            }
+        }
+    } else if constexpr (FMT == OXQ_GGUF_Q4_K || FMT == OXQ_GGUF_Q5_K) {
+        const u32x4_t q = *(const u32x4_t *)(chunk + lane * 16);
+        const uint32_t hb = FMT == OXQ_GGUF_Q5_K ? *(const uint32_t *)(chunk + L::H_OFF + lane * 4) : 0u;
         const uint8_t *hd = blk + L::BH_OFF + ni * 16;
         const float d = (float)__builtin_bit_cast(_Float16, *(const uint16_t *)hd);
         const float dmin = (float)__builtin_bit_cast(_Float16, *(const uint16_t *)(hd + 2));
@@ -197,7 +256,8 @@ __global__ __launch_bounds__(256) void ggm_dequant_kernel(const uint8_t *__restr
             const float d1 = d * (float)scv, m1 = dmin * (float)mnv;
 #pragma unroll
             for (int i = 0; i < 8; ++i)
-                o[32 * t + i] = d1 * (float)((q[t] >> (4 * (i >> 1) + 16 * (i & 1))) & 0xFu) - m1;
+                o[32 * t + i] = d1 * (float)(((q[t] >> (4 * (i >> 1) + 16 * (i & 1))) & 0xFu) |
+                                             (((hb >> (4 * t + (i >> 1) + 16 * (i & 1))) & 1u) << 4)) - m1;
         }
     } else if constexpr (FMT == OXQ_GGUF_Q6_K) {
         const u32x4_t lw = *(const u32x4_t *)(chunk + lane * 16);
@@ -240,10 +300,10 @@ template <int FMT> struct GgmChunk {
     typedef GgmFmt<FMT> F;
     typedef GgmLayout<FMT> L;
     static constexpr int NSTEP = FMT == OXQ_GGUF_Q6_K ? 8 : 4;
-    static constexpr bool HAS_MIN = FMT == OXQ_GGUF_Q4_K;
+    static constexpr bool HAS_MIN = ggm_has_min<FMT>;
     u32x4_t q[F::WQ];
     uint32_t qh[FMT == OXQ_GGUF_Q6_K ? 2 : 1];
-    uint32_t uh[F::UH ? 2 : 1];   // unit headers of the column: four f16 d (Q4_0, Q8_0), eight int8 scales (Q6_K)
+    uint32_t uh[F::UH == 16 ? 4 : F::UH ? 2 : 1];   // unit headers of the column: four f16 d or {d, m} pairs, eight int8 scales (Q6_K)
     uint32_t bh[F::BH == 16 ? 4 : 1];  // block header of the column
 
     // c: the chunk's index in its strip
@@ -254,6 +314,9 @@ template <int FMT> struct GgmChunk {
         if constexpr (F::UH == 8) {
             const u32x2_t v = __builtin_amdgcn_raw_buffer_load_b64(rs, ni * 8, soff + L::UH_OFF, 2);
             uh[0] = v[0], uh[1] = v[1];
+        } else if constexpr (F::UH == 16) {
+            const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(rs, ni * 16, soff + L::UH_OFF, 2);
+            uh[0] = v[0], uh[1] = v[1], uh[2] = v[2], uh[3] = v[3];
         }
         if constexpr (F::BH == 16) {
             const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(rs, ni * 16, blk + L::BH_OFF, 0);
@@ -266,12 +329,14 @@ template <int FMT> struct GgmChunk {
         if constexpr (FMT == OXQ_GGUF_Q6_K) {
             const u32x2_t v = __builtin_amdgcn_raw_buffer_load_b64(rs, lane * 8, soff + L::H_OFF, 2);
             qh[0] = v[0], qh[1] = v[1];
+        } else if constexpr (ggm_fifth_bit<FMT>) {
+            qh[0] = __builtin_amdgcn_raw_buffer_load_b32(rs, lane * 4, soff + L::H_OFF, 2);
         }
     }
     // The factors of the chunk's steps, once per chunk when its registers have arrived; half = c % 2 (wave-uniform).
     // f0[st] multiplies the step's sum, f1[st] (formats with a minimum) the bias term -128 sum(x).
     __device__ __forceinline__ void factors(int half, int ni, float (&f0)[NSTEP], float (&f1)[NSTEP]) const {
-        if constexpr (FMT == OXQ_GGUF_Q4_K) {
+        if constexpr (FMT == OXQ_GGUF_Q4_K || FMT == OXQ_GGUF_Q5_K) {
             // get_scale_min_k4 (quant_kernels.metal:2438-2450) for the chunk's four sub-blocks at once, a byte each
             // (selected by mask: as a branch on the chunk's parity the two sides kept twice the registers alive)
             const uint32_t hm = half ? 0xFFFFFFFFu : 0u;
@@ -287,6 +352,9 @@ template <int FMT> struct GgmChunk {
             const float d = ggm_f16((ni & 1) ? (bh[0] >> 16) : (bh[0] & 0xFFFFu));
 #pragma unroll
             for (int st = 0; st < 8; ++st) f0[st] = d * (float)(int)(int8_t)((uh[st >> 2] >> (8 * (st & 3))) & 0xFFu), f1[st] = 0.f;
+        } else if constexpr (F::UH == 16) {  // w = d q + m: the minimum times sum(x) = -m / 128 times the bias term
+#pragma unroll
+            for (int st = 0; st < 4; ++st) f0[st] = ggm_f16(uh[st] & 0xFFFFu), f1[st] = ggm_f16(uh[st] >> 16) * -0.0078125f;
         } else {
 #pragma unroll
             for (int st = 0; st < 4; ++st) f0[st] = ggm_f16((st & 1) ? (uh[st >> 1] >> 16) : (uh[st >> 1] & 0xFFFFu)), f1[st] = 0.f;
@@ -294,9 +362,16 @@ template <int FMT> struct GgmChunk {
     }
     // B operand of step st: bias + q as bf16 pairs (four for a step of 32 elements, two for one of 16)
     __device__ __forceinline__ void operand(int st, uint32_t (&b)[4], const NibbleMasks &nm) const {
-        if constexpr (FMT == OXQ_GGUF_Q4_0 || FMT == OXQ_GGUF_Q4_K) {
+        if constexpr (FMT == OXQ_GGUF_Q4_0 || FMT == OXQ_GGUF_Q4_K || FMT == OXQ_GGUF_Q4_1) {
 #pragma unroll
             for (int pp = 0; pp < 4; ++pp) b[pp] = BF16Traits::unpack1(q[0][st], pp, nm);
+        } else if constexpr (ggm_fifth_bit<FMT>) {  // nibble | fifth bit << 4; m1: the bits' mask, in a register
+#pragma unroll
+            for (int pp = 0; pp < 4; ++pp) {
+                const int sft = 4 * st + pp - 4;
+                const uint32_t hs = sft < 0 ? (qh[0] << -sft) : (qh[0] >> sft);
+                b[pp] = (hs & nm.m1) | BF16Traits::unpack1(q[0][st], pp, nm);
+            }
         } else if constexpr (FMT == OXQ_GGUF_Q8_0) {
             const uint32_t w0 = q[st >> 1][2 * (st & 1)], w1 = q[st >> 1][2 * (st & 1) + 1];
             b[0] = ggm_bytes02(w0), b[1] = ggm_bytes13(w0), b[2] = ggm_bytes02(w1), b[3] = ggm_bytes13(w1);
@@ -370,7 +445,8 @@ __global__ __launch_bounds__(NW * 64) void ggm_kernel(const uint16_t *__restrict
     for (int st = 0; st < NSTEP; ++st)
         a_rd[st] = K16 ? ni * 256 + (((2 * st + (kb >> 1)) ^ ni) << 4) + (kb & 1) * 8 : ni * 256 + (((4 * st + kb) ^ ni) << 4);
     // both masks in registers: v_and_or_b32 takes one literal, and the exponent pattern is it
-    const NibbleMasks nm = FMT == OXQ_GGUF_Q6_K ? NibbleMasks{vgpr_const(0x000F000Fu), vgpr_const(0x00300030u)} : nibble_masks();
+    const NibbleMasks nm = FMT == OXQ_GGUF_Q6_K ? NibbleMasks{vgpr_const(0x000F000Fu), vgpr_const(0x00300030u)}
+                           : ggm_fifth_bit<FMT> ? NibbleMasks{vgpr_const(0x000F000Fu), vgpr_const(0x00100010u)} : nibble_masks();
 #pragma unroll
     for (int q = AQ; q < 4 * MT; ++q) {  // rows no call of this instantiation brings stay zero
         const int row = 4 * q + kb;
@@ -503,13 +579,18 @@ __global__ __launch_bounds__(NW * 64) void ggm_kernel(const uint16_t *__restrict
 // host side
 // ---------------------------------------------------------------------------
 static bool ggm_format(int quant) {
-    return quant == OXQ_GGUF_Q4_0 || quant == OXQ_GGUF_Q8_0 || quant == OXQ_GGUF_Q4_K || quant == OXQ_GGUF_Q6_K;
+    return quant == OXQ_GGUF_Q4_0 || quant == OXQ_GGUF_Q8_0 || quant == OXQ_GGUF_Q4_K || quant == OXQ_GGUF_Q6_K ||
+           quant == OXQ_GGUF_Q4_1 || quant == OXQ_GGUF_Q5_0 || quant == OXQ_GGUF_Q5_1 || quant == OXQ_GGUF_Q5_K;
 }
 static const char *ggm_name(int q) {
     switch (q) {
     case OXQ_GGUF_Q4_0: return "q4_0";
     case OXQ_GGUF_Q8_0: return "q8_0";
     case OXQ_GGUF_Q4_K: return "q4k";
+    case OXQ_GGUF_Q4_1: return "q4_1";
+    case OXQ_GGUF_Q5_0: return "q5_0";
+    case OXQ_GGUF_Q5_1: return "q5_1";
+    case OXQ_GGUF_Q5_K: return "q5k";
     default: return "q6k";
     }
 }
@@ -531,6 +612,10 @@ int launch_gguf_mfma_repack(oxq_ctx *ctx, hipStream_t s, int quant, const uint8_
     case OXQ_GGUF_Q8_0: hipLaunchKernelGGL((ggm_repack_kernel<OXQ_GGUF_Q8_0>), grid, block, 0, s, w, (uint8_t *)pw, (int)K, (int)N); break;
     case OXQ_GGUF_Q4_K: hipLaunchKernelGGL((ggm_repack_kernel<OXQ_GGUF_Q4_K>), grid, block, 0, s, w, (uint8_t *)pw, (int)K, (int)N); break;
     case OXQ_GGUF_Q6_K: hipLaunchKernelGGL((ggm_repack_kernel<OXQ_GGUF_Q6_K>), grid, block, 0, s, w, (uint8_t *)pw, (int)K, (int)N); break;
+    case OXQ_GGUF_Q4_1: hipLaunchKernelGGL((ggm_repack_kernel<OXQ_GGUF_Q4_1>), grid, block, 0, s, w, (uint8_t *)pw, (int)K, (int)N); break;
+    case OXQ_GGUF_Q5_0: hipLaunchKernelGGL((ggm_repack_kernel<OXQ_GGUF_Q5_0>), grid, block, 0, s, w, (uint8_t *)pw, (int)K, (int)N); break;
+    case OXQ_GGUF_Q5_1: hipLaunchKernelGGL((ggm_repack_kernel<OXQ_GGUF_Q5_1>), grid, block, 0, s, w, (uint8_t *)pw, (int)K, (int)N); break;
+    case OXQ_GGUF_Q5_K: hipLaunchKernelGGL((ggm_repack_kernel<OXQ_GGUF_Q5_K>), grid, block, 0, s, w, (uint8_t *)pw, (int)K, (int)N); break;
     default: return fail(OXQ_ERR_UNSUPPORTED, "gguf repack: format %d has no matrix-core layout", quant);
     }
     OXQ_HIP_CHECK(hipGetLastError());
@@ -549,6 +634,10 @@ int launch_gguf_mfma_dequant(oxq_ctx *ctx, hipStream_t s, int quant, const void 
     case OXQ_GGUF_Q8_0: hipLaunchKernelGGL((ggm_dequant_kernel<OXQ_GGUF_Q8_0>), grid, block, 0, s, (const uint8_t *)pw, out_nk, (int)K, (int)N); break;
     case OXQ_GGUF_Q4_K: hipLaunchKernelGGL((ggm_dequant_kernel<OXQ_GGUF_Q4_K>), grid, block, 0, s, (const uint8_t *)pw, out_nk, (int)K, (int)N); break;
     case OXQ_GGUF_Q6_K: hipLaunchKernelGGL((ggm_dequant_kernel<OXQ_GGUF_Q6_K>), grid, block, 0, s, (const uint8_t *)pw, out_nk, (int)K, (int)N); break;
+    case OXQ_GGUF_Q4_1: hipLaunchKernelGGL((ggm_dequant_kernel<OXQ_GGUF_Q4_1>), grid, block, 0, s, (const uint8_t *)pw, out_nk, (int)K, (int)N); break;
+    case OXQ_GGUF_Q5_0: hipLaunchKernelGGL((ggm_dequant_kernel<OXQ_GGUF_Q5_0>), grid, block, 0, s, (const uint8_t *)pw, out_nk, (int)K, (int)N); break;
+    case OXQ_GGUF_Q5_1: hipLaunchKernelGGL((ggm_dequant_kernel<OXQ_GGUF_Q5_1>), grid, block, 0, s, (const uint8_t *)pw, out_nk, (int)K, (int)N); break;
+    case OXQ_GGUF_Q5_K: hipLaunchKernelGGL((ggm_dequant_kernel<OXQ_GGUF_Q5_K>), grid, block, 0, s, (const uint8_t *)pw, out_nk, (int)K, (int)N); break;
     default: return fail(OXQ_ERR_UNSUPPORTED, "gguf dequant: format %d has no matrix-core layout", quant);
     }
     OXQ_HIP_CHECK(hipGetLastError());
@@ -622,6 +711,10 @@ int launch_gguf_mfma(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p) {
     case OXQ_GGUF_Q8_0: return ggm_by_shape<OXQ_GGUF_Q8_0>(s, grid, p, nullptr, cslice, mt, xq, nw, ns);
     case OXQ_GGUF_Q4_K: return ggm_by_shape<OXQ_GGUF_Q4_K>(s, grid, p, nullptr, cslice, mt, xq, nw, ns);
     case OXQ_GGUF_Q6_K: return ggm_by_shape<OXQ_GGUF_Q6_K>(s, grid, p, nullptr, cslice, mt, xq, nw, ns);
+    case OXQ_GGUF_Q4_1: return ggm_by_shape<OXQ_GGUF_Q4_1>(s, grid, p, nullptr, cslice, mt, xq, nw, ns);
+    case OXQ_GGUF_Q5_0: return ggm_by_shape<OXQ_GGUF_Q5_0>(s, grid, p, nullptr, cslice, mt, xq, nw, ns);
+    case OXQ_GGUF_Q5_1: return ggm_by_shape<OXQ_GGUF_Q5_1>(s, grid, p, nullptr, cslice, mt, xq, nw, ns);
+    case OXQ_GGUF_Q5_K: return ggm_by_shape<OXQ_GGUF_Q5_K>(s, grid, p, nullptr, cslice, mt, xq, nw, ns);
     default: return fail(OXQ_ERR_UNSUPPORTED, "gguf matrix-core matmul: format %d", p.quant);
     }
 }

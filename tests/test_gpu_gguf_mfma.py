@@ -1,6 +1,7 @@
 """Resident bf16 GGUF layers on the matrix-core layout (csrc/gguf_mfma.hip), through the C ABI.
 
-A bf16 QLinear (linear.rs:197-284, the reference's GPU contract: bf16 x and y) of Q4_0, Q8_0, Q4_K or Q6_K keeps
+A bf16 QLinear (linear.rs:197-284, the reference's GPU contract: bf16 x and y) of Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q4_K,
+Q5_K or Q6_K keeps
 a copy of its blocks in which a strip of 16 columns and a step of 32 (Q6_K: 16) elements of K are one MFMA whose
 rows are rows of x; 1 - 32 rows run on it in one launch.  The arithmetic is the GEMV's at every row count
 (quant_kernels.metal:1097-1221, 1681-1838: integer sums, one f32 scale per sub-block): the weights are never
@@ -27,9 +28,10 @@ from tests.helpers import as_f32, assert_close, bits_of, gguf_on_matrix_cores, r
 
 pytestmark = pytest.mark.gpu
 ops = None
-MC = [synth.GGUF_Q4_0, synth.GGUF_Q8_0, synth.GGUF_Q4_K, synth.GGUF_Q6_K]
+MC = [synth.GGUF_Q4_0, synth.GGUF_Q8_0, synth.GGUF_Q4_K, synth.GGUF_Q6_K, synth.GGUF_Q4_1, synth.GGUF_Q5_0, synth.GGUF_Q5_1, synth.GGUF_Q5_K]
 FMTS = [pytest.param(f, id=synth.GGUF_NAMES[f]) for f in MC]
-TAG = {synth.GGUF_Q4_0: "q4_0", synth.GGUF_Q8_0: "q8_0", synth.GGUF_Q4_K: "q4k", synth.GGUF_Q6_K: "q6k"}
+TAG = {synth.GGUF_Q4_0: "q4_0", synth.GGUF_Q8_0: "q8_0", synth.GGUF_Q4_K: "q4k", synth.GGUF_Q6_K: "q6k",
+       synth.GGUF_Q4_1: "q4_1", synth.GGUF_Q5_0: "q5_0", synth.GGUF_Q5_1: "q5_1", synth.GGUF_Q5_K: "q5k"}
 
 
 def setup_module(module):
