@@ -138,9 +138,9 @@ int oxq_ctx_reset_tuning(oxq_ctx *ctx, const char *name);
  * weights, f32 fold; above: tile GEMM on weights rounded to the activation type).  Shapes the
  * resident layout does not cover take the usual path.  The copy costs the packed tensors' size
  * again; least recently used copies go when max_bytes is reached.  oxq_gguf_quant_matmul does the
- * same for the GGUF formats that have a strip-major form (see oxq_qlinear_new) at 1 - 4 rows of x (f32: 1 - 8),
- * keyed by the address of the block
- * bytes, with the strip-major copy that oxq_qlinear_new builds.
+ * same for the GGUF formats that have a strip-major form (see oxq_qlinear_new) at the rows that form takes
+ * (f32: 1 - 8; bf16: 1 - 32 on the matrix-core copy, there also for oxq_gguf_quant_mul_mm), keyed by the
+ * address of the block bytes and the layout, with the copy that oxq_qlinear_new builds.
  *
  * A copy that served a call while the stream was being captured is part of that graph: it stays, and
  * counts against max_bytes, until oxq_ctx_forget_weights or oxq_ctx_destroy frees it - either of which
@@ -473,7 +473,12 @@ int oxq_qlinear_forward(oxq_qlinear *layer, void *stream, const oxq_tensor *x,
  * builds a layer-owned copy of the blocks in strips of 16 rows (the file's bytes per weight; Q3_K: 112 for
  * 110 bytes a super-block; so twice the
  * layer's bytes while the caller keeps weight_bytes); forward then runs 1 - 4 rows of x on that copy (f32
- * rows up to 8, in two passes of four) and everything else on weight_bytes as before.  OXQ_PREPACK=0 in the environment turns the copy off.
+ * rows up to 8, in two passes of four) and everything else on weight_bytes as before.  A BF16 layer of Q4_0,
+ * Q4_1, Q5_0, Q5_1, Q8_0, Q4_K, Q5_K or Q6_K holds the copy in the matrix-core layout instead (the same size), on
+ * which one launch takes 1 - 32 rows (16 from 768 strips of 16 columns on) with the GEMV's arithmetic at every
+ * row count: integer sums, one f32 scale per sub-block, the weights never rounded to bf16 (the reference's
+ * prefill tiles round them above 8 rows).  The tuning switch OXQ_PREPACK=0 turns the copy off, OXQ_GGUF_MFMA=0
+ * keeps the first layout for BF16 layers too.
  * *resident = 1 if the layer holds the copy. */
 int oxq_qlinear_is_resident(const oxq_qlinear *layer, int *resident);
 /* Dense f32 [out_features, in_features] of the layer's weights, read from the copy when there is one:
