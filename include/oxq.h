@@ -475,7 +475,7 @@ int oxq_qlinear_forward(oxq_qlinear *layer, void *stream, const oxq_tensor *x,
  * layer's bytes while the caller keeps weight_bytes); forward then runs 1 - 4 rows of x on that copy (f32
  * rows up to 8, in two passes of four) and everything else on weight_bytes as before.  A BF16 layer of Q4_0,
  * Q4_1, Q5_0, Q5_1, Q8_0, Q4_K, Q5_K or Q6_K holds the copy in the matrix-core layout instead (the same size), on
- * which one launch takes 1 - 32 rows (16 from 768 strips of 16 columns on) with the GEMV's arithmetic at every
+ * which one launch takes 1 - 32 rows with the GEMV's arithmetic at every
  * row count: integer sums, one f32 scale per sub-block, the weights never rounded to bf16 (the reference's
  * prefill tiles round them above 8 rows).  The tuning switch OXQ_PREPACK=0 turns the copy off, OXQ_GGUF_MFMA=0
  * keeps the first layout for BF16 layers too.

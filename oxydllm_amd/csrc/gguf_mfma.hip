@@ -404,8 +404,8 @@ __global__ __launch_bounds__(NW * 64) void ggm_kernel(const uint16_t *__restrict
     typedef GgmLayout<FMT> L;
     typedef GgmChunk<FMT> C;
     constexpr int ROWS = 16 * MT, AQ = XQ, SLOT = ROWS * 256, OOB = 0x7FFFFF00, NSTEP = C::NSTEP;
-    // chunks in flight a wave: three, two where block headers and factors take the registers (measured on
-    // 4096 x 4096 at one row, Q8_0: 5.06 us with three, 5.87 with two)
+    // chunks in flight a wave: three (4096 x 4096 at one row, Q8_0: 5.06 us with three, 5.87 with two); two
+    // where a workgroup takes four strips, whose quants are four times the registers
     constexpr int RD = NS > 1 ? 2 : 3;
     constexpr bool K16 = NSTEP == 8;  // steps of 16 elements
     extern __shared__ __attribute__((aligned(16))) unsigned char pk4_lds[];
@@ -530,25 +530,28 @@ __global__ __launch_bounds__(NW * 64) void ggm_kernel(const uint16_t *__restrict
                 }
             }
         } else {  // more row tiles: step by step, the registers do not hold a chunk's operands
-            static_assert(MT == 1 || NS == 1, "two row tiles take one strip");
-            const C &w = wr[CUR][0];
-            w.factors((cc0 + i) & 1, ni, f0, f1);
 #pragma unroll
-            for (int st = 0; st < NSTEP; ++st) {
-                uint32_t b[4];
-                w.operand(st, b, nm);
+            for (int f = 0; f < NS; ++f) {
+                const C &w = wr[CUR][f];
+                w.factors((cc0 + i) & 1, ni, f0, f1);
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt) {
-                    uint32_t a[4];
-                    load_a(st, mt, a);
-                    const float4_t tn = mma(a, neg, zero4);
-                    const float4_t t = mma(a, b, tn);
+                for (int st = 0; st < NSTEP; ++st) {
+                    uint32_t b[4];
+                    w.operand(st, b, nm);
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        acc[mt][0][e] = fmaf(f0[st], t[e], acc[mt][0][e]);
-                        if constexpr (C::HAS_MIN) acc[mt][0][e] = fmaf(f1[st], tn[e], acc[mt][0][e]);
+                    for (int mt = 0; mt < MT; ++mt) {
+                        uint32_t a[4];
+                        load_a(st, mt, a);
+                        const float4_t tn = mma(a, neg, zero4);
+                        const float4_t t = mma(a, b, tn);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            acc[mt][f][e] = fmaf(f0[st], t[e], acc[mt][f][e]);
+                            if constexpr (C::HAS_MIN) acc[mt][f][e] = fmaf(f1[st], tn[e], acc[mt][f][e]);
+                        }
                     }
                 }
+                if constexpr (NS > 1) __builtin_amdgcn_sched_barrier(0);  // one strip's operands at a time
             }
         }
         if (more) request(i + RD, wr[CUR], ar[CUR]);
@@ -657,6 +660,7 @@ static int ggm_go(hipStream_t s, dim3 grid, const GgufProblem &p, float *ws, int
 template <int FMT>
 static int ggm_by_shape(hipStream_t s, dim3 grid, const GgufProblem &p, float *ws, int cslice, int mt, int xq, int nw, int ns) {
     if (ns == 4) {  // 8 waves: four strips' quants in flight take the registers of two waves of a 16-wave workgroup
+        if (mt == 2) return ggm_go<FMT, 2, 8, 8, 4>(s, grid, p, ws, cslice);
         if (xq == 1) return ggm_go<FMT, 1, 1, 8, 4>(s, grid, p, ws, cslice);
         if (xq == 2) return ggm_go<FMT, 1, 2, 8, 4>(s, grid, p, ws, cslice);
         return ggm_go<FMT, 1, 4, 8, 4>(s, grid, p, ws, cslice);
@@ -681,16 +685,14 @@ static int ggm_strips(const oxq_ctx *ctx, int64_t N) {
     return (N / 16 >= 768 && (N / 16) % 4 == 0) ? 4 : 1;
 }
 
-// rows of x a launch of the matrix-core kernel takes (more go to the tile matmul on the file layout): 32, 16 where
-// a workgroup takes four strips (two row tiles of four strips do not fit the registers)
-bool gguf_mfma_takes(const oxq_ctx *ctx, int64_t M, int64_t N, int act_dtype) {
-    const int64_t cap = ggm_strips(ctx, N) == 4 ? 16 : 32;
-    return act_dtype == OXQ_BF16 && M >= 1 && M <= std::min<int64_t>(cap, tune(ctx, OXQ_TUNE_GGUF_MFMA_MAX_M, 32));
+// rows of x a launch of the matrix-core kernel takes (more go to the tile matmul on the file layout)
+bool gguf_mfma_takes(const oxq_ctx *ctx, int64_t M, int64_t, int act_dtype) {
+    return act_dtype == OXQ_BF16 && M >= 1 && M <= std::min<int64_t>(32, tune(ctx, OXQ_TUNE_GGUF_MFMA_MAX_M, 32));
 }
 
 // p.w is the matrix-core copy
 int launch_gguf_mfma(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p) {
-    const int ns = p.M <= 16 ? ggm_strips(ctx, p.N) : 1;
+    const int ns = ggm_strips(ctx, p.N);
     const int mt = p.M > 16 ? 2 : 1;
     const int rows = (int)std::min<int64_t>(p.M, 16 * mt);
     const int xq = rows <= 4 ? 1 : rows <= 8 ? 2 : 4;

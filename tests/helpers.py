@@ -93,8 +93,7 @@ def gguf_on_matrix_cores(fmt: int, n: int, k: int, m: int, bf16: bool = True) ->
                                synth.GGUF_Q5_0, synth.GGUF_Q5_1, synth.GGUF_Q5_K):
         return False
     kq = fmt in (synth.GGUF_Q4_K, synth.GGUF_Q6_K, synth.GGUF_Q5_K)
-    wide = n // 16 >= 768 and n % 64 == 0  # four strips a workgroup: one row tile
-    return n % 16 == 0 and k % (256 if kq else 128) == 0 and 1 <= m <= (16 if wide else GGUF_MATRIX_CORE_ROWS)
+    return n % 16 == 0 and k % (256 if kq else 128) == 0 and 1 <= m <= GGUF_MATRIX_CORE_ROWS
 
 
 def round_x(x_f32: np.ndarray, dt: int) -> np.ndarray:
