@@ -466,6 +466,20 @@ typedef struct oxq_qlinear oxq_qlinear;
 int oxq_qlinear_new(oxq_ctx *ctx, int quant, const oxq_tensor *weight_bytes, int64_t in_features,
                     int64_t out_features, const oxq_tensor *bias_or_null, int out_dtype,
                     oxq_qlinear **out);
+/* ffn.rs:307-373, 386-413: the fused gate|up projection of a block-quantized FFN (GateUpProjection::Packed: rows
+ * 0 .. I - 1 of weight_bytes are gate_proj, I .. 2I - 1 up_proj; a loader fuses separate ffn_gate / ffn_up tensors
+ * by concatenating their bytes) with gated_silu_fused / gated_gelu_tanh_fused (ffn_kernels.metal:19-160) run in the
+ * matmul's epilogue: out_features = 2I, forward writes [.., I] = act(gate(x)) * up(x), bit for bit what
+ * oxq_gated_activation gives on the plain layer's output.  Needs a BF16 layer that takes the matrix-core copy (see
+ * oxq_qlinear_is_resident below), else OXQ_ERR_UNSUPPORTED.  Every row count runs in one launch, in row tiles of 32
+ * that each read the weights again (and, above 32 rows, with the unrounded weights that the plain layer's tile
+ * matmul rounds to bf16): oxq_mlp_forward sends more than OXQ_GGUF_FUSED_ACT_ROWS rows through the plain layer's
+ * path and the activation by itself, so that a FeedForward over this layer gives the plain layers' bits at every
+ * row count. */
+#define OXQ_GGUF_FUSED_ACT_ROWS 32
+int oxq_qlinear_new_gate_up(oxq_ctx *ctx, int quant, const oxq_tensor *weight_bytes, int64_t in_features,
+                            int64_t out_features, const oxq_tensor *bias_or_null, int act, int out_dtype,
+                            oxq_qlinear **out);
 int oxq_qlinear_forward(oxq_qlinear *layer, void *stream, const oxq_tensor *x,
                         const oxq_tensor *out);
 /* linear.rs:225-240 (the fast path's own copy of the block bytes).  For layers of any of the ten formats

@@ -139,6 +139,8 @@ SIGNATURES = {
     "oxq_packed_quant_linear_free": (None, [_VP]),
     "oxq_qlinear_new": (C.c_int, [_VP, C.c_int, _TP, C.c_int64, C.c_int64, _TP, C.c_int,
                                   C.POINTER(_VP)]),
+    "oxq_qlinear_new_gate_up": (C.c_int, [_VP, C.c_int, _TP, C.c_int64, C.c_int64, _TP, C.c_int, C.c_int,
+                                          C.POINTER(_VP)]),
     "oxq_qlinear_forward": (C.c_int, [_VP, _VP, _TP, _TP]),
     "oxq_qlinear_is_resident": (C.c_int, [_VP, C.POINTER(C.c_int)]),
     "oxq_qlinear_dequantize": (C.c_int, [_VP, _VP, _TP]),

@@ -282,9 +282,14 @@ class GgufWeights(TensorFile):
         return ops.QLinear(t.gguf_quant, w, in_f, out_f, bias, out_dtype or torch.bfloat16, ctx=ctx)
 
     def feed_forward(self, layer_idx: int, intermediate_size: int, activation: Optional[int] = None, out_dtype=None,
-                     ctx=None):
+                     ctx=None, fuse: bool = True):
         """ffn.rs:307-373 FeedForward::load_gguf: ``blk.{i}.ffn_{gate,up,down}.weight`` kept quantized.
-        Separate when ``ffn_gate`` exists, packed when ``ffn_up`` holds gate and up, ungated otherwise."""
+        Separate when ``ffn_gate`` exists, packed when ``ffn_up`` holds gate and up, ungated otherwise.
+
+        With ``fuse`` a gated bf16 layer whose format and shape have the matrix-core copy becomes one projection with
+        the activation in its epilogue (separate ``ffn_gate`` / ``ffn_up`` tensors of one format are fused by
+        concatenating their bytes): two launches a forward instead of four, the same bits."""
+        import torch
         from . import ops
         activation = ops.ACT_GATED_SILU if activation is None else activation
         prefix = f"blk.{layer_idx}"
@@ -303,15 +308,40 @@ class GgufWeights(TensorFile):
             if up_out != intermediate_size:
                 raise OxqError(-3, f"GGUF ffn_up shape mismatch at {prefix}: expected dim0={intermediate_size}, "
                                    f"got {up_out}")
-            kind, a, b = ops.GATE_UP_SEPARATE, mk("gate"), mk("up")
+            a = None
+            if fuse and gate_t.gguf_quant == up_t.gguf_quant and gate_t.shape == up_t.shape:
+                both = torch.cat([gate_t.to_device(ctx).reshape(-1), up_t.to_device(ctx).reshape(-1)])
+                a = self._fused_gate_up(up_t.gguf_quant, both, up_t.shape[1], 2 * intermediate_size, activation, out_dtype, ctx)
+            if a is not None:
+                kind, b = ops.GATE_UP_FUSED, None
+            else:
+                kind, a, b = ops.GATE_UP_SEPARATE, mk("gate"), mk("up")
         elif up_out == 2 * intermediate_size:
-            kind, a, b = ops.GATE_UP_FUSED, mk("up"), None
+            a = self._fused_gate_up(up_t.gguf_quant, up_t.to_device(ctx), up_t.shape[1], up_out, activation, out_dtype,
+                                    ctx) if fuse else None
+            kind, a, b = ops.GATE_UP_FUSED, a if a is not None else mk("up"), None
         elif up_out == intermediate_size:
             kind, a, b = ops.GATE_UP_SIMPLE, mk("up"), None
         else:
             raise OxqError(-3, f"Unsupported GGUF FFN up-proj shape at {prefix}: dim0={up_out} (expected "
                                f"{intermediate_size} or {2 * intermediate_size})")
         return ops.FeedForward(kind, a, b, mk("down"), intermediate_size, activation, ctx=ctx)
+
+
+    @staticmethod
+    def _fused_gate_up(quant: int, both, in_f: int, out_f: int, activation: int, out_dtype, ctx):
+        """The gate|up bytes as one layer with the activation in its epilogue, or None where that layer cannot be
+        built (format, shape or dtype without the matrix-core copy)."""
+        import torch
+        from . import ops
+        if quant < 0 or (out_dtype or torch.bfloat16) != torch.bfloat16:
+            return None
+        try:
+            return ops.QLinear(quant, both, in_f, out_f, None, torch.bfloat16, ctx=ctx, gate_up_act=activation)
+        except OxqError as e:
+            if e.status != -11:  # OXQ_ERR_UNSUPPORTED: take the plain layers
+                raise
+            return None
 
 
 @dataclass

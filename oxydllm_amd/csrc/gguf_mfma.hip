@@ -68,9 +68,18 @@ template <int FMT> struct GgmLayout {
 // ---------------------------------------------------------------------------
 // repack: one thread per (strip, chunk, lane)
 // ---------------------------------------------------------------------------
+// Resident column -> row of the file.  A fused gate|up layer (half = N / 2 gate rows followed by as many up rows)
+// keeps, in every strip of 16, 8 gate columns followed by the 8 up columns they are multiplied with, so that one
+// workgroup holds both factors of its outputs.
+__device__ __forceinline__ int ggm_src_row(int c, int half) {
+    if (!half) return c;
+    const int j = c >> 4, cc = c & 15;
+    return cc < 8 ? 8 * j + cc : half + 8 * j + (cc - 8);
+}
+
 template <int FMT>
 __global__ __launch_bounds__(256) void ggm_repack_kernel(const uint8_t *__restrict__ w, uint8_t *__restrict__ pw, int K,
-                                                         int N) {
+                                                         int N, int half) {
     typedef GgmFmt<FMT> F;
     typedef GgmLayout<FMT> L;
     const int nch = K >> 7;
@@ -79,7 +88,7 @@ __global__ __launch_bounds__(256) void ggm_repack_kernel(const uint8_t *__restri
     const int lane = (int)(idx & 63), c = (int)((idx >> 6) % nch), strip = (int)((idx >> 6) / nch);
     const int ni = lane & 15, kb = lane >> 4;
     const size_t row_bytes = (size_t)(K / GgufFmt<FMT>::BE) * GgufFmt<FMT>::BB;
-    const uint8_t *row = w + (size_t)(16 * strip + ni) * row_bytes;
+    const uint8_t *row = w + (size_t)ggm_src_row(16 * strip + ni, half) * row_bytes;
     uint8_t *blk = pw + ((size_t)strip * (nch / F::CH) + c / F::CH) * L::BLKB;
     uint8_t *chunk = blk + (c % F::CH) * L::CHB;
     if constexpr (FMT == OXQ_GGUF_Q4_0) {
@@ -192,7 +201,7 @@ __global__ __launch_bounds__(256) void ggm_repack_kernel(const uint8_t *__restri
 // dense [N, K] f32 from the copy, with the arithmetic of the file-layout dequant (pins the repack bit for bit)
 template <int FMT>
 __global__ __launch_bounds__(256) void ggm_dequant_kernel(const uint8_t *__restrict__ pw, float *__restrict__ out, int K,
-                                                          int N) {
+                                                          int N, int half) {
     typedef GgmFmt<FMT> F;
     typedef GgmLayout<FMT> L;
     const int nch = K >> 7;
@@ -202,7 +211,8 @@ __global__ __launch_bounds__(256) void ggm_dequant_kernel(const uint8_t *__restr
     const int ni = lane & 15, kb = lane >> 4;
     const uint8_t *blk = pw + ((size_t)strip * (nch / F::CH) + c / F::CH) * L::BLKB;
     const uint8_t *chunk = blk + (c % F::CH) * L::CHB;
-    float *o = out + (size_t)(16 * strip + ni) * K + (size_t)c * 128 + 8 * kb;
+    const size_t orow = (size_t)ggm_src_row(16 * strip + ni, half);
+    float *o = out + orow * K + (size_t)c * 128 + 8 * kb;
     if constexpr (FMT == OXQ_GGUF_Q4_0) {
         const u32x4_t q = *(const u32x4_t *)(chunk + lane * 16);
 #pragma unroll
@@ -263,7 +273,7 @@ __global__ __launch_bounds__(256) void ggm_dequant_kernel(const uint8_t *__restr
         const u32x4_t lw = *(const u32x4_t *)(chunk + lane * 16);
         const uint2 hw = *(const uint2 *)(chunk + L::H_OFF + lane * 8);
         const float d = (float)__builtin_bit_cast(_Float16, *(const uint16_t *)(blk + L::BH_OFF + ni * 2));
-        float *o6 = out + (size_t)(16 * strip + ni) * K + (size_t)c * 128 + 4 * kb;
+        float *o6 = out + orow * K + (size_t)c * 128 + 4 * kb;
 #pragma unroll
         for (int s2 = 0; s2 < 8; ++s2) {
             const float ds = d * (float)(int)*(const int8_t *)(chunk + L::UH_OFF + ni * 8 + s2);
@@ -394,10 +404,53 @@ __device__ __forceinline__ float4_t ggm_mfma16(uint32_t a0, uint32_t a1, uint32_
                                                      __builtin_bit_cast(short4_t, u32x2_t{b0, b1}), c, 0, 0, 0);
 }
 
+// Epilogue of a fused gate|up layer (ffn.rs:386-400 runs gated_silu_fused / gated_gelu_tanh_fused on the fused
+// projection's output): the waves' partial tiles meet in LDS as in pk4n_epilogue; a thread then owns (row, gate
+// column p of a strip and its up column p + 8), adds the waves in order, rounds both factors to bf16 as the
+// projection's own output would be, and writes act(gate) * up to y [M, N / 2].
+template <int MT, int NS, int NW>
+__device__ __forceinline__ void ggm_epilogue_act(const float4_t (&acc)[MT][NS], const uint16_t *__restrict__ bias,
+                                                 uint16_t *__restrict__ y, int M, int N, int j, int m0, int act,
+                                                 int wave, int lane) {
+    typedef BF16Traits TT;
+    constexpr int NT = NW * 64, ROWS = 16 * MT;
+    extern __shared__ __attribute__((aligned(16))) unsigned char pk4_lds[];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            float *dst = (float *)(pk4_lds + (size_t)wave * MT * 4096) + ((mt * 4 + e) * 64 + lane) * NS;
+#pragma unroll
+            for (int f = 0; f < NS; ++f) dst[f] = acc[mt][f][e];
+        }
+    __syncthreads();
+    const int half = N >> 1;
+    for (int t = threadIdx.x; t < ROWS * 8 * NS; t += NT) {
+        const int p = t & 7, f = (t >> 3) % NS, ml = t / (8 * NS);
+        if (m0 + ml >= M) continue;
+        const int mt = ml >> 4, r = ml & 15, kb = r >> 2, e = r & 3;
+        float g = 0.f, u = 0.f;
+#pragma unroll
+        for (int s = 0; s < NW; ++s) {
+            const float *src = (const float *)(pk4_lds + (size_t)s * MT * 4096) + ((mt * 4 + e) * 64 + kb * 16 + p) * NS + f;
+            g += src[0];
+            u += src[8 * NS];
+        }
+        const int n = 8 * (NS * j + f) + p;
+        if (bias) {
+            g += TT::to_f32(bias[n]);
+            u += TT::to_f32(bias[half + n]);
+        }
+        g = TT::to_f32(TT::from_f32(g));
+        u = TT::to_f32(TT::from_f32(u));
+        y[(size_t)(m0 + ml) * half + n] = TT::from_f32(mul_f32_rn(act == 1 ? silu_f32(g) : gelu_tanh_f32(g), u));
+    }
+}
+
 template <int FMT, int MT, int XQ, int NW, int NS>
 __global__ __launch_bounds__(NW * 64) void ggm_kernel(const uint16_t *__restrict__ x, const uint8_t *__restrict__ pw,
                                                       const uint16_t *__restrict__ bias, uint16_t *__restrict__ y,
-                                                      float *__restrict__ ws, int M, int K, int N, int cslice) {
+                                                      float *__restrict__ ws, int M, int K, int N, int cslice, int act) {
     typedef BF16Traits TT;
     typedef MfmaOps<TT> Ops;
     typedef GgmFmt<FMT> F;
@@ -575,7 +628,8 @@ __global__ __launch_bounds__(NW * 64) void ggm_kernel(const uint16_t *__restrict
             if (i + 1 < nloc) chunk(i + 1, std::integral_constant<int, 1>{}, false);
         }
     }
-    pk4n_epilogue<TT, MT, NS, NW>(acc, bias, y, ws, M, N, j, m0, wave, lane);
+    if (act) ggm_epilogue_act<MT, NS, NW>(acc, bias, y, M, N, j, m0, act, wave, lane);
+    else pk4n_epilogue<TT, MT, NS, NW>(acc, bias, y, ws, M, N, j, m0, wave, lane);
 }
 
 // ---------------------------------------------------------------------------
@@ -603,7 +657,8 @@ bool gguf_mfma_eligible(const oxq_ctx *ctx, int quant, int64_t K, int64_t N) {
     return gguf_res_eligible(quant, K, N);  // the same strips, chunks and 32-bit offsets
 }
 
-int launch_gguf_mfma_repack(oxq_ctx *ctx, hipStream_t s, int quant, const uint8_t *w, void *pw, int64_t K, int64_t N) {
+int launch_gguf_mfma_repack(oxq_ctx *ctx, hipStream_t s, int quant, const uint8_t *w, void *pw, int64_t K, int64_t N,
+                            int64_t gate_half) {
     const size_t threads = (size_t)(N / 16) * (K / 128) * 64;
     dim3 grid((unsigned)ceil_div((int64_t)threads, 256)), block(256);
     char name[64];
@@ -611,21 +666,22 @@ int launch_gguf_mfma_repack(oxq_ctx *ctx, hipStream_t s, int quant, const uint8_
     set_plan(ctx, name, grid, block, 1, 1, 0);
     if (ctx->plan_only) return OXQ_OK;
     switch (quant) {
-    case OXQ_GGUF_Q4_0: hipLaunchKernelGGL((ggm_repack_kernel<OXQ_GGUF_Q4_0>), grid, block, 0, s, w, (uint8_t *)pw, (int)K, (int)N); break;
-    case OXQ_GGUF_Q8_0: hipLaunchKernelGGL((ggm_repack_kernel<OXQ_GGUF_Q8_0>), grid, block, 0, s, w, (uint8_t *)pw, (int)K, (int)N); break;
-    case OXQ_GGUF_Q4_K: hipLaunchKernelGGL((ggm_repack_kernel<OXQ_GGUF_Q4_K>), grid, block, 0, s, w, (uint8_t *)pw, (int)K, (int)N); break;
-    case OXQ_GGUF_Q6_K: hipLaunchKernelGGL((ggm_repack_kernel<OXQ_GGUF_Q6_K>), grid, block, 0, s, w, (uint8_t *)pw, (int)K, (int)N); break;
-    case OXQ_GGUF_Q4_1: hipLaunchKernelGGL((ggm_repack_kernel<OXQ_GGUF_Q4_1>), grid, block, 0, s, w, (uint8_t *)pw, (int)K, (int)N); break;
-    case OXQ_GGUF_Q5_0: hipLaunchKernelGGL((ggm_repack_kernel<OXQ_GGUF_Q5_0>), grid, block, 0, s, w, (uint8_t *)pw, (int)K, (int)N); break;
-    case OXQ_GGUF_Q5_1: hipLaunchKernelGGL((ggm_repack_kernel<OXQ_GGUF_Q5_1>), grid, block, 0, s, w, (uint8_t *)pw, (int)K, (int)N); break;
-    case OXQ_GGUF_Q5_K: hipLaunchKernelGGL((ggm_repack_kernel<OXQ_GGUF_Q5_K>), grid, block, 0, s, w, (uint8_t *)pw, (int)K, (int)N); break;
+    case OXQ_GGUF_Q4_0: hipLaunchKernelGGL((ggm_repack_kernel<OXQ_GGUF_Q4_0>), grid, block, 0, s, w, (uint8_t *)pw, (int)K, (int)N, (int)gate_half); break;
+    case OXQ_GGUF_Q8_0: hipLaunchKernelGGL((ggm_repack_kernel<OXQ_GGUF_Q8_0>), grid, block, 0, s, w, (uint8_t *)pw, (int)K, (int)N, (int)gate_half); break;
+    case OXQ_GGUF_Q4_K: hipLaunchKernelGGL((ggm_repack_kernel<OXQ_GGUF_Q4_K>), grid, block, 0, s, w, (uint8_t *)pw, (int)K, (int)N, (int)gate_half); break;
+    case OXQ_GGUF_Q6_K: hipLaunchKernelGGL((ggm_repack_kernel<OXQ_GGUF_Q6_K>), grid, block, 0, s, w, (uint8_t *)pw, (int)K, (int)N, (int)gate_half); break;
+    case OXQ_GGUF_Q4_1: hipLaunchKernelGGL((ggm_repack_kernel<OXQ_GGUF_Q4_1>), grid, block, 0, s, w, (uint8_t *)pw, (int)K, (int)N, (int)gate_half); break;
+    case OXQ_GGUF_Q5_0: hipLaunchKernelGGL((ggm_repack_kernel<OXQ_GGUF_Q5_0>), grid, block, 0, s, w, (uint8_t *)pw, (int)K, (int)N, (int)gate_half); break;
+    case OXQ_GGUF_Q5_1: hipLaunchKernelGGL((ggm_repack_kernel<OXQ_GGUF_Q5_1>), grid, block, 0, s, w, (uint8_t *)pw, (int)K, (int)N, (int)gate_half); break;
+    case OXQ_GGUF_Q5_K: hipLaunchKernelGGL((ggm_repack_kernel<OXQ_GGUF_Q5_K>), grid, block, 0, s, w, (uint8_t *)pw, (int)K, (int)N, (int)gate_half); break;
     default: return fail(OXQ_ERR_UNSUPPORTED, "gguf repack: format %d has no matrix-core layout", quant);
     }
     OXQ_HIP_CHECK(hipGetLastError());
     return OXQ_OK;
 }
 
-int launch_gguf_mfma_dequant(oxq_ctx *ctx, hipStream_t s, int quant, const void *pw, int64_t K, int64_t N, float *out_nk) {
+int launch_gguf_mfma_dequant(oxq_ctx *ctx, hipStream_t s, int quant, const void *pw, int64_t K, int64_t N, float *out_nk,
+                             int64_t gate_half) {
     const size_t threads = (size_t)(N / 16) * (K / 128) * 64;
     dim3 grid((unsigned)ceil_div((int64_t)threads, 256)), block(256);
     char name[64];
@@ -633,14 +689,14 @@ int launch_gguf_mfma_dequant(oxq_ctx *ctx, hipStream_t s, int quant, const void 
     set_plan(ctx, name, grid, block, 1, 1, 0);
     if (ctx->plan_only) return OXQ_OK;
     switch (quant) {
-    case OXQ_GGUF_Q4_0: hipLaunchKernelGGL((ggm_dequant_kernel<OXQ_GGUF_Q4_0>), grid, block, 0, s, (const uint8_t *)pw, out_nk, (int)K, (int)N); break;
-    case OXQ_GGUF_Q8_0: hipLaunchKernelGGL((ggm_dequant_kernel<OXQ_GGUF_Q8_0>), grid, block, 0, s, (const uint8_t *)pw, out_nk, (int)K, (int)N); break;
-    case OXQ_GGUF_Q4_K: hipLaunchKernelGGL((ggm_dequant_kernel<OXQ_GGUF_Q4_K>), grid, block, 0, s, (const uint8_t *)pw, out_nk, (int)K, (int)N); break;
-    case OXQ_GGUF_Q6_K: hipLaunchKernelGGL((ggm_dequant_kernel<OXQ_GGUF_Q6_K>), grid, block, 0, s, (const uint8_t *)pw, out_nk, (int)K, (int)N); break;
-    case OXQ_GGUF_Q4_1: hipLaunchKernelGGL((ggm_dequant_kernel<OXQ_GGUF_Q4_1>), grid, block, 0, s, (const uint8_t *)pw, out_nk, (int)K, (int)N); break;
-    case OXQ_GGUF_Q5_0: hipLaunchKernelGGL((ggm_dequant_kernel<OXQ_GGUF_Q5_0>), grid, block, 0, s, (const uint8_t *)pw, out_nk, (int)K, (int)N); break;
-    case OXQ_GGUF_Q5_1: hipLaunchKernelGGL((ggm_dequant_kernel<OXQ_GGUF_Q5_1>), grid, block, 0, s, (const uint8_t *)pw, out_nk, (int)K, (int)N); break;
-    case OXQ_GGUF_Q5_K: hipLaunchKernelGGL((ggm_dequant_kernel<OXQ_GGUF_Q5_K>), grid, block, 0, s, (const uint8_t *)pw, out_nk, (int)K, (int)N); break;
+    case OXQ_GGUF_Q4_0: hipLaunchKernelGGL((ggm_dequant_kernel<OXQ_GGUF_Q4_0>), grid, block, 0, s, (const uint8_t *)pw, out_nk, (int)K, (int)N, (int)gate_half); break;
+    case OXQ_GGUF_Q8_0: hipLaunchKernelGGL((ggm_dequant_kernel<OXQ_GGUF_Q8_0>), grid, block, 0, s, (const uint8_t *)pw, out_nk, (int)K, (int)N, (int)gate_half); break;
+    case OXQ_GGUF_Q4_K: hipLaunchKernelGGL((ggm_dequant_kernel<OXQ_GGUF_Q4_K>), grid, block, 0, s, (const uint8_t *)pw, out_nk, (int)K, (int)N, (int)gate_half); break;
+    case OXQ_GGUF_Q6_K: hipLaunchKernelGGL((ggm_dequant_kernel<OXQ_GGUF_Q6_K>), grid, block, 0, s, (const uint8_t *)pw, out_nk, (int)K, (int)N, (int)gate_half); break;
+    case OXQ_GGUF_Q4_1: hipLaunchKernelGGL((ggm_dequant_kernel<OXQ_GGUF_Q4_1>), grid, block, 0, s, (const uint8_t *)pw, out_nk, (int)K, (int)N, (int)gate_half); break;
+    case OXQ_GGUF_Q5_0: hipLaunchKernelGGL((ggm_dequant_kernel<OXQ_GGUF_Q5_0>), grid, block, 0, s, (const uint8_t *)pw, out_nk, (int)K, (int)N, (int)gate_half); break;
+    case OXQ_GGUF_Q5_1: hipLaunchKernelGGL((ggm_dequant_kernel<OXQ_GGUF_Q5_1>), grid, block, 0, s, (const uint8_t *)pw, out_nk, (int)K, (int)N, (int)gate_half); break;
+    case OXQ_GGUF_Q5_K: hipLaunchKernelGGL((ggm_dequant_kernel<OXQ_GGUF_Q5_K>), grid, block, 0, s, (const uint8_t *)pw, out_nk, (int)K, (int)N, (int)gate_half); break;
     default: return fail(OXQ_ERR_UNSUPPORTED, "gguf dequant: format %d has no matrix-core layout", quant);
     }
     OXQ_HIP_CHECK(hipGetLastError());
@@ -653,7 +709,7 @@ static int ggm_go(hipStream_t s, dim3 grid, const GgufProblem &p, float *ws, int
     const size_t lds = (size_t)NW * MT * 4096;
     OXQ_HIP_CHECK(lds_grant.ensure((const void *)ggm_kernel<FMT, MT, XQ, NW, NS>, lds));
     hipLaunchKernelGGL((ggm_kernel<FMT, MT, XQ, NW, NS>), grid, dim3(NW * 64), lds, s, (const uint16_t *)p.x, p.w,
-                       (const uint16_t *)p.bias, (uint16_t *)p.y, ws, (int)p.M, (int)p.K, (int)p.N, cslice);
+                       (const uint16_t *)p.bias, (uint16_t *)p.y, ws, (int)p.M, (int)p.K, (int)p.N, cslice, p.act);
     OXQ_HIP_CHECK(hipGetLastError());
     return OXQ_OK;
 }
@@ -690,7 +746,10 @@ bool gguf_mfma_takes(const oxq_ctx *ctx, int64_t M, int64_t, int act_dtype) {
     return act_dtype == OXQ_BF16 && M >= 1 && M <= std::min<int64_t>(32, tune(ctx, OXQ_TUNE_GGUF_MFMA_MAX_M, 32));
 }
 
-// p.w is the matrix-core copy
+// p.w is the matrix-core copy; p.act: 0, or 1 + the gated activation of a fused gate|up layer, whose y is [M, N / 2].
+// More rows than gguf_mfma_takes allows run as row tiles of the grid (every tile reads the weights again: the
+// callers send such calls elsewhere where they can).
+
 int launch_gguf_mfma(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p) {
     const int ns = ggm_strips(ctx, p.N);
     const int mt = p.M > 16 ? 2 : 1;
@@ -700,7 +759,7 @@ int launch_gguf_mfma(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p) {
     const int nw = (p.K / 128 < 16 || mt == 2 || ns == 4) ? 8 : 16;
     dim3 grid((unsigned)(p.N / (16 * ns)), 1, (unsigned)ceil_div(p.M, (int64_t)16 * mt));
     char name[64];
-    snprintf(name, sizeof name, "gguf_%s_mfma_bf16_mt%d%s", ggm_name(p.quant), mt, ns == 4 ? "_n64" : "");
+    snprintf(name, sizeof name, "gguf_%s_mfma_bf16_mt%d%s%s", ggm_name(p.quant), mt, ns == 4 ? "_n64" : "", p.act ? "_act" : "");
     set_plan(ctx, name, grid, dim3(nw * 64), 1, 1, 0);
     if (ctx->plan_only) return OXQ_OK;
     if (p.act_dtype != OXQ_BF16) return fail(OXQ_ERR_UNSUPPORTED, "gguf matrix-core matmul: activations must be BF16");

@@ -874,7 +874,7 @@ static bool wcache_forward_gguf(oxq_ctx *ctx, hipStream_t s, const GgufProblem &
         }
         oxq_weight_cache::Entry e{p.w, nullptr, nullptr, p.K, p.N, 0, 0, p.quant, kind,
                                   Pk4Weights{(uint32_t *)mem, nullptr, p.K, p.N, 0, 0, 0, 0, 0, 0}, bytes, 0, false};
-        const int prc = (mfma ? launch_gguf_mfma_repack : launch_gguf_res_repack)(ctx, s, p.quant, p.w, mem, p.K, p.N);
+        const int prc = mfma ? launch_gguf_mfma_repack(ctx, s, p.quant, p.w, mem, p.K, p.N) : launch_gguf_res_repack(ctx, s, p.quant, p.w, mem, p.K, p.N);
         if (prc != OXQ_OK) {
             (void)hipFree(mem);
             *rc = prc;
@@ -1922,6 +1922,7 @@ struct oxq_qlinear {
     void *res = nullptr;    // layer-owned strip-major copy of the blocks
     bool resident = false;
     bool mfma = false;      // the copy is the matrix-core layout (bf16 layers), else the rotated one of the vector GEMV
+    int act = 0;            // 0, or 1 + oxq_gated_act of a fused gate|up layer (matrix-core copy only)
 };
 
 // linear.rs:225-240: the fast path copies the block bytes at build; here the copy is strip-major
@@ -1932,6 +1933,7 @@ static int build_resident_gguf(oxq_qlinear *l) {
     oxq_ctx *ctx = l->ctx;
     // a bf16 layer (the reference's GPU path: bf16 x and y) of a format that has it takes the matrix-core layout
     l->mfma = l->out_dtype == OXQ_BF16 && gguf_mfma_eligible(ctx, l->quant, l->in_features, l->out_features);
+    if (l->act && !l->mfma) return OXQ_OK;  // the caller reports it
     if (ctx->plan_only) {
         l->resident = true;
         return OXQ_OK;
@@ -1945,8 +1947,10 @@ static int build_resident_gguf(oxq_qlinear *l) {
         l->res = nullptr;
         rc = fail(OXQ_ERR_RUNTIME, "QLinear: repack allocation failed: %s", hipGetErrorString(e));
     } else {
-        rc = (l->mfma ? launch_gguf_mfma_repack : launch_gguf_res_repack)(
-            ctx, nullptr, l->quant, (const uint8_t *)l->weight_bytes.data, l->res, l->in_features, l->out_features);
+        const uint8_t *src = (const uint8_t *)l->weight_bytes.data;
+        rc = l->mfma ? launch_gguf_mfma_repack(ctx, nullptr, l->quant, src, l->res, l->in_features, l->out_features,
+                                               l->act ? l->out_features / 2 : 0)
+                     : launch_gguf_res_repack(ctx, nullptr, l->quant, src, l->res, l->in_features, l->out_features);
         if (rc == OXQ_OK && (e = hipStreamSynchronize(nullptr)) != hipSuccess)
             rc = fail(OXQ_ERR_RUNTIME, "QLinear: repack failed: %s", hipGetErrorString(e));
     }
@@ -2127,9 +2131,8 @@ void oxq_packed_quant_linear_free(oxq_packed_quant_linear *l) {
 }
 
 // linear.rs:197-247 GgufFastPath::build
-int oxq_qlinear_new(oxq_ctx *ctx, int quant, const oxq_tensor *weight_bytes, int64_t in_features,
-                    int64_t out_features, const oxq_tensor *bias, int out_dtype, oxq_qlinear **out) {
-    const char *op = "QLinear";
+static int new_qlinear(const char *op, oxq_ctx *ctx, int quant, const oxq_tensor *weight_bytes, int64_t in_features,
+                       int64_t out_features, const oxq_tensor *bias, int act, int out_dtype, oxq_qlinear **out) {
     if (!ctx || !out) return fail(OXQ_ERR_ARG, "%s: NULL argument", op);
     *out = nullptr;
     int64_t be, bb;
@@ -2158,13 +2161,40 @@ int oxq_qlinear_new(oxq_ctx *ctx, int quant, const oxq_tensor *weight_bytes, int
     l->out_features = out_features;
     l->quant = quant;
     l->out_dtype = out_dtype;
-    const int rc = build_resident_gguf(l);
+    l->act = act;
+    int rc = build_resident_gguf(l);
+    if (rc == OXQ_OK && act && !(l->resident && l->mfma))
+        rc = fail(OXQ_ERR_UNSUPPORTED,
+                  "%s: the fused activation needs a BF16 layer on the matrix-core copy (Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, "
+                  "Q4_K, Q5_K or Q6_K, out_features a multiple of 16, in_features of 128 or 256, OXQ_PREPACK and "
+                  "OXQ_GGUF_MFMA not 0); build a plain layer and call oxq_gated_activation on its output instead",
+                  op);
     if (rc != OXQ_OK) {
         oxq_qlinear_free(l);
         return rc;
     }
     *out = l;
     return OXQ_OK;
+}
+
+int oxq_qlinear_new(oxq_ctx *ctx, int quant, const oxq_tensor *weight_bytes, int64_t in_features,
+                    int64_t out_features, const oxq_tensor *bias, int out_dtype, oxq_qlinear **out) {
+    return new_qlinear("QLinear", ctx, quant, weight_bytes, in_features, out_features, bias, 0, out_dtype, out);
+}
+
+int oxq_qlinear_new_gate_up(oxq_ctx *ctx, int quant, const oxq_tensor *weight_bytes, int64_t in_features,
+                            int64_t out_features, const oxq_tensor *bias, int act, int out_dtype, oxq_qlinear **out) {
+    const char *op = "QLinear(gate|up)";
+    if (act != OXQ_ACT_GATED_SILU && act != OXQ_ACT_GATED_GELU_TANH)
+        return fail(OXQ_ERR_ARG, "%s: activation must be OXQ_ACT_GATED_SILU or OXQ_ACT_GATED_GELU_TANH, got %d", op, act);
+    if (out_features % 2 != 0) return fail(OXQ_ERR_SHAPE, "%s: out_features %lld is not gate and up halves", op, (long long)out_features);
+    return new_qlinear(op, ctx, quant, weight_bytes, in_features, out_features, bias, act + 1, out_dtype, out);
+}
+
+// what forward does when the layer has no copy, or more rows than the copy's kernels take: the file layout
+static int qlinear_forward_file_layout(oxq_qlinear *l, void *stream, const GgufProblem &p) {
+    if (gguf_mm_eligible(l->ctx, p)) return launch_gguf_mm(l->ctx, (hipStream_t)stream, p);
+    return launch_gguf_gemv(l->ctx, (hipStream_t)stream, p);
 }
 
 // linear.rs:324-351 QLinear::forward (fast-path arm), 250-284 forward_decode/prefill
@@ -2174,12 +2204,24 @@ int oxq_qlinear_forward(oxq_qlinear *l, void *stream, const oxq_tensor *x, const
     oxq_tensor x2, o2;
     int64_t m;
     OXQ_TRY(flatten_rows(op, x, l->in_features, &x2, &m));
-    OXQ_TRY(flatten_out(op, out, m, l->out_features, &o2));
+    OXQ_TRY(flatten_out(op, out, m, l->act ? l->out_features / 2 : l->out_features, &o2));
     if (out->dtype != l->out_dtype)
         return fail(OXQ_ERR_DTYPE, "%s: out dtype %s != layer out dtype %s", op,
                     dtype_name(out->dtype), dtype_name(l->out_dtype));
     GgufProblem p;
     const bool decode = m >= 1 && m <= 8;  // GGUF_BATCH_MAX, metal_ops.rs:5324
+    if (l->act) {
+        // the fused activation lives in the matrix-core kernel: every row count runs there, in row tiles of 32
+        oxq_tensor full = o2;  // check_gguf sees the projection's own shape
+        full.dims[full.rank - 1] = l->out_features;
+        OXQ_TRY(check_gguf(l->ctx, "GgufQuantMulMM", false, false, &x2, &l->weight_bytes, l->in_features, l->out_features,
+                           l->quant, &full, &p));
+        if ((uintptr_t)p.x & 15) return fail(OXQ_ERR_UNSUPPORTED, "%s: x must be 16-byte aligned", op);
+        p.bias = l->has_bias ? l->bias.data : nullptr;
+        p.w = (const uint8_t *)l->res;
+        p.act = l->act;
+        return launch_gguf_mfma(l->ctx, (hipStream_t)stream, p);
+    }
     OXQ_TRY(check_gguf(l->ctx, decode ? "GgufQuantMatmul" : "GgufQuantMulMM", decode, false, &x2,
                        &l->weight_bytes, l->in_features, l->out_features, l->quant, &o2, &p));
     p.bias = l->has_bias ? l->bias.data : nullptr;
@@ -2192,8 +2234,18 @@ int oxq_qlinear_forward(oxq_qlinear *l, void *stream, const oxq_tensor *x, const
         p.w = (const uint8_t *)l->res;
         return launch_gguf_res_gemv(l->ctx, (hipStream_t)stream, p);
     }
-    if (gguf_mm_eligible(l->ctx, p)) return launch_gguf_mm(l->ctx, (hipStream_t)stream, p);
-    return launch_gguf_gemv(l->ctx, (hipStream_t)stream, p);
+    return qlinear_forward_file_layout(l, stream, p);
+}
+
+// The projection of a fused gate|up layer without its activation, [m, out_features], from the file layout: for
+// callers that hold scratch for it (FeedForward at more rows than the fused kernel should take).
+static int qlinear_forward_unfused(oxq_qlinear *l, void *stream, const oxq_tensor *x2, const oxq_tensor *gu) {
+    GgufProblem p;
+    const bool decode = x2->dims[0] >= 1 && x2->dims[0] <= 8;
+    OXQ_TRY(check_gguf(l->ctx, decode ? "GgufQuantMatmul" : "GgufQuantMulMM", decode, false, x2, &l->weight_bytes,
+                       l->in_features, l->out_features, l->quant, gu, &p));
+    p.bias = l->has_bias ? l->bias.data : nullptr;
+    return qlinear_forward_file_layout(l, stream, p);
 }
 
 int oxq_qlinear_is_resident(const oxq_qlinear *l, int *resident) {
@@ -2210,9 +2262,12 @@ int oxq_qlinear_dequantize(oxq_qlinear *l, void *stream, const oxq_tensor *out) 
         return fail(OXQ_ERR_SHAPE, "%s: out must be F32 [%lld, %lld]", op, (long long)l->out_features,
                     (long long)l->in_features);
     if (!out->contiguous) return fail(OXQ_ERR_CONTIGUOUS, "%s: out must be contiguous", op);
+    if (l->resident && l->mfma)
+        return launch_gguf_mfma_dequant(l->ctx, (hipStream_t)stream, l->quant, l->res, l->in_features, l->out_features,
+                                        (float *)out->data, l->act ? l->out_features / 2 : 0);
     if (l->resident)
-        return (l->mfma ? launch_gguf_mfma_dequant : launch_gguf_res_dequant)(
-            l->ctx, (hipStream_t)stream, l->quant, l->res, l->in_features, l->out_features, (float *)out->data);
+        return launch_gguf_res_dequant(l->ctx, (hipStream_t)stream, l->quant, l->res, l->in_features, l->out_features,
+                                       (float *)out->data);
     GgufProblem p{};
     p.w = (const uint8_t *)l->weight_bytes.data;
     p.K = l->in_features, p.N = l->out_features, p.quant = l->quant, p.act_dtype = OXQ_F32;
@@ -2314,7 +2369,7 @@ static int linear_info(const char *op, const char *name, const oxq_any_linear *l
     }
     case OXQ_LINEAR_GGUF: {
         const oxq_qlinear *q = (const oxq_qlinear *)l->layer;
-        *info = LinearInfo{q->ctx, q->in_features, q->out_features, q->out_dtype, 0};
+        *info = LinearInfo{q->ctx, q->in_features, q->act ? q->out_features / 2 : q->out_features, q->out_dtype, q->act};
         return OXQ_OK;
     }
     case OXQ_LINEAR_MXFP4: {
@@ -2341,7 +2396,8 @@ static int linear_forward(const oxq_any_linear &l, void *stream, const oxq_tenso
 // elements of `mid_dtype` that forward keeps between the projections, per row of x
 static int64_t mlp_scratch_per_row(const oxq_mlp *m) {
     switch (m->gate_up_kind) {
-    case OXQ_GATE_UP_FUSED: return m->epilogue ? m->intermediate : 3 * m->intermediate;
+    // (a GGUF layer with the fused activation runs many rows unfused, on the file layout)
+    case OXQ_GATE_UP_FUSED: return (m->epilogue && m->a.kind != OXQ_LINEAR_GGUF) ? m->intermediate : 3 * m->intermediate;
     case OXQ_GATE_UP_SEPARATE: return 2 * m->intermediate;
     default: return m->intermediate;
     }
@@ -2444,7 +2500,13 @@ int oxq_mlp_forward(oxq_mlp *m, void *stream, const oxq_tensor *x, const oxq_ten
     oxq_tensor h;  // [rows, I]: act(gate) * up, the input of down_proj
     switch (m->gate_up_kind) {
     case OXQ_GATE_UP_FUSED:
-        if (m->epilogue) {
+        if (m->epilogue && m->a.kind == OXQ_LINEAR_GGUF && rows > OXQ_GGUF_FUSED_ACT_ROWS) {
+            // every row tile of the fused kernel reads the weights again: the tile matmul and the activation by itself
+            const oxq_tensor gu = rows_view(scratch, 0, rows, 2 * I);
+            h = rows_view(scratch, rows * 2 * I, rows, I);
+            OXQ_TRY(qlinear_forward_unfused((oxq_qlinear *)m->a.layer, stream, &x2, &gu));
+            OXQ_TRY(oxq_gated_activation(m->ctx, stream, &gu, m->activation, 0.0f, &h));
+        } else if (m->epilogue) {
             h = rows_view(scratch, 0, rows, I);
             OXQ_TRY(linear_forward(m->a, stream, &x2, &h));
         } else {

@@ -141,6 +141,7 @@ struct GgufProblem {
     int64_t M, K, N;
     int quant;
     int act_dtype;          // OXQ_BF16 or OXQ_F32
+    int act = 0;            // matrix-core copy of a fused gate|up layer: 1 + the gated activation (y is [M, N / 2])
 };
 
 struct Mxfp4Problem {
@@ -229,8 +230,10 @@ int launch_gguf_res_gemv(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p);  //
 // matrix-core copy of a GGUF weight for 16-bit activations and its matmul (gguf_mfma.hip)
 bool gguf_mfma_eligible(const oxq_ctx *ctx, int quant, int64_t K, int64_t N);
 bool gguf_mfma_takes(const oxq_ctx *ctx, int64_t M, int64_t N, int act_dtype);
-int launch_gguf_mfma_repack(oxq_ctx *ctx, hipStream_t s, int quant, const uint8_t *w, void *pw, int64_t K, int64_t N);
-int launch_gguf_mfma_dequant(oxq_ctx *ctx, hipStream_t s, int quant, const void *pw, int64_t K, int64_t N, float *out_nk);
+int launch_gguf_mfma_repack(oxq_ctx *ctx, hipStream_t s, int quant, const uint8_t *w, void *pw, int64_t K, int64_t N,
+                            int64_t gate_half = 0);
+int launch_gguf_mfma_dequant(oxq_ctx *ctx, hipStream_t s, int quant, const void *pw, int64_t K, int64_t N, float *out_nk,
+                             int64_t gate_half = 0);
 int launch_gguf_mfma(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p);  // p.w = the copy
 bool gguf_mm_eligible(const oxq_ctx *ctx, const GgufProblem &p);
 int launch_gguf_mm(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p);

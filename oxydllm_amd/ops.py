@@ -654,15 +654,24 @@ class QLinear:
     """linear.rs:179-393 (GGUF fast path)."""
 
     def __init__(self, quant: int, weight_bytes, in_features: int, out_features: int, bias=None,
-                 out_dtype=torch.bfloat16, ctx: Optional[Context] = None):
+                 out_dtype=torch.bfloat16, ctx: Optional[Context] = None, gate_up_act: Optional[int] = None):
+        """``gate_up_act`` (ACT_GATED_SILU / ACT_GATED_GELU_TANH) makes this the fused gate|up projection of a
+        block-quantized FFN (ffn.rs:307-373 GateUpProjection::Packed): ``weight_bytes`` holds the gate rows followed
+        by the up rows (``out_features`` = 2 I) and forward returns act(gate(x)) * up(x), [.., I]."""
         self.ctx = _ctx(ctx)
         self._keep = (weight_bytes, bias)
         self.handle = C.c_void_p()
         self.in_features = in_features
-        self.out_features = out_features
-        _lib.check(self.ctx._lib.oxq_qlinear_new(
-            self.ctx.handle, quant, desc(weight_bytes), in_features, out_features, desc(bias),
-            _DTYPES[out_dtype], C.byref(self.handle)))
+        self.weight_rows = out_features
+        self.out_features = out_features if gate_up_act is None else out_features // 2
+        if gate_up_act is None:
+            _lib.check(self.ctx._lib.oxq_qlinear_new(
+                self.ctx.handle, quant, desc(weight_bytes), in_features, out_features, desc(bias),
+                _DTYPES[out_dtype], C.byref(self.handle)))
+        else:
+            _lib.check(self.ctx._lib.oxq_qlinear_new_gate_up(
+                self.ctx.handle, quant, desc(weight_bytes), in_features, out_features, desc(bias), gate_up_act,
+                _DTYPES[out_dtype], C.byref(self.handle)))
 
     def forward(self, x: torch.Tensor, out=None) -> torch.Tensor:
         if out is None:
@@ -681,7 +690,7 @@ class QLinear:
 
     def dequantize(self) -> torch.Tensor:
         """Dense f32 [out_features, in_features], read from the layer's copy when it holds one."""
-        out = torch.empty((self.out_features, self.in_features), dtype=torch.float32,
+        out = torch.empty((self.weight_rows, self.in_features), dtype=torch.float32,
                           device=self._keep[0].device)
         _lib.check(self.ctx._lib.oxq_qlinear_dequantize(self.handle, self.ctx.stream(), desc(out)))
         return out

@@ -337,6 +337,27 @@ def test_feed_forward_validates_and_plans(lib, ctx):
                                C.byref(fake((1, H), BF16))) == 0, err(lib)
     assert plan(lib, ctx).kernel.decode().startswith("gguf_q4k_mfma_bf16_mt1")  # a bf16 layer: the matrix-core copy
     lib.oxq_mlp_free(m)
+    # the fused gate|up projection of a block-quantized FFN with the activation in its epilogue (ffn.rs:307-373 Packed)
+    both_bytes = fake((2 * I * (H // 256) * 144,), U8)
+    qf = C.c_void_p()
+    assert lib.oxq_qlinear_new_gate_up(ctx, _lib.GGUF_Q4_K, C.byref(both_bytes), H, 2 * I, None, 2, BF16, C.byref(qf)) == -1
+    assert "activation must be" in err(lib)
+    assert lib.oxq_qlinear_new_gate_up(ctx, _lib.GGUF_Q4_K, C.byref(both_bytes), H, 2 * I, None, 0, F32, C.byref(qf)) == -11
+    assert "needs a BF16 layer on the matrix-core copy" in err(lib)
+    assert lib.oxq_qlinear_new_gate_up(ctx, _lib.GGUF_Q4_K, C.byref(both_bytes), H, 2 * I, None, 0, BF16, C.byref(qf)) == 0, err(lib)
+    assert lib.oxq_qlinear_forward(qf, None, C.byref(fake((3, H), BF16)), C.byref(fake((3, 2 * I), BF16))) == -3
+    assert lib.oxq_qlinear_forward(qf, None, C.byref(fake((3, H), BF16)), C.byref(fake((3, I), BF16))) == 0, err(lib)
+    assert plan(lib, ctx).kernel.decode() == "gguf_q4k_mfma_bf16_mt1_n64_act"
+    rc, m = new(0, qf, None, qd, lk=1)
+    assert rc == 0, err(lib)
+    elems = C.c_int64()
+    assert lib.oxq_mlp_scratch_elems(m, 2, C.byref(elems)) == 0 and elems.value == 2 * 3 * I
+    for rows, kern in [(2, "gguf_q4k_mfma_bf16_mt1"), (100, "gguf_q4k_mul_mm_bf16")]:  # the down projection ran last
+        assert lib.oxq_mlp_forward(m, None, C.byref(fake((rows, H), BF16)), C.byref(fake((rows * 3 * I,), BF16)),
+                                   C.byref(fake((rows, H), BF16))) == 0, err(lib)
+        assert plan(lib, ctx).kernel.decode().startswith(kern), plan(lib, ctx).kernel
+    lib.oxq_mlp_free(m)
+    lib.oxq_qlinear_free(qf)
     for h in (qg, qu, qd):
         lib.oxq_qlinear_free(h)
     for h in (gate, up, both, epi, down):

@@ -58,6 +58,40 @@ def test_gguf_file_to_qlinear(tmp_path):
                 d.qlinear("dense")
 
 
+@pytest.mark.parametrize("layout", ["separate", "packed"])
+def test_gguf_file_to_feed_forward_fuses_gate_and_up(tmp_path, layout):
+    """ffn.rs:307-373 FeedForward::load_gguf.  With fuse (the default) a bf16 layer of a format with the matrix-core
+    copy becomes one gate|up projection with the activation in its epilogue - separate ffn_gate / ffn_up tensors by
+    concatenating their bytes - and gives the bits of the layer built the reference's way; a format without that
+    copy keeps its layout."""
+    from oxydllm_amd import ops
+    H, I = 512, 256
+    for fmt, fusable in [(synth.GGUF_Q4_K, True), (synth.GGUF_Q5_0, True), (synth.GGUF_Q2_K, False)]:
+        gate, up = synth.gguf_weight(fmt, I, H, seed=1), synth.gguf_weight(fmt, I, H, seed=2)
+        down = synth.gguf_weight(fmt, H, I, seed=3)
+        G_ = G.GGML_OF_QUANT[fmt]
+        if layout == "separate":
+            tensors = [("blk.0.ffn_gate.weight", (I, H), G_, gate.tobytes()), ("blk.0.ffn_up.weight", (I, H), G_, up.tobytes())]
+        else:
+            tensors = [("blk.0.ffn_up.weight", (2 * I, H), G_, gate.tobytes() + up.tobytes())]
+        tensors.append(("blk.0.ffn_down.weight", (H, I), G_, down.tobytes()))
+        path = str(tmp_path / f"ffn_{fmt}.gguf")
+        G.write_gguf(path, [("general.architecture", G.STRING, "llama")], tensors)
+        with ck.GgufWeights.load(path) as w:
+            ff = w.feed_forward(0, I)
+            ref = w.feed_forward(0, I, fuse=False)
+            assert ref.gate_up_kind == (ops.GATE_UP_SEPARATE if layout == "separate" else ops.GATE_UP_FUSED)
+            assert ff.gate_up_kind == (ops.GATE_UP_FUSED if fusable else ref.gate_up_kind)
+            for m in (1, 8, 40):
+                x = to_dev(_x(m, H, seed=m) * 0.25, torch.bfloat16)
+                y = ff.forward(x)
+                np.testing.assert_array_equal(y.view(torch.int16).cpu().numpy(), ref.forward(x).view(torch.int16).cpu().numpy())
+            if fusable:
+                a = ff._keep[0]
+                a.forward(to_dev(_x(2, H, seed=5), torch.bfloat16))
+                assert ops.default_context().last_plan()["kernel"].endswith("_act")
+
+
 @pytest.mark.parametrize("method, bits", [("awq", 4), ("awq", 8), ("gptq", 4), ("gptq", 8)])
 def test_safetensors_file_to_packed_linear(tmp_path, method, bits):
     from safetensors.numpy import save_file

@@ -171,3 +171,100 @@ def test_matrix_core_layer_replays_in_a_graph(fmt):
         g.replay()
         torch.cuda.synchronize()
         assert np.array_equal(bits_of(y), want), f"replay {i}"
+
+
+# ------------------------------------------------------------------ fused gate|up activation
+@pytest.mark.parametrize("fmt", FMTS)
+@pytest.mark.parametrize("act", ["silu", "gelu_tanh"])
+def test_fused_gate_up_activation_gives_the_two_call_bits(fmt, act):
+    """ffn.rs:386-413: the fused projection's output goes through gated_silu_fused / gated_gelu_tanh_fused.  The layer
+    built with gate_up_act runs that in its epilogue; it must give, bit for bit, what the plain layer followed by
+    oxq_gated_activation gives - at every row count the plain layer runs on the same kernel (up to 32), with and
+    without bias, one strip and four strips a workgroup.  The paired repack is pinned by the dense dequant."""
+    kind = ops.ACT_GATED_SILU if act == "silu" else ops.ACT_GATED_GELU_TANH
+    name = synth.GGUF_NAMES[fmt]
+    for K, I, ns in [(1024, 64, 1), (2304 + 256, 96, 1), (512, 128, 4)]:
+        N = 2 * I
+        data = synth.gguf_weight(fmt, N, K, seed=K + I + fmt)
+        wd = to_dev(data)
+        for with_bias in (False, True):
+            bias = ((np.arange(N, dtype=np.float32) % 9) - 4) * np.float32(0.5) if with_bias else None
+            bd = None if bias is None else to_dev(bias, torch.bfloat16)
+            tune("OXQ_GGUF_MFMA_NS", ns)
+            plain = ops.QLinear(fmt, wd, K, N, bd, torch.bfloat16)
+            fused = ops.QLinear(fmt, wd, K, N, bd, torch.bfloat16, gate_up_act=kind)
+            assert fused.resident and fused.out_features == I
+            want = oracle.dequantize_gguf(fmt, data, N, K)
+            assert np.array_equal(fused.dequantize().cpu().numpy().view(np.uint32), want.view(np.uint32)), "paired repack"
+            for m in (1, 3, 8, 13, 16, 17, 32):
+                say(f"gguf fused gate|up {name} {act} K={K} I={I} ns={ns} bias={with_bias} m={m}")
+                x = np.random.default_rng(K + m).standard_normal((m, K)).astype(np.float32)
+                xd = to_dev(x, torch.bfloat16)
+                y = fused.forward(xd)
+                plan = ops.default_context().last_plan()
+                assert plan["kernel"].endswith("_act") and "_mfma_bf16_mt" in plan["kernel"] and plan["launches"] == 1, plan
+                assert tuple(y.shape) == (m, I)
+                gu = plain.forward(xd)
+                assert "_mfma_bf16_mt" in ops.default_context().last_plan()["kernel"]
+                two = ops.gated_activation(gu, kind)
+                np.testing.assert_array_equal(bits_of(y), bits_of(two))
+            tune("OXQ_GGUF_MFMA_NS", None)
+
+
+@pytest.mark.parametrize("fmt", [synth.GGUF_Q4_K, synth.GGUF_Q6_K])
+def test_fused_gate_up_rows_beyond_a_tile_and_refusals(fmt):
+    """More than 32 rows run as row tiles of the same launch: every tile gives what a call on its rows gives (8-wave
+    workgroups at this K for every row count, so the sums run in the same order)."""
+    K, I = 1024, 64
+    N = 2 * I
+    data = synth.gguf_weight(fmt, N, K, seed=71 + fmt)
+    wd = to_dev(data)
+    fused = ops.QLinear(fmt, wd, K, N, None, torch.bfloat16, gate_up_act=ops.ACT_GATED_SILU)
+    x = np.random.default_rng(72).standard_normal((70, K)).astype(np.float32)
+    xd = to_dev(x, torch.bfloat16)
+    say(f"gguf fused gate|up {synth.GGUF_NAMES[fmt]} 70 rows")
+    y = bits_of(fused.forward(xd))
+    plan = ops.default_context().last_plan()
+    assert plan["grid"] == (N // 16, 1, 3) and plan["kernel"].endswith("_mt2_act"), plan
+    for r0 in (0, 32):
+        np.testing.assert_array_equal(y[r0:r0 + 32], bits_of(fused.forward(xd[r0:r0 + 32].contiguous())))
+    g, u = oracle.matmul_nt_f32(round_x(x, oracle.BF16), oracle.dequantize_gguf(fmt, data, N, K)).reshape(70, 2, I).transpose(1, 0, 2)
+    g, u = oracle.round_through(g, oracle.BF16), oracle.round_through(u, oracle.BF16)
+    ref = g / (1.0 + np.exp(-g.astype(np.float64))) * u
+    # both factors are rounded to bf16 before the product: where the f32 sums of kernel and oracle fall on either side
+    # of a rounding boundary, a whole bf16 ulp of that factor shows in the product
+    assert_close(torch.from_numpy(y.view(np.int16)).view(torch.bfloat16), ref.astype(np.float32), "70 rows against the oracle",
+                 rtol=2.0 ** -6)
+    with pytest.raises(ops.OxqError, match="needs a BF16 layer on the matrix-core copy"):
+        ops.QLinear(fmt, wd, K, N, None, torch.float32, gate_up_act=ops.ACT_GATED_SILU)
+    with pytest.raises(ops.OxqError, match="needs a BF16 layer on the matrix-core copy"):
+        ops.QLinear(synth.GGUF_Q2_K, to_dev(synth.gguf_weight(synth.GGUF_Q2_K, N, K, seed=1)), K, N, None, torch.bfloat16,
+                    gate_up_act=ops.ACT_GATED_SILU)
+    with pytest.raises(ops.OxqError, match="activation must be"):
+        ops.QLinear(fmt, wd, K, N, None, torch.bfloat16, gate_up_act=ops.ACT_GPT_OSS_SWIGLU)
+    with pytest.raises(ops.OxqError, match="out dtype"):
+        fused.forward(to_dev(x[:2]))
+
+
+@pytest.mark.parametrize("fmt", [synth.GGUF_Q4_0, synth.GGUF_Q4_K, synth.GGUF_Q5_K, synth.GGUF_Q6_K])
+def test_feed_forward_over_a_fused_gguf_layer(fmt):
+    """FeedForward (ffn.rs:386-474) with the fused-activation layer as gate_up_proj gives the bits of the layer built
+    over the plain fused projection: through the fused kernel up to 32 rows (where the plain projection runs on the
+    same kernel), through the file-layout matmul and the stand-alone activation above."""
+    H, I = 512, 256
+    gu = to_dev(synth.gguf_weight(fmt, 2 * I, H, seed=81 + fmt))
+    dn = to_dev(synth.gguf_weight(fmt, H, I, seed=82 + fmt))
+    down = ops.QLinear(fmt, dn, I, H, None, torch.bfloat16)
+    plain = ops.QLinear(fmt, gu, H, 2 * I, None, torch.bfloat16)
+    fused = ops.QLinear(fmt, gu, H, 2 * I, None, torch.bfloat16, gate_up_act=ops.ACT_GATED_GELU_TANH)
+    ff_plain = ops.FeedForward(ops.GATE_UP_FUSED, plain, None, down, I, ops.ACT_GATED_GELU_TANH)
+    ff_fused = ops.FeedForward(ops.GATE_UP_FUSED, fused, None, down, I, ops.ACT_GATED_GELU_TANH)
+    assert ff_fused.scratch_elems(5) == 5 * 3 * I  # room for the unfused path at many rows
+    for m in (1, 8, 32, 33, 100):
+        say(f"gguf FeedForward over a fused layer {synth.GGUF_NAMES[fmt]} m={m}")
+        x = to_dev(np.random.default_rng(m).standard_normal((m, H)).astype(np.float32) * 0.25, torch.bfloat16)
+        np.testing.assert_array_equal(bits_of(ff_fused.forward(x)), bits_of(ff_plain.forward(x)))
+    with pytest.raises(ops.OxqError, match="another activation"):
+        ops.FeedForward(ops.GATE_UP_FUSED, fused, None, down, I, ops.ACT_GATED_SILU)
+    with pytest.raises(ops.OxqError, match="only be the fused gate_up_proj"):
+        ops.FeedForward(ops.GATE_UP_SEPARATE, fused, plain, down, I, ops.ACT_GATED_GELU_TANH)
