@@ -2,6 +2,7 @@
 
 GPTQ 4/8-bit GEMV (K=5120, N=13824, g=128, M in {1, 8}); GGUF Q4_0 / Q8_0 / Q4_K /
 Q6_K ... GEMV (M=1, K=N=4096, f32 activations) and tile matmul (M=64..2048, bf16); MXFP4
+gated GGUF FFN at decode (four launches against the fused gate|up layer's two); MXFP4
 MoE expert GEMV (32 experts, top-4, 8 tokens, hidden 2880, gate_up N=5760, down K=2880),
 the same layer at 512 tokens, and one expert's gate_up at prefill sizes.  Every case rotates
 over enough weight copies to exceed the 256 MB memory-side cache and replays a
@@ -124,6 +125,35 @@ def run(ops, ctx, stream, steps, warmup, time_graph):
                                  warmup, stream, time_graph, data.nbytes + m * K * 2 + m * N * 2,
                                  2.0 * m * K * N, ctx))
         del d
+
+    # ---- a gated GGUF FFN at decode (ffn.rs:307-474): the reference's layout (gate, up, activation, down: four
+    # launches) against the fused gate|up layer with the activation in its epilogue (two launches)
+    H, I = 4096, 14336
+    for fmt in (synth.GGUF_Q4_K, synth.GGUF_Q6_K):
+        parts = [synth.gguf_weight(fmt, I, H, seed=1), synth.gguf_weight(fmt, I, H, seed=2), synth.gguf_weight(fmt, H, I, seed=3)]
+        nb_w = sum(p.nbytes for p in parts)
+        nc = 3  # 3 x 100 MB and more: beyond the memory-side cache
+        sep, fus = [], []
+        for _ in range(nc):
+            gd, ud, dd = (torch.from_numpy(p).to(dev) for p in parts)
+            down = ops.QLinear(fmt, dd, I, H, None, torch.bfloat16, ctx=ctx)
+            sep.append(ops.FeedForward(ops.GATE_UP_SEPARATE, ops.QLinear(fmt, gd, H, I, None, torch.bfloat16, ctx=ctx),
+                                       ops.QLinear(fmt, ud, H, I, None, torch.bfloat16, ctx=ctx), down, I, ctx=ctx))
+            both = torch.cat([gd.reshape(-1), ud.reshape(-1)])
+            fus.append(ops.FeedForward(ops.GATE_UP_FUSED, ops.QLinear(fmt, both, H, 2 * I, None, torch.bfloat16, ctx=ctx,
+                                                                      gate_up_act=ops.ACT_GATED_SILU), None, down, I, ctx=ctx))
+        for m in (1, 8):
+            xb = torch.randn((m, H), device=dev, dtype=torch.bfloat16) * 0.1
+            yb = torch.empty((m, H), device=dev, dtype=torch.bfloat16)
+            sc = torch.empty(m * 3 * I, device=dev, dtype=torch.bfloat16)
+            for tag, ffs, launches in (("gate, up, activation, down", sep, 4), ("fused gate|up with the activation, down", fus, 2)):
+                def ffstep(i, ffs=ffs, xb=xb, yb=yb, sc=sc):
+                    ffs[i % nc].forward(xb, out=yb, scratch=sc)
+                r = _case(f"gguf {synth.GGUF_NAMES[fmt]} FFN {H}/{I} M={m} bf16 SiLU: {tag}", ffstep, steps, warmup, stream,
+                          time_graph, nb_w + 2 * m * H * 2, 6.0 * m * H * I, ctx)
+                r["launches"] = launches
+                out.append(r)
+        del sep, fus
 
     # ---- block-scaled F8E4M3 (sibling path: streamed FP8 experts) -----------------------
     for (n8, k8) in ((4096, 4096), (2048, 512)):
