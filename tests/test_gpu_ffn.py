@@ -236,8 +236,11 @@ def test_gguf_mlp_from_file(tmp_path, layout):
     G.write_gguf(path, [("general.architecture", G.STRING, "llama")], tensors)
     with ck.GgufWeights.load(path) as w:
         ff = w.feed_forward(0, I, ops.ACT_GATED_SILU)
-        assert ff.gate_up_kind == {"separate": ops.GATE_UP_SEPARATE, "packed": ops.GATE_UP_FUSED,
+        # gate and up of one format with the matrix-core copy: fused into one projection by default
+        assert ff.gate_up_kind == {"separate": ops.GATE_UP_FUSED, "packed": ops.GATE_UP_FUSED,
                                    "simple": ops.GATE_UP_SIMPLE}[layout]
+        assert w.feed_forward(0, I, ops.ACT_GATED_SILU, fuse=False).gate_up_kind == {
+            "separate": ops.GATE_UP_SEPARATE, "packed": ops.GATE_UP_FUSED, "simple": ops.GATE_UP_SIMPLE}[layout]
         for m in (1, 6):    # the decode kernels multiply the unrounded dequantized weights
             x = _x(m, H, seed=m)
             ref = oracle_ffn(x, None if layout == "simple" else w_gate, w_up, w_down, ops.ACT_GATED_SILU, oracle.BF16)

@@ -72,7 +72,7 @@ def test_matrix_core_layer_against_oracle(fmt, N, K, ns):
         four = ns == 4
         assert plan["kernel"] == f"gguf_{TAG[fmt]}_mfma_bf16_mt{mt}" + ("_n64" if four else "") and plan["launches"] == 1, plan
         assert plan["grid"] == (N // (64 if four else 16), 1, 1), plan
-        assert plan["block"][0] == (512 if (K // 128 < 16 or mt == 2 or four) else 1024), plan
+        assert plan["block"][0] == (512 if (K // 128 < 16 or K // 128 >= 64 or mt == 2 or four) else 1024), plan
         xr = round_x(x, oracle.BF16)
         ref = oracle.matmul_nt_f32(xr, w, br)
         assert_close(y, ref, f"matrix-core {name} N={N} K={K} m={m}", bf16_out=True)
