@@ -18,11 +18,12 @@
 // call costs no getenv and two engine threads cannot race on the process environment.
 #define OXQ_TUNE_LIST(X)                                                                                      \
     X(ACT_VEC) X(F8_MM_KS) X(F8_MM_MIN_M) X(F8_MM_MT) X(FORCE_GENERIC) X(GEMV_CFG) X(GEMV_GPW) X(GEMV_TILE)   \
-    X(GGR_GRID) X(GGR_WAVES) X(GGUF_BIG_LDS) X(GGUF_MM_KS) X(GGUF_MM_MIN_M) X(GGUF_MM_MT) X(GGUF_MFMA) X(GGUF_MFMA_MAX_M) X(GGUF_MFMA_NS) X(GGUF_PW)          \
-    X(GGUF_RPWG) X(GPTQ_TILE) X(GPTQ_TILE_KS) X(MFMA_MT) X(MFMA_SPLITK) X(MFMA_VARIANT) X(MXFP4_FR)           \
-    X(MXFP4_MM) X(MXFP4_MM_KS) X(MXFP4_MM_MT) X(MXFP4_VARIANT) X(PK4N_NS1_ROWS) X(PK4N_W16)                   \
-    X(PK4_CONTIGUOUS) X(PK4_FOLD) X(PK4_FRONT) X(PK4_KS) X(PK4_PLACE64) X(PK4_STRIP16) X(PK4_T64) X(PK4_XQ)   \
-    X(PREPACK) X(SPLITK_MODE) X(TRANSIENT_REPACK)
+    X(GGR_GRID) X(GGR_WAVES) X(GGUF_BIG_LDS) X(GGUF_MFMA) X(GGUF_MFMA_MAX_M) X(GGUF_MFMA_NS) X(GGUF_MM_KS)    \
+    X(GGUF_MM_MIN_M) X(GGUF_MM_MT) X(GGUF_PW) X(GGUF_RPWG) X(GPTQ_TILE) X(GPTQ_TILE_KS) X(MFMA_MT)            \
+    X(MFMA_SPLITK) X(MFMA_VARIANT) X(MXFP4_FR) X(MXFP4_MM) X(MXFP4_MM_KS) X(MXFP4_MM_MT) X(MXFP4_VARIANT)     \
+    X(PK4N_NS1_ROWS) X(PK4N_W16) X(PK4_CONTIGUOUS) X(PK4_FOLD) X(PK4_FRONT) X(PK4_GEMM_MIN_M)                 \
+    X(PK4_GEMM_ROWS) X(PK4_KS) X(PK4_PLACE64) X(PK4_STRIP16) X(PK4_T64) X(PK4_XQ) X(PREPACK)                  \
+    X(SPLITK_MODE) X(TRANSIENT_REPACK)
 enum oxq_tune_key {
 #define OXQ_TUNE_ENUM(n) OXQ_TUNE_##n,
     OXQ_TUNE_LIST(OXQ_TUNE_ENUM)
@@ -202,6 +203,9 @@ struct Pk4Problem {
 
 // ---- launchers (defined in the .hip files) ---------------------------------
 bool pk4_eligible(const Wna16Problem &p);
+// resident 4-bit layers at prefill sizes: 64 rows x eight strips a workgroup (pk4_gemm.hip)
+bool pk4_gemm_takes(const oxq_ctx *ctx, const Pk4Problem &p);
+int launch_pk4_gemm(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p);
 size_t pk4_weight_bytes(int64_t K, int64_t N, int bits);
 int pk4_choose_strip(const oxq_ctx *ctx, int64_t K, int64_t N, int bits, int64_t gate_half);
 size_t pk4_zs_bytes(int64_t K, int64_t N, int group_shift);

@@ -1420,6 +1420,7 @@ static int launch_pk4n_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p)
 
 int launch_pk4_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p) {
     if (p.w.strip == 16) return launch_pk4n_forward(ctx, s, p);
+    if (pk4_gemm_takes(ctx, p)) return launch_pk4_gemm(ctx, s, p);
     const int64_t M = p.M;
     const int mt = M > 48 ? 4 : (int)ceil_div(M, 16);
     const int NB = (int)(p.w.K / 128);

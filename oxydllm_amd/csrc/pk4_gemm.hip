@@ -1,0 +1,225 @@
+// Resident 4-bit layers at prefill sizes (linear.rs:494-509: m >= 64 takes the staged tile GEMM,
+// mpp_gemm.metal:101-266): the tile arithmetic of pk4_mfma_kernel - B = T((q - z) * s) rounded once to the
+// activation type, f32 accumulate - in a decomposition for many rows.
+//
+// pk4_mfma_kernel gives a workgroup one strip of 64 columns and 64 rows of x, and its 8 waves split K: every
+// (row tile, strip) pair reads its 64 rows of x again, each wave for itself through the vector-memory unit.
+// At 2048 rows of a 4096 x 14336 layer that is 7168 workgroups x 512 KB = 3.7 GB of activations out of L2 for
+// 16.8 MB of x, and the kernel runs at the speed it has at 64 rows (0.6 PFLOP/s).  Here a workgroup takes 64
+// rows and EIGHT strips: its waves share one copy of the rows in LDS (loaded once per 128 elements of K by
+// all 512 threads, two buffers, one barrier a block), each wave owns a strip, streams its blocks with the
+// one-block ring of pk4_mfma_kernel and keeps the whole K in its own accumulators - no partial tiles, no
+// second launch.  x out of L2 falls to an eighth.  Workgroups are numbered so that 64 neighbours form a square
+// of 8 row tiles x 8 strip groups, whose rows of x and weights the neighbours find in L2.
+#include "oxq_device.hpp"
+#include "oxq_internal.hpp"
+#include "oxq_mfma.hpp"
+#include "pk4_common.hpp"
+
+#include <algorithm>
+#include <cmath>
+
+namespace oxq {
+
+constexpr int PK4G_STRIPS = 8;  // strips (= waves) of a workgroup
+
+template <typename TT, int MT>
+__global__ __launch_bounds__(512) void pk4_gemm_kernel(const uint16_t *__restrict__ x, const uint32_t *__restrict__ pw,
+                                                       const uint16_t *__restrict__ bias, uint16_t *__restrict__ y,
+                                                       int M, int K, int N, int NG, int RT) {
+    typedef MfmaOps<TT> Ops;
+    constexpr int ROWS = 16 * MT, BB = pk4_block_words(4) * 4, OOB = 0x7FFFFF00, XBUF = ROWS * 256;
+    constexpr int XV = ROWS / 32;  // 16-byte chunks of x a thread brings per block: 512 threads, 16 chunks a row
+    extern __shared__ __attribute__((aligned(16))) unsigned char pk4_lds[];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int ni = lane & 15, kb = lane >> 4;
+    // Bands of 8 row tiles are cut into squares of 8 row tiles x 8 strip groups, 64 neighbouring workgroups each
+    // (neighbour i runs on XCD i % 8: a row tile stays on one XCD); the last RT % 8 row tiles are numbered row
+    // tile first, so that no XCD is handed only idle workgroups.
+    const int full = (RT >> 3) * ((NG + 7) >> 3) * 64, tail = RT & 7;
+    int rt, g;
+    if ((int)blockIdx.x < full) {
+        const int sq = blockIdx.x >> 6, within = blockIdx.x & 63, bands = RT >> 3;
+        rt = (sq % bands) * 8 + (within & 7), g = (sq / bands) * 8 + (within >> 3);
+    } else {
+        const int id = blockIdx.x - full;
+        rt = (RT & ~7) + id % tail, g = id / tail;
+    }
+    if (g >= NG) return;  // the whole workgroup, before any barrier: the ragged last column of squares
+    const int j = g * PK4G_STRIPS + wave;
+    const bool live = j < (N >> 6);  // wave-uniform: the last group of a layer may have fewer than eight strips
+    const int m0 = rt * ROWS;
+    const int NB = K >> 7;
+    const int xrows = min(M - m0, ROWS);
+
+    const __amdgpu_buffer_rsrc_t rs_none = make_rsrc(pw, 0u);
+    const __amdgpu_buffer_rsrc_t rs_wl = make_rsrc(pw + (size_t)(live ? j : 0) * NB * (BB / 4), (uint32_t)NB * (uint32_t)BB);
+    const __amdgpu_buffer_rsrc_t rs_w = live ? rs_wl : rs_none;
+    const __amdgpu_buffer_rsrc_t rs_x = make_rsrc(x + (size_t)m0 * K, (uint32_t)xrows * (uint32_t)K * 2u);
+    const int voff_w = lane * 16;
+    const int voff_z = 1024 * 4 + (ni * 4 + kb) * 4;
+    // x: thread t brings XV neighbouring chunks of row t / (16 / XV) of the block; rows past M read zeros
+    const int xr = threadIdx.x / (16 / XV), xc = (threadIdx.x % (16 / XV)) * XV;
+    const int voff_x = xr < xrows ? (xr * K * 2 + xc * 16) : OOB;
+    int x_wr[XV];
+#pragma unroll
+    for (int v = 0; v < XV; ++v) x_wr[v] = xr * 256 + (((xc + v) ^ (xr & 15)) << 4);
+    int a_rd[4];  // fragment of step st, row tile mt (+ 4096 mt): row ni, chunk 8 (st / 2) + 2 kb + st % 2
+#pragma unroll
+    for (int st = 0; st < 4; ++st) a_rd[st] = ni * 256 + (((8 * (st >> 1) + 2 * kb + (st & 1)) ^ ni) << 4);
+    const NibbleMasks nm = nibble_masks();
+
+    u32x4_t xq[XV], wring[4];
+    uint32_t zring;
+    auto load_x = [&](int i) {
+        const __amdgpu_buffer_rsrc_t rs = i < NB ? rs_x : rs_none;
+#pragma unroll
+        for (int v = 0; v < XV; ++v) xq[v] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff_x + 16 * v, i * 256, 0);
+    };
+    auto store_x = [&](int i) {
+        unsigned char *buf = pk4_lds + (i & 1) * XBUF;
+#pragma unroll
+        for (int v = 0; v < XV; ++v) *(u32x4_t *)(buf + x_wr[v]) = xq[v];
+    };
+    auto load_w = [&](int i, int st) {
+        const __amdgpu_buffer_rsrc_t rs = i < NB ? rs_w : rs_none;
+        wring[st] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff_w, i * BB + st * 1024, 0);
+    };
+    auto load_z = [&](int i) {
+        const __amdgpu_buffer_rsrc_t rs = i < NB ? rs_w : rs_none;
+        zring = __builtin_amdgcn_raw_buffer_load_b32(rs, voff_z, i * BB, 0);
+    };
+    auto zs_words = [&](uint32_t z, uint32_t (&zv)[4]) {
+        const auto p16 = __builtin_amdgcn_permlane16_swap(z, z, false, false);
+        const uint32_t even = p16[0], odd = p16[1];
+        const auto pe = __builtin_amdgcn_permlane32_swap(even, even, false, false);
+        const auto po = __builtin_amdgcn_permlane32_swap(odd, odd, false, false);
+        zv[0] = pe[0], zv[2] = pe[1], zv[1] = po[0], zv[3] = po[1];
+    };
+
+    load_x(0);
+    load_z(0);
+#pragma unroll
+    for (int st = 0; st < 4; ++st) load_w(0, st);
+    float4_t acc[MT][4];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int f = 0; f < 4; ++f) acc[mt][f] = float4_t{0.f, 0.f, 0.f, 0.f};
+    store_x(0);
+    __syncthreads();
+
+    for (int i = 0; i < NB; ++i) {
+        load_x(i + 1);  // lands while this block is multiplied; stored behind it
+        const unsigned char *buf = pk4_lds + (i & 1) * XBUF;
+        uint32_t zv[4], negzb[4], sp[4];
+        zs_words(zring, zv);
+#pragma unroll
+        for (int f = 0; f < 4; ++f) Pk4T<TT>::prep(zv[f], negzb[f], sp[f]);
+        load_z(i + 1);
+#pragma unroll
+        for (int st = 0; st < 4; ++st) {
+            const u32x4_t wv = wring[st];
+            const uint32_t wp[4] = {wv[0], wv[1], wv[2], wv[3]};
+            uint32_t a[MT][4];
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const u32x4_t av = *(const u32x4_t *)(buf + mt * 4096 + a_rd[st]);
+                a[mt][0] = av[0], a[mt][1] = av[1], a[mt][2] = av[2], a[mt][3] = av[3];
+            }
+#pragma unroll
+            for (int f = 0; f < 4; ++f) {
+                uint32_t b[4];
+#pragma unroll
+                for (int pp = 0; pp < 4; ++pp) b[pp] = Pk4T<TT>::deq(TT::unpack1(wp[pp], f, nm), negzb[f], sp[f]);
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) acc[mt][f] = Ops::mfma(a[mt], b, acc[mt][f]);
+            }
+            load_w(i + 1, st);  // into the registers this step has just left
+        }
+        // the other buffer was last read in the previous block, which every wave has left (the barrier below)
+        store_x(i + 1);
+        __syncthreads();
+    }
+
+    if (!live) return;
+    // row 16 mt + 4 kb + e, columns 64 j + 4 ni + f: four neighbours, one 8-byte store
+    float bv[4] = {0.f, 0.f, 0.f, 0.f};
+    if (bias) {
+        const uint2 bw = *(const uint2 *)(bias + 64 * j + 4 * ni);
+        bv[0] = TT::to_f32((uint16_t)(bw.x & 0xFFFFu)), bv[1] = TT::to_f32((uint16_t)(bw.x >> 16));
+        bv[2] = TT::to_f32((uint16_t)(bw.y & 0xFFFFu)), bv[3] = TT::to_f32((uint16_t)(bw.y >> 16));
+    }
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int row = m0 + 16 * mt + 4 * kb + e;
+            if (row >= M) continue;
+            const uint32_t o0 = TT::from_f32(acc[mt][0][e] + bv[0]), o1 = TT::from_f32(acc[mt][1][e] + bv[1]);
+            const uint32_t o2 = TT::from_f32(acc[mt][2][e] + bv[2]), o3 = TT::from_f32(acc[mt][3][e] + bv[3]);
+            *(uint2 *)(y + (size_t)row * N + 64 * j + 4 * ni) = uint2{o0 | (o1 << 16), o2 | (o3 << 16)};
+        }
+}
+
+// Which decomposition a resident 4-bit layer runs at M rows: 0 = the split-K tiles of pk4_mfma_kernel, else the
+// rows of a workgroup here.  Costs are in units of one 64-row workgroup's time, measured at 4096 x 14336 and
+// 8192 x 28672 (both types, 128..4096 rows):
+//   - 128-row workgroups (one per CU: 220..256 registers) take 1.4 (f16) or 1.6 (bf16) units and run in whole
+//     rounds of num_cus;
+//   - 64-row workgroups in bf16 (143 registers, one per CU) run in whole rounds too; in f16 (125 registers)
+//     two share a CU, each then at 0.6 of its speed alone, and past two a CU the time follows the count;
+//   - the split-K tiles reach two thirds of a full round's rate at any M, in small workgroups that leave no
+//     ragged round.
+// OXQ_PK4_GEMM_ROWS = 64 | 128 takes the choice (tests, sweeps); OXQ_PK4_GEMM_MIN_M = 0 switches the kernel off.
+static int pk4_gemm_rows(const oxq_ctx *ctx, const Pk4Problem &p) {
+    const int64_t min_m = tune(ctx, OXQ_TUNE_PK4_GEMM_MIN_M, 65);
+    if (min_m <= 0 || p.w.bits != 4 || p.w.strip == 16 || p.act || p.M < min_m) return 0;
+    const int forced = tune(ctx, OXQ_TUNE_PK4_GEMM_ROWS, 0);
+    if (forced == 64 || forced == 128) return forced;
+    const double cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
+    const int64_t groups = ceil_div(p.w.N / 64, (int64_t)PK4G_STRIPS);
+    const double w64 = (double)(groups * ceil_div(p.M, (int64_t)64)) / cus, w128 = (double)(groups * ceil_div(p.M, (int64_t)128)) / cus;
+    const bool f16 = p.w.dtype == OXQ_F16;
+    const double c_split = 1.5 * w64;
+    const double c64 = !f16 ? std::ceil(w64) : w64 <= 1.0 ? 1.0 : std::max(1.6, 0.95 * w64);
+    const double c128 = (f16 ? 1.4 : 1.6) * std::ceil(w128);
+    if (c_split <= c64 && c_split <= c128) return 0;
+    return c128 < c64 ? 128 : 64;
+}
+bool pk4_gemm_takes(const oxq_ctx *ctx, const Pk4Problem &p) { return pk4_gemm_rows(ctx, p) != 0; }
+
+template <typename TT, int MT>
+static int pk4_gemm_go(hipStream_t s, dim3 grid, const Pk4Problem &p, int NG, int RT) {
+    static LdsGrant grant;  // one per instantiation
+    const size_t lds = 2 * 16 * MT * 256;
+    OXQ_HIP_CHECK(grant.ensure((const void *)pk4_gemm_kernel<TT, MT>, lds));
+    hipLaunchKernelGGL((pk4_gemm_kernel<TT, MT>), grid, dim3(512), lds, s, (const uint16_t *)p.x, p.w.pw,
+                       (const uint16_t *)p.bias, (uint16_t *)p.y, (int)p.M, (int)p.w.K, (int)p.w.N, NG, RT);
+    OXQ_HIP_CHECK(hipGetLastError());
+    return OXQ_OK;
+}
+
+int launch_pk4_gemm(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p) {
+    const int rows = pk4_gemm_rows(ctx, p);
+    const int64_t NG = ceil_div(p.w.N / 64, (int64_t)PK4G_STRIPS), RT = ceil_div(p.M, (int64_t)rows);
+    // whole bands of 8 row tiles in squares of 64 workgroups, then the last RT % 8 row tiles x NG groups
+    const int64_t wgs = (RT / 8) * ceil_div(NG, (int64_t)8) * 64 + (RT % 8) * NG;
+    if (wgs > 0x7FFFFFFF) return fail(OXQ_ERR_UNSUPPORTED, "repacked matmul: m = %lld exceeds the grid", (long long)p.M);
+    dim3 grid((unsigned)wgs);
+    char name[64];
+    snprintf(name, sizeof name, "pk4_gemm_%s_r%dx8", p.w.dtype == OXQ_F16 ? "f16" : "bf16", rows);
+    set_plan(ctx, name, grid, dim3(512), 1, 1, 0);
+    if (ctx->plan_only) return OXQ_OK;
+    if ((uint64_t)rows * (uint64_t)p.w.K * 2 >= (1ull << 31)) return fail(OXQ_ERR_UNSUPPORTED, "repacked matmul: K too large");
+    if (((uintptr_t)p.x | (uintptr_t)p.y) & 15) return fail(OXQ_ERR_UNSUPPORTED, "repacked matmul: x and y must be 16-byte aligned");
+    if (p.bias && ((uintptr_t)p.bias & 7)) return fail(OXQ_ERR_UNSUPPORTED, "repacked matmul: bias must be 8-byte aligned");
+    const bool f16 = p.w.dtype == OXQ_F16;
+    if (rows == 128)
+        return f16 ? pk4_gemm_go<F16Traits, 8>(s, grid, p, (int)NG, (int)RT) : pk4_gemm_go<BF16Traits, 8>(s, grid, p, (int)NG, (int)RT);
+    return f16 ? pk4_gemm_go<F16Traits, 4>(s, grid, p, (int)NG, (int)RT) : pk4_gemm_go<BF16Traits, 4>(s, grid, p, (int)NG, (int)RT);
+}
+
+}  // namespace oxq

@@ -392,6 +392,19 @@ def test_layers_validate_like_reference(lib, ctx):
         out = fake(shape[:-1] + (14336,), BF16)
         assert lib.oxq_packed_quant_linear_forward(h, None, C.byref(x), C.byref(out)) == 0, err(lib)
         assert plan(lib, ctx).kernel.decode().startswith(kern), plan(lib, ctx).kernel
+    # prefill sizes: 28 groups of eight strips x row tiles of 64 or 128; the split-K tiles while those would
+    # leave most of the chip idle, then whichever row count needs the cheaper rounds of 256 workgroups
+    for rows, kern, wgs in [(256, "pk4_mfma_bf16_mt4", None), (512, "pk4_gemm_bf16_r64x8", 4 * 64),
+                            (768, "pk4_gemm_bf16_r128x8", 6 * 28), (1000, "pk4_gemm_bf16_r128x8", 4 * 64),
+                            (1536, "pk4_gemm_bf16_r64x8", 3 * 4 * 64), (1537, "pk4_gemm_bf16_r64x8", 3 * 4 * 64 + 28),
+                            (2100, "pk4_gemm_bf16_r128x8", 2 * 4 * 64 + 28),
+                            (4096, "pk4_gemm_bf16_r128x8", 4 * 4 * 64)]:
+        x = fake((rows, 4096), BF16)
+        assert lib.oxq_packed_quant_linear_forward(h, None, C.byref(x), C.byref(fake((rows, 14336), BF16))) == 0, err(lib)
+        pl = plan(lib, ctx)
+        assert pl.kernel.decode().startswith(kern), (rows, pl.kernel)
+        if wgs is not None:
+            assert (pl.grid[0], pl.block[0], pl.launches) == (wgs, 512, 1), (rows, tuple(pl.grid))
     x = fake((1, 4000), BF16)
     assert lib.oxq_packed_quant_linear_forward(h, None, C.byref(x), C.byref(fake((1, 14336), BF16))) == -3
     assert "input last dim 4000 != in_features 4096" in err(lib)

@@ -146,6 +146,80 @@ def front_rule(K, ks, m, bits=4):
 
 @pytest.mark.parametrize("kind", ["awq", "gptq"])
 @pytest.mark.parametrize("dtn", ["f16", "bf16"])
+@pytest.mark.parametrize("rows", [64, 128])
+@pytest.mark.parametrize("K,N,g", [(512, 576, 128), (1280, 1088, 128), (256, 64, 128)])
+def test_prefill_rows_by_eight_strips(kind, dtn, rows, K, N, g):
+    """The prefill decomposition (a workgroup = 64 or 128 rows x eight strips, x shared in LDS, a strip per
+    wave): N = 576 and 1088 leave the last group one live strip of eight, N = 64 a single group of one; m covers
+    one ragged row tile, whole bands of eight row tiles with a ragged remainder (581 rows: 8 + 2 tiles of 64,
+    5 of 128; 1100: 16 + 2, 8 + 1) and a band alone; K of 2, 4 and 10 blocks.  Against the tile-GEMM oracle
+    (mpp_gemm.metal:115-184: B rounded to the activation type), the reference's own bound against the
+    unrounded weights (metal_ops.rs:3713-3716), run to run bitwise, and rows of y independent of m."""
+    tune("OXQ_PK4_STRIP16", 0)
+    tune("OXQ_PK4_GEMM_ROWS", rows)
+    dt = DT[dtn]
+    trip, pack_dim = make(kind, K, N, g, seed=K + 5 * N)
+    bias = (np.arange(N, dtype=np.float32) % 13 - 6) * np.float32(0.125)
+    layer = layer_of(trip, pack_dim, dt, bias)
+    assert layer.prepacked
+    w = dense(kind, trip, dt)
+    wt = oracle.round_through(w, dt)
+    rng = np.random.default_rng(K + N + rows)
+    x_all = rng.standard_normal((1100, K)).astype(np.float32)
+    xd_all = to_dev(x_all, TORCH_DT[dt])
+    tile_all = oracle.matmul_nt_f32(round_x(x_all, dt), wt, bias)
+    ref_all = oracle.matmul_nt_f32(round_x(x_all, dt), w, bias)
+    first = None
+    for m in (1100, 65, 128, 300, 512, 581, 1024):
+        say(f"pk4 prefill {kind} {dtn} r{rows} K={K} N={N} m={m}")
+        xd = xd_all[:m]
+        y = layer.forward(xd)
+        plan = ops.default_context().last_plan()
+        rt, ng = -(-m // rows), -(-(N // 64) // 8)
+        assert plan["kernel"] == f"pk4_gemm_{dtn}_r{rows}x8", plan
+        assert plan["grid"][0] == (rt // 8) * (-(-ng // 8)) * 64 + (rt % 8) * ng and plan["launches"] == 1, plan
+        assert y.shape == (m, N)
+        assert_close(y, tile_all[:m], f"pk4 prefill {kind} {dtn} r{rows} m{m}")
+        assert np.abs(as_f32(y) - ref_all[:m]).max() < 0.06 * np.abs(ref_all[:m]).max() + 1e-2
+        np.testing.assert_array_equal(bits_of(layer.forward(xd)), bits_of(y))
+        if first is None:
+            first = bits_of(y)
+        else:
+            # a row's result does not depend on how many rows ride along or on which tile it falls
+            np.testing.assert_array_equal(bits_of(y), first[:m])
+    # without a bias, into a caller's buffer that holds other values
+    plain = layer_of(trip, pack_dim, dt, None)
+    out = torch.full((300, N), 7.0, device="cuda", dtype=TORCH_DT[dt])
+    plain.forward(xd_all[:300], out=out)
+    assert ops.default_context().last_plan()["kernel"] == f"pk4_gemm_{dtn}_r{rows}x8"
+    assert_close(out, tile_all[:300] - bias[None, :], f"pk4 prefill {kind} {dtn} no bias")
+
+
+def test_prefill_takes_over_where_it_fills_the_chip():
+    """With the switches at their defaults a 4096 x 14336 layer moves from the split-K tiles to 64-row and
+    then 128-row workgroups as m grows (28 groups of eight strips: 512 rows are 224 workgroups of 64 rows,
+    1000 rows 224 of 128), OXQ_PK4_GEMM_MIN_M = 0 keeps the split-K tiles, and the two agree within the
+    tolerance of one f16 rounding of y."""
+    K, N, g = 4096, 14336, 128
+    trip, pack_dim = make("awq", K, N, g, seed=11)
+    layer = layer_of(trip, pack_dim, oracle.F16, None)
+    rng = np.random.default_rng(5)
+    xd = to_dev(rng.standard_normal((1000, K)).astype(np.float32), torch.float16)
+    for m, kern in [(64, "pk4_mfma_f16_mt4"), (256, "pk4_mfma_f16_mt4"), (512, "pk4_gemm_f16_r64x8"), (1000, "pk4_gemm_f16_r128x8")]:
+        say(f"pk4 prefill rule m={m}")
+        y = layer.forward(xd[:m])
+        plan = ops.default_context().last_plan()
+        assert plan["kernel"].startswith(kern), (m, plan)
+        tune("OXQ_PK4_GEMM_MIN_M", 0)
+        y0 = layer.forward(xd[:m])
+        assert ops.default_context().last_plan()["kernel"].startswith("pk4_mfma_f16_mt4")
+        tune("OXQ_PK4_GEMM_MIN_M", None)
+        a, b = y.float(), y0.float()
+        assert bool(((a - b).abs() <= 2.0 ** -9 * b.abs() + 2e-2).all()), (m, float((a - b).abs().max()))
+
+
+@pytest.mark.parametrize("kind", ["awq", "gptq"])
+@pytest.mark.parametrize("dtn", ["f16", "bf16"])
 @pytest.mark.parametrize("K,N,g,ks", [(2048, 256, 128, 1), (4096 + 640, 128, 128, 1), (6144, 64, 128, 1),
                                       (4096, 192, 256, 1), (128 * 21, 64, 128, 1), (4096, 128, 128, 3),
                                       (8192, 64, 128, 1), (8192 - 384, 128, 128, 1), (5120, 128, 128, 1),
