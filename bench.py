@@ -161,6 +161,9 @@ def main():
                     help="skip the plain-read calibration (`roofline.bare_read_us`)")
     ap.add_argument("--all", action="store_true",
                     help="also the long list: prefill sizes, fused FFN entry, F8, all ten GGUF formats (`extra_configs`)")
+    ap.add_argument("--prefill-only", action="store_true",
+                    help="only the resident layers at prefill sizes (the first part of --all), as one JSON line "
+                         "{\"prefill\": [...]}: a short run for a profiler")
     ap.add_argument("--calib-copy", action="store_true",
                     help="first run a plain 256 MiB device copy 4 times: a kernel of known HBM "
                          "traffic to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings with")
@@ -189,6 +192,15 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+
+    if args.prefill_only:
+        import bench_extra
+        rows = bench_extra.run_prefill(ops, ctx, stream, args.steps, args.warmup, time_graph)
+        for r in rows:
+            print(f"[bench] {r['case']}: {r['us_per_call']} us, {r['TFLOP_per_s']} TFLOP/s "
+                  f"({r['mfma_frac']:.3f} of the dense MFMA peak), {r['kernel']}", file=sys.stderr, flush=True)
+        print(json.dumps({"prefill": rows}), flush=True)
+        return
 
     qw, qz, sc = synth.awq_checkpoint(K, N, G, 4, seed=0x0A0D11E6)
     copies = max(1, args.copies)

@@ -1,5 +1,6 @@
-"""Timings of the other benchmark configurations (`bench.py --all`).
+"""Timings of the other benchmark configurations (`bench.py --all`; `--prefill-only`: its first part alone).
 
+Resident AWQ layers at prefill sizes (256 - 4096 rows; 4096 x 14336 and 8192 x 28672, f16 and bf16);
 GPTQ 4/8-bit GEMV (K=5120, N=13824, g=128, M in {1, 8}); GGUF Q4_0 / Q8_0 / Q4_K /
 Q6_K ... GEMV (M=1, K=N=4096, f32 activations) and tile matmul (M=64..2048, bf16); MXFP4
 gated GGUF FFN at decode (four launches against the fused gate|up layer's two); MXFP4
@@ -34,9 +35,43 @@ def _case(name, fn_of_step, steps, warmup, stream, time_graph, nbytes, flops, ct
             "TFLOP_per_s": round(flops / us / 1e6, 3)}
 
 
-def run(ops, ctx, stream, steps, warmup, time_graph):
+def run_prefill(ops, ctx, stream, steps, warmup, time_graph):
+    """Config 1's layer and a 70B-class one at prefill sizes (PackedQuantLinear.forward): the rows x eight
+    strips kernel where the launcher chooses it, beside the split-K tiles it replaces there."""
     dev = torch.device("cuda:0")
     out = []
+    steps, warmup = max(4, steps // 8), max(2, warmup // 8)
+    for K, N, rows in ((4096, 14336, (256, 512, 1024, 2048, 4096)), (8192, 28672, (512, 4096))):
+        qw, qz, sc = synth.awq_checkpoint(K, N, 128, 4, seed=0x0A0D11F3)
+        wbytes = qw.nbytes + qz.nbytes + sc.size * 2
+        for tdt, tn in ((torch.float16, "f16"), (torch.bfloat16, "bf16")):
+            layer = ops.PackedQuantLinear(4, ops.PACK_OUT, torch.from_numpy(qw).to(dev), torch.from_numpy(qz).to(dev),
+                                          torch.from_numpy(sc).to(dev, tdt), None, tdt, ctx=ctx)
+            for m in rows:
+                x = torch.randn((m, K), device=dev, dtype=tdt)
+                y = torch.empty((m, N), device=dev, dtype=tdt)
+
+                def step(i, x=x, y=y, layer=layer):
+                    layer.forward(x, out=y)
+                nb, fl = wbytes + m * K * 2 + m * N * 2, 2.0 * m * K * N
+                r = _case(f"awq4 prefill M={m} K={K} N={N} {tn} (PackedQuantLinear)", step, steps, warmup, stream,
+                          time_graph, nb, fl, ctx)
+                r["mfma_frac"] = round(r["TFLOP_per_s"] / 2500.0, 4)
+                out.append(r)
+                if r["kernel"].startswith("pk4_gemm"):
+                    ctx.set_tuning("OXQ_PK4_GEMM_MIN_M", 0)
+                    r0 = _case(f"awq4 prefill M={m} K={K} N={N} {tn} (split-K tiles, OXQ_PK4_GEMM_MIN_M=0)", step,
+                               steps, warmup, stream, time_graph, nb, fl, ctx)
+                    ctx.set_tuning("OXQ_PK4_GEMM_MIN_M", None)
+                    r0["mfma_frac"] = round(r0["TFLOP_per_s"] / 2500.0, 4)
+                    out.append(r0)
+            del layer
+    return out
+
+
+def run(ops, ctx, stream, steps, warmup, time_graph):
+    dev = torch.device("cuda:0")
+    out = run_prefill(ops, ctx, stream, steps, warmup, time_graph)
 
     # ---- config 2: GPTQ ------------------------------------------------------
     K, N, G = 5120, 13824, 128

@@ -6,8 +6,9 @@
 // (row tile, strip) pair reads its 64 rows of x again, each wave for itself through the vector-memory unit.
 // At 2048 rows of a 4096 x 14336 layer that is 7168 workgroups x 512 KB = 3.7 GB of activations out of L2 for
 // 16.8 MB of x, and the kernel runs at the speed it has at 64 rows (0.6 PFLOP/s).  Here a workgroup takes 64
-// rows and EIGHT strips: its waves share one copy of the rows in LDS (loaded once per 128 elements of K by
-// all 512 threads, two buffers, one barrier a block), each wave owns a strip, streams its blocks with the
+// rows and EIGHT strips: its waves share one copy of the rows in LDS (a block of 128 elements of K at a time,
+// loaded from global memory straight into LDS - no registers, nothing for the compiler to sink behind the
+// arithmetic - two buffers, one barrier a block), each wave owns a strip, streams its blocks with the
 // one-block ring of pk4_mfma_kernel and keeps the whole K in its own accumulators - no partial tiles, no
 // second launch.  x out of L2 falls to an eighth.  Workgroups are numbered so that 64 neighbours form a square
 // of 8 row tiles x 8 strip groups, whose rows of x and weights the neighbours find in L2.
@@ -23,13 +24,23 @@ namespace oxq {
 
 constexpr int PK4G_STRIPS = 8;  // strips (= waves) of a workgroup
 
+typedef __attribute__((address_space(3))) void *pk4g_lds_ptr_t;
+// 16 bytes a lane from global memory into LDS at lds + 16 lane.  Kept out of the kernel template: the host pass
+// rejects the 16-byte form where it instantiates a template, and then drops the kernel's stub without a word.
+__device__ __forceinline__ void pk4g_load_lds16(__amdgpu_buffer_rsrc_t rs, unsigned char *lds, int voff, int soff) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (pk4g_lds_ptr_t)lds, 16, voff, soff, 0, 0);
+}
+template <int N> __device__ __forceinline__ void pk4g_wait_vmcnt() {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
 template <typename TT, int MT>
 __global__ __launch_bounds__(512) void pk4_gemm_kernel(const uint16_t *__restrict__ x, const uint32_t *__restrict__ pw,
                                                        const uint16_t *__restrict__ bias, uint16_t *__restrict__ y,
                                                        int M, int K, int N, int NG, int RT) {
     typedef MfmaOps<TT> Ops;
-    constexpr int ROWS = 16 * MT, BB = pk4_block_words(4) * 4, OOB = 0x7FFFFF00, XBUF = ROWS * 256;
-    constexpr int XV = ROWS / 32;  // 16-byte chunks of x a thread brings per block: 512 threads, 16 chunks a row
+    constexpr int ROWS = 16 * MT, BB = pk4_block_words(4) * 4, XBUF = ROWS * 256;
+    constexpr int XV = ROWS / 32;  // loads of x a wave issues per block: 64 lanes x 16 bytes = 4 rows each
     extern __shared__ __attribute__((aligned(16))) unsigned char pk4_lds[];
 
     const int lane = threadIdx.x & 63;
@@ -60,28 +71,29 @@ __global__ __launch_bounds__(512) void pk4_gemm_kernel(const uint16_t *__restric
     const __amdgpu_buffer_rsrc_t rs_x = make_rsrc(x + (size_t)m0 * K, (uint32_t)xrows * (uint32_t)K * 2u);
     const int voff_w = lane * 16;
     const int voff_z = 1024 * 4 + (ni * 4 + kb) * 4;
-    // x: thread t brings XV neighbouring chunks of row t / (16 / XV) of the block; rows past M read zeros
-    const int xr = threadIdx.x / (16 / XV), xc = (threadIdx.x % (16 / XV)) * XV;
-    const int voff_x = xr < xrows ? (xr * K * 2 + xc * 16) : OOB;
-    int x_wr[XV];
+    // x: load q of a wave brings rows 4 (XV wave + q) .. + 3 of the block straight into LDS, lane l the 16 bytes
+    // that belong at position l % 16 of row l / 16 - chunk (l % 16) ^ (row % 16) of the row, the swizzle the
+    // fragment reads undo.  Rows past M lie beyond the descriptor: LDS receives zeros.
+    int xo[XV];
 #pragma unroll
-    for (int v = 0; v < XV; ++v) x_wr[v] = xr * 256 + (((xc + v) ^ (xr & 15)) << 4);
+    for (int q = 0; q < XV; ++q) {
+        const int r = 4 * (wave * XV + q) + (lane >> 4);
+        xo[q] = r * K * 2 + (((lane & 15) ^ (r & 15)) << 4);
+    }
     int a_rd[4];  // fragment of step st, row tile mt (+ 4096 mt): row ni, chunk 8 (st / 2) + 2 kb + st % 2
 #pragma unroll
     for (int st = 0; st < 4; ++st) a_rd[st] = ni * 256 + (((8 * (st >> 1) + 2 * kb + (st & 1)) ^ ni) << 4);
     const NibbleMasks nm = nibble_masks();
 
-    u32x4_t xq[XV], wring[4];
+    u32x4_t wring[4];
     uint32_t zring;
-    auto load_x = [&](int i) {
+    // The compiler orders nothing against these loads: the wait for them (the five ring loads of a block are
+    // younger) is written out in front of the barrier that publishes the block.
+    auto dma_x = [&](int i) {
         const __amdgpu_buffer_rsrc_t rs = i < NB ? rs_x : rs_none;
 #pragma unroll
-        for (int v = 0; v < XV; ++v) xq[v] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff_x + 16 * v, i * 256, 0);
-    };
-    auto store_x = [&](int i) {
-        unsigned char *buf = pk4_lds + (i & 1) * XBUF;
-#pragma unroll
-        for (int v = 0; v < XV; ++v) *(u32x4_t *)(buf + x_wr[v]) = xq[v];
+        for (int q = 0; q < XV; ++q)
+            pk4g_load_lds16(rs, pk4_lds + (i & 1) * XBUF + (wave * XV + q) * 1024, xo[q], i * 256);
     };
     auto load_w = [&](int i, int st) {
         const __amdgpu_buffer_rsrc_t rs = i < NB ? rs_w : rs_none;
@@ -99,20 +111,24 @@ __global__ __launch_bounds__(512) void pk4_gemm_kernel(const uint16_t *__restric
         zv[0] = pe[0], zv[2] = pe[1], zv[1] = po[0], zv[3] = po[1];
     };
 
-    load_x(0);
+    dma_x(0);
+    __builtin_amdgcn_sched_barrier(0);  // requests keep this order: the wait counts rely on it
     load_z(0);
 #pragma unroll
     for (int st = 0; st < 4; ++st) load_w(0, st);
+    __builtin_amdgcn_sched_barrier(0);
     float4_t acc[MT][4];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
         for (int f = 0; f < 4; ++f) acc[mt][f] = float4_t{0.f, 0.f, 0.f, 0.f};
-    store_x(0);
+    pk4g_wait_vmcnt<5>();
     __syncthreads();
 
     for (int i = 0; i < NB; ++i) {
-        load_x(i + 1);  // lands while this block is multiplied; stored behind it
+        // the other buffer was last read in the previous block, which every wave has left (the barrier below)
+        dma_x(i + 1);
+        __builtin_amdgcn_sched_barrier(0);
         const unsigned char *buf = pk4_lds + (i & 1) * XBUF;
         uint32_t zv[4], negzb[4], sp[4];
         zs_words(zring, zv);
@@ -139,8 +155,8 @@ __global__ __launch_bounds__(512) void pk4_gemm_kernel(const uint16_t *__restric
             }
             load_w(i + 1, st);  // into the registers this step has just left
         }
-        // the other buffer was last read in the previous block, which every wave has left (the barrier below)
-        store_x(i + 1);
+        __builtin_amdgcn_sched_barrier(0);
+        pk4g_wait_vmcnt<5>();  // this wave's part of the next block is in LDS; its ring loads may still fly
         __syncthreads();
     }
 
@@ -165,27 +181,33 @@ __global__ __launch_bounds__(512) void pk4_gemm_kernel(const uint16_t *__restric
 }
 
 // Which decomposition a resident 4-bit layer runs at M rows: 0 = the split-K tiles of pk4_mfma_kernel, else the
-// rows of a workgroup here.  Costs are in units of one 64-row workgroup's time, measured at 4096 x 14336 and
-// 8192 x 28672 (both types, 128..4096 rows):
-//   - 128-row workgroups (one per CU: 220..256 registers) take 1.4 (f16) or 1.6 (bf16) units and run in whole
-//     rounds of num_cus;
-//   - 64-row workgroups in bf16 (143 registers, one per CU) run in whole rounds too; in f16 (125 registers)
-//     two share a CU, each then at 0.6 of its speed alone, and past two a CU the time follows the count;
-//   - the split-K tiles reach two thirds of a full round's rate at any M, in small workgroups that leave no
-//     ragged round.
+// rows of a workgroup here.  Costs are in units of a full round (one 64-row workgroup on every CU), fitted to
+// sweeps of 4096 x 14336 and 8192 x 28672 over 128..4096 rows in both types:
+//   - 128-row workgroups (203 registers: one a CU) run in whole rounds; a round costs `full128`, a last round
+//     that fills at most 0.7 of the CUs `part128`;
+//   - 64-row workgroups (121 registers) share a CU in pairs: up to one a CU the launch costs 1 (`part64` up to
+//     three quarters of the CUs), up to two a CU a64 + b64 w, beyond that slope64 w (w = workgroups / CUs);
+//   - the split-K tiles cost `split_lo` (below one round) or `split_hi` times w at any M: small workgroups, no
+//     ragged round, but the rate they have at 64 rows.
 // OXQ_PK4_GEMM_ROWS = 64 | 128 takes the choice (tests, sweeps); OXQ_PK4_GEMM_MIN_M = 0 switches the kernel off.
+struct Pk4GemmCost {
+    double part64, a64, b64, slope64, full128, part128, split_lo, split_hi;
+};
 static int pk4_gemm_rows(const oxq_ctx *ctx, const Pk4Problem &p) {
     const int64_t min_m = tune(ctx, OXQ_TUNE_PK4_GEMM_MIN_M, 65);
     if (min_m <= 0 || p.w.bits != 4 || p.w.strip == 16 || p.act || p.M < min_m) return 0;
     const int forced = tune(ctx, OXQ_TUNE_PK4_GEMM_ROWS, 0);
     if (forced == 64 || forced == 128) return forced;
+    static const Pk4GemmCost F16 = {0.88, 1.20, 0.30, 0.97, 1.50, 1.27, 1.70, 1.50};
+    static const Pk4GemmCost BF16 = {0.98, 1.45, 0.20, 0.98, 1.39, 1.32, 1.60, 1.42};
+    const Pk4GemmCost &c = p.w.dtype == OXQ_F16 ? F16 : BF16;
     const double cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
     const int64_t groups = ceil_div(p.w.N / 64, (int64_t)PK4G_STRIPS);
     const double w64 = (double)(groups * ceil_div(p.M, (int64_t)64)) / cus, w128 = (double)(groups * ceil_div(p.M, (int64_t)128)) / cus;
-    const bool f16 = p.w.dtype == OXQ_F16;
-    const double c_split = 1.5 * w64;
-    const double c64 = !f16 ? std::ceil(w64) : w64 <= 1.0 ? 1.0 : std::max(1.6, 0.95 * w64);
-    const double c128 = (f16 ? 1.4 : 1.6) * std::ceil(w128);
+    const double c64 = w64 <= 0.75 ? c.part64 : w64 <= 1.0 ? 1.0 : w64 <= 2.0 ? c.a64 + c.b64 * w64 : c.slope64 * w64;
+    const double whole = std::floor(w128), rest = w128 - whole;
+    const double c128 = whole * c.full128 + (rest <= 0.0 ? 0.0 : rest <= 0.7 ? c.part128 : c.full128);
+    const double c_split = (w64 < 1.0 ? c.split_lo : c.split_hi) * w64;
     if (c_split <= c64 && c_split <= c128) return 0;
     return c128 < c64 ? 128 : 64;
 }

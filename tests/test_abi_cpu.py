@@ -394,7 +394,8 @@ def test_layers_validate_like_reference(lib, ctx):
         assert plan(lib, ctx).kernel.decode().startswith(kern), plan(lib, ctx).kernel
     # prefill sizes: 28 groups of eight strips x row tiles of 64 or 128; the split-K tiles while those would
     # leave most of the chip idle, then whichever row count needs the cheaper rounds of 256 workgroups
-    for rows, kern, wgs in [(256, "pk4_mfma_bf16_mt4", None), (512, "pk4_gemm_bf16_r64x8", 4 * 64),
+    for rows, kern, wgs in [(256, "pk4_mfma_bf16_mt4", None), (384, "pk4_gemm_bf16_r64x8", 6 * 28),
+                            (512, "pk4_gemm_bf16_r64x8", 4 * 64),
                             (768, "pk4_gemm_bf16_r128x8", 6 * 28), (1000, "pk4_gemm_bf16_r128x8", 4 * 64),
                             (1536, "pk4_gemm_bf16_r64x8", 3 * 4 * 64), (1537, "pk4_gemm_bf16_r64x8", 3 * 4 * 64 + 28),
                             (2100, "pk4_gemm_bf16_r128x8", 2 * 4 * 64 + 28),
