@@ -639,7 +639,6 @@ __global__ __launch_bounds__(NW * 64) void pk4_front_kernel(const uint16_t *__re
 // odd pp; bf16: 128): the pairs hold -z alone, the folded form takes the biases out with a second row
 // sum (x against a fragment of the biases), the tile form keeps one constant per bias and column.
 // ---------------------------------------------------------------------------
-constexpr int PK4N_BW = 272;  // words of one block: 256 of weights, 16 of pairs
 
 template <typename TT, bool GPTQ>
 __global__ __launch_bounds__(256) void pk4n_prepack_kernel(const uint32_t *__restrict__ qw,
@@ -667,46 +666,6 @@ __global__ __launch_bounds__(256) void pk4n_prepack_kernel(const uint32_t *__res
         pw[idx] = (uint32_t)TT::from_f32(-(float)z) | ((uint32_t)sc[(size_t)g * N + col] << 16);
     }
 }
-
-// The constants of one column and block from its pair word {-z, s}; deq() = T((q - z) * s) of a row pair.
-template <typename TT> struct Pk4N;
-template <> struct Pk4N<F16Traits> {
-    uint32_t ce, co, sp;  // -(1024 + z), -(64 + z), s, each in both halves
-    __device__ __forceinline__ void prep(uint32_t zw) {
-        const uint32_t nz = perm_b32(zw, zw, 0x01000100u);
-        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
-        ce = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, nz) + __builtin_bit_cast(h2, 0xE400E400u));
-        co = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, nz) + __builtin_bit_cast(h2, 0xD400D400u));
-        sp = perm_b32(zw, zw, 0x03020302u);
-    }
-    // the odd pairs' constant from the even pairs': -(1024 + z) + 960 (exact); for kernels short of registers
-    __device__ __forceinline__ void odd_from_even() {
-        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
-        uint32_t e = ce;
-        asm volatile("" : "+v"(e));
-        co = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, e) + __builtin_bit_cast(h2, 0x63806380u));
-    }
-    __device__ __forceinline__ uint32_t deq(uint32_t p, int pp) const {
-        return MfmaOps<F16Traits>::dequant_pair(p, (pp & 1) ? co : ce, sp);
-    }
-    // (bias + q) - (bias + z): the exact integers q - z as a pair of f16
-    __device__ __forceinline__ uint32_t minus_zero(uint32_t p, int pp) const {
-        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
-        return __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, p) + __builtin_bit_cast(h2, (pp & 1) ? co : ce));
-    }
-};
-template <> struct Pk4N<BF16Traits> {
-    uint32_t c0, c1;
-    __device__ __forceinline__ void prep(uint32_t zw) {
-        const float sf = __builtin_bit_cast(float, zw & 0xFFFF0000u);
-        const float nz = __builtin_bit_cast(float, zw << 16);
-        c0 = __builtin_bit_cast(uint32_t, sf);
-        c1 = __builtin_bit_cast(uint32_t, (nz - 128.0f) * sf);
-    }
-    __device__ __forceinline__ uint32_t deq(uint32_t p, int) const { return Pk4T<BF16Traits>::deq(p, c0, c1); }
-    __device__ __forceinline__ uint32_t minus_zero(uint32_t p, int) const { return p; }  // f16 only
-    __device__ __forceinline__ void odd_from_even() {}
-};
 
 template <typename TT>
 __global__ __launch_bounds__(256) void pk4n_dequant_kernel(const uint32_t *__restrict__ pw,
@@ -1419,8 +1378,8 @@ static int launch_pk4n_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p)
 }
 
 int launch_pk4_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p) {
+    if (pk4_gemm_takes(ctx, p)) return launch_pk4_gemm(ctx, s, p);  // prefill sizes, either layout
     if (p.w.strip == 16) return launch_pk4n_forward(ctx, s, p);
-    if (pk4_gemm_takes(ctx, p)) return launch_pk4_gemm(ctx, s, p);
     const int64_t M = p.M;
     const int mt = M > 48 ? 4 : (int)ceil_div(M, 16);
     const int NB = (int)(p.w.K / 128);

@@ -42,6 +42,48 @@ template <> struct Pk4T<BF16Traits> {
     }
 };
 
+constexpr int PK4N_BW = 272;  // 16-column strips: words of one block, 256 of weights and 16 of pairs
+
+// The constants of one column and block from its pair word {-z, s}; deq() = T((q - z) * s) of a row pair.
+template <typename TT> struct Pk4N;
+template <> struct Pk4N<F16Traits> {
+    uint32_t ce, co, sp;  // -(1024 + z), -(64 + z), s, each in both halves
+    __device__ __forceinline__ void prep(uint32_t zw) {
+        const uint32_t nz = perm_b32(zw, zw, 0x01000100u);
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        ce = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, nz) + __builtin_bit_cast(h2, 0xE400E400u));
+        co = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, nz) + __builtin_bit_cast(h2, 0xD400D400u));
+        sp = perm_b32(zw, zw, 0x03020302u);
+    }
+    // the odd pairs' constant from the even pairs': -(1024 + z) + 960 (exact); for kernels short of registers
+    __device__ __forceinline__ void odd_from_even() {
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        uint32_t e = ce;
+        asm volatile("" : "+v"(e));
+        co = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, e) + __builtin_bit_cast(h2, 0x63806380u));
+    }
+    __device__ __forceinline__ uint32_t deq(uint32_t p, int pp) const {
+        return MfmaOps<F16Traits>::dequant_pair(p, (pp & 1) ? co : ce, sp);
+    }
+    // (bias + q) - (bias + z): the exact integers q - z as a pair of f16
+    __device__ __forceinline__ uint32_t minus_zero(uint32_t p, int pp) const {
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        return __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, p) + __builtin_bit_cast(h2, (pp & 1) ? co : ce));
+    }
+};
+template <> struct Pk4N<BF16Traits> {
+    uint32_t c0, c1;
+    __device__ __forceinline__ void prep(uint32_t zw) {
+        const float sf = __builtin_bit_cast(float, zw & 0xFFFF0000u);
+        const float nz = __builtin_bit_cast(float, zw << 16);
+        c0 = __builtin_bit_cast(uint32_t, sf);
+        c1 = __builtin_bit_cast(uint32_t, (nz - 128.0f) * sf);
+    }
+    __device__ __forceinline__ uint32_t deq(uint32_t p, int) const { return Pk4T<BF16Traits>::deq(p, c0, c1); }
+    __device__ __forceinline__ uint32_t minus_zero(uint32_t p, int) const { return p; }  // f16 only
+    __device__ __forceinline__ void odd_from_even() {}
+};
+
 __device__ __forceinline__ int pk4_kk(int t, int kb) { return ((t >> 1) << 6) + (kb << 4) + ((t & 1) << 3); }
 
 // Resident column -> checkpoint column.  A fused gate|up layer (half = N/2) keeps, in every strip

@@ -19,6 +19,7 @@
 
 #include <algorithm>
 #include <cmath>
+#include <type_traits>
 
 namespace oxq {
 
@@ -34,6 +35,19 @@ template <int N> __device__ __forceinline__ void pk4g_wait_vmcnt() {
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
+// Workgroup -> (row tile, strip group).  Bands of 8 row tiles are cut into squares of 8 row tiles x 8 strip groups,
+// 64 neighbouring workgroups each (neighbour i runs on XCD i % 8: a row tile stays on one XCD); the last RT % 8
+// row tiles are numbered row tile first, so that no XCD is handed only idle workgroups.
+__device__ __forceinline__ void pk4g_tile_of(int id, int RT, int NG, int &rt, int &g) {
+    const int full = (RT >> 3) * ((NG + 7) >> 3) * 64, tail = RT & 7;
+    if (id < full) {
+        const int sq = id >> 6, within = id & 63, bands = RT >> 3;
+        rt = (sq % bands) * 8 + (within & 7), g = (sq / bands) * 8 + (within >> 3);
+    } else {
+        rt = (RT & ~7) + (id - full) % tail, g = (id - full) / tail;
+    }
+}
+
 template <typename TT, int MT>
 __global__ __launch_bounds__(512) void pk4_gemm_kernel(const uint16_t *__restrict__ x, const uint32_t *__restrict__ pw,
                                                        const uint16_t *__restrict__ bias, uint16_t *__restrict__ y,
@@ -46,18 +60,8 @@ __global__ __launch_bounds__(512) void pk4_gemm_kernel(const uint16_t *__restric
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int ni = lane & 15, kb = lane >> 4;
-    // Bands of 8 row tiles are cut into squares of 8 row tiles x 8 strip groups, 64 neighbouring workgroups each
-    // (neighbour i runs on XCD i % 8: a row tile stays on one XCD); the last RT % 8 row tiles are numbered row
-    // tile first, so that no XCD is handed only idle workgroups.
-    const int full = (RT >> 3) * ((NG + 7) >> 3) * 64, tail = RT & 7;
     int rt, g;
-    if ((int)blockIdx.x < full) {
-        const int sq = blockIdx.x >> 6, within = blockIdx.x & 63, bands = RT >> 3;
-        rt = (sq % bands) * 8 + (within & 7), g = (sq / bands) * 8 + (within >> 3);
-    } else {
-        const int id = blockIdx.x - full;
-        rt = (RT & ~7) + id % tail, g = id / tail;
-    }
+    pk4g_tile_of((int)blockIdx.x, RT, NG, rt, g);
     if (g >= NG) return;  // the whole workgroup, before any barrier: the ragged last column of squares
     const int j = g * PK4G_STRIPS + wave;
     const bool live = j < (N >> 6);  // wave-uniform: the last group of a layer may have fewer than eight strips
@@ -180,48 +184,196 @@ __global__ __launch_bounds__(512) void pk4_gemm_kernel(const uint16_t *__restric
         }
 }
 
-// Which decomposition a resident 4-bit layer runs at M rows: 0 = the split-K tiles of pk4_mfma_kernel, else the
-// rows of a workgroup here.  Costs are in units of a full round (one 64-row workgroup on every CU), fitted to
-// sweeps of 4096 x 14336 and 8192 x 28672 over 128..4096 rows in both types:
-//   - 128-row workgroups (203 registers: one a CU) run in whole rounds; a round costs `full128`, a last round
-//     that fills at most 0.7 of the CUs `part128`;
-//   - 64-row workgroups (121 registers) share a CU in pairs: up to one a CU the launch costs 1 (`part64` up to
-//     three quarters of the CUs), up to two a CU a64 + b64 w, beyond that slope64 w (w = workgroups / CUs);
+// The same decomposition on a layer stored in 16-column strips (the narrow layout of attention and down
+// projections): a wave's 64 columns are four neighbouring strips, a strip's block is one 16-byte load a lane
+// whose words are the block's four steps - so the ring holds whole blocks, two of them: the next block is
+// requested into the other half when a block starts.  Lane (ni, kb) holds column 16 f + ni of strip f.
+template <typename TT, int MT>
+__global__ __launch_bounds__(512) void pk4n_gemm_kernel(const uint16_t *__restrict__ x, const uint32_t *__restrict__ pw,
+                                                        const uint16_t *__restrict__ bias, uint16_t *__restrict__ y,
+                                                        int M, int K, int N, int NG, int RT) {
+    typedef MfmaOps<TT> Ops;
+    constexpr int ROWS = 16 * MT, BB = PK4N_BW * 4, XBUF = ROWS * 256, XV = ROWS / 32;
+    extern __shared__ __attribute__((aligned(16))) unsigned char pk4_lds[];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int ni = lane & 15, kb = lane >> 4;
+    int rt, g;
+    pk4g_tile_of((int)blockIdx.x, RT, NG, rt, g);
+    if (g >= NG) return;  // the whole workgroup, before any barrier
+    const int j = g * PK4G_STRIPS + wave;  // the wave's 64 columns: strips 4 j .. 4 j + 3
+    const bool live = j < (N >> 6);
+    const int m0 = rt * ROWS;
+    const int NB = K >> 7;
+    const int xrows = min(M - m0, ROWS);
+
+    const __amdgpu_buffer_rsrc_t rs_none = make_rsrc(pw, 0u);
+    const __amdgpu_buffer_rsrc_t rs_wl =
+        make_rsrc(pw + (size_t)(live ? 4 * j : 0) * NB * PK4N_BW, 4u * (uint32_t)NB * (uint32_t)BB);
+    const __amdgpu_buffer_rsrc_t rs_w = live ? rs_wl : rs_none;
+    const __amdgpu_buffer_rsrc_t rs_x = make_rsrc(x + (size_t)m0 * K, (uint32_t)xrows * (uint32_t)K * 2u);
+    const int voff_w = lane * 16, voff_z = 1024 + ni * 4;
+    int xo[XV];
+#pragma unroll
+    for (int q = 0; q < XV; ++q) {
+        const int r = 4 * (wave * XV + q) + (lane >> 4);
+        xo[q] = r * K * 2 + (((lane & 15) ^ (r & 15)) << 4);
+    }
+    int a_rd[4];
+#pragma unroll
+    for (int st = 0; st < 4; ++st) a_rd[st] = ni * 256 + (((8 * (st >> 1) + 2 * kb + (st & 1)) ^ ni) << 4);
+    const NibbleMasks nm = nibble_masks();
+
+    u32x4_t wring[2][4];
+    uint32_t zring[4];
+    auto dma_x = [&](int i) {
+        const __amdgpu_buffer_rsrc_t rs = i < NB ? rs_x : rs_none;
+#pragma unroll
+        for (int q = 0; q < XV; ++q)
+            pk4g_load_lds16(rs, pk4_lds + (i & 1) * XBUF + (wave * XV + q) * 1024, xo[q], i * 256);
+    };
+    auto load_w = [&](int i, u32x4_t (&w)[4]) {
+        const __amdgpu_buffer_rsrc_t rs = i < NB ? rs_w : rs_none;
+#pragma unroll
+        for (int f = 0; f < 4; ++f) w[f] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff_w, (f * NB + i) * BB, 0);
+    };
+    auto load_z = [&](int i) {
+        const __amdgpu_buffer_rsrc_t rs = i < NB ? rs_w : rs_none;
+#pragma unroll
+        for (int f = 0; f < 4; ++f) zring[f] = __builtin_amdgcn_raw_buffer_load_b32(rs, voff_z, (f * NB + i) * BB, 0);
+    };
+
+    dma_x(0);
+    __builtin_amdgcn_sched_barrier(0);  // requests keep this order: the wait counts rely on it
+    load_z(0);
+    load_w(0, wring[0]);
+    __builtin_amdgcn_sched_barrier(0);
+    float4_t acc[MT][4];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int f = 0; f < 4; ++f) acc[mt][f] = float4_t{0.f, 0.f, 0.f, 0.f};
+    pk4g_wait_vmcnt<8>();
+    __syncthreads();
+
+    // one block, its weights in ring half CUR; eight ring loads are younger than the block's loads of x
+    auto block = [&](int i, auto cur_c) {
+        constexpr int CUR = decltype(cur_c)::value;
+        dma_x(i + 1);
+        __builtin_amdgcn_sched_barrier(0);
+        load_w(i + 1, wring[CUR ^ 1]);
+        __builtin_amdgcn_sched_barrier(0);  // not sunk to the block's end, where the next block would wait for them
+        const unsigned char *buf = pk4_lds + (i & 1) * XBUF;
+        Pk4N<TT> cst[4];
+#pragma unroll
+        for (int f = 0; f < 4; ++f) cst[f].prep(zring[f]);
+        load_z(i + 1);
+#pragma unroll
+        for (int st = 0; st < 4; ++st) {
+            uint32_t a[MT][4];
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const u32x4_t av = *(const u32x4_t *)(buf + mt * 4096 + a_rd[st]);
+                a[mt][0] = av[0], a[mt][1] = av[1], a[mt][2] = av[2], a[mt][3] = av[3];
+            }
+#pragma unroll
+            for (int f = 0; f < 4; ++f) {
+                const uint32_t w = wring[CUR][f][st];
+                uint32_t b[4];
+#pragma unroll
+                for (int pp = 0; pp < 4; ++pp) b[pp] = cst[f].deq(TT::unpack1(w, pp, nm), pp);
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) acc[mt][f] = Ops::mfma(a[mt], b, acc[mt][f]);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        pk4g_wait_vmcnt<8>();  // this wave's part of the next block of x is in LDS
+        __syncthreads();
+    };
+    {
+        int i = 0;
+        for (; i + 1 < NB; i += 2) {
+            block(i, std::integral_constant<int, 0>{});
+            block(i + 1, std::integral_constant<int, 1>{});
+        }
+        if (i < NB) block(i, std::integral_constant<int, 0>{});
+    }
+
+    if (!live) return;
+    // row 16 mt + 4 kb + e, column 64 j + 16 f + ni
+    float bv[4] = {0.f, 0.f, 0.f, 0.f};
+    if (bias) {
+#pragma unroll
+        for (int f = 0; f < 4; ++f) bv[f] = TT::to_f32(bias[64 * j + 16 * f + ni]);
+    }
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int row = m0 + 16 * mt + 4 * kb + e;
+            if (row >= M) continue;
+#pragma unroll
+            for (int f = 0; f < 4; ++f) y[(size_t)row * N + 64 * j + 16 * f + ni] = TT::from_f32(acc[mt][f][e] + bv[f]);
+        }
+}
+
+// Which decomposition a resident 4-bit layer runs at M rows: 0 = the split-K tiles of pk4_mfma_kernel /
+// pk4n_mfma_kernel, else the rows of a workgroup here.  Costs are in units of a full round (one 64-row workgroup
+// on every CU), fitted to sweeps over 128..8192 rows in both types (64-column strips: 4096 x 14336, 8192 x 28672;
+// 16-column strips: 4096 x 4096, 4096 x 6144, 14336 x 4096, 8192 x 8192):
+//   - 128-row workgroups (203..256 registers: one a CU) run in whole rounds; a round costs `full128`, a last
+//     round that fills at most 0.7 of the CUs `part128`;
+//   - 64-row workgroups of the 64-column layout (121 registers) share a CU in pairs: up to one a CU the launch
+//     costs 1 (`part64` up to three quarters of the CUs), up to two a CU a64 + b64 w, beyond that slope64 w
+//     (w = workgroups / CUs); those of the 16-column layout (140..144 registers) run in whole rounds;
 //   - the split-K tiles cost `split_lo` (below one round) or `split_hi` times w at any M: small workgroups, no
 //     ragged round, but the rate they have at 64 rows.
-// OXQ_PK4_GEMM_ROWS = 64 | 128 takes the choice (tests, sweeps); OXQ_PK4_GEMM_MIN_M = 0 switches the kernel off.
+// OXQ_PK4_GEMM_ROWS = 64 | 128 takes the choice (tests, sweeps); OXQ_PK4_GEMM_MIN_M = 0 switches the kernels off.
 struct Pk4GemmCost {
+    bool pairs64;
     double part64, a64, b64, slope64, full128, part128, split_lo, split_hi;
 };
 static int pk4_gemm_rows(const oxq_ctx *ctx, const Pk4Problem &p) {
     const int64_t min_m = tune(ctx, OXQ_TUNE_PK4_GEMM_MIN_M, 65);
-    if (min_m <= 0 || p.w.bits != 4 || p.w.strip == 16 || p.act || p.M < min_m) return 0;
+    if (min_m <= 0 || p.w.bits != 4 || p.act || p.M < min_m) return 0;
     const int forced = tune(ctx, OXQ_TUNE_PK4_GEMM_ROWS, 0);
     if (forced == 64 || forced == 128) return forced;
-    static const Pk4GemmCost F16 = {0.88, 1.20, 0.30, 0.97, 1.50, 1.27, 1.70, 1.50};
-    static const Pk4GemmCost BF16 = {0.98, 1.45, 0.20, 0.98, 1.39, 1.32, 1.60, 1.42};
-    const Pk4GemmCost &c = p.w.dtype == OXQ_F16 ? F16 : BF16;
+    static const Pk4GemmCost WIDE_F16 = {true, 0.88, 1.20, 0.30, 0.97, 1.50, 1.27, 1.70, 1.50};
+    static const Pk4GemmCost WIDE_BF16 = {true, 0.98, 1.45, 0.20, 0.98, 1.39, 1.32, 1.60, 1.42};
+    static const Pk4GemmCost NARROW_F16 = {false, 0.86, 0, 0, 0, 1.64, 1.30, 1.60, 1.50};
+    static const Pk4GemmCost NARROW_BF16 = {false, 0.97, 0, 0, 0, 1.68, 1.65, 1.50, 1.40};
+    const bool f16 = p.w.dtype == OXQ_F16;
+    const Pk4GemmCost &c = p.w.strip == 16 ? (f16 ? NARROW_F16 : NARROW_BF16) : (f16 ? WIDE_F16 : WIDE_BF16);
     const double cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
     const int64_t groups = ceil_div(p.w.N / 64, (int64_t)PK4G_STRIPS);
     const double w64 = (double)(groups * ceil_div(p.M, (int64_t)64)) / cus, w128 = (double)(groups * ceil_div(p.M, (int64_t)128)) / cus;
-    const double c64 = w64 <= 0.75 ? c.part64 : w64 <= 1.0 ? 1.0 : w64 <= 2.0 ? c.a64 + c.b64 * w64 : c.slope64 * w64;
-    const double whole = std::floor(w128), rest = w128 - whole;
-    const double c128 = whole * c.full128 + (rest <= 0.0 ? 0.0 : rest <= 0.7 ? c.part128 : c.full128);
+    auto rounds = [](double w, double full, double part, double part_upto) {
+        const double whole = std::floor(w), rest = w - whole;
+        return whole * full + (rest <= 0.0 ? 0.0 : rest <= part_upto ? part : full);
+    };
+    const double c64 = !c.pairs64 || w64 <= 1.0 ? rounds(w64, 1.0, c.part64, 0.75) : w64 <= 2.0 ? c.a64 + c.b64 * w64 : c.slope64 * w64;
+    const double c128 = rounds(w128, c.full128, c.part128, 0.7);
     const double c_split = (w64 < 1.0 ? c.split_lo : c.split_hi) * w64;
     if (c_split <= c64 && c_split <= c128) return 0;
     return c128 < c64 ? 128 : 64;
 }
 bool pk4_gemm_takes(const oxq_ctx *ctx, const Pk4Problem &p) { return pk4_gemm_rows(ctx, p) != 0; }
 
-template <typename TT, int MT>
+template <typename TT, int MT, bool N16>
 static int pk4_gemm_go(hipStream_t s, dim3 grid, const Pk4Problem &p, int NG, int RT) {
     static LdsGrant grant;  // one per instantiation
     const size_t lds = 2 * 16 * MT * 256;
-    OXQ_HIP_CHECK(grant.ensure((const void *)pk4_gemm_kernel<TT, MT>, lds));
-    hipLaunchKernelGGL((pk4_gemm_kernel<TT, MT>), grid, dim3(512), lds, s, (const uint16_t *)p.x, p.w.pw,
-                       (const uint16_t *)p.bias, (uint16_t *)p.y, (int)p.M, (int)p.w.K, (int)p.w.N, NG, RT);
+    auto kernel = N16 ? pk4n_gemm_kernel<TT, MT> : pk4_gemm_kernel<TT, MT>;
+    OXQ_HIP_CHECK(grant.ensure((const void *)kernel, lds));
+    hipLaunchKernelGGL(kernel, grid, dim3(512), lds, s, (const uint16_t *)p.x, p.w.pw, (const uint16_t *)p.bias,
+                       (uint16_t *)p.y, (int)p.M, (int)p.w.K, (int)p.w.N, NG, RT);
     OXQ_HIP_CHECK(hipGetLastError());
     return OXQ_OK;
+}
+template <typename TT, int MT>
+static int pk4_gemm_go_layout(hipStream_t s, dim3 grid, const Pk4Problem &p, int NG, int RT) {
+    return p.w.strip == 16 ? pk4_gemm_go<TT, MT, true>(s, grid, p, NG, RT) : pk4_gemm_go<TT, MT, false>(s, grid, p, NG, RT);
 }
 
 int launch_pk4_gemm(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p) {
@@ -232,7 +384,7 @@ int launch_pk4_gemm(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p) {
     if (wgs > 0x7FFFFFFF) return fail(OXQ_ERR_UNSUPPORTED, "repacked matmul: m = %lld exceeds the grid", (long long)p.M);
     dim3 grid((unsigned)wgs);
     char name[64];
-    snprintf(name, sizeof name, "pk4_gemm_%s_r%dx8", p.w.dtype == OXQ_F16 ? "f16" : "bf16", rows);
+    snprintf(name, sizeof name, "pk4_gemm_%s_r%dx8%s", p.w.dtype == OXQ_F16 ? "f16" : "bf16", rows, p.w.strip == 16 ? "_n16" : "");
     set_plan(ctx, name, grid, dim3(512), 1, 1, 0);
     if (ctx->plan_only) return OXQ_OK;
     if ((uint64_t)rows * (uint64_t)p.w.K * 2 >= (1ull << 31)) return fail(OXQ_ERR_UNSUPPORTED, "repacked matmul: K too large");
@@ -240,8 +392,8 @@ int launch_pk4_gemm(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p) {
     if (p.bias && ((uintptr_t)p.bias & 7)) return fail(OXQ_ERR_UNSUPPORTED, "repacked matmul: bias must be 8-byte aligned");
     const bool f16 = p.w.dtype == OXQ_F16;
     if (rows == 128)
-        return f16 ? pk4_gemm_go<F16Traits, 8>(s, grid, p, (int)NG, (int)RT) : pk4_gemm_go<BF16Traits, 8>(s, grid, p, (int)NG, (int)RT);
-    return f16 ? pk4_gemm_go<F16Traits, 4>(s, grid, p, (int)NG, (int)RT) : pk4_gemm_go<BF16Traits, 4>(s, grid, p, (int)NG, (int)RT);
+        return f16 ? pk4_gemm_go_layout<F16Traits, 8>(s, grid, p, (int)NG, (int)RT) : pk4_gemm_go_layout<BF16Traits, 8>(s, grid, p, (int)NG, (int)RT);
+    return f16 ? pk4_gemm_go_layout<F16Traits, 4>(s, grid, p, (int)NG, (int)RT) : pk4_gemm_go_layout<BF16Traits, 4>(s, grid, p, (int)NG, (int)RT);
 }
 
 }  // namespace oxq

@@ -410,6 +410,20 @@ def test_layers_validate_like_reference(lib, ctx):
     assert lib.oxq_packed_quant_linear_forward(h, None, C.byref(x), C.byref(fake((1, 14336), BF16))) == -3
     assert "input last dim 4000 != in_features 4096" in err(lib)
     lib.oxq_packed_quant_linear_free(h)
+    # a narrow layer (16-column strips): eight groups of 512 columns fill the chip from 2048 rows on
+    nqw, nqz, nsc = _awq(4096, 4096, 128, F16)
+    assert lib.oxq_packed_quant_linear_new(ctx, 4, 0, C.byref(nqw), C.byref(nqz), C.byref(nsc), None,
+                                           F16, C.byref(h)) == 0, err(lib)
+    for rows, kern, wgs in [(64, "pk4_mfma_f16_mt4_n16x4", None), (1024, "pk4_mfma_f16_mt4_n16x4", None),
+                            (2048, "pk4_gemm_f16_r64x8_n16", 256), (4096, "pk4_gemm_f16_r128x8_n16", 256),
+                            (4100, "pk4_gemm_f16_r64x8_n16", 512 + 8)]:
+        assert lib.oxq_packed_quant_linear_forward(h, None, C.byref(fake((rows, 4096), F16)),
+                                                   C.byref(fake((rows, 4096), F16))) == 0, err(lib)
+        pl = plan(lib, ctx)
+        assert pl.kernel.decode().startswith(kern), (rows, pl.kernel)
+        if wgs is not None:
+            assert (pl.grid[0], pl.block[0], pl.launches) == (wgs, 512, 1), (rows, tuple(pl.grid))
+    lib.oxq_packed_quant_linear_free(h)
 
     # Mxfp4Linear::new (mxfp4.rs:85-105)
     m = C.c_void_p()

@@ -147,16 +147,20 @@ def front_rule(K, ks, m, bits=4):
 @pytest.mark.parametrize("kind", ["awq", "gptq"])
 @pytest.mark.parametrize("dtn", ["f16", "bf16"])
 @pytest.mark.parametrize("rows", [64, 128])
+@pytest.mark.parametrize("strip16", [0, 2])
 @pytest.mark.parametrize("K,N,g", [(512, 576, 128), (1280, 1088, 128), (256, 64, 128)])
-def test_prefill_rows_by_eight_strips(kind, dtn, rows, K, N, g):
+def test_prefill_rows_by_eight_strips(kind, dtn, rows, K, N, g, strip16):
     """The prefill decomposition (a workgroup = 64 or 128 rows x eight strips, x shared in LDS, a strip per
     wave): N = 576 and 1088 leave the last group one live strip of eight, N = 64 a single group of one; m covers
     one ragged row tile, whole bands of eight row tiles with a ragged remainder (581 rows: 8 + 2 tiles of 64,
     5 of 128; 1100: 16 + 2, 8 + 1) and a band alone; K of 2, 4 and 10 blocks.  Against the tile-GEMM oracle
     (mpp_gemm.metal:115-184: B rounded to the activation type), the reference's own bound against the
-    unrounded weights (metal_ops.rs:3713-3716), run to run bitwise, and rows of y independent of m."""
-    tune("OXQ_PK4_STRIP16", 0)
+    unrounded weights (metal_ops.rs:3713-3716), run to run bitwise, and rows of y independent of m.  Both resident
+    layouts: 64-column strips and (strip16 = 2) the 16-column strips of narrow layers, whose kernel rings whole
+    blocks in two halves (K of 2, 4 and 10 blocks: both halves, and an odd count)."""
+    tune("OXQ_PK4_STRIP16", strip16)
     tune("OXQ_PK4_GEMM_ROWS", rows)
+    kname = f"pk4_gemm_{dtn}_r{rows}x8" + ("_n16" if strip16 else "")
     dt = DT[dtn]
     trip, pack_dim = make(kind, K, N, g, seed=K + 5 * N)
     bias = (np.arange(N, dtype=np.float32) % 13 - 6) * np.float32(0.125)
@@ -176,7 +180,7 @@ def test_prefill_rows_by_eight_strips(kind, dtn, rows, K, N, g):
         y = layer.forward(xd)
         plan = ops.default_context().last_plan()
         rt, ng = -(-m // rows), -(-(N // 64) // 8)
-        assert plan["kernel"] == f"pk4_gemm_{dtn}_r{rows}x8", plan
+        assert plan["kernel"] == kname, plan
         assert plan["grid"][0] == (rt // 8) * (-(-ng // 8)) * 64 + (rt % 8) * ng and plan["launches"] == 1, plan
         assert y.shape == (m, N)
         assert_close(y, tile_all[:m], f"pk4 prefill {kind} {dtn} r{rows} m{m}")
@@ -191,7 +195,7 @@ def test_prefill_rows_by_eight_strips(kind, dtn, rows, K, N, g):
     plain = layer_of(trip, pack_dim, dt, None)
     out = torch.full((300, N), 7.0, device="cuda", dtype=TORCH_DT[dt])
     plain.forward(xd_all[:300], out=out)
-    assert ops.default_context().last_plan()["kernel"] == f"pk4_gemm_{dtn}_r{rows}x8"
+    assert ops.default_context().last_plan()["kernel"] == kname
     assert_close(out, tile_all[:300] - bias[None, :], f"pk4 prefill {kind} {dtn} no bias")
 
 
