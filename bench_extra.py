@@ -1,6 +1,7 @@
 """Timings of the other benchmark configurations (`bench.py --all`; `--prefill-only`: its first part alone).
 
-Resident AWQ layers at prefill sizes (256 - 4096 rows; 4096 x 14336 and 8192 x 28672, f16 and bf16);
+Resident AWQ layers at prefill sizes (256 - 4096 rows; 4096 x 14336, 14336 x 4096, 4096 x 4096 and
+8192 x 28672, f16 and bf16);
 GPTQ 4/8-bit GEMV (K=5120, N=13824, g=128, M in {1, 8}); GGUF Q4_0 / Q8_0 / Q4_K /
 Q6_K ... GEMV (M=1, K=N=4096, f32 activations) and tile matmul (M=64..2048, bf16); MXFP4
 gated GGUF FFN at decode (four launches against the fused gate|up layer's two); MXFP4
@@ -36,12 +37,14 @@ def _case(name, fn_of_step, steps, warmup, stream, time_graph, nbytes, flops, ct
 
 
 def run_prefill(ops, ctx, stream, steps, warmup, time_graph):
-    """Config 1's layer and a 70B-class one at prefill sizes (PackedQuantLinear.forward): the rows x eight
-    strips kernel where the launcher chooses it, beside the split-K tiles it replaces there."""
+    """Config 1's layer, its down projection, an attention projection (both stored in 16-column strips) and a
+    70B-class layer at prefill sizes (PackedQuantLinear.forward): the rows x eight strips kernels where the
+    launcher chooses them, beside the split-K tiles they replace there."""
     dev = torch.device("cuda:0")
     out = []
     steps, warmup = max(4, steps // 8), max(2, warmup // 8)
-    for K, N, rows in ((4096, 14336, (256, 512, 1024, 2048, 4096)), (8192, 28672, (512, 4096))):
+    for K, N, rows in ((4096, 14336, (256, 512, 1024, 2048, 4096)), (14336, 4096, (1024, 2048, 4096)),
+                       (4096, 4096, (2048, 4096)), (8192, 28672, (512, 4096))):
         qw, qz, sc = synth.awq_checkpoint(K, N, 128, 4, seed=0x0A0D11F3)
         wbytes = qw.nbytes + qz.nbytes + sc.size * 2
         for tdt, tn in ((torch.float16, "f16"), (torch.bfloat16, "bf16")):
