@@ -31,6 +31,24 @@ typedef __attribute__((address_space(3))) void *pk4g_lds_ptr_t;
 __device__ __forceinline__ void pk4g_load_lds16(__amdgpu_buffer_rsrc_t rs, unsigned char *lds, int voff, int soff) {
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (pk4g_lds_ptr_t)lds, 16, voff, soff, 0, 0);
 }
+// bf16 has no packed 16-bit arithmetic: a weight goes nibble -> f32 -> fma -> (a pair at a time) bf16.  Masked in
+// place, a byte of the word holds q (low nibbles) or 16 q (high nibbles), which v_cvt_f32_ubyteN widens in one
+// instruction; the high nibbles' fma takes s / 16.  (q - z) s is exact in f32 either way: the same bits as
+// Pk4T<BF16Traits>::deq, with a sixth fewer instructions.
+struct Pk4gBf16 {
+    float s, s16, c;  // scale, scale / 16, -z * scale
+    __device__ __forceinline__ void set(float scale, float minus_z) { s = scale, s16 = scale * 0.0625f, c = minus_z * scale; }
+    // the pair in bytes B and B + 2 of v; HIGH: v holds high nibbles
+    template <int B, bool HIGH> __device__ __forceinline__ uint32_t pair(uint32_t v) const {
+        const float lo = (float)((v >> (8 * B)) & 0xFFu), hi = (float)((v >> (8 * B + 16)) & 0xFFu);
+        const float m = HIGH ? s16 : s;
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(float2_t{__builtin_fmaf(lo, m, c), __builtin_fmaf(hi, m, c)}, bf16x2_t));
+    }
+};
+__device__ __forceinline__ void pk4g_nibbles(uint32_t w, uint32_t &lo, uint32_t &hi) {
+    lo = w & 0x0F0F0F0Fu, hi = w & 0xF0F0F0F0u;
+    asm volatile("" : "+v"(lo), "+v"(hi));  // keep the masks here: folded into the byte extracts they cost one each
+}
 template <int N> __device__ __forceinline__ void pk4g_wait_vmcnt() {
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
@@ -54,6 +72,7 @@ __global__ __launch_bounds__(512) void pk4_gemm_kernel(const uint16_t *__restric
                                                        int M, int K, int N, int NG, int RT) {
     typedef MfmaOps<TT> Ops;
     constexpr int ROWS = 16 * MT, BB = pk4_block_words(4) * 4, XBUF = ROWS * 256;
+    constexpr bool BF = TT::DTYPE == BF16Traits::DTYPE;
     constexpr int XV = ROWS / 32;  // loads of x a wave issues per block: 64 lanes x 16 bytes = 4 rows each
     extern __shared__ __attribute__((aligned(16))) unsigned char pk4_lds[];
 
@@ -135,9 +154,16 @@ __global__ __launch_bounds__(512) void pk4_gemm_kernel(const uint16_t *__restric
         __builtin_amdgcn_sched_barrier(0);
         const unsigned char *buf = pk4_lds + (i & 1) * XBUF;
         uint32_t zv[4], negzb[4], sp[4];
+        Pk4gBf16 cb[4];
         zs_words(zring, zv);
 #pragma unroll
-        for (int f = 0; f < 4; ++f) Pk4T<TT>::prep(zv[f], negzb[f], sp[f]);
+        for (int f = 0; f < 4; ++f) {
+            if constexpr (BF) {  // the pair word holds {-(128 + z), s}
+                cb[f].set(__builtin_bit_cast(float, zv[f] & 0xFFFF0000u), __builtin_bit_cast(float, zv[f] << 16) + 128.0f);
+            } else {
+                Pk4T<TT>::prep(zv[f], negzb[f], sp[f]);
+            }
+        }
         load_z(i + 1);
 #pragma unroll
         for (int st = 0; st < 4; ++st) {
@@ -149,11 +175,23 @@ __global__ __launch_bounds__(512) void pk4_gemm_kernel(const uint16_t *__restric
                 const u32x4_t av = *(const u32x4_t *)(buf + mt * 4096 + a_rd[st]);
                 a[mt][0] = av[0], a[mt][1] = av[1], a[mt][2] = av[2], a[mt][3] = av[3];
             }
+            uint32_t tl[4], th[4];
+            if constexpr (BF) {
+#pragma unroll
+                for (int pp = 0; pp < 4; ++pp) pk4g_nibbles(wp[pp], tl[pp], th[pp]);
+            }
 #pragma unroll
             for (int f = 0; f < 4; ++f) {
                 uint32_t b[4];
 #pragma unroll
-                for (int pp = 0; pp < 4; ++pp) b[pp] = Pk4T<TT>::deq(TT::unpack1(wp[pp], f, nm), negzb[f], sp[f]);
+                for (int pp = 0; pp < 4; ++pp) {
+                    // column f of word pp: nibble f of each 16-bit half = the low or high nibble of bytes f / 2 and 2 + f / 2
+                    if constexpr (!BF) b[pp] = Pk4T<TT>::deq(TT::unpack1(wp[pp], f, nm), negzb[f], sp[f]);
+                    else if (f == 0) b[pp] = cb[0].template pair<0, false>(tl[pp]);
+                    else if (f == 1) b[pp] = cb[1].template pair<0, true>(th[pp]);
+                    else if (f == 2) b[pp] = cb[2].template pair<1, false>(tl[pp]);
+                    else b[pp] = cb[3].template pair<1, true>(th[pp]);
+                }
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt) acc[mt][f] = Ops::mfma(a[mt], b, acc[mt][f]);
             }
@@ -194,6 +232,7 @@ __global__ __launch_bounds__(512) void pk4n_gemm_kernel(const uint16_t *__restri
                                                         int M, int K, int N, int NG, int RT) {
     typedef MfmaOps<TT> Ops;
     constexpr int ROWS = 16 * MT, BB = PK4N_BW * 4, XBUF = ROWS * 256, XV = ROWS / 32;
+    constexpr bool BF = TT::DTYPE == BF16Traits::DTYPE;
     extern __shared__ __attribute__((aligned(16))) unsigned char pk4_lds[];
 
     const int lane = threadIdx.x & 63;
@@ -266,8 +305,15 @@ __global__ __launch_bounds__(512) void pk4n_gemm_kernel(const uint16_t *__restri
         __builtin_amdgcn_sched_barrier(0);  // not sunk to the block's end, where the next block would wait for them
         const unsigned char *buf = pk4_lds + (i & 1) * XBUF;
         Pk4N<TT> cst[4];
+        Pk4gBf16 cb[4];
 #pragma unroll
-        for (int f = 0; f < 4; ++f) cst[f].prep(zring[f]);
+        for (int f = 0; f < 4; ++f) {
+            if constexpr (BF) {  // the pair word holds {-z, s}
+                cb[f].set(__builtin_bit_cast(float, zring[f] & 0xFFFF0000u), __builtin_bit_cast(float, zring[f] << 16));
+            } else {
+                cst[f].prep(zring[f]);
+            }
+        }
         load_z(i + 1);
 #pragma unroll
         for (int st = 0; st < 4; ++st) {
@@ -281,8 +327,15 @@ __global__ __launch_bounds__(512) void pk4n_gemm_kernel(const uint16_t *__restri
             for (int f = 0; f < 4; ++f) {
                 const uint32_t w = wring[CUR][f][st];
                 uint32_t b[4];
+                if constexpr (BF) {  // row pair pp: nibble pp of each 16-bit half
+                    uint32_t tl, th;
+                    pk4g_nibbles(w, tl, th);
+                    b[0] = cb[f].template pair<0, false>(tl), b[1] = cb[f].template pair<0, true>(th);
+                    b[2] = cb[f].template pair<1, false>(tl), b[3] = cb[f].template pair<1, true>(th);
+                } else {
 #pragma unroll
-                for (int pp = 0; pp < 4; ++pp) b[pp] = cst[f].deq(TT::unpack1(w, pp, nm), pp);
+                    for (int pp = 0; pp < 4; ++pp) b[pp] = cst[f].deq(TT::unpack1(w, pp, nm), pp);
+                }
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt) acc[mt][f] = Ops::mfma(a[mt], b, acc[mt][f]);
             }
@@ -322,11 +375,11 @@ __global__ __launch_bounds__(512) void pk4n_gemm_kernel(const uint16_t *__restri
 // pk4n_mfma_kernel, else the rows of a workgroup here.  Costs are in units of a full round (one 64-row workgroup
 // on every CU), fitted to sweeps over 128..8192 rows in both types (64-column strips: 4096 x 14336, 8192 x 28672;
 // 16-column strips: 4096 x 4096, 4096 x 6144, 14336 x 4096, 8192 x 8192):
-//   - 128-row workgroups (203..256 registers: one a CU) run in whole rounds; a round costs `full128`, a last
+//   - 128-row workgroups (203..230 registers: one a CU) run in whole rounds; a round costs `full128`, a last
 //     round that fills at most 0.7 of the CUs `part128`;
-//   - 64-row workgroups of the 64-column layout (121 registers) share a CU in pairs: up to one a CU the launch
+//   - 64-row workgroups of the 64-column layout (121..125 registers) share a CU in pairs: up to one a CU the launch
 //     costs 1 (`part64` up to three quarters of the CUs), up to two a CU a64 + b64 w, beyond that slope64 w
-//     (w = workgroups / CUs); those of the 16-column layout (140..144 registers) run in whole rounds;
+//     (w = workgroups / CUs); those of the 16-column layout (144..145 registers) run in whole rounds;
 //   - the split-K tiles cost `split_lo` (below one round) or `split_hi` times w at any M: small workgroups, no
 //     ragged round, but the rate they have at 64 rows.
 // OXQ_PK4_GEMM_ROWS = 64 | 128 takes the choice (tests, sweeps); OXQ_PK4_GEMM_MIN_M = 0 switches the kernels off.
@@ -340,9 +393,9 @@ static int pk4_gemm_rows(const oxq_ctx *ctx, const Pk4Problem &p) {
     const int forced = tune(ctx, OXQ_TUNE_PK4_GEMM_ROWS, 0);
     if (forced == 64 || forced == 128) return forced;
     static const Pk4GemmCost WIDE_F16 = {true, 0.88, 1.20, 0.30, 0.97, 1.50, 1.27, 1.70, 1.50};
-    static const Pk4GemmCost WIDE_BF16 = {true, 0.98, 1.45, 0.20, 0.98, 1.39, 1.32, 1.60, 1.42};
+    static const Pk4GemmCost WIDE_BF16 = {true, 0.93, 1.29, 0.27, 0.98, 1.44, 1.35, 1.75, 1.53};
     static const Pk4GemmCost NARROW_F16 = {false, 0.86, 0, 0, 0, 1.64, 1.30, 1.60, 1.50};
-    static const Pk4GemmCost NARROW_BF16 = {false, 0.97, 0, 0, 0, 1.68, 1.65, 1.50, 1.40};
+    static const Pk4GemmCost NARROW_BF16 = {false, 0.94, 0, 0, 0, 1.51, 1.35, 1.60, 1.50};
     const bool f16 = p.w.dtype == OXQ_F16;
     const Pk4GemmCost &c = p.w.strip == 16 ? (f16 ? NARROW_F16 : NARROW_BF16) : (f16 ? WIDE_F16 : WIDE_BF16);
     const double cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
