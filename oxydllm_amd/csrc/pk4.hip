@@ -1378,6 +1378,8 @@ static int launch_pk4n_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p)
 }
 
 int launch_pk4_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p) {
+    if (p.act && (!p.w.gate_half || p.act > 2))
+        return fail(OXQ_ERR_ARG, "repacked matmul: activation %d on a layer that is not a fused gate|up layer", p.act);
     if (pk4_gemm_takes(ctx, p)) return launch_pk4_gemm(ctx, s, p);  // prefill sizes, either layout
     if (p.w.strip == 16) return launch_pk4n_forward(ctx, s, p);
     const int64_t M = p.M;
@@ -1407,8 +1409,6 @@ int launch_pk4_forward(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p) {
         return fail(OXQ_ERR_UNSUPPORTED, "repacked matmul: m = %lld exceeds the grid limit (65535 row tiles)", (long long)M);
     dim3 grid((unsigned)(p.w.N / 64), (unsigned)ks, (unsigned)ceil_div(M, 16 * mt));
     char name[64];
-    if (p.act && (!p.w.gate_half || p.act > 2))
-        return fail(OXQ_ERR_ARG, "repacked matmul: activation %d on a layer that is not a fused gate|up layer", p.act);
     // A single row tile (up to 16 rows) runs straight-line kernels (pk4_front_kernel) where one exists for the
     // slice: no loop, so no loop-carried ring registers to copy (and wait for) at its end, and every request
     // placed where the source puts it.  Which form, measured side by side on one box (f16, us; "ring" is

@@ -69,7 +69,7 @@ __device__ __forceinline__ void pk4g_tile_of(int id, int RT, int NG, int &rt, in
 template <typename TT, int MT>
 __global__ __launch_bounds__(512) void pk4_gemm_kernel(const uint16_t *__restrict__ x, const uint32_t *__restrict__ pw,
                                                        const uint16_t *__restrict__ bias, uint16_t *__restrict__ y,
-                                                       int M, int K, int N, int NG, int RT) {
+                                                       int M, int K, int N, int NG, int RT, int act) {
     typedef MfmaOps<TT> Ops;
     constexpr int ROWS = 16 * MT, BB = pk4_block_words(4) * 4, XBUF = ROWS * 256;
     constexpr bool BF = TT::DTYPE == BF16Traits::DTYPE;
@@ -203,6 +203,35 @@ __global__ __launch_bounds__(512) void pk4_gemm_kernel(const uint16_t *__restric
     }
 
     if (!live) return;
+    if (act) {
+        // Fused gate|up layer (pk4_src_col): columns 0..31 of the strip are gate columns 32 j .. 32 j + 31, columns
+        // 32..63 the up columns they meet - lane ni < 8 holds four gate columns, lane ni + 8 of the same row of 16
+        // their up columns.  As in pk4_epilogue: both factors rounded to the layer type (what the projection's own
+        // output would hold, ffn.rs:388-400), act(gate) * up in f32, one rounding; y is [M, N / 2].
+        const int half = N >> 1, col = 32 * j + 4 * (ni & 7);
+        float bv[4] = {0.f, 0.f, 0.f, 0.f};
+        if (bias) {
+            const uint2 bw = *(const uint2 *)(bias + (ni < 8 ? 0 : half) + col);
+            bv[0] = TT::to_f32((uint16_t)(bw.x & 0xFFFFu)), bv[1] = TT::to_f32((uint16_t)(bw.x >> 16));
+            bv[2] = TT::to_f32((uint16_t)(bw.y & 0xFFFFu)), bv[3] = TT::to_f32((uint16_t)(bw.y >> 16));
+        }
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int row = m0 + 16 * mt + 4 * kb + e;
+                uint32_t o[4];
+#pragma unroll
+                for (int f = 0; f < 4; ++f) {
+                    const float mine = TT::to_f32(TT::from_f32(acc[mt][f][e] + bv[f]));
+                    // the other half of the row of 16 lanes (row_ror:8)
+                    const float other = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, mine), 0x128, 0xF, 0xF, false));
+                    o[f] = TT::from_f32(mul_f32_rn(act == 1 ? silu_f32(mine) : gelu_tanh_f32(mine), other));
+                }
+                if (ni < 8 && row < M) *(uint2 *)(y + (size_t)row * half + col) = uint2{o[0] | (o[1] << 16), o[2] | (o[3] << 16)};
+            }
+        return;
+    }
     // row 16 mt + 4 kb + e, columns 64 j + 4 ni + f: four neighbours, one 8-byte store
     float bv[4] = {0.f, 0.f, 0.f, 0.f};
     if (bias) {
@@ -389,7 +418,7 @@ struct Pk4GemmCost {
 };
 static int pk4_gemm_rows(const oxq_ctx *ctx, const Pk4Problem &p) {
     const int64_t min_m = tune(ctx, OXQ_TUNE_PK4_GEMM_MIN_M, 65);
-    if (min_m <= 0 || p.w.bits != 4 || p.act || p.M < min_m) return 0;
+    if (min_m <= 0 || p.w.bits != 4 || (p.act && p.w.strip == 16) || p.M < min_m) return 0;
     const int forced = tune(ctx, OXQ_TUNE_PK4_GEMM_ROWS, 0);
     if (forced == 64 || forced == 128) return forced;
     static const Pk4GemmCost WIDE_F16 = {true, 0.88, 1.20, 0.30, 0.97, 1.50, 1.27, 1.70, 1.50};
@@ -417,10 +446,15 @@ template <typename TT, int MT, bool N16>
 static int pk4_gemm_go(hipStream_t s, dim3 grid, const Pk4Problem &p, int NG, int RT) {
     static LdsGrant grant;  // one per instantiation
     const size_t lds = 2 * 16 * MT * 256;
-    auto kernel = N16 ? pk4n_gemm_kernel<TT, MT> : pk4_gemm_kernel<TT, MT>;
-    OXQ_HIP_CHECK(grant.ensure((const void *)kernel, lds));
-    hipLaunchKernelGGL(kernel, grid, dim3(512), lds, s, (const uint16_t *)p.x, p.w.pw, (const uint16_t *)p.bias,
-                       (uint16_t *)p.y, (int)p.M, (int)p.w.K, (int)p.w.N, NG, RT);
+    if constexpr (N16) {
+        OXQ_HIP_CHECK(grant.ensure((const void *)pk4n_gemm_kernel<TT, MT>, lds));
+        hipLaunchKernelGGL((pk4n_gemm_kernel<TT, MT>), grid, dim3(512), lds, s, (const uint16_t *)p.x, p.w.pw, (const uint16_t *)p.bias,
+                           (uint16_t *)p.y, (int)p.M, (int)p.w.K, (int)p.w.N, NG, RT);
+    } else {
+        OXQ_HIP_CHECK(grant.ensure((const void *)pk4_gemm_kernel<TT, MT>, lds));
+        hipLaunchKernelGGL((pk4_gemm_kernel<TT, MT>), grid, dim3(512), lds, s, (const uint16_t *)p.x, p.w.pw, (const uint16_t *)p.bias,
+                           (uint16_t *)p.y, (int)p.M, (int)p.w.K, (int)p.w.N, NG, RT, p.act);
+    }
     OXQ_HIP_CHECK(hipGetLastError());
     return OXQ_OK;
 }
@@ -437,7 +471,8 @@ int launch_pk4_gemm(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p) {
     if (wgs > 0x7FFFFFFF) return fail(OXQ_ERR_UNSUPPORTED, "repacked matmul: m = %lld exceeds the grid", (long long)p.M);
     dim3 grid((unsigned)wgs);
     char name[64];
-    snprintf(name, sizeof name, "pk4_gemm_%s_r%dx8%s", p.w.dtype == OXQ_F16 ? "f16" : "bf16", rows, p.w.strip == 16 ? "_n16" : "");
+    snprintf(name, sizeof name, "pk4_gemm_%s_r%dx8%s%s", p.w.dtype == OXQ_F16 ? "f16" : "bf16", rows, p.w.strip == 16 ? "_n16" : "",
+             p.act == 1 ? "_silu" : p.act == 2 ? "_gelu" : "");
     set_plan(ctx, name, grid, dim3(512), 1, 1, 0);
     if (ctx->plan_only) return OXQ_OK;
     if ((uint64_t)rows * (uint64_t)p.w.K * 2 >= (1ull << 31)) return fail(OXQ_ERR_UNSUPPORTED, "repacked matmul: K too large");

@@ -506,6 +506,41 @@ def test_fused_gate_up_activation(kind, dtn, act, K, I, g):
             assert_close(y, ref, f"gate|up {kind} {dtn} {act} m{m}")
 
 
+@pytest.mark.parametrize("kind", ["awq", "gptq"])
+@pytest.mark.parametrize("dtn", ["f16", "bf16"])
+@pytest.mark.parametrize("act", ["silu", "gelu"])
+@pytest.mark.parametrize("rows", [64, 128])
+def test_fused_gate_up_activation_at_prefill(kind, dtn, act, rows):
+    """The prefill kernel's own activation epilogue (gate and up columns of an output sit in lanes 8 apart of the
+    accumulator layout): bit for bit the plain layer through the same kernel followed by the activation kernel,
+    with and without bias, ragged row tiles, a last strip group of one strip (I = 288: nine strips)."""
+    tune("OXQ_PK4_GEMM_ROWS", rows)
+    dt = DT[dtn]
+    tdt = TORCH_DT[dt]
+    K, I, g = 512, 288, 128
+    trip, pack_dim = make(kind, K, 2 * I, g, seed=17)
+    bias = (np.arange(2 * I, dtype=np.float32) % 7 - 3) * np.float32(0.0625)
+    kind_id = ops.ACT_GATED_SILU if act == "silu" else ops.ACT_GATED_GELU_TANH
+    rng = np.random.default_rng(rows)
+    xd = to_dev(rng.standard_normal((581, K)).astype(np.float32), tdt)
+    for b in (None, bias):
+        plain = layer_of(trip, pack_dim, dt, b)
+        bd = None if b is None else to_dev(b, tdt)
+        fused = ops.PackedQuantLinear(4, pack_dim, to_dev(trip[0]), to_dev(trip[1]), to_dev(trip[2], tdt), bd, tdt,
+                                      gate_up_act=kind_id)
+        for m in (65, 300, 581):
+            say(f"gate|up prefill {kind} {dtn} {act} r{rows} m={m} bias={b is not None}")
+            y = fused.forward(xd[:m])
+            plan = ops.default_context().last_plan()
+            assert plan["kernel"] == f"pk4_gemm_{dtn}_r{rows}x8_{act}" and plan["launches"] == 1, plan
+            assert y.shape == (m, I)
+            gu = plain.forward(xd[:m])
+            assert ops.default_context().last_plan()["kernel"] == f"pk4_gemm_{dtn}_r{rows}x8"
+            np.testing.assert_array_equal(bits_of(y), bits_of(ops.gated_activation(gu, kind_id)))
+            ref = oracle.gated_silu(as_f32(gu)) if act == "silu" else oracle.gated_gelu_tanh(as_f32(gu))
+            assert_close(y, ref, f"gate|up prefill {kind} {dtn} {act} m{m}")
+
+
 def test_fused_gate_up_benchmark_shape_and_refusals():
     K, I, g = 4096, 14336, 128
     trip = synth.awq_checkpoint(K, 2 * I, g, 4, seed=11)
@@ -513,10 +548,11 @@ def test_fused_gate_up_benchmark_shape_and_refusals():
     plain = ops.PackedQuantLinear(*args)
     fused = ops.PackedQuantLinear(*args, gate_up_act=ops.ACT_GATED_SILU)
     rng = np.random.default_rng(2)
-    for m in (1, 16, 64):
+    for m in (1, 16, 64, 300, 1000):  # 300 rows: 64-row workgroups of the prefill kernel, 1000: 128-row
         x = to_dev(rng.standard_normal((m, K)).astype(np.float32), torch.float16)
         y = fused.forward(x)
         assert ops.default_context().last_plan()["kernel"].endswith("_silu")
+        assert ops.default_context().last_plan()["kernel"].startswith("pk4_gemm_f16_r") == (m > 64)
         assert ops.default_context().last_plan()["launches"] == 1
         np.testing.assert_array_equal(bits_of(y), bits_of(ops.gated_activation(plain.forward(x), ops.ACT_GATED_SILU)))
         with pytest.raises(ops.OxqError):
