@@ -69,6 +69,37 @@ def run_prefill(ops, ctx, stream, steps, warmup, time_graph):
                     r0["mfma_frac"] = round(r0["TFLOP_per_s"] / 2500.0, 4)
                     out.append(r0)
             del layer
+
+    # the whole gated FFN of config 1's model (hidden 4096, intermediate 14336, bf16): the gate|up projection with
+    # the activation in its epilogue, then the down projection (stored in 16-column strips) - two launches
+    H, I = 4096, 14336
+    gu = synth.awq_checkpoint(H, 2 * I, 128, 4, seed=0x0A0D11F4)
+    dn = synth.awq_checkpoint(I, H, 128, 4, seed=0x0A0D11F5)
+    wbytes = sum(t[0].nbytes + t[1].nbytes + t[2].size * 2 for t in (gu, dn))
+    tdt = torch.bfloat16
+
+    def lin(t, **kw):
+        return ops.PackedQuantLinear(4, ops.PACK_OUT, torch.from_numpy(t[0]).to(dev), torch.from_numpy(t[1]).to(dev),
+                                     torch.from_numpy(t[2]).to(dev, tdt), None, tdt, ctx=ctx, **kw)
+    ffn = ops.FeedForward(ops.GATE_UP_FUSED, lin(gu, gate_up_act=ops.ACT_GATED_SILU), None, lin(dn), I,
+                          ops.ACT_GATED_SILU, ctx=ctx)
+    for m in (512, 2048, 4096):
+        x = torch.randn((m, H), device=dev, dtype=tdt)
+        y = torch.empty((m, H), device=dev, dtype=tdt)
+        scratch = torch.empty(max(ffn.scratch_elems(m), 1), device=dev, dtype=tdt)
+
+        def fstep(i, x=x, y=y, scratch=scratch):
+            ffn.forward(x, out=y, scratch=scratch)
+        nb, fl = wbytes + 2 * m * H * 2 + 2 * m * I * 2, 6.0 * m * H * I
+        for label, min_m in (("", None), (" (split-K tiles, OXQ_PK4_GEMM_MIN_M=0)", 0)):
+            ctx.set_tuning("OXQ_PK4_GEMM_MIN_M", min_m)
+            r = _case(f"awq4 gated FFN prefill M={m} H={H} I={I} bf16 (FeedForward, fused gate|up + down){label}",
+                      fstep, steps, warmup, stream, time_graph, nb, fl, ctx)
+            r["launches"] = 2
+            r["mfma_frac"] = round(r["TFLOP_per_s"] / 2500.0, 4)
+            out.append(r)
+        ctx.set_tuning("OXQ_PK4_GEMM_MIN_M", None)
+    del ffn
     return out
 
 

@@ -150,17 +150,26 @@ __device__ __forceinline__ float mul_f32_rn(float a, float b) {
     asm("v_mul_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
     return r;
 }
-__device__ __forceinline__ float silu_f32(float x) { return x / (1.0f + expf(-x)); }
+// The logistic function through the hardware's exp2 and reciprocal (v_exp_f32, v_rcp_f32: an ulp each), five
+// instructions where expf and an IEEE division take about forty - in a matmul epilogue that nothing overlaps
+// (one workgroup a CU at prefill sizes) the difference is a tenth of the kernel.  The results are rounded to a
+// 16-bit type afterwards; every kernel here takes these same functions, so they agree among themselves bit for
+// bit.  e^-x = inf for very negative x gives 1 / inf = 0: the limit.
+__device__ __forceinline__ float logistic_f32(float x) {
+    return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * -1.4426950408889634f));
+}
+__device__ __forceinline__ float silu_f32(float x) { return x * logistic_f32(x); }
 // GPT-OSS clamped SwiGLU of one (gate, up) pair, alpha = 1.702 (moe.rs:152-173)
 __device__ __forceinline__ float gpt_oss_swiglu_f32(float gate, float up, float limit) {
     gate = fminf(gate, limit);
     up = fminf(fmaxf(up, -limit), limit);
-    const float sig = 1.0f / (1.0f + expf(-(gate * 1.702f)));
+    const float sig = logistic_f32(gate * 1.702f);
     return mul_f32_rn(up + 1.0f, gate * sig);
 }
 __device__ __forceinline__ float gelu_tanh_f32(float x) {
+    // 0.5 x (1 + tanh t) = x / (1 + e^(-2t)): no cancellation in the negative tail, where 1 + tanh t is tiny
     const float k0 = 0.7978845608028654f, k1 = 0.044715f;
-    return 0.5f * x * (1.0f + tanhf(k0 * (x + k1 * x * x * x)));
+    return x * logistic_f32(2.0f * (k0 * (x + k1 * x * x * x)));
 }
 
 __device__ __forceinline__ float e8m0_to_f32(uint32_t s) {

@@ -208,10 +208,13 @@ __global__ __launch_bounds__(512) void pk4_gemm_kernel(const uint16_t *__restric
         // 32..63 the up columns they meet - lane ni < 8 holds four gate columns, lane ni + 8 of the same row of 16
         // their up columns.  As in pk4_epilogue: both factors rounded to the layer type (what the projection's own
         // output would hold, ffn.rs:388-400), act(gate) * up in f32, one rounding; y is [M, N / 2].
+        // The two lanes of a pair exchange all four values (row_ror:8) and share the work: lane ni takes outputs
+        // 0 and 1 of its four columns, lane ni + 8 outputs 2 and 3.
         const int half = N >> 1, col = 32 * j + 4 * (ni & 7);
+        const bool low = ni < 8;
         float bv[4] = {0.f, 0.f, 0.f, 0.f};
         if (bias) {
-            const uint2 bw = *(const uint2 *)(bias + (ni < 8 ? 0 : half) + col);
+            const uint2 bw = *(const uint2 *)(bias + (low ? 0 : half) + col);
             bv[0] = TT::to_f32((uint16_t)(bw.x & 0xFFFFu)), bv[1] = TT::to_f32((uint16_t)(bw.x >> 16));
             bv[2] = TT::to_f32((uint16_t)(bw.y & 0xFFFFu)), bv[3] = TT::to_f32((uint16_t)(bw.y >> 16));
         }
@@ -220,15 +223,19 @@ __global__ __launch_bounds__(512) void pk4_gemm_kernel(const uint16_t *__restric
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const int row = m0 + 16 * mt + 4 * kb + e;
-                uint32_t o[4];
+                float mine[4], other[4];
 #pragma unroll
                 for (int f = 0; f < 4; ++f) {
-                    const float mine = TT::to_f32(TT::from_f32(acc[mt][f][e] + bv[f]));
-                    // the other half of the row of 16 lanes (row_ror:8)
-                    const float other = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, mine), 0x128, 0xF, 0xF, false));
-                    o[f] = TT::from_f32(mul_f32_rn(act == 1 ? silu_f32(mine) : gelu_tanh_f32(mine), other));
+                    mine[f] = TT::to_f32(TT::from_f32(acc[mt][f][e] + bv[f]));
+                    other[f] = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, mine[f]), 0x128, 0xF, 0xF, false));
                 }
-                if (ni < 8 && row < M) *(uint2 *)(y + (size_t)row * half + col) = uint2{o[0] | (o[1] << 16), o[2] | (o[3] << 16)};
+                uint32_t o[2];
+#pragma unroll
+                for (int q = 0; q < 2; ++q) {
+                    const float gq = low ? mine[q] : other[2 + q], uq = low ? other[q] : mine[2 + q];
+                    o[q] = TT::from_f32(mul_f32_rn(act == 1 ? silu_f32(gq) : gelu_tanh_f32(gq), uq));
+                }
+                if (row < M) *(uint32_t *)(y + (size_t)row * half + col + (low ? 0 : 2)) = o[0] | (o[1] << 16);
             }
         return;
     }
