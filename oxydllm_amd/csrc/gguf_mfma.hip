@@ -311,6 +311,8 @@ template <int FMT> struct GgmChunk {
     typedef GgmLayout<FMT> L;
     static constexpr int NSTEP = FMT == OXQ_GGUF_Q6_K ? 8 : 4;
     static constexpr bool HAS_MIN = ggm_has_min<FMT>;
+    // vector loads of one request()
+    static constexpr int LOADS = (F::UH ? 1 : 0) + (F::BH ? 1 : 0) + F::WQ + ((FMT == OXQ_GGUF_Q6_K || ggm_fifth_bit<FMT>) ? 1 : 0);
     u32x4_t q[F::WQ];
     uint32_t qh[FMT == OXQ_GGUF_Q6_K ? 2 : 1];
     uint32_t uh[F::UH == 16 ? 4 : F::UH ? 2 : 1];   // unit headers of the column: four f16 d or {d, m} pairs, eight int8 scales (Q6_K)
@@ -633,6 +635,225 @@ __global__ __launch_bounds__(NW * 64) void ggm_kernel(const uint16_t *__restrict
 }
 
 // ---------------------------------------------------------------------------
+// prefill: the decomposition of pk4n_gemm_kernel on the matrix-core copy
+// ---------------------------------------------------------------------------
+// More rows than the integer kernel above should take (every 32 of them read the weights again, and the scale is
+// applied per unit and output) run the tile arithmetic of the reference's mul_mm (quant_kernels.metal strips,
+// linear.rs:270-284 forward_prefill): B = the dequantized weight rounded once to bf16, f32 accumulation.  A
+// workgroup takes 64 rows of x and eight waves x four neighbouring strips (512 columns); a chunk (128 elements of
+// K) of the rows goes from global memory straight into LDS once for all eight waves (two buffers, one barrier a
+// chunk); a wave rings its four strips' chunks in two halves, turns a step's integers into the weight with one
+// fma each (two where a five-bit format has a minimum) from the integer kernel's own factors, and keeps the whole
+// K in its accumulators: one launch, no partial tiles.
+template <int FMT, int MT>
+__global__ __launch_bounds__(512) void ggm_gemm_kernel(const uint16_t *__restrict__ x, const uint8_t *__restrict__ pw,
+                                                       const uint16_t *__restrict__ bias, uint16_t *__restrict__ y,
+                                                       int M, int K, int N, int NG, int RT, int act) {
+    typedef BF16Traits TT;
+    typedef MfmaOps<TT> Ops;
+    typedef GgmFmt<FMT> F;
+    typedef GgmLayout<FMT> L;
+    typedef GgmChunk<FMT> C;
+    constexpr int ROWS = 16 * MT, XBUF = ROWS * 256, XV = ROWS / 32, NSTEP = C::NSTEP;
+    constexpr bool K16 = NSTEP == 8;
+    constexpr int RING = 4 * C::LOADS;  // vector loads of a chunk's weights: younger than the chunk's loads of x
+    extern __shared__ __attribute__((aligned(16))) unsigned char pk4_lds[];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int ni = lane & 15, kb = lane >> 4;
+    int rt, g;
+    pk4g_tile_of((int)blockIdx.x, RT, NG, rt, g);
+    if (g >= NG) return;  // the whole workgroup, before any barrier
+    const int j = g * 8 + wave;  // the wave's 64 columns: strips 4 j .. 4 j + 3
+    const bool live = j < (N >> 6);
+    const int m0 = rt * ROWS;
+    const int NC = K >> 7;
+    const int xrows = min(M - m0, ROWS);
+
+    const uint32_t strip_bytes = (uint32_t)(NC / F::CH) * (uint32_t)L::BLKB;
+    const __amdgpu_buffer_rsrc_t rs_none = make_rsrc(pw, 0u);
+    const __amdgpu_buffer_rsrc_t rs_wl = make_rsrc(pw + (size_t)(live ? 4 * j : 0) * strip_bytes, 4u * strip_bytes);
+    const __amdgpu_buffer_rsrc_t rs_w = live ? rs_wl : rs_none;
+    const __amdgpu_buffer_rsrc_t rs_x = make_rsrc(x + (size_t)m0 * K, (uint32_t)xrows * (uint32_t)K * 2u);
+    // x: load q of a wave brings rows 4 (XV wave + q) .. + 3 of the chunk, lane l the 16 bytes that belong at
+    // position l % 16 of row l / 16 (piece (l % 16) ^ (row % 16): the swizzle the fragment reads undo); rows past
+    // M lie beyond the descriptor and arrive as zeros
+    int xo[XV];
+#pragma unroll
+    for (int q = 0; q < XV; ++q) {
+        const int r = 4 * (wave * XV + q) + (lane >> 4);
+        xo[q] = r * K * 2 + (((lane & 15) ^ (r & 15)) << 4);
+    }
+    int a_rd[NSTEP];
+#pragma unroll
+    for (int st = 0; st < NSTEP; ++st)
+        a_rd[st] = K16 ? ni * 256 + (((2 * st + (kb >> 1)) ^ ni) << 4) + (kb & 1) * 8 : ni * 256 + (((4 * st + kb) ^ ni) << 4);
+    const NibbleMasks nm = FMT == OXQ_GGUF_Q6_K ? NibbleMasks{vgpr_const(0x000F000Fu), vgpr_const(0x00300030u)}
+                           : ggm_fifth_bit<FMT> ? NibbleMasks{vgpr_const(0x000F000Fu), vgpr_const(0x00100010u)} : nibble_masks();
+    constexpr float NEGF = __builtin_bit_cast(float, (F::NEG & 0xFFFFu) << 16);
+    constexpr bool NIB = FMT == OXQ_GGUF_Q4_0 || FMT == OXQ_GGUF_Q4_1 || FMT == OXQ_GGUF_Q4_K;
+
+    C wr[2][4];
+    auto dma_x = [&](int i) {
+        const __amdgpu_buffer_rsrc_t rs = i < NC ? rs_x : rs_none;
+#pragma unroll
+        for (int q = 0; q < XV; ++q)
+            pk4g_load_lds16(rs, pk4_lds + (i & 1) * XBUF + (wave * XV + q) * 1024, xo[q], i * 256);
+    };
+    auto request = [&](int i, C (&w)[4]) {
+        const __amdgpu_buffer_rsrc_t rs = i < NC ? rs_w : rs_none;
+#pragma unroll
+        for (int f = 0; f < 4; ++f) w[f].request(rs, lane, ni, i, (int)(f * strip_bytes));
+    };
+
+    dma_x(0);
+    __builtin_amdgcn_sched_barrier(0);  // requests keep this order: the wait counts rely on it
+    request(0, wr[0]);
+    __builtin_amdgcn_sched_barrier(0);
+    float4_t acc[MT][4];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int f = 0; f < 4; ++f) acc[mt][f] = float4_t{0.f, 0.f, 0.f, 0.f};
+    pk4g_wait_vmcnt<RING>();
+    __syncthreads();
+
+    auto chunk = [&](int i, auto cur_c) {
+        constexpr int CUR = decltype(cur_c)::value;
+        dma_x(i + 1);
+        __builtin_amdgcn_sched_barrier(0);
+        request(i + 1, wr[CUR ^ 1]);
+        __builtin_amdgcn_sched_barrier(0);  // not sunk to the chunk's end, where the next chunk would wait for them
+        const unsigned char *buf = pk4_lds + (i & 1) * XBUF;
+        // w = f0 q' + c2 with q' = q minus the format's offset and c2 = -(minimum): exact products, one rounding -
+        // the bits of the dense dequant (ggm_dequant_kernel), so the tile the matrix cores see is the reference's
+        float f0[4][NSTEP], c2[4][C::HAS_MIN ? NSTEP : 1];
+#pragma unroll
+        for (int f = 0; f < 4; ++f) {
+            float f1[NSTEP];
+            wr[CUR][f].factors(i & 1, ni, f0[f], f1);
+            if constexpr (C::HAS_MIN) {
+#pragma unroll
+                for (int st = 0; st < NSTEP; ++st) c2[f][st] = -128.0f * f1[st];
+            }
+        }
+#pragma unroll
+        for (int st = 0; st < NSTEP; ++st) {
+            uint32_t a[MT][4];
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                if constexpr (K16) {
+                    const uint2 av = *(const uint2 *)(buf + mt * 4096 + a_rd[st]);
+                    a[mt][0] = av.x, a[mt][1] = av.y, a[mt][2] = 0u, a[mt][3] = 0u;
+                } else {
+                    const u32x4_t av = *(const u32x4_t *)(buf + mt * 4096 + a_rd[st]);
+                    a[mt][0] = av[0], a[mt][1] = av[1], a[mt][2] = av[2], a[mt][3] = av[3];
+                }
+            }
+#pragma unroll
+            for (int f = 0; f < 4; ++f) {
+                uint32_t b[4];
+                const float sc = f0[f][st];
+                if constexpr (NIB) {
+                    // plain nibbles (pair pp = nibble pp of each 16-bit half): masked in place a byte holds q or 16 q,
+                    // which v_cvt_f32_ubyteN widens; one fma a weight
+                    uint32_t tl, th;
+                    pk4g_nibbles(wr[CUR][f].q[0][st], tl, th);
+                    Pk4gBf16 cv;
+                    cv.s = sc, cv.s16 = sc * 0.0625f, cv.c = C::HAS_MIN ? c2[f][st] : (NEGF + 128.0f) * sc;
+                    b[0] = cv.template pair<0, false>(tl), b[1] = cv.template pair<0, true>(th);
+                    b[2] = cv.template pair<1, false>(tl), b[3] = cv.template pair<1, true>(th);
+                } else if constexpr (FMT == OXQ_GGUF_Q8_0) {
+                    // bytes q + 128, elements 0, 2, 1, 3 of a word's four: pairs in bytes (0, 2) and (1, 3)
+                    const uint32_t w0 = wr[CUR][f].q[st >> 1][2 * (st & 1)], w1 = wr[CUR][f].q[st >> 1][2 * (st & 1) + 1];
+                    Pk4gBf16 cv;
+                    cv.s = sc, cv.s16 = 0.f, cv.c = -128.0f * sc;
+                    b[0] = cv.template pair<0, false>(w0), b[1] = cv.template pair<1, false>(w0);
+                    b[2] = cv.template pair<0, false>(w1), b[3] = cv.template pair<1, false>(w1);
+                } else {
+                    // bias + q as bf16 (the integer kernel's operand): f0 (bias + q) + NEG f0 is exact in one fma
+                    wr[CUR][f].operand(st, b, nm);
+                    const float c = NEGF * sc;
+#pragma unroll
+                    for (int pp = 0; pp < (K16 ? 2 : 4); ++pp) {
+                        float lo = __builtin_fmaf(__builtin_bit_cast(float, b[pp] << 16), sc, c);
+                        float hi = __builtin_fmaf(__builtin_bit_cast(float, b[pp] & 0xFFFF0000u), sc, c);
+                        if constexpr (C::HAS_MIN) lo += c2[f][st], hi += c2[f][st];
+                        b[pp] = __builtin_bit_cast(uint32_t, __builtin_convertvector(float2_t{lo, hi}, bf16x2_t));
+                    }
+                }
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+                    if constexpr (K16) acc[mt][f] = ggm_mfma16(a[mt][0], a[mt][1], b[0], b[1], acc[mt][f]);
+                    else acc[mt][f] = Ops::mfma(a[mt], b, acc[mt][f]);
+                }
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        pk4g_wait_vmcnt<RING>();  // this wave's part of the next chunk of x is in LDS
+        __syncthreads();
+    };
+    {
+        int i = 0;
+        for (; i + 1 < NC; i += 2) {
+            chunk(i, std::integral_constant<int, 0>{});
+            chunk(i + 1, std::integral_constant<int, 1>{});
+        }
+        if (i < NC) chunk(i, std::integral_constant<int, 0>{});
+    }
+
+    if (!live) return;
+    if (act) {
+        // Fused gate|up layer (ggm_src_row): strip 4 j + f holds gate columns 8 (4 j + f) .. + 7 in lanes ni < 8 and
+        // the up columns they meet in lanes ni + 8.  The two lanes of a pair exchange their four values (row_ror:8)
+        // and finish two outputs each; both factors rounded to bf16 first, as in ggm_epilogue_act.  y is [M, N / 2].
+        const int half = N >> 1, p = ni & 7;
+        const bool low = ni < 8;
+        float bv[4] = {0.f, 0.f, 0.f, 0.f};
+        if (bias) {
+#pragma unroll
+            for (int f = 0; f < 4; ++f) bv[f] = TT::to_f32(bias[(low ? 0 : half) + 8 * (4 * j + f) + p]);
+        }
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int row = m0 + 16 * mt + 4 * kb + e;
+                float mine[4], other[4];
+#pragma unroll
+                for (int f = 0; f < 4; ++f) {
+                    mine[f] = TT::to_f32(TT::from_f32(acc[mt][f][e] + bv[f]));
+                    other[f] = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, mine[f]), 0x128, 0xF, 0xF, false));
+                }
+#pragma unroll
+                for (int q = 0; q < 2; ++q) {
+                    const int f = low ? q : 2 + q;
+                    const float gq = low ? mine[q] : other[2 + q], uq = low ? other[q] : mine[2 + q];
+                    const uint16_t o = TT::from_f32(mul_f32_rn(act == 1 ? silu_f32(gq) : gelu_tanh_f32(gq), uq));
+                    if (row < M) y[(size_t)row * half + 8 * (4 * j + f) + p] = o;
+                }
+            }
+        return;
+    }
+    // row 16 mt + 4 kb + e, column 64 j + 16 f + ni
+    float bv[4] = {0.f, 0.f, 0.f, 0.f};
+    if (bias) {
+#pragma unroll
+        for (int f = 0; f < 4; ++f) bv[f] = TT::to_f32(bias[64 * j + 16 * f + ni]);
+    }
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int row = m0 + 16 * mt + 4 * kb + e;
+            if (row >= M) continue;
+#pragma unroll
+            for (int f = 0; f < 4; ++f) y[(size_t)row * N + 64 * j + 16 * f + ni] = TT::from_f32(acc[mt][f][e] + bv[f]);
+        }
+}
+
+// ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
 static bool ggm_format(int quant) {
@@ -781,6 +1002,67 @@ int launch_gguf_mfma(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p) {
     case OXQ_GGUF_Q5_1: return ggm_by_shape<OXQ_GGUF_Q5_1>(s, grid, p, nullptr, cslice, mt, xq, nw, ns);
     case OXQ_GGUF_Q5_K: return ggm_by_shape<OXQ_GGUF_Q5_K>(s, grid, p, nullptr, cslice, mt, xq, nw, ns);
     default: return fail(OXQ_ERR_UNSUPPORTED, "gguf matrix-core matmul: format %d", p.quant);
+    }
+}
+
+// Rows from which a bf16 layer's matrix-core copy runs the prefill kernel instead of the tile matmul on the file
+// layout (gguf_mm: a workgroup of 64 rows x 64 columns with K slices).  Costs in rounds of 256 workgroups of 64
+// rows x 512 columns (one a CU), as for the packed layers (pk4_gemm_rows).
+bool gguf_gemm_takes(const oxq_ctx *ctx, int quant, int64_t M, int64_t K, int64_t N, int act_dtype) {
+    (void)K;
+    // OXQ_GGUF_GEMM_MIN_M: unset = by cost, 0 = never, n = from n rows on whatever the cost
+    const int64_t v = tune(ctx, OXQ_TUNE_GGUF_GEMM_MIN_M, -1);
+    if (v == 0 || act_dtype != OXQ_BF16 || !ggm_format(quant) || M <= 32 || N % 64 != 0) return false;
+    if (v > 0) return M >= v;
+    // Costs in rounds of one 64-row workgroup a CU (154 - 210 registers: no second one fits).  A last round that
+    // fills at most three quarters of the CUs costs 0.95; the file-layout tile matmul 1.55 w (1.75 w below one
+    // round) for the formats whose conversion is one fma a weight, 1.3 w (1.45 w) for the five- and six-bit ones.
+    // Fitted to 4096 x 4096, 4096 x 14336 and 14336 x 4096 at 64 - 4096 rows.
+    const bool light = quant == OXQ_GGUF_Q4_0 || quant == OXQ_GGUF_Q4_1 || quant == OXQ_GGUF_Q4_K || quant == OXQ_GGUF_Q8_0;
+    const double cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
+    const double w64 = (double)(ceil_div(N / 64, (int64_t)8) * ceil_div(M, (int64_t)64)) / cus;
+    const double whole = std::floor(w64), rest = w64 - whole;
+    const double c64 = whole + (rest <= 0.0 ? 0.0 : rest <= 0.75 ? 0.95 : 1.0);
+    const double split = w64 < 1.0 ? (light ? 1.75 : 1.45) : (light ? 1.55 : 1.3);
+    return split * w64 > c64;
+}
+
+template <int FMT>
+static int ggm_gemm_go(hipStream_t s, dim3 grid, const GgufProblem &p, int NG, int RT) {
+    static LdsGrant grant;  // one per instantiation
+    constexpr int MT = 4;
+    const size_t lds = 2 * 16 * MT * 256;
+    OXQ_HIP_CHECK(grant.ensure((const void *)ggm_gemm_kernel<FMT, MT>, lds));
+    hipLaunchKernelGGL((ggm_gemm_kernel<FMT, MT>), grid, dim3(512), lds, s, (const uint16_t *)p.x, p.w, (const uint16_t *)p.bias,
+                       (uint16_t *)p.y, (int)p.M, (int)p.K, (int)p.N, NG, RT, p.act);
+    OXQ_HIP_CHECK(hipGetLastError());
+    return OXQ_OK;
+}
+
+// p.w is the matrix-core copy; p.act as for launch_gguf_mfma
+int launch_gguf_gemm(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p) {
+    const int rows = 64;
+    const int64_t NG = ceil_div(p.N / 64, (int64_t)8), RT = ceil_div(p.M, (int64_t)rows);
+    const int64_t wgs = (RT / 8) * ceil_div(NG, (int64_t)8) * 64 + (RT % 8) * NG;
+    if (wgs > 0x7FFFFFFF) return fail(OXQ_ERR_UNSUPPORTED, "gguf prefill matmul: m = %lld exceeds the grid", (long long)p.M);
+    dim3 grid((unsigned)wgs);
+    char name[64];
+    snprintf(name, sizeof name, "gguf_%s_gemm_bf16_r%dx8%s", ggm_name(p.quant), rows, p.act == 1 ? "_silu" : p.act == 2 ? "_gelu" : "");
+    set_plan(ctx, name, grid, dim3(512), 1, 1, 0);
+    if (ctx->plan_only) return OXQ_OK;
+    if (p.act_dtype != OXQ_BF16) return fail(OXQ_ERR_UNSUPPORTED, "gguf prefill matmul: activations must be BF16");
+    if ((uint64_t)rows * (uint64_t)p.K * 2 >= (1ull << 31)) return fail(OXQ_ERR_UNSUPPORTED, "gguf prefill matmul: K too large");
+    if (((uintptr_t)p.x & 15) || ((uintptr_t)p.y & 1)) return fail(OXQ_ERR_UNSUPPORTED, "gguf prefill matmul: x must be 16-byte aligned");
+    switch (p.quant) {
+    case OXQ_GGUF_Q4_0: return ggm_gemm_go<OXQ_GGUF_Q4_0>(s, grid, p, (int)NG, (int)RT);
+    case OXQ_GGUF_Q8_0: return ggm_gemm_go<OXQ_GGUF_Q8_0>(s, grid, p, (int)NG, (int)RT);
+    case OXQ_GGUF_Q4_K: return ggm_gemm_go<OXQ_GGUF_Q4_K>(s, grid, p, (int)NG, (int)RT);
+    case OXQ_GGUF_Q6_K: return ggm_gemm_go<OXQ_GGUF_Q6_K>(s, grid, p, (int)NG, (int)RT);
+    case OXQ_GGUF_Q4_1: return ggm_gemm_go<OXQ_GGUF_Q4_1>(s, grid, p, (int)NG, (int)RT);
+    case OXQ_GGUF_Q5_0: return ggm_gemm_go<OXQ_GGUF_Q5_0>(s, grid, p, (int)NG, (int)RT);
+    case OXQ_GGUF_Q5_1: return ggm_gemm_go<OXQ_GGUF_Q5_1>(s, grid, p, (int)NG, (int)RT);
+    case OXQ_GGUF_Q5_K: return ggm_gemm_go<OXQ_GGUF_Q5_K>(s, grid, p, (int)NG, (int)RT);
+    default: return fail(OXQ_ERR_UNSUPPORTED, "gguf prefill matmul: format %d has no matrix-core layout", p.quant);
     }
 }
 

@@ -2220,6 +2220,7 @@ int oxq_qlinear_forward(oxq_qlinear *l, void *stream, const oxq_tensor *x, const
         p.bias = l->has_bias ? l->bias.data : nullptr;
         p.w = (const uint8_t *)l->res;
         p.act = l->act;
+        if (gguf_gemm_takes(l->ctx, l->quant, p.M, p.K, p.N, p.act_dtype)) return launch_gguf_gemm(l->ctx, (hipStream_t)stream, p);
         return launch_gguf_mfma(l->ctx, (hipStream_t)stream, p);
     }
     OXQ_TRY(check_gguf(l->ctx, decode ? "GgufQuantMatmul" : "GgufQuantMulMM", decode, false, &x2,
@@ -2229,6 +2230,10 @@ int oxq_qlinear_forward(oxq_qlinear *l, void *stream, const oxq_tensor *x, const
         if (gguf_mfma_takes(l->ctx, p.M, p.N, p.act_dtype) && ((uintptr_t)p.x & 15) == 0) {
             p.w = (const uint8_t *)l->res;
             return launch_gguf_mfma(l->ctx, (hipStream_t)stream, p);
+        }
+        if (gguf_gemm_takes(l->ctx, l->quant, p.M, p.K, p.N, p.act_dtype) && ((uintptr_t)p.x & 15) == 0) {
+            p.w = (const uint8_t *)l->res;
+            return launch_gguf_gemm(l->ctx, (hipStream_t)stream, p);
         }
     } else if (l->resident && gguf_res_takes(p.K, p.M, p.act_dtype) && ((uintptr_t)p.x & 15) == 0) {
         p.w = (const uint8_t *)l->res;
@@ -2246,6 +2251,12 @@ static int qlinear_forward_unfused(oxq_qlinear *l, void *stream, const oxq_tenso
                        l->in_features, l->out_features, l->quant, gu, &p));
     p.bias = l->has_bias ? l->bias.data : nullptr;
     return qlinear_forward_file_layout(l, stream, p);
+}
+
+// whether `rows` rows of a bf16 layer run the prefill kernel on its matrix-core copy (a fused gate|up layer then
+// keeps its activation in that kernel's epilogue, and the plain layer takes the same kernel: the same bits)
+static bool qlinear_prefill_on_copy(const oxq_qlinear *l, int64_t rows) {
+    return l->resident && l->mfma && gguf_gemm_takes(l->ctx, l->quant, rows, l->in_features, l->out_features, l->out_dtype);
 }
 
 int oxq_qlinear_is_resident(const oxq_qlinear *l, int *resident) {
@@ -2500,7 +2511,8 @@ int oxq_mlp_forward(oxq_mlp *m, void *stream, const oxq_tensor *x, const oxq_ten
     oxq_tensor h;  // [rows, I]: act(gate) * up, the input of down_proj
     switch (m->gate_up_kind) {
     case OXQ_GATE_UP_FUSED:
-        if (m->epilogue && m->a.kind == OXQ_LINEAR_GGUF && rows > OXQ_GGUF_FUSED_ACT_ROWS) {
+        if (m->epilogue && m->a.kind == OXQ_LINEAR_GGUF && rows > OXQ_GGUF_FUSED_ACT_ROWS &&
+            !qlinear_prefill_on_copy((const oxq_qlinear *)m->a.layer, rows)) {
             // every row tile of the fused kernel reads the weights again: the tile matmul and the activation by itself
             const oxq_tensor gu = rows_view(scratch, 0, rows, 2 * I);
             h = rows_view(scratch, rows * 2 * I, rows, I);

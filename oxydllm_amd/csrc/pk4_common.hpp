@@ -42,6 +42,49 @@ template <> struct Pk4T<BF16Traits> {
     }
 };
 
+// ---- shared by the prefill kernels (rows x eight waves of 64 columns a workgroup, x through LDS) ----
+typedef __attribute__((address_space(3))) void *pk4g_lds_ptr_t;
+// 16 bytes a lane from global memory into LDS at lds + 16 lane.  Kept out of the kernel template: the host pass
+// rejects the 16-byte form where it instantiates a template, and then drops the kernel's stub without a word.
+__device__ __forceinline__ void pk4g_load_lds16(__amdgpu_buffer_rsrc_t rs, unsigned char *lds, int voff, int soff) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (pk4g_lds_ptr_t)lds, 16, voff, soff, 0, 0);
+}
+template <int N> __device__ __forceinline__ void pk4g_wait_vmcnt() {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+// Workgroup -> (row tile, strip group).  Bands of 8 row tiles are cut into squares of 8 row tiles x 8 strip groups,
+// 64 neighbouring workgroups each (neighbour i runs on XCD i % 8: a row tile stays on one XCD); the last RT % 8
+// row tiles are numbered row tile first, so that no XCD is handed only idle workgroups.
+__device__ __forceinline__ void pk4g_tile_of(int id, int RT, int NG, int &rt, int &g) {
+    const int full = (RT >> 3) * ((NG + 7) >> 3) * 64, tail = RT & 7;
+    if (id < full) {
+        const int sq = id >> 6, within = id & 63, bands = RT >> 3;
+        rt = (sq % bands) * 8 + (within & 7), g = (sq / bands) * 8 + (within >> 3);
+    } else {
+        rt = (RT & ~7) + (id - full) % tail, g = (id - full) / tail;
+    }
+}
+
+// bf16 has no packed 16-bit arithmetic: a weight goes nibble -> f32 -> fma -> (a pair at a time) bf16.  Masked in
+// place, a byte of the word holds q (low nibbles) or 16 q (high nibbles), which v_cvt_f32_ubyteN widens in one
+// instruction; the high nibbles' fma takes s / 16.  (q - z) s is exact in f32 either way: the same bits as
+// Pk4T<BF16Traits>::deq, with a sixth fewer instructions.
+struct Pk4gBf16 {
+    float s, s16, c;  // scale, scale / 16, -z * scale
+    __device__ __forceinline__ void set(float scale, float minus_z) { s = scale, s16 = scale * 0.0625f, c = minus_z * scale; }
+    // the pair in bytes B and B + 2 of v; HIGH: v holds high nibbles
+    template <int B, bool HIGH> __device__ __forceinline__ uint32_t pair(uint32_t v) const {
+        const float lo = (float)((v >> (8 * B)) & 0xFFu), hi = (float)((v >> (8 * B + 16)) & 0xFFu);
+        const float m = HIGH ? s16 : s;
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(float2_t{__builtin_fmaf(lo, m, c), __builtin_fmaf(hi, m, c)}, bf16x2_t));
+    }
+};
+__device__ __forceinline__ void pk4g_nibbles(uint32_t w, uint32_t &lo, uint32_t &hi) {
+    lo = w & 0x0F0F0F0Fu, hi = w & 0xF0F0F0F0u;
+    asm volatile("" : "+v"(lo), "+v"(hi));  // keep the masks here: folded into the byte extracts they cost one each
+}
+
 constexpr int PK4N_BW = 272;  // 16-column strips: words of one block, 256 of weights and 16 of pairs
 
 // The constants of one column and block from its pair word {-z, s}; deq() = T((q - z) * s) of a row pair.

@@ -447,7 +447,11 @@ def test_layers_validate_like_reference(lib, ctx):
     # rows 1-4: the GEMV on the layer's strip-major copy; 5-8 the tile matmul with unrounded weights
     for m_rows, kern in [(1, "gguf_q4k_mfma_bf16_mt1"), (2, "gguf_q4k_mfma_bf16_mt1"),
                          (4, "gguf_q4k_mfma_bf16_mt1"), (8, "gguf_q4k_mfma_bf16_mt1"),
-                         (16, "gguf_q4k_mfma_bf16_mt1"), (32, "gguf_q4k_mfma_bf16_mt2"), (33, "gguf_q4k_mul_mm_bf16_mt4")]:
+                         (16, "gguf_q4k_mfma_bf16_mt1"), (32, "gguf_q4k_mfma_bf16_mt2"), (33, "gguf_q4k_mul_mm_bf16_mt4"),
+                         # prefill: the tile matmul on the file layout until eight groups of 512 columns x row tiles
+                         # of 64 fill the chip, then the kernel on the layer's copy
+                         (1024, "gguf_q4k_mul_mm_bf16_mt4"), (1536, "gguf_q4k_gemm_bf16_r64x8"),
+                         (4096, "gguf_q4k_gemm_bf16_r64x8")]:
         assert lib.oxq_qlinear_forward(q, None, C.byref(fake((m_rows, 4096), BF16)),
                                        C.byref(fake((m_rows, 4096), BF16))) == 0, err(lib)
         p = plan(lib, ctx)

@@ -247,6 +247,76 @@ def test_fused_gate_up_rows_beyond_a_tile_and_refusals(fmt):
         fused.forward(to_dev(x[:2]))
 
 
+@pytest.mark.parametrize("fmt", FMTS)
+@pytest.mark.parametrize("N,K", [(576, 512), (1088, 1280), (64, 256)])
+def test_prefill_kernel_on_the_matrix_core_copy(fmt, N, K):
+    """linear.rs:270-284 forward_prefill: more rows than the integer kernel takes run the tile arithmetic (the
+    dequantized weight rounded to bf16, f32 accumulation) from the same copy - a workgroup of 64 rows x eight waves
+    of 64 columns, x shared in LDS.  N = 576 and 1088 leave the last group one live wave of eight, N = 64 is one
+    wave; m covers a ragged row tile, a whole band of eight row tiles with a remainder (581 rows) and two bands;
+    K of 2, 4 and 10 chunks (both ring halves, an odd count, both halves of a K-quant block).  The weights the
+    matrix cores see are bit for bit the dense dequant's, so the tile oracle holds at the GEMV tolerance; run to run
+    bitwise; a row's bits do not depend on m."""
+    name = synth.GGUF_NAMES[fmt]
+    tune("OXQ_GGUF_GEMM_MIN_M", 33)
+    bias = ((np.arange(N, dtype=np.float32) % 13) - 6) * np.float32(0.25)
+    data, layer = _layer(fmt, N, K, seed=N + K + fmt, bias=bias)
+    w = oracle.round_through(oracle.dequantize_gguf(fmt, data, N, K), oracle.BF16)
+    x = np.random.default_rng(K + N).standard_normal((1030, K)).astype(np.float32)
+    xd = to_dev(x, torch.bfloat16)
+    tile_all = oracle.matmul_nt_f32(round_x(x, oracle.BF16), w, round_x(bias, oracle.BF16))
+    first = None
+    for m in (1030, 33, 64, 65, 300, 581):
+        say(f"gguf prefill {name} N={N} K={K} m={m}")
+        y = layer.forward(xd[:m])
+        plan = ops.default_context().last_plan()
+        rt, ng = -(-m // 64), -(-(N // 64) // 8)
+        assert plan["kernel"] == f"gguf_{TAG[fmt]}_gemm_bf16_r64x8" and plan["launches"] == 1, plan
+        assert plan["grid"][0] == (rt // 8) * (-(-ng // 8)) * 64 + (rt % 8) * ng and plan["block"][0] == 512, plan
+        assert tuple(y.shape) == (m, N)
+        assert_close(y, tile_all[:m], f"gguf prefill {name} N={N} K={K} m={m}", bf16_out=True)
+        assert np.array_equal(bits_of(layer.forward(xd[:m])), bits_of(y)), "run to run"
+        if first is None:
+            first = bits_of(y)
+        else:
+            np.testing.assert_array_equal(bits_of(y), first[:m])
+    # OXQ_GGUF_GEMM_MIN_M = 0: the tile matmul on the file layout, same arithmetic in another order
+    tune("OXQ_GGUF_GEMM_MIN_M", 0)
+    y0 = layer.forward(xd[:300])
+    assert "_mul_mm_bf16" in ops.default_context().last_plan()["kernel"]
+    assert_close(y0, tile_all[:300], f"gguf tile matmul {name}", bf16_out=True)
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+@pytest.mark.parametrize("act", ["silu", "gelu_tanh"])
+def test_fused_gate_up_activation_at_prefill(fmt, act):
+    """The prefill kernel's own activation epilogue (gate and up columns of an output sit in lanes 8 apart of the
+    accumulator layout) against the plain layer through the same kernel followed by oxq_gated_activation: the same
+    bits, with and without bias; I = 288 leaves the last group one live wave."""
+    kind = ops.ACT_GATED_SILU if act == "silu" else ops.ACT_GATED_GELU_TANH
+    name = synth.GGUF_NAMES[fmt]
+    tune("OXQ_GGUF_GEMM_MIN_M", 33)
+    K, I = 512, 288
+    N = 2 * I
+    data = synth.gguf_weight(fmt, N, K, seed=K + I + fmt)
+    wd = to_dev(data)
+    xd = to_dev(np.random.default_rng(5).standard_normal((300, K)).astype(np.float32), torch.bfloat16)
+    for with_bias in (False, True):
+        bias = ((np.arange(N, dtype=np.float32) % 9) - 4) * np.float32(0.5) if with_bias else None
+        bd = None if bias is None else to_dev(bias, torch.bfloat16)
+        plain = ops.QLinear(fmt, wd, K, N, bd, torch.bfloat16)
+        fused = ops.QLinear(fmt, wd, K, N, bd, torch.bfloat16, gate_up_act=kind)
+        for m in (33, 65, 300):
+            say(f"gguf fused gate|up prefill {name} {act} bias={with_bias} m={m}")
+            y = fused.forward(xd[:m])
+            plan = ops.default_context().last_plan()
+            assert plan["kernel"] == f"gguf_{TAG[fmt]}_gemm_bf16_r64x8_" + ("silu" if act == "silu" else "gelu"), plan
+            assert tuple(y.shape) == (m, I) and plan["launches"] == 1
+            gu = plain.forward(xd[:m])
+            assert ops.default_context().last_plan()["kernel"] == f"gguf_{TAG[fmt]}_gemm_bf16_r64x8"
+            np.testing.assert_array_equal(bits_of(y), bits_of(ops.gated_activation(gu, kind)))
+
+
 @pytest.mark.parametrize("fmt", [synth.GGUF_Q4_0, synth.GGUF_Q4_K, synth.GGUF_Q5_K, synth.GGUF_Q6_K])
 def test_feed_forward_over_a_fused_gguf_layer(fmt):
     """FeedForward (ffn.rs:386-474) with the fused-activation layer as gate_up_proj gives the bits of the layer built
