@@ -1,7 +1,7 @@
 """Timings of the other benchmark configurations (`bench.py --all`; `--prefill-only`: its first part alone).
 
 Resident AWQ layers at prefill sizes (256 - 4096 rows; 4096 x 14336, 14336 x 4096, 4096 x 4096 and
-8192 x 28672, f16 and bf16);
+8192 x 28672, f16 and bf16), GGUF layers and a GGUF FFN at prefill sizes;
 GPTQ 4/8-bit GEMV (K=5120, N=13824, g=128, M in {1, 8}); GGUF Q4_0 / Q8_0 / Q4_K /
 Q6_K ... GEMV (M=1, K=N=4096, f32 activations) and tile matmul (M=64..2048, bf16); MXFP4
 gated GGUF FFN at decode (four launches against the fused gate|up layer's two); MXFP4
@@ -99,6 +99,51 @@ def run_prefill(ops, ctx, stream, steps, warmup, time_graph):
             r["mfma_frac"] = round(r["TFLOP_per_s"] / 2500.0, 4)
             out.append(r)
         ctx.set_tuning("OXQ_PK4_GEMM_MIN_M", None)
+    del ffn
+
+    # GGUF layers (bf16 QLinear.forward): the prefill kernel on the layer's matrix-core copy where the launcher
+    # chooses it, beside the tile matmul on the file layout
+    for fmt in (synth.GGUF_Q4_0, synth.GGUF_Q8_0, synth.GGUF_Q4_K, synth.GGUF_Q6_K):
+        for K, N, rows in ((4096, 14336, (512, 2048)), (4096, 4096, (2048, 4096))):
+            data = synth.gguf_weight(fmt, N, K, seed=0x0A0D11F6 + fmt)
+            layer = ops.QLinear(fmt, torch.from_numpy(data).to(dev), K, N, None, torch.bfloat16, ctx=ctx)
+            for m in rows:
+                x = torch.randn((m, K), device=dev, dtype=torch.bfloat16)
+                y = torch.empty((m, N), device=dev, dtype=torch.bfloat16)
+
+                def gstep(i, x=x, y=y, layer=layer):
+                    layer.forward(x, out=y)
+                nb, fl = data.nbytes + m * K * 2 + m * N * 2, 2.0 * m * K * N
+                for label, min_m in (("", None), (" (tile matmul on the file layout, OXQ_GGUF_GEMM_MIN_M=0)", 0)):
+                    ctx.set_tuning("OXQ_GGUF_GEMM_MIN_M", min_m)
+                    r = _case(f"gguf {synth.GGUF_NAMES[fmt]} prefill M={m} K={K} N={N} bf16 (QLinear){label}", gstep, steps,
+                              warmup, stream, time_graph, nb, fl, ctx)
+                    r["mfma_frac"] = round(r["TFLOP_per_s"] / 2500.0, 4)
+                    out.append(r)
+                ctx.set_tuning("OXQ_GGUF_GEMM_MIN_M", None)
+            del layer
+    # the whole gated FFN as a GGUF file holds it (Q4_K): fused gate|up with the activation in the epilogue + down
+    fmt = synth.GGUF_Q4_K
+    gd, ud, dd = (torch.from_numpy(synth.gguf_weight(fmt, n, k, seed=sd)).to(dev) for n, k, sd in ((I, H, 1), (I, H, 2), (H, I, 3)))
+    ffn = ops.FeedForward(ops.GATE_UP_FUSED, ops.QLinear(fmt, torch.cat([gd.reshape(-1), ud.reshape(-1)]), H, 2 * I, None,
+                                                          torch.bfloat16, ctx=ctx, gate_up_act=ops.ACT_GATED_SILU),
+                          None, ops.QLinear(fmt, dd, I, H, None, torch.bfloat16, ctx=ctx), I, ctx=ctx)
+    for m in (2048,):
+        x = torch.randn((m, H), device=dev, dtype=tdt) * 0.1
+        y = torch.empty((m, H), device=dev, dtype=tdt)
+        scratch = torch.empty(m * 3 * I, device=dev, dtype=tdt)
+
+        def gfstep(i, x=x, y=y, scratch=scratch):
+            ffn.forward(x, out=y, scratch=scratch)
+        nb, fl = gd.numel() + ud.numel() + dd.numel() + 2 * m * H * 2, 6.0 * m * H * I
+        for label, min_m in (("fused gate|up with the activation + down, on the layers' copies", None),
+                             ("tile matmul on the file layout, activation kernel, OXQ_GGUF_GEMM_MIN_M=0", 0)):
+            ctx.set_tuning("OXQ_GGUF_GEMM_MIN_M", min_m)
+            r = _case(f"gguf Q4_K gated FFN prefill M={m} H={H} I={I} bf16 (FeedForward: {label})", gfstep, steps, warmup,
+                      stream, time_graph, nb, fl, ctx)
+            r["mfma_frac"] = round(r["TFLOP_per_s"] / 2500.0, 4)
+            out.append(r)
+        ctx.set_tuning("OXQ_GGUF_GEMM_MIN_M", None)
     del ffn
     return out
 

@@ -837,13 +837,14 @@ static bool wcache_forward(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p, i
 }
 
 // The same for a GGUF weight: the copy is the strip-major one of the QLinear layers - the matrix-core layout
-// for bf16 activations (up to the rows its kernel takes), the rotated one of the vector GEMV for f32 (1 - 8
-// rows).  Entry fields: qw = the block bytes, bits = the ggml format, pack_dim = -1 (rotated) or -2
+// for bf16 activations (the rows its kernels take: up to 32, and prefill sizes), the rotated one of the vector
+// GEMV for f32 (1 - 8 rows).  Entry fields: qw = the block bytes, bits = the ggml format, pack_dim = -1 (rotated) or -2
 // (matrix-core), w.pw = the copy.
 static bool wcache_forward_gguf(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p, int *rc) {
     if (!ctx->wcache_limit || ctx->plan_only || !gguf_res_eligible(p.quant, p.K, p.N)) return false;
     const bool mfma = p.act_dtype == OXQ_BF16 && gguf_mfma_eligible(ctx, p.quant, p.K, p.N);
-    if (!(mfma ? gguf_mfma_takes(ctx, p.M, p.N, p.act_dtype) : gguf_res_takes(p.K, p.M, p.act_dtype))) return false;
+    const bool gemm = mfma && gguf_gemm_takes(ctx, p.quant, p.M, p.K, p.N, p.act_dtype);  // prefill sizes, same copy
+    if (!gemm && !(mfma ? gguf_mfma_takes(ctx, p.M, p.N, p.act_dtype) : gguf_res_takes(p.K, p.M, p.act_dtype))) return false;
     const int kind = mfma ? -2 : -1;
     if (((uintptr_t)p.x & 15) || ((uintptr_t)p.w & 1)) return false;
     if (!ctx->wcache) {
@@ -893,7 +894,7 @@ static bool wcache_forward_gguf(oxq_ctx *ctx, hipStream_t s, const GgufProblem &
     wcache_pin_if_capturing(s, hit);
     GgufProblem q = p;
     q.w = (const uint8_t *)hit->w.pw;
-    *rc = mfma ? launch_gguf_mfma(ctx, s, q) : launch_gguf_res_gemv(ctx, s, q);
+    *rc = gemm ? launch_gguf_gemm(ctx, s, q) : mfma ? launch_gguf_mfma(ctx, s, q) : launch_gguf_res_gemv(ctx, s, q);
     return true;
 }
 

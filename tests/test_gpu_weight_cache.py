@@ -18,7 +18,7 @@ import torch
 
 import oracle
 from oxydllm_amd import synth
-from tests.helpers import TORCH_DT, as_f32, assert_close, bits_of, resident_rounds_weights, round_x, to_dev
+from tests.helpers import TORCH_DT, as_f32, assert_close, bits_of, resident_rounds_weights, round_x, to_dev, tune
 
 pytestmark = pytest.mark.gpu
 ops = None
@@ -232,8 +232,16 @@ def test_cached_gguf_op_with_bf16_activations_runs_on_the_matrix_core_copy(fmt):
             np.testing.assert_array_equal(bits_of(y), bits_of(layer.forward(xd)))
             assert_close(y, oracle.matmul_nt_f32(round_x(x, oracle.BF16), w), f"cached gguf bf16 op m={m}", bf16_out=True)
         assert ctx.weight_cache_usage() == (nbytes, 1)
-        ops.gguf_quant_mul_mm(to_dev(x[:1].repeat(33, 0), torch.bfloat16), wd, K, N, fmt, ctx=ctx)
-        assert "_mul_mm_" in ctx.last_plan()["kernel"]  # more rows than the kernel takes: the file layout
+        x33 = to_dev(x[:1].repeat(33, 0), torch.bfloat16)
+        ops.gguf_quant_mul_mm(x33, wd, K, N, fmt, ctx=ctx)
+        assert "_mul_mm_" in ctx.last_plan()["kernel"]  # more rows than the integer kernel takes: the file layout
+        ctx.set_tuning("OXQ_GGUF_GEMM_MIN_M", 33)       # or, where it pays, the prefill kernel on the same copy
+        y33 = ops.gguf_quant_mul_mm(x33, wd, K, N, fmt, ctx=ctx)
+        assert "_gemm_bf16_r64x8" in ctx.last_plan()["kernel"] and ctx.weight_cache_usage() == (nbytes, 1)
+        tune("OXQ_GGUF_GEMM_MIN_M", 33)
+        np.testing.assert_array_equal(bits_of(y33), bits_of(layer.forward(x33)))
+        tune("OXQ_GGUF_GEMM_MIN_M", None)
+        ctx.set_tuning("OXQ_GGUF_GEMM_MIN_M", None)
         ops.gguf_quant_matmul(to_dev(x[:2]), wd, K, N, fmt, ctx=ctx)
         assert "_res_gemv_f32" in ctx.last_plan()["kernel"]
         assert ctx.weight_cache_usage() == (2 * nbytes, 2)
