@@ -70,6 +70,29 @@ def run_prefill(ops, ctx, stream, steps, warmup, time_graph):
                     out.append(r0)
             del layer
 
+    # 8-bit layers (config 2's GPTQ shape): the same kernel with two loads a step
+    K, N = 5120, 13824
+    qw, qz, sc = synth.gptq_checkpoint(K, N, 128, 8, seed=0x0A0D11F7)
+    wbytes = qw.nbytes + qz.nbytes + sc.size * 2
+    for tdt, tn in ((torch.float16, "f16"), (torch.bfloat16, "bf16")):
+        layer = ops.PackedQuantLinear(8, ops.PACK_IN, torch.from_numpy(qw).to(dev), torch.from_numpy(qz).to(dev),
+                                      torch.from_numpy(sc).to(dev, tdt), None, tdt, ctx=ctx)
+        for m in (512, 2048):
+            x = torch.randn((m, K), device=dev, dtype=tdt)
+            y = torch.empty((m, N), device=dev, dtype=tdt)
+
+            def step8(i, x=x, y=y, layer=layer):
+                layer.forward(x, out=y)
+            nb, fl = wbytes + m * K * 2 + m * N * 2, 2.0 * m * K * N
+            for label, min_m in (("", None), (" (split-K tiles, OXQ_PK4_GEMM_MIN_M=0)", 0)):
+                ctx.set_tuning("OXQ_PK4_GEMM_MIN_M", min_m)
+                r = _case(f"gptq8 prefill M={m} K={K} N={N} {tn} (PackedQuantLinear){label}", step8, steps, warmup, stream,
+                          time_graph, nb, fl, ctx)
+                r["mfma_frac"] = round(r["TFLOP_per_s"] / 2500.0, 4)
+                out.append(r)
+            ctx.set_tuning("OXQ_PK4_GEMM_MIN_M", None)
+        del layer
+
     # the whole gated FFN of config 1's model (hidden 4096, intermediate 14336, bf16): the gate|up projection with
     # the activation in its epilogue, then the down projection (stored in 16-column strips) - two launches
     H, I = 4096, 14336

@@ -1,4 +1,4 @@
-// Resident 4-bit layers at prefill sizes (linear.rs:494-509: m >= 64 takes the staged tile GEMM,
+// Resident layers at prefill sizes (linear.rs:494-509: m >= 64 takes the staged tile GEMM,
 // mpp_gemm.metal:101-266): the tile arithmetic of pk4_mfma_kernel - B = T((q - z) * s) rounded once to the
 // activation type, f32 accumulate - in a decomposition for many rows.
 //
@@ -25,12 +25,14 @@ namespace oxq {
 
 constexpr int PK4G_STRIPS = 8;  // strips (= waves) of a workgroup
 
-template <typename TT, int MT>
+template <typename TT, int MT, int BITS>
 __global__ __launch_bounds__(512) void pk4_gemm_kernel(const uint16_t *__restrict__ x, const uint32_t *__restrict__ pw,
                                                        const uint16_t *__restrict__ bias, uint16_t *__restrict__ y,
                                                        int M, int K, int N, int NG, int RT, int act) {
     typedef MfmaOps<TT> Ops;
-    constexpr int ROWS = 16 * MT, BB = pk4_block_words(4) * 4, XBUF = ROWS * 256;
+    constexpr int ROWS = 16 * MT, BB = pk4_block_words(BITS) * 4, XBUF = ROWS * 256;
+    constexpr int WL = BITS / 4;          // 1 KB weight loads a step (8-bit: column pairs 0, 1 and 2, 3)
+    constexpr int RING = 4 * WL + 1;      // ring loads of a block: younger than the block's loads of x
     constexpr bool BF = TT::DTYPE == BF16Traits::DTYPE;
     constexpr int XV = ROWS / 32;  // loads of x a wave issues per block: 64 lanes x 16 bytes = 4 rows each
     extern __shared__ __attribute__((aligned(16))) unsigned char pk4_lds[];
@@ -52,7 +54,7 @@ __global__ __launch_bounds__(512) void pk4_gemm_kernel(const uint16_t *__restric
     const __amdgpu_buffer_rsrc_t rs_w = live ? rs_wl : rs_none;
     const __amdgpu_buffer_rsrc_t rs_x = make_rsrc(x + (size_t)m0 * K, (uint32_t)xrows * (uint32_t)K * 2u);
     const int voff_w = lane * 16;
-    const int voff_z = 1024 * 4 + (ni * 4 + kb) * 4;
+    const int voff_z = 1024 * WL * 4 + (ni * 4 + kb) * 4;
     // x: load q of a wave brings rows 4 (XV wave + q) .. + 3 of the block straight into LDS, lane l the 16 bytes
     // that belong at position l % 16 of row l / 16 - chunk (l % 16) ^ (row % 16) of the row, the swizzle the
     // fragment reads undo.  Rows past M lie beyond the descriptor: LDS receives zeros.
@@ -67,9 +69,9 @@ __global__ __launch_bounds__(512) void pk4_gemm_kernel(const uint16_t *__restric
     for (int st = 0; st < 4; ++st) a_rd[st] = ni * 256 + (((8 * (st >> 1) + 2 * kb + (st & 1)) ^ ni) << 4);
     const NibbleMasks nm = nibble_masks();
 
-    u32x4_t wring[4];
+    u32x4_t wring[4][WL];
     uint32_t zring;
-    // The compiler orders nothing against these loads: the wait for them (the five ring loads of a block are
+    // The compiler orders nothing against these loads: the wait for them (the ring loads of a block are
     // younger) is written out in front of the barrier that publishes the block.
     auto dma_x = [&](int i) {
         const __amdgpu_buffer_rsrc_t rs = i < NB ? rs_x : rs_none;
@@ -79,7 +81,8 @@ __global__ __launch_bounds__(512) void pk4_gemm_kernel(const uint16_t *__restric
     };
     auto load_w = [&](int i, int st) {
         const __amdgpu_buffer_rsrc_t rs = i < NB ? rs_w : rs_none;
-        wring[st] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff_w, i * BB + st * 1024, 0);
+#pragma unroll
+        for (int h = 0; h < WL; ++h) wring[st][h] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff_w, i * BB + (st * WL + h) * 1024, 0);
     };
     auto load_z = [&](int i) {
         const __amdgpu_buffer_rsrc_t rs = i < NB ? rs_w : rs_none;
@@ -104,7 +107,7 @@ __global__ __launch_bounds__(512) void pk4_gemm_kernel(const uint16_t *__restric
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
         for (int f = 0; f < 4; ++f) acc[mt][f] = float4_t{0.f, 0.f, 0.f, 0.f};
-    pk4g_wait_vmcnt<5>();
+    pk4g_wait_vmcnt<RING>();
     __syncthreads();
 
     for (int i = 0; i < NB; ++i) {
@@ -117,8 +120,8 @@ __global__ __launch_bounds__(512) void pk4_gemm_kernel(const uint16_t *__restric
         zs_words(zring, zv);
 #pragma unroll
         for (int f = 0; f < 4; ++f) {
-            if constexpr (BF) {  // the pair word holds {-(128 + z), s}
-                cb[f].set(__builtin_bit_cast(float, zv[f] & 0xFFFF0000u), __builtin_bit_cast(float, zv[f] << 16) + 128.0f);
+            if constexpr (BF) {  // the pair word holds {-(bias + z), s}, bias = 128 for nibbles and 0 for bytes
+                cb[f].set(__builtin_bit_cast(float, zv[f] & 0xFFFF0000u), __builtin_bit_cast(float, zv[f] << 16) + (BITS == 4 ? 128.0f : 0.0f));
             } else {
                 Pk4T<TT>::prep(zv[f], negzb[f], sp[f]);
             }
@@ -126,8 +129,12 @@ __global__ __launch_bounds__(512) void pk4_gemm_kernel(const uint16_t *__restric
         load_z(i + 1);
 #pragma unroll
         for (int st = 0; st < 4; ++st) {
-            const u32x4_t wv = wring[st];
-            const uint32_t wp[4] = {wv[0], wv[1], wv[2], wv[3]};
+            uint32_t wp[WL][4];
+#pragma unroll
+            for (int h = 0; h < WL; ++h) {
+                const u32x4_t wv = wring[st][h];
+                wp[h][0] = wv[0], wp[h][1] = wv[1], wp[h][2] = wv[2], wp[h][3] = wv[3];
+            }
             uint32_t a[MT][4];
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
@@ -135,21 +142,29 @@ __global__ __launch_bounds__(512) void pk4_gemm_kernel(const uint16_t *__restric
                 a[mt][0] = av[0], a[mt][1] = av[1], a[mt][2] = av[2], a[mt][3] = av[3];
             }
             uint32_t tl[4], th[4];
-            if constexpr (BF) {
+            if constexpr (BF && BITS == 4) {
 #pragma unroll
-                for (int pp = 0; pp < 4; ++pp) pk4g_nibbles(wp[pp], tl[pp], th[pp]);
+                for (int pp = 0; pp < 4; ++pp) pk4g_nibbles(wp[0][pp], tl[pp], th[pp]);
             }
 #pragma unroll
             for (int f = 0; f < 4; ++f) {
                 uint32_t b[4];
 #pragma unroll
                 for (int pp = 0; pp < 4; ++pp) {
-                    // column f of word pp: nibble f of each 16-bit half = the low or high nibble of bytes f / 2 and 2 + f / 2
-                    if constexpr (!BF) b[pp] = Pk4T<TT>::deq(TT::unpack1(wp[pp], f, nm), negzb[f], sp[f]);
-                    else if (f == 0) b[pp] = cb[0].template pair<0, false>(tl[pp]);
-                    else if (f == 1) b[pp] = cb[1].template pair<0, true>(th[pp]);
-                    else if (f == 2) b[pp] = cb[2].template pair<1, false>(tl[pp]);
-                    else b[pp] = cb[3].template pair<1, true>(th[pp]);
+                    if constexpr (BITS == 8) {
+                        // word pp of half f / 2: bytes {row 2 pp, row 2 pp + 1} x {column 2 h, 2 h + 1}: the pair of
+                        // column f in bytes f % 2 and f % 2 + 2
+                        const uint32_t word = wp[f >> 1][pp];
+                        if constexpr (BF) b[pp] = (f & 1) ? cb[f].template pair<1, false>(word) : cb[f].template pair<0, false>(word);
+                        else b[pp] = Pk4T<TT>::deq(TT::unpack_bytes((f & 1) ? (word >> 8) : word), negzb[f], sp[f]);
+                    } else {
+                        // column f of word pp: nibble f of each 16-bit half = the low or high nibble of bytes f / 2 and 2 + f / 2
+                        if constexpr (!BF) b[pp] = Pk4T<TT>::deq(TT::unpack1(wp[0][pp], f, nm), negzb[f], sp[f]);
+                        else if (f == 0) b[pp] = cb[0].template pair<0, false>(tl[pp]);
+                        else if (f == 1) b[pp] = cb[1].template pair<0, true>(th[pp]);
+                        else if (f == 2) b[pp] = cb[2].template pair<1, false>(tl[pp]);
+                        else b[pp] = cb[3].template pair<1, true>(th[pp]);
+                    }
                 }
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt) acc[mt][f] = Ops::mfma(a[mt], b, acc[mt][f]);
@@ -157,7 +172,7 @@ __global__ __launch_bounds__(512) void pk4_gemm_kernel(const uint16_t *__restric
             load_w(i + 1, st);  // into the registers this step has just left
         }
         __builtin_amdgcn_sched_barrier(0);
-        pk4g_wait_vmcnt<5>();  // this wave's part of the next block is in LDS; its ring loads may still fly
+        pk4g_wait_vmcnt<RING>();  // this wave's part of the next block is in LDS; its ring loads may still fly
         __syncthreads();
     }
 
@@ -366,10 +381,10 @@ __global__ __launch_bounds__(512) void pk4n_gemm_kernel(const uint16_t *__restri
         }
 }
 
-// Which decomposition a resident 4-bit layer runs at M rows: 0 = the split-K tiles of pk4_mfma_kernel /
+// Which decomposition a resident layer runs at M rows: 0 = the split-K tiles of pk4_mfma_kernel /
 // pk4n_mfma_kernel, else the rows of a workgroup here.  Costs are in units of a full round (one 64-row workgroup
 // on every CU), fitted to sweeps over 128..8192 rows in both types (64-column strips: 4096 x 14336, 8192 x 28672;
-// 16-column strips: 4096 x 4096, 4096 x 6144, 14336 x 4096, 8192 x 8192):
+// 16-column strips: 4096 x 4096, 4096 x 6144, 14336 x 4096, 8192 x 8192; 8-bit: 4096 x 14336, 5120 x 13824):
 //   - 128-row workgroups (203..230 registers: one a CU) run in whole rounds; a round costs `full128`, a last
 //     round that fills at most 0.7 of the CUs `part128`;
 //   - 64-row workgroups of the 64-column layout (121..125 registers) share a CU in pairs: up to one a CU the launch
@@ -384,15 +399,20 @@ struct Pk4GemmCost {
 };
 static int pk4_gemm_rows(const oxq_ctx *ctx, const Pk4Problem &p) {
     const int64_t min_m = tune(ctx, OXQ_TUNE_PK4_GEMM_MIN_M, 65);
-    if (min_m <= 0 || p.w.bits != 4 || (p.act && p.w.strip == 16) || p.M < min_m) return 0;
+    if (min_m <= 0 || (p.w.bits != 4 && p.w.bits != 8) || (p.act && p.w.strip == 16) || p.M < min_m) return 0;
+    if (p.w.bits == 8 && p.w.strip == 16) return 0;  // (16-column strips are a 4-bit layout)
     const int forced = tune(ctx, OXQ_TUNE_PK4_GEMM_ROWS, 0);
     if (forced == 64 || forced == 128) return forced;
     static const Pk4GemmCost WIDE_F16 = {true, 0.88, 1.20, 0.30, 0.97, 1.50, 1.27, 1.70, 1.50};
     static const Pk4GemmCost WIDE_BF16 = {true, 0.93, 1.29, 0.27, 0.98, 1.44, 1.35, 1.75, 1.53};
     static const Pk4GemmCost NARROW_F16 = {false, 0.86, 0, 0, 0, 1.64, 1.30, 1.60, 1.50};
     static const Pk4GemmCost NARROW_BF16 = {false, 0.94, 0, 0, 0, 1.51, 1.35, 1.60, 1.50};
+    static const Pk4GemmCost WIDE8_F16 = {false, 0.88, 0, 0, 0, 1.47, 1.27, 1.92, 1.71};  // 8-bit: 137 registers at 64 rows
+    static const Pk4GemmCost WIDE8_BF16 = {false, 0.91, 0, 0, 0, 1.47, 1.32, 2.00, 1.78};
     const bool f16 = p.w.dtype == OXQ_F16;
-    const Pk4GemmCost &c = p.w.strip == 16 ? (f16 ? NARROW_F16 : NARROW_BF16) : (f16 ? WIDE_F16 : WIDE_BF16);
+    const Pk4GemmCost &c = p.w.bits == 8      ? (f16 ? WIDE8_F16 : WIDE8_BF16)
+                           : p.w.strip == 16 ? (f16 ? NARROW_F16 : NARROW_BF16)
+                                             : (f16 ? WIDE_F16 : WIDE_BF16);
     const double cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
     const int64_t groups = ceil_div(p.w.N / 64, (int64_t)PK4G_STRIPS);
     const double w64 = (double)(groups * ceil_div(p.M, (int64_t)64)) / cus, w128 = (double)(groups * ceil_div(p.M, (int64_t)128)) / cus;
@@ -408,17 +428,17 @@ static int pk4_gemm_rows(const oxq_ctx *ctx, const Pk4Problem &p) {
 }
 bool pk4_gemm_takes(const oxq_ctx *ctx, const Pk4Problem &p) { return pk4_gemm_rows(ctx, p) != 0; }
 
-template <typename TT, int MT, bool N16>
+template <typename TT, int MT, int LAYOUT>  // LAYOUT: 4 / 8 = bits of a layer in 64-column strips, 16 = 4-bit in 16-column strips
 static int pk4_gemm_go(hipStream_t s, dim3 grid, const Pk4Problem &p, int NG, int RT) {
     static LdsGrant grant;  // one per instantiation
     const size_t lds = 2 * 16 * MT * 256;
-    if constexpr (N16) {
+    if constexpr (LAYOUT == 16) {
         OXQ_HIP_CHECK(grant.ensure((const void *)pk4n_gemm_kernel<TT, MT>, lds));
         hipLaunchKernelGGL((pk4n_gemm_kernel<TT, MT>), grid, dim3(512), lds, s, (const uint16_t *)p.x, p.w.pw, (const uint16_t *)p.bias,
                            (uint16_t *)p.y, (int)p.M, (int)p.w.K, (int)p.w.N, NG, RT);
     } else {
-        OXQ_HIP_CHECK(grant.ensure((const void *)pk4_gemm_kernel<TT, MT>, lds));
-        hipLaunchKernelGGL((pk4_gemm_kernel<TT, MT>), grid, dim3(512), lds, s, (const uint16_t *)p.x, p.w.pw, (const uint16_t *)p.bias,
+        OXQ_HIP_CHECK(grant.ensure((const void *)pk4_gemm_kernel<TT, MT, LAYOUT>, lds));
+        hipLaunchKernelGGL((pk4_gemm_kernel<TT, MT, LAYOUT>), grid, dim3(512), lds, s, (const uint16_t *)p.x, p.w.pw, (const uint16_t *)p.bias,
                            (uint16_t *)p.y, (int)p.M, (int)p.w.K, (int)p.w.N, NG, RT, p.act);
     }
     OXQ_HIP_CHECK(hipGetLastError());
@@ -426,7 +446,8 @@ static int pk4_gemm_go(hipStream_t s, dim3 grid, const Pk4Problem &p, int NG, in
 }
 template <typename TT, int MT>
 static int pk4_gemm_go_layout(hipStream_t s, dim3 grid, const Pk4Problem &p, int NG, int RT) {
-    return p.w.strip == 16 ? pk4_gemm_go<TT, MT, true>(s, grid, p, NG, RT) : pk4_gemm_go<TT, MT, false>(s, grid, p, NG, RT);
+    if (p.w.strip == 16) return pk4_gemm_go<TT, MT, 16>(s, grid, p, NG, RT);
+    return p.w.bits == 8 ? pk4_gemm_go<TT, MT, 8>(s, grid, p, NG, RT) : pk4_gemm_go<TT, MT, 4>(s, grid, p, NG, RT);
 }
 
 int launch_pk4_gemm(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p) {
@@ -437,7 +458,7 @@ int launch_pk4_gemm(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p) {
     if (wgs > 0x7FFFFFFF) return fail(OXQ_ERR_UNSUPPORTED, "repacked matmul: m = %lld exceeds the grid", (long long)p.M);
     dim3 grid((unsigned)wgs);
     char name[64];
-    snprintf(name, sizeof name, "pk4_gemm_%s_r%dx8%s%s", p.w.dtype == OXQ_F16 ? "f16" : "bf16", rows, p.w.strip == 16 ? "_n16" : "",
+    snprintf(name, sizeof name, "pk%d_gemm_%s_r%dx8%s%s", p.w.bits, p.w.dtype == OXQ_F16 ? "f16" : "bf16", rows, p.w.strip == 16 ? "_n16" : "",
              p.act == 1 ? "_silu" : p.act == 2 ? "_gelu" : "");
     set_plan(ctx, name, grid, dim3(512), 1, 1, 0);
     if (ctx->plan_only) return OXQ_OK;

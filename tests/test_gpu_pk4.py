@@ -144,10 +144,9 @@ def front_rule(K, ks, m, bits=4):
     return "line" if bslice % 8 == 0 and share8 in (1, 2, 3, 4, 5, 6, 8) else ""
 
 
-@pytest.mark.parametrize("kind", ["awq", "gptq"])
+@pytest.mark.parametrize("kind,strip16", [(k, s16) for k in KINDS for s16 in (0, 2) if not (s16 and k.endswith("8"))])
 @pytest.mark.parametrize("dtn", ["f16", "bf16"])
 @pytest.mark.parametrize("rows", [64, 128])
-@pytest.mark.parametrize("strip16", [0, 2])
 @pytest.mark.parametrize("K,N,g", [(512, 576, 128), (1280, 1088, 128), (256, 64, 128)])
 def test_prefill_rows_by_eight_strips(kind, dtn, rows, K, N, g, strip16):
     """The prefill decomposition (a workgroup = 64 or 128 rows x eight strips, x shared in LDS, a strip per
@@ -156,15 +155,16 @@ def test_prefill_rows_by_eight_strips(kind, dtn, rows, K, N, g, strip16):
     5 of 128; 1100: 16 + 2, 8 + 1) and a band alone; K of 2, 4 and 10 blocks.  Against the tile-GEMM oracle
     (mpp_gemm.metal:115-184: B rounded to the activation type), the reference's own bound against the
     unrounded weights (metal_ops.rs:3713-3716), run to run bitwise, and rows of y independent of m.  Both resident
-    layouts: 64-column strips and (strip16 = 2) the 16-column strips of narrow layers, whose kernel rings whole
-    blocks in two halves (K of 2, 4 and 10 blocks: both halves, and an odd count)."""
+    layouts: 64-column strips (4- and 8-bit) and (strip16 = 2) the 16-column strips of narrow layers, whose kernel
+    rings whole blocks in two halves (K of 2, 4 and 10 blocks: both halves, and an odd count)."""
+    bits = bits_of_kind(kind)  # (16-column strips are a 4-bit layout)
     tune("OXQ_PK4_STRIP16", strip16)
     tune("OXQ_PK4_GEMM_ROWS", rows)
-    kname = f"pk4_gemm_{dtn}_r{rows}x8" + ("_n16" if strip16 else "")
+    kname = f"pk{bits}_gemm_{dtn}_r{rows}x8" + ("_n16" if strip16 else "")
     dt = DT[dtn]
     trip, pack_dim = make(kind, K, N, g, seed=K + 5 * N)
     bias = (np.arange(N, dtype=np.float32) % 13 - 6) * np.float32(0.125)
-    layer = layer_of(trip, pack_dim, dt, bias)
+    layer = layer_of(trip, pack_dim, dt, bias, bits=bits)
     assert layer.prepacked
     w = dense(kind, trip, dt)
     wt = oracle.round_through(w, dt)
@@ -192,7 +192,7 @@ def test_prefill_rows_by_eight_strips(kind, dtn, rows, K, N, g, strip16):
             # a row's result does not depend on how many rows ride along or on which tile it falls
             np.testing.assert_array_equal(bits_of(y), first[:m])
     # without a bias, into a caller's buffer that holds other values
-    plain = layer_of(trip, pack_dim, dt, None)
+    plain = layer_of(trip, pack_dim, dt, None, bits=bits)
     out = torch.full((300, N), 7.0, device="cuda", dtype=TORCH_DT[dt])
     plain.forward(xd_all[:300], out=out)
     assert ops.default_context().last_plan()["kernel"] == kname
@@ -506,7 +506,7 @@ def test_fused_gate_up_activation(kind, dtn, act, K, I, g):
             assert_close(y, ref, f"gate|up {kind} {dtn} {act} m{m}")
 
 
-@pytest.mark.parametrize("kind", ["awq", "gptq"])
+@pytest.mark.parametrize("kind", KINDS)
 @pytest.mark.parametrize("dtn", ["f16", "bf16"])
 @pytest.mark.parametrize("act", ["silu", "gelu"])
 @pytest.mark.parametrize("rows", [64, 128])
@@ -523,19 +523,20 @@ def test_fused_gate_up_activation_at_prefill(kind, dtn, act, rows):
     kind_id = ops.ACT_GATED_SILU if act == "silu" else ops.ACT_GATED_GELU_TANH
     rng = np.random.default_rng(rows)
     xd = to_dev(rng.standard_normal((581, K)).astype(np.float32), tdt)
+    bits = bits_of_kind(kind)
     for b in (None, bias):
-        plain = layer_of(trip, pack_dim, dt, b)
+        plain = layer_of(trip, pack_dim, dt, b, bits=bits)
         bd = None if b is None else to_dev(b, tdt)
-        fused = ops.PackedQuantLinear(4, pack_dim, to_dev(trip[0]), to_dev(trip[1]), to_dev(trip[2], tdt), bd, tdt,
+        fused = ops.PackedQuantLinear(bits, pack_dim, to_dev(trip[0]), to_dev(trip[1]), to_dev(trip[2], tdt), bd, tdt,
                                       gate_up_act=kind_id)
         for m in (65, 300, 581):
             say(f"gate|up prefill {kind} {dtn} {act} r{rows} m={m} bias={b is not None}")
             y = fused.forward(xd[:m])
             plan = ops.default_context().last_plan()
-            assert plan["kernel"] == f"pk4_gemm_{dtn}_r{rows}x8_{act}" and plan["launches"] == 1, plan
+            assert plan["kernel"] == f"pk{bits}_gemm_{dtn}_r{rows}x8_{act}" and plan["launches"] == 1, plan
             assert y.shape == (m, I)
             gu = plain.forward(xd[:m])
-            assert ops.default_context().last_plan()["kernel"] == f"pk4_gemm_{dtn}_r{rows}x8"
+            assert ops.default_context().last_plan()["kernel"] == f"pk{bits}_gemm_{dtn}_r{rows}x8"
             np.testing.assert_array_equal(bits_of(y), bits_of(ops.gated_activation(gu, kind_id)))
             ref = oracle.gated_silu(as_f32(gu)) if act == "silu" else oracle.gated_gelu_tanh(as_f32(gu))
             assert_close(y, ref, f"gate|up prefill {kind} {dtn} {act} m{m}")
