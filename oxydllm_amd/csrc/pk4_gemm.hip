@@ -25,28 +25,42 @@ namespace oxq {
 
 constexpr int PK4G_STRIPS = 8;  // strips (= waves) of a workgroup
 
-template <typename TT, int MT, int BITS>
+// KS = 1: eight strips a workgroup, a wave takes every block of its strip.  KS = 4 (the form for 65 to a few hundred
+// rows, where workgroups of eight strips are too few to fill the chip): two strips a workgroup, the four waves of
+// a strip take every fourth block; a round brings four blocks of x into LDS, each loaded by the two waves that use
+// it; at the end the waves' partial tiles meet in LDS (where x was) and wave kq of a strip finishes row tile kq,
+// adding the four partials in K order - the epilogue then runs on the accumulator layout as for KS = 1.
+template <typename TT, int MT, int BITS, int KS>
 __global__ __launch_bounds__(512) void pk4_gemm_kernel(const uint16_t *__restrict__ x, const uint32_t *__restrict__ pw,
                                                        const uint16_t *__restrict__ bias, uint16_t *__restrict__ y,
                                                        int M, int K, int N, int NG, int RT, int act) {
     typedef MfmaOps<TT> Ops;
-    constexpr int ROWS = 16 * MT, BB = pk4_block_words(BITS) * 4, XBUF = ROWS * 256;
+    static_assert(KS == 1 || KS == MT, "wave kq of a strip finishes row tile kq");
+    constexpr int SPW = PK4G_STRIPS / KS;  // strips a workgroup
+    constexpr int ROWS = 16 * MT, BB = pk4_block_words(BITS) * 4, XBUF = KS * ROWS * 256;
     constexpr int WL = BITS / 4;          // 1 KB weight loads a step (8-bit: column pairs 0, 1 and 2, 3)
     constexpr int RING = 4 * WL + 1;      // ring loads of a block: younger than the block's loads of x
     constexpr bool BF = TT::DTYPE == BF16Traits::DTYPE;
-    constexpr int XV = ROWS / 32;  // loads of x a wave issues per block: 64 lanes x 16 bytes = 4 rows each
+    constexpr int XV = ROWS / 4 / SPW;  // loads of x a wave issues per round: 64 lanes x 16 bytes = 4 rows each
     extern __shared__ __attribute__((aligned(16))) unsigned char pk4_lds[];
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int ni = lane & 15, kb = lane >> 4;
+    const int ws = wave % SPW, kq = wave / SPW;  // the wave's strip of the workgroup, and its share of K
     int rt, g;
-    pk4g_tile_of((int)blockIdx.x, RT, NG, rt, g);
-    if (g >= NG) return;  // the whole workgroup, before any barrier: the ragged last column of squares
-    const int j = g * PK4G_STRIPS + wave;
-    const bool live = j < (N >> 6);  // wave-uniform: the last group of a layer may have fewer than eight strips
+    if constexpr (KS == 1) {
+        pk4g_tile_of((int)blockIdx.x, RT, NG, rt, g);
+        if (g >= NG) return;  // the whole workgroup, before any barrier: the ragged last column of squares
+    } else {
+        // a row tile's strip groups are neighbours: the eight XCDs share its rows of x, and with NG a multiple of 8
+        // the row tiles of a strip group meet on one XCD, whose L2 then holds the group's weights
+        rt = (int)blockIdx.x / NG, g = (int)blockIdx.x % NG;
+    }
+    const int j = g * SPW + ws;
+    const bool live = j < (N >> 6);  // wave-uniform: the last group of a layer may have fewer strips
     const int m0 = rt * ROWS;
-    const int NB = K >> 7;
+    const int NB = K >> 7, NR = (NB + KS - 1) / KS;  // blocks; rounds of KS blocks
     const int xrows = min(M - m0, ROWS);
 
     const __amdgpu_buffer_rsrc_t rs_none = make_rsrc(pw, 0u);
@@ -55,13 +69,13 @@ __global__ __launch_bounds__(512) void pk4_gemm_kernel(const uint16_t *__restric
     const __amdgpu_buffer_rsrc_t rs_x = make_rsrc(x + (size_t)m0 * K, (uint32_t)xrows * (uint32_t)K * 2u);
     const int voff_w = lane * 16;
     const int voff_z = 1024 * WL * 4 + (ni * 4 + kb) * 4;
-    // x: load q of a wave brings rows 4 (XV wave + q) .. + 3 of the block straight into LDS, lane l the 16 bytes
-    // that belong at position l % 16 of row l / 16 - chunk (l % 16) ^ (row % 16) of the row, the swizzle the
-    // fragment reads undo.  Rows past M lie beyond the descriptor: LDS receives zeros.
+    // x: load q of a wave brings rows 4 (XV ws + q) .. + 3 of the wave's block of the round straight into LDS, lane l
+    // the 16 bytes that belong at position l % 16 of row l / 16 - chunk (l % 16) ^ (row % 16) of the row, the
+    // swizzle the fragment reads undo.  Rows past M lie beyond the descriptor: LDS receives zeros.
     int xo[XV];
 #pragma unroll
     for (int q = 0; q < XV; ++q) {
-        const int r = 4 * (wave * XV + q) + (lane >> 4);
+        const int r = 4 * (ws * XV + q) + (lane >> 4);
         xo[q] = r * K * 2 + (((lane & 15) ^ (r & 15)) << 4);
     }
     int a_rd[4];  // fragment of step st, row tile mt (+ 4096 mt): row ni, chunk 8 (st / 2) + 2 kb + st % 2
@@ -73,11 +87,13 @@ __global__ __launch_bounds__(512) void pk4_gemm_kernel(const uint16_t *__restric
     uint32_t zring;
     // The compiler orders nothing against these loads: the wait for them (the ring loads of a block are
     // younger) is written out in front of the barrier that publishes the block.
-    auto dma_x = [&](int i) {
+    // round r: the wave's block is KS r + kq; its tile of x lies at kq ROWS 256 of the round's buffer
+    auto dma_x = [&](int r) {
+        const int i = KS * r + kq;
         const __amdgpu_buffer_rsrc_t rs = i < NB ? rs_x : rs_none;
 #pragma unroll
         for (int q = 0; q < XV; ++q)
-            pk4g_load_lds16(rs, pk4_lds + (i & 1) * XBUF + (wave * XV + q) * 1024, xo[q], i * 256);
+            pk4g_load_lds16(rs, pk4_lds + (r & 1) * XBUF + kq * (ROWS * 256) + (ws * XV + q) * 1024, xo[q], i * 256);
     };
     auto load_w = [&](int i, int st) {
         const __amdgpu_buffer_rsrc_t rs = i < NB ? rs_w : rs_none;
@@ -98,9 +114,9 @@ __global__ __launch_bounds__(512) void pk4_gemm_kernel(const uint16_t *__restric
 
     dma_x(0);
     __builtin_amdgcn_sched_barrier(0);  // requests keep this order: the wait counts rely on it
-    load_z(0);
+    load_z(kq);
 #pragma unroll
-    for (int st = 0; st < 4; ++st) load_w(0, st);
+    for (int st = 0; st < 4; ++st) load_w(kq, st);
     __builtin_amdgcn_sched_barrier(0);
     float4_t acc[MT][4];
 #pragma unroll
@@ -110,11 +126,12 @@ __global__ __launch_bounds__(512) void pk4_gemm_kernel(const uint16_t *__restric
     pk4g_wait_vmcnt<RING>();
     __syncthreads();
 
-    for (int i = 0; i < NB; ++i) {
-        // the other buffer was last read in the previous block, which every wave has left (the barrier below)
-        dma_x(i + 1);
+    for (int r = 0; r < NR; ++r) {
+        const int i = KS * r + kq;  // past NB (a ragged last round): zeros from both streams
+        // the other buffer was last read in the previous round, which every wave has left (the barrier below)
+        dma_x(r + 1);
         __builtin_amdgcn_sched_barrier(0);
-        const unsigned char *buf = pk4_lds + (i & 1) * XBUF;
+        const unsigned char *buf = pk4_lds + (r & 1) * XBUF + kq * (ROWS * 256);
         uint32_t zv[4], negzb[4], sp[4];
         Pk4gBf16 cb[4];
         zs_words(zring, zv);
@@ -126,7 +143,7 @@ __global__ __launch_bounds__(512) void pk4_gemm_kernel(const uint16_t *__restric
                 Pk4T<TT>::prep(zv[f], negzb[f], sp[f]);
             }
         }
-        load_z(i + 1);
+        load_z(i + KS);
 #pragma unroll
         for (int st = 0; st < 4; ++st) {
             uint32_t wp[WL][4];
@@ -169,14 +186,41 @@ __global__ __launch_bounds__(512) void pk4_gemm_kernel(const uint16_t *__restric
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt) acc[mt][f] = Ops::mfma(a[mt], b, acc[mt][f]);
             }
-            load_w(i + 1, st);  // into the registers this step has just left
+            load_w(i + KS, st);  // into the registers this step has just left
         }
         __builtin_amdgcn_sched_barrier(0);
-        pk4g_wait_vmcnt<RING>();  // this wave's part of the next block is in LDS; its ring loads may still fly
+        pk4g_wait_vmcnt<RING>();  // this wave's part of the next round of x is in LDS; its ring loads may still fly
         __syncthreads();
     }
 
+    // the finished tile rows of this wave: all of them (KS = 1), or row tile kq summed over the strip's waves
+    float4_t fin[KS == 1 ? MT : 1][4];
+    if constexpr (KS == 1) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int f = 0; f < 4; ++f) fin[mt][f] = acc[mt][f];
+    } else {
+        // slot of wave w: [mt][e][lane] x float4 (f = 0..3), 16 KB; the last round's barrier has freed the buffers
+        float4_t *red = (float4_t *)pk4_lds;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                red[((wave * MT + mt) * 4 + e) * 64 + lane] = float4_t{acc[mt][0][e], acc[mt][1][e], acc[mt][2][e], acc[mt][3][e]};
+        __syncthreads();
+#pragma unroll
+        for (int f = 0; f < 4; ++f) fin[0][f] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int k = 0; k < KS; ++k)  // K order: the same sum whatever the timing
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float4_t v = red[(((k * SPW + ws) * MT + kq) * 4 + e) * 64 + lane];
+                fin[0][0][e] += v[0], fin[0][1][e] += v[1], fin[0][2][e] += v[2], fin[0][3][e] += v[3];
+            }
+    }
     if (!live) return;
+    constexpr int FT = KS == 1 ? MT : 1;  // row tiles this wave stores: fin[t] is row tile (KS == 1 ? t : kq)
     if (act) {
         // Fused gate|up layer (pk4_src_col): columns 0..31 of the strip are gate columns 32 j .. 32 j + 31, columns
         // 32..63 the up columns they meet - lane ni < 8 holds four gate columns, lane ni + 8 of the same row of 16
@@ -193,14 +237,14 @@ __global__ __launch_bounds__(512) void pk4_gemm_kernel(const uint16_t *__restric
             bv[2] = TT::to_f32((uint16_t)(bw.y & 0xFFFFu)), bv[3] = TT::to_f32((uint16_t)(bw.y >> 16));
         }
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
+        for (int t = 0; t < FT; ++t)
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                const int row = m0 + 16 * mt + 4 * kb + e;
+                const int row = m0 + 16 * (KS == 1 ? t : kq) + 4 * kb + e;
                 float mine[4], other[4];
 #pragma unroll
                 for (int f = 0; f < 4; ++f) {
-                    mine[f] = TT::to_f32(TT::from_f32(acc[mt][f][e] + bv[f]));
+                    mine[f] = TT::to_f32(TT::from_f32(fin[t][f][e] + bv[f]));
                     other[f] = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, mine[f]), 0x128, 0xF, 0xF, false));
                 }
                 uint32_t o[2];
@@ -221,13 +265,13 @@ __global__ __launch_bounds__(512) void pk4_gemm_kernel(const uint16_t *__restric
         bv[2] = TT::to_f32((uint16_t)(bw.y & 0xFFFFu)), bv[3] = TT::to_f32((uint16_t)(bw.y >> 16));
     }
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
+    for (int t = 0; t < FT; ++t)
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            const int row = m0 + 16 * mt + 4 * kb + e;
+            const int row = m0 + 16 * (KS == 1 ? t : kq) + 4 * kb + e;
             if (row >= M) continue;
-            const uint32_t o0 = TT::from_f32(acc[mt][0][e] + bv[0]), o1 = TT::from_f32(acc[mt][1][e] + bv[1]);
-            const uint32_t o2 = TT::from_f32(acc[mt][2][e] + bv[2]), o3 = TT::from_f32(acc[mt][3][e] + bv[3]);
+            const uint32_t o0 = TT::from_f32(fin[t][0][e] + bv[0]), o1 = TT::from_f32(fin[t][1][e] + bv[1]);
+            const uint32_t o2 = TT::from_f32(fin[t][2][e] + bv[2]), o3 = TT::from_f32(fin[t][3][e] + bv[3]);
             *(uint2 *)(y + (size_t)row * N + 64 * j + 4 * ni) = uint2{o0 | (o1 << 16), o2 | (o3 << 16)};
         }
 }
@@ -393,18 +437,28 @@ __global__ __launch_bounds__(512) void pk4n_gemm_kernel(const uint16_t *__restri
 //   - the split-K tiles cost `split_lo` (below one round) or `split_hi` times w at any M: small workgroups, no
 //     ragged round, but the rate they have at 64 rows.
 // OXQ_PK4_GEMM_ROWS = 64 | 128 takes the choice (tests, sweeps); OXQ_PK4_GEMM_MIN_M = 0 switches the kernels off.
+// a round of the two-strip form (one workgroup a CU) against a full round of 64-row workgroups of eight strips:
+// 19 - 24 us against 65 - 78 at K = 4096 over both widths and types
+constexpr double PK4_MID_ROUND = 0.31;
+
 struct Pk4GemmCost {
     bool pairs64;
     double part64, a64, b64, slope64, full128, part128, split_lo, split_hi;
 };
-static int pk4_gemm_rows(const oxq_ctx *ctx, const Pk4Problem &p) {
+// rows of a workgroup (0: the split-K tiles) and the K split inside it (4: two strips a workgroup)
+struct Pk4GemmForm {
+    int rows, ks;
+};
+static Pk4GemmForm pk4_gemm_form(const oxq_ctx *ctx, const Pk4Problem &p) {
     const int64_t min_m = tune(ctx, OXQ_TUNE_PK4_GEMM_MIN_M, 65);
-    if (min_m <= 0 || (p.w.bits != 4 && p.w.bits != 8) || (p.act && p.w.strip == 16) || p.M < min_m) return 0;
-    if (p.w.bits == 8 && p.w.strip == 16) return 0;  // (16-column strips are a 4-bit layout)
-    const int forced = tune(ctx, OXQ_TUNE_PK4_GEMM_ROWS, 0);
-    if (forced == 64 || forced == 128) return forced;
-    static const Pk4GemmCost WIDE_F16 = {true, 0.88, 1.20, 0.30, 0.97, 1.50, 1.27, 1.70, 1.50};
-    static const Pk4GemmCost WIDE_BF16 = {true, 0.93, 1.29, 0.27, 0.98, 1.44, 1.35, 1.75, 1.53};
+    if (min_m <= 0 || (p.w.bits != 4 && p.w.bits != 8) || (p.act && p.w.strip == 16) || p.M < min_m) return {0, 1};
+    if (p.w.bits == 8 && p.w.strip == 16) return {0, 1};  // (16-column strips are a 4-bit layout)
+    const bool mid_ok = p.w.strip != 16;  // the K split inside a workgroup: 64-column strips only
+    const int forced = tune(ctx, OXQ_TUNE_PK4_GEMM_ROWS, 0), forced_ks = tune(ctx, OXQ_TUNE_PK4_GEMM_KS, 0);
+    if (forced_ks == 4 && mid_ok) return {64, 4};
+    if (forced == 64 || forced == 128) return {forced, 1};
+    static const Pk4GemmCost WIDE_F16 = {true, 0.88, 1.20, 0.30, 0.97, 1.50, 1.27, 1.93, 1.50};
+    static const Pk4GemmCost WIDE_BF16 = {true, 0.93, 1.29, 0.27, 0.98, 1.44, 1.35, 2.00, 1.53};
     static const Pk4GemmCost NARROW_F16 = {false, 0.86, 0, 0, 0, 1.64, 1.30, 1.60, 1.50};
     static const Pk4GemmCost NARROW_BF16 = {false, 0.94, 0, 0, 0, 1.51, 1.35, 1.60, 1.50};
     static const Pk4GemmCost WIDE8_F16 = {false, 0.88, 0, 0, 0, 1.47, 1.27, 1.92, 1.71};  // 8-bit: 137 registers at 64 rows
@@ -423,52 +477,62 @@ static int pk4_gemm_rows(const oxq_ctx *ctx, const Pk4Problem &p) {
     const double c64 = !c.pairs64 || w64 <= 1.0 ? rounds(w64, 1.0, c.part64, 0.75) : w64 <= 2.0 ? c.a64 + c.b64 * w64 : c.slope64 * w64;
     const double c128 = rounds(w128, c.full128, c.part128, 0.7);
     const double c_split = (w64 < 1.0 ? c.split_lo : c.split_hi) * w64;
-    if (c_split <= c64 && c_split <= c128) return 0;
-    return c128 < c64 ? 128 : 64;
+    // two strips a workgroup (128 KB of LDS: one a CU), whole rounds of `PK4_MID_ROUND` each
+    const double w_mid = (double)(ceil_div(p.w.N / 64, (int64_t)2) * ceil_div(p.M, (int64_t)64)) / cus;
+    const double c_mid = mid_ok && forced_ks != 1 ? std::ceil(w_mid) * PK4_MID_ROUND : 1e30;
+    if (c_split <= c64 && c_split <= c128 && c_split <= c_mid) return {0, 1};
+    if (c_mid < c64 && c_mid < c128) return {64, 4};
+    return {c128 < c64 ? 128 : 64, 1};
 }
-bool pk4_gemm_takes(const oxq_ctx *ctx, const Pk4Problem &p) { return pk4_gemm_rows(ctx, p) != 0; }
+bool pk4_gemm_takes(const oxq_ctx *ctx, const Pk4Problem &p) { return pk4_gemm_form(ctx, p).rows != 0; }
 
-template <typename TT, int MT, int LAYOUT>  // LAYOUT: 4 / 8 = bits of a layer in 64-column strips, 16 = 4-bit in 16-column strips
+template <typename TT, int MT, int LAYOUT, int KS>  // LAYOUT: 4 / 8 = bits of a layer in 64-column strips, 16 = 4-bit in 16-column strips
 static int pk4_gemm_go(hipStream_t s, dim3 grid, const Pk4Problem &p, int NG, int RT) {
     static LdsGrant grant;  // one per instantiation
-    const size_t lds = 2 * 16 * MT * 256;
+    const size_t lds = (size_t)2 * KS * 16 * MT * 256;
     if constexpr (LAYOUT == 16) {
         OXQ_HIP_CHECK(grant.ensure((const void *)pk4n_gemm_kernel<TT, MT>, lds));
         hipLaunchKernelGGL((pk4n_gemm_kernel<TT, MT>), grid, dim3(512), lds, s, (const uint16_t *)p.x, p.w.pw, (const uint16_t *)p.bias,
                            (uint16_t *)p.y, (int)p.M, (int)p.w.K, (int)p.w.N, NG, RT);
     } else {
-        OXQ_HIP_CHECK(grant.ensure((const void *)pk4_gemm_kernel<TT, MT, LAYOUT>, lds));
-        hipLaunchKernelGGL((pk4_gemm_kernel<TT, MT, LAYOUT>), grid, dim3(512), lds, s, (const uint16_t *)p.x, p.w.pw, (const uint16_t *)p.bias,
+        OXQ_HIP_CHECK(grant.ensure((const void *)pk4_gemm_kernel<TT, MT, LAYOUT, KS>, lds));
+        hipLaunchKernelGGL((pk4_gemm_kernel<TT, MT, LAYOUT, KS>), grid, dim3(512), lds, s, (const uint16_t *)p.x, p.w.pw, (const uint16_t *)p.bias,
                            (uint16_t *)p.y, (int)p.M, (int)p.w.K, (int)p.w.N, NG, RT, p.act);
     }
     OXQ_HIP_CHECK(hipGetLastError());
     return OXQ_OK;
 }
-template <typename TT, int MT>
+template <typename TT, int MT, int KS>
 static int pk4_gemm_go_layout(hipStream_t s, dim3 grid, const Pk4Problem &p, int NG, int RT) {
-    if (p.w.strip == 16) return pk4_gemm_go<TT, MT, 16>(s, grid, p, NG, RT);
-    return p.w.bits == 8 ? pk4_gemm_go<TT, MT, 8>(s, grid, p, NG, RT) : pk4_gemm_go<TT, MT, 4>(s, grid, p, NG, RT);
+    if constexpr (KS == 1) {
+        if (p.w.strip == 16) return pk4_gemm_go<TT, MT, 16, 1>(s, grid, p, NG, RT);
+    }
+    return p.w.bits == 8 ? pk4_gemm_go<TT, MT, 8, KS>(s, grid, p, NG, RT) : pk4_gemm_go<TT, MT, 4, KS>(s, grid, p, NG, RT);
 }
 
 int launch_pk4_gemm(oxq_ctx *ctx, hipStream_t s, const Pk4Problem &p) {
-    const int rows = pk4_gemm_rows(ctx, p);
-    const int64_t NG = ceil_div(p.w.N / 64, (int64_t)PK4G_STRIPS), RT = ceil_div(p.M, (int64_t)rows);
-    // whole bands of 8 row tiles in squares of 64 workgroups, then the last RT % 8 row tiles x NG groups
-    const int64_t wgs = (RT / 8) * ceil_div(NG, (int64_t)8) * 64 + (RT % 8) * NG;
+    const Pk4GemmForm form = pk4_gemm_form(ctx, p);
+    const int rows = form.rows, spw = PK4G_STRIPS / form.ks;
+    const int64_t NG = ceil_div(p.w.N / 64, (int64_t)spw), RT = ceil_div(p.M, (int64_t)rows);
+    // eight strips a workgroup: whole bands of 8 row tiles in squares of 64 workgroups, then the last RT % 8 row
+    // tiles x NG groups; two strips: row tile by row tile
+    const int64_t wgs = form.ks == 1 ? (RT / 8) * ceil_div(NG, (int64_t)8) * 64 + (RT % 8) * NG : RT * NG;
     if (wgs > 0x7FFFFFFF) return fail(OXQ_ERR_UNSUPPORTED, "repacked matmul: m = %lld exceeds the grid", (long long)p.M);
     dim3 grid((unsigned)wgs);
     char name[64];
-    snprintf(name, sizeof name, "pk%d_gemm_%s_r%dx8%s%s", p.w.bits, p.w.dtype == OXQ_F16 ? "f16" : "bf16", rows, p.w.strip == 16 ? "_n16" : "",
-             p.act == 1 ? "_silu" : p.act == 2 ? "_gelu" : "");
+    snprintf(name, sizeof name, "pk%d_gemm_%s_r%dx%d%s%s%s", p.w.bits, p.w.dtype == OXQ_F16 ? "f16" : "bf16", rows, spw,
+             form.ks > 1 ? "k4" : "", p.w.strip == 16 ? "_n16" : "", p.act == 1 ? "_silu" : p.act == 2 ? "_gelu" : "");
     set_plan(ctx, name, grid, dim3(512), 1, 1, 0);
     if (ctx->plan_only) return OXQ_OK;
     if ((uint64_t)rows * (uint64_t)p.w.K * 2 >= (1ull << 31)) return fail(OXQ_ERR_UNSUPPORTED, "repacked matmul: K too large");
     if (((uintptr_t)p.x | (uintptr_t)p.y) & 15) return fail(OXQ_ERR_UNSUPPORTED, "repacked matmul: x and y must be 16-byte aligned");
     if (p.bias && ((uintptr_t)p.bias & 7)) return fail(OXQ_ERR_UNSUPPORTED, "repacked matmul: bias must be 8-byte aligned");
     const bool f16 = p.w.dtype == OXQ_F16;
+    if (form.ks == 4)
+        return f16 ? pk4_gemm_go_layout<F16Traits, 4, 4>(s, grid, p, (int)NG, (int)RT) : pk4_gemm_go_layout<BF16Traits, 4, 4>(s, grid, p, (int)NG, (int)RT);
     if (rows == 128)
-        return f16 ? pk4_gemm_go_layout<F16Traits, 8>(s, grid, p, (int)NG, (int)RT) : pk4_gemm_go_layout<BF16Traits, 8>(s, grid, p, (int)NG, (int)RT);
-    return f16 ? pk4_gemm_go_layout<F16Traits, 4>(s, grid, p, (int)NG, (int)RT) : pk4_gemm_go_layout<BF16Traits, 4>(s, grid, p, (int)NG, (int)RT);
+        return f16 ? pk4_gemm_go_layout<F16Traits, 8, 1>(s, grid, p, (int)NG, (int)RT) : pk4_gemm_go_layout<BF16Traits, 8, 1>(s, grid, p, (int)NG, (int)RT);
+    return f16 ? pk4_gemm_go_layout<F16Traits, 4, 1>(s, grid, p, (int)NG, (int)RT) : pk4_gemm_go_layout<BF16Traits, 4, 1>(s, grid, p, (int)NG, (int)RT);
 }
 
 }  // namespace oxq

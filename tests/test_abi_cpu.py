@@ -392,9 +392,11 @@ def test_layers_validate_like_reference(lib, ctx):
         out = fake(shape[:-1] + (14336,), BF16)
         assert lib.oxq_packed_quant_linear_forward(h, None, C.byref(x), C.byref(out)) == 0, err(lib)
         assert plan(lib, ctx).kernel.decode().startswith(kern), plan(lib, ctx).kernel
-    # prefill sizes: 28 groups of eight strips x row tiles of 64 or 128; the split-K tiles while those would
-    # leave most of the chip idle, then whichever row count needs the cheaper rounds of 256 workgroups
-    for rows, kern, wgs in [(256, "pk4_mfma_bf16_mt4", None), (384, "pk4_gemm_bf16_r64x8", 6 * 28),
+    # beyond one row tile: 112 pairs of strips x row tiles of 64 with K split inside the workgroup while 28 groups
+    # of eight strips would leave most of the chip idle, then row tiles of 64 or 128 x eight strips, whichever needs
+    # the cheaper rounds of 256 workgroups
+    for rows, kern, wgs in [(64, "pk4_mfma_bf16_mt4", None), (65, "pk4_gemm_bf16_r64x2k4", 2 * 112),
+                            (256, "pk4_gemm_bf16_r64x2k4", 4 * 112), (384, "pk4_gemm_bf16_r64x2k4", 6 * 112), (448, "pk4_gemm_bf16_r64x8", 7 * 28),
                             (512, "pk4_gemm_bf16_r64x8", 4 * 64),
                             (768, "pk4_gemm_bf16_r128x8", 6 * 28), (1000, "pk4_gemm_bf16_r128x8", 4 * 64),
                             (1536, "pk4_gemm_bf16_r64x8", 3 * 4 * 64), (1537, "pk4_gemm_bf16_r64x8", 3 * 4 * 64 + 28),

@@ -199,17 +199,65 @@ def test_prefill_rows_by_eight_strips(kind, dtn, rows, K, N, g, strip16):
     assert_close(out, tile_all[:300] - bias[None, :], f"pk4 prefill {kind} {dtn} no bias")
 
 
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("dtn", ["f16", "bf16"])
+@pytest.mark.parametrize("K,N,g", [(512, 576, 128), (1280, 1088, 128), (256, 64, 128), (4096, 128, 128)])
+def test_prefill_two_strips_with_k_split(kind, dtn, K, N, g):
+    """The form for 65 to a few hundred rows: a workgroup = 64 rows x two strips, the four waves of a strip take every
+    fourth block of K and wave kq finishes row tile kq from the four partial tiles in LDS.  N = 576 and 1088 leave
+    the last workgroup one live strip; K of 2 blocks (half the waves have none), 4 (one round), 10 (a ragged third
+    round) and 32; ragged row tiles.  Against the tile-GEMM oracle, run to run bitwise, rows independent of m."""
+    bits = bits_of_kind(kind)
+    tune("OXQ_PK4_STRIP16", 0)
+    tune("OXQ_PK4_GEMM_KS", 4)
+    dt = DT[dtn]
+    trip, pack_dim = make(kind, K, N, g, seed=K + 7 * N)
+    bias = (np.arange(N, dtype=np.float32) % 13 - 6) * np.float32(0.125)
+    layer = layer_of(trip, pack_dim, dt, bias, bits=bits)
+    w = dense(kind, trip, dt)
+    wt = oracle.round_through(w, dt)
+    rng = np.random.default_rng(K + N)
+    x_all = rng.standard_normal((330, K)).astype(np.float32)
+    xd_all = to_dev(x_all, TORCH_DT[dt])
+    tile_all = oracle.matmul_nt_f32(round_x(x_all, dt), wt, bias)
+    ref_all = oracle.matmul_nt_f32(round_x(x_all, dt), w, bias)
+    first = None
+    for m in (330, 65, 128, 200):
+        say(f"pk{bits} prefill two strips {kind} {dtn} K={K} N={N} m={m}")
+        y = layer.forward(xd_all[:m])
+        plan = ops.default_context().last_plan()
+        assert plan["kernel"] == f"pk{bits}_gemm_{dtn}_r64x2k4" and plan["launches"] == 1, plan
+        assert plan["grid"][0] == -(-m // 64) * -(-(N // 64) // 2) and plan["block"][0] == 512, plan
+        assert_close(y, tile_all[:m], f"pk{bits} two strips {kind} {dtn} m{m}")
+        assert np.abs(as_f32(y) - ref_all[:m]).max() < 0.06 * np.abs(ref_all[:m]).max() + 1e-2
+        np.testing.assert_array_equal(bits_of(layer.forward(xd_all[:m])), bits_of(y))
+        if first is None:
+            first = bits_of(y)
+        else:
+            np.testing.assert_array_equal(bits_of(y), first[:m])
+    if N % 128 == 0 and N >= 128:
+        # the same layer as a fused gate|up projection: the activation epilogue on the summed tile
+        kind_id = ops.ACT_GATED_SILU
+        tdt = TORCH_DT[dt]
+        fused = ops.PackedQuantLinear(bits, pack_dim, to_dev(trip[0]), to_dev(trip[1]), to_dev(trip[2], tdt), to_dev(bias, tdt), tdt,
+                                      gate_up_act=kind_id)
+        y = fused.forward(xd_all[:200])
+        assert ops.default_context().last_plan()["kernel"] == f"pk{bits}_gemm_{dtn}_r64x2k4_silu"
+        np.testing.assert_array_equal(bits_of(y), bits_of(ops.gated_activation(layer.forward(xd_all[:200]), kind_id)))
+
+
 def test_prefill_takes_over_where_it_fills_the_chip():
-    """With the switches at their defaults a 4096 x 14336 layer moves from the split-K tiles to 64-row and
-    then 128-row workgroups as m grows (28 groups of eight strips: 512 rows are 224 workgroups of 64 rows,
-    1000 rows 224 of 128), OXQ_PK4_GEMM_MIN_M = 0 keeps the split-K tiles, and the two agree within the
-    tolerance of one f16 rounding of y."""
+    """With the switches at their defaults a 4096 x 14336 layer moves from the split-K tiles (one row tile) to
+    workgroups of two strips with K split inside (128 rows: 224 of them), then to 64-row and 128-row workgroups of
+    eight strips as m grows (512 rows are 224 workgroups of 64 rows, 1000 rows 224 of 128), OXQ_PK4_GEMM_MIN_M = 0
+    keeps the split-K tiles, and the two agree within the tolerance of one f16 rounding of y."""
     K, N, g = 4096, 14336, 128
     trip, pack_dim = make("awq", K, N, g, seed=11)
     layer = layer_of(trip, pack_dim, oracle.F16, None)
     rng = np.random.default_rng(5)
     xd = to_dev(rng.standard_normal((1000, K)).astype(np.float32), torch.float16)
-    for m, kern in [(64, "pk4_mfma_f16_mt4"), (256, "pk4_mfma_f16_mt4"), (512, "pk4_gemm_f16_r64x8"), (1000, "pk4_gemm_f16_r128x8")]:
+    for m, kern in [(64, "pk4_mfma_f16_mt4"), (128, "pk4_gemm_f16_r64x2k4"), (256, "pk4_gemm_f16_r64x2k4"), (512, "pk4_gemm_f16_r64x8"),
+                    (1000, "pk4_gemm_f16_r128x8")]:
         say(f"pk4 prefill rule m={m}")
         y = layer.forward(xd[:m])
         plan = ops.default_context().last_plan()
