@@ -472,12 +472,12 @@ int oxq_qlinear_new(oxq_ctx *ctx, int quant, const oxq_tensor *weight_bytes, int
  * matmul's epilogue: out_features = 2I, forward writes [.., I] = act(gate(x)) * up(x), bit for bit what
  * oxq_gated_activation gives on the plain layer's output.  Needs a BF16 layer that takes the matrix-core copy (see
  * oxq_qlinear_is_resident below), else OXQ_ERR_UNSUPPORTED.  Every row count runs in one launch: up to 32 rows
- * the integer kernel of the copy; prefill sizes, where enough workgroups of 64 rows x 512 columns fill the chip,
- * the copy's prefill kernel (the plain layer takes the same kernel at the same sizes: the same bits); in between, row
- * tiles of 32 that each read the weights again (with the unrounded weights that the plain layer's tile matmul
- * rounds to bf16) - oxq_mlp_forward sends those row counts (more than OXQ_GGUF_FUSED_ACT_ROWS, fewer than the
- * prefill kernel takes) through the plain layer's path and the activation by itself, so that a FeedForward over
- * this layer gives the plain layers' bits at every row count. */
+ * the integer kernel of the copy; above that, where enough workgroups of 64 rows fill the chip, the copy's prefill
+ * kernel (the plain layer takes the same kernel at the same sizes: the same bits); otherwise row tiles of 32 that
+ * each read the weights again (with the unrounded weights that the plain layer's tile matmul rounds to bf16) -
+ * oxq_mlp_forward sends those row counts (more than OXQ_GGUF_FUSED_ACT_ROWS where the prefill kernel does not take
+ * the call) through the plain layer's path and the activation by itself, so that a FeedForward over this layer
+ * gives the plain layers' bits at every row count. */
 #define OXQ_GGUF_FUSED_ACT_ROWS 32
 int oxq_qlinear_new_gate_up(oxq_ctx *ctx, int quant, const oxq_tensor *weight_bytes, int64_t in_features,
                             int64_t out_features, const oxq_tensor *bias_or_null, int act, int out_dtype,

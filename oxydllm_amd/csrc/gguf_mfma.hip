@@ -645,7 +645,9 @@ __global__ __launch_bounds__(NW * 64) void ggm_kernel(const uint16_t *__restrict
 // chunk); a wave rings its four strips' chunks in two halves, turns a step's integers into the weight with one
 // fma each (two where a five-bit format has a minimum) from the integer kernel's own factors, and keeps the whole
 // K in its accumulators: one launch, no partial tiles.
-template <int FMT, int MT>
+// KS = 4: two waves of 64 columns a workgroup and the four waves of a column group take every fourth chunk, as in
+// pk4_gemm_kernel - the form for 33 to a few hundred rows of a wide layer.
+template <int FMT, int MT, int KS>
 __global__ __launch_bounds__(512) void ggm_gemm_kernel(const uint16_t *__restrict__ x, const uint8_t *__restrict__ pw,
                                                        const uint16_t *__restrict__ bias, uint16_t *__restrict__ y,
                                                        int M, int K, int N, int NG, int RT, int act) {
@@ -654,7 +656,9 @@ __global__ __launch_bounds__(512) void ggm_gemm_kernel(const uint16_t *__restric
     typedef GgmFmt<FMT> F;
     typedef GgmLayout<FMT> L;
     typedef GgmChunk<FMT> C;
-    constexpr int ROWS = 16 * MT, XBUF = ROWS * 256, XV = ROWS / 32, NSTEP = C::NSTEP;
+    static_assert(KS == 1 || KS == MT, "wave kq of a column group finishes row tile kq");
+    constexpr int SPW = 8 / KS;  // waves of 64 columns a workgroup
+    constexpr int ROWS = 16 * MT, XBUF = KS * ROWS * 256, XV = ROWS / 4 / SPW, NSTEP = C::NSTEP;
     constexpr bool K16 = NSTEP == 8;
     constexpr int RING = 4 * C::LOADS;  // vector loads of a chunk's weights: younger than the chunk's loads of x
     extern __shared__ __attribute__((aligned(16))) unsigned char pk4_lds[];
@@ -662,13 +666,18 @@ __global__ __launch_bounds__(512) void ggm_gemm_kernel(const uint16_t *__restric
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int ni = lane & 15, kb = lane >> 4;
+    const int ws = wave % SPW, kq = wave / SPW;  // the wave's column group of the workgroup, and its share of K
     int rt, g;
-    pk4g_tile_of((int)blockIdx.x, RT, NG, rt, g);
-    if (g >= NG) return;  // the whole workgroup, before any barrier
-    const int j = g * 8 + wave;  // the wave's 64 columns: strips 4 j .. 4 j + 3
+    if constexpr (KS == 1) {
+        pk4g_tile_of((int)blockIdx.x, RT, NG, rt, g);
+        if (g >= NG) return;  // the whole workgroup, before any barrier
+    } else {
+        rt = (int)blockIdx.x / NG, g = (int)blockIdx.x % NG;
+    }
+    const int j = g * SPW + ws;  // the wave's 64 columns: strips 4 j .. 4 j + 3
     const bool live = j < (N >> 6);
     const int m0 = rt * ROWS;
-    const int NC = K >> 7;
+    const int NC = K >> 7, NR = (NC + KS - 1) / KS;  // chunks; rounds of KS chunks
     const int xrows = min(M - m0, ROWS);
 
     const uint32_t strip_bytes = (uint32_t)(NC / F::CH) * (uint32_t)L::BLKB;
@@ -682,7 +691,7 @@ __global__ __launch_bounds__(512) void ggm_gemm_kernel(const uint16_t *__restric
     int xo[XV];
 #pragma unroll
     for (int q = 0; q < XV; ++q) {
-        const int r = 4 * (wave * XV + q) + (lane >> 4);
+        const int r = 4 * (ws * XV + q) + (lane >> 4);
         xo[q] = r * K * 2 + (((lane & 15) ^ (r & 15)) << 4);
     }
     int a_rd[NSTEP];
@@ -695,11 +704,12 @@ __global__ __launch_bounds__(512) void ggm_gemm_kernel(const uint16_t *__restric
     constexpr bool NIB = FMT == OXQ_GGUF_Q4_0 || FMT == OXQ_GGUF_Q4_1 || FMT == OXQ_GGUF_Q4_K;
 
     C wr[2][4];
-    auto dma_x = [&](int i) {
+    auto dma_x = [&](int r) {  // round r: the wave's chunk is KS r + kq, its tile of x at kq ROWS 256 of the round's buffer
+        const int i = KS * r + kq;
         const __amdgpu_buffer_rsrc_t rs = i < NC ? rs_x : rs_none;
 #pragma unroll
         for (int q = 0; q < XV; ++q)
-            pk4g_load_lds16(rs, pk4_lds + (i & 1) * XBUF + (wave * XV + q) * 1024, xo[q], i * 256);
+            pk4g_load_lds16(rs, pk4_lds + (r & 1) * XBUF + kq * (ROWS * 256) + (ws * XV + q) * 1024, xo[q], i * 256);
     };
     auto request = [&](int i, C (&w)[4]) {
         const __amdgpu_buffer_rsrc_t rs = i < NC ? rs_w : rs_none;
@@ -709,7 +719,7 @@ __global__ __launch_bounds__(512) void ggm_gemm_kernel(const uint16_t *__restric
 
     dma_x(0);
     __builtin_amdgcn_sched_barrier(0);  // requests keep this order: the wait counts rely on it
-    request(0, wr[0]);
+    request(kq, wr[0]);
     __builtin_amdgcn_sched_barrier(0);
     float4_t acc[MT][4];
 #pragma unroll
@@ -719,13 +729,14 @@ __global__ __launch_bounds__(512) void ggm_gemm_kernel(const uint16_t *__restric
     pk4g_wait_vmcnt<RING>();
     __syncthreads();
 
-    auto chunk = [&](int i, auto cur_c) {
+    auto chunk = [&](int r, auto cur_c) {
         constexpr int CUR = decltype(cur_c)::value;
-        dma_x(i + 1);
+        const int i = KS * r + kq;  // past NC (a ragged last round): zeros from both streams
+        dma_x(r + 1);
         __builtin_amdgcn_sched_barrier(0);
-        request(i + 1, wr[CUR ^ 1]);
+        request(i + KS, wr[CUR ^ 1]);
         __builtin_amdgcn_sched_barrier(0);  // not sunk to the chunk's end, where the next chunk would wait for them
-        const unsigned char *buf = pk4_lds + (i & 1) * XBUF;
+        const unsigned char *buf = pk4_lds + (r & 1) * XBUF + kq * (ROWS * 256);
         // w = f0 q' + c2 with q' = q minus the format's offset and c2 = -(minimum): exact products, one rounding -
         // the bits of the dense dequant (ggm_dequant_kernel), so the tile the matrix cores see is the reference's
         float f0[4][NSTEP], c2[4][C::HAS_MIN ? NSTEP : 1];
@@ -795,14 +806,41 @@ __global__ __launch_bounds__(512) void ggm_gemm_kernel(const uint16_t *__restric
         __syncthreads();
     };
     {
-        int i = 0;
-        for (; i + 1 < NC; i += 2) {
-            chunk(i, std::integral_constant<int, 0>{});
-            chunk(i + 1, std::integral_constant<int, 1>{});
+        int r = 0;
+        for (; r + 1 < NR; r += 2) {
+            chunk(r, std::integral_constant<int, 0>{});
+            chunk(r + 1, std::integral_constant<int, 1>{});
         }
-        if (i < NC) chunk(i, std::integral_constant<int, 0>{});
+        if (r < NR) chunk(r, std::integral_constant<int, 0>{});
     }
 
+    // the finished tile rows of this wave: all of them (KS = 1), or row tile kq summed over the column group's waves
+    constexpr int FT = KS == 1 ? MT : 1;
+    float4_t fin[FT][4];
+    if constexpr (KS == 1) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int f = 0; f < 4; ++f) fin[mt][f] = acc[mt][f];
+    } else {
+        // slot of wave w: [mt][e][lane] x float4 (f = 0..3), 16 KB; the last round's barrier has freed the buffers
+        float4_t *red = (float4_t *)pk4_lds;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                red[((wave * MT + mt) * 4 + e) * 64 + lane] = float4_t{acc[mt][0][e], acc[mt][1][e], acc[mt][2][e], acc[mt][3][e]};
+        __syncthreads();
+#pragma unroll
+        for (int f = 0; f < 4; ++f) fin[0][f] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int k = 0; k < KS; ++k)  // K order: the same sum whatever the timing
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float4_t v = red[(((k * SPW + ws) * MT + kq) * 4 + e) * 64 + lane];
+                fin[0][0][e] += v[0], fin[0][1][e] += v[1], fin[0][2][e] += v[2], fin[0][3][e] += v[3];
+            }
+    }
     if (!live) return;
     if (act) {
         // Fused gate|up layer (ggm_src_row): strip 4 j + f holds gate columns 8 (4 j + f) .. + 7 in lanes ni < 8 and
@@ -816,14 +854,14 @@ __global__ __launch_bounds__(512) void ggm_gemm_kernel(const uint16_t *__restric
             for (int f = 0; f < 4; ++f) bv[f] = TT::to_f32(bias[(low ? 0 : half) + 8 * (4 * j + f) + p]);
         }
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
+        for (int t = 0; t < FT; ++t)
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                const int row = m0 + 16 * mt + 4 * kb + e;
+                const int row = m0 + 16 * (KS == 1 ? t : kq) + 4 * kb + e;
                 float mine[4], other[4];
 #pragma unroll
                 for (int f = 0; f < 4; ++f) {
-                    mine[f] = TT::to_f32(TT::from_f32(acc[mt][f][e] + bv[f]));
+                    mine[f] = TT::to_f32(TT::from_f32(fin[t][f][e] + bv[f]));
                     other[f] = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, mine[f]), 0x128, 0xF, 0xF, false));
                 }
 #pragma unroll
@@ -843,13 +881,13 @@ __global__ __launch_bounds__(512) void ggm_gemm_kernel(const uint16_t *__restric
         for (int f = 0; f < 4; ++f) bv[f] = TT::to_f32(bias[64 * j + 16 * f + ni]);
     }
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
+    for (int t = 0; t < FT; ++t)
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            const int row = m0 + 16 * mt + 4 * kb + e;
+            const int row = m0 + 16 * (KS == 1 ? t : kq) + 4 * kb + e;
             if (row >= M) continue;
 #pragma unroll
-            for (int f = 0; f < 4; ++f) y[(size_t)row * N + 64 * j + 16 * f + ni] = TT::from_f32(acc[mt][f][e] + bv[f]);
+            for (int f = 0; f < 4; ++f) y[(size_t)row * N + 64 * j + 16 * f + ni] = TT::from_f32(fin[t][f][e] + bv[f]);
         }
 }
 
@@ -1006,62 +1044,81 @@ int launch_gguf_mfma(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p) {
 }
 
 // Rows from which a bf16 layer's matrix-core copy runs the prefill kernel instead of the tile matmul on the file
-// layout (gguf_mm: a workgroup of 64 rows x 64 columns with K slices).  Costs in rounds of 256 workgroups of 64
-// rows x 512 columns (one a CU), as for the packed layers (pk4_gemm_rows).
-bool gguf_gemm_takes(const oxq_ctx *ctx, int quant, int64_t M, int64_t K, int64_t N, int act_dtype) {
-    (void)K;
-    // OXQ_GGUF_GEMM_MIN_M: unset = by cost, 0 = never, n = from n rows on whatever the cost
+// layout (gguf_mm: a workgroup of 64 rows x 64 columns with K slices), and in which form: 1 = eight waves of 64
+// columns a workgroup, 4 = two, with K split across the waves inside (0: the file layout).  Costs in rounds of 256
+// workgroups of 64 rows x 512 columns (one a CU: 154 - 210 registers), as for the packed layers (pk4_gemm_form): a
+// last round that fills at most three quarters of the CUs costs 0.95; a round of the two-wave form GGM_MID_ROUND
+// (25 - 35 us against 82 - 120 at K = 4096); the file-layout tile matmul 0.17 + 1.45 w (1.3 w for the five- and
+// six-bit formats, whose conversion weighs on the prefill kernel too): two launches or a latency floor, then about
+// two thirds of a full round's rate.  Fitted to 4096 x 4096, 4096 x 14336 and 14336 x 4096 at
+// 64 - 4096 rows.  OXQ_GGUF_GEMM_MIN_M: unset = by cost, 0 = never, n = the eight-wave form from n rows on whatever
+// the cost; OXQ_GGUF_GEMM_KS = 4 | 1: always | never the two-wave form.
+constexpr double GGM_MID_ROUND = 0.31;
+static int gguf_gemm_form(const oxq_ctx *ctx, int quant, int64_t M, int64_t N, int act_dtype) {
     const int64_t v = tune(ctx, OXQ_TUNE_GGUF_GEMM_MIN_M, -1);
-    if (v == 0 || act_dtype != OXQ_BF16 || !ggm_format(quant) || M <= 32 || N % 64 != 0) return false;
-    if (v > 0) return M >= v;
-    // Costs in rounds of one 64-row workgroup a CU (154 - 210 registers: no second one fits).  A last round that
-    // fills at most three quarters of the CUs costs 0.95; the file-layout tile matmul 1.55 w (1.75 w below one
-    // round) for the formats whose conversion is one fma a weight, 1.3 w (1.45 w) for the five- and six-bit ones.
-    // Fitted to 4096 x 4096, 4096 x 14336 and 14336 x 4096 at 64 - 4096 rows.
+    if (v == 0 || act_dtype != OXQ_BF16 || !ggm_format(quant) || M <= 32 || N % 64 != 0) return 0;
+    const int ks = tune(ctx, OXQ_TUNE_GGUF_GEMM_KS, 0);
+    if (ks == 4) return 4;
+    if (v > 0) return M >= v ? 1 : 0;
     const bool light = quant == OXQ_GGUF_Q4_0 || quant == OXQ_GGUF_Q4_1 || quant == OXQ_GGUF_Q4_K || quant == OXQ_GGUF_Q8_0;
     const double cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
-    const double w64 = (double)(ceil_div(N / 64, (int64_t)8) * ceil_div(M, (int64_t)64)) / cus;
+    const int64_t row_tiles = ceil_div(M, (int64_t)64);
+    const double w64 = (double)(ceil_div(N / 64, (int64_t)8) * row_tiles) / cus;
     const double whole = std::floor(w64), rest = w64 - whole;
     const double c64 = whole + (rest <= 0.0 ? 0.0 : rest <= 0.75 ? 0.95 : 1.0);
-    const double split = w64 < 1.0 ? (light ? 1.75 : 1.45) : (light ? 1.55 : 1.3);
-    return split * w64 > c64;
+    const double c_mid = ks == 1 ? 1e30 : std::ceil((double)(ceil_div(N / 64, (int64_t)2) * row_tiles) / cus) * GGM_MID_ROUND;
+    const double c_file = 0.17 + (light ? 1.45 : 1.3) * w64;
+    if (c_file <= c64 && c_file <= c_mid) return 0;
+    return c_mid < c64 ? 4 : 1;
+}
+bool gguf_gemm_takes(const oxq_ctx *ctx, int quant, int64_t M, int64_t K, int64_t N, int act_dtype) {
+    (void)K;
+    return gguf_gemm_form(ctx, quant, M, N, act_dtype) != 0;
 }
 
-template <int FMT>
+template <int FMT, int KS>
 static int ggm_gemm_go(hipStream_t s, dim3 grid, const GgufProblem &p, int NG, int RT) {
     static LdsGrant grant;  // one per instantiation
     constexpr int MT = 4;
-    const size_t lds = 2 * 16 * MT * 256;
-    OXQ_HIP_CHECK(grant.ensure((const void *)ggm_gemm_kernel<FMT, MT>, lds));
-    hipLaunchKernelGGL((ggm_gemm_kernel<FMT, MT>), grid, dim3(512), lds, s, (const uint16_t *)p.x, p.w, (const uint16_t *)p.bias,
+    const size_t lds = (size_t)2 * KS * 16 * MT * 256;
+    OXQ_HIP_CHECK(grant.ensure((const void *)ggm_gemm_kernel<FMT, MT, KS>, lds));
+    hipLaunchKernelGGL((ggm_gemm_kernel<FMT, MT, KS>), grid, dim3(512), lds, s, (const uint16_t *)p.x, p.w, (const uint16_t *)p.bias,
                        (uint16_t *)p.y, (int)p.M, (int)p.K, (int)p.N, NG, RT, p.act);
     OXQ_HIP_CHECK(hipGetLastError());
     return OXQ_OK;
+}
+template <int FMT>
+static int ggm_gemm_go_form(hipStream_t s, dim3 grid, const GgufProblem &p, int NG, int RT, int ks) {
+    return ks == 4 ? ggm_gemm_go<FMT, 4>(s, grid, p, NG, RT) : ggm_gemm_go<FMT, 1>(s, grid, p, NG, RT);
 }
 
 // p.w is the matrix-core copy; p.act as for launch_gguf_mfma
 int launch_gguf_gemm(oxq_ctx *ctx, hipStream_t s, const GgufProblem &p) {
     const int rows = 64;
-    const int64_t NG = ceil_div(p.N / 64, (int64_t)8), RT = ceil_div(p.M, (int64_t)rows);
-    const int64_t wgs = (RT / 8) * ceil_div(NG, (int64_t)8) * 64 + (RT % 8) * NG;
+    int ks = gguf_gemm_form(ctx, p.quant, p.M, p.N, p.act_dtype);
+    if (ks == 0) ks = 1;  // a caller that asks for this kernel gets it
+    const int spw = 8 / ks;
+    const int64_t NG = ceil_div(p.N / 64, (int64_t)spw), RT = ceil_div(p.M, (int64_t)rows);
+    const int64_t wgs = ks == 1 ? (RT / 8) * ceil_div(NG, (int64_t)8) * 64 + (RT % 8) * NG : RT * NG;
     if (wgs > 0x7FFFFFFF) return fail(OXQ_ERR_UNSUPPORTED, "gguf prefill matmul: m = %lld exceeds the grid", (long long)p.M);
     dim3 grid((unsigned)wgs);
     char name[64];
-    snprintf(name, sizeof name, "gguf_%s_gemm_bf16_r%dx8%s", ggm_name(p.quant), rows, p.act == 1 ? "_silu" : p.act == 2 ? "_gelu" : "");
+    snprintf(name, sizeof name, "gguf_%s_gemm_bf16_r%dx%d%s%s", ggm_name(p.quant), rows, spw, ks > 1 ? "k4" : "",
+             p.act == 1 ? "_silu" : p.act == 2 ? "_gelu" : "");
     set_plan(ctx, name, grid, dim3(512), 1, 1, 0);
     if (ctx->plan_only) return OXQ_OK;
     if (p.act_dtype != OXQ_BF16) return fail(OXQ_ERR_UNSUPPORTED, "gguf prefill matmul: activations must be BF16");
     if ((uint64_t)rows * (uint64_t)p.K * 2 >= (1ull << 31)) return fail(OXQ_ERR_UNSUPPORTED, "gguf prefill matmul: K too large");
     if (((uintptr_t)p.x & 15) || ((uintptr_t)p.y & 1)) return fail(OXQ_ERR_UNSUPPORTED, "gguf prefill matmul: x must be 16-byte aligned");
     switch (p.quant) {
-    case OXQ_GGUF_Q4_0: return ggm_gemm_go<OXQ_GGUF_Q4_0>(s, grid, p, (int)NG, (int)RT);
-    case OXQ_GGUF_Q8_0: return ggm_gemm_go<OXQ_GGUF_Q8_0>(s, grid, p, (int)NG, (int)RT);
-    case OXQ_GGUF_Q4_K: return ggm_gemm_go<OXQ_GGUF_Q4_K>(s, grid, p, (int)NG, (int)RT);
-    case OXQ_GGUF_Q6_K: return ggm_gemm_go<OXQ_GGUF_Q6_K>(s, grid, p, (int)NG, (int)RT);
-    case OXQ_GGUF_Q4_1: return ggm_gemm_go<OXQ_GGUF_Q4_1>(s, grid, p, (int)NG, (int)RT);
-    case OXQ_GGUF_Q5_0: return ggm_gemm_go<OXQ_GGUF_Q5_0>(s, grid, p, (int)NG, (int)RT);
-    case OXQ_GGUF_Q5_1: return ggm_gemm_go<OXQ_GGUF_Q5_1>(s, grid, p, (int)NG, (int)RT);
-    case OXQ_GGUF_Q5_K: return ggm_gemm_go<OXQ_GGUF_Q5_K>(s, grid, p, (int)NG, (int)RT);
+    case OXQ_GGUF_Q4_0: return ggm_gemm_go_form<OXQ_GGUF_Q4_0>(s, grid, p, (int)NG, (int)RT, ks);
+    case OXQ_GGUF_Q8_0: return ggm_gemm_go_form<OXQ_GGUF_Q8_0>(s, grid, p, (int)NG, (int)RT, ks);
+    case OXQ_GGUF_Q4_K: return ggm_gemm_go_form<OXQ_GGUF_Q4_K>(s, grid, p, (int)NG, (int)RT, ks);
+    case OXQ_GGUF_Q6_K: return ggm_gemm_go_form<OXQ_GGUF_Q6_K>(s, grid, p, (int)NG, (int)RT, ks);
+    case OXQ_GGUF_Q4_1: return ggm_gemm_go_form<OXQ_GGUF_Q4_1>(s, grid, p, (int)NG, (int)RT, ks);
+    case OXQ_GGUF_Q5_0: return ggm_gemm_go_form<OXQ_GGUF_Q5_0>(s, grid, p, (int)NG, (int)RT, ks);
+    case OXQ_GGUF_Q5_1: return ggm_gemm_go_form<OXQ_GGUF_Q5_1>(s, grid, p, (int)NG, (int)RT, ks);
+    case OXQ_GGUF_Q5_K: return ggm_gemm_go_form<OXQ_GGUF_Q5_K>(s, grid, p, (int)NG, (int)RT, ks);
     default: return fail(OXQ_ERR_UNSUPPORTED, "gguf prefill matmul: format %d has no matrix-core layout", p.quant);
     }
 }

@@ -18,12 +18,12 @@
 // call costs no getenv and two engine threads cannot race on the process environment.
 #define OXQ_TUNE_LIST(X)                                                                                      \
     X(ACT_VEC) X(F8_MM_KS) X(F8_MM_MIN_M) X(F8_MM_MT) X(FORCE_GENERIC) X(GEMV_CFG) X(GEMV_GPW) X(GEMV_TILE)   \
-    X(GGR_GRID) X(GGR_WAVES) X(GGUF_BIG_LDS) X(GGUF_GEMM_MIN_M) X(GGUF_MFMA) X(GGUF_MFMA_MAX_M)               \
-    X(GGUF_MFMA_NS) X(GGUF_MM_KS) X(GGUF_MM_MIN_M) X(GGUF_MM_MT) X(GGUF_PW) X(GGUF_RPWG) X(GPTQ_TILE)         \
-    X(GPTQ_TILE_KS) X(MFMA_MT) X(MFMA_SPLITK) X(MFMA_VARIANT) X(MXFP4_FR) X(MXFP4_MM) X(MXFP4_MM_KS)          \
-    X(MXFP4_MM_MT) X(MXFP4_VARIANT) X(PK4N_NS1_ROWS) X(PK4N_W16) X(PK4_CONTIGUOUS) X(PK4_FOLD) X(PK4_FRONT)   \
-    X(PK4_GEMM_KS) X(PK4_GEMM_MIN_M) X(PK4_GEMM_ROWS) X(PK4_KS) X(PK4_PLACE64) X(PK4_STRIP16) X(PK4_T64)      \
-    X(PK4_XQ) X(PREPACK) X(SPLITK_MODE) X(TRANSIENT_REPACK)
+    X(GGR_GRID) X(GGR_WAVES) X(GGUF_BIG_LDS) X(GGUF_GEMM_KS) X(GGUF_GEMM_MIN_M) X(GGUF_MFMA)                  \
+    X(GGUF_MFMA_MAX_M) X(GGUF_MFMA_NS) X(GGUF_MM_KS) X(GGUF_MM_MIN_M) X(GGUF_MM_MT) X(GGUF_PW) X(GGUF_RPWG)   \
+    X(GPTQ_TILE) X(GPTQ_TILE_KS) X(MFMA_MT) X(MFMA_SPLITK) X(MFMA_VARIANT) X(MXFP4_FR) X(MXFP4_MM)            \
+    X(MXFP4_MM_KS) X(MXFP4_MM_MT) X(MXFP4_VARIANT) X(PK4N_NS1_ROWS) X(PK4N_W16) X(PK4_CONTIGUOUS)             \
+    X(PK4_FOLD) X(PK4_FRONT) X(PK4_GEMM_KS) X(PK4_GEMM_MIN_M) X(PK4_GEMM_ROWS) X(PK4_KS) X(PK4_PLACE64)       \
+    X(PK4_STRIP16) X(PK4_T64) X(PK4_XQ) X(PREPACK) X(SPLITK_MODE) X(TRANSIENT_REPACK)
 enum oxq_tune_key {
 #define OXQ_TUNE_ENUM(n) OXQ_TUNE_##n,
     OXQ_TUNE_LIST(OXQ_TUNE_ENUM)

@@ -450,9 +450,11 @@ def test_layers_validate_like_reference(lib, ctx):
     for m_rows, kern in [(1, "gguf_q4k_mfma_bf16_mt1"), (2, "gguf_q4k_mfma_bf16_mt1"),
                          (4, "gguf_q4k_mfma_bf16_mt1"), (8, "gguf_q4k_mfma_bf16_mt1"),
                          (16, "gguf_q4k_mfma_bf16_mt1"), (32, "gguf_q4k_mfma_bf16_mt2"), (33, "gguf_q4k_mul_mm_bf16_mt4"),
-                         # prefill: the tile matmul on the file layout until eight groups of 512 columns x row tiles
-                         # of 64 fill the chip, then the kernel on the layer's copy
-                         (1024, "gguf_q4k_mul_mm_bf16_mt4"), (1536, "gguf_q4k_gemm_bf16_r64x8"),
+                         # more rows: the tile matmul on the file layout, then the kernels on the layer's copy - 32
+                         # pairs of column groups x row tiles of 64 with K split inside the workgroup, and eight groups
+                         # of 512 columns x row tiles once those fill the chip
+                         (128, "gguf_q4k_mul_mm_bf16_mt4"), (256, "gguf_q4k_gemm_bf16_r64x2k4"),
+                         (1024, "gguf_q4k_gemm_bf16_r64x2k4"), (2048, "gguf_q4k_gemm_bf16_r64x8"),
                          (4096, "gguf_q4k_gemm_bf16_r64x8")]:
         assert lib.oxq_qlinear_forward(q, None, C.byref(fake((m_rows, 4096), BF16)),
                                        C.byref(fake((m_rows, 4096), BF16))) == 0, err(lib)

@@ -248,17 +248,22 @@ def test_fused_gate_up_rows_beyond_a_tile_and_refusals(fmt):
 
 
 @pytest.mark.parametrize("fmt", FMTS)
+@pytest.mark.parametrize("ks", [1, 4])
 @pytest.mark.parametrize("N,K", [(576, 512), (1088, 1280), (64, 256)])
-def test_prefill_kernel_on_the_matrix_core_copy(fmt, N, K):
+def test_prefill_kernel_on_the_matrix_core_copy(fmt, N, K, ks):
     """linear.rs:270-284 forward_prefill: more rows than the integer kernel takes run the tile arithmetic (the
     dequantized weight rounded to bf16, f32 accumulation) from the same copy - a workgroup of 64 rows x eight waves
     of 64 columns, x shared in LDS.  N = 576 and 1088 leave the last group one live wave of eight, N = 64 is one
     wave; m covers a ragged row tile, a whole band of eight row tiles with a remainder (581 rows) and two bands;
     K of 2, 4 and 10 chunks (both ring halves, an odd count, both halves of a K-quant block).  The weights the
     matrix cores see are bit for bit the dense dequant's, so the tile oracle holds at the GEMV tolerance; run to run
-    bitwise; a row's bits do not depend on m."""
+    bitwise; a row's bits do not depend on m.  ks = 4: the form for fewer rows - two waves of 64 columns a workgroup,
+    the four waves of a column group take every fourth chunk (K of 2 chunks: half of them have none; 10: a ragged
+    third round) and meet in LDS."""
     name = synth.GGUF_NAMES[fmt]
     tune("OXQ_GGUF_GEMM_MIN_M", 33)
+    tune("OXQ_GGUF_GEMM_KS", ks)
+    kname = f"gguf_{TAG[fmt]}_gemm_bf16_r64x" + ("8" if ks == 1 else "2k4")
     bias = ((np.arange(N, dtype=np.float32) % 13) - 6) * np.float32(0.25)
     data, layer = _layer(fmt, N, K, seed=N + K + fmt, bias=bias)
     w = oracle.round_through(oracle.dequantize_gguf(fmt, data, N, K), oracle.BF16)
@@ -270,9 +275,9 @@ def test_prefill_kernel_on_the_matrix_core_copy(fmt, N, K):
         say(f"gguf prefill {name} N={N} K={K} m={m}")
         y = layer.forward(xd[:m])
         plan = ops.default_context().last_plan()
-        rt, ng = -(-m // 64), -(-(N // 64) // 8)
-        assert plan["kernel"] == f"gguf_{TAG[fmt]}_gemm_bf16_r64x8" and plan["launches"] == 1, plan
-        assert plan["grid"][0] == (rt // 8) * (-(-ng // 8)) * 64 + (rt % 8) * ng and plan["block"][0] == 512, plan
+        rt, ng = -(-m // 64), -(-(N // 64) // (8 // ks))
+        assert plan["kernel"] == kname and plan["launches"] == 1, plan
+        assert plan["grid"][0] == ((rt // 8) * (-(-ng // 8)) * 64 + (rt % 8) * ng if ks == 1 else rt * ng) and plan["block"][0] == 512, plan
         assert tuple(y.shape) == (m, N)
         assert_close(y, tile_all[:m], f"gguf prefill {name} N={N} K={K} m={m}", bf16_out=True)
         assert np.array_equal(bits_of(layer.forward(xd[:m])), bits_of(y)), "run to run"
@@ -288,14 +293,17 @@ def test_prefill_kernel_on_the_matrix_core_copy(fmt, N, K):
 
 
 @pytest.mark.parametrize("fmt", FMTS)
+@pytest.mark.parametrize("ks", [1, 4])
 @pytest.mark.parametrize("act", ["silu", "gelu_tanh"])
-def test_fused_gate_up_activation_at_prefill(fmt, act):
+def test_fused_gate_up_activation_at_prefill(fmt, act, ks):
     """The prefill kernel's own activation epilogue (gate and up columns of an output sit in lanes 8 apart of the
     accumulator layout) against the plain layer through the same kernel followed by oxq_gated_activation: the same
     bits, with and without bias; I = 288 leaves the last group one live wave."""
     kind = ops.ACT_GATED_SILU if act == "silu" else ops.ACT_GATED_GELU_TANH
     name = synth.GGUF_NAMES[fmt]
     tune("OXQ_GGUF_GEMM_MIN_M", 33)
+    tune("OXQ_GGUF_GEMM_KS", ks)
+    kname = f"gguf_{TAG[fmt]}_gemm_bf16_r64x" + ("8" if ks == 1 else "2k4")
     K, I = 512, 288
     N = 2 * I
     data = synth.gguf_weight(fmt, N, K, seed=K + I + fmt)
@@ -310,10 +318,10 @@ def test_fused_gate_up_activation_at_prefill(fmt, act):
             say(f"gguf fused gate|up prefill {name} {act} bias={with_bias} m={m}")
             y = fused.forward(xd[:m])
             plan = ops.default_context().last_plan()
-            assert plan["kernel"] == f"gguf_{TAG[fmt]}_gemm_bf16_r64x8_" + ("silu" if act == "silu" else "gelu"), plan
+            assert plan["kernel"] == kname + ("_silu" if act == "silu" else "_gelu"), plan
             assert tuple(y.shape) == (m, I) and plan["launches"] == 1
             gu = plain.forward(xd[:m])
-            assert ops.default_context().last_plan()["kernel"] == f"gguf_{TAG[fmt]}_gemm_bf16_r64x8"
+            assert ops.default_context().last_plan()["kernel"] == kname
             np.testing.assert_array_equal(bits_of(y), bits_of(ops.gated_activation(gu, kind)))
 
 
