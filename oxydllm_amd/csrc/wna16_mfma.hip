@@ -692,38 +692,52 @@ bool awq4_mfma_ok(const Wna16Problem &p) {
     return true;
 }
 
+// The tile-major copy built in the ctx workspace, then the resident-layer kernels on it: two launches (the repack
+// is one pass over the weights: about 45 us at 5120 x 13824, 4-bit).  A caller that holds the layer should hold a
+// PackedQuantLinear, which repacks once.
+static bool transient_repack_fits(const oxq_ctx *ctx, const Wna16Problem &p) {
+    return p.M > 8 && pk4_eligible(p) && !ctx->plan_only && tune(ctx, OXQ_TUNE_TRANSIENT_REPACK, 1) &&
+           !tune(ctx, OXQ_TUNE_FORCE_GENERIC, 0) &&
+           ((pk4_weight_bytes(p.K, p.N, p.bits) + 255) & ~(size_t)255) <= ctx->workspace_bytes;
+}
+static int launch_transient_repack(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p) {
+    Pk4Weights w{(uint32_t *)ctx->workspace, nullptr, p.K, p.N, p.group_shift, p.dtype, p.bits, 0,
+                   p.pack_dim == OXQ_PACK_IN ? 32 : 16, 64};
+    int rc = launch_pk4_prepack(ctx, s, p, w);
+    if (rc != OXQ_OK) return rc;
+    Pk4Problem q;
+    q.x = p.x;
+    q.bias = p.bias;
+    q.y = p.y;
+    q.M = p.M;
+    q.act = 0;
+    q.no_split = 1;  // the workspace holds the copy: no room for K slices' partials
+    q.w = w;
+    rc = launch_pk4_forward(ctx, s, q);
+    ctx->plan.launches = 2;
+    return rc;
+}
+
 int launch_wna16_mfma(oxq_ctx *ctx, hipStream_t s, const Wna16Problem &p) {
+    // Prefill sizes: the resident layout's kernels (x shared in LDS by eight strips, or two with K split inside
+    // the workgroup) run at two to six times the rate of the kernels on the checkpoint layout - 4096 x 14336 at
+    // 2048 rows: 197 (f16) / 216 (bf16) us against 377 / 1313 - which pays for the repack (36 us on that layer) from
+    // a few hundred rows on in f16 (the checkpoint-layout kernel does 0.19 us a row there) and from under a
+    // hundred in bf16 (0.64 us a row): 2048 rows 377 -> 232 and 1313 -> 252 us with the repack included.
+    // The GPTQ kernel on the checkpoint layout holds 0.6 PFLOP/s in both types: the repack pays from 640 rows too
+    // (5120 x 13824 at 2048 rows: 430 / 478 -> 269 / 289 us).
+    const bool awq = awq4_mfma_ok(p), gptq = !awq && gptq_tile_ok(p) && tune(ctx, OXQ_TUNE_GPTQ_TILE, 1) != 2;
+    const int64_t repack_from = awq && p.dtype != OXQ_F16 ? 80 : 640;
+    if (p.M >= repack_from && (awq || gptq) && transient_repack_fits(ctx, p)) return launch_transient_repack(ctx, s, p);
     if (awq4_mfma_ok(p) && !tune(ctx, OXQ_TUNE_FORCE_GENERIC, 0))
         return p.dtype == OXQ_F16 ? launch_awq4_mfma<F16Traits>(ctx, s, p)
                                   : launch_awq4_mfma<BF16Traits>(ctx, s, p);
     if (gptq_tile_ok(p) && tune(ctx, OXQ_TUNE_GPTQ_TILE, 1) && !tune(ctx, OXQ_TUNE_FORCE_GENERIC, 0))
         return launch_gptq_tile(ctx, s, p);
     // Layouts without a tile kernel of their own on the checkpoint layout (8-bit AWQ, unaligned GPTQ): when the
-    // tile-major copy fits the ctx workspace, build it there and run the resident-layer kernel on it.
-    // One launch more (about 45 us at 5120 x 13824, 4-bit) instead of one GEMV pass over the weights
-    // per 8 rows (35 - 45 us each): ahead from m = 9.  A caller that holds the layer should hold a
-    // PackedQuantLinear, which repacks once.
-    if (p.M > 8 && pk4_eligible(p) && !ctx->plan_only && tune(ctx, OXQ_TUNE_TRANSIENT_REPACK, 1) &&
-        !tune(ctx, OXQ_TUNE_FORCE_GENERIC, 0)) {
-        const size_t wb = (pk4_weight_bytes(p.K, p.N, p.bits) + 255) & ~(size_t)255;
-        if (wb <= ctx->workspace_bytes) {
-            Pk4Weights w{(uint32_t *)ctx->workspace, nullptr, p.K, p.N, p.group_shift, p.dtype, p.bits, 0,
-                           p.pack_dim == OXQ_PACK_IN ? 32 : 16, 64};
-            int rc = launch_pk4_prepack(ctx, s, p, w);
-            if (rc != OXQ_OK) return rc;
-            Pk4Problem q;
-            q.x = p.x;
-            q.bias = p.bias;
-            q.y = p.y;
-            q.M = p.M;
-            q.act = 0;
-            q.no_split = 1;
-            q.w = w;
-            rc = launch_pk4_forward(ctx, s, q);
-            ctx->plan.launches = 2;
-            return rc;
-        }
-    }
+    // tile-major copy fits the ctx workspace, build it there and run the resident-layer kernel on it: one launch
+    // more instead of one GEMV pass over the weights per 8 rows (35 - 45 us each): ahead from m = 9.
+    if (transient_repack_fits(ctx, p)) return launch_transient_repack(ctx, s, p);
     // Otherwise (unaligned shapes, copies larger than the workspace): the GEMV kernel over chunks of 8
     // rows, as the reference does below its tile-GEMM threshold (linear.rs:457-480).
     uint32_t launches = 0;

@@ -436,6 +436,43 @@ def test_stateless_tile_op_on_layouts_without_a_tile_kernel(method, bits, dtn, m
     assert_close(ya, oracle.matmul_nt_f32(round_x(xa, dt), oracle.round_through(wa, dt)), "awq4 after a repacked call")
 
 
+@pytest.mark.parametrize("method", ["awq", "gptq"])
+@pytest.mark.parametrize("dtn", ["f16", "bf16"])
+def test_stateless_tile_op_repacks_at_prefill_sizes(method, dtn):
+    """mpp_quant_matmul at prefill sizes: the kernels of the resident layout run at two to six times the rate of
+    those on the checkpoint layout, so from 640 rows (bf16 AWQ: 80) the op builds the tile-major copy in the ctx
+    workspace and runs them (two launches); below that, and with OXQ_TRANSIENT_REPACK = 0, the checkpoint-layout
+    kernel.  Both against the tile oracle."""
+    dt = DT[dtn]
+    K, N, g = 512, 640, 128
+    make = synth.awq_checkpoint if method == "awq" else synth.gptq_checkpoint
+    qw, qz, sc = make(K, N, g, 4, seed=K + N)
+    d = dev_triplet(qw, qz, sc, dt)
+    s_r = oracle.round_through(sc, dt)
+    w = oracle.dequantize_awq(qw, qz, s_r) if method == "awq" else oracle.dequantize_gptq(qw, qz, s_r, 4)
+    wt = oracle.round_through(w, dt)
+    pd = ops.PACK_OUT if method == "awq" else ops.PACK_IN
+    own = "awq4_mfma_pipe" if method == "awq" else "gptq4_tile"
+    first = 80 if (method, dtn) == ("awq", "bf16") else 640
+    x = np.random.default_rng(6).standard_normal((700, K)).astype(np.float32)
+    xd = to_dev(x, TORCH_DT[dt])
+    ref = oracle.matmul_nt_f32(round_x(x, dt), wt)
+    for m in (64, first - 1, first, 700):
+        say(f"prefill repack {method} {dtn} m={m}")
+        y = ops.mpp_quant_matmul(xd[:m], *d, 4, pd)
+        plan = ops.default_context().last_plan()
+        if m >= first:
+            assert plan["kernel"].startswith("pk4_") and plan["launches"] == 2, (m, plan)
+        else:
+            assert plan["kernel"].startswith(own), (m, plan)
+        assert_close(y, ref[:m], f"{method} {dtn} m{m}")
+        tune("OXQ_TRANSIENT_REPACK", 0)
+        y0 = ops.mpp_quant_matmul(xd[:m], *d, 4, pd)
+        assert ops.default_context().last_plan()["kernel"].startswith(own)
+        assert_close(y0, ref[:m], f"{method} {dtn} m{m} on the checkpoint layout")
+        tune("OXQ_TRANSIENT_REPACK", None)
+
+
 # ------------------------------------------------------------------ split-K: fused sum against the second launch
 @pytest.mark.parametrize("route", ["awq4", "awq8", "gptq4", "gptq8", "awq4_generic", "gptq4_generic"])
 @pytest.mark.parametrize("dtn", ["f16", "bf16"])
