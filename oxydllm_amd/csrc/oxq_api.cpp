@@ -1078,6 +1078,21 @@ int oxq_gguf_quant_matmul(oxq_ctx *ctx, void *stream, const oxq_tensor *x,
                        out_features, quant, out, &p));
     int rc = OXQ_OK;
     if (wcache_forward_gguf(ctx, (hipStream_t)stream, p, &rc)) return rc;
+    // Prefill sizes without a cached copy: the matrix-core copy built in the ctx workspace (one pass over the
+    // blocks: 10 us for 4096 x 4096 Q4_K), then its prefill kernel, which runs at 1.5 - 1.8 x the tile matmul on the
+    // file layout - ahead from about a thousand rows.  Two launches.
+    if (!ctx->plan_only && p.act_dtype == OXQ_BF16 && p.M >= 1024 && tune(ctx, OXQ_TUNE_TRANSIENT_REPACK, 1) &&
+        gguf_mfma_eligible(ctx, quant, p.K, p.N) && gguf_gemm_takes(ctx, quant, p.M, p.K, p.N, p.act_dtype) &&
+        ((uintptr_t)p.x & 15) == 0 && ((uintptr_t)p.w & 1) == 0 &&
+        ((gguf_res_bytes(quant, p.K, p.N) + 255) & ~(size_t)255) <= ctx->workspace_bytes) {
+        rc = launch_gguf_mfma_repack(ctx, (hipStream_t)stream, quant, p.w, ctx->workspace, p.K, p.N);
+        if (rc != OXQ_OK) return rc;
+        GgufProblem q = p;
+        q.w = (const uint8_t *)ctx->workspace;
+        rc = launch_gguf_gemm(ctx, (hipStream_t)stream, q);
+        ctx->plan.launches = 2;
+        return rc;
+    }
     if (gguf_mm_eligible(ctx, p)) return launch_gguf_mm(ctx, (hipStream_t)stream, p);
     return launch_gguf_gemv(ctx, (hipStream_t)stream, p);
 }
@@ -1090,6 +1105,21 @@ int oxq_gguf_quant_mul_mm(oxq_ctx *ctx, void *stream, const oxq_tensor *x,
                        out_features, quant, out, &p));
     int rc = OXQ_OK;
     if (wcache_forward_gguf(ctx, (hipStream_t)stream, p, &rc)) return rc;
+    // Prefill sizes without a cached copy: the matrix-core copy built in the ctx workspace (one pass over the
+    // blocks: 10 us for 4096 x 4096 Q4_K), then its prefill kernel, which runs at 1.5 - 1.8 x the tile matmul on the
+    // file layout - ahead from about a thousand rows.  Two launches.
+    if (!ctx->plan_only && p.act_dtype == OXQ_BF16 && p.M >= 1024 && tune(ctx, OXQ_TUNE_TRANSIENT_REPACK, 1) &&
+        gguf_mfma_eligible(ctx, quant, p.K, p.N) && gguf_gemm_takes(ctx, quant, p.M, p.K, p.N, p.act_dtype) &&
+        ((uintptr_t)p.x & 15) == 0 && ((uintptr_t)p.w & 1) == 0 &&
+        ((gguf_res_bytes(quant, p.K, p.N) + 255) & ~(size_t)255) <= ctx->workspace_bytes) {
+        rc = launch_gguf_mfma_repack(ctx, (hipStream_t)stream, quant, p.w, ctx->workspace, p.K, p.N);
+        if (rc != OXQ_OK) return rc;
+        GgufProblem q = p;
+        q.w = (const uint8_t *)ctx->workspace;
+        rc = launch_gguf_gemm(ctx, (hipStream_t)stream, q);
+        ctx->plan.launches = 2;
+        return rc;
+    }
     if (gguf_mm_eligible(ctx, p)) return launch_gguf_mm(ctx, (hipStream_t)stream, p);
     return launch_gguf_gemv(ctx, (hipStream_t)stream, p);
 }

@@ -325,6 +325,38 @@ def test_fused_gate_up_activation_at_prefill(fmt, act, ks):
             np.testing.assert_array_equal(bits_of(y), bits_of(ops.gated_activation(gu, kind)))
 
 
+@pytest.mark.parametrize("fmt", FMTS)
+def test_stateless_prefill_op_builds_the_copy_in_the_workspace(fmt):
+    """oxq_gguf_quant_mul_mm without a layer or a cached copy: from 1024 rows, where the prefill kernel would take the
+    call, the op builds the matrix-core copy in the ctx workspace and runs that kernel (two launches, the layer's
+    bits); fewer rows, f32 activations and OXQ_TRANSIENT_REPACK = 0 keep the tile matmul on the file layout."""
+    name = synth.GGUF_NAMES[fmt]
+    N, K = 128, 512
+    tune("OXQ_GGUF_GEMM_MIN_M", 33)
+    data, layer = _layer(fmt, N, K, seed=7 + fmt)
+    wd = to_dev(data)
+    w = oracle.round_through(oracle.dequantize_gguf(fmt, data, N, K), oracle.BF16)
+    x = np.random.default_rng(8).standard_normal((1030, K)).astype(np.float32)
+    xd = to_dev(x, torch.bfloat16)
+    ref = oracle.matmul_nt_f32(round_x(x, oracle.BF16), w)
+    for m in (1023, 1024, 1030):
+        say(f"gguf stateless prefill {name} m={m}")
+        y = ops.gguf_quant_mul_mm(xd[:m], wd, K, N, fmt)
+        plan = ops.default_context().last_plan()
+        if m >= 1024:
+            assert plan["kernel"] == f"gguf_{TAG[fmt]}_gemm_bf16_r64x8" and plan["launches"] == 2, plan
+            np.testing.assert_array_equal(bits_of(y), bits_of(layer.forward(xd[:m])))
+        else:
+            assert "_mul_mm_bf16" in plan["kernel"], plan
+        assert_close(y, ref[:m], f"gguf stateless prefill {name} m={m}", bf16_out=True)
+    tune("OXQ_TRANSIENT_REPACK", 0)
+    ops.gguf_quant_mul_mm(xd, wd, K, N, fmt)
+    assert "_mul_mm_bf16" in ops.default_context().last_plan()["kernel"]
+    tune("OXQ_TRANSIENT_REPACK", None)
+    ops.gguf_quant_mul_mm(to_dev(x), wd, K, N, fmt)
+    assert "_gemm_" not in ops.default_context().last_plan()["kernel"]
+
+
 @pytest.mark.parametrize("fmt", [synth.GGUF_Q4_0, synth.GGUF_Q4_K, synth.GGUF_Q5_K, synth.GGUF_Q6_K])
 def test_feed_forward_over_a_fused_gguf_layer(fmt):
     """FeedForward (ffn.rs:386-474) with the fused-activation layer as gate_up_proj gives the bits of the layer built
