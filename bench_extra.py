@@ -43,8 +43,8 @@ def run_prefill(ops, ctx, stream, steps, warmup, time_graph):
     dev = torch.device("cuda:0")
     out = []
     steps, warmup = max(4, steps // 8), max(2, warmup // 8)
-    for K, N, rows in ((4096, 14336, (128, 256, 512, 1024, 2048, 4096)), (14336, 4096, (1024, 2048, 4096)),
-                       (4096, 4096, (2048, 4096)), (8192, 28672, (512, 4096))):
+    for K, N, rows in ((4096, 14336, (128, 256, 512, 1024, 2048, 4096)), (14336, 4096, (512, 1024, 2048, 4096)),
+                       (4096, 4096, (512, 1024, 2048, 4096)), (8192, 28672, (512, 4096))):
         qw, qz, sc = synth.awq_checkpoint(K, N, 128, 4, seed=0x0A0D11F3)
         wbytes = qw.nbytes + qz.nbytes + sc.size * 2
         for tdt, tn in ((torch.float16, "f16"), (torch.bfloat16, "bf16")):

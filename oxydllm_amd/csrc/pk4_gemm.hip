@@ -280,25 +280,32 @@ __global__ __launch_bounds__(512) void pk4_gemm_kernel(const uint16_t *__restric
 // projections): a wave's 64 columns are four neighbouring strips, a strip's block is one 16-byte load a lane
 // whose words are the block's four steps - so the ring holds whole blocks, two of them: the next block is
 // requested into the other half when a block starts.  Lane (ni, kb) holds column 16 f + ni of strip f.
-template <typename TT, int MT>
+template <typename TT, int MT, int KS>
 __global__ __launch_bounds__(512) void pk4n_gemm_kernel(const uint16_t *__restrict__ x, const uint32_t *__restrict__ pw,
                                                         const uint16_t *__restrict__ bias, uint16_t *__restrict__ y,
                                                         int M, int K, int N, int NG, int RT) {
     typedef MfmaOps<TT> Ops;
-    constexpr int ROWS = 16 * MT, BB = PK4N_BW * 4, XBUF = ROWS * 256, XV = ROWS / 32;
+    static_assert(KS == 1 || KS == MT, "wave kq of a column group finishes row tile kq");
+    constexpr int SPW = PK4G_STRIPS / KS;  // 64-column groups a workgroup
+    constexpr int ROWS = 16 * MT, BB = PK4N_BW * 4, XBUF = KS * ROWS * 256, XV = ROWS / 4 / SPW;
     constexpr bool BF = TT::DTYPE == BF16Traits::DTYPE;
     extern __shared__ __attribute__((aligned(16))) unsigned char pk4_lds[];
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int ni = lane & 15, kb = lane >> 4;
+    const int ws = wave % SPW, kq = wave / SPW;  // as in pk4_gemm_kernel
     int rt, g;
-    pk4g_tile_of((int)blockIdx.x, RT, NG, rt, g);
-    if (g >= NG) return;  // the whole workgroup, before any barrier
-    const int j = g * PK4G_STRIPS + wave;  // the wave's 64 columns: strips 4 j .. 4 j + 3
+    if constexpr (KS == 1) {
+        pk4g_tile_of((int)blockIdx.x, RT, NG, rt, g);
+        if (g >= NG) return;  // the whole workgroup, before any barrier
+    } else {
+        rt = (int)blockIdx.x / NG, g = (int)blockIdx.x % NG;
+    }
+    const int j = g * SPW + ws;  // the wave's 64 columns: strips 4 j .. 4 j + 3
     const bool live = j < (N >> 6);
     const int m0 = rt * ROWS;
-    const int NB = K >> 7;
+    const int NB = K >> 7, NR = (NB + KS - 1) / KS;
     const int xrows = min(M - m0, ROWS);
 
     const __amdgpu_buffer_rsrc_t rs_none = make_rsrc(pw, 0u);
@@ -310,7 +317,7 @@ __global__ __launch_bounds__(512) void pk4n_gemm_kernel(const uint16_t *__restri
     int xo[XV];
 #pragma unroll
     for (int q = 0; q < XV; ++q) {
-        const int r = 4 * (wave * XV + q) + (lane >> 4);
+        const int r = 4 * (ws * XV + q) + (lane >> 4);
         xo[q] = r * K * 2 + (((lane & 15) ^ (r & 15)) << 4);
     }
     int a_rd[4];
@@ -320,11 +327,13 @@ __global__ __launch_bounds__(512) void pk4n_gemm_kernel(const uint16_t *__restri
 
     u32x4_t wring[2][4];
     uint32_t zring[4];
-    auto dma_x = [&](int i) {
+    // round r: the wave's block is KS r + kq, its tile of x at kq ROWS 256 of the round's buffer
+    auto dma_x = [&](int r) {
+        const int i = KS * r + kq;
         const __amdgpu_buffer_rsrc_t rs = i < NB ? rs_x : rs_none;
 #pragma unroll
         for (int q = 0; q < XV; ++q)
-            pk4g_load_lds16(rs, pk4_lds + (i & 1) * XBUF + (wave * XV + q) * 1024, xo[q], i * 256);
+            pk4g_load_lds16(rs, pk4_lds + (r & 1) * XBUF + kq * (ROWS * 256) + (ws * XV + q) * 1024, xo[q], i * 256);
     };
     auto load_w = [&](int i, u32x4_t (&w)[4]) {
         const __amdgpu_buffer_rsrc_t rs = i < NB ? rs_w : rs_none;
@@ -339,8 +348,8 @@ __global__ __launch_bounds__(512) void pk4n_gemm_kernel(const uint16_t *__restri
 
     dma_x(0);
     __builtin_amdgcn_sched_barrier(0);  // requests keep this order: the wait counts rely on it
-    load_z(0);
-    load_w(0, wring[0]);
+    load_z(kq);
+    load_w(kq, wring[0]);
     __builtin_amdgcn_sched_barrier(0);
     float4_t acc[MT][4];
 #pragma unroll
@@ -350,14 +359,15 @@ __global__ __launch_bounds__(512) void pk4n_gemm_kernel(const uint16_t *__restri
     pk4g_wait_vmcnt<8>();
     __syncthreads();
 
-    // one block, its weights in ring half CUR; eight ring loads are younger than the block's loads of x
-    auto block = [&](int i, auto cur_c) {
+    // one round, the block's weights in ring half CUR; eight ring loads are younger than the round's loads of x
+    auto block = [&](int r, auto cur_c) {
         constexpr int CUR = decltype(cur_c)::value;
-        dma_x(i + 1);
+        const int i = KS * r + kq;  // past NB (a ragged last round): zeros from both streams
+        dma_x(r + 1);
         __builtin_amdgcn_sched_barrier(0);
-        load_w(i + 1, wring[CUR ^ 1]);
+        load_w(i + KS, wring[CUR ^ 1]);
         __builtin_amdgcn_sched_barrier(0);  // not sunk to the block's end, where the next block would wait for them
-        const unsigned char *buf = pk4_lds + (i & 1) * XBUF;
+        const unsigned char *buf = pk4_lds + (r & 1) * XBUF + kq * (ROWS * 256);
         Pk4N<TT> cst[4];
         Pk4gBf16 cb[4];
 #pragma unroll
@@ -368,7 +378,7 @@ __global__ __launch_bounds__(512) void pk4n_gemm_kernel(const uint16_t *__restri
                 cst[f].prep(zring[f]);
             }
         }
-        load_z(i + 1);
+        load_z(i + KS);
 #pragma unroll
         for (int st = 0; st < 4; ++st) {
             uint32_t a[MT][4];
@@ -395,18 +405,43 @@ __global__ __launch_bounds__(512) void pk4n_gemm_kernel(const uint16_t *__restri
             }
         }
         __builtin_amdgcn_sched_barrier(0);
-        pk4g_wait_vmcnt<8>();  // this wave's part of the next block of x is in LDS
+        pk4g_wait_vmcnt<8>();  // this wave's part of the next round of x is in LDS
         __syncthreads();
     };
     {
-        int i = 0;
-        for (; i + 1 < NB; i += 2) {
-            block(i, std::integral_constant<int, 0>{});
-            block(i + 1, std::integral_constant<int, 1>{});
+        int r = 0;
+        for (; r + 1 < NR; r += 2) {
+            block(r, std::integral_constant<int, 0>{});
+            block(r + 1, std::integral_constant<int, 1>{});
         }
-        if (i < NB) block(i, std::integral_constant<int, 0>{});
+        if (r < NR) block(r, std::integral_constant<int, 0>{});
     }
 
+    // the finished tile rows of this wave, as in pk4_gemm_kernel
+    float4_t fin[KS == 1 ? MT : 1][4];
+    if constexpr (KS == 1) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int f = 0; f < 4; ++f) fin[mt][f] = acc[mt][f];
+    } else {
+        float4_t *red = (float4_t *)pk4_lds;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                red[((wave * MT + mt) * 4 + e) * 64 + lane] = float4_t{acc[mt][0][e], acc[mt][1][e], acc[mt][2][e], acc[mt][3][e]};
+        __syncthreads();
+#pragma unroll
+        for (int f = 0; f < 4; ++f) fin[0][f] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int k = 0; k < KS; ++k)  // K order: the same sum whatever the timing
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float4_t v = red[(((k * SPW + ws) * MT + kq) * 4 + e) * 64 + lane];
+                fin[0][0][e] += v[0], fin[0][1][e] += v[1], fin[0][2][e] += v[2], fin[0][3][e] += v[3];
+            }
+    }
     if (!live) return;
     // row 16 mt + 4 kb + e, column 64 j + 16 f + ni
     float bv[4] = {0.f, 0.f, 0.f, 0.f};
@@ -414,14 +449,15 @@ __global__ __launch_bounds__(512) void pk4n_gemm_kernel(const uint16_t *__restri
 #pragma unroll
         for (int f = 0; f < 4; ++f) bv[f] = TT::to_f32(bias[64 * j + 16 * f + ni]);
     }
+    constexpr int FT = KS == 1 ? MT : 1;
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
+    for (int t = 0; t < FT; ++t)
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            const int row = m0 + 16 * mt + 4 * kb + e;
+            const int row = m0 + 16 * (KS == 1 ? t : kq) + 4 * kb + e;
             if (row >= M) continue;
 #pragma unroll
-            for (int f = 0; f < 4; ++f) y[(size_t)row * N + 64 * j + 16 * f + ni] = TT::from_f32(acc[mt][f][e] + bv[f]);
+            for (int f = 0; f < 4; ++f) y[(size_t)row * N + 64 * j + 16 * f + ni] = TT::from_f32(fin[t][f][e] + bv[f]);
         }
 }
 
@@ -440,6 +476,9 @@ __global__ __launch_bounds__(512) void pk4n_gemm_kernel(const uint16_t *__restri
 // a round of the two-strip form (one workgroup a CU) against a full round of 64-row workgroups of eight strips:
 // 19 - 24 us against 65 - 78 at K = 4096 over both widths and types
 constexpr double PK4_MID_ROUND = 0.31;
+// 16-column strips: the same for a whole round, 0.27 for a last round on at most half of the CUs (4096 x 4096,
+// 4096 x 6144, 8192 x 8192, 14336 x 4096 over 65..2048 rows in both types: 18.7 - 24.4 us a round at K = 4096)
+constexpr double PK4N_MID_ROUND = 0.31, PK4N_MID_PART = 0.27;
 
 struct Pk4GemmCost {
     bool pairs64;
@@ -453,9 +492,8 @@ static Pk4GemmForm pk4_gemm_form(const oxq_ctx *ctx, const Pk4Problem &p) {
     const int64_t min_m = tune(ctx, OXQ_TUNE_PK4_GEMM_MIN_M, 65);
     if (min_m <= 0 || (p.w.bits != 4 && p.w.bits != 8) || (p.act && p.w.strip == 16) || p.M < min_m) return {0, 1};
     if (p.w.bits == 8 && p.w.strip == 16) return {0, 1};  // (16-column strips are a 4-bit layout)
-    const bool mid_ok = p.w.strip != 16;  // the K split inside a workgroup: 64-column strips only
     const int forced = tune(ctx, OXQ_TUNE_PK4_GEMM_ROWS, 0), forced_ks = tune(ctx, OXQ_TUNE_PK4_GEMM_KS, 0);
-    if (forced_ks == 4 && mid_ok) return {64, 4};
+    if (forced_ks == 4) return {64, 4};
     if (forced == 64 || forced == 128) return {forced, 1};
     static const Pk4GemmCost WIDE_F16 = {true, 0.88, 1.20, 0.30, 0.97, 1.50, 1.27, 1.93, 1.50};
     static const Pk4GemmCost WIDE_BF16 = {true, 0.93, 1.29, 0.27, 0.98, 1.44, 1.35, 2.00, 1.53};
@@ -476,10 +514,13 @@ static Pk4GemmForm pk4_gemm_form(const oxq_ctx *ctx, const Pk4Problem &p) {
     };
     const double c64 = !c.pairs64 || w64 <= 1.0 ? rounds(w64, 1.0, c.part64, 0.75) : w64 <= 2.0 ? c.a64 + c.b64 * w64 : c.slope64 * w64;
     const double c128 = rounds(w128, c.full128, c.part128, 0.7);
-    const double c_split = (w64 < 1.0 ? c.split_lo : c.split_hi) * w64;
+    // the split-K tiles of the 16-column layout are one workgroup a row tile and 64 columns, in whole rounds too
+    const double c_split = (w64 < 1.0 ? c.split_lo : c.split_hi) * (p.w.strip == 16 ? std::ceil(8.0 * w64 - 1e-9) / 8.0 : w64);
     // two strips a workgroup (128 KB of LDS: one a CU), whole rounds of `PK4_MID_ROUND` each
     const double w_mid = (double)(ceil_div(p.w.N / 64, (int64_t)2) * ceil_div(p.M, (int64_t)64)) / cus;
-    const double c_mid = mid_ok && forced_ks != 1 ? std::ceil(w_mid) * PK4_MID_ROUND : 1e30;
+    const double c_mid = forced_ks == 1        ? 1e30
+                         : p.w.strip == 16 ? rounds(w_mid, PK4N_MID_ROUND, PK4N_MID_PART, 0.5)
+                                           : std::ceil(w_mid) * PK4_MID_ROUND;
     if (c_split <= c64 && c_split <= c128 && c_split <= c_mid) return {0, 1};
     if (c_mid < c64 && c_mid < c128) return {64, 4};
     return {c128 < c64 ? 128 : 64, 1};
@@ -491,8 +532,8 @@ static int pk4_gemm_go(hipStream_t s, dim3 grid, const Pk4Problem &p, int NG, in
     static LdsGrant grant;  // one per instantiation
     const size_t lds = (size_t)2 * KS * 16 * MT * 256;
     if constexpr (LAYOUT == 16) {
-        OXQ_HIP_CHECK(grant.ensure((const void *)pk4n_gemm_kernel<TT, MT>, lds));
-        hipLaunchKernelGGL((pk4n_gemm_kernel<TT, MT>), grid, dim3(512), lds, s, (const uint16_t *)p.x, p.w.pw, (const uint16_t *)p.bias,
+        OXQ_HIP_CHECK(grant.ensure((const void *)pk4n_gemm_kernel<TT, MT, KS>, lds));
+        hipLaunchKernelGGL((pk4n_gemm_kernel<TT, MT, KS>), grid, dim3(512), lds, s, (const uint16_t *)p.x, p.w.pw, (const uint16_t *)p.bias,
                            (uint16_t *)p.y, (int)p.M, (int)p.w.K, (int)p.w.N, NG, RT);
     } else {
         OXQ_HIP_CHECK(grant.ensure((const void *)pk4_gemm_kernel<TT, MT, LAYOUT, KS>, lds));
@@ -504,9 +545,7 @@ static int pk4_gemm_go(hipStream_t s, dim3 grid, const Pk4Problem &p, int NG, in
 }
 template <typename TT, int MT, int KS>
 static int pk4_gemm_go_layout(hipStream_t s, dim3 grid, const Pk4Problem &p, int NG, int RT) {
-    if constexpr (KS == 1) {
-        if (p.w.strip == 16) return pk4_gemm_go<TT, MT, 16, 1>(s, grid, p, NG, RT);
-    }
+    if (p.w.strip == 16) return pk4_gemm_go<TT, MT, 16, KS>(s, grid, p, NG, RT);
     return p.w.bits == 8 ? pk4_gemm_go<TT, MT, 8, KS>(s, grid, p, NG, RT) : pk4_gemm_go<TT, MT, 4, KS>(s, grid, p, NG, RT);
 }
 

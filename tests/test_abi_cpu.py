@@ -412,13 +412,16 @@ def test_layers_validate_like_reference(lib, ctx):
     assert lib.oxq_packed_quant_linear_forward(h, None, C.byref(x), C.byref(fake((1, 14336), BF16))) == -3
     assert "input last dim 4000 != in_features 4096" in err(lib)
     lib.oxq_packed_quant_linear_free(h)
-    # a narrow layer (16-column strips): eight groups of 512 columns fill the chip from 2048 rows on
+    # a narrow layer (16-column strips): eight groups of 512 columns fill the chip from 2048 rows on; below, 32 pairs
+    # of 64-column groups x row tiles with K split inside the workgroup, from where the split-K tiles need a second
+    # round of 256 workgroups
     nqw, nqz, nsc = _awq(4096, 4096, 128, F16)
     assert lib.oxq_packed_quant_linear_new(ctx, 4, 0, C.byref(nqw), C.byref(nqz), C.byref(nsc), None,
                                            F16, C.byref(h)) == 0, err(lib)
-    for rows, kern, wgs in [(64, "pk4_mfma_f16_mt4_n16x4", None), (1024, "pk4_mfma_f16_mt4_n16x4", None),
-                            (2048, "pk4_gemm_f16_r64x8_n16", 256), (4096, "pk4_gemm_f16_r128x8_n16", 256),
-                            (4100, "pk4_gemm_f16_r64x8_n16", 512 + 8)]:
+    for rows, kern, wgs in [(64, "pk4_mfma_f16_mt4_n16x4", None), (256, "pk4_mfma_f16_mt4_n16x4", None),
+                            (384, "pk4_gemm_f16_r64x2k4_n16", 6 * 32), (1024, "pk4_gemm_f16_r64x2k4_n16", 16 * 32),
+                            (1536, "pk4_gemm_f16_r64x8_n16", 192), (2048, "pk4_gemm_f16_r64x8_n16", 256), (4096, "pk4_gemm_f16_r128x8_n16", 256),
+                            (4100, "pk4_gemm_f16_r64x2k4_n16", 65 * 32)]:  # four rows past two rounds of 128-row workgroups
         assert lib.oxq_packed_quant_linear_forward(h, None, C.byref(fake((rows, 4096), F16)),
                                                    C.byref(fake((rows, 4096), F16))) == 0, err(lib)
         pl = plan(lib, ctx)

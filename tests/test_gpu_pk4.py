@@ -199,17 +199,19 @@ def test_prefill_rows_by_eight_strips(kind, dtn, rows, K, N, g, strip16):
     assert_close(out, tile_all[:300] - bias[None, :], f"pk4 prefill {kind} {dtn} no bias")
 
 
-@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("kind,strip16", [(k, s16) for k in KINDS for s16 in (0, 2) if not (s16 and k.endswith("8"))])
 @pytest.mark.parametrize("dtn", ["f16", "bf16"])
 @pytest.mark.parametrize("K,N,g", [(512, 576, 128), (1280, 1088, 128), (256, 64, 128), (4096, 128, 128)])
-def test_prefill_two_strips_with_k_split(kind, dtn, K, N, g):
+def test_prefill_two_strips_with_k_split(kind, dtn, K, N, g, strip16):
     """The form for 65 to a few hundred rows: a workgroup = 64 rows x two strips, the four waves of a strip take every
     fourth block of K and wave kq finishes row tile kq from the four partial tiles in LDS.  N = 576 and 1088 leave
     the last workgroup one live strip; K of 2 blocks (half the waves have none), 4 (one round), 10 (a ragged third
-    round) and 32; ragged row tiles.  Against the tile-GEMM oracle, run to run bitwise, rows independent of m."""
+    round: both ring halves of the 16-column layout, and an odd count) and 32; ragged row tiles.  Both resident
+    layouts.  Against the tile-GEMM oracle, run to run bitwise, rows independent of m."""
     bits = bits_of_kind(kind)
-    tune("OXQ_PK4_STRIP16", 0)
+    tune("OXQ_PK4_STRIP16", strip16)
     tune("OXQ_PK4_GEMM_KS", 4)
+    n16 = "_n16" if strip16 else ""
     dt = DT[dtn]
     trip, pack_dim = make(kind, K, N, g, seed=K + 7 * N)
     bias = (np.arange(N, dtype=np.float32) % 13 - 6) * np.float32(0.125)
@@ -226,7 +228,7 @@ def test_prefill_two_strips_with_k_split(kind, dtn, K, N, g):
         say(f"pk{bits} prefill two strips {kind} {dtn} K={K} N={N} m={m}")
         y = layer.forward(xd_all[:m])
         plan = ops.default_context().last_plan()
-        assert plan["kernel"] == f"pk{bits}_gemm_{dtn}_r64x2k4" and plan["launches"] == 1, plan
+        assert plan["kernel"] == f"pk{bits}_gemm_{dtn}_r64x2k4{n16}" and plan["launches"] == 1, plan
         assert plan["grid"][0] == -(-m // 64) * -(-(N // 64) // 2) and plan["block"][0] == 512, plan
         assert_close(y, tile_all[:m], f"pk{bits} two strips {kind} {dtn} m{m}")
         assert np.abs(as_f32(y) - ref_all[:m]).max() < 0.06 * np.abs(ref_all[:m]).max() + 1e-2
@@ -235,7 +237,7 @@ def test_prefill_two_strips_with_k_split(kind, dtn, K, N, g):
             first = bits_of(y)
         else:
             np.testing.assert_array_equal(bits_of(y), first[:m])
-    if N % 128 == 0 and N >= 128:
+    if N % 128 == 0 and N >= 128 and not strip16:
         # the same layer as a fused gate|up projection: the activation epilogue on the summed tile
         kind_id = ops.ACT_GATED_SILU
         tdt = TORCH_DT[dt]
