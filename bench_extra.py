@@ -13,6 +13,8 @@ bytes, TFLOP/s, fraction of the 8 TB/s HBM peak).
 """
 from __future__ import annotations
 
+import sys
+
 import numpy as np
 import torch
 
@@ -30,6 +32,7 @@ def _case(name, fn_of_step, steps, warmup, stream, time_graph, nbytes, flops, ct
     plan = ctx.last_plan()
     _, ev_ms = time_graph(fn_of_step, steps, warmup, stream)
     us = ev_ms * 1e3 / steps
+    print(f"[bench] {name}: {us:.3f} us, {plan['kernel']}", file=sys.stderr, flush=True)  # a long run shows it is alive
     return {"case": name, "kernel": plan["kernel"], "launches": plan["launches"],
             "us_per_call": round(us, 3), "algorithmic_bytes": int(nbytes),
             "GB_per_s": round(nbytes / us / 1e3, 1), "hbm_frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
@@ -375,25 +378,48 @@ def run(ops, ctx, stream, steps, warmup, time_graph):
             ops.mxfp4_matmul(xm, gub[0][:nb1 * 16], gub[1][:nb1], H, 2 * I, out=ym, ctx=ctx)
         out.append(_case(f"mxfp4 M={m} K={H} N={2 * I} bf16 (mxfp4_matmul, prefill)", pstep, steps, warmup, stream,
                          time_graph, nb1 * 17 + m * (H + 2 * I) * 2, 2.0 * m * H * 2 * I, ctx))
-    Tp = 512
-    logits_p = torch.randn((Tp, E), device=dev, dtype=torch.float32)
-    xp = torch.randn((Tp, H), device=dev, dtype=torch.bfloat16)
-    np_p = Tp * top_k
-    ygu_p = torch.empty((np_p, 2 * I), device=dev, dtype=torch.bfloat16)
-    h_p = torch.empty((np_p, I), device=dev, dtype=torch.bfloat16)
-    ydn_p = torch.empty((np_p, H), device=dev, dtype=torch.bfloat16)
-    out_p = torch.empty((Tp, H), device=dev, dtype=torch.bfloat16)
+    # a MoE layer step at prefill sizes: through the stateless ops on the checkpoint layout (tile matmul + activation
+    # kernel), and on the resident experts (tiles of an expert's pairs on the tile-major copy, SwiGLU in the epilogue)
+    gu_res = ops.Mxfp4Experts(gub[0], gub[1], gu_bias, E, H, 2 * I, ctx=ctx)
+    dn_res = ops.Mxfp4Experts(dnb[0], dnb[1], dn_bias, E, I, H, ctx=ctx)
+    for Tp in (512, 2048):
+        logits_p = torch.randn((Tp, E), device=dev, dtype=torch.float32)
+        xp = torch.randn((Tp, H), device=dev, dtype=torch.bfloat16)
+        np_p = Tp * top_k
+        ygu_p = torch.empty((np_p, 2 * I), device=dev, dtype=torch.bfloat16)
+        h_p = torch.empty((np_p, I), device=dev, dtype=torch.bfloat16)
+        ydn_p = torch.empty((np_p, H), device=dev, dtype=torch.bfloat16)
+        out_p = torch.empty((Tp, H), device=dev, dtype=torch.bfloat16)
 
-    def prefill_step(i):
-        idx, vals = ops.moe_route(logits_p, top_k, True, ctx=ctx)
-        off, tok, _, pos = ops.moe_group(idx, vals, E, ctx=ctx)
-        ops.mxfp4_moe_matmul(xp, gub[0], gub[1], gu_bias, off, tok, H, 2 * I, out=ygu_p, ctx=ctx)
-        ops.gated_activation(ygu_p, ops.ACT_GPT_OSS_SWIGLU, 7.0, out=h_p, ctx=ctx)
-        ops.mxfp4_moe_matmul(h_p, dnb[0], dnb[1], dn_bias, off, None, I, H, out=ydn_p, ctx=ctx)
-        ops.moe_combine(ydn_p, pos, vals, out=out_p, ctx=ctx)
-    r3 = _case(f"mxfp4 moe layer step, prefill: {Tp} tokens, {np_p} pairs over {E} experts", prefill_step, steps,
-               warmup, stream, time_graph, E * per_expert + np_p * (H + 2 * I + I + H) * 2,
-               2.0 * np_p * (2 * I * H + H * I), ctx)
-    r3["launches"] = 6
-    out.append(r3)
+        def prefill_step(i):
+            idx, vals = ops.moe_route(logits_p, top_k, True, ctx=ctx)
+            off, tok, _, pos = ops.moe_group(idx, vals, E, ctx=ctx)
+            ops.mxfp4_moe_matmul(xp, gub[0], gub[1], gu_bias, off, tok, H, 2 * I, out=ygu_p, ctx=ctx)
+            ops.gated_activation(ygu_p, ops.ACT_GPT_OSS_SWIGLU, 7.0, out=h_p, ctx=ctx)
+            ops.mxfp4_moe_matmul(h_p, dnb[0], dnb[1], dn_bias, off, None, I, H, out=ydn_p, ctx=ctx)
+            ops.moe_combine(ydn_p, pos, vals, out=out_p, ctx=ctx)
+
+        def prefill_step_res(i):
+            idx, vals = ops.moe_route(logits_p, top_k, True, ctx=ctx)
+            off, tok, _, pos = ops.moe_group(idx, vals, E, ctx=ctx)
+            gu_res.gate_up_swiglu(xp, off, tok, 7.0, out=h_p)
+            dn_res.matmul(h_p, off, None, out=ydn_p)
+            ops.moe_combine(ydn_p, pos, vals, out=out_p, ctx=ctx)
+        nbytes = E * per_expert + np_p * (H + 2 * I + I + H) * 2
+        fl = 2.0 * np_p * (2 * I * H + H * I)
+        r3 = _case(f"mxfp4 moe layer step, prefill: {Tp} tokens, {np_p} pairs over {E} experts (stateless ops, checkpoint layout)",
+                   prefill_step, steps, warmup, stream, time_graph, nbytes, fl, ctx)
+        r3["launches"] = 6
+        r3["mfma_frac"] = round(r3["TFLOP_per_s"] / 2500.0, 4)
+        out.append(r3)
+        r4 = _case(f"mxfp4 moe layer step, prefill: {Tp} tokens, {np_p} pairs over {E} experts (resident experts, fused SwiGLU)",
+                   prefill_step_res, steps, warmup, stream, time_graph, nbytes - np_p * 2 * I * 2 * 2, fl, ctx)
+        r4["launches"] = 5
+        off0, tok0 = ops.moe_group(*ops.moe_route(logits_p, top_k, True, ctx=ctx), E, ctx=ctx)[:2]
+        gu_res.gate_up_swiglu(xp, off0, tok0, 7.0, out=h_p)
+        r4["kernel"] = ctx.last_plan()["kernel"]
+        r4["mfma_frac"] = round(r4["TFLOP_per_s"] / 2500.0, 4)
+        out.append(r4)
+        del logits_p, xp, ygu_p, h_p, ydn_p, out_p
+    del gu_res, dn_res
     return out

@@ -345,9 +345,10 @@ int oxq_mxfp4_moe_gate_up_swiglu(oxq_ctx *ctx, void *stream, const oxq_tensor *x
  * [E, n, k/32] scales, for the life of the model) and moe.rs:563-607 (dispatch_sparse runs them).
  * `new` is the load-time step: when n is a multiple of 16 it builds a tile-major copy in device memory
  * owned by the handle (matrix-core operand order, one contiguous run per 16 rows; the checkpoint tensors'
- * size plus at most one block in four per row) and synchronises the null stream once; decode sizes then
- * stream that copy.  The caller's tensors are borrowed and must outlive the handle: many pairs per expert
- * (n_pairs >= 8 * n_experts) and shapes that do not qualify run on them, with the stateless ops' kernels.
+ * size plus at most one block in four per row) and synchronises the null stream once; every call then
+ * runs on that copy: the decode GEMV below three pairs an expert on average, tiles of 16 - 128 of an expert's
+ * pairs above, both with the fused SwiGLU.  The caller's tensors are borrowed and must outlive the handle:
+ * shapes that do not qualify (and an x of 2 GiB or more) run on them, with the stateless ops' kernels.
  * OXQ_PREPACK=0 in the environment disables the copy. */
 typedef struct oxq_mxfp4_experts oxq_mxfp4_experts;
 int oxq_mxfp4_experts_new(oxq_ctx *ctx, const oxq_tensor *blocks, const oxq_tensor *scales,

@@ -17,7 +17,7 @@ LIB = os.path.join(HERE, "liboxq_hip.so")
 OBJ_DIR = os.path.join(HERE, "csrc", "build")
 
 SOURCES = ["oxq_api.cpp", "wna16_gemv.hip", "wna16_mfma.hip", "wna16_dequant.hip", "awq_transforms.hip", "pk4.hip", "pk4_tile.hip", "pk4_gemm.hip", "gptq_tile.hip",
-           "gguf_gemv.hip", "gguf_res.hip", "gguf_mfma.hip", "blockq_mm.hip", "mxfp4_gemv.hip", "moe_glue.hip", "f8_block.hip", "calib.hip",
+           "gguf_gemv.hip", "gguf_res.hip", "gguf_mfma.hip", "blockq_mm.hip", "mxfp4_gemv.hip", "mxfp4_gemm.hip", "moe_glue.hip", "f8_block.hip", "calib.hip",
            "checkpoint_files.cpp"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")

@@ -1580,9 +1580,12 @@ static int experts_forward(oxq_mxfp4_experts *h, void *stream, const oxq_tensor 
         return fail(OXQ_ERR_SHAPE, "%s: expert_offsets must be a contiguous I32 [%lld]", op, (long long)h->n_experts + 1);
     const bool resident = h->pw != nullptr;
     const int64_t n_pairs = (out && out->rank == 2) ? out->dims[0] : 0;
-    // many pairs per expert (prefill) convert a weight once per 64 tokens in the tile matmul, which reads the
-    // checkpoint layout
-    if (!resident || n_pairs >= 8 * h->n_experts)
+    // many pairs per expert (prefill) convert a weight once per 64 tokens: the prefill kernel on the copy, or
+    // (sizes it does not take) the tile matmul, which reads the checkpoint layout
+    // (its 32-bit offsets into x hold up to 2 GiB; more than that takes the tile matmul as before)
+    const bool prefill = resident && x && x->rank == 2 && (uint64_t)x->dims[0] * (uint64_t)h->k * 2u < (1ull << 31) &&
+                         mxfp4_gemm_form(ctx, n_pairs, h->n_experts, h->k, h->n) != 0;
+    if (!resident || (!prefill && n_pairs >= 8 * h->n_experts))
         return moe_matmul_impl(op, ctx, stream, x, &h->blocks, &h->scales, h->has_bias ? &h->bias : nullptr, expert_offsets,
                                token_ids, gather_rows, h->k, h->n, swiglu, limit, out, fused);
     Mxfp4Problem p;
@@ -1607,7 +1610,9 @@ static int experts_forward(oxq_mxfp4_experts *h, void *stream, const oxq_tensor 
     p.n_pairs = n_pairs;
     p.swiglu = swiglu ? 1 : 0;
     p.swiglu_limit = limit;
-    const int rc = launch_mxfp4_res_gemv(ctx, (hipStream_t)stream, p);
+    p.M = x->dims[0];
+    // many pairs an expert (prefill): 64-row tiles on the same copy
+    const int rc = prefill ? launch_mxfp4_res_gemm(ctx, (hipStream_t)stream, p) : launch_mxfp4_res_gemv(ctx, (hipStream_t)stream, p);
     if (rc == OXQ_OK && fused) *fused = 1;
     return rc;
 }

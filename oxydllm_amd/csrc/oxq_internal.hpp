@@ -20,7 +20,8 @@
     X(ACT_VEC) X(F8_MM_KS) X(F8_MM_MIN_M) X(F8_MM_MT) X(FORCE_GENERIC) X(GEMV_CFG) X(GEMV_GPW) X(GEMV_TILE)   \
     X(GGR_GRID) X(GGR_WAVES) X(GGUF_BIG_LDS) X(GGUF_GEMM_KS) X(GGUF_GEMM_MIN_M) X(GGUF_MFMA)                  \
     X(GGUF_MFMA_MAX_M) X(GGUF_MFMA_NS) X(GGUF_MM_KS) X(GGUF_MM_MIN_M) X(GGUF_MM_MT) X(GGUF_PW) X(GGUF_RPWG)   \
-    X(GPTQ_TILE) X(GPTQ_TILE_KS) X(MFMA_MT) X(MFMA_SPLITK) X(MFMA_VARIANT) X(MXFP4_FR) X(MXFP4_MM)            \
+    X(GPTQ_TILE) X(GPTQ_TILE_KS) X(MFMA_MT) X(MFMA_SPLITK) X(MFMA_VARIANT) X(MXFP4_FR) X(MXFP4_GEMM_MIN_PAIRS) \
+    X(MXFP4_GEMM_ROWS) X(MXFP4_MM)      \
     X(MXFP4_MM_KS) X(MXFP4_MM_MT) X(MXFP4_VARIANT) X(PK4N_NS1_ROWS) X(PK4N_W16) X(PK4_CONTIGUOUS)             \
     X(PK4_FOLD) X(PK4_FRONT) X(PK4_GEMM_KS) X(PK4_GEMM_MIN_M) X(PK4_GEMM_ROWS) X(PK4_KS) X(PK4_PLACE64)       \
     X(PK4_STRIP16) X(PK4_T64) X(PK4_XQ) X(PREPACK) X(SPLITK_MODE) X(TRANSIENT_REPACK)
@@ -273,6 +274,9 @@ int launch_mxfp4_repack(oxq_ctx *ctx, hipStream_t s, const uint8_t *blocks, cons
 int launch_mxfp4_res_dequant(oxq_ctx *ctx, hipStream_t s, const void *pw, const void *ps, int64_t expert, int64_t K,
                              int64_t N, float *out_nk);
 int launch_mxfp4_res_gemv(oxq_ctx *ctx, hipStream_t s, const Mxfp4Problem &p);
+// prefill on the resident copy: 0 = not taken, else the rows of a tile; p.M = rows of x
+int mxfp4_gemm_form(const oxq_ctx *ctx, int64_t n_pairs, int64_t E, int64_t K, int64_t N);
+int launch_mxfp4_res_gemm(oxq_ctx *ctx, hipStream_t s, const Mxfp4Problem &p);
 // mixture-of-experts glue (moe_glue.hip)
 int launch_moe_route(oxq_ctx *ctx, hipStream_t s, const void *logits, int dtype, int64_t T, int64_t E, int64_t top_k,
                      int norm_topk, int32_t *top_idx, float *top_vals);

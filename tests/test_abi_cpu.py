@@ -267,6 +267,38 @@ def test_mxfp4_validation(lib, ctx):
     assert call(out=fake((7, N), BF16)) == -3 and "output shape" in err(lib)
 
 
+def test_resident_experts_pick_their_kernel_by_pairs(lib, ctx):
+    """oxq_mxfp4_experts_* (moe.rs:366-417, 563-607): below three pairs an expert on average the decode GEMV on the
+    copy, above it tiles of an expert's pairs whose rows follow the average; a shape without whole tiles of 16
+    weight rows keeps the checkpoint-layout kernels."""
+    E, K, N = 32, 2880, 5760
+    nb = K // 32
+    blocks, scales = fake((E * N * nb * 16,), U8), fake((E * N * nb,), U8)
+    h = C.c_void_p()
+    assert lib.oxq_mxfp4_experts_new(ctx, C.byref(blocks), C.byref(scales), None, E, K, N, C.byref(h)) == 0, err(lib)
+    off = fake((E + 1,), I32)
+    for tokens, kern, ytiles in [(8, "mxfp4_experts_gemv_bf16_t4", None), (24, "mxfp4_experts_gemm_bf16_r16x8", 96 // 16 + E),
+                                 (96, "mxfp4_experts_gemm_bf16_r16x8", 384 // 16 + E), (128, "mxfp4_experts_gemm_bf16_r32x8", 512 // 32 + E),
+                                 (512, "mxfp4_experts_gemm_bf16_r32x8", 2048 // 32 + E), (1024, "mxfp4_experts_gemm_bf16_r64x8", 4096 // 64 + E),
+                                 (4096, "mxfp4_experts_gemm_bf16_r128x8", 16384 // 128 + E)]:
+        pairs = 4 * tokens
+        x, tok = fake((tokens, K), BF16), fake((pairs,), I32)
+        assert lib.oxq_mxfp4_experts_matmul(h, None, C.byref(x), C.byref(off), C.byref(tok), 1, C.byref(fake((pairs, N), BF16))) == 0, err(lib)
+        pl = plan(lib, ctx)
+        assert pl.kernel.decode() == kern and pl.launches == 1, (tokens, pl.kernel)
+        if ytiles is not None:
+            assert (pl.grid[0], pl.grid[1], pl.block[0]) == (12, ytiles, 512), (tokens, tuple(pl.grid))
+        fused = C.c_int(-1)
+        assert lib.oxq_mxfp4_experts_gate_up_swiglu(h, None, C.byref(x), C.byref(off), C.byref(tok), 1, 7.0,
+                                                    C.byref(fake((pairs, N // 2), BF16)), C.byref(fused)) == 0, err(lib)
+        assert fused.value == 1 and plan(lib, ctx).kernel.decode() == kern + "_swiglu"
+    x, tok = fake((128, K), BF16), fake((512,), I32)
+    assert lib.oxq_mxfp4_experts_matmul(h, None, C.byref(x), C.byref(off), C.byref(tok), 1, C.byref(fake((512, N + 16), BF16))) == -3
+    assert lib.oxq_mxfp4_experts_matmul(h, None, C.byref(x), C.byref(off), C.byref(fake((500,), I32)), 1, C.byref(fake((512, N), BF16))) == -3
+    assert "token_ids" in err(lib)
+    lib.oxq_mxfp4_experts_free(h)
+
+
 def test_feed_forward_validates_and_plans(lib, ctx):
     """ffn.rs:22-474 at the benchmark's layer size: layouts, shape checks, scratch sizes, launch plans."""
     H, I = 4096, 14336

@@ -81,6 +81,7 @@ def test_experts_dequantize_is_bit_exact(E, N, K):
 def test_experts_matmul_matches_oracle_and_the_stateless_op(E, N, K, counts, gather):
     from oxydllm_amd import ops
     say(f"experts matmul E={E} N={N} K={K} counts={counts} gather={gather}")
+    tune("OXQ_MXFP4_GEMM_MIN_PAIRS", 0)  # the decode kernel at every pair count, also where the tiles would take over
     blocks, scales, bias = _experts(E, N, K, seed=7 * E + N)
     offsets, tokens, n_tok = _lists(counts)
     n_pairs = int(offsets[-1])
@@ -113,6 +114,7 @@ def test_experts_matmul_matches_oracle_and_the_stateless_op(E, N, K, counts, gat
 def test_experts_gate_up_swiglu_equals_the_two_calls(E, N, K, counts):
     from oxydllm_amd import ops
     say(f"experts swiglu E={E} N={N} K={K}")
+    tune("OXQ_MXFP4_GEMM_MIN_PAIRS", 0)
     blocks, scales, bias = _experts(E, N, K, seed=N + K)
     offsets, tokens, n_tok = _lists(counts)
     x = np.random.default_rng(1).standard_normal((n_tok, K)).astype(np.float32) * 2
@@ -125,6 +127,61 @@ def test_experts_gate_up_swiglu_equals_the_two_calls(E, N, K, counts):
     assert np.array_equal(bits_of(fused), bits_of(two))
     want = oracle.gpt_oss_swiglu(gu.float().cpu().numpy(), 7.0)
     assert_close(fused, want, "swiglu on the resident copy")
+
+
+@pytest.mark.parametrize("E,N,K,counts", [
+    (3, 80, 2880, [70, 0, 130]),      # 22.5 chunks; five tiles: a wave with one live tile of its four
+    (2, 192, 96, [5, 64]),            # three blocks: one chunk, cut off; a whole row tile and a sliver
+    (4, 64, 512, [1, 65, 0, 128]),    # four chunks; an idle expert
+    (2, 640, 1280, [33, 200]),        # ten chunks: both ring halves; two column groups, the second two waves wide
+])
+@pytest.mark.parametrize("rows", [16, 32, 64, 128])
+@pytest.mark.parametrize("gather", [True, False])
+def test_experts_prefill_kernel_on_the_copy(E, N, K, counts, rows, gather):
+    """Many pairs an expert: tiles of 16 - 128 of an expert's pairs x the waves' four tiles of 16 weight rows, x
+    gathered through the token list straight into LDS, whole K in a wave's accumulators.  Against the
+    f32-accumulated oracle on the dense dequant (the weights are exact in bf16, so this is the tile matmul's
+    arithmetic too), run to run bitwise, and with the fused SwiGLU epilogue bit-identical to matmul + activation."""
+    from oxydllm_amd import ops
+    say(f"experts prefill E={E} N={N} K={K} counts={counts} rows={rows} gather={gather}")
+    tune("OXQ_MXFP4_GEMM_MIN_PAIRS", 1)
+    tune("OXQ_MXFP4_GEMM_ROWS", rows)
+    blocks, scales, bias = _experts(E, N, K, seed=3 * E + N)
+    offsets, tokens, n_tok = _lists(counts)
+    n_pairs = int(offsets[-1])
+    x = np.random.default_rng(K + 1).standard_normal((n_tok, K)).astype(np.float32)
+    xb, bb = round_x(x, oracle.BF16), round_x(bias, oracle.BF16)
+    ref = np.zeros((n_pairs, N), np.float32)
+    for e in range(E):
+        lo, hi = int(offsets[e]), int(offsets[e + 1])
+        if hi > lo:
+            ref[lo:hi] = oracle.matmul_nt_f32(xb[tokens[lo:hi]], _dense(blocks, scales, e, N, K), bb[e])
+    bd, sd, biasd = to_dev(blocks), to_dev(scales), to_dev(bias, torch.bfloat16)
+    ex = ops.Mxfp4Experts(bd, sd, biasd, E, K, N)
+    assert ex.resident
+    off_d = to_dev(offsets)
+    if gather:
+        xd, tok_d = to_dev(x, torch.bfloat16), to_dev(tokens)
+    else:
+        xd, tok_d = to_dev(x[tokens], torch.bfloat16), None
+    y = ex.matmul(xd, off_d, tok_d)
+    plan = ops.default_context().last_plan()
+    kname = f"mxfp4_experts_gemm_bf16_r{rows}x8"
+    assert plan["kernel"] == kname and plan["launches"] == 1, plan
+    assert plan["grid"][0] == -(-(N // 16) // 32) and plan["grid"][1] == n_pairs // rows + E, plan
+    assert_close(y, ref, "experts prefill matmul")
+    assert np.array_equal(bits_of(ex.matmul(xd, off_d, tok_d)), bits_of(y))
+    # without a bias, into a buffer that holds other values
+    plain = ops.Mxfp4Experts(bd, sd, None, E, K, N)
+    out = torch.full((n_pairs, N), 3.0, device="cuda", dtype=torch.bfloat16)
+    plain.matmul(xd, off_d, tok_d, out=out)
+    assert ops.default_context().last_plan()["kernel"] == kname
+    assert_close(out, ref - np.repeat(bb, counts, axis=0), "experts prefill matmul, no bias")
+    # interleaved gate / up rows with the clamped SwiGLU in the epilogue
+    fused = ex.gate_up_swiglu(xd * 2, off_d, tok_d, 7.0)
+    assert ops.default_context().last_plan()["kernel"] == kname + "_swiglu"
+    two = ops.gated_activation(ex.matmul(xd * 2, off_d, tok_d), ops.ACT_GPT_OSS_SWIGLU, 7.0)
+    assert np.array_equal(bits_of(fused), bits_of(two))
 
 
 def test_experts_fall_back_where_the_copy_does_not_apply(monkeypatch):
@@ -140,7 +197,9 @@ def test_experts_fall_back_where_the_copy_does_not_apply(monkeypatch):
     y = ex.matmul(to_dev(x, torch.bfloat16), to_dev(offsets), to_dev(tokens))
     y0 = ops.mxfp4_moe_matmul(to_dev(x, torch.bfloat16), bd, sd, biasd, to_dev(offsets), to_dev(tokens), K, N)
     assert np.array_equal(bits_of(y), bits_of(y0))
-    # many pairs per expert: the tile matmul on the checkpoint layout, same result as the stateless op
+    # the prefill kernel switched off: many pairs per expert take the tile matmul on the checkpoint layout, same
+    # result as the stateless op
+    tune("OXQ_MXFP4_GEMM_MIN_PAIRS", 0)
     E, N, K = 2, 64, 128
     blocks, scales, bias = _experts(E, N, K, seed=4)
     offsets, tokens, n_tok = _lists([20, 13])
