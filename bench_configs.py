@@ -286,6 +286,13 @@ def run(ops, ctx, stream, steps, warmup, time_graph, with_cpu=True):
               warmup, stream, time_graph, nb, flops, ctx)
     r1["launches"] = 2
     rows.append(r1)
+    ctx.set_weight_cache(1 << 30)  # the op remembers the stacked expert tensors by address: the resident experts' copy
+    step_ops(0)
+    r1c = _row("cfg4", "the same step through the stateless mxfp4_moe_matmul op with the ctx weight cache on", step_ops, steps,
+               warmup, stream, time_graph, nb, flops, ctx)
+    r1c["launches"] = 2
+    rows.append(r1c)
+    ctx.set_weight_cache(0)
 
     logits_d = torch.from_numpy(logits).to(dev)
     out_d = torch.empty((T, H), device=dev, dtype=torch.bfloat16)

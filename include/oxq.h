@@ -140,7 +140,10 @@ int oxq_ctx_reset_tuning(oxq_ctx *ctx, const char *name);
  * again; least recently used copies go when max_bytes is reached.  oxq_gguf_quant_matmul does the
  * same for the GGUF formats that have a strip-major form (see oxq_qlinear_new) at the rows that form takes
  * (f32: 1 - 8; bf16: 1 - 32 on the matrix-core copy, there also for oxq_gguf_quant_mul_mm), keyed by the
- * address of the block bytes and the layout, with the copy that oxq_qlinear_new builds.
+ * address of the block bytes and the layout, with the copy that oxq_qlinear_new builds; and
+ * oxq_mxfp4_moe_matmul / oxq_mxfp4_moe_gate_up_swiglu for stacked expert tensors with n a multiple of 16,
+ * keyed by the addresses of blocks and scales, with the copy and the kernels of oxq_mxfp4_experts_new (the
+ * SwiGLU then fused at every size).
  *
  * A copy that served a call while the stream was being captured is part of that graph: it stays, and
  * counts against max_bytes, until oxq_ctx_forget_weights or oxq_ctx_destroy frees it - either of which
@@ -151,7 +154,7 @@ int oxq_ctx_reset_tuning(oxq_ctx *ctx, const char *name);
  * a copy.
  *
  * Contract: while a triple is cached its tensors must neither change nor be freed and reused - the
- * ctx cannot see that.  Call oxq_ctx_forget_weights(ctx, qweight->data) (for a GGUF weight: the
+ * ctx cannot see that.  Call oxq_ctx_forget_weights(ctx, qweight->data) (for a GGUF or MXFP4 weight: the
  * address of its block bytes) before doing so (NULL drops every copy).  Off by default (max_bytes = 0, or OXQ_WEIGHT_CACHE_MB in the environment).
  * No counterpart in the reference, whose ops read the checkpoint layout directly. */
 int oxq_ctx_set_weight_cache(oxq_ctx *ctx, int64_t max_bytes);

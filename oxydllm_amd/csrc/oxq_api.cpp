@@ -1431,6 +1431,68 @@ int oxq_mxfp4_dequantize(oxq_ctx *ctx, void *stream, const oxq_tensor *blocks,
     return launch_mxfp4_dequant(ctx, (hipStream_t)stream, p, (float *)out->data);
 }
 
+// The grouped MXFP4 op behind the weight cache: the stacked expert tensors of a projection (keyed by the addresses
+// of blocks and scales) get the resident experts' tile-major copy on their first call; later calls run the decode
+// GEMV or the tiles of an expert's pairs on it, as an oxq_mxfp4_experts handle would.
+static bool wcache_forward_mxfp4(oxq_ctx *ctx, hipStream_t s, const Mxfp4Problem &p, int *rc) {
+    if (!ctx->wcache_limit || ctx->plan_only || p.n_experts <= 0 || !mxfp4_res_eligible(p.K, p.N)) return false;
+    if (((uintptr_t)p.x & 15) || ((uintptr_t)p.blocks & 15)) return false;
+    const bool prefill = (uint64_t)p.M * (uint64_t)p.K * 2u < (1ull << 31) && mxfp4_gemm_form(ctx, p.n_pairs, p.n_experts, p.K, p.N) != 0;
+    if (!prefill && p.n_pairs >= 8 * p.n_experts) return false;  // the tile matmul on the caller's tensors
+    const int kind = -3;
+    if (!ctx->wcache) {
+        ctx->wcache = new (std::nothrow) oxq_weight_cache();
+        if (!ctx->wcache) return false;
+    }
+    oxq_weight_cache *c = ctx->wcache;
+    ++c->tick;
+    oxq_weight_cache::Entry *hit = nullptr;
+    for (auto &e : c->entries)
+        if (e.qw == p.blocks && e.qz == nullptr && e.sc == p.scales && e.K == p.K && e.N == p.N && e.bits == (int)p.n_experts &&
+            e.pack_dim == kind) {
+            hit = &e;
+            break;
+        }
+    const size_t w_bytes = (mxfp4_res_weight_bytes(p.n_experts, p.K, p.N) + 255) & ~(size_t)255;
+    if (!hit) {
+        hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(s, &cs) != hipSuccess || cs != hipStreamCaptureStatusNone) {
+            (void)hipGetLastError();
+            return false;
+        }
+        const size_t bytes = w_bytes + ((mxfp4_res_scale_bytes(p.n_experts, p.K, p.N) + 255) & ~(size_t)255);
+        if (!wcache_make_room(ctx, bytes)) return false;
+        void *mem = nullptr;
+        if (hipMalloc(&mem, bytes) != hipSuccess) {
+            (void)hipGetLastError();
+            return false;
+        }
+        oxq_weight_cache::Entry e{p.blocks, nullptr, p.scales, p.K, p.N, 0, 0, (int)p.n_experts, kind,
+                                  Pk4Weights{(uint32_t *)mem, nullptr, p.K, p.N, 0, 0, 0, 0, 0, 0}, bytes, 0, false};
+        const int prc = launch_mxfp4_repack(ctx, s, p.blocks, p.scales, mem, (unsigned char *)mem + w_bytes, p.n_experts, p.K, p.N);
+        if (prc != OXQ_OK) {
+            (void)hipFree(mem);
+            *rc = prc;
+            return true;
+        }
+        try {
+            c->entries.push_back(e);
+        } catch (...) {
+            (void)hipFree(mem);
+            return false;
+        }
+        c->bytes += bytes;
+        hit = &c->entries.back();
+    }
+    hit->last_use = c->tick;
+    wcache_pin_if_capturing(s, hit);
+    Mxfp4Problem q = p;
+    q.blocks = (const uint8_t *)hit->w.pw;
+    q.scales = (const uint8_t *)hit->w.pw + w_bytes;
+    *rc = prefill ? launch_mxfp4_res_gemm(ctx, s, q) : launch_mxfp4_res_gemv(ctx, s, q);
+    return true;
+}
+
 static int moe_matmul_impl(const char *op, oxq_ctx *ctx, void *stream, const oxq_tensor *x, const oxq_tensor *blocks,
                            const oxq_tensor *scales, const oxq_tensor *bias, const oxq_tensor *expert_offsets,
                            const oxq_tensor *token_ids, int gather_rows, int64_t k, int64_t n, bool swiglu, float limit,
@@ -1471,6 +1533,11 @@ static int moe_matmul_impl(const char *op, oxq_ctx *ctx, void *stream, const oxq
     p.n_pairs = n_pairs;
     p.swiglu = swiglu ? 1 : 0;
     p.swiglu_limit = limit;
+    int crc = OXQ_OK;
+    if (wcache_forward_mxfp4(ctx, (hipStream_t)stream, p, &crc)) {
+        if (crc == OXQ_OK && fused) *fused = 1;
+        return crc;
+    }
     const int rc = launch_mxfp4_gemv(ctx, (hipStream_t)stream, p);
     if (rc == OXQ_DECLINED) return OXQ_OK;  // *fused stays 0, nothing was enqueued
     if (rc == OXQ_OK && fused) *fused = 1;

@@ -249,6 +249,53 @@ def test_cached_gguf_op_with_bf16_activations_runs_on_the_matrix_core_copy(fmt):
         ctx.close()
 
 
+def test_cached_mxfp4_moe_op_runs_on_the_resident_experts_copy():
+    """The grouped MXFP4 op with the cache on: the stacked expert tensors get the resident experts' tile-major copy on
+    the first call; decode sizes then run its GEMV, many pairs an expert its tiles, with the handle's bits and the
+    fused SwiGLU; forgetting the blocks goes back to the checkpoint-layout kernels."""
+    E, N, K = 4, 96, 2880
+    blocks, scales = synth.mxfp4_weight(E * N, K, seed=77)
+    bias = np.random.default_rng(78).standard_normal((E, N)).astype(np.float32) * 0.1
+    bd, sd, biasd = to_dev(blocks), to_dev(scales), to_dev(bias, torch.bfloat16)
+    ex = ops.Mxfp4Experts(bd, sd, biasd, E, K, N)
+    nb = K // 32
+    want_bytes = E * (N // 16) * nb * 256 + E * (N // 16) * -(-(-(-nb // 4)) // 4) * 256
+    ctx = ops.Context()
+    try:
+        ctx.set_weight_cache(1 << 24)
+        for counts, kern in [([1, 0, 2, 1], "mxfp4_experts_gemv_bf16_t4"), ([20, 0, 13, 7], "mxfp4_experts_gemm_bf16_r16x8"),
+                             ([70, 1, 40, 30], "mxfp4_experts_gemm_bf16_r32x8")]:
+            say(f"weight cache mxfp4 moe counts={counts}")
+            offsets = np.zeros(E + 1, np.int32)
+            offsets[1:] = np.cumsum(counts)
+            n_tok = max(counts)
+            tokens = np.concatenate([np.arange(c, dtype=np.int32) % n_tok for c in counts]).astype(np.int32)
+            x = np.random.default_rng(sum(counts)).standard_normal((n_tok, K)).astype(np.float32)
+            xd, off_d, tok_d = to_dev(x, torch.bfloat16), to_dev(offsets), to_dev(tokens)
+            y = ops.mxfp4_moe_matmul(xd, bd, sd, biasd, off_d, tok_d, K, N, ctx=ctx)
+            assert ctx.last_plan()["kernel"] == kern, ctx.last_plan()
+            np.testing.assert_array_equal(bits_of(y), bits_of(ex.matmul(xd, off_d, tok_d)))
+            ref = np.zeros((int(offsets[-1]), N), np.float32)
+            xb, bb = round_x(x, oracle.BF16), round_x(bias, oracle.BF16)
+            for e in range(E):
+                lo, hi = int(offsets[e]), int(offsets[e + 1])
+                if hi > lo:
+                    w = oracle.dequantize_mxfp4_f32(blocks[e * N * nb * 16:(e + 1) * N * nb * 16], scales[e * N * nb:(e + 1) * N * nb], N, K)
+                    ref[lo:hi] = oracle.matmul_nt_f32(xb[tokens[lo:hi]], w, bb[e])
+            assert_close(y, ref, f"cached mxfp4 moe op {counts}")
+            h = ops.mxfp4_moe_gate_up_swiglu(xd, bd, sd, biasd, off_d, tok_d, K, N, 7.0, ctx=ctx)
+            assert ctx.last_plan()["kernel"] == kern + "_swiglu"
+            np.testing.assert_array_equal(bits_of(h), bits_of(ex.gate_up_swiglu(xd, off_d, tok_d, 7.0)))
+        assert ctx.weight_cache_usage() == (want_bytes, 1)
+        ctx.forget_weights(bd)
+        assert ctx.weight_cache_usage() == (0, 0)
+        ctx.set_weight_cache(0)
+        ops.mxfp4_moe_matmul(xd, bd, sd, biasd, off_d, tok_d, K, N, ctx=ctx)
+        assert "experts" not in ctx.last_plan()["kernel"]
+    finally:
+        ctx.close()
+
+
 def test_capture_allocates_nothing_and_replays_the_cached_kernel():
     K, N, g, m = 2048, 512, 128, 4
     tdt = torch.float16
