@@ -164,6 +164,9 @@ def main():
     ap.add_argument("--prefill-only", action="store_true",
                     help="only the resident layers at prefill sizes (the first part of --all), as one JSON line "
                          "{\"prefill\": [...]}: a short run for a profiler")
+    ap.add_argument("--moe-only", action="store_true",
+                    help="only config 4's MXFP4 mixture-of-experts rows of --all (decode step, prefill layer steps), as one "
+                         "JSON line {\"moe\": [...]}: a short run for a profiler")
     ap.add_argument("--calib-copy", action="store_true",
                     help="first run a plain 256 MiB device copy 4 times: a kernel of known HBM "
                          "traffic to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings with")
@@ -193,6 +196,10 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
+    if args.moe_only:
+        import bench_extra
+        print(json.dumps({"moe": bench_extra.run_moe(ops, ctx, stream, args.steps, args.warmup, time_graph)}), flush=True)
+        return
     if args.prefill_only:
         import bench_extra
         rows = bench_extra.run_prefill(ops, ctx, stream, args.steps, args.warmup, time_graph)

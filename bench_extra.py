@@ -312,6 +312,16 @@ def run(ops, ctx, stream, steps, warmup, time_graph):
                              time_graph, wb.nbytes + scl.nbytes + m * (k8 + n8) * 2, 2.0 * m * k8 * n8, ctx))
         del d8
 
+    out.extend(run_moe(ops, ctx, stream, steps, warmup, time_graph))
+    return out
+
+
+def run_moe(ops, ctx, stream, steps, warmup, time_graph):
+    """Config 4's MXFP4 mixture-of-experts layer: the decode step through the stateless ops, one expert's projection
+    as a plain layer at prefill sizes, and whole layer steps at 512 and 2048 tokens through the stateless ops and on
+    the resident experts."""
+    dev = torch.device("cuda:0")
+    out = []
     # ---- config 4: MXFP4 MoE -----------------------------------------------------
     E, top_k, H, I, T = 32, 4, 2880, 2880, 8
     rng = np.random.default_rng(0x0A0D11E9)

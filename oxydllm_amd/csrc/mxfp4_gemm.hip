@@ -57,16 +57,19 @@ __global__ __launch_bounds__(512) void mxfp4_gemm_kernel(const uint16_t *__restr
     const __amdgpu_buffer_rsrc_t rs_s = make_rsrc(ps + et * NG * 256, live ? (uint32_t)live_tiles * (uint32_t)NG * 256u : 0u);
     const __amdgpu_buffer_rsrc_t rs_x = make_rsrc(x, x_bytes);
     const int voff_w = lane * 16, voff_s = lane * 4;
-    // x: load q of a wave brings rows 4 (XV wave + q) .. + 3 of a chunk straight into LDS, lane l
-    // the 16 bytes that belong at position l % 16 of row l / 16: chunk (l % 16) ^ (row % 16) of the row's 128
-    // elements, the swizzle the fragment reads undo.  Rows past the expert's pairs, and the elements past K in the
-    // last chunk, get an offset beyond the descriptor: LDS receives zeros.
+    // x: load q of a wave brings rows 4 (XV wave + q) .. + 3 of a chunk straight into LDS, lane l the 16 bytes that
+    // belong at position l % 16 of row l / 16.  Piece p = 4 kb + st of a row's 128 elements (what lane group kb reads
+    // in step st) is kept at position (4 st + kb) ^ (row % 16): the four lane groups of a fragment read then start in
+    // different banks (at position p ^ row, groups 0 and 2 would meet 128 bytes apart: four conflict cycles a read).
+    // Rows past the expert's pairs, and the elements past K in the last chunk, get an offset beyond the descriptor:
+    // LDS receives zeros.
     int xo[XV], xc[XV];
 #pragma unroll
     for (int q = 0; q < XV; ++q) {
         const int r = 4 * (wave * XV + q) + (lane >> 4);
         const int m = m0 + r;
-        xc[q] = (lane & 15) ^ (r & 15);
+        const int pos = (lane & 15) ^ (r & 15);
+        xc[q] = ((pos & 3) << 2) | (pos >> 2);  // the piece kept at this position
         int src = 0;
         if (m < m_end) src = token_ids ? token_ids[m] : m;
         xo[q] = m < m_end ? src * K * 2 + (xc[q] << 4) : OOB;
@@ -74,7 +77,7 @@ __global__ __launch_bounds__(512) void mxfp4_gemm_kernel(const uint16_t *__restr
     // fragment of step st, row tile mt (+ 4096 mt): row ni, elements 32 kb + 8 st .. + 7 of the chunk = piece 4 kb + st
     int a_rd[4];
 #pragma unroll
-    for (int st = 0; st < 4; ++st) a_rd[st] = ni * 256 + (((4 * kb + st) ^ ni) << 4);
+    for (int st = 0; st < 4; ++st) a_rd[st] = ni * 256 + (((4 * st + kb) ^ ni) << 4);
 
     u32x4_t wring[2][4];
     uint32_t sring[4];
@@ -169,24 +172,32 @@ __global__ __launch_bounds__(512) void mxfp4_gemm_kernel(const uint16_t *__restr
 #pragma unroll
     for (int f = 0; f < 4; ++f)
         if (bias && f < live_tiles) bv[f] = BF16Traits::to_f32(bias[(size_t)e * N + 64 * j + 16 * f + ni]);
+    // Neighbouring lanes hold neighbouring weight rows: the two lanes of a pair exchange their values (quad_perm
+    // [1, 0, 3, 2]) and share the work - the even lane finishes pairs i = 0 and 2 of the four, the odd lane 1 and 3.
+    const bool odd = ni & 1;
 #pragma unroll
     for (int t = 0; t < MT; ++t)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int m = m0 + 16 * t + 4 * kb + i;
+        for (int f = 0; f < 4; ++f) {
+            const int n = 64 * j + 16 * f + (ni & ~1);  // the lane pair's two weight rows: n, n + 1
+            float mine[4], other[4];
 #pragma unroll
-            for (int f = 0; f < 4; ++f) {
-                const int n = 64 * j + 16 * f + ni;
+            for (int i = 0; i < 4; ++i) {
+                // rounded to bf16 as the projection's own output is (for the SwiGLU: what it would read)
+                mine[i] = BF16Traits::to_f32(BF16Traits::from_f32(acc[t][f][i] + bv[f]));
+                other[i] = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, mine[i]), 0xB1, 0xF, 0xF, false));
+            }
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int i = 2 * h + (odd ? 1 : 0);
+                const int m = m0 + 16 * t + 4 * kb + i;
+                const float lo = odd ? other[2 * h + 1] : mine[2 * h], hi = odd ? mine[2 * h + 1] : other[2 * h];  // rows n, n + 1
+                if (m >= m_end || f >= live_tiles) continue;
                 if (swiglu) {
-                    // rows 2 c / 2 c + 1 are the gate / up of output c (moe.rs:152-173) and sit in neighbouring lanes:
-                    // each is rounded to bf16 as the projection's own output would be, the even lane takes its
-                    // neighbour's value (quad_perm [1, 0, 3, 2]) and stores the activation
-                    const float v = BF16Traits::to_f32(BF16Traits::from_f32(acc[t][f][i] + bv[f]));
-                    const float other = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, false));
-                    if (!(ni & 1) && m < m_end && f < live_tiles)
-                        y[(size_t)m * (N >> 1) + (n >> 1)] = BF16Traits::from_f32(gpt_oss_swiglu_f32(v, other, limit));
-                } else if (m < m_end && f < live_tiles) {
-                    y[(size_t)m * N + n] = BF16Traits::from_f32(acc[t][f][i] + bv[f]);
+                    // rows 2 c / 2 c + 1 are the gate / up of output c (moe.rs:152-173)
+                    y[(size_t)m * (N >> 1) + (n >> 1)] = BF16Traits::from_f32(gpt_oss_swiglu_f32(lo, hi, limit));
+                } else {
+                    *(uint32_t *)(y + (size_t)m * N + n) = (uint32_t)BF16Traits::from_f32(lo) | ((uint32_t)BF16Traits::from_f32(hi) << 16);
                 }
             }
         }
