@@ -247,6 +247,7 @@ int launch_mxfp4_res_gemm(oxq_ctx *ctx, hipStream_t s, const Mxfp4Problem &p) {
     const uint64_t x_bytes = (uint64_t)p.M * (uint64_t)p.K * 2u;
     if (x_bytes >= (1ull << 31)) return fail(OXQ_ERR_UNSUPPORTED, "mxfp4 experts prefill: x of %llu bytes exceeds 2 GiB", (unsigned long long)x_bytes);
     if ((uintptr_t)p.x & 15) return fail(OXQ_ERR_UNSUPPORTED, "mxfp4 experts prefill: x must be 16-byte aligned");
+    if ((uintptr_t)p.y & 3) return fail(OXQ_ERR_UNSUPPORTED, "mxfp4 experts prefill: out must be 4-byte aligned");
     switch (rows) {
     case 16: return mxfp4_gemm_go<1>(s, grid, p, NC, NG, (uint32_t)x_bytes);
     case 32: return mxfp4_gemm_go<2>(s, grid, p, NC, NG, (uint32_t)x_bytes);

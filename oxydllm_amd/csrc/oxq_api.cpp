@@ -1437,7 +1437,8 @@ int oxq_mxfp4_dequantize(oxq_ctx *ctx, void *stream, const oxq_tensor *blocks,
 static bool wcache_forward_mxfp4(oxq_ctx *ctx, hipStream_t s, const Mxfp4Problem &p, int *rc) {
     if (!ctx->wcache_limit || ctx->plan_only || p.n_experts <= 0 || !mxfp4_res_eligible(p.K, p.N)) return false;
     if (((uintptr_t)p.x & 15) || ((uintptr_t)p.blocks & 15)) return false;
-    const bool prefill = (uint64_t)p.M * (uint64_t)p.K * 2u < (1ull << 31) && mxfp4_gemm_form(ctx, p.n_pairs, p.n_experts, p.K, p.N) != 0;
+    const bool prefill = (uint64_t)p.M * (uint64_t)p.K * 2u < (1ull << 31) && ((uintptr_t)p.y & 3) == 0 &&
+                         mxfp4_gemm_form(ctx, p.n_pairs, p.n_experts, p.K, p.N) != 0;
     if (!prefill && p.n_pairs >= 8 * p.n_experts) return false;  // the tile matmul on the caller's tensors
     const int kind = -3;
     if (!ctx->wcache) {
@@ -1651,6 +1652,7 @@ static int experts_forward(oxq_mxfp4_experts *h, void *stream, const oxq_tensor 
     // (sizes it does not take) the tile matmul, which reads the checkpoint layout
     // (its 32-bit offsets into x hold up to 2 GiB; more than that takes the tile matmul as before)
     const bool prefill = resident && x && x->rank == 2 && (uint64_t)x->dims[0] * (uint64_t)h->k * 2u < (1ull << 31) &&
+                         ((uintptr_t)x->data & 15) == 0 && out && ((uintptr_t)out->data & 3) == 0 &&  // (two outputs a store)
                          mxfp4_gemm_form(ctx, n_pairs, h->n_experts, h->k, h->n) != 0;
     if (!resident || (!prefill && n_pairs >= 8 * h->n_experts))
         return moe_matmul_impl(op, ctx, stream, x, &h->blocks, &h->scales, h->has_bias ? &h->bias : nullptr, expert_offsets,

@@ -177,6 +177,13 @@ def test_experts_prefill_kernel_on_the_copy(E, N, K, counts, rows, gather):
     plain.matmul(xd, off_d, tok_d, out=out)
     assert ops.default_context().last_plan()["kernel"] == kname
     assert_close(out, ref - np.repeat(bb, counts, axis=0), "experts prefill matmul, no bias")
+    if rows == 32:
+        # an output that starts at an odd element (the tiles store two neighbouring outputs as one word): the tile
+        # matmul on the caller's tensors takes the call
+        buf = torch.zeros(n_pairs * N + 1, device="cuda", dtype=torch.bfloat16)
+        ex.matmul(xd, off_d, tok_d, out=buf[1:].view(n_pairs, N))
+        assert "mul_mm" in ops.default_context().last_plan()["kernel"], ops.default_context().last_plan()
+        assert_close(buf[1:].view(n_pairs, N), ref, "experts prefill matmul, odd output address")
     # interleaved gate / up rows with the clamped SwiGLU in the epilogue
     fused = ex.gate_up_swiglu(xd * 2, off_d, tok_d, 7.0)
     assert ops.default_context().last_plan()["kernel"] == kname + "_swiglu"
