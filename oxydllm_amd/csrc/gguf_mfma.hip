@@ -1067,7 +1067,8 @@ static int gguf_gemm_form(const oxq_ctx *ctx, int quant, int64_t M, int64_t N, i
     const double whole = std::floor(w64), rest = w64 - whole;
     const double c64 = whole + (rest <= 0.0 ? 0.0 : rest <= 0.75 ? 0.95 : 1.0);
     const double c_mid = ks == 1 ? 1e30 : std::ceil((double)(ceil_div(N / 64, (int64_t)2) * row_tiles) / cus) * GGM_MID_ROUND;
-    const double c_file = 0.17 + (light ? 1.45 : 1.3) * w64;
+    // (Q8_0's 34-byte blocks make the file layout's matmul 1.2 - 1.35 x the 4-bit formats' at the same shape)
+    const double c_file = 0.17 + (quant == OXQ_GGUF_Q8_0 ? 1.75 : light ? 1.45 : 1.3) * w64;
     if (c_file <= c64 && c_file <= c_mid) return 0;
     return c_mid < c64 ? 4 : 1;
 }
