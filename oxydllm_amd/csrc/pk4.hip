@@ -1221,8 +1221,8 @@ static int pk4_by_mt(oxq_ctx *ctx, hipStream_t s, dim3 grid, const Pk4Problem &p
 }
 
 // Strip width of a layer's resident copy: 16 columns for 4-bit layers of at most 128 64-column strips and a
-// K of 32 - 112 blocks (the shapes that otherwise leave CUs idle or need K slices and a second launch),
-// 64 otherwise.
+// K of 32 - 112 blocks, or at most 80 strips and 16 - 31 blocks (the shapes that otherwise leave CUs idle or need
+// K slices and a second launch), 64 otherwise.
 int pk4_choose_strip(const oxq_ctx *ctx, int64_t K, int64_t N, int bits, int64_t gate_half) {
     // Measured (f16; 64-column strips, with K slices where few -> 16-column strips, one launch up to 8 rows),
     // at 1 / 4 / 16 / 64 rows of x:
@@ -1239,7 +1239,13 @@ int pk4_choose_strip(const oxq_ctx *ctx, int64_t K, int64_t N, int bits, int64_t
     const int mode = tune(ctx, OXQ_TUNE_PK4_STRIP16, 1);  // 0 never, 1 by shape, 2 wherever the layout applies
     if (!mode || bits != 4 || gate_half || N % 64 != 0) return 64;
     if (mode == 2) return 16;
-    return (N / 64 <= 128 && N / 16 >= 128 && K / 128 >= 32 && K / 128 <= 112) ? 16 : 64;
+    // Shorter K (16 - 31 blocks: hidden sizes of 2048 - 3968) gains on layers up to 5120 columns, whose 64-column
+    // strips leave most CUs idle (3584 x 3584 at 1 / 8 / 16 / 64 rows 5.79 / 6.08 / 6.80 / 13.6 -> 3.57 / 4.08 / 5.05 /
+    // 12.45 us; 3072 x 3072 4.99 -> 3.41, 2048 x 2048 3.95 -> 3.14, 3584 x 4608 5.87 -> 4.28 at one row), and loses
+    // from 16 rows on at 8192 columns (3072 x 8192: 5.32 / 6.35 -> 4.66 / 7.06 at 1 / 16 rows).  A K beyond 112 blocks
+    // gains at 1 - 4 rows only (18944 x 3584: 9.88 / 10.52 -> 8.18 / 11.64 at 1 / 8 rows).
+    const int64_t nb = K / 128, wide = N / 64;
+    return (N / 16 >= 128 && ((nb >= 32 && nb <= 112 && wide <= 128) || (nb >= 16 && nb < 32 && wide <= 80))) ? 16 : 64;
 }
 
 template <typename TT, int MT, bool GS, int NS, int XQ, int NW = 8>

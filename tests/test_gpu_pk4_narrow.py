@@ -113,7 +113,7 @@ def test_narrow_layout_k_slices(ks, monkeypatch):
 
 
 @pytest.mark.parametrize("K,N", [(4096, 4096), (4096, 6144), (8192, 2048), (14336, 4096), (4096, 8192), (8192, 4096),
-                                 (6144, 4096)])
+                                 (6144, 4096), (3584, 3584), (2048, 2048), (3072, 5120)])
 def test_attention_and_down_projection_shapes_take_the_narrow_layout(K, N, monkeypatch):
     """By shape alone (no switch): one launch up to eight rows, up to 16 on whole rounds of strips and K <= 8192
     (16 waves a workgroup), the wide layout's answer within tolerance."""
@@ -178,11 +178,18 @@ def test_sixteen_wave_workgroups_on_a_long_k(kind, dtn, monkeypatch):
 
 
 def test_shapes_outside_the_rule_keep_the_wide_layout():
-    for K, N in [(14464, 2048), (4096, 1024), (4096, 14336), (2048, 4096)]:
+    """K beyond 112 blocks, fewer than 128 strips of 16, a layer that fills the chip with 64-column strips, a short K
+    (16 - 31 blocks) on more than 5120 columns, a K below 16 blocks; and the short K the rule does take."""
+    for K, N in [(14464, 2048), (4096, 1024), (4096, 14336), (2048, 8192), (1920, 2048)]:
         trip, pack_dim = make("awq", K, N, 128, seed=1)
         layer = layer_of(trip, pack_dim, oracle.F16)
         layer.forward(torch.zeros((1, K), device="cuda", dtype=torch.float16))
         assert "_n16x" not in kernel_of_last_call()["kernel"], (K, N)
+    for K, N in [(2048, 4096), (3584, 3584), (3968, 5120)]:
+        trip, pack_dim = make("awq", K, N, 128, seed=1)
+        layer = layer_of(trip, pack_dim, oracle.F16)
+        layer.forward(torch.zeros((1, K), device="cuda", dtype=torch.float16))
+        assert "_n16x" in kernel_of_last_call()["kernel"], (K, N)
     trip = synth.gptq_checkpoint(4096, 4096, 128, 8, seed=2)
     l8 = ops.PackedQuantLinear(8, ops.PACK_IN, to_dev(trip[0]), to_dev(trip[1]), to_dev(trip[2], torch.float16), None,
                                torch.float16)
