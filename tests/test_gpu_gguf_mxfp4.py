@@ -610,6 +610,35 @@ def test_moe_step_config4_end_to_end():
     assert err.max() < 2e-2 * np.abs(out_ref).max() + 1e-2, err.max()
 
 
+@pytest.mark.parametrize("dtn", ["bf16", "f16"])
+@pytest.mark.parametrize("T,H,k", [(700, 768, 4), (260, 2880, 4), (1200, 512, 8), (300, 2884, 4)])
+def test_moe_combine_at_prefill_sizes(dtn, T, H, k):
+    """moe.rs:592-605 at prefill sizes: from 2^19 outputs on, 16-bit types and H a multiple of 8 take eight columns a
+    thread (16-byte loads and stores); the sums run in slot order in f32 either way, so the result equals the slot
+    loop restated in torch bit for bit, and the scalar kernel's (an output buffer that starts 8 bytes off a 16-byte
+    boundary takes that one).  H = 2884 is not a multiple of 8: the scalar kernel."""
+    tdt = torch.bfloat16 if dtn == "bf16" else torch.float16
+    say(f"moe combine {dtn} T={T} H={H} k={k}")
+    g = torch.Generator(device="cpu").manual_seed(T + H)
+    P = T * k
+    eo = torch.randn((P, H), generator=g).to(tdt).cuda()
+    pos = torch.randperm(P, generator=g).to(torch.int32).view(T, k).cuda()
+    vals = torch.rand((T, k), generator=g).cuda()
+    out = ops.moe_combine(eo, pos, vals)
+    vec = H % 8 == 0
+    assert ops.default_context().last_plan()["kernel"] == ("moe_combine_x8" if vec else "moe_combine")
+    acc = torch.zeros((T, H), device="cuda", dtype=torch.float32)
+    for s in range(k):  # fmaf(w, v, acc) in slot order; the product of a 16-bit value and an f32 weight needs the fma
+        acc = torch.addcmul(acc.double(), vals[:, s:s + 1].double(), eo[pos[:, s].long()].double()).float()
+    want = acc.to(tdt)
+    assert torch.equal(out.view(torch.int16), want.view(torch.int16))
+    buf = torch.zeros(T * H + 4, device="cuda", dtype=tdt)
+    off = buf[4:].view(T, H)
+    ops.moe_combine(eo, pos, vals, out=off)
+    assert ops.default_context().last_plan()["kernel"] == "moe_combine"
+    assert torch.equal(off.view(torch.int16), out.view(torch.int16))
+
+
 @pytest.mark.parametrize("E,N,K,counts,bias", [(4, 64, 64, (1, 0, 3, 2), True), (3, 38, 96, (5, 1, 0), False),
                                                (2, 6, 32, (9, 4), True), (5, 130, 160, (0, 0, 2, 0, 1), True)])
 def test_mxfp4_moe_gate_up_swiglu_fused(E, N, K, counts, bias, monkeypatch):
